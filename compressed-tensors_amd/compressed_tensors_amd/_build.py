@@ -1,0 +1,61 @@
+"""Compile libctmi.so (HIP, gfx950) in-tree with hipcc.
+
+    python -m compressed_tensors_amd._build        # or  build_library()
+
+hipcc cross-compiles for gfx950 without a GPU.  The library lands next to this
+file (lib/libctmi.so); it is git-ignored but travels with the source tree.
+"""
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC_DIR = PKG_DIR.parent / "csrc"
+INCLUDE_DIR = PKG_DIR.parent.parent / "include"
+LIB_DIR = PKG_DIR / "lib"
+LIB_PATH = LIB_DIR / "libctmi.so"
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-shared",
+    # correctly rounded fp32 division and no contraction: results must match torch bit for bit
+    "-fhip-fp32-correctly-rounded-divide-sqrt",
+    "-ffp-contract=off",
+    "-fno-fast-math",
+    # do not let the compiler form packed-fp32 instructions
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+]
+
+
+def sources():
+    return sorted(str(p) for p in CSRC_DIR.glob("*.hip"))
+
+
+def build_library(verbose: bool = False) -> Path:
+    LIB_DIR.mkdir(parents=True, exist_ok=True)
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    cmd = [HIPCC, *FLAGS, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", *sources(), "-o", str(tmp)]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    proc = subprocess.run(cmd, capture_output=True, text=True)
+    noise = "is not a recognized feature for this target"
+    err = "\n".join(l for l in proc.stderr.splitlines() if noise not in l)
+    if proc.returncode != 0:
+        raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
+    if verbose and err.strip():
+        print(err, file=sys.stderr)
+    os.replace(tmp, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

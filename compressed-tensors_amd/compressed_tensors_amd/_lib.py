@@ -1,0 +1,207 @@
+"""ctypes binding of libctmi.so (the C ABI declared in include/ctmi.h).
+
+torch is imported first on purpose: libctmi.so needs the HIP runtime by soname,
+and importing torch maps the one torch itself uses, so both share a single
+runtime (and therefore streams and allocations).
+
+There is no CPU fallback: every call needs the compiled library, and every
+tensor handed to a kernel must live on a GPU.
+"""
+import ctypes
+from ctypes import POINTER, c_char_p, c_float, c_int32, c_int64, c_void_p
+from pathlib import Path
+from typing import Optional
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libctmi.so"
+
+CTMI_OK = 0
+CTMI_ERR_VALUE = -1
+CTMI_ERR_UNSUPPORTED = -2
+CTMI_ERR_ASSERT = -3
+CTMI_ERR_HIP = -4
+
+F32, F16, BF16, F8E4M3, I8, I16, I32, I64, U8, BOOL = range(10)
+QTYPE_INT, QTYPE_FLOAT = 0, 1
+
+_DTYPE_CODE = {
+    torch.float32: F32,
+    torch.float16: F16,
+    torch.bfloat16: BF16,
+    torch.float8_e4m3fn: F8E4M3,
+    torch.int8: I8,
+    torch.int16: I16,
+    torch.int32: I32,
+    torch.int64: I64,
+    torch.uint8: U8,
+    torch.bool: BOOL,
+}
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise NotImplementedError(f"dtype {dtype} is not supported by the HIP kernels")
+
+
+class QParams(ctypes.Structure):
+    """mirror of `struct ctmi_qparams`"""
+
+    _fields_ = [
+        ("scale", c_void_p),
+        ("zero_point", c_void_p),
+        ("global_scale", c_void_p),
+        ("col_group", c_void_p),
+        ("s_rows", c_int64),
+        ("s_cols", c_int64),
+        ("blk_rows", c_int64),
+        ("blk_cols", c_int64),
+        ("scale_dtype", c_int32),
+        ("zp_dtype", c_int32),
+        ("qtype", c_int32),
+        ("num_bits", c_int32),
+    ]
+
+
+_QP = POINTER(QParams)
+
+# name -> (restype, argtypes); must list every symbol of include/ctmi.h
+SIGNATURES = {
+    "ctmi_last_error": (c_char_p, []),
+    "ctmi_version": (c_int32, []),
+    "ctmi_qdq": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int64, _QP, c_int32, c_int32, c_void_p],
+    ),
+    "ctmi_pack_to_int32": (
+        c_int32,
+        [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p],
+    ),
+    "ctmi_unpack_from_int32": (
+        c_int32,
+        [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p],
+    ),
+    "ctmi_pack_quantized_compress": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int64, c_int64, _QP, c_void_p],
+    ),
+    "ctmi_pack_quantized_decompress": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int64, c_int64, _QP, c_void_p],
+    ),
+    "ctmi_pack_fp4_to_uint8": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_void_p]),
+    "ctmi_unpack_fp4_from_uint8": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int64, c_int64, c_void_p],
+    ),
+    "ctmi_nvfp4_compress": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int64, c_int64, _QP, c_void_p],
+    ),
+    "ctmi_nvfp4_decompress": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int64, c_int64, _QP, c_void_p],
+    ),
+    "ctmi_pack_bitmasks": (c_int32, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "ctmi_unpack_bitmasks": (c_int32, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "ctmi_bitmask_tmp_bytes": (c_int64, [c_int64]),
+    "ctmi_bitmask_count": (
+        c_int32,
+        [c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64,
+         c_void_p],
+    ),
+    "ctmi_bitmask_compact": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    ),
+    "ctmi_bitmask_decompress": (
+        c_int32,
+        [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    ),
+    "ctmi_get_24_bytemasks": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
+    "ctmi_sparse24_compress": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    ),
+    "ctmi_topk24_lut": (None, [c_void_p]),
+    "ctmi_calculate_qparams": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32, c_void_p,
+         c_void_p, c_int32, c_void_p, c_int32, c_void_p],
+    ),
+    "ctmi_generate_gparam": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p]),
+    "ctmi_minmax_tmp_bytes": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int32]),
+    "ctmi_minmax": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
+         c_void_p],
+    ),
+    "ctmi_observe_qparams": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p,
+         c_void_p, c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_void_p],
+    ),
+}
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def load() -> ctypes.CDLL:
+    """Load libctmi.so (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with "
+                "`python -m compressed_tensors_amd._build` (there is no CPU fallback)"
+            )
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = restype
+            fn.argtypes = argtypes
+        _lib = lib
+    return _lib
+
+
+_EXC = {
+    CTMI_ERR_VALUE: ValueError,
+    CTMI_ERR_UNSUPPORTED: NotImplementedError,
+    CTMI_ERR_ASSERT: AssertionError,
+    CTMI_ERR_HIP: RuntimeError,
+}
+
+
+def check(rc: int) -> None:
+    if rc != CTMI_OK:
+        msg = load().ctmi_last_error().decode("utf-8", "replace")
+        raise _EXC.get(rc, RuntimeError)(msg)
+
+
+def require_gpu(*tensors: Optional[torch.Tensor]) -> torch.device:
+    """All given tensors must sit on one GPU; returns that device."""
+    dev = None
+    for t in tensors:
+        if t is None:
+            continue
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                f"compressed_tensors_amd kernels run on the GPU only, got a tensor on {t.device}"
+            )
+        if dev is None:
+            dev = t.device
+        elif t.device != dev:
+            raise RuntimeError(f"tensors live on different devices: {dev} and {t.device}")
+    if dev is None:
+        raise RuntimeError("no tensor given")
+    return dev
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def stream_of(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

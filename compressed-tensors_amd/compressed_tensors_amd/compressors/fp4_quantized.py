@@ -1,0 +1,148 @@
+"""`nvfp4-pack-quantized`: e2m1 codes, two per byte.
+
+Reference: compressors/quantized_compressors/fp4_quantized.py
+(NVFP4PackedCompressor :44-123, pack_fp4_to_uint8 :135-178,
+unpack_fp4_from_uint8 :187-221).
+"""
+import ctypes
+from typing import Dict, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from compressed_tensors_amd import _lib
+from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
+from compressed_tensors_amd.compressors.quantized_base import BaseQuantizationCompressor
+from compressed_tensors_amd.config import CompressionFormat
+from compressed_tensors_amd.quantization.forward import (
+    _ShapeOnly,
+    build_qparams,
+    infer_dequant_args,
+)
+from compressed_tensors_amd.quantization.quant_args import QuantizationArgs
+
+__all__ = [
+    "NVFP4PackedCompressor",
+    "MXFP4PackedCompressor",
+    "pack_fp4_to_uint8",
+    "unpack_fp4_from_uint8",
+    "FLOAT_TO_E2M1",
+]
+
+FLOAT_TO_E2M1 = [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+_FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+
+def pack_fp4_to_uint8(x: Tensor) -> Tensor:
+    """[m, n] e2m1-valued tensor -> uint8 [m, n/2]; low nibble first, sign in bit 3."""
+    m, n = x.shape
+    if n % 2 != 0:
+        raise ValueError("tensor must have an even number of columns for nvfp4 compression")
+    x = to_gpu(x).contiguous()
+    if x.dtype not in _FLOATS:
+        raise NotImplementedError(f"fp4 packing of dtype {x.dtype} is not supported")
+    out = torch.empty((m, n // 2), dtype=torch.uint8, device=x.device)
+    _lib.check(
+        _lib.load().ctmi_pack_fp4_to_uint8(
+            x.data_ptr(), _lib.dtype_code(x.dtype), out.data_ptr(), m, n,
+            _lib.stream_of(x.device),
+        )
+    )
+    return out
+
+
+def unpack_fp4_from_uint8(
+    a: Tensor, m: int, n: int, dtype: Optional[torch.dtype] = torch.bfloat16
+) -> Tensor:
+    """uint8 [m, n/2] -> [m, n] of `dtype`"""
+    assert a.dtype == torch.uint8
+    a = to_gpu(a).contiguous()
+    if a.numel() * 2 != m * n:
+        raise RuntimeError(f"cannot unpack {a.numel()} bytes into [{m}, {n}]")
+    out = torch.empty((m, n), dtype=dtype, device=a.device)
+    _lib.check(
+        _lib.load().ctmi_unpack_fp4_from_uint8(
+            a.data_ptr(), out.data_ptr(), _lib.dtype_code(dtype), m, n, _lib.stream_of(a.device)
+        )
+    )
+    return out
+
+
+@BaseCompressor.register(name=CompressionFormat.nvfp4_pack_quantized.value)
+class NVFP4PackedCompressor(BaseQuantizationCompressor):
+    @property
+    def compression_param_names(self) -> Tuple[str]:
+        return ("weight_packed", "weight_scale", "weight_zero_point", "weight_global_scale")
+
+    def compression_param_info(
+        self, weight_shape: torch.Size, quantization_args: Optional[QuantizationArgs] = None
+    ) -> Dict[str, Tuple[torch.Size, torch.dtype]]:
+        return {
+            "weight_packed": (torch.Size((weight_shape[0], weight_shape[1] // 2)), torch.uint8)
+        }
+
+    def compress_weight(
+        self,
+        weight: Tensor,
+        scale: Tensor,
+        global_scale: Tensor,
+        quantization_args: QuantizationArgs,
+        device: Optional[torch.device] = None,
+        zero_point: Optional[Tensor] = None,
+        g_idx: Optional[Tensor] = None,
+    ) -> Dict[str, Tensor]:
+        weight, scale, global_scale, zero_point = (
+            to_gpu(t) for t in (weight, scale, global_scale, zero_point)
+        )
+        if weight.ndim != 2:
+            raise ValueError(f"expected a 2-D weight, got shape {tuple(weight.shape)}")
+        # the reference does not forward g_idx to quantize()
+        plan = build_qparams(weight, scale, zero_point, quantization_args, None, global_scale)
+        w = weight.contiguous()
+        rows, cols = w.shape
+        if cols % 2 != 0:
+            raise ValueError("tensor must have an even number of columns for nvfp4 compression")
+        packed = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
+        _lib.check(
+            _lib.load().ctmi_nvfp4_compress(
+                w.data_ptr(), _lib.dtype_code(w.dtype), packed.data_ptr(), rows, cols,
+                ctypes.byref(plan.qp), _lib.stream_of(w.device),
+            )
+        )
+        if device is not None:
+            packed = packed.to(device)
+        return {"weight_packed": packed}
+
+    def decompress_weight(
+        self,
+        compressed_data: Dict[str, Tensor],
+        quantization_args: Optional[QuantizationArgs] = None,
+    ) -> Tensor:
+        packed = to_gpu(compressed_data["weight_packed"]).contiguous()
+        scale = to_gpu(compressed_data["weight_scale"])
+        global_scale = to_gpu(compressed_data["weight_global_scale"])
+        assert packed.dtype == torch.uint8
+        m, half = packed.shape
+        shape = torch.Size((m, half * 2))
+        # unpack to bf16, then dequantize(x_q, scale, global_scale, dtype=bf16) with
+        # the strategy inferred from the scale's shape
+        carrier = _ShapeOnly(shape, torch.bfloat16)
+        dq_args = infer_dequant_args(carrier, scale)
+        plan = build_qparams(carrier, scale, None, dq_args, None, global_scale)
+        plan.qp.qtype = _lib.QTYPE_FLOAT
+        plan.qp.num_bits = 4
+        # only the group path of the reference honours the requested bf16 output
+        out_dtype = torch.bfloat16 if plan.grouped else plan.dequant_dtype
+        out = torch.empty(shape, dtype=out_dtype, device=packed.device)
+        _lib.check(
+            _lib.load().ctmi_nvfp4_decompress(
+                packed.data_ptr(), out.data_ptr(), _lib.dtype_code(out_dtype), shape[0], shape[1],
+                ctypes.byref(plan.qp), _lib.stream_of(packed.device),
+            )
+        )
+        return out
+
+
+@BaseCompressor.register(name=CompressionFormat.mxfp4_pack_quantized.value)
+class MXFP4PackedCompressor(NVFP4PackedCompressor):
+    pass

@@ -1,0 +1,213 @@
+"""`pack-quantized`: integer weights packed 32/num_bits to an int32.
+
+Reference: compressors/quantized_compressors/pack_quantized.py
+(PackedQuantizationCompressor :33-183, pack_to_int32 :186-246,
+unpack_from_int32 :249-309).  compress_weight / decompress_weight run as one
+fused kernel each (quantize+pack, unpack+dequantize); the free functions pack
+and unpack int8 tensors on their own.
+"""
+import ctypes
+import math
+from typing import Dict, Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from compressed_tensors_amd import _lib
+from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
+from compressed_tensors_amd.compressors.quantized_base import BaseQuantizationCompressor
+from compressed_tensors_amd.config import CompressionFormat
+from compressed_tensors_amd.quantization.forward import (
+    _ShapeOnly,
+    build_qparams,
+    infer_dequant_args,
+)
+from compressed_tensors_amd.quantization.helpers import can_quantize
+from compressed_tensors_amd.quantization.quant_args import QuantizationArgs, QuantizationStrategy
+
+__all__ = ["PackedQuantizationCompressor", "pack_to_int32", "unpack_from_int32"]
+
+_PACKABLE = (QuantizationStrategy.GROUP.value, QuantizationStrategy.CHANNEL.value)
+
+
+def pack_to_int32(value: Tensor, num_bits: int, packed_dim: int = 1) -> Tensor:
+    """int8 [R, C] -> int32 [R, ceil(C/pf)] (or [ceil(R/pf), C] for packed_dim=0)."""
+    if value.dtype is not torch.int8:
+        raise ValueError("Tensor must be quantized to torch.int8 before packing")
+    if num_bits > 8:
+        raise ValueError("Packing is only supported for less than 8 bits")
+    if num_bits < 1:
+        raise ValueError(f"num_bits must be at least 1, got {num_bits}")
+    if value.ndim != 2:
+        raise ValueError(f"expected a 2-D tensor, got shape {tuple(value.shape)}")
+    value = to_gpu(value).contiguous()
+    rows, cols = value.shape
+    pf = 32 // num_bits
+    shape = (rows, math.ceil(cols / pf)) if packed_dim == 1 else (math.ceil(rows / pf), cols)
+    out = torch.empty(shape, dtype=torch.int32, device=value.device)
+    _lib.check(
+        _lib.load().ctmi_pack_to_int32(
+            value.data_ptr(), out.data_ptr(), rows, cols, num_bits, packed_dim,
+            _lib.stream_of(value.device),
+        )
+    )
+    return out
+
+
+def unpack_from_int32(
+    value: Tensor, num_bits: int, shape: torch.Size, packed_dim: int = 1
+) -> Tensor:
+    """inverse of pack_to_int32; `shape` is the unpacked shape (padding is cut off)."""
+    if value.dtype is not torch.int32:
+        raise ValueError(f"Expected {torch.int32} but got {value.dtype}, Aborting unpack.")
+    if num_bits > 8:
+        raise ValueError("Unpacking is only supported for less than 8 bits")
+    value = to_gpu(value)
+    pf = 32 // num_bits
+    if packed_dim == 1:
+        rows = value.shape[0]
+        cols = min(int(shape[1]), value.shape[1] * pf)
+        need = math.ceil(cols / pf)
+        if value.shape[1] != need:
+            value = value[:, :need]
+    else:
+        cols = value.shape[1]
+        rows = min(int(shape[0]), value.shape[0] * pf)
+        need = math.ceil(rows / pf)
+        if value.shape[0] != need:
+            value = value[:need, :]
+    value = value.contiguous()
+    out = torch.empty((rows, cols), dtype=torch.int8, device=value.device)
+    _lib.check(
+        _lib.load().ctmi_unpack_from_int32(
+            value.data_ptr(), out.data_ptr(), rows, cols, num_bits, packed_dim,
+            _lib.stream_of(value.device),
+        )
+    )
+    return out
+
+
+@BaseCompressor.register(name=CompressionFormat.pack_quantized.value)
+class PackedQuantizationCompressor(BaseQuantizationCompressor):
+    packs_zero_points = True
+
+    @property
+    def compression_param_names(self) -> Tuple[str]:
+        return (
+            "weight_packed",
+            "weight_scale",
+            "weight_zero_point",
+            "weight_g_idx",
+            "weight_shape",
+        )
+
+    def compression_param_info(
+        self, weight_shape: torch.Size, quantization_args: Optional[QuantizationArgs] = None
+    ) -> Dict[str, Tuple[torch.Size, torch.dtype]]:
+        pf = 32 // quantization_args.num_bits
+        info = {
+            "weight_packed": (
+                torch.Size((weight_shape[0], math.ceil(weight_shape[1] / pf))),
+                torch.int32,
+            ),
+            "weight_shape": (torch.Size((2,)), torch.int32),
+        }
+        if not quantization_args.symmetric and quantization_args.strategy in _PACKABLE:
+            zp_factor = (
+                quantization_args.group_size
+                if quantization_args.strategy == QuantizationStrategy.GROUP.value
+                else weight_shape[-1]
+            )
+            info["weight_zero_point"] = (
+                torch.Size((math.ceil(weight_shape[0] / pf), weight_shape[-1] // zp_factor)),
+                torch.int32,
+            )
+        return info
+
+    def compress_weight(
+        self,
+        weight: Tensor,
+        scale: Tensor,
+        quantization_args: QuantizationArgs,
+        zero_point: Optional[Tensor] = None,
+        g_idx: Optional[Tensor] = None,
+        device: Optional[torch.device] = None,
+        global_scale: Optional[Tensor] = None,
+    ) -> Dict[str, Tensor]:
+        if global_scale is not None:
+            raise ValueError("global_scale is not supported for the PackQuantizationCompressor")
+        args = quantization_args
+        weight, scale, zero_point, g_idx = (to_gpu(t) for t in (weight, scale, zero_point, g_idx))
+
+        if can_quantize(weight, args):
+            if weight.ndim != 2:
+                raise ValueError(f"expected a 2-D weight, got shape {tuple(weight.shape)}")
+            plan = build_qparams(weight, scale, zero_point, args, g_idx, None)
+            w = weight.contiguous()
+            rows, cols = w.shape
+            pf = 32 // max(1, min(args.num_bits, 32))
+            packed = torch.empty(
+                (rows, math.ceil(cols / max(pf, 1))), dtype=torch.int32, device=w.device
+            )
+            _lib.check(
+                _lib.load().ctmi_pack_quantized_compress(
+                    w.data_ptr(), _lib.dtype_code(w.dtype), packed.data_ptr(), rows, cols,
+                    ctypes.byref(plan.qp), _lib.stream_of(w.device),
+                )
+            )
+        else:
+            packed = pack_to_int32(weight, args.num_bits)
+
+        weight_shape = torch.tensor(weight.shape)
+        if device is not None:
+            packed = packed.to(device)
+            weight_shape = weight_shape.to(device)
+        out = {"weight_shape": weight_shape, "weight_packed": packed}
+        if not args.symmetric and args.strategy in _PACKABLE:
+            out["weight_zero_point"] = pack_to_int32(zero_point, args.num_bits, packed_dim=0)
+        return out
+
+    def decompress_weight(
+        self,
+        compressed_data: Dict[str, Tensor],
+        quantization_args: Optional[QuantizationArgs] = None,
+    ) -> Tensor:
+        args = quantization_args
+        packed = to_gpu(compressed_data["weight_packed"])
+        scale = to_gpu(compressed_data["weight_scale"])
+        zero_point = to_gpu(compressed_data.get("weight_zero_point", None))
+        g_idx = to_gpu(compressed_data.get("weight_g_idx", None))
+        shape = torch.Size(int(d) for d in compressed_data["weight_shape"])
+        num_bits = args.num_bits
+        if packed.dtype is not torch.int32:
+            raise ValueError(f"Expected {torch.int32} but got {packed.dtype}, Aborting unpack.")
+        if num_bits > 8:
+            raise ValueError("Unpacking is only supported for less than 8 bits")
+
+        if not args.symmetric and args.strategy in _PACKABLE:
+            assert zero_point is not None, "Asymmetric quantization requires zero-point values"
+            zero_point = unpack_from_int32(
+                zero_point, num_bits, (shape[0], scale.shape[-1]), packed_dim=0
+            )
+
+        # dequantize(x_q, scale, zero_point, g_idx) with args=None: strategy is
+        # inferred from the scale's shape, output dtype is the scale's
+        carrier = _ShapeOnly(shape, torch.int8)
+        dq_args = infer_dequant_args(carrier, scale)
+        plan = build_qparams(carrier, scale, zero_point, dq_args, g_idx, None)
+        plan.qp.qtype = _lib.QTYPE_INT
+        plan.qp.num_bits = num_bits
+        rows, cols = shape
+        pf = 32 // num_bits
+        need = math.ceil(cols / pf)
+        if packed.shape[1] != need:
+            packed = packed[:, :need]
+        packed = packed.contiguous()
+        out = torch.empty(shape, dtype=scale.dtype, device=packed.device)
+        _lib.check(
+            _lib.load().ctmi_pack_quantized_decompress(
+                packed.data_ptr(), out.data_ptr(), _lib.dtype_code(scale.dtype), rows, cols,
+                ctypes.byref(plan.qp), _lib.stream_of(packed.device),
+            )
+        )
+        return out

@@ -1,0 +1,150 @@
+"""`sparse-24-bitmask`: the two survivors of every group of four + packed bitmask.
+
+Reference: compressors/sparse_compressors/sparse_24_bitmask.py
+(Sparse24BitMaskCompressor :37-67, Sparse24BitMaskTensor :70-159,
+sparse24_bitmask_compress :162-203, sparse24_bitmask_decompress :206-224,
+get_24_bytemasks :227-260).
+"""
+from dataclasses import dataclass
+from typing import Dict, List, Tuple, Union
+
+import torch
+from torch import Tensor
+
+from compressed_tensors_amd import _lib
+from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
+from compressed_tensors_amd.compressors.sparse_base import BaseSparseCompressor
+from compressed_tensors_amd.compressors.sparse_bitmask import _scatter
+from compressed_tensors_amd.config import CompressionFormat, SparsityStructure
+from compressed_tensors_amd.utils.helpers import merge_names
+
+__all__ = [
+    "Sparse24BitMaskCompressor",
+    "Sparse24BitMaskTensor",
+    "sparse24_bitmask_compress",
+    "sparse24_bitmask_decompress",
+    "get_24_bytemasks",
+]
+
+_RANKABLE = (torch.float32, torch.float16, torch.bfloat16, torch.float8_e4m3fn, torch.int8)
+
+
+def _check_dtype(dtype: torch.dtype) -> None:
+    if dtype not in _RANKABLE:
+        raise NotImplementedError(f"2:4 masks of dtype {dtype} are not supported")
+
+
+def get_24_bytemasks(tensor: Tensor) -> Tensor:
+    """bool mask keeping, in every run of four elements, the two that
+    `abs().topk(2)` keeps (float8 tensors are ranked through their int8 view)."""
+    x = to_gpu(tensor).contiguous()
+    _check_dtype(x.dtype)
+    if x.numel() % 4 != 0:
+        raise ValueError("Tensor size must be a multiple of 4 for TWO_FOUR sparsity")
+    mask = torch.empty(x.shape, dtype=torch.bool, device=x.device)
+    _lib.check(
+        _lib.load().ctmi_get_24_bytemasks(
+            x.data_ptr(), _lib.dtype_code(x.dtype), mask.data_ptr(), x.numel(),
+            _lib.stream_of(x.device),
+        )
+    )
+    return mask
+
+
+def sparse24_bitmask_compress(
+    tensor: Tensor,
+    sparsity_structure: Union[SparsityStructure, str] = SparsityStructure.TWO_FOUR,
+) -> Tuple[Tensor, Tensor]:
+    """dense [R, C] -> (values [R, C/2], bitmask uint8 [R, ceil(C/8)])"""
+    assert len(tensor.shape) == 2, "Only 2D tensors are supported"
+    assert (
+        SparsityStructure(sparsity_structure) == SparsityStructure.TWO_FOUR
+    ), "Only 2:4 sparsity is supported"
+    rows, cols = tensor.shape
+    if tensor.is_meta:
+        return (
+            torch.empty((rows, cols // 2), dtype=tensor.dtype, device="meta"),
+            torch.empty((rows, (cols + 7) // 8), dtype=torch.uint8, device="meta"),
+        )
+    x = to_gpu(tensor).contiguous()
+    _check_dtype(x.dtype)
+    if x.numel() % 4 != 0:
+        raise ValueError("Tensor size must be a multiple of 4 for TWO_FOUR sparsity")
+    values = torch.empty((rows, cols // 2), dtype=x.dtype, device=x.device)
+    bitmask = torch.empty((rows, (cols + 7) // 8), dtype=torch.uint8, device=x.device)
+    _lib.check(
+        _lib.load().ctmi_sparse24_compress(
+            x.data_ptr(), _lib.dtype_code(x.dtype), values.data_ptr(), bitmask.data_ptr(), rows,
+            cols, _lib.stream_of(x.device),
+        )
+    )
+    return values, bitmask
+
+
+def sparse24_bitmask_decompress(
+    values: Tensor, bitmasks: Tensor, original_shape: torch.Size
+) -> Tensor:
+    return _scatter(values, bitmasks, None, original_shape)
+
+
+@dataclass
+class Sparse24BitMaskTensor:
+    shape: List[int]
+    compressed: Tensor
+    bitmask: Tensor
+
+    @staticmethod
+    def from_dense(
+        tensor: Tensor,
+        sparsity_structure: Union[SparsityStructure, str] = SparsityStructure.TWO_FOUR,
+    ) -> "Sparse24BitMaskTensor":
+        compressed, bitmask = sparse24_bitmask_compress(tensor, sparsity_structure)
+        return Sparse24BitMaskTensor(shape=list(tensor.shape), compressed=compressed,
+                                     bitmask=bitmask)
+
+    @staticmethod
+    def from_compressed_data(
+        shape: Union[List[int], Tensor], compressed: Tensor, bitmask: Tensor
+    ) -> "Sparse24BitMaskTensor":
+        if isinstance(shape, Tensor):
+            shape = shape.flatten().tolist()
+        return Sparse24BitMaskTensor(shape=[int(d) for d in shape], compressed=compressed,
+                                     bitmask=bitmask)
+
+    def decompress(self) -> Tensor:
+        return sparse24_bitmask_decompress(self.compressed, self.bitmask, self.shape)
+
+    def curr_memory_size_bytes(self) -> int:
+        return sum(t.element_size() * t.nelement() for t in (self.compressed, self.bitmask))
+
+    def dict(self, name_prefix: str, device=None) -> Dict[str, Tensor]:
+        if name_prefix.endswith(".weight"):
+            name_prefix = name_prefix[: -len(".weight")]
+
+        def mv(t):
+            return t if device is None else t.to(device)
+
+        return {
+            merge_names(name_prefix, "shape"): mv(torch.tensor(self.shape).reshape(-1, 1)),
+            merge_names(name_prefix, "compressed"): mv(self.compressed),
+            merge_names(name_prefix, "bitmask"): mv(self.bitmask),
+        }
+
+    def __repr__(self) -> str:
+        return f"BitMaskTensor(shape={self.shape}, compressed=True)"
+
+
+@BaseCompressor.register(name=CompressionFormat.sparse_24_bitmask.value)
+class Sparse24BitMaskCompressor(BaseSparseCompressor):
+    @property
+    def compression_param_names(self) -> Tuple[str]:
+        return ("shape", "compressed", "bitmask")
+
+    def compress_weight(self, name, value):
+        structure = getattr(self.config, "sparsity_structure", SparsityStructure.TWO_FOUR.value)
+        tensor = Sparse24BitMaskTensor.from_dense(value, structure)
+        return tensor.dict(name_prefix=name,
+                           device="meta" if value.is_meta else self.output_device)
+
+    def decompress_weight(self, weight_data):
+        return Sparse24BitMaskTensor.from_compressed_data(**weight_data).decompress()

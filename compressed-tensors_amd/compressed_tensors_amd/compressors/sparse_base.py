@@ -1,0 +1,78 @@
+"""State-dict harness shared by the sparsity compressors.
+
+Mirrors BaseSparseCompressor (reference: compressors/sparse_compressors/base.py:66-202):
+only entries named `*.weight` (and, if given, listed in compression_targets)
+are compressed; the key prefix of the emitted entries is the name without
+`.weight`.
+"""
+from typing import Dict, Generator, Optional, Set, Tuple
+
+from torch import Tensor
+
+from compressed_tensors_amd.compressors.base import BaseCompressor
+from compressed_tensors_amd.utils.helpers import (
+    load_safetensors_state_dict,
+    merge_names,
+    nest_state_dict,
+)
+
+__all__ = ["BaseSparseCompressor"]
+
+
+class BaseSparseCompressor(BaseCompressor):
+    # device the emitted tensors are moved to; None leaves them on the GPU
+    # (the reference always returns host tensors)
+    output_device = None
+
+    def compress(
+        self,
+        model_state: Dict[str, Tensor],
+        compression_targets: Optional[Set[str]] = None,
+        show_progress: bool = False,
+    ) -> Dict[str, Tensor]:
+        out: Dict[str, Tensor] = {}
+        for name, value in model_state.items():
+            if not self.should_compress(name, compression_targets):
+                out[name] = value
+                continue
+            prefix = name[: -len(".weight")] if name.endswith(".weight") else name
+            out.update(self.compress_weight(prefix, value))
+        return out
+
+    def decompress(
+        self,
+        path_to_model_or_tensors,
+        device: str = "cpu",
+        params_to_skip_load: Optional[Tuple] = None,
+        **kwargs,
+    ) -> Generator[Tuple[str, Tensor], None, None]:
+        if isinstance(path_to_model_or_tensors, dict):
+            state = path_to_model_or_tensors
+        else:
+            state = load_safetensors_state_dict(path_to_model_or_tensors, device=device)
+        nested, ignored = nest_state_dict(
+            state, self.compression_param_names, return_unmatched_params=True
+        )
+        for module_path, weight_data in nested.items():
+            yield merge_names(module_path, "weight"), self.decompress_weight(dict(weight_data))
+        for name, value in ignored.items():
+            if params_to_skip_load is not None and any(p in name for p in params_to_skip_load):
+                continue
+            yield name, value
+
+    def decompress_from_state_dict(
+        self, state_dict: Dict[str, Tensor]
+    ) -> Generator[Tuple[str, Tensor], None, None]:
+        nested, ignored = nest_state_dict(
+            state_dict, self.compression_param_names, return_unmatched_params=True
+        )
+        for module_path, weight_data in nested.items():
+            yield merge_names(module_path, "weight"), self.decompress_weight(dict(weight_data))
+        for name, value in ignored.items():
+            yield name, value
+
+    @staticmethod
+    def should_compress(name: str, expanded_targets: Optional[Set[str]] = None) -> bool:
+        if expanded_targets is None:
+            return name.endswith(".weight")
+        return name.endswith(".weight") and name[: -len(".weight")] in expanded_targets

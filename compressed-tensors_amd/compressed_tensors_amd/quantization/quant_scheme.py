@@ -1,0 +1,169 @@
+"""QuantizationScheme and the preset table (W4A16, FP8_DYNAMIC, NVFP4, ...).
+
+Field names and preset contents follow the reference's
+quantization/quant_scheme.py:36-339 so that scheme names used in recipes map
+to the same arguments.
+"""
+from copy import deepcopy
+from typing import Any, Dict, List, Optional
+
+from compressed_tensors_amd.quantization.quant_args import (
+    DynamicType,
+    QuantizationArgs,
+    QuantizationStrategy,
+    QuantizationType,
+)
+
+__all__ = [
+    "QuantizationScheme",
+    "QuantizationConfig",
+    "preset_name_to_scheme",
+    "is_preset_scheme",
+    "PRESET_SCHEMES",
+]
+
+
+class QuantizationScheme:
+    def __init__(
+        self,
+        targets: List[str],
+        weights: Optional[QuantizationArgs] = None,
+        input_activations: Optional[QuantizationArgs] = None,
+        output_activations: Optional[QuantizationArgs] = None,
+        format: Optional[str] = None,
+    ):
+        self.targets = list(targets)
+        self.weights = QuantizationArgs.model_validate(weights) if weights is not None else None
+        self.input_activations = (
+            QuantizationArgs.model_validate(input_activations)
+            if input_activations is not None
+            else None
+        )
+        self.output_activations = (
+            QuantizationArgs.model_validate(output_activations)
+            if output_activations is not None
+            else None
+        )
+        self.format = format
+        for args in (self.input_activations, self.output_activations):
+            if args is not None and args.actorder is not None:
+                raise ValueError("Cannot apply actorder to activations")
+
+    def model_dump(self) -> Dict[str, Any]:
+        return {
+            "targets": self.targets,
+            "weights": self.weights.model_dump() if self.weights else None,
+            "input_activations": self.input_activations.model_dump()
+            if self.input_activations
+            else None,
+            "output_activations": self.output_activations.model_dump()
+            if self.output_activations
+            else None,
+            "format": self.format,
+        }
+
+
+class QuantizationConfig:
+    """config_groups / format / quantization_status / ignore
+    (reference: quantization/quant_config.py:105-283, fields only)."""
+
+    def __init__(
+        self,
+        config_groups: Dict[str, QuantizationScheme],
+        format: str = "fakequant",
+        quantization_status: str = "initialized",
+        global_compression_ratio: Optional[float] = None,
+        ignore: Optional[List[str]] = None,
+        kv_cache_scheme: Optional[QuantizationArgs] = None,
+        quant_method: str = "compressed-tensors",
+    ):
+        groups = {}
+        for name, scheme in config_groups.items():
+            if isinstance(scheme, dict):
+                scheme = QuantizationScheme(**scheme)
+            groups[name] = scheme
+        self.config_groups = groups
+        self.format = format
+        self.quantization_status = quantization_status
+        self.global_compression_ratio = global_compression_ratio
+        self.ignore = ignore or []
+        self.kv_cache_scheme = kv_cache_scheme
+        self.quant_method = quant_method
+
+
+def _w(**kw) -> Dict[str, QuantizationArgs]:
+    return {"weights": QuantizationArgs(**kw)}
+
+
+_INT8_W_CHANNEL = dict(num_bits=8, type=QuantizationType.INT, strategy=QuantizationStrategy.CHANNEL,
+                       symmetric=True, dynamic=False)
+_FP8_W_TENSOR = dict(num_bits=8, type=QuantizationType.FLOAT, strategy=QuantizationStrategy.TENSOR,
+                     symmetric=True, dynamic=False)
+
+PRESET_SCHEMES: Dict[str, Dict[str, QuantizationArgs]] = {
+    "UNQUANTIZED": {},
+    "W8A16": _w(**_INT8_W_CHANNEL),
+    "W4A16": _w(num_bits=4, type=QuantizationType.INT, strategy=QuantizationStrategy.GROUP,
+                group_size=128, symmetric=True, dynamic=False),
+    "W4A16_ASYM": _w(num_bits=4, type=QuantizationType.INT, strategy=QuantizationStrategy.GROUP,
+                     group_size=128, symmetric=False, dynamic=False),
+    "W8A8": {
+        "weights": QuantizationArgs(**_INT8_W_CHANNEL),
+        "input_activations": QuantizationArgs(
+            num_bits=8, type=QuantizationType.INT, strategy=QuantizationStrategy.TOKEN,
+            symmetric=True, dynamic=True, observer=None),
+    },
+    "W4A8": {
+        "weights": QuantizationArgs(num_bits=4, type=QuantizationType.INT,
+                                    strategy=QuantizationStrategy.GROUP, group_size=128,
+                                    symmetric=True, dynamic=False),
+        "input_activations": QuantizationArgs(
+            num_bits=8, type=QuantizationType.INT, strategy=QuantizationStrategy.TOKEN,
+            symmetric=True, dynamic=True, observer=None),
+    },
+    "FP8": {
+        "weights": QuantizationArgs(**_FP8_W_TENSOR),
+        "input_activations": QuantizationArgs(**_FP8_W_TENSOR),
+    },
+    "FP8_DYNAMIC": {
+        "weights": QuantizationArgs(num_bits=8, type=QuantizationType.FLOAT,
+                                    strategy=QuantizationStrategy.CHANNEL, symmetric=True,
+                                    dynamic=False),
+        "input_activations": QuantizationArgs(
+            num_bits=8, type=QuantizationType.FLOAT, strategy=QuantizationStrategy.TOKEN,
+            symmetric=True, dynamic=True, observer=None),
+    },
+    "FP8_BLOCK": {
+        "weights": QuantizationArgs(num_bits=8, type=QuantizationType.FLOAT,
+                                    strategy=QuantizationStrategy.BLOCK, symmetric=True,
+                                    dynamic=False, block_structure=[128, 128]),
+        "input_activations": QuantizationArgs(
+            num_bits=8, type=QuantizationType.FLOAT, strategy=QuantizationStrategy.GROUP,
+            symmetric=True, dynamic=True, observer=None, group_size=128),
+    },
+    "NVFP4A16": _w(num_bits=4, type=QuantizationType.FLOAT,
+                   strategy=QuantizationStrategy.TENSOR_GROUP, symmetric=True, dynamic=False,
+                   group_size=16),
+    "NVFP4": {
+        "weights": QuantizationArgs(num_bits=4, type=QuantizationType.FLOAT,
+                                    strategy=QuantizationStrategy.TENSOR_GROUP, symmetric=True,
+                                    dynamic=False, group_size=16),
+        "input_activations": QuantizationArgs(
+            num_bits=4, type=QuantizationType.FLOAT, strategy=QuantizationStrategy.TENSOR_GROUP,
+            symmetric=True, dynamic=DynamicType.LOCAL, group_size=16),
+    },
+}
+PRESET_SCHEMES["INT8"] = PRESET_SCHEMES["W8A8"]
+
+
+def preset_name_to_scheme(name: str, targets: List[str]) -> QuantizationScheme:
+    name = name.upper()
+    if name not in PRESET_SCHEMES:
+        raise KeyError(
+            f"Unknown preset scheme name {name}, available names: {list(PRESET_SCHEMES.keys())}"
+        )
+    return QuantizationScheme(targets=targets, **deepcopy(PRESET_SCHEMES[name]))
+
+
+def is_preset_scheme(name: str) -> bool:
+    return name.upper() in PRESET_SCHEMES

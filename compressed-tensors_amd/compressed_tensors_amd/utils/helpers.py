@@ -1,0 +1,142 @@
+"""Bitmask packing and small tensor utilities.
+
+pack_bitmasks / unpack_bitmasks reproduce numpy.packbits / unpackbits with
+bitorder="little" (reference: utils/helpers.py:302-339) on the GPU; shard /
+combine helpers mirror utils/helpers.py:237-299; merge_names mirrors
+utils/safetensors_load.py:115-125.
+"""
+from typing import List
+
+import torch
+
+from compressed_tensors_amd import _lib
+
+__all__ = [
+    "pack_bitmasks",
+    "unpack_bitmasks",
+    "shard_tensor",
+    "combine_shards",
+    "merge_names",
+    "tensor_follows_mask_structure",
+    "split_param_name",
+    "nest_state_dict",
+    "load_safetensors_state_dict",
+]
+
+
+def pack_bitmasks(bytemasks: torch.Tensor) -> torch.Tensor:
+    """[..., C] bool -> [..., ceil(C/8)] uint8, bit j of byte k = column 8k+j."""
+    _lib.require_gpu(bytemasks)
+    m = bytemasks.contiguous()
+    if m.dtype not in (torch.bool, torch.uint8, torch.int8):
+        m = m != 0
+    cols = m.shape[-1]
+    rows = m.numel() // cols if cols else 0
+    out = torch.empty(tuple(m.shape[:-1]) + ((cols + 7) // 8,), dtype=torch.uint8, device=m.device)
+    _lib.check(
+        _lib.load().ctmi_pack_bitmasks(m.data_ptr(), out.data_ptr(), rows, cols,
+                                       _lib.stream_of(m.device))
+    )
+    return out
+
+
+def unpack_bitmasks(packed_bitmasks: torch.Tensor, original_shape: List[int]) -> torch.Tensor:
+    """inverse of pack_bitmasks; returns a bool tensor of `original_shape`"""
+    _lib.require_gpu(packed_bitmasks)
+    p = packed_bitmasks.contiguous()
+    shape = [int(d) for d in original_shape]
+    cols = shape[-1]
+    rows = 1
+    for d in shape[:-1]:
+        rows *= d
+    if p.numel() != rows * ((cols + 7) // 8):
+        raise ValueError(
+            f"cannot reshape {p.numel()} bitmask bytes into shape {shape}"
+        )
+    out = torch.empty(shape, dtype=torch.bool, device=p.device)
+    _lib.check(
+        _lib.load().ctmi_unpack_bitmasks(p.data_ptr(), out.data_ptr(), rows, cols,
+                                         _lib.stream_of(p.device))
+    )
+    return out
+
+
+def shard_tensor(tensor: torch.Tensor, shard_sizes: List[int], dim: int = 0) -> List[torch.Tensor]:
+    if sum(shard_sizes) != tensor.size(dim):
+        raise ValueError(
+            "Sum of shard_sizes must equal the size of the tensor along the specified dimension."
+        )
+    out, start = [], 0
+    for size in shard_sizes:
+        out.append(tensor.narrow(dim, start, size))
+        start += size
+    return out
+
+
+def combine_shards(shards, dim=0):
+    if not shards:
+        raise ValueError("The list of shards is empty.")
+    if len({s.dtype for s in shards}) > 1:
+        raise ValueError("All shards must have the same dtype.")
+    return torch.cat(list(shards), dim=dim)
+
+
+def merge_names(parent_name: str, child_name: str) -> str:
+    if not parent_name:
+        return child_name
+    if not child_name:
+        return parent_name
+    return parent_name + "." + child_name
+
+
+def tensor_follows_mask_structure(tensor: torch.Tensor, mask: str = "2:4") -> bool:
+    n, m = (int(p) for p in mask.split(":"))
+    zero_counts = (tensor.reshape(-1, m) == 0).sum(dim=1)
+    if not bool(torch.all(zero_counts >= n)):
+        raise ValueError()
+    return True
+
+
+def split_param_name(full_name: str, param_name: str):
+    """'a.b.<param_name>' -> 'a.b'; None when full_name does not end in '.<param_name>'"""
+    suffix = "." + param_name
+    if full_name.endswith(suffix) and len(full_name) > len(suffix):
+        return full_name[: -len(suffix)]
+    return None
+
+
+def nest_state_dict(state_dict, params_to_nest, return_unmatched_params: bool = False):
+    """Group compression parameters by owning module:
+    {module_path: {param_name: tensor}} (+ the entries that matched nothing).
+    Reference: utils/safetensors_load.py:251-291."""
+    nested, unmatched = {}, {}
+    for key, value in state_dict.items():
+        hit = False
+        for param_name in params_to_nest:
+            module_path = split_param_name(key, param_name)
+            if module_path:
+                nested.setdefault(module_path, {})[param_name] = value
+                hit = True
+        if not hit:
+            unmatched[key] = value
+    return (nested, unmatched) if return_unmatched_params else nested
+
+
+def load_safetensors_state_dict(path, device="cpu"):
+    """All tensors of a .safetensors file, or of every such file in a directory."""
+    import os
+
+    from safetensors import safe_open
+
+    path = str(path)
+    files = (
+        sorted(os.path.join(path, f) for f in os.listdir(path) if f.endswith(".safetensors"))
+        if os.path.isdir(path)
+        else [path]
+    )
+    out = {}
+    for f in files:
+        with safe_open(f, framework="pt", device=str(device)) as fh:
+            for k in fh.keys():
+                out[k] = fh.get_tensor(k)
+    return out

@@ -1,0 +1,402 @@
+// FP4 e2m1 nibble packing (nvfp4-pack-quantized format).
+//
+//   pack_fp4_to_uint8      compressors/quantized_compressors/fp4_quantized.py:135-178
+//   unpack_fp4_from_uint8  fp4_quantized.py:187-221
+//   NVFP4PackedCompressor.compress_weight / decompress_weight  fp4_quantized.py:84-123
+//
+// Code = 3-bit index into {0,.5,1,1.5,2,3,4,6} | sign bit << 3; element 2j is
+// the low nibble of byte j, element 2j+1 the high nibble.
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "quant_core.h"
+#include "vec_geom.h"
+
+namespace ctmi {
+
+// Index chosen by the reference for one element: argmin_k |(|x| - lut[k])|
+// with the subtraction rounded to x's dtype (the reference subtracts tensors
+// of that dtype) and the first minimum winning; NaN distances win outright,
+// as in torch.argmin.  Values that sit on the e2m1 grid — the only ones a
+// quantized tensor holds — take the short path.
+template <int XDT>
+__device__ __forceinline__ int fp4_nearest_code(float x) {
+  const float a = fabsf(x);
+  int c = fp4_bucket(a);
+  if (fp4_code_to_f32(c) != a) {
+    c = 0;
+    float best = fabsf(round_ct<XDT>(a - 0.0f));
+    if (best == best) {
+#pragma unroll
+      for (int k = 1; k < 8; ++k) {
+        const float d = fabsf(round_ct<XDT>(a - fp4_code_to_f32(k)));
+        if (d != d) { c = k; break; }
+        if (d < best) { best = d; c = k; }
+      }
+    }
+  }
+  return c | ((int)(f2u(x) >> 31) << 3);
+}
+
+__device__ __forceinline__ int fp4_nearest_code_rt(float x, int xdt) {
+  if (xdt == CTMI_BF16) return fp4_nearest_code<CTMI_BF16>(x);
+  if (xdt == CTMI_F16) return fp4_nearest_code<CTMI_F16>(x);
+  return fp4_nearest_code<CTMI_F32>(x);
+}
+
+__device__ __forceinline__ float fp4_decode(int code) {
+  const float m = fp4_code_to_f32(code & 7);
+  return (code & 8) ? -m : m;
+}
+
+// ------------------------------------------------------------------ standalone pack / unpack
+// one thread per 8 elements (cols % 8 == 0) -> one 32-bit store
+template <typename XT>
+__global__ void __launch_bounds__(256)
+fp4_pack_vec_kernel(const typename XT::raw* __restrict__ x, uint32_t* __restrict__ out,
+                    int64_t nvec) {
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
+       v += (int64_t)gridDim.x * blockDim.x) {
+    Vec<typename XT::raw, 8> a = ldg<typename XT::raw, 8>(x + v * 8);
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      acc |= (uint32_t)fp4_nearest_code<XT::id>(XT::to_f32(a.v[i])) << (4 * i);
+    out[v] = acc;
+  }
+}
+
+// one thread per output byte
+__global__ void __launch_bounds__(256)
+fp4_pack_kernel(const void* __restrict__ x, int x_dtype, uint8_t* __restrict__ out, int64_t nbytes) {
+  for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < nbytes;
+       b += (int64_t)gridDim.x * blockDim.x) {
+    const int lo = fp4_nearest_code_rt(load_f32(x, x_dtype, 2 * b), x_dtype);
+    const int hi = fp4_nearest_code_rt(load_f32(x, x_dtype, 2 * b + 1), x_dtype);
+    out[b] = (uint8_t)(lo | (hi << 4));
+  }
+}
+
+template <typename OT>
+__global__ void __launch_bounds__(256)
+fp4_unpack_vec_kernel(const uint32_t* __restrict__ in, typename OT::raw* __restrict__ out,
+                      int64_t nvec) {
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
+       v += (int64_t)gridDim.x * blockDim.x) {
+    const uint32_t w = in[v];
+    Vec<typename OT::raw, 8> o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o.v[i] = OT::from_f32(fp4_decode((int)((w >> (4 * i)) & 15u)));
+    stg<typename OT::raw, 8>(out + v * 8, o);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+fp4_unpack_kernel(const uint8_t* __restrict__ in, void* __restrict__ out, int out_dtype,
+                  int64_t nbytes) {
+  for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < nbytes;
+       b += (int64_t)gridDim.x * blockDim.x) {
+    const int w = in[b];
+    store_from_f32(out, out_dtype, 2 * b, fp4_decode(w & 15));
+    store_from_f32(out, out_dtype, 2 * b + 1, fp4_decode(w >> 4));
+  }
+}
+
+// ------------------------------------------------------------------ fused nvfp4, generic
+struct Fp4Args {
+  const void* x;
+  void* out;
+  const void* scale;
+  const void* zp;
+  const float* gscale;
+  const int32_t* col_group;
+  int64_t rows, cols;
+  int64_t s_rows, s_cols, blk_rows, blk_cols;
+  int x_dtype, out_dtype, scale_dtype, zp_dtype;
+  QuantCfg q;
+};
+
+__device__ __forceinline__ float fp4_eff_scale(const Fp4Args& a, int64_t r, int64_t c,
+                                               int64_t* si_out) {
+  const int64_t srow = (r / a.blk_rows) % a.s_rows;
+  const int64_t scol = a.col_group ? (int64_t)a.col_group[c] : c / a.blk_cols;
+  const int64_t si = srow * a.s_cols + scol;
+  *si_out = si;
+  float s = load_f32(a.scale, a.scale_dtype, si);
+  if (a.gscale) s = s / a.gscale[0];
+  return s;
+}
+
+// The reference quantizes to e2m1 values held in x.dtype (forward.py:327 casts
+// the group result back), then indexes them; a value on the grid survives that
+// cast unchanged, so the code can be taken straight from the quantized value.
+__device__ __forceinline__ int fp4_code_of_quantized(float v) {
+  return fp4_bucket(fabsf(v)) | ((int)(f2u(v) >> 31) << 3);
+}
+
+__global__ void __launch_bounds__(256) nvfp4_compress_generic_kernel(Fp4Args a) {
+  const int64_t hc = a.cols / 2;
+  const int64_t total = a.rows * hc;
+  for (int64_t b = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; b < total;
+       b += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = b / hc, j = b - r * hc;
+    int code[2];
+    for (int h = 0; h < 2; ++h) {
+      const int64_t c = 2 * j + h;
+      int64_t si;
+      const float s = fp4_eff_scale(a, r, c, &si);
+      const float z = a.zp ? round_to(load_f32(a.zp, a.zp_dtype, si), a.x_dtype) : 0.0f;
+      const float v =
+          quantize_value(load_f32(a.x, a.x_dtype, r * a.cols + c), s, z, a.zp != nullptr, a.q);
+      code[h] = fp4_code_of_quantized(v);
+    }
+    ((uint8_t*)a.out)[b] = (uint8_t)(code[0] | (code[1] << 4));
+  }
+}
+
+__global__ void __launch_bounds__(256) nvfp4_decompress_generic_kernel(Fp4Args a) {
+  const int64_t hc = a.cols / 2;
+  const int64_t total = a.rows * a.cols;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = e / a.cols, c = e - r * a.cols;
+    const int w = ((const uint8_t*)a.x)[r * hc + c / 2];
+    const float qv = fp4_decode((c & 1) ? (w >> 4) : (w & 15));
+    int64_t si;
+    const float s = fp4_eff_scale(a, r, c, &si);
+    store_from_f32(a.out, a.out_dtype, e, dequantize_value(qv, s, 0.0f, false, a.q.dt));
+  }
+}
+
+// ------------------------------------------------------------------ fused nvfp4, vectorised
+// fp8 e4m3 local scales + fp32 global scale; arithmetic in fp32 (bf16/fp16/fp32
+// input divided by an fp32 scale promotes to fp32).
+template <typename XT, bool HAS_ZP>
+__global__ void __launch_bounds__(256)
+nvfp4_compress_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __restrict__ scale,
+                          const uint8_t* __restrict__ zp, const float* __restrict__ gscale,
+                          uint32_t* __restrict__ out, VecGeom g) {
+  const float gs = gscale[0];
+  const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
+  for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
+    const uint32_t v0 = chunk * (256 * kU) + threadIdx.x;
+    Vec<typename XT::raw, 8> xv[kU];
+    float sv[kU], zv[kU];
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        xv[k] = ldg<typename XT::raw, 8>(x + (size_t)v * 8);
+        const uint32_t si = scale_index(v, g);
+        sv[k] = f8e4m3_to_f32(scale[si]) / gs;
+        // zero_point.to(x.dtype): an fp8 value is exact in every wider float type
+        zv[k] = HAS_ZP ? f8e4m3_to_f32(zp[si]) : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        uint32_t acc = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          float t = XT::to_f32(xv[k].v[i]) / sv[k];
+          if (HAS_ZP) t = t + zv[k];
+          t = clamp_nan(t, -6.0f, 6.0f);
+          // sign of cast_to_fp4's product: exact zeros lose their sign
+          const uint32_t neg = (t < 0.0f) ? 8u : 0u;
+          acc |= ((uint32_t)fp4_bucket(fabsf(t)) | neg) << (4 * i);
+        }
+        out[v] = acc;
+      }
+    }
+  }
+}
+
+template <typename OT>
+__global__ void __launch_bounds__(256)
+nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* __restrict__ scale,
+                            const float* __restrict__ gscale, typename OT::raw* __restrict__ out,
+                            VecGeom g) {
+  const float gs = gscale[0];
+  const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
+  for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
+    const uint32_t v0 = chunk * (256 * kU) + threadIdx.x;
+    uint32_t pv[kU];
+    float sv[kU];
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        pv[k] = packed[v];
+        sv[k] = f8e4m3_to_f32(scale[scale_index(v, g)]) / gs;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        Vec<typename OT::raw, 8> o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          o.v[i] = OT::from_f32(fp4_decode((int)((pv[k] >> (4 * i)) & 15u)) * sv[k]);
+        stg<typename OT::raw, 8>(out + (size_t)v * 8, o);
+      }
+    }
+  }
+}
+
+static int fill_fp4(Fp4Args* a, const ctmi_qparams* qp, int64_t rows, int64_t cols) {
+  a->scale = qp->scale;
+  a->zp = qp->zero_point;
+  a->gscale = qp->global_scale;
+  a->col_group = qp->col_group;
+  a->rows = rows;
+  a->cols = cols;
+  a->s_rows = qp->s_rows;
+  a->s_cols = qp->s_cols;
+  a->blk_rows = qp->blk_rows;
+  a->blk_cols = qp->blk_cols;
+  a->scale_dtype = qp->scale_dtype;
+  a->zp_dtype = qp->zp_dtype;
+  a->q.qtype = CTMI_QTYPE_FLOAT;
+  a->q.num_bits = 4;
+  a->q.qmin = -6.0f;
+  a->q.qmax = 6.0f;
+  a->q.dt = qp->global_scale ? CTMI_F32 : qp->scale_dtype;
+  return CTMI_OK;
+}
+
+}  // namespace ctmi
+
+using namespace ctmi;
+
+static int check_float3(int dtype, const char* what) {
+  CTMI_REQUIRE(dtype == CTMI_F32 || dtype == CTMI_F16 || dtype == CTMI_BF16, CTMI_ERR_UNSUPPORTED,
+               "%s must be float16/bfloat16/float32", what);
+  return CTMI_OK;
+}
+
+extern "C" int ctmi_pack_fp4_to_uint8(const void* x, int32_t x_dtype, uint8_t* out, int64_t rows,
+                                      int64_t cols, void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  CTMI_REQUIRE(cols % 2 == 0, CTMI_ERR_VALUE,
+               "tensor must have an even number of columns for nvfp4 compression");
+  int rc = check_float3(x_dtype, "fp4 input");
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(x && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n = rows * cols;
+  if (n % 8 == 0 && (uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)out % 4 == 0) {
+    const int64_t nvec = n / 8;
+    const int grid = grid_for(nvec, 256);
+    if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(fp4_pack_vec_kernel<BF16>, grid, 256, 0, st, (const uint16_t*)x, (uint32_t*)out, nvec);
+    else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(fp4_pack_vec_kernel<F16>, grid, 256, 0, st, (const uint16_t*)x, (uint32_t*)out, nvec);
+    else hipLaunchKernelGGL(fp4_pack_vec_kernel<F32>, grid, 256, 0, st, (const float*)x, (uint32_t*)out, nvec);
+  } else {
+    hipLaunchKernelGGL(fp4_pack_kernel, grid_for(n / 2, 256), 256, 0, st, x, x_dtype, out, n / 2);
+  }
+  return check_launch("ctmi_pack_fp4_to_uint8");
+}
+
+extern "C" int ctmi_unpack_fp4_from_uint8(const uint8_t* in, void* out, int32_t out_dtype,
+                                          int64_t rows, int64_t cols, void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  CTMI_REQUIRE(cols % 2 == 0, CTMI_ERR_VALUE, "unpacked fp4 column count must be even");
+  int rc = check_float3(out_dtype, "fp4 output");
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(in && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n = rows * cols;
+  if (n % 8 == 0 && (uintptr_t)out % (8 * dtype_size(out_dtype)) == 0 && (uintptr_t)in % 4 == 0) {
+    const int64_t nvec = n / 8;
+    const int grid = grid_for(nvec, 256);
+    if (out_dtype == CTMI_BF16) hipLaunchKernelGGL(fp4_unpack_vec_kernel<BF16>, grid, 256, 0, st, (const uint32_t*)in, (uint16_t*)out, nvec);
+    else if (out_dtype == CTMI_F16) hipLaunchKernelGGL(fp4_unpack_vec_kernel<F16>, grid, 256, 0, st, (const uint32_t*)in, (uint16_t*)out, nvec);
+    else hipLaunchKernelGGL(fp4_unpack_vec_kernel<F32>, grid, 256, 0, st, (const uint32_t*)in, (float*)out, nvec);
+  } else {
+    hipLaunchKernelGGL(fp4_unpack_kernel, grid_for(n / 2, 256), 256, 0, st, in, out, out_dtype, n / 2);
+  }
+  return check_launch("ctmi_unpack_fp4_from_uint8");
+}
+
+extern "C" int ctmi_nvfp4_compress(const void* x, int32_t x_dtype, uint8_t* out, int64_t rows,
+                                   int64_t cols, const ctmi_qparams* qp, void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  int rc = check_float3(x_dtype, "quantize input");
+  if (rc) return rc;
+  rc = check_qparams(qp, rows, cols);
+  if (rc) return rc;
+  CTMI_REQUIRE(qp->qtype == CTMI_QTYPE_FLOAT && qp->num_bits == 4, CTMI_ERR_VALUE,
+               "nvfp4 compression needs float 4-bit quantization args");
+  CTMI_REQUIRE(cols % 2 == 0, CTMI_ERR_VALUE,
+               "tensor must have an even number of columns for nvfp4 compression");
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(x && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+
+  VecGeom g;
+  const bool zp_ok = qp->zero_point == nullptr || qp->zp_dtype == CTMI_F8E4M3;
+  if (qp->scale_dtype == CTMI_F8E4M3 && qp->global_scale && zp_ok &&
+      (uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)out % 4 == 0 &&
+      vec_geometry(qp, rows, cols, &g, true)) {
+    const int grid = grid_for(g.nvec, 256 * kU);
+    const auto* sc = (const uint8_t*)qp->scale;
+    const auto* zp = (const uint8_t*)qp->zero_point;
+#define CTMI_LAUNCH(XT, RAW)                                                                      \
+  if (zp) hipLaunchKernelGGL((nvfp4_compress_vec_kernel<XT, true>), grid, 256, 0, st, (const RAW*)x, sc, zp, qp->global_scale, (uint32_t*)out, g); \
+  else hipLaunchKernelGGL((nvfp4_compress_vec_kernel<XT, false>), grid, 256, 0, st, (const RAW*)x, sc, zp, qp->global_scale, (uint32_t*)out, g);
+    if (x_dtype == CTMI_BF16) { CTMI_LAUNCH(BF16, uint16_t) }
+    else if (x_dtype == CTMI_F16) { CTMI_LAUNCH(F16, uint16_t) }
+    else { CTMI_LAUNCH(F32, float) }
+#undef CTMI_LAUNCH
+    return check_launch("ctmi_nvfp4_compress");
+  }
+
+  Fp4Args a;
+  fill_fp4(&a, qp, rows, cols);
+  a.x = x;
+  a.out = out;
+  a.x_dtype = x_dtype;
+  a.out_dtype = CTMI_U8;
+  a.q.ct = promote_float(x_dtype, a.q.dt);
+  hipLaunchKernelGGL(nvfp4_compress_generic_kernel, grid_for(rows * cols / 2, 256), 256, 0, st, a);
+  return check_launch("ctmi_nvfp4_compress");
+}
+
+extern "C" int ctmi_nvfp4_decompress(const uint8_t* packed, void* out, int32_t out_dtype,
+                                     int64_t rows, int64_t cols, const ctmi_qparams* qp,
+                                     void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  int rc = check_float3(out_dtype, "dequantize output");
+  if (rc) return rc;
+  rc = check_qparams(qp, rows, cols);
+  if (rc) return rc;
+  CTMI_REQUIRE(cols % 2 == 0, CTMI_ERR_VALUE, "unpacked fp4 column count must be even");
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(packed && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+
+  VecGeom g;
+  if (qp->scale_dtype == CTMI_F8E4M3 && qp->global_scale && qp->zero_point == nullptr &&
+      (uintptr_t)out % (8 * dtype_size(out_dtype)) == 0 && (uintptr_t)packed % 4 == 0 &&
+      vec_geometry(qp, rows, cols, &g, true)) {
+    const int grid = grid_for(g.nvec, 256 * kU);
+    const auto* sc = (const uint8_t*)qp->scale;
+    if (out_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<BF16>, grid, 256, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (uint16_t*)out, g);
+    else if (out_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<F16>, grid, 256, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (uint16_t*)out, g);
+    else hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<F32>, grid, 256, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (float*)out, g);
+    return check_launch("ctmi_nvfp4_decompress");
+  }
+
+  Fp4Args a;
+  fill_fp4(&a, qp, rows, cols);
+  a.x = packed;
+  a.out = out;
+  a.x_dtype = CTMI_U8;
+  a.out_dtype = out_dtype;
+  a.q.ct = a.q.dt;
+  hipLaunchKernelGGL(nvfp4_decompress_generic_kernel, grid_for(rows * cols, 256), 256, 0, st, a);
+  return check_launch("ctmi_nvfp4_decompress");
+}

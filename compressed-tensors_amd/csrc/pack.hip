@@ -1,0 +1,494 @@
+// int4/int8 -> int32 packing (pack-quantized format): standalone pack / unpack
+// and the fused quantize+pack / unpack+dequantize passes.
+//
+//   pack_to_int32      compressors/quantized_compressors/pack_quantized.py:186-246
+//   unpack_from_int32  pack_quantized.py:249-309
+//   compress_weight / decompress_weight  pack_quantized.py:88-183
+//
+// Layout: element i of a run of pf = 32/num_bits neighbours sits in bits
+// [b*i, b*i+b) of the word, stored as (value + 2^(b-1)) mod 256; a ragged tail
+// is padded with zero bits.
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "quant_core.h"
+#include "vec_geom.h"
+
+namespace ctmi {
+
+// ------------------------------------------------------------------ standalone pack / unpack
+// packed_dim == 1: one thread per output word.
+__global__ void __launch_bounds__(256)
+pack_dim1_kernel(const int8_t* __restrict__ in, int32_t* __restrict__ out, int64_t rows,
+                 int64_t cols, int64_t pcols, int bits) {
+  const int pf = 32 / bits;
+  const int offset = 1 << (bits - 1);
+  const int64_t total = rows * pcols;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total;
+       w += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = w / pcols, j = w - r * pcols;
+    const int8_t* src = in + r * cols + j * pf;
+    const int n = (int)((cols - j * pf) < pf ? (cols - j * pf) : pf);
+    uint32_t acc = 0;
+    for (int i = 0; i < n; ++i) {
+      uint32_t u = (uint8_t)(src[i] + offset);
+      acc += u << (bits * i);  // the reference sums shifted terms (carries included)
+    }
+    out[w] = (int32_t)acc;
+  }
+}
+
+// 4- or 8-bit, cols % 16 == 0: 16 input bytes per thread.
+template <int BITS>
+__global__ void __launch_bounds__(256)
+pack_dim1_vec_kernel(const int8_t* __restrict__ in, int32_t* __restrict__ out, int64_t nvec) {
+  constexpr int W = BITS * 16 / 32;  // words produced per 16 inputs
+  constexpr int PF = 32 / BITS;
+  constexpr int OFF = 1 << (BITS - 1);
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
+       v += (int64_t)gridDim.x * blockDim.x) {
+    Vec<int8_t, 16> a = ldg<int8_t, 16>(in + v * 16);
+    Vec<int32_t, W> o;
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      uint32_t acc = 0;
+#pragma unroll
+      for (int i = 0; i < PF; ++i) acc += (uint32_t)(uint8_t)(a.v[w * PF + i] + OFF) << (BITS * i);
+      o.v[w] = (int32_t)acc;
+    }
+    stg<int32_t, W>(out + v * W, o);
+  }
+}
+
+// packed_dim == 0: out[j, c] packs in[j*pf + i, c]; one thread per output word.
+__global__ void __launch_bounds__(256)
+pack_dim0_kernel(const int8_t* __restrict__ in, int32_t* __restrict__ out, int64_t rows,
+                 int64_t cols, int64_t prows, int bits) {
+  const int pf = 32 / bits;
+  const int offset = 1 << (bits - 1);
+  const int64_t total = prows * cols;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total;
+       w += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t j = w / cols, c = w - j * cols;
+    uint32_t acc = 0;
+    for (int i = 0; i < pf; ++i) {
+      const int64_t r = j * pf + i;
+      if (r < rows) acc += (uint32_t)(uint8_t)(in[r * cols + c] + offset) << (bits * i);
+    }
+    out[w] = (int32_t)acc;
+  }
+}
+
+// one thread per output element, either packed dim
+__global__ void __launch_bounds__(256)
+unpack_kernel(const int32_t* __restrict__ in, int8_t* __restrict__ out, int64_t rows, int64_t cols,
+              int bits, int packed_dim) {
+  const int pf = 32 / bits;
+  const uint32_t mask = (bits == 32) ? 0xffffffffu : ((1u << bits) - 1u);
+  const int offset = 1 << (bits - 1);
+  const int64_t pcols = packed_dim == 1 ? (cols + pf - 1) / pf : cols;
+  const int64_t total = rows * cols;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = e / cols, c = e - r * cols;
+    uint32_t word;
+    int i;
+    if (packed_dim == 1) {
+      word = (uint32_t)in[r * pcols + c / pf];
+      i = (int)(c % pf);
+    } else {
+      word = (uint32_t)in[(r / pf) * pcols + c];
+      i = (int)(r % pf);
+    }
+    out[e] = (int8_t)((int)((word >> (bits * i)) & mask) - offset);
+  }
+}
+
+// 4- or 8-bit, packed_dim 1, cols % 16 == 0: 16 output bytes per thread.
+template <int BITS>
+__global__ void __launch_bounds__(256)
+unpack_dim1_vec_kernel(const int32_t* __restrict__ in, int8_t* __restrict__ out, int64_t nvec) {
+  constexpr int W = BITS * 16 / 32;
+  constexpr int PF = 32 / BITS;
+  constexpr int OFF = 1 << (BITS - 1);
+  constexpr uint32_t MASK = (1u << BITS) - 1u;
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
+       v += (int64_t)gridDim.x * blockDim.x) {
+    Vec<int32_t, W> a = ldg<int32_t, W>(in + v * W);
+    Vec<int8_t, 16> o;
+#pragma unroll
+    for (int w = 0; w < W; ++w)
+#pragma unroll
+      for (int i = 0; i < PF; ++i)
+        o.v[w * PF + i] = (int8_t)((int)(((uint32_t)a.v[w] >> (BITS * i)) & MASK) - OFF);
+    stg<int8_t, 16>(out + v * 16, o);
+  }
+}
+
+// ------------------------------------------------------------------ fused, generic
+struct FusedArgs {
+  const void* x;        // compress: dense input; decompress: packed words
+  void* out;            // compress: packed words; decompress: dense output
+  const void* scale;
+  const void* zp;
+  const float* gscale;
+  const int32_t* col_group;
+  int64_t rows, cols, pcols;
+  int64_t s_rows, s_cols, blk_rows, blk_cols;
+  int x_dtype, out_dtype, scale_dtype, zp_dtype;
+  QuantCfg q;
+};
+
+__device__ __forceinline__ void load_qp(const FusedArgs& a, int64_t r, int64_t c, int zq_dtype,
+                                        float* s, float* z) {
+  const int64_t srow = (r / a.blk_rows) % a.s_rows;
+  const int64_t scol = a.col_group ? (int64_t)a.col_group[c] : c / a.blk_cols;
+  const int64_t si = srow * a.s_cols + scol;
+  float sv = load_f32(a.scale, a.scale_dtype, si);
+  if (a.gscale) sv = sv / a.gscale[0];
+  *s = sv;
+  *z = a.zp ? round_to(load_f32(a.zp, a.zp_dtype, si), zq_dtype) : 0.0f;
+}
+
+__global__ void __launch_bounds__(256) pq_compress_generic_kernel(FusedArgs a) {
+  const int bits = a.q.num_bits;
+  const int pf = 32 / bits;
+  const int offset = 1 << (bits - 1);
+  const int64_t total = a.rows * a.pcols;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total;
+       w += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = w / a.pcols, j = w - r * a.pcols;
+    uint32_t acc = 0;
+    for (int i = 0; i < pf; ++i) {
+      const int64_t c = j * pf + i;
+      if (c >= a.cols) break;
+      float s, z;
+      load_qp(a, r, c, a.x_dtype, &s, &z);
+      float v = quantize_value(load_f32(a.x, a.x_dtype, r * a.cols + c), s, z, a.zp != nullptr, a.q);
+      acc += (uint32_t)(uint8_t)((int8_t)f32_to_int(v) + offset) << (bits * i);
+    }
+    ((int32_t*)a.out)[w] = (int32_t)acc;
+  }
+}
+
+__global__ void __launch_bounds__(256) pq_decompress_generic_kernel(FusedArgs a) {
+  const int bits = a.q.num_bits;
+  const int pf = 32 / bits;
+  const uint32_t mask = (1u << bits) - 1u;
+  const int offset = 1 << (bits - 1);
+  const int64_t total = a.rows * a.cols;
+  for (int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; e < total;
+       e += (int64_t)gridDim.x * blockDim.x) {
+    const int64_t r = e / a.cols, c = e - r * a.cols;
+    const uint32_t word = (uint32_t)((const int32_t*)a.x)[r * a.pcols + c / pf];
+    const int8_t qv = (int8_t)((int)((word >> (bits * (int)(c % pf))) & mask) - offset);
+    float s, z;
+    load_qp(a, r, c, a.q.dt, &s, &z);
+    float v = dequantize_value((float)qv, s, z, a.zp != nullptr, a.q.dt);
+    store_from_f32(a.out, a.out_dtype, e, v);
+  }
+}
+
+// ------------------------------------------------------------------ fused, vectorised
+// Work item = 8 neighbouring elements of one row that share a scale (the scale
+// block is a multiple of 8 columns wide): a 16-byte load for 2-byte inputs.
+// A workgroup walks chunks of 256*U items; all loads of a chunk are issued
+// before the arithmetic so that U*16 bytes per lane are in flight.
+template <typename XT, typename ST, int BITS, bool HAS_ZP>
+__global__ void __launch_bounds__(256)
+pq_compress_vec_kernel(const typename XT::raw* __restrict__ x,
+                       const typename ST::raw* __restrict__ scale,
+                       const int8_t* __restrict__ zp, int32_t* __restrict__ out, VecGeom g,
+                       float qmin, float qmax) {
+  constexpr int CT = Promote<XT::id, ST::id>::value;
+  constexpr int W = BITS / 4;  // output words per item
+  constexpr int PF = 32 / BITS;
+  constexpr int OFF = 1 << (BITS - 1);
+  using XV = Vec<typename XT::raw, 8>;
+  const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
+  for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
+    const uint32_t v0 = chunk * (256 * kU) + threadIdx.x;
+    XV xv[kU];
+    float sv[kU], zv[kU];
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        xv[k] = ldg<typename XT::raw, 8>(x + (size_t)v * 8);
+        const uint32_t si = scale_index(v, g);
+        sv[k] = ST::to_f32(scale[si]);
+        zv[k] = HAS_ZP ? (float)zp[si] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        Vec<int32_t, W> o;
+#pragma unroll
+        for (int w = 0; w < W; ++w) {
+          uint32_t acc = 0;
+#pragma unroll
+          for (int i = 0; i < PF; ++i) {
+            float t = round_ct<CT>(XT::to_f32(xv[k].v[w * PF + i]) / sv[k]);
+            if (HAS_ZP) t = round_ct<CT>(t + zv[k]);
+            t = rintf(clamp_nan(t, qmin, qmax));
+            acc |= ((uint32_t)(f32_to_int(t) + OFF) & ((1u << BITS) - 1u)) << (BITS * i);
+          }
+          o.v[w] = (int32_t)acc;
+        }
+        stg<int32_t, W>(out + (size_t)v * W, o);
+      }
+    }
+  }
+}
+
+template <typename ST, int BITS, bool HAS_ZP>
+__global__ void __launch_bounds__(256)
+pq_decompress_vec_kernel(const int32_t* __restrict__ packed,
+                         const typename ST::raw* __restrict__ scale,
+                         const int8_t* __restrict__ zp, typename ST::raw* __restrict__ out,
+                         VecGeom g) {
+  constexpr int DT = ST::id;
+  constexpr int W = BITS / 4;
+  constexpr int PF = 32 / BITS;
+  constexpr int OFF = 1 << (BITS - 1);
+  constexpr uint32_t MASK = (1u << BITS) - 1u;
+  const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
+  for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
+    const uint32_t v0 = chunk * (256 * kU) + threadIdx.x;
+    Vec<int32_t, W> pv[kU];
+    float sv[kU], zv[kU];
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        pv[k] = ldg<int32_t, W>(packed + (size_t)v * W);
+        const uint32_t si = scale_index(v, g);
+        sv[k] = ST::to_f32(scale[si]);
+        zv[k] = HAS_ZP ? (float)zp[si] : 0.0f;
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kU; ++k) {
+      const uint32_t v = v0 + k * 256;
+      if (v < g.nvec) {
+        Vec<typename ST::raw, 8> o;
+#pragma unroll
+        for (int w = 0; w < W; ++w)
+#pragma unroll
+          for (int i = 0; i < PF; ++i) {
+            float t = (float)((int)(((uint32_t)pv[k].v[w] >> (BITS * i)) & MASK) - OFF);
+            if (HAS_ZP) t = round_ct<DT>(t - zv[k]);
+            o.v[w * PF + i] = ST::from_f32(t * sv[k]);
+          }
+        stg<typename ST::raw, 8>(out + (size_t)v * 8, o);
+      }
+    }
+  }
+}
+
+template <typename XT, typename ST>
+static void launch_compress_vec(const void* x, const ctmi_qparams* qp, int32_t* out,
+                                const VecGeom& g, float qmin, float qmax, hipStream_t st) {
+  const int grid = grid_for(g.nvec, 256 * kU);
+  const auto* xs = (const typename XT::raw*)x;
+  const auto* sc = (const typename ST::raw*)qp->scale;
+  const auto* zp = (const int8_t*)qp->zero_point;
+  const bool z = zp != nullptr;
+  if (qp->num_bits == 4) {
+    if (z) hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 4, true>), grid, 256, 0, st, xs, sc, zp, out, g, qmin, qmax);
+    else hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 4, false>), grid, 256, 0, st, xs, sc, zp, out, g, qmin, qmax);
+  } else {
+    if (z) hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 8, true>), grid, 256, 0, st, xs, sc, zp, out, g, qmin, qmax);
+    else hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 8, false>), grid, 256, 0, st, xs, sc, zp, out, g, qmin, qmax);
+  }
+}
+
+template <typename ST>
+static void launch_decompress_vec(const int32_t* packed, const ctmi_qparams* qp, void* out,
+                                  const VecGeom& g, hipStream_t st) {
+  const int grid = grid_for(g.nvec, 256 * kU);
+  const auto* sc = (const typename ST::raw*)qp->scale;
+  const auto* zp = (const int8_t*)qp->zero_point;
+  auto* o = (typename ST::raw*)out;
+  const bool z = zp != nullptr;
+  if (qp->num_bits == 4) {
+    if (z) hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 4, true>), grid, 256, 0, st, packed, sc, zp, o, g);
+    else hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 4, false>), grid, 256, 0, st, packed, sc, zp, o, g);
+  } else {
+    if (z) hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 8, true>), grid, 256, 0, st, packed, sc, zp, o, g);
+    else hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 8, false>), grid, 256, 0, st, packed, sc, zp, o, g);
+  }
+}
+
+static int fill_fused(FusedArgs* a, const ctmi_qparams* qp, int64_t rows, int64_t cols) {
+  a->scale = qp->scale;
+  a->zp = qp->zero_point;
+  a->gscale = qp->global_scale;
+  a->col_group = qp->col_group;
+  a->rows = rows;
+  a->cols = cols;
+  a->pcols = cdiv(cols, 32 / qp->num_bits);
+  a->s_rows = qp->s_rows;
+  a->s_cols = qp->s_cols;
+  a->blk_rows = qp->blk_rows;
+  a->blk_cols = qp->blk_cols;
+  a->scale_dtype = qp->scale_dtype;
+  a->zp_dtype = qp->zp_dtype;
+  a->q.qtype = qp->qtype;
+  a->q.num_bits = qp->num_bits;
+  return quant_range(qp->qtype, qp->num_bits, &a->q.qmin, &a->q.qmax);
+}
+
+}  // namespace ctmi
+
+using namespace ctmi;
+
+static int check_bits(int32_t num_bits) {
+  CTMI_REQUIRE(num_bits <= 8, CTMI_ERR_VALUE, "Packing is only supported for less than 8 bits");
+  CTMI_REQUIRE(num_bits >= 1, CTMI_ERR_VALUE, "num_bits must be at least 1, got %d", num_bits);
+  return CTMI_OK;
+}
+
+extern "C" int ctmi_pack_to_int32(const int8_t* in, int32_t* out, int64_t rows, int64_t cols,
+                                  int32_t num_bits, int32_t packed_dim, void* stream) {
+  int rc = check_bits(num_bits);
+  if (rc) return rc;
+  CTMI_REQUIRE(packed_dim == 0 || packed_dim == 1, CTMI_ERR_VALUE, "packed_dim must be 0 or 1");
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(in && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const int pf = 32 / num_bits;
+  if (packed_dim == 1) {
+    const bool vec = (num_bits == 4 || num_bits == 8) && cols % 16 == 0 &&
+                     ((uintptr_t)in % 16 == 0) && ((uintptr_t)out % 8 == 0);
+    if (vec) {
+      const int64_t nvec = rows * cols / 16;
+      const int grid = grid_for(nvec, 256);
+      if (num_bits == 4) hipLaunchKernelGGL(pack_dim1_vec_kernel<4>, grid, 256, 0, st, in, out, nvec);
+      else hipLaunchKernelGGL(pack_dim1_vec_kernel<8>, grid, 256, 0, st, in, out, nvec);
+    } else {
+      const int64_t pcols = cdiv(cols, pf);
+      hipLaunchKernelGGL(pack_dim1_kernel, grid_for(rows * pcols, 256), 256, 0, st, in, out, rows,
+                         cols, pcols, num_bits);
+    }
+  } else {
+    const int64_t prows = cdiv(rows, pf);
+    hipLaunchKernelGGL(pack_dim0_kernel, grid_for(prows * cols, 256), 256, 0, st, in, out, rows,
+                       cols, prows, num_bits);
+  }
+  return check_launch("ctmi_pack_to_int32");
+}
+
+extern "C" int ctmi_unpack_from_int32(const int32_t* in, int8_t* out, int64_t rows, int64_t cols,
+                                      int32_t num_bits, int32_t packed_dim, void* stream) {
+  CTMI_REQUIRE(num_bits <= 8, CTMI_ERR_VALUE, "Unpacking is only supported for less than 8 bits");
+  CTMI_REQUIRE(num_bits >= 1, CTMI_ERR_VALUE, "num_bits must be at least 1, got %d", num_bits);
+  CTMI_REQUIRE(packed_dim == 0 || packed_dim == 1, CTMI_ERR_VALUE, "packed_dim must be 0 or 1");
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(in && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const bool vec = packed_dim == 1 && (num_bits == 4 || num_bits == 8) && cols % 16 == 0 &&
+                   ((uintptr_t)out % 16 == 0) && ((uintptr_t)in % 8 == 0);
+  if (vec) {
+    const int64_t nvec = rows * cols / 16;
+    const int grid = grid_for(nvec, 256);
+    if (num_bits == 4) hipLaunchKernelGGL(unpack_dim1_vec_kernel<4>, grid, 256, 0, st, in, out, nvec);
+    else hipLaunchKernelGGL(unpack_dim1_vec_kernel<8>, grid, 256, 0, st, in, out, nvec);
+  } else {
+    hipLaunchKernelGGL(unpack_kernel, grid_for(rows * cols, 256), 256, 0, st, in, out, rows, cols,
+                       num_bits, packed_dim);
+  }
+  return check_launch("ctmi_unpack_from_int32");
+}
+
+extern "C" int ctmi_pack_quantized_compress(const void* x, int32_t x_dtype, int32_t* out,
+                                            int64_t rows, int64_t cols, const ctmi_qparams* qp,
+                                            void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  CTMI_REQUIRE(x_dtype == CTMI_F32 || x_dtype == CTMI_F16 || x_dtype == CTMI_BF16,
+               CTMI_ERR_UNSUPPORTED, "quantize needs a float16/bfloat16/float32 input");
+  int rc = check_qparams(qp, rows, cols);
+  if (rc) return rc;
+  CTMI_REQUIRE(qp->global_scale == nullptr, CTMI_ERR_VALUE,
+               "global_scale is not supported for the PackQuantizationCompressor");
+  CTMI_REQUIRE(qp->qtype == CTMI_QTYPE_INT, CTMI_ERR_VALUE,
+               "Tensor must be quantized to torch.int8 before packing");
+  rc = check_bits(qp->num_bits);
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(x && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+
+  VecGeom g;
+  const bool zp_ok = qp->zero_point == nullptr || qp->zp_dtype == CTMI_I8;
+  const bool aligned = ((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0) && ((uintptr_t)out % 8 == 0);
+  if ((qp->num_bits == 4 || qp->num_bits == 8) && zp_ok && aligned &&
+      qp->scale_dtype != CTMI_F8E4M3 && vec_geometry(qp, rows, cols, &g)) {
+    float qmin, qmax;
+    quant_range(qp->qtype, qp->num_bits, &qmin, &qmax);
+    const int sd = qp->scale_dtype;
+#define CTMI_DISPATCH_X(XT)                                                        \
+  if (sd == CTMI_BF16) launch_compress_vec<XT, BF16>(x, qp, out, g, qmin, qmax, st); \
+  else if (sd == CTMI_F16) launch_compress_vec<XT, F16>(x, qp, out, g, qmin, qmax, st); \
+  else launch_compress_vec<XT, F32>(x, qp, out, g, qmin, qmax, st);
+    if (x_dtype == CTMI_BF16) { CTMI_DISPATCH_X(BF16) }
+    else if (x_dtype == CTMI_F16) { CTMI_DISPATCH_X(F16) }
+    else { CTMI_DISPATCH_X(F32) }
+#undef CTMI_DISPATCH_X
+    return check_launch("ctmi_pack_quantized_compress");
+  }
+
+  FusedArgs a;
+  rc = fill_fused(&a, qp, rows, cols);
+  if (rc) return rc;
+  a.x = x;
+  a.out = out;
+  a.x_dtype = x_dtype;
+  a.out_dtype = CTMI_I32;
+  a.q.dt = qp->scale_dtype;
+  a.q.ct = promote_float(x_dtype, qp->scale_dtype);
+  hipLaunchKernelGGL(pq_compress_generic_kernel, grid_for(rows * a.pcols, 256), 256, 0, st, a);
+  return check_launch("ctmi_pack_quantized_compress");
+}
+
+extern "C" int ctmi_pack_quantized_decompress(const int32_t* packed, void* out, int32_t out_dtype,
+                                              int64_t rows, int64_t cols, const ctmi_qparams* qp,
+                                              void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  CTMI_REQUIRE(out_dtype == CTMI_F32 || out_dtype == CTMI_F16 || out_dtype == CTMI_BF16,
+               CTMI_ERR_UNSUPPORTED, "dequantize output must be float16/bfloat16/float32");
+  int rc = check_qparams(qp, rows, cols);
+  if (rc) return rc;
+  CTMI_REQUIRE(qp->num_bits <= 8, CTMI_ERR_VALUE,
+               "Unpacking is only supported for less than 8 bits");
+  CTMI_REQUIRE(qp->qtype == CTMI_QTYPE_INT, CTMI_ERR_VALUE, "pack-quantized holds integer codes");
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(packed && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+
+  VecGeom g;
+  const bool zp_ok = qp->zero_point == nullptr || qp->zp_dtype == CTMI_I8;
+  const bool aligned = ((uintptr_t)out % (8 * dtype_size(out_dtype)) == 0) && ((uintptr_t)packed % 8 == 0);
+  if ((qp->num_bits == 4 || qp->num_bits == 8) && zp_ok && aligned &&
+      out_dtype == qp->scale_dtype && vec_geometry(qp, rows, cols, &g)) {
+    if (out_dtype == CTMI_BF16) launch_decompress_vec<BF16>(packed, qp, out, g, st);
+    else if (out_dtype == CTMI_F16) launch_decompress_vec<F16>(packed, qp, out, g, st);
+    else launch_decompress_vec<F32>(packed, qp, out, g, st);
+    return check_launch("ctmi_pack_quantized_decompress");
+  }
+
+  FusedArgs a;
+  rc = fill_fused(&a, qp, rows, cols);
+  if (rc) return rc;
+  a.x = packed;
+  a.out = out;
+  a.x_dtype = CTMI_I32;
+  a.out_dtype = out_dtype;
+  a.q.dt = qp->global_scale ? CTMI_F32 : qp->scale_dtype;
+  a.q.ct = a.q.dt;
+  hipLaunchKernelGGL(pq_decompress_generic_kernel, grid_for(rows * cols, 256), 256, 0, st, a);
+  return check_launch("ctmi_pack_quantized_decompress");
+}

@@ -1,0 +1,120 @@
+// quantize / dequantize / fake-quantize kernels.
+//
+// Numerics contract: the reference evaluates an op chain in torch, one op at a
+// time, each op computed in fp32 and rounded to the tensor dtype torch's type
+// promotion picked.  The kernels here replay the same chain per element in
+// registers: every intermediate is rounded to that dtype (`round_to`) before
+// the next op, so results are bit-identical while the tensor is read once and
+// written once.
+//
+//   _quantize   (quantization/lifecycle/forward.py:455-487)
+//   _dequantize (forward.py:491-514)
+//   round_to_quantized_type / cast_to_fp4 (quantization/quant_args.py:55-68, 384-408)
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "quant_core.h"
+
+namespace ctmi {
+
+// ------------------------------------------------------------------ generic kernel
+// One element per thread, any dtype / strategy combination.  Used whenever no
+// vectorised specialisation applies.
+struct QdqArgs {
+  const void* x;
+  void* out;
+  const void* scale;
+  const void* zp;
+  const float* gscale;
+  const int32_t* col_group;
+  int64_t rows, cols;
+  int64_t s_rows, s_cols, blk_rows, blk_cols;
+  int x_dtype, out_dtype, scale_dtype, zp_dtype;
+  QuantCfg q;
+  int do_q, do_dq;
+};
+
+__global__ void __launch_bounds__(256) qdq_generic_kernel(QdqArgs a) {
+  const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (c >= a.cols) return;
+  const int64_t scol = a.col_group ? (int64_t)a.col_group[c] : c / a.blk_cols;
+  const float gs = a.gscale ? a.gscale[0] : 1.0f;
+  for (int64_t r = blockIdx.y; r < a.rows; r += gridDim.y) {
+    const int64_t srow = (r / a.blk_rows) % a.s_rows;
+    const int64_t si = srow * a.s_cols + scol;
+    float s = load_f32(a.scale, a.scale_dtype, si);
+    if (a.gscale) s = s / gs;  // scale.to(float32) / global_scale
+    float zq = 0.0f, zd = 0.0f;
+    if (a.zp) {
+      float z = load_f32(a.zp, a.zp_dtype, si);
+      zq = round_to(z, a.x_dtype);   // zero_point.to(x.dtype)
+      zd = round_to(z, a.q.dt);      // zero_point.to(scale.dtype)
+    }
+    const int64_t i = r * a.cols + c;
+    float v = load_f32(a.x, a.x_dtype, i);
+    if (a.do_q) v = quantize_value(v, s, zq, a.zp != nullptr, a.q);
+    if (a.do_dq) v = dequantize_value(v, s, zd, a.zp != nullptr, a.q.dt);
+    store_from_f32(a.out, a.out_dtype, i, v);
+  }
+}
+
+// ------------------------------------------------------------------ host side
+static int fill_cfg(const ctmi_qparams* qp, int x_dtype, QuantCfg* q) {
+  int rc = quant_range(qp->qtype, qp->num_bits, &q->qmin, &q->qmax);
+  if (rc) return rc;
+  q->qtype = qp->qtype;
+  q->num_bits = qp->num_bits;
+  const int sdt = qp->global_scale ? CTMI_F32 : qp->scale_dtype;
+  q->dt = sdt;
+  q->ct = is_float_dtype(x_dtype) && x_dtype != CTMI_F8E4M3 ? promote_float(x_dtype, sdt) : sdt;
+  return CTMI_OK;
+}
+
+}  // namespace ctmi
+
+using namespace ctmi;
+
+extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_dtype, int64_t rows,
+                        int64_t cols, const ctmi_qparams* qp, int32_t do_quantize,
+                        int32_t do_dequantize, void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  CTMI_REQUIRE(do_quantize || do_dequantize, CTMI_ERR_VALUE, "nothing to do");
+  CTMI_REQUIRE(dtype_size(x_dtype) > 0 && x_dtype != CTMI_I64, CTMI_ERR_UNSUPPORTED,
+               "unsupported input dtype %d", x_dtype);
+  CTMI_REQUIRE(dtype_size(out_dtype) > 0 && out_dtype != CTMI_I64 && out_dtype != CTMI_BOOL,
+               CTMI_ERR_UNSUPPORTED, "unsupported output dtype %d", out_dtype);
+  if (do_quantize) {
+    CTMI_REQUIRE(x_dtype == CTMI_F32 || x_dtype == CTMI_F16 || x_dtype == CTMI_BF16,
+                 CTMI_ERR_UNSUPPORTED, "quantize needs a float16/bfloat16/float32 input");
+  }
+  int rc = check_qparams(qp, rows, cols);
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(x != nullptr && out != nullptr, CTMI_ERR_VALUE, "NULL tensor pointer");
+
+  QdqArgs a;
+  a.x = x;
+  a.out = out;
+  a.scale = qp->scale;
+  a.zp = qp->zero_point;
+  a.gscale = qp->global_scale;
+  a.col_group = qp->col_group;
+  a.rows = rows;
+  a.cols = cols;
+  a.s_rows = qp->s_rows;
+  a.s_cols = qp->s_cols;
+  a.blk_rows = qp->blk_rows;
+  a.blk_cols = qp->blk_cols;
+  a.x_dtype = x_dtype;
+  a.out_dtype = out_dtype;
+  a.scale_dtype = qp->scale_dtype;
+  a.zp_dtype = qp->zp_dtype;
+  a.do_q = do_quantize;
+  a.do_dq = do_dequantize;
+  rc = fill_cfg(qp, x_dtype, &a.q);
+  if (rc) return rc;
+
+  dim3 block(256);
+  dim3 grid((unsigned)cdiv(cols, 256), (unsigned)(rows < 32768 ? rows : 32768));
+  hipLaunchKernelGGL(qdq_generic_kernel, grid, block, 0, (hipStream_t)stream, a);
+  return check_launch("ctmi_qdq");
+}

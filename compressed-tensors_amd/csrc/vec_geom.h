@@ -1,0 +1,78 @@
+// Geometry shared by the vectorised streaming kernels: a work item is 8
+// neighbouring elements of one row that share one scale; items are numbered
+// row-major and mapped to their scale with two invariant-divisor divisions.
+#pragma once
+
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+
+namespace ctmi {
+
+// 32-bit division by an invariant divisor: q = (n * m) >> (31 + s), exact for
+// n < 2^31 and 1 <= d < 2^31.
+struct FastDiv {
+  uint32_t d, m, s;
+};
+static inline FastDiv make_fastdiv(uint32_t d) {
+  FastDiv f;
+  f.d = d;
+  uint32_t s = 0;
+  while ((1ull << s) < d) ++s;
+  f.s = s;
+  f.m = (uint32_t)(((1ull << (31 + s)) + d - 1) / d);
+  return f;
+}
+__device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv& f) {
+  return (uint32_t)(((uint64_t)n * f.m) >> 31) >> f.s;
+}
+
+struct VecGeom {
+  FastDiv vpr;        // items per row
+  FastDiv vpb;        // items per scale block (blk_cols / 8)
+  uint32_t nvec;      // total items
+  uint32_t s_cols;
+  uint32_t row_scaled;  // 1: scale row = tensor row; 0: a single scale row
+};
+
+__device__ __forceinline__ uint32_t scale_index(uint32_t v, const VecGeom& g) {
+  const uint32_t r = fdiv(v, g.vpr);
+  const uint32_t cv = v - r * g.vpr.d;
+  return (g.row_scaled ? r * g.s_cols : 0u) + fdiv(cv, g.vpb);
+}
+
+template <int A, int B>
+struct Promote {
+  static constexpr int value = (A == B) ? A : CTMI_F32;
+};
+
+constexpr int kU = 4;
+
+static inline int grid_for(int64_t work_items, int per_block) {
+  int64_t b = cdiv(work_items, per_block);
+  const int64_t cap = 256 * 16;  // 16 resident workgroups per CU is plenty for streaming
+  if (b > cap) b = cap;
+  if (b < 1) b = 1;
+  return (int)b;
+}
+
+// Can the vectorised kernels take this problem?
+static inline bool vec_geometry(const ctmi_qparams* qp, int64_t rows, int64_t cols, VecGeom* g,
+                                bool allow_gscale = false) {
+  if (qp->col_group || (qp->global_scale && !allow_gscale)) return false;
+  if (cols % 8 || qp->blk_cols % 8) return false;
+  if (rows * cols / 8 >= (1ll << 31) || cols / 8 < 1) return false;
+  if (cols % qp->blk_cols) return false;
+  const bool row_scaled = (qp->blk_rows == 1 && qp->s_rows == rows);
+  const bool single_row = (qp->s_rows == 1 && qp->blk_rows >= rows);
+  if (!row_scaled && !single_row) return false;
+  if (qp->s_cols >= (1ll << 31) || rows * qp->s_cols >= (1ll << 31)) return false;
+  g->vpr = make_fastdiv((uint32_t)(cols / 8));
+  g->vpb = make_fastdiv((uint32_t)(qp->blk_cols / 8));
+  g->nvec = (uint32_t)(rows * cols / 8);
+  g->s_cols = (uint32_t)qp->s_cols;
+  g->row_scaled = row_scaled ? 1u : 0u;
+  return true;
+}
+
+
+}  // namespace ctmi

@@ -1,0 +1,226 @@
+/*
+ * ctmi.h — C ABI of libctmi.so, the MI355X (gfx950) implementation of the
+ * compressed-tensors weight compress/decompress hot path.
+ *
+ * Conventions shared by every entry point
+ *   - All tensor pointers are DEVICE pointers owned and pre-allocated by the
+ *     caller; tensors are dense, row-major ("contiguous") unless a stride is
+ *     passed explicitly.  Nothing is allocated, freed or retained.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Work
+ *     is enqueued on it; no entry point synchronises.
+ *   - Return value: CTMI_OK (0) or a negative CTMI_ERR_* code.  Arguments are
+ *     validated BEFORE the first HIP call, so every error path can be exercised
+ *     on a host without a GPU.  ctmi_last_error() returns a thread-local,
+ *     human-readable message for the most recent failure on this thread.
+ *   - The reference implementation is pure Python (torch op chains); each entry
+ *     point names the reference function (file:line under
+ *     src/compressed_tensors/) whose arithmetic it reproduces bit-for-bit.
+ */
+#ifndef CTMI_H_
+#define CTMI_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- return codes (the Python layer maps them to the reference's exception
+ *      classes: ValueError / NotImplementedError / AssertionError / RuntimeError) */
+#define CTMI_OK 0
+#define CTMI_ERR_VALUE (-1)        /* bad argument            -> ValueError          */
+#define CTMI_ERR_UNSUPPORTED (-2)  /* valid but not built     -> NotImplementedError */
+#define CTMI_ERR_ASSERT (-3)       /* reference `assert` site -> AssertionError      */
+#define CTMI_ERR_HIP (-4)          /* HIP runtime failure     -> RuntimeError        */
+
+/* ---- element types */
+#define CTMI_F32 0
+#define CTMI_F16 1
+#define CTMI_BF16 2
+#define CTMI_F8E4M3 3 /* torch.float8_e4m3fn */
+#define CTMI_I8 4
+#define CTMI_I16 5
+#define CTMI_I32 6
+#define CTMI_I64 7
+#define CTMI_U8 8
+#define CTMI_BOOL 9
+
+/* ---- quantized number formats (QuantizationType + num_bits, quant_args.py:85-91) */
+#define CTMI_QTYPE_INT 0
+#define CTMI_QTYPE_FLOAT 1
+
+/* Quantization parameters of one tensor viewed as a 2-D [rows, cols] matrix.
+ *
+ * Scale element (i, j) of a logical [s_rows, s_cols] grid covers the elements
+ *   i == (r / blk_rows) % s_rows     and     j == c / blk_cols
+ * (or j == col_group[c] when col_group is given).  That one rule expresses every
+ * strategy of quantization/lifecycle/forward.py:193-353:
+ *   tensor   s=[1,1]     blk=[rows, cols]        channel  s=[R,1]   blk=[1, cols]
+ *   group    s=[R,C/g]   blk=[1, g]              token    s=[T,1]   blk=[1, cols]
+ *   block    s=[R/bh,C/bw] blk=[bh,bw]           attn_head s=[H,1]  blk=[S, cols]
+ * zero_point (optional) has the same grid.  global_scale (optional) points to
+ * one fp32 on the device: the effective scale is fp32(scale)/global_scale
+ * (forward.py:468-469, 501-502).
+ */
+typedef struct ctmi_qparams {
+  const void* scale;
+  const void* zero_point;     /* NULL = reference called with zero_point=None */
+  const float* global_scale;  /* NULL = none */
+  const int32_t* col_group;   /* NULL = column order; else int32[cols] (act-order g_idx) */
+  int64_t s_rows, s_cols;
+  int64_t blk_rows, blk_cols;
+  int32_t scale_dtype;        /* CTMI_F32 / F16 / BF16 / F8E4M3 */
+  int32_t zp_dtype;           /* any CTMI_* numeric type */
+  int32_t qtype;              /* CTMI_QTYPE_* */
+  int32_t num_bits;           /* INT: 1..32, FLOAT: 4 (e2m1) or 8 (e4m3fn) */
+} ctmi_qparams;
+
+const char* ctmi_last_error(void);
+int ctmi_version(void);
+
+/* A5-A8.  quantize / dequantize / fake_quantize
+ * (quantization/lifecycle/forward.py:45-189, _quantize :455-487, _dequantize
+ * :491-514, round_to_quantized_type quant_args.py:384-408).
+ * do_quantize / do_dequantize select among the three reference functions.
+ * x is [rows, cols] of x_dtype; out is [rows, cols] of out_dtype.  The
+ * arithmetic dtype is derived exactly as torch type promotion would derive it
+ * from (x_dtype, scale_dtype, global_scale). */
+int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_dtype, int64_t rows,
+             int64_t cols, const ctmi_qparams* qp, int32_t do_quantize, int32_t do_dequantize,
+             void* stream);
+
+/* A9.  pack_to_int32 (compressors/quantized_compressors/pack_quantized.py:186-246).
+ * in: int8 [rows, cols]; out: int32 [rows, ceil(cols/pf)] (packed_dim=1) or
+ * int32 [ceil(rows/pf), cols] (packed_dim=0), pf = 32/num_bits. */
+int ctmi_pack_to_int32(const int8_t* in, int32_t* out, int64_t rows, int64_t cols,
+                       int32_t num_bits, int32_t packed_dim, void* stream);
+
+/* A10.  unpack_from_int32 (pack_quantized.py:249-309).  rows/cols are the
+ * ORIGINAL (unpacked) shape; `in` has the packed shape described above. */
+int ctmi_unpack_from_int32(const int32_t* in, int8_t* out, int64_t rows, int64_t cols,
+                           int32_t num_bits, int32_t packed_dim, void* stream);
+
+/* A11 fused.  PackedQuantizationCompressor.compress_weight
+ * (pack_quantized.py:88-145): quantize(dtype=int8) + pack_to_int32 in one pass.
+ * out: int32 [rows, ceil(cols/pf)]. */
+int ctmi_pack_quantized_compress(const void* x, int32_t x_dtype, int32_t* out, int64_t rows,
+                                 int64_t cols, const ctmi_qparams* qp, void* stream);
+
+/* A11 fused.  PackedQuantizationCompressor.decompress_weight
+ * (pack_quantized.py:147-183): unpack_from_int32 + dequantize in one pass.
+ * zero_point in qp is the UNPACKED int8 zero point (or NULL). */
+int ctmi_pack_quantized_decompress(const int32_t* packed, void* out, int32_t out_dtype,
+                                   int64_t rows, int64_t cols, const ctmi_qparams* qp,
+                                   void* stream);
+
+/* A13.  pack_fp4_to_uint8 (compressors/quantized_compressors/fp4_quantized.py:135-178).
+ * x: [rows, cols] float type; out: uint8 [rows, cols/2]. */
+int ctmi_pack_fp4_to_uint8(const void* x, int32_t x_dtype, uint8_t* out, int64_t rows,
+                           int64_t cols, void* stream);
+
+/* A14.  unpack_fp4_from_uint8 (fp4_quantized.py:187-221).  rows/cols = unpacked shape. */
+int ctmi_unpack_fp4_from_uint8(const uint8_t* in, void* out, int32_t out_dtype, int64_t rows,
+                               int64_t cols, void* stream);
+
+/* A15 fused.  NVFP4PackedCompressor.compress_weight (fp4_quantized.py:84-106):
+ * quantize (fp4, global scale) + pack_fp4_to_uint8.  out: uint8 [rows, cols/2]. */
+int ctmi_nvfp4_compress(const void* x, int32_t x_dtype, uint8_t* out, int64_t rows, int64_t cols,
+                        const ctmi_qparams* qp, void* stream);
+
+/* A15 fused.  NVFP4PackedCompressor.decompress_weight (fp4_quantized.py:108-123):
+ * unpack_fp4_from_uint8 (to bf16) + dequantize.  out: [rows, cols] out_dtype. */
+int ctmi_nvfp4_decompress(const uint8_t* packed, void* out, int32_t out_dtype, int64_t rows,
+                          int64_t cols, const ctmi_qparams* qp, void* stream);
+
+/* A19.  pack_bitmasks / unpack_bitmasks (utils/helpers.py:302-339):
+ * numpy.packbits(axis=-1, bitorder="little").  mask: bool/uint8 [rows, cols];
+ * packed: uint8 [rows, ceil(cols/8)]. */
+int ctmi_pack_bitmasks(const uint8_t* mask, uint8_t* packed, int64_t rows, int64_t cols,
+                       void* stream);
+int ctmi_unpack_bitmasks(const uint8_t* packed, uint8_t* mask, int64_t rows, int64_t cols,
+                         void* stream);
+
+/* A17.  bitmask_compress (compressors/sparse_compressors/sparse_bitmask.py:131-149)
+ * in two calls, because the size of `values` is data dependent:
+ *   ctmi_bitmask_count    writes bitmask [rows, ceil(cols/8)], row_offsets int64 [rows]
+ *                         (exclusive prefix sum of per-row non-zero counts) and
+ *                         *total_nnz (int64, device);
+ *   ctmi_bitmask_compact  writes values[total_nnz] (row-major order of the non-zeros).
+ * elem_size is the element width in bytes (1, 2 or 4); `x != 0` is evaluated on
+ * the value of a floating type (so -0.0 is dropped, NaN kept) when
+ * is_float != 0, on the raw integer otherwise.  fp8 tensors are passed as
+ * floats with elem_size 1 (sparse_bitmask.py:141-145 views them as int8 only to
+ * index them; the mask itself comes from `tensor != 0`).
+ * tmp: device scratch of ctmi_bitmask_tmp_bytes(rows) bytes. */
+int64_t ctmi_bitmask_tmp_bytes(int64_t rows);
+int ctmi_bitmask_count(const void* x, int32_t elem_size, int32_t is_float, uint8_t* bitmask,
+                       int64_t* row_offsets, int64_t* total_nnz, void* tmp, int64_t rows,
+                       int64_t cols, void* stream);
+int ctmi_bitmask_compact(const void* x, int32_t elem_size, const uint8_t* bitmask,
+                         const int64_t* row_offsets, void* values, int64_t rows, int64_t cols,
+                         void* stream);
+
+/* A18 / A22.  bitmask_decompress (sparse_bitmask.py:152-169) and
+ * sparse24_bitmask_decompress (sparse_24_bitmask.py:206-224): scatter `values`
+ * (nvalues elements, consumed in row-major order of the set bits; set bits
+ * beyond nvalues read as zero) into a zero-filled [rows, cols].
+ * row_offsets may be NULL: it is then recomputed from the bitmask into tmp
+ * (ctmi_bitmask_tmp_bytes(rows) bytes + rows*8 bytes for the offsets). */
+int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_size,
+                            const uint8_t* bitmask,
+                            const int64_t* row_offsets, void* out, void* tmp, int64_t rows,
+                            int64_t cols, void* stream);
+
+/* A20.  get_24_bytemasks (sparse_24_bitmask.py:227-260): top-2-of-4 by
+ * |value| with torch.topk's tie order.  kind: 0 = float type of elem_size
+ * bytes (bf16 when elem_size==2 && is_bf16), 1 = int8 view of fp8 / int8
+ * (ranked by abs() computed in int8, so abs(-128) == -128).
+ * mask: bool [numel]. */
+int ctmi_get_24_bytemasks(const void* x, int32_t x_dtype, uint8_t* mask, int64_t numel,
+                          void* stream);
+
+/* A21.  sparse24_bitmask_compress (sparse_24_bitmask.py:162-203): values
+ * [rows, cols/2] + packed bitmask [rows, ceil(cols/8)] in one pass. */
+int ctmi_sparse24_compress(const void* x, int32_t x_dtype, void* values, uint8_t* bitmask,
+                           int64_t rows, int64_t cols, void* stream);
+
+/* A1.  calculate_qparams (quantization/utils/helpers.py:67-146), elementwise
+ * over n (min, max) pairs of dtype mm_dtype.  mm_is_0d != 0 when the reference
+ * would see 0-d min/max tensors (their zero-point subtraction then promotes to
+ * fp32).  scale_dtype must be mm_dtype, or CTMI_F8E4M3 for fp4 with a global
+ * scale; zero_point may be NULL. */
+int ctmi_calculate_qparams(const void* min_vals, const void* max_vals, int32_t mm_dtype,
+                           int32_t mm_is_0d, int64_t n, int32_t qtype, int32_t num_bits,
+                           int32_t symmetric, const float* global_scale, void* scale,
+                           int32_t scale_dtype, void* zero_point, int32_t zp_dtype, void* stream);
+
+/* A16.  generate_gparam (helpers.py:414-434): out[i] = fp32(448*6 / max|min,max|). */
+int ctmi_generate_gparam(const void* min_vals, const void* max_vals, int32_t mm_dtype, int64_t n,
+                         float* out, void* stream);
+
+/* A2 / A3.  amin / amax over cells of blk_rows x blk_cols elements of a
+ * [rows, cols] tensor (observer reduction: tests/mock_observer.py:38-56,
+ * helpers.py:199-203).  Outputs have x_dtype and shape
+ * [ceil(rows/blk_rows), ceil(cols/blk_cols)].  tmp: ctmi_minmax_tmp_bytes()
+ * bytes of device scratch, only needed when blk_rows > 1. */
+int64_t ctmi_minmax_tmp_bytes(int64_t rows, int64_t cols, int64_t blk_rows, int64_t blk_cols,
+                              int32_t x_dtype);
+int ctmi_minmax(const void* x, int32_t x_dtype, int64_t rows, int64_t cols, int64_t blk_rows,
+                int64_t blk_cols, void* min_out, void* max_out, void* tmp, void* stream);
+
+/* A2 + A1 fused for cells one row tall (group / channel / token): min-max
+ * reduction and calculate_qparams in one pass over x.  scale / zero_point:
+ * [rows, ceil(cols/blk_cols)]; min_out / max_out optional (x_dtype). */
+int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows, int64_t cols,
+                         int64_t blk_cols, int32_t qtype, int32_t num_bits, int32_t symmetric,
+                         const float* global_scale, void* scale, int32_t scale_dtype,
+                         void* zero_point, int32_t zp_dtype, void* min_out, void* max_out,
+                         void* stream);
+
+/* The 4096-entry keep table used by the 2:4 kernels (host copy, for tests). */
+void ctmi_topk24_lut(uint8_t* out4096);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CTMI_H_ */
