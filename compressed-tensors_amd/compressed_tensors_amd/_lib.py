@@ -67,6 +67,21 @@ class QParams(ctypes.Structure):
 
 _QP = POINTER(QParams)
 
+
+class WeightJob(ctypes.Structure):
+    """mirror of `struct ctmi_weight_job`"""
+
+    _fields_ = [
+        ("src", c_void_p),
+        ("dst", c_void_p),
+        ("rows", c_int64),
+        ("cols", c_int64),
+        ("dense_dtype", c_int32),
+        ("reserved", c_int32),
+        ("qp", QParams),
+    ]
+
+
 # name -> (restype, argtypes); must list every symbol of include/ctmi.h
 SIGNATURES = {
     "ctmi_last_error": (c_char_p, []),
@@ -91,6 +106,8 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int64, c_int64, _QP, c_void_p],
     ),
+    "ctmi_pack_quantized_compress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
+    "ctmi_pack_quantized_decompress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
     "ctmi_pack_fp4_to_uint8": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_void_p]),
     "ctmi_unpack_fp4_from_uint8": (
         c_int32,

@@ -211,3 +211,68 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
             )
         )
         return out
+
+
+class PackedWeightBatch:
+    """Every weight of a state dict prepared for one-call compress / decompress.
+
+    Holds the dense weights, their qparams, the packed outputs and the job
+    tables the C ABI consumes (ctmi_pack_quantized_{compress,decompress}_many).
+    Buffers are allocated once; `compress()` / `decompress()` only enqueue
+    kernels, so a serving or benchmarking loop can call them repeatedly.
+    """
+
+    def __init__(self, entries, device=None):
+        """entries: list of dicts with keys weight, scale, quantization_args and
+        optionally zero_point, g_idx (tensors on the GPU, or moved there)."""
+        self.n = len(entries)
+        self.names = [e.get("name", str(i)) for i, e in enumerate(entries)]
+        self._keep = []
+        self.weights, self.packed, self.dense, self.scales = [], [], [], []
+        self._cjobs = (_lib.WeightJob * max(self.n, 1))()
+        self._djobs = (_lib.WeightJob * max(self.n, 1))()
+        self.device = device
+        for i, e in enumerate(entries):
+            args = e["quantization_args"]
+            w, scale, zp, g_idx = (to_gpu(e.get(k)) for k in ("weight", "scale", "zero_point", "g_idx"))
+            if w.ndim != 2:
+                raise ValueError(f"expected a 2-D weight, got shape {tuple(w.shape)}")
+            if self.device is None:
+                self.device = w.device
+            w = w.contiguous()
+            rows, cols = w.shape
+            if args.num_bits > 8:
+                raise ValueError("Packing is only supported for less than 8 bits")
+            pf = 32 // args.num_bits
+            packed = torch.empty((rows, math.ceil(cols / pf)), dtype=torch.int32, device=w.device)
+            dense = torch.empty((rows, cols), dtype=scale.dtype, device=w.device)
+            cplan = build_qparams(w, scale, zp, args, g_idx, None)
+            dq_args = infer_dequant_args(_ShapeOnly(w.shape, torch.int8), scale)
+            dplan = build_qparams(_ShapeOnly(w.shape, torch.int8), scale, zp, dq_args, g_idx, None)
+            dplan.qp.qtype, dplan.qp.num_bits = _lib.QTYPE_INT, args.num_bits
+            self._keep += [cplan, dplan]
+            cj, dj = self._cjobs[i], self._djobs[i]
+            cj.src, cj.dst, cj.rows, cj.cols = w.data_ptr(), packed.data_ptr(), rows, cols
+            cj.dense_dtype, cj.qp = _lib.dtype_code(w.dtype), cplan.qp
+            dj.src, dj.dst, dj.rows, dj.cols = packed.data_ptr(), dense.data_ptr(), rows, cols
+            dj.dense_dtype, dj.qp = _lib.dtype_code(scale.dtype), dplan.qp
+            self.weights.append(w)
+            self.packed.append(packed)
+            self.dense.append(dense)
+            self.scales.append(scale)
+
+    def compress(self):
+        """enqueue quantize+pack of every weight; returns the packed tensors"""
+        _lib.check(
+            _lib.load().ctmi_pack_quantized_compress_many(self._cjobs, self.n,
+                                                          _lib.stream_of(self.device))
+        )
+        return self.packed
+
+    def decompress(self):
+        """enqueue unpack+dequantize of every packed weight; returns the dense tensors"""
+        _lib.check(
+            _lib.load().ctmi_pack_quantized_decompress_many(self._djobs, self.n,
+                                                            _lib.stream_of(self.device))
+        )
+        return self.dense

@@ -53,7 +53,7 @@ __device__ __forceinline__ float f8e4m3_to_f32(uint8_t b) {
 }
 
 // fp32 -> e4m3fn, round-to-nearest-even including the subnormal range (step
-// 2^-9).  Magnitudes that round above 448 (>= 464) and NaN give the NaN code,
+// 2^-9).  Magnitudes that round above 448 (> 464) and NaN give the NaN code,
 // which is what torch's cast does (it does not saturate).
 __device__ __forceinline__ uint8_t f32_to_f8e4m3(float f) {
   uint32_t u = f2u(f);
@@ -70,7 +70,7 @@ __device__ __forceinline__ uint8_t f32_to_f8e4m3(float f) {
     uint32_t odd = (u >> 20) & 1u;
     u += 0x7FFFFu + odd;        // RNE at bit 20
     u -= (120u << 23);          // rebias 127 -> 7
-    r = (uint8_t)(u >> 20);     // 464 <= |f| < 480 lands on 0x7F (NaN), as in torch
+    r = (uint8_t)(u >> 20);     // 464 < |f| < 480 lands on 0x7F (NaN), as in torch
   }
   return r | sign;
 }

@@ -492,3 +492,31 @@ extern "C" int ctmi_pack_quantized_decompress(const int32_t* packed, void* out, 
   hipLaunchKernelGGL(pq_decompress_generic_kernel, grid_for(rows * cols, 256), 256, 0, st, a);
   return check_launch("ctmi_pack_quantized_decompress");
 }
+
+// ------------------------------------------------------------------ many weights, one call
+// The state-dict loops of the compressors hand over every weight of a model at
+// once; launching them from one host call keeps the GPU queue full (a Python
+// round trip per tensor costs more than the kernels of a 4096 x 4096 weight).
+extern "C" int ctmi_pack_quantized_compress_many(const ctmi_weight_job* jobs, int64_t n,
+                                                 void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_weight_job& j = jobs[i];
+    int rc = ctmi_pack_quantized_compress(j.src, j.dense_dtype, (int32_t*)j.dst, j.rows, j.cols,
+                                          &j.qp, stream);
+    if (rc) return rc;
+  }
+  return CTMI_OK;
+}
+
+extern "C" int ctmi_pack_quantized_decompress_many(const ctmi_weight_job* jobs, int64_t n,
+                                                   void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_weight_job& j = jobs[i];
+    int rc = ctmi_pack_quantized_decompress((const int32_t*)j.src, j.dst, j.dense_dtype, j.rows,
+                                            j.cols, &j.qp, stream);
+    if (rc) return rc;
+  }
+  return CTMI_OK;
+}

@@ -113,6 +113,26 @@ int ctmi_pack_quantized_decompress(const int32_t* packed, void* out, int32_t out
                                    int64_t rows, int64_t cols, const ctmi_qparams* qp,
                                    void* stream);
 
+/* One weight of a state dict.  src/dst: for compress, dense weight -> packed
+ * words; for decompress, packed words -> dense weight.  dense_dtype is the
+ * dtype of the dense side. */
+typedef struct ctmi_weight_job {
+  const void* src;
+  void* dst;
+  int64_t rows, cols;
+  int32_t dense_dtype;
+  int32_t reserved;
+  ctmi_qparams qp;
+} ctmi_weight_job;
+
+/* A27.  The per-weight loop of BaseQuantizationCompressor.compress /
+ * decompress_from_state_dict (compressors/quantized_compressors/base.py:91-125,
+ * 213-230) for the pack-quantized format: n fused launches from one call.
+ * Jobs are validated and enqueued in order; on the first invalid job the call
+ * returns its error (earlier jobs stay enqueued). */
+int ctmi_pack_quantized_compress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
+int ctmi_pack_quantized_decompress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
+
 /* A13.  pack_fp4_to_uint8 (compressors/quantized_compressors/fp4_quantized.py:135-178).
  * x: [rows, cols] float type; out: uint8 [rows, cols/2]. */
 int ctmi_pack_fp4_to_uint8(const void* x, int32_t x_dtype, uint8_t* out, int64_t rows,

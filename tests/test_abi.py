@@ -1,0 +1,135 @@
+"""The C-ABI library: it loads, exports every symbol the header declares, and
+rejects bad arguments before touching a device (so this runs without a GPU)."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from compressed_tensors_amd import _lib
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def _declared_symbols():
+    text = (ROOT / "include" / "ctmi.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ctmi_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(ctmi):
+    names = _declared_symbols()
+    assert len(names) >= 25
+    for name in names:
+        assert hasattr(ctmi, name), f"{name} declared in ctmi.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert set(_lib.SIGNATURES) == set(names)
+
+
+def test_version_and_struct_layout(ctmi):
+    assert ctmi.ctmi_version() == 1
+    assert ctypes.sizeof(_lib.QParams) == 4 * 8 + 4 * 8 + 4 * 4
+
+
+def _err(ctmi):
+    return ctmi.ctmi_last_error().decode()
+
+
+def test_pack_argument_errors(ctmi):
+    assert ctmi.ctmi_pack_to_int32(None, None, 4, 4, 9, 1, None) == _lib.CTMI_ERR_VALUE
+    assert "less than 8 bits" in _err(ctmi)
+    assert ctmi.ctmi_pack_to_int32(None, None, 4, 4, 0, 1, None) == _lib.CTMI_ERR_VALUE
+    assert "at least 1" in _err(ctmi)
+    assert ctmi.ctmi_pack_to_int32(None, None, 4, 4, 4, 2, None) == _lib.CTMI_ERR_VALUE
+    assert ctmi.ctmi_unpack_from_int32(None, None, 4, 4, 16, 1, None) == _lib.CTMI_ERR_VALUE
+    # empty tensors are fine and launch nothing
+    assert ctmi.ctmi_pack_to_int32(None, None, 0, 8, 4, 1, None) == _lib.CTMI_OK
+    # NULL data with a non-empty shape is refused on the host
+    assert ctmi.ctmi_pack_to_int32(None, None, 2, 8, 4, 1, None) == _lib.CTMI_ERR_VALUE
+
+
+def _qp(**kw):
+    qp = _lib.QParams()
+    qp.scale = 0x1000  # never dereferenced on these paths
+    qp.s_rows, qp.s_cols, qp.blk_rows, qp.blk_cols = 1, 1, 4, 8
+    qp.scale_dtype = _lib.BF16
+    qp.qtype, qp.num_bits = _lib.QTYPE_INT, 4
+    for k, v in kw.items():
+        setattr(qp, k, v)
+    return qp
+
+
+def test_quant_argument_errors(ctmi):
+    qp = _qp(num_bits=6, qtype=_lib.QTYPE_FLOAT)
+    rc = ctmi.ctmi_qdq(None, _lib.BF16, None, _lib.BF16, 4, 8, ctypes.byref(qp), 1, 0, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "4 and 8 bits" in _err(ctmi)
+    qp = _qp(qtype=7)
+    rc = ctmi.ctmi_qdq(None, _lib.BF16, None, _lib.BF16, 4, 8, ctypes.byref(qp), 1, 0, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "Invalid quantization type" in _err(ctmi)
+    qp = _qp()
+    rc = ctmi.ctmi_qdq(None, _lib.I8, None, _lib.I8, 4, 8, ctypes.byref(qp), 1, 0, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED  # cannot quantize an int8 tensor
+    qp = _qp(global_scale=0x1000)
+    rc = ctmi.ctmi_pack_quantized_compress(None, _lib.BF16, None, 4, 8, ctypes.byref(qp), None)
+    assert rc == _lib.CTMI_ERR_VALUE and "global_scale is not supported" in _err(ctmi)
+    qp = _qp(num_bits=16)
+    rc = ctmi.ctmi_pack_quantized_compress(None, _lib.BF16, None, 4, 8, ctypes.byref(qp), None)
+    assert rc == _lib.CTMI_ERR_VALUE and "less than 8 bits" in _err(ctmi)
+    qp = _qp(scale_dtype=_lib.F8E4M3)
+    rc = ctmi.ctmi_qdq(None, _lib.BF16, None, _lib.BF16, 4, 8, ctypes.byref(qp), 1, 0, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "global_scale" in _err(ctmi)
+    qp = _qp(s_cols=1, blk_cols=4)  # grid too small for 8 columns
+    rc = ctmi.ctmi_qdq(None, _lib.BF16, None, _lib.BF16, 4, 8, ctypes.byref(qp), 1, 0, None)
+    assert rc == _lib.CTMI_ERR_VALUE
+
+
+def test_fp4_and_sparse_argument_errors(ctmi):
+    assert ctmi.ctmi_pack_fp4_to_uint8(None, _lib.BF16, None, 3, 7, None) == _lib.CTMI_ERR_VALUE
+    assert "even number of columns" in _err(ctmi)
+    assert ctmi.ctmi_pack_fp4_to_uint8(None, _lib.I8, None, 3, 8, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert ctmi.ctmi_get_24_bytemasks(None, _lib.BF16, None, 6, None) == _lib.CTMI_ERR_VALUE
+    assert "multiple of 4" in _err(ctmi)
+    assert ctmi.ctmi_sparse24_compress(None, _lib.BF16, None, None, 3, 2, None) == _lib.CTMI_ERR_VALUE
+    assert ctmi.ctmi_bitmask_count(None, 3, 1, None, None, 0x1000, None, 2, 2, None) == \
+        _lib.CTMI_ERR_UNSUPPORTED
+    assert ctmi.ctmi_calculate_qparams(None, None, _lib.BF16, 0, 4, _lib.QTYPE_FLOAT, 4, 0, None,
+                                       None, _lib.BF16, None, _lib.F8E4M3, None) == \
+        _lib.CTMI_ERR_UNSUPPORTED
+    assert "Asymmetric Quantization is not supported for FP4" in _err(ctmi)
+
+
+def test_topk24_table_matches_installed_torch(ctmi):
+    """the 2:4 keep table compiled into the library against torch.topk on every
+    weak ordering of four keys"""
+    import itertools
+
+    import torch
+
+    buf = (ctypes.c_uint8 * 4096)()
+    ctmi.ctmi_topk24_lut(buf)
+    pairs = [(0, 1), (0, 2), (0, 3), (1, 2), (1, 3), (2, 3)]
+    seen = 0
+    for t in itertools.product(range(4), repeat=4):
+        if sorted(set(t)) != list(range(len(set(t)))):
+            continue
+        idx = 0
+        for p, (i, j) in enumerate(pairs):
+            idx |= (2 if t[i] > t[j] else (1 if t[i] == t[j] else 0)) << (2 * p)
+        for dtype in (torch.float32, torch.bfloat16, torch.int8):
+            keep = torch.tensor([t], dtype=dtype).topk(2, dim=1).indices[0].tolist()
+            assert buf[idx] == (1 << keep[0]) | (1 << keep[1]), (t, dtype)
+        seen += 1
+    assert seen == 75
+
+
+def test_product_refuses_cpu_tensors():
+    import torch
+
+    from compressed_tensors_amd.quantization import QuantizationArgs, quantize
+
+    if torch.cuda.is_available():
+        pytest.skip("needs a host without GPU")
+    x = torch.zeros(4, 8, dtype=torch.bfloat16)
+    s = torch.ones(1, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU"):
+        quantize(x, s, None, QuantizationArgs(num_bits=4))

@@ -1,0 +1,240 @@
+"""GPU parity: int32 packing, fp4 nibble packing and the quantization
+compressors (pack-quantized, naive/int/float-quantized, nvfp4-pack-quantized)
+vs the oracle, bit-exact."""
+import json
+from pathlib import Path
+
+import pytest
+import torch
+
+from gpu_util import announce, assert_bit_equal
+from oracle import pack as op
+from oracle import quant as oq
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).parent / "golden"
+
+
+def _pair(d):
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    return QuantizationArgs(**d), oq._Args(**d)
+
+
+def test_pack_known_answers_on_gpu(gpu):
+    from compressed_tensors_amd.compressors import pack_to_int32, unpack_from_int32
+
+    for case in json.loads((GOLDEN / "pack_int32.json").read_text())["cases"]:
+        announce("pack golden", case["num_bits"], case["values"])
+        values = torch.tensor(case["values"], dtype=torch.int8)
+        packed = torch.tensor(case["packed"], dtype=torch.int32)
+        assert_bit_equal(pack_to_int32(values.to(gpu), case["num_bits"]), packed, "pack")
+        assert_bit_equal(unpack_from_int32(packed.to(gpu), case["num_bits"], values.shape), values, "unpack")
+
+
+@pytest.mark.parametrize("bits", [1, 2, 3, 4, 5, 7, 8])
+@pytest.mark.parametrize("shape", [(1, 1), (5, 37), (16, 64), (3, 1024), (130, 48)])
+def test_pack_unpack_random(bits, shape, gpu):
+    from compressed_tensors_amd.compressors import pack_to_int32, unpack_from_int32
+
+    announce("pack random", bits, shape)
+    g = torch.Generator().manual_seed(bits * 1000 + shape[0])
+    v = torch.randint(-(1 << (bits - 1)), 1 << (bits - 1), shape, generator=g, dtype=torch.int8)
+    for dim in (1, 0):
+        p = pack_to_int32(v.to(gpu), bits, packed_dim=dim)
+        want = op.pack_to_int32(v, bits, packed_dim=dim).contiguous()
+        assert_bit_equal(p, want, f"pack dim{dim}")
+        u = unpack_from_int32(p, bits, v.shape, packed_dim=dim)
+        assert_bit_equal(u, v, f"unpack dim{dim}")
+    # out-of-range int8 input: the reference adds the shifted terms, carries and all
+    wild = torch.randint(-128, 128, shape, generator=g, dtype=torch.int8)
+    assert_bit_equal(pack_to_int32(wild.to(gpu), bits), op.pack_to_int32(wild, bits), "wild pack")
+
+
+def test_pack_errors(gpu):
+    from compressed_tensors_amd.compressors import pack_to_int32, unpack_from_int32
+
+    with pytest.raises(ValueError, match="int8"):
+        pack_to_int32(torch.zeros(2, 2, dtype=torch.int32, device=gpu), 4)
+    with pytest.raises(ValueError, match="less than 8"):
+        pack_to_int32(torch.zeros(2, 2, dtype=torch.int8, device=gpu), 9)
+    with pytest.raises(ValueError, match="at least 1"):
+        pack_to_int32(torch.zeros(2, 2, dtype=torch.int8, device=gpu), 0)
+    with pytest.raises(ValueError, match="Expected"):
+        unpack_from_int32(torch.zeros(2, 2, dtype=torch.int8, device=gpu), 4, (2, 2))
+    e = pack_to_int32(torch.zeros(0, 8, dtype=torch.int8, device=gpu), 4)
+    assert e.shape == (0, 1) and e.dtype == torch.int32
+
+
+PQ = [
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (128, 1024), torch.bfloat16),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=128), (128, 512), torch.bfloat16),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="channel"), (64, 520), torch.bfloat16),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="channel"), (19, 256), torch.float16),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=64), (32, 256), torch.float32),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="tensor"), (32, 256), torch.bfloat16),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="tensor"), (7, 36), torch.bfloat16),  # ragged: generic kernel
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=12), (10, 36), torch.bfloat16),
+    (dict(num_bits=3, type="int", symmetric=True, strategy="channel"), (10, 40), torch.bfloat16),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="block", block_structure=[4, 16]), (16, 64), torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype", PQ, ids=[f"pq{i}-{c[0]['strategy']}" for i, c in enumerate(PQ)])
+def test_pack_quantized_compressor(spec, shape, dtype, gpu):
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("pack-quantized", spec, shape, dtype)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(31)
+    w = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+    w.view(-1)[0] = -0.0
+    scale, zp = oq.observe_weight(w, oargs)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    want = op.pack_quantized_compress(w, scale, oargs, zero_point=zp)
+    for zero_point in ((zp,) if not spec["symmetric"] else (zp, None)):
+        got = comp.compress_weight(
+            weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+            zero_point=None if zero_point is None else zero_point.to(gpu))
+        assert set(got) == set(want)
+        assert_bit_equal(got["weight_packed"], want["weight_packed"], "weight_packed")
+        assert_bit_equal(got["weight_shape"], want["weight_shape"], "weight_shape")
+        if "weight_zero_point" in want:
+            assert_bit_equal(got["weight_zero_point"], want["weight_zero_point"], "packed zp")
+    data = dict(want, weight_scale=scale)
+    dense_want = op.pack_quantized_decompress(dict(data), oargs)
+    dense = comp.decompress_weight({k: v.to(gpu) for k, v in data.items()}, quantization_args=args)
+    assert_bit_equal(dense, dense_want, "decompress")
+    # the reference's own property: compress -> decompress == fake_quantize
+    assert_bit_equal(dense, oq.fake_quantize(w, scale, zp, oargs).to(scale.dtype), "== fake_quantize")
+
+
+def test_pack_quantized_state_dict_and_g_idx(gpu):
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.quantization import QuantizationScheme
+
+    announce("pack-quantized state dict")
+    spec = dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=32)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(33)
+    w = (torch.randn(16, 128, generator=g) * 0.02).bfloat16()
+    g_idx = (torch.randperm(128, generator=g) // 32).to(torch.int32)
+    scale, zp = oq.observe_weight(w.index_select(-1, torch.argsort(g_idx)), oargs)
+    state = {
+        "m.weight": w, "m.weight_scale": scale, "m.weight_zero_point": zp, "m.weight_g_idx": g_idx,
+        "m.bias": torch.ones(16), "other.weight": torch.ones(4, 4),
+    }
+    scheme = QuantizationScheme(targets=["Linear"], weights=args)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    out = comp.compress({k: v.to(gpu) for k, v in state.items()}, names_to_scheme={"m": scheme})
+    assert set(out) == {"m.weight_packed", "m.weight_shape", "m.weight_scale", "m.weight_zero_point",
+                        "m.weight_g_idx", "m.bias", "other.weight"}
+    want = op.pack_quantized_compress(w, scale, oargs, zero_point=zp, g_idx=g_idx)
+    assert_bit_equal(out["m.weight_packed"], want["weight_packed"], "packed (g_idx)")
+    assert_bit_equal(out["m.weight_zero_point"], want["weight_zero_point"], "zp packed")
+    assert out["m.weight_zero_point"].dtype == torch.int32 and out["m.weight_shape"].dtype == torch.int64
+    (path, data), = list(comp.decompress(out, names_to_scheme={"m": scheme}))
+    assert path == "m"
+    want_dense = op.pack_quantized_decompress(
+        dict(want, weight_scale=scale, weight_g_idx=g_idx), oargs)
+    assert_bit_equal(data["weight"], want_dense, "state-dict decompress")
+    with pytest.raises(ValueError, match="global_scale"):
+        comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+                             global_scale=torch.ones(1, device=gpu))
+
+
+NQ = [
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (96, 512), torch.bfloat16),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="tensor"), (31, 65), torch.float16),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (96, 512), torch.bfloat16),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=128), (16, 256), torch.bfloat16),
+    ("naive-quantized", dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (16, 64), torch.float32),
+]
+
+
+@pytest.mark.parametrize("fmt,spec,shape,dtype", NQ, ids=[f"{c[0]}-{i}" for i, c in enumerate(NQ)])
+def test_naive_compressors(fmt, spec, shape, dtype, gpu):
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce(fmt, spec, shape, dtype)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(41)
+    w = torch.randn(shape, generator=g) * 0.02
+    w[torch.rand(shape, generator=g) < 0.001] *= 20
+    w = w.to(dtype)
+    w.view(-1)[1] = -0.0
+    scale, zp = oq.observe_weight(w, oargs)
+    comp = BaseCompressor.load_from_registry(fmt)
+    for zero_point in ((zp,) if not spec["symmetric"] else (zp, None)):
+        got = comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+                                   zero_point=None if zero_point is None else zero_point.to(gpu))
+        want = op.naive_compress(w, scale, oargs, zero_point=zero_point)
+        assert list(got) == ["weight"]
+        assert_bit_equal(got["weight"], want, "codes")
+        data = {"weight": want, "weight_scale": scale}
+        if zero_point is not None:
+            data["weight_zero_point"] = zero_point
+        dense = comp.decompress_weight({k: v.to(gpu) for k, v in data.items()}, quantization_args=args)
+        assert_bit_equal(dense, op.naive_decompress(data), "decompress")
+
+
+def test_fp4_pack_golden_on_gpu(gpu):
+    from compressed_tensors_amd.compressors import pack_fp4_to_uint8, unpack_fp4_from_uint8
+
+    announce("fp4 golden")
+    gold = json.loads((GOLDEN / "fp4_pack.json").read_text())
+    x = torch.tensor(gold["roundtrip"]).to(torch.bfloat16)
+    packed = pack_fp4_to_uint8(x.to(gpu))
+    assert_bit_equal(packed, op.pack_fp4_to_uint8(x), "fp4 pack")
+    back = unpack_fp4_from_uint8(packed, 4, 8, dtype=torch.bfloat16)
+    assert_bit_equal(back, x, "fp4 unpack (sign of zero included)")
+    with pytest.raises(ValueError, match="even number of columns"):
+        pack_fp4_to_uint8(torch.tensor(gold["odd_columns_raise"]).to(gpu))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("shape", [(3, 6), (16, 64), (5, 1026)])
+def test_fp4_pack_off_grid_inputs(dtype, shape, gpu):
+    """values off the e2m1 grid go to the nearest entry exactly as the reference's
+    argmin over |x - lut| (computed in x's dtype) picks it"""
+    from compressed_tensors_amd.compressors import pack_fp4_to_uint8, unpack_fp4_from_uint8
+
+    announce("fp4 off grid", dtype, shape)
+    g = torch.Generator().manual_seed(17)
+    x = (torch.randn(shape, generator=g) * 3).to(dtype)
+    x.view(-1)[:6] = torch.tensor([0.25, 0.75, -1.25, 2.5, 5.0, -7.5]).to(dtype)
+    packed = pack_fp4_to_uint8(x.to(gpu))
+    want = op.pack_fp4_to_uint8(x)
+    assert_bit_equal(packed, want, "fp4 pack off-grid")
+    for out_dtype in (torch.bfloat16, torch.float32):
+        assert_bit_equal(unpack_fp4_from_uint8(packed, *shape, dtype=out_dtype),
+                         op.unpack_fp4_from_uint8(want, *shape, dtype=out_dtype), "fp4 unpack")
+
+
+@pytest.mark.parametrize("shape,dtype", [((64, 256), torch.bfloat16), ((24, 48), torch.bfloat16),
+                                         ((32, 128), torch.float16), ((8, 64), torch.float32)])
+def test_nvfp4_compressor(shape, dtype, gpu):
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("nvfp4", shape, dtype)
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(51)
+    w = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+    w.view(-1)[:3] = torch.tensor([0.0, -0.0, -1e-6]).to(dtype)
+    gs = oq.generate_gparam(*[t.reshape(1) for t in torch.aminmax(w)])
+    scale, zp = oq.observe_weight(w, oargs, global_scale=gs)
+    assert scale.dtype == torch.float8_e4m3fn and gs.dtype == torch.float32
+    comp = BaseCompressor.load_from_registry("nvfp4-pack-quantized")
+    for zero_point in (zp, None):
+        got = comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), global_scale=gs.to(gpu),
+                                   quantization_args=args,
+                                   zero_point=None if zero_point is None else zero_point.to(gpu))
+        want = op.nvfp4_compress(w, scale, gs, oargs, zero_point=zero_point)
+        assert list(got) == ["weight_packed"]
+        assert_bit_equal(got["weight_packed"], want, f"nvfp4 codes (zp={'yes' if zero_point is not None else 'no'})")
+    dense = comp.decompress_weight(
+        {"weight_packed": want.to(gpu), "weight_scale": scale.to(gpu),
+         "weight_global_scale": gs.to(gpu)}, quantization_args=args)
+    assert_bit_equal(dense, op.nvfp4_decompress(want, scale, gs), "nvfp4 decompress")
+    assert dense.dtype == torch.bfloat16

@@ -1,0 +1,224 @@
+"""GPU parity: quantize / dequantize / fake_quantize and qparams vs the oracle
+(bit-exact), called through the Python mirror of the reference API -> C ABI."""
+import json
+from pathlib import Path
+
+import pytest
+import torch
+
+from gpu_util import announce, assert_bit_equal
+from oracle import quant as oq
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).parent / "golden"
+
+
+def _pair(d):
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    d = dict(d)
+    dyn = d.pop("dynamic", False)
+    return QuantizationArgs(dynamic=dyn, **d), oq._Args(**d)
+
+
+def _weights(shape, dtype, seed, std=0.02):
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(shape, generator=g) * std).to(dtype)
+    flat = w.view(-1)
+    flat[0] = 0.0
+    if flat.numel() > 8:
+        flat[3] = -0.0
+        flat[5] = flat[4].abs() * 20
+    return w
+
+
+CASES = [
+    # (args, shape, x dtype, scale dtype override)
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (64, 512), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=128), (64, 512), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (33, 96), torch.float16, None),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (48, 200), torch.bfloat16, None),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="channel"), (48, 200), torch.float32, None),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="tensor"), (17, 129), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="tensor"), (17, 129), torch.float16, None),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (40, 256), torch.bfloat16, None),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="tensor"), (40, 250), torch.float16, None),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[16, 32]), (64, 128), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="block", block_structure=[2, 3]), (4, 6), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (32, 256), torch.bfloat16, torch.float32),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=64), (32, 256), torch.float16, torch.bfloat16),
+    (dict(num_bits=2, type="int", symmetric=True, strategy="channel"), (8, 64), torch.bfloat16, None),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype,sdt", CASES,
+                         ids=[f"{c[0]['type']}{c[0]['num_bits']}-{c[0]['strategy']}-{str(c[2])[6:]}-{i}"
+                              for i, c in enumerate(CASES)])
+def test_static_qdq_matches_oracle(spec, shape, dtype, sdt, gpu):
+    from compressed_tensors_amd.quantization import (
+        dequantize, fake_quantize, observe_weight_qparams, quantize,
+    )
+
+    announce("static_qdq", spec, shape, dtype, sdt)
+    args, oargs = _pair(spec)
+    w = _weights(shape, dtype, seed=11)
+    o_scale, o_zp = oq.observe_weight(w, oargs)
+    # observer + calculate_qparams on the GPU
+    scale, zp = observe_weight_qparams(w.to(gpu), args)
+    assert_bit_equal(scale, o_scale, "scale")
+    assert_bit_equal(zp, o_zp, "zero_point")
+    if sdt is not None:
+        o_scale = o_scale.to(sdt)
+        scale = o_scale.to(gpu)
+    qdt = oq.pytorch_dtype(oargs)
+    for zero_point, o_zero_point in ((zp, o_zp), (None, None)):
+        if zero_point is None and not spec["symmetric"]:
+            continue
+        q = quantize(w.to(gpu), scale, zero_point, args, dtype=qdt)
+        oq_ = oq.quantize(w, o_scale, o_zero_point, oargs, dtype=qdt)
+        assert_bit_equal(q, oq_, "quantize")
+        qf = quantize(w.to(gpu), scale, zero_point, args)  # no dtype: stays floating
+        assert_bit_equal(qf, oq.quantize(w, o_scale, o_zero_point, oargs), "quantize(no dtype)")
+        dq = dequantize(q, scale, zero_point, args)
+        assert_bit_equal(dq, oq.dequantize(oq_, o_scale, o_zero_point, oargs), "dequantize")
+        dq2 = dequantize(q, scale, zero_point)  # strategy inferred from the scale's shape
+        assert_bit_equal(dq2, oq.dequantize(oq_, o_scale, o_zero_point), "dequantize(inferred)")
+        fq = fake_quantize(w.to(gpu), scale, zero_point, args)
+        assert_bit_equal(fq, oq.fake_quantize(w, o_scale, o_zero_point, oargs), "fake_quantize")
+
+
+def test_reference_golden_qdq_on_gpu(gpu):
+    """the reference's own expected QDQ matrices, reproduced by the HIP path"""
+    from compressed_tensors_amd.quantization import (
+        fake_quantize, generate_gparam, observe_weight_qparams,
+    )
+
+    gold = json.loads((GOLDEN / "static_lifecycle.json").read_text())
+    w = torch.arange(24, dtype=torch.bfloat16).reshape(4, 6)
+    for case in gold["weight_cases"]:
+        announce("golden", case["args"])
+        args, oargs = _pair(case["args"])
+        gs = o_gs = None
+        if args.strategy == "tensor_group":
+            mn, mx = torch.aminmax(w)
+            o_gs = oq.generate_gparam(mn.reshape(1), mx.reshape(1))
+            gs = generate_gparam(mn.reshape(1).to(gpu), mx.reshape(1).to(gpu))
+            assert_bit_equal(gs, o_gs, "global scale")
+        scale, zp = observe_weight_qparams(w.to(gpu), args, global_scale=gs)
+        o_scale, o_zp = oq.observe_weight(w, oargs, global_scale=o_gs)
+        assert_bit_equal(scale, o_scale, "scale")
+        assert_bit_equal(zp, o_zp, "zp")
+        out = fake_quantize(w.to(gpu), scale, zp, args, global_scale=gs)
+        assert_bit_equal(out, oq.fake_quantize(w, o_scale, o_zp, oargs, global_scale=o_gs), "qdq")
+        assert torch.allclose(out.cpu(), torch.tensor(case["qdq"]).to(out.dtype))
+
+
+def test_act_order_g_idx(gpu):
+    from compressed_tensors_amd.quantization import dequantize, quantize
+
+    announce("g_idx")
+    spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32)
+    args, oargs = _pair(spec)
+    w = _weights((24, 128), torch.bfloat16, seed=5)
+    g = torch.Generator().manual_seed(6)
+    g_idx = (torch.randperm(128, generator=g) // 32).to(torch.int32)
+    perm = torch.argsort(g_idx)
+    o_scale, o_zp = oq.observe_weight(w.index_select(-1, perm), oargs)
+    q = quantize(w.to(gpu), o_scale.to(gpu), o_zp.to(gpu), args, dtype=torch.int8, g_idx=g_idx.to(gpu))
+    want = oq.quantize(w, o_scale, o_zp, oargs, dtype=torch.int8, g_idx=g_idx)
+    assert_bit_equal(q, want, "quantize g_idx")
+    dq = dequantize(q, o_scale.to(gpu), o_zp.to(gpu), g_idx=g_idx.to(gpu))
+    assert_bit_equal(dq, oq.dequantize(want, o_scale, o_zp, g_idx=g_idx), "dequantize g_idx")
+    # g_idx full of -1 means column order
+    unset = torch.full((128,), -1, dtype=torch.int32)
+    q2 = quantize(w.to(gpu), o_scale.to(gpu), None, args, dtype=torch.int8, g_idx=unset.to(gpu))
+    assert_bit_equal(q2, oq.quantize(w, o_scale, None, oargs, dtype=torch.int8, g_idx=unset), "unset g_idx")
+
+
+DYN = [
+    (dict(num_bits=8, type="float", symmetric=True, strategy="token", dynamic=True), (2, 40, 256), torch.bfloat16),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="token", dynamic=True), (1, 33, 100), torch.float16),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="token", dynamic=True), (3, 8, 64), torch.bfloat16),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="token", dynamic=True), (16, 64), torch.bfloat16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="tensor", dynamic=True), (4, 9, 31), torch.bfloat16),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="tensor", dynamic=True), (7, 33), torch.bfloat16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=128, dynamic=True), (1, 16, 512), torch.bfloat16),
+    (dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16, dynamic="local"), (1, 32, 256), torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype", DYN, ids=[f"{c[0]['strategy']}-{i}" for i, c in enumerate(DYN)])
+def test_dynamic_activation_quant(spec, shape, dtype, gpu):
+    from compressed_tensors_amd.quantization import (
+        compute_dynamic_scales_and_zp, fake_quantize, generate_gparam,
+    )
+
+    announce("dynamic", spec, shape, dtype)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(shape, generator=g)
+    x[..., 3] *= 50
+    x = x.to(dtype)
+    gs = o_gs = None
+    if args.strategy == "tensor_group":
+        mn, mx = torch.aminmax(x)
+        o_gs = oq.generate_gparam(mn.reshape(1), mx.reshape(1))
+        gs = o_gs.to(gpu)
+    o_scale, o_zp = oq.compute_dynamic_scales_and_zp(x, oargs, global_scale=o_gs)
+    scale, zp = compute_dynamic_scales_and_zp(x.to(gpu), args, None, global_scale=gs)
+    assert_bit_equal(scale, o_scale, "dynamic scale")
+    assert_bit_equal(zp, o_zp, "dynamic zp")
+    out = fake_quantize(x.to(gpu), scale, zp, args, global_scale=gs)
+    assert_bit_equal(out, oq.fake_quantize(x, o_scale, o_zp, oargs, global_scale=o_gs), "dynamic qdq")
+
+
+def test_attn_head_and_errors(gpu):
+    from compressed_tensors_amd.quantization import QuantizationArgs, fake_quantize, quantize
+
+    announce("attn_head")
+    args = QuantizationArgs(num_bits=8, type="float", strategy="attn_head")
+    oargs = oq._Args(num_bits=8, type="float", strategy="attn_head")
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(2, 4, 6, 16, generator=g).bfloat16()
+    scale = (x.float().abs().amax(dim=(0, 2, 3), keepdim=False) / 448).bfloat16().reshape(4, 1, 1)
+    out = fake_quantize(x.to(gpu), scale.to(gpu), None, args)
+    assert_bit_equal(out, oq.fake_quantize(x, scale, None, oargs), "attn_head")
+    gargs = QuantizationArgs(num_bits=4, strategy="group", group_size=48)
+    with pytest.raises(ValueError, match="divisble"):
+        quantize(x.reshape(48, 16).repeat(1, 4).to(gpu), scale.reshape(-1)[:1].to(gpu), None, gargs)
+    bargs = QuantizationArgs(num_bits=8, type="float", strategy="block", block_structure=[5, 16])
+    with pytest.raises(ValueError, match="block_height"):
+        quantize(x.reshape(48, 16).to(gpu), torch.ones(9, 1, dtype=torch.bfloat16, device=gpu), None, bargs)
+    with pytest.raises(NotImplementedError):
+        quantize(x.to(gpu), scale.to(gpu), None, QuantizationArgs(num_bits=6, type="float", strategy="tensor"))
+
+
+def test_large_w4a16_properties(gpu):
+    """BASELINE-sized weight: sampled-row parity plus size-independent properties"""
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, dequantize, observe_weight_qparams, quantize,
+    )
+
+    announce("large w4a16")
+    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    oargs = oq._Args(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn(4096, 4096, generator=g) * 0.02).bfloat16()
+    wg = w.to(gpu)
+    scale, zp = observe_weight_qparams(wg, args)
+    q = quantize(wg, scale, zp, args, dtype=torch.int8)
+    dq = dequantize(q, scale, zp)
+    rows = torch.arange(0, 4096, 97)
+    o_scale, o_zp = oq.observe_weight(w[rows], oargs)
+    assert_bit_equal(scale[rows.to(gpu)], o_scale, "scale rows")
+    want_q = oq.quantize(w[rows], o_scale, o_zp, oargs, dtype=torch.int8)
+    assert_bit_equal(q[rows.to(gpu)], want_q, "q rows")
+    assert_bit_equal(dq[rows.to(gpu)], oq.dequantize(want_q, o_scale, o_zp), "dq rows")
+    # idempotence: quantizing the dequantized weight with the same scales gives the same codes
+    assert torch.equal(quantize(dq, scale, zp, args, dtype=torch.int8), q)
+    assert int(q.min()) >= -8 and int(q.max()) <= 7
+    # |w - dq| <= scale/2 plus the bf16 roundings of w/scale and q*scale (each
+    # below 2^-8 of 8 code steps) wherever no clamping happened
+    err = (wg.float() - dq.float()).abs()
+    bound = scale.float().repeat_interleave(128, dim=1) * 0.57 + 1e-12
+    assert bool(((err <= bound) | (q == 7) | (q == -8)).all())

@@ -1,0 +1,179 @@
+"""GPU parity: bitmask packing, sparse-bitmask and sparse-24-bitmask vs the oracle."""
+import pytest
+import torch
+
+from gpu_util import announce, assert_bit_equal
+from oracle import quant as oq
+from oracle import sparse as osp
+
+pytestmark = pytest.mark.gpu
+FP8 = torch.float8_e4m3fn
+
+
+@pytest.mark.parametrize("shape", [(1, 1), (3, 7), (4, 8), (5, 17), (64, 4096), (2, 3, 20)])
+def test_pack_unpack_bitmasks(shape, gpu):
+    from compressed_tensors_amd.utils import pack_bitmasks, unpack_bitmasks
+
+    announce("bitmasks", shape)
+    g = torch.Generator().manual_seed(sum(shape))
+    mask = torch.rand(shape, generator=g) > 0.5
+    packed = pack_bitmasks(mask.to(gpu))
+    assert_bit_equal(packed, osp.pack_bitmasks(mask), "pack_bitmasks")
+    assert_bit_equal(unpack_bitmasks(packed, list(shape)), mask, "unpack_bitmasks")
+
+
+def _sparse_tensor(shape, dtype, sparsity, seed):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(shape, generator=g) * 0.02
+    x[torch.rand(shape, generator=g) < sparsity] = 0
+    if dtype == FP8:
+        x = (x * 1000).to(FP8)
+    else:
+        x = x.to(dtype)
+    if x.numel() > 4:
+        flat = x.view(torch.uint8 if dtype == FP8 else dtype).view(-1)
+        if dtype == FP8:
+            flat[1] = 0x80  # -0.0
+            flat[2] = 0x7F  # NaN counts as non-zero
+        else:
+            flat[1] = -0.0
+            flat[2] = float("nan")
+    return x
+
+
+BM = [
+    ((2, 10), torch.float32, 0.5), ((16, 50), torch.bfloat16, 0.9), ((7, 64), torch.float16, 0.0),
+    ((3, 9), torch.bfloat16, 1.0), ((33, 2050), torch.bfloat16, 0.5), ((64, 4096), torch.bfloat16, 0.5),
+    ((9, 300), FP8, 0.6), ((5, 100), torch.int8, 0.7), ((300, 24), torch.bfloat16, 0.3),
+]
+
+
+@pytest.mark.parametrize("shape,dtype,sparsity", BM, ids=[f"bm{i}" for i in range(len(BM))])
+def test_bitmask_compress_decompress(shape, dtype, sparsity, gpu):
+    from compressed_tensors_amd.compressors import (
+        BaseCompressor, BitmaskTensor, bitmask_compress, bitmask_decompress,
+    )
+
+    announce("sparse-bitmask", shape, dtype, sparsity)
+    if dtype == torch.int8:
+        g = torch.Generator().manual_seed(3)
+        x = torch.randint(-128, 128, shape, generator=g, dtype=torch.int8)
+        x[torch.rand(shape, generator=g) < sparsity] = 0
+    else:
+        x = _sparse_tensor(shape, dtype, sparsity, seed=shape[1])
+    values, bitmask, row_offsets = bitmask_compress(x.to(gpu))
+    o_values, o_bitmask, o_offsets = osp.bitmask_compress(x)
+    assert_bit_equal(values, o_values, "values")
+    assert_bit_equal(bitmask, o_bitmask, "bitmask")
+    assert_bit_equal(row_offsets, o_offsets, "row_offsets")
+    dense = bitmask_decompress(o_values.to(gpu), o_bitmask.to(gpu), list(shape))
+    assert_bit_equal(dense, osp.bitmask_decompress(o_values, o_bitmask, list(shape)), "decompress")
+    comp = BaseCompressor.load_from_registry("sparse-bitmask")
+    out = comp.compress_weight("layer", x.to(gpu))
+    assert set(out) == {"layer.shape", "layer.compressed", "layer.bitmask", "layer.row_offsets"}
+    assert out["layer.shape"].tolist() == list(shape) and out["layer.shape"].dtype == torch.int64
+    back = comp.decompress_weight({k.split(".", 1)[1]: v for k, v in out.items()})
+    want = osp.bitmask_decompress(o_values, o_bitmask, list(shape))
+    assert_bit_equal(back, want, "compressor round trip")
+    assert BitmaskTensor.from_dense(x.to(gpu)).curr_memory_size_bytes() == (
+        o_values.numel() * o_values.element_size() + o_bitmask.numel() + 8 * shape[0])
+
+
+def test_bitmask_empty_and_state_dict(gpu):
+    from compressed_tensors_amd.compressors import BaseCompressor, bitmask_compress
+
+    announce("sparse-bitmask edge")
+    z = torch.zeros(4, 16, dtype=torch.bfloat16, device=gpu)
+    values, bitmask, row_offsets = bitmask_compress(z)
+    assert values.numel() == 0 and int(bitmask.sum()) == 0 and row_offsets.tolist() == [0, 0, 0, 0]
+    comp = BaseCompressor.load_from_registry("sparse-bitmask")
+    g = torch.Generator().manual_seed(8)
+    w = torch.randn(8, 24, generator=g).bfloat16()
+    w[w.abs() < 0.7] = 0
+    state = {"a.weight": w.to(gpu), "a.bias": torch.ones(8, device=gpu), "b.weight": w.t().contiguous().to(gpu)}
+    out = comp.compress(state, compression_targets={"a"})
+    assert set(out) == {"a.shape", "a.compressed", "a.bitmask", "a.row_offsets", "a.bias", "b.weight"}
+    restored = dict(comp.decompress(out))
+    assert_bit_equal(restored["a.weight"], w, "state-dict round trip")
+    assert "a.bias" in restored and "b.weight" in restored
+
+
+def _prune24(x):
+    keep = osp.get_24_bytemasks(x)
+    return torch.where(keep, x, torch.zeros_like(x))
+
+
+S24 = [((8, 16), torch.bfloat16), ((64, 4096), torch.bfloat16), ((33, 40), torch.float16),
+       ((16, 64), torch.float32), ((32, 256), FP8), ((12, 32), torch.int8), ((6, 10), torch.bfloat16),
+       ((3, 12), torch.bfloat16)]
+
+
+@pytest.mark.parametrize("shape,dtype", S24, ids=[f"s24-{i}" for i in range(len(S24))])
+def test_sparse24(shape, dtype, gpu):
+    from compressed_tensors_amd.compressors import (
+        BaseCompressor, get_24_bytemasks, sparse24_bitmask_compress, sparse24_bitmask_decompress,
+    )
+
+    announce("sparse-24", shape, dtype)
+    g = torch.Generator().manual_seed(shape[0] * 7 + shape[1])
+    if dtype == FP8:
+        base = (torch.randn(shape, generator=g) * 0.02).bfloat16()
+        base = _prune24(base)
+        scale = (base.float().abs().amax(-1, keepdim=True) / 448).bfloat16()
+        args = oq._Args(num_bits=8, type="float", strategy="channel")
+        x = oq.quantize(base, scale, None, args, dtype=FP8)  # many groups with < 2 non-zeros, -0.0 codes
+    elif dtype == torch.int8:
+        x = torch.randint(-128, 128, shape, generator=g, dtype=torch.int8)
+        x[torch.rand(shape, generator=g) < 0.5] = 0
+    else:
+        x = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+        x[torch.rand(shape, generator=g) < 0.4] = 0  # ties between zeros
+        x.view(-1)[0] = float("nan")
+    mask = get_24_bytemasks(x.to(gpu))
+    assert_bit_equal(mask, osp.get_24_bytemasks(x), "24 mask")
+    if (shape[1] % 2) == 0:
+        values, bitmask = sparse24_bitmask_compress(x.to(gpu))
+        o_values, o_bitmask = osp.sparse24_bitmask_compress(x)
+        assert_bit_equal(values, o_values, "24 values")
+        assert_bit_equal(bitmask, o_bitmask, "24 bitmask")
+        dense = sparse24_bitmask_decompress(values, bitmask, torch.Size(shape))
+        assert_bit_equal(dense, osp.sparse24_bitmask_decompress(o_values, o_bitmask, shape), "24 decompress")
+        comp = BaseCompressor.load_from_registry("sparse-24-bitmask")
+        out = comp.compress_weight("l.weight", x.to(gpu))
+        assert set(out) == {"l.shape", "l.compressed", "l.bitmask"}
+        assert tuple(out["l.shape"].shape) == (2, 1)
+        back = comp.decompress_weight({k.split(".", 1)[1]: v for k, v in out.items()})
+        assert_bit_equal(back, osp.sparse24_bitmask_decompress(o_values, o_bitmask, shape), "24 round trip")
+
+
+def test_sparse24_errors(gpu):
+    from compressed_tensors_amd.compressors import get_24_bytemasks, sparse24_bitmask_compress
+
+    with pytest.raises(ValueError, match="multiple of 4"):
+        get_24_bytemasks(torch.zeros(3, 5, dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(AssertionError, match="2D"):
+        sparse24_bitmask_compress(torch.zeros(2, 2, 4, dtype=torch.bfloat16, device=gpu))
+    with pytest.raises(AssertionError, match="2:4"):
+        sparse24_bitmask_compress(torch.zeros(4, 8, dtype=torch.bfloat16, device=gpu), "unstructured")
+
+
+def test_large_bitmask_roundtrip_properties(gpu):
+    """BASELINE-sized (8192 x 8192, 50 % magnitude pruned): sampled parity and a lossless round trip"""
+    from compressed_tensors_amd.compressors import bitmask_compress, bitmask_decompress
+
+    announce("large bitmask")
+    g = torch.Generator().manual_seed(0)
+    w = (torch.randn(8192, 8192, generator=g) * 0.02).bfloat16()
+    thr = w.float().abs().flatten().kthvalue(w.numel() // 2).values
+    w[w.float().abs() <= thr] = 0
+    wg = w.to(gpu)
+    values, bitmask, row_offsets = bitmask_compress(wg)
+    nnz_rows = (w != 0).sum(-1)
+    assert_bit_equal(row_offsets, torch.cumsum(nnz_rows, 0) - nnz_rows, "row offsets")
+    assert values.numel() == int(nnz_rows.sum())
+    rows = [0, 1, 4097, 8191]
+    for r in rows:
+        lo = int(row_offsets[r])
+        assert_bit_equal(values[lo: lo + int(nnz_rows[r])], w[r][w[r] != 0], f"values row {r}")
+    assert_bit_equal(bitmask[:64], osp.pack_bitmasks(w[:64] != 0), "bitmask head")
+    assert torch.equal(bitmask_decompress(values, bitmask, list(w.shape)), wg)
