@@ -126,7 +126,10 @@ def main():
         scale, zp = observe_weight_qparams(w, args)
         entries.append(dict(name=name, weight=w, scale=scale, zero_point=zp,
                             quantization_args=args))
-    batch = PackedWeightBatch(entries)
+    # The compress side sees the (all-zero, int8) zero points the observer emits, as the
+    # reference's state-dict loop passes them on; the decompress side does not, because a
+    # symmetric scheme's zero points are not part of the compressed state dict.
+    batch = PackedWeightBatch(entries, decompress_zero_points=False)
     per_dir, n_elems = algorithmic_bytes(shapes)
     torch.cuda.synchronize()
 

@@ -222,9 +222,11 @@ class PackedWeightBatch:
     kernels, so a serving or benchmarking loop can call them repeatedly.
     """
 
-    def __init__(self, entries, device=None):
+    def __init__(self, entries, device=None, decompress_zero_points=None):
         """entries: list of dicts with keys weight, scale, quantization_args and
-        optionally zero_point, g_idx (tensors on the GPU, or moved there)."""
+        optionally zero_point, g_idx (tensors on the GPU, or moved there).
+        decompress_zero_points: whether decompression subtracts the zero points;
+        default = only for asymmetric schemes (symmetric ones do not store any)."""
         self.n = len(entries)
         self.names = [e.get("name", str(i)) for i, e in enumerate(entries)]
         self._keep = []
@@ -248,7 +250,9 @@ class PackedWeightBatch:
             dense = torch.empty((rows, cols), dtype=scale.dtype, device=w.device)
             cplan = build_qparams(w, scale, zp, args, g_idx, None)
             dq_args = infer_dequant_args(_ShapeOnly(w.shape, torch.int8), scale)
-            dplan = build_qparams(_ShapeOnly(w.shape, torch.int8), scale, zp, dq_args, g_idx, None)
+            use_zp = (not args.symmetric) if decompress_zero_points is None else decompress_zero_points
+            dplan = build_qparams(_ShapeOnly(w.shape, torch.int8), scale, zp if use_zp else None,
+                                  dq_args, g_idx, None)
             dplan.qp.qtype, dplan.qp.num_bits = _lib.QTYPE_INT, args.num_bits
             self._keep += [cplan, dplan]
             cj, dj = self._cjobs[i], self._djobs[i]

@@ -91,12 +91,19 @@ __device__ __forceinline__ int fp4_bucket(float a) {
   return c;
 }
 
-__device__ __forceinline__ float fp4_code_to_f32(int code3) {
-  // 0,.5,1,1.5,2,3,4,6 : exponent = code>>1 (bias 1), mantissa = code&1
-  const uint32_t e = ((uint32_t)code3 >> 1) & 3u, m = (uint32_t)code3 & 1u;
-  const uint32_t normal = ((e + 126u) << 23) | (m << 22);
-  const uint32_t sub = m ? 0x3F000000u : 0u;
-  return u2f(e ? normal : sub);
+// fp32 bit pattern of the e2m1 magnitude {0,.5,1,1.5,2,3,4,6}[code3]: from 1.0 on
+// the patterns are consecutive multiples of 2^22 starting at 254 << 22.
+__device__ __forceinline__ uint32_t fp4_mag_bits(int code3) {
+  const uint32_t c = (uint32_t)code3 & 7u;
+  const uint32_t k = c + 252u - (c == 1u ? 1u : 0u);
+  return c ? (k << 22) : 0u;
+}
+
+__device__ __forceinline__ float fp4_code_to_f32(int code3) { return u2f(fp4_mag_bits(code3)); }
+
+// signed value of a 4-bit code (bit 3 = sign), assembled in the integer domain
+__device__ __forceinline__ float fp4_decode(int code) {
+  return u2f(fp4_mag_bits(code) | (((uint32_t)code & 8u) << 28));
 }
 
 // ---------------------------------------------------------------- dtype-generic scalar access

@@ -43,11 +43,6 @@ __device__ __forceinline__ int fp4_nearest_code_rt(float x, int xdt) {
   return fp4_nearest_code<CTMI_F32>(x);
 }
 
-__device__ __forceinline__ float fp4_decode(int code) {
-  const float m = fp4_code_to_f32(code & 7);
-  return (code & 8) ? -m : m;
-}
-
 // ------------------------------------------------------------------ standalone pack / unpack
 // one thread per 8 elements (cols % 8 == 0) -> one 32-bit store
 template <typename XT>
