@@ -11,6 +11,7 @@
 #include "ctmi_device.h"
 #include "ctmi_host.h"
 #include "quant_core.h"
+#include "quant_fast.h"
 #include "vec_geom.h"
 
 namespace ctmi {
@@ -199,10 +200,7 @@ pq_compress_vec_kernel(const typename XT::raw* __restrict__ x,
                        const typename ST::raw* __restrict__ scale,
                        const int8_t* __restrict__ zp, int32_t* __restrict__ out, VecGeom g,
                        float qmin, float qmax) {
-  constexpr int CT = Promote<XT::id, ST::id>::value;
   constexpr int W = BITS / 4;  // output words per item
-  constexpr int PF = 32 / BITS;
-  constexpr int OFF = 1 << (BITS - 1);
   using XV = Vec<typename XT::raw, 8>;
   const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
   for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
@@ -223,20 +221,8 @@ pq_compress_vec_kernel(const typename XT::raw* __restrict__ x,
     for (int k = 0; k < kU; ++k) {
       const uint32_t v = v0 + k * 256;
       if (v < g.nvec) {
-        Vec<int32_t, W> o;
-#pragma unroll
-        for (int w = 0; w < W; ++w) {
-          uint32_t acc = 0;
-#pragma unroll
-          for (int i = 0; i < PF; ++i) {
-            float t = round_ct<CT>(XT::to_f32(xv[k].v[w * PF + i]) / sv[k]);
-            if (HAS_ZP) t = round_ct<CT>(t + zv[k]);
-            t = rintf(clamp_nan(t, qmin, qmax));
-            acc |= ((uint32_t)(f32_to_int(t) + OFF) & ((1u << BITS) - 1u)) << (BITS * i);
-          }
-          o.v[w] = (int32_t)acc;
-        }
-        stg<int32_t, W>(out + (size_t)v * W, o);
+        stg<int32_t, W>(out + (size_t)v * W,
+                        quant_pack8<XT, ST, BITS, HAS_ZP>(xv[k], sv[k], zv[k], qmin, qmax));
       }
     }
   }
@@ -248,11 +234,7 @@ pq_decompress_vec_kernel(const int32_t* __restrict__ packed,
                          const typename ST::raw* __restrict__ scale,
                          const int8_t* __restrict__ zp, typename ST::raw* __restrict__ out,
                          VecGeom g) {
-  constexpr int DT = ST::id;
   constexpr int W = BITS / 4;
-  constexpr int PF = 32 / BITS;
-  constexpr int OFF = 1 << (BITS - 1);
-  constexpr uint32_t MASK = (1u << BITS) - 1u;
   const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
   for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
     const uint32_t v0 = chunk * (256 * kU) + threadIdx.x;
@@ -272,16 +254,8 @@ pq_decompress_vec_kernel(const int32_t* __restrict__ packed,
     for (int k = 0; k < kU; ++k) {
       const uint32_t v = v0 + k * 256;
       if (v < g.nvec) {
-        Vec<typename ST::raw, 8> o;
-#pragma unroll
-        for (int w = 0; w < W; ++w)
-#pragma unroll
-          for (int i = 0; i < PF; ++i) {
-            float t = (float)((int)(((uint32_t)pv[k].v[w] >> (BITS * i)) & MASK) - OFF);
-            if (HAS_ZP) t = round_ct<DT>(t - zv[k]);
-            o.v[w * PF + i] = ST::from_f32(t * sv[k]);
-          }
-        stg<typename ST::raw, 8>(out + (size_t)v * 8, o);
+        stg<typename ST::raw, 8>(out + (size_t)v * 8,
+                                 unpack_dequant8<ST, BITS, HAS_ZP>(pv[k], sv[k], zv[k]));
       }
     }
   }
