@@ -14,7 +14,10 @@ from typing import Optional
 
 import torch
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "libctmi.so"
+import os
+
+# CTMI_LIB points at an alternative build of the library (kernel tuning experiments)
+LIB_PATH = Path(os.environ.get("CTMI_LIB") or Path(__file__).resolve().parent / "lib" / "libctmi.so")
 
 CTMI_OK = 0
 CTMI_ERR_VALUE = -1

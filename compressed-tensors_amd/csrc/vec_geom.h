@@ -32,9 +32,15 @@ struct VecGeom {
   uint32_t nvec;      // total items
   uint32_t s_cols;
   uint32_t row_scaled;  // 1: scale row = tensor row; 0: a single scale row
+  // When every row has its own scales and scale blocks tile the rows exactly,
+  // scales are numbered like the items: index = item / vpb, a shift if vpb is a
+  // power of two.  mode 0: shift, 1: one division, 2: row/column split.
+  uint32_t mode, shift;
 };
 
 __device__ __forceinline__ uint32_t scale_index(uint32_t v, const VecGeom& g) {
+  if (g.mode == 0) return v >> g.shift;
+  if (g.mode == 1) return fdiv(v, g.vpb);
   const uint32_t r = fdiv(v, g.vpr);
   const uint32_t cv = v - r * g.vpr.d;
   return (g.row_scaled ? r * g.s_cols : 0u) + fdiv(cv, g.vpb);
@@ -71,6 +77,17 @@ static inline bool vec_geometry(const ctmi_qparams* qp, int64_t rows, int64_t co
   g->nvec = (uint32_t)(rows * cols / 8);
   g->s_cols = (uint32_t)qp->s_cols;
   g->row_scaled = row_scaled ? 1u : 0u;
+  g->mode = 2;
+  g->shift = 0;
+  if (row_scaled && g->vpr.d % g->vpb.d == 0 && qp->s_cols == cols / qp->blk_cols) {
+    const uint32_t d = g->vpb.d;
+    if ((d & (d - 1)) == 0) {
+      g->mode = 0;
+      while ((1u << g->shift) < d) ++g->shift;
+    } else {
+      g->mode = 1;
+    }
+  }
   return true;
 }
 

@@ -128,8 +128,8 @@ typedef struct ctmi_weight_job {
 /* A27.  The per-weight loop of BaseQuantizationCompressor.compress /
  * decompress_from_state_dict (compressors/quantized_compressors/base.py:91-125,
  * 213-230) for the pack-quantized format: n fused launches from one call.
- * Jobs are validated and enqueued in order; on the first invalid job the call
- * returns its error (earlier jobs stay enqueued). */
+ * Every job is validated before anything is enqueued; weights that share a
+ * dtype / bit-width combination are chained into common launches. */
 int ctmi_pack_quantized_compress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
 int ctmi_pack_quantized_decompress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
 
