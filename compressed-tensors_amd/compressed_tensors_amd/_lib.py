@@ -146,6 +146,16 @@ SIGNATURES = {
         [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     ),
     "ctmi_topk24_lut": (None, [c_void_p]),
+    "ctmi_hadamard_supported": (c_int32, [c_int32, c_int32, c_int32]),
+    "ctmi_hadamard_apply": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_void_p],
+    ),
+    "ctmi_block_matmul": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p],
+    ),
     "ctmi_calculate_qparams": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int32, c_int64, c_int32, c_int32, c_int32, c_void_p,

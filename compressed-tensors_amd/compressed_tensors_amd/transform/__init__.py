@@ -1,0 +1,1 @@
+from .hadamard import *  # noqa: F401,F403

@@ -1,0 +1,356 @@
+// Hadamard transform apply on the matrix cores.
+//
+//   apply_transform_weight / _multihead_matmul   transform/utils/matrix.py:65-171
+//   HadamardTransform.forward                    transform/factory/hadamard.py:104-121
+//
+// The reference multiplies by an explicit n x n matrix (fp32 online, fp64 when
+// fused into weights) and divides by sqrt(n).  Here the matrix is taken in
+// factored form  W = diag(s_in) * (Ma (x) Mb) * diag(s_out)  with Ma (a x a) and
+// Mb (b x b) small +-1 matrices (Sylvester blocks for Hadamard transforms; a = 1
+// for block sizes up to 128).  Viewing each length-n run of the last dimension
+// as an a x b matrix X,
+//        x * (Ma (x) Mb)  =  vec( Ma^T * X * Mb ),
+// two small dense products that run on bf16 MFMA (v_mfma_f32_16x16x32_bf16)
+// out of LDS.  +-1 is exact in bf16 and inputs are split into bf16 terms that
+// sum to the input exactly (1 term for bf16, 2 for fp16, 3 for fp32), so stage
+// 1 accumulates exact products in fp32.  The fp32 intermediate is split three
+// ways (24 significant bits) before stage 2.  Results differ from the
+// reference only by fp32 summation order: within one ulp of the output dtype.
+//
+// Tile = S sub-rows of b elements = one contiguous span of memory, staged
+// through LDS in both directions so that every HBM access is a full 16-byte
+// lane access on consecutive addresses.
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+
+namespace ctmi {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kHadThreads = 256;
+constexpr int kHadWaves = kHadThreads / kWave;
+
+struct HadArgs {
+  const void* x;
+  void* out;
+  const uint16_t* mbt;   // Mb^T, [b][b] bf16
+  const uint16_t* mat;   // Ma^T, [a][a] bf16 (a > 1)
+  const float* s_in;     // [n] or NULL
+  const float* s_out;    // [n] or NULL
+  int64_t n_sub;         // number of sub-rows (numel / b)
+  float sqrt_n;
+};
+
+template <int A, int B, typename IO>
+struct HadCfg {
+  static constexpr int NS = IO::id == CTMI_BF16 ? 1 : (IO::id == CTMI_F16 ? 2 : 3);
+  static constexpr int S = A > 64 ? A : 64;  // sub-rows per tile, a multiple of A
+  static constexpr int XP = B + 8;           // padded row pitch (elements): conflict-free 16-byte reads
+  static constexpr int TP = S + 8;
+  static constexpr int AP = A + 8;
+  static constexpr int OP = B + 16 / (int)sizeof(typename IO::raw);
+  static constexpr size_t xs_bytes = (size_t)NS * S * XP * 2;
+  static constexpr size_t mbt_bytes = (size_t)B * XP * 2;
+  static constexpr size_t mat_bytes = A > 1 ? (size_t)A * AP * 2 : 0;
+  static constexpr size_t tt_bytes = A > 1 ? (size_t)3 * B * TP * 2 : 0;
+  static constexpr size_t os_bytes = (size_t)S * OP * sizeof(typename IO::raw);
+  static constexpr size_t lds_bytes = xs_bytes + mbt_bytes + mat_bytes + tt_bytes + os_bytes;
+};
+
+// split an fp32 value into bf16 terms that add up to it (exactly when the
+// value has at most 8 * NS significant bits)
+template <int NS>
+__device__ __forceinline__ void split_bf16(float v, uint16_t* parts) {
+  float rest = v;
+#pragma unroll
+  for (int s = 0; s < NS; ++s) {
+    const uint16_t h = f32_to_bf16(rest);
+    parts[s] = h;
+    rest -= bf16_to_f32(h);
+  }
+}
+
+template <int A, int B, typename IO>
+__global__ void __launch_bounds__(kHadThreads) hadamard_mfma_kernel(HadArgs a) {
+  using C = HadCfg<A, B, IO>;
+  using R = typename IO::raw;
+  constexpr int NS = C::NS, S = C::S, XP = C::XP, TP = C::TP, AP = C::AP, OP = C::OP;
+  constexpr int N = A * B;
+  constexpr int VE = 16 / (int)sizeof(R);  // elements per 16-byte global access
+  extern __shared__ __align__(16) unsigned char lds[];
+  uint16_t* Xs = reinterpret_cast<uint16_t*>(lds);
+  uint16_t* Mbt = reinterpret_cast<uint16_t*>(lds + C::xs_bytes);
+  uint16_t* Mat = reinterpret_cast<uint16_t*>(lds + C::xs_bytes + C::mbt_bytes);
+  uint16_t* Tt = reinterpret_cast<uint16_t*>(lds + C::xs_bytes + C::mbt_bytes + C::mat_bytes);
+  R* Os = reinterpret_cast<R*>(lds + C::xs_bytes + C::mbt_bytes + C::mat_bytes + C::tt_bytes);
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int l16 = lane & 15, lq = lane >> 4;
+
+  // ---- the small matrices, once per workgroup
+  for (int i = tid; i < B * B / 8; i += kHadThreads) {
+    const int r = (i * 8) / B, c = (i * 8) % B;
+    *reinterpret_cast<uint4*>(&Mbt[r * XP + c]) = *reinterpret_cast<const uint4*>(&a.mbt[r * B + c]);
+  }
+  if constexpr (A > 1) {
+    for (int i = tid; i < A * A / 8; i += kHadThreads) {
+      const int r = (i * 8) / A, c = (i * 8) % A;
+      *reinterpret_cast<uint4*>(&Mat[r * AP + c]) = *reinterpret_cast<const uint4*>(&a.mat[r * A + c]);
+    }
+  }
+
+  const int64_t n_tiles = (a.n_sub + S - 1) / S;
+  for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    const int64_t sub0 = tile * S;
+    const R* src = reinterpret_cast<const R*>(a.x) + sub0 * B;
+    R* dst = reinterpret_cast<R*>(a.out) + sub0 * B;
+    const int64_t live = (a.n_sub - sub0 < S ? a.n_sub - sub0 : S) * B;  // elements in this tile
+
+    __syncthreads();  // previous tile fully written out before Xs / Os are reused
+    // ---- global -> LDS, with the input signs and the bf16 split
+    for (int e = tid * VE; e < S * B; e += kHadThreads * VE) {
+      Vec<R, VE> v;
+      if (e < live) {
+        v = ldg_nt<R, VE>(src + e);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VE; ++j) v.v[j] = IO::from_f32(0.0f);
+      }
+      const int row = e / B, col = e % B;
+      const int pos = e % N;  // a tile starts on a multiple of N elements
+#pragma unroll
+      for (int j = 0; j < VE; ++j) {
+        float f = IO::to_f32(v.v[j]);
+        if (a.s_in) f *= a.s_in[pos + j];
+        uint16_t parts[NS];
+        split_bf16<NS>(f, parts);
+#pragma unroll
+        for (int s = 0; s < NS; ++s) Xs[(s * S + row) * XP + col + j] = parts[s];
+      }
+    }
+    __syncthreads();
+
+    // ---- stage 1: T = X * Mb  (per 16 x 16 output tile: K = B in steps of 32)
+    for (int mt = wave; mt < S / 16; mt += kHadWaves) {
+#pragma unroll
+      for (int nt = 0; nt < B / 16; ++nt) {
+        f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < B / 32; ++ks) {
+          const bf16x8_t hf =
+              *reinterpret_cast<const bf16x8_t*>(&Mbt[(nt * 16 + l16) * XP + ks * 32 + 8 * lq]);
+#pragma unroll
+          for (int s = 0; s < NS; ++s) {
+            const bf16x8_t xf = *reinterpret_cast<const bf16x8_t*>(
+                &Xs[(s * S + mt * 16 + l16) * XP + ks * 32 + 8 * lq]);
+            if constexpr (A == 1) {
+              // D^T = Mb^T * X^T: lane holds 4 neighbouring output columns of one sub-row
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(hf, xf, acc, 0, 0, 0);
+            } else {
+              // D = X * Mb: lane holds 4 neighbouring sub-rows of one column
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf, hf, acc, 0, 0, 0);
+            }
+          }
+        }
+        if constexpr (A == 1) {
+          const int row = mt * 16 + l16, col = nt * 16 + 4 * lq;
+          Vec<R, 4> o;
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            float v = acc[r] / a.sqrt_n;
+            if (a.s_out) v *= a.s_out[col + r];
+            o.v[r] = IO::from_f32(v);
+          }
+          *reinterpret_cast<Vec<R, 4>*>(&Os[row * OP + col]) = o;
+        } else {
+          const int col = nt * 16 + l16, row = mt * 16 + 4 * lq;
+          Vec<uint16_t, 4> p[3];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            uint16_t parts[3];
+            split_bf16<3>(acc[r], parts);
+            p[0].v[r] = parts[0];
+            p[1].v[r] = parts[1];
+            p[2].v[r] = parts[2];
+          }
+#pragma unroll
+          for (int s = 0; s < 3; ++s)
+            *reinterpret_cast<Vec<uint16_t, 4>*>(&Tt[(s * B + col) * TP + row]) = p[s];
+        }
+      }
+    }
+
+    if constexpr (A > 1) {
+      __syncthreads();
+      // ---- stage 2: Y = Ma^T * T per data row; computed as Y^T = T^T * Ma so that a
+      // lane ends up with 4 neighbouring columns of one output sub-row
+      constexpr int MT = B / 16, NT = A / 16, PER_ROW = MT * NT;
+      for (int q = wave; q < (S / A) * PER_ROW; q += kHadWaves) {
+        const int d = q / PER_ROW, mt = (q % PER_ROW) / NT, nt = q % NT;
+        f32x4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < A / 32; ++ks) {
+          const bf16x8_t mf =
+              *reinterpret_cast<const bf16x8_t*>(&Mat[(nt * 16 + l16) * AP + ks * 32 + 8 * lq]);
+#pragma unroll
+          for (int s = 0; s < 3; ++s) {
+            const bf16x8_t tf = *reinterpret_cast<const bf16x8_t*>(
+                &Tt[(s * B + mt * 16 + l16) * TP + d * A + ks * 32 + 8 * lq]);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf, mf, acc, 0, 0, 0);
+          }
+        }
+        const int i = nt * 16 + l16;           // output sub-row inside the data row
+        const int col = mt * 16 + 4 * lq;
+        Vec<R, 4> o;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = acc[r] / a.sqrt_n;
+          if (a.s_out) v *= a.s_out[i * B + col + r];
+          o.v[r] = IO::from_f32(v);
+        }
+        *reinterpret_cast<Vec<R, 4>*>(&Os[(d * A + i) * OP + col]) = o;
+      }
+    }
+    __syncthreads();
+
+    // ---- LDS -> global
+    for (int e = tid * VE; e < S * B; e += kHadThreads * VE) {
+      if (e < live) {
+        const int row = e / B, col = e % B;
+        stg_nt<R, VE>(dst + e, *reinterpret_cast<const Vec<R, VE>*>(&Os[row * OP + col]));
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------- any small dense matrix (VALU)
+// y[r, g*h + j] = sum_k x[r, g*h + k] * w[k, j] / sqrt_n for an explicit fp32
+// h x h matrix: covers sizes and matrices the MFMA path does not (h < 32,
+// non-Kronecker sizes, matrices that are not +-1).  One workgroup per h-chunk.
+template <typename IO>
+__global__ void __launch_bounds__(256)
+block_matmul_kernel(const typename IO::raw* __restrict__ x, const float* __restrict__ w,
+                    typename IO::raw* __restrict__ out, int64_t n_chunks, int h, float sqrt_n) {
+  extern __shared__ float xrow[];
+  for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+    __syncthreads();
+    for (int k = threadIdx.x; k < h; k += blockDim.x) xrow[k] = IO::to_f32(x[c * h + k]);
+    __syncthreads();
+    for (int j = threadIdx.x; j < h; j += blockDim.x) {
+      float acc = 0.0f;
+      for (int k = 0; k < h; ++k) acc = fmaf(xrow[k], w[(int64_t)k * h + j], acc);
+      out[c * h + j] = IO::from_f32(acc / sqrt_n);
+    }
+  }
+}
+
+template <int A, int B, typename IO>
+static int launch_had(const HadArgs& a, hipStream_t st) {
+  using C = HadCfg<A, B, IO>;
+  static bool configured = false;
+  auto kern = hadamard_mfma_kernel<A, B, IO>;
+  if (!configured && C::lds_bytes > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)C::lds_bytes);
+    if (e != hipSuccess)
+      return set_error(CTMI_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    configured = true;
+  }
+  const int64_t tiles = cdiv(a.n_sub, C::S);
+  const int64_t cap = 256 * 8;
+  const unsigned grid = (unsigned)(tiles < cap ? tiles : cap);
+  hipLaunchKernelGGL(kern, grid, kHadThreads, C::lds_bytes, st, a);
+  return CTMI_OK;
+}
+
+template <typename IO>
+static int dispatch_had(int a_dim, int b_dim, const HadArgs& a, hipStream_t st) {
+#define CTMI_HAD(AA, BB) \
+  if (a_dim == AA && b_dim == BB) return launch_had<AA, BB, IO>(a, st);
+  CTMI_HAD(1, 32) CTMI_HAD(1, 64) CTMI_HAD(1, 128)
+  CTMI_HAD(32, 32) CTMI_HAD(32, 64) CTMI_HAD(64, 64) CTMI_HAD(64, 128)
+#undef CTMI_HAD
+  return set_error(CTMI_ERR_UNSUPPORTED, "no MFMA kernel for the factorisation %d x %d", a_dim,
+                   b_dim);
+}
+
+}  // namespace ctmi
+
+using namespace ctmi;
+
+extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
+  const bool pair = (a_dim == 1 && (b_dim == 32 || b_dim == 64 || b_dim == 128)) ||
+                    (a_dim == 32 && (b_dim == 32 || b_dim == 64)) ||
+                    (a_dim == 64 && (b_dim == 64 || b_dim == 128));
+  if (!pair) return 0;
+  if (io_dtype == CTMI_BF16) return 1;
+  // wider inputs need 2-3 staged copies: the largest factorisation does not fit in LDS
+  if (io_dtype == CTMI_F16 || io_dtype == CTMI_F32) return !(a_dim == 64 && b_dim == 128);
+  return 0;
+}
+
+extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel,
+                                   int32_t a_dim, int32_t b_dim, const void* ma_t,
+                                   const void* mb_t, const float* sign_in, const float* sign_out,
+                                   void* stream) {
+  CTMI_REQUIRE(numel >= 0, CTMI_ERR_VALUE, "negative size");
+  CTMI_REQUIRE(a_dim >= 1 && b_dim >= 1, CTMI_ERR_VALUE, "bad factor sizes");
+  CTMI_REQUIRE(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32,
+               CTMI_ERR_UNSUPPORTED, "transforms take float16/bfloat16/float32 tensors");
+  const int64_t n = (int64_t)a_dim * b_dim;
+  CTMI_REQUIRE(numel % n == 0, CTMI_ERR_VALUE,
+               "tensor size %lld is not a multiple of the transform size %lld", (long long)numel,
+               (long long)n);
+  CTMI_REQUIRE(ctmi_hadamard_supported(a_dim, b_dim, io_dtype), CTMI_ERR_UNSUPPORTED,
+               "no MFMA kernel for the factorisation %d x %d with this dtype", a_dim, b_dim);
+  if (numel == 0) return CTMI_OK;
+  CTMI_REQUIRE(x && out && mb_t && (a_dim == 1 || ma_t), CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)mb_t % 16 == 0 &&
+                   (uintptr_t)ma_t % 16 == 0,
+               CTMI_ERR_VALUE, "tensors must be 16-byte aligned");
+  HadArgs a;
+  a.x = x;
+  a.out = out;
+  a.mbt = (const uint16_t*)mb_t;
+  a.mat = (const uint16_t*)ma_t;
+  a.s_in = sign_in;
+  a.s_out = sign_out;
+  a.n_sub = numel / b_dim;
+  a.sqrt_n = sqrtf((float)n);
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (io_dtype == CTMI_BF16) rc = dispatch_had<BF16>(a_dim, b_dim, a, st);
+  else if (io_dtype == CTMI_F16) rc = dispatch_had<F16>(a_dim, b_dim, a, st);
+  else rc = dispatch_had<F32>(a_dim, b_dim, a, st);
+  if (rc) return rc;
+  return check_launch("ctmi_hadamard_apply");
+}
+
+extern "C" int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel,
+                                 int32_t h, const float* w, void* stream) {
+  CTMI_REQUIRE(numel >= 0, CTMI_ERR_VALUE, "negative size");
+  CTMI_REQUIRE(h >= 1 && h <= 8192, CTMI_ERR_UNSUPPORTED, "block size must be in 1..8192");
+  CTMI_REQUIRE(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32,
+               CTMI_ERR_UNSUPPORTED, "transforms take float16/bfloat16/float32 tensors");
+  CTMI_REQUIRE(numel % h == 0, CTMI_ERR_VALUE,
+               "tensor size %lld is not a multiple of the transform size %d", (long long)numel, h);
+  if (numel == 0) return CTMI_OK;
+  CTMI_REQUIRE(x && out && w, CTMI_ERR_VALUE, "NULL tensor pointer");
+  const int64_t chunks = numel / h;
+  const unsigned grid = (unsigned)(chunks < 256 * 32 ? chunks : 256 * 32);
+  const float sqrt_n = sqrtf((float)h);
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = (size_t)h * sizeof(float);
+  if (io_dtype == CTMI_BF16)
+    hipLaunchKernelGGL(block_matmul_kernel<BF16>, grid, 256, lds, st, (const uint16_t*)x, w,
+                       (uint16_t*)out, chunks, h, sqrt_n);
+  else if (io_dtype == CTMI_F16)
+    hipLaunchKernelGGL(block_matmul_kernel<F16>, grid, 256, lds, st, (const uint16_t*)x, w,
+                       (uint16_t*)out, chunks, h, sqrt_n);
+  else
+    hipLaunchKernelGGL(block_matmul_kernel<F32>, grid, 256, lds, st, (const float*)x, w,
+                       (float*)out, chunks, h, sqrt_n);
+  return check_launch("ctmi_block_matmul");
+}

@@ -237,6 +237,26 @@ int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows, int64_t c
                          void* zero_point, int32_t zp_dtype, void* min_out, void* max_out,
                          void* stream);
 
+/* A24 / A25.  Hadamard transform apply (transform/utils/matrix.py:65-171,
+ * transform/factory/hadamard.py:104-121) for a matrix given in factored form
+ *     W = diag(sign_in) * (Ma (x) Mb) * diag(sign_out),      n = a_dim * b_dim:
+ * every run of n consecutive elements x of the tensor (numel % n == 0) becomes
+ *     x * W / sqrt(n)
+ * rounded to io_dtype.  ma_t / mb_t: Ma^T [a,a] and Mb^T [b,b] as bf16 (entries
+ * must be exact in bf16, e.g. +-1); ma_t is ignored when a_dim == 1.  sign_in /
+ * sign_out: fp32 [n] or NULL.  Runs on bf16 MFMA; ctmi_hadamard_supported says
+ * which (a_dim, b_dim, dtype) combinations are built. */
+int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype);
+int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t a_dim,
+                        int32_t b_dim, const void* ma_t, const void* mb_t, const float* sign_in,
+                        const float* sign_out, void* stream);
+
+/* A24 for an arbitrary explicit fp32 matrix w [h,h] (small h, or matrices that
+ * are not +-1): every run of h consecutive elements x becomes x * w / sqrt(h).
+ * fp32 accumulation on the vector ALUs. */
+int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t h,
+                      const float* w, void* stream);
+
 /* The 4096-entry keep table used by the 2:4 kernels (host copy, for tests). */
 void ctmi_topk24_lut(uint8_t* out4096);
 

@@ -1,0 +1,165 @@
+"""GPU parity: Hadamard transform apply vs the oracle (fp64 / fp32 matmul by the
+explicit matrix): within one ulp of the output dtype."""
+import pytest
+import torch
+
+from gpu_util import announce
+from oracle import hadamard as oh
+
+pytestmark = pytest.mark.gpu
+
+
+def _ulp(t: torch.Tensor) -> torch.Tensor:
+    """spacing of t's dtype at |t| (as float64)"""
+    bits = {torch.bfloat16: 8, torch.float16: 11, torch.float32: 24}[t.dtype]
+    mag = t.double().abs().clamp_min(2.0 ** (-14 if t.dtype == torch.float16 else -126))
+    return torch.exp2(torch.floor(torch.log2(mag)) - (bits - 1))
+
+
+def _assert_within_ulp(got, exact, what, ulps=1.0):
+    got = got.cpu()
+    assert got.dtype == exact.dtype and got.shape == exact.shape, what
+    err = (got.double() - exact.double()).abs()
+    if exact.dtype == torch.float32:
+        # fp32 accumulation of n terms: rtol 1e-5 of the value plus the same fraction of the
+        # largest term scale of the row (cancellation makes a pure per-value bound meaningless)
+        tol = 1e-5 * exact.double().abs() + 1e-5 * exact.double().abs().amax(-1, keepdim=True)
+    else:
+        tol = ulps * _ulp(exact)
+    bad = err > tol
+    assert not bool(bad.any()), f"{what}: {int(bad.sum())} elements off by more than {ulps} ulp; max ratio {(err / tol).max():.2f}"
+
+
+def _reference(weight64, value, location, inverse=False, module_type=torch.nn.Linear, perm=None):
+    """fp64 application rounded once to value.dtype: the exact answer"""
+    return oh.hadamard_forward(weight64, value, location, module_type, inverse, perm)
+
+
+SIZES = [32, 64, 128, 1024, 2048, 4096, 8192]
+
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_sylvester_apply(n, dtype, gpu):
+    from compressed_tensors_amd import _lib
+    from compressed_tensors_amd.transform import hadamard_apply, hadamard_factors
+
+    announce("hadamard_apply", n, dtype)
+    a, b = hadamard_factors(n)
+    if not _lib.load().ctmi_hadamard_supported(a, b, _lib.dtype_code(dtype)):
+        pytest.skip("factorisation not built for this dtype")
+    g = torch.Generator().manual_seed(n)
+    rows = 37 if n <= 2048 else 9
+    x = torch.randn(rows, 2 * n if n <= 1024 else n, generator=g).to(dtype)
+    q = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).double()
+    h = oh.deterministic_hadamard_matrix(n, torch.float64)
+    y = hadamard_apply(x.to(gpu), n)
+    _assert_within_ulp(y, _reference(h, x, "input"), "plain")
+    y = hadamard_apply(x.to(gpu), n, sign_in=q.float())
+    _assert_within_ulp(y, _reference(q.unsqueeze(1) * h, x, "input"), "sign_in")
+    y = hadamard_apply(x.to(gpu), n, sign_out=q.float())
+    _assert_within_ulp(y, _reference((q.unsqueeze(1) * h).T, x, "input"), "sign_out")
+
+
+def test_explicit_small_matrix(gpu):
+    from compressed_tensors_amd.transform import hadamard_apply
+
+    announce("explicit matrix 64")
+    g = torch.Generator().manual_seed(3)
+    m = (torch.randint(0, 2, (64, 64), generator=g) * 2 - 1).double()  # any +-1 matrix
+    x = torch.randn(50, 192, generator=g).bfloat16()
+    y = hadamard_apply(x.to(gpu), 64, matrix_t=m.T.contiguous())
+    _assert_within_ulp(y, _reference(m, x, "input"), "explicit")
+
+
+LOCS = [("input", False), ("input", True), ("weight_input", False), ("weight_input", True),
+        ("weight_output", False), ("weight_output", True), ("output", False)]
+
+
+@pytest.mark.parametrize("kind", ["hadamard", "random-hadamard"])
+@pytest.mark.parametrize("location,inverse", LOCS)
+def test_transform_objects(kind, location, inverse, gpu):
+    from compressed_tensors_amd.transform import (
+        TransformArgs, TransformFactory, TransformScheme,
+    )
+
+    announce("transform", kind, location, inverse)
+    scheme = TransformScheme(type=kind, apply=[], head_dim=None)
+    factory = TransformFactory.from_scheme(scheme, name="t", seed=11)
+    linear = torch.nn.Linear(256 if location != "weight_output" else 128, 128, bias=False)
+    if location in ("weight_output", "output"):
+        linear = torch.nn.Linear(64, 128, bias=False)
+    else:
+        linear = torch.nn.Linear(128, 64, bias=False)
+    args = TransformArgs(targets=["Linear"], location=location, inverse=inverse)
+    tfm = factory.create_transform(linear, args)
+    weight64 = tfm.weight.double()
+    g = torch.Generator().manual_seed(5)
+    if location in ("weight_input", "weight_output"):
+        value = (torch.randn(linear.out_features, linear.in_features, generator=g) * 0.02).bfloat16()
+    elif location == "input":
+        value = torch.randn(3, 7, 128, generator=g).bfloat16()
+    else:
+        value = torch.randn(3, 7, 128, generator=g).bfloat16()
+    got = tfm(value.to(gpu))
+    want = _reference(weight64, value, location, inverse)
+    _assert_within_ulp(got, want, f"{kind} {location} inverse={inverse}")
+
+
+def test_multihead_and_permutation(gpu):
+    from compressed_tensors_amd.transform import (
+        TransformArgs, TransformFactory, TransformScheme,
+    )
+
+    announce("transform head_dim + randomize")
+    scheme = TransformScheme(type="random-hadamard", head_dim=64, randomize=True)
+    factory = TransformFactory.from_scheme(scheme, name="t", seed=3)
+    linear = torch.nn.Linear(256, 128, bias=False)
+    g = torch.Generator().manual_seed(6)
+    for location, value in (("input", torch.randn(4, 9, 256, generator=g).bfloat16()),
+                            ("weight_input", (torch.randn(128, 256, generator=g) * 0.02).bfloat16())):
+        tfm = factory.create_transform(linear, TransformArgs(["Linear"], location))
+        assert tfm.size == 64 and tfm.perm is not None
+        want = _reference(tfm.weight.double(), value, location, perm=tfm.perm)
+        _assert_within_ulp(tfm(value.to(gpu)), want, f"multihead {location}")
+
+
+def test_transform_algebra_on_gpu(gpu):
+    """output_tfm(input_tfm(x) @ (U W V)^T) == x W^T at atol 1e-5 in fp32"""
+    from compressed_tensors_amd.transform import (
+        TransformArgs, TransformFactory, TransformScheme,
+    )
+
+    announce("transform algebra")
+    scheme = TransformScheme(type="random-hadamard")
+    fac = TransformFactory.from_scheme(scheme, name="t", seed=0)
+    lin = torch.nn.Linear(128, 64, bias=False)
+    g = torch.Generator().manual_seed(9)
+    w = torch.randn(64, 128, generator=g).to(gpu)
+    x = torch.randn(5, 128, generator=g).to(gpu)
+    t_in = fac.create_transform(lin, TransformArgs(["Linear"], "input"))
+    t_wi = fac.create_transform(lin, TransformArgs(["Linear"], "weight_input", inverse=True))
+    t_wo = fac.create_transform(lin, TransformArgs(["Linear"], "weight_output"))
+    t_out = fac.create_transform(lin, TransformArgs(["Linear"], "output", inverse=True))
+    y = t_out(t_in(x) @ t_wo(t_wi(w)).T)
+    assert torch.allclose(y, x @ w.T, atol=1e-4)
+
+
+def test_large_activation_properties(gpu):
+    """BASELINE-sized: 8192 x 4096 bf16 activations, block 128 and full 4096: sampled
+    rows against fp64, and an involution check (H H^T / n = I) on the whole tensor"""
+    from compressed_tensors_amd.transform import hadamard_apply
+
+    announce("hadamard large")
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(8192, 4096, generator=g).bfloat16()
+    xg = x.to(gpu)
+    for n in (128, 4096):
+        q = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+        y = hadamard_apply(xg, n, sign_in=q)
+        rows = torch.tensor([0, 1, 4095, 8191])
+        w = q.double().unsqueeze(1) * oh.deterministic_hadamard_matrix(n, torch.float64)
+        _assert_within_ulp(y[rows.to(gpu)], _reference(w, x[rows], "input"), f"rows n={n}")
+        back = hadamard_apply(y, n, sign_out=q)  # times W^T / sqrt(n): undoes it up to bf16 rounding
+        rel = (back.float() - xg.float()).abs().max() / xg.float().abs().max()
+        assert float(rel) < 2e-2
