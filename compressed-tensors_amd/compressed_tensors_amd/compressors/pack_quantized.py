@@ -280,3 +280,71 @@ class PackedWeightBatch:
                                                             _lib.stream_of(self.device))
         )
         return self.dense
+
+
+def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,
+                                 compression_device=None, **kwargs):
+    """BaseQuantizationCompressor.compress for pack-quantized with every weight
+    handed to the C ABI in one call (same keys, dtypes and shapes as the
+    per-weight loop)."""
+    jobs, order = [], []
+    for name in list(model_state.keys()):
+        if not name.endswith("weight"):
+            continue
+        prefix = name[: -len("weight")]
+        scale = model_state.get(prefix + "weight_scale", None)
+        if scale is None:
+            continue
+        module_path = prefix[:-1] if prefix.endswith(".") else prefix
+        args = names_to_scheme[module_path].weights
+        weight = model_state[name]
+        if model_state.get(prefix + "weight_global_scale", None) is not None:
+            raise ValueError("global_scale is not supported for the PackQuantizationCompressor")
+        if not can_quantize(weight, args) or weight.ndim != 2:
+            continue  # handled by the per-weight path below
+        jobs.append(dict(name=name, weight=weight, scale=scale,
+                         zero_point=model_state.get(prefix + "weight_zero_point", None),
+                         g_idx=model_state.get(prefix + "weight_g_idx", None),
+                         quantization_args=args))
+        order.append((name, prefix, args))
+    packed_by_name = {}
+    if jobs:
+        batch = PackedWeightBatch(jobs)
+        for (name, prefix, args), packed in zip(order, batch.compress()):
+            packed_by_name[name] = packed
+
+    def move(t):
+        return t if compression_device is None else t.to(compression_device)
+
+    out = {}
+    for name in list(model_state.keys()):
+        value = model_state[name]
+        if name in packed_by_name:
+            prefix = name[: -len("weight")]
+            module_path = prefix[:-1] if prefix.endswith(".") else prefix
+            args = names_to_scheme[module_path].weights
+            out[prefix + "weight_shape"] = move(torch.tensor(value.shape))
+            out[prefix + "weight_packed"] = move(packed_by_name[name])
+            if not args.symmetric and args.strategy in _PACKABLE:
+                zp = to_gpu(model_state[prefix + "weight_zero_point"])
+                out[prefix + "weight_zero_point"] = move(
+                    pack_to_int32(zp, args.num_bits, packed_dim=0))
+        elif name.endswith("weight") and model_state.get(name[: -len("weight")] + "weight_scale") is not None:
+            prefix = name[: -len("weight")]
+            module_path = prefix[:-1] if prefix.endswith(".") else prefix
+            single = self.compress_weight(
+                weight=value, scale=model_state[prefix + "weight_scale"],
+                zero_point=model_state.get(prefix + "weight_zero_point", None),
+                g_idx=model_state.get(prefix + "weight_g_idx", None),
+                quantization_args=names_to_scheme[module_path].weights,
+                device=compression_device)
+            for key, tensor in single.items():
+                out[prefix + key] = move(tensor)
+        elif name.endswith("zero_point") and self._skip_zp(name, names_to_scheme):
+            continue
+        elif name not in out:
+            out[name] = move(value)
+    return out
+
+
+PackedQuantizationCompressor.compress = _compress_state_dict_batched

@@ -1,0 +1,136 @@
+"""GPU: ModelCompressor on a small Llama-shaped module tree vs the oracle."""
+import pytest
+import torch
+
+from gpu_util import announce, assert_bit_equal
+from oracle import pack as op
+from oracle import quant as oq
+from oracle import sparse as osp
+
+pytestmark = pytest.mark.gpu
+
+
+class Block(torch.nn.Module):
+    def __init__(self, d, f):
+        super().__init__()
+        self.q_proj = torch.nn.Linear(d, d, bias=False)
+        self.k_proj = torch.nn.Linear(d, d // 4, bias=False)
+        self.down_proj = torch.nn.Linear(f, d, bias=False)
+        self.norm = torch.nn.LayerNorm(d)
+
+
+class Tiny(torch.nn.Module):
+    def __init__(self, d=256, f=512, layers=2):
+        super().__init__()
+        self.layers = torch.nn.ModuleList([Block(d, f) for _ in range(layers)])
+        self.lm_head = torch.nn.Linear(d, 64, bias=False)
+
+
+def _prepare(model, args, oargs, gpu):
+    """calibrate with the GPU observer, keep a CPU copy for the oracle"""
+    from compressed_tensors_amd.quantization import observe_weight_qparams
+
+    cpu = {}
+    for name, m in model.named_modules():
+        if getattr(m, "quantization_scheme", None) is None:
+            continue
+        w = m.weight.data
+        scale, zp = observe_weight_qparams(w, args)
+        o_scale, o_zp = oq.observe_weight(w.cpu(), oargs)
+        assert_bit_equal(scale, o_scale, "scale")
+        m.register_parameter("weight_scale", torch.nn.Parameter(scale, requires_grad=False))
+        m.register_parameter("weight_zero_point", torch.nn.Parameter(zp, requires_grad=False))
+        cpu[name] = (w.cpu(), o_scale, o_zp)
+    return cpu
+
+
+@pytest.mark.parametrize("symmetric", [True, False])
+def test_pack_quantized_model_roundtrip(symmetric, gpu):
+    from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme,
+    )
+
+    announce("ModelCompressor pack-quantized", symmetric)
+    torch.manual_seed(0)
+    model = Tiny().to(torch.bfloat16).to(gpu)
+    spec = dict(num_bits=4, type="int", symmetric=symmetric, strategy="group", group_size=128)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    config = QuantizationConfig(
+        config_groups={"g0": QuantizationScheme(targets=["Linear"], weights=args)},
+        format="pack-quantized", ignore=["lm_head"])
+    apply_quantization_scheme(model, config)
+    cpu = _prepare(model, args, oargs, gpu)
+    assert set(cpu) == {f"layers.{i}.{p}" for i in range(2) for p in ("q_proj", "k_proj", "down_proj")}
+
+    mc = ModelCompressor(quantization_config=config)
+    state = mc.compress(model)
+    for name, (w, s, z) in cpu.items():
+        want = op.pack_quantized_compress(w, s, oargs, zero_point=z)
+        assert_bit_equal(state[f"{name}.weight_packed"], want["weight_packed"], name)
+        assert state[f"{name}.weight_shape"].tolist() == list(w.shape)
+        assert f"{name}.weight" not in state
+        assert (f"{name}.weight_zero_point" in state) == (not symmetric)
+    assert "lm_head.weight" in state and "layers.0.norm.weight" in state
+
+    # in-memory: compress_model / decompress_model
+    mc.compress_model(model)
+    q = model.layers[0].q_proj
+    assert hasattr(q, "weight_packed") and not hasattr(q, "weight")
+    assert str(q.quantization_status.value) == "compressed"
+    mc.decompress_model(model)
+    for name, (w, s, z) in cpu.items():
+        want = op.pack_quantized_compress(w, s, oargs, zero_point=z)
+        data = dict(want, weight_scale=s)
+        dense = op.pack_quantized_decompress(data, oargs)
+        assert_bit_equal(model.get_submodule(name).weight.data, dense, f"{name} decompressed")
+
+    # state-dict decompress into a fresh model
+    fresh = Tiny().to(torch.bfloat16).to(gpu)
+    apply_quantization_scheme(fresh, config)
+    mc.decompress(state, fresh)
+    for name, (w, s, z) in cpu.items():
+        want = op.pack_quantized_compress(w, s, oargs, zero_point=z)
+        dense = op.pack_quantized_decompress(dict(want, weight_scale=s), oargs)
+        assert_bit_equal(fresh.get_submodule(name).weight.data, dense, f"{name} loaded")
+
+
+def test_fp8_plus_sparse24_stack(gpu):
+    """quantization first, sparsity second (float-quantized + sparse-24-bitmask)"""
+    from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
+    from compressed_tensors_amd.config import SparsityCompressionConfig
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme,
+    )
+
+    announce("ModelCompressor fp8 + 2:4")
+    torch.manual_seed(1)
+    model = Tiny(layers=1).to(torch.bfloat16).to(gpu)
+    for m in model.modules():
+        if isinstance(m, torch.nn.Linear):
+            keep = osp.get_24_bytemasks(m.weight.data.cpu()).to(gpu)
+            m.weight.data = torch.where(keep, m.weight.data, torch.zeros_like(m.weight.data))
+    spec = dict(num_bits=8, type="float", symmetric=True, strategy="channel")
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    qcfg = QuantizationConfig(
+        config_groups={"g0": QuantizationScheme(targets=["Linear"], weights=args)},
+        format="float-quantized", ignore=["lm_head"])
+    scfg = SparsityCompressionConfig(format="sparse-24-bitmask", targets=["Linear"],
+                                     ignore=["lm_head"], sparsity_structure="2:4")
+    apply_quantization_scheme(model, qcfg)
+    cpu = _prepare(model, args, oargs, gpu)
+    mc = ModelCompressor(sparsity_config=scfg, quantization_config=qcfg)
+    state = mc.compress(model)
+    for name, (w, s, z) in cpu.items():
+        codes = op.naive_compress(w, s, oargs, zero_point=z)
+        vals, bm = osp.sparse24_bitmask_compress(codes)
+        assert_bit_equal(state[f"{name}.compressed"], vals, f"{name}.compressed")
+        assert_bit_equal(state[f"{name}.bitmask"], bm, f"{name}.bitmask")
+        assert state[f"{name}.shape"].flatten().tolist() == list(w.shape)
+        assert f"{name}.weight" not in state and f"{name}.weight_scale" in state
+    mc.compress_model(model)
+    mc.decompress_model(model)
+    for name, (w, s, z) in cpu.items():
+        codes = op.naive_compress(w, s, oargs, zero_point=z)
+        dense = op.naive_decompress({"weight": codes, "weight_scale": s})
+        assert_bit_equal(model.get_submodule(name).weight.data, dense, f"{name} decompressed")
