@@ -1,0 +1,229 @@
+// Vectorised quantize / dequantize / fake-quantize for the common layouts:
+// input, scale and (for the float side) output share one float dtype, scales
+// cover runs of at least 8 columns (per tensor, channel, token or group), codes
+// are int8 or float8_e4m3fn.  Same arithmetic as the generic kernel in
+// quant.hip (forward.py:455-514), 8 elements per lane, 16-byte accesses, one
+// workgroup per chunk, streaming hints on the dense data.
+//
+// bf16 tensors quantize with a reciprocal multiply (same bits as the division,
+// see quant_fast.h); fp8 codes use the hardware converters
+// (v_cvt_pk_fp8_f32 / v_cvt_f32_fp8: OCP e4m3, round-to-nearest-even), which the
+// GPU tests compare with torch's cast on every bf16 bit pattern.
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "quant_core.h"
+#include "quant_fast.h"
+#include "vec_geom.h"
+
+namespace ctmi {
+
+constexpr int kKindFloat = 0, kKindI8 = 1, kKindF8 = 2;
+constexpr int kQdqBlock = 512, kQdqUnroll = 2;
+
+template <int CT>
+__device__ __forceinline__ void round2(float& a, float& b) {
+  if constexpr (CT == CTMI_BF16) {
+    const uint32_t p = pack_bf16x2(a, b);
+    a = bf16_lo(p);
+    b = bf16_hi(p);
+  } else if constexpr (CT == CTMI_F16) {
+    a = f16_to_f32(f32_to_f16(a));
+    b = f16_to_f32(f32_to_f16(b));
+  }
+}
+
+__device__ __forceinline__ float fp8_hw_decode(uint32_t word, int byte) {
+  switch (byte) {
+    case 0: return __builtin_amdgcn_cvt_f32_fp8((int)word, 0);
+    case 1: return __builtin_amdgcn_cvt_f32_fp8((int)word, 1);
+    case 2: return __builtin_amdgcn_cvt_f32_fp8((int)word, 2);
+    default: return __builtin_amdgcn_cvt_f32_fp8((int)word, 3);
+  }
+}
+
+// FT: float dtype tag of x / scale / float output.  IN / OUT: element kind of the
+// input and output tensors.  QK: 0 = integer grid, 1 = fp8 grid.
+template <typename FT, int IN, int OUT, int QK, bool HAS_ZP>
+__global__ void __launch_bounds__(kQdqBlock)
+qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict__ scale,
+               const uint8_t* __restrict__ zp, void* __restrict__ yout, VecGeom g, float qmin,
+               float qmax) {
+  constexpr int CT = FT::id;
+  constexpr int B = kQdqBlock, U = kQdqUnroll;
+  constexpr bool DO_Q = IN == kKindFloat;
+  constexpr bool DO_DQ = OUT == kKindFloat;
+  using FR = typename FT::raw;
+  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  Vec<FR, 8> xf[U];
+  Vec<uint8_t, 8> xc[U];
+  float sv[U], zv[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    if (v < g.nvec) {
+      if constexpr (DO_Q) xf[k] = ldg_nt<FR, 8>((const FR*)xin + (size_t)v * 8);
+      else xc[k] = ldg_nt<uint8_t, 8>((const uint8_t*)xin + (size_t)v * 8);
+      const uint32_t si = scale_index(v, g);
+      sv[k] = FT::to_f32(scale[si]);
+      if constexpr (HAS_ZP) {
+        zv[k] = QK == 0 ? (float)(int8_t)zp[si] : f8e4m3_to_f32(zp[si]);
+      } else {
+        zv[k] = 0.0f;
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    if (v >= g.nvec) continue;
+    const float s = sv[k], z = zv[k];
+    float t[8];
+    uint32_t codes[2] = {0u, 0u};  // 8 one-byte codes
+    if constexpr (DO_Q) {
+      const bool fast = CT == CTMI_BF16 && scale_is_tame(s);
+      const float r = __builtin_amdgcn_rcpf(s);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float a = FT::to_f32(xf[k].v[2 * j]), b = FT::to_f32(xf[k].v[2 * j + 1]);
+        if (fast) { a *= r; b *= r; } else { a /= s; b /= s; }
+        round2<CT>(a, b);
+        if (HAS_ZP) { a += z; b += z; round2<CT>(a, b); }
+        a = clamp_nan(a, qmin, qmax);
+        b = clamp_nan(b, qmin, qmax);
+        if constexpr (QK == 0) {
+          a = rintf(a);
+          b = rintf(b);
+          if constexpr (OUT == kKindI8) {
+            codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(a)) << (16 * (j % 2));
+            codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(b)) << (16 * (j % 2) + 8);
+          }
+        } else {
+          // two fp8 codes into the low or high half of the word
+          if (j % 2 == 0) codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], false);
+          else codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], true);
+          if constexpr (DO_DQ) {
+            a = fp8_hw_decode(codes[j / 2], 2 * (j % 2));
+            b = fp8_hw_decode(codes[j / 2], 2 * (j % 2) + 1);
+          }
+        }
+        t[2 * j] = a;
+        t[2 * j + 1] = b;
+      }
+    } else {
+      const Vec<uint32_t, 2> w = __builtin_bit_cast(Vec<uint32_t, 2>, xc[k]);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        if constexpr (IN == kKindI8) t[i] = (float)(int8_t)((w.v[i / 4] >> (8 * (i % 4))) & 0xffu);
+        else t[i] = fp8_hw_decode(w.v[i / 4], i % 4);
+      }
+    }
+    if constexpr (DO_DQ) {
+      Vec<FR, 8> o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float a = t[2 * j], b = t[2 * j + 1];
+        if (HAS_ZP) { a -= z; b -= z; round2<CT>(a, b); }
+        a *= s;
+        b *= s;
+        if constexpr (CT == CTMI_BF16) {
+          const uint32_t p = pack_bf16x2(a, b);
+          o.v[2 * j] = (uint16_t)(p & 0xffffu);
+          o.v[2 * j + 1] = (uint16_t)(p >> 16);
+        } else {
+          o.v[2 * j] = FT::from_f32(a);
+          o.v[2 * j + 1] = FT::from_f32(b);
+        }
+      }
+      stg_nt<FR, 8>((FR*)yout + (size_t)v * 8, o);
+    } else {
+      Vec<uint32_t, 2> w;
+      w.v[0] = codes[0];
+      w.v[1] = codes[1];
+      stg_nt<uint8_t, 8>((uint8_t*)yout + (size_t)v * 8, __builtin_bit_cast(Vec<uint8_t, 8>, w));
+    }
+  }
+}
+
+template <typename FT, int IN, int OUT, int QK>
+static void launch_qdq(bool has_zp, const void* x, const void* scale, const void* zp, void* out,
+                       const VecGeom& g, float qmin, float qmax, hipStream_t st) {
+  const unsigned grid = (unsigned)cdiv(g.nvec, kQdqBlock * kQdqUnroll);
+  using FR = typename FT::raw;
+  if (has_zp)
+    hipLaunchKernelGGL((qdq_vec_kernel<FT, IN, OUT, QK, true>), grid, kQdqBlock, 0, st, x,
+                       (const FR*)scale, (const uint8_t*)zp, out, g, qmin, qmax);
+  else
+    hipLaunchKernelGGL((qdq_vec_kernel<FT, IN, OUT, QK, false>), grid, kQdqBlock, 0, st, x,
+                       (const FR*)scale, (const uint8_t*)zp, out, g, qmin, qmax);
+}
+
+template <typename FT>
+static void dispatch_mode(int in_kind, int out_kind, int qk, bool has_zp, const void* x,
+                          const void* scale, const void* zp, void* out, const VecGeom& g,
+                          float qmin, float qmax, hipStream_t st) {
+#define CTMI_QDQ(IN, OUT, QK)                              \
+  if (in_kind == IN && out_kind == OUT && qk == QK) {      \
+    launch_qdq<FT, IN, OUT, QK>(has_zp, x, scale, zp, out, g, qmin, qmax, st); \
+    return;                                                \
+  }
+  CTMI_QDQ(kKindFloat, kKindI8, 0)
+  CTMI_QDQ(kKindFloat, kKindF8, 1)
+  CTMI_QDQ(kKindI8, kKindFloat, 0)
+  CTMI_QDQ(kKindF8, kKindFloat, 1)
+  CTMI_QDQ(kKindFloat, kKindFloat, 0)
+  CTMI_QDQ(kKindFloat, kKindFloat, 1)
+#undef CTMI_QDQ
+}
+
+// Tries the vectorised path; returns false (nothing launched) if the problem
+// does not fit it.  All arguments have been validated by the caller.
+bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
+                        int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq,
+                        hipStream_t st) {
+  const int sd = qp->scale_dtype;
+  if (sd != CTMI_BF16 && sd != CTMI_F16 && sd != CTMI_F32) return false;
+  int in_kind, out_kind, qk;
+  if (!do_q) {
+    // dequantize only looks at the stored codes, whatever grid produced them
+    if (x_dtype == CTMI_I8) qk = 0;
+    else if (x_dtype == CTMI_F8E4M3) qk = 1;
+    else return false;
+  } else if (qp->qtype == CTMI_QTYPE_INT && qp->num_bits <= 8) {
+    qk = 0;
+  } else if (qp->qtype == CTMI_QTYPE_FLOAT && qp->num_bits == 8) {
+    qk = 1;
+  } else {
+    return false;
+  }
+  const int code_dtype = qk == 0 ? CTMI_I8 : CTMI_F8E4M3;
+  if (do_q && do_dq) {
+    if (x_dtype != sd || out_dtype != sd) return false;
+    in_kind = out_kind = kKindFloat;
+  } else if (do_q) {
+    if (x_dtype != sd || out_dtype != code_dtype) return false;
+    in_kind = kKindFloat;
+    out_kind = qk == 0 ? kKindI8 : kKindF8;
+  } else {
+    if (x_dtype != code_dtype || out_dtype != sd) return false;
+    in_kind = qk == 0 ? kKindI8 : kKindF8;
+    out_kind = kKindFloat;
+  }
+  if (qp->zero_point && qp->zp_dtype != code_dtype) return false;
+  VecGeom g;
+  if (!vec_geometry(qp, rows, cols, &g)) return false;
+  if (cdiv(g.nvec, kQdqBlock * kQdqUnroll) >= (1ll << 31)) return false;
+  const int in_bytes = 8 * dtype_size(x_dtype), out_bytes = 8 * dtype_size(out_dtype);
+  if ((uintptr_t)x % in_bytes || (uintptr_t)out % out_bytes) return false;
+  float qmin, qmax;
+  if (quant_range(qp->qtype, qp->num_bits, &qmin, &qmax)) return false;
+  const bool has_zp = qp->zero_point != nullptr;
+  if (sd == CTMI_BF16)
+    dispatch_mode<BF16>(in_kind, out_kind, qk, has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
+  else if (sd == CTMI_F16)
+    dispatch_mode<F16>(in_kind, out_kind, qk, has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
+  else
+    dispatch_mode<F32>(in_kind, out_kind, qk, has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
+  return true;
+}
+
+}  // namespace ctmi

@@ -57,6 +57,9 @@ __global__ void __launch_bounds__(256) qdq_generic_kernel(QdqArgs a) {
   }
 }
 
+bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
+                        int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq, hipStream_t st);
+
 // ------------------------------------------------------------------ host side
 static int fill_cfg(const ctmi_qparams* qp, int x_dtype, QuantCfg* q) {
   int rc = quant_range(qp->qtype, qp->num_bits, &q->qmin, &q->qmax);
@@ -90,6 +93,10 @@ extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_d
   if (rc) return rc;
   if (rows == 0 || cols == 0) return CTMI_OK;
   CTMI_REQUIRE(x != nullptr && out != nullptr, CTMI_ERR_VALUE, "NULL tensor pointer");
+
+  if (qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize,
+                         (hipStream_t)stream))
+    return check_launch("ctmi_qdq");
 
   QdqArgs a;
   a.x = x;

@@ -222,3 +222,71 @@ def test_large_w4a16_properties(gpu):
     err = (wg.float() - dq.float()).abs()
     bound = scale.float().repeat_interleave(128, dim=1) * 0.57 + 1e-12
     assert bool(((err <= bound) | (q == 7) | (q == -8)).all())
+
+
+def test_fp8_codes_on_every_bf16_pattern(gpu):
+    """scale 1: the quantize chain reduces to clamp + cast, so every bf16 bit pattern
+    (NaN aside) goes through the fp8 conversion; likewise every fp8 code is decoded"""
+    from compressed_tensors_amd.quantization import QuantizationArgs, dequantize, quantize
+
+    announce("fp8 exhaustive")
+    args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
+    oargs = oq._Args(num_bits=8, type="float", symmetric=True, strategy="channel")
+    allbits = torch.arange(0, 65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    x = allbits[~torch.isnan(allbits.float())]
+    x = torch.cat([x, x[: (-x.numel()) % 512]]).reshape(-1, 512)
+    for s_val in (1.0, 0.5, 3.0, 0.0123):
+        scale = torch.full((x.shape[0], 1), s_val, dtype=torch.bfloat16)
+        q = quantize(x.to(gpu), scale.to(gpu), None, args, dtype=torch.float8_e4m3fn)
+        assert_bit_equal(q, oq.quantize(x, scale, None, oargs, dtype=torch.float8_e4m3fn), f"fp8 codes s={s_val}")
+    codes = torch.arange(0, 256, dtype=torch.int32).to(torch.uint8).repeat(16).reshape(8, 512)
+    codes = codes[:, [c for c in range(512) if (c % 256) & 0x7F != 0x7F]]  # drop the NaN codes
+    codes = codes[:, :504].contiguous().view(torch.float8_e4m3fn)
+    scale = torch.full((8, 1), 1.0, dtype=torch.bfloat16)
+    dq = dequantize(codes.to(gpu), scale.to(gpu))
+    assert_bit_equal(dq, oq.dequantize(codes, scale), "fp8 decode")
+    for dt in (torch.float16, torch.float32):
+        xs = x.to(dt)
+        scale = torch.full((x.shape[0], 1), 0.37, dtype=dt)
+        q = quantize(xs.to(gpu), scale.to(gpu), None, args, dtype=torch.float8_e4m3fn)
+        assert_bit_equal(q, oq.quantize(xs, scale, None, oargs, dtype=torch.float8_e4m3fn), f"fp8 codes {dt}")
+
+
+def test_large_fp8_channel_and_token(gpu):
+    """BASELINE-sized fp8 paths: per-channel weight codes and per-token activation QDQ,
+    sampled rows against the oracle"""
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, compute_dynamic_scales_and_zp, dequantize, fake_quantize,
+        observe_weight_qparams, quantize,
+    )
+
+    announce("large fp8")
+    g = torch.Generator().manual_seed(1)
+    w = torch.randn(14336, 4096, generator=g) * 0.02
+    w[torch.rand(w.shape, generator=g) < 0.001] *= 20
+    w = w.bfloat16()
+    args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
+    oargs = oq._Args(num_bits=8, type="float", symmetric=True, strategy="channel")
+    wg = w.to(gpu)
+    scale, zp = observe_weight_qparams(wg, args)
+    q = quantize(wg, scale, zp, args, dtype=torch.float8_e4m3fn)
+    dq = dequantize(q, scale)
+    rows = torch.arange(0, 14336, 211)
+    o_scale, o_zp = oq.observe_weight(w[rows], oargs)
+    assert_bit_equal(scale[rows.to(gpu)], o_scale, "fp8 scale rows")
+    want = oq.quantize(w[rows], o_scale, o_zp, oargs, dtype=torch.float8_e4m3fn)
+    assert_bit_equal(q[rows.to(gpu)], want, "fp8 code rows")
+    assert_bit_equal(dq[rows.to(gpu)], oq.dequantize(want, o_scale), "fp8 dequant rows")
+    assert float(q.float().abs().max()) == 448.0  # every row's extreme value hits the fp8 maximum
+    x = torch.randn(1, 8192, 4096, generator=g)
+    x[..., torch.rand(4096, generator=g) < 0.005] *= 50
+    x = x.bfloat16()
+    targs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="token", dynamic=True)
+    toargs = oq._Args(num_bits=8, type="float", symmetric=True, strategy="token")
+    xg = x.to(gpu)
+    s, z = compute_dynamic_scales_and_zp(xg, targs)
+    y = fake_quantize(xg, s, z, targs)
+    toks = torch.arange(0, 8192, 301)
+    os_, oz_ = oq.compute_dynamic_scales_and_zp(x[:, toks], toargs)
+    assert_bit_equal(s[:, toks.to(gpu)], os_, "token scales")
+    assert_bit_equal(y[:, toks.to(gpu)], oq.fake_quantize(x[:, toks], os_, oz_, toargs), "token qdq")
