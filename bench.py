@@ -38,6 +38,15 @@ LLAMA3_8B_LAYER = [
 ]
 GROUP = 128
 
+# HBM bytes per launch of the two fused kernels, averaged over the launches of one
+# pass: rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch), each scaled
+# by what the same counter reads for a plain 1 GiB copy (FETCH_SIZE reads 0.5000 of the
+# bytes copied, WRITE_SIZE 1.0000).  The summaries are profiles/pmc_traffic_*.txt.
+MEASURED_TRAFFIC = {
+    ("llama3-8b-w4a16", "pq_compress_vec_kernel"): 629.1e6,
+    ("llama3-8b-w4a16", "pq_decompress_vec_kernel"): 631.1e6,
+}
+
 
 def shapes_for(workload: str):
     if workload == "llama3-8b-w4a16":
@@ -98,6 +107,8 @@ def main():
     ap.add_argument("--workload", default="llama3-8b-w4a16")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--calib-copies", type=int, default=0,
+                    help="launch N plain 1 GiB copies first (byte-counter calibration when profiling)")
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit(
@@ -117,6 +128,15 @@ def main():
     shapes = shapes_for(a.workload)
     args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group",
                             group_size=GROUP)
+
+    if a.calib_copies:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        for _ in range(a.calib_copies):
+            _lib.check(_lib.load().ctmi_calib_copy(src.data_ptr(), dst.data_ptr(), src.numel(),
+                                                   _lib.stream_of(dev)))
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- synthetic, seeded inputs resident in HBM
     entries = []
@@ -169,13 +189,15 @@ def main():
 
     ms_per_step = wall / a.steps * 1e3
     value = 2 * per_dir / (wall / a.steps) / 1e9
-    n_launch = len(shapes)
     comp_gbs = per_dir / (comp_ms * 1e-3) / 1e9
     deco_gbs = per_dir / (deco_ms * 1e-3) / 1e9
     # the compress kernel does the arithmetic (division, rounding, packing): it is the dominant one
-    dom, dom_gbs, dom_ms = ("pq_compress_vec_kernel", comp_gbs, comp_ms)
+    dom, dom_gbs, dom_ms, n_launch = ("pq_compress_vec_kernel", comp_gbs, comp_ms,
+                                      batch.launches(compress=True))
     if deco_ms > comp_ms:
-        dom, dom_gbs, dom_ms = ("pq_decompress_vec_kernel", deco_gbs, deco_ms)
+        dom, dom_gbs, dom_ms, n_launch = ("pq_decompress_vec_kernel", deco_gbs, deco_ms,
+                                          batch.launches(compress=False))
+    traffic = MEASURED_TRAFFIC.get((a.workload, dom))
 
     out = {
         "metric": "compress+decompress GB/s & % HBM roofline, Llama-3-8B-shaped W4A16 g128",
@@ -192,7 +214,7 @@ def main():
         "data": "synthetic",
         "config": {
             "workload": a.workload,
-            "tensors": n_launch,
+            "tensors": len(shapes),
             "elements": n_elems,
             "group_size": GROUP,
             "algorithmic_bytes_per_step": 2 * per_dir,
@@ -207,7 +229,9 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": dom_gbs / HBM_PEAK_GBS,
-            "traffic": None,
+            "achieved_bytes_per_launch": per_dir / n_launch,
+            "traffic": traffic,
+            "traffic_unit": "HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, copy-calibrated)",
             "avg_launch_ms": dom_ms / n_launch,
             "launches_per_step": n_launch,
             "compress_GBs": comp_gbs,

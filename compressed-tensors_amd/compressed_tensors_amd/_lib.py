@@ -111,6 +111,7 @@ SIGNATURES = {
     ),
     "ctmi_pack_quantized_compress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
     "ctmi_pack_quantized_decompress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
+    "ctmi_pack_quantized_launches": (c_int64, [POINTER(WeightJob), c_int64, c_int32]),
     "ctmi_pack_fp4_to_uint8": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_void_p]),
     "ctmi_unpack_fp4_from_uint8": (
         c_int32,
@@ -146,6 +147,7 @@ SIGNATURES = {
         [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     ),
     "ctmi_topk24_lut": (None, [c_void_p]),
+    "ctmi_calib_copy": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "ctmi_hadamard_supported": (c_int32, [c_int32, c_int32, c_int32]),
     "ctmi_hadamard_apply": (
         c_int32,

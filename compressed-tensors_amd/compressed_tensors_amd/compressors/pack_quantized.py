@@ -273,6 +273,14 @@ class PackedWeightBatch:
         )
         return self.packed
 
+    def launches(self, compress=True):
+        """number of kernel launches one compress() (or decompress()) pass enqueues"""
+        jobs = self._cjobs if compress else self._djobs
+        count = _lib.load().ctmi_pack_quantized_launches(jobs, self.n, 1 if compress else 0)
+        if count < 0:
+            _lib.check(int(count))
+        return int(count)
+
     def decompress(self):
         """enqueue unpack+dequantize of every packed weight; returns the dense tensors"""
         _lib.check(

@@ -544,7 +544,10 @@ static int plan_decompress(const int32_t* packed, void* out, int32_t out_dtype, 
 
 // Enqueue validated plans: vectorised ones are chained, kMaxJobs per launch and
 // per template instance; the others get a launch of the generic kernel each.
-static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, const char* what) {
+// With `count_only` set nothing is enqueued and the number of launches is stored there.
+static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, const char* what,
+                     int64_t* count_only = nullptr) {
+  int64_t launches = 0;
   const int per_block = compress ? kCompressBlock * kCompressUnroll
                                  : kDecompressBlock * kDecompressUnroll;
   std::vector<char> done((size_t)n, 0);
@@ -552,7 +555,9 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
     if (done[i] || plans[i].empty) continue;
     if (!plans[i].vec) {
       const FusedArgs& a = plans[i].generic;
-      if (compress)
+      ++launches;
+      if (count_only) {
+      } else if (compress)
         hipLaunchKernelGGL(pq_compress_generic_kernel, grid_for(a.rows * a.pcols, 256), 256, 0, st, a);
       else
         hipLaunchKernelGGL(pq_decompress_generic_kernel, grid_for(a.rows * a.cols, 256), 256, 0, st, a);
@@ -572,7 +577,9 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
     quant_range(CTMI_QTYPE_INT, key.bits, &t.qmin, &t.qmax);
     auto flush = [&]() {
       if (t.n == 0) return;
-      if (compress) launch_compress_vec(key, t, (unsigned)chunks, st);
+      ++launches;
+      if (count_only) {
+      } else if (compress) launch_compress_vec(key, t, (unsigned)chunks, st);
       else launch_decompress_vec(key, t, (unsigned)chunks, st);
       reset();
     };
@@ -587,6 +594,10 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
       done[j] = 1;
     }
     flush();
+  }
+  if (count_only) {
+    *count_only = launches;
+    return CTMI_OK;
   }
   return check_launch(what);
 }
@@ -622,6 +633,21 @@ extern "C" int ctmi_pack_quantized_compress_many(const ctmi_weight_job* jobs, in
     if (rc) return rc;
   }
   return run_plans(plans.data(), n, true, (hipStream_t)stream, "ctmi_pack_quantized_compress_many");
+}
+
+extern "C" int64_t ctmi_pack_quantized_launches(const ctmi_weight_job* jobs, int64_t n,
+                                                int32_t compress) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  std::vector<PqPlan> plans((size_t)n);
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_weight_job& j = jobs[i];
+    int rc = compress ? plan_compress(j.src, j.dense_dtype, (int32_t*)j.dst, j.rows, j.cols, &j.qp, &plans[i])
+                      : plan_decompress((const int32_t*)j.src, j.dst, j.dense_dtype, j.rows, j.cols, &j.qp, &plans[i]);
+    if (rc) return rc;
+  }
+  int64_t count = 0;
+  run_plans(plans.data(), n, compress != 0, nullptr, "ctmi_pack_quantized_launches", &count);
+  return count;
 }
 
 extern "C" int ctmi_pack_quantized_decompress_many(const ctmi_weight_job* jobs, int64_t n,

@@ -132,6 +132,10 @@ typedef struct ctmi_weight_job {
  * dtype / bit-width combination are chained into common launches. */
 int ctmi_pack_quantized_compress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
 int ctmi_pack_quantized_decompress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
+/* Number of kernel launches the call above (compress != 0) or its inverse
+ * (compress == 0) would enqueue for this job list, without enqueueing any:
+ * what a profiler divides a pass's time by.  Negative = error code. */
+int64_t ctmi_pack_quantized_launches(const ctmi_weight_job* jobs, int64_t n, int32_t compress);
 
 /* A13.  pack_fp4_to_uint8 (compressors/quantized_compressors/fp4_quantized.py:135-178).
  * x: [rows, cols] float type; out: uint8 [rows, cols/2]. */
@@ -256,6 +260,11 @@ int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t nume
  * fp32 accumulation on the vector ALUs. */
 int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t h,
                       const float* w, void* stream);
+
+/* Plain device-to-device copy of `bytes` bytes (a multiple of 16): the known
+ * quantity against which hardware byte counters are calibrated when profiling.
+ * No counterpart in the reference. */
+int ctmi_calib_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
 /* The 4096-entry keep table used by the 2:4 kernels (host copy, for tests). */
 void ctmi_topk24_lut(uint8_t* out4096);
