@@ -196,10 +196,10 @@ int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_si
                             int64_t cols, void* stream);
 
 /* A20.  get_24_bytemasks (sparse_24_bitmask.py:227-260): top-2-of-4 by
- * |value| with torch.topk's tie order.  kind: 0 = float type of elem_size
- * bytes (bf16 when elem_size==2 && is_bf16), 1 = int8 view of fp8 / int8
- * (ranked by abs() computed in int8, so abs(-128) == -128).
- * mask: bool [numel]. */
+ * |value| with torch.topk's tie order.  x_dtype: a float type (ranked on the
+ * value), or CTMI_I8 / CTMI_F8E4M3, which are ranked as the reference ranks
+ * its int8 view of fp8 data: abs() computed in int8, so abs(-128) == -128.
+ * numel must be a multiple of 4.  mask: bool [numel]. */
 int ctmi_get_24_bytemasks(const void* x, int32_t x_dtype, uint8_t* mask, int64_t numel,
                           void* stream);
 
