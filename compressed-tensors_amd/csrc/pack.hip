@@ -10,6 +10,9 @@
 // is padded with zero bits.
 #include <vector>
 
+#include <cstddef>
+#include <cstring>
+
 #include "ctmi_device.h"
 #include "ctmi_host.h"
 #include "quant_core.h"
@@ -221,50 +224,114 @@ struct VecJob {
   VecGeom g;
 };
 
-struct VecJobTable {
-  VecJob job[kMaxJobs];
+// What a workgroup needs of its weight, 64 bytes so that one scalar load brings
+// it in.  Scale of item v (8 elements): `v >> shift` when scales are numbered
+// like the items (FLAT), else row r = v / vpr, column block (v - r*vpr) / vpb,
+// index r * s_stride + block (s_stride 0 when all rows share one scale row).
+struct alignas(64) PqJob {
+  const void* src;
+  void* dst;
+  const void* scale;
+  const int8_t* zp;
+  uint32_t shift, reserved;
+  uint32_t vpr_d, vpr_m, vpr_s;
+  uint32_t vpb_m, vpb_s;
+  uint32_t s_stride;
+};
+static_assert(sizeof(PqJob) == 64, "one scalar load per job");
+
+// Kernel argument of a chained launch.  What decides which job a workgroup
+// belongs to and whether a lane has work comes first, in one scalar load; unused
+// chunk_end entries hold 0xFFFFFFFF.
+struct PqJobTable {
   uint32_t chunk_end[kMaxJobs];  // running total of chunks, job 0 .. j
-  int32_t n;
+  uint32_t nvec[kMaxJobs];       // items of job j
+  PqJob job[kMaxJobs];
   float qmin, qmax;
+  int32_t n;
 };
 
-__device__ __forceinline__ int find_job(const VecJobTable& t, uint32_t chunk, uint32_t* local) {
-  // branch-free over the whole table (unused entries hold 0xFFFFFFFF): the
-  // loads are independent, so they are fetched together instead of one
-  // dependent scalar load per step
-  int j = 0;
-  uint32_t first = 0;
-#pragma unroll
-  for (int i = 0; i < kMaxJobs - 1; ++i) {
-    const uint32_t e = t.chunk_end[i];
-    const bool past = chunk >= e;
-    j += past ? 1 : 0;
-    first = past ? e : first;
-  }
-  *local = chunk - first;
-  return j;
+static inline bool flat_geometry(const VecGeom& g) { return g.mode == 0; }
+
+static inline PqJob make_pq_job(const VecJob& j) {
+  PqJob o;
+  o.src = j.src;
+  o.dst = j.dst;
+  o.scale = j.scale;
+  o.zp = j.zp;
+  o.shift = j.g.shift;
+  o.reserved = 0;
+  o.vpr_d = j.g.vpr.d;
+  o.vpr_m = j.g.vpr.m;
+  o.vpr_s = j.g.vpr.s;
+  o.vpb_m = j.g.vpb.m;
+  o.vpb_s = j.g.vpb.s;
+  o.s_stride = j.g.row_scaled ? j.g.s_cols : 0u;
+  return o;
 }
 
-template <typename XT, typename ST, int BITS, bool HAS_ZP>
-__global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const VecJobTable t) {
+static_assert(kMaxJobs == 8 && offsetof(PqJobTable, chunk_end) == 0 &&
+                  offsetof(PqJobTable, nvec) == 32,
+              "find_job reads chunk_end and nvec as the first 16 dwords of the kernel argument");
+
+// The job of workgroup `chunk`, the chunk's number within that job and the job's
+// item count.  The table must be the kernel's only argument.  Its head (chunk_end
+// and nvec) is fetched with one 64-byte scalar load written out by hand: left to
+// itself the compiler turns the search into a chain of dependent loads, and a
+// wave of these kernels lives too short to hide several scalar round trips.
+// The search itself is then compares and selects on registers, and the job's 64
+// bytes follow as one more batch of scalar loads.
+__device__ __forceinline__ PqJob find_job(const PqJobTable& t, uint32_t chunk, uint32_t* local,
+                                          uint32_t* nvec) {
+  typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
+  u32x16 head;
+  asm volatile("s_load_dwordx16 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)"
+               : "=s"(head)
+               : "s"(__builtin_amdgcn_kernarg_segment_ptr()));
+  uint32_t j = 0, first = 0, nv = head[8];
+#pragma unroll
+  for (int i = 0; i < kMaxJobs - 1; ++i) {
+    const uint32_t e = head[i];
+    const bool past = chunk >= e;
+    j = past ? (uint32_t)(i + 1) : j;  // chunk_end ascends: the last hit wins
+    first = past ? e : first;
+    nv = past ? head[9 + i] : nv;
+  }
+  *local = chunk - first;
+  *nvec = nv;
+  return t.job[j];
+}
+
+template <bool FLAT>
+__device__ __forceinline__ uint32_t pq_scale_index(uint32_t v, const PqJob& job) {
+  if constexpr (FLAT) {
+    return v >> job.shift;
+  } else {
+    const uint32_t r = (uint32_t)(((uint64_t)v * job.vpr_m) >> 31) >> job.vpr_s;
+    const uint32_t cv = v - r * job.vpr_d;
+    return r * job.s_stride + ((uint32_t)(((uint64_t)cv * job.vpb_m) >> 31) >> job.vpb_s);
+  }
+}
+
+template <typename XT, typename ST, int BITS, bool HAS_ZP, bool FLAT>
+__global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const PqJobTable t) {
   constexpr int W = BITS / 4;  // output words per item
   constexpr int B = kCompressBlock, U = kCompressUnroll;
-  uint32_t chunk;
-  const VecJob& job = t.job[find_job(t, blockIdx.x, &chunk)];
+  uint32_t chunk, nvec;
+  const PqJob job = find_job(t, blockIdx.x, &chunk, &nvec);
   const auto* __restrict__ x = (const typename XT::raw*)job.src;
   const auto* __restrict__ scale = (const typename ST::raw*)job.scale;
   const int8_t* __restrict__ zp = job.zp;
   int32_t* __restrict__ out = (int32_t*)job.dst;
-  const VecGeom g = job.g;
   const uint32_t v0 = chunk * (B * U) + threadIdx.x;
   Vec<typename XT::raw, 8> xv[U];
   float sv[U], zv[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
-    if (v < g.nvec) {
+    if (v < nvec) {
       xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
-      const uint32_t si = scale_index(v, g);
+      const uint32_t si = pq_scale_index<FLAT>(v, job);
       sv[k] = ST::to_f32(scale[si]);
       zv[k] = HAS_ZP ? (float)zp[si] : 0.0f;
     }
@@ -272,33 +339,32 @@ __global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const V
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
-    if (v < g.nvec) {
+    if (v < nvec) {
       stg_nt<int32_t, W>(out + (size_t)v * W,
                          quant_pack8<XT, ST, BITS, HAS_ZP>(xv[k], sv[k], zv[k], t.qmin, t.qmax));
     }
   }
 }
 
-template <typename ST, int BITS, bool HAS_ZP>
-__global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(const VecJobTable t) {
+template <typename ST, int BITS, bool HAS_ZP, bool FLAT>
+__global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(const PqJobTable t) {
   constexpr int W = BITS / 4;
   constexpr int B = kDecompressBlock, U = kDecompressUnroll;
-  uint32_t chunk;
-  const VecJob& job = t.job[find_job(t, blockIdx.x, &chunk)];
+  uint32_t chunk, nvec;
+  const PqJob job = find_job(t, blockIdx.x, &chunk, &nvec);
   const int32_t* __restrict__ packed = (const int32_t*)job.src;
   const auto* __restrict__ scale = (const typename ST::raw*)job.scale;
   const int8_t* __restrict__ zp = job.zp;
   auto* __restrict__ out = (typename ST::raw*)job.dst;
-  const VecGeom g = job.g;
   const uint32_t v0 = chunk * (B * U) + threadIdx.x;
   Vec<int32_t, W> pv[U];
   float sv[U], zv[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
-    if (v < g.nvec) {
+    if (v < nvec) {
       pv[k] = ldg<int32_t, W>(packed + (size_t)v * W);
-      const uint32_t si = scale_index(v, g);
+      const uint32_t si = pq_scale_index<FLAT>(v, job);
       sv[k] = ST::to_f32(scale[si]);
       zv[k] = HAS_ZP ? (float)zp[si] : 0.0f;
     }
@@ -306,7 +372,7 @@ __global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(con
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
-    if (v < g.nvec) {
+    if (v < nvec) {
       stg_nt<typename ST::raw, 8>(out + (size_t)v * 8,
                                   unpack_dequant8<ST, BITS, HAS_ZP>(pv[k], sv[k], zv[k]));
     }
@@ -315,27 +381,34 @@ __global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(con
 
 // key of a vectorised job: which template instance runs it
 struct VecKey {
-  int x_dtype, scale_dtype, bits, has_zp;
+  int x_dtype, scale_dtype, bits, has_zp, flat;
   bool operator==(const VecKey& o) const {
     return x_dtype == o.x_dtype && scale_dtype == o.scale_dtype && bits == o.bits &&
-           has_zp == o.has_zp;
+           has_zp == o.has_zp && flat == o.flat;
   }
 };
 
-template <typename XT, typename ST>
-static void launch_compress_table(const VecKey& k, const VecJobTable& t, unsigned grid,
-                                  hipStream_t st) {
+template <typename XT, typename ST, bool FLAT>
+static void launch_compress_flat(const VecKey& k, const PqJobTable& t, unsigned grid,
+                                 hipStream_t st) {
   constexpr int B = kCompressBlock;
   if (k.bits == 4) {
-    if (k.has_zp) hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 4, true>), grid, B, 0, st, t);
-    else hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 4, false>), grid, B, 0, st, t);
+    if (k.has_zp) hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 4, true, FLAT>), grid, B, 0, st, t);
+    else hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 4, false, FLAT>), grid, B, 0, st, t);
   } else {
-    if (k.has_zp) hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 8, true>), grid, B, 0, st, t);
-    else hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 8, false>), grid, B, 0, st, t);
+    if (k.has_zp) hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 8, true, FLAT>), grid, B, 0, st, t);
+    else hipLaunchKernelGGL((pq_compress_vec_kernel<XT, ST, 8, false, FLAT>), grid, B, 0, st, t);
   }
 }
 
-static void launch_compress_vec(const VecKey& k, const VecJobTable& t, unsigned grid,
+template <typename XT, typename ST>
+static void launch_compress_table(const VecKey& k, const PqJobTable& t, unsigned grid,
+                                  hipStream_t st) {
+  if (k.flat) launch_compress_flat<XT, ST, true>(k, t, grid, st);
+  else launch_compress_flat<XT, ST, false>(k, t, grid, st);
+}
+
+static void launch_compress_vec(const VecKey& k, const PqJobTable& t, unsigned grid,
                                 hipStream_t st) {
 #define CTMI_DISPATCH_S(XT)                                                              \
   if (k.scale_dtype == CTMI_BF16) launch_compress_table<XT, BF16>(k, t, grid, st);       \
@@ -347,20 +420,27 @@ static void launch_compress_vec(const VecKey& k, const VecJobTable& t, unsigned 
 #undef CTMI_DISPATCH_S
 }
 
-template <typename ST>
-static void launch_decompress_table(const VecKey& k, const VecJobTable& t, unsigned grid,
-                                    hipStream_t st) {
+template <typename ST, bool FLAT>
+static void launch_decompress_flat(const VecKey& k, const PqJobTable& t, unsigned grid,
+                                   hipStream_t st) {
   constexpr int B = kDecompressBlock;
   if (k.bits == 4) {
-    if (k.has_zp) hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 4, true>), grid, B, 0, st, t);
-    else hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 4, false>), grid, B, 0, st, t);
+    if (k.has_zp) hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 4, true, FLAT>), grid, B, 0, st, t);
+    else hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 4, false, FLAT>), grid, B, 0, st, t);
   } else {
-    if (k.has_zp) hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 8, true>), grid, B, 0, st, t);
-    else hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 8, false>), grid, B, 0, st, t);
+    if (k.has_zp) hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 8, true, FLAT>), grid, B, 0, st, t);
+    else hipLaunchKernelGGL((pq_decompress_vec_kernel<ST, 8, false, FLAT>), grid, B, 0, st, t);
   }
 }
 
-static void launch_decompress_vec(const VecKey& k, const VecJobTable& t, unsigned grid,
+template <typename ST>
+static void launch_decompress_table(const VecKey& k, const PqJobTable& t, unsigned grid,
+                                    hipStream_t st) {
+  if (k.flat) launch_decompress_flat<ST, true>(k, t, grid, st);
+  else launch_decompress_flat<ST, false>(k, t, grid, st);
+}
+
+static void launch_decompress_vec(const VecKey& k, const PqJobTable& t, unsigned grid,
                                   hipStream_t st) {
   if (k.scale_dtype == CTMI_BF16) launch_decompress_table<BF16>(k, t, grid, st);
   else if (k.scale_dtype == CTMI_F16) launch_decompress_table<F16>(k, t, grid, st);
@@ -483,7 +563,8 @@ static int plan_compress(const void* x, int32_t x_dtype, int32_t* out, int64_t r
            qp->scale_dtype != CTMI_F8E4M3 && vec_geometry(qp, rows, cols, &p->job.g) &&
            cdiv(p->job.g.nvec, kCompressBlock * kCompressUnroll) < (1ll << 30);
   if (p->vec) {
-    p->key = VecKey{x_dtype, qp->scale_dtype, qp->num_bits, qp->zero_point != nullptr};
+    p->key = VecKey{x_dtype, qp->scale_dtype, qp->num_bits, qp->zero_point != nullptr,
+                    flat_geometry(p->job.g)};
     p->job.src = x;
     p->job.dst = out;
     p->job.scale = qp->scale;
@@ -523,7 +604,8 @@ static int plan_decompress(const int32_t* packed, void* out, int32_t out_dtype, 
            out_dtype == qp->scale_dtype && vec_geometry(qp, rows, cols, &p->job.g) &&
            cdiv(p->job.g.nvec, kDecompressBlock * kDecompressUnroll) < (1ll << 30);
   if (p->vec) {
-    p->key = VecKey{out_dtype, qp->scale_dtype, qp->num_bits, qp->zero_point != nullptr};
+    p->key = VecKey{out_dtype, qp->scale_dtype, qp->num_bits, qp->zero_point != nullptr,
+                    flat_geometry(p->job.g)};
     p->job.src = packed;
     p->job.dst = out;
     p->job.scale = qp->scale;
@@ -566,7 +648,8 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
     }
     // gather every remaining job with the same key, kMaxJobs at a time
     const VecKey key = plans[i].key;
-    VecJobTable t;
+    PqJobTable t;
+    std::memset(&t, 0, sizeof(t));
     uint64_t chunks = 0;
     auto reset = [&]() {
       t.n = 0;
@@ -587,7 +670,8 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
       if (done[j] || plans[j].empty || !plans[j].vec || !(plans[j].key == key)) continue;
       const uint64_t c = (uint64_t)cdiv(plans[j].job.g.nvec, per_block);
       if (t.n == kMaxJobs || chunks + c >= (1ull << 31)) flush();
-      t.job[t.n] = plans[j].job;
+      t.job[t.n] = make_pq_job(plans[j].job);
+      t.nvec[t.n] = plans[j].job.g.nvec;
       chunks += c;
       t.chunk_end[t.n] = (uint32_t)chunks;
       ++t.n;

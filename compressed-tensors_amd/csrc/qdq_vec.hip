@@ -80,7 +80,7 @@ qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict_
     float t[8];
     uint32_t codes[2] = {0u, 0u};  // 8 one-byte codes
     if constexpr (DO_Q) {
-      const bool fast = CT == CTMI_BF16 && scale_is_tame(s);
+      const bool fast = CT == CTMI_BF16 && wave_all(scale_is_tame(s));
       const float r = __builtin_amdgcn_rcpf(s);
 #pragma unroll
       for (int j = 0; j < 4; ++j) {

@@ -35,6 +35,10 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000u); }
 
+// True when `p` holds on every active lane of the wavefront.  Branching on it is a
+// scalar branch: a rare slow path then costs the common one nothing.
+__device__ __forceinline__ bool wave_all(bool p) { return __builtin_amdgcn_ballot_w64(!p) == 0; }
+
 __device__ __forceinline__ bool scale_is_tame(float s) {
   const float a = fabsf(s);
   return a >= 7.888609052210118e-31f && a <= 1.2676506002282294e30f;  // 2^-100 .. 2^100
@@ -84,7 +88,8 @@ __device__ __forceinline__ Vec<int32_t, BITS / 4> quant_pack8_bf16(const Vec<uin
                                                                   float qmax) {
   using PC = PackConst<BITS>;
   constexpr int W = BITS / 4;
-  if (!scale_is_tame(s)) return quant_pack8_exact<BF16, CTMI_BF16, BITS, HAS_ZP>(xv, s, z, qmin, qmax);
+  if (!wave_all(scale_is_tame(s)))
+    return quant_pack8_exact<BF16, CTMI_BF16, BITS, HAS_ZP>(xv, s, z, qmin, qmax);
   const float r = __builtin_amdgcn_rcpf(s);
   const Vec<uint32_t, 4> xw = __builtin_bit_cast(Vec<uint32_t, 4>, xv);
   // a zero point of 0 leaves every code unchanged (it only turns -0 into +0)
@@ -121,36 +126,73 @@ __device__ __forceinline__ Vec<int32_t, BITS / 4> quant_pack8(const Vec<typename
 }
 
 // ---------------------------------------------------------------- unpack + dequantize, 8 elements
-// (q - z) is an integer of at most 8 bits, exact in every float type here, so
-// the chain float(q) -> minus zero point -> times scale rounds once, at the end.
+// Byte k of a word as a float, in one instruction (extract + convert).
+template <int K>
+__device__ __forceinline__ float ubyte_to_f32(uint32_t w) {
+  float f;
+  if constexpr (K == 0) asm("v_cvt_f32_ubyte0 %0, %1" : "=v"(f) : "v"(w));
+  else if constexpr (K == 1) asm("v_cvt_f32_ubyte1 %0, %1" : "=v"(f) : "v"(w));
+  else if constexpr (K == 2) asm("v_cvt_f32_ubyte2 %0, %1" : "=v"(f) : "v"(w));
+  else asm("v_cvt_f32_ubyte3 %0, %1" : "=v"(f) : "v"(w));
+  return f;
+}
+
+// The reference computes (float(q) - zp) * scale with every step in the scale's
+// dtype (forward.py:504-509).  q - zp is an integer of at most 8 bits, exact in
+// every float type here, so the chain rounds once, at the end.  With u = q + OFF
+// the stored code and off = OFF + zp:
+//   fused form   fma(u, s, -(off * s)): u*s and off*s are exact in fp32 when s
+//                has at most 11 significant bits (bf16 / fp16 scales) or off is a
+//                power of two (no zero point), and the fma rounds the exact
+//                (u - off) * s once: the same value as the two-step form.  Only
+//                taken for scales of ordinary magnitude, where off * s can
+//                neither overflow nor lose bits to underflow;
+//   two-step     (u - off) * s, always valid.
 template <typename ST, int BITS, bool HAS_ZP>
 __device__ __forceinline__ Vec<typename ST::raw, 8> unpack_dequant8(const Vec<int32_t, BITS / 4>& pv,
                                                                     float s, float z) {
   constexpr int OFF = 1 << (BITS - 1);
+  constexpr bool kFusable = ST::id != CTMI_F32 || !HAS_ZP;
   const float off = (float)OFF + (HAS_ZP ? z : 0.0f);
-  float f[8];
+  uint32_t b[2];  // the 8 codes, one per byte
   if constexpr (BITS == 4) {
     const uint32_t w = (uint32_t)pv.v[0];
-    const uint32_t even = w & 0x0F0F0F0Fu, odd = (w >> 4) & 0x0F0F0F0Fu;
+    b[0] = w & 0x0F0F0F0Fu;         // elements 0, 2, 4, 6
+    b[1] = (w >> 4) & 0x0F0F0F0Fu;  // elements 1, 3, 5, 7
+  } else {
+    b[0] = (uint32_t)pv.v[0];
+    b[1] = (uint32_t)pv.v[1];
+  }
+  float f[8];
+  if constexpr (BITS == 4) {
+    f[0] = ubyte_to_f32<0>(b[0]); f[1] = ubyte_to_f32<0>(b[1]);
+    f[2] = ubyte_to_f32<1>(b[0]); f[3] = ubyte_to_f32<1>(b[1]);
+    f[4] = ubyte_to_f32<2>(b[0]); f[5] = ubyte_to_f32<2>(b[1]);
+    f[6] = ubyte_to_f32<3>(b[0]); f[7] = ubyte_to_f32<3>(b[1]);
+  } else {
+    f[0] = ubyte_to_f32<0>(b[0]); f[1] = ubyte_to_f32<1>(b[0]);
+    f[2] = ubyte_to_f32<2>(b[0]); f[3] = ubyte_to_f32<3>(b[0]);
+    f[4] = ubyte_to_f32<0>(b[1]); f[5] = ubyte_to_f32<1>(b[1]);
+    f[6] = ubyte_to_f32<2>(b[1]); f[7] = ubyte_to_f32<3>(b[1]);
+  }
+  // (a negative scale takes the two-step form too: it gives -0 where the fma gives +0)
+  if (kFusable && wave_all(s >= 7.888609052210118e-31f && s <= 1.2676506002282294e30f)) {
+    const float c = -(off * s);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
-      f[2 * b] = (float)((even >> (8 * b)) & 0xffu);
-      f[2 * b + 1] = (float)((odd >> (8 * b)) & 0xffu);
-    }
+    for (int i = 0; i < 8; ++i) f[i] = __builtin_fmaf(f[i], s, c);
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = (float)(((uint32_t)pv.v[i / 4] >> (8 * (i % 4))) & 0xffu);
+    for (int i = 0; i < 8; ++i) f[i] = (f[i] - off) * s;
   }
   Vec<typename ST::raw, 8> o;
   if constexpr (ST::id == CTMI_BF16) {
     Vec<uint32_t, 4> ow;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      ow.v[j] = pack_bf16x2((f[2 * j] - off) * s, (f[2 * j + 1] - off) * s);
+    for (int j = 0; j < 4; ++j) ow.v[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
     o = __builtin_bit_cast(Vec<uint16_t, 8>, ow);
   } else {
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o.v[i] = ST::from_f32((f[i] - off) * s);
+    for (int i = 0; i < 8; ++i) o.v[i] = ST::from_f32(f[i]);
   }
   return o;
 }

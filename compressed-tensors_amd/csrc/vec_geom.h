@@ -87,6 +87,9 @@ static inline bool vec_geometry(const ctmi_qparams* qp, int64_t rows, int64_t co
     } else {
       g->mode = 1;
     }
+  } else if (single_row && qp->s_cols == 1) {
+    g->mode = 0;  // one scale for everything: items are < 2^31, so the index is 0
+    g->shift = 31;
   }
   return true;
 }
