@@ -12,6 +12,7 @@
 
 #include <cstddef>
 #include <cstring>
+#include <type_traits>
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
@@ -209,7 +210,7 @@ __global__ void __launch_bounds__(256) pq_decompress_generic_kernel(FusedArgs a)
 // travels in the kernel arguments; a workgroup finds its tensor by a scan over
 // the running chunk counts (uniform, scalar registers).
 #ifndef CTMI_PQ_TUNING
-#define CTMI_PQ_TUNING 512, 4, 512, 1, 8
+#define CTMI_PQ_TUNING 512, 2, 512, 2, 8
 #endif
 constexpr int kPqTuning[5] = {CTMI_PQ_TUNING};
 constexpr int kCompressBlock = kPqTuning[0], kCompressUnroll = kPqTuning[1];
@@ -324,26 +325,37 @@ __global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const P
   const int8_t* __restrict__ zp = job.zp;
   int32_t* __restrict__ out = (int32_t*)job.dst;
   const uint32_t v0 = chunk * (B * U) + threadIdx.x;
-  Vec<typename XT::raw, 8> xv[U];
-  float sv[U], zv[U];
+  // A chunk that lies wholly inside its weight (all but the last one) runs
+  // without per-lane bounds checks: straight-line code, every load of the
+  // workgroup issued before the first value is looked at.
+  const bool full = (chunk + 1) * (uint32_t)(B * U) <= nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    Vec<typename XT::raw, 8> xv[U];
+    typename ST::raw sraw[U];
+    int8_t zraw[U];
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const uint32_t v = v0 + k * B;
-    if (v < nvec) {
-      xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
-      const uint32_t si = pq_scale_index<FLAT>(v, job);
-      sv[k] = ST::to_f32(scale[si]);
-      zv[k] = HAS_ZP ? (float)zp[si] : 0.0f;
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
+        const uint32_t si = pq_scale_index<FLAT>(v, job);
+        sraw[k] = scale[si];
+        if constexpr (HAS_ZP) zraw[k] = zp[si];
+      }
     }
-  }
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const uint32_t v = v0 + k * B;
-    if (v < nvec) {
-      stg_nt<int32_t, W>(out + (size_t)v * W,
-                         quant_pack8<XT, ST, BITS, HAS_ZP>(xv[k], sv[k], zv[k], t.qmin, t.qmax));
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        const float s = ST::to_f32(sraw[k]), z = HAS_ZP ? (float)zraw[k] : 0.0f;
+        stg_nt<int32_t, W>(out + (size_t)v * W,
+                           quant_pack8<XT, ST, BITS, HAS_ZP>(xv[k], s, z, t.qmin, t.qmax));
+      }
     }
-  }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
 }
 
 template <typename ST, int BITS, bool HAS_ZP, bool FLAT>
@@ -357,26 +369,34 @@ __global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(con
   const int8_t* __restrict__ zp = job.zp;
   auto* __restrict__ out = (typename ST::raw*)job.dst;
   const uint32_t v0 = chunk * (B * U) + threadIdx.x;
-  Vec<int32_t, W> pv[U];
-  float sv[U], zv[U];
+  const bool full = (chunk + 1) * (uint32_t)(B * U) <= nvec;  // see pq_compress_vec_kernel
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    Vec<int32_t, W> pv[U];
+    typename ST::raw sraw[U];
+    int8_t zraw[U];
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const uint32_t v = v0 + k * B;
-    if (v < nvec) {
-      pv[k] = ldg<int32_t, W>(packed + (size_t)v * W);
-      const uint32_t si = pq_scale_index<FLAT>(v, job);
-      sv[k] = ST::to_f32(scale[si]);
-      zv[k] = HAS_ZP ? (float)zp[si] : 0.0f;
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        pv[k] = ldg<int32_t, W>(packed + (size_t)v * W);
+        const uint32_t si = pq_scale_index<FLAT>(v, job);
+        sraw[k] = scale[si];
+        if constexpr (HAS_ZP) zraw[k] = zp[si];
+      }
     }
-  }
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const uint32_t v = v0 + k * B;
-    if (v < nvec) {
-      stg_nt<typename ST::raw, 8>(out + (size_t)v * 8,
-                                  unpack_dequant8<ST, BITS, HAS_ZP>(pv[k], sv[k], zv[k]));
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        const float s = ST::to_f32(sraw[k]), z = HAS_ZP ? (float)zraw[k] : 0.0f;
+        stg_nt<typename ST::raw, 8>(out + (size_t)v * 8,
+                                    unpack_dequant8<ST, BITS, HAS_ZP>(pv[k], s, z));
+      }
     }
-  }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
 }
 
 // key of a vectorised job: which template instance runs it

@@ -9,6 +9,8 @@
 // see quant_fast.h); fp8 codes use the hardware converters
 // (v_cvt_pk_fp8_f32 / v_cvt_f32_fp8: OCP e4m3, round-to-nearest-even), which the
 // GPU tests compare with torch's cast on every bf16 bit pattern.
+#include <type_traits>
+
 #include "ctmi_device.h"
 #include "ctmi_host.h"
 #include "quant_core.h"
@@ -54,94 +56,104 @@ qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict_
   constexpr bool DO_DQ = OUT == kKindFloat;
   using FR = typename FT::raw;
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
-  Vec<FR, 8> xf[U];
-  Vec<uint8_t, 8> xc[U];
-  float sv[U], zv[U];
+  // A chunk wholly inside the tensor (all but the last) runs without per-lane
+  // bounds checks: straight-line code, every load of the workgroup issued before
+  // the first loaded value is looked at.
+  const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    Vec<FR, 8> xf[U];
+    Vec<uint8_t, 8> xc[U];
+    FR sraw[U];
+    uint8_t zraw[U];
+    uint32_t si[U];
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const uint32_t v = v0 + k * B;
-    if (v < g.nvec) {
-      if constexpr (DO_Q) xf[k] = ldg_nt<FR, 8>((const FR*)xin + (size_t)v * 8);
-      else xc[k] = ldg_nt<uint8_t, 8>((const uint8_t*)xin + (size_t)v * 8);
-      const uint32_t si = scale_index(v, g);
-      sv[k] = FT::to_f32(scale[si]);
-      if constexpr (HAS_ZP) {
-        zv[k] = QK == 0 ? (float)(int8_t)zp[si] : f8e4m3_to_f32(zp[si]);
+    for (int k = 0; k < U; ++k) si[k] = scale_index(min(v0 + k * B, g.nvec - 1), g);
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
+        if constexpr (DO_Q) xf[k] = ldg_nt<FR, 8>((const FR*)xin + (size_t)v * 8);
+        else xc[k] = ldg_nt<uint8_t, 8>((const uint8_t*)xin + (size_t)v * 8);
+        sraw[k] = scale[si[k]];
+        if constexpr (HAS_ZP) zraw[k] = zp[si[k]];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (GUARD && v >= g.nvec) continue;
+      const float s = FT::to_f32(sraw[k]);
+      float z = 0.0f;
+      if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw[k] : f8e4m3_to_f32(zraw[k]);
+      float t[8];
+      uint32_t codes[2] = {0u, 0u};  // 8 one-byte codes
+      if constexpr (DO_Q) {
+        const bool fast = CT == CTMI_BF16 && wave_all(scale_is_tame(s));
+        const float r = __builtin_amdgcn_rcpf(s);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float a = FT::to_f32(xf[k].v[2 * j]), b = FT::to_f32(xf[k].v[2 * j + 1]);
+          if (fast) { a *= r; b *= r; } else { a /= s; b /= s; }
+          round2<CT>(a, b);
+          if (HAS_ZP) { a += z; b += z; round2<CT>(a, b); }
+          a = clamp_nan(a, qmin, qmax);
+          b = clamp_nan(b, qmin, qmax);
+          if constexpr (QK == 0) {
+            a = rintf(a);
+            b = rintf(b);
+            if constexpr (OUT == kKindI8) {
+              codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(a)) << (16 * (j % 2));
+              codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(b)) << (16 * (j % 2) + 8);
+            }
+          } else {
+            // two fp8 codes into the low or high half of the word
+            if (j % 2 == 0) codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], false);
+            else codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], true);
+            if constexpr (DO_DQ) {
+              a = fp8_hw_decode(codes[j / 2], 2 * (j % 2));
+              b = fp8_hw_decode(codes[j / 2], 2 * (j % 2) + 1);
+            }
+          }
+          t[2 * j] = a;
+          t[2 * j + 1] = b;
+        }
       } else {
-        zv[k] = 0.0f;
-      }
-    }
-  }
+        const Vec<uint32_t, 2> w = __builtin_bit_cast(Vec<uint32_t, 2>, xc[k]);
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const uint32_t v = v0 + k * B;
-    if (v >= g.nvec) continue;
-    const float s = sv[k], z = zv[k];
-    float t[8];
-    uint32_t codes[2] = {0u, 0u};  // 8 one-byte codes
-    if constexpr (DO_Q) {
-      const bool fast = CT == CTMI_BF16 && wave_all(scale_is_tame(s));
-      const float r = __builtin_amdgcn_rcpf(s);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float a = FT::to_f32(xf[k].v[2 * j]), b = FT::to_f32(xf[k].v[2 * j + 1]);
-        if (fast) { a *= r; b *= r; } else { a /= s; b /= s; }
-        round2<CT>(a, b);
-        if (HAS_ZP) { a += z; b += z; round2<CT>(a, b); }
-        a = clamp_nan(a, qmin, qmax);
-        b = clamp_nan(b, qmin, qmax);
-        if constexpr (QK == 0) {
-          a = rintf(a);
-          b = rintf(b);
-          if constexpr (OUT == kKindI8) {
-            codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(a)) << (16 * (j % 2));
-            codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(b)) << (16 * (j % 2) + 8);
-          }
-        } else {
-          // two fp8 codes into the low or high half of the word
-          if (j % 2 == 0) codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], false);
-          else codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], true);
-          if constexpr (DO_DQ) {
-            a = fp8_hw_decode(codes[j / 2], 2 * (j % 2));
-            b = fp8_hw_decode(codes[j / 2], 2 * (j % 2) + 1);
-          }
-        }
-        t[2 * j] = a;
-        t[2 * j + 1] = b;
-      }
-    } else {
-      const Vec<uint32_t, 2> w = __builtin_bit_cast(Vec<uint32_t, 2>, xc[k]);
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        if constexpr (IN == kKindI8) t[i] = (float)(int8_t)((w.v[i / 4] >> (8 * (i % 4))) & 0xffu);
-        else t[i] = fp8_hw_decode(w.v[i / 4], i % 4);
-      }
-    }
-    if constexpr (DO_DQ) {
-      Vec<FR, 8> o;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float a = t[2 * j], b = t[2 * j + 1];
-        if (HAS_ZP) { a -= z; b -= z; round2<CT>(a, b); }
-        a *= s;
-        b *= s;
-        if constexpr (CT == CTMI_BF16) {
-          const uint32_t p = pack_bf16x2(a, b);
-          o.v[2 * j] = (uint16_t)(p & 0xffffu);
-          o.v[2 * j + 1] = (uint16_t)(p >> 16);
-        } else {
-          o.v[2 * j] = FT::from_f32(a);
-          o.v[2 * j + 1] = FT::from_f32(b);
+        for (int i = 0; i < 8; ++i) {
+          if constexpr (IN == kKindI8) t[i] = (float)(int8_t)((w.v[i / 4] >> (8 * (i % 4))) & 0xffu);
+          else t[i] = fp8_hw_decode(w.v[i / 4], i % 4);
         }
       }
-      stg_nt<FR, 8>((FR*)yout + (size_t)v * 8, o);
-    } else {
-      Vec<uint32_t, 2> w;
-      w.v[0] = codes[0];
-      w.v[1] = codes[1];
-      stg_nt<uint8_t, 8>((uint8_t*)yout + (size_t)v * 8, __builtin_bit_cast(Vec<uint8_t, 8>, w));
+      if constexpr (DO_DQ) {
+        Vec<FR, 8> o;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          float a = t[2 * j], b = t[2 * j + 1];
+          if (HAS_ZP) { a -= z; b -= z; round2<CT>(a, b); }
+          a *= s;
+          b *= s;
+          if constexpr (CT == CTMI_BF16) {
+            const uint32_t p = pack_bf16x2(a, b);
+            o.v[2 * j] = (uint16_t)(p & 0xffffu);
+            o.v[2 * j + 1] = (uint16_t)(p >> 16);
+          } else {
+            o.v[2 * j] = FT::from_f32(a);
+            o.v[2 * j + 1] = FT::from_f32(b);
+          }
+        }
+        stg_nt<FR, 8>((FR*)yout + (size_t)v * 8, o);
+      } else {
+        Vec<uint32_t, 2> w;
+        w.v[0] = codes[0];
+        w.v[1] = codes[1];
+        stg_nt<uint8_t, 8>((uint8_t*)yout + (size_t)v * 8, __builtin_bit_cast(Vec<uint8_t, 8>, w));
+      }
     }
-  }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
 }
 
 template <typename FT, int IN, int OUT, int QK>
