@@ -22,6 +22,7 @@
 // lane access on consecutive addresses.
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "quant_fast.h"
 
 namespace ctmi {
 
@@ -30,6 +31,9 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kHadThreads = 256;
 constexpr int kHadWaves = kHadThreads / kWave;
+#ifndef CTMI_HAD_KRON_WAVES
+#define CTMI_HAD_KRON_WAVES 2  // waves per SIMD the kernel for 64 x 64 is built for (measured best)
+#endif
 
 struct HadArgs {
   const void* x;
@@ -224,6 +228,335 @@ __global__ void __launch_bounds__(kHadThreads) hadamard_mfma_kernel(HadArgs a) {
   }
 }
 
+// ---------------------------------------------------------------- block sizes up to 128, bf16, no LDS
+// One wavefront owns 16 sub-rows at a time and never talks to another wave.
+// Accesses are plain (not streaming) ones: a lane group touches half a cache
+// line per instruction and the other half with the next, which the streaming
+// hint turns into two trips to memory.
+// With D^T = Mb^T * X^T on v_mfma_f32_16x16x32_bf16 the operand layouts line up
+// with memory on both sides:
+//   B operand (X^T): lane (i + 16 q) holds X[row i][32 ks + 8 q .. + 8], one
+//                    16-byte global load;
+//   A operand:       rows of Mb^T, fetched once per wave and kept in registers
+//                    for every tile the wave handles, with the signs folded in
+//                    (row c times sign_out[c], column k times sign_in[k]);
+//   D^T:             lane (i + 16 jq) holds 4 output columns of row i.  Which 4
+//                    is a matter of labelling the rows of the A operand: tiles
+//                    2p and 2p+1 are given the columns 32 p + 8 jq + {0..3} and
+//                    + {4..7}, so a lane ends up with 8 neighbouring outputs,
+//                    one 16-byte global store.
+// Sign vectors are used as signs: their entries must be +1 or -1.
+template <int B>
+__global__ void __launch_bounds__(kHadThreads)
+hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
+                     const uint16_t* __restrict__ mbt, const float* __restrict__ s_in,
+                     const float* __restrict__ s_out, int64_t n_sub, float inv_sqrt_n) {
+  constexpr int KS = B / 32;  // k steps
+  constexpr int NP = B / 32;  // pairs of 16-column output tiles
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: loop control stays scalar
+  const int l16 = lane & 15, lq = lane >> 4;
+
+  // The matrix fragments are the same in every wave of the workgroup: each wave
+  // fetches a quarter of them, and all pick up the whole set from LDS.
+  __shared__ u32x4_t frag_lds[2 * NP * KS][kWave];
+  for (int f = wave; f < 2 * NP * KS; f += kHadWaves) {
+    const int nt = f / KS, ks = f % KS;
+    const int col = 32 * (nt / 2) + 8 * (l16 / 4) + 4 * (nt % 2) + (l16 % 4);
+    frag_lds[f][lane] = *reinterpret_cast<const u32x4_t*>(mbt + col * B + 32 * ks + 8 * lq);
+  }
+  __syncthreads();
+  bf16x8_t mb[2 * NP][KS];
+#pragma unroll
+  for (int nt = 0; nt < 2 * NP; ++nt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      mb[nt][ks] = __builtin_bit_cast(bf16x8_t, frag_lds[nt * KS + ks][lane]);
+  if (s_in || s_out) {
+    // Sign bits, XORed into the fragments (bit 15 of each half word).  An absent
+    // vector reads the matrix instead (any valid address) and is masked out: no
+    // branches, so these loads overlap too.
+    const uint32_t* pin = reinterpret_cast<const uint32_t*>(s_in ? (const void*)s_in : (const void*)mbt);
+    const uint32_t* pout = reinterpret_cast<const uint32_t*>(s_out ? (const void*)s_out : (const void*)mbt);
+    const uint32_t use_in = s_in ? 1u : 0u, use_out = s_out ? 0x80008000u : 0u;
+    uint32_t raw_in[KS][8], raw_out[2 * NP];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) raw_in[ks][e] = pin[32 * ks + 8 * lq + e];
+#pragma unroll
+    for (int nt = 0; nt < 2 * NP; ++nt)
+      raw_out[nt] = pout[32 * (nt / 2) + 8 * (l16 / 4) + 4 * (nt % 2) + (l16 % 4)];
+#pragma unroll
+    for (int nt = 0; nt < 2 * NP; ++nt) {
+      const uint32_t fo = (raw_out[nt] >> 31) * use_out;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        Vec<uint32_t, 4> m = __builtin_bit_cast(Vec<uint32_t, 4>, mb[nt][ks]);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t lo = (raw_in[ks][2 * w] >> 31) & use_in, hi = (raw_in[ks][2 * w + 1] >> 31) & use_in;
+          m.v[w] ^= ((lo << 15) | (hi << 31)) ^ fo;
+        }
+        mb[nt][ks] = __builtin_bit_cast(bf16x8_t, m);
+      }
+    }
+  }
+
+  const int64_t n_full = n_sub / 16;  // whole groups of 16 sub-rows
+  const int64_t stride = (int64_t)gridDim.x * kHadWaves;
+  const int64_t first = (int64_t)blockIdx.x * kHadWaves + wave;
+
+  // Loads are never conditional (a group past the end re-reads the last whole
+  // one) and the stores of whole groups are not either: with a fixed number of
+  // memory operations per step the waits can say exactly how many newer
+  // operations may still be in flight.
+  auto load_group = [&](int64_t grp, bf16x8_t* xf) {
+    if (grp >= n_full) grp = n_full - 1;
+    const uint16_t* src = x + (grp * 16 + l16) * B + 8 * lq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      xf[ks] = __builtin_bit_cast(bf16x8_t, ldg<uint16_t, 8>(src + 32 * ks));
+  };
+  auto transform_rows = [&](const bf16x8_t* xf, uint16_t* dst, bool keep) {
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      f32x4_t a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p][ks], xf[ks], a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p + 1][ks], xf[ks], a1, 0, 0, 0);
+      }
+      Vec<uint32_t, 4> o;
+      o.v[0] = pack_bf16x2(a0[0] * inv_sqrt_n, a0[1] * inv_sqrt_n);
+      o.v[1] = pack_bf16x2(a0[2] * inv_sqrt_n, a0[3] * inv_sqrt_n);
+      o.v[2] = pack_bf16x2(a1[0] * inv_sqrt_n, a1[1] * inv_sqrt_n);
+      o.v[3] = pack_bf16x2(a1[2] * inv_sqrt_n, a1[3] * inv_sqrt_n);
+      if (keep) stg<uint16_t, 8>(dst + 32 * p, __builtin_bit_cast(Vec<uint16_t, 8>, o));
+    }
+  };
+  auto transform_group = [&](int64_t grp, const bf16x8_t* xf) {
+    transform_rows(xf, out + (grp * 16 + l16) * B + 8 * lq, true);
+  };
+
+  if (first < n_full) {
+    // Software pipeline one group ahead, two register sets taking turns (no
+    // copies).  The first group is handled ahead of the loop so that the loop is
+    // entered with the same operations in flight as on its back edge (one set's
+    // loads, then a group's stores): a wait for loads then never has to cover
+    // the stores issued after them, which would cost a store latency per group.
+    bf16x8_t xa[KS], xb[KS];
+    int64_t g = first;
+    load_group(g, xa);
+    load_group(g + stride, xb);
+    transform_group(g, xa);
+    g += stride;
+    while (g < n_full) {  // invariant: group g is in xb
+      load_group(g + stride, xa);
+      transform_group(g, xb);
+      g += stride;
+      if (g >= n_full) break;
+      load_group(g + stride, xb);
+      transform_group(g, xa);
+      g += stride;
+    }
+  }
+  // the ragged last group (fewer than 16 sub-rows), by the wave whose turn it is
+  if (n_sub % 16 != 0 && n_full % stride == first) {
+    int64_t row = n_full * 16 + l16;
+    const bool keep = row < n_sub;
+    if (!keep) row = n_sub - 1;
+    bf16x8_t xt[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      xt[ks] = __builtin_bit_cast(bf16x8_t, ldg<uint16_t, 8>(x + row * B + 8 * lq + 32 * ks));
+    transform_rows(xt, out + row * B + 8 * lq, keep);
+  }
+}
+
+template <int B>
+static int launch_had_rows(const HadArgs& a, hipStream_t st) {
+  const int64_t groups = cdiv(a.n_sub, 16);
+  const int64_t wgs = cdiv(groups, kHadWaves);
+  // a wave keeps the matrix in registers: give it several groups to use it on
+  // (as many workgroups as fit on the chip at once: 2 per CU at 128, where a wave
+  // needs some 190 registers, more below)
+  const int64_t cap = 256 * (B == 32 ? 4 : 2);
+  const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
+  hipLaunchKernelGGL(hadamard_rows_kernel<B>, grid, kHadThreads, 0, st, (const uint16_t*)a.x,
+                     (uint16_t*)a.out, a.mbt, a.s_in, a.s_out, a.n_sub, 1.0f / a.sqrt_n);
+  return CTMI_OK;
+}
+
+// ---------------------------------------------------------------- Kronecker sizes, bf16, no LDS staging
+// n = A * B (1024 = 32 x 32, 2048 = 32 x 64, 4096 = 64 x 64): one wavefront per
+// data row, the row viewed as X [A sub-rows][B].  Both stages run on
+// v_mfma_f32_16x16x32_bf16 with operands that never leave the registers:
+//
+//   stage 1   T = X * Mb.  A operand = X: lane (i + 16 q) holds 8 neighbouring
+//             elements of a sub-row (one 16-byte global load); B operand = Mb,
+//             kept in registers.  The result tile has lane (j + 16 iq) holding 4
+//             sub-rows of column j.  Sub-rows are handed to the row labels of
+//             two tiles so that these come out as 8 neighbouring sub-rows
+//             32 P + 8 iq + {0..7}: exactly the 8 k-values a lane supplies to
+//             the next product.
+//   stage 2   Y^T = T^T * Ma, i.e. D[c][a'] = sum_a T[a][c] Ma[a][a'].  A operand
+//             = the T values just computed (fp32 split into three bf16 terms, so
+//             the contraction is fp32-accurate), B operand = Ma, in registers.
+//             Lane (a' + 16 cq) ends up with 4 columns of output sub-row a';
+//             columns are handed to the column labels of stage 1 so that two
+//             tiles give 8 neighbouring columns: one 16-byte global store.
+//
+// Signs (entries +1 / -1) are XOR masks on the bf16 sign bits of X and of the
+// output; they are per position within the row, the same for every row, and sit
+// in LDS in the lanes' own layout.
+template <int A, int B>
+__global__ void __launch_bounds__(kHadThreads) __attribute__((amdgpu_waves_per_eu(CTMI_HAD_KRON_WAVES)))
+hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
+                     const uint16_t* __restrict__ mbt, const uint16_t* __restrict__ mat,
+                     const float* __restrict__ s_in, const float* __restrict__ s_out,
+                     int64_t n_rows, float inv_sqrt_n) {
+  constexpr int N = A * B;
+  constexpr int KS = B / 32;   // k steps of stage 1
+  constexpr int MT = A / 16;   // sub-row tiles
+  constexpr int NT = B / 16;   // column tiles
+  constexpr int PS = A / 32;   // k steps of stage 2 (pairs of sub-row tiles)
+  constexpr int AT = A / 16;   // output sub-row tiles
+  constexpr int NSPLIT = 3;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & 15, lq = lane >> 4;
+  const int perm = 8 * (l16 / 4) + (l16 % 4);  // label -> position within a pair of tiles
+
+  __shared__ u32x4_t sign_in_lds[MT * KS][kWave];
+  __shared__ u32x4_t sign_out_lds[AT * (NT / 2)][kWave];
+  const bool signed_io = s_in || s_out;
+  if (signed_io) {
+    const uint32_t* pin = reinterpret_cast<const uint32_t*>(s_in ? (const void*)s_in : (const void*)mbt);
+    const uint32_t* pout = reinterpret_cast<const uint32_t*>(s_out ? (const void*)s_out : (const void*)mbt);
+    const uint32_t use_in = s_in ? 1u : 0u, use_out = s_out ? 1u : 0u;
+    for (int f = wave; f < MT * KS; f += kHadWaves) {
+      const int m = f / KS, ks = f % KS;
+      const int pos = (32 * (m / 2) + 4 * (m % 2) + perm) * B + 32 * ks + 8 * lq;
+      u32x4_t w;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        w[d] = (((pin[pos + 2 * d] >> 31) & use_in) << 15) | (((pin[pos + 2 * d + 1] >> 31) & use_in) << 31);
+      sign_in_lds[f][lane] = w;
+    }
+    for (int f = wave; f < AT * (NT / 2); f += kHadWaves) {
+      const int at = f / (NT / 2), p = f % (NT / 2);
+      const int pos = (16 * at + l16) * B + 32 * p + 8 * lq;
+      u32x4_t w;
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+        w[d] = (((pout[pos + 2 * d] >> 31) & use_out) << 15) | (((pout[pos + 2 * d + 1] >> 31) & use_out) << 31);
+      sign_out_lds[f][lane] = w;
+    }
+    __syncthreads();
+  }
+
+  // the two small matrices, as B operands
+  bf16x8_t mbf[NT][KS], maf[AT][PS];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      mbf[nt][ks] = __builtin_bit_cast(
+          bf16x8_t, ldg<uint16_t, 8>(mbt + (32 * (nt / 2) + 4 * (nt % 2) + perm) * B + 32 * ks + 8 * lq));
+#pragma unroll
+  for (int at = 0; at < AT; ++at)
+#pragma unroll
+    for (int ps = 0; ps < PS; ++ps)
+      maf[at][ps] = __builtin_bit_cast(
+          bf16x8_t, ldg<uint16_t, 8>(mat + (16 * at + l16) * A + 32 * ps + 8 * lq));
+
+  const int64_t stride = (int64_t)gridDim.x * kHadWaves;
+  for (int64_t row = (int64_t)blockIdx.x * kHadWaves + wave; row < n_rows; row += stride) {
+    const uint16_t* src = x + row * N;
+    uint16_t* dst = out + row * N;
+    bf16x8_t xf[MT][KS];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        xf[m][ks] = __builtin_bit_cast(
+            bf16x8_t,
+            ldg<uint16_t, 8>(src + (32 * (m / 2) + 4 * (m % 2) + perm) * B + 32 * ks + 8 * lq));
+    if (signed_io) {
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const u32x4_t f = sign_in_lds[m * KS + ks][lane];
+          xf[m][ks] = __builtin_bit_cast(bf16x8_t, __builtin_bit_cast(u32x4_t, xf[m][ks]) ^ f);
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < NT / 2; ++p) {
+      // ---- stage 1 for column tiles 2p and 2p+1, split for stage 2
+      bf16x8_t tf[2][PS][NSPLIT];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int nt = 2 * p + h;
+#pragma unroll
+        for (int ps = 0; ps < PS; ++ps) {
+          f32x4_t lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[2 * ps][ks], mbf[nt][ks], lo, 0, 0, 0);
+            hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[2 * ps + 1][ks], mbf[nt][ks], hi, 0, 0, 0);
+          }
+          float t[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+          u32x4_t parts[NSPLIT];
+#pragma unroll
+          for (int sp = 0; sp < NSPLIT; ++sp) {
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const uint32_t w = pack_bf16x2(t[2 * d], t[2 * d + 1]);
+              parts[sp][d] = w;
+              t[2 * d] -= bf16_lo(w);
+              t[2 * d + 1] -= bf16_hi(w);
+            }
+            tf[h][ps][sp] = __builtin_bit_cast(bf16x8_t, parts[sp]);
+          }
+        }
+      }
+      // ---- stage 2: every output sub-row tile for these 32 columns
+#pragma unroll
+      for (int at = 0; at < AT; ++at) {
+        f32x4_t y0 = {0.0f, 0.0f, 0.0f, 0.0f}, y1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ps = 0; ps < PS; ++ps)
+#pragma unroll
+          for (int sp = NSPLIT - 1; sp >= 0; --sp) {  // small terms first
+            y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf[0][ps][sp], maf[at][ps], y0, 0, 0, 0);
+            y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf[1][ps][sp], maf[at][ps], y1, 0, 0, 0);
+          }
+        u32x4_t o;
+        o[0] = pack_bf16x2(y0[0] * inv_sqrt_n, y0[1] * inv_sqrt_n);
+        o[1] = pack_bf16x2(y0[2] * inv_sqrt_n, y0[3] * inv_sqrt_n);
+        o[2] = pack_bf16x2(y1[0] * inv_sqrt_n, y1[1] * inv_sqrt_n);
+        o[3] = pack_bf16x2(y1[2] * inv_sqrt_n, y1[3] * inv_sqrt_n);
+        if (signed_io) o ^= sign_out_lds[at * (NT / 2) + p][lane];
+        stg<uint16_t, 8>(dst + (16 * at + l16) * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o));
+      }
+    }
+  }
+}
+
+template <int A, int B>
+static int launch_had_kron(const HadArgs& a, hipStream_t st) {
+  const int64_t n_rows = a.n_sub / A;
+  const int64_t wgs = cdiv(n_rows, kHadWaves);
+  // as many workgroups as are resident at once (register-limited)
+  const int64_t cap = 256 * (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES));
+  const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
+  hipLaunchKernelGGL((hadamard_kron_kernel<A, B>), grid, kHadThreads, 0, st, (const uint16_t*)a.x,
+                     (uint16_t*)a.out, a.mbt, a.mat, a.s_in, a.s_out, n_rows, 1.0f / a.sqrt_n);
+  return CTMI_OK;
+}
+
 // ---------------------------------------------------------------- any small dense matrix (VALU)
 // y[r, g*h + j] = sum_k x[r, g*h + k] * w[k, j] / sqrt_n for an explicit fp32
 // h x h matrix: covers sizes and matrices the MFMA path does not (h < 32,
@@ -321,7 +654,16 @@ extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, i
   a.sqrt_n = sqrtf((float)n);
   hipStream_t st = (hipStream_t)stream;
   int rc;
-  if (io_dtype == CTMI_BF16) rc = dispatch_had<BF16>(a_dim, b_dim, a, st);
+  if (io_dtype == CTMI_BF16 && a_dim == 1) {
+    rc = b_dim == 32 ? launch_had_rows<32>(a, st)
+                     : (b_dim == 64 ? launch_had_rows<64>(a, st) : launch_had_rows<128>(a, st));
+  } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 32) {
+    rc = launch_had_kron<32, 32>(a, st);
+  } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 64) {
+    rc = launch_had_kron<32, 64>(a, st);
+  } else if (io_dtype == CTMI_BF16 && a_dim == 64 && b_dim == 64) {
+    rc = launch_had_kron<64, 64>(a, st);
+  } else if (io_dtype == CTMI_BF16) rc = dispatch_had<BF16>(a_dim, b_dim, a, st);
   else if (io_dtype == CTMI_F16) rc = dispatch_had<F16>(a_dim, b_dim, a, st);
   else rc = dispatch_had<F32>(a_dim, b_dim, a, st);
   if (rc) return rc;
