@@ -184,6 +184,173 @@ observe_rows_kernel(const typename XT::raw* __restrict__ x, const float* gscale,
   }
 }
 
+// ---- streaming forms of stage 1 (+ calculate_qparams) for 16-byte-aligned tensors whose
+// segments are whole numbers of 8-element vectors and tile the rows exactly.
+// Memory is then one run of vectors, numbered like the segments.  Both kernels
+// issue every load of a workgroup's share before looking at any value, one
+// workgroup per share (no grid-stride loop).
+struct ObserveOut {
+  void* scale;   // NULL: min/max only
+  void* zp;
+  void* mn;
+  void* mx;
+};
+
+// min / max of 8 elements folded into lo / hi with the hardware's 3-operand min
+// and max (which skip NaNs); `unordered` collects whether a NaN was seen, for the
+// caller to put back (torch's amin / amax propagate it).
+template <typename XT>
+__device__ __forceinline__ void vec_minmax(const Vec<typename XT::raw, 8>& a, float* lo, float* hi,
+                                           bool* unordered) {
+#pragma unroll
+  for (int j = 0; j < 8; j += 2) {
+    const float f0 = XT::to_f32(a.v[j]), f1 = XT::to_f32(a.v[j + 1]);
+    *lo = __builtin_fminf(__builtin_fminf(*lo, f0), f1);
+    *hi = __builtin_fmaxf(__builtin_fmaxf(*hi, f0), f1);
+    *unordered |= __builtin_isunordered(f0, f1);
+  }
+}
+
+// one step of a min / max reduction over neighbouring lanes, on the data-parallel
+// permute path of the vector ALU (no LDS traffic): CTRL names the lane exchange
+template <int CTRL>
+__device__ __forceinline__ void dpp_minmax_step(float* lo, float* hi) {
+  const float l = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, *lo), CTRL, 0xf, 0xf, false));
+  const float h = __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, *hi), CTRL, 0xf, 0xf, false));
+  *lo = __builtin_fminf(*lo, l);
+  *hi = __builtin_fmaxf(*hi, h);
+}
+
+// all-reduce over aligned groups of L lanes (L a power of two <= 64)
+__device__ __forceinline__ void group_minmax(int L, float* lo, float* hi) {
+  if (L >= 2) dpp_minmax_step<0xB1>(lo, hi);   // quad_perm [1,0,3,2]
+  if (L >= 4) dpp_minmax_step<0x4E>(lo, hi);   // quad_perm [2,3,0,1]
+  if (L >= 8) dpp_minmax_step<0x141>(lo, hi);  // row_half_mirror
+  if (L >= 16) dpp_minmax_step<0x140>(lo, hi); // row_mirror
+  for (int d = 16; d < L; d <<= 1) {
+    *lo = __builtin_fminf(__shfl_xor(*lo, d, kWave), *lo);
+    *hi = __builtin_fmaxf(__shfl_xor(*hi, d, kWave), *hi);
+  }
+}
+
+// did any lane of this lane's group of L see a NaN?
+__device__ __forceinline__ bool group_any(int L, bool flag) {
+  const uint64_t m = __builtin_amdgcn_ballot_w64(flag);
+  const uint64_t group = L >= 64 ? ~0ull : (((1ull << L) - 1) << (lane_id() & ~(L - 1)));
+  return (m & group) != 0;
+}
+
+template <typename XT>
+__device__ __forceinline__ void emit_segment(const ObserveOut& o, int64_t s, float lo, float hi,
+                                             float gs, const QpCfg& c) {
+  if (o.scale) {
+    float sv, zv;
+    qparams_value(lo, hi, gs, c, &sv, &zv);
+    store_from_f32(o.scale, c.scale_dtype, s, sv);
+    if (o.zp) store_from_f32(o.zp, c.zp_dtype, s, zv);
+  }
+  if (o.mn) ((typename XT::raw*)o.mn)[s] = XT::from_f32(lo);
+  if (o.mx) ((typename XT::raw*)o.mx)[s] = XT::from_f32(hi);
+}
+
+constexpr int kObsUnroll = 4;
+
+// L vectors per segment, L a power of two <= 64: L neighbouring lanes own a segment
+template <typename XT>
+__global__ void __launch_bounds__(256)
+observe_flat_kernel(const typename XT::raw* __restrict__ x, const float* gscale, ObserveOut o,
+                    int64_t nvec, int L, QpCfg c) {
+  constexpr int U = kObsUnroll;
+  const float gs = gscale ? gscale[0] : 1.0f;
+  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  Vec<typename XT::raw, 8> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    // past the end: re-read the last vector (nothing is emitted for it)
+    const int64_t v = v0 + k * 256;
+    a[k] = ldg<typename XT::raw, 8>(x + (v < nvec ? v : nvec - 1) * 8);
+  }
+  // The segments' results go through LDS so that the scale arithmetic and the
+  // stores run on full wavefronts, one segment per lane, instead of on one lane
+  // in L.  A workgroup covers 256 * U vectors = 256 * U / L whole segments.
+  __shared__ float seg_lo[256 * U], seg_hi[256 * U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    bool unordered = false;
+    vec_minmax<XT>(a[k], &lo, &hi, &unordered);
+    group_minmax(L, &lo, &hi);
+    if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
+    if ((threadIdx.x & (L - 1)) == 0) {
+      const int slot = (k * 256 + threadIdx.x) / L;
+      seg_lo[slot] = lo;
+      seg_hi[slot] = hi;
+    }
+  }
+  __syncthreads();
+  const int per_wg = 256 * U / L;
+  const int64_t first = (int64_t)blockIdx.x * per_wg, n_seg = nvec / L;
+  for (int i = threadIdx.x; i < per_wg && first + i < n_seg; i += 256)
+    emit_segment<XT>(o, first + i, seg_lo[i], seg_hi[i], gs, c);
+}
+
+// more than 64 vectors per segment: one wavefront per segment
+template <typename XT>
+__global__ void __launch_bounds__(256)
+observe_wide_kernel(const typename XT::raw* __restrict__ x, const float* gscale, ObserveOut o,
+                    int64_t n_segments, int64_t items, QpCfg c) {
+  constexpr int U = 8;
+  const float gs = gscale ? gscale[0] : 1.0f;
+  const int lane = threadIdx.x & 63;
+  const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (s >= n_segments) return;
+  const typename XT::raw* p = x + s * items * 8;
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  bool unordered = false;
+  for (int64_t t = 0; t < items; t += 64 * U) {
+    Vec<typename XT::raw, 8> a[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      // min / max do not mind seeing an element twice: no bounds branches
+      const int64_t i = t + k * 64 + lane;
+      a[k] = ldg<typename XT::raw, 8>(p + (i < items ? i : items - 1) * 8);
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) vec_minmax<XT>(a[k], &lo, &hi, &unordered);
+  }
+  group_minmax(64, &lo, &hi);
+  if (group_any(64, unordered)) lo = hi = __builtin_nanf("");
+  if (lane == 0) emit_segment<XT>(o, s, lo, hi, gs, c);
+}
+
+// launches a streaming form if the geometry allows; false = nothing launched
+template <typename XT>
+static bool observe_streaming(const void* x, const float* gscale, const ObserveOut& o,
+                              const SegGeom& g, const QpCfg& c, hipStream_t st) {
+  if (!g.vec || g.cols % g.seg_cols != 0) return false;
+  const int64_t items = g.seg_cols / 8;
+  const int64_t nvec = g.rows * g.cols / 8;
+  const int64_t n_segments = g.rows * g.n_seg;
+  using R = typename XT::raw;
+  if (items <= 64 && (items & (items - 1)) == 0) {
+    const int64_t blocks = cdiv(nvec, 256 * kObsUnroll);
+    if (blocks >= (1ll << 31)) return false;
+    hipLaunchKernelGGL(observe_flat_kernel<XT>, (unsigned)blocks, 256, 0, st, (const R*)x, gscale, o,
+                       nvec, (int)items, c);
+    return true;
+  }
+  if (items > 64) {
+    const int64_t blocks = cdiv(n_segments, 4);
+    if (blocks >= (1ll << 31)) return false;
+    hipLaunchKernelGGL(observe_wide_kernel<XT>, (unsigned)blocks, 256, 0, st, (const R*)x, gscale, o,
+                       n_segments, items, c);
+    return true;
+  }
+  return false;
+}
+
 // stage 2: fold `blk_rows` consecutive rows of a [rows, n_seg] min/max table;
 // one workgroup per output cell
 template <typename XT>
@@ -329,10 +496,14 @@ extern "C" int ctmi_minmax(const void* x, int32_t x_dtype, int64_t rows, int64_t
   SegGeom g;
   seg_geometry(&g, x, dtype_size(x_dtype), rows, cols, blk_cols);
   const int grid = seg_grid(g);
+  QpCfg none{};
   if (blk_rows == 1) {
-    CTMI_DISPATCH_XT(x_dtype, hipLaunchKernelGGL(minmax_rows_kernel<XT>, grid, 256, 0, st,
-                                                 (const XT::raw*)x, (XT::raw*)min_out,
-                                                 (XT::raw*)max_out, g));
+    const ObserveOut o{nullptr, nullptr, min_out, max_out};
+    CTMI_DISPATCH_XT(x_dtype, {
+      if (!observe_streaming<XT>(x, nullptr, o, g, none, st))
+        hipLaunchKernelGGL(minmax_rows_kernel<XT>, grid, 256, 0, st, (const XT::raw*)x,
+                           (XT::raw*)min_out, (XT::raw*)max_out, g);
+    });
     return check_launch("ctmi_minmax");
   }
   const int64_t out_rows = cdiv(rows, blk_rows);
@@ -340,9 +511,11 @@ extern "C" int ctmi_minmax(const void* x, int32_t x_dtype, int64_t rows, int64_t
   const int es = dtype_size(x_dtype);
   void* tmn = tmp;
   void* tmx = (char*)tmp + rows * g.n_seg * es;
+  const ObserveOut stage1{nullptr, nullptr, tmn, tmx};
   CTMI_DISPATCH_XT(x_dtype, {
-    hipLaunchKernelGGL(minmax_rows_kernel<XT>, grid, 256, 0, st, (const XT::raw*)x, (XT::raw*)tmn,
-                       (XT::raw*)tmx, g);
+    if (!observe_streaming<XT>(x, nullptr, stage1, g, none, st))
+      hipLaunchKernelGGL(minmax_rows_kernel<XT>, grid, 256, 0, st, (const XT::raw*)x,
+                         (XT::raw*)tmn, (XT::raw*)tmx, g);
     hipLaunchKernelGGL(minmax_fold_kernel<XT>, (int)(cells < 4096 ? cells : 4096), 256, 0, st,
                        (const XT::raw*)tmn, (const XT::raw*)tmx, (XT::raw*)min_out,
                        (XT::raw*)max_out, rows, g.n_seg, blk_rows, out_rows);
@@ -364,9 +537,12 @@ extern "C" int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows
   CTMI_REQUIRE(x && scale, CTMI_ERR_VALUE, "NULL tensor pointer");
   SegGeom g;
   seg_geometry(&g, x, dtype_size(x_dtype), rows, cols, blk_cols);
-  CTMI_DISPATCH_XT(x_dtype, hipLaunchKernelGGL(observe_rows_kernel<XT>, seg_grid(g), 256, 0,
-                                               (hipStream_t)stream, (const XT::raw*)x,
-                                               global_scale, scale, zero_point,
-                                               (XT::raw*)min_out, (XT::raw*)max_out, g, c));
+  const ObserveOut o{scale, zero_point, min_out, max_out};
+  CTMI_DISPATCH_XT(x_dtype, {
+    if (!observe_streaming<XT>(x, global_scale, o, g, c, (hipStream_t)stream))
+      hipLaunchKernelGGL(observe_rows_kernel<XT>, seg_grid(g), 256, 0, (hipStream_t)stream,
+                         (const XT::raw*)x, global_scale, scale, zero_point, (XT::raw*)min_out,
+                         (XT::raw*)max_out, g, c);
+  });
   return check_launch("ctmi_observe_qparams");
 }
