@@ -6,9 +6,12 @@
 //
 // Code = 3-bit index into {0,.5,1,1.5,2,3,4,6} | sign bit << 3; element 2j is
 // the low nibble of byte j, element 2j+1 the high nibble.
+#include <type_traits>
+
 #include "ctmi_device.h"
 #include "ctmi_host.h"
 #include "quant_core.h"
+#include "quant_fast.h"
 #include "vec_geom.h"
 
 namespace ctmi {
@@ -164,80 +167,233 @@ __global__ void __launch_bounds__(256) nvfp4_decompress_generic_kernel(Fp4Args a
 
 // ------------------------------------------------------------------ fused nvfp4, vectorised
 // fp8 e4m3 local scales + fp32 global scale; arithmetic in fp32 (bf16/fp16/fp32
-// input divided by an fp32 scale promotes to fp32).
+// input divided by an fp32 scale promotes to fp32).  One workgroup per chunk,
+// every load of a chunk issued before the first value is looked at; chunks that
+// lie wholly inside the tensor run without per-lane bounds checks.
+#ifndef CTMI_FP4_TUNING
+#define CTMI_FP4_TUNING 256, 1
+#endif
+constexpr int kFp4Tuning[2] = {CTMI_FP4_TUNING};
+constexpr int kFp4Block = kFp4Tuning[0], kFp4Unroll = kFp4Tuning[1];
+
+// 8 fp32 values -> 8 e2m1 codes (element i in bits [4i, 4i+4)) with the hardware
+// converter: round to nearest even on the e2m1 grid = the reference's bucket
+// boundaries (quant_args.py:55-68), saturating at +-6, sign kept.
+__device__ __forceinline__ uint32_t fp4_pack8_hw(const float* t) {
+  uint32_t w = 0;
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[0], t[1], 1.0f, 0);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[2], t[3], 1.0f, 1);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[4], t[5], 1.0f, 2);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[6], t[7], 1.0f, 3);
+  return w;
+}
+
+// 8 codes of a dword -> 8 fp32 values (exact; code 8 is -0.0)
+__device__ __forceinline__ void fp4_unpack8_hw(uint32_t w, float* t) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  f32x2 r;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0); t[0] = r.x; t[1] = r.y;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1); t[2] = r.x; t[3] = r.y;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2); t[4] = r.x; t[5] = r.y;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3); t[6] = r.x; t[7] = r.y;
+}
+
+// The reference's chain for 8 elements: x / s, + zp, clamp to +-6, cast_to_fp4
+// (forward.py:471-482, quant_args.py:55-68), one exact division per element.
 template <typename XT, bool HAS_ZP>
-__global__ void __launch_bounds__(256)
+__device__ __forceinline__ uint32_t nvfp4_codes_exact(const Vec<typename XT::raw, 8>& xv, float s,
+                                                      float z) {
+  uint32_t acc = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float t = XT::to_f32(xv.v[i]) / s;
+    if (HAS_ZP) t = t + z;
+    t = clamp_nan(t, -6.0f, 6.0f);
+    // sign of cast_to_fp4's product: exact zeros lose their sign
+    const uint32_t neg = (t < 0.0f) ? 8u : 0u;
+    acc |= ((uint32_t)fp4_bucket(fabsf(t)) | neg) << (4 * i);
+  }
+  return acc;
+}
+
+// Same codes without the divisions.  The exact quotient q = x / s lies between
+// x * r_lo and x * r_hi, r = rcp(s) widened by 2^-20 either way (rcp and the
+// product are each good to 2^-23); rounding to e2m1 is monotonic, so when both
+// ends convert to the same code that is q's code.  Otherwise (about one value in
+// 10^5 sits that close to a boundary) the wavefront redoes the vector exactly.
+// fma(x, r, +0) instead of x * r turns a -0 quotient into +0, as the reference's
+// sign(0) = 0 does.  NaNs take the exact path.
+template <typename XT, bool HAS_ZP>
+__device__ __forceinline__ uint32_t nvfp4_codes(const Vec<typename XT::raw, 8>& xv, float s,
+                                                float z) {
+  const float r = __builtin_amdgcn_rcpf(s);
+  const float r_lo = r * 0.99999904632568359375f, r_hi = r * 1.00000095367431640625f;
+  float lo[8], hi[8];
+  bool ok = s >= 7.888609052210118e-31f && s <= 1.2676506002282294e30f;
+  // a zero point of zero (what symmetric schemes carry) only turns -0 into +0,
+  // which the fma below does as well; any other takes the exact path
+  if constexpr (HAS_ZP) ok &= z == 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; i += 2) {
+    const float x0 = XT::to_f32(xv.v[i]), x1 = XT::to_f32(xv.v[i + 1]);
+    ok &= !__builtin_isunordered(x0, x1);
+    lo[i] = __builtin_fmaf(x0, r_lo, 0.0f);
+    hi[i] = __builtin_fmaf(x0, r_hi, 0.0f);
+    lo[i + 1] = __builtin_fmaf(x1, r_lo, 0.0f);
+    hi[i + 1] = __builtin_fmaf(x1, r_hi, 0.0f);
+  }
+  const uint32_t c_lo = fp4_pack8_hw(lo), c_hi = fp4_pack8_hw(hi);
+  ok &= c_lo == c_hi;
+  if (wave_all(ok)) return c_lo;
+  return nvfp4_codes_exact<XT, HAS_ZP>(xv, s, z);
+}
+
+template <typename XT, bool HAS_ZP>
+__global__ void __launch_bounds__(kFp4Block)
 nvfp4_compress_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __restrict__ scale,
                           const uint8_t* __restrict__ zp, const float* __restrict__ gscale,
                           uint32_t* __restrict__ out, VecGeom g) {
+  constexpr int B = kFp4Block, U = kFp4Unroll;
   const float gs = gscale[0];
-  const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
-  for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
-    const uint32_t v0 = chunk * (256 * kU) + threadIdx.x;
-    Vec<typename XT::raw, 8> xv[kU];
-    float sv[kU], zv[kU];
+  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    uint32_t si[U];
 #pragma unroll
-    for (int k = 0; k < kU; ++k) {
-      const uint32_t v = v0 + k * 256;
-      if (v < g.nvec) {
-        xv[k] = ldg<typename XT::raw, 8>(x + (size_t)v * 8);
-        const uint32_t si = scale_index(v, g);
-        sv[k] = f8e4m3_to_f32(scale[si]) / gs;
+    for (int k = 0; k < U; ++k) si[k] = scale_index(min(v0 + k * B, g.nvec - 1), g);
+    Vec<typename XT::raw, 8> xv[U];
+    uint8_t sraw[U], zraw[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
+        xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
+        sraw[k] = scale[si[k]];
+        if constexpr (HAS_ZP) zraw[k] = zp[si[k]];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
+        const float s = f8e4m3_to_f32(sraw[k]) / gs;
         // zero_point.to(x.dtype): an fp8 value is exact in every wider float type
-        zv[k] = HAS_ZP ? f8e4m3_to_f32(zp[si]) : 0.0f;
+        const float z = HAS_ZP ? f8e4m3_to_f32(zraw[k]) : 0.0f;
+        __builtin_nontemporal_store(nvfp4_codes<XT, HAS_ZP>(xv[k], s, z), out + v);
       }
     }
-#pragma unroll
-    for (int k = 0; k < kU; ++k) {
-      const uint32_t v = v0 + k * 256;
-      if (v < g.nvec) {
-        uint32_t acc = 0;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          float t = XT::to_f32(xv[k].v[i]) / sv[k];
-          if (HAS_ZP) t = t + zv[k];
-          t = clamp_nan(t, -6.0f, 6.0f);
-          // sign of cast_to_fp4's product: exact zeros lose their sign
-          const uint32_t neg = (t < 0.0f) ? 8u : 0u;
-          acc |= ((uint32_t)fp4_bucket(fabsf(t)) | neg) << (4 * i);
-        }
-        out[v] = acc;
-      }
-    }
-  }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
 }
 
 template <typename OT>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(kFp4Block)
 nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* __restrict__ scale,
                             const float* __restrict__ gscale, typename OT::raw* __restrict__ out,
                             VecGeom g) {
+  constexpr int B = kFp4Block, U = kFp4Unroll;
   const float gs = gscale[0];
-  const uint32_t nchunk = (g.nvec + 256 * kU - 1) / (256 * kU);
-  for (uint32_t chunk = blockIdx.x; chunk < nchunk; chunk += gridDim.x) {
-    const uint32_t v0 = chunk * (256 * kU) + threadIdx.x;
-    uint32_t pv[kU];
-    float sv[kU];
+  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    uint32_t si[U];
 #pragma unroll
-    for (int k = 0; k < kU; ++k) {
-      const uint32_t v = v0 + k * 256;
-      if (v < g.nvec) {
+    for (int k = 0; k < U; ++k) si[k] = scale_index(min(v0 + k * B, g.nvec - 1), g);
+    uint32_t pv[U];
+    uint8_t sraw[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
         pv[k] = packed[v];
-        sv[k] = f8e4m3_to_f32(scale[scale_index(v, g)]) / gs;
+        sraw[k] = scale[si[k]];
       }
     }
 #pragma unroll
-    for (int k = 0; k < kU; ++k) {
-      const uint32_t v = v0 + k * 256;
-      if (v < g.nvec) {
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
+        const float s = f8e4m3_to_f32(sraw[k]) / gs;
+        float t[8];
+        fp4_unpack8_hw(pv[k], t);
         Vec<typename OT::raw, 8> o;
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          o.v[i] = OT::from_f32(fp4_decode((int)((pv[k] >> (4 * i)) & 15u)) * sv[k]);
-        stg<typename OT::raw, 8>(out + (size_t)v * 8, o);
+        for (int i = 0; i < 8; ++i) o.v[i] = OT::from_f32(t[i] * s);
+        stg_nt<typename OT::raw, 8>(out + (size_t)v * 8, o);
       }
     }
-  }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
+}
+
+// quantize + dequantize in one pass (fake_quantize of forward.py:150-189 for the
+// nvfp4 scheme): out = XT(e2m1(x / s) * s), s = fp32(scale) / global_scale
+template <typename XT>
+__global__ void __launch_bounds__(kFp4Block)
+nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __restrict__ scale,
+                     const float* __restrict__ gscale, typename XT::raw* __restrict__ out,
+                     VecGeom g) {
+  constexpr int B = kFp4Block, U = kFp4Unroll;
+  const float gs = gscale[0];
+  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    uint32_t si[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) si[k] = scale_index(min(v0 + k * B, g.nvec - 1), g);
+    Vec<typename XT::raw, 8> xv[U];
+    uint8_t sraw[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
+        xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
+        sraw[k] = scale[si[k]];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
+        const float s = f8e4m3_to_f32(sraw[k]) / gs;
+        float t[8];
+        fp4_unpack8_hw(nvfp4_codes<XT, false>(xv[k], s, 0.0f), t);
+        Vec<typename XT::raw, 8> o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float xi = XT::to_f32(xv[k].v[i]);
+          o.v[i] = XT::from_f32(xi != xi ? xi : t[i] * s);  // a NaN stays one (no code stands for it)
+        }
+        stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
+      }
+    }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
+}
+
+// fake-quantize entry for ctmi_qdq; false = not this kernel's case, nothing launched
+bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
+                              int64_t cols, const ctmi_qparams* qp, hipStream_t st) {
+  if (qp->qtype != CTMI_QTYPE_FLOAT || qp->num_bits != 4 || !qp->global_scale ||
+      qp->scale_dtype != CTMI_F8E4M3 || qp->zero_point || x_dtype != out_dtype)
+    return false;
+  if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16 && x_dtype != CTMI_F32) return false;
+  const int bytes = 8 * dtype_size(x_dtype);
+  if ((uintptr_t)x % bytes || (uintptr_t)out % bytes) return false;
+  VecGeom g;
+  if (!vec_geometry(qp, rows, cols, &g, true)) return false;
+  const int64_t grid = cdiv(g.nvec, kFp4Block * kFp4Unroll);
+  const auto* sc = (const uint8_t*)qp->scale;
+  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
+  else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
+  else hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, sc, qp->global_scale, (float*)out, g);
+  return true;
 }
 
 static int fill_fp4(Fp4Args* a, const ctmi_qparams* qp, int64_t rows, int64_t cols) {
@@ -336,12 +492,12 @@ extern "C" int ctmi_nvfp4_compress(const void* x, int32_t x_dtype, uint8_t* out,
   if (qp->scale_dtype == CTMI_F8E4M3 && qp->global_scale && zp_ok &&
       (uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)out % 4 == 0 &&
       vec_geometry(qp, rows, cols, &g, true)) {
-    const int grid = grid_for(g.nvec, 256 * kU);
+    const unsigned grid = (unsigned)cdiv(g.nvec, kFp4Block * kFp4Unroll);
     const auto* sc = (const uint8_t*)qp->scale;
     const auto* zp = (const uint8_t*)qp->zero_point;
 #define CTMI_LAUNCH(XT, RAW)                                                                      \
-  if (zp) hipLaunchKernelGGL((nvfp4_compress_vec_kernel<XT, true>), grid, 256, 0, st, (const RAW*)x, sc, zp, qp->global_scale, (uint32_t*)out, g); \
-  else hipLaunchKernelGGL((nvfp4_compress_vec_kernel<XT, false>), grid, 256, 0, st, (const RAW*)x, sc, zp, qp->global_scale, (uint32_t*)out, g);
+  if (zp) hipLaunchKernelGGL((nvfp4_compress_vec_kernel<XT, true>), grid, kFp4Block, 0, st, (const RAW*)x, sc, zp, qp->global_scale, (uint32_t*)out, g); \
+  else hipLaunchKernelGGL((nvfp4_compress_vec_kernel<XT, false>), grid, kFp4Block, 0, st, (const RAW*)x, sc, zp, qp->global_scale, (uint32_t*)out, g);
     if (x_dtype == CTMI_BF16) { CTMI_LAUNCH(BF16, uint16_t) }
     else if (x_dtype == CTMI_F16) { CTMI_LAUNCH(F16, uint16_t) }
     else { CTMI_LAUNCH(F32, float) }
@@ -377,11 +533,11 @@ extern "C" int ctmi_nvfp4_decompress(const uint8_t* packed, void* out, int32_t o
   if (qp->scale_dtype == CTMI_F8E4M3 && qp->global_scale && qp->zero_point == nullptr &&
       (uintptr_t)out % (8 * dtype_size(out_dtype)) == 0 && (uintptr_t)packed % 4 == 0 &&
       vec_geometry(qp, rows, cols, &g, true)) {
-    const int grid = grid_for(g.nvec, 256 * kU);
+    const unsigned grid = (unsigned)cdiv(g.nvec, kFp4Block * kFp4Unroll);
     const auto* sc = (const uint8_t*)qp->scale;
-    if (out_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<BF16>, grid, 256, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (uint16_t*)out, g);
-    else if (out_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<F16>, grid, 256, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (uint16_t*)out, g);
-    else hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<F32>, grid, 256, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (float*)out, g);
+    if (out_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<BF16>, grid, kFp4Block, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (uint16_t*)out, g);
+    else if (out_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<F16>, grid, kFp4Block, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (uint16_t*)out, g);
+    else hipLaunchKernelGGL(nvfp4_decompress_vec_kernel<F32>, grid, kFp4Block, 0, st, (const uint32_t*)packed, sc, qp->global_scale, (float*)out, g);
     return check_launch("ctmi_nvfp4_decompress");
   }
 

@@ -59,6 +59,8 @@ __global__ void __launch_bounds__(256) qdq_generic_kernel(QdqArgs a) {
 
 bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
                         int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq, hipStream_t st);
+bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
+                              int64_t cols, const ctmi_qparams* qp, hipStream_t st);
 
 // ------------------------------------------------------------------ host side
 static int fill_cfg(const ctmi_qparams* qp, int x_dtype, QuantCfg* q) {
@@ -96,6 +98,9 @@ extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_d
 
   if (qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize,
                          (hipStream_t)stream))
+    return check_launch("ctmi_qdq");
+  if (do_quantize && do_dequantize &&
+      nvfp4_qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, (hipStream_t)stream))
     return check_launch("ctmi_qdq");
 
   QdqArgs a;

@@ -241,3 +241,38 @@ def test_nvfp4_compressor(shape, dtype, gpu):
          "weight_global_scale": gs.to(gpu)}, quantization_args=args)
     assert_bit_equal(dense, op.nvfp4_decompress(want, scale, gs), "nvfp4 decompress")
     assert dense.dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("scale_value,global_scale", [(1.0, 1.0), (0.75, 3.0), (448.0, 1234.5),
+                                                      (2.0 ** -9, 0.37)])
+def test_nvfp4_every_bf16_pattern(scale_value, global_scale, gpu):
+    """The no-division fast path and the hardware e2m1 converters against the
+    oracle on all 65 536 bf16 inputs (zeros of both signs, subnormals, every
+    rounding boundary when the effective scale is 1, infinities, NaNs), for
+    compress, decompress and fake-quantize."""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.quantization import fake_quantize
+
+    announce("nvfp4 all bf16 patterns", scale_value, global_scale)
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+    args, oargs = _pair(spec)
+    w = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).reshape(512, 128)
+    scale = torch.full((512, 8), scale_value).to(torch.float8_e4m3fn)
+    gs = torch.tensor([global_scale], dtype=torch.float32)
+    comp = BaseCompressor.load_from_registry("nvfp4-pack-quantized")
+    got = comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), global_scale=gs.to(gpu),
+                               quantization_args=args)["weight_packed"]
+    want = op.nvfp4_compress(w, scale, gs, oargs)
+    # A NaN input has no defined code: the reference's comes from the sign of a NaN
+    # product, which differs between platforms.  Compare the nibbles of all other inputs.
+    not_nan = ~torch.isnan(w.float())
+    nib = lambda t: torch.stack([t & 15, t >> 4], dim=-1).reshape(512, 128)
+    assert_bit_equal(nib(got.cpu())[not_nan], nib(want)[not_nan], "nvfp4 codes")
+    dense = comp.decompress_weight({"weight_packed": want.to(gpu), "weight_scale": scale.to(gpu),
+                                    "weight_global_scale": gs.to(gpu)}, quantization_args=args)
+    assert_bit_equal(dense, op.nvfp4_decompress(want, scale, gs), "nvfp4 decompress")
+    finite = ~torch.isnan(w.float())
+    fq = fake_quantize(w.to(gpu), scale.to(gpu), None, args, global_scale=gs.to(gpu)).cpu()
+    want_fq = oq.fake_quantize(w, scale, None, oargs, global_scale=gs)
+    assert_bit_equal(fq[finite], want_fq[finite], "nvfp4 fake-quantize")
+    assert bool(torch.isnan(fq[~finite].float()).all() == torch.isnan(want_fq[~finite].float()).all())
