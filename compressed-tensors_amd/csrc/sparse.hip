@@ -8,8 +8,11 @@
 // Bit j of bitmask byte k of a row flags column 8k+j (numpy packbits,
 // bitorder="little"); the last byte of a row is zero padded.  Compacted values
 // are stored in row-major order of the set bits.
+#include <type_traits>
+
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "quant_fast.h"
 #include "topk24_lut.h"
 #include "vec_geom.h"
 
@@ -142,37 +145,61 @@ bitmask_count_kernel(const R* __restrict__ x, uint32_t nz_mask, uint8_t* __restr
   }
 }
 
-// per-row popcount of an existing bitmask (bits at columns >= cols ignored)
+// per-row popcount of an existing bitmask (bits at columns >= cols ignored):
+// one wavefront per row, 4 bitmask bytes per lane and step when rows are whole
+// words
+// (`only_if`, when given, points at a flag that must be non-zero for the kernel to do anything)
 __global__ void __launch_bounds__(kBlock)
 bitmask_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t* __restrict__ counts,
-                        int64_t rows, int64_t cols, int64_t pc) {
-  __shared__ int64_t red[kWaves];
+                        int64_t rows, int64_t cols, int64_t pc, const int* only_if) {
+  if (only_if && *only_if == 0) return;
+  const int lane = lane_id();
   const uint32_t tail = (cols % 8) ? ((1u << (cols % 8)) - 1u) : 0xffu;
-  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
-    int64_t cnt = 0;
-    for (int64_t b = threadIdx.x; b < pc; b += kBlock) {
-      uint32_t bits = bitmask[r * pc + b];
+  for (int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave; r < rows;
+       r += (int64_t)gridDim.x * kWaves) {
+  const uint8_t* row = bitmask + r * pc;
+  int cnt = 0;
+  if (pc % 4 == 0 && (uintptr_t)bitmask % 4 == 0) {
+    const uint32_t* w = reinterpret_cast<const uint32_t*>(row);
+    const int64_t nw = pc / 4;
+    const uint32_t last = 0x00ffffffu | (tail << 24);
+    for (int64_t i = lane; i < nw; i += kWave) {
+      uint32_t bits = w[i];
+      if (i == nw - 1) bits &= last;
+      cnt += __popc(bits);
+    }
+  } else {
+    for (int64_t b = lane; b < pc; b += kWave) {
+      uint32_t bits = row[b];
       if (b == pc - 1) bits &= tail;
       cnt += __popc(bits);
     }
-    const int64_t t = block_sum(cnt, red);
-    if (threadIdx.x == 0) counts[r] = t;
+  }
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) cnt += __shfl_xor(cnt, d, kWave);
+  if (lane == 0) counts[r] = cnt;
   }
 }
 
-// exclusive scan of counts[rows] -> offsets[rows], total; single workgroup
-__global__ void __launch_bounds__(1024)
+// exclusive scan of counts[rows] -> offsets[rows], total; single workgroup, 8
+// neighbouring rows per thread and step
+constexpr int kScanThreads = 1024, kScanPer = 8;
+__global__ void __launch_bounds__(kScanThreads)
 row_offsets_kernel(const int64_t* __restrict__ counts, int64_t* __restrict__ offsets,
-                   int64_t* __restrict__ total, int64_t rows) {
-  __shared__ int64_t wsum[16];
-  __shared__ int64_t carry_s;
-  if (threadIdx.x == 0) carry_s = 0;
-  __syncthreads();
+                   int64_t* __restrict__ total, int64_t rows, const int* only_if) {
+  if (only_if && *only_if == 0) return;
+  __shared__ int64_t wsum[kScanThreads / kWave];
+  int64_t carry = 0;
   const int lane = lane_id(), wave = threadIdx.x / kWave;
-  for (int64_t base = 0; base < rows; base += 1024) {
-    const int64_t i = base + threadIdx.x;
-    const int64_t c = i < rows ? counts[i] : 0;
-    int64_t inc = c;
+  for (int64_t base = 0; base < rows; base += kScanThreads * kScanPer) {
+    const int64_t i0 = base + (int64_t)threadIdx.x * kScanPer;
+    int64_t c[kScanPer];
+#pragma unroll
+    for (int k = 0; k < kScanPer; ++k) c[k] = i0 + k < rows ? counts[i0 + k] : 0;
+    int64_t mine = 0;
+#pragma unroll
+    for (int k = 0; k < kScanPer; ++k) mine += c[k];
+    int64_t inc = mine;
 #pragma unroll
     for (int d = 1; d < kWave; d <<= 1) {
       const int64_t t = __shfl_up(inc, d, kWave);
@@ -181,18 +208,22 @@ row_offsets_kernel(const int64_t* __restrict__ counts, int64_t* __restrict__ off
     if (lane == kWave - 1) wsum[wave] = inc;
     __syncthreads();
     int64_t woff = 0, tot = 0;
-    for (int w = 0; w < 16; ++w) {
-      const int64_t s = wsum[w];
-      if (w < wave) woff += s;
-      tot += s;
+#pragma unroll
+    for (int w = 0; w < kScanThreads / kWave; ++w) {
+      const int64_t sv = wsum[w];
+      if (w < wave) woff += sv;
+      tot += sv;
     }
-    const int64_t carry = carry_s;
-    if (i < rows) offsets[i] = carry + woff + inc - c;
-    __syncthreads();
-    if (threadIdx.x == 0) carry_s = carry + tot;
+    int64_t run = carry + woff + inc - mine;
+#pragma unroll
+    for (int k = 0; k < kScanPer; ++k) {
+      if (i0 + k < rows) offsets[i0 + k] = run;
+      run += c[k];
+    }
+    carry += tot;
     __syncthreads();
   }
-  if (threadIdx.x == 0 && total) *total = carry_s;
+  if (threadIdx.x == 0 && total) *total = carry;
 }
 
 // ------------------------------------------------------------------ sparse-bitmask: compaction
@@ -248,7 +279,8 @@ __global__ void __launch_bounds__(kBlock)
 bitmask_scatter_kernel(const R* __restrict__ values, int64_t nvalues,
                        const uint8_t* __restrict__ bitmask,
                        const int64_t* __restrict__ row_offsets, R* __restrict__ out, int64_t rows,
-                       int64_t cols, int64_t pc) {
+                       int64_t cols, int64_t pc, const int* only_if) {
+  if (only_if && *only_if == 0) return;
   __shared__ int scan_s[kWaves];
   __shared__ R stage[kBlock * 8];
   const bool vec = (cols % 8 == 0) && ((uintptr_t)out % (8 * sizeof(R)) == 0);
@@ -288,6 +320,73 @@ bitmask_scatter_kernel(const R* __restrict__ values, int64_t nvalues,
   }
 }
 
+// ------------------------------------------------------------------ 2:4 decompress, streaming
+// In a well-formed 2:4 bitmask every group of 4 columns keeps exactly 2, so the
+// values of group g are values[2g], values[2g+1] and no prefix sum over the
+// bitmask is needed: a lane turns E columns' worth of mask bits and E/2 values
+// into one 16-byte store.  Whether the bitmask IS well formed is only known once
+// all of it has been looked at: every lane checks its own bits and raises
+// *malformed otherwise, and the general kernels, enqueued behind this one, do
+// their work (and overwrite the output) only if the flag went up.
+template <typename R>
+struct Scatter24 {
+  static constexpr int E = sizeof(R) == 1 ? 16 : 8;  // columns per lane
+  using MaskT = typename std::conditional<E == 16, uint16_t, uint8_t>::type;
+};
+
+template <typename R>
+__global__ void __launch_bounds__(kBlock)
+sparse24_scatter_kernel(const R* __restrict__ values, const uint8_t* __restrict__ bitmask,
+                        R* __restrict__ out, int64_t n_items, int* __restrict__ malformed) {
+  constexpr int E = Scatter24<R>::E, U = 2;
+  using MaskT = typename Scatter24<R>::MaskT;
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  MaskT m[U];
+  Vec<R, E / 2> v[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    // past the end: re-read the last item (not stored)
+    int64_t i = i0 + k * kBlock;
+    if (i >= n_items) i = n_items - 1;
+    m[k] = reinterpret_cast<const MaskT*>(bitmask)[i];
+    v[k] = ldg<R, E / 2>(values + i * (E / 2));
+  }
+  bool bad = false;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    const uint32_t bits = m[k];
+    uint32_t n = bits - ((bits >> 1) & 0x5555u);
+    n = (n & 0x3333u) + ((n >> 2) & 0x3333u);  // set bits per group of 4
+    bad |= i < n_items && n != (E == 16 ? 0x2222u : 0x22u);
+    Vec<R, E> o;
+#pragma unroll
+    for (int g = 0; g < E / 4; ++g) {
+      const uint32_t gm = (bits >> (4 * g)) & 15u;
+      const R a = v[k].v[2 * g], b = v[k].v[2 * g + 1];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool keep = (gm >> j) & 1u, second = (gm & ((1u << j) - 1u)) != 0;
+        o.v[4 * g + j] = keep ? (second ? b : a) : (R)0;
+      }
+    }
+    if (i < n_items) {
+      if constexpr (sizeof(R) * E == 16) {
+        stg_nt<R, E>(out + i * E, o);
+      } else {  // 4-byte elements: two 16-byte halves
+        Vec<R, 4> lo, hi;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) { lo.v[j] = o.v[j]; hi.v[j] = o.v[4 + j]; }
+        stg<R, 4>(out + i * E, lo);
+        stg<R, 4>(out + i * E + 4, hi);
+      }
+    }
+  }
+  if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane_id() == 0) atomicOr(malformed, 1);
+}
+
+__global__ void zero_flag_kernel(int* flag) { *flag = 0; }
+
 // ------------------------------------------------------------------ 2:4 selection
 // Ranking key of one element: |value| compared the way torch.topk compares
 // it (NaN above everything, all NaNs equal); for 1-byte integer views abs() is
@@ -322,23 +421,83 @@ __device__ __forceinline__ uint32_t keep24(uint32_t k0, uint32_t k1, uint32_t k2
   return lut[idx];
 }
 
-__device__ __forceinline__ void load_lut(uint8_t* lds_lut) {
-  // 4096 bytes, 16 per thread of a 256-thread workgroup
-  reinterpret_cast<uint4*>(lds_lut)[threadIdx.x] =
-      reinterpret_cast<const uint4*>(kTopk24LutDev)[threadIdx.x];
-  __syncthreads();
+// Keep masks of the N/4 groups of one work item (group q in bits [4q, 4q+4)).
+// A group with exactly two keys above zero (what a 2:4-pruned tensor holds
+// nearly everywhere) keeps those two whatever order torch.topk gives the rest;
+// only when some lane of the wavefront meets another kind of group are the ties
+// resolved through the comparison table (read from memory then: no per-workgroup
+// copy of it for the common case).
+template <typename R, int DT, int N>
+__device__ __forceinline__ uint32_t keep_masks24(const Vec<R, N>& a) {
+  uint32_t keys[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) keys[i] = key24<DT>(a.v[i]);
+  uint32_t keep = 0;
+  bool clear = true;
+#pragma unroll
+  for (int q = 0; q < N / 4; ++q) {
+    uint32_t pos = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      // above zero as the ranking sees it (int8-view keys are biased by 128, and
+      // -128, whose abs() stays -128, ranks below zero)
+      const bool gt = DT == CTMI_I8 ? keys[4 * q + j] > 128u : keys[4 * q + j] != 0;
+      pos |= (gt ? 1u : 0u) << j;
+    }
+    clear &= __popc(pos) == 2;
+    keep |= pos << (4 * q);
+  }
+  if (wave_all(clear)) return keep;
+  keep = 0;
+#pragma unroll
+  for (int q = 0; q < N / 4; ++q)
+    keep |= keep24(keys[4 * q], keys[4 * q + 1], keys[4 * q + 2], keys[4 * q + 3], kTopk24LutDev)
+            << (4 * q);
+  return keep;
+}
+
+// get_24_bytemasks: one bool per element; work item = 16 elements (numel % 16 == 0)
+template <typename R, int DT>
+__global__ void __launch_bounds__(kBlock)
+bytemask24_vec_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64_t nitems) {
+  constexpr int N = 16, U = 2;
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  Vec<R, N> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    int64_t i = i0 + k * kBlock;
+    if (i >= nitems) i = nitems - 1;  // re-read, not stored
+    if constexpr (sizeof(R) * N == 16) {
+      a[k] = ldg<R, N>(x + i * N);
+    } else {
+#pragma unroll
+      for (int h = 0; h < (int)(sizeof(R) * N / 16); ++h) {
+        constexpr int PER = 16 / sizeof(R);
+        const Vec<R, PER> part = ldg<R, PER>(x + i * N + h * PER);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) a[k].v[h * PER + j] = part.v[j];
+      }
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    const uint32_t keep = keep_masks24<R, DT, N>(a[k]);
+    Vec<uint8_t, N> o;
+#pragma unroll
+    for (int j = 0; j < N; ++j) o.v[j] = (uint8_t)((keep >> j) & 1u);
+    if (i < nitems) stg<uint8_t, N>(mask + i * N, o);
+  }
 }
 
 template <typename R, int DT>
 __global__ void __launch_bounds__(kBlock)
 bytemask24_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64_t ngroups) {
-  __shared__ __align__(16) uint8_t lut[4096];
-  load_lut(lut);
   for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < ngroups;
        g += (int64_t)gridDim.x * blockDim.x) {
     const R* p = x + g * 4;
     const uint32_t keep = keep24(key24<DT>(p[0]), key24<DT>(p[1]), key24<DT>(p[2]),
-                                 key24<DT>(p[3]), lut);
+                                 key24<DT>(p[3]), kTopk24LutDev);
     uint32_t w = 0;
 #pragma unroll
     for (int j = 0; j < 4; ++j) w |= ((keep >> j) & 1u) << (8 * j);
@@ -348,31 +507,41 @@ bytemask24_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64_t n
 
 // Fused 2:4 compress, cols % 8 == 0.  Work item = N elements (N/4 groups):
 // one 16-byte load, N/2 survivors stored as one vector, N/8 bitmask bytes.
+// One workgroup per chunk of items, every load issued before the first use.
 template <typename R, int DT, int N>
 __global__ void __launch_bounds__(kBlock)
 sparse24_compress_kernel(const R* __restrict__ x, R* __restrict__ values,
                          uint8_t* __restrict__ bitmask, int64_t nitems) {
-  __shared__ __align__(16) uint8_t lut[4096];
-  load_lut(lut);
-  for (int64_t it = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; it < nitems;
-       it += (int64_t)gridDim.x * blockDim.x) {
-    Vec<R, N> a = ldg<R, N>(x + it * N);
+  constexpr int U = 2;
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  Vec<R, N> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    a[k] = ldg<R, N>(x + (i < nitems ? i : nitems - 1) * N);  // past the end: re-read, not stored
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    const uint32_t keep_all = keep_masks24<R, DT, N>(a[k]);
     Vec<R, N / 2> o;
     Vec<uint8_t, N / 8> m;
 #pragma unroll
     for (int q = 0; q < N / 4; ++q) {
-      const uint32_t keep = keep24(key24<DT>(a.v[4 * q]), key24<DT>(a.v[4 * q + 1]),
-                                   key24<DT>(a.v[4 * q + 2]), key24<DT>(a.v[4 * q + 3]), lut);
-      // the two survivors in column order
-      const int lo = __ffs(keep) - 1;
-      const int hi = 31 - __clz(keep);
-      o.v[2 * q] = a.v[4 * q + lo];
-      o.v[2 * q + 1] = a.v[4 * q + hi];
-      if (q & 1) m.v[q / 2] |= (uint8_t)(keep << 4);
-      else m.v[q / 2] = (uint8_t)keep;
+      const uint32_t keep = (keep_all >> (4 * q)) & 15u;
+      // the two survivors in column order: the lower one is element 0, 1 or 2,
+      // the upper one element 1, 2 or 3
+      const R e0 = a[k].v[4 * q], e1 = a[k].v[4 * q + 1], e2 = a[k].v[4 * q + 2],
+              e3 = a[k].v[4 * q + 3];
+      o.v[2 * q] = (keep & 1u) ? e0 : ((keep & 2u) ? e1 : e2);
+      o.v[2 * q + 1] = (keep & 8u) ? e3 : ((keep & 4u) ? e2 : e1);
     }
-    stg<R, N / 2>(values + it * (N / 2), o);
-    stg<uint8_t, N / 8>(bitmask + it * (N / 8), m);
+#pragma unroll
+    for (int bq = 0; bq < N / 8; ++bq) m.v[bq] = (uint8_t)((keep_all >> (8 * bq)) & 0xffu);
+    if (i < nitems) {
+      stg<R, N / 2>(values + i * (N / 2), o);
+      stg<uint8_t, N / 8>(bitmask + i * (N / 8), m);
+    }
   }
 }
 
@@ -380,13 +549,11 @@ sparse24_compress_kernel(const R* __restrict__ x, R* __restrict__ values,
 template <typename R, int DT>
 __global__ void __launch_bounds__(kBlock)
 sparse24_values_kernel(const R* __restrict__ x, R* __restrict__ values, int64_t ngroups) {
-  __shared__ __align__(16) uint8_t lut[4096];
-  load_lut(lut);
   for (int64_t g = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; g < ngroups;
        g += (int64_t)gridDim.x * blockDim.x) {
     const R* p = x + g * 4;
     const uint32_t keep = keep24(key24<DT>(p[0]), key24<DT>(p[1]), key24<DT>(p[2]),
-                                 key24<DT>(p[3]), lut);
+                                 key24<DT>(p[3]), kTopk24LutDev);
     values[2 * g] = p[__ffs(keep) - 1];
     values[2 * g + 1] = p[31 - __clz(keep)];
   }
@@ -397,8 +564,6 @@ template <typename R, int DT>
 __global__ void __launch_bounds__(kBlock)
 sparse24_bitmask_kernel(const R* __restrict__ x, uint8_t* __restrict__ bitmask, int64_t rows,
                         int64_t cols, int64_t pc) {
-  __shared__ __align__(16) uint8_t lut[4096];
-  load_lut(lut);
   const int64_t total = rows * pc;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
        i += (int64_t)gridDim.x * blockDim.x) {
@@ -410,7 +575,7 @@ sparse24_bitmask_kernel(const R* __restrict__ x, uint8_t* __restrict__ bitmask, 
       const int64_t e = r * cols + c;
       const R* p = x + (e / 4) * 4;
       const uint32_t keep = keep24(key24<DT>(p[0]), key24<DT>(p[1]), key24<DT>(p[2]),
-                                   key24<DT>(p[3]), lut);
+                                   key24<DT>(p[3]), kTopk24LutDev);
       bits |= ((keep >> (e % 4)) & 1u) << j;
     }
     bitmask[i] = (uint8_t)bits;
@@ -495,7 +660,8 @@ extern "C" int ctmi_bitmask_count(const void* x, int32_t elem_size, int32_t is_f
     hipLaunchKernelGGL(bitmask_count_kernel<uint32_t>, grid, kBlock, 0, st, (const uint32_t*)x,
                        is_float ? 0x7FFFFFFFu : 0xFFFFFFFFu, bitmask, counts, rows, cols, pc);
   }
-  hipLaunchKernelGGL(row_offsets_kernel, 1, 1024, 0, st, counts, row_offsets, total_nnz, rows);
+  hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, row_offsets, total_nnz, rows,
+                     (const int*)nullptr);
   return check_launch("ctmi_bitmask_count");
 }
 
@@ -536,23 +702,55 @@ extern "C" int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int3
   CTMI_REQUIRE(row_offsets || tmp, CTMI_ERR_VALUE, "row_offsets and tmp are both NULL");
   hipStream_t st = (hipStream_t)stream;
   const int64_t pc = cdiv(cols, 8);
-  const int grid = rows_grid(rows);
+  int grid = rows_grid(rows);
+  int64_t pop_grid = cdiv(rows, kWaves);
+  const int* only_if = nullptr;
   if (!row_offsets) {
     int64_t* counts = (int64_t*)tmp;
     int64_t* offs = counts + rows;
-    hipLaunchKernelGGL(bitmask_popcount_kernel, grid, kBlock, 0, st, bitmask, counts, rows, cols, pc);
-    hipLaunchKernelGGL(row_offsets_kernel, 1, 1024, 0, st, counts, offs, (int64_t*)nullptr, rows);
+    // exactly half as many values as elements, rows of whole bitmask bytes: try
+    // the 2:4 streaming kernel first (see sparse24_scatter_kernel)
+    const int64_t numel = rows * cols;
+    const int e = elem_size == 1 ? 16 : 8;
+    if (nvalues * 2 == numel && cols % 8 == 0 && numel % e == 0 && (uintptr_t)out % 16 == 0 &&
+        (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 2 == 0 && numel / e < (1ll << 40)) {
+      int* flag = (int*)(offs + rows);
+      const int64_t n_items = numel / e;
+      const unsigned g24 = (unsigned)cdiv(n_items, kBlock * 2);
+      hipLaunchKernelGGL(zero_flag_kernel, 1, 1, 0, st, flag);
+      if (elem_size == 1)
+        hipLaunchKernelGGL(sparse24_scatter_kernel<uint8_t>, g24, kBlock, 0, st,
+                           (const uint8_t*)values, bitmask, (uint8_t*)out, n_items, flag);
+      else if (elem_size == 2)
+        hipLaunchKernelGGL(sparse24_scatter_kernel<uint16_t>, g24, kBlock, 0, st,
+                           (const uint16_t*)values, bitmask, (uint16_t*)out, n_items, flag);
+      else
+        hipLaunchKernelGGL(sparse24_scatter_kernel<uint32_t>, g24, kBlock, 0, st,
+                           (const uint32_t*)values, bitmask, (uint32_t*)out, n_items, flag);
+      only_if = flag;
+      // the kernels below now only run in the rare malformed case: keep their
+      // grids small, an empty launch costs by the workgroup
+      if (grid > 1024) grid = 1024;
+      if (pop_grid > 512) pop_grid = 512;
+    }
+    if (pop_grid > (1 << 20)) pop_grid = 1 << 20;
+    hipLaunchKernelGGL(bitmask_popcount_kernel, (unsigned)pop_grid, kBlock, 0, st, bitmask,
+                       counts, rows, cols, pc, only_if);
+    hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, offs, (int64_t*)nullptr,
+                       rows, only_if);
     row_offsets = offs;
   }
   if (elem_size == 1)
     hipLaunchKernelGGL(bitmask_scatter_kernel<uint8_t>, grid, kBlock, 0, st, (const uint8_t*)values,
-                       nvalues, bitmask, row_offsets, (uint8_t*)out, rows, cols, pc);
+                       nvalues, bitmask, row_offsets, (uint8_t*)out, rows, cols, pc, only_if);
   else if (elem_size == 2)
     hipLaunchKernelGGL(bitmask_scatter_kernel<uint16_t>, grid, kBlock, 0, st,
-                       (const uint16_t*)values, nvalues, bitmask, row_offsets, (uint16_t*)out, rows, cols, pc);
+                       (const uint16_t*)values, nvalues, bitmask, row_offsets, (uint16_t*)out, rows,
+                       cols, pc, only_if);
   else
     hipLaunchKernelGGL(bitmask_scatter_kernel<uint32_t>, grid, kBlock, 0, st,
-                       (const uint32_t*)values, nvalues, bitmask, row_offsets, (uint32_t*)out, rows, cols, pc);
+                       (const uint32_t*)values, nvalues, bitmask, row_offsets, (uint32_t*)out, rows,
+                       cols, pc, only_if);
   return check_launch("ctmi_bitmask_decompress");
 }
 
@@ -585,6 +783,13 @@ extern "C" int ctmi_get_24_bytemasks(const void* x, int32_t x_dtype, uint8_t* ma
   const int64_t ng = numel / 4;
   const int grid = grid_for(ng, kBlock);
   hipStream_t st = (hipStream_t)stream;
+  if (numel % 16 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)mask % 16 == 0) {
+    const int64_t items = numel / 16;
+    CTMI_DISPATCH_24(x_dtype, hipLaunchKernelGGL((bytemask24_vec_kernel<R, DT>),
+                                                  (unsigned)cdiv(items, kBlock * 2), kBlock, 0, st,
+                                                  (const R*)x, mask, items));
+    return check_launch("ctmi_get_24_bytemasks");
+  }
   CTMI_DISPATCH_24(x_dtype, hipLaunchKernelGGL((bytemask24_kernel<R, DT>), grid, kBlock, 0, st,
                                                 (const R*)x, mask, ng));
   return check_launch("ctmi_get_24_bytemasks");
@@ -611,22 +816,23 @@ extern "C" int ctmi_sparse24_compress(const void* x, int32_t x_dtype, void* valu
   if (fast) {
     if (es == 1) {
       const int64_t items = n / 16;
-      hipLaunchKernelGGL((sparse24_compress_kernel<uint8_t, CTMI_I8, 16>), grid_for(items, kBlock),
+      hipLaunchKernelGGL((sparse24_compress_kernel<uint8_t, CTMI_I8, 16>), (unsigned)cdiv(items, kBlock * 2),
                          kBlock, 0, st, (const uint8_t*)x, (uint8_t*)values, bitmask, items);
     } else if (es == 2) {
       const int64_t items = n / 8;
       if (x_dtype == CTMI_BF16)
         hipLaunchKernelGGL((sparse24_compress_kernel<uint16_t, CTMI_BF16, 8>),
-                           grid_for(items, kBlock), kBlock, 0, st, (const uint16_t*)x,
+                           (unsigned)cdiv(items, kBlock * 2), kBlock, 0, st, (const uint16_t*)x,
                            (uint16_t*)values, bitmask, items);
       else
         hipLaunchKernelGGL((sparse24_compress_kernel<uint16_t, CTMI_F16, 8>),
-                           grid_for(items, kBlock), kBlock, 0, st, (const uint16_t*)x,
+                           (unsigned)cdiv(items, kBlock * 2), kBlock, 0, st, (const uint16_t*)x,
                            (uint16_t*)values, bitmask, items);
     } else {
       const int64_t items = n / 8;
-      hipLaunchKernelGGL((sparse24_compress_kernel<uint32_t, CTMI_F32, 8>), grid_for(items, kBlock),
-                         kBlock, 0, st, (const uint32_t*)x, (uint32_t*)values, bitmask, items);
+      hipLaunchKernelGGL((sparse24_compress_kernel<uint32_t, CTMI_F32, 8>),
+                         (unsigned)cdiv(items, kBlock * 2), kBlock, 0, st, (const uint32_t*)x,
+                         (uint32_t*)values, bitmask, items);
     }
     return check_launch("ctmi_sparse24_compress");
   }

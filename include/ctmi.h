@@ -189,7 +189,11 @@ int ctmi_bitmask_compact(const void* x, int32_t elem_size, const uint8_t* bitmas
  * (nvalues elements, consumed in row-major order of the set bits; set bits
  * beyond nvalues read as zero) into a zero-filled [rows, cols].
  * row_offsets may be NULL: it is then recomputed from the bitmask into tmp
- * (ctmi_bitmask_tmp_bytes(rows) bytes + rows*8 bytes for the offsets). */
+ * (ctmi_bitmask_tmp_bytes(rows) bytes + rows*8 bytes for the offsets + 8 bytes
+ * for a flag).  With NULL row_offsets and exactly half as many values as
+ * elements the bitmask is first taken to be a 2:4 one (2 kept per group of 4),
+ * which needs no prefix sums; the general path runs behind it only if some
+ * group turns out not to keep exactly 2. */
 int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_size,
                             const uint8_t* bitmask,
                             const int64_t* row_offsets, void* out, void* tmp, int64_t rows,

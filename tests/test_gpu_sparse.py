@@ -177,3 +177,31 @@ def test_large_bitmask_roundtrip_properties(gpu):
         assert_bit_equal(values[lo: lo + int(nnz_rows[r])], w[r][w[r] != 0], f"values row {r}")
     assert_bit_equal(bitmask[:64], osp.pack_bitmasks(w[:64] != 0), "bitmask head")
     assert torch.equal(bitmask_decompress(values, bitmask, list(w.shape)), wg)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn, torch.float32])
+def test_sparse24_decompress_of_a_bitmask_that_is_not_2_4(dtype, gpu):
+    """sparse24_bitmask_decompress is `out[mask] = values` for ANY mask
+    (sparse_24_bitmask.py:206-224).  Half of the elements kept, but not 2 per group
+    of 4: the streaming 2:4 kernel must notice and the general path take over."""
+    from compressed_tensors_amd.compressors import sparse24_bitmask_decompress
+    from compressed_tensors_amd.utils.helpers import pack_bitmasks
+
+    announce("sparse24 decompress, malformed mask", dtype)
+    g = torch.Generator().manual_seed(7)
+    rows, cols = 48, 256
+    x = torch.randn(rows, cols, generator=g).clamp(-3, 3)
+    x[x == 0] = 1.0
+    mask = torch.zeros(rows, cols, dtype=torch.bool)
+    mask[:, : cols // 2] = True              # 4 kept in the first groups, none in the last
+    mask[5] = torch.arange(cols) % 2 == 0    # one well-formed row in between
+    mask[6, :8] = torch.tensor([1, 1, 1, 0, 1, 0, 0, 0], dtype=torch.bool)  # 3 + 1: right total, wrong groups
+    mask[6, 8:] = torch.arange(cols - 8) % 2 == 0
+    x = torch.where(mask, x, torch.zeros_like(x)).to(dtype)
+    raw = x.view(torch.int8) if dtype == torch.float8_e4m3fn else x
+    values = raw[mask].reshape(rows, cols // 2)
+    if dtype == torch.float8_e4m3fn:
+        values = values.view(torch.float8_e4m3fn)
+    bitmask = pack_bitmasks(mask.to(gpu))
+    dense = sparse24_bitmask_decompress(values.to(gpu), bitmask, torch.Size((rows, cols)))
+    assert_bit_equal(dense, x, "general path behind the 2:4 kernel")
