@@ -12,6 +12,17 @@ Workloads
   llama3-8b-w4a16   (default) 32 x {q,o 4096x4096; k,v 1024x4096; gate,up 14336x4096;
                     down 4096x14336} bf16 N(0, 0.02), symmetric int4, group 128
   w4a16-4096        one 4096 x 4096 weight of the same recipe
+The other configurations of the same path, each a list of operations timed one
+by one (HIP events on the launch stream) over rotating copies of the inputs, so
+that no pass finds its input in the last-level cache:
+  fp8-w8a8          per-channel fp8 weights of the same 224 shapes (0.1 % outliers x20)
+                    + dynamic per-token fp8 activation quantization, 8192 x 4096
+  sparse            sparse-bitmask on a 50 % pruned 8192 x 8192 bf16 weight; sparse-24-bitmask
+                    on a 2:4 pruned, fp8-quantized 14336 x 4096 weight
+  nvfp4             nvfp4-pack-quantized on 14336 x 4096 and 4096 x 14336 bf16 weights
+                    + dynamic nvfp4 activation quantization, 4096 x 4096
+  hadamard          block-128 and full 4096 rotations of 8192 x 4096 activations and of
+                    4096 x 4096 / 14336 x 4096 weights
 """
 import argparse
 import json
@@ -99,6 +110,254 @@ def cpu_baseline(torch, sample_shapes, seed):
     }
 
 
+# ---------------------------------------------------------------------------------------------
+# The other configurations: lists of operations on the C ABI, prepared once and timed one by one
+class Op:
+    def __init__(self, name, calls, nbytes, kernel):
+        self.name, self.calls, self.nbytes, self.kernel = name, calls, nbytes, kernel
+        self.ms = 0.0
+
+
+def time_ops(torch, ops, steps, warmup):
+    """every op is a list of enqueue closures (one per rotating input copy); per-op GPU time from
+    events recorded on the launch stream around each op"""
+    def one_pass(record):
+        marks = []
+        for op in ops:
+            if record:
+                e = torch.cuda.Event(enable_timing=True); e.record(); marks.append(e)
+            for call in op.calls:
+                call()
+        if record:
+            e = torch.cuda.Event(enable_timing=True); e.record(); marks.append(e)
+        return marks
+    for _ in range(warmup):
+        one_pass(False)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    all_marks = [one_pass(True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    for i, op in enumerate(ops):
+        op.ms = sum(m[i].elapsed_time(m[i + 1]) for m in all_marks) / steps
+    return wall / steps
+
+
+def other_workload(torch, name, seed):
+    """-> (metric, ops, keep-alive list)"""
+    import ctypes
+    from compressed_tensors_amd import _lib
+    from compressed_tensors_amd.quantization import (QuantizationArgs, compute_dynamic_scales_and_zp,
+                                                     generate_gparam, observe_weight_qparams)
+    from compressed_tensors_amd.quantization.forward import build_qparams
+    from compressed_tensors_amd.transform.hadamard import deterministic_hadamard_matrix
+
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    st = _lib.stream_of(dev)
+    code = _lib.dtype_code
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    keep = []
+    FP8 = torch.float8_e4m3fn
+
+    def randn(r, c, std=1.0):
+        return (torch.randn(r, c, generator=gen, device=dev) * std).to(torch.bfloat16)
+
+    def qdq(x, out, plan, do_q, do_dq):
+        keep.extend([x, out, plan])
+        rows = x.numel() // x.shape[-1]
+        args = (x.data_ptr(), code(x.dtype), out.data_ptr(), code(out.dtype), rows, x.shape[-1],
+                ctypes.byref(plan.qp), do_q, do_dq, st)
+        return lambda: _lib.check(lib.ctmi_qdq(*args))
+
+    def observe(x, blk_cols, args, scale, zp, gscale=None):
+        keep.extend([x, scale, zp, gscale])
+        rows = x.numel() // x.shape[-1]
+        qtype = _lib.QTYPE_FLOAT if args.type == "float" else _lib.QTYPE_INT
+        a = (x.data_ptr(), code(x.dtype), rows, x.shape[-1], blk_cols, qtype, args.num_bits,
+             int(args.symmetric), _lib.ptr(gscale), scale.data_ptr(), code(scale.dtype),
+             zp.data_ptr(), code(zp.dtype), None, None, st)
+        return lambda: _lib.check(lib.ctmi_observe_qparams(*a))
+
+    if name == "fp8-w8a8":
+        args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
+        q_calls, d_calls, n = [], [], 0
+        for _, r, c in shapes_for("llama3-8b-w4a16"):
+            w = randn(r, c, 0.02)
+            hot = torch.rand(r, c, generator=gen, device=dev) < 1e-3
+            w = torch.where(hot, w * 20, w)
+            scale, zp = observe_weight_qparams(w, args)
+            codes = torch.empty(r, c, dtype=FP8, device=dev)
+            dense = torch.empty(r, c, dtype=torch.bfloat16, device=dev)
+            q_calls.append(qdq(w, codes, build_qparams(w, scale, None, args), 1, 0))
+            d_calls.append(qdq(codes, dense, build_qparams(codes, scale, None, args), 0, 1))
+            n += r * c
+        acts, a_obs, a_fq = [], [], []
+        targs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="token",
+                                 dynamic=True)
+        for _ in range(8):  # 8 x 67 MB: more than the last-level cache
+            x = randn(8192, 4096)
+            x[:, torch.rand(4096, generator=gen, device=dev) < 5e-3] *= 50
+            x = x.reshape(1, 8192, 4096)
+            s, z = compute_dynamic_scales_and_zp(x, targs)
+            out = torch.empty_like(x)
+            a_obs.append(observe(x, 4096, targs, s, z))
+            a_fq.append(qdq(x, out, build_qparams(x, s, z, targs), 1, 1))
+            acts.append(x)
+        na = 8 * 8192 * 4096
+        ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_kernel"),
+               Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_kernel"),
+               Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
+               Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel")]
+        return "fp8 W8A8 quantize/dequantize GB/s, Llama-3-8B-shaped weights + per-token activations", ops, keep
+
+    if name == "sparse":
+        copies = 6
+        c_calls, d_calls, s_calls, t_calls = [], [], [], []
+        nb = 8192 * 8192
+        nnz_total = 0
+        for _ in range(copies):
+            w = randn(8192, 8192, 0.02)
+            thr = w.float().abs().flatten().kthvalue(nb // 2).values
+            w = torch.where(w.float().abs() <= thr, torch.zeros_like(w), w)
+            rows, cols = w.shape
+            bitmask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=dev)
+            offs = torch.empty(rows, dtype=torch.int64, device=dev)
+            total = torch.empty(1, dtype=torch.int64, device=dev)
+            tmp = torch.empty(lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8, dtype=torch.uint8, device=dev)
+            a = (w.data_ptr(), 2, 1, bitmask.data_ptr(), offs.data_ptr(), total.data_ptr(), tmp.data_ptr(), rows, cols, st)
+            _lib.check(lib.ctmi_bitmask_count(*a))
+            nnz = int(total.item())
+            nnz_total += nnz
+            values = torch.empty(nnz, dtype=torch.bfloat16, device=dev)
+            b = (w.data_ptr(), 2, bitmask.data_ptr(), offs.data_ptr(), values.data_ptr(), rows, cols, st)
+            dense = torch.empty_like(w)
+            d = (values.data_ptr(), nnz, 2, bitmask.data_ptr(), None, dense.data_ptr(), tmp.data_ptr(), rows, cols, st)
+            keep.extend([w, bitmask, offs, total, tmp, values, dense])
+            c_calls.append(lambda a=a, b=b: (_lib.check(lib.ctmi_bitmask_count(*a)), _lib.check(lib.ctmi_bitmask_compact(*b))))
+            d_calls.append(lambda d=d: _lib.check(lib.ctmi_bitmask_decompress(*d)))
+        n24 = 14336 * 4096
+        cargs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
+        from compressed_tensors_amd.compressors import get_24_bytemasks
+        from compressed_tensors_amd.quantization import quantize
+        for _ in range(copies):
+            w = randn(14336, 4096, 0.02)
+            w = torch.where(get_24_bytemasks(w), w, torch.zeros_like(w))
+            scale, _ = observe_weight_qparams(w, cargs)
+            q = quantize(w, scale, None, cargs, dtype=FP8)
+            rows, cols = q.shape
+            values = torch.empty(rows, cols // 2, dtype=FP8, device=dev)
+            bitmask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=dev)
+            dense = torch.empty_like(q)
+            tmp = torch.empty(lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8, dtype=torch.uint8, device=dev)
+            a = (q.data_ptr(), code(FP8), values.data_ptr(), bitmask.data_ptr(), rows, cols, st)
+            d = (values.data_ptr(), values.numel(), 1, bitmask.data_ptr(), None, dense.data_ptr(), tmp.data_ptr(), rows, cols, st)
+            _lib.check(lib.ctmi_sparse24_compress(*a))
+            keep.extend([q, values, bitmask, dense, tmp])
+            s_calls.append(lambda a=a: _lib.check(lib.ctmi_sparse24_compress(*a)))
+            t_calls.append(lambda d=d: _lib.check(lib.ctmi_bitmask_decompress(*d)))
+        bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
+        s24_bytes = copies * (n24 + n24 // 2 + n24 // 8)
+        ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_kernel"),
+               Op("sparse-bitmask decompress (row offsets recomputed from the bitmask)", d_calls, bm_bytes, "bitmask_scatter_kernel"),
+               Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
+               Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel")]
+        return "sparse-bitmask / sparse-24-bitmask compress+decompress GB/s", ops, keep
+
+    if name == "nvfp4":
+        args = QuantizationArgs(num_bits=4, type="float", symmetric=True, strategy="tensor_group",
+                                group_size=16)
+        ops = []
+        for r, c in ((14336, 4096), (4096, 14336)):
+            c_calls, d_calls = [], []
+            for _ in range(5):
+                w = randn(r, c, 0.02)
+                gs = generate_gparam(w.min().reshape(1), w.max().reshape(1))
+                scale, zp = observe_weight_qparams(w, args, global_scale=gs)
+                packed = torch.empty(r, c // 2, dtype=torch.uint8, device=dev)
+                dense = torch.empty_like(w)
+                cp = build_qparams(w, scale, zp, args, None, gs)
+                dp = build_qparams(w, scale, None, args, None, gs)
+                keep.extend([w, gs, scale, zp, packed, dense, cp, dp])
+                ca = (w.data_ptr(), code(w.dtype), packed.data_ptr(), r, c, ctypes.byref(cp.qp), st)
+                da = (packed.data_ptr(), dense.data_ptr(), code(dense.dtype), r, c, ctypes.byref(dp.qp), st)
+                c_calls.append(lambda ca=ca: _lib.check(lib.ctmi_nvfp4_compress(*ca)))
+                d_calls.append(lambda da=da: _lib.check(lib.ctmi_nvfp4_decompress(*da)))
+            nbytes = 5 * (2 * r * c + r * c // 16 + r * c // 2)
+            ops += [Op(f"nvfp4 compress {r}x{c} (x5)", c_calls, nbytes, "nvfp4_compress_vec_kernel"),
+                    Op(f"nvfp4 decompress {r}x{c} (x5)", d_calls, nbytes, "nvfp4_decompress_vec_kernel")]
+        aargs = QuantizationArgs(num_bits=4, type="float", symmetric=True, strategy="tensor_group",
+                                 group_size=16, dynamic="local")
+        o_calls, f_calls = [], []
+        for _ in range(16):
+            x = randn(4096, 4096)
+            gs = generate_gparam(x.min().reshape(1), x.max().reshape(1))
+            s, z = compute_dynamic_scales_and_zp(x, aargs, None, global_scale=gs)
+            out = torch.empty_like(x)
+            o_calls.append(observe(x, 16, aargs, s, z, gs))
+            f_calls.append(qdq(x, out, build_qparams(x, s, None, aargs, None, gs), 1, 1))
+        na = 16 * 4096 * 4096
+        ops += [Op("nvfp4 activations: group-16 scales (16 x 4096x4096)", o_calls, 2 * na + na // 16, "observe_flat_kernel"),
+                Op("nvfp4 activations: fake-quantize (16 x 4096x4096)", f_calls, 4 * na + na // 16, "nvfp4_qdq_vec_kernel")]
+        return "nvfp4-pack-quantized compress/decompress + activation fake-quantize GB/s", ops, keep
+
+    if name == "hadamard":
+        ops = []
+        tensors = {"activations 8192x4096 (x8)": [randn(8192, 4096) for _ in range(8)],
+                   "weights 4096x4096 (x16)": [randn(4096, 4096, 0.02) for _ in range(16)],
+                   "weights 14336x4096 (x5)": [randn(14336, 4096, 0.02) for _ in range(5)]}
+        for n, (a_dim, b_dim) in ((128, (1, 128)), (4096, (64, 64))):
+            q = (torch.randint(0, 2, (n,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
+            mb = deterministic_hadamard_matrix(b_dim, torch.bfloat16, dev).contiguous()
+            ma = deterministic_hadamard_matrix(a_dim, torch.bfloat16, dev).contiguous() if a_dim > 1 else None
+            keep.extend([q, mb, ma])
+            for label, xs in tensors.items():
+                calls = []
+                for x in xs:
+                    out = torch.empty_like(x)
+                    keep.extend([x, out])
+                    a = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), a_dim, b_dim,
+                         _lib.ptr(ma), mb.data_ptr(), q.data_ptr(), None, st)
+                    calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
+                nb = sum(4 * x.numel() for x in xs)
+                ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb,
+                              "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel"))
+        return "Hadamard rotation GB/s (bf16 MFMA), block 128 and full 4096", ops, keep
+
+    raise SystemExit(f"unknown workload {name}")
+
+
+def run_other(torch, a):
+    metric, ops, keep = other_workload(torch, a.workload, a.seed)
+    step_s = time_ops(torch, ops, a.steps, a.warmup)
+    total_bytes = sum(op.nbytes for op in ops)
+    gpu_ms = sum(op.ms for op in ops)
+    slow = min(ops, key=lambda op: op.nbytes / op.ms)
+    n_launch = len(slow.calls)
+    out = {
+        "metric": metric,
+        "value": total_bytes / (gpu_ms * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "ms_per_step": step_s * 1e3,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 in, codes as the format says (arithmetic in the reference's promoted dtype)",
+        "data": "synthetic",
+        "config": {"workload": a.workload, "seed": a.seed,
+                   "value_is": "algorithmic bytes of all operations / sum of their GPU times"},
+        "roofline": {"bound": "hbm", "kernel": slow.kernel, "operation": slow.name,
+                     "achieved": slow.nbytes / (slow.ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": slow.nbytes / (slow.ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                     "traffic": None, "avg_launch_ms": slow.ms / n_launch,
+                     "launches_per_step": n_launch},
+        "operations": [{"name": op.name, "GBs": op.nbytes / (op.ms * 1e-3) / 1e9,
+                        "frac_of_hbm_peak": op.nbytes / (op.ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                        "ms": op.ms, "algorithmic_bytes": op.nbytes} for op in ops],
+        "ms_per_step_gpu": gpu_ms,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -125,6 +384,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     _lib.load()
     dev = torch.device("cuda:0")
+    if a.workload in ("fp8-w8a8", "sparse", "nvfp4", "hadamard"):
+        return run_other(torch, a)
     shapes = shapes_for(a.workload)
     args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group",
                             group_size=GROUP)
