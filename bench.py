@@ -251,11 +251,11 @@ def other_workload(torch, name, seed):
             dense = torch.empty_like(q)
             tmp = torch.empty(lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8, dtype=torch.uint8, device=dev)
             a = (q.data_ptr(), code(FP8), values.data_ptr(), bitmask.data_ptr(), rows, cols, st)
-            d = (values.data_ptr(), values.numel(), 1, bitmask.data_ptr(), None, dense.data_ptr(), tmp.data_ptr(), rows, cols, st)
+            d = (values.data_ptr(), values.numel(), 1, bitmask.data_ptr(), dense.data_ptr(), tmp.data_ptr(), rows, cols, st)
             _lib.check(lib.ctmi_sparse24_compress(*a))
             keep.extend([q, values, bitmask, dense, tmp])
             s_calls.append(lambda a=a: _lib.check(lib.ctmi_sparse24_compress(*a)))
-            t_calls.append(lambda d=d: _lib.check(lib.ctmi_bitmask_decompress(*d)))
+            t_calls.append(lambda d=d: _lib.check(lib.ctmi_sparse24_decompress(*d)))
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies * (n24 + n24 // 2 + n24 // 8)
         ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_kernel"),
@@ -322,7 +322,23 @@ def other_workload(torch, name, seed):
                 nb = sum(4 * x.numel() for x in xs)
                 ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb,
                               "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel"))
-        return "Hadamard rotation GB/s (bf16 MFMA), block 128 and full 4096", ops, keep
+        # rotation (block 128) + symmetric int4 group-128 quantization + pack_to_int32, one pass
+        mb = deterministic_hadamard_matrix(128, torch.bfloat16, dev).contiguous()
+        q = (torch.randint(0, 2, (128,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
+        keep.extend([mb, q])
+        for label in ("weights 4096x4096 (x16)", "weights 14336x4096 (x5)"):
+            calls = []
+            for x in tensors[label]:
+                packed = torch.empty(x.shape[0], x.shape[1] // 8, dtype=torch.int32, device=dev)
+                scale = torch.empty(x.shape[0], x.shape[1] // 128, dtype=torch.bfloat16, device=dev)
+                keep.extend([packed, scale])
+                a = (x.data_ptr(), code(x.dtype), x.numel(), 128, mb.data_ptr(), q.data_ptr(), None,
+                     4, 1, packed.data_ptr(), scale.data_ptr(), None, st)
+                calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_quant_pack(*a)))
+            nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in tensors[label])
+            ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}", calls, nb,
+                          "hadamard_quant_pack_kernel"))
+        return "Hadamard rotation GB/s (bf16 MFMA), block 128 and full 4096, and fused with int4 packing", ops, keep
 
     raise SystemExit(f"unknown workload {name}")
 

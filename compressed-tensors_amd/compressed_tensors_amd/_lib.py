@@ -141,6 +141,15 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     ),
+    "ctmi_hadamard_quant_pack": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int32,
+         c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "ctmi_sparse24_decompress": (
+        c_int32,
+        [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    ),
     "ctmi_get_24_bytemasks": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_void_p]),
     "ctmi_sparse24_compress": (
         c_int32,

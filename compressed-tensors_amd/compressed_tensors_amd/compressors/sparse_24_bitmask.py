@@ -84,7 +84,7 @@ def sparse24_bitmask_compress(
 def sparse24_bitmask_decompress(
     values: Tensor, bitmasks: Tensor, original_shape: torch.Size
 ) -> Tensor:
-    return _scatter(values, bitmasks, None, original_shape)
+    return _scatter(values, bitmasks, None, original_shape, two_four=True)
 
 
 @dataclass

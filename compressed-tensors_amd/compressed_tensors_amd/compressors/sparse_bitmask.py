@@ -67,7 +67,7 @@ def bitmask_compress(tensor: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
     return values, bitmask, row_offsets
 
 
-def _scatter(values: Tensor, bitmasks: Tensor, row_offsets, shape) -> Tensor:
+def _scatter(values: Tensor, bitmasks: Tensor, row_offsets, shape, two_four: bool = False) -> Tensor:
     values = to_gpu(values).contiguous().reshape(-1)
     bitmasks = to_gpu(bitmasks).contiguous()
     shape = [int(d) for d in shape]
@@ -87,12 +87,17 @@ def _scatter(values: Tensor, bitmasks: Tensor, row_offsets, shape) -> Tensor:
     if row_offsets is not None:
         row_offsets = to_gpu(row_offsets).to(torch.int64).contiguous()
         ro_ptr = row_offsets.data_ptr()
-    _lib.check(
-        lib.ctmi_bitmask_decompress(
-            values.data_ptr(), values.numel(), esize, bitmasks.data_ptr(), ro_ptr, out.data_ptr(), tmp.data_ptr(),
-            rows, cols, _lib.stream_of(dev),
+    if two_four:
+        rc = lib.ctmi_sparse24_decompress(
+            values.data_ptr(), values.numel(), esize, bitmasks.data_ptr(), out.data_ptr(),
+            tmp.data_ptr(), rows, cols, _lib.stream_of(dev),
         )
-    )
+    else:
+        rc = lib.ctmi_bitmask_decompress(
+            values.data_ptr(), values.numel(), esize, bitmasks.data_ptr(), ro_ptr, out.data_ptr(),
+            tmp.data_ptr(), rows, cols, _lib.stream_of(dev),
+        )
+    _lib.check(rc)
     return out
 
 

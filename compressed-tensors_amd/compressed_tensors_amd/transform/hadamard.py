@@ -37,6 +37,7 @@ __all__ = [
     "random_hadamard_signs",
     "hadamard_factors",
     "hadamard_apply",
+    "hadamard_quantize_pack",
     "apply_transform_weight",
     "TransformLocation",
     "TransformArgs",
@@ -152,6 +153,55 @@ def hadamard_apply(
             _lib.ptr(s_in), _lib.ptr(s_out), _lib.stream_of(dev),
         )
     )
+    return out
+
+
+def hadamard_quantize_pack(
+    value: Tensor,
+    n: int,
+    quantization_args,
+    sign_in: Optional[Tensor] = None,
+    sign_out: Optional[Tensor] = None,
+    matrix_t: Optional[Tensor] = None,
+    return_rotated: bool = False,
+) -> Dict[str, Tensor]:
+    """hadamard_apply, the min-max observer and pack-quantized compression in one
+    pass over a bf16 [rows, cols] tensor, for block size n (32, 64 or 128) equal
+    to the group size of a symmetric 4-bit integer scheme.  Returns what the
+    three steps return, bit for bit: weight_packed int32 [rows, cols / 8],
+    weight_scale bf16 [rows, cols / n], weight_shape int64 [2] (and the rotated
+    tensor under "rotated" if asked for)."""
+    x = to_gpu(value).contiguous()
+    args = quantization_args
+    if x.ndim != 2 or x.dtype != torch.bfloat16:
+        raise NotImplementedError("the fused path takes 2-D bfloat16 tensors")
+    if not (args.num_bits == 4 and str(getattr(args.type, "value", args.type)) == "int" and args.symmetric
+            and str(getattr(args.strategy, "value", args.strategy)) == "group" and args.group_size == n):
+        raise NotImplementedError(
+            "the fused path covers symmetric int4 group quantization with group_size == block size")
+    if n not in (32, 64, 128):
+        raise NotImplementedError("block size must be 32, 64 or 128")
+    rows, cols = x.shape
+    if cols % n != 0:
+        raise ValueError(f"{n} must divide the last dimension {cols}")
+    dev = x.device
+    mb_t = (_sylvester_bf16(n, dev) if matrix_t is None
+            else matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous())
+    s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
+    s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
+    packed = torch.empty((rows, cols // 8), dtype=torch.int32, device=dev)
+    scale = torch.empty((rows, cols // n), dtype=torch.bfloat16, device=dev)
+    rotated = torch.empty_like(x) if return_rotated else None
+    _lib.check(
+        _lib.load().ctmi_hadamard_quant_pack(
+            x.data_ptr(), _lib.dtype_code(x.dtype), x.numel(), n, mb_t.data_ptr(), _lib.ptr(s_in),
+            _lib.ptr(s_out), 4, 1, packed.data_ptr(), scale.data_ptr(), _lib.ptr(rotated),
+            _lib.stream_of(dev),
+        )
+    )
+    out = {"weight_packed": packed, "weight_scale": scale, "weight_shape": torch.tensor(x.shape)}
+    if return_rotated:
+        out["rotated"] = rotated
     return out
 
 

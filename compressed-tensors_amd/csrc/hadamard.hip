@@ -22,6 +22,8 @@
 // lane access on consecutive addresses.
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "qparams.h"
+#include "quant_core.h"
 #include "quant_fast.h"
 
 namespace ctmi {
@@ -31,6 +33,9 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kHadThreads = 256;
 constexpr int kHadWaves = kHadThreads / kWave;
+#ifndef CTMI_HQP_WG_PER_CU
+#define CTMI_HQP_WG_PER_CU 4  // workgroups per CU of the fused rotation + quantization kernel
+#endif
 #ifndef CTMI_HAD_KRON_WAVES
 #define CTMI_HAD_KRON_WAVES 2  // waves per SIMD the kernel for 64 x 64 is built for (measured best)
 #endif
@@ -388,6 +393,126 @@ static int launch_had_rows(const HadArgs& a, hipStream_t st) {
   return CTMI_OK;
 }
 
+// ---------------------------------------------------------------- rotation + int4 group quantization + packing
+// hadamard_rows_kernel with the rest of the W4A16 pipeline in its epilogue, for
+// group size == block size B: the rotated sub-row (rounded to bf16, as the
+// stand-alone transform stores it) IS one quantization group, so its min / max,
+// calculate_qparams (helpers.py:67-146, symmetric), _quantize (forward.py:455-487)
+// and pack_to_int32 (pack_quantized.py:186-246) follow in registers.  The bits are
+// those of the three separate steps; the rotated tensor never goes to memory
+// (unless `rotated` asks for it).  A sub-row's 128 outputs sit in the 4 lanes
+// l16 + 16 q; they agree on min / max through two lane exchanges.
+template <int B>
+__global__ void __launch_bounds__(kHadThreads)
+hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ mbt,
+                           const float* __restrict__ s_in, const float* __restrict__ s_out,
+                           int32_t* __restrict__ packed, uint16_t* __restrict__ scale,
+                           uint16_t* __restrict__ rotated, int64_t n_sub, float inv_sqrt_n,
+                           QpCfg cfg) {
+  constexpr int KS = B / 32, NP = B / 32;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & 15, lq = lane >> 4;
+
+  // The matrix fragments stay in LDS, in the lanes' own layout, and are read at
+  // each use (16 bytes per lane, conflict free): with the epilogue's registers on
+  // top of 128 for the matrix only one wavefront per SIMD would fit, and it is
+  // the number of wavefronts in flight that hides the memory latency here.
+  __shared__ u32x4_t frag_lds[2 * NP * KS][kWave];
+  __shared__ __align__(16) int32_t swap_lds[kHadWaves][16][16];
+  for (int f = wave; f < 2 * NP * KS; f += kHadWaves) {
+    const int nt = f / KS, ks = f % KS;
+    const int col = 32 * (nt / 2) + 8 * (l16 / 4) + 4 * (nt % 2) + (l16 % 4);
+    u32x4_t m = *reinterpret_cast<const u32x4_t*>(mbt + col * B + 32 * ks + 8 * lq);
+    if (s_in || s_out) {
+      const uint32_t fo = s_out ? ((f2u(s_out[col]) >> 31) * 0x80008000u) : 0u;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        const int k0 = 32 * ks + 8 * lq + 2 * w;
+        const uint32_t lo = s_in ? (f2u(s_in[k0]) >> 31) : 0u, hi = s_in ? (f2u(s_in[k0 + 1]) >> 31) : 0u;
+        m[w] ^= ((lo << 15) | (hi << 31)) ^ fo;
+      }
+    }
+    frag_lds[f][lane] = m;
+  }
+  __syncthreads();
+
+  const int64_t n_groups = (n_sub + 15) / 16;
+  const int64_t stride = (int64_t)gridDim.x * kHadWaves;
+  for (int64_t g = (int64_t)blockIdx.x * kHadWaves + wave; g < n_groups; g += stride) {
+    int64_t row = g * 16 + l16;
+    const bool keep = row < n_sub;
+    if (!keep) row = n_sub - 1;  // ragged last group: recompute the last sub-row, store nothing
+    const uint16_t* src = x + row * B + 8 * lq;
+    bf16x8_t xf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      xf[ks] = __builtin_bit_cast(bf16x8_t, ldg<uint16_t, 8>(src + 32 * ks));
+    Vec<uint32_t, 4> o[NP];  // the rotated sub-row in bf16: columns 32 p + 8 lq .. + 8
+    // A symmetric scale only needs max |x| of the group (min(min,0) and max(max,0)
+    // enter through their magnitudes, helpers.py:87-104).  Magnitudes of bf16
+    // values order like their bit patterns, a NaN above everything: the maximum is
+    // taken on the packed 16-bit halves, two elements per instruction.
+    typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+    u16x2_t top = {0, 0};
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      f32x4_t a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = {0.0f, 0.0f, 0.0f, 0.0f};
+      // keeps the compiler from hoisting these (loop-invariant) LDS reads out of
+      // the loop, back into 128 registers
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bf16x8_t m0 = __builtin_bit_cast(bf16x8_t, frag_lds[(2 * p) * KS + ks][lane]);
+        const bf16x8_t m1 = __builtin_bit_cast(bf16x8_t, frag_lds[(2 * p + 1) * KS + ks][lane]);
+        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(m0, xf[ks], a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(m1, xf[ks], a1, 0, 0, 0);
+      }
+      o[p].v[0] = pack_bf16x2(a0[0] * inv_sqrt_n, a0[1] * inv_sqrt_n);
+      o[p].v[1] = pack_bf16x2(a0[2] * inv_sqrt_n, a0[3] * inv_sqrt_n);
+      o[p].v[2] = pack_bf16x2(a1[0] * inv_sqrt_n, a1[1] * inv_sqrt_n);
+      o[p].v[3] = pack_bf16x2(a1[2] * inv_sqrt_n, a1[3] * inv_sqrt_n);
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2_t, o[p].v[w] & 0x7FFF7FFFu));
+    }
+    uint32_t mag = top.x > top.y ? top.x : top.y;
+#pragma unroll
+    for (int d = 16; d < 64; d <<= 1) {
+      const uint32_t other = (uint32_t)__shfl_xor((int)mag, d, kWave);
+      mag = other > mag ? other : mag;
+    }
+    // calculate_qparams, symmetric, in bf16 (helpers.py:101-122): the scheme is fixed
+    // here, so the general routine's dtype switches are spelled out instead
+    float sv = bf16_to_f32(f32_to_bf16(bf16_to_f32((uint16_t)mag) / cfg.sym_div));
+    sv = (sv != sv) ? sv : fmaxf(sv, 1.1920928955078125e-07f);
+    // Packed word 4 p + lq of the sub-row comes out of lane (l16, lq) for pair p.
+    // The 4 lanes of a sub-row swap words through a wave-private patch of LDS so
+    // that each stores NP neighbouring words (16 bytes at B = 128) instead of NP
+    // single ones 16 bytes apart.
+    int32_t* swap = &swap_lds[wave][l16][0];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      const Vec<int32_t, 1> w = quant_pack8<BF16, BF16, 4, false>(
+          __builtin_bit_cast(Vec<uint16_t, 8>, o[p]), sv, 0.0f, cfg.bit_min, cfg.bit_max);
+      swap[4 * p + lq] = w.v[0];
+      if (rotated && keep)
+        stg<uint16_t, 8>(rotated + row * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o[p]));
+    }
+    asm volatile("" ::: "memory");  // the reads below are of other lanes' words
+    if (keep) {
+      if (lq == 0) scale[row] = f32_to_bf16(sv);
+      if (lq < NP) {
+        Vec<int32_t, 4> out4;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) out4.v[j] = swap[4 * lq + j];
+        stg<int32_t, 4>(packed + row * (B / 8) + 4 * lq, out4);
+      }
+    }
+    asm volatile("" ::: "memory");  // the next group's words must not overtake these reads
+  }
+}
+
 // ---------------------------------------------------------------- Kronecker sizes, bf16, no LDS staging
 // n = A * B (1024 = 32 x 32, 2048 = 32 x 64, 4096 = 64 x 64): one wavefront per
 // data row, the row viewed as X [A sub-rows][B].  Both stages run on
@@ -695,4 +820,48 @@ extern "C" int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int
     hipLaunchKernelGGL(block_matmul_kernel<F32>, grid, 256, lds, st, (const float*)x, w,
                        (float*)out, chunks, h, sqrt_n);
   return check_launch("ctmi_block_matmul");
+}
+
+extern "C" int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t numel, int32_t b_dim,
+                                        const void* mb_t, const float* sign_in,
+                                        const float* sign_out, int32_t num_bits, int32_t symmetric,
+                                        int32_t* packed, void* scale, void* rotated, void* stream) {
+  CTMI_REQUIRE(numel >= 0, CTMI_ERR_VALUE, "negative size");
+  CTMI_REQUIRE(io_dtype == CTMI_BF16, CTMI_ERR_UNSUPPORTED,
+               "the fused rotation + quantization takes bfloat16 tensors");
+  CTMI_REQUIRE(b_dim == 32 || b_dim == 64 || b_dim == 128, CTMI_ERR_UNSUPPORTED,
+               "block (= group) size must be 32, 64 or 128, got %d", b_dim);
+  CTMI_REQUIRE(num_bits == 4 && symmetric, CTMI_ERR_UNSUPPORTED,
+               "only symmetric 4-bit integer quantization is fused");
+  CTMI_REQUIRE(numel % b_dim == 0, CTMI_ERR_VALUE,
+               "tensor size %lld is not a multiple of the block size %d", (long long)numel, b_dim);
+  if (numel == 0) return CTMI_OK;
+  CTMI_REQUIRE(x && mb_t && packed && scale, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)mb_t % 16 == 0 && (uintptr_t)rotated % 16 == 0 &&
+                   (uintptr_t)packed % 4 == 0 && (uintptr_t)scale % 2 == 0,
+               CTMI_ERR_VALUE, "tensors must be 16-byte aligned");
+  QpCfg c{};
+  quant_range(CTMI_QTYPE_INT, num_bits, &c.bit_min, &c.bit_max);
+  c.range = c.bit_max - c.bit_min;
+  c.sym_div = (float)((double)c.range / 2.0);
+  c.qtype = CTMI_QTYPE_INT;
+  c.num_bits = num_bits;
+  c.symmetric = 1;
+  c.mt = c.zp_sub_dtype = c.scale_dtype = CTMI_BF16;
+  c.zp_dtype = CTMI_I8;
+  const int64_t n_sub = numel / b_dim;
+  const int64_t wgs = cdiv(cdiv(n_sub, 16), kHadWaves);
+  const int64_t cap = 256 * CTMI_HQP_WG_PER_CU;
+  const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
+  const float inv = 1.0f / sqrtf((float)b_dim);
+  hipStream_t st = (hipStream_t)stream;
+#define CTMI_HQP(BB)                                                                              \
+  hipLaunchKernelGGL(hadamard_quant_pack_kernel<BB>, grid, kHadThreads, 0, st, (const uint16_t*)x, \
+                     (const uint16_t*)mb_t, sign_in, sign_out, packed, (uint16_t*)scale,          \
+                     (uint16_t*)rotated, n_sub, inv, c)
+  if (b_dim == 32) CTMI_HQP(32);
+  else if (b_dim == 64) CTMI_HQP(64);
+  else CTMI_HQP(128);
+#undef CTMI_HQP
+  return check_launch("ctmi_hadamard_quant_pack");
 }

@@ -689,10 +689,9 @@ extern "C" int ctmi_bitmask_compact(const void* x, int32_t elem_size, const uint
   return check_launch("ctmi_bitmask_compact");
 }
 
-extern "C" int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_size,
-                                       const uint8_t* bitmask, const int64_t* row_offsets,
-                                       void* out, void* tmp, int64_t rows, int64_t cols,
-                                       void* stream) {
+static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
+                         const uint8_t* bitmask, const int64_t* row_offsets, void* out, void* tmp,
+                         int64_t rows, int64_t cols, void* stream, bool try_24, const char* what) {
   CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
   int rc = check_elem(elem_size);
   if (rc) return rc;
@@ -712,7 +711,7 @@ extern "C" int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int3
     // the 2:4 streaming kernel first (see sparse24_scatter_kernel)
     const int64_t numel = rows * cols;
     const int e = elem_size == 1 ? 16 : 8;
-    if (nvalues * 2 == numel && cols % 8 == 0 && numel % e == 0 && (uintptr_t)out % 16 == 0 &&
+    if (try_24 && nvalues * 2 == numel && cols % 8 == 0 && numel % e == 0 && (uintptr_t)out % 16 == 0 &&
         (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 2 == 0 && numel / e < (1ll << 40)) {
       int* flag = (int*)(offs + rows);
       const int64_t n_items = numel / e;
@@ -751,8 +750,25 @@ extern "C" int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int3
     hipLaunchKernelGGL(bitmask_scatter_kernel<uint32_t>, grid, kBlock, 0, st,
                        (const uint32_t*)values, nvalues, bitmask, row_offsets, (uint32_t*)out, rows,
                        cols, pc, only_if);
-  return check_launch("ctmi_bitmask_decompress");
+  return check_launch(what);
 }
+
+extern "C" int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_size,
+                                       const uint8_t* bitmask, const int64_t* row_offsets,
+                                       void* out, void* tmp, int64_t rows, int64_t cols,
+                                       void* stream) {
+  return scatter_entry(values, nvalues, elem_size, bitmask, row_offsets, out, tmp, rows, cols,
+                       stream, false, "ctmi_bitmask_decompress");
+}
+
+extern "C" int ctmi_sparse24_decompress(const void* values, int64_t nvalues, int32_t elem_size,
+                                        const uint8_t* bitmask, void* out, void* tmp, int64_t rows,
+                                        int64_t cols, void* stream) {
+  CTMI_REQUIRE(tmp != nullptr || rows == 0 || cols == 0, CTMI_ERR_VALUE, "tmp is NULL");
+  return scatter_entry(values, nvalues, elem_size, bitmask, nullptr, out, tmp, rows, cols, stream,
+                       true, "ctmi_sparse24_decompress");
+}
+
 
 // dispatch over the element types get_24_bytemasks can rank
 #define CTMI_DISPATCH_24(DTYPE, ...)                                        \

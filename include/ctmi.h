@@ -184,20 +184,25 @@ int ctmi_bitmask_compact(const void* x, int32_t elem_size, const uint8_t* bitmas
                          const int64_t* row_offsets, void* values, int64_t rows, int64_t cols,
                          void* stream);
 
-/* A18 / A22.  bitmask_decompress (sparse_bitmask.py:152-169) and
- * sparse24_bitmask_decompress (sparse_24_bitmask.py:206-224): scatter `values`
+/* A18.  bitmask_decompress (sparse_bitmask.py:152-169): scatter `values`
  * (nvalues elements, consumed in row-major order of the set bits; set bits
  * beyond nvalues read as zero) into a zero-filled [rows, cols].
  * row_offsets may be NULL: it is then recomputed from the bitmask into tmp
- * (ctmi_bitmask_tmp_bytes(rows) bytes + rows*8 bytes for the offsets + 8 bytes
- * for a flag).  With NULL row_offsets and exactly half as many values as
- * elements the bitmask is first taken to be a 2:4 one (2 kept per group of 4),
- * which needs no prefix sums; the general path runs behind it only if some
- * group turns out not to keep exactly 2. */
+ * (ctmi_bitmask_tmp_bytes(rows) + rows*8 + 8 bytes). */
 int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_size,
                             const uint8_t* bitmask,
                             const int64_t* row_offsets, void* out, void* tmp, int64_t rows,
                             int64_t cols, void* stream);
+
+/* A22.  sparse24_bitmask_decompress (sparse_24_bitmask.py:206-224): the same
+ * scatter, `out[mask] = values`, for any bitmask.  A bitmask that keeps exactly 2
+ * of every 4 columns (what the format holds) needs no prefix sums and is
+ * expanded in one streaming pass; the general path of ctmi_bitmask_decompress is
+ * enqueued behind it and does its work only if some group turned out not to
+ * keep exactly 2.  tmp: ctmi_bitmask_tmp_bytes(rows) + rows*8 + 8 bytes. */
+int ctmi_sparse24_decompress(const void* values, int64_t nvalues, int32_t elem_size,
+                             const uint8_t* bitmask, void* out, void* tmp, int64_t rows,
+                             int64_t cols, void* stream);
 
 /* A20.  get_24_bytemasks (sparse_24_bitmask.py:227-260): top-2-of-4 by
  * |value| with torch.topk's tie order.  x_dtype: a float type (ranked on the
@@ -258,6 +263,18 @@ int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype);
 int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t a_dim,
                         int32_t b_dim, const void* ma_t, const void* mb_t, const float* sign_in,
                         const float* sign_out, void* stream);
+
+/* A24 / A25 + A2 + A1 + A11 in one pass, for bf16 tensors, block size b_dim (32,
+ * 64 or 128) equal to the quantization group size, symmetric 4-bit integers:
+ * the rotation of ctmi_hadamard_apply (a_dim == 1) followed, per rotated block,
+ * by the min-max observer, calculate_qparams and the quantize + pack_to_int32 of
+ * ctmi_pack_quantized_compress.  Same bits as those calls in sequence.
+ * packed: int32 [numel / 8]; scale: bf16 [numel / b_dim] (the group scales, row
+ * major); rotated: optional bf16 [numel] copy of the rotated tensor, or NULL. */
+int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t numel, int32_t b_dim,
+                             const void* mb_t, const float* sign_in, const float* sign_out,
+                             int32_t num_bits, int32_t symmetric, int32_t* packed, void* scale,
+                             void* rotated, void* stream);
 
 /* A24 for an arbitrary explicit fp32 matrix w [h,h] (small h, or matrices that
  * are not +-1): every run of h consecutive elements x becomes x * w / sqrt(h).
