@@ -125,20 +125,38 @@ bitmask_count_kernel(const R* __restrict__ x, uint32_t nz_mask, uint8_t* __restr
   for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
     const R* row = x + r * cols;
     int64_t cnt = 0;
-    for (int64_t b = threadIdx.x; b < pc; b += kBlock) {
-      uint32_t bits = 0;
-      if (vec) {
-        Vec<R, 8> a = ldg<R, 8>(row + b * 8);
+    if (vec) {
+      // 4 vectors per thread and step, all loads first
+      constexpr int U = 4;
+      for (int64_t b0 = threadIdx.x; b0 < pc; b0 += kBlock * U) {
+        Vec<R, 8> a[U];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) bits |= (uint32_t)(((uint32_t)a.v[j] & nz_mask) != 0) << j;
-      } else {
+        for (int k = 0; k < U; ++k) {
+          const int64_t b = b0 + k * kBlock;
+          a[k] = ldg<R, 8>(row + (b < pc ? b : pc - 1) * 8);  // past the end: re-read, not used
+        }
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+          const int64_t b = b0 + k * kBlock;
+          if (b < pc) {
+            uint32_t bits = 0;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) bits |= (uint32_t)(((uint32_t)a[k].v[j] & nz_mask) != 0) << j;
+            bitmask[r * pc + b] = (uint8_t)bits;
+            cnt += __popc(bits);
+          }
+        }
+      }
+    } else {
+      for (int64_t b = threadIdx.x; b < pc; b += kBlock) {
+        uint32_t bits = 0;
         for (int j = 0; j < 8; ++j) {
           const int64_t c = b * 8 + j;
           if (c < cols) bits |= (uint32_t)(((uint32_t)row[c] & nz_mask) != 0) << j;
         }
+        bitmask[r * pc + b] = (uint8_t)bits;
+        cnt += __popc(bits);
       }
-      bitmask[r * pc + b] = (uint8_t)bits;
-      cnt += __popc(bits);
     }
     const int64_t t = block_sum(cnt, red);
     if (threadIdx.x == 0) counts[r] = t;
@@ -318,6 +336,97 @@ bitmask_scatter_kernel(const R* __restrict__ values, int64_t nvalues,
       __syncthreads();
     }
   }
+}
+
+// ------------------------------------------------------------------ bitmask decompress, one wavefront per row
+// For rows that are whole 16-column words (cols % 16 == 0) and 16-byte aligned
+// buffers.  A lane owns 16 neighbouring columns of a 1024-column span; the
+// wavefront's scan of the lanes' popcounts says where each lane's values start,
+// the values of the span are copied into a wave-private patch of LDS with
+// aligned 16-byte loads, and every lane picks its own out of it.  No workgroup
+// barrier anywhere: LDS operations of one wavefront complete in order.  The
+// row's bitmask is fetched in one go before anything depends on it.
+constexpr int kScatterSpan = 1024;      // columns per wavefront and step
+constexpr int kScatterMaxSteps = 16;    // rows of up to 16384 columns
+template <typename R>
+__global__ void __launch_bounds__(kBlock)
+bitmask_scatter_wave_kernel(const R* __restrict__ values, int64_t nvalues,
+                            const uint8_t* __restrict__ bitmask,
+                            const int64_t* __restrict__ row_offsets, R* __restrict__ out,
+                            int64_t rows, int64_t cols, int64_t pc, const int* only_if) {
+  if (only_if && *only_if == 0) return;
+  constexpr int VE = 16 / (int)sizeof(R);  // elements per 16-byte vector
+  __shared__ __align__(16) R stage_all[kWaves][kScatterSpan + 2 * VE];
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  R* stage = stage_all[wave];
+  for (int64_t r = (int64_t)blockIdx.x * kWaves + wave; r < rows; r += (int64_t)gridDim.x * kWaves) {
+  const uint16_t* words = reinterpret_cast<const uint16_t*>(bitmask + r * pc);
+  const int steps = (int)((cols + kScatterSpan - 1) / kScatterSpan);
+  uint32_t bits_of[kScatterMaxSteps];
+#pragma unroll
+  for (int it = 0; it < kScatterMaxSteps; ++it) {
+    const int64_t col = (int64_t)it * kScatterSpan + 16 * lane;
+    bits_of[it] = (it < steps && col < cols) ? words[col / 16] : 0u;
+  }
+  int64_t src = row_offsets[r];
+  R* row = out + r * cols;
+#pragma unroll
+  for (int it = 0; it < kScatterMaxSteps; ++it) {
+    if (it >= steps) break;
+    const uint32_t bits = bits_of[it];
+    const int cnt = __popc(bits);
+    const int inc = wave_inclusive_scan(cnt);
+    const int total = __shfl(inc, kWave - 1, kWave);
+    // values [src, src + total) -> stage, from the 16-byte boundary below src
+    const int64_t base = src & ~(int64_t)(VE - 1);
+    const int off = (int)(src - base);
+    const int nvecs = (off + total + VE - 1) / VE;
+    for (int i = lane; i < nvecs; i += kWave) {
+      const int64_t e0 = base + (int64_t)i * VE;
+      Vec<R, VE> v;
+      if (e0 < nvalues) {
+        // an aligned vector that starts inside the buffer never leaves its page
+        v = ldg<R, VE>(values + e0);
+#pragma unroll
+        for (int e = 0; e < VE; ++e)
+          if (e0 + e >= nvalues) v.v[e] = (R)0;  // more set bits than values: zeros
+      } else {
+#pragma unroll
+        for (int e = 0; e < VE; ++e) v.v[e] = (R)0;
+      }
+      *reinterpret_cast<Vec<R, VE>*>(stage + i * VE) = v;
+    }
+    asm volatile("" ::: "memory");  // the reads below are of other lanes' writes
+    const int64_t col = (int64_t)it * kScatterSpan + 16 * lane;
+    if (col < cols) {
+      int idx = off + inc - cnt;
+      Vec<R, 16> o;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const bool set = (bits >> j) & 1u;
+        o.v[j] = set ? stage[idx] : (R)0;
+        idx += set ? 1 : 0;
+      }
+#pragma unroll
+      for (int h = 0; h < 16 / VE; ++h) {
+        Vec<R, VE> part;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) part.v[e] = o.v[h * VE + e];
+        stg<R, VE>(row + col + h * VE, part);
+      }
+    }
+    asm volatile("" ::: "memory");  // the next step's writes must not overtake these reads
+    src += total;
+  }
+  }
+}
+
+template <typename R>
+static bool scatter_wave_ok(const void* values, const uint8_t* bitmask, const void* out,
+                            int64_t cols) {
+  return cols % 16 == 0 && cols <= (int64_t)kScatterSpan * kScatterMaxSteps &&
+         (uintptr_t)values % 16 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)bitmask % 2 == 0 &&
+         (cols * sizeof(R)) % 16 == 0;
 }
 
 // ------------------------------------------------------------------ 2:4 decompress, streaming
@@ -739,17 +848,21 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
                        rows, only_if);
     row_offsets = offs;
   }
-  if (elem_size == 1)
-    hipLaunchKernelGGL(bitmask_scatter_kernel<uint8_t>, grid, kBlock, 0, st, (const uint8_t*)values,
-                       nvalues, bitmask, row_offsets, (uint8_t*)out, rows, cols, pc, only_if);
-  else if (elem_size == 2)
-    hipLaunchKernelGGL(bitmask_scatter_kernel<uint16_t>, grid, kBlock, 0, st,
-                       (const uint16_t*)values, nvalues, bitmask, row_offsets, (uint16_t*)out, rows,
-                       cols, pc, only_if);
-  else
-    hipLaunchKernelGGL(bitmask_scatter_kernel<uint32_t>, grid, kBlock, 0, st,
-                       (const uint32_t*)values, nvalues, bitmask, row_offsets, (uint32_t*)out, rows,
-                       cols, pc, only_if);
+#define CTMI_SCATTER(R)                                                                           \
+  if (scatter_wave_ok<R>(values, bitmask, out, cols))                                             \
+    hipLaunchKernelGGL(bitmask_scatter_wave_kernel<R>, (unsigned)wave_grid, kBlock, 0, st,        \
+                       (const R*)values, nvalues, bitmask, row_offsets, (R*)out, rows, cols, pc,  \
+                       only_if);                                                                  \
+  else                                                                                            \
+    hipLaunchKernelGGL(bitmask_scatter_kernel<R>, grid, kBlock, 0, st, (const R*)values, nvalues, \
+                       bitmask, row_offsets, (R*)out, rows, cols, pc, only_if)
+  int64_t wave_grid = cdiv(rows, kWaves);
+  if (wave_grid > (1 << 24)) wave_grid = 1 << 24;
+  if (only_if && wave_grid > 512) wave_grid = 512;  // rarely does anything: keep the launch small
+  if (elem_size == 1) { CTMI_SCATTER(uint8_t); }
+  else if (elem_size == 2) { CTMI_SCATTER(uint16_t); }
+  else { CTMI_SCATTER(uint32_t); }
+#undef CTMI_SCATTER
   return check_launch(what);
 }
 

@@ -45,6 +45,10 @@ BM = [
     ((2, 10), torch.float32, 0.5), ((16, 50), torch.bfloat16, 0.9), ((7, 64), torch.float16, 0.0),
     ((3, 9), torch.bfloat16, 1.0), ((33, 2050), torch.bfloat16, 0.5), ((64, 4096), torch.bfloat16, 0.5),
     ((9, 300), FP8, 0.6), ((5, 100), torch.int8, 0.7), ((300, 24), torch.bfloat16, 0.3),
+    # rows of whole 16-column words: the one-wavefront-per-row scatter (several 1024-column
+    # steps, a partial last one, row counts that do not fill a workgroup, dense and empty rows)
+    ((33, 2064), torch.bfloat16, 0.5), ((6, 16384), FP8, 0.3), ((5, 1040), torch.float32, 0.8),
+    ((10, 48), torch.bfloat16, 0.0), ((7, 1024), torch.float16, 1.0), ((3, 16400), torch.bfloat16, 0.5),
 ]
 
 
