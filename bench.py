@@ -181,17 +181,18 @@ def other_workload(torch, name, seed):
 
     if name == "fp8-w8a8":
         args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
-        q_calls, d_calls, n = [], [], 0
+        from compressed_tensors_amd.compressors import QuantizedWeightBatch
+        entries, n = [], 0
         for _, r, c in shapes_for("llama3-8b-w4a16"):
             w = randn(r, c, 0.02)
             hot = torch.rand(r, c, generator=gen, device=dev) < 1e-3
             w = torch.where(hot, w * 20, w)
             scale, zp = observe_weight_qparams(w, args)
-            codes = torch.empty(r, c, dtype=FP8, device=dev)
-            dense = torch.empty(r, c, dtype=torch.bfloat16, device=dev)
-            q_calls.append(qdq(w, codes, build_qparams(w, scale, None, args), 1, 0))
-            d_calls.append(qdq(codes, dense, build_qparams(codes, scale, None, args), 0, 1))
+            entries.append(dict(weight=w, scale=scale, zero_point=None, quantization_args=args))
             n += r * c
+        batch = QuantizedWeightBatch(entries)   # one ctmi_qdq_many call per direction
+        keep.append(batch)
+        q_calls, d_calls = [batch.compress], [batch.decompress]
         acts, a_obs, a_fq = [], [], []
         targs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="token",
                                  dynamic=True)

@@ -85,6 +85,20 @@ class WeightJob(ctypes.Structure):
     ]
 
 
+class QdqJob(ctypes.Structure):
+    """ctmi_qdq_job"""
+
+    _fields_ = [
+        ("x", c_void_p),
+        ("out", c_void_p),
+        ("rows", c_int64),
+        ("cols", c_int64),
+        ("x_dtype", c_int32),
+        ("out_dtype", c_int32),
+        ("qp", QParams),
+    ]
+
+
 # name -> (restype, argtypes); must list every symbol of include/ctmi.h
 SIGNATURES = {
     "ctmi_last_error": (c_char_p, []),
@@ -93,6 +107,7 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int64, _QP, c_int32, c_int32, c_void_p],
     ),
+    "ctmi_qdq_many": (c_int32, [POINTER(QdqJob), c_int64, c_int32, c_int32, c_void_p]),
     "ctmi_pack_to_int32": (
         c_int32,
         [c_void_p, c_void_p, c_int64, c_int64, c_int32, c_int32, c_void_p],

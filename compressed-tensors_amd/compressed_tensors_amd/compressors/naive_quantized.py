@@ -8,18 +8,71 @@ from typing import Dict, Optional, Tuple
 import torch
 from torch import Tensor
 
+from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
 from compressed_tensors_amd.compressors.quantized_base import BaseQuantizationCompressor
 from compressed_tensors_amd.config import CompressionFormat
-from compressed_tensors_amd.quantization.forward import dequantize, quantize
+from compressed_tensors_amd.quantization.forward import (
+    _rows_cols, _ShapeOnly, build_qparams, dequantize, infer_dequant_args, quantize,
+)
 from compressed_tensors_amd.quantization.helpers import can_quantize
 from compressed_tensors_amd.quantization.quant_args import QuantizationArgs
 
 __all__ = [
+    "QuantizedWeightBatch",
     "NaiveQuantizationCompressor",
     "IntQuantizationCompressor",
     "FloatQuantizationCompressor",
 ]
+
+
+class QuantizedWeightBatch:
+    """Every weight of a state dict prepared for one-call quantize / dequantize
+    (ctmi_qdq_many): codes in int8 or float8_e4m3fn as the scheme says, buffers
+    allocated once, `compress()` / `decompress()` only enqueue kernels."""
+
+    def __init__(self, entries, device=None):
+        """entries: dicts with weight, scale, quantization_args and optionally
+        zero_point, g_idx (tensors on the GPU, or moved there)"""
+        self.n = len(entries)
+        self.device = device
+        self._keep = []
+        self.weights, self.codes, self.dense = [], [], []
+        self._cjobs = (_lib.QdqJob * max(self.n, 1))()
+        self._djobs = (_lib.QdqJob * max(self.n, 1))()
+        for i, e in enumerate(entries):
+            args = e["quantization_args"]
+            w, scale, zp, g_idx = (to_gpu(e.get(k)) for k in ("weight", "scale", "zero_point", "g_idx"))
+            if self.device is None:
+                self.device = w.device
+            w = w.contiguous()
+            rows, cols = _rows_cols(w)
+            codes = torch.empty(w.shape, dtype=args.pytorch_dtype(), device=w.device)
+            dense = torch.empty(w.shape, dtype=scale.dtype, device=w.device)
+            cplan = build_qparams(w, scale, zp, args, g_idx, None)
+            dq_args = infer_dequant_args(_ShapeOnly(w.shape, codes.dtype), scale)
+            # a symmetric scheme stores no zero points: its decompression sees none
+            dplan = build_qparams(_ShapeOnly(w.shape, codes.dtype), scale,
+                                  None if args.symmetric else zp, dq_args, g_idx, None)
+            self._keep += [cplan, dplan, scale, zp, g_idx]
+            cj, dj = self._cjobs[i], self._djobs[i]
+            cj.x, cj.out, cj.rows, cj.cols = w.data_ptr(), codes.data_ptr(), rows, cols
+            cj.x_dtype, cj.out_dtype, cj.qp = _lib.dtype_code(w.dtype), _lib.dtype_code(codes.dtype), cplan.qp
+            dj.x, dj.out, dj.rows, dj.cols = codes.data_ptr(), dense.data_ptr(), rows, cols
+            dj.x_dtype, dj.out_dtype, dj.qp = _lib.dtype_code(codes.dtype), _lib.dtype_code(dense.dtype), dplan.qp
+            self.weights.append(w)
+            self.codes.append(codes)
+            self.dense.append(dense)
+
+    def compress(self):
+        """enqueue the quantization of every weight; returns the code tensors"""
+        _lib.check(_lib.load().ctmi_qdq_many(self._cjobs, self.n, 1, 0, _lib.stream_of(self.device)))
+        return self.codes
+
+    def decompress(self):
+        """enqueue the dequantization of every code tensor; returns the dense tensors"""
+        _lib.check(_lib.load().ctmi_qdq_many(self._djobs, self.n, 0, 1, _lib.stream_of(self.device)))
+        return self.dense
 
 
 @BaseCompressor.register(name=CompressionFormat.naive_quantized.value)
@@ -72,6 +125,61 @@ class NaiveQuantizationCompressor(BaseQuantizationCompressor):
             zero_point=to_gpu(compressed_data.get("weight_zero_point", None)),
             g_idx=to_gpu(compressed_data.get("weight_g_idx", None)),
         )
+
+
+def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,
+                                 compression_device=None, **kwargs):
+    """BaseQuantizationCompressor.compress (quantized_compressors/base.py:69-161) with
+    every quantizable weight handed to the C ABI in one call: same keys, dtypes and
+    values as the per-weight loop."""
+    jobs, names = [], []
+    for name in list(model_state.keys()):
+        if not name.endswith("weight"):
+            continue
+        prefix = name[: -len("weight")]
+        scale = model_state.get(prefix + "weight_scale", None)
+        if scale is None:
+            continue
+        if model_state.get(prefix + "weight_global_scale", None) is not None:
+            raise ValueError("global_scale is not supported for the NaiveQuantizationCompressor")
+        module_path = prefix[:-1] if prefix.endswith(".") else prefix
+        args = names_to_scheme[module_path].weights
+        weight = model_state[name]
+        if not can_quantize(weight, args) or weight.ndim < 1 or weight.numel() == 0:
+            continue  # the per-weight path below passes it through
+        jobs.append(dict(weight=weight, scale=scale, quantization_args=args,
+                         zero_point=model_state.get(prefix + "weight_zero_point", None),
+                         g_idx=model_state.get(prefix + "weight_g_idx", None)))
+        names.append(name)
+    codes_by_name = dict(zip(names, QuantizedWeightBatch(jobs).compress())) if jobs else {}
+
+    def move(t):
+        return t if compression_device is None else t.to(compression_device)
+
+    out = {}
+    for name in list(model_state.keys()):
+        value = model_state[name]
+        if name in codes_by_name:
+            out[name] = move(codes_by_name[name])
+        elif name.endswith("weight") and model_state.get(name[: -len("weight")] + "weight_scale") is not None:
+            prefix = name[: -len("weight")]
+            module_path = prefix[:-1] if prefix.endswith(".") else prefix
+            single = self.compress_weight(
+                weight=value, scale=model_state[prefix + "weight_scale"],
+                zero_point=model_state.get(prefix + "weight_zero_point", None),
+                g_idx=model_state.get(prefix + "weight_g_idx", None),
+                quantization_args=names_to_scheme[module_path].weights,
+                device=compression_device)
+            for key, tensor in single.items():
+                out[prefix + key] = move(tensor)
+        elif name.endswith("zero_point") and self._skip_zp(name, names_to_scheme):
+            continue
+        else:
+            out[name] = move(value)
+    return out
+
+
+NaiveQuantizationCompressor.compress = _compress_state_dict_batched
 
 
 @BaseCompressor.register(name=CompressionFormat.int_quantized.value)

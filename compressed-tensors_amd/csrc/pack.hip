@@ -19,6 +19,7 @@
 #include "quant_core.h"
 #include "quant_fast.h"
 #include "vec_geom.h"
+#include "job_table.h"
 
 namespace ctmi {
 
@@ -215,111 +216,14 @@ __global__ void __launch_bounds__(256) pq_decompress_generic_kernel(FusedArgs a)
 constexpr int kPqTuning[5] = {CTMI_PQ_TUNING};
 constexpr int kCompressBlock = kPqTuning[0], kCompressUnroll = kPqTuning[1];
 constexpr int kDecompressBlock = kPqTuning[2], kDecompressUnroll = kPqTuning[3];
-constexpr int kMaxJobs = kPqTuning[4];
-
-struct VecJob {
-  const void* src;
-  void* dst;
-  const void* scale;
-  const int8_t* zp;
-  VecGeom g;
-};
-
-// What a workgroup needs of its weight, 64 bytes so that one scalar load brings
-// it in.  Scale of item v (8 elements): `v >> shift` when scales are numbered
-// like the items (FLAT), else row r = v / vpr, column block (v - r*vpr) / vpb,
-// index r * s_stride + block (s_stride 0 when all rows share one scale row).
-struct alignas(64) PqJob {
-  const void* src;
-  void* dst;
-  const void* scale;
-  const int8_t* zp;
-  uint32_t shift, reserved;
-  uint32_t vpr_d, vpr_m, vpr_s;
-  uint32_t vpb_m, vpb_s;
-  uint32_t s_stride;
-};
-static_assert(sizeof(PqJob) == 64, "one scalar load per job");
-
-// Kernel argument of a chained launch.  What decides which job a workgroup
-// belongs to and whether a lane has work comes first, in one scalar load; unused
-// chunk_end entries hold 0xFFFFFFFF.
-struct PqJobTable {
-  uint32_t chunk_end[kMaxJobs];  // running total of chunks, job 0 .. j
-  uint32_t nvec[kMaxJobs];       // items of job j
-  PqJob job[kMaxJobs];
-  float qmin, qmax;
-  int32_t n;
-};
-
-static inline bool flat_geometry(const VecGeom& g) { return g.mode == 0; }
-
-static inline PqJob make_pq_job(const VecJob& j) {
-  PqJob o;
-  o.src = j.src;
-  o.dst = j.dst;
-  o.scale = j.scale;
-  o.zp = j.zp;
-  o.shift = j.g.shift;
-  o.reserved = 0;
-  o.vpr_d = j.g.vpr.d;
-  o.vpr_m = j.g.vpr.m;
-  o.vpr_s = j.g.vpr.s;
-  o.vpb_m = j.g.vpb.m;
-  o.vpb_s = j.g.vpb.s;
-  o.s_stride = j.g.row_scaled ? j.g.s_cols : 0u;
-  return o;
-}
-
-static_assert(kMaxJobs == 8 && offsetof(PqJobTable, chunk_end) == 0 &&
-                  offsetof(PqJobTable, nvec) == 32,
-              "find_job reads chunk_end and nvec as the first 16 dwords of the kernel argument");
-
-// The job of workgroup `chunk`, the chunk's number within that job and the job's
-// item count.  The table must be the kernel's only argument.  Its head (chunk_end
-// and nvec) is fetched with one 64-byte scalar load written out by hand: left to
-// itself the compiler turns the search into a chain of dependent loads, and a
-// wave of these kernels lives too short to hide several scalar round trips.
-// The search itself is then compares and selects on registers, and the job's 64
-// bytes follow as one more batch of scalar loads.
-__device__ __forceinline__ PqJob find_job(const PqJobTable& t, uint32_t chunk, uint32_t* local,
-                                          uint32_t* nvec) {
-  typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
-  u32x16 head;
-  asm volatile("s_load_dwordx16 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)"
-               : "=s"(head)
-               : "s"(__builtin_amdgcn_kernarg_segment_ptr()));
-  uint32_t j = 0, first = 0, nv = head[8];
-#pragma unroll
-  for (int i = 0; i < kMaxJobs - 1; ++i) {
-    const uint32_t e = head[i];
-    const bool past = chunk >= e;
-    j = past ? (uint32_t)(i + 1) : j;  // chunk_end ascends: the last hit wins
-    first = past ? e : first;
-    nv = past ? head[9 + i] : nv;
-  }
-  *local = chunk - first;
-  *nvec = nv;
-  return t.job[j];
-}
-
-template <bool FLAT>
-__device__ __forceinline__ uint32_t pq_scale_index(uint32_t v, const PqJob& job) {
-  if constexpr (FLAT) {
-    return v >> job.shift;
-  } else {
-    const uint32_t r = (uint32_t)(((uint64_t)v * job.vpr_m) >> 31) >> job.vpr_s;
-    const uint32_t cv = v - r * job.vpr_d;
-    return r * job.s_stride + ((uint32_t)(((uint64_t)cv * job.vpb_m) >> 31) >> job.vpb_s);
-  }
-}
+static_assert(kPqTuning[4] == kMaxJobs, "jobs per launch are fixed by job_table.h");
 
 template <typename XT, typename ST, int BITS, bool HAS_ZP, bool FLAT>
-__global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const PqJobTable t) {
+__global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const ChainTable t) {
   constexpr int W = BITS / 4;  // output words per item
   constexpr int B = kCompressBlock, U = kCompressUnroll;
   uint32_t chunk, nvec;
-  const PqJob job = find_job(t, blockIdx.x, &chunk, &nvec);
+  const ChainJob job = find_job(t, blockIdx.x, &chunk, &nvec);
   const auto* __restrict__ x = (const typename XT::raw*)job.src;
   const auto* __restrict__ scale = (const typename ST::raw*)job.scale;
   const int8_t* __restrict__ zp = job.zp;
@@ -339,7 +243,7 @@ __global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const P
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < nvec) {
         xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
-        const uint32_t si = pq_scale_index<FLAT>(v, job);
+        const uint32_t si = chain_scale_index<FLAT>(v, job);
         sraw[k] = scale[si];
         if constexpr (HAS_ZP) zraw[k] = zp[si];
       }
@@ -359,11 +263,11 @@ __global__ void __launch_bounds__(kCompressBlock) pq_compress_vec_kernel(const P
 }
 
 template <typename ST, int BITS, bool HAS_ZP, bool FLAT>
-__global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(const PqJobTable t) {
+__global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(const ChainTable t) {
   constexpr int W = BITS / 4;
   constexpr int B = kDecompressBlock, U = kDecompressUnroll;
   uint32_t chunk, nvec;
-  const PqJob job = find_job(t, blockIdx.x, &chunk, &nvec);
+  const ChainJob job = find_job(t, blockIdx.x, &chunk, &nvec);
   const int32_t* __restrict__ packed = (const int32_t*)job.src;
   const auto* __restrict__ scale = (const typename ST::raw*)job.scale;
   const int8_t* __restrict__ zp = job.zp;
@@ -380,7 +284,7 @@ __global__ void __launch_bounds__(kDecompressBlock) pq_decompress_vec_kernel(con
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < nvec) {
         pv[k] = ldg<int32_t, W>(packed + (size_t)v * W);
-        const uint32_t si = pq_scale_index<FLAT>(v, job);
+        const uint32_t si = chain_scale_index<FLAT>(v, job);
         sraw[k] = scale[si];
         if constexpr (HAS_ZP) zraw[k] = zp[si];
       }
@@ -409,7 +313,7 @@ struct VecKey {
 };
 
 template <typename XT, typename ST, bool FLAT>
-static void launch_compress_flat(const VecKey& k, const PqJobTable& t, unsigned grid,
+static void launch_compress_flat(const VecKey& k, const ChainTable& t, unsigned grid,
                                  hipStream_t st) {
   constexpr int B = kCompressBlock;
   if (k.bits == 4) {
@@ -422,13 +326,13 @@ static void launch_compress_flat(const VecKey& k, const PqJobTable& t, unsigned 
 }
 
 template <typename XT, typename ST>
-static void launch_compress_table(const VecKey& k, const PqJobTable& t, unsigned grid,
+static void launch_compress_table(const VecKey& k, const ChainTable& t, unsigned grid,
                                   hipStream_t st) {
   if (k.flat) launch_compress_flat<XT, ST, true>(k, t, grid, st);
   else launch_compress_flat<XT, ST, false>(k, t, grid, st);
 }
 
-static void launch_compress_vec(const VecKey& k, const PqJobTable& t, unsigned grid,
+static void launch_compress_vec(const VecKey& k, const ChainTable& t, unsigned grid,
                                 hipStream_t st) {
 #define CTMI_DISPATCH_S(XT)                                                              \
   if (k.scale_dtype == CTMI_BF16) launch_compress_table<XT, BF16>(k, t, grid, st);       \
@@ -441,7 +345,7 @@ static void launch_compress_vec(const VecKey& k, const PqJobTable& t, unsigned g
 }
 
 template <typename ST, bool FLAT>
-static void launch_decompress_flat(const VecKey& k, const PqJobTable& t, unsigned grid,
+static void launch_decompress_flat(const VecKey& k, const ChainTable& t, unsigned grid,
                                    hipStream_t st) {
   constexpr int B = kDecompressBlock;
   if (k.bits == 4) {
@@ -454,13 +358,13 @@ static void launch_decompress_flat(const VecKey& k, const PqJobTable& t, unsigne
 }
 
 template <typename ST>
-static void launch_decompress_table(const VecKey& k, const PqJobTable& t, unsigned grid,
+static void launch_decompress_table(const VecKey& k, const ChainTable& t, unsigned grid,
                                     hipStream_t st) {
   if (k.flat) launch_decompress_flat<ST, true>(k, t, grid, st);
   else launch_decompress_flat<ST, false>(k, t, grid, st);
 }
 
-static void launch_decompress_vec(const VecKey& k, const PqJobTable& t, unsigned grid,
+static void launch_decompress_vec(const VecKey& k, const ChainTable& t, unsigned grid,
                                   hipStream_t st) {
   if (k.scale_dtype == CTMI_BF16) launch_decompress_table<BF16>(k, t, grid, st);
   else if (k.scale_dtype == CTMI_F16) launch_decompress_table<F16>(k, t, grid, st);
@@ -668,7 +572,7 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
     }
     // gather every remaining job with the same key, kMaxJobs at a time
     const VecKey key = plans[i].key;
-    PqJobTable t;
+    ChainTable t;
     std::memset(&t, 0, sizeof(t));
     uint64_t chunks = 0;
     auto reset = [&]() {
@@ -690,7 +594,7 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
       if (done[j] || plans[j].empty || !plans[j].vec || !(plans[j].key == key)) continue;
       const uint64_t c = (uint64_t)cdiv(plans[j].job.g.nvec, per_block);
       if (t.n == kMaxJobs || chunks + c >= (1ull << 31)) flush();
-      t.job[t.n] = make_pq_job(plans[j].job);
+      t.job[t.n] = make_chain_job(plans[j].job);
       t.nvec[t.n] = plans[j].job.g.nvec;
       chunks += c;
       t.chunk_end[t.n] = (uint32_t)chunks;

@@ -16,6 +16,7 @@
 #include "quant_core.h"
 #include "quant_fast.h"
 #include "vec_geom.h"
+#include "job_table.h"
 
 namespace ctmi {
 
@@ -45,21 +46,24 @@ __device__ __forceinline__ float fp8_hw_decode(uint32_t word, int byte) {
 
 // FT: float dtype tag of x / scale / float output.  IN / OUT: element kind of the
 // input and output tensors.  QK: 0 = integer grid, 1 = fp8 grid.
-template <typename FT, int IN, int OUT, int QK, bool HAS_ZP>
-__global__ void __launch_bounds__(kQdqBlock)
-qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict__ scale,
-               const uint8_t* __restrict__ zp, void* __restrict__ yout, VecGeom g, float qmin,
-               float qmax) {
+// One chunk (kQdqBlock * kQdqUnroll items) of one tensor; `index_of` maps an item
+// to its scale.
+template <typename FT, int IN, int OUT, int QK, bool HAS_ZP, typename IndexOf>
+__device__ __forceinline__ void qdq_chunk(const void* __restrict__ xin,
+                                          const typename FT::raw* __restrict__ scale,
+                                          const uint8_t* __restrict__ zp, void* __restrict__ yout,
+                                          uint32_t nvec, uint32_t chunk, IndexOf index_of,
+                                          float qmin, float qmax) {
   constexpr int CT = FT::id;
   constexpr int B = kQdqBlock, U = kQdqUnroll;
   constexpr bool DO_Q = IN == kKindFloat;
   constexpr bool DO_DQ = OUT == kKindFloat;
   using FR = typename FT::raw;
-  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  const uint32_t v0 = chunk * (B * U) + threadIdx.x;
   // A chunk wholly inside the tensor (all but the last) runs without per-lane
   // bounds checks: straight-line code, every load of the workgroup issued before
   // the first loaded value is looked at.
-  const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
+  const bool full = (chunk + 1) * (uint32_t)(B * U) <= nvec;
   auto body = [&](auto guard) {
     constexpr bool GUARD = decltype(guard)::value;
     Vec<FR, 8> xf[U];
@@ -68,11 +72,11 @@ qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict_
     uint8_t zraw[U];
     uint32_t si[U];
 #pragma unroll
-    for (int k = 0; k < U; ++k) si[k] = scale_index(min(v0 + k * B, g.nvec - 1), g);
+    for (int k = 0; k < U; ++k) si[k] = index_of(min(v0 + k * B, nvec - 1));
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
-      if (!GUARD || v < g.nvec) {
+      if (!GUARD || v < nvec) {
         if constexpr (DO_Q) xf[k] = ldg_nt<FR, 8>((const FR*)xin + (size_t)v * 8);
         else xc[k] = ldg_nt<uint8_t, 8>((const uint8_t*)xin + (size_t)v * 8);
         sraw[k] = scale[si[k]];
@@ -82,7 +86,7 @@ qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict_
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
-      if (GUARD && v >= g.nvec) continue;
+      if (GUARD && v >= nvec) continue;
       const float s = FT::to_f32(sraw[k]);
       float z = 0.0f;
       if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw[k] : f8e4m3_to_f32(zraw[k]);
@@ -156,6 +160,26 @@ qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict_
   else body(std::true_type{});
 }
 
+template <typename FT, int IN, int OUT, int QK, bool HAS_ZP>
+__global__ void __launch_bounds__(kQdqBlock)
+qdq_vec_kernel(const void* __restrict__ xin, const typename FT::raw* __restrict__ scale,
+               const uint8_t* __restrict__ zp, void* __restrict__ yout, VecGeom g, float qmin,
+               float qmax) {
+  qdq_chunk<FT, IN, OUT, QK, HAS_ZP>(xin, scale, zp, yout, g.nvec, blockIdx.x,
+                                     [&](uint32_t v) { return scale_index(v, g); }, qmin, qmax);
+}
+
+// several tensors per launch (job_table.h); the table must be the only argument
+template <typename FT, int IN, int OUT, int QK, bool HAS_ZP, bool FLAT>
+__global__ void __launch_bounds__(kQdqBlock) qdq_vec_many_kernel(const ChainTable t) {
+  uint32_t chunk, nvec;
+  const ChainJob job = find_job(t, blockIdx.x, &chunk, &nvec);
+  qdq_chunk<FT, IN, OUT, QK, HAS_ZP>(job.src, (const typename FT::raw*)job.scale,
+                                     (const uint8_t*)job.zp, job.dst, nvec, chunk,
+                                     [&](uint32_t v) { return chain_scale_index<FLAT>(v, job); },
+                                     t.qmin, t.qmax);
+}
+
 template <typename FT, int IN, int OUT, int QK>
 static void launch_qdq(bool has_zp, const void* x, const void* scale, const void* zp, void* out,
                        const VecGeom& g, float qmin, float qmax, hipStream_t st) {
@@ -187,11 +211,19 @@ static void dispatch_mode(int in_kind, int out_kind, int qk, bool has_zp, const 
 #undef CTMI_QDQ
 }
 
-// Tries the vectorised path; returns false (nothing launched) if the problem
-// does not fit it.  All arguments have been validated by the caller.
-bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
-                        int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq,
-                        hipStream_t st) {
+// Which instance of the vectorised kernels takes this problem, if any.
+struct QdqKey {
+  int sd, in_kind, out_kind, qk, has_zp, flat;
+  bool operator==(const QdqKey& o) const {
+    return sd == o.sd && in_kind == o.in_kind && out_kind == o.out_kind && qk == o.qk &&
+           has_zp == o.has_zp && flat == o.flat;
+  }
+};
+
+// All arguments have been validated by the caller.  false = does not fit.
+bool qdq_classify(const void* x, int x_dtype, const void* out, int out_dtype, int64_t rows,
+                  int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq, QdqKey* key,
+                  VecGeom* g, float* qmin, float* qmax) {
   const int sd = qp->scale_dtype;
   if (sd != CTMI_BF16 && sd != CTMI_F16 && sd != CTMI_F32) return false;
   int in_kind, out_kind, qk;
@@ -221,21 +253,66 @@ bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, in
     out_kind = kKindFloat;
   }
   if (qp->zero_point && qp->zp_dtype != code_dtype) return false;
-  VecGeom g;
-  if (!vec_geometry(qp, rows, cols, &g)) return false;
-  if (cdiv(g.nvec, kQdqBlock * kQdqUnroll) >= (1ll << 31)) return false;
+  if (!vec_geometry(qp, rows, cols, g)) return false;
+  if (cdiv(g->nvec, kQdqBlock * kQdqUnroll) >= (1ll << 30)) return false;
   const int in_bytes = 8 * dtype_size(x_dtype), out_bytes = 8 * dtype_size(out_dtype);
   if ((uintptr_t)x % in_bytes || (uintptr_t)out % out_bytes) return false;
-  float qmin, qmax;
-  if (quant_range(qp->qtype, qp->num_bits, &qmin, &qmax)) return false;
-  const bool has_zp = qp->zero_point != nullptr;
-  if (sd == CTMI_BF16)
-    dispatch_mode<BF16>(in_kind, out_kind, qk, has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
-  else if (sd == CTMI_F16)
-    dispatch_mode<F16>(in_kind, out_kind, qk, has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
-  else
-    dispatch_mode<F32>(in_kind, out_kind, qk, has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
+  if (quant_range(qp->qtype, qp->num_bits, qmin, qmax)) return false;
+  *key = QdqKey{sd, in_kind, out_kind, qk, qp->zero_point != nullptr, g->mode == 0};
   return true;
 }
+
+// Tries the vectorised path; returns false (nothing launched) if the problem
+// does not fit it.
+bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
+                        int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq,
+                        hipStream_t st) {
+  QdqKey k;
+  VecGeom g;
+  float qmin, qmax;
+  if (!qdq_classify(x, x_dtype, out, out_dtype, rows, cols, qp, do_q, do_dq, &k, &g, &qmin, &qmax))
+    return false;
+  if (k.sd == CTMI_BF16)
+    dispatch_mode<BF16>(k.in_kind, k.out_kind, k.qk, k.has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
+  else if (k.sd == CTMI_F16)
+    dispatch_mode<F16>(k.in_kind, k.out_kind, k.qk, k.has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
+  else
+    dispatch_mode<F32>(k.in_kind, k.out_kind, k.qk, k.has_zp, x, qp->scale, qp->zero_point, out, g, qmin, qmax, st);
+  return true;
+}
+
+// ---- chained launches
+template <typename FT, int IN, int OUT, int QK>
+static void launch_many2(const QdqKey& k, const ChainTable& t, unsigned grid, hipStream_t st) {
+#define CTMI_QM(ZP, FLAT) \
+  hipLaunchKernelGGL((qdq_vec_many_kernel<FT, IN, OUT, QK, ZP, FLAT>), grid, kQdqBlock, 0, st, t)
+  if (k.has_zp) { if (k.flat) CTMI_QM(true, true); else CTMI_QM(true, false); }
+  else { if (k.flat) CTMI_QM(false, true); else CTMI_QM(false, false); }
+#undef CTMI_QM
+}
+
+template <typename FT>
+static void launch_many1(const QdqKey& k, const ChainTable& t, unsigned grid, hipStream_t st) {
+#define CTMI_QDQ(IN, OUT, QK)                                        \
+  if (k.in_kind == IN && k.out_kind == OUT && k.qk == QK) {          \
+    launch_many2<FT, IN, OUT, QK>(k, t, grid, st);                   \
+    return;                                                          \
+  }
+  CTMI_QDQ(kKindFloat, kKindI8, 0)
+  CTMI_QDQ(kKindFloat, kKindF8, 1)
+  CTMI_QDQ(kKindI8, kKindFloat, 0)
+  CTMI_QDQ(kKindF8, kKindFloat, 1)
+  CTMI_QDQ(kKindFloat, kKindFloat, 0)
+  CTMI_QDQ(kKindFloat, kKindFloat, 1)
+#undef CTMI_QDQ
+}
+
+void qdq_launch_chain(const QdqKey& k, const ChainTable& t, unsigned grid, hipStream_t st) {
+  if (k.sd == CTMI_BF16) launch_many1<BF16>(k, t, grid, st);
+  else if (k.sd == CTMI_F16) launch_many1<F16>(k, t, grid, st);
+  else launch_many1<F32>(k, t, grid, st);
+}
+
+int qdq_chunk_items() { return kQdqBlock * kQdqUnroll; }
 
 }  // namespace ctmi

@@ -13,6 +13,11 @@
 #include "ctmi_device.h"
 #include "ctmi_host.h"
 #include "quant_core.h"
+#include "vec_geom.h"
+#include "job_table.h"
+
+#include <cstring>
+#include <vector>
 
 namespace ctmi {
 
@@ -57,6 +62,18 @@ __global__ void __launch_bounds__(256) qdq_generic_kernel(QdqArgs a) {
   }
 }
 
+struct QdqKey {
+  int sd, in_kind, out_kind, qk, has_zp, flat;
+  bool operator==(const QdqKey& o) const {
+    return sd == o.sd && in_kind == o.in_kind && out_kind == o.out_kind && qk == o.qk &&
+           has_zp == o.has_zp && flat == o.flat;
+  }
+};
+bool qdq_classify(const void* x, int x_dtype, const void* out, int out_dtype, int64_t rows,
+                  int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq, QdqKey* key,
+                  VecGeom* g, float* qmin, float* qmax);
+void qdq_launch_chain(const QdqKey& k, const ChainTable& t, unsigned grid, hipStream_t st);
+int qdq_chunk_items();
 bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
                         int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq, hipStream_t st);
 bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
@@ -78,9 +95,9 @@ static int fill_cfg(const ctmi_qparams* qp, int x_dtype, QuantCfg* q) {
 
 using namespace ctmi;
 
-extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_dtype, int64_t rows,
-                        int64_t cols, const ctmi_qparams* qp, int32_t do_quantize,
-                        int32_t do_dequantize, void* stream) {
+static int qdq_validate(const void* x, int32_t x_dtype, const void* out, int32_t out_dtype,
+                        int64_t rows, int64_t cols, const ctmi_qparams* qp, int32_t do_quantize,
+                        int32_t do_dequantize) {
   CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
   CTMI_REQUIRE(do_quantize || do_dequantize, CTMI_ERR_VALUE, "nothing to do");
   CTMI_REQUIRE(dtype_size(x_dtype) > 0 && x_dtype != CTMI_I64, CTMI_ERR_UNSUPPORTED,
@@ -95,14 +112,14 @@ extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_d
   if (rc) return rc;
   if (rows == 0 || cols == 0) return CTMI_OK;
   CTMI_REQUIRE(x != nullptr && out != nullptr, CTMI_ERR_VALUE, "NULL tensor pointer");
+  QuantCfg q;
+  return fill_cfg(qp, x_dtype, &q);
+}
 
-  if (qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize,
-                         (hipStream_t)stream))
-    return check_launch("ctmi_qdq");
-  if (do_quantize && do_dequantize &&
-      nvfp4_qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, (hipStream_t)stream))
-    return check_launch("ctmi_qdq");
-
+// the any-layout kernel, for a validated problem
+static void qdq_enqueue_generic(const void* x, int32_t x_dtype, void* out, int32_t out_dtype,
+                                int64_t rows, int64_t cols, const ctmi_qparams* qp,
+                                int32_t do_quantize, int32_t do_dequantize, hipStream_t st) {
   QdqArgs a;
   a.x = x;
   a.out = out;
@@ -122,11 +139,102 @@ extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_d
   a.zp_dtype = qp->zp_dtype;
   a.do_q = do_quantize;
   a.do_dq = do_dequantize;
-  rc = fill_cfg(qp, x_dtype, &a.q);
-  if (rc) return rc;
-
+  fill_cfg(qp, x_dtype, &a.q);
   dim3 block(256);
   dim3 grid((unsigned)cdiv(cols, 256), (unsigned)(rows < 32768 ? rows : 32768));
-  hipLaunchKernelGGL(qdq_generic_kernel, grid, block, 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(qdq_generic_kernel, grid, block, 0, st, a);
+}
+
+extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_dtype, int64_t rows,
+                        int64_t cols, const ctmi_qparams* qp, int32_t do_quantize,
+                        int32_t do_dequantize, void* stream) {
+  int rc = qdq_validate(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize);
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  hipStream_t st = (hipStream_t)stream;
+  if (qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize, st))
+    return check_launch("ctmi_qdq");
+  if (do_quantize && do_dequantize &&
+      nvfp4_qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, st))
+    return check_launch("ctmi_qdq");
+  qdq_enqueue_generic(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize, st);
   return check_launch("ctmi_qdq");
+}
+
+// Every job is validated before anything is enqueued; jobs the vectorised
+// kernels take are chained, kMaxJobs per launch and kernel instance, the others
+// run as ctmi_qdq would run them.
+extern "C" int ctmi_qdq_many(const ctmi_qdq_job* jobs, int64_t n, int32_t do_quantize,
+                             int32_t do_dequantize, void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_qdq_job& j = jobs[i];
+    int rc = qdq_validate(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, do_quantize,
+                          do_dequantize);
+    if (rc) return rc;
+  }
+  hipStream_t st = (hipStream_t)stream;
+  struct Plan {
+    bool vec;
+    QdqKey key;
+    VecJob job;
+    float qmin, qmax;
+  };
+  std::vector<Plan> plans((size_t)n);
+  std::vector<char> done((size_t)n, 0);
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_qdq_job& j = jobs[i];
+    Plan& p = plans[i];
+    if (j.rows == 0 || j.cols == 0) { done[i] = 1; continue; }
+    p.vec = qdq_classify(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, do_quantize,
+                         do_dequantize, &p.key, &p.job.g, &p.qmin, &p.qmax);
+    if (p.vec) {
+      p.job.src = j.x;
+      p.job.dst = j.out;
+      p.job.scale = j.qp.scale;
+      p.job.zp = (const int8_t*)j.qp.zero_point;
+      continue;
+    }
+    if (!(do_quantize && do_dequantize &&
+          nvfp4_qdq_try_vectorised(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, st)))
+      qdq_enqueue_generic(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, do_quantize,
+                          do_dequantize, st);
+    done[i] = 1;
+  }
+  const int per_chunk = qdq_chunk_items();
+  for (int64_t i = 0; i < n; ++i) {
+    if (done[i]) continue;
+    const QdqKey key = plans[i].key;
+    ChainTable t;
+    std::memset(&t, 0, sizeof(t));
+    uint64_t chunks = 0;
+    auto reset = [&]() {
+      t.n = 0;
+      chunks = 0;
+      for (int k = 0; k < kMaxJobs; ++k) t.chunk_end[k] = 0xFFFFFFFFu;
+    };
+    reset();
+    t.qmin = plans[i].qmin;
+    t.qmax = plans[i].qmax;
+    auto flush = [&]() {
+      if (t.n == 0) return;
+      qdq_launch_chain(key, t, (unsigned)chunks, st);
+      reset();
+    };
+    for (int64_t j = i; j < n; ++j) {
+      // quantization range is part of the key: it follows from qk only for fp8, not for ints
+      if (done[j] || !(plans[j].key == key) || plans[j].qmin != t.qmin || plans[j].qmax != t.qmax)
+        continue;
+      const uint64_t c = (uint64_t)cdiv(plans[j].job.g.nvec, per_chunk);
+      if (t.n == kMaxJobs || chunks + c >= (1ull << 31)) flush();
+      t.job[t.n] = make_chain_job(plans[j].job);
+      t.nvec[t.n] = plans[j].job.g.nvec;
+      chunks += c;
+      t.chunk_end[t.n] = (uint32_t)chunks;
+      ++t.n;
+      done[j] = 1;
+    }
+    flush();
+  }
+  return check_launch("ctmi_qdq_many");
 }

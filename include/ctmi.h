@@ -89,6 +89,24 @@ int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_dtype, int64
              int64_t cols, const ctmi_qparams* qp, int32_t do_quantize, int32_t do_dequantize,
              void* stream);
 
+/* One tensor of a state dict for ctmi_qdq_many. */
+typedef struct ctmi_qdq_job {
+  const void* x;
+  void* out;
+  int64_t rows, cols;
+  int32_t x_dtype, out_dtype;
+  ctmi_qparams qp;
+} ctmi_qdq_job;
+
+/* A27 for the naive / int / float-quantized formats: the per-weight loop of
+ * BaseQuantizationCompressor.compress / decompress_from_state_dict
+ * (compressors/quantized_compressors/base.py:91-125, 213-230) around quantize /
+ * dequantize, n tensors from one call.  Every job is validated before anything
+ * is enqueued; tensors that share a kernel instance are chained into common
+ * launches.  Same results as n calls of ctmi_qdq. */
+int ctmi_qdq_many(const ctmi_qdq_job* jobs, int64_t n, int32_t do_quantize, int32_t do_dequantize,
+                  void* stream);
+
 /* A9.  pack_to_int32 (compressors/quantized_compressors/pack_quantized.py:186-246).
  * in: int8 [rows, cols]; out: int32 [rows, ceil(cols/pf)] (packed_dim=1) or
  * int32 [ceil(rows/pf), cols] (packed_dim=0), pf = 32/num_bits. */

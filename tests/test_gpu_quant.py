@@ -290,3 +290,38 @@ def test_large_fp8_channel_and_token(gpu):
     os_, oz_ = oq.compute_dynamic_scales_and_zp(x[:, toks], toargs)
     assert_bit_equal(s[:, toks.to(gpu)], os_, "token scales")
     assert_bit_equal(y[:, toks.to(gpu)], oq.fake_quantize(x[:, toks], os_, oz_, toargs), "token qdq")
+
+
+def test_quantized_weight_batch_matches_single_calls(gpu):
+    """ctmi_qdq_many (chained launches) == one ctmi_qdq per tensor, for a mix of kernel
+    instances: fp8 and int8 codes, with and without zero points, channel / group / tensor
+    scales, a shape the vectorised kernels do not take, and more than 8 tensors of a kind."""
+    from compressed_tensors_amd.compressors import QuantizedWeightBatch
+    from compressed_tensors_amd.quantization import (QuantizationArgs, dequantize,
+                                                     observe_weight_qparams, quantize)
+
+    announce("qdq_many")
+    g = torch.Generator().manual_seed(11)
+    specs = [dict(num_bits=8, type="float", symmetric=True, strategy="channel")] * 11 + [
+        dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=32),
+        dict(num_bits=8, type="int", symmetric=True, strategy="tensor"),
+        dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128),
+        dict(num_bits=8, type="int", symmetric=False, strategy="channel"),
+    ]
+    shapes = [(64, 256), (8, 4096), (33, 128), (1, 8), (128, 1024), (5, 72), (16, 16), (256, 256),
+              (3, 4104), (40, 640), (7, 56), (48, 96), (20, 200), (12, 384), (9, 30)]
+    entries = []
+    for spec, shape in zip(specs, shapes):
+        args = QuantizationArgs(**spec)
+        w = (torch.randn(shape, generator=g) * 0.05).bfloat16().to(gpu)
+        scale, zp = observe_weight_qparams(w, args)
+        entries.append(dict(weight=w, scale=scale, zero_point=zp, quantization_args=args))
+    batch = QuantizedWeightBatch(entries)
+    codes = batch.compress()
+    dense = batch.decompress()
+    for e, c, d in zip(entries, codes, dense):
+        args = e["quantization_args"]
+        want = quantize(e["weight"], e["scale"], e["zero_point"], args, dtype=args.pytorch_dtype())
+        assert c.dtype == want.dtype and torch.equal(c.view(torch.int8), want.view(torch.int8))
+        back = dequantize(want, e["scale"], None if args.symmetric else e["zero_point"])
+        assert d.dtype == back.dtype and torch.equal(d.view(torch.int16), back.view(torch.int16))
