@@ -343,9 +343,12 @@ def fake_quantize(
 def forward_quantize(
     module: torch.nn.Module, value: torch.Tensor, base_name: str, args: QuantizationArgs
 ) -> torch.Tensor:
-    """reference: forward.py:414-451 (dynamic scales come from the fused
-    min/max + qparams kernels)."""
-    from compressed_tensors_amd.quantization.helpers import compute_dynamic_scales_and_zp
+    """reference: forward.py:414-451.  Dynamic schemes take one pass over `value`
+    (scales and fake-quantization in one kernel) where a fused kernel exists, else
+    the fused min/max + qparams kernel followed by fake_quantize."""
+    from compressed_tensors_amd.quantization.helpers import (
+        compute_dynamic_scales_and_zp, dynamic_fake_quantize,
+    )
 
     status = getattr(module, "quantization_status", None)
     if status is not None and str(getattr(status, "value", status)) == "compressed":
@@ -358,6 +361,10 @@ def forward_quantize(
     global_scale = getattr(module, f"{base_name}_global_scale", None)
 
     if args.dynamic in (True, DynamicType.LOCAL.value):
+        if g_idx is None:
+            fused = dynamic_fake_quantize(value, args, global_scale)
+            if fused is not None:
+                return fused
         scale, zero_point = compute_dynamic_scales_and_zp(
             value=value, args=args, module=module, global_scale=global_scale
         )

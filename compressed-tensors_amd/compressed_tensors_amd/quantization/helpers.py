@@ -28,6 +28,7 @@ __all__ = [
     "calculate_range",
     "calculate_qparams",
     "compute_dynamic_scales_and_zp",
+    "dynamic_fake_quantize",
     "generate_gparam",
     "observe_weight_qparams",
     "minmax",
@@ -168,6 +169,68 @@ def _observe_rows(
         )
     )
     return scales, zps
+
+
+def dynamic_fake_quantize(
+    value: torch.Tensor,
+    args: QuantizationArgs,
+    global_scale: Optional[torch.Tensor] = None,
+    return_qparams: bool = False,
+):
+    """compute_dynamic_scales_and_zp (helpers.py:149-205) followed by fake_quantize
+    (forward.py:150-189) in one pass over `value` (ctmi_dynamic_qdq).  Returns None
+    when the layout has no fused kernel; the caller then makes the two calls."""
+    _lib.require_gpu(value)
+    if value.dtype not in _FLOATS or value.numel() == 0:
+        return None
+    strategy = args.strategy
+    if strategy == QuantizationStrategy.TOKEN.value:
+        if value.ndim <= 2:
+            return None  # one scale for the whole tensor: two passes by nature
+        rows = value.shape[0] * value.shape[1]
+        cols = value.numel() // rows
+        blk_cols = cols
+        out_shape = (value.shape[0], value.shape[1]) + (1,) * (value.ndim - 2)
+    elif strategy in (QuantizationStrategy.TENSOR_GROUP.value, QuantizationStrategy.GROUP.value):
+        cols = value.shape[-1]
+        blk_cols = args.group_size
+        if value.ndim < 1 or cols % blk_cols:
+            return None
+        rows = value.numel() // cols
+        out_shape = tuple(value.shape[:-1]) + (cols // blk_cols,)
+    else:
+        return None
+    fp4 = is_fp4(args)
+    if fp4 and not args.symmetric:
+        return None
+    if (global_scale is not None) != fp4:
+        return None  # a global scale that calculate_qparams ignores, or fp4 without one
+    lib = _lib.load()
+    if not lib.ctmi_dynamic_qdq_supported(_lib.dtype_code(value.dtype), rows, cols, blk_cols,
+                                          _qtype(args), args.num_bits, int(fp4)):
+        return None
+    v = value.contiguous()
+    if v.data_ptr() % (8 * v.element_size()):
+        return None  # a view that starts in the middle of a vector
+    keep = []
+    gs_ptr = _gscale_ptr(global_scale, keep)
+    scale_dtype = _scale_dtype(args, v.dtype, fp4)
+    zp_dtype = _zp_dtype(args)
+    out = torch.empty_like(v)
+    scales = zps = None
+    if return_qparams:
+        scales = torch.empty(out_shape, dtype=scale_dtype, device=v.device)
+        zps = torch.empty(out_shape, dtype=zp_dtype, device=v.device)
+    _lib.check(
+        lib.ctmi_dynamic_qdq(
+            v.data_ptr(), _lib.dtype_code(v.dtype), out.data_ptr(), rows, cols, blk_cols,
+            _qtype(args), args.num_bits, int(args.symmetric), gs_ptr,
+            scales.data_ptr() if return_qparams else None, _lib.dtype_code(scale_dtype),
+            zps.data_ptr() if return_qparams else None, _lib.dtype_code(zp_dtype),
+            _lib.stream_of(v.device),
+        )
+    )
+    return (out, scales, zps) if return_qparams else out
 
 
 def compute_dynamic_scales_and_zp(

@@ -32,7 +32,11 @@ __device__ __forceinline__ uint16_t f32_to_bf16(float f) {
 __device__ __forceinline__ float f16_to_f32(uint16_t h) {
   return (float)__builtin_bit_cast(_Float16, h);
 }
+// The empty asm keeps the conversion an instruction of its own.  Left to itself the
+// compiler folds a preceding multiplication into it as fma_mix(a, b, +0), and the
+// +0 addend turns a product of -0 into +0.
 __device__ __forceinline__ uint16_t f32_to_f16(float f) {
+  asm("" : "+v"(f));
   return __builtin_bit_cast(uint16_t, (_Float16)f);
 }
 

@@ -1,0 +1,204 @@
+// Dynamic activation quantization in one pass: the scales come from the tensor
+// itself, which is then fake-quantized with them while still in registers.
+//
+//   forward_quantize, args.dynamic            quantization/lifecycle/forward.py:414-451
+//     compute_dynamic_scales_and_zp           quantization/utils/helpers.py:149-205
+//     calculate_qparams                       helpers.py:67-146
+//     fake_quantize                           forward.py:150-189
+//
+// The reference runs these one after the other (the tensor is read for the
+// min / max, read again and written by fake_quantize); the arithmetic here is the
+// same, step for step, on data that is read once: 4 bytes per bf16 element
+// instead of 6.
+#include <type_traits>
+
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "minmax.h"
+#include "qdq_core.h"
+#include "qparams.h"
+#include "quant_core.h"
+#include "quant_fast.h"
+
+namespace ctmi {
+
+int fill_qpcfg(QpCfg* c, int qtype, int num_bits, int symmetric, int mt, int mm_is_0d,
+               bool has_gscale, int scale_dtype, int zp_dtype);
+bool nvfp4_dynamic_try(const void* x, int x_dtype, void* out, int64_t rows, int64_t cols,
+                       int64_t blk_cols, const float* gscale, void* scale_out, void* zp_out,
+                       const QpCfg& c, hipStream_t st);
+
+struct DynOut {
+  void* scale;  // optional
+  void* zp;     // optional
+};
+
+// The zero point as fake_quantize reads it back from its storage dtype: fp8 rounds
+// it, an integer dtype has no -0 (rint of a small negative value gives one).
+__device__ __forceinline__ float stored_zero_point(float z, const QpCfg& c) {
+  return c.qtype == CTMI_QTYPE_INT ? z + 0.0f : round_to(z, c.zp_dtype);
+}
+
+// One wavefront per row-long segment (token / channel): up to 64 * U vectors of
+// 8 elements, all loaded before anything is looked at.
+template <typename FT, int QK, int U>
+__global__ void __launch_bounds__(256)
+dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __restrict__ out,
+                    DynOut o, int64_t n_segments, int items, QpCfg c) {
+  using FR = typename FT::raw;
+  const int lane = threadIdx.x & 63;
+  const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (s >= n_segments) return;
+  const FR* p = x + s * (int64_t)items * 8;
+  Vec<FR, 8> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int i = k * 64 + lane;
+    a[k] = ldg_nt<FR, 8>(p + (int64_t)(i < items ? i : items - 1) * 8);  // re-reads do not change min / max
+  }
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  bool unordered = false;
+#pragma unroll
+  for (int k = 0; k < U; ++k) vec_minmax<FT>(a[k], &lo, &hi, &unordered);
+  group_minmax(64, &lo, &hi);
+  if (group_any(64, unordered)) lo = hi = __builtin_nanf("");
+  float sv, zv;
+  qparams_value(lo, hi, 1.0f, c, &sv, &zv);
+  zv = stored_zero_point(zv, c);
+  if (lane == 0) {
+    if (o.scale) store_from_f32(o.scale, c.scale_dtype, s, sv);
+    if (o.zp) store_from_f32(o.zp, c.zp_dtype, s, zv);
+  }
+  FR* q = out + s * (int64_t)items * 8;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int i = k * 64 + lane;
+    Vec<FR, 8> of;
+    Vec<uint8_t, 8> oc;
+    qdq_vec8<FT, kKindFloat, kKindFloat, QK, true>(a[k], oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
+    if (i < items) stg_nt<FR, 8>(q + (int64_t)i * 8, of);
+  }
+}
+
+// Segments of L vectors, L a power of two <= 64 (group strategies): L neighbouring
+// lanes own a segment; memory is one run of vectors numbered like the segments.
+template <typename FT, int QK>
+__global__ void __launch_bounds__(256)
+dynamic_flat_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __restrict__ out,
+                    DynOut o, int64_t nvec, int L, QpCfg c) {
+  using FR = typename FT::raw;
+  constexpr int U = 2;
+  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  Vec<FR, 8> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    a[k] = ldg_nt<FR, 8>(x + (v < nvec ? v : nvec - 1) * 8);
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    bool unordered = false;
+    vec_minmax<FT>(a[k], &lo, &hi, &unordered);
+    group_minmax(L, &lo, &hi);
+    if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
+    float sv, zv;
+    qparams_value(lo, hi, 1.0f, c, &sv, &zv);
+    zv = stored_zero_point(zv, c);
+  zv = stored_zero_point(zv, c);
+    if (v < nvec && (threadIdx.x & (L - 1)) == 0) {
+      if (o.scale) store_from_f32(o.scale, c.scale_dtype, v / L, sv);
+      if (o.zp) store_from_f32(o.zp, c.zp_dtype, v / L, zv);
+    }
+    Vec<FR, 8> of;
+    Vec<uint8_t, 8> oc;
+    qdq_vec8<FT, kKindFloat, kKindFloat, QK, true>(a[k], oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
+    if (v < nvec) stg_nt<FR, 8>(out + v * 8, of);
+  }
+}
+
+template <typename FT, int QK>
+static bool launch_dynamic(const void* x, void* out, const DynOut& o, int64_t rows, int64_t cols,
+                           int64_t blk_cols, const QpCfg& c, hipStream_t st) {
+  using FR = typename FT::raw;
+  const int64_t seg = blk_cols < cols ? blk_cols : cols;
+  if (seg % 8 || cols % seg) return false;
+  const int64_t items = seg / 8, nvec = rows * cols / 8, n_segments = rows * (cols / seg);
+  if (items <= 64 && (items & (items - 1)) == 0) {
+    const int64_t blocks = cdiv(nvec, 256 * 2);
+    if (blocks >= (1ll << 31)) return false;
+    hipLaunchKernelGGL((dynamic_flat_kernel<FT, QK>), (unsigned)blocks, 256, 0, st, (const FR*)x,
+                       (FR*)out, o, nvec, (int)items, c);
+    return true;
+  }
+  const int64_t blocks = cdiv(n_segments, 4);
+  if (blocks >= (1ll << 31)) return false;
+#define CTMI_DYN(UU)                                                                              \
+  hipLaunchKernelGGL((dynamic_rows_kernel<FT, QK, UU>), (unsigned)blocks, 256, 0, st, (const FR*)x, \
+                     (FR*)out, o, n_segments, (int)items, c)
+  if (items <= 64 * 2) CTMI_DYN(2);
+  else if (items <= 64 * 4) CTMI_DYN(4);
+  else if (items <= 64 * 8) CTMI_DYN(8);
+  else if (items <= 64 * 16) CTMI_DYN(16);
+  else return false;
+#undef CTMI_DYN
+  return true;
+}
+
+}  // namespace ctmi
+
+using namespace ctmi;
+
+extern "C" int ctmi_dynamic_qdq_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                          int64_t blk_cols, int32_t qtype, int32_t num_bits,
+                                          int32_t has_global_scale) {
+  if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16 && x_dtype != CTMI_F32) return 0;
+  if (rows < 1 || cols < 1 || blk_cols < 1) return 0;
+  const int64_t seg = blk_cols < cols ? blk_cols : cols;
+  if (seg % 8 || cols % seg) return 0;
+  const int64_t items = seg / 8;
+  if (qtype == CTMI_QTYPE_FLOAT && num_bits == 4)
+    return has_global_scale && items == 2;  // nvfp4: groups of 16
+  if (has_global_scale) return 0;
+  if (!((qtype == CTMI_QTYPE_INT && num_bits <= 8) || (qtype == CTMI_QTYPE_FLOAT && num_bits == 8)))
+    return 0;
+  return items <= 1024;
+}
+
+extern "C" int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64_t rows,
+                                int64_t cols, int64_t blk_cols, int32_t qtype, int32_t num_bits,
+                                int32_t symmetric, const float* global_scale, void* scale_out,
+                                int32_t scale_dtype, void* zp_out, int32_t zp_dtype, void* stream) {
+  CTMI_REQUIRE(rows >= 1 && cols >= 1, CTMI_ERR_VALUE, "cannot observe an empty tensor");
+  CTMI_REQUIRE(blk_cols >= 1, CTMI_ERR_VALUE, "empty cell");
+  QpCfg c;
+  int rc = fill_qpcfg(&c, qtype, num_bits, symmetric, x_dtype, 0, global_scale != nullptr,
+                      scale_dtype, zp_dtype);
+  if (rc) return rc;
+  CTMI_REQUIRE(x && out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE(ctmi_dynamic_qdq_supported(x_dtype, rows, cols, blk_cols, qtype, num_bits,
+                                          global_scale != nullptr),
+               CTMI_ERR_UNSUPPORTED,
+               "no fused kernel for this layout: compute the scales and fake-quantize separately");
+  const int bytes = 8 * dtype_size(x_dtype);
+  CTMI_REQUIRE((uintptr_t)x % bytes == 0 && (uintptr_t)out % bytes == 0, CTMI_ERR_VALUE,
+               "tensors must be aligned to 8 elements");
+  hipStream_t st = (hipStream_t)stream;
+  const DynOut o{scale_out, zp_out};
+  bool ok;
+  if (qtype == CTMI_QTYPE_FLOAT && num_bits == 4) {
+    ok = nvfp4_dynamic_try(x, x_dtype, out, rows, cols, blk_cols, global_scale, scale_out, zp_out,
+                           c, st);
+  } else {
+    const int qk = qtype == CTMI_QTYPE_INT ? 0 : 1;
+#define CTMI_DYN_FT(FT)                                                                  \
+  (qk == 0 ? launch_dynamic<FT, 0>(x, out, o, rows, cols, blk_cols, c, st)              \
+           : launch_dynamic<FT, 1>(x, out, o, rows, cols, blk_cols, c, st))
+    ok = x_dtype == CTMI_BF16 ? CTMI_DYN_FT(BF16)
+                              : (x_dtype == CTMI_F16 ? CTMI_DYN_FT(F16) : CTMI_DYN_FT(F32));
+#undef CTMI_DYN_FT
+  }
+  CTMI_REQUIRE(ok, CTMI_ERR_UNSUPPORTED, "no fused kernel for this layout");
+  return check_launch("ctmi_dynamic_qdq");
+}

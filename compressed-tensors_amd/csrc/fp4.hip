@@ -10,6 +10,8 @@
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "minmax.h"
+#include "qparams.h"
 #include "quant_core.h"
 #include "quant_fast.h"
 #include "vec_geom.h"
@@ -393,6 +395,67 @@ bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dty
   if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
   else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
   else hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, sc, qp->global_scale, (float*)out, g);
+  return true;
+}
+
+// Dynamic nvfp4 activations (forward.py:414-451 with a tensor_group scheme): the
+// group scales come from the 16 elements themselves (helpers.py:149-205, :67-146),
+// which are then fake-quantized with them without leaving the registers.  Two
+// neighbouring lanes hold one group.
+template <typename XT>
+__global__ void __launch_bounds__(kFp4Block)
+nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __restrict__ gscale,
+                     typename XT::raw* __restrict__ out, uint8_t* __restrict__ scale_out,
+                     uint8_t* __restrict__ zp_out, uint32_t nvec, QpCfg c) {
+  constexpr int B = kFp4Block, U = 2;
+  const float gs = gscale[0];
+  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  Vec<typename XT::raw, 8> xv[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)(v < nvec ? v : nvec - 1) * 8);
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    bool unordered = false;
+    vec_minmax<XT>(xv[k], &lo, &hi, &unordered);
+    group_minmax(2, &lo, &hi);
+    if (group_any(2, unordered)) lo = hi = __builtin_nanf("");
+    float sv, zv;
+    qparams_value(lo, hi, gs, c, &sv, &zv);
+    if (v < nvec && (threadIdx.x & 1) == 0) {
+      if (scale_out) scale_out[v >> 1] = f32_to_f8e4m3(sv);
+      if (zp_out) zp_out[v >> 1] = 0;  // fp8 zero
+    }
+    const float s = sv / gs;
+    float t[8];
+    fp4_unpack8_hw(nvfp4_codes<XT, true>(xv[k], s, 0.0f), t);
+    Vec<typename XT::raw, 8> o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float xi = XT::to_f32(xv[k].v[i]);
+      o.v[i] = XT::from_f32(xi != xi ? xi : t[i] * s);
+    }
+    if (v < nvec) stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
+  }
+}
+
+bool nvfp4_dynamic_try(const void* x, int x_dtype, void* out, int64_t rows, int64_t cols,
+                       int64_t blk_cols, const float* gscale, void* scale_out, void* zp_out,
+                       const QpCfg& c, hipStream_t st) {
+  if (!gscale || blk_cols != 16 || cols % 16 || !c.fp4_global) return false;
+  const int64_t nvec = rows * cols / 8;
+  const int64_t grid = cdiv(nvec, kFp4Block * 2);
+  if (nvec >= (1ll << 32) || grid >= (1ll << 31)) return false;
+  auto* so = (uint8_t*)scale_out;
+  auto* zo = (uint8_t*)zp_out;
+  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_dynamic_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, (uint16_t*)out, so, zo, (uint32_t)nvec, c);
+  else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_dynamic_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, (uint16_t*)out, so, zo, (uint32_t)nvec, c);
+  else if (x_dtype == CTMI_F32) hipLaunchKernelGGL(nvfp4_dynamic_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, gscale, (float*)out, so, zo, (uint32_t)nvec, c);
+  else return false;
   return true;
 }
 

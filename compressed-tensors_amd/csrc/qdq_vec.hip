@@ -15,34 +15,13 @@
 #include "ctmi_host.h"
 #include "quant_core.h"
 #include "quant_fast.h"
+#include "qdq_core.h"
 #include "vec_geom.h"
 #include "job_table.h"
 
 namespace ctmi {
 
-constexpr int kKindFloat = 0, kKindI8 = 1, kKindF8 = 2;
 constexpr int kQdqBlock = 512, kQdqUnroll = 2;
-
-template <int CT>
-__device__ __forceinline__ void round2(float& a, float& b) {
-  if constexpr (CT == CTMI_BF16) {
-    const uint32_t p = pack_bf16x2(a, b);
-    a = bf16_lo(p);
-    b = bf16_hi(p);
-  } else if constexpr (CT == CTMI_F16) {
-    a = f16_to_f32(f32_to_f16(a));
-    b = f16_to_f32(f32_to_f16(b));
-  }
-}
-
-__device__ __forceinline__ float fp8_hw_decode(uint32_t word, int byte) {
-  switch (byte) {
-    case 0: return __builtin_amdgcn_cvt_f32_fp8((int)word, 0);
-    case 1: return __builtin_amdgcn_cvt_f32_fp8((int)word, 1);
-    case 2: return __builtin_amdgcn_cvt_f32_fp8((int)word, 2);
-    default: return __builtin_amdgcn_cvt_f32_fp8((int)word, 3);
-  }
-}
 
 // FT: float dtype tag of x / scale / float output.  IN / OUT: element kind of the
 // input and output tensors.  QK: 0 = integer grid, 1 = fp8 grid.
@@ -90,70 +69,11 @@ __device__ __forceinline__ void qdq_chunk(const void* __restrict__ xin,
       const float s = FT::to_f32(sraw[k]);
       float z = 0.0f;
       if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw[k] : f8e4m3_to_f32(zraw[k]);
-      float t[8];
-      uint32_t codes[2] = {0u, 0u};  // 8 one-byte codes
-      if constexpr (DO_Q) {
-        const bool fast = CT == CTMI_BF16 && wave_all(scale_is_tame(s));
-        const float r = __builtin_amdgcn_rcpf(s);
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float a = FT::to_f32(xf[k].v[2 * j]), b = FT::to_f32(xf[k].v[2 * j + 1]);
-          if (fast) { a *= r; b *= r; } else { a /= s; b /= s; }
-          round2<CT>(a, b);
-          if (HAS_ZP) { a += z; b += z; round2<CT>(a, b); }
-          a = clamp_nan(a, qmin, qmax);
-          b = clamp_nan(b, qmin, qmax);
-          if constexpr (QK == 0) {
-            a = rintf(a);
-            b = rintf(b);
-            if constexpr (OUT == kKindI8) {
-              codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(a)) << (16 * (j % 2));
-              codes[j / 2] |= ((uint32_t)(uint8_t)(int8_t)f32_to_int(b)) << (16 * (j % 2) + 8);
-            }
-          } else {
-            // two fp8 codes into the low or high half of the word
-            if (j % 2 == 0) codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], false);
-            else codes[j / 2] = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)codes[j / 2], true);
-            if constexpr (DO_DQ) {
-              a = fp8_hw_decode(codes[j / 2], 2 * (j % 2));
-              b = fp8_hw_decode(codes[j / 2], 2 * (j % 2) + 1);
-            }
-          }
-          t[2 * j] = a;
-          t[2 * j + 1] = b;
-        }
-      } else {
-        const Vec<uint32_t, 2> w = __builtin_bit_cast(Vec<uint32_t, 2>, xc[k]);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          if constexpr (IN == kKindI8) t[i] = (float)(int8_t)((w.v[i / 4] >> (8 * (i % 4))) & 0xffu);
-          else t[i] = fp8_hw_decode(w.v[i / 4], i % 4);
-        }
-      }
-      if constexpr (DO_DQ) {
-        Vec<FR, 8> o;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          float a = t[2 * j], b = t[2 * j + 1];
-          if (HAS_ZP) { a -= z; b -= z; round2<CT>(a, b); }
-          a *= s;
-          b *= s;
-          if constexpr (CT == CTMI_BF16) {
-            const uint32_t p = pack_bf16x2(a, b);
-            o.v[2 * j] = (uint16_t)(p & 0xffffu);
-            o.v[2 * j + 1] = (uint16_t)(p >> 16);
-          } else {
-            o.v[2 * j] = FT::from_f32(a);
-            o.v[2 * j + 1] = FT::from_f32(b);
-          }
-        }
-        stg_nt<FR, 8>((FR*)yout + (size_t)v * 8, o);
-      } else {
-        Vec<uint32_t, 2> w;
-        w.v[0] = codes[0];
-        w.v[1] = codes[1];
-        stg_nt<uint8_t, 8>((uint8_t*)yout + (size_t)v * 8, __builtin_bit_cast(Vec<uint8_t, 8>, w));
-      }
+      Vec<FR, 8> of;
+      Vec<uint8_t, 8> oc;
+      qdq_vec8<FT, IN, OUT, QK, HAS_ZP>(xf[k], xc[k], s, z, qmin, qmax, &of, &oc);
+      if constexpr (DO_DQ) stg_nt<FR, 8>((FR*)yout + (size_t)v * 8, of);
+      else stg_nt<uint8_t, 8>((uint8_t*)yout + (size_t)v * 8, oc);
     }
   };
   if (full) body(std::false_type{});

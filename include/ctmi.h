@@ -268,6 +268,26 @@ int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows, int64_t c
                          void* zero_point, int32_t zp_dtype, void* min_out, void* max_out,
                          void* stream);
 
+/* A26.  Dynamic activation quantization in one pass (forward_quantize with
+ * args.dynamic, quantization/lifecycle/forward.py:414-451): the scales of
+ * compute_dynamic_scales_and_zp (quantization/utils/helpers.py:149-205, via
+ * calculate_qparams :67-146) for cells of 1 x blk_cols elements of x[rows, cols]
+ * (token: blk_cols = cols; group / tensor_group: blk_cols = group_size), then
+ * fake_quantize (forward.py:150-189) of x with them: out has x's dtype and
+ * shape.  The tensor is read once.  scale_out / zp_out are optional
+ * [rows, cols / blk_cols] outputs with the dtypes ctmi_observe_qparams documents.
+ * global_scale: the fp32 scalar of a tensor_group (nvfp4) scheme, else NULL.
+ * ctmi_dynamic_qdq_supported() says whether a layout has a fused kernel (int
+ * <= 8 bits and fp8: cells of up to 8192 elements in multiples of 8; fp4 with
+ * a global scale: cells of 16); CTMI_ERR_UNSUPPORTED otherwise,
+ * and the caller runs ctmi_observe_qparams + ctmi_qdq. */
+int ctmi_dynamic_qdq_supported(int32_t x_dtype, int64_t rows, int64_t cols, int64_t blk_cols,
+                               int32_t qtype, int32_t num_bits, int32_t has_global_scale);
+int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64_t rows, int64_t cols,
+                     int64_t blk_cols, int32_t qtype, int32_t num_bits, int32_t symmetric,
+                     const float* global_scale, void* scale_out, int32_t scale_dtype,
+                     void* zp_out, int32_t zp_dtype, void* stream);
+
 /* A24 / A25.  Hadamard transform apply (transform/utils/matrix.py:65-171,
  * transform/factory/hadamard.py:104-121) for a matrix given in factored form
  *     W = diag(sign_in) * (Ma (x) Mb) * diag(sign_out),      n = a_dim * b_dim:

@@ -6,7 +6,7 @@ from pathlib import Path
 import pytest
 import torch
 
-from gpu_util import announce, assert_bit_equal
+from gpu_util import announce, assert_bit_equal, bits as bits_of
 from oracle import quant as oq
 
 pytestmark = pytest.mark.gpu
@@ -170,6 +170,120 @@ def test_dynamic_activation_quant(spec, shape, dtype, gpu):
     assert_bit_equal(zp, o_zp, "dynamic zp")
     out = fake_quantize(x.to(gpu), scale, zp, args, global_scale=gs)
     assert_bit_equal(out, oq.fake_quantize(x, o_scale, o_zp, oargs, global_scale=o_gs), "dynamic qdq")
+
+
+FUSED = [
+    # (args, shape, dtype, fused kernel expected)
+    (dict(num_bits=8, type="float", symmetric=True, strategy="token", dynamic=True), (2, 40, 256), torch.bfloat16, True),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="token", dynamic=True), (1, 19, 4096), torch.bfloat16, True),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="token", dynamic=True), (1, 5, 8192), torch.float16, True),
+    (dict(num_bits=8, type="float", symmetric=False, strategy="token", dynamic=True), (2, 7, 1024), torch.bfloat16, True),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="token", dynamic=True), (3, 33, 320), torch.bfloat16, True),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="token", dynamic=True), (3, 8, 64), torch.bfloat16, True),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="token", dynamic=True), (2, 9, 2, 760), torch.float32, True),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="token", dynamic=True), (1, 70, 5120), torch.float16, True),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="token", dynamic=True), (1, 33, 100), torch.float16, False),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="token", dynamic=True), (16, 64), torch.bfloat16, False),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=128, dynamic=True), (1, 16, 512), torch.bfloat16, True),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=32, dynamic=True), (45, 96), torch.bfloat16, True),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=8, dynamic=True), (3, 11, 72), torch.float32, True),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=24, dynamic=True), (7, 48), torch.bfloat16, True),
+    (dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16, dynamic="local"), (1, 32, 256), torch.bfloat16, True),
+    (dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16, dynamic="local"), (77, 48), torch.float16, True),
+    (dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16, dynamic="local"), (2, 3, 4112), torch.float32, True),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype,fusable", FUSED,
+                         ids=[f"{c[0]['type']}{c[0]['num_bits']}-{c[0]['strategy']}-{i}" for i, c in enumerate(FUSED)])
+def test_dynamic_quant_in_one_pass(spec, shape, dtype, fusable, gpu):
+    """scales + fake-quantization from one kernel: same bits as the oracle's
+    compute_dynamic_scales_and_zp followed by fake_quantize, special values included"""
+    from compressed_tensors_amd.quantization import forward_quantize
+    from compressed_tensors_amd.quantization.helpers import dynamic_fake_quantize
+
+    announce("dynamic one pass", spec, shape, dtype)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(shape, generator=g)
+    x[..., 3] *= 50
+    x = x.to(dtype)
+    flat = x.view(-1, x.shape[-1])
+    flat[0, :8] = 0.0                      # a stretch of zeros
+    flat[0, 1] = -0.0
+    flat[-1] = 0.0                         # a row of zeros: the scale floor
+    if flat.shape[0] > 2:
+        flat[1, 5] = float("nan")          # poisons its group / token
+        flat[2, 0] = float("inf")
+    gs = o_gs = None
+    module = torch.nn.Module()
+    if args.strategy == "tensor_group":
+        finite = torch.nan_to_num(x.float(), nan=0.0, posinf=1.0, neginf=-1.0)
+        mn, mx = torch.aminmax(finite)
+        o_gs = oq.generate_gparam(mn.reshape(1), mx.reshape(1))
+        gs = o_gs.to(gpu)
+        module.input_global_scale = gs
+    o_scale, o_zp = oq.compute_dynamic_scales_and_zp(x, oargs, global_scale=o_gs)
+    want = oq.fake_quantize(x, o_scale, o_zp, oargs, global_scale=o_gs)
+    if args.strategy == "tensor_group":
+        # the reference's fp4 cast of a NaN is platform dependent: a group that holds one
+        # comes out as NaN here, the oracle's choice for the other 15 values is not binding
+        bad = torch.isnan(o_scale.float()).repeat_interleave(16, dim=-1)
+        want = torch.where(bad, torch.full_like(want, float("nan")), want)
+
+    def canon(t):  # one NaN pattern: which payload a NaN result carries is not part of the contract
+        return torch.where(torch.isnan(t.float()).to(t.device), torch.full_like(t, float("nan")), t)
+
+    want, o_scale = canon(want), canon(o_scale)
+    res = dynamic_fake_quantize(x.to(gpu), args, gs, return_qparams=True)
+    assert (res is not None) == fusable
+    if res is not None:
+        out, scale, zp = res
+        assert_bit_equal(canon(scale), o_scale, "one-pass scale")
+        assert_bit_equal(zp, o_zp, "one-pass zp")
+        assert_bit_equal(canon(out), want, "one-pass qdq")
+        assert_bit_equal(canon(dynamic_fake_quantize(x.to(gpu), args, gs)), want, "one-pass qdq, no qparams")
+    routed = forward_quantize(module, x.to(gpu), "input", args)
+    if args.strategy == "tensor_group":
+        routed = torch.where(bad.to(gpu), torch.full_like(routed, float("nan")), routed)
+    assert_bit_equal(canon(routed), want, "forward_quantize")
+
+
+@pytest.mark.parametrize("spec", [
+    dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128),
+    dict(num_bits=8, type="int", symmetric=True, strategy="channel"),
+    dict(num_bits=8, type="float", symmetric=True, strategy="channel"),
+    dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16),
+], ids=["int4-group", "int8-channel", "fp8-channel", "nvfp4"])
+@pytest.mark.parametrize("with_zp", [False, True], ids=["nozp", "zp"])
+def test_float16_results_keep_the_sign_of_zero(spec, with_zp, gpu):
+    """small negative values quantize to -0 and must dequantize to -0 in float16 too
+    (a multiplication folded into the float16 conversion would give +0)"""
+    from compressed_tensors_amd.quantization import dequantize, fake_quantize, quantize
+
+    announce("f16 negative zero", spec, with_zp)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(77)
+    w = (torch.randn(64, 512, generator=g) * 0.02).to(torch.float16)
+    w[:, ::3] = -w[:, ::3].abs() * 1e-3            # far below half a quantization step
+    w[:, 5] = 0.3
+    gs = None
+    if args.strategy == "tensor_group":
+        gs = oq.generate_gparam(*[t.reshape(1) for t in torch.aminmax(w)])
+    scale, zp = oq.observe_weight(w, oargs, global_scale=gs)
+    if not with_zp:
+        zp = None
+    dev = lambda t: None if t is None else t.to(gpu)
+    want = oq.fake_quantize(w, scale, zp, oargs, global_scale=gs)
+    assert (bits_of(want) == -32768).sum() > 100  # the case is there: float16 -0 is 0x8000
+    got = fake_quantize(w.to(gpu), dev(scale), dev(zp), args, global_scale=dev(gs))
+    assert_bit_equal(got, want, "fake_quantize f16")
+    if args.num_bits == 8:
+        q = quantize(w.to(gpu), dev(scale), dev(zp), args, dtype=args.pytorch_dtype())
+        o_q = oq.quantize(w, scale, zp, oargs, dtype=args.pytorch_dtype())
+        assert_bit_equal(q, o_q, "quantize f16")
+        assert_bit_equal(dequantize(q, dev(scale), dev(zp), args=args),
+                         oq.dequantize(o_q, scale, zp, args=oargs), "dequantize f16")
 
 
 def test_attn_head_and_errors(gpu):
