@@ -179,6 +179,16 @@ def other_workload(torch, name, seed):
              zp.data_ptr(), code(zp.dtype), None, None, st)
         return lambda: _lib.check(lib.ctmi_observe_qparams(*a))
 
+    def dynamic(x, out, blk_cols, args, gscale=None):
+        keep.extend([x, out, gscale])
+        rows = x.numel() // x.shape[-1]
+        qtype = _lib.QTYPE_FLOAT if args.type == "float" else _lib.QTYPE_INT
+        fp4 = args.num_bits == 4 and args.type == "float"
+        a = (x.data_ptr(), code(x.dtype), out.data_ptr(), rows, x.shape[-1], blk_cols, qtype,
+             args.num_bits, int(args.symmetric), _lib.ptr(gscale), None,
+             code(FP8 if fp4 else x.dtype), None, code(FP8 if args.type == "float" else torch.int8), st)
+        return lambda: _lib.check(lib.ctmi_dynamic_qdq(*a))
+
     if name == "fp8-w8a8":
         args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
         from compressed_tensors_amd.compressors import QuantizedWeightBatch
@@ -193,7 +203,7 @@ def other_workload(torch, name, seed):
         batch = QuantizedWeightBatch(entries)   # one ctmi_qdq_many call per direction
         keep.append(batch)
         q_calls, d_calls = [batch.compress], [batch.decompress]
-        acts, a_obs, a_fq = [], [], []
+        acts, a_obs, a_fq, a_dyn = [], [], [], []
         targs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="token",
                                  dynamic=True)
         for _ in range(8):  # 8 x 67 MB: more than the last-level cache
@@ -204,12 +214,14 @@ def other_workload(torch, name, seed):
             out = torch.empty_like(x)
             a_obs.append(observe(x, 4096, targs, s, z))
             a_fq.append(qdq(x, out, build_qparams(x, s, z, targs), 1, 1))
+            a_dyn.append(dynamic(x, out, 4096, targs))
             acts.append(x)
         na = 8 * 8192 * 4096
         ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_kernel"),
                Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_kernel"),
                Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
-               Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel")]
+               Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel"),
+               Op("activations: scales + fake-quantize in one pass (8 x 8192x4096)", a_dyn, 4 * na, "dynamic_rows_kernel")]
         return "fp8 W8A8 quantize/dequantize GB/s, Llama-3-8B-shaped weights + per-token activations", ops, keep
 
     if name == "sparse":
@@ -289,7 +301,7 @@ def other_workload(torch, name, seed):
                     Op(f"nvfp4 decompress {r}x{c} (x5)", d_calls, nbytes, "nvfp4_decompress_vec_kernel")]
         aargs = QuantizationArgs(num_bits=4, type="float", symmetric=True, strategy="tensor_group",
                                  group_size=16, dynamic="local")
-        o_calls, f_calls = [], []
+        o_calls, f_calls, y_calls = [], [], []
         for _ in range(16):
             x = randn(4096, 4096)
             gs = generate_gparam(x.min().reshape(1), x.max().reshape(1))
@@ -297,9 +309,11 @@ def other_workload(torch, name, seed):
             out = torch.empty_like(x)
             o_calls.append(observe(x, 16, aargs, s, z, gs))
             f_calls.append(qdq(x, out, build_qparams(x, s, None, aargs, None, gs), 1, 1))
+            y_calls.append(dynamic(x, out, 16, aargs, gs))
         na = 16 * 4096 * 4096
         ops += [Op("nvfp4 activations: group-16 scales (16 x 4096x4096)", o_calls, 2 * na + na // 16, "observe_flat_kernel"),
-                Op("nvfp4 activations: fake-quantize (16 x 4096x4096)", f_calls, 4 * na + na // 16, "nvfp4_qdq_vec_kernel")]
+                Op("nvfp4 activations: fake-quantize (16 x 4096x4096)", f_calls, 4 * na + na // 16, "nvfp4_qdq_vec_kernel"),
+                Op("nvfp4 activations: scales + fake-quantize in one pass (16 x 4096x4096)", y_calls, 4 * na, "nvfp4_dynamic_kernel")]
         return "nvfp4-pack-quantized compress/decompress + activation fake-quantize GB/s", ops, keep
 
     if name == "hadamard":

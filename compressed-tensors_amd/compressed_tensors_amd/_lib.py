@@ -194,6 +194,14 @@ SIGNATURES = {
         [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
          c_void_p],
     ),
+    "ctmi_observe_pack_quantized_supported": (
+        c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32],
+    ),
+    "ctmi_observe_pack_quantized": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p,
+         c_void_p, c_void_p],
+    ),
     "ctmi_dynamic_qdq_supported": (
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32],
     ),

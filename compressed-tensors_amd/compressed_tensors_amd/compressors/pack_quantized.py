@@ -167,6 +167,63 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
             out["weight_zero_point"] = pack_to_int32(zero_point, args.num_bits, packed_dim=0)
         return out
 
+    def observe_and_compress_weight(
+        self, weight: Tensor, quantization_args: QuantizationArgs,
+        device: Optional[torch.device] = None,
+    ) -> Dict[str, Tensor]:
+        """One-shot (round-to-nearest) compression of a weight that has no scales yet:
+        the min-max observer (tests/mock_observer.py:38-113), calculate_qparams
+        (quantization/utils/helpers.py:67-146) and compress_weight
+        (pack_quantized.py:88-146) in one pass over the weight.  Returns
+        compress_weight's dict plus "weight_scale" (and the packed
+        "weight_zero_point" of an asymmetric scheme)."""
+        args = quantization_args
+        weight = to_gpu(weight)
+        if weight.ndim != 2:
+            raise ValueError(f"expected a 2-D weight, got shape {tuple(weight.shape)}")
+        rows, cols = weight.shape
+        if args.strategy == QuantizationStrategy.GROUP.value:
+            blk_cols = args.group_size
+        elif args.strategy == QuantizationStrategy.CHANNEL.value:
+            blk_cols = cols
+        else:
+            blk_cols = 0
+        lib = _lib.load()
+        w = weight.contiguous()
+        fused = (
+            blk_cols > 0 and args.type == "int" and can_quantize(weight, args)
+            and w.data_ptr() % (8 * w.element_size()) == 0
+            and lib.ctmi_observe_pack_quantized_supported(
+                _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits)
+        )
+        if not fused:
+            from compressed_tensors_amd.quantization.helpers import observe_weight_qparams
+
+            scale, zero_point = observe_weight_qparams(weight, args)
+            out = self.compress_weight(weight, scale, args, zero_point=zero_point, device=device)
+            out["weight_scale"] = scale if device is None else scale.to(device)
+            return out
+        n_cells = cols // min(blk_cols, cols)
+        packed = torch.empty((rows, cols * args.num_bits // 32), dtype=torch.int32, device=w.device)
+        scale = torch.empty((rows, n_cells), dtype=w.dtype, device=w.device)
+        zero_point = None
+        if not args.symmetric:
+            zero_point = torch.empty((rows, n_cells), dtype=torch.int8, device=w.device)
+        _lib.check(
+            lib.ctmi_observe_pack_quantized(
+                w.data_ptr(), _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits,
+                int(args.symmetric), packed.data_ptr(), scale.data_ptr(), _lib.ptr(zero_point),
+                _lib.stream_of(w.device),
+            )
+        )
+        out = {"weight_shape": torch.tensor(weight.shape), "weight_packed": packed,
+               "weight_scale": scale}
+        if zero_point is not None:
+            out["weight_zero_point"] = pack_to_int32(zero_point, args.num_bits, packed_dim=0)
+        if device is not None:
+            out = {k: v.to(device) for k, v in out.items()}
+        return out
+
     def decompress_weight(
         self,
         compressed_data: Dict[str, Tensor],

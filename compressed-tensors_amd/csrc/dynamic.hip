@@ -33,27 +33,22 @@ struct DynOut {
   void* zp;     // optional
 };
 
-// The zero point as fake_quantize reads it back from its storage dtype: fp8 rounds
-// it, an integer dtype has no -0 (rint of a small negative value gives one).
-__device__ __forceinline__ float stored_zero_point(float z, const QpCfg& c) {
-  return c.qtype == CTMI_QTYPE_INT ? z + 0.0f : round_to(z, c.zp_dtype);
-}
-
-// One wavefront per row-long segment (token / channel): up to 64 * U vectors of
-// 8 elements, all loaded before anything is looked at.
+// One workgroup of 256 threads per row-long segment (token / channel) of up to
+// 256 * U vectors of 8 elements: every vector is loaded before anything is looked
+// at; the four wavefronts meet once, over 8 floats in LDS.
 template <typename FT, int QK, int U>
 __global__ void __launch_bounds__(256)
 dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __restrict__ out,
-                    DynOut o, int64_t n_segments, int items, QpCfg c) {
+                    DynOut o, int items, QpCfg c) {
   using FR = typename FT::raw;
-  const int lane = threadIdx.x & 63;
-  const int64_t s = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (s >= n_segments) return;
+  __shared__ float part_lo[4], part_hi[4];
+  __shared__ int part_nan[4];
+  const int64_t s = blockIdx.x;
   const FR* p = x + s * (int64_t)items * 8;
   Vec<FR, 8> a[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
-    const int i = k * 64 + lane;
+    const int i = k * 256 + threadIdx.x;
     a[k] = ldg_nt<FR, 8>(p + (int64_t)(i < items ? i : items - 1) * 8);  // re-reads do not change min / max
   }
   float lo = __builtin_inff(), hi = -__builtin_inff();
@@ -61,18 +56,27 @@ dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
 #pragma unroll
   for (int k = 0; k < U; ++k) vec_minmax<FT>(a[k], &lo, &hi, &unordered);
   group_minmax(64, &lo, &hi);
-  if (group_any(64, unordered)) lo = hi = __builtin_nanf("");
+  unordered = group_any(64, unordered);
+  if ((threadIdx.x & 63) == 0) {
+    part_lo[threadIdx.x >> 6] = lo;
+    part_hi[threadIdx.x >> 6] = hi;
+    part_nan[threadIdx.x >> 6] = unordered;
+  }
+  __syncthreads();
+  lo = __builtin_fminf(__builtin_fminf(part_lo[0], part_lo[1]), __builtin_fminf(part_lo[2], part_lo[3]));
+  hi = __builtin_fmaxf(__builtin_fmaxf(part_hi[0], part_hi[1]), __builtin_fmaxf(part_hi[2], part_hi[3]));
+  if (part_nan[0] | part_nan[1] | part_nan[2] | part_nan[3]) lo = hi = __builtin_nanf("");
   float sv, zv;
-  qparams_value(lo, hi, 1.0f, c, &sv, &zv);
+  qparams_value<FT::id>(lo, hi, 1.0f, c, &sv, &zv);
   zv = stored_zero_point(zv, c);
-  if (lane == 0) {
+  if (threadIdx.x == 0) {
     if (o.scale) store_from_f32(o.scale, c.scale_dtype, s, sv);
     if (o.zp) store_from_f32(o.zp, c.zp_dtype, s, zv);
   }
   FR* q = out + s * (int64_t)items * 8;
 #pragma unroll
   for (int k = 0; k < U; ++k) {
-    const int i = k * 64 + lane;
+    const int i = k * 256 + threadIdx.x;
     Vec<FR, 8> of;
     Vec<uint8_t, 8> oc;
     qdq_vec8<FT, kKindFloat, kKindFloat, QK, true>(a[k], oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
@@ -104,9 +108,8 @@ dynamic_flat_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
     group_minmax(L, &lo, &hi);
     if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
     float sv, zv;
-    qparams_value(lo, hi, 1.0f, c, &sv, &zv);
+    qparams_value<FT::id>(lo, hi, 1.0f, c, &sv, &zv);
     zv = stored_zero_point(zv, c);
-  zv = stored_zero_point(zv, c);
     if (v < nvec && (threadIdx.x & (L - 1)) == 0) {
       if (o.scale) store_from_f32(o.scale, c.scale_dtype, v / L, sv);
       if (o.zp) store_from_f32(o.zp, c.zp_dtype, v / L, zv);
@@ -132,15 +135,13 @@ static bool launch_dynamic(const void* x, void* out, const DynOut& o, int64_t ro
                        (FR*)out, o, nvec, (int)items, c);
     return true;
   }
-  const int64_t blocks = cdiv(n_segments, 4);
-  if (blocks >= (1ll << 31)) return false;
-#define CTMI_DYN(UU)                                                                              \
-  hipLaunchKernelGGL((dynamic_rows_kernel<FT, QK, UU>), (unsigned)blocks, 256, 0, st, (const FR*)x, \
-                     (FR*)out, o, n_segments, (int)items, c)
-  if (items <= 64 * 2) CTMI_DYN(2);
-  else if (items <= 64 * 4) CTMI_DYN(4);
-  else if (items <= 64 * 8) CTMI_DYN(8);
-  else if (items <= 64 * 16) CTMI_DYN(16);
+  if (n_segments >= (1ll << 31)) return false;
+#define CTMI_DYN(UU)                                                                    \
+  hipLaunchKernelGGL((dynamic_rows_kernel<FT, QK, UU>), (unsigned)n_segments, 256, 0, st, \
+                     (const FR*)x, (FR*)out, o, (int)items, c)
+  if (items <= 256) CTMI_DYN(1);
+  else if (items <= 256 * 2) CTMI_DYN(2);
+  else if (items <= 256 * 4) CTMI_DYN(4);
   else return false;
 #undef CTMI_DYN
   return true;

@@ -11,6 +11,7 @@
 #include "ctmi_device.h"
 #include "ctmi_host.h"
 #include "minmax.h"
+#include "qdq_core.h"
 #include "qparams.h"
 #include "quant_core.h"
 #include "quant_fast.h"
@@ -398,6 +399,33 @@ bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dty
   return true;
 }
 
+// calculate_qparams (helpers.py:67-146) for one group of an fp4 scheme with a
+// global scale, min / max in XT: scale = fp8(clamp(gs * XT(max|x| / 6), +-448)),
+// zero replaced by 0.125.  Returns the fp8 code, *sv = its value.
+template <typename XT>
+__device__ __forceinline__ uint8_t nvfp4_group_scale(float lo, float hi, bool has_nan, float gs,
+                                                     float* sv) {
+  // max(|min(lo, 0)|, |max(hi, 0)|)
+  const float m = __builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f);
+  float t = m / 6.0f, same = t;
+  round2<XT::id>(t, same);
+  float s = gs * t;
+  has_nan |= s != s;  // inf * 0
+  s = __builtin_fminf(__builtin_fmaxf(s, -448.0f), 448.0f);
+  uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s, s, 0, false) & 0xffu;
+  float value = __builtin_amdgcn_cvt_f32_fp8((int)code, 0);
+  if (value == 0.0f) {
+    code = 0x20u;  // 0.125
+    value = 0.125f;
+  }
+  if (has_nan) {
+    code = 0x7fu;
+    value = __builtin_nanf("");
+  }
+  *sv = value;
+  return (uint8_t)code;
+}
+
 // Dynamic nvfp4 activations (forward.py:414-451 with a tensor_group scheme): the
 // group scales come from the 16 elements themselves (helpers.py:149-205, :67-146),
 // which are then fake-quantized with them without leaving the registers.  Two
@@ -406,7 +434,7 @@ template <typename XT>
 __global__ void __launch_bounds__(kFp4Block)
 nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __restrict__ gscale,
                      typename XT::raw* __restrict__ out, uint8_t* __restrict__ scale_out,
-                     uint8_t* __restrict__ zp_out, uint32_t nvec, QpCfg c) {
+                     uint8_t* __restrict__ zp_out, uint32_t nvec) {
   constexpr int B = kFp4Block, U = 2;
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
@@ -423,11 +451,10 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
     bool unordered = false;
     vec_minmax<XT>(xv[k], &lo, &hi, &unordered);
     group_minmax(2, &lo, &hi);
-    if (group_any(2, unordered)) lo = hi = __builtin_nanf("");
-    float sv, zv;
-    qparams_value(lo, hi, gs, c, &sv, &zv);
+    float sv;
+    const uint8_t code = nvfp4_group_scale<XT>(lo, hi, group_any(2, unordered), gs, &sv);
     if (v < nvec && (threadIdx.x & 1) == 0) {
-      if (scale_out) scale_out[v >> 1] = f32_to_f8e4m3(sv);
+      if (scale_out) scale_out[v >> 1] = code;
       if (zp_out) zp_out[v >> 1] = 0;  // fp8 zero
     }
     const float s = sv / gs;
@@ -452,9 +479,9 @@ bool nvfp4_dynamic_try(const void* x, int x_dtype, void* out, int64_t rows, int6
   if (nvec >= (1ll << 32) || grid >= (1ll << 31)) return false;
   auto* so = (uint8_t*)scale_out;
   auto* zo = (uint8_t*)zp_out;
-  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_dynamic_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, (uint16_t*)out, so, zo, (uint32_t)nvec, c);
-  else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_dynamic_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, (uint16_t*)out, so, zo, (uint32_t)nvec, c);
-  else if (x_dtype == CTMI_F32) hipLaunchKernelGGL(nvfp4_dynamic_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, gscale, (float*)out, so, zo, (uint32_t)nvec, c);
+  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_dynamic_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, (uint16_t*)out, so, zo, (uint32_t)nvec);
+  else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_dynamic_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, (uint16_t*)out, so, zo, (uint32_t)nvec);
+  else if (x_dtype == CTMI_F32) hipLaunchKernelGGL(nvfp4_dynamic_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, gscale, (float*)out, so, zo, (uint32_t)nvec);
   else return false;
   return true;
 }

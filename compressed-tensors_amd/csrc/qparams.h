@@ -21,10 +21,19 @@ struct QpCfg {
   int scale_dtype, zp_dtype;
 };
 
-// returns scale and zero point as fp32 values already rounded to their storage dtypes
-__device__ __forceinline__ void qparams_value(float mn, float mx, float gs, const QpCfg& c,
+// Returns the scale rounded to its storage dtype, and the zero point before its
+// storage cast, both as fp32.  MT >= 0 fixes the dtype of min / max at compile
+// time (c.mt and c.zp_sub_dtype are then not looked at), which removes the dtype
+// dispatch from every rounding step.
+template <int MT = -1>
+__device__ __forceinline__ void qparams_value(float mn, float mx, float gs, const QpCfg& cfg,
                                               float* scale, float* zp) {
   constexpr float kEps = 1.1920928955078125e-07f;  // torch.finfo(torch.float32).eps
+  struct {
+    float bit_min, bit_max, sym_div, range;
+    int qtype, symmetric, mt, zp_sub_dtype, fp4_global;
+  } c = {cfg.bit_min, cfg.bit_max, cfg.sym_div, cfg.range, cfg.qtype, cfg.symmetric,
+         MT >= 0 ? MT : cfg.mt, MT >= 0 ? MT : cfg.zp_sub_dtype, cfg.fp4_global};
   mn = nan_min(mn, 0.0f);
   mx = nan_max(mx, 0.0f);
   float s, z;
@@ -49,6 +58,12 @@ __device__ __forceinline__ void qparams_value(float mn, float mx, float gs, cons
   }
   *scale = s;
   *zp = z;
+}
+
+// The zero point as quantize / dequantize read it back from its storage dtype: fp8
+// rounds it, an integer dtype has no -0 (rint of a small negative value gives one).
+__device__ __forceinline__ float stored_zero_point(float z, const QpCfg& c) {
+  return c.qtype == CTMI_QTYPE_INT ? z + 0.0f : round_to(z, c.zp_dtype);
 }
 
 }  // namespace ctmi

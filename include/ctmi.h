@@ -268,6 +268,25 @@ int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows, int64_t c
                          void* zero_point, int32_t zp_dtype, void* min_out, void* max_out,
                          void* stream);
 
+/* A2 + A1 + A5 + A9 fused: min-max observer (tests/mock_observer.py:38-113),
+ * calculate_qparams (quantization/utils/helpers.py:67-146), quantize
+ * (quantization/lifecycle/forward.py:45-81, 455-487) and pack_to_int32
+ * (compressors/quantized_compressors/pack_quantized.py:186-246) in one pass over
+ * a weight x[rows, cols], for cells of 1 x blk_cols elements (group: blk_cols =
+ * group_size, channel: blk_cols = cols) and 4- or 8-bit integer codes: what
+ * PackedQuantizationCompressor.compress_weight (pack_quantized.py:88-146)
+ * returns for scales a min-max observer has just produced, with the weight read
+ * once.  packed: int32 [rows, cols * num_bits / 32].  scale: [rows, cols /
+ * blk_cols] in x_dtype.  zero_point: optional int8 [rows, cols / blk_cols]
+ * (unpacked; asymmetric schemes pack it with ctmi_pack_to_int32, packed_dim 0).
+ * ctmi_observe_pack_quantized_supported() says whether the layout has a kernel
+ * (cells of up to 16384 elements in multiples of 8 that tile the rows). */
+int ctmi_observe_pack_quantized_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                          int64_t blk_cols, int32_t num_bits);
+int ctmi_observe_pack_quantized(const void* x, int32_t x_dtype, int64_t rows, int64_t cols,
+                                int64_t blk_cols, int32_t num_bits, int32_t symmetric,
+                                int32_t* packed, void* scale, int8_t* zero_point, void* stream);
+
 /* A26.  Dynamic activation quantization in one pass (forward_quantize with
  * args.dynamic, quantization/lifecycle/forward.py:414-451): the scales of
  * compute_dynamic_scales_and_zp (quantization/utils/helpers.py:149-205, via

@@ -112,6 +112,72 @@ def test_pack_quantized_compressor(spec, shape, dtype, gpu):
     assert torch.equal(dense.cpu(), oq.fake_quantize(w, scale, zp, oargs).to(scale.dtype))
 
 
+ONE_SHOT = [
+    # (args, shape, dtype, fused kernel expected)
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (128, 1024), torch.bfloat16, True),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=128), (77, 512), torch.bfloat16, True),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (33, 96), torch.float16, True),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=64), (32, 256), torch.float32, True),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=24), (16, 48), torch.bfloat16, True),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="channel"), (64, 520), torch.bfloat16, True),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="channel"), (19, 4096), torch.float16, True),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (5, 14336), torch.bfloat16, True),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=12), (10, 36), torch.bfloat16, False),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="tensor"), (16, 64), torch.bfloat16, False),
+    (dict(num_bits=3, type="int", symmetric=True, strategy="channel"), (10, 40), torch.bfloat16, False),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype,fused", ONE_SHOT,
+                         ids=[f"os{i}-{c[0]['strategy']}" for i, c in enumerate(ONE_SHOT)])
+def test_observe_and_compress_in_one_pass(spec, shape, dtype, fused, gpu):
+    """observer + calculate_qparams + quantize + pack from one kernel: the oracle's
+    observe_weight followed by its pack_quantized_compress, bit for bit"""
+    from compressed_tensors_amd import _lib
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("one-shot pack-quantized", spec, shape, dtype)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(32)
+    w = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+    w[0, :8] = 0.0
+    w[0, 1] = -0.0
+    w[-1] = 0.0                     # a row of zeros: the scale floor
+    w[1] = w[1].abs()               # one-sided rows: min / max are clamped to include 0
+    w[2] = -w[2].abs()
+    w[3, 5] = float("nan")
+    w[4, 0] = float("inf")
+    rows, cols = shape
+    blk = {"group": spec.get("group_size", 0), "channel": cols}.get(spec["strategy"], 0)
+    assert bool(blk and _lib.load().ctmi_observe_pack_quantized_supported(
+        _lib.dtype_code(dtype), rows, cols, blk, spec["num_bits"])) == fused
+    scale, zp = oq.observe_weight(w, oargs)
+    want = op.pack_quantized_compress(w, scale, oargs, zero_point=zp)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    got = comp.observe_and_compress_weight(w.to(gpu), args)
+    assert set(got) == set(want) | {"weight_scale"}
+    # a NaN in a cell makes its scale NaN; the codes of such a cell are an int cast of NaN,
+    # which is not defined: compare the others
+    bad_cells = torch.isnan(scale.float())
+    if spec["strategy"] == "tensor":
+        ok = torch.full(shape, not bool(bad_cells.any()))
+    else:
+        ok = ~bad_cells.repeat_interleave(cols // scale.shape[-1], dim=-1)
+    nan = torch.full_like(scale, float("nan"))
+    assert_bit_equal(torch.where(bad_cells.to(gpu), nan.to(gpu), got["weight_scale"]),
+                     torch.where(bad_cells, nan, scale), "scale")
+    from oracle.pack import unpack_from_int32 as o_unpack
+    got_codes = o_unpack(got["weight_packed"].cpu(), spec["num_bits"], torch.Size(shape))
+    want_codes = o_unpack(want["weight_packed"], spec["num_bits"], torch.Size(shape))
+    assert torch.equal(got_codes[ok], want_codes[ok]), "codes"
+    assert_bit_equal(got["weight_shape"], want["weight_shape"], "weight_shape")
+    if "weight_zero_point" in want:
+        n_cells = scale.shape[-1]
+        gz = o_unpack(got["weight_zero_point"].cpu(), spec["num_bits"], torch.Size((rows, n_cells)), packed_dim=0)
+        wz = o_unpack(want["weight_zero_point"], spec["num_bits"], torch.Size((rows, n_cells)), packed_dim=0)
+        assert torch.equal(gz[~bad_cells], wz[~bad_cells]), "zero points"
+
+
 def test_pack_quantized_state_dict_and_g_idx(gpu):
     from compressed_tensors_amd.compressors import BaseCompressor
     from compressed_tensors_amd.quantization import QuantizationScheme

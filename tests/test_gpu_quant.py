@@ -215,6 +215,9 @@ def test_dynamic_quant_in_one_pass(spec, shape, dtype, fusable, gpu):
     if flat.shape[0] > 2:
         flat[1, 5] = float("nan")          # poisons its group / token
         flat[2, 0] = float("inf")
+    if flat.shape[0] > 6:
+        flat[3] *= 1e-5                    # group scales down in the subnormal range of fp8
+        flat[4] *= 3e-4
     gs = o_gs = None
     module = torch.nn.Module()
     if args.strategy == "tensor_group":
