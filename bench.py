@@ -21,6 +21,8 @@ that no pass finds its input in the last-level cache:
                     on a 2:4 pruned, fp8-quantized 14336 x 4096 weight
   nvfp4             nvfp4-pack-quantized on 14336 x 4096 and 4096 x 14336 bf16 weights
                     + dynamic nvfp4 activation quantization, 4096 x 4096
+  one-shot          the default set with no scales given: min-max observer, qparams,
+                    quantize and pack, as separate passes and as one
   hadamard          block-128 and full 4096 rotations of 8192 x 4096 activations and of
                     4096 x 4096 / 14336 x 4096 weights
 """
@@ -316,6 +318,37 @@ def other_workload(torch, name, seed):
                 Op("nvfp4 activations: scales + fake-quantize in one pass (16 x 4096x4096)", y_calls, 4 * na, "nvfp4_dynamic_kernel")]
         return "nvfp4-pack-quantized compress/decompress + activation fake-quantize GB/s", ops, keep
 
+    if name == "one-shot":
+        # the Llama-3-8B-shaped set, no scales yet: observer + qparams + quantize + pack
+        args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
+        sep_obs, sep_cmp, fused, job_fields, n = [], [], [], [], 0
+        for _, r, c in shapes_for("llama3-8b-w4a16"):
+            w = randn(r, c, 0.02)
+            scale, zp = observe_weight_qparams(w, args)
+            packed = torch.empty(r, c // 8, dtype=torch.int32, device=dev)
+            plan = build_qparams(w, scale, None, args, None, None)
+            keep.extend([w, scale, zp, packed, plan])
+            sep_obs.append(observe(w, GROUP, args, scale, zp))
+            ca = (w.data_ptr(), code(w.dtype), packed.data_ptr(), r, c, ctypes.byref(plan.qp), st)
+            sep_cmp.append(lambda ca=ca: _lib.check(lib.ctmi_pack_quantized_compress(*ca)))
+            fa = (w.data_ptr(), code(w.dtype), r, c, GROUP, 4, 1, packed.data_ptr(), scale.data_ptr(), None, st)
+            fused.append(lambda fa=fa: _lib.check(lib.ctmi_observe_pack_quantized(*fa)))
+            job_fields.append((w.data_ptr(), packed.data_ptr(), scale.data_ptr(), None, r, c, GROUP,
+                               code(w.dtype), 4, 1))
+            n += r * c
+        jobs = (_lib.ObservePackJob * len(job_fields))()
+        for j, f in zip(jobs, job_fields):
+            (j.x, j.packed, j.scale, j.zero_point, j.rows, j.cols, j.blk_cols, j.x_dtype,
+             j.num_bits, j.symmetric) = f
+        keep.append(jobs)
+        many = [lambda: _lib.check(lib.ctmi_observe_pack_quantized_many(jobs, len(job_fields), st))]
+        g = n // GROUP
+        ops = [Op("observer + qparams, group 128 (224 tensors, one call each)", sep_obs, 2 * n + 3 * g, "observe_flat_kernel"),
+               Op("quantize + pack with those scales (one call each)", sep_cmp, 2 * n + 2 * g + n // 2, "pq_compress_vec_kernel"),
+               Op("observer + qparams + quantize + pack in one pass (one call each)", fused, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel"),
+               Op("the same, all 224 tensors in one call (8 per launch)", many, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel")]
+        return "one-shot W4A16 g128 compression GB/s (no scales given), Llama-3-8B-shaped weights", ops, keep
+
     if name == "hadamard":
         ops = []
         tensors = {"activations 8192x4096 (x8)": [randn(8192, 4096) for _ in range(8)],
@@ -415,7 +448,7 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     _lib.load()
     dev = torch.device("cuda:0")
-    if a.workload in ("fp8-w8a8", "sparse", "nvfp4", "hadamard"):
+    if a.workload in ("fp8-w8a8", "sparse", "nvfp4", "hadamard", "one-shot"):
         return run_other(torch, a)
     shapes = shapes_for(a.workload)
     args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group",

@@ -85,6 +85,15 @@ class WeightJob(ctypes.Structure):
     ]
 
 
+class ObservePackJob(ctypes.Structure):
+    """ctmi_observe_pack_job"""
+    _fields_ = [
+        ("x", c_void_p), ("packed", c_void_p), ("scale", c_void_p), ("zero_point", c_void_p),
+        ("rows", c_int64), ("cols", c_int64), ("blk_cols", c_int64),
+        ("x_dtype", c_int32), ("num_bits", c_int32), ("symmetric", c_int32),
+    ]
+
+
 class QdqJob(ctypes.Structure):
     """ctmi_qdq_job"""
 
@@ -197,6 +206,7 @@ SIGNATURES = {
     "ctmi_observe_pack_quantized_supported": (
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32],
     ),
+    "ctmi_observe_pack_quantized_many": (c_int32, [c_void_p, c_int64, c_void_p]),
     "ctmi_observe_pack_quantized": (
         c_int32,
         [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p,

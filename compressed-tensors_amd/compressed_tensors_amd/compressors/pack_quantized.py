@@ -25,7 +25,8 @@ from compressed_tensors_amd.quantization.forward import (
 from compressed_tensors_amd.quantization.helpers import can_quantize
 from compressed_tensors_amd.quantization.quant_args import QuantizationArgs, QuantizationStrategy
 
-__all__ = ["PackedQuantizationCompressor", "pack_to_int32", "unpack_from_int32"]
+__all__ = ["PackedQuantizationCompressor", "PackedWeightBatch", "ObservedWeightBatch",
+           "pack_to_int32", "unpack_from_int32"]
 
 _PACKABLE = (QuantizationStrategy.GROUP.value, QuantizationStrategy.CHANNEL.value)
 
@@ -345,6 +346,63 @@ class PackedWeightBatch:
                                                             _lib.stream_of(self.device))
         )
         return self.dense
+
+
+class ObservedWeightBatch:
+    """Every weight of a model that has no scales yet, prepared for a one-call,
+    one-pass compression: min-max observer, calculate_qparams, quantize and pack
+    (ctmi_observe_pack_quantized_many).  Buffers are allocated once; `compress()`
+    only enqueues kernels and returns, per weight, what
+    PackedQuantizationCompressor.observe_and_compress_weight returns."""
+
+    def __init__(self, entries, device=None):
+        """entries: dicts with weight (2-D float tensor) and quantization_args
+        (int, 4 or 8 bits, group or channel strategy)"""
+        lib = _lib.load()
+        self.n = len(entries)
+        self.device = device
+        self.weights, self.packed, self.scales, self.zero_points, self.args = [], [], [], [], []
+        self._jobs = (_lib.ObservePackJob * max(self.n, 1))()
+        for i, e in enumerate(entries):
+            args = e["quantization_args"]
+            w = to_gpu(e["weight"]).contiguous()
+            if w.ndim != 2:
+                raise ValueError(f"expected a 2-D weight, got shape {tuple(w.shape)}")
+            if self.device is None:
+                self.device = w.device
+            rows, cols = w.shape
+            blk_cols = {QuantizationStrategy.GROUP.value: args.group_size,
+                        QuantizationStrategy.CHANNEL.value: cols}.get(args.strategy, 0)
+            if not (blk_cols and args.type == "int" and lib.ctmi_observe_pack_quantized_supported(
+                    _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits)):
+                raise NotImplementedError(
+                    f"no one-pass kernel for {args.strategy} / {args.num_bits} bits on a "
+                    f"{tuple(w.shape)} {w.dtype} weight: use observe_and_compress_weight")
+            n_cells = cols // min(blk_cols, cols)
+            packed = torch.empty((rows, cols * args.num_bits // 32), dtype=torch.int32, device=w.device)
+            scale = torch.empty((rows, n_cells), dtype=w.dtype, device=w.device)
+            zp = None if args.symmetric else torch.empty((rows, n_cells), dtype=torch.int8, device=w.device)
+            j = self._jobs[i]
+            j.x, j.packed, j.scale, j.zero_point = w.data_ptr(), packed.data_ptr(), scale.data_ptr(), _lib.ptr(zp)
+            j.rows, j.cols, j.blk_cols = rows, cols, blk_cols
+            j.x_dtype, j.num_bits, j.symmetric = _lib.dtype_code(w.dtype), args.num_bits, int(args.symmetric)
+            self.weights.append(w)
+            self.packed.append(packed)
+            self.scales.append(scale)
+            self.zero_points.append(zp)
+            self.args.append(args)
+
+    def compress(self):
+        _lib.check(_lib.load().ctmi_observe_pack_quantized_many(self._jobs, self.n,
+                                                                _lib.stream_of(self.device)))
+        out = []
+        for w, packed, scale, zp, args in zip(self.weights, self.packed, self.scales,
+                                              self.zero_points, self.args):
+            d = {"weight_shape": torch.tensor(w.shape), "weight_packed": packed, "weight_scale": scale}
+            if zp is not None:
+                d["weight_zero_point"] = pack_to_int32(zp, args.num_bits, packed_dim=0)
+            out.append(d)
+        return out
 
 
 def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,

@@ -9,75 +9,172 @@
 //
 // Traffic per element of a bf16 weight: 2 bytes in, num_bits / 8 out (+ scales),
 // against 2 in for the observer and 2 in again for the compressor.
+#include <cstring>
 #include <type_traits>
+#include <vector>
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "job_table.h"
 #include "minmax.h"
+#include "qdq_core.h"
 #include "qparams.h"
 #include "quant_core.h"
 #include "quant_fast.h"
 
 namespace ctmi {
 
-int fill_qpcfg(QpCfg* c, int qtype, int num_bits, int symmetric, int mt, int mm_is_0d,
-               bool has_gscale, int scale_dtype, int zp_dtype);
+constexpr float kScaleFloor = 1.1920928955078125e-07f;  // torch.finfo(torch.float32).eps
 
-struct ObservePackOut {
-  int32_t* packed;
-  void* scale;
-  int8_t* zp;  // optional, unpacked
-};
+// ------------------------------------------------------------------ |x| maximum on the raw bits
+// For a symmetric scheme only max|x| matters (helpers.py:87-110 with min <= 0 <= max:
+// max(|min|, |max|) = max|x|).  The magnitude bits of a 16-bit float order like
+// unsigned integers, NaNs above infinity, so two elements go through one packed
+// integer maximum and a NaN shows in the result by itself.
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
 
-template <typename XT, int BITS>
-__device__ __forceinline__ Vec<int32_t, BITS / 4> observe_pack_codes(
-    const Vec<typename XT::raw, 8>& a, float sv, float zv, const QpCfg& c) {
-  // a symmetric scheme's zero point is 0: adding it changes no code
-  if (c.symmetric) return quant_pack8<XT, XT, BITS, false>(a, sv, 0.0f, c.bit_min, c.bit_max);
-  return quant_pack8<XT, XT, BITS, true>(a, sv, zv, c.bit_min, c.bit_max);
+template <typename XT>
+__device__ __forceinline__ uint32_t absmax8_bits(const Vec<typename XT::raw, 8>& a) {
+  static_assert(sizeof(typename XT::raw) == 2, "16-bit floats only");
+  const Vec<uint32_t, 4> w = __builtin_bit_cast(Vec<uint32_t, 4>, a);
+  u16x2_t m[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) m[j] = __builtin_bit_cast(u16x2_t, w.v[j] & 0x7fff7fffu);
+  const u16x2_t r = __builtin_elementwise_max(__builtin_elementwise_max(m[0], m[1]),
+                                              __builtin_elementwise_max(m[2], m[3]));
+  return r.x > r.y ? (uint32_t)r.x : (uint32_t)r.y;
 }
 
-// Groups of L vectors of 8 elements, L a power of two <= 64: L neighbouring lanes
-// own a group; vectors, words and groups are all numbered row-major.
-template <typename XT, int BITS, int U>
-__global__ void __launch_bounds__(256)
-observe_pack_flat_kernel(const typename XT::raw* __restrict__ x, ObservePackOut o, int64_t nvec,
-                         int L, QpCfg c) {
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_umax_step(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+  return o > v ? o : v;
+}
+
+// all-reduce over aligned groups of L lanes (L a power of two <= 64)
+__device__ __forceinline__ uint32_t group_umax(int L, uint32_t v) {
+  if (L >= 2) v = dpp_umax_step<0xB1>(v);
+  if (L >= 4) v = dpp_umax_step<0x4E>(v);
+  if (L >= 8) v = dpp_umax_step<0x141>(v);
+  if (L >= 16) v = dpp_umax_step<0x140>(v);
+  for (int d = 16; d < L; d <<= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)v, d, kWave);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+// ------------------------------------------------------------------ scale and zero point of a group
+// calculate_qparams for an integer scheme with min / max in XT, the dtype dispatch
+// and the scheme dispatch of the general routine resolved at compile time.
+template <typename XT>
+__device__ __forceinline__ float round_xt(float v) {
+  float same = v;
+  round2<XT::id>(v, same);
+  return v;
+}
+
+// symmetric: scale = max(XT(max|x| / (range / 2)), eps)
+template <typename XT>
+__device__ __forceinline__ float symmetric_scale(float absmax, bool has_nan, float half_range) {
+  float t;
+  if constexpr (XT::id == CTMI_BF16) {
+    // bf16 / bf16 (7.5 and 127.5 are bf16 values): the product with the reciprocal
+    // rounds to the same bf16 as the quotient
+    t = absmax * __builtin_amdgcn_rcpf(half_range);
+  } else {
+    t = absmax / half_range;
+  }
+  const float s = __builtin_fmaxf(round_xt<XT>(t), kScaleFloor);
+  return has_nan ? __builtin_nanf("") : s;
+}
+
+// asymmetric: scale = max(XT(XT(max - min) / range), eps),
+//             zp = round(clamp(XT(qmin - XT(min / scale)), qmin, qmax))
+template <typename XT>
+__device__ __forceinline__ void asymmetric_qparams(float lo, float hi, bool has_nan, float qmin,
+                                                   float qmax, float* scale, float* zp) {
+  const float mn = __builtin_fminf(lo, 0.0f), mx = __builtin_fmaxf(hi, 0.0f);
+  float s = round_xt<XT>(round_xt<XT>(mx - mn) / (qmax - qmin));
+  s = (s != s) ? s : __builtin_fmaxf(s, kScaleFloor);  // inf - inf
+  float z = round_xt<XT>(qmin - round_xt<XT>(mn / s));
+  z = (z != z) ? z : __builtin_fminf(__builtin_fmaxf(z, qmin), qmax);
+  z = rintf(z) + 0.0f;  // an int8 zero point has no -0
+  const float nan = __builtin_nanf("");
+  *scale = has_nan ? nan : s;
+  *zp = has_nan ? nan : z;
+}
+
+// ------------------------------------------------------------------ groups within a row
+constexpr int kOpBlock = 512, kOpUnroll = 2;
+
+// One item = 8 neighbouring elements; L = 2^job.shift neighbouring lanes own a
+// group.  Items, words and groups are numbered row-major, so a chunk of
+// kOpBlock * kOpUnroll items never splits a group.  job.scale / job.zp are outputs.
+template <typename XT, int BITS, bool SYM>
+__global__ void __launch_bounds__(kOpBlock) observe_pack_groups_kernel(const ChainTable t) {
   using XR = typename XT::raw;
   constexpr int W = BITS / 4;
-  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
-  Vec<XR, 8> a[U];
+  constexpr int B = kOpBlock, U = kOpUnroll;
+  uint32_t chunk, nvec;
+  const ChainJob job = find_job(t, blockIdx.x, &chunk, &nvec);
+  const auto* __restrict__ x = (const XR*)job.src;
+  int32_t* __restrict__ out = (int32_t*)job.dst;
+  XR* __restrict__ scale = (XR*)const_cast<void*>(job.scale);
+  int8_t* __restrict__ zp = const_cast<int8_t*>(job.zp);
+  const int L = 1 << job.shift;
+  const uint32_t v0 = chunk * (B * U) + threadIdx.x;
+  const bool full = (chunk + 1) * (uint32_t)(B * U) <= nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    Vec<XR, 8> a[U];
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const int64_t v = v0 + k * 256;
-    a[k] = ldg_nt<XR, 8>(x + (v < nvec ? v : nvec - 1) * 8);
-  }
-#pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const int64_t v = v0 + k * 256;
-    float lo = __builtin_inff(), hi = -__builtin_inff();
-    bool unordered = false;
-    vec_minmax<XT>(a[k], &lo, &hi, &unordered);
-    group_minmax(L, &lo, &hi);
-    if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
-    float sv, zv;
-    qparams_value<XT::id>(lo, hi, 1.0f, c, &sv, &zv);
-    zv = stored_zero_point(zv, c);
-    if (v < nvec && (threadIdx.x & (L - 1)) == 0) {
-      ((XR*)o.scale)[v / L] = XT::from_f32(sv);
-      if (o.zp) o.zp[v / L] = (int8_t)f32_to_int(zv);
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      // past the end: read the last item again, it changes no group it belongs to
+      a[k] = ldg_nt<XR, 8>(x + (size_t)(GUARD && v >= nvec ? nvec - 1 : v) * 8);
     }
-    const Vec<int32_t, W> w = observe_pack_codes<XT, BITS>(a[k], sv, zv, c);
-    if (v < nvec) stg_nt<int32_t, W>(o.packed + v * W, w);
-  }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      float sv, zv = 0.0f;
+      if constexpr (SYM && sizeof(XR) == 2) {
+        const uint32_t m = group_umax(L, absmax8_bits<XT>(a[k]));
+        constexpr uint32_t kInf = XT::id == CTMI_BF16 ? 0x7f80u : 0x7c00u;
+        sv = symmetric_scale<XT>(XT::to_f32((XR)m), m > kInf, (t.qmax - t.qmin) * 0.5f);
+      } else {
+        float lo = __builtin_inff(), hi = -__builtin_inff();
+        bool unordered = false;
+        vec_minmax<XT>(a[k], &lo, &hi, &unordered);
+        group_minmax(L, &lo, &hi);
+        unordered = group_any(L, unordered);
+        if constexpr (SYM) {
+          const float m = __builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f);
+          sv = symmetric_scale<XT>(m, unordered, (t.qmax - t.qmin) * 0.5f);
+        } else {
+          asymmetric_qparams<XT>(lo, hi, unordered, t.qmin, t.qmax, &sv, &zv);
+        }
+      }
+      if ((!GUARD || v < nvec) && (threadIdx.x & (L - 1)) == 0) {
+        scale[v >> job.shift] = XT::from_f32(sv);
+        if (zp) zp[v >> job.shift] = SYM ? (int8_t)0 : (int8_t)f32_to_int(zv);
+      }
+      // a symmetric scheme's zero point is 0: adding it changes no code
+      const Vec<int32_t, W> w = quant_pack8<XT, XT, BITS, !SYM>(a[k], sv, zv, t.qmin, t.qmax);
+      if (!GUARD || v < nvec) stg_nt<int32_t, W>(out + (size_t)v * W, w);
+    }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
 }
 
-// One workgroup of 256 threads per row-long group (channel strategy) of up to
-// 256 * U vectors.
-template <typename XT, int BITS, int U>
+// ------------------------------------------------------------------ one group per row
+// One workgroup of 256 threads per row (channel strategy) of up to 256 * U items.
+template <typename XT, int BITS, bool SYM, int U>
 __global__ void __launch_bounds__(256)
-observe_pack_rows_kernel(const typename XT::raw* __restrict__ x, ObservePackOut o, int items,
-                         QpCfg c) {
+observe_pack_rows_kernel(const typename XT::raw* __restrict__ x, int32_t* __restrict__ packed,
+                         typename XT::raw* __restrict__ scale, int8_t* __restrict__ zp, int items,
+                         float qmin, float qmax) {
   using XR = typename XT::raw;
   constexpr int W = BITS / 4;
   __shared__ float part_lo[4], part_hi[4];
@@ -104,48 +201,188 @@ observe_pack_rows_kernel(const typename XT::raw* __restrict__ x, ObservePackOut 
   __syncthreads();
   lo = __builtin_fminf(__builtin_fminf(part_lo[0], part_lo[1]), __builtin_fminf(part_lo[2], part_lo[3]));
   hi = __builtin_fmaxf(__builtin_fmaxf(part_hi[0], part_hi[1]), __builtin_fmaxf(part_hi[2], part_hi[3]));
-  if (part_nan[0] | part_nan[1] | part_nan[2] | part_nan[3]) lo = hi = __builtin_nanf("");
-  float sv, zv;
-  qparams_value<XT::id>(lo, hi, 1.0f, c, &sv, &zv);
-  zv = stored_zero_point(zv, c);
-  if (threadIdx.x == 0) {
-    ((XR*)o.scale)[s] = XT::from_f32(sv);
-    if (o.zp) o.zp[s] = (int8_t)f32_to_int(zv);
+  unordered = (part_nan[0] | part_nan[1] | part_nan[2] | part_nan[3]) != 0;
+  float sv, zv = 0.0f;
+  if constexpr (SYM) {
+    sv = symmetric_scale<XT>(__builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f), unordered,
+                             (qmax - qmin) * 0.5f);
+  } else {
+    asymmetric_qparams<XT>(lo, hi, unordered, qmin, qmax, &sv, &zv);
   }
-  int32_t* q = o.packed + s * (int64_t)items * W;
+  if (threadIdx.x == 0) {
+    scale[s] = XT::from_f32(sv);
+    if (zp) zp[s] = SYM ? (int8_t)0 : (int8_t)f32_to_int(zv);
+  }
+  int32_t* q = packed + s * (int64_t)items * W;
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int i = k * 256 + threadIdx.x;
-    const Vec<int32_t, W> w = observe_pack_codes<XT, BITS>(a[k], sv, zv, c);
+    const Vec<int32_t, W> w = quant_pack8<XT, XT, BITS, !SYM>(a[k], sv, zv, qmin, qmax);
     if (i < items) stg_nt<int32_t, W>(q + (int64_t)i * W, w);
   }
 }
 
 constexpr int kObservePackMaxItems = 256 * 8;
 
-template <typename XT, int BITS>
-static bool launch_observe_pack(const void* x, const ObservePackOut& o, int64_t rows, int64_t cols,
-                                int64_t seg, const QpCfg& c, hipStream_t st) {
-  using XR = typename XT::raw;
-  const int64_t items = seg / 8, nvec = rows * cols / 8, n_segments = rows * (cols / seg);
-  if (items <= 64 && (items & (items - 1)) == 0) {
-    constexpr int U = 2;
-    const int64_t blocks = cdiv(nvec, 256 * U);
-    if (blocks >= (1ll << 31)) return false;
-    hipLaunchKernelGGL((observe_pack_flat_kernel<XT, BITS, U>), (unsigned)blocks, 256, 0, st,
-                       (const XR*)x, o, nvec, (int)items, c);
-    return true;
+// ------------------------------------------------------------------ host side
+struct OpKey {
+  int x_dtype, bits, symmetric;
+  bool operator==(const OpKey& o) const {
+    return x_dtype == o.x_dtype && bits == o.bits && symmetric == o.symmetric;
   }
-  if (n_segments >= (1ll << 31) || items > kObservePackMaxItems) return false;
-#define CTMI_OP(UU)                                                                          \
-  hipLaunchKernelGGL((observe_pack_rows_kernel<XT, BITS, UU>), (unsigned)n_segments, 256, 0, st, \
-                     (const XR*)x, o, (int)items, c)
-  if (items <= 256) CTMI_OP(1);
-  else if (items <= 256 * 2) CTMI_OP(2);
-  else if (items <= 256 * 4) CTMI_OP(4);
+};
+
+struct OpPlan {
+  OpKey key;
+  bool grouped;  // groups within a row (chained launches) or one group per row
+  const void* x;
+  int32_t* packed;
+  void* scale;
+  int8_t* zp;
+  int64_t rows, items;  // items per group
+  uint32_t nvec, shift;
+};
+
+template <typename XT, int BITS>
+static void launch_groups_sym(const OpKey& k, const ChainTable& t, unsigned grid, hipStream_t st) {
+  if (k.symmetric) hipLaunchKernelGGL((observe_pack_groups_kernel<XT, BITS, true>), grid, kOpBlock, 0, st, t);
+  else hipLaunchKernelGGL((observe_pack_groups_kernel<XT, BITS, false>), grid, kOpBlock, 0, st, t);
+}
+
+template <typename XT>
+static void launch_groups_bits(const OpKey& k, const ChainTable& t, unsigned grid, hipStream_t st) {
+  if (k.bits == 4) launch_groups_sym<XT, 4>(k, t, grid, st);
+  else launch_groups_sym<XT, 8>(k, t, grid, st);
+}
+
+static void launch_groups(const OpKey& k, const ChainTable& t, unsigned grid, hipStream_t st) {
+  if (k.x_dtype == CTMI_BF16) launch_groups_bits<BF16>(k, t, grid, st);
+  else if (k.x_dtype == CTMI_F16) launch_groups_bits<F16>(k, t, grid, st);
+  else launch_groups_bits<F32>(k, t, grid, st);
+}
+
+template <typename XT, int BITS, bool SYM>
+static void launch_rows_u(const OpPlan& p, float qmin, float qmax, hipStream_t st) {
+  using XR = typename XT::raw;
+#define CTMI_OP(UU)                                                                            \
+  hipLaunchKernelGGL((observe_pack_rows_kernel<XT, BITS, SYM, UU>), (unsigned)p.rows, 256, 0, st, \
+                     (const XR*)p.x, p.packed, (XR*)p.scale, p.zp, (int)p.items, qmin, qmax)
+  if (p.items <= 256) CTMI_OP(1);
+  else if (p.items <= 256 * 2) CTMI_OP(2);
+  else if (p.items <= 256 * 4) CTMI_OP(4);
   else CTMI_OP(8);
 #undef CTMI_OP
-  return true;
+}
+
+template <typename XT>
+static void launch_rows_xt(const OpPlan& p, float qmin, float qmax, hipStream_t st) {
+  if (p.key.bits == 4) {
+    if (p.key.symmetric) launch_rows_u<XT, 4, true>(p, qmin, qmax, st);
+    else launch_rows_u<XT, 4, false>(p, qmin, qmax, st);
+  } else {
+    if (p.key.symmetric) launch_rows_u<XT, 8, true>(p, qmin, qmax, st);
+    else launch_rows_u<XT, 8, false>(p, qmin, qmax, st);
+  }
+}
+
+static void launch_rows(const OpPlan& p, float qmin, float qmax, hipStream_t st) {
+  if (p.key.x_dtype == CTMI_BF16) launch_rows_xt<BF16>(p, qmin, qmax, st);
+  else if (p.key.x_dtype == CTMI_F16) launch_rows_xt<F16>(p, qmin, qmax, st);
+  else launch_rows_xt<F32>(p, qmin, qmax, st);
+}
+
+static bool op_supported(int x_dtype, int64_t rows, int64_t cols, int64_t blk_cols, int num_bits) {
+  if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16 && x_dtype != CTMI_F32) return false;
+  if (num_bits != 4 && num_bits != 8) return false;
+  if (rows < 1 || cols < 1 || blk_cols < 1) return false;
+  const int64_t seg = blk_cols < cols ? blk_cols : cols;
+  if (seg % 8 || cols % seg) return false;
+  const int64_t items = seg / 8;
+  if (rows * cols / 8 >= (1ll << 31)) return false;
+  if (items <= 64 && (items & (items - 1)) == 0) return true;  // groups of neighbouring lanes
+  return seg == cols && items <= kObservePackMaxItems;         // one workgroup per row
+}
+
+static int plan_observe_pack(const ctmi_observe_pack_job& j, OpPlan* p) {
+  CTMI_REQUIRE(j.rows >= 1 && j.cols >= 1, CTMI_ERR_VALUE, "cannot observe an empty tensor");
+  CTMI_REQUIRE(j.blk_cols >= 1, CTMI_ERR_VALUE, "empty cell");
+  float qmin, qmax;
+  int rc = quant_range(CTMI_QTYPE_INT, j.num_bits, &qmin, &qmax);
+  if (rc) return rc;
+  CTMI_REQUIRE(j.x_dtype == CTMI_F32 || j.x_dtype == CTMI_F16 || j.x_dtype == CTMI_BF16,
+               CTMI_ERR_UNSUPPORTED, "weights must be float16/bfloat16/float32");
+  CTMI_REQUIRE(j.x && j.packed && j.scale, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE(op_supported(j.x_dtype, j.rows, j.cols, j.blk_cols, j.num_bits), CTMI_ERR_UNSUPPORTED,
+               "no fused kernel for this layout: run the observer and the compressor separately");
+  CTMI_REQUIRE((uintptr_t)j.x % (8 * dtype_size(j.x_dtype)) == 0 &&
+                   (uintptr_t)j.packed % (4 * (j.num_bits / 4)) == 0 &&
+                   (uintptr_t)j.scale % dtype_size(j.x_dtype) == 0,
+               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+  const int64_t seg = j.blk_cols < j.cols ? j.blk_cols : j.cols;
+  p->key = OpKey{j.x_dtype, j.num_bits, j.symmetric ? 1 : 0};
+  p->x = j.x;
+  p->packed = j.packed;
+  p->scale = j.scale;
+  p->zp = j.zero_point;
+  p->rows = j.rows;
+  p->items = seg / 8;
+  p->nvec = (uint32_t)(j.rows * j.cols / 8);
+  p->grouped = p->items <= 64 && (p->items & (p->items - 1)) == 0;
+  p->shift = 0;
+  while ((1ll << p->shift) < p->items) ++p->shift;
+  return CTMI_OK;
+}
+
+static int run_observe_pack(const OpPlan* plans, int64_t n, hipStream_t st, const char* what) {
+  std::vector<char> done((size_t)n, 0);
+  const int per_block = kOpBlock * kOpUnroll;
+  for (int64_t i = 0; i < n; ++i) {
+    if (done[i]) continue;
+    const OpKey key = plans[i].key;
+    float qmin, qmax;
+    quant_range(CTMI_QTYPE_INT, key.bits, &qmin, &qmax);
+    if (!plans[i].grouped) {
+      launch_rows(plans[i], qmin, qmax, st);
+      done[i] = 1;
+      continue;
+    }
+    ChainTable t;
+    std::memset(&t, 0, sizeof(t));
+    t.qmin = qmin;
+    t.qmax = qmax;
+    uint64_t chunks = 0;
+    auto reset = [&]() {
+      t.n = 0;
+      chunks = 0;
+      for (int k = 0; k < kMaxJobs; ++k) t.chunk_end[k] = 0xFFFFFFFFu;
+    };
+    reset();
+    auto flush = [&]() {
+      if (t.n == 0) return;
+      launch_groups(key, t, (unsigned)chunks, st);
+      reset();
+    };
+    for (int64_t j = i; j < n; ++j) {
+      if (done[j] || !plans[j].grouped || !(plans[j].key == key)) continue;
+      const uint64_t c = (uint64_t)cdiv(plans[j].nvec, per_block);
+      if (t.n == kMaxJobs || chunks + c >= (1ull << 31)) flush();
+      ChainJob cj;
+      std::memset(&cj, 0, sizeof(cj));
+      cj.src = plans[j].x;
+      cj.dst = plans[j].packed;
+      cj.scale = plans[j].scale;
+      cj.zp = plans[j].zp;
+      cj.shift = plans[j].shift;
+      t.job[t.n] = cj;
+      t.nvec[t.n] = plans[j].nvec;
+      chunks += c;
+      t.chunk_end[t.n] = (uint32_t)chunks;
+      ++t.n;
+      done[j] = 1;
+    }
+    flush();
+  }
+  return check_launch(what);
 }
 
 }  // namespace ctmi
@@ -154,39 +391,28 @@ using namespace ctmi;
 
 extern "C" int ctmi_observe_pack_quantized_supported(int32_t x_dtype, int64_t rows, int64_t cols,
                                                      int64_t blk_cols, int32_t num_bits) {
-  if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16 && x_dtype != CTMI_F32) return 0;
-  if (num_bits != 4 && num_bits != 8) return 0;
-  if (rows < 1 || cols < 1 || blk_cols < 1) return 0;
-  const int64_t seg = blk_cols < cols ? blk_cols : cols;
-  if (seg % 8 || cols % seg) return 0;
-  return seg / 8 <= kObservePackMaxItems;
+  return op_supported(x_dtype, rows, cols, blk_cols, num_bits) ? 1 : 0;
+}
+
+extern "C" int ctmi_observe_pack_quantized_many(const ctmi_observe_pack_job* jobs, int64_t n,
+                                                void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  std::vector<OpPlan> plans((size_t)n);
+  for (int64_t i = 0; i < n; ++i) {  // every job is validated before anything is enqueued
+    int rc = plan_observe_pack(jobs[i], &plans[i]);
+    if (rc) return rc;
+  }
+  return run_observe_pack(plans.data(), n, (hipStream_t)stream, "ctmi_observe_pack_quantized_many");
 }
 
 extern "C" int ctmi_observe_pack_quantized(const void* x, int32_t x_dtype, int64_t rows,
                                            int64_t cols, int64_t blk_cols, int32_t num_bits,
                                            int32_t symmetric, int32_t* packed, void* scale,
                                            int8_t* zero_point, void* stream) {
-  CTMI_REQUIRE(rows >= 1 && cols >= 1, CTMI_ERR_VALUE, "cannot observe an empty tensor");
-  CTMI_REQUIRE(blk_cols >= 1, CTMI_ERR_VALUE, "empty cell");
-  QpCfg c;
-  int rc = fill_qpcfg(&c, CTMI_QTYPE_INT, num_bits, symmetric, x_dtype, 0, false, x_dtype, CTMI_I8);
+  const ctmi_observe_pack_job j{x, packed, scale, zero_point, rows, cols, blk_cols, x_dtype,
+                                num_bits, symmetric};
+  OpPlan p;
+  int rc = plan_observe_pack(j, &p);
   if (rc) return rc;
-  CTMI_REQUIRE(x && packed && scale, CTMI_ERR_VALUE, "NULL tensor pointer");
-  CTMI_REQUIRE(ctmi_observe_pack_quantized_supported(x_dtype, rows, cols, blk_cols, num_bits),
-               CTMI_ERR_UNSUPPORTED,
-               "no fused kernel for this layout: run the observer and the compressor separately");
-  CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)packed % (4 * (num_bits / 4)) == 0,
-               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
-  const int64_t seg = blk_cols < cols ? blk_cols : cols;
-  const ObservePackOut o{packed, scale, zero_point};
-  hipStream_t st = (hipStream_t)stream;
-  bool ok;
-#define CTMI_OP_XT(XT)                                                          \
-  (num_bits == 4 ? launch_observe_pack<XT, 4>(x, o, rows, cols, seg, c, st)     \
-                 : launch_observe_pack<XT, 8>(x, o, rows, cols, seg, c, st))
-  ok = x_dtype == CTMI_BF16 ? CTMI_OP_XT(BF16)
-                            : (x_dtype == CTMI_F16 ? CTMI_OP_XT(F16) : CTMI_OP_XT(F32));
-#undef CTMI_OP_XT
-  CTMI_REQUIRE(ok, CTMI_ERR_UNSUPPORTED, "no fused kernel for this layout");
-  return check_launch("ctmi_observe_pack_quantized");
+  return run_observe_pack(&p, 1, (hipStream_t)stream, "ctmi_observe_pack_quantized");
 }

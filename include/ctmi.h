@@ -280,9 +280,21 @@ int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows, int64_t c
  * blk_cols] in x_dtype.  zero_point: optional int8 [rows, cols / blk_cols]
  * (unpacked; asymmetric schemes pack it with ctmi_pack_to_int32, packed_dim 0).
  * ctmi_observe_pack_quantized_supported() says whether the layout has a kernel
- * (cells of up to 16384 elements in multiples of 8 that tile the rows). */
+ * (groups of 8, 16, ... 512 elements that tile the rows, or one cell per row of
+ * up to 16384 elements, a multiple of 8). */
+typedef struct ctmi_observe_pack_job {
+  const void* x;
+  int32_t* packed;
+  void* scale;
+  int8_t* zero_point; /* optional */
+  int64_t rows, cols, blk_cols;
+  int32_t x_dtype, num_bits, symmetric;
+} ctmi_observe_pack_job;
 int ctmi_observe_pack_quantized_supported(int32_t x_dtype, int64_t rows, int64_t cols,
                                           int64_t blk_cols, int32_t num_bits);
+/* every weight of a state dict in one call: the group layouts share launches,
+ * eight weights at a time */
+int ctmi_observe_pack_quantized_many(const ctmi_observe_pack_job* jobs, int64_t n, void* stream);
 int ctmi_observe_pack_quantized(const void* x, int32_t x_dtype, int64_t rows, int64_t cols,
                                 int64_t blk_cols, int32_t num_bits, int32_t symmetric,
                                 int32_t* packed, void* scale, int8_t* zero_point, void* stream);

@@ -118,7 +118,10 @@ ONE_SHOT = [
     (dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=128), (77, 512), torch.bfloat16, True),
     (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (33, 96), torch.float16, True),
     (dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=64), (32, 256), torch.float32, True),
-    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=24), (16, 48), torch.bfloat16, True),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=24), (16, 48), torch.bfloat16, False),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=512), (9, 2048), torch.float16, True),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=8), (700, 1504), torch.bfloat16, True),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (40, 256), torch.float32, True),
     (dict(num_bits=4, type="int", symmetric=True, strategy="channel"), (64, 520), torch.bfloat16, True),
     (dict(num_bits=4, type="int", symmetric=False, strategy="channel"), (19, 4096), torch.float16, True),
     (dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (5, 14336), torch.bfloat16, True),
@@ -176,6 +179,41 @@ def test_observe_and_compress_in_one_pass(spec, shape, dtype, fused, gpu):
         gz = o_unpack(got["weight_zero_point"].cpu(), spec["num_bits"], torch.Size((rows, n_cells)), packed_dim=0)
         wz = o_unpack(want["weight_zero_point"], spec["num_bits"], torch.Size((rows, n_cells)), packed_dim=0)
         assert torch.equal(gz[~bad_cells], wz[~bad_cells]), "zero points"
+
+
+def test_observed_weight_batch_matches_single_calls(gpu):
+    """a state dict's worth of weights through one ctmi_observe_pack_quantized_many call
+    (mixed schemes and dtypes, more weights of one kind than a launch takes) gives what
+    the per-weight calls give"""
+    from compressed_tensors_amd.compressors import BaseCompressor, ObservedWeightBatch
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    announce("observed weight batch")
+    g = torch.Generator().manual_seed(8)
+    sym = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    asym = QuantizationArgs(num_bits=4, type="int", symmetric=False, strategy="group", group_size=64)
+    chan = QuantizationArgs(num_bits=8, type="int", symmetric=True, strategy="channel")
+    entries = []
+    for i in range(11):
+        entries.append(dict(weight=(torch.randn(24 + 8 * i, 1024, generator=g) * 0.02).bfloat16(),
+                            quantization_args=sym))
+    entries.insert(3, dict(weight=(torch.randn(40, 512, generator=g) * 0.02).half(), quantization_args=asym))
+    entries.insert(7, dict(weight=(torch.randn(9, 2056, generator=g) * 0.02).bfloat16(), quantization_args=chan))
+    entries.append(dict(weight=(torch.randn(1100, 128, generator=g) * 0.02).bfloat16(), quantization_args=sym))
+    for e in entries:
+        e["weight"] = e["weight"].to(gpu)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    batch = ObservedWeightBatch(entries)
+    for _ in range(2):  # buffers are reused
+        got = batch.compress()
+    for e, d in zip(entries, got):
+        want = comp.observe_and_compress_weight(e["weight"], e["quantization_args"])
+        assert set(d) == set(want)
+        for k in want:
+            assert_bit_equal(d[k], want[k], k)
+    with pytest.raises(NotImplementedError):
+        ObservedWeightBatch([dict(weight=entries[0]["weight"], quantization_args=QuantizationArgs(
+            num_bits=4, type="int", symmetric=True, strategy="tensor"))])
 
 
 def test_pack_quantized_state_dict_and_g_idx(gpu):
