@@ -33,16 +33,36 @@ struct DynOut {
   void* zp;     // optional
 };
 
+// scale and zero point of a cell from its min / max (float path) -- the caller has
+// folded NaNs into has_nan
+template <typename FT, int QK, bool SYM>
+__device__ __forceinline__ void cell_qparams(float lo, float hi, bool has_nan, float qmin,
+                                             float qmax, float* sv, float* zv) {
+  if constexpr (SYM) {
+    *sv = symmetric_scale<FT>(__builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f), has_nan,
+                              (qmax - qmin) * 0.5f);
+    *zv = 0.0f;  // zeros whatever the data holds
+  } else {
+    asymmetric_qparams<FT, QK>(lo, hi, has_nan, qmin, qmax, sv, zv);
+  }
+}
+
+__device__ __forceinline__ void store_cell(const DynOut& o, int64_t cell, float sv, float zv,
+                                           int scale_dtype, int zp_dtype) {
+  if (o.scale) store_from_f32(o.scale, scale_dtype, cell, sv);
+  if (o.zp) store_from_f32(o.zp, zp_dtype, cell, zv);
+}
+
 // One workgroup of 256 threads per row-long segment (token / channel) of up to
 // 256 * U vectors of 8 elements: every vector is loaded before anything is looked
-// at; the four wavefronts meet once, over 8 floats in LDS.
-template <typename FT, int QK, int U>
+// at; the four wavefronts meet once, over a few words in LDS.
+template <typename FT, int QK, bool SYM, int U>
 __global__ void __launch_bounds__(256)
 dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __restrict__ out,
                     DynOut o, int items, QpCfg c) {
   using FR = typename FT::raw;
   __shared__ float part_lo[4], part_hi[4];
-  __shared__ int part_nan[4];
+  __shared__ int part_word[4];
   const int64_t s = blockIdx.x;
   const FR* p = x + s * (int64_t)items * 8;
   Vec<FR, 8> a[U];
@@ -51,28 +71,42 @@ dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
     const int i = k * 256 + threadIdx.x;
     a[k] = ldg_nt<FR, 8>(p + (int64_t)(i < items ? i : items - 1) * 8);  // re-reads do not change min / max
   }
-  float lo = __builtin_inff(), hi = -__builtin_inff();
-  bool unordered = false;
-#pragma unroll
-  for (int k = 0; k < U; ++k) vec_minmax<FT>(a[k], &lo, &hi, &unordered);
-  group_minmax(64, &lo, &hi);
-  unordered = group_any(64, unordered);
-  if ((threadIdx.x & 63) == 0) {
-    part_lo[threadIdx.x >> 6] = lo;
-    part_hi[threadIdx.x >> 6] = hi;
-    part_nan[threadIdx.x >> 6] = unordered;
-  }
-  __syncthreads();
-  lo = __builtin_fminf(__builtin_fminf(part_lo[0], part_lo[1]), __builtin_fminf(part_lo[2], part_lo[3]));
-  hi = __builtin_fmaxf(__builtin_fmaxf(part_hi[0], part_hi[1]), __builtin_fmaxf(part_hi[2], part_hi[3]));
-  if (part_nan[0] | part_nan[1] | part_nan[2] | part_nan[3]) lo = hi = __builtin_nanf("");
   float sv, zv;
-  qparams_value<FT::id>(lo, hi, 1.0f, c, &sv, &zv);
-  zv = stored_zero_point(zv, c);
-  if (threadIdx.x == 0) {
-    if (o.scale) store_from_f32(o.scale, c.scale_dtype, s, sv);
-    if (o.zp) store_from_f32(o.zp, c.zp_dtype, s, zv);
+  if constexpr (SYM && sizeof(FR) == 2) {
+    uint32_t m = 0;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t mk = absmax8_bits<FT>(a[k]);
+      m = mk > m ? mk : m;
+    }
+    m = group_umax(64, m);
+    if ((threadIdx.x & 63) == 0) part_word[threadIdx.x >> 6] = (int)m;
+    __syncthreads();
+    const uint32_t m01 = max((uint32_t)part_word[0], (uint32_t)part_word[1]);
+    const uint32_t m23 = max((uint32_t)part_word[2], (uint32_t)part_word[3]);
+    m = max(m01, m23);
+    constexpr uint32_t kInf = FT::id == CTMI_BF16 ? 0x7f80u : 0x7c00u;
+    sv = symmetric_scale<FT>(FT::to_f32((FR)m), m > kInf, (c.bit_max - c.bit_min) * 0.5f);
+    zv = 0.0f;
+  } else {
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    bool unordered = false;
+#pragma unroll
+    for (int k = 0; k < U; ++k) vec_minmax<FT>(a[k], &lo, &hi, &unordered);
+    group_minmax(64, &lo, &hi);
+    unordered = group_any(64, unordered);
+    if ((threadIdx.x & 63) == 0) {
+      part_lo[threadIdx.x >> 6] = lo;
+      part_hi[threadIdx.x >> 6] = hi;
+      part_word[threadIdx.x >> 6] = unordered;
+    }
+    __syncthreads();
+    lo = __builtin_fminf(__builtin_fminf(part_lo[0], part_lo[1]), __builtin_fminf(part_lo[2], part_lo[3]));
+    hi = __builtin_fmaxf(__builtin_fmaxf(part_hi[0], part_hi[1]), __builtin_fmaxf(part_hi[2], part_hi[3]));
+    unordered = (part_word[0] | part_word[1] | part_word[2] | part_word[3]) != 0;
+    cell_qparams<FT, QK, SYM>(lo, hi, unordered, c.bit_min, c.bit_max, &sv, &zv);
   }
+  if (threadIdx.x == 0) store_cell(o, s, sv, zv, c.scale_dtype, c.zp_dtype);
   FR* q = out + s * (int64_t)items * 8;
 #pragma unroll
   for (int k = 0; k < U; ++k) {
@@ -86,7 +120,7 @@ dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
 
 // Segments of L vectors, L a power of two <= 64 (group strategies): L neighbouring
 // lanes own a segment; memory is one run of vectors numbered like the segments.
-template <typename FT, int QK>
+template <typename FT, int QK, bool SYM>
 __global__ void __launch_bounds__(256)
 dynamic_flat_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __restrict__ out,
                     DynOut o, int64_t nvec, int L, QpCfg c) {
@@ -102,18 +136,20 @@ dynamic_flat_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int64_t v = v0 + k * 256;
-    float lo = __builtin_inff(), hi = -__builtin_inff();
-    bool unordered = false;
-    vec_minmax<FT>(a[k], &lo, &hi, &unordered);
-    group_minmax(L, &lo, &hi);
-    if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
     float sv, zv;
-    qparams_value<FT::id>(lo, hi, 1.0f, c, &sv, &zv);
-    zv = stored_zero_point(zv, c);
-    if (v < nvec && (threadIdx.x & (L - 1)) == 0) {
-      if (o.scale) store_from_f32(o.scale, c.scale_dtype, v / L, sv);
-      if (o.zp) store_from_f32(o.zp, c.zp_dtype, v / L, zv);
+    if constexpr (SYM && sizeof(FR) == 2) {
+      const uint32_t m = group_umax(L, absmax8_bits<FT>(a[k]));
+      constexpr uint32_t kInf = FT::id == CTMI_BF16 ? 0x7f80u : 0x7c00u;
+      sv = symmetric_scale<FT>(FT::to_f32((FR)m), m > kInf, (c.bit_max - c.bit_min) * 0.5f);
+      zv = 0.0f;
+    } else {
+      float lo = __builtin_inff(), hi = -__builtin_inff();
+      bool unordered = false;
+      vec_minmax<FT>(a[k], &lo, &hi, &unordered);
+      group_minmax(L, &lo, &hi);
+      cell_qparams<FT, QK, SYM>(lo, hi, group_any(L, unordered), c.bit_min, c.bit_max, &sv, &zv);
     }
+    if (v < nvec && (threadIdx.x & (L - 1)) == 0) store_cell(o, v / L, sv, zv, c.scale_dtype, c.zp_dtype);
     Vec<FR, 8> of;
     Vec<uint8_t, 8> oc;
     qdq_vec8<FT, kKindFloat, kKindFloat, QK, true>(a[k], oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
@@ -121,7 +157,7 @@ dynamic_flat_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
   }
 }
 
-template <typename FT, int QK>
+template <typename FT, int QK, bool SYM>
 static bool launch_dynamic(const void* x, void* out, const DynOut& o, int64_t rows, int64_t cols,
                            int64_t blk_cols, const QpCfg& c, hipStream_t st) {
   using FR = typename FT::raw;
@@ -131,13 +167,13 @@ static bool launch_dynamic(const void* x, void* out, const DynOut& o, int64_t ro
   if (items <= 64 && (items & (items - 1)) == 0) {
     const int64_t blocks = cdiv(nvec, 256 * 2);
     if (blocks >= (1ll << 31)) return false;
-    hipLaunchKernelGGL((dynamic_flat_kernel<FT, QK>), (unsigned)blocks, 256, 0, st, (const FR*)x,
+    hipLaunchKernelGGL((dynamic_flat_kernel<FT, QK, SYM>), (unsigned)blocks, 256, 0, st, (const FR*)x,
                        (FR*)out, o, nvec, (int)items, c);
     return true;
   }
   if (n_segments >= (1ll << 31)) return false;
 #define CTMI_DYN(UU)                                                                    \
-  hipLaunchKernelGGL((dynamic_rows_kernel<FT, QK, UU>), (unsigned)n_segments, 256, 0, st, \
+  hipLaunchKernelGGL((dynamic_rows_kernel<FT, QK, SYM, UU>), (unsigned)n_segments, 256, 0, st, \
                      (const FR*)x, (FR*)out, o, (int)items, c)
   if (items <= 256) CTMI_DYN(1);
   else if (items <= 256 * 2) CTMI_DYN(2);
@@ -193,11 +229,13 @@ extern "C" int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64
                            c, st);
   } else {
     const int qk = qtype == CTMI_QTYPE_INT ? 0 : 1;
-#define CTMI_DYN_FT(FT)                                                                  \
-  (qk == 0 ? launch_dynamic<FT, 0>(x, out, o, rows, cols, blk_cols, c, st)              \
-           : launch_dynamic<FT, 1>(x, out, o, rows, cols, blk_cols, c, st))
+#define CTMI_DYN_SYM(FT, QK)                                                               \
+  (symmetric ? launch_dynamic<FT, QK, true>(x, out, o, rows, cols, blk_cols, c, st)        \
+             : launch_dynamic<FT, QK, false>(x, out, o, rows, cols, blk_cols, c, st))
+#define CTMI_DYN_FT(FT) (qk == 0 ? CTMI_DYN_SYM(FT, 0) : CTMI_DYN_SYM(FT, 1))
     ok = x_dtype == CTMI_BF16 ? CTMI_DYN_FT(BF16)
                               : (x_dtype == CTMI_F16 ? CTMI_DYN_FT(F16) : CTMI_DYN_FT(F32));
+#undef CTMI_DYN_SYM
 #undef CTMI_DYN_FT
   }
   CTMI_REQUIRE(ok, CTMI_ERR_UNSUPPORTED, "no fused kernel for this layout");

@@ -52,4 +52,42 @@ __device__ __forceinline__ bool group_any(int L, bool flag) {
   return (m & group) != 0;
 }
 
+// ------------------------------------------------------------------ |x| maximum on the raw bits
+// For a symmetric scheme only max|x| matters (helpers.py:87-110 with min <= 0 <= max:
+// max(|min|, |max|) = max|x|).  The magnitude bits of a 16-bit float order like
+// unsigned integers, NaNs above infinity, so two elements go through one packed
+// integer maximum and a NaN shows in the result by itself.
+typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+
+template <typename XT>
+__device__ __forceinline__ uint32_t absmax8_bits(const Vec<typename XT::raw, 8>& a) {
+  static_assert(sizeof(typename XT::raw) == 2, "16-bit floats only");
+  const Vec<uint32_t, 4> w = __builtin_bit_cast(Vec<uint32_t, 4>, a);
+  u16x2_t m[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) m[j] = __builtin_bit_cast(u16x2_t, w.v[j] & 0x7fff7fffu);
+  const u16x2_t r = __builtin_elementwise_max(__builtin_elementwise_max(m[0], m[1]),
+                                              __builtin_elementwise_max(m[2], m[3]));
+  return r.x > r.y ? (uint32_t)r.x : (uint32_t)r.y;
+}
+
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_umax_step(uint32_t v) {
+  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
+  return o > v ? o : v;
+}
+
+// all-reduce over aligned groups of L lanes (L a power of two <= 64)
+__device__ __forceinline__ uint32_t group_umax(int L, uint32_t v) {
+  if (L >= 2) v = dpp_umax_step<0xB1>(v);
+  if (L >= 4) v = dpp_umax_step<0x4E>(v);
+  if (L >= 8) v = dpp_umax_step<0x141>(v);
+  if (L >= 16) v = dpp_umax_step<0x140>(v);
+  for (int d = 16; d < L; d <<= 1) {
+    const uint32_t o = (uint32_t)__shfl_xor((int)v, d, kWave);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
 }  // namespace ctmi

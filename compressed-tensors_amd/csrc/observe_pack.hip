@@ -24,87 +24,6 @@
 
 namespace ctmi {
 
-constexpr float kScaleFloor = 1.1920928955078125e-07f;  // torch.finfo(torch.float32).eps
-
-// ------------------------------------------------------------------ |x| maximum on the raw bits
-// For a symmetric scheme only max|x| matters (helpers.py:87-110 with min <= 0 <= max:
-// max(|min|, |max|) = max|x|).  The magnitude bits of a 16-bit float order like
-// unsigned integers, NaNs above infinity, so two elements go through one packed
-// integer maximum and a NaN shows in the result by itself.
-typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
-
-template <typename XT>
-__device__ __forceinline__ uint32_t absmax8_bits(const Vec<typename XT::raw, 8>& a) {
-  static_assert(sizeof(typename XT::raw) == 2, "16-bit floats only");
-  const Vec<uint32_t, 4> w = __builtin_bit_cast(Vec<uint32_t, 4>, a);
-  u16x2_t m[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) m[j] = __builtin_bit_cast(u16x2_t, w.v[j] & 0x7fff7fffu);
-  const u16x2_t r = __builtin_elementwise_max(__builtin_elementwise_max(m[0], m[1]),
-                                              __builtin_elementwise_max(m[2], m[3]));
-  return r.x > r.y ? (uint32_t)r.x : (uint32_t)r.y;
-}
-
-template <int CTRL>
-__device__ __forceinline__ uint32_t dpp_umax_step(uint32_t v) {
-  const uint32_t o = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false);
-  return o > v ? o : v;
-}
-
-// all-reduce over aligned groups of L lanes (L a power of two <= 64)
-__device__ __forceinline__ uint32_t group_umax(int L, uint32_t v) {
-  if (L >= 2) v = dpp_umax_step<0xB1>(v);
-  if (L >= 4) v = dpp_umax_step<0x4E>(v);
-  if (L >= 8) v = dpp_umax_step<0x141>(v);
-  if (L >= 16) v = dpp_umax_step<0x140>(v);
-  for (int d = 16; d < L; d <<= 1) {
-    const uint32_t o = (uint32_t)__shfl_xor((int)v, d, kWave);
-    v = o > v ? o : v;
-  }
-  return v;
-}
-
-// ------------------------------------------------------------------ scale and zero point of a group
-// calculate_qparams for an integer scheme with min / max in XT, the dtype dispatch
-// and the scheme dispatch of the general routine resolved at compile time.
-template <typename XT>
-__device__ __forceinline__ float round_xt(float v) {
-  float same = v;
-  round2<XT::id>(v, same);
-  return v;
-}
-
-// symmetric: scale = max(XT(max|x| / (range / 2)), eps)
-template <typename XT>
-__device__ __forceinline__ float symmetric_scale(float absmax, bool has_nan, float half_range) {
-  float t;
-  if constexpr (XT::id == CTMI_BF16) {
-    // bf16 / bf16 (7.5 and 127.5 are bf16 values): the product with the reciprocal
-    // rounds to the same bf16 as the quotient
-    t = absmax * __builtin_amdgcn_rcpf(half_range);
-  } else {
-    t = absmax / half_range;
-  }
-  const float s = __builtin_fmaxf(round_xt<XT>(t), kScaleFloor);
-  return has_nan ? __builtin_nanf("") : s;
-}
-
-// asymmetric: scale = max(XT(XT(max - min) / range), eps),
-//             zp = round(clamp(XT(qmin - XT(min / scale)), qmin, qmax))
-template <typename XT>
-__device__ __forceinline__ void asymmetric_qparams(float lo, float hi, bool has_nan, float qmin,
-                                                   float qmax, float* scale, float* zp) {
-  const float mn = __builtin_fminf(lo, 0.0f), mx = __builtin_fmaxf(hi, 0.0f);
-  float s = round_xt<XT>(round_xt<XT>(mx - mn) / (qmax - qmin));
-  s = (s != s) ? s : __builtin_fmaxf(s, kScaleFloor);  // inf - inf
-  float z = round_xt<XT>(qmin - round_xt<XT>(mn / s));
-  z = (z != z) ? z : __builtin_fminf(__builtin_fmaxf(z, qmin), qmax);
-  z = rintf(z) + 0.0f;  // an int8 zero point has no -0
-  const float nan = __builtin_nanf("");
-  *scale = has_nan ? nan : s;
-  *zp = has_nan ? nan : z;
-}
-
 // ------------------------------------------------------------------ groups within a row
 constexpr int kOpBlock = 512, kOpUnroll = 2;
 
@@ -152,7 +71,7 @@ __global__ void __launch_bounds__(kOpBlock) observe_pack_groups_kernel(const Cha
           const float m = __builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f);
           sv = symmetric_scale<XT>(m, unordered, (t.qmax - t.qmin) * 0.5f);
         } else {
-          asymmetric_qparams<XT>(lo, hi, unordered, t.qmin, t.qmax, &sv, &zv);
+          asymmetric_qparams<XT, 0>(lo, hi, unordered, t.qmin, t.qmax, &sv, &zv);
         }
       }
       if ((!GUARD || v < nvec) && (threadIdx.x & (L - 1)) == 0) {
@@ -207,7 +126,7 @@ observe_pack_rows_kernel(const typename XT::raw* __restrict__ x, int32_t* __rest
     sv = symmetric_scale<XT>(__builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f), unordered,
                              (qmax - qmin) * 0.5f);
   } else {
-    asymmetric_qparams<XT>(lo, hi, unordered, qmin, qmax, &sv, &zv);
+    asymmetric_qparams<XT, 0>(lo, hi, unordered, qmin, qmax, &sv, &zv);
   }
   if (threadIdx.x == 0) {
     scale[s] = XT::from_f32(sv);

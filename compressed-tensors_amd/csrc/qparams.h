@@ -3,6 +3,7 @@
 #pragma once
 
 #include "ctmi_device.h"
+#include "qdq_core.h"
 
 namespace ctmi {
 
@@ -64,6 +65,55 @@ __device__ __forceinline__ void qparams_value(float mn, float mx, float gs, cons
 // rounds it, an integer dtype has no -0 (rint of a small negative value gives one).
 __device__ __forceinline__ float stored_zero_point(float z, const QpCfg& c) {
   return c.qtype == CTMI_QTYPE_INT ? z + 0.0f : round_to(z, c.zp_dtype);
+}
+
+// ------------------------------------------------------------------ compile-time forms
+// calculate_qparams for an int or fp8 scheme without a global scale, min / max in
+// XT, with the dtype and scheme dispatch of qparams_value resolved at compile time
+// and the NaN bookkeeping left to the caller (has_nan: the cell holds a NaN).
+constexpr float kScaleFloor = 1.1920928955078125e-07f;  // torch.finfo(torch.float32).eps
+
+template <typename XT>
+__device__ __forceinline__ float round_xt(float v) {
+  float same = v;
+  round2<XT::id>(v, same);
+  return v;
+}
+
+// symmetric: scale = max(XT(max|x| / (range / 2)), eps)
+template <typename XT>
+__device__ __forceinline__ float symmetric_scale(float absmax, bool has_nan, float half_range) {
+  float t;
+  if constexpr (XT::id == CTMI_BF16) {
+    // bf16 / bf16 (7.5, 127.5 and 448 are bf16 values): the product with the
+    // reciprocal rounds to the same bf16 as the quotient
+    t = absmax * __builtin_amdgcn_rcpf(half_range);
+  } else {
+    t = absmax / half_range;
+  }
+  const float s = __builtin_fmaxf(round_xt<XT>(t), kScaleFloor);
+  return has_nan ? __builtin_nanf("") : s;
+}
+
+// asymmetric: scale = max(XT(XT(max - min) / range), eps),
+//             zp = clamp(XT(qmin - XT(min / scale)), qmin, qmax), rounded to an integer
+// (QK 0, stored as int8) or to fp8 (QK 1), as quantize / dequantize read it back
+template <typename XT, int QK>
+__device__ __forceinline__ void asymmetric_qparams(float lo, float hi, bool has_nan, float qmin,
+                                                   float qmax, float* scale, float* zp) {
+  const float mn = __builtin_fminf(lo, 0.0f), mx = __builtin_fmaxf(hi, 0.0f);
+  float s = round_xt<XT>(round_xt<XT>(mx - mn) / (qmax - qmin));
+  s = (s != s) ? s : __builtin_fmaxf(s, kScaleFloor);  // inf - inf
+  float z = round_xt<XT>(qmin - round_xt<XT>(mn / s));
+  z = (z != z) ? z : __builtin_fminf(__builtin_fmaxf(z, qmin), qmax);
+  if constexpr (QK == 0) {
+    z = rintf(z) + 0.0f;  // an int8 zero point has no -0
+  } else {
+    if (z == z) z = __builtin_amdgcn_cvt_f32_fp8(__builtin_amdgcn_cvt_pk_fp8_f32(z, z, 0, false), 0);
+  }
+  const float nan = __builtin_nanf("");
+  *scale = has_nan ? nan : s;
+  *zp = has_nan ? nan : z;
 }
 
 }  // namespace ctmi
