@@ -403,13 +403,17 @@ bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dty
 // global scale, min / max in XT: scale = fp8(clamp(gs * XT(max|x| / 6), +-448)),
 // zero replaced by 0.125.  Returns the fp8 code, *sv = its value.
 template <typename XT>
-__device__ __forceinline__ uint8_t nvfp4_group_scale(float lo, float hi, bool has_nan, float gs,
+__device__ __forceinline__ uint8_t nvfp4_group_scale(float absmax, bool has_nan, float gs,
                                                      float* sv) {
-  // max(|min(lo, 0)|, |max(hi, 0)|)
-  const float m = __builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f);
-  float t = m / 6.0f, same = t;
-  round2<XT::id>(t, same);
-  float s = gs * t;
+  float t;
+  if constexpr (XT::id == CTMI_BF16) {
+    // bf16 / bf16 (6 is a bf16 value): the product with the reciprocal rounds to
+    // the same bf16 as the quotient
+    t = absmax * 0.16666667163372039794921875f;
+  } else {
+    t = absmax / 6.0f;
+  }
+  float s = gs * round_xt<XT>(t);
   has_nan |= s != s;  // inf * 0
   s = __builtin_fminf(__builtin_fmaxf(s, -448.0f), 448.0f);
   uint32_t code = (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(s, s, 0, false) & 0xffu;
@@ -447,12 +451,21 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
-    float lo = __builtin_inff(), hi = -__builtin_inff();
-    bool unordered = false;
-    vec_minmax<XT>(xv[k], &lo, &hi, &unordered);
-    group_minmax(2, &lo, &hi);
     float sv;
-    const uint8_t code = nvfp4_group_scale<XT>(lo, hi, group_any(2, unordered), gs, &sv);
+    uint8_t code;
+    if constexpr (sizeof(typename XT::raw) == 2) {
+      const uint32_t m = group_umax(2, absmax8_bits<XT>(xv[k]));
+      constexpr uint32_t kInf = XT::id == CTMI_BF16 ? 0x7f80u : 0x7c00u;
+      code = nvfp4_group_scale<XT>(XT::to_f32((typename XT::raw)m), m > kInf, gs, &sv);
+    } else {
+      float lo = __builtin_inff(), hi = -__builtin_inff();
+      bool unordered = false;
+      vec_minmax<XT>(xv[k], &lo, &hi, &unordered);
+      group_minmax(2, &lo, &hi);
+      // max(|min(lo, 0)|, |max(hi, 0)|)
+      code = nvfp4_group_scale<XT>(__builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f),
+                                   group_any(2, unordered), gs, &sv);
+    }
     if (v < nvec && (threadIdx.x & 1) == 0) {
       if (scale_out) scale_out[v >> 1] = code;
       if (zp_out) zp_out[v >> 1] = 0;  // fp8 zero
@@ -462,10 +475,7 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
     fp4_unpack8_hw(nvfp4_codes<XT, true>(xv[k], s, 0.0f), t);
     Vec<typename XT::raw, 8> o;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float xi = XT::to_f32(xv[k].v[i]);
-      o.v[i] = XT::from_f32(xi != xi ? xi : t[i] * s);
-    }
+    for (int i = 0; i < 8; ++i) o.v[i] = XT::from_f32(t[i] * s);  // a NaN in the group made s NaN
     if (v < nvec) stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
   }
 }
