@@ -11,5 +11,6 @@ from compressed_tensors_amd.config import *  # noqa: F401,F403
 from compressed_tensors_amd.quantization import *  # noqa: F401,F403
 from compressed_tensors_amd.utils import *  # noqa: F401,F403
 from compressed_tensors_amd.compressors import *  # noqa: F401,F403
+from compressed_tensors_amd.linear import *  # noqa: F401,F403
 
 __version__ = "0.1.0"

@@ -2,3 +2,4 @@ from .quant_args import *  # noqa: F401,F403
 from .quant_scheme import *  # noqa: F401,F403
 from .helpers import *  # noqa: F401,F403
 from .forward import *  # noqa: F401,F403
+from .initialize import *  # noqa: F401,F403

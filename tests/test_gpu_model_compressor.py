@@ -134,3 +134,66 @@ def test_fp8_plus_sparse24_stack(gpu):
         codes = op.naive_compress(w, s, oargs, zero_point=z)
         dense = op.naive_decompress({"weight": codes, "weight_scale": s})
         assert_bit_equal(model.get_submodule(name).weight.data, dense, f"{name} decompressed")
+
+
+@pytest.mark.parametrize("fmt,spec,dtype", [
+    ("pack-quantized", dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), torch.bfloat16),
+    ("pack-quantized", dict(num_bits=4, type="int", symmetric=False, strategy="channel"), torch.float16),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), torch.bfloat16),
+    ("nvfp4-pack-quantized", dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16), torch.bfloat16),
+], ids=["w4a16", "w4a16-asym-channel", "fp8", "nvfp4"])
+def test_compressed_linear_runs_from_compressed_parameters(fmt, spec, dtype, gpu):
+    """CompressedLinear.from_linear gives empty parameters of the compressed shapes;
+    filled from a compressed state dict, the first forward decompresses (on the GPU)
+    and every forward equals a Linear holding the oracle's decompressed weight"""
+    from compressed_tensors_amd import CompressedLinear
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.config import QuantizationStatus
+    from compressed_tensors_amd.quantization import QuantizationArgs, QuantizationScheme
+
+    announce("CompressedLinear", fmt, spec, dtype)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    g = torch.Generator().manual_seed(12)
+    w = (torch.randn(96, 256, generator=g) * 0.02).to(dtype)
+    bias = torch.randn(96, generator=g).to(dtype)
+    gs = None
+    if spec["strategy"] == "tensor_group":
+        gs = oq.generate_gparam(*[t.reshape(1) for t in torch.aminmax(w)])
+    scale, zp = oq.observe_weight(w, oargs, global_scale=gs)
+    if fmt == "pack-quantized":
+        compressed = op.pack_quantized_compress(w, scale, oargs, zero_point=zp)
+        compressed["weight_scale"] = scale
+        dense = op.pack_quantized_decompress(dict(compressed), oargs)
+    elif fmt == "float-quantized":
+        compressed = dict(weight=op.naive_compress(w, scale, oargs, zero_point=zp), weight_scale=scale)
+        dense = op.naive_decompress(dict(compressed))
+    else:
+        compressed = {"weight_packed": op.nvfp4_compress(w, scale, gs, oargs), "weight_scale": scale,
+                      "weight_global_scale": gs}
+        dense = op.nvfp4_decompress(compressed["weight_packed"], scale, gs)
+
+    layer = torch.nn.Linear(256, 96, bias=True).to(dtype).to(gpu)
+    layer.bias.data.copy_(bias)
+    scheme = QuantizationScheme(targets=["Linear"], weights=args)
+    with pytest.warns(UserWarning):
+        CompressedLinear(4, 4)
+    module = CompressedLinear.from_linear(layer, scheme, fmt)
+    assert isinstance(module, CompressedLinear) and module is layer
+    assert module.quantization_status == QuantizationStatus.COMPRESSED
+    info = BaseCompressor.load_from_registry(fmt).compression_param_info(w.shape, args)
+    assert ("weight" in info) == hasattr(module, "weight")  # the naive formats keep the name
+    for name, (shape, pdtype) in info.items():
+        p = getattr(module, name)
+        assert tuple(p.shape) == tuple(shape) and p.dtype == pdtype and p.device.type == "cuda"
+    assert module.weight_scale.shape == scale.shape and module.weight_scale.dtype == scale.dtype
+    for name, value in compressed.items():  # what loading a checkpoint does
+        assert tuple(getattr(module, name).shape) == tuple(value.shape), name
+        getattr(module, name).data.copy_(value.to(gpu))
+
+    x = torch.randn(5, 256, generator=g).to(dtype).to(gpu)
+    want = torch.nn.functional.linear(x, dense.to(dtype).to(gpu), bias.to(gpu))
+    for _ in range(2):
+        got = module(x)
+        assert module.quantization_status == QuantizationStatus.FROZEN
+        assert_bit_equal(got, want.cpu(), "forward")
+    assert_bit_equal(module.weight.data, dense.to(module.weight.dtype), "decompressed weight")
