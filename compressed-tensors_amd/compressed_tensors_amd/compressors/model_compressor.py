@@ -17,6 +17,8 @@ from torch.nn import Module
 
 from compressed_tensors_amd.compressors.base import BaseCompressor
 from compressed_tensors_amd.config import (
+    QUANTIZATION_CONFIG_NAME,
+    SPARSITY_CONFIG_NAME,
     CompressionFormat,
     QuantizationStatus,
     SparsityCompressionConfig,
@@ -136,10 +138,27 @@ class ModelCompressor:
     def decompress(self, model_path, model: Module) -> None:
         """overwrite the weights of `model` with the ones decompressed from a
         safetensors file / directory or from a compressed state dict"""
-        state = (model_path if isinstance(model_path, dict)
-                 else load_safetensors_state_dict(model_path, device="cpu"))
         quant_compressor = (next(iter(self.quantization_compressor.values()))
                             if self.quantization_compressor is not None else None)
+        has_sparsity = (self.sparsity_compressor is not None
+                        and self.sparsity_config.format != CompressionFormat.dense.value)
+        if not isinstance(model_path, dict):
+            first = next(model.parameters(), None)
+            device = str(first.device) if first is not None else "cpu"
+            if quant_compressor is not None and not has_sparsity:
+                # one module at a time, read from the files straight onto the model's device
+                names_to_scheme = map_module_to_scheme(model)
+                for mod_path, data in quant_compressor.decompress(
+                        str(model_path), names_to_scheme=names_to_scheme, device=device):
+                    for param_name, param_data in data.items():
+                        if param_name == "weight" or hasattr(self._module(model, mod_path), param_name):
+                            self._assign(model, f"{mod_path}.{param_name}", param_data)
+                for module in model.modules():
+                    if getattr(module, "quantization_scheme", None) is not None:
+                        module.quantization_status = QuantizationStatus.FROZEN
+                return
+            model_path = load_safetensors_state_dict(model_path, device=device)
+        state = model_path
         if (self.sparsity_compressor is not None
                 and self.sparsity_config.format != CompressionFormat.dense.value):
             skip = quant_compressor.compression_param_names if quant_compressor else None
@@ -156,6 +175,59 @@ class ModelCompressor:
             for module in model.modules():
                 if getattr(module, "quantization_scheme", None) is not None:
                     module.quantization_status = QuantizationStatus.FROZEN
+
+    def update_config(self, save_directory: str) -> None:
+        """write the compression configs into `config.json` under `save_directory`, next
+        to whatever the file already holds (model_compressor.py:769-817)"""
+        import json
+        import os
+
+        import compressed_tensors_amd
+
+        if not any((self.quantization_config, self.sparsity_config, self.transform_config)):
+            return
+        config_file_path = os.path.join(save_directory, "config.json")
+        if os.path.exists(config_file_path):
+            with open(config_file_path, "r") as file:
+                config_data = json.load(file)
+        else:
+            config_data = {}
+        qconfig_data = {}
+        if self.quantization_config is not None:
+            qconfig_data = self.quantization_config.model_dump(exclude=["quant_method"])
+        sconfig_data = self.sparsity_config.model_dump() if self.sparsity_config is not None else {}
+        tconfig_data = {}
+        if self.transform_config is not None and hasattr(self.transform_config, "model_dump"):
+            tconfig_data = self.transform_config.model_dump()
+        config_data[QUANTIZATION_CONFIG_NAME] = {
+            "version": compressed_tensors_amd.__version__,
+            "quant_method": "compressed-tensors",
+            SPARSITY_CONFIG_NAME: sconfig_data,
+            "transform_config": tconfig_data,
+            **qconfig_data,
+        }
+        with open(config_file_path, "w") as config_file:
+            json.dump(config_data, config_file, indent=2, sort_keys=True)
+
+    @classmethod
+    def from_compression_config(cls, compression_config: Optional[Dict]):
+        """a compressor from the `quantization_config` entry of a config.json (the
+        dict form; model_compressor.py:164-206)"""
+        if not compression_config:
+            return None
+        data = dict(compression_config)
+        sparsity = data.pop(SPARSITY_CONFIG_NAME, None) or None
+        data.pop("transform_config", None)
+        data.pop("version", None)
+        sparsity_config = SparsityCompressionConfig(**sparsity) if sparsity else None
+        quantization_config = None
+        if data.get("config_groups"):
+            allowed = ("config_groups", "format", "quantization_status", "global_compression_ratio",
+                       "ignore", "kv_cache_scheme", "quant_method")
+            quantization_config = QuantizationConfig(**{k: v for k, v in data.items() if k in allowed})
+        if sparsity_config is None and quantization_config is None:
+            return None
+        return cls(sparsity_config=sparsity_config, quantization_config=quantization_config)
 
     # ----- in-memory pathways ----- #
     def compress_model(self, model: Module) -> None:

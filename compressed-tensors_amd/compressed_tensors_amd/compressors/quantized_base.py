@@ -15,7 +15,8 @@ from torch import Tensor
 
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
 from compressed_tensors_amd.quantization.quant_args import QuantizationStrategy
-from compressed_tensors_amd.utils.helpers import load_safetensors_state_dict, nest_state_dict
+from compressed_tensors_amd.utils.helpers import nest_state_dict
+from compressed_tensors_amd.utils.safetensors_io import CheckpointReader, get_nested_weight_mappings
 
 __all__ = ["BaseQuantizationCompressor"]
 
@@ -83,11 +84,23 @@ class BaseQuantizationCompressor(BaseCompressor):
         names_to_scheme: Dict[str, Any],
         device: str = "cpu",
     ) -> Generator[Tuple[str, Dict[str, Tensor]], None, None]:
-        if isinstance(path_to_model_or_tensors, (str, Path)):
-            state = load_safetensors_state_dict(path_to_model_or_tensors, device=device)
-        else:
-            state = path_to_model_or_tensors
-        yield from self.decompress_from_state_dict(state, names_to_scheme)
+        if not isinstance(path_to_model_or_tensors, (str, Path)):
+            yield from self.decompress_from_state_dict(path_to_model_or_tensors, names_to_scheme)
+            return
+        # one module at a time: only its compression parameters are in memory
+        # (quantized_compressors/base.py:186-220)
+        path = str(path_to_model_or_tensors)
+        nested = get_nested_weight_mappings(path, self.compression_param_names)
+        with CheckpointReader(path, device=device) as reader:
+            for module_path, params in nested.items():
+                if "weight_scale" not in params:
+                    continue
+                weight_data = {name: reader.get(f"{module_path}.{name}") for name in params}
+                quant_args = names_to_scheme[module_path].weights
+                weight_data["weight"] = self.decompress_weight(
+                    compressed_data=weight_data, quantization_args=quant_args
+                )
+                yield module_path, weight_data
 
     def decompress_from_state_dict(
         self, state_dict: Dict[str, Tensor], names_to_scheme: Dict[str, Any]

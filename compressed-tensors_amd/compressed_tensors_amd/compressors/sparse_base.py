@@ -10,11 +10,8 @@ from typing import Dict, Generator, Optional, Set, Tuple
 from torch import Tensor
 
 from compressed_tensors_amd.compressors.base import BaseCompressor
-from compressed_tensors_amd.utils.helpers import (
-    load_safetensors_state_dict,
-    merge_names,
-    nest_state_dict,
-)
+from compressed_tensors_amd.utils.helpers import merge_names, nest_state_dict
+from compressed_tensors_amd.utils.safetensors_io import CheckpointReader, get_nested_weight_mappings
 
 __all__ = ["BaseSparseCompressor"]
 
@@ -47,18 +44,29 @@ class BaseSparseCompressor(BaseCompressor):
         **kwargs,
     ) -> Generator[Tuple[str, Tensor], None, None]:
         if isinstance(path_to_model_or_tensors, dict):
-            state = path_to_model_or_tensors
-        else:
-            state = load_safetensors_state_dict(path_to_model_or_tensors, device=device)
-        nested, ignored = nest_state_dict(
-            state, self.compression_param_names, return_unmatched_params=True
+            nested, ignored = nest_state_dict(
+                path_to_model_or_tensors, self.compression_param_names, return_unmatched_params=True
+            )
+            for module_path, weight_data in nested.items():
+                yield merge_names(module_path, "weight"), self.decompress_weight(dict(weight_data))
+            for name, value in ignored.items():
+                if params_to_skip_load is not None and any(p in name for p in params_to_skip_load):
+                    continue
+                yield name, value
+            return
+        # one module at a time from the files (sparse_compressors/base.py:114-152)
+        path = str(path_to_model_or_tensors)
+        nested, ignored = get_nested_weight_mappings(
+            path, self.compression_param_names, return_unmatched_params=True
         )
-        for module_path, weight_data in nested.items():
-            yield merge_names(module_path, "weight"), self.decompress_weight(dict(weight_data))
-        for name, value in ignored.items():
-            if params_to_skip_load is not None and any(p in name for p in params_to_skip_load):
-                continue
-            yield name, value
+        with CheckpointReader(path, device=device) as reader:
+            for module_path, params in nested.items():
+                weight_data = {name: reader.get(merge_names(module_path, name)) for name in params}
+                yield merge_names(module_path, "weight"), self.decompress_weight(weight_data)
+            for name in ignored:
+                if params_to_skip_load is not None and any(p in name for p in params_to_skip_load):
+                    continue
+                yield name, reader.get(name)
 
     def decompress_from_state_dict(
         self, state_dict: Dict[str, Tensor]

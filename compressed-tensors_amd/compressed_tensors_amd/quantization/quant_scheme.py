@@ -90,6 +90,21 @@ class QuantizationConfig:
         self.kv_cache_scheme = kv_cache_scheme
         self.quant_method = quant_method
 
+    def model_dump(self, exclude=None) -> Dict[str, Any]:
+        """plain-dict form, as written into a model's config.json"""
+        data = {
+            "config_groups": {name: scheme.model_dump() for name, scheme in self.config_groups.items()},
+            "format": self.format,
+            "quantization_status": getattr(self.quantization_status, "value", self.quantization_status),
+            "global_compression_ratio": self.global_compression_ratio,
+            "ignore": list(self.ignore),
+            "kv_cache_scheme": self.kv_cache_scheme.model_dump() if self.kv_cache_scheme else None,
+            "quant_method": self.quant_method,
+        }
+        for key in exclude or ():
+            data.pop(key, None)
+        return data
+
 
 def _w(**kw) -> Dict[str, QuantizationArgs]:
     return {"weights": QuantizationArgs(**kw)}

@@ -197,3 +197,70 @@ def test_compressed_linear_runs_from_compressed_parameters(fmt, spec, dtype, gpu
         assert module.quantization_status == QuantizationStatus.FROZEN
         assert_bit_equal(got, want.cpu(), "forward")
     assert_bit_equal(module.weight.data, dense.to(module.weight.dtype), "decompressed weight")
+
+
+def test_checkpoint_on_disk_roundtrip(tmp_path, gpu):
+    """compress on the GPU -> stream into a safetensors file (tensors bigger than the
+    staging buffers) + config.json -> a fresh process-side view: the library's own reader
+    sees the same tensors, and decompress(path, model) restores the oracle's weights"""
+    import json
+
+    from safetensors.torch import load_file
+
+    from compressed_tensors_amd.compressors import (
+        ModelCompressor, apply_quantization_scheme, load_compressed, save_compressed,
+    )
+    from compressed_tensors_amd.config import SparsityCompressionConfig
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme,
+    )
+    from compressed_tensors_amd.utils.safetensors_io import save_file
+
+    announce("checkpoint on disk")
+    torch.manual_seed(4)
+    model = Tiny().to(torch.bfloat16).to(gpu)
+    spec = dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=128)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    config = QuantizationConfig(
+        config_groups={"g0": QuantizationScheme(targets=["Linear"], weights=args)},
+        format="pack-quantized", ignore=["lm_head"])
+    apply_quantization_scheme(model, config)
+    cpu = _prepare(model, args, oargs, gpu)
+    mc = ModelCompressor(quantization_config=config)
+    state = mc.compress(model)
+    assert all(t.is_cuda for t in state.values() if t.numel() > 2)
+
+    path = tmp_path / "model.safetensors"
+    save_file(state, str(path), metadata={"format": "pt"}, staging_bytes=4096)  # many pieces per tensor
+    mc.update_config(str(tmp_path))
+    on_disk = load_file(str(path))
+    assert set(on_disk) == set(state)
+    for k, v in state.items():
+        assert_bit_equal(on_disk[k], v.cpu(), k)
+
+    q = json.loads((tmp_path / "config.json").read_text())["quantization_config"]
+    loaded_mc = ModelCompressor.from_compression_config(q)
+    fresh = Tiny().to(torch.bfloat16).to(gpu)
+    apply_quantization_scheme(fresh, loaded_mc.quantization_config)
+    loaded_mc.decompress(str(tmp_path), fresh)
+    for name, (w, s, z) in cpu.items():
+        want = op.pack_quantized_compress(w, s, oargs, zero_point=z)
+        dense = op.pack_quantized_decompress(dict(want, weight_scale=s), oargs)
+        assert_bit_equal(fresh.get_submodule(name).weight.data, dense, f"{name} from disk")
+
+    # the sparse helpers: save_compressed / load_compressed through a file
+    w = torch.randn(64, 96, device=gpu).bfloat16()
+    w = torch.where(torch.rand_like(w.float()) < 0.6, torch.zeros_like(w), w)
+    sparse_path = tmp_path / "sparse.safetensors"
+    save_compressed({"a.weight": w, "b.bias": torch.ones(3, device=gpu)}, sparse_path, "sparse-bitmask")
+    assert set(load_file(str(sparse_path))) == {"a.compressed", "a.bitmask", "a.shape", "a.row_offsets", "b.bias"}
+    back = dict(load_compressed(sparse_path, SparsityCompressionConfig(format="sparse-bitmask"),
+                                device=str(gpu)))
+    assert_bit_equal(back["a.weight"], w.cpu(), "sparse round trip through a file")
+    assert_bit_equal(back["b.bias"], torch.ones(3), "passed through")
+    dense_back = dict(load_compressed(sparse_path, None))
+    assert set(dense_back) == {"a.compressed", "a.bitmask", "a.shape", "a.row_offsets", "b.bias"}
+    with pytest.raises(ValueError):
+        save_compressed({}, sparse_path, "sparse-bitmask")
+    with pytest.raises(ValueError, match="Unknown compression format"):
+        save_compressed({"a.weight": w}, sparse_path, "no-such-format")
