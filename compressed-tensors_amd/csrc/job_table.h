@@ -27,13 +27,14 @@ struct VecJob {
 // What a workgroup needs of its weight, 64 bytes so that one scalar load brings
 // it in.  Scale of item v (8 elements): `v >> shift` when scales are numbered
 // like the items (FLAT), else row r = v / vpr, column block (v - r*vpr) / vpb,
-// index r * s_stride + block (s_stride 0 when all rows share one scale row).
+// index (r >> row_shift) * s_stride + block (s_stride 0 when all rows share one
+// scale row; row_shift > 0 for blocks several rows tall).
 struct alignas(64) ChainJob {
   const void* src;
   void* dst;
   const void* scale;
   const int8_t* zp;
-  uint32_t shift, reserved;
+  uint32_t shift, row_shift;
   uint32_t vpr_d, vpr_m, vpr_s;
   uint32_t vpb_m, vpb_s;
   uint32_t s_stride;
@@ -60,7 +61,7 @@ static inline ChainJob make_chain_job(const VecJob& j) {
   o.scale = j.scale;
   o.zp = j.zp;
   o.shift = j.g.shift;
-  o.reserved = 0;
+  o.row_shift = j.g.row_shift;
   o.vpr_d = j.g.vpr.d;
   o.vpr_m = j.g.vpr.m;
   o.vpr_s = j.g.vpr.s;
@@ -109,7 +110,8 @@ __device__ __forceinline__ uint32_t chain_scale_index(uint32_t v, const ChainJob
   } else {
     const uint32_t r = (uint32_t)(((uint64_t)v * job.vpr_m) >> 31) >> job.vpr_s;
     const uint32_t cv = v - r * job.vpr_d;
-    return r * job.s_stride + ((uint32_t)(((uint64_t)cv * job.vpb_m) >> 31) >> job.vpb_s);
+    return (r >> job.row_shift) * job.s_stride +
+           ((uint32_t)(((uint64_t)cv * job.vpb_m) >> 31) >> job.vpb_s);
   }
 }
 

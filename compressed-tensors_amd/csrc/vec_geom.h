@@ -31,7 +31,8 @@ struct VecGeom {
   FastDiv vpb;        // items per scale block (blk_cols / 8)
   uint32_t nvec;      // total items
   uint32_t s_cols;
-  uint32_t row_scaled;  // 1: scale row = tensor row; 0: a single scale row
+  uint32_t row_scaled;  // 1: scale row = tensor row >> row_shift; 0: a single scale row
+  uint32_t row_shift;   // log2 of the rows that share a scale row (blocks: 2^k rows tall)
   // When every row has its own scales and scale blocks tile the rows exactly,
   // scales are numbered like the items: index = item / vpb, a shift if vpb is a
   // power of two.  mode 0: shift, 1: one division, 2: row/column split.
@@ -43,7 +44,7 @@ __device__ __forceinline__ uint32_t scale_index(uint32_t v, const VecGeom& g) {
   if (g.mode == 1) return fdiv(v, g.vpb);
   const uint32_t r = fdiv(v, g.vpr);
   const uint32_t cv = v - r * g.vpr.d;
-  return (g.row_scaled ? r * g.s_cols : 0u) + fdiv(cv, g.vpb);
+  return (g.row_scaled ? (r >> g.row_shift) * g.s_cols : 0u) + fdiv(cv, g.vpb);
 }
 
 template <int A, int B>
@@ -68,8 +69,10 @@ static inline bool vec_geometry(const ctmi_qparams* qp, int64_t rows, int64_t co
   if (cols % 8 || qp->blk_cols % 8) return false;
   if (rows * cols / 8 >= (1ll << 31) || cols / 8 < 1) return false;
   if (cols % qp->blk_cols) return false;
-  const bool row_scaled = (qp->blk_rows == 1 && qp->s_rows == rows);
   const bool single_row = (qp->s_rows == 1 && qp->blk_rows >= rows);
+  // every row its own scales, or blocks a power of two rows tall
+  const bool pow2_rows = qp->blk_rows >= 1 && (qp->blk_rows & (qp->blk_rows - 1)) == 0;
+  const bool row_scaled = pow2_rows && qp->s_rows == cdiv(rows, qp->blk_rows);
   if (!row_scaled && !single_row) return false;
   if (qp->s_cols >= (1ll << 31) || rows * qp->s_cols >= (1ll << 31)) return false;
   g->vpr = make_fastdiv((uint32_t)(cols / 8));
@@ -77,9 +80,13 @@ static inline bool vec_geometry(const ctmi_qparams* qp, int64_t rows, int64_t co
   g->nvec = (uint32_t)(rows * cols / 8);
   g->s_cols = (uint32_t)qp->s_cols;
   g->row_scaled = row_scaled ? 1u : 0u;
+  g->row_shift = 0;
+  if (row_scaled)
+    while ((1ll << g->row_shift) < qp->blk_rows) ++g->row_shift;
   g->mode = 2;
   g->shift = 0;
-  if (row_scaled && g->vpr.d % g->vpb.d == 0 && qp->s_cols == cols / qp->blk_cols) {
+  if (row_scaled && g->row_shift == 0 && g->vpr.d % g->vpb.d == 0 &&
+      qp->s_cols == cols / qp->blk_cols) {
     const uint32_t d = g->vpb.d;
     if ((d & (d - 1)) == 0) {
       g->mode = 0;

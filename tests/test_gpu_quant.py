@@ -45,6 +45,10 @@ CASES = [
     (dict(num_bits=8, type="float", symmetric=True, strategy="tensor"), (40, 250), torch.float16, None),
     (dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[16, 32]), (64, 128), torch.bfloat16, None),
     (dict(num_bits=4, type="int", symmetric=True, strategy="block", block_structure=[2, 3]), (4, 6), torch.bfloat16, None),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[128, 128]), (256, 384), torch.bfloat16, None),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="block", block_structure=[8, 64]), (64, 256), torch.float16, None),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[6, 32]), (12, 64), torch.bfloat16, None),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[1, 16]), (5, 64), torch.float32, None),
     (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (32, 256), torch.bfloat16, torch.float32),
     (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=64), (32, 256), torch.float16, torch.bfloat16),
     (dict(num_bits=2, type="int", symmetric=True, strategy="channel"), (8, 64), torch.bfloat16, None),
