@@ -319,6 +319,17 @@ int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64_t rows, in
                      const float* global_scale, void* scale_out, int32_t scale_dtype,
                      void* zp_out, int32_t zp_dtype, void* stream);
 
+/* MXFP4 group scales (quantization/utils/mxfp4_utils.py): powers of two held as
+ * uint8 exponents.  x / out of the first two are bfloat16 group maxima, n values.
+ *   ctmi_mxfp4_round_to_power_2   :41-73  (x + 32) & 0xFF80 on the bf16 bits
+ *   ctmi_mxfp4_generate_scales    :76-97  127 + floor(log2(round_to_power_2(x))) - 2,
+ *                                         clamped to [0, 255]
+ *   ctmi_mxfp4_convert_exp_scale  :24-38  2 ** (e - 127) in out_dtype (f32 / f16 / bf16) */
+int ctmi_mxfp4_round_to_power_2(const void* x, void* out, int64_t n, void* stream);
+int ctmi_mxfp4_generate_scales(const void* x, uint8_t* out, int64_t n, void* stream);
+int ctmi_mxfp4_convert_exp_scale(const uint8_t* exps, void* out, int32_t out_dtype, int64_t n,
+                                 void* stream);
+
 /* A24 / A25.  Hadamard transform apply (transform/utils/matrix.py:65-171,
  * transform/factory/hadamard.py:104-121) for a matrix given in factored form
  *     W = diag(sign_in) * (Ma (x) Mb) * diag(sign_out),      n = a_dim * b_dim:

@@ -446,3 +446,31 @@ def test_quantized_weight_batch_matches_single_calls(gpu):
         assert c.dtype == want.dtype and torch.equal(c.view(torch.int8), want.view(torch.int8))
         back = dequantize(want, e["scale"], None if args.symmetric else e["zero_point"])
         assert d.dtype == back.dtype and torch.equal(d.view(torch.int16), back.view(torch.int16))
+
+
+def test_mxfp4_scale_helpers_on_every_input(gpu):
+    """round_to_power_2 and generate_mxfp4_scales on all 65 536 bfloat16 patterns,
+    convert_mxfp4_exp_scale on all 256 exponents, against the oracle"""
+    from compressed_tensors_amd.quantization import (
+        convert_mxfp4_exp_scale, generate_mxfp4_scales, round_to_power_2,
+    )
+    from oracle import mxfp4 as om
+
+    announce("mxfp4 scales")
+    x = torch.arange(65536, dtype=torch.int32).to(torch.uint16).view(torch.bfloat16).reshape(256, 256)
+    assert_bit_equal(round_to_power_2(x.to(gpu)), om.round_to_power_2(x), "round_to_power_2")
+    got = generate_mxfp4_scales(x.to(gpu)).cpu()
+    want = om.generate_mxfp4_scales(x)
+    # a group maximum is never negative; for negative, infinite and NaN inputs the
+    # reference casts a NaN / infinity to int32, which the language leaves undefined
+    defined = (x.view(torch.int16) >= 0) & torch.isfinite(x.float()) \
+        & torch.isfinite(om.round_to_power_2(x).float())
+    assert torch.equal(got[defined], want[defined])
+    assert int(defined.sum()) > 32000
+    e = torch.arange(256, dtype=torch.int32).to(torch.uint8)
+    for dtype in (torch.bfloat16, torch.float16, torch.float32):
+        assert_bit_equal(convert_mxfp4_exp_scale(e.to(gpu), dtype), om.convert_mxfp4_exp_scale(e, dtype),
+                         f"convert {dtype}")
+    assert convert_mxfp4_exp_scale(e[:0].to(gpu)).shape == (0,)
+    with pytest.raises(AssertionError):
+        round_to_power_2(torch.zeros(4, device=gpu))

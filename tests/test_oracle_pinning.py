@@ -360,3 +360,45 @@ def test_24_mask_fp8_uses_int8_view():
     assert torch.equal(mask, want.reshape(1, 8))
     # abs(int8(-128)) wraps to -128 and so ranks below zero
     assert not bool(mask[0, 0])
+
+
+# ---------------------------------------------------------------- MXFP4 scales
+def test_mxfp4_round_to_power_2_reference_vector():
+    from oracle import mxfp4
+
+    gold = json.loads((GOLDEN / "mxfp4.json").read_text())
+    x = torch.tensor(gold["x"]).to(torch.bfloat16)
+    want = torch.tensor(gold["rounded"]).to(torch.bfloat16)
+    assert torch.equal(mxfp4.round_to_power_2(x), want)
+
+
+def test_mxfp4_noisy_powers_round_back():
+    """the reference's second test (test_mxfp4_utils.py:22-38): a power of two times
+    (1 + up to 20 % noise) rounds back to it"""
+    from oracle import mxfp4
+
+    g = torch.Generator().manual_seed(0)
+    powers = (2.0 ** torch.arange(-10, 2).float()).repeat(50).to(torch.bfloat16)
+    noisy = powers * (1 + torch.rand(powers.shape, generator=g).to(torch.bfloat16) * 0.2)
+    assert torch.equal(mxfp4.round_to_power_2(noisy), powers)
+
+
+def test_mxfp4_scales_closed_form():
+    """every positive normal bfloat16: the exponent is that of the rounded power of two
+    minus 2 (clamped at 0), and 2 ** (e - 127) gives it back (test_mxfp4_utils.py:64-80)"""
+    from oracle import mxfp4
+
+    bits = torch.arange(0x0080, 0x7F80, dtype=torch.int32).to(torch.uint16)
+    x = bits.view(torch.bfloat16)
+    e = mxfp4.generate_mxfp4_scales(x)
+    rounded_bits = (bits.to(torch.int32) + 32) & 0xFF80
+    biased = rounded_bits >> 7
+    want = torch.where(biased == 255, torch.zeros_like(biased), torch.clamp(biased - 2, min=0))
+    assert torch.equal(e.to(torch.int32), want)
+    ok = (biased >= 2) & (biased < 255)
+    back = mxfp4.convert_mxfp4_exp_scale(e)
+    assert torch.equal(torch.log2(back.float())[ok], (biased[ok] - 2 - 127).float())
+    # all 256 exponents: exact powers of two, subnormal at the bottom, infinite at the top
+    every = mxfp4.convert_mxfp4_exp_scale(torch.arange(256, dtype=torch.int32).to(torch.uint8), torch.float32)
+    assert every[0].item() == 2.0 ** -127 and every[127].item() == 1.0 and every[254].item() == 2.0 ** 127
+    assert torch.isinf(every[255])
