@@ -380,3 +380,43 @@ def test_nvfp4_every_bf16_pattern(scale_value, global_scale, gpu):
     want_fq = oq.fake_quantize(w, scale, None, oargs, global_scale=gs)
     assert_bit_equal(fq[finite], want_fq[finite], "nvfp4 fake-quantize")
     assert bool(torch.isnan(fq[~finite].float()).all() == torch.isnan(want_fq[~finite].float()).all())
+
+
+def test_weight_larger_than_4_gib(gpu):
+    """a 140 000 x 16 384 bf16 weight (4.6 GB: byte offsets beyond 32 bits, an lm_head of
+    a large model): slices at both ends and in the middle against the oracle, and the
+    round trip compress(decompress(compress(w))) == compress(w) over the whole tensor"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.quantization import observe_weight_qparams
+
+    announce("4.6 GB weight")
+    rows, cols = 140_000, 16_384
+    spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    args, oargs = _pair(spec)
+    gen = torch.Generator(device=gpu).manual_seed(99)
+    w = torch.empty(rows, cols, dtype=torch.bfloat16, device=gpu)
+    for r0 in range(0, rows, 20_000):  # in pieces: the fp32 draw of the whole tensor would be 9 GB
+        r1 = min(r0 + 20_000, rows)
+        w[r0:r1] = (torch.randn(r1 - r0, cols, generator=gen, device=gpu) * 0.02).bfloat16()
+    assert w.numel() * 2 > 1 << 32
+    scale, zp = observe_weight_qparams(w, args)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    packed = comp.compress_weight(weight=w, scale=scale, quantization_args=args)["weight_packed"]
+    fused = comp.observe_and_compress_weight(w, args)
+    assert torch.equal(fused["weight_packed"], packed) and torch.equal(fused["weight_scale"], scale)
+    dense = comp.decompress_weight(
+        {"weight_packed": packed, "weight_scale": scale, "weight_shape": torch.tensor([rows, cols])},
+        quantization_args=args)
+    for r0 in (0, 70_001, rows - 48):
+        sl = slice(r0, r0 + 48)
+        w_cpu = w[sl].cpu()
+        o_scale, o_zp = oq.observe_weight(w_cpu, oargs)
+        assert_bit_equal(scale[sl], o_scale, f"scale rows {r0}")
+        want = op.pack_quantized_compress(w_cpu, o_scale, oargs, zero_point=None)
+        assert_bit_equal(packed[sl], want["weight_packed"], f"packed rows {r0}")
+        want_dense = op.pack_quantized_decompress(
+            dict(want, weight_scale=o_scale, weight_shape=torch.tensor([48, cols])), oargs)
+        assert_bit_equal(dense[sl], want_dense, f"dense rows {r0}")
+    del w
+    again = comp.compress_weight(weight=dense, scale=scale, quantization_args=args)["weight_packed"]
+    assert torch.equal(again, packed)
