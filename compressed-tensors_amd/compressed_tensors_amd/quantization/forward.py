@@ -74,11 +74,19 @@ def _leading_grid(x_shape, s_shape) -> Tuple[int, int]:
 def _column_groups(g_idx: Optional[torch.Tensor], group_size: int) -> Optional[torch.Tensor]:
     """act-order: the reference sorts columns by g_idx and cuts the sorted order
     into runs of group_size (forward.py:286-303, 329-331)."""
-    if g_idx is None or bool((g_idx == -1).any()):
+    if g_idx is None:
         return None
-    perm = torch.argsort(g_idx)
-    position = torch.argsort(perm)
-    return (position // group_size).to(torch.int32).contiguous()
+    cols = g_idx.numel()
+    if cols >= 1 << 16:  # beyond the counting kernel: torch's sort, with a host read-back
+        if bool((g_idx == -1).any()):
+            return None
+        position = torch.argsort(torch.argsort(g_idx, stable=True))
+        return (position // group_size).to(torch.int32).contiguous()
+    g = g_idx.reshape(-1).to(torch.int32).contiguous()
+    out = torch.empty_like(g)
+    _lib.check(_lib.load().ctmi_column_groups(g.data_ptr(), cols, group_size, out.data_ptr(),
+                                              _lib.stream_of(g.device)))
+    return out
 
 
 class QPlan:

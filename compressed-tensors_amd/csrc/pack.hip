@@ -454,11 +454,26 @@ extern "C" int ctmi_unpack_from_int32(const int32_t* in, int8_t* out, int64_t ro
   return check_launch("ctmi_unpack_from_int32");
 }
 
+namespace ctmi {
+bool gidx_geometry(const ctmi_qparams* qp, int64_t rows, int64_t cols, int dense_dtype,
+                   const void* dense, const void* packed);
+void gidx_launch_compress(const void* x, int x_dtype, int32_t* out, int64_t rows, int64_t cols,
+                          const ctmi_qparams* qp, hipStream_t st);
+void gidx_launch_decompress(const int32_t* packed, void* out, int64_t rows, int64_t cols,
+                            const ctmi_qparams* qp, hipStream_t st);
+}  // namespace ctmi
+
 // ---- pack-quantized compress / decompress: validate (no HIP call), then launch.
 // A plan is the validated, classified form of one weight.
 struct PqPlan {
   bool empty;   // nothing to launch
   bool vec;     // runs in the vectorised multi-tensor kernel
+  bool gidx;    // activation-ordered groups: runs in the streaming g_idx kernel
+  ctmi_qparams qp;  // for the g_idx launch
+  const void* src;
+  void* dst;
+  int64_t rows, cols;
+  int dense_dtype;
   VecKey key;
   VecJob job;
   FusedArgs generic;
@@ -478,6 +493,7 @@ static int plan_compress(const void* x, int32_t x_dtype, int32_t* out, int64_t r
   rc = check_bits(qp->num_bits);
   if (rc) return rc;
   p->empty = rows == 0 || cols == 0;
+  p->vec = p->gidx = false;
   if (p->empty) return CTMI_OK;
   CTMI_REQUIRE(x && out, CTMI_ERR_VALUE, "NULL tensor pointer");
 
@@ -493,6 +509,16 @@ static int plan_compress(const void* x, int32_t x_dtype, int32_t* out, int64_t r
     p->job.dst = out;
     p->job.scale = qp->scale;
     p->job.zp = (const int8_t*)qp->zero_point;
+    return CTMI_OK;
+  }
+  p->gidx = gidx_geometry(qp, rows, cols, x_dtype, x, out);
+  if (p->gidx) {
+    p->qp = *qp;
+    p->src = x;
+    p->dst = out;
+    p->rows = rows;
+    p->cols = cols;
+    p->dense_dtype = x_dtype;
     return CTMI_OK;
   }
   FusedArgs& a = p->generic;
@@ -518,6 +544,7 @@ static int plan_decompress(const int32_t* packed, void* out, int32_t out_dtype, 
                "Unpacking is only supported for less than 8 bits");
   CTMI_REQUIRE(qp->qtype == CTMI_QTYPE_INT, CTMI_ERR_VALUE, "pack-quantized holds integer codes");
   p->empty = rows == 0 || cols == 0;
+  p->vec = p->gidx = false;
   if (p->empty) return CTMI_OK;
   CTMI_REQUIRE(packed && out, CTMI_ERR_VALUE, "NULL tensor pointer");
 
@@ -534,6 +561,16 @@ static int plan_decompress(const int32_t* packed, void* out, int32_t out_dtype, 
     p->job.dst = out;
     p->job.scale = qp->scale;
     p->job.zp = (const int8_t*)qp->zero_point;
+    return CTMI_OK;
+  }
+  p->gidx = out_dtype == qp->scale_dtype && gidx_geometry(qp, rows, cols, out_dtype, out, packed);
+  if (p->gidx) {
+    p->qp = *qp;
+    p->src = packed;
+    p->dst = out;
+    p->rows = rows;
+    p->cols = cols;
+    p->dense_dtype = out_dtype;
     return CTMI_OK;
   }
   FusedArgs& a = p->generic;
@@ -559,6 +596,17 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
   std::vector<char> done((size_t)n, 0);
   for (int64_t i = 0; i < n; ++i) {
     if (done[i] || plans[i].empty) continue;
+    if (plans[i].gidx) {
+      const PqPlan& g = plans[i];
+      ++launches;
+      if (count_only) {
+      } else if (compress)
+        gidx_launch_compress(g.src, g.dense_dtype, (int32_t*)g.dst, g.rows, g.cols, &g.qp, st);
+      else
+        gidx_launch_decompress((const int32_t*)g.src, g.dst, g.rows, g.cols, &g.qp, st);
+      done[i] = 1;
+      continue;
+    }
     if (!plans[i].vec) {
       const FusedArgs& a = plans[i].generic;
       ++launches;

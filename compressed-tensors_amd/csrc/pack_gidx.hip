@@ -1,0 +1,404 @@
+// pack-quantized compress / decompress for activation-ordered weights: the group
+// of a column is g_idx[column] instead of column / group_size
+// (quantization/lifecycle/forward.py:286-296, pack_quantized.py:88-183).
+//
+// A workgroup takes RB rows of a tile of 256 x 8 columns.  A lane keeps the group
+// indices of its 8 columns in registers for all RB rows; the RB rows of scales
+// (and zero points) are staged in LDS as fp32 once and gathered from there, so the
+// only per-element global traffic is the dense / packed data itself, in 16-byte
+// pieces as in the column-ordered kernels.
+#include <type_traits>
+
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "quant_core.h"
+#include "quant_fast.h"
+
+namespace ctmi {
+
+struct GidxArgs {
+  const void* dense;          // compress: input; decompress: output
+  const int32_t* packed_in;   // decompress
+  int32_t* packed_out;        // compress
+  const void* scale;
+  const int8_t* zp;
+  const int32_t* col_group;
+  uint32_t rows, vpr, s_cols, tiles;  // vpr: items (8 elements) per row
+  float qmin, qmax;
+};
+
+constexpr int kGidxThreads = 256;
+
+// quantize + pack 8 elements, every element with its own scale / zero point: the
+// reference chain with one IEEE division per element
+template <typename XT, typename ST, int BITS, bool HAS_ZP>
+__device__ __forceinline__ Vec<int32_t, BITS / 4> quant_pack8_each_exact(
+    const Vec<typename XT::raw, 8>& xv, const float* s, const float* z, float qmin, float qmax) {
+  constexpr int W = BITS / 4;
+  constexpr int PF = 32 / BITS;
+  constexpr int OFF = 1 << (BITS - 1);
+  constexpr int CT = (XT::id == ST::id) ? XT::id : CTMI_F32;
+  Vec<int32_t, W> o;
+#pragma unroll
+  for (int w = 0; w < W; ++w) {
+    uint32_t acc = 0;
+#pragma unroll
+    for (int i = 0; i < PF; ++i) {
+      const int e = w * PF + i;
+      float t = round_ct<CT>(XT::to_f32(xv.v[e]) / s[e]);
+      if (HAS_ZP) t = round_ct<CT>(t + z[e]);
+      t = rintf(clamp_nan(t, qmin, qmax));
+      acc |= ((uint32_t)(f32_to_int(t) + OFF) & ((1u << BITS) - 1u)) << (BITS * i);
+    }
+    o.v[w] = (int32_t)acc;
+  }
+  return o;
+}
+
+// bf16 input, bf16 scales of ordinary magnitude: products with the staged
+// reciprocals (they round to the same bf16 as the quotients), hardware bf16
+// conversions, integer rounding and packing by the magic-number addition
+template <int BITS, bool HAS_ZP>
+__device__ __forceinline__ Vec<int32_t, BITS / 4> quant_pack8_each_bf16(
+    const Vec<uint16_t, 8>& xv, const float* r, const float* z, float qmin, float qmax) {
+  using PC = PackConst<BITS>;
+  constexpr int W = BITS / 4;
+  const Vec<uint32_t, 4> xw = __builtin_bit_cast(Vec<uint32_t, 4>, xv);
+  uint32_t acc[W];
+#pragma unroll
+  for (int w = 0; w < W; ++w) acc[w] = 0u - PC::bias();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int e0 = 2 * j, e1 = 2 * j + 1;
+    uint32_t t = pack_bf16x2(bf16_lo(xw.v[j]) * r[e0], bf16_hi(xw.v[j]) * r[e1]);
+    if (HAS_ZP) t = pack_bf16x2(bf16_lo(t) + z[e0], bf16_hi(t) + z[e1]);
+    const float c0 = __builtin_amdgcn_fmed3f(bf16_lo(t), qmin, qmax) + PC::MAGIC;
+    const float c1 = __builtin_amdgcn_fmed3f(bf16_hi(t), qmin, qmax) + PC::MAGIC;
+    acc[e0 / PC::PF] += f2u(c0) << (BITS * (e0 % PC::PF));
+    acc[e1 / PC::PF] += f2u(c1) << (BITS * (e1 % PC::PF));
+  }
+  Vec<int32_t, W> o;
+#pragma unroll
+  for (int w = 0; w < W; ++w) o.v[w] = (int32_t)acc[w];
+  return o;
+}
+
+// unpack + dequantize 8 elements: (q - zp) is an integer of at most 8 bits, exact in
+// every float type here, so the reference's chain rounds once, in the product
+template <typename ST, int BITS, bool HAS_ZP>
+__device__ __forceinline__ Vec<typename ST::raw, 8> unpack_dequant8_each(
+    const Vec<int32_t, BITS / 4>& pv, const float* s, const float* z) {
+  constexpr int PF = 32 / BITS;
+  constexpr int OFF = 1 << (BITS - 1);
+  Vec<typename ST::raw, 8> o;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    const uint32_t word = (uint32_t)pv.v[e / PF];
+    const int q = (int)((word >> (BITS * (e % PF))) & ((1u << BITS) - 1u)) - OFF;
+    float t = (float)q;
+    if (HAS_ZP) t -= z[e];
+    o.v[e] = ST::from_f32(t * s[e]);
+  }
+  return o;
+}
+
+// stage RB rows of scales (zero points) as fp32: lds_s[rb * s_cols + j]; with lds_r
+// also their reciprocals.  Returns whether a staged scale is outside the range
+// where the reciprocal path is exact.
+template <typename ST, bool HAS_ZP, int RB>
+__device__ __forceinline__ bool stage_qparams(const GidxArgs& a, uint32_t row0, float* lds_s,
+                                              float* lds_z, float* lds_r) {
+  const auto* scale = (const typename ST::raw*)a.scale;
+  bool wild = false;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const uint32_t row = min(row0 + rb, a.rows - 1);
+    for (uint32_t j = threadIdx.x; j < a.s_cols; j += kGidxThreads) {
+      const size_t si = (size_t)row * a.s_cols + j;
+      const float sv = ST::to_f32(scale[si]);
+      lds_s[rb * a.s_cols + j] = sv;
+      if (lds_r) {
+        lds_r[rb * a.s_cols + j] = __builtin_amdgcn_rcpf(sv);
+        wild |= !scale_is_tame(sv);
+      }
+      if constexpr (HAS_ZP) lds_z[rb * a.s_cols + j] = (float)a.zp[si];
+    }
+  }
+  return wild;
+}
+
+__device__ __forceinline__ void load_groups(const GidxArgs& a, uint32_t cv, uint32_t* g) {
+  const Vec<int32_t, 4> lo = ldg<int32_t, 4>(a.col_group + (size_t)cv * 8);
+  const Vec<int32_t, 4> hi = ldg<int32_t, 4>(a.col_group + (size_t)cv * 8 + 4);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    // an index outside the scale row must not leave the staged window
+    g[k] = min((uint32_t)max(lo.v[k], 0), a.s_cols - 1);
+    g[4 + k] = min((uint32_t)max(hi.v[k], 0), a.s_cols - 1);
+  }
+}
+
+template <typename XT, typename ST, int BITS, bool HAS_ZP, int RB>
+__global__ void __launch_bounds__(kGidxThreads) pq_gidx_compress_kernel(GidxArgs a) {
+  using XR = typename XT::raw;
+  constexpr int W = BITS / 4;
+  constexpr bool kBf16 = XT::id == CTMI_BF16 && ST::id == CTMI_BF16;
+  extern __shared__ float lds[];
+  float* lds_s = lds;
+  float* lds_r = lds + RB * a.s_cols;
+  float* lds_z = lds + 2 * RB * a.s_cols;
+  const uint32_t rowblk = blockIdx.x / a.tiles, tile = blockIdx.x - rowblk * a.tiles;
+  const uint32_t row0 = rowblk * RB;
+  const uint32_t cv = tile * kGidxThreads + threadIdx.x;
+  const bool lane_ok = cv < a.vpr;
+  const uint32_t cvc = lane_ok ? cv : a.vpr - 1;
+  const XR* x = (const XR*)a.dense;
+  Vec<XR, 8> xv[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const uint32_t row = min(row0 + rb, a.rows - 1);
+    xv[rb] = ldg_nt<XR, 8>(x + ((size_t)row * a.vpr + cvc) * 8);
+  }
+  uint32_t g[8];
+  load_groups(a, cvc, g);
+  const bool wild = stage_qparams<ST, HAS_ZP, RB>(a, row0, lds_s, lds_z, lds_r);
+  const bool fast = kBf16 && !__syncthreads_or(wild);  // the barrier that publishes the staged rows
+  if constexpr (!kBf16) __syncthreads();
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    float s[8], z[8];
+    const float* from = fast ? lds_r : lds_s;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      s[k] = from[rb * a.s_cols + g[k]];
+      z[k] = HAS_ZP ? lds_z[rb * a.s_cols + g[k]] : 0.0f;
+    }
+    Vec<int32_t, W> w;
+    if constexpr (kBf16) {
+      if (fast) w = quant_pack8_each_bf16<BITS, HAS_ZP>(xv[rb], s, z, a.qmin, a.qmax);
+      else w = quant_pack8_each_exact<XT, ST, BITS, HAS_ZP>(xv[rb], s, z, a.qmin, a.qmax);
+    } else {
+      w = quant_pack8_each_exact<XT, ST, BITS, HAS_ZP>(xv[rb], s, z, a.qmin, a.qmax);
+    }
+    const uint32_t row = row0 + rb;
+    if (lane_ok && row < a.rows)
+      stg_nt<int32_t, W>(a.packed_out + ((size_t)row * a.vpr + cv) * W, w);
+  }
+}
+
+template <typename ST, int BITS, bool HAS_ZP, int RB>
+__global__ void __launch_bounds__(kGidxThreads) pq_gidx_decompress_kernel(GidxArgs a) {
+  using SR = typename ST::raw;
+  constexpr int W = BITS / 4;
+  extern __shared__ float lds[];
+  float* lds_s = lds;
+  float* lds_z = lds + RB * a.s_cols;
+  const uint32_t rowblk = blockIdx.x / a.tiles, tile = blockIdx.x - rowblk * a.tiles;
+  const uint32_t row0 = rowblk * RB;
+  const uint32_t cv = tile * kGidxThreads + threadIdx.x;
+  const bool lane_ok = cv < a.vpr;
+  const uint32_t cvc = lane_ok ? cv : a.vpr - 1;
+  Vec<int32_t, W> pv[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const uint32_t row = min(row0 + rb, a.rows - 1);
+    pv[rb] = ldg_nt<int32_t, W>(a.packed_in + ((size_t)row * a.vpr + cvc) * W);
+  }
+  uint32_t g[8];
+  load_groups(a, cvc, g);
+  stage_qparams<ST, HAS_ZP, RB>(a, row0, lds_s, lds_z, nullptr);
+  __syncthreads();
+  SR* out = (SR*)a.dense;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    float s[8], z[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      s[k] = lds_s[rb * a.s_cols + g[k]];
+      z[k] = HAS_ZP ? lds_z[rb * a.s_cols + g[k]] : 0.0f;
+    }
+    const Vec<SR, 8> o = unpack_dequant8_each<ST, BITS, HAS_ZP>(pv[rb], s, z);
+    const uint32_t row = row0 + rb;
+    if (lane_ok && row < a.rows) stg_nt<SR, 8>(out + ((size_t)row * a.vpr + cv) * 8, o);
+  }
+}
+
+// rows per workgroup so that the staged fp32 arrays (scales, for compression their
+// reciprocals, zero points) stay within 32 KB
+static int gidx_rows_per_block(int64_t s_cols, int arrays) {
+  const int64_t per_row = s_cols * 4 * arrays;
+  for (int rb = 8; rb >= 1; rb >>= 1)
+    if (rb * per_row <= 32 * 1024) return rb;
+  return 0;
+}
+
+template <typename XT, typename ST, int BITS, bool HAS_ZP>
+static void launch_gidx_compress_rb(const GidxArgs& a, int rb, size_t lds, hipStream_t st) {
+  const unsigned grid = (unsigned)(cdiv(a.rows, rb) * a.tiles);
+#define CTMI_G(RB) hipLaunchKernelGGL((pq_gidx_compress_kernel<XT, ST, BITS, HAS_ZP, RB>), grid, kGidxThreads, lds, st, a)
+  if (rb == 8) CTMI_G(8); else if (rb == 4) CTMI_G(4); else if (rb == 2) CTMI_G(2); else CTMI_G(1);
+#undef CTMI_G
+}
+
+template <typename ST, int BITS, bool HAS_ZP>
+static void launch_gidx_decompress_rb(const GidxArgs& a, int rb, size_t lds, hipStream_t st) {
+  const unsigned grid = (unsigned)(cdiv(a.rows, rb) * a.tiles);
+#define CTMI_G(RB) hipLaunchKernelGGL((pq_gidx_decompress_kernel<ST, BITS, HAS_ZP, RB>), grid, kGidxThreads, lds, st, a)
+  if (rb == 8) CTMI_G(8); else if (rb == 4) CTMI_G(4); else if (rb == 2) CTMI_G(2); else CTMI_G(1);
+#undef CTMI_G
+}
+
+template <typename XT, typename ST>
+static void launch_gidx_compress_st(const GidxArgs& a, int bits, int rb, size_t lds, hipStream_t st) {
+  const bool has_zp = a.zp != nullptr;
+  if (bits == 4) {
+    if (has_zp) launch_gidx_compress_rb<XT, ST, 4, true>(a, rb, lds, st);
+    else launch_gidx_compress_rb<XT, ST, 4, false>(a, rb, lds, st);
+  } else {
+    if (has_zp) launch_gidx_compress_rb<XT, ST, 8, true>(a, rb, lds, st);
+    else launch_gidx_compress_rb<XT, ST, 8, false>(a, rb, lds, st);
+  }
+}
+
+template <typename XT>
+static void launch_gidx_compress_xt(const GidxArgs& a, int scale_dtype, int bits, int rb,
+                                    size_t lds, hipStream_t st) {
+  if (scale_dtype == CTMI_BF16) launch_gidx_compress_st<XT, BF16>(a, bits, rb, lds, st);
+  else if (scale_dtype == CTMI_F16) launch_gidx_compress_st<XT, F16>(a, bits, rb, lds, st);
+  else launch_gidx_compress_st<XT, F32>(a, bits, rb, lds, st);
+}
+
+template <typename ST>
+static void launch_gidx_decompress_st(const GidxArgs& a, int bits, int rb, size_t lds, hipStream_t st) {
+  const bool has_zp = a.zp != nullptr;
+  if (bits == 4) {
+    if (has_zp) launch_gidx_decompress_rb<ST, 4, true>(a, rb, lds, st);
+    else launch_gidx_decompress_rb<ST, 4, false>(a, rb, lds, st);
+  } else {
+    if (has_zp) launch_gidx_decompress_rb<ST, 8, true>(a, rb, lds, st);
+    else launch_gidx_decompress_rb<ST, 8, false>(a, rb, lds, st);
+  }
+}
+
+// Can the streaming act-order kernels take this weight?  (every row its own scale
+// row, 4- or 8-bit codes, columns in multiples of 8, int8 zero points)
+bool gidx_geometry(const ctmi_qparams* qp, int64_t rows, int64_t cols, int dense_dtype,
+                   const void* dense, const void* packed) {
+  if (!qp->col_group || qp->global_scale) return false;
+  if (qp->num_bits != 4 && qp->num_bits != 8) return false;
+  if (qp->blk_rows != 1 || qp->s_rows != rows) return false;
+  if (cols % 8 || rows * (cols / 8) >= (1ll << 31) || rows >= (1ll << 31)) return false;
+  if (qp->scale_dtype != CTMI_BF16 && qp->scale_dtype != CTMI_F16 && qp->scale_dtype != CTMI_F32)
+    return false;
+  if (qp->zero_point && qp->zp_dtype != CTMI_I8) return false;
+  if (gidx_rows_per_block(qp->s_cols, 3) == 0) return false;
+  if ((uintptr_t)dense % (8 * dtype_size(dense_dtype)) || (uintptr_t)packed % 8 ||
+      (uintptr_t)qp->col_group % 16)
+    return false;
+  const int64_t tiles = cdiv(cols / 8, kGidxThreads);
+  return cdiv(rows, 1) * tiles < (1ll << 31);
+}
+
+static GidxArgs gidx_args(const ctmi_qparams* qp, int64_t rows, int64_t cols) {
+  GidxArgs a;
+  a.dense = nullptr;
+  a.packed_in = nullptr;
+  a.packed_out = nullptr;
+  a.scale = qp->scale;
+  a.zp = (const int8_t*)qp->zero_point;
+  a.col_group = qp->col_group;
+  a.rows = (uint32_t)rows;
+  a.vpr = (uint32_t)(cols / 8);
+  a.s_cols = (uint32_t)qp->s_cols;
+  a.tiles = (uint32_t)cdiv(cols / 8, kGidxThreads);
+  quant_range(CTMI_QTYPE_INT, qp->num_bits, &a.qmin, &a.qmax);
+  return a;
+}
+
+void gidx_launch_compress(const void* x, int x_dtype, int32_t* out, int64_t rows, int64_t cols,
+                          const ctmi_qparams* qp, hipStream_t st) {
+  GidxArgs a = gidx_args(qp, rows, cols);
+  a.dense = x;
+  a.packed_out = out;
+  const int arrays = qp->zero_point ? 3 : 2;
+  const int rb = gidx_rows_per_block(qp->s_cols, arrays);
+  const size_t lds = (size_t)rb * qp->s_cols * 4 * arrays;
+  if (x_dtype == CTMI_BF16) launch_gidx_compress_xt<BF16>(a, qp->scale_dtype, qp->num_bits, rb, lds, st);
+  else if (x_dtype == CTMI_F16) launch_gidx_compress_xt<F16>(a, qp->scale_dtype, qp->num_bits, rb, lds, st);
+  else launch_gidx_compress_xt<F32>(a, qp->scale_dtype, qp->num_bits, rb, lds, st);
+}
+
+void gidx_launch_decompress(const int32_t* packed, void* out, int64_t rows, int64_t cols,
+                            const ctmi_qparams* qp, hipStream_t st) {
+  GidxArgs a = gidx_args(qp, rows, cols);
+  a.dense = out;
+  a.packed_in = packed;
+  const int arrays = qp->zero_point ? 2 : 1;
+  const int rb = gidx_rows_per_block(qp->s_cols, arrays);
+  const size_t lds = (size_t)rb * qp->s_cols * 4 * arrays;
+  if (qp->scale_dtype == CTMI_BF16) launch_gidx_decompress_st<BF16>(a, qp->num_bits, rb, lds, st);
+  else if (qp->scale_dtype == CTMI_F16) launch_gidx_decompress_st<F16>(a, qp->num_bits, rb, lds, st);
+  else launch_gidx_decompress_st<F32>(a, qp->num_bits, rb, lds, st);
+}
+
+// ------------------------------------------------------------------ g_idx -> group of a column
+// The reference sorts the columns by g_idx and cuts the sorted order into runs of
+// group_size (forward.py:286-303): the group of column c is position(c) / group_size
+// with position(c) = #{c' : (g[c'], c') < (g[c], c)}, the place of c in a stable
+// sort.  Counted directly, tiled over (c, c') with integer atomics (the sum does not
+// depend on their order); a g_idx that holds a -1 is unset and means column order.
+constexpr int kRankTile = 1024;
+
+__global__ void __launch_bounds__(256)
+column_rank_zero_kernel(int32_t* __restrict__ rank, int cols) {
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  if (c < cols) rank[c] = 0;
+}
+
+__global__ void __launch_bounds__(256)
+column_rank_kernel(const int32_t* __restrict__ g, int32_t* __restrict__ rank, int cols) {
+  __shared__ uint32_t key[kRankTile];
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int base = blockIdx.y * kRankTile;
+  // (g, column) as one unsigned key: cols < 2^16 and g < 2^15 (checked on the host)
+  for (int i = threadIdx.x; i < kRankTile; i += 256) {
+    const int c2 = base + i;
+    key[i] = c2 < cols ? (((uint32_t)g[c2] & 0x7fffu) << 16) | (uint32_t)c2 : 0xffffffffu;
+  }
+  __syncthreads();
+  if (c >= cols) return;
+  const uint32_t mine = (((uint32_t)g[c] & 0x7fffu) << 16) | (uint32_t)c;
+  int below = 0;
+#pragma unroll 8
+  for (int i = 0; i < kRankTile; ++i) below += key[i] < mine ? 1 : 0;
+  if (below) atomicAdd(rank + c, below);
+}
+
+__global__ void __launch_bounds__(1024)
+column_group_finish_kernel(const int32_t* __restrict__ g, int32_t* __restrict__ rank_to_group,
+                           int cols, int group_size) {
+  bool unset = false;
+  for (int c = threadIdx.x; c < cols; c += 1024) unset |= g[c] == -1;
+  unset = __syncthreads_or(unset);
+  for (int c = threadIdx.x; c < cols; c += 1024)
+    rank_to_group[c] = (unset ? c : rank_to_group[c]) / group_size;
+}
+
+}  // namespace ctmi
+
+extern "C" int ctmi_column_groups(const int32_t* g_idx, int64_t cols, int64_t group_size,
+                                  int32_t* col_group, void* stream) {
+  using namespace ctmi;
+  CTMI_REQUIRE(cols >= 0 && group_size >= 1, CTMI_ERR_VALUE, "bad shape");
+  CTMI_REQUIRE(cols < (1 << 16), CTMI_ERR_UNSUPPORTED, "at most 65535 columns");
+  if (cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(g_idx && col_group, CTMI_ERR_VALUE, "NULL tensor pointer");
+  hipStream_t st = (hipStream_t)stream;
+  const unsigned col_blocks = (unsigned)cdiv(cols, 256);
+  hipLaunchKernelGGL(column_rank_zero_kernel, col_blocks, 256, 0, st, col_group, (int)cols);
+  hipLaunchKernelGGL(column_rank_kernel, dim3(col_blocks, (unsigned)cdiv(cols, kRankTile)), 256, 0,
+                     st, g_idx, col_group, (int)cols);
+  hipLaunchKernelGGL(column_group_finish_kernel, 1, 1024, 0, st, g_idx, col_group, (int)cols,
+                     (int)group_size);
+  return check_launch("ctmi_column_groups");
+}

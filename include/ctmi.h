@@ -330,6 +330,15 @@ int ctmi_mxfp4_generate_scales(const void* x, uint8_t* out, int64_t n, void* str
 int ctmi_mxfp4_convert_exp_scale(const uint8_t* exps, void* out, int32_t out_dtype, int64_t n,
                                  void* stream);
 
+/* Activation ordering (quantization/lifecycle/forward.py:286-303): the reference
+ * sorts the columns of a weight by g_idx and cuts the sorted order into runs of
+ * group_size.  col_group[c] = (place of column c in a stable sort by g_idx) /
+ * group_size is that rule as a per-column group index, the form ctmi_qparams
+ * takes; a g_idx that holds a -1 is unset and gives column order (c / group_size).
+ * g_idx values must lie in [-1, 32767], cols < 65536.  No scratch, no host sync. */
+int ctmi_column_groups(const int32_t* g_idx, int64_t cols, int64_t group_size,
+                       int32_t* col_group, void* stream);
+
 /* A24 / A25.  Hadamard transform apply (transform/utils/matrix.py:65-171,
  * transform/factory/hadamard.py:104-121) for a matrix given in factored form
  *     W = diag(sign_in) * (Ma (x) Mb) * diag(sign_out),      n = a_dim * b_dim:

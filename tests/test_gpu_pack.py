@@ -250,6 +250,47 @@ def test_pack_quantized_state_dict_and_g_idx(gpu):
                              global_scale=torch.ones(1, device=gpu))
 
 
+GIDX = [
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (64, 1024), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=128), (33, 4096), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=64), (19, 512), torch.float16, None),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=8), (13, 2056), torch.bfloat16, None),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (9, 256), torch.float32, None),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (16, 512), torch.bfloat16, torch.float32),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=16), (3, 20480), torch.bfloat16, None),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype,sdt", GIDX, ids=[f"gidx{i}" for i in range(len(GIDX))])
+def test_pack_quantized_with_activation_ordering(spec, shape, dtype, sdt, gpu):
+    """weights whose columns were grouped by activation order (a g_idx per column): the
+    streaming kernels gather the scales of every element's own group"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("pack-quantized g_idx", spec, shape, dtype, sdt)
+    args, oargs = _pair(spec)
+    rows, cols = shape
+    g = torch.Generator().manual_seed(34)
+    w = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+    w.view(-1)[:3] = torch.tensor([0.0, -0.0, -1e-6]).to(dtype)
+    n_groups = cols // spec["group_size"]
+    g_idx = (torch.randperm(cols, generator=g) // spec["group_size"]).to(torch.int32)
+    scale, zp = oq.observe_weight(w.index_select(-1, torch.argsort(g_idx)), oargs)
+    assert scale.shape == (rows, n_groups)
+    if sdt is not None:
+        scale = scale.to(sdt)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    got = comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+                               zero_point=None if spec["symmetric"] else zp.to(gpu), g_idx=g_idx.to(gpu))
+    want = op.pack_quantized_compress(w, scale, oargs, zero_point=None if spec["symmetric"] else zp,
+                                      g_idx=g_idx)
+    assert_bit_equal(got["weight_packed"], want["weight_packed"], "packed")
+    data = dict(want, weight_scale=scale, weight_g_idx=g_idx)
+    dense_want = op.pack_quantized_decompress(dict(data), oargs)
+    dense = comp.decompress_weight({k: v.to(gpu) for k, v in data.items()}, quantization_args=args)
+    assert_bit_equal(dense, dense_want, "decompress")
+
+
 NQ = [
     ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (96, 512), torch.bfloat16),
     ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="tensor"), (31, 65), torch.float16),

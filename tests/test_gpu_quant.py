@@ -474,3 +474,24 @@ def test_mxfp4_scale_helpers_on_every_input(gpu):
     assert convert_mxfp4_exp_scale(e[:0].to(gpu)).shape == (0,)
     with pytest.raises(AssertionError):
         round_to_power_2(torch.zeros(4, device=gpu))
+
+
+@pytest.mark.parametrize("cols,group_size", [(128, 32), (4096, 128), (1000, 8), (14336, 128), (40, 7)])
+def test_column_groups_from_g_idx(cols, group_size, gpu):
+    """g_idx -> group of every column: the place of the column in a stable sort by g_idx,
+    cut into runs of group_size; also with uneven group populations, and unset (-1)"""
+    from compressed_tensors_amd.quantization.forward import _column_groups
+
+    announce("column groups", cols, group_size)
+    g = torch.Generator().manual_seed(cols)
+    even = (torch.randperm(cols, generator=g) // group_size).to(torch.int32)
+    uneven = torch.randint(0, max(cols // group_size, 1), (cols,), generator=g, dtype=torch.int32)
+    for g_idx in (even, uneven, torch.arange(cols, dtype=torch.int32) // group_size):
+        want = (torch.argsort(torch.argsort(g_idx, stable=True), stable=True) // group_size).to(torch.int32)
+        assert_bit_equal(_column_groups(g_idx.to(gpu), group_size), want, "col_group")
+        assert_bit_equal(_column_groups(g_idx.to(torch.int64).to(gpu), group_size), want, "int64 g_idx")
+    unset = even.clone()
+    unset[cols // 2] = -1
+    assert_bit_equal(_column_groups(unset.to(gpu), group_size),
+                     (torch.arange(cols) // group_size).to(torch.int32), "unset g_idx")
+    assert _column_groups(None, group_size) is None
