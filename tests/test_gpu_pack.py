@@ -461,3 +461,48 @@ def test_weight_larger_than_4_gib(gpu):
     del w
     again = comp.compress_weight(weight=dense, scale=scale, quantization_args=args)["weight_packed"]
     assert torch.equal(again, packed)
+
+
+def test_batches_replay_from_a_captured_graph(gpu):
+    """the entry points allocate nothing and never synchronise, so a whole pass over a
+    state dict can be captured once and replayed: every replay (with eager work and
+    synchronisations in between) reproduces the eager result on fresh inputs"""
+    from compressed_tensors_amd.compressors import ObservedWeightBatch, PackedWeightBatch
+    from compressed_tensors_amd.quantization import QuantizationArgs, observe_weight_qparams
+
+    announce("graph replay")
+    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    g = torch.Generator(device=gpu).manual_seed(5)
+    shapes = [(256, 1024), (64, 512), (512, 256)] * 4  # 12 weights: more than one launch
+    weights = [(torch.randn(s, generator=g, device=gpu) * 0.02).bfloat16() for s in shapes]
+    entries = []
+    for w in weights:
+        scale, _ = observe_weight_qparams(w, args)
+        entries.append(dict(weight=w, scale=scale, quantization_args=args))
+    batch = PackedWeightBatch(entries)
+    one_shot = ObservedWeightBatch([dict(weight=w, quantization_args=args) for w in batch.weights])
+    lib_stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    batch.compress(), batch.decompress(), one_shot.compress()  # warm up outside the capture
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=lib_stream):
+        batch.compress()
+        batch.decompress()
+        one_shot.compress()
+    for replay in range(3):
+        for w in batch.weights:  # new data in the captured buffers
+            w.copy_((torch.randn(w.shape, generator=g, device=gpu) * 0.02).bfloat16())
+        for e, w in zip(entries, batch.weights):  # the scales the captured compress reads
+            e["scale"].copy_(observe_weight_qparams(w, args)[0])
+        for t in batch.packed + batch.dense + one_shot.packed + one_shot.scales:
+            t.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in batch.packed + batch.dense + one_shot.packed + one_shot.scales]
+        batch.compress(), batch.decompress(), one_shot.compress()  # eager, same buffers
+        torch.cuda.synchronize()
+        want = batch.packed + batch.dense + one_shot.packed + one_shot.scales
+        for i, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a, b), f"replay {replay}, tensor {i}"
+        assert all(torch.equal(p, q) for p, q in zip(batch.packed, one_shot.packed))
