@@ -264,7 +264,7 @@ def other_workload(torch, name, seed):
             values = torch.empty(rows, cols // 2, dtype=FP8, device=dev)
             bitmask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=dev)
             dense = torch.empty_like(q)
-            tmp = torch.empty(lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8, dtype=torch.uint8, device=dev)
+            tmp = torch.empty(lib.ctmi_sparse24_tmp_bytes(rows, cols, 1), dtype=torch.uint8, device=dev)
             a = (q.data_ptr(), code(FP8), values.data_ptr(), bitmask.data_ptr(), rows, cols, st)
             d = (values.data_ptr(), values.numel(), 1, bitmask.data_ptr(), dense.data_ptr(), tmp.data_ptr(), rows, cols, st)
             _lib.check(lib.ctmi_sparse24_compress(*a))

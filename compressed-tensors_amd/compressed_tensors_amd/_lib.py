@@ -216,6 +216,7 @@ SIGNATURES = {
     "ctmi_mxfp4_generate_scales": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "ctmi_mxfp4_convert_exp_scale": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
     "ctmi_column_groups": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
+    "ctmi_sparse24_tmp_bytes": (c_int64, [c_int64, c_int64, c_int32]),
     "ctmi_dynamic_qdq_supported": (
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32],
     ),

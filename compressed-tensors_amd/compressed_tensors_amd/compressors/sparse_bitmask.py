@@ -81,8 +81,9 @@ def _scatter(values: Tensor, bitmasks: Tensor, row_offsets, shape, two_four: boo
     if bitmasks.numel() != rows * ((cols + 7) // 8):
         raise ValueError(f"bitmask of {bitmasks.numel()} bytes does not describe shape {shape}")
     out = torch.empty(shape, dtype=values.dtype, device=dev)
-    tmp = torch.empty((lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8,), dtype=torch.uint8,
-                      device=dev)
+    tmp_bytes = (lib.ctmi_sparse24_tmp_bytes(rows, cols, esize) if two_four
+                 else lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8)
+    tmp = torch.empty((tmp_bytes,), dtype=torch.uint8, device=dev)
     ro_ptr = None
     if row_offsets is not None:
         row_offsets = to_gpu(row_offsets).to(torch.int64).contiguous()

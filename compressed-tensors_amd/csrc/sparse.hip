@@ -166,47 +166,51 @@ bitmask_count_kernel(const R* __restrict__ x, uint32_t nz_mask, uint8_t* __restr
 // per-row popcount of an existing bitmask (bits at columns >= cols ignored):
 // one wavefront per row, 4 bitmask bytes per lane and step when rows are whole
 // words
-// (`only_if`, when given, points at a flag that must be non-zero for the kernel to do anything)
-__global__ void __launch_bounds__(kBlock)
-bitmask_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t* __restrict__ counts,
-                        int64_t rows, int64_t cols, int64_t pc, const int* only_if) {
-  if (only_if && *only_if == 0) return;
+__device__ __forceinline__ void popcount_rows(const uint8_t* __restrict__ bitmask,
+                                              int64_t* __restrict__ counts, int64_t rows,
+                                              int64_t cols, int64_t pc, int64_t first_row,
+                                              int64_t row_stride) {
   const int lane = lane_id();
   const uint32_t tail = (cols % 8) ? ((1u << (cols % 8)) - 1u) : 0xffu;
-  for (int64_t r = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave; r < rows;
-       r += (int64_t)gridDim.x * kWaves) {
-  const uint8_t* row = bitmask + r * pc;
-  int cnt = 0;
-  if (pc % 4 == 0 && (uintptr_t)bitmask % 4 == 0) {
-    const uint32_t* w = reinterpret_cast<const uint32_t*>(row);
-    const int64_t nw = pc / 4;
-    const uint32_t last = 0x00ffffffu | (tail << 24);
-    for (int64_t i = lane; i < nw; i += kWave) {
-      uint32_t bits = w[i];
-      if (i == nw - 1) bits &= last;
-      cnt += __popc(bits);
+  for (int64_t r = first_row; r < rows; r += row_stride) {
+    const uint8_t* row = bitmask + r * pc;
+    int cnt = 0;
+    if (pc % 4 == 0 && (uintptr_t)bitmask % 4 == 0) {
+      const uint32_t* w = reinterpret_cast<const uint32_t*>(row);
+      const int64_t nw = pc / 4;
+      const uint32_t last = 0x00ffffffu | (tail << 24);
+      for (int64_t i = lane; i < nw; i += kWave) {
+        uint32_t bits = w[i];
+        if (i == nw - 1) bits &= last;
+        cnt += __popc(bits);
+      }
+    } else {
+      for (int64_t b = lane; b < pc; b += kWave) {
+        uint32_t bits = row[b];
+        if (b == pc - 1) bits &= tail;
+        cnt += __popc(bits);
+      }
     }
-  } else {
-    for (int64_t b = lane; b < pc; b += kWave) {
-      uint32_t bits = row[b];
-      if (b == pc - 1) bits &= tail;
-      cnt += __popc(bits);
-    }
-  }
 #pragma unroll
-  for (int d = kWave / 2; d > 0; d >>= 1) cnt += __shfl_xor(cnt, d, kWave);
-  if (lane == 0) counts[r] = cnt;
+    for (int d = kWave / 2; d > 0; d >>= 1) cnt += __shfl_xor(cnt, d, kWave);
+    if (lane == 0) counts[r] = cnt;
   }
+}
+
+__global__ void __launch_bounds__(kBlock)
+bitmask_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t* __restrict__ counts,
+                        int64_t rows, int64_t cols, int64_t pc) {
+  popcount_rows(bitmask, counts, rows, cols, pc, (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave,
+                (int64_t)gridDim.x * kWaves);
 }
 
 // exclusive scan of counts[rows] -> offsets[rows], total; single workgroup, 8
 // neighbouring rows per thread and step
 constexpr int kScanThreads = 1024, kScanPer = 8;
-__global__ void __launch_bounds__(kScanThreads)
-row_offsets_kernel(const int64_t* __restrict__ counts, int64_t* __restrict__ offsets,
-                   int64_t* __restrict__ total, int64_t rows, const int* only_if) {
-  if (only_if && *only_if == 0) return;
-  __shared__ int64_t wsum[kScanThreads / kWave];
+__device__ __forceinline__ void scan_rows(const int64_t* __restrict__ counts,
+                                          int64_t* __restrict__ offsets,
+                                          int64_t* __restrict__ total, int64_t rows,
+                                          int64_t* wsum) {
   int64_t carry = 0;
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   for (int64_t base = 0; base < rows; base += kScanThreads * kScanPer) {
@@ -242,6 +246,32 @@ row_offsets_kernel(const int64_t* __restrict__ counts, int64_t* __restrict__ off
     __syncthreads();
   }
   if (threadIdx.x == 0 && total) *total = carry;
+}
+
+__global__ void __launch_bounds__(kScanThreads)
+row_offsets_kernel(const int64_t* __restrict__ counts, int64_t* __restrict__ offsets,
+                   int64_t* __restrict__ total, int64_t rows) {
+  __shared__ int64_t wsum[kScanThreads / kWave];
+  scan_rows(counts, offsets, total, rows, wsum);
+}
+
+// What follows a 2:4 streaming pass (sparse24_scatter_kernel): one workgroup looks at
+// the verdicts the streaming workgroups left, one word each, and publishes the
+// answer in *flag for the scatter kernel behind it.  If a group did not keep exactly
+// 2 of 4 it also prepares the general scatter: per-row popcounts and their prefix.
+__global__ void __launch_bounds__(kScanThreads)
+sparse24_verdict_kernel(const int* __restrict__ verdicts, int64_t n_verdicts, int* __restrict__ flag,
+                        const uint8_t* __restrict__ bitmask, int64_t* __restrict__ counts,
+                        int64_t* __restrict__ offsets, int64_t rows, int64_t cols, int64_t pc) {
+  __shared__ int64_t wsum[kScanThreads / kWave];
+  int bad = 0;
+  for (int64_t i = threadIdx.x; i < n_verdicts; i += kScanThreads) bad |= verdicts[i];
+  bad = __syncthreads_or(bad);
+  if (threadIdx.x == 0) *flag = bad ? 1 : 0;
+  if (!bad) return;
+  popcount_rows(bitmask, counts, rows, cols, pc, threadIdx.x / kWave, kScanThreads / kWave);
+  __syncthreads();  // counts are read back by other wavefronts of this workgroup
+  scan_rows(counts, offsets, nullptr, rows, wsum);
 }
 
 // ------------------------------------------------------------------ sparse-bitmask: compaction
@@ -435,7 +465,7 @@ static bool scatter_wave_ok(const void* values, const uint8_t* bitmask, const vo
 // bitmask is needed: a lane turns E columns' worth of mask bits and E/2 values
 // into one 16-byte store.  Whether the bitmask IS well formed is only known once
 // all of it has been looked at: every lane checks its own bits and raises
-// *malformed otherwise, and the general kernels, enqueued behind this one, do
+// a verdict for its workgroup otherwise, and the general kernels, enqueued behind this one, do
 // their work (and overwrite the output) only if the flag went up.
 template <typename R>
 struct Scatter24 {
@@ -446,7 +476,7 @@ struct Scatter24 {
 template <typename R>
 __global__ void __launch_bounds__(kBlock)
 sparse24_scatter_kernel(const R* __restrict__ values, const uint8_t* __restrict__ bitmask,
-                        R* __restrict__ out, int64_t n_items, int* __restrict__ malformed) {
+                        R* __restrict__ out, int64_t n_items, int* __restrict__ verdicts) {
   constexpr int E = Scatter24<R>::E, U = 2;
   using MaskT = typename Scatter24<R>::MaskT;
   const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
@@ -491,10 +521,10 @@ sparse24_scatter_kernel(const R* __restrict__ values, const uint8_t* __restrict_
       }
     }
   }
-  if (__builtin_amdgcn_ballot_w64(bad) != 0 && lane_id() == 0) atomicOr(malformed, 1);
+  // every workgroup leaves its verdict, good or bad: nothing has to be cleared beforehand
+  const int any_bad = __syncthreads_or(bad);
+  if (threadIdx.x == 0) verdicts[blockIdx.x] = any_bad ? 1 : 0;
 }
-
-__global__ void zero_flag_kernel(int* flag) { *flag = 0; }
 
 // ------------------------------------------------------------------ 2:4 selection
 // Ranking key of one element: |value| compared the way torch.topk compares
@@ -734,6 +764,13 @@ extern "C" int ctmi_unpack_bitmasks(const uint8_t* packed, uint8_t* mask, int64_
 
 extern "C" int64_t ctmi_bitmask_tmp_bytes(int64_t rows) { return (rows < 1 ? 1 : rows) * 8; }
 
+// per-row counts and offsets, the flag, one verdict per streaming workgroup
+extern "C" int64_t ctmi_sparse24_tmp_bytes(int64_t rows, int64_t cols, int32_t elem_size) {
+  const int64_t r = rows < 1 ? 1 : rows, c = cols < 1 ? 1 : cols;
+  const int64_t items = cdiv(r * c, elem_size == 1 ? 16 : 8);
+  return r * 16 + 8 + 4 * cdiv(items, kBlock * 2) + 8;
+}
+
 static int check_elem(int32_t elem_size) {
   CTMI_REQUIRE(elem_size == 1 || elem_size == 2 || elem_size == 4, CTMI_ERR_UNSUPPORTED,
                "element size must be 1, 2 or 4 bytes, got %d", elem_size);
@@ -769,8 +806,7 @@ extern "C" int ctmi_bitmask_count(const void* x, int32_t elem_size, int32_t is_f
     hipLaunchKernelGGL(bitmask_count_kernel<uint32_t>, grid, kBlock, 0, st, (const uint32_t*)x,
                        is_float ? 0x7FFFFFFFu : 0xFFFFFFFFu, bitmask, counts, rows, cols, pc);
   }
-  hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, row_offsets, total_nnz, rows,
-                     (const int*)nullptr);
+  hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, row_offsets, total_nnz, rows);
   return check_launch("ctmi_bitmask_count");
 }
 
@@ -823,29 +859,31 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
     if (try_24 && nvalues * 2 == numel && cols % 8 == 0 && numel % e == 0 && (uintptr_t)out % 16 == 0 &&
         (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 2 == 0 && numel / e < (1ll << 40)) {
       int* flag = (int*)(offs + rows);
+      int* verdicts = flag + 2;
       const int64_t n_items = numel / e;
       const unsigned g24 = (unsigned)cdiv(n_items, kBlock * 2);
-      hipLaunchKernelGGL(zero_flag_kernel, 1, 1, 0, st, flag);
       if (elem_size == 1)
         hipLaunchKernelGGL(sparse24_scatter_kernel<uint8_t>, g24, kBlock, 0, st,
-                           (const uint8_t*)values, bitmask, (uint8_t*)out, n_items, flag);
+                           (const uint8_t*)values, bitmask, (uint8_t*)out, n_items, verdicts);
       else if (elem_size == 2)
         hipLaunchKernelGGL(sparse24_scatter_kernel<uint16_t>, g24, kBlock, 0, st,
-                           (const uint16_t*)values, bitmask, (uint16_t*)out, n_items, flag);
+                           (const uint16_t*)values, bitmask, (uint16_t*)out, n_items, verdicts);
       else
         hipLaunchKernelGGL(sparse24_scatter_kernel<uint32_t>, g24, kBlock, 0, st,
-                           (const uint32_t*)values, bitmask, (uint32_t*)out, n_items, flag);
+                           (const uint32_t*)values, bitmask, (uint32_t*)out, n_items, verdicts);
+      hipLaunchKernelGGL(sparse24_verdict_kernel, 1, kScanThreads, 0, st, verdicts, (int64_t)g24,
+                         flag, bitmask, counts, offs, rows, cols, pc);
       only_if = flag;
-      // the kernels below now only run in the rare malformed case: keep their
-      // grids small, an empty launch costs by the workgroup
+      // the scatter below now only runs in the rare malformed case: keep its grid
+      // small, an empty launch costs by the workgroup
       if (grid > 1024) grid = 1024;
-      if (pop_grid > 512) pop_grid = 512;
+    } else {
+      if (pop_grid > (1 << 20)) pop_grid = 1 << 20;
+      hipLaunchKernelGGL(bitmask_popcount_kernel, (unsigned)pop_grid, kBlock, 0, st, bitmask,
+                         counts, rows, cols, pc);
+      hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, offs,
+                         (int64_t*)nullptr, rows);
     }
-    if (pop_grid > (1 << 20)) pop_grid = 1 << 20;
-    hipLaunchKernelGGL(bitmask_popcount_kernel, (unsigned)pop_grid, kBlock, 0, st, bitmask,
-                       counts, rows, cols, pc, only_if);
-    hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, offs, (int64_t*)nullptr,
-                       rows, only_if);
     row_offsets = offs;
   }
 #define CTMI_SCATTER(R)                                                                           \

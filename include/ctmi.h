@@ -217,7 +217,9 @@ int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_si
  * of every 4 columns (what the format holds) needs no prefix sums and is
  * expanded in one streaming pass; the general path of ctmi_bitmask_decompress is
  * enqueued behind it and does its work only if some group turned out not to
- * keep exactly 2.  tmp: ctmi_bitmask_tmp_bytes(rows) + rows*8 + 8 bytes. */
+ * keep exactly 2.  tmp: ctmi_sparse24_tmp_bytes(rows, cols, elem_size) bytes of
+ * device scratch; it needs no initialisation. */
+int64_t ctmi_sparse24_tmp_bytes(int64_t rows, int64_t cols, int32_t elem_size);
 int ctmi_sparse24_decompress(const void* values, int64_t nvalues, int32_t elem_size,
                              const uint8_t* bitmask, void* out, void* tmp, int64_t rows,
                              int64_t cols, void* stream);
