@@ -217,6 +217,9 @@ SIGNATURES = {
     "ctmi_mxfp4_convert_exp_scale": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_void_p]),
     "ctmi_column_groups": (c_int32, [c_void_p, c_int64, c_int64, c_void_p, c_void_p]),
     "ctmi_sparse24_tmp_bytes": (c_int64, [c_int64, c_int64, c_int32]),
+    "ctmi_observe_nvfp4_compress": (
+        c_int32, [c_void_p, c_int32, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
     "ctmi_dynamic_qdq_supported": (
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32],
     ),

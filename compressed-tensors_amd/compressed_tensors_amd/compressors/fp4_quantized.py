@@ -113,6 +113,41 @@ class NVFP4PackedCompressor(BaseQuantizationCompressor):
             packed = packed.to(device)
         return {"weight_packed": packed}
 
+    def observe_and_compress_weight(
+        self, weight: Tensor, quantization_args: QuantizationArgs,
+        global_scale: Optional[Tensor] = None, device: Optional[torch.device] = None,
+    ) -> Dict[str, Tensor]:
+        """One-shot compression of a weight that has no scales yet: the global scale
+        (generate_gparam of the tensor's min / max, helpers.py:414-434, unless given),
+        then the group scales of the min-max observer and compress_weight in one pass
+        over the weight.  Returns weight_packed, weight_scale and weight_global_scale."""
+        from compressed_tensors_amd.quantization.helpers import generate_gparam, minmax
+
+        args = quantization_args
+        weight = to_gpu(weight)
+        if weight.ndim != 2:
+            raise ValueError(f"expected a 2-D weight, got shape {tuple(weight.shape)}")
+        w = weight.contiguous()
+        rows, cols = w.shape
+        if args.group_size != 16 or cols % 16 or w.data_ptr() % (8 * w.element_size()):
+            raise NotImplementedError("one-pass nvfp4 compression needs groups of 16 columns")
+        if global_scale is None:
+            mn, mx = minmax(w, rows, cols)
+            global_scale = generate_gparam(mn.reshape(1), mx.reshape(1))
+        gs = to_gpu(global_scale).to(torch.float32).reshape(-1).contiguous()
+        packed = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
+        scale = torch.empty((rows, cols // 16), dtype=torch.float8_e4m3fn, device=w.device)
+        _lib.check(
+            _lib.load().ctmi_observe_nvfp4_compress(
+                w.data_ptr(), _lib.dtype_code(w.dtype), rows, cols, gs.data_ptr(),
+                packed.data_ptr(), scale.data_ptr(), _lib.stream_of(w.device),
+            )
+        )
+        out = {"weight_packed": packed, "weight_scale": scale, "weight_global_scale": gs}
+        if device is not None:
+            out = {k: v.to(device) for k, v in out.items()}
+        return out
+
     def decompress_weight(
         self,
         compressed_data: Dict[str, Tensor],

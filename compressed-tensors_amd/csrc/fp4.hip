@@ -480,6 +480,49 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
   }
 }
 
+// One-shot nvfp4 compression of a weight whose global scale is known: group scales
+// (min-max observer + calculate_qparams, tests/mock_observer.py:38-113,
+// helpers.py:101-120) and NVFP4PackedCompressor.compress_weight
+// (fp4_quantized.py:84-107) with those scales and their all-zero zero points, the
+// weight read once.
+template <typename XT>
+__global__ void __launch_bounds__(kFp4Block)
+nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
+                              const float* __restrict__ gscale, uint32_t* __restrict__ packed,
+                              uint8_t* __restrict__ scale_out, uint32_t nvec) {
+  constexpr int B = kFp4Block, U = 2;
+  const float gs = gscale[0];
+  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  Vec<typename XT::raw, 8> xv[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)(v < nvec ? v : nvec - 1) * 8);
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    float sv;
+    uint8_t code;
+    if constexpr (sizeof(typename XT::raw) == 2) {
+      const uint32_t m = group_umax(2, absmax8_bits<XT>(xv[k]));
+      constexpr uint32_t kInf = XT::id == CTMI_BF16 ? 0x7f80u : 0x7c00u;
+      code = nvfp4_group_scale<XT>(XT::to_f32((typename XT::raw)m), m > kInf, gs, &sv);
+    } else {
+      float lo = __builtin_inff(), hi = -__builtin_inff();
+      bool unordered = false;
+      vec_minmax<XT>(xv[k], &lo, &hi, &unordered);
+      group_minmax(2, &lo, &hi);
+      code = nvfp4_group_scale<XT>(__builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f),
+                                   group_any(2, unordered), gs, &sv);
+    }
+    if (v < nvec) {
+      if ((threadIdx.x & 1) == 0) scale_out[v >> 1] = code;
+      __builtin_nontemporal_store(nvfp4_codes<XT, true>(xv[k], sv / gs, 0.0f), packed + v);
+    }
+  }
+}
+
 bool nvfp4_dynamic_try(const void* x, int x_dtype, void* out, int64_t rows, int64_t cols,
                        int64_t blk_cols, const float* gscale, void* scale_out, void* zp_out,
                        const QpCfg& c, hipStream_t st) {
@@ -650,4 +693,25 @@ extern "C" int ctmi_nvfp4_decompress(const uint8_t* packed, void* out, int32_t o
   a.q.ct = a.q.dt;
   hipLaunchKernelGGL(nvfp4_decompress_generic_kernel, grid_for(rows * cols, 256), 256, 0, st, a);
   return check_launch("ctmi_nvfp4_decompress");
+}
+
+extern "C" int ctmi_observe_nvfp4_compress(const void* x, int32_t x_dtype, int64_t rows,
+                                           int64_t cols, const float* global_scale,
+                                           uint8_t* packed, uint8_t* scale, void* stream) {
+  CTMI_REQUIRE(rows >= 1 && cols >= 1, CTMI_ERR_VALUE, "cannot observe an empty tensor");
+  int rc = check_float3(x_dtype, "nvfp4 input");
+  if (rc) return rc;
+  CTMI_REQUIRE(cols % 16 == 0, CTMI_ERR_UNSUPPORTED, "columns must come in groups of 16");
+  CTMI_REQUIRE(x && global_scale && packed && scale, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)packed % 4 == 0,
+               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+  const int64_t nvec = rows * cols / 8;
+  const int64_t grid = cdiv(nvec, kFp4Block * 2);
+  CTMI_REQUIRE(nvec < (1ll << 32) && grid < (1ll << 31), CTMI_ERR_UNSUPPORTED, "tensor too large");
+  hipStream_t st = (hipStream_t)stream;
+  auto* out = (uint32_t*)packed;
+  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_observe_compress_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, global_scale, out, scale, (uint32_t)nvec);
+  else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_observe_compress_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, global_scale, out, scale, (uint32_t)nvec);
+  else hipLaunchKernelGGL(nvfp4_observe_compress_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, global_scale, out, scale, (uint32_t)nvec);
+  return check_launch("ctmi_observe_nvfp4_compress");
 }

@@ -35,7 +35,10 @@ gparam_kernel(const void* __restrict__ mn, const void* __restrict__ mx, int mt,
     const float a = nan_min(load_f32(mn, mt, i), 0.0f);
     const float b = nan_max(load_f32(mx, mt, i), 0.0f);
     const float m = nan_max(fabsf(a), fabsf(b));
-    out[i] = round_to(2688.0f / m, mt);  // 448 * 6 / max|x| in the min/max dtype, then -> fp32
+    // `448 * 6 / max_val_pos` with a Python float on the left runs as
+    // max_val_pos.reciprocal() * 2688 (Tensor.__rtruediv__): two roundings in the
+    // min / max dtype, then the cast to fp32
+    out[i] = round_to(round_to(1.0f / m, mt) * 2688.0f, mt);
   }
 }
 

@@ -247,7 +247,9 @@ int ctmi_calculate_qparams(const void* min_vals, const void* max_vals, int32_t m
                            int32_t symmetric, const float* global_scale, void* scale,
                            int32_t scale_dtype, void* zero_point, int32_t zp_dtype, void* stream);
 
-/* A16.  generate_gparam (helpers.py:414-434): out[i] = fp32(448*6 / max|min,max|). */
+/* A16.  generate_gparam (helpers.py:414-434): out[i] = fp32(448*6 / max|min,max|),
+ * evaluated as torch evaluates `float / tensor`: reciprocal, then the product, each
+ * rounded to the dtype of min / max. */
 int ctmi_generate_gparam(const void* min_vals, const void* max_vals, int32_t mm_dtype, int64_t n,
                          float* out, void* stream);
 
@@ -300,6 +302,15 @@ int ctmi_observe_pack_quantized_many(const ctmi_observe_pack_job* jobs, int64_t 
 int ctmi_observe_pack_quantized(const void* x, int32_t x_dtype, int64_t rows, int64_t cols,
                                 int64_t blk_cols, int32_t num_bits, int32_t symmetric,
                                 int32_t* packed, void* scale, int8_t* zero_point, void* stream);
+
+/* The same for the nvfp4 format with a known global scale: group-16 scales of the
+ * observer (tests/mock_observer.py:38-113, helpers.py:101-120: fp8 e4m3, zeros
+ * replaced by 0.125) and NVFP4PackedCompressor.compress_weight
+ * (fp4_quantized.py:84-107) with those scales and their zero points (all zero),
+ * the weight read once.  packed: uint8 [rows, cols/2]; scale: fp8 [rows, cols/16]. */
+int ctmi_observe_nvfp4_compress(const void* x, int32_t x_dtype, int64_t rows, int64_t cols,
+                                const float* global_scale, uint8_t* packed, uint8_t* scale,
+                                void* stream);
 
 /* A26.  Dynamic activation quantization in one pass (forward_quantize with
  * args.dynamic, quantization/lifecycle/forward.py:414-451): the scales of

@@ -388,6 +388,37 @@ def test_nvfp4_compressor(shape, dtype, gpu):
     assert dense.dtype == torch.bfloat16
 
 
+@pytest.mark.parametrize("shape,dtype", [((64, 256), torch.bfloat16), ((37, 48), torch.bfloat16),
+                                         ((32, 4112), torch.float16), ((8, 64), torch.float32)])
+def test_nvfp4_observe_and_compress_in_one_pass(shape, dtype, gpu):
+    """global scale, then group scales + codes from one kernel: the oracle's
+    generate_gparam, observe_weight and nvfp4_compress, bit for bit"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("one-shot nvfp4", shape, dtype)
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(52)
+    w = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+    w[0, :16] = 0.0                       # a group of zeros: the 0.125 replacement
+    w[0, 17] = -0.0
+    w[1, :16] *= 1e-4                     # a scale in the subnormal range of fp8
+    w[2, 3] *= 40                         # an outlier that sets the global scale
+    gs = oq.generate_gparam(*[t.reshape(1) for t in torch.aminmax(w)])
+    scale, zp = oq.observe_weight(w, oargs, global_scale=gs)
+    want = op.nvfp4_compress(w, scale, gs, oargs, zero_point=zp)
+    comp = BaseCompressor.load_from_registry("nvfp4-pack-quantized")
+    got = comp.observe_and_compress_weight(w.to(gpu), args)
+    assert set(got) == {"weight_packed", "weight_scale", "weight_global_scale"}
+    assert_bit_equal(got["weight_global_scale"], gs, "global scale")
+    assert_bit_equal(got["weight_scale"], scale, "group scales")
+    assert_bit_equal(got["weight_packed"], want, "codes")
+    again = comp.observe_and_compress_weight(w.to(gpu), args, global_scale=gs.to(gpu))
+    assert_bit_equal(again["weight_packed"], want, "codes, global scale given")
+    with pytest.raises(NotImplementedError):
+        comp.observe_and_compress_weight(w.to(gpu)[:, :24].contiguous(), args)
+
+
 @pytest.mark.parametrize("scale_value,global_scale", [(1.0, 1.0), (0.75, 3.0), (448.0, 1234.5),
                                                       (2.0 ** -9, 0.37)])
 def test_nvfp4_every_bf16_pattern(scale_value, global_scale, gpu):

@@ -495,3 +495,35 @@ def test_column_groups_from_g_idx(cols, group_size, gpu):
     assert_bit_equal(_column_groups(unset.to(gpu), group_size),
                      (torch.arange(cols) // group_size).to(torch.int32), "unset g_idx")
     assert _column_groups(None, group_size) is None
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_generate_gparam_on_many_values(dtype, gpu):
+    """448 * 6 / max|x| as torch evaluates it (reciprocal, then product, each rounded to
+    the dtype of min / max): every positive bfloat16 / float16 pattern, a random draw of
+    float32 values, on either side of zero"""
+    from compressed_tensors_amd import _lib
+    from compressed_tensors_amd.quantization import generate_gparam
+
+    announce("generate_gparam", dtype)
+    if dtype == torch.float32:
+        g = torch.Generator().manual_seed(1)
+        v = torch.cat([torch.rand(50000, generator=g) * 4, torch.randn(50000, generator=g).abs() * 1e-3,
+                       torch.tensor([0.0, 1e-30, 3e38, float("inf")])])
+    else:
+        v = torch.arange(0, 0x7c01 if dtype == torch.float16 else 0x7f81, dtype=torch.int32) \
+            .to(torch.int16).view(dtype).clone()
+    lib = _lib.load()
+    for mn, mx in ((torch.zeros_like(v), v), (-v, v / 2), (v / 4, v)):
+        # the elementwise arithmetic on all values at once, through the C ABI
+        a, b = mn.to(gpu), mx.to(gpu)
+        out = torch.empty(v.numel(), dtype=torch.float32, device=gpu)
+        _lib.check(lib.ctmi_generate_gparam(a.data_ptr(), b.data_ptr(), _lib.dtype_code(dtype), v.numel(),
+                                            out.data_ptr(), _lib.stream_of(gpu)))
+        zero = torch.zeros_like(mn)
+        m = torch.max(torch.abs(torch.min(mn, zero)), torch.abs(torch.max(mx, zero)))
+        assert_bit_equal(out, (448.0 * 6.0 / m).to(torch.float32), "generate_gparam (all values)")
+        # and the wrapper against the oracle, one value per call as the reference uses it
+        for i in range(1, v.numel(), v.numel() // 7):
+            assert_bit_equal(generate_gparam(a[i:i + 1], b[i:i + 1]),
+                             oq.generate_gparam(mn[i:i + 1], mx[i:i + 1]), f"generate_gparam [{i}]")

@@ -402,3 +402,23 @@ def test_mxfp4_scales_closed_form():
     every = mxfp4.convert_mxfp4_exp_scale(torch.arange(256, dtype=torch.int32).to(torch.uint8), torch.float32)
     assert every[0].item() == 2.0 ** -127 and every[127].item() == 1.0 and every[254].item() == 2.0 ** 127
     assert torch.isinf(every[255])
+
+
+# ---------------------------------------------------------------- NVFP4 global scale (A16)
+def test_generate_gparam_is_reciprocal_times_constant():
+    """`448 * 6 / max_val_pos` (helpers.py:431) has a Python float on the left, so torch
+    runs Tensor.__rtruediv__: reciprocal, then the product, each rounded to the tensor's
+    dtype.  For max|x| = 1.1953125 in bfloat16 that is bf16(bf16(0.8366) * 2688) = 2240,
+    where a single division would give bf16(2248.78) = 2256."""
+    m = torch.tensor([1.1953125], dtype=torch.bfloat16)
+    got = quant.generate_gparam(-m, m / 2)
+    assert got.dtype == torch.float32 and got.shape == (1,)
+    assert got.item() == 2240.0
+    r = torch.tensor(1.0 / 1.1953125).to(torch.bfloat16)
+    assert (r.float() * 2688.0).to(torch.bfloat16).item() == 2240.0
+    assert torch.tensor(2688.0 / 1.1953125).to(torch.bfloat16).item() == 2256.0
+    # and on every positive normal bfloat16: the two-step closed form
+    v = torch.arange(0x0080, 0x7f80, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    closed = ((1.0 / v.float()).to(torch.bfloat16).float() * 2688.0).to(torch.bfloat16).float()
+    every = (448.0 * 6.0 / v).float()
+    assert torch.equal(every, closed)
