@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from gpu_util import announce, assert_bit_equal, bits as bits_of
+from oracle import pack as op
 from oracle import quant as oq
 
 pytestmark = pytest.mark.gpu
@@ -527,3 +528,146 @@ def test_generate_gparam_on_many_values(dtype, gpu):
         for i in range(1, v.numel(), v.numel() // 7):
             assert_bit_equal(generate_gparam(a[i:i + 1], b[i:i + 1]),
                              oq.generate_gparam(mn[i:i + 1], mx[i:i + 1]), f"generate_gparam [{i}]")
+
+
+QP_SPECS = [
+    dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128),
+    dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=128),
+    dict(num_bits=8, type="int", symmetric=True, strategy="channel"),
+    dict(num_bits=8, type="int", symmetric=False, strategy="channel"),
+    dict(num_bits=8, type="float", symmetric=True, strategy="channel"),
+    dict(num_bits=8, type="float", symmetric=False, strategy="channel"),
+    dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16),
+    dict(num_bits=2, type="int", symmetric=False, strategy="channel"),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "f16", "f32"])
+@pytest.mark.parametrize("spec", QP_SPECS, ids=[f"{s['type']}{s['num_bits']}-{'sym' if s['symmetric'] else 'asym'}" for s in QP_SPECS])
+def test_calculate_qparams_on_many_pairs(spec, dtype, gpu):
+    """calculate_qparams on 200 000 (min, max) pairs per scheme and dtype: magnitudes from
+    1e-9 to 1e4, one-sided ranges, exact zeros, equal ends, infinities and NaNs"""
+    from compressed_tensors_amd.quantization import calculate_qparams
+
+    announce("calculate_qparams many", spec, dtype)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(17)
+    n = 200_000
+    mag = 10.0 ** (torch.rand(n, generator=g) * 13 - 9)
+    lo = -mag * torch.rand(n, generator=g)
+    hi = mag * torch.rand(n, generator=g)
+    kind = torch.randint(0, 8, (n,), generator=g)
+    lo = torch.where(kind == 0, hi * 0.5, lo)          # all positive
+    hi = torch.where(kind == 1, lo * 0.5, hi)          # all negative
+    lo = torch.where(kind == 2, torch.zeros(n), lo)
+    hi = torch.where(kind == 3, lo, hi)                # equal ends
+    special = torch.tensor([0.0, -0.0, float("inf"), -float("inf"), float("nan"), 1e-45, 65504.0, 3e38])
+    lo[:8], hi[:8] = special, special.flip(0)
+    lo[8:16], hi[8:16] = -special.abs(), special.abs()
+    lo, hi = torch.minimum(lo, hi).to(dtype), torch.maximum(lo, hi).to(dtype)
+    lo[4], hi[11] = float("nan"), float("nan")
+    gs = o_gs = None
+    if spec["strategy"] == "tensor_group":
+        o_gs = torch.tensor([37.5], dtype=torch.float32)
+        gs = o_gs.to(gpu)
+    o_scale, o_zp = oq.calculate_qparams(lo, hi, oargs, global_scale=o_gs)
+    scale, zp = calculate_qparams(lo.to(gpu), hi.to(gpu), args, global_scale=gs)
+    nan = torch.isnan(o_scale.float())
+    assert torch.equal(torch.isnan(scale.float()).cpu(), nan)
+    assert_bit_equal(torch.where(nan.to(gpu), torch.zeros_like(scale.float()), scale.float()),
+                     torch.where(nan, torch.zeros_like(o_scale.float()), o_scale.float()), "scale")
+    assert scale.dtype == o_scale.dtype and zp.dtype == o_zp.dtype
+    # where the scale is NaN, or an end is infinite (inf / inf), the zero point is a cast
+    # of a NaN to int8 or fp8: not defined / sign and payload not part of the contract
+    ok = ~nan & torch.isfinite(lo.float()) & torch.isfinite(hi.float())
+    assert torch.equal(zp.cpu().view(torch.uint8 if zp.element_size() == 1 else zp.dtype)[ok],
+                       o_zp.view(torch.uint8 if o_zp.element_size() == 1 else o_zp.dtype)[ok]), "zero points"
+
+
+@pytest.mark.parametrize("xdt,sdt", [(torch.bfloat16, torch.bfloat16), (torch.float16, torch.float16),
+                                     (torch.bfloat16, torch.float32), (torch.float16, torch.bfloat16)],
+                         ids=["bf16", "f16", "bf16-f32scale", "f16-bf16scale"])
+@pytest.mark.parametrize("bits,symmetric", [(4, True), (4, False), (8, True), (8, False)])
+def test_int_codes_on_every_16_bit_pattern(bits, symmetric, xdt, sdt, gpu):
+    """all 65 536 patterns of a 16-bit float as inputs, one row of 128 per scale, 512
+    scales from 1e-12 to 1e6 (and the clamp floor, and powers of two), random zero
+    points: quantize, fake_quantize, pack-quantized compress and decompress against the
+    oracle (NaN inputs have no defined integer code and are left out of the code checks)"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.quantization import fake_quantize, quantize
+
+    announce("every 16-bit pattern", bits, symmetric, xdt, sdt)
+    spec = dict(num_bits=bits, type="int", symmetric=symmetric, strategy="group", group_size=128)
+    args, oargs = _pair(spec)
+    x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(xdt).reshape(512, 128).clone()
+    g = torch.Generator().manual_seed(bits * 2 + symmetric)
+    scale = (10.0 ** (torch.rand(512, 1, generator=g) * 18 - 12))
+    scale[:4, 0] = torch.tensor([1.1920928955078125e-07, 1.0, 0.5, 2.0 ** -20])
+    scale = scale.to(sdt)
+    lo, hi = -(1 << (bits - 1)), (1 << (bits - 1)) - 1
+    zp = None if symmetric else torch.randint(lo, hi + 1, (512, 1), generator=g).to(torch.int8)
+    dev = lambda t: None if t is None else t.to(gpu)
+    finite_code = ~torch.isnan(x.float())
+    want_q = oq.quantize(x, scale, zp, oargs, dtype=torch.int8)
+    got_q = quantize(x.to(gpu), dev(scale), dev(zp), args, dtype=torch.int8).cpu()
+    assert torch.equal(got_q[finite_code], want_q[finite_code]), "quantize"
+    want_fq = oq.fake_quantize(x, scale, zp, oargs)
+    got_fq = fake_quantize(x.to(gpu), dev(scale), dev(zp), args).cpu()
+    nan = torch.isnan(want_fq.float())
+    assert torch.equal(torch.isnan(got_fq.float()), nan), "fake_quantize NaNs"
+    assert torch.equal(bits_of(got_fq)[~nan], bits_of(want_fq)[~nan]), "fake_quantize"
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    want_c = op.pack_quantized_compress(x, scale, oargs, zero_point=zp)
+    got_c = comp.compress_weight(weight=x.to(gpu), scale=dev(scale), quantization_args=args, zero_point=dev(zp))
+    from oracle.pack import unpack_from_int32 as o_unpack
+    gc = o_unpack(got_c["weight_packed"].cpu(), bits, torch.Size((512, 128)))
+    wc = o_unpack(want_c["weight_packed"], bits, torch.Size((512, 128)))
+    assert torch.equal(gc[finite_code], wc[finite_code]), "packed codes"
+    data = dict(want_c, weight_scale=scale)
+    want_d = op.pack_quantized_decompress(dict(data), oargs)
+    got_d = comp.decompress_weight({k: v.to(gpu) for k, v in data.items()}, quantization_args=args)
+    assert_bit_equal(got_d, want_d, "decompress")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_scales_computed_in_kernels_for_every_maximum(dtype, gpu):
+    """the kernels that derive scales themselves (one-shot compression, dynamic
+    quantization) against calculate_qparams for every finite positive 16-bit value as the
+    group maximum: max / 7.5, / 127.5, / 448 and / 6 (the bf16 paths multiply by a reciprocal)"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.quantization.helpers import dynamic_fake_quantize
+
+    announce("in-kernel scales, every maximum", dtype)
+    top = 0x7f80 if dtype == torch.bfloat16 else 0x7c00
+    m = torch.arange(1, top, dtype=torch.int32).to(torch.int16).view(dtype)
+    rows = m.numel()
+    x = torch.zeros(rows, 128, dtype=dtype)
+    x[:, 5] = m
+    x[::2, 5] = -m[::2]          # the maximum on either side
+    x[:, 77] = (m.float() * 0.37).to(dtype)
+    xg = x.to(gpu)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    for bits in (4, 8):
+        spec = dict(num_bits=bits, type="int", symmetric=True, strategy="group", group_size=128)
+        args, oargs = _pair(spec)
+        o_scale, _ = oq.observe_weight(x, oargs)
+        got = comp.observe_and_compress_weight(xg, args)
+        assert_bit_equal(got["weight_scale"], o_scale, f"one-shot int{bits} scales")
+        want = op.pack_quantized_compress(x, o_scale, oargs)
+        assert_bit_equal(got["weight_packed"], want["weight_packed"], f"one-shot int{bits} codes")
+    for spec in (dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=128, dynamic=True),
+                 dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=128, dynamic=True)):
+        args, oargs = _pair(spec)
+        o_scale, o_zp = oq.compute_dynamic_scales_and_zp(x, oargs)
+        out, scale, zp = dynamic_fake_quantize(xg, args, None, return_qparams=True)
+        assert_bit_equal(scale, o_scale, f"dynamic {spec['type']}8 scales")
+        assert_bit_equal(out, oq.fake_quantize(x, o_scale, o_zp, oargs), f"dynamic {spec['type']}8 qdq")
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16, dynamic="local")
+    args, oargs = _pair(spec)
+    for gs_value in (1.0, 37.5, 2688.0 / 3.0):
+        o_gs = torch.tensor([gs_value], dtype=torch.float32)
+        o_scale, o_zp = oq.compute_dynamic_scales_and_zp(x, oargs, global_scale=o_gs)
+        out, scale, zp = dynamic_fake_quantize(xg, args, o_gs.to(gpu), return_qparams=True)
+        assert_bit_equal(scale, o_scale, f"dynamic nvfp4 scales, gs {gs_value}")
+        assert_bit_equal(out, oq.fake_quantize(x, o_scale, o_zp, oargs, global_scale=o_gs),
+                         f"dynamic nvfp4 qdq, gs {gs_value}")
