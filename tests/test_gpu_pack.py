@@ -537,3 +537,51 @@ def test_batches_replay_from_a_captured_graph(gpu):
         for i, (a, b) in enumerate(zip(got, want)):
             assert torch.equal(a, b), f"replay {replay}, tensor {i}"
         assert all(torch.equal(p, q) for p, q in zip(batch.packed, one_shot.packed))
+
+
+def test_random_shapes_sweep(gpu):
+    """random shapes, bit widths and packed dims for pack / unpack; random shapes, group
+    sizes, dtypes and symmetry for the pack-quantized compressor (vector, ragged and
+    generic kernels alike), against the oracle"""
+    from compressed_tensors_amd.compressors import BaseCompressor, pack_to_int32, unpack_from_int32
+
+    g = torch.Generator().manual_seed(77)
+    ri = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    for case in range(40):
+        bits, dim = ri(1, 8), ri(0, 1)
+        rows, cols = ri(1, 40), ri(1, 300)
+        announce("pack sweep", case, bits, dim, (rows, cols))
+        lo, hi = -(1 << (bits - 1)), (1 << (bits - 1)) - 1
+        v = torch.randint(lo, hi + 1, (rows, cols), generator=g).to(torch.int8)
+        packed = pack_to_int32(v.to(gpu), bits, packed_dim=dim)
+        assert_bit_equal(packed, op.pack_to_int32(v, bits, packed_dim=dim), f"pack {case}")
+        assert_bit_equal(unpack_from_int32(packed, bits, torch.Size((rows, cols)), packed_dim=dim), v,
+                         f"unpack {case}")
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    for case in range(40):
+        bits = (4, 8, 4, 2, 6)[case % 5]
+        group = (8, 16, 32, 64, 128, 24, 4)[case % 7]
+        rows, n_groups = ri(1, 70), ri(1, 40)
+        cols = group * n_groups
+        dtype = (torch.bfloat16, torch.float16, torch.float32)[case % 3]
+        symmetric = bool(case % 2)
+        strategy = ("group", "channel", "tensor")[ri(0, 2)]
+        spec = dict(num_bits=bits, type="int", symmetric=symmetric, strategy=strategy)
+        if strategy == "group":
+            spec["group_size"] = group
+        announce("pack-quantized sweep", case, spec, (rows, cols), dtype)
+        args, oargs = _pair(spec)
+        w = (torch.randn(rows, cols, generator=g) * 0.02).to(dtype)
+        scale, zp = oq.observe_weight(w, oargs)
+        zp_arg = None if symmetric else zp
+        want = op.pack_quantized_compress(w, scale, oargs, zero_point=zp_arg)
+        got = comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+                                   zero_point=None if zp_arg is None else zp_arg.to(gpu))
+        assert set(got) == set(want)
+        for k in want:
+            assert_bit_equal(got[k], want[k], f"{k} {case}")
+        data = dict(want, weight_scale=scale)
+        if not symmetric and strategy == "tensor":
+            data["weight_zero_point"] = zp
+        dense = comp.decompress_weight({k: v.to(gpu) for k, v in data.items()}, quantization_args=args)
+        assert_bit_equal(dense, op.pack_quantized_decompress(dict(data), oargs), f"decompress {case}")

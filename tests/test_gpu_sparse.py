@@ -209,3 +209,41 @@ def test_sparse24_decompress_of_a_bitmask_that_is_not_2_4(dtype, gpu):
     bitmask = pack_bitmasks(mask.to(gpu))
     dense = sparse24_bitmask_decompress(values.to(gpu), bitmask, torch.Size((rows, cols)))
     assert_bit_equal(dense, x, "general path behind the 2:4 kernel")
+
+
+def test_random_shapes_sweep(gpu):
+    """60 random shapes (row lengths around the 8 / 16 / 1024 / 16384 column boundaries of
+    the kernels, 1 to 70 rows, four dtypes, sparsities from 0 to 1): both sparse formats
+    against the oracle"""
+    from compressed_tensors_amd.compressors import (
+        bitmask_compress, bitmask_decompress, get_24_bytemasks, sparse24_bitmask_compress,
+        sparse24_bitmask_decompress,
+    )
+
+    g = torch.Generator().manual_seed(2024)
+    edges = [8, 16, 64, 1024, 2048, 4096, 16384]
+    dtypes = [torch.bfloat16, torch.float16, torch.float32, FP8]
+    for case in range(60):
+        rows = int(torch.randint(1, 71, (1,), generator=g))
+        edge = edges[int(torch.randint(0, len(edges), (1,), generator=g))]
+        cols = max(1, edge + int(torch.randint(-17, 18, (1,), generator=g)))
+        dtype = dtypes[case % 4]
+        sparsity = float(torch.rand(1, generator=g)) if case % 7 else float(case % 2)
+        announce("sparse sweep", case, (rows, cols), dtype, round(sparsity, 2))
+        x = _sparse_tensor((rows, cols), dtype, sparsity, seed=case)
+        values, bitmask, offsets = bitmask_compress(x.to(gpu))
+        o_values, o_bitmask, o_offsets = osp.bitmask_compress(x)
+        assert_bit_equal(values, o_values, f"values {case}")
+        assert_bit_equal(bitmask, o_bitmask, f"bitmask {case}")
+        assert_bit_equal(offsets, o_offsets, f"offsets {case}")
+        assert_bit_equal(bitmask_decompress(values, bitmask, [rows, cols]),
+                         osp.bitmask_decompress(o_values, o_bitmask, [rows, cols]), f"decompress {case}")
+        cols4 = max(4, cols // 4 * 4)
+        y = _sparse_tensor((rows, cols4), dtype, min(sparsity, 0.6), seed=1000 + case)
+        assert_bit_equal(get_24_bytemasks(y.to(gpu)), osp.get_24_bytemasks(y), f"24 mask {case}")
+        v24, b24 = sparse24_bitmask_compress(y.to(gpu))
+        o_v24, o_b24 = osp.sparse24_bitmask_compress(y)
+        assert_bit_equal(v24, o_v24, f"24 values {case}")
+        assert_bit_equal(b24, o_b24, f"24 bitmask {case}")
+        assert_bit_equal(sparse24_bitmask_decompress(v24, b24, torch.Size((rows, cols4))),
+                         osp.sparse24_bitmask_decompress(o_v24, o_b24, (rows, cols4)), f"24 decompress {case}")
