@@ -40,10 +40,7 @@ def sources():
     return sorted(str(p) for p in CSRC_DIR.glob("*.hip"))
 
 
-def build_library(verbose: bool = False) -> Path:
-    LIB_DIR.mkdir(parents=True, exist_ok=True)
-    tmp = LIB_PATH.with_suffix(".so.tmp")
-    cmd = [HIPCC, *FLAGS, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", *sources(), "-o", str(tmp)]
+def _run(cmd, verbose):
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -53,6 +50,26 @@ def build_library(verbose: bool = False) -> Path:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build_library(verbose: bool = False, jobs: int = 0) -> Path:
+    """compile every source file (one hipcc process each, `jobs` at a time) and link"""
+    from concurrent.futures import ThreadPoolExecutor
+
+    LIB_DIR.mkdir(parents=True, exist_ok=True)
+    obj_dir = LIB_DIR / "obj"
+    obj_dir.mkdir(exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+    srcs = sources()
+    objs = [str(obj_dir / (Path(src).stem + ".o")) for src in srcs]
+    jobs = jobs or min(len(srcs), os.cpu_count() or 1, 16)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(
+            lambda so: _run([HIPCC, *compile_flags, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", "-c", so[0],
+                             "-o", so[1]], verbose),
+            zip(srcs, objs)))
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", str(tmp)], verbose)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 
