@@ -29,6 +29,7 @@
 namespace ctmi {
 
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kHadThreads = 256;
@@ -251,7 +252,7 @@ __global__ void __launch_bounds__(kHadThreads) hadamard_mfma_kernel(HadArgs a) {
 //                    + {4..7}, so a lane ends up with 8 neighbouring outputs,
 //                    one 16-byte global store.
 // Sign vectors are used as signs: their entries must be +1 or -1.
-template <int B>
+template <int B, bool HALF>
 __global__ void __launch_bounds__(kHadThreads)
 hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
                      const uint16_t* __restrict__ mbt, const float* __restrict__ s_in,
@@ -261,6 +262,9 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // uniform: loop control stays scalar
   const int l16 = lane & 15, lq = lane >> 4;
+  // HALF: float16 tensors on v_mfma_f32_16x16x32_f16; the matrix arrives in bfloat16
+  // and converts to float16 exactly (more significand bits, entries of order 1)
+  using frag_t = typename std::conditional<HALF, f16x8_t, bf16x8_t>::type;
 
   // The matrix fragments are the same in every wave of the workgroup: each wave
   // fetches a quarter of them, and all pick up the whole set from LDS.
@@ -268,15 +272,21 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   for (int f = wave; f < 2 * NP * KS; f += kHadWaves) {
     const int nt = f / KS, ks = f % KS;
     const int col = 32 * (nt / 2) + 8 * (l16 / 4) + 4 * (nt % 2) + (l16 % 4);
-    frag_lds[f][lane] = *reinterpret_cast<const u32x4_t*>(mbt + col * B + 32 * ks + 8 * lq);
+    u32x4_t m = *reinterpret_cast<const u32x4_t*>(mbt + col * B + 32 * ks + 8 * lq);
+    if constexpr (HALF) {
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        m[w] = (uint32_t)f32_to_f16(bf16_lo(m[w])) | ((uint32_t)f32_to_f16(bf16_hi(m[w])) << 16);
+    }
+    frag_lds[f][lane] = m;
   }
   __syncthreads();
-  bf16x8_t mb[2 * NP][KS];
+  frag_t mb[2 * NP][KS];
 #pragma unroll
   for (int nt = 0; nt < 2 * NP; ++nt)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      mb[nt][ks] = __builtin_bit_cast(bf16x8_t, frag_lds[nt * KS + ks][lane]);
+      mb[nt][ks] = __builtin_bit_cast(frag_t, frag_lds[nt * KS + ks][lane]);
   if (s_in || s_out) {
     // Sign bits, XORed into the fragments (bit 15 of each half word).  An absent
     // vector reads the matrix instead (any valid address) and is masked out: no
@@ -303,7 +313,7 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
           const uint32_t lo = (raw_in[ks][2 * w] >> 31) & use_in, hi = (raw_in[ks][2 * w + 1] >> 31) & use_in;
           m.v[w] ^= ((lo << 15) | (hi << 31)) ^ fo;
         }
-        mb[nt][ks] = __builtin_bit_cast(bf16x8_t, m);
+        mb[nt][ks] = __builtin_bit_cast(frag_t, m);
       }
     }
   }
@@ -316,31 +326,40 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   // one) and the stores of whole groups are not either: with a fixed number of
   // memory operations per step the waits can say exactly how many newer
   // operations may still be in flight.
-  auto load_group = [&](int64_t grp, bf16x8_t* xf) {
+  auto load_group = [&](int64_t grp, frag_t* xf) {
     if (grp >= n_full) grp = n_full - 1;
     const uint16_t* src = x + (grp * 16 + l16) * B + 8 * lq;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      xf[ks] = __builtin_bit_cast(bf16x8_t, ldg<uint16_t, 8>(src + 32 * ks));
+      xf[ks] = __builtin_bit_cast(frag_t, ldg<uint16_t, 8>(src + 32 * ks));
   };
-  auto transform_rows = [&](const bf16x8_t* xf, uint16_t* dst, bool keep) {
+  auto pack2 = [&](float lo, float hi) -> uint32_t {
+    if constexpr (HALF) return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
+    else return pack_bf16x2(lo, hi);
+  };
+  auto transform_rows = [&](const frag_t* xf, uint16_t* dst, bool keep) {
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
       f32x4_t a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p][ks], xf[ks], a0, 0, 0, 0);
-        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p + 1][ks], xf[ks], a1, 0, 0, 0);
+        if constexpr (HALF) {
+          a0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(mb[2 * p][ks], xf[ks], a0, 0, 0, 0);
+          a1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(mb[2 * p + 1][ks], xf[ks], a1, 0, 0, 0);
+        } else {
+          a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p][ks], xf[ks], a0, 0, 0, 0);
+          a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p + 1][ks], xf[ks], a1, 0, 0, 0);
+        }
       }
       Vec<uint32_t, 4> o;
-      o.v[0] = pack_bf16x2(a0[0] * inv_sqrt_n, a0[1] * inv_sqrt_n);
-      o.v[1] = pack_bf16x2(a0[2] * inv_sqrt_n, a0[3] * inv_sqrt_n);
-      o.v[2] = pack_bf16x2(a1[0] * inv_sqrt_n, a1[1] * inv_sqrt_n);
-      o.v[3] = pack_bf16x2(a1[2] * inv_sqrt_n, a1[3] * inv_sqrt_n);
+      o.v[0] = pack2(a0[0] * inv_sqrt_n, a0[1] * inv_sqrt_n);
+      o.v[1] = pack2(a0[2] * inv_sqrt_n, a0[3] * inv_sqrt_n);
+      o.v[2] = pack2(a1[0] * inv_sqrt_n, a1[1] * inv_sqrt_n);
+      o.v[3] = pack2(a1[2] * inv_sqrt_n, a1[3] * inv_sqrt_n);
       if (keep) stg<uint16_t, 8>(dst + 32 * p, __builtin_bit_cast(Vec<uint16_t, 8>, o));
     }
   };
-  auto transform_group = [&](int64_t grp, const bf16x8_t* xf) {
+  auto transform_group = [&](int64_t grp, const frag_t* xf) {
     transform_rows(xf, out + (grp * 16 + l16) * B + 8 * lq, true);
   };
 
@@ -350,7 +369,7 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
     // entered with the same operations in flight as on its back edge (one set's
     // loads, then a group's stores): a wait for loads then never has to cover
     // the stores issued after them, which would cost a store latency per group.
-    bf16x8_t xa[KS], xb[KS];
+    frag_t xa[KS], xb[KS];
     int64_t g = first;
     load_group(g, xa);
     load_group(g + stride, xb);
@@ -371,15 +390,15 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
     int64_t row = n_full * 16 + l16;
     const bool keep = row < n_sub;
     if (!keep) row = n_sub - 1;
-    bf16x8_t xt[KS];
+    frag_t xt[KS];
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      xt[ks] = __builtin_bit_cast(bf16x8_t, ldg<uint16_t, 8>(x + row * B + 8 * lq + 32 * ks));
+      xt[ks] = __builtin_bit_cast(frag_t, ldg<uint16_t, 8>(x + row * B + 8 * lq + 32 * ks));
     transform_rows(xt, out + row * B + 8 * lq, keep);
   }
 }
 
-template <int B>
+template <int B, bool HALF>
 static int launch_had_rows(const HadArgs& a, hipStream_t st) {
   const int64_t groups = cdiv(a.n_sub, 16);
   const int64_t wgs = cdiv(groups, kHadWaves);
@@ -388,7 +407,7 @@ static int launch_had_rows(const HadArgs& a, hipStream_t st) {
   // needs some 190 registers, more below)
   const int64_t cap = 256 * (B == 32 ? 4 : 2);
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
-  hipLaunchKernelGGL(hadamard_rows_kernel<B>, grid, kHadThreads, 0, st, (const uint16_t*)a.x,
+  hipLaunchKernelGGL((hadamard_rows_kernel<B, HALF>), grid, kHadThreads, 0, st, (const uint16_t*)a.x,
                      (uint16_t*)a.out, a.mbt, a.s_in, a.s_out, a.n_sub, 1.0f / a.sqrt_n);
   return CTMI_OK;
 }
@@ -780,8 +799,13 @@ extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, i
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (io_dtype == CTMI_BF16 && a_dim == 1) {
-    rc = b_dim == 32 ? launch_had_rows<32>(a, st)
-                     : (b_dim == 64 ? launch_had_rows<64>(a, st) : launch_had_rows<128>(a, st));
+    rc = b_dim == 32 ? launch_had_rows<32, false>(a, st)
+                     : (b_dim == 64 ? launch_had_rows<64, false>(a, st)
+                                    : launch_had_rows<128, false>(a, st));
+  } else if (io_dtype == CTMI_F16 && a_dim == 1) {
+    rc = b_dim == 32 ? launch_had_rows<32, true>(a, st)
+                     : (b_dim == 64 ? launch_had_rows<64, true>(a, st)
+                                    : launch_had_rows<128, true>(a, st));
   } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 32) {
     rc = launch_had_kron<32, 32>(a, st);
   } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 64) {
