@@ -554,7 +554,7 @@ hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __res
 // Signs (entries +1 / -1) are XOR masks on the bf16 sign bits of X and of the
 // output; they are per position within the row, the same for every row, and sit
 // in LDS in the lanes' own layout.
-template <int A, int B>
+template <int A, int B, bool HALF>
 __global__ void __launch_bounds__(kHadThreads) __attribute__((amdgpu_waves_per_eu(CTMI_HAD_KRON_WAVES)))
 hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
                      const uint16_t* __restrict__ mbt, const uint16_t* __restrict__ mat,
@@ -571,6 +571,9 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l16 = lane & 15, lq = lane >> 4;
   const int perm = 8 * (l16 / 4) + (l16 % 4);  // label -> position within a pair of tiles
+  // HALF: float16 tensors.  Stage 1 runs on v_mfma_f32_16x16x32_f16 (Mb converts from
+  // bfloat16 to float16 exactly); stage 2 works on the fp32 intermediate as before.
+  using xfrag_t = typename std::conditional<HALF, f16x8_t, bf16x8_t>::type;
 
   __shared__ u32x4_t sign_in_lds[MT * KS][kWave];
   __shared__ u32x4_t sign_out_lds[AT * (NT / 2)][kWave];
@@ -601,13 +604,22 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   }
 
   // the two small matrices, as B operands
-  bf16x8_t mbf[NT][KS], maf[AT][PS];
+  xfrag_t mbf[NT][KS];
+  bf16x8_t maf[AT][PS];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      mbf[nt][ks] = __builtin_bit_cast(
-          bf16x8_t, ldg<uint16_t, 8>(mbt + (32 * (nt / 2) + 4 * (nt % 2) + perm) * B + 32 * ks + 8 * lq));
+    for (int ks = 0; ks < KS; ++ks) {
+      Vec<uint32_t, 4> m = __builtin_bit_cast(
+          Vec<uint32_t, 4>,
+          ldg<uint16_t, 8>(mbt + (32 * (nt / 2) + 4 * (nt % 2) + perm) * B + 32 * ks + 8 * lq));
+      if constexpr (HALF) {
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          m.v[w] = (uint32_t)f32_to_f16(bf16_lo(m.v[w])) | ((uint32_t)f32_to_f16(bf16_hi(m.v[w])) << 16);
+      }
+      mbf[nt][ks] = __builtin_bit_cast(xfrag_t, m);
+    }
 #pragma unroll
   for (int at = 0; at < AT; ++at)
 #pragma unroll
@@ -619,13 +631,13 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   for (int64_t row = (int64_t)blockIdx.x * kHadWaves + wave; row < n_rows; row += stride) {
     const uint16_t* src = x + row * N;
     uint16_t* dst = out + row * N;
-    bf16x8_t xf[MT][KS];
+    xfrag_t xf[MT][KS];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks)
         xf[m][ks] = __builtin_bit_cast(
-            bf16x8_t,
+            xfrag_t,
             ldg<uint16_t, 8>(src + (32 * (m / 2) + 4 * (m % 2) + perm) * B + 32 * ks + 8 * lq));
     if (signed_io) {
 #pragma unroll
@@ -633,7 +645,7 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
           const u32x4_t f = sign_in_lds[m * KS + ks][lane];
-          xf[m][ks] = __builtin_bit_cast(bf16x8_t, __builtin_bit_cast(u32x4_t, xf[m][ks]) ^ f);
+          xf[m][ks] = __builtin_bit_cast(xfrag_t, __builtin_bit_cast(u32x4_t, xf[m][ks]) ^ f);
         }
     }
 #pragma unroll
@@ -648,8 +660,13 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
           f32x4_t lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
           for (int ks = 0; ks < KS; ++ks) {
-            lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[2 * ps][ks], mbf[nt][ks], lo, 0, 0, 0);
-            hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[2 * ps + 1][ks], mbf[nt][ks], hi, 0, 0, 0);
+            if constexpr (HALF) {
+              lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[2 * ps][ks], mbf[nt][ks], lo, 0, 0, 0);
+              hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[2 * ps + 1][ks], mbf[nt][ks], hi, 0, 0, 0);
+            } else {
+              lo = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[2 * ps][ks], mbf[nt][ks], lo, 0, 0, 0);
+              hi = __builtin_amdgcn_mfma_f32_16x16x32_bf16(xf[2 * ps + 1][ks], mbf[nt][ks], hi, 0, 0, 0);
+            }
           }
           float t[8] = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
           u32x4_t parts[NSPLIT];
@@ -678,10 +695,20 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
             y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf[1][ps][sp], maf[at][ps], y1, 0, 0, 0);
           }
         u32x4_t o;
-        o[0] = pack_bf16x2(y0[0] * inv_sqrt_n, y0[1] * inv_sqrt_n);
-        o[1] = pack_bf16x2(y0[2] * inv_sqrt_n, y0[3] * inv_sqrt_n);
-        o[2] = pack_bf16x2(y1[0] * inv_sqrt_n, y1[1] * inv_sqrt_n);
-        o[3] = pack_bf16x2(y1[2] * inv_sqrt_n, y1[3] * inv_sqrt_n);
+        if constexpr (HALF) {
+#pragma unroll
+          for (int d = 0; d < 2; ++d) {
+            o[d] = (uint32_t)f32_to_f16(y0[2 * d] * inv_sqrt_n) |
+                   ((uint32_t)f32_to_f16(y0[2 * d + 1] * inv_sqrt_n) << 16);
+            o[2 + d] = (uint32_t)f32_to_f16(y1[2 * d] * inv_sqrt_n) |
+                       ((uint32_t)f32_to_f16(y1[2 * d + 1] * inv_sqrt_n) << 16);
+          }
+        } else {
+          o[0] = pack_bf16x2(y0[0] * inv_sqrt_n, y0[1] * inv_sqrt_n);
+          o[1] = pack_bf16x2(y0[2] * inv_sqrt_n, y0[3] * inv_sqrt_n);
+          o[2] = pack_bf16x2(y1[0] * inv_sqrt_n, y1[1] * inv_sqrt_n);
+          o[3] = pack_bf16x2(y1[2] * inv_sqrt_n, y1[3] * inv_sqrt_n);
+        }
         if (signed_io) o ^= sign_out_lds[at * (NT / 2) + p][lane];
         stg<uint16_t, 8>(dst + (16 * at + l16) * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o));
       }
@@ -689,14 +716,14 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   }
 }
 
-template <int A, int B>
+template <int A, int B, bool HALF>
 static int launch_had_kron(const HadArgs& a, hipStream_t st) {
   const int64_t n_rows = a.n_sub / A;
   const int64_t wgs = cdiv(n_rows, kHadWaves);
   // as many workgroups as are resident at once (register-limited)
   const int64_t cap = 256 * (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES));
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
-  hipLaunchKernelGGL((hadamard_kron_kernel<A, B>), grid, kHadThreads, 0, st, (const uint16_t*)a.x,
+  hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF>), grid, kHadThreads, 0, st, (const uint16_t*)a.x,
                      (uint16_t*)a.out, a.mbt, a.mat, a.s_in, a.s_out, n_rows, 1.0f / a.sqrt_n);
   return CTMI_OK;
 }
@@ -807,11 +834,17 @@ extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, i
                      : (b_dim == 64 ? launch_had_rows<64, true>(a, st)
                                     : launch_had_rows<128, true>(a, st));
   } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 32) {
-    rc = launch_had_kron<32, 32>(a, st);
+    rc = launch_had_kron<32, 32, false>(a, st);
   } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 64) {
-    rc = launch_had_kron<32, 64>(a, st);
+    rc = launch_had_kron<32, 64, false>(a, st);
   } else if (io_dtype == CTMI_BF16 && a_dim == 64 && b_dim == 64) {
-    rc = launch_had_kron<64, 64>(a, st);
+    rc = launch_had_kron<64, 64, false>(a, st);
+  } else if (io_dtype == CTMI_F16 && a_dim == 32 && b_dim == 32) {
+    rc = launch_had_kron<32, 32, true>(a, st);
+  } else if (io_dtype == CTMI_F16 && a_dim == 32 && b_dim == 64) {
+    rc = launch_had_kron<32, 64, true>(a, st);
+  } else if (io_dtype == CTMI_F16 && a_dim == 64 && b_dim == 64) {
+    rc = launch_had_kron<64, 64, true>(a, st);
   } else if (io_dtype == CTMI_BF16) rc = dispatch_had<BF16>(a_dim, b_dim, a, st);
   else if (io_dtype == CTMI_F16) rc = dispatch_had<F16>(a_dim, b_dim, a, st);
   else rc = dispatch_had<F32>(a_dim, b_dim, a, st);
