@@ -1,0 +1,76 @@
+// Shared by the kernels for activation-ordered weights (the group of a column is
+// g_idx[column], quantization/lifecycle/forward.py:286-296): a workgroup takes RB
+// rows of a tile of 256 x 8 columns; a lane keeps the group indices of its 8
+// columns in registers, the RB rows of scales (zero points) are staged in LDS as
+// fp32 and gathered per element.
+#pragma once
+
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "quant_core.h"
+#include "quant_fast.h"
+
+namespace ctmi {
+
+struct GidxArgs {
+  const void* dense;          // pack-quantized: compress input / decompress output
+  const int32_t* packed_in;   // pack-quantized decompress
+  int32_t* packed_out;        // pack-quantized compress
+  const void* in;             // quantize / dequantize: input and output tensors
+  void* out;
+  const void* scale;
+  const int8_t* zp;
+  const int32_t* col_group;
+  uint32_t rows, vpr, s_cols, tiles;  // vpr: items (8 elements) per row
+  float qmin, qmax;
+};
+
+constexpr int kGidxThreads = 256;
+
+// stage RB rows of scales (zero points) as fp32: lds_s[rb * s_cols + j]; with lds_r
+// also their reciprocals.  Returns whether a staged scale is outside the range
+// where the reciprocal path is exact.
+template <typename ST, bool HAS_ZP, int RB, bool ZP_FP8 = false>
+__device__ __forceinline__ bool stage_qparams(const GidxArgs& a, uint32_t row0, float* lds_s,
+                                              float* lds_z, float* lds_r) {
+  const auto* scale = (const typename ST::raw*)a.scale;
+  bool wild = false;
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    const uint32_t row = min(row0 + rb, a.rows - 1);
+    for (uint32_t j = threadIdx.x; j < a.s_cols; j += kGidxThreads) {
+      const size_t si = (size_t)row * a.s_cols + j;
+      const float sv = ST::to_f32(scale[si]);
+      lds_s[rb * a.s_cols + j] = sv;
+      if (lds_r) {
+        lds_r[rb * a.s_cols + j] = __builtin_amdgcn_rcpf(sv);
+        wild |= !scale_is_tame(sv);
+      }
+      if constexpr (HAS_ZP)
+        lds_z[rb * a.s_cols + j] = ZP_FP8 ? f8e4m3_to_f32((uint8_t)a.zp[si]) : (float)a.zp[si];
+    }
+  }
+  return wild;
+}
+
+__device__ __forceinline__ void load_groups(const GidxArgs& a, uint32_t cv, uint32_t* g) {
+  const Vec<int32_t, 4> lo = ldg<int32_t, 4>(a.col_group + (size_t)cv * 8);
+  const Vec<int32_t, 4> hi = ldg<int32_t, 4>(a.col_group + (size_t)cv * 8 + 4);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    // an index outside the scale row must not leave the staged window
+    g[k] = min((uint32_t)max(lo.v[k], 0), a.s_cols - 1);
+    g[4 + k] = min((uint32_t)max(hi.v[k], 0), a.s_cols - 1);
+  }
+}
+
+// rows per workgroup so that the staged fp32 arrays (scales, for compression their
+// reciprocals, zero points) stay within 32 KB
+static inline int gidx_rows_per_block(int64_t s_cols, int arrays) {
+  const int64_t per_row = s_cols * 4 * arrays;
+  for (int rb = 8; rb >= 1; rb >>= 1)
+    if (rb * per_row <= 32 * 1024) return rb;
+  return 0;
+}
+
+}  // namespace ctmi

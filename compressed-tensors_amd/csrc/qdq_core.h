@@ -37,11 +37,14 @@ __device__ __forceinline__ float fp8_hw_decode(uint32_t word, int byte) {
 // input and output (kKindFloat, kKindI8, kKindF8).  QK: 0 = integer grid, 1 = fp8
 // grid.  xf is read when IN is float, xc otherwise; out_float is written when OUT
 // is float, out_codes otherwise.
-template <typename FT, int IN, int OUT, int QK, bool HAS_ZP>
-__device__ __forceinline__ void qdq_vec8(const Vec<typename FT::raw, 8>& xf,
-                                         const Vec<uint8_t, 8>& xc, float s, float z, float qmin,
-                                         float qmax, Vec<typename FT::raw, 8>* out_float,
-                                         Vec<uint8_t, 8>* out_codes) {
+// SS: 0 = one scale / zero point for the 8 elements (s[0], z[0]), 1 = one per
+// element (s[i], z[i]: activation-ordered groups).
+template <typename FT, int IN, int OUT, int QK, bool HAS_ZP, int SS>
+__device__ __forceinline__ void qdq_vec8_impl(const Vec<typename FT::raw, 8>& xf,
+                                              const Vec<uint8_t, 8>& xc, const float* s,
+                                              const float* z, float qmin, float qmax,
+                                              Vec<typename FT::raw, 8>* out_float,
+                                              Vec<uint8_t, 8>* out_codes) {
   constexpr int CT = FT::id;
   constexpr bool DO_Q = IN == kKindFloat;
   constexpr bool DO_DQ = OUT == kKindFloat;
@@ -49,14 +52,19 @@ __device__ __forceinline__ void qdq_vec8(const Vec<typename FT::raw, 8>& xf,
   float t[8];
   uint32_t codes[2] = {0u, 0u};  // 8 one-byte codes
   if constexpr (DO_Q) {
-    const bool fast = CT == CTMI_BF16 && wave_all(scale_is_tame(s));
-    const float r = __builtin_amdgcn_rcpf(s);
+    bool tame = scale_is_tame(s[0]);
+    if constexpr (SS != 0) {
+#pragma unroll
+      for (int i = 1; i < 8; ++i) tame &= scale_is_tame(s[i]);
+    }
+    const bool fast = CT == CTMI_BF16 && wave_all(tame);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float a = FT::to_f32(xf.v[2 * j]), b = FT::to_f32(xf.v[2 * j + 1]);
-      if (fast) { a *= r; b *= r; } else { a /= s; b /= s; }
+      const float sa = s[SS * 2 * j], sb = s[SS * (2 * j + 1)];
+      if (fast) { a *= __builtin_amdgcn_rcpf(sa); b *= __builtin_amdgcn_rcpf(sb); } else { a /= sa; b /= sb; }
       round2<CT>(a, b);
-      if (HAS_ZP) { a += z; b += z; round2<CT>(a, b); }
+      if (HAS_ZP) { a += z[SS * 2 * j]; b += z[SS * (2 * j + 1)]; round2<CT>(a, b); }
       a = clamp_nan(a, qmin, qmax);
       b = clamp_nan(b, qmin, qmax);
       if constexpr (QK == 0) {
@@ -91,9 +99,9 @@ __device__ __forceinline__ void qdq_vec8(const Vec<typename FT::raw, 8>& xf,
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float a = t[2 * j], b = t[2 * j + 1];
-      if (HAS_ZP) { a -= z; b -= z; round2<CT>(a, b); }
-      a *= s;
-      b *= s;
+      if (HAS_ZP) { a -= z[SS * 2 * j]; b -= z[SS * (2 * j + 1)]; round2<CT>(a, b); }
+      a *= s[SS * 2 * j];
+      b *= s[SS * (2 * j + 1)];
       if constexpr (CT == CTMI_BF16) {
         const uint32_t p = pack_bf16x2(a, b);
         o.v[2 * j] = (uint16_t)(p & 0xffffu);
@@ -110,6 +118,14 @@ __device__ __forceinline__ void qdq_vec8(const Vec<typename FT::raw, 8>& xf,
     w.v[1] = codes[1];
     *out_codes = __builtin_bit_cast(Vec<uint8_t, 8>, w);
   }
+}
+
+template <typename FT, int IN, int OUT, int QK, bool HAS_ZP>
+__device__ __forceinline__ void qdq_vec8(const Vec<typename FT::raw, 8>& xf,
+                                         const Vec<uint8_t, 8>& xc, float s, float z, float qmin,
+                                         float qmax, Vec<typename FT::raw, 8>* out_float,
+                                         Vec<uint8_t, 8>* out_codes) {
+  qdq_vec8_impl<FT, IN, OUT, QK, HAS_ZP, 0>(xf, xc, &s, &z, qmin, qmax, out_float, out_codes);
 }
 
 }  // namespace ctmi

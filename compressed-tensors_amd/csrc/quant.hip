@@ -78,6 +78,8 @@ bool qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, in
                         int64_t cols, const ctmi_qparams* qp, int do_q, int do_dq, hipStream_t st);
 bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows,
                               int64_t cols, const ctmi_qparams* qp, hipStream_t st);
+bool qdq_gidx_try(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows, int64_t cols,
+                  const ctmi_qparams* qp, int do_q, int do_dq, hipStream_t st);
 
 // ------------------------------------------------------------------ host side
 static int fill_cfg(const ctmi_qparams* qp, int x_dtype, QuantCfg* q) {
@@ -157,6 +159,8 @@ extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_d
   if (do_quantize && do_dequantize &&
       nvfp4_qdq_try_vectorised(x, x_dtype, out, out_dtype, rows, cols, qp, st))
     return check_launch("ctmi_qdq");
+  if (qdq_gidx_try(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize, st))
+    return check_launch("ctmi_qdq");
   qdq_enqueue_generic(x, x_dtype, out, out_dtype, rows, cols, qp, do_quantize, do_dequantize, st);
   return check_launch("ctmi_qdq");
 }
@@ -196,7 +200,9 @@ extern "C" int ctmi_qdq_many(const ctmi_qdq_job* jobs, int64_t n, int32_t do_qua
       continue;
     }
     if (!(do_quantize && do_dequantize &&
-          nvfp4_qdq_try_vectorised(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, st)))
+          nvfp4_qdq_try_vectorised(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, st)) &&
+        !qdq_gidx_try(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, do_quantize,
+                      do_dequantize, st))
       qdq_enqueue_generic(j.x, j.x_dtype, j.out, j.out_dtype, j.rows, j.cols, &j.qp, do_quantize,
                           do_dequantize, st);
     done[i] = 1;

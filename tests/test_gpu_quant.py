@@ -671,3 +671,39 @@ def test_scales_computed_in_kernels_for_every_maximum(dtype, gpu):
         assert_bit_equal(scale, o_scale, f"dynamic nvfp4 scales, gs {gs_value}")
         assert_bit_equal(out, oq.fake_quantize(x, o_scale, o_zp, oargs, global_scale=o_gs),
                          f"dynamic nvfp4 qdq, gs {gs_value}")
+
+
+QG = [
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128), (64, 1024), torch.bfloat16),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=64), (33, 4096), torch.bfloat16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=32), (19, 512), torch.float16),
+    (dict(num_bits=8, type="float", symmetric=False, strategy="group", group_size=128), (9, 2048), torch.bfloat16),
+    (dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=8), (13, 2056), torch.float32),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=16), (3, 20480), torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype", QG, ids=[f"qg{i}" for i in range(len(QG))])
+def test_quantize_dequantize_with_activation_ordering(spec, shape, dtype, gpu):
+    """quantize, dequantize and fake_quantize with a g_idx per column (the streaming
+    kernels gather every element's scale and zero point) against the oracle"""
+    from compressed_tensors_amd.quantization import dequantize, fake_quantize, quantize
+
+    announce("qdq g_idx", spec, shape, dtype)
+    args, oargs = _pair(spec)
+    rows, cols = shape
+    g = torch.Generator().manual_seed(rows)
+    w = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+    w.view(-1)[:3] = torch.tensor([0.0, -0.0, -1e-6]).to(dtype)
+    g_idx = (torch.randperm(cols, generator=g) // spec["group_size"]).to(torch.int32)
+    scale, zp = oq.observe_weight(w.index_select(-1, torch.argsort(g_idx)), oargs)
+    zp_arg = None if spec["symmetric"] else zp
+    dev = lambda t: None if t is None else t.to(gpu)
+    code_dtype = torch.int8 if spec["type"] == "int" else torch.float8_e4m3fn
+    want_q = oq.quantize(w, scale, zp_arg, oargs, dtype=code_dtype, g_idx=g_idx)
+    got_q = quantize(w.to(gpu), dev(scale), dev(zp_arg), args, dtype=code_dtype, g_idx=dev(g_idx))
+    assert_bit_equal(got_q, want_q, "quantize")
+    assert_bit_equal(dequantize(got_q, dev(scale), dev(zp_arg), args=args, g_idx=dev(g_idx)),
+                     oq.dequantize(want_q, scale, zp_arg, args=oargs, g_idx=g_idx), "dequantize")
+    assert_bit_equal(fake_quantize(w.to(gpu), dev(scale), dev(zp_arg), args, g_idx=dev(g_idx)),
+                     oq.fake_quantize(w, scale, zp_arg, oargs, g_idx=g_idx), "fake_quantize")
