@@ -247,7 +247,7 @@ __device__ __forceinline__ uint32_t nvfp4_codes(const Vec<typename XT::raw, 8>& 
   }
   const uint32_t c_lo = fp4_pack8_hw(lo), c_hi = fp4_pack8_hw(hi);
   ok &= c_lo == c_hi;
-  if (wave_all(ok)) return c_lo;
+  if (__builtin_expect(wave_all(ok), 1)) return c_lo;
   return nvfp4_codes_exact<XT, HAS_ZP>(xv, s, z);
 }
 
@@ -280,9 +280,9 @@ nvfp4_compress_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t*
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < g.nvec) {
-        const float s = f8e4m3_to_f32(sraw[k]) / gs;
+        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
         // zero_point.to(x.dtype): an fp8 value is exact in every wider float type
-        const float z = HAS_ZP ? f8e4m3_to_f32(zraw[k]) : 0.0f;
+        const float z = HAS_ZP ? __builtin_amdgcn_cvt_f32_fp8((int)zraw[k], 0) : 0.0f;
         __builtin_nontemporal_store(nvfp4_codes<XT, HAS_ZP>(xv[k], s, z), out + v);
       }
     }
@@ -319,7 +319,7 @@ nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* 
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < g.nvec) {
-        const float s = f8e4m3_to_f32(sraw[k]) / gs;
+        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
         float t[8];
         fp4_unpack8_hw(pv[k], t);
         Vec<typename OT::raw, 8> o;
@@ -363,7 +363,7 @@ nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __re
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < g.nvec) {
-        const float s = f8e4m3_to_f32(sraw[k]) / gs;
+        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
         float t[8];
         fp4_unpack8_hw(nvfp4_codes<XT, false>(xv[k], s, 0.0f), t);
         Vec<typename XT::raw, 8> o;

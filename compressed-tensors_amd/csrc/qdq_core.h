@@ -57,7 +57,7 @@ __device__ __forceinline__ void qdq_vec8_impl(const Vec<typename FT::raw, 8>& xf
 #pragma unroll
       for (int i = 1; i < 8; ++i) tame &= scale_is_tame(s[i]);
     }
-    const bool fast = CT == CTMI_BF16 && wave_all(tame);
+    const bool fast = CT == CTMI_BF16 && __builtin_expect(wave_all(tame), 1);
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float a = FT::to_f32(xf.v[2 * j]), b = FT::to_f32(xf.v[2 * j + 1]);

@@ -88,7 +88,7 @@ __device__ __forceinline__ Vec<int32_t, BITS / 4> quant_pack8_bf16(const Vec<uin
                                                                   float qmax) {
   using PC = PackConst<BITS>;
   constexpr int W = BITS / 4;
-  if (!wave_all(scale_is_tame(s)))
+  if (__builtin_expect(!wave_all(scale_is_tame(s)), 0))
     return quant_pack8_exact<BF16, CTMI_BF16, BITS, HAS_ZP>(xv, s, z, qmin, qmax);
   const float r = __builtin_amdgcn_rcpf(s);
   const Vec<uint32_t, 4> xw = __builtin_bit_cast(Vec<uint32_t, 4>, xv);
@@ -176,7 +176,7 @@ __device__ __forceinline__ Vec<typename ST::raw, 8> unpack_dequant8(const Vec<in
     f[6] = ubyte_to_f32<2>(b[1]); f[7] = ubyte_to_f32<3>(b[1]);
   }
   // (a negative scale takes the two-step form too: it gives -0 where the fma gives +0)
-  if (kFusable && wave_all(s >= 7.888609052210118e-31f && s <= 1.2676506002282294e30f)) {
+  if (kFusable && __builtin_expect(wave_all(s >= 7.888609052210118e-31f && s <= 1.2676506002282294e30f), 1)) {
     const float c = -(off * s);
 #pragma unroll
     for (int i = 0; i < 8; ++i) f[i] = __builtin_fmaf(f[i], s, c);
