@@ -174,7 +174,7 @@ __global__ void __launch_bounds__(256) nvfp4_decompress_generic_kernel(Fp4Args a
 // every load of a chunk issued before the first value is looked at; chunks that
 // lie wholly inside the tensor run without per-lane bounds checks.
 #ifndef CTMI_FP4_TUNING
-#define CTMI_FP4_TUNING 256, 1
+#define CTMI_FP4_TUNING 512, 2
 #endif
 constexpr int kFp4Tuning[2] = {CTMI_FP4_TUNING};
 constexpr int kFp4Block = kFp4Tuning[0], kFp4Unroll = kFp4Tuning[1];
@@ -335,12 +335,14 @@ nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* 
 
 // quantize + dequantize in one pass (fake_quantize of forward.py:150-189 for the
 // nvfp4 scheme): out = XT(e2m1(x / s) * s), s = fp32(scale) / global_scale
+// (fake-quantize moves 4 bytes per element: one item per lane in flight is enough)
+constexpr int kFp4QdqBlock = 256, kFp4QdqUnroll = 1;
 template <typename XT>
-__global__ void __launch_bounds__(kFp4Block)
+__global__ void __launch_bounds__(kFp4QdqBlock)
 nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __restrict__ scale,
                      const float* __restrict__ gscale, typename XT::raw* __restrict__ out,
                      VecGeom g) {
-  constexpr int B = kFp4Block, U = kFp4Unroll;
+  constexpr int B = kFp4QdqBlock, U = kFp4QdqUnroll;
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
@@ -391,11 +393,11 @@ bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dty
   if ((uintptr_t)x % bytes || (uintptr_t)out % bytes) return false;
   VecGeom g;
   if (!vec_geometry(qp, rows, cols, &g, true)) return false;
-  const int64_t grid = cdiv(g.nvec, kFp4Block * kFp4Unroll);
+  const int64_t grid = cdiv(g.nvec, kFp4QdqBlock * kFp4QdqUnroll);
   const auto* sc = (const uint8_t*)qp->scale;
-  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
-  else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
-  else hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, sc, qp->global_scale, (float*)out, g);
+  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<BF16>, (unsigned)grid, kFp4QdqBlock, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
+  else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F16>, (unsigned)grid, kFp4QdqBlock, 0, st, (const uint16_t*)x, sc, qp->global_scale, (uint16_t*)out, g);
+  else hipLaunchKernelGGL(nvfp4_qdq_vec_kernel<F32>, (unsigned)grid, kFp4QdqBlock, 0, st, (const float*)x, sc, qp->global_scale, (float*)out, g);
   return true;
 }
 
