@@ -25,7 +25,11 @@
 namespace ctmi {
 
 // ------------------------------------------------------------------ groups within a row
-constexpr int kOpBlock = 512, kOpUnroll = 2;
+#ifndef CTMI_OP_TUNING
+#define CTMI_OP_TUNING 512, 4
+#endif
+constexpr int kOpTuning[2] = {CTMI_OP_TUNING};
+constexpr int kOpBlock = kOpTuning[0], kOpUnroll = kOpTuning[1];
 
 // One item = 8 neighbouring elements; L = 2^job.shift neighbouring lanes own a
 // group.  Items, words and groups are numbered row-major, so a chunk of
