@@ -239,7 +239,7 @@ def other_workload(torch, name, seed):
             bitmask = torch.empty(rows, cols // 8, dtype=torch.uint8, device=dev)
             offs = torch.empty(rows, dtype=torch.int64, device=dev)
             total = torch.empty(1, dtype=torch.int64, device=dev)
-            tmp = torch.empty(lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8, dtype=torch.uint8, device=dev)
+            tmp = torch.empty(lib.ctmi_bitmask_tmp_bytes(rows, cols), dtype=torch.uint8, device=dev)
             a = (w.data_ptr(), 2, 1, bitmask.data_ptr(), offs.data_ptr(), total.data_ptr(), tmp.data_ptr(), rows, cols, st)
             _lib.check(lib.ctmi_bitmask_count(*a))
             nnz = int(total.item())
@@ -274,7 +274,7 @@ def other_workload(torch, name, seed):
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies * (n24 + n24 // 2 + n24 // 8)
         ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_kernel"),
-               Op("sparse-bitmask decompress (row offsets recomputed from the bitmask)", d_calls, bm_bytes, "bitmask_scatter_kernel"),
+               Op("sparse-bitmask decompress (positions from the bitmask alone)", d_calls, bm_bytes, "bitmask_scatter_tiles_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel")]
         return "sparse-bitmask / sparse-24-bitmask compress+decompress GB/s", ops, keep

@@ -48,7 +48,7 @@ def bitmask_compress(tensor: Tensor) -> Tuple[Tensor, Tensor, Tensor]:
         raise NotImplementedError("bitmask compression expects a 2-D tensor")
     row_offsets = torch.empty((rows,), dtype=torch.int64, device=dev)
     total = torch.empty((1,), dtype=torch.int64, device=dev)
-    tmp = torch.empty((max(lib.ctmi_bitmask_tmp_bytes(rows), 8),), dtype=torch.uint8, device=dev)
+    tmp = torch.empty((lib.ctmi_bitmask_tmp_bytes(rows, cols),), dtype=torch.uint8, device=dev)
     stream = _lib.stream_of(dev)
     _lib.check(
         lib.ctmi_bitmask_count(
@@ -82,7 +82,7 @@ def _scatter(values: Tensor, bitmasks: Tensor, row_offsets, shape, two_four: boo
         raise ValueError(f"bitmask of {bitmasks.numel()} bytes does not describe shape {shape}")
     out = torch.empty(shape, dtype=values.dtype, device=dev)
     tmp_bytes = (lib.ctmi_sparse24_tmp_bytes(rows, cols, esize) if two_four
-                 else lib.ctmi_bitmask_tmp_bytes(rows) + rows * 8 + 8)
+                 else lib.ctmi_bitmask_tmp_bytes(rows, cols))
     tmp = torch.empty((tmp_bytes,), dtype=torch.uint8, device=dev)
     ro_ptr = None
     if row_offsets is not None:

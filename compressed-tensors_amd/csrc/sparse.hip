@@ -459,6 +459,205 @@ static bool scatter_wave_ok(const void* values, const uint8_t* bitmask, const vo
          (cols * sizeof(R)) % 16 == 0;
 }
 
+// ------------------------------------------------------------------ bitmask decompress by tiles
+// With rows of whole bitmask bytes the bitmask is one flat run of bits and the
+// values one flat run in the same order, so rows do not matter.  The tensor is
+// cut into tiles of kTileElems elements; a first pass counts the set bits of
+// every tile (one wavefront per tile), row_offsets_kernel turns the counts into
+// where each tile's values start, and the scatter then knows before it has looked
+// at anything which values a tile needs: it fetches them together with the tile's
+// bitmask, stages them in LDS and every lane picks its own.
+#ifndef CTMI_TILE_U
+#define CTMI_TILE_U 1
+#endif
+constexpr int kTileU = CTMI_TILE_U;            // 16-element items per lane
+constexpr int kTileItems = kBlock * kTileU;
+constexpr int kTileElems = kTileItems * 16;
+constexpr int kTileBytes = kTileElems / 8;     // bitmask bytes per tile
+
+__global__ void __launch_bounds__(kBlock)
+tile_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
+                     int64_t* __restrict__ counts, int64_t ntiles) {
+  const int lane = lane_id();
+  const int64_t tile = (int64_t)blockIdx.x * kWaves + threadIdx.x / kWave;
+  if (tile >= ntiles) return;
+  int cnt = 0;
+#pragma unroll
+  for (int i = 0; i < kTileBytes; i += kWave * 16) {
+    const int64_t b0 = tile * kTileBytes + i + lane * 16;
+    if (i + lane * 16 >= kTileBytes) {
+      // a tile shorter than one step of the wavefront
+    } else if (b0 + 16 <= nbytes) {
+      const u32x4_t q = *reinterpret_cast<const u32x4_t*>(bitmask + b0);
+      cnt += __popc(q.x) + __popc(q.y) + __popc(q.z) + __popc(q.w);
+    } else {
+      for (int64_t b = b0; b < nbytes; ++b) cnt += __popc((uint32_t)bitmask[b]);
+    }
+  }
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) cnt += __shfl_xor(cnt, d, kWave);
+  if (lane == 0) counts[tile] = cnt;
+}
+
+// The same count for tensors of up to kGroupTiles * kMaxGroups tiles, without the
+// scan in between: a workgroup counts a group of kGroupTiles neighbouring tiles
+// and leaves, per tile, the count of the group's earlier tiles and its own, and per
+// group its total; a scatter workgroup adds up the totals of the groups before its
+// own by itself (at most kMaxGroups words, from L2).
+constexpr int kGroupTiles = 64;
+constexpr int kGroupThreads = 1024;
+constexpr int kMaxGroups = 1024;
+struct TileInfo {
+  int32_t before;  // set bits in the group's earlier tiles
+  int32_t count;   // set bits in the tile
+};
+
+__global__ void __launch_bounds__(kGroupThreads)
+tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
+                            TileInfo* __restrict__ info, int32_t* __restrict__ group_total,
+                            int64_t ntiles) {
+  constexpr int kPerWave = kGroupTiles / (kGroupThreads / kWave);  // tiles per wavefront
+  __shared__ int cnt_s[kGroupTiles];
+  const int lane = lane_id(), wave = threadIdx.x / kWave;
+  const int64_t tile0 = (int64_t)blockIdx.x * kGroupTiles;
+  int cnt[kPerWave];
+#pragma unroll
+  for (int t = 0; t < kPerWave; ++t) {
+    const int64_t tile = tile0 + wave * kPerWave + t;
+    cnt[t] = 0;
+#pragma unroll
+    for (int i = 0; i < kTileBytes; i += kWave * 16) {
+      const int64_t b0 = tile * kTileBytes + i + lane * 16;
+      if (i + lane * 16 >= kTileBytes) {
+        // a tile shorter than one step of the wavefront
+      } else if (b0 + 16 <= nbytes) {
+        const u32x4_t q = *reinterpret_cast<const u32x4_t*>(bitmask + b0);
+        cnt[t] += __popc(q.x) + __popc(q.y) + __popc(q.z) + __popc(q.w);
+      } else {
+        for (int64_t b = b0; b < nbytes; ++b) cnt[t] += __popc((uint32_t)bitmask[b]);
+      }
+    }
+  }
+#pragma unroll
+  for (int t = 0; t < kPerWave; ++t) {
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) cnt[t] += __shfl_xor(cnt[t], d, kWave);
+    if (lane == 0) cnt_s[wave * kPerWave + t] = cnt[t];
+  }
+  __syncthreads();
+  if (wave == 0) {
+    const int c = cnt_s[lane];
+    const int inc = wave_inclusive_scan(c);
+    if (tile0 + lane < ntiles) info[tile0 + lane] = TileInfo{inc - c, c};
+    if (lane == kWave - 1) group_total[blockIdx.x] = inc;
+  }
+}
+
+// Set bits beyond nvalues read as zero.  GROUPED: positions from
+// tile_popcount_groups_kernel (info, group_total), else from tile_popcount_kernel
+// and the scan behind it (tile_counts, tile_offsets).
+template <typename R, bool GROUPED>
+__global__ void __launch_bounds__(kBlock)
+bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
+                             const uint16_t* __restrict__ words,
+                             const int64_t* __restrict__ tile_counts,
+                             const int64_t* __restrict__ tile_offsets,
+                             const TileInfo* __restrict__ info,
+                             const int32_t* __restrict__ group_total, R* __restrict__ out,
+                             int64_t n_items) {
+  constexpr int E = 16, U = kTileU;
+  constexpr int VE = 16 / (int)sizeof(R);
+  __shared__ int wtot[U][kWaves];
+  __shared__ __align__(16) R stage[kTileElems + 2 * VE];
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid / kWave;
+  const int64_t tile = blockIdx.x;
+  const int64_t item0 = tile * kTileItems;
+  int64_t excl;
+  int total;
+  if constexpr (GROUPED) {
+    // every wavefront adds up the earlier groups by itself: no barrier
+    const int group = (int)(tile / kGroupTiles);
+    int64_t before = 0;
+    for (int g = lane; g < group; g += kWave) before += group_total[g];
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) before += __shfl_xor(before, d, kWave);
+    const TileInfo ti = info[tile];
+    excl = before + ti.before;
+    total = ti.count;
+  } else {
+    excl = tile_offsets[tile];
+    total = (int)tile_counts[tile];
+  }
+
+  uint32_t bits[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t item = item0 + k * kBlock + tid;
+    bits[k] = item < n_items ? (uint32_t)words[item] : 0u;
+  }
+  // values [excl, excl + total) -> LDS, from the 16-byte boundary below excl
+  const int64_t base = excl & ~(int64_t)(VE - 1);
+  const int off = (int)(excl - base);
+  const int nvecs = (off + total + VE - 1) / VE;
+  for (int i = tid; i < nvecs; i += kBlock) {
+    const int64_t e0 = base + (int64_t)i * VE;
+    Vec<R, VE> v;
+    if (e0 < nvalues) {
+      // an aligned vector that starts inside the buffer never leaves its page
+      v = ldg<R, VE>(values + e0);
+#pragma unroll
+      for (int e = 0; e < VE; ++e)
+        if (e0 + e >= nvalues) v.v[e] = (R)0;
+    } else {
+#pragma unroll
+      for (int e = 0; e < VE; ++e) v.v[e] = (R)0;
+    }
+    *reinterpret_cast<Vec<R, VE>*>(stage + i * VE) = v;
+  }
+  // ranks: item k of a lane comes after every item k' < k and after item k of the lanes below
+  int cnt[U], inc[U], pre[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    cnt[k] = __popc(bits[k]);
+    inc[k] = wave_inclusive_scan(cnt[k]);
+    if (lane == kWave - 1) wtot[k][wave] = inc[k];
+  }
+  __syncthreads();
+  int before = 0;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    int mine = before;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const int s = wtot[k][w];
+      if (w < wave) mine += s;
+      before += s;
+    }
+    pre[k] = mine + inc[k] - cnt[k];
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t item = item0 + k * kBlock + tid;
+    if (item < n_items) {
+      int idx = off + pre[k];
+      Vec<R, E> o;
+#pragma unroll
+      for (int j = 0; j < E; ++j) {
+        const bool set = (bits[k] >> j) & 1u;
+        o.v[j] = set ? stage[idx] : (R)0;
+        idx += set ? 1 : 0;
+      }
+#pragma unroll
+      for (int h = 0; h < E / VE; ++h) {
+        Vec<R, VE> part;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) part.v[e] = o.v[h * VE + e];
+        stg_nt<R, VE>(out + item * E + h * VE, part);
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------------ 2:4 decompress, streaming
 // In a well-formed 2:4 bitmask every group of 4 columns keeps exactly 2, so the
 // values of group g are values[2g], values[2g+1] and no prefix sum over the
@@ -762,7 +961,11 @@ extern "C" int ctmi_unpack_bitmasks(const uint8_t* packed, uint8_t* mask, int64_
   return check_launch("ctmi_unpack_bitmasks");
 }
 
-extern "C" int64_t ctmi_bitmask_tmp_bytes(int64_t rows) { return (rows < 1 ? 1 : rows) * 8; }
+// per-row counts and offsets for the row kernels, per-tile ones for the tile kernels
+extern "C" int64_t ctmi_bitmask_tmp_bytes(int64_t rows, int64_t cols) {
+  const int64_t r = rows < 1 ? 1 : rows, c = cols < 1 ? 1 : cols;
+  return 16 * r + 16 * cdiv(r * c, kTileElems) + 32;
+}
 
 // per-row counts and offsets, the flag, one verdict per streaming workgroup
 extern "C" int64_t ctmi_sparse24_tmp_bytes(int64_t rows, int64_t cols, int32_t elem_size) {
@@ -846,6 +1049,47 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
   CTMI_REQUIRE(row_offsets || tmp, CTMI_ERR_VALUE, "row_offsets and tmp are both NULL");
   hipStream_t st = (hipStream_t)stream;
   const int64_t pc = cdiv(cols, 8);
+  if (!try_24 && tmp && cols % 8 == 0 && (rows * cols) % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+      (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 16 == 0 && (uintptr_t)tmp % 8 == 0 &&
+      cdiv(rows * cols, kTileElems) < (1ll << 31)) {
+    // positions from the bitmask alone, as in the reference (sparse_bitmask.py:152-169)
+    const int64_t n_items = rows * cols / 16;
+    const int64_t ntiles = cdiv(n_items, kTileItems);
+    const uint16_t* words = reinterpret_cast<const uint16_t*>(bitmask);
+    const int64_t ngroups = cdiv(ntiles, kGroupTiles);
+    int64_t* counts = nullptr;
+    int64_t* offs = nullptr;
+    TileInfo* info = nullptr;
+    int32_t* totals = nullptr;
+    const bool grouped = ngroups <= kMaxGroups;
+    if (grouped) {
+      info = (TileInfo*)tmp;
+      totals = (int32_t*)(info + ntiles);
+      hipLaunchKernelGGL(tile_popcount_groups_kernel, (unsigned)ngroups, kGroupThreads, 0, st,
+                         bitmask, rows * pc, info, totals, ntiles);
+    } else {
+      counts = (int64_t*)tmp;
+      offs = counts + ntiles;
+      hipLaunchKernelGGL(tile_popcount_kernel, (unsigned)cdiv(ntiles, kWaves), kBlock, 0, st,
+                         bitmask, rows * pc, counts, ntiles);
+      hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, offs,
+                         (int64_t*)nullptr, ntiles);
+    }
+#define CTMI_TILES(R)                                                                              \
+  if (grouped)                                                                                     \
+    hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, true>), (unsigned)ntiles, kBlock, 0, st,   \
+                       (const R*)values, nvalues, words, counts, offs, info, totals, (R*)out,      \
+                       n_items);                                                                   \
+  else                                                                                             \
+    hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, false>), (unsigned)ntiles, kBlock, 0, st,  \
+                       (const R*)values, nvalues, words, counts, offs, info, totals, (R*)out,      \
+                       n_items)
+    if (elem_size == 1) { CTMI_TILES(uint8_t); }
+    else if (elem_size == 2) { CTMI_TILES(uint16_t); }
+    else { CTMI_TILES(uint32_t); }
+#undef CTMI_TILES
+    return check_launch(what);
+  }
   int grid = rows_grid(rows);
   int64_t pop_grid = cdiv(rows, kWaves);
   const int* only_if = nullptr;

@@ -193,8 +193,8 @@ int ctmi_unpack_bitmasks(const uint8_t* packed, uint8_t* mask, int64_t rows, int
  * is_float != 0, on the raw integer otherwise.  fp8 tensors are passed as
  * floats with elem_size 1 (sparse_bitmask.py:141-145 views them as int8 only to
  * index them; the mask itself comes from `tensor != 0`).
- * tmp: device scratch of ctmi_bitmask_tmp_bytes(rows) bytes. */
-int64_t ctmi_bitmask_tmp_bytes(int64_t rows);
+ * tmp: device scratch of ctmi_bitmask_tmp_bytes(rows, cols) bytes, 8-byte aligned. */
+int64_t ctmi_bitmask_tmp_bytes(int64_t rows, int64_t cols);
 int ctmi_bitmask_count(const void* x, int32_t elem_size, int32_t is_float, uint8_t* bitmask,
                        int64_t* row_offsets, int64_t* total_nnz, void* tmp, int64_t rows,
                        int64_t cols, void* stream);
@@ -205,8 +205,9 @@ int ctmi_bitmask_compact(const void* x, int32_t elem_size, const uint8_t* bitmas
 /* A18.  bitmask_decompress (sparse_bitmask.py:152-169): scatter `values`
  * (nvalues elements, consumed in row-major order of the set bits; set bits
  * beyond nvalues read as zero) into a zero-filled [rows, cols].
- * row_offsets may be NULL: it is then recomputed from the bitmask into tmp
- * (ctmi_bitmask_tmp_bytes(rows) + rows*8 + 8 bytes). */
+ * With tmp (ctmi_bitmask_tmp_bytes(rows, cols) bytes) the positions come from
+ * the bitmask alone, as in the reference, and row_offsets may be NULL.  Without
+ * tmp, row_offsets is required and trusted. */
 int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_size,
                             const uint8_t* bitmask,
                             const int64_t* row_offsets, void* out, void* tmp, int64_t rows,

@@ -247,3 +247,59 @@ def test_random_shapes_sweep(gpu):
         assert_bit_equal(b24, o_b24, f"24 bitmask {case}")
         assert_bit_equal(sparse24_bitmask_decompress(v24, b24, torch.Size((rows, cols4))),
                          osp.sparse24_bitmask_decompress(o_v24, o_b24, (rows, cols4)), f"24 decompress {case}")
+
+
+def test_bitmask_decompress_with_few_values(gpu):
+    """set bits beyond the values that exist read as zero, also across tiles of the scatter"""
+    from compressed_tensors_amd.compressors import bitmask_decompress
+
+    announce("bitmask decompress, short values")
+    x = _sparse_tensor((64, 4096), torch.bfloat16, 0.5, seed=5)
+    o_values, o_bitmask, _ = osp.bitmask_compress(x)
+    for keep in (o_values.numel() - 1, o_values.numel() // 3, 9, 0):
+        short = o_values[:keep]
+        padded = torch.cat([short, torch.zeros(o_values.numel() - keep, dtype=o_values.dtype)])
+        want = osp.bitmask_decompress(padded, o_bitmask, [64, 4096])
+        assert_bit_equal(bitmask_decompress(short.to(gpu), o_bitmask.to(gpu), [64, 4096]), want, f"keep {keep}")
+
+
+def test_bitmask_many_tiles(gpu):
+    """tensors of several hundred scatter tiles (8192 elements each, whatever the row
+    length), all element sizes, sparsities from empty to full, a ragged last tile"""
+    from compressed_tensors_amd.compressors import bitmask_compress, bitmask_decompress
+
+    cases = [((1024, 4096), torch.bfloat16, 0.5), ((4096, 512), torch.float16, 0.9), ((3, 1048576), torch.bfloat16, 0.1),
+             ((2048, 1032), FP8, 0.5), ((512, 2056), torch.float32, 0.7), ((70000, 8), torch.bfloat16, 0.5),
+             ((512, 4096), torch.bfloat16, 1.0), ((512, 4096), torch.bfloat16, 0.0), ((1001, 24), torch.bfloat16, 0.4)]
+    for shape, dtype, sparsity in cases:
+        announce("bitmask, many tiles", shape, dtype, sparsity)
+        x = _sparse_tensor(shape, dtype, sparsity, seed=shape[1] + 1)
+        o_values, o_bitmask, o_offsets = osp.bitmask_compress(x)
+        values, bitmask, offsets = bitmask_compress(x.to(gpu))
+        assert_bit_equal(values, o_values, "values")
+        assert_bit_equal(bitmask, o_bitmask, "bitmask")
+        assert_bit_equal(offsets, o_offsets, "offsets")
+        assert_bit_equal(bitmask_decompress(values, bitmask, list(shape)),
+                         osp.bitmask_decompress(o_values, o_bitmask, list(shape)), "decompress")
+
+
+def test_bitmask_decompress_of_a_very_large_tensor(gpu):
+    """more tiles than the grouped count handles (> 65536 tiles of 8192 elements): the scatter
+    then takes its positions from a scan over all tiles.  Round trip on the GPU, values and
+    offsets spot-checked against torch."""
+    from compressed_tensors_amd.compressors import bitmask_compress, bitmask_decompress
+
+    announce("bitmask, 537M elements")
+    rows, cols = 65600, 8192
+    g = torch.Generator(device=gpu).manual_seed(1)
+    x = torch.randint(-128, 128, (rows, cols), generator=g, dtype=torch.int8, device=gpu)
+    x[torch.rand((rows, cols), generator=g, device=gpu) < 0.5] = 0
+    values, bitmask, offsets = bitmask_compress(x)
+    nnz_rows = (x != 0).sum(-1)
+    assert values.numel() == int(nnz_rows.sum())
+    assert torch.equal(offsets, torch.cumsum(nnz_rows, 0) - nnz_rows)
+    for r in (0, 1, 40000, rows - 1):
+        lo = int(offsets[r])
+        assert torch.equal(values[lo: lo + int(nnz_rows[r])], x[r][x[r] != 0])
+    back = bitmask_decompress(values, bitmask, [rows, cols])
+    assert torch.equal(back, x)
