@@ -21,10 +21,11 @@ from compressed_tensors_amd.quantization.quant_args import (
 )
 from compressed_tensors_amd.quantization.quant_scheme import QuantizationScheme
 
-__all__ = ["initialize_module_for_quantization", "initialize_qparams", "clear_qparams"]
+__all__ = ["initialize_module_for_quantization", "initialize_qparams", "clear_qparams",
+           "is_attention_module", "initialize_attn_qparams"]
 
 _QPARAM_SUFFIXES = ("_scale", "_zero_point", "_global_scale", "_g_idx")
-_BASE_NAMES = ("input", "weight", "output")
+_BASE_NAMES = ("input", "weight", "output", "q", "k", "v")
 
 
 def clear_qparams(module: Module) -> None:
@@ -34,6 +35,18 @@ def clear_qparams(module: Module) -> None:
             name = base + suffix
             if name in module._parameters:
                 delattr(module, name)
+
+
+def _device_of(module: Module) -> torch.device:
+    """where the module computes: its weight, else its first parameter or buffer (those of
+    its children included), else the CPU"""
+    if isinstance(getattr(module, "weight", None), torch.Tensor):
+        return module.weight.device
+    for t in module.parameters():
+        return t.device
+    for t in module.buffers():
+        return t.device
+    return torch.device("cpu")
 
 
 def _register(module: Module, name: str, value: torch.Tensor) -> None:
@@ -54,7 +67,7 @@ def initialize_qparams(
     args = quantization_args
     strategy = args.strategy
     dynamic = args.dynamic
-    device = module.weight.device if hasattr(module, "weight") else torch.device("cpu")
+    device = _device_of(module)
 
     if dynamic is True:  # scales are computed on the fly: nothing to hold
         return
@@ -120,6 +133,11 @@ def initialize_module_for_quantization(
     if scheme is None:
         return
     clear_qparams(module)
+    if is_attention_module(module):
+        initialize_attn_qparams(module, scheme, force_zero_point)
+        module.quantization_scheme = scheme
+        module.quantization_status = QuantizationStatus.INITIALIZED
+        return
     if not hasattr(module, "weight"):
         return  # a weight is needed to know shapes and dtypes
     weight = module.weight
@@ -134,3 +152,42 @@ def initialize_module_for_quantization(
                            weight.dtype, force_zero_point)
     module.quantization_scheme = scheme
     module.quantization_status = QuantizationStatus.INITIALIZED
+
+
+def is_attention_module(module: Module) -> bool:
+    """reference: initialize.py:147-152"""
+    return "attention" in module.__class__.__name__.lower() and (
+        hasattr(module, "k_proj") or hasattr(module, "v_proj") or hasattr(module, "qkv_proj"))
+
+
+def initialize_attn_qparams(module: Module, scheme: QuantizationScheme, force_zero_point: bool) -> None:
+    """`q_*` parameters if the module calls attention through a QuantizedAttentionImpl, `k_*`
+    and `v_*` if it writes through a QuantizedKVCache; observed shapes are
+    (heads, None, head_dim) (reference: initialize.py:283-337)"""
+    from compressed_tensors_amd.modeling import IMPL_ATTR, KV_CACHE_ATTR
+    from compressed_tensors_amd.utils.helpers import get_head_dim, get_num_attn_heads, get_num_kv_heads
+
+    impl = getattr(module, IMPL_ATTR, None)
+    kv_cache = getattr(module, KV_CACHE_ATTR, None)
+    if impl is None and kv_cache is None:
+        raise ValueError(
+            f"Attention module has quantization scheme but no {IMPL_ATTR} or {KV_CACHE_ATTR} "
+            "attributes. Please ensure that these attributes are initialized using "
+            "`initialize_hooked_attention`.")
+    if scheme.weights is not None:
+        raise ValueError("Cannot apply weight quantization to attention. Instead, target the "
+                         "(q|k|v)_proj submodule layers of attention")
+    if scheme.input_activations is None:
+        raise ValueError("Cannot apply attention quantization without specifying input activations")
+    if scheme.output_activations is not None:
+        raise ValueError("Cannot apply output quantization to attention")
+    config = (kv_cache if kv_cache is not None else impl).config
+    head_dim = get_head_dim(config)
+    dtype = next(module.parameters()).dtype
+    if impl is not None:
+        initialize_qparams(module, "q", scheme.input_activations,
+                           (get_num_attn_heads(config), None, head_dim), dtype, force_zero_point)
+    if kv_cache is not None:
+        kv_shape = (get_num_kv_heads(config), None, head_dim)
+        initialize_qparams(module, "k", scheme.input_activations, kv_shape, dtype, force_zero_point)
+        initialize_qparams(module, "v", scheme.input_activations, kv_shape, dtype, force_zero_point)

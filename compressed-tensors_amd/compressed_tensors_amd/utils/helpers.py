@@ -21,6 +21,10 @@ __all__ = [
     "split_param_name",
     "nest_state_dict",
     "load_safetensors_state_dict",
+    "getattr_chain",
+    "get_num_attn_heads",
+    "get_num_kv_heads",
+    "get_head_dim",
 ]
 
 
@@ -140,3 +144,46 @@ def load_safetensors_state_dict(path, device="cpu"):
             for k in fh.keys():
                 out[k] = fh.get_tensor(k)
     return out
+
+
+_MISSING = object()
+
+
+def getattr_chain(obj, chain_str: str, default=_MISSING):
+    """getattr along a dotted path; `default` (if given) when a link is missing
+    (reference: utils/helpers.py:145-171)"""
+    for name in chain_str.split("."):
+        if not hasattr(obj, name):
+            if default is _MISSING:
+                raise AttributeError(f"{obj} object has no attribute {name}")
+            return default
+        obj = getattr(obj, name)
+    return obj
+
+
+def get_num_attn_heads(config) -> int:
+    """reference: utils/helpers.py:404-422"""
+    if hasattr(config, "num_attention_heads"):
+        return config.num_attention_heads
+    if hasattr(config, "hidden_size") and hasattr(config, "head_dim"):
+        return config.hidden_size // config.head_dim
+    raise ValueError("Cannot determine num_attention_heads from config. Config must define either "
+                     f"`num_attention_heads` or both `hidden_size` and `head_dim`. {config}")
+
+
+def get_num_kv_heads(config) -> int:
+    """reference: utils/helpers.py:425-439"""
+    if hasattr(config, "num_key_value_heads"):
+        return config.num_key_value_heads
+    raise ValueError("Cannot determine num_key_value_heads from config. Config must define "
+                     f"`num_key_value_heads`. {config}")
+
+
+def get_head_dim(config) -> int:
+    """reference: utils/helpers.py:442-460"""
+    if hasattr(config, "head_dim"):
+        return config.head_dim
+    if hasattr(config, "hidden_size") and hasattr(config, "num_attention_heads"):
+        return config.hidden_size // config.num_attention_heads
+    raise ValueError("Cannot determine head_dim from config. Config must define either `head_dim` "
+                     f"or both `hidden_size` and `num_attention_heads`. {config}")

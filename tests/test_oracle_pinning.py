@@ -422,3 +422,23 @@ def test_generate_gparam_is_reciprocal_times_constant():
     closed = ((1.0 / v.float()).to(torch.bfloat16).float() * 2688.0).to(torch.bfloat16).float()
     every = (448.0 * 6.0 / v).float()
     assert torch.equal(every, closed)
+
+
+@pytest.mark.parametrize("case", GOLD_LC["attention_cases"], ids=lambda c: c["args"]["strategy"])
+def test_static_attention_golden(case):
+    """keys of shape (batch, heads, seq, head_dim) quantized per tensor and per head
+    (test_static_lifecycle.py:278-386); the observer reduces everything but the head"""
+    args = _args(case["args"])
+    x = torch.arange(24, dtype=torch.bfloat16).reshape(1, 2, 3, 4)
+    if args.strategy == "tensor":
+        mn, mx = torch.aminmax(x)
+        mn, mx = mn.reshape(1), mx.reshape(1)
+    else:
+        mn = torch.amin(x, dim=(0, 2, 3)).reshape(2, 1, 1)
+        mx = torch.amax(x, dim=(0, 2, 3)).reshape(2, 1, 1)
+    assert torch.equal(mn.float(), torch.tensor(case["min"]))
+    assert torch.equal(mx.float(), torch.tensor(case["max"]))
+    scale, zp = quant.calculate_qparams(mn, mx, args)
+    out = quant.fake_quantize(x, scale, zp, args)
+    assert torch.allclose(out, torch.tensor(case["qdq"]).to(out.dtype))
+    assert torch.nn.functional.mse_loss(out.float(), x.float()) <= case["max_mse"]
