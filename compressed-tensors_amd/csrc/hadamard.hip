@@ -34,9 +34,23 @@ typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int kHadThreads = 256;
 constexpr int kHadWaves = kHadThreads / kWave;
-#ifndef CTMI_HQP_WG_PER_CU
-#define CTMI_HQP_WG_PER_CU 4  // workgroups per CU of the fused rotation + quantization kernel
+#ifndef CTMI_HAD_ROWS_THREADS
+#define CTMI_HAD_ROWS_THREADS 512  // the matrix set-up of hadamard_rows_kernel is shared by a workgroup
 #endif
+constexpr int kRowsThreads = CTMI_HAD_ROWS_THREADS;
+constexpr int kRowsWaves = kRowsThreads / kWave;
+#ifndef CTMI_HAD_KRON_THREADS
+#define CTMI_HAD_KRON_THREADS 256  // measured: 512 is 4 % slower at 64 x 64
+#endif
+constexpr int kKronThreads = CTMI_HAD_KRON_THREADS;
+constexpr int kKronWaves = kKronThreads / kWave;
+#ifndef CTMI_HQP_TUNING
+#define CTMI_HQP_TUNING 1024, 1  // fused rotation + quantization kernel: threads, workgroups per CU
+#endif
+constexpr int kHqpTuning[] = {CTMI_HQP_TUNING};
+constexpr int kHqpThreads = kHqpTuning[0];
+constexpr int kHqpWaves = kHqpThreads / kWave;
+#define CTMI_HQP_WG_PER_CU kHqpTuning[1]
 #ifndef CTMI_HAD_KRON_WAVES
 #define CTMI_HAD_KRON_WAVES 2  // waves per SIMD the kernel for 64 x 64 is built for (measured best)
 #endif
@@ -253,7 +267,7 @@ __global__ void __launch_bounds__(kHadThreads) hadamard_mfma_kernel(HadArgs a) {
 //                    one 16-byte global store.
 // Sign vectors are used as signs: their entries must be +1 or -1.
 template <int B, bool HALF>
-__global__ void __launch_bounds__(kHadThreads)
+__global__ void __launch_bounds__(kRowsThreads)
 hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
                      const uint16_t* __restrict__ mbt, const float* __restrict__ s_in,
                      const float* __restrict__ s_out, int64_t n_sub, float inv_sqrt_n) {
@@ -269,7 +283,7 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   // The matrix fragments are the same in every wave of the workgroup: each wave
   // fetches a quarter of them, and all pick up the whole set from LDS.
   __shared__ u32x4_t frag_lds[2 * NP * KS][kWave];
-  for (int f = wave; f < 2 * NP * KS; f += kHadWaves) {
+  for (int f = wave; f < 2 * NP * KS; f += kRowsWaves) {
     const int nt = f / KS, ks = f % KS;
     const int col = 32 * (nt / 2) + 8 * (l16 / 4) + 4 * (nt % 2) + (l16 % 4);
     u32x4_t m = *reinterpret_cast<const u32x4_t*>(mbt + col * B + 32 * ks + 8 * lq);
@@ -319,8 +333,8 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   }
 
   const int64_t n_full = n_sub / 16;  // whole groups of 16 sub-rows
-  const int64_t stride = (int64_t)gridDim.x * kHadWaves;
-  const int64_t first = (int64_t)blockIdx.x * kHadWaves + wave;
+  const int64_t stride = (int64_t)gridDim.x * kRowsWaves;
+  const int64_t first = (int64_t)blockIdx.x * kRowsWaves + wave;
 
   // Loads are never conditional (a group past the end re-reads the last whole
   // one) and the stores of whole groups are not either: with a fixed number of
@@ -401,13 +415,13 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
 template <int B, bool HALF>
 static int launch_had_rows(const HadArgs& a, hipStream_t st) {
   const int64_t groups = cdiv(a.n_sub, 16);
-  const int64_t wgs = cdiv(groups, kHadWaves);
+  const int64_t wgs = cdiv(groups, kRowsWaves);
   // a wave keeps the matrix in registers: give it several groups to use it on
-  // (as many workgroups as fit on the chip at once: 2 per CU at 128, where a wave
+  // (as many wavefronts as fit on the chip at once: 8 per CU at 128, where a wave
   // needs some 190 registers, more below)
-  const int64_t cap = 256 * (B == 32 ? 4 : 2);
+  const int64_t cap = 256 * (B == 32 ? 16 : 8) / kRowsWaves;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
-  hipLaunchKernelGGL((hadamard_rows_kernel<B, HALF>), grid, kHadThreads, 0, st, (const uint16_t*)a.x,
+  hipLaunchKernelGGL((hadamard_rows_kernel<B, HALF>), grid, kRowsThreads, 0, st, (const uint16_t*)a.x,
                      (uint16_t*)a.out, a.mbt, a.s_in, a.s_out, a.n_sub, 1.0f / a.sqrt_n);
   return CTMI_OK;
 }
@@ -422,7 +436,7 @@ static int launch_had_rows(const HadArgs& a, hipStream_t st) {
 // (unless `rotated` asks for it).  A sub-row's 128 outputs sit in the 4 lanes
 // l16 + 16 q; they agree on min / max through two lane exchanges.
 template <int B>
-__global__ void __launch_bounds__(kHadThreads)
+__global__ void __launch_bounds__(kHqpThreads)
 hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ mbt,
                            const float* __restrict__ s_in, const float* __restrict__ s_out,
                            int32_t* __restrict__ packed, uint16_t* __restrict__ scale,
@@ -438,8 +452,8 @@ hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __res
   // top of 128 for the matrix only one wavefront per SIMD would fit, and it is
   // the number of wavefronts in flight that hides the memory latency here.
   __shared__ u32x4_t frag_lds[2 * NP * KS][kWave];
-  __shared__ __align__(16) int32_t swap_lds[kHadWaves][16][16];
-  for (int f = wave; f < 2 * NP * KS; f += kHadWaves) {
+  __shared__ __align__(16) int32_t swap_lds[kHqpWaves][16][16];
+  for (int f = wave; f < 2 * NP * KS; f += kHqpWaves) {
     const int nt = f / KS, ks = f % KS;
     const int col = 32 * (nt / 2) + 8 * (l16 / 4) + 4 * (nt % 2) + (l16 % 4);
     u32x4_t m = *reinterpret_cast<const u32x4_t*>(mbt + col * B + 32 * ks + 8 * lq);
@@ -457,8 +471,8 @@ hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __res
   __syncthreads();
 
   const int64_t n_groups = (n_sub + 15) / 16;
-  const int64_t stride = (int64_t)gridDim.x * kHadWaves;
-  for (int64_t g = (int64_t)blockIdx.x * kHadWaves + wave; g < n_groups; g += stride) {
+  const int64_t stride = (int64_t)gridDim.x * kHqpWaves;
+  for (int64_t g = (int64_t)blockIdx.x * kHqpWaves + wave; g < n_groups; g += stride) {
     int64_t row = g * 16 + l16;
     const bool keep = row < n_sub;
     if (!keep) row = n_sub - 1;  // ragged last group: recompute the last sub-row, store nothing
@@ -555,7 +569,7 @@ hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __res
 // output; they are per position within the row, the same for every row, and sit
 // in LDS in the lanes' own layout.
 template <int A, int B, bool HALF>
-__global__ void __launch_bounds__(kHadThreads) __attribute__((amdgpu_waves_per_eu(CTMI_HAD_KRON_WAVES)))
+__global__ void __launch_bounds__(kKronThreads) __attribute__((amdgpu_waves_per_eu(CTMI_HAD_KRON_WAVES)))
 hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
                      const uint16_t* __restrict__ mbt, const uint16_t* __restrict__ mat,
                      const float* __restrict__ s_in, const float* __restrict__ s_out,
@@ -582,7 +596,7 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
     const uint32_t* pin = reinterpret_cast<const uint32_t*>(s_in ? (const void*)s_in : (const void*)mbt);
     const uint32_t* pout = reinterpret_cast<const uint32_t*>(s_out ? (const void*)s_out : (const void*)mbt);
     const uint32_t use_in = s_in ? 1u : 0u, use_out = s_out ? 1u : 0u;
-    for (int f = wave; f < MT * KS; f += kHadWaves) {
+    for (int f = wave; f < MT * KS; f += kKronWaves) {
       const int m = f / KS, ks = f % KS;
       const int pos = (32 * (m / 2) + 4 * (m % 2) + perm) * B + 32 * ks + 8 * lq;
       u32x4_t w;
@@ -591,7 +605,7 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
         w[d] = (((pin[pos + 2 * d] >> 31) & use_in) << 15) | (((pin[pos + 2 * d + 1] >> 31) & use_in) << 31);
       sign_in_lds[f][lane] = w;
     }
-    for (int f = wave; f < AT * (NT / 2); f += kHadWaves) {
+    for (int f = wave; f < AT * (NT / 2); f += kKronWaves) {
       const int at = f / (NT / 2), p = f % (NT / 2);
       const int pos = (16 * at + l16) * B + 32 * p + 8 * lq;
       u32x4_t w;
@@ -627,8 +641,8 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
       maf[at][ps] = __builtin_bit_cast(
           bf16x8_t, ldg<uint16_t, 8>(mat + (16 * at + l16) * A + 32 * ps + 8 * lq));
 
-  const int64_t stride = (int64_t)gridDim.x * kHadWaves;
-  for (int64_t row = (int64_t)blockIdx.x * kHadWaves + wave; row < n_rows; row += stride) {
+  const int64_t stride = (int64_t)gridDim.x * kKronWaves;
+  for (int64_t row = (int64_t)blockIdx.x * kKronWaves + wave; row < n_rows; row += stride) {
     const uint16_t* src = x + row * N;
     uint16_t* dst = out + row * N;
     xfrag_t xf[MT][KS];
@@ -719,11 +733,11 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
 template <int A, int B, bool HALF>
 static int launch_had_kron(const HadArgs& a, hipStream_t st) {
   const int64_t n_rows = a.n_sub / A;
-  const int64_t wgs = cdiv(n_rows, kHadWaves);
+  const int64_t wgs = cdiv(n_rows, kKronWaves);
   // as many workgroups as are resident at once (register-limited)
-  const int64_t cap = 256 * (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES));
+  const int64_t cap = 256 * 4 * (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES)) / kKronWaves;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
-  hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF>), grid, kHadThreads, 0, st, (const uint16_t*)a.x,
+  hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF>), grid, kKronThreads, 0, st, (const uint16_t*)a.x,
                      (uint16_t*)a.out, a.mbt, a.mat, a.s_in, a.s_out, n_rows, 1.0f / a.sqrt_n);
   return CTMI_OK;
 }
@@ -907,13 +921,13 @@ extern "C" int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t
   c.mt = c.zp_sub_dtype = c.scale_dtype = CTMI_BF16;
   c.zp_dtype = CTMI_I8;
   const int64_t n_sub = numel / b_dim;
-  const int64_t wgs = cdiv(cdiv(n_sub, 16), kHadWaves);
+  const int64_t wgs = cdiv(cdiv(n_sub, 16), kHqpWaves);
   const int64_t cap = 256 * CTMI_HQP_WG_PER_CU;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
   const float inv = 1.0f / sqrtf((float)b_dim);
   hipStream_t st = (hipStream_t)stream;
 #define CTMI_HQP(BB)                                                                              \
-  hipLaunchKernelGGL(hadamard_quant_pack_kernel<BB>, grid, kHadThreads, 0, st, (const uint16_t*)x, \
+  hipLaunchKernelGGL(hadamard_quant_pack_kernel<BB>, grid, kHqpThreads, 0, st, (const uint16_t*)x, \
                      (const uint16_t*)mb_t, sign_in, sign_out, packed, (uint16_t*)scale,          \
                      (uint16_t*)rotated, n_sub, inv, c)
   if (b_dim == 32) CTMI_HQP(32);
