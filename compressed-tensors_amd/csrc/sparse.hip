@@ -255,25 +255,6 @@ row_offsets_kernel(const int64_t* __restrict__ counts, int64_t* __restrict__ off
   scan_rows(counts, offsets, total, rows, wsum);
 }
 
-// What follows a 2:4 streaming pass (sparse24_scatter_kernel): one workgroup looks at
-// the verdicts the streaming workgroups left, one word each, and publishes the
-// answer in *flag for the scatter kernel behind it.  If a group did not keep exactly
-// 2 of 4 it also prepares the general scatter: per-row popcounts and their prefix.
-__global__ void __launch_bounds__(kScanThreads)
-sparse24_verdict_kernel(const int* __restrict__ verdicts, int64_t n_verdicts, int* __restrict__ flag,
-                        const uint8_t* __restrict__ bitmask, int64_t* __restrict__ counts,
-                        int64_t* __restrict__ offsets, int64_t rows, int64_t cols, int64_t pc) {
-  __shared__ int64_t wsum[kScanThreads / kWave];
-  int bad = 0;
-  for (int64_t i = threadIdx.x; i < n_verdicts; i += kScanThreads) bad |= verdicts[i];
-  bad = __syncthreads_or(bad);
-  if (threadIdx.x == 0) *flag = bad ? 1 : 0;
-  if (!bad) return;
-  popcount_rows(bitmask, counts, rows, cols, pc, threadIdx.x / kWave, kScanThreads / kWave);
-  __syncthreads();  // counts are read back by other wavefronts of this workgroup
-  scan_rows(counts, offsets, nullptr, rows, wsum);
-}
-
 // ------------------------------------------------------------------ sparse-bitmask: compaction
 // One workgroup per row, 2048 columns per iteration.  Survivors are first
 // gathered into LDS at their rank within the iteration, then the contiguous
@@ -322,49 +303,59 @@ bitmask_compact_kernel(const R* __restrict__ x, const uint8_t* __restrict__ bitm
 }
 
 // ------------------------------------------------------------------ bitmask decompress (scatter)
+// One row by one workgroup, 2048 columns per step: the step's values are staged in
+// LDS, every thread picks its own 8.  `src` is where the row's values start and is
+// moved past them.  A bitmask with more set bits than there are values reads
+// zeros, never past the end.
+template <typename R>
+__device__ __forceinline__ void scatter_row(const R* __restrict__ values, int64_t nvalues,
+                                            const uint8_t* __restrict__ mask_row, int64_t& src,
+                                            R* __restrict__ row, int64_t cols, int64_t pc, bool vec,
+                                            uint32_t tail, int* scan_s, R* stage) {
+  for (int64_t b0 = 0; b0 < pc; b0 += kBlock) {
+    const int64_t b = b0 + threadIdx.x;
+    uint32_t bits = 0;
+    if (b < pc) {
+      bits = mask_row[b];
+      if (b == pc - 1) bits &= tail;
+    }
+    int pre, total;
+    block_exclusive_scan(__popc(bits), &pre, &total, scan_s);
+    for (int i = threadIdx.x; i < total; i += kBlock)
+      stage[i] = (src + i < nvalues) ? values[src + i] : (R)0;
+    src += total;
+    __syncthreads();
+    if (b < pc) {
+      Vec<R, 8> o;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o.v[j] = ((bits >> j) & 1u) ? stage[pre++] : (R)0;
+      if (vec) {
+        stg<R, 8>(row + b * 8, o);
+      } else {
+        for (int j = 0; j < 8; ++j) {
+          const int64_t c = b * 8 + j;
+          if (c < cols) row[c] = o.v[j];
+        }
+      }
+    }
+    __syncthreads();
+  }
+}
+
 template <typename R>
 __global__ void __launch_bounds__(kBlock)
 bitmask_scatter_kernel(const R* __restrict__ values, int64_t nvalues,
                        const uint8_t* __restrict__ bitmask,
                        const int64_t* __restrict__ row_offsets, R* __restrict__ out, int64_t rows,
-                       int64_t cols, int64_t pc, const int* only_if) {
-  if (only_if && *only_if == 0) return;
+                       int64_t cols, int64_t pc) {
   __shared__ int scan_s[kWaves];
   __shared__ R stage[kBlock * 8];
   const bool vec = (cols % 8 == 0) && ((uintptr_t)out % (8 * sizeof(R)) == 0);
   const uint32_t tail = (cols % 8) ? ((1u << (cols % 8)) - 1u) : 0xffu;
   for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
-    R* row = out + r * cols;
     int64_t src = row_offsets[r];
-    for (int64_t b0 = 0; b0 < pc; b0 += kBlock) {
-      const int64_t b = b0 + threadIdx.x;
-      uint32_t bits = 0;
-      if (b < pc) {
-        bits = bitmask[r * pc + b];
-        if (b == pc - 1) bits &= tail;
-      }
-      int pre, total;
-      block_exclusive_scan(__popc(bits), &pre, &total, scan_s);
-      // a bitmask with more set bits than there are values reads zeros, never past the end
-      for (int i = threadIdx.x; i < total; i += kBlock)
-        stage[i] = (src + i < nvalues) ? values[src + i] : (R)0;
-      src += total;
-      __syncthreads();
-      if (b < pc) {
-        Vec<R, 8> o;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) o.v[j] = ((bits >> j) & 1u) ? stage[pre++] : (R)0;
-        if (vec) {
-          stg<R, 8>(row + b * 8, o);
-        } else {
-          for (int j = 0; j < 8; ++j) {
-            const int64_t c = b * 8 + j;
-            if (c < cols) row[c] = o.v[j];
-          }
-        }
-      }
-      __syncthreads();
-    }
+    scatter_row<R>(values, nvalues, bitmask + r * pc, src, out + r * cols, cols, pc, vec, tail, scan_s,
+                   stage);
   }
 }
 
@@ -383,8 +374,7 @@ __global__ void __launch_bounds__(kBlock)
 bitmask_scatter_wave_kernel(const R* __restrict__ values, int64_t nvalues,
                             const uint8_t* __restrict__ bitmask,
                             const int64_t* __restrict__ row_offsets, R* __restrict__ out,
-                            int64_t rows, int64_t cols, int64_t pc, const int* only_if) {
-  if (only_if && *only_if == 0) return;
+                            int64_t rows, int64_t cols, int64_t pc) {
   constexpr int VE = 16 / (int)sizeof(R);  // elements per 16-byte vector
   __shared__ __align__(16) R stage_all[kWaves][kScatterSpan + 2 * VE];
   const int lane = lane_id(), wave = threadIdx.x / kWave;
@@ -664,8 +654,9 @@ bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
 // bitmask is needed: a lane turns E columns' worth of mask bits and E/2 values
 // into one 16-byte store.  Whether the bitmask IS well formed is only known once
 // all of it has been looked at: every lane checks its own bits and raises
-// a verdict for its workgroup otherwise, and the general kernels, enqueued behind this one, do
-// their work (and overwrite the output) only if the flag went up.
+// a verdict for its workgroup otherwise, and sparse24_repair_kernel, enqueued behind
+// this one, does the general scatter (and overwrites the output) only if a verdict
+// went up.
 template <typename R>
 struct Scatter24 {
   static constexpr int E = sizeof(R) == 1 ? 16 : 8;  // columns per lane
@@ -723,6 +714,43 @@ sparse24_scatter_kernel(const R* __restrict__ values, const uint8_t* __restrict_
   // every workgroup leaves its verdict, good or bad: nothing has to be cleared beforehand
   const int any_bad = __syncthreads_or(bad);
   if (threadIdx.x == 0) verdicts[blockIdx.x] = any_bad ? 1 : 0;
+}
+
+// What follows the streaming pass: every workgroup looks at all the verdicts (a few
+// KB, from L2) and is done if none is up.  Otherwise the bitmask is not 2:4 and the
+// workgroups redo the tensor as a general scatter, rows dealt round-robin; where a
+// row's values start is the number of set bits before it, which each workgroup
+// counts by itself as it moves from one of its rows to the next (rows are whole
+// bitmask bytes here, so the rows in between are one run of bytes).  Slow next to
+// the streaming pass, but it only runs for a bitmask that no 2:4 compressor wrote.
+template <typename R>
+__global__ void __launch_bounds__(kBlock)
+sparse24_repair_kernel(const R* __restrict__ values, int64_t nvalues,
+                       const uint8_t* __restrict__ bitmask, R* __restrict__ out, int64_t rows,
+                       int64_t cols, int64_t pc, const int* __restrict__ verdicts,
+                       int64_t n_verdicts) {
+  __shared__ int scan_s[kWaves];
+  __shared__ int64_t red[kWaves];
+  __shared__ R stage[kBlock * 8];
+  uint32_t bad = 0;
+  const int64_t quads = n_verdicts / 4;  // 16 bytes per load; verdicts is 16-byte aligned
+  const u32x4_t* v4 = reinterpret_cast<const u32x4_t*>(verdicts);
+  for (int64_t i = threadIdx.x; i < quads; i += kBlock) {
+    const u32x4_t q = v4[i];
+    bad |= q.x | q.y | q.z | q.w;
+  }
+  for (int64_t i = quads * 4 + threadIdx.x; i < n_verdicts; i += kBlock) bad |= (uint32_t)verdicts[i];
+  if (!__syncthreads_or((int)bad)) return;
+  const bool vec = (uintptr_t)out % (8 * sizeof(R)) == 0;
+  int64_t src = 0, counted = 0;  // set bits in rows [0, counted)
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    int64_t c = 0;
+    for (int64_t b = counted * pc + threadIdx.x; b < r * pc; b += kBlock) c += __popc((uint32_t)bitmask[b]);
+    src += block_sum(c, red);
+    scatter_row<R>(values, nvalues, bitmask + r * pc, src, out + r * cols, cols, pc, vec, 0xffu, scan_s,
+                   stage);
+    counted = r + 1;
+  }
 }
 
 // ------------------------------------------------------------------ 2:4 selection
@@ -967,11 +995,13 @@ extern "C" int64_t ctmi_bitmask_tmp_bytes(int64_t rows, int64_t cols) {
   return 16 * r + 16 * cdiv(r * c, kTileElems) + 32;
 }
 
-// per-row counts and offsets, the flag, one verdict per streaming workgroup
+// one verdict per streaming workgroup, or what the general kernels need
 extern "C" int64_t ctmi_sparse24_tmp_bytes(int64_t rows, int64_t cols, int32_t elem_size) {
   const int64_t r = rows < 1 ? 1 : rows, c = cols < 1 ? 1 : cols;
   const int64_t items = cdiv(r * c, elem_size == 1 ? 16 : 8);
-  return r * 16 + 8 + 4 * cdiv(items, kBlock * 2) + 8;
+  const int64_t verdicts = 4 * cdiv(items, kBlock * 2) + 8;
+  const int64_t general = ctmi_bitmask_tmp_bytes(rows, cols);
+  return verdicts > general ? verdicts : general;
 }
 
 static int check_elem(int32_t elem_size) {
@@ -1049,11 +1079,34 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
   CTMI_REQUIRE(row_offsets || tmp, CTMI_ERR_VALUE, "row_offsets and tmp are both NULL");
   hipStream_t st = (hipStream_t)stream;
   const int64_t pc = cdiv(cols, 8);
-  if (!try_24 && tmp && cols % 8 == 0 && (rows * cols) % 16 == 0 && (uintptr_t)out % 16 == 0 &&
+  const int64_t numel = rows * cols;
+  // exactly half as many values as elements, rows of whole bitmask bytes: the 2:4
+  // streaming kernel, and behind it the kernel that redoes the work if the bitmask
+  // turns out not to be 2:4 (see sparse24_scatter_kernel)
+  const int e24 = elem_size == 1 ? 16 : 8;
+  if (try_24 && tmp && nvalues * 2 == numel && cols % 8 == 0 && numel % e24 == 0 &&
+      (uintptr_t)out % 16 == 0 && (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 2 == 0 &&
+      (uintptr_t)tmp % 16 == 0 && numel / e24 < (1ll << 40)) {
+    int* verdicts = (int*)tmp;
+    const int64_t n_items = numel / e24;
+    const unsigned g24 = (unsigned)cdiv(n_items, kBlock * 2);
+    const unsigned repair_grid = (unsigned)(rows < 32 ? rows : 32);
+#define CTMI_24(R)                                                                               \
+  hipLaunchKernelGGL(sparse24_scatter_kernel<R>, g24, kBlock, 0, st, (const R*)values, bitmask,  \
+                     (R*)out, n_items, verdicts);                                                \
+  hipLaunchKernelGGL(sparse24_repair_kernel<R>, repair_grid, kBlock, 0, st, (const R*)values,    \
+                     nvalues, bitmask, (R*)out, rows, cols, pc, verdicts, (int64_t)g24)
+    if (elem_size == 1) { CTMI_24(uint8_t); }
+    else if (elem_size == 2) { CTMI_24(uint16_t); }
+    else { CTMI_24(uint32_t); }
+#undef CTMI_24
+    return check_launch(what);
+  }
+  if (tmp && cols % 8 == 0 && numel % 16 == 0 && (uintptr_t)out % 16 == 0 &&
       (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 16 == 0 && (uintptr_t)tmp % 8 == 0 &&
-      cdiv(rows * cols, kTileElems) < (1ll << 31)) {
+      cdiv(numel, kTileElems) < (1ll << 31)) {
     // positions from the bitmask alone, as in the reference (sparse_bitmask.py:152-169)
-    const int64_t n_items = rows * cols / 16;
+    const int64_t n_items = numel / 16;
     const int64_t ntiles = cdiv(n_items, kTileItems);
     const uint16_t* words = reinterpret_cast<const uint16_t*>(bitmask);
     const int64_t ngroups = cdiv(ntiles, kGroupTiles);
@@ -1090,57 +1143,28 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
 #undef CTMI_TILES
     return check_launch(what);
   }
-  int grid = rows_grid(rows);
-  int64_t pop_grid = cdiv(rows, kWaves);
-  const int* only_if = nullptr;
+  // any other shape: per-row counts, their prefix, one wavefront or workgroup per row
+  const int grid = rows_grid(rows);
   if (!row_offsets) {
     int64_t* counts = (int64_t*)tmp;
     int64_t* offs = counts + rows;
-    // exactly half as many values as elements, rows of whole bitmask bytes: try
-    // the 2:4 streaming kernel first (see sparse24_scatter_kernel)
-    const int64_t numel = rows * cols;
-    const int e = elem_size == 1 ? 16 : 8;
-    if (try_24 && nvalues * 2 == numel && cols % 8 == 0 && numel % e == 0 && (uintptr_t)out % 16 == 0 &&
-        (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 2 == 0 && numel / e < (1ll << 40)) {
-      int* flag = (int*)(offs + rows);
-      int* verdicts = flag + 2;
-      const int64_t n_items = numel / e;
-      const unsigned g24 = (unsigned)cdiv(n_items, kBlock * 2);
-      if (elem_size == 1)
-        hipLaunchKernelGGL(sparse24_scatter_kernel<uint8_t>, g24, kBlock, 0, st,
-                           (const uint8_t*)values, bitmask, (uint8_t*)out, n_items, verdicts);
-      else if (elem_size == 2)
-        hipLaunchKernelGGL(sparse24_scatter_kernel<uint16_t>, g24, kBlock, 0, st,
-                           (const uint16_t*)values, bitmask, (uint16_t*)out, n_items, verdicts);
-      else
-        hipLaunchKernelGGL(sparse24_scatter_kernel<uint32_t>, g24, kBlock, 0, st,
-                           (const uint32_t*)values, bitmask, (uint32_t*)out, n_items, verdicts);
-      hipLaunchKernelGGL(sparse24_verdict_kernel, 1, kScanThreads, 0, st, verdicts, (int64_t)g24,
-                         flag, bitmask, counts, offs, rows, cols, pc);
-      only_if = flag;
-      // the scatter below now only runs in the rare malformed case: keep its grid
-      // small, an empty launch costs by the workgroup
-      if (grid > 1024) grid = 1024;
-    } else {
-      if (pop_grid > (1 << 20)) pop_grid = 1 << 20;
-      hipLaunchKernelGGL(bitmask_popcount_kernel, (unsigned)pop_grid, kBlock, 0, st, bitmask,
-                         counts, rows, cols, pc);
-      hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, offs,
-                         (int64_t*)nullptr, rows);
-    }
+    int64_t pop_grid = cdiv(rows, kWaves);
+    if (pop_grid > (1 << 20)) pop_grid = 1 << 20;
+    hipLaunchKernelGGL(bitmask_popcount_kernel, (unsigned)pop_grid, kBlock, 0, st, bitmask, counts,
+                       rows, cols, pc);
+    hipLaunchKernelGGL(row_offsets_kernel, 1, kScanThreads, 0, st, counts, offs, (int64_t*)nullptr,
+                       rows);
     row_offsets = offs;
   }
 #define CTMI_SCATTER(R)                                                                           \
   if (scatter_wave_ok<R>(values, bitmask, out, cols))                                             \
     hipLaunchKernelGGL(bitmask_scatter_wave_kernel<R>, (unsigned)wave_grid, kBlock, 0, st,        \
-                       (const R*)values, nvalues, bitmask, row_offsets, (R*)out, rows, cols, pc,  \
-                       only_if);                                                                  \
+                       (const R*)values, nvalues, bitmask, row_offsets, (R*)out, rows, cols, pc); \
   else                                                                                            \
     hipLaunchKernelGGL(bitmask_scatter_kernel<R>, grid, kBlock, 0, st, (const R*)values, nvalues, \
-                       bitmask, row_offsets, (R*)out, rows, cols, pc, only_if)
+                       bitmask, row_offsets, (R*)out, rows, cols, pc)
   int64_t wave_grid = cdiv(rows, kWaves);
   if (wave_grid > (1 << 24)) wave_grid = 1 << 24;
-  if (only_if && wave_grid > 512) wave_grid = 512;  // rarely does anything: keep the launch small
   if (elem_size == 1) { CTMI_SCATTER(uint8_t); }
   else if (elem_size == 2) { CTMI_SCATTER(uint16_t); }
   else { CTMI_SCATTER(uint32_t); }
