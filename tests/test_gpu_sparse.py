@@ -303,3 +303,51 @@ def test_bitmask_decompress_of_a_very_large_tensor(gpu):
         assert torch.equal(values[lo: lo + int(nnz_rows[r])], x[r][x[r] != 0])
     back = bitmask_decompress(values, bitmask, [rows, cols])
     assert torch.equal(back, x)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, FP8])
+@pytest.mark.parametrize("shard_dim,shard_sizes", [(0, [256, 128, 128]), (1, [64, 64, 128]), (1, [128, 128])])
+def test_sparse24_shards_recombine(dtype, shard_dim, shard_sizes, gpu):
+    """compressed values and bitmask cut into shards along either dimension decompress
+    shard by shard into the pieces of the dense tensor
+    (reference: tests/test_compressors/sparse_compressors/test_sparse_24_bitmask.py:99-145)"""
+    from compressed_tensors_amd.compressors import Sparse24BitMaskTensor
+    from compressed_tensors_amd.utils import combine_shards, shard_tensor
+
+    announce("sparse24 shards", dtype, shard_dim, shard_sizes)
+    m, k = (512, 256)
+    x = _prune24(_sparse_tensor((m, k), torch.bfloat16, 0.0, seed=3).float()).to(torch.bfloat16)
+    if dtype == FP8:
+        x = (x.float() * 50).to(FP8)
+    t = Sparse24BitMaskTensor.from_dense(x.to(gpu))
+    v_sizes = [s // 2 for s in shard_sizes] if shard_dim == 1 else shard_sizes
+    b_sizes = [s // 8 for s in shard_sizes] if shard_dim == 1 else shard_sizes
+    pieces = []
+    for values, bitmask in zip(shard_tensor(t.compressed, v_sizes, dim=shard_dim),
+                               shard_tensor(t.bitmask, b_sizes, dim=shard_dim)):
+        shape = (bitmask.shape[0], bitmask.shape[1] * 8)
+        pieces.append(Sparse24BitMaskTensor(shape=shape, compressed=values.contiguous(),
+                                            bitmask=bitmask.contiguous()).decompress())
+    want = osp.sparse24_bitmask_decompress(*osp.sparse24_bitmask_compress(x), (m, k))
+    assert_bit_equal(combine_shards(pieces, dim=shard_dim), want, "recombined")
+
+
+def test_sparse24_repair_over_many_rows(gpu):
+    """a bitmask that is not 2:4 in a tensor of thousands of rows: the kernel behind the
+    streaming pass redoes every row, each workgroup counting the set bits before its rows"""
+    from compressed_tensors_amd.compressors import sparse24_bitmask_decompress
+    from compressed_tensors_amd.utils.helpers import pack_bitmasks
+
+    announce("sparse24 repair, 3000 rows")
+    rows, cols = 3000, 512
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn(rows, cols, generator=g).bfloat16()
+    x[x == 0] = 1.0
+    # half of the elements kept, row by row, at random places: right total, wrong groups
+    keep = torch.zeros(rows, cols, dtype=torch.bool)
+    order = torch.rand(rows, cols, generator=g).argsort(dim=1)[:, : cols // 2]
+    keep.scatter_(1, order, True)
+    x = torch.where(keep, x, torch.zeros_like(x))
+    values = x[keep].reshape(rows, cols // 2)
+    dense = sparse24_bitmask_decompress(values.to(gpu), pack_bitmasks(keep.to(gpu)), torch.Size((rows, cols)))
+    assert_bit_equal(dense, x, "repaired")
