@@ -301,6 +301,28 @@ def other_workload(torch, name, seed):
             nbytes = 5 * (2 * r * c + r * c // 16 + r * c // 2)
             ops += [Op(f"nvfp4 compress {r}x{c} (x5)", c_calls, nbytes, "nvfp4_compress_vec_kernel"),
                     Op(f"nvfp4 decompress {r}x{c} (x5)", d_calls, nbytes, "nvfp4_decompress_vec_kernel")]
+        # the Llama-3-8B-shaped set: one call per weight against all 224 in one call
+        from compressed_tensors_amd.compressors import Fp4WeightBatch
+        entries, single_c, single_d, n_set = [], [], [], 0
+        for _, r, c in shapes_for("llama3-8b-w4a16"):
+            w = randn(r, c, 0.02)
+            gs = generate_gparam(w.min().reshape(1), w.max().reshape(1))
+            scale, zp = observe_weight_qparams(w, args, global_scale=gs)
+            entries.append(dict(weight=w, scale=scale, global_scale=gs, quantization_args=args))
+            n_set += r * c
+        batch = Fp4WeightBatch(entries)
+        keep.append(batch)
+        for i in range(batch.n):
+            cj, dj = batch._cjobs[i], batch._djobs[i]
+            ca = (cj.src, cj.dense_dtype, cj.dst, cj.rows, cj.cols, ctypes.byref(cj.qp), st)
+            da = (dj.src, dj.dst, dj.dense_dtype, dj.rows, dj.cols, ctypes.byref(dj.qp), st)
+            single_c.append(lambda ca=ca: _lib.check(lib.ctmi_nvfp4_compress(*ca)))
+            single_d.append(lambda da=da: _lib.check(lib.ctmi_nvfp4_decompress(*da)))
+        set_bytes = 2 * n_set + n_set // 16 + n_set // 2
+        ops += [Op("nvfp4 compress, Llama-3-8B set, one call per weight (224)", single_c, set_bytes, "nvfp4_compress_vec_kernel"),
+                Op("nvfp4 compress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.compress], set_bytes, "nvfp4_compress_chain_kernel"),
+                Op("nvfp4 decompress, Llama-3-8B set, one call per weight (224)", single_d, set_bytes, "nvfp4_decompress_vec_kernel"),
+                Op("nvfp4 decompress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.decompress], set_bytes, "nvfp4_decompress_chain_kernel")]
         aargs = QuantizationArgs(num_bits=4, type="float", symmetric=True, strategy="tensor_group",
                                  group_size=16, dynamic="local")
         o_calls, f_calls, y_calls = [], [], []

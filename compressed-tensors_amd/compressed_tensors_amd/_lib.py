@@ -134,6 +134,8 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_int32, c_int64, c_int64, _QP, c_void_p],
     ),
     "ctmi_pack_quantized_compress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
+    "ctmi_nvfp4_compress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
+    "ctmi_nvfp4_decompress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
     "ctmi_pack_quantized_decompress_many": (c_int32, [POINTER(WeightJob), c_int64, c_void_p]),
     "ctmi_pack_quantized_launches": (c_int64, [POINTER(WeightJob), c_int64, c_int32]),
     "ctmi_pack_fp4_to_uint8": (c_int32, [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_void_p]),

@@ -22,6 +22,7 @@ from compressed_tensors_amd.quantization.forward import (
 from compressed_tensors_amd.quantization.quant_args import QuantizationArgs
 
 __all__ = [
+    "Fp4WeightBatch",
     "NVFP4PackedCompressor",
     "MXFP4PackedCompressor",
     "pack_fp4_to_uint8",
@@ -176,6 +177,114 @@ class NVFP4PackedCompressor(BaseQuantizationCompressor):
             )
         )
         return out
+
+
+class Fp4WeightBatch:
+    """Every nvfp4 weight of a state dict prepared for one-call compress / decompress
+    (ctmi_nvfp4_{compress,decompress}_many).  Buffers are allocated once; `compress()`
+    and `decompress()` only enqueue kernels."""
+
+    def __init__(self, entries):
+        """entries: dicts with keys weight, scale (fp8 group scales), global_scale,
+        quantization_args, optionally zero_point"""
+        self.n = len(entries)
+        self._keep = []
+        self.weights, self.packed, self.dense = [], [], []
+        self._cjobs = (_lib.WeightJob * max(self.n, 1))()
+        self._djobs = (_lib.WeightJob * max(self.n, 1))()
+        self.device = None
+        for i, e in enumerate(entries):
+            args = e["quantization_args"]
+            w, scale, gs, zp = (to_gpu(e.get(k)) for k in ("weight", "scale", "global_scale", "zero_point"))
+            if w.ndim != 2:
+                raise ValueError(f"expected a 2-D weight, got shape {tuple(w.shape)}")
+            if self.device is None:
+                self.device = w.device
+            w = w.contiguous()
+            rows, cols = w.shape
+            if cols % 2 != 0:
+                raise ValueError("tensor must have an even number of columns for nvfp4 compression")
+            packed = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
+            cplan = build_qparams(w, scale, zp, args, None, gs)
+            carrier = _ShapeOnly(w.shape, torch.bfloat16)
+            dq_args = infer_dequant_args(carrier, scale)
+            dplan = build_qparams(carrier, scale, None, dq_args, None, gs)
+            dplan.qp.qtype, dplan.qp.num_bits = _lib.QTYPE_FLOAT, 4
+            out_dtype = torch.bfloat16 if dplan.grouped else dplan.dequant_dtype
+            dense = torch.empty((rows, cols), dtype=out_dtype, device=w.device)
+            self._keep += [cplan, dplan]
+            cj, dj = self._cjobs[i], self._djobs[i]
+            cj.src, cj.dst, cj.rows, cj.cols = w.data_ptr(), packed.data_ptr(), rows, cols
+            cj.dense_dtype, cj.qp = _lib.dtype_code(w.dtype), cplan.qp
+            dj.src, dj.dst, dj.rows, dj.cols = packed.data_ptr(), dense.data_ptr(), rows, cols
+            dj.dense_dtype, dj.qp = _lib.dtype_code(out_dtype), dplan.qp
+            self.weights.append(w)
+            self.packed.append(packed)
+            self.dense.append(dense)
+
+    def compress(self):
+        """enqueue quantize + pack of every weight; returns the packed tensors"""
+        if self.n:
+            _lib.check(_lib.load().ctmi_nvfp4_compress_many(self._cjobs, self.n, _lib.stream_of(self.device)))
+        return self.packed
+
+    def decompress(self):
+        """enqueue unpack + dequantize of every packed weight; returns the dense tensors"""
+        if self.n:
+            _lib.check(_lib.load().ctmi_nvfp4_decompress_many(self._djobs, self.n, _lib.stream_of(self.device)))
+        return self.dense
+
+
+def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,
+                                 compression_device=None, **kwargs):
+    """BaseQuantizationCompressor.compress (quantized_compressors/base.py:69-161) with
+    every nvfp4 weight handed to the C ABI in one call: same keys, dtypes and values as
+    the per-weight loop."""
+    jobs, names = [], []
+    for name in list(model_state.keys()):
+        if not name.endswith("weight"):
+            continue
+        prefix = name[: -len("weight")]
+        scale = model_state.get(prefix + "weight_scale", None)
+        gs = model_state.get(prefix + "weight_global_scale", None)
+        weight = model_state[name]
+        if scale is None or gs is None or weight.ndim != 2 or weight.numel() == 0:
+            continue  # the per-weight path below deals with it (or raises as the reference does)
+        module_path = prefix[:-1] if prefix.endswith(".") else prefix
+        jobs.append(dict(weight=weight, scale=scale, global_scale=gs,
+                         zero_point=model_state.get(prefix + "weight_zero_point", None),
+                         quantization_args=names_to_scheme[module_path].weights))
+        names.append(name)
+    packed_by_name = dict(zip(names, Fp4WeightBatch(jobs).compress())) if jobs else {}
+
+    def move(t):
+        return t if compression_device is None else t.to(compression_device)
+
+    out = {}
+    for name in list(model_state.keys()):
+        value = model_state[name]
+        prefix = name[: -len("weight")] if name.endswith("weight") else None
+        if name in packed_by_name:
+            out[prefix + "weight_packed"] = move(packed_by_name[name])
+        elif prefix is not None and model_state.get(prefix + "weight_scale") is not None:
+            module_path = prefix[:-1] if prefix.endswith(".") else prefix
+            single = self.compress_weight(
+                weight=value, scale=model_state[prefix + "weight_scale"],
+                global_scale=model_state.get(prefix + "weight_global_scale", None),
+                zero_point=model_state.get(prefix + "weight_zero_point", None),
+                g_idx=model_state.get(prefix + "weight_g_idx", None),
+                quantization_args=names_to_scheme[module_path].weights,
+                device=compression_device)
+            for key, tensor in single.items():
+                out[prefix + key] = move(tensor)
+        elif name.endswith("zero_point") and self._skip_zp(name, names_to_scheme):
+            continue
+        else:
+            out[name] = move(value)
+    return out
+
+
+NVFP4PackedCompressor.compress = _compress_state_dict_batched
 
 
 @BaseCompressor.register(name=CompressionFormat.mxfp4_pack_quantized.value)

@@ -15,6 +15,7 @@
 #include "qparams.h"
 #include "quant_core.h"
 #include "quant_fast.h"
+#include "job_table.h"
 #include "vec_geom.h"
 
 namespace ctmi {
@@ -325,6 +326,87 @@ nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* 
         Vec<typename OT::raw, 8> o;
 #pragma unroll
         for (int i = 0; i < 8; ++i) o.v[i] = OT::from_f32(t[i] * s);
+        stg_nt<typename OT::raw, 8>(out + (size_t)v * 8, o);
+      }
+    }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
+}
+
+// The two kernels above for up to kMaxJobs weights per launch (job_table.h), for
+// scales numbered like the items (rows of whole groups, which is every nvfp4 weight
+// the compressor sees).  A job's zero-point slot carries its global scale: the
+// format is symmetric and stores no zero points.
+template <typename XT>
+__global__ void __launch_bounds__(kFp4Block) nvfp4_compress_chain_kernel(ChainTable t) {
+  constexpr int B = kFp4Block, U = kFp4Unroll;
+  uint32_t local, nvec;
+  const ChainJob job = find_job(t, blockIdx.x, &local, &nvec);
+  const auto* x = static_cast<const typename XT::raw*>(job.src);
+  const auto* scale = static_cast<const uint8_t*>(job.scale);
+  auto* out = static_cast<uint32_t*>(job.dst);
+  const float gs = reinterpret_cast<const float*>(job.zp)[0];
+  const uint32_t v0 = local * (B * U) + threadIdx.x;
+  const bool full = (local + 1) * (uint32_t)(B * U) <= nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    Vec<typename XT::raw, 8> xv[U];
+    uint8_t sraw[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
+        sraw[k] = scale[v >> job.shift];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
+        __builtin_nontemporal_store(nvfp4_codes<XT, false>(xv[k], s, 0.0f), out + v);
+      }
+    }
+  };
+  if (full) body(std::false_type{});
+  else body(std::true_type{});
+}
+
+template <typename OT>
+__global__ void __launch_bounds__(kFp4Block) nvfp4_decompress_chain_kernel(ChainTable t) {
+  constexpr int B = kFp4Block, U = kFp4Unroll;
+  uint32_t local, nvec;
+  const ChainJob job = find_job(t, blockIdx.x, &local, &nvec);
+  const auto* packed = static_cast<const uint32_t*>(job.src);
+  const auto* scale = static_cast<const uint8_t*>(job.scale);
+  auto* out = static_cast<typename OT::raw*>(job.dst);
+  const float gs = reinterpret_cast<const float*>(job.zp)[0];
+  const uint32_t v0 = local * (B * U) + threadIdx.x;
+  const bool full = (local + 1) * (uint32_t)(B * U) <= nvec;
+  auto body = [&](auto guard) {
+    constexpr bool GUARD = decltype(guard)::value;
+    uint32_t pv[U];
+    uint8_t sraw[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        pv[k] = packed[v];
+        sraw[k] = scale[v >> job.shift];
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) {
+        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
+        float f[8];
+        fp4_unpack8_hw(pv[k], f);
+        Vec<typename OT::raw, 8> o;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) o.v[i] = OT::from_f32(f[i] * s);
         stg_nt<typename OT::raw, 8>(out + (size_t)v * 8, o);
       }
     }
@@ -695,6 +777,102 @@ extern "C" int ctmi_nvfp4_decompress(const uint8_t* packed, void* out, int32_t o
   a.q.ct = a.q.dt;
   hipLaunchKernelGGL(nvfp4_decompress_generic_kernel, grid_for(rows * cols, 256), 256, 0, st, a);
   return check_launch("ctmi_nvfp4_decompress");
+}
+
+// Can this weight go into a chained launch?  (the fast path of the single-call entry
+// points, with scales numbered like the items and no zero point)
+static bool fp4_chainable(const ctmi_weight_job& j, bool compress, VecGeom* g) {
+  const ctmi_qparams* qp = &j.qp;
+  const uintptr_t dense = (uintptr_t)(compress ? j.src : j.dst);
+  const uintptr_t packed = (uintptr_t)(compress ? j.dst : j.src);
+  return j.rows > 0 && j.cols > 0 && qp->scale_dtype == CTMI_F8E4M3 && qp->global_scale &&
+         qp->zero_point == nullptr && dense % (8 * dtype_size(j.dense_dtype)) == 0 &&
+         packed % 4 == 0 && vec_geometry(qp, j.rows, j.cols, g, true) && flat_geometry(*g);
+}
+
+static int fp4_many(const ctmi_weight_job* jobs, int64_t n, bool compress, void* stream,
+                    const char* what) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  hipStream_t st = (hipStream_t)stream;
+  constexpr uint32_t per = kFp4Block * kFp4Unroll;
+  // validate everything before anything is enqueued
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_weight_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 0 && j.cols >= 0, CTMI_ERR_VALUE, "job %lld: negative shape", (long long)i);
+    int rc = check_float3(j.dense_dtype, "dense side");
+    if (rc) return rc;
+    rc = check_qparams(&j.qp, j.rows, j.cols);
+    if (rc) return rc;
+    CTMI_REQUIRE(j.cols % 2 == 0, CTMI_ERR_VALUE,
+                 "tensor must have an even number of columns for nvfp4 compression");
+    CTMI_REQUIRE(!compress || (j.qp.qtype == CTMI_QTYPE_FLOAT && j.qp.num_bits == 4), CTMI_ERR_VALUE,
+                 "nvfp4 compression needs float 4-bit quantization args");
+    CTMI_REQUIRE((j.src && j.dst) || j.rows == 0 || j.cols == 0, CTMI_ERR_VALUE,
+                 "job %lld: NULL tensor pointer", (long long)i);
+  }
+  // chain per dense dtype, kMaxJobs weights per launch; the rest one call each
+  const int dts[3] = {CTMI_BF16, CTMI_F16, CTMI_F32};
+  for (int d = 0; d < 3; ++d) {
+    ChainTable t;
+    auto reset = [&]() {
+      t.n = 0;
+      for (int k = 0; k < kMaxJobs; ++k) { t.chunk_end[k] = 0xFFFFFFFFu; t.nvec[k] = 0; }
+    };
+    auto flush = [&]() {
+      if (t.n == 0) return;
+      const unsigned grid = t.chunk_end[t.n - 1];
+      if (compress) {
+        if (dts[d] == CTMI_BF16) hipLaunchKernelGGL(nvfp4_compress_chain_kernel<BF16>, grid, kFp4Block, 0, st, t);
+        else if (dts[d] == CTMI_F16) hipLaunchKernelGGL(nvfp4_compress_chain_kernel<F16>, grid, kFp4Block, 0, st, t);
+        else hipLaunchKernelGGL(nvfp4_compress_chain_kernel<F32>, grid, kFp4Block, 0, st, t);
+      } else {
+        if (dts[d] == CTMI_BF16) hipLaunchKernelGGL(nvfp4_decompress_chain_kernel<BF16>, grid, kFp4Block, 0, st, t);
+        else if (dts[d] == CTMI_F16) hipLaunchKernelGGL(nvfp4_decompress_chain_kernel<F16>, grid, kFp4Block, 0, st, t);
+        else hipLaunchKernelGGL(nvfp4_decompress_chain_kernel<F32>, grid, kFp4Block, 0, st, t);
+      }
+      reset();
+    };
+    reset();
+    for (int64_t i = 0; i < n; ++i) {
+      const ctmi_weight_job& j = jobs[i];
+      VecGeom g;
+      if (j.dense_dtype != dts[d] || !fp4_chainable(j, compress, &g)) continue;
+      const uint64_t chunks = cdiv(g.nvec, per);
+      const uint64_t before = t.n ? t.chunk_end[t.n - 1] : 0;
+      if (t.n == kMaxJobs || before + chunks >= 0x7FFFFFFFull) flush();
+      VecJob vj;
+      vj.src = j.src;
+      vj.dst = j.dst;
+      vj.scale = j.qp.scale;
+      vj.zp = reinterpret_cast<const int8_t*>(j.qp.global_scale);
+      vj.g = g;
+      t.job[t.n] = make_chain_job(vj);
+      t.nvec[t.n] = g.nvec;
+      t.chunk_end[t.n] = (uint32_t)((t.n ? t.chunk_end[t.n - 1] : 0) + chunks);
+      ++t.n;
+    }
+    flush();
+  }
+  int rc = check_launch(what);
+  if (rc) return rc;
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_weight_job& j = jobs[i];
+    VecGeom g;
+    if (j.rows == 0 || j.cols == 0 || fp4_chainable(j, compress, &g)) continue;
+    rc = compress ? ctmi_nvfp4_compress(j.src, j.dense_dtype, (uint8_t*)j.dst, j.rows, j.cols, &j.qp, stream)
+                  : ctmi_nvfp4_decompress((const uint8_t*)j.src, j.dst, j.dense_dtype, j.rows, j.cols,
+                                          &j.qp, stream);
+    if (rc) return rc;
+  }
+  return CTMI_OK;
+}
+
+extern "C" int ctmi_nvfp4_compress_many(const ctmi_weight_job* jobs, int64_t n, void* stream) {
+  return fp4_many(jobs, n, true, stream, "ctmi_nvfp4_compress_many");
+}
+
+extern "C" int ctmi_nvfp4_decompress_many(const ctmi_weight_job* jobs, int64_t n, void* stream) {
+  return fp4_many(jobs, n, false, stream, "ctmi_nvfp4_decompress_many");
 }
 
 extern "C" int ctmi_observe_nvfp4_compress(const void* x, int32_t x_dtype, int64_t rows,

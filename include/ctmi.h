@@ -174,6 +174,15 @@ int ctmi_nvfp4_compress(const void* x, int32_t x_dtype, uint8_t* out, int64_t ro
 int ctmi_nvfp4_decompress(const uint8_t* packed, void* out, int32_t out_dtype, int64_t rows,
                           int64_t cols, const ctmi_qparams* qp, void* stream);
 
+/* A27 for the nvfp4 format: the per-weight loop of BaseQuantizationCompressor.compress /
+ * decompress_from_state_dict (compressors/quantized_compressors/base.py:91-125, 213-230)
+ * in one call.  src/dst as in ctmi_weight_job (dense weight -> packed bytes, or back);
+ * qp carries the fp8 group scales and the weight's global scale.  Every job is
+ * validated before anything is enqueued; weights of one dense dtype are chained
+ * into common launches, 8 per launch. */
+int ctmi_nvfp4_compress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
+int ctmi_nvfp4_decompress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
+
 /* A19.  pack_bitmasks / unpack_bitmasks (utils/helpers.py:302-339):
  * numpy.packbits(axis=-1, bitorder="little").  mask: bool/uint8 [rows, cols];
  * packed: uint8 [rows, ceil(cols/8)]. */

@@ -585,3 +585,58 @@ def test_random_shapes_sweep(gpu):
             data["weight_zero_point"] = zp
         dense = comp.decompress_weight({k: v.to(gpu) for k, v in data.items()}, quantization_args=args)
         assert_bit_equal(dense, op.pack_quantized_decompress(dict(data), oargs), f"decompress {case}")
+
+
+def test_nvfp4_weight_batch_and_state_dict(gpu):
+    """Fp4WeightBatch (ctmi_nvfp4_{compress,decompress}_many: 8 weights per launch, more
+    than 8 weights, mixed dtypes, a weight whose rows are not whole 16-byte items and so
+    falls back to a call of its own) against the per-weight compressor and the oracle; the
+    compressor's state-dict compress emits the per-weight loop's keys and values"""
+    from compressed_tensors_amd.compressors import BaseCompressor, Fp4WeightBatch
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationScheme, generate_gparam, observe_weight_qparams,
+    )
+
+    announce("nvfp4 batch")
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    comp = BaseCompressor.load_from_registry("nvfp4-pack-quantized")
+    shapes = [(64, 256, torch.bfloat16), (8, 4096, torch.bfloat16), (33, 48, torch.float16), (128, 512, torch.bfloat16),
+              (5, 16, torch.float32), (256, 1024, torch.bfloat16), (16, 32, torch.bfloat16), (40, 80, torch.float16),
+              (300, 64, torch.bfloat16), (64, 4112, torch.bfloat16), (7, 16, torch.bfloat16), (96, 160, torch.bfloat16)]
+    entries, state, schemes = [], {}, {}
+    for i, (r, c, dt) in enumerate(shapes):
+        w = (torch.randn((r, c), generator=torch.Generator().manual_seed(40 + i)) * 0.02).to(dt)
+        w.view(-1)[:3] = torch.tensor([0.0, -0.0, -1e-6]).to(dt)
+        mn, mx = torch.aminmax(w)
+        gs = generate_gparam(mn.reshape(1).to(gpu), mx.reshape(1).to(gpu))
+        scale, zp = observe_weight_qparams(w.to(gpu), args, global_scale=gs)
+        entries.append(dict(weight=w.to(gpu), scale=scale, global_scale=gs, quantization_args=args))
+        state[f"m{i}.weight"] = w.to(gpu)
+        state[f"m{i}.weight_scale"] = scale
+        state[f"m{i}.weight_global_scale"] = gs
+        state[f"m{i}.weight_zero_point"] = zp
+        schemes[f"m{i}"] = QuantizationScheme(targets=["Linear"], weights=args)
+    state["m0.bias"] = torch.ones(64, device=gpu)
+    batch = Fp4WeightBatch(entries)
+    packed = batch.compress()
+    dense = batch.decompress()
+    for i, e in enumerate(entries):
+        single = comp.compress_weight(weight=e["weight"], scale=e["scale"], global_scale=e["global_scale"],
+                                      quantization_args=args)["weight_packed"]
+        assert_bit_equal(packed[i], single, f"packed {i} vs single call")
+        w, s, g = e["weight"].cpu(), e["scale"].cpu(), e["global_scale"].cpu()
+        want = op.nvfp4_compress(w, s, g, oargs)
+        assert_bit_equal(packed[i], want, f"packed {i} vs oracle")
+        back = comp.decompress_weight({"weight_packed": single, "weight_scale": e["scale"],
+                                       "weight_global_scale": e["global_scale"]})
+        assert_bit_equal(dense[i], back, f"dense {i} vs single call")
+    out = comp.compress(state, names_to_scheme=schemes)
+    assert set(out) == ({f"m{i}.weight_packed" for i in range(len(shapes))}
+                        | {f"m{i}.weight_scale" for i in range(len(shapes))}
+                        | {f"m{i}.weight_global_scale" for i in range(len(shapes))} | {"m0.bias"})
+    for i in range(len(shapes)):
+        assert_bit_equal(out[f"m{i}.weight_packed"], packed[i], f"state dict {i}")
+    restored = dict(comp.decompress_from_state_dict(out, names_to_scheme=schemes))
+    for i in range(len(shapes)):
+        assert_bit_equal(restored[f"m{i}"]["weight"], dense[i], f"state dict decompress {i}")
