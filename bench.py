@@ -392,6 +392,17 @@ def other_workload(torch, name, seed):
                 nb = sum(4 * x.numel() for x in xs)
                 ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb,
                               "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel"))
+                if label.startswith("weights 4096x4096"):
+                    jobs = (_lib.HadamardJob * len(xs))()
+                    outs = [torch.empty_like(x) for x in xs]
+                    for job, x, out in zip(jobs, xs, outs):
+                        job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()
+                    keep.extend([jobs, outs])
+                    m = (jobs, len(xs), code(xs[0].dtype), a_dim, b_dim, _lib.ptr(ma), mb.data_ptr(),
+                         q.data_ptr(), None, st)
+                    ops.append(Op(f"random-sign Hadamard, size {n}: {label}, one call (8 per launch)",
+                                  [lambda m=m: _lib.check(lib.ctmi_hadamard_apply_many(*m))], nb,
+                                  "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel"))
         # rotation (block 128) + symmetric int4 group-128 quantization + pack_to_int32, one pass
         mb = deterministic_hadamard_matrix(128, torch.bfloat16, dev).contiguous()
         q = (torch.randint(0, 2, (128,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
@@ -408,6 +419,20 @@ def other_workload(torch, name, seed):
             nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in tensors[label])
             ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}", calls, nb,
                           "hadamard_quant_pack_kernel"))
+            if label.startswith("weights 4096x4096"):
+                xs = tensors[label]
+                jobs = (_lib.HadamardPackJob * len(xs))()
+                for job, x in zip(jobs, xs):
+                    packed = torch.empty(x.shape[0], x.shape[1] // 8, dtype=torch.int32, device=dev)
+                    scale = torch.empty(x.shape[0], x.shape[1] // 128, dtype=torch.bfloat16, device=dev)
+                    keep.extend([packed, scale])
+                    job.x, job.packed, job.scale, job.rotated, job.numel = (
+                        x.data_ptr(), packed.data_ptr(), scale.data_ptr(), None, x.numel())
+                keep.append(jobs)
+                m = (jobs, len(xs), code(xs[0].dtype), 128, mb.data_ptr(), q.data_ptr(), None, 4, 1, st)
+                ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
+                              [lambda m=m: _lib.check(lib.ctmi_hadamard_quant_pack_many(*m))], nb,
+                              "hadamard_quant_pack_kernel"))
         return "Hadamard rotation GB/s (bf16 MFMA), block 128 and full 4096, and fused with int4 packing", ops, keep
 
     raise SystemExit(f"unknown workload {name}")

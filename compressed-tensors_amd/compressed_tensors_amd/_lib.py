@@ -85,6 +85,19 @@ class WeightJob(ctypes.Structure):
     ]
 
 
+class HadamardJob(ctypes.Structure):
+    """mirror of `struct ctmi_hadamard_job`"""
+
+    _fields_ = [("x", c_void_p), ("out", c_void_p), ("numel", c_int64)]
+
+
+class HadamardPackJob(ctypes.Structure):
+    """mirror of `struct ctmi_hadamard_pack_job`"""
+
+    _fields_ = [("x", c_void_p), ("packed", c_void_p), ("scale", c_void_p), ("rotated", c_void_p),
+                ("numel", c_int64)]
+
+
 class ObservePackJob(ctypes.Structure):
     """ctmi_observe_pack_job"""
     _fields_ = [
@@ -184,6 +197,16 @@ SIGNATURES = {
     "ctmi_topk24_lut": (None, [c_void_p]),
     "ctmi_calib_copy": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "ctmi_hadamard_supported": (c_int32, [c_int32, c_int32, c_int32]),
+    "ctmi_hadamard_apply_many": (
+        c_int32,
+        [POINTER(HadamardJob), c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_void_p],
+    ),
+    "ctmi_hadamard_quant_pack_many": (
+        c_int32,
+        [POINTER(HadamardPackJob), c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
+         c_int32, c_void_p],
+    ),
     "ctmi_hadamard_apply": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p,

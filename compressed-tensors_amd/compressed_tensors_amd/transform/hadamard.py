@@ -38,6 +38,8 @@ __all__ = [
     "hadamard_factors",
     "hadamard_apply",
     "hadamard_quantize_pack",
+    "hadamard_apply_many",
+    "hadamard_quantize_pack_many",
     "apply_transform_weight",
     "TransformLocation",
     "TransformArgs",
@@ -203,6 +205,101 @@ def hadamard_quantize_pack(
     if return_rotated:
         out["rotated"] = rotated
     return out
+
+
+def hadamard_apply_many(
+    values: List[Tensor],
+    n: int,
+    sign_in: Optional[Tensor] = None,
+    sign_out: Optional[Tensor] = None,
+    matrix_t: Optional[Tensor] = None,
+) -> List[Tensor]:
+    """hadamard_apply on several tensors of one dtype that share the matrix and the
+    signs (the weights of a model under one transform scheme), from one call: the
+    kernels take 8 tensors per launch."""
+    if not values:
+        return []
+    xs = [to_gpu(v).contiguous() for v in values]
+    dtype, dev = xs[0].dtype, xs[0].device
+    if dtype not in _FLOATS:
+        raise NotImplementedError(f"transforms of dtype {dtype} are not supported")
+    for x in xs:
+        if x.dtype != dtype or x.device != dev:
+            raise ValueError("tensors of one call share dtype and device")
+        if x.shape[-1] % n != 0:
+            raise ValueError(f"{n} must divide the last dimension {x.shape[-1]}")
+    fac = hadamard_factors(n)
+    lib = _lib.load()
+    code = _lib.dtype_code(dtype)
+    if fac is None or not lib.ctmi_hadamard_supported(fac[0], fac[1], code):
+        raise NotImplementedError(f"no MFMA Hadamard kernel for size {n} and dtype {dtype}")
+    a, b = fac
+    if matrix_t is not None:
+        if a != 1:
+            raise NotImplementedError("explicit matrices are supported for sizes 32, 64 and 128")
+        mb_t, ma_t = matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous(), None
+    else:
+        mb_t = _sylvester_bf16(b, dev)
+        ma_t = _sylvester_bf16(a, dev) if a > 1 else None
+    s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
+    s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
+    outs = [torch.empty_like(x) for x in xs]
+    jobs = (_lib.HadamardJob * len(xs))()
+    for job, x, out in zip(jobs, xs, outs):
+        job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()
+    _lib.check(
+        lib.ctmi_hadamard_apply_many(jobs, len(xs), code, a, b, _lib.ptr(ma_t), mb_t.data_ptr(),
+                                     _lib.ptr(s_in), _lib.ptr(s_out), _lib.stream_of(dev))
+    )
+    return outs
+
+
+def hadamard_quantize_pack_many(
+    values: List[Tensor],
+    n: int,
+    quantization_args,
+    sign_in: Optional[Tensor] = None,
+    sign_out: Optional[Tensor] = None,
+    matrix_t: Optional[Tensor] = None,
+) -> List[Dict[str, Tensor]]:
+    """hadamard_quantize_pack on several bf16 [rows, cols] tensors from one call (8 per
+    launch); one dict per tensor, as hadamard_quantize_pack returns it"""
+    if not values:
+        return []
+    xs = [to_gpu(v).contiguous() for v in values]
+    args = quantization_args
+    if not (args.num_bits == 4 and str(getattr(args.type, "value", args.type)) == "int" and args.symmetric
+            and str(getattr(args.strategy, "value", args.strategy)) == "group" and args.group_size == n):
+        raise NotImplementedError(
+            "the fused path covers symmetric int4 group quantization with group_size == block size")
+    if n not in (32, 64, 128):
+        raise NotImplementedError("block size must be 32, 64 or 128")
+    dev = xs[0].device
+    for x in xs:
+        if x.ndim != 2 or x.dtype != torch.bfloat16 or x.device != dev:
+            raise NotImplementedError("the fused path takes 2-D bfloat16 tensors on one device")
+        if x.shape[1] % n != 0:
+            raise ValueError(f"{n} must divide the last dimension {x.shape[1]}")
+    mb_t = (_sylvester_bf16(n, dev) if matrix_t is None
+            else matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous())
+    s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
+    s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
+    jobs = (_lib.HadamardPackJob * len(xs))()
+    results = []
+    for job, x in zip(jobs, xs):
+        rows, cols = x.shape
+        packed = torch.empty((rows, cols // 8), dtype=torch.int32, device=dev)
+        scale = torch.empty((rows, cols // n), dtype=torch.bfloat16, device=dev)
+        job.x, job.packed, job.scale, job.rotated, job.numel = (
+            x.data_ptr(), packed.data_ptr(), scale.data_ptr(), None, x.numel())
+        results.append({"weight_packed": packed, "weight_scale": scale,
+                        "weight_shape": torch.tensor(x.shape)})
+    _lib.check(
+        _lib.load().ctmi_hadamard_quant_pack_many(
+            jobs, len(xs), _lib.dtype_code(torch.bfloat16), n, mb_t.data_ptr(), _lib.ptr(s_in),
+            _lib.ptr(s_out), 4, 1, _lib.stream_of(dev))
+    )
+    return results
 
 
 # ------------------------------------------------------------------ vocabulary

@@ -55,6 +55,39 @@ constexpr int kHqpWaves = kHqpThreads / kWave;
 #define CTMI_HAD_KRON_WAVES 2  // waves per SIMD the kernel for 64 x 64 is built for (measured best)
 #endif
 
+// Up to kHadMaxJobs tensors for one launch of a kernel whose workgroups stay for the
+// whole launch (the matrix set-up is then paid once for all of them).  A unit is
+// what a wavefront takes at a time: 16 sub-rows, or a data row.
+constexpr int kHadMaxJobs = 8;
+struct HadJobs {
+  const void* x[kHadMaxJobs];
+  void* out[kHadMaxJobs];
+  void* scale[kHadMaxJobs];    // fused rotation + quantization only
+  void* rotated[kHadMaxJobs];  // fused rotation + quantization only
+  int64_t end[kHadMaxJobs];    // running total of units, job 0 .. j (unused: INT64_MAX)
+  int64_t n_sub[kHadMaxJobs];  // sub-rows of job j
+};
+
+// the job of a unit and the unit's number within that job (all wave-uniform); launches
+// of a single tensor skip the search and the indexed loads behind it
+template <bool MANY>
+__device__ __forceinline__ int had_job(const HadJobs& t, int64_t unit, int64_t* local) {
+  if constexpr (!MANY) {
+    *local = unit;
+    return 0;
+  }
+  int j = 0;
+  int64_t first = 0;
+#pragma unroll
+  for (int i = 0; i < kHadMaxJobs - 1; ++i) {
+    const bool past = unit >= t.end[i];
+    j = past ? i + 1 : j;
+    first = past ? t.end[i] : first;
+  }
+  *local = unit - first;
+  return j;
+}
+
 struct HadArgs {
   const void* x;
   void* out;
@@ -266,11 +299,11 @@ __global__ void __launch_bounds__(kHadThreads) hadamard_mfma_kernel(HadArgs a) {
 //                    + {4..7}, so a lane ends up with 8 neighbouring outputs,
 //                    one 16-byte global store.
 // Sign vectors are used as signs: their entries must be +1 or -1.
-template <int B, bool HALF>
+template <int B, bool HALF, bool MANY>
 __global__ void __launch_bounds__(kRowsThreads)
-hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
+hadamard_rows_kernel(HadJobs jobs, int64_t n_full, int ragged_sub,
                      const uint16_t* __restrict__ mbt, const float* __restrict__ s_in,
-                     const float* __restrict__ s_out, int64_t n_sub, float inv_sqrt_n) {
+                     const float* __restrict__ s_out, float inv_sqrt_n) {
   constexpr int KS = B / 32;  // k steps
   constexpr int NP = B / 32;  // pairs of 16-column output tiles
   const int lane = threadIdx.x & 63;
@@ -332,17 +365,22 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
     }
   }
 
-  const int64_t n_full = n_sub / 16;  // whole groups of 16 sub-rows
+  // n_full: whole groups of 16 sub-rows, over all jobs
   const int64_t stride = (int64_t)gridDim.x * kRowsWaves;
   const int64_t first = (int64_t)blockIdx.x * kRowsWaves + wave;
 
   // Loads are never conditional (a group past the end re-reads the last whole
   // one) and the stores of whole groups are not either: with a fixed number of
   // memory operations per step the waits can say exactly how many newer
-  // operations may still be in flight.
-  auto load_group = [&](int64_t grp, frag_t* xf) {
+  // operations may still be in flight.  Where the group's outputs go is looked up
+  // together with where its inputs are.
+  auto load_group = [&](int64_t grp, frag_t* xf, uint16_t** dst) {
     if (grp >= n_full) grp = n_full - 1;
-    const uint16_t* src = x + (grp * 16 + l16) * B + 8 * lq;
+    int64_t local;
+    const int j = had_job<MANY>(jobs, grp, &local);
+    const int64_t at = (local * 16 + l16) * B + 8 * lq;
+    const uint16_t* src = static_cast<const uint16_t*>(jobs.x[j]) + at;
+    *dst = static_cast<uint16_t*>(jobs.out[j]) + at;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
       xf[ks] = __builtin_bit_cast(frag_t, ldg<uint16_t, 8>(src + 32 * ks));
@@ -373,10 +411,6 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
       if (keep) stg<uint16_t, 8>(dst + 32 * p, __builtin_bit_cast(Vec<uint16_t, 8>, o));
     }
   };
-  auto transform_group = [&](int64_t grp, const frag_t* xf) {
-    transform_rows(xf, out + (grp * 16 + l16) * B + 8 * lq, true);
-  };
-
   if (first < n_full) {
     // Software pipeline one group ahead, two register sets taking turns (no
     // copies).  The first group is handled ahead of the loop so that the loop is
@@ -384,23 +418,28 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
     // loads, then a group's stores): a wait for loads then never has to cover
     // the stores issued after them, which would cost a store latency per group.
     frag_t xa[KS], xb[KS];
+    uint16_t *da, *db;
     int64_t g = first;
-    load_group(g, xa);
-    load_group(g + stride, xb);
-    transform_group(g, xa);
+    load_group(g, xa, &da);
+    load_group(g + stride, xb, &db);
+    transform_rows(xa, da, true);
     g += stride;
     while (g < n_full) {  // invariant: group g is in xb
-      load_group(g + stride, xa);
-      transform_group(g, xb);
+      load_group(g + stride, xa, &da);
+      transform_rows(xb, db, true);
       g += stride;
       if (g >= n_full) break;
-      load_group(g + stride, xb);
-      transform_group(g, xa);
+      load_group(g + stride, xb, &db);
+      transform_rows(xa, da, true);
       g += stride;
     }
   }
-  // the ragged last group (fewer than 16 sub-rows), by the wave whose turn it is
-  if (n_sub % 16 != 0 && n_full % stride == first) {
+  // the ragged last group (fewer than 16 sub-rows; single tensors only), by the wave
+  // whose turn it is
+  if (ragged_sub != 0 && n_full % stride == first) {
+    const int64_t n_sub = n_full * 16 + ragged_sub;
+    const uint16_t* x = static_cast<const uint16_t*>(jobs.x[0]);
+    uint16_t* out = static_cast<uint16_t*>(jobs.out[0]);
     int64_t row = n_full * 16 + l16;
     const bool keep = row < n_sub;
     if (!keep) row = n_sub - 1;
@@ -412,17 +451,33 @@ hadamard_rows_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   }
 }
 
+static void clear_jobs(HadJobs* t) {
+  for (int k = 0; k < kHadMaxJobs; ++k) {
+    t->x[k] = nullptr;
+    t->out[k] = t->scale[k] = t->rotated[k] = nullptr;
+    t->end[k] = INT64_MAX;
+    t->n_sub[k] = 0;
+  }
+}
+
+// jobs: whole groups of 16 sub-rows per tensor, except that a single tensor may end
+// in a ragged group
 template <int B, bool HALF>
-static int launch_had_rows(const HadArgs& a, hipStream_t st) {
-  const int64_t groups = cdiv(a.n_sub, 16);
-  const int64_t wgs = cdiv(groups, kRowsWaves);
+static int launch_had_rows_jobs(const HadJobs& jobs, int n_jobs, const HadArgs& a, hipStream_t st) {
+  const int64_t n_full = n_jobs == 1 ? jobs.n_sub[0] / 16 : jobs.end[n_jobs - 1];
+  const int ragged = n_jobs == 1 ? (int)(jobs.n_sub[0] % 16) : 0;
+  const int64_t wgs = cdiv(n_full + (ragged ? 1 : 0), kRowsWaves);
   // a wave keeps the matrix in registers: give it several groups to use it on
   // (as many wavefronts as fit on the chip at once: 8 per CU at 128, where a wave
   // needs some 190 registers, more below)
   const int64_t cap = 256 * (B == 32 ? 16 : 8) / kRowsWaves;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
-  hipLaunchKernelGGL((hadamard_rows_kernel<B, HALF>), grid, kRowsThreads, 0, st, (const uint16_t*)a.x,
-                     (uint16_t*)a.out, a.mbt, a.s_in, a.s_out, a.n_sub, 1.0f / a.sqrt_n);
+  if (n_jobs == 1)
+    hipLaunchKernelGGL((hadamard_rows_kernel<B, HALF, false>), grid, kRowsThreads, 0, st, jobs, n_full,
+                       ragged, a.mbt, a.s_in, a.s_out, 1.0f / a.sqrt_n);
+  else
+    hipLaunchKernelGGL((hadamard_rows_kernel<B, HALF, true>), grid, kRowsThreads, 0, st, jobs, n_full,
+                       ragged, a.mbt, a.s_in, a.s_out, 1.0f / a.sqrt_n);
   return CTMI_OK;
 }
 
@@ -435,13 +490,11 @@ static int launch_had_rows(const HadArgs& a, hipStream_t st) {
 // those of the three separate steps; the rotated tensor never goes to memory
 // (unless `rotated` asks for it).  A sub-row's 128 outputs sit in the 4 lanes
 // l16 + 16 q; they agree on min / max through two lane exchanges.
-template <int B>
+template <int B, bool MANY>
 __global__ void __launch_bounds__(kHqpThreads)
-hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __restrict__ mbt,
+hadamard_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const uint16_t* __restrict__ mbt,
                            const float* __restrict__ s_in, const float* __restrict__ s_out,
-                           int32_t* __restrict__ packed, uint16_t* __restrict__ scale,
-                           uint16_t* __restrict__ rotated, int64_t n_sub, float inv_sqrt_n,
-                           QpCfg cfg) {
+                           float inv_sqrt_n, QpCfg cfg) {
   constexpr int KS = B / 32, NP = B / 32;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -470,10 +523,17 @@ hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __res
   }
   __syncthreads();
 
-  const int64_t n_groups = (n_sub + 15) / 16;
+  // n_groups: groups of 16 sub-rows over all jobs (a job's last one may be ragged)
   const int64_t stride = (int64_t)gridDim.x * kHqpWaves;
   for (int64_t g = (int64_t)blockIdx.x * kHqpWaves + wave; g < n_groups; g += stride) {
-    int64_t row = g * 16 + l16;
+    int64_t local;
+    const int j = had_job<MANY>(jobs, g, &local);
+    const int64_t n_sub = jobs.n_sub[j];
+    const uint16_t* x = static_cast<const uint16_t*>(jobs.x[j]);
+    int32_t* packed = static_cast<int32_t*>(jobs.out[j]);
+    uint16_t* scale = static_cast<uint16_t*>(jobs.scale[j]);
+    uint16_t* rotated = static_cast<uint16_t*>(jobs.rotated[j]);
+    int64_t row = local * 16 + l16;
     const bool keep = row < n_sub;
     if (!keep) row = n_sub - 1;  // ragged last group: recompute the last sub-row, store nothing
     const uint16_t* src = x + row * B + 8 * lq;
@@ -568,12 +628,11 @@ hadamard_quant_pack_kernel(const uint16_t* __restrict__ x, const uint16_t* __res
 // Signs (entries +1 / -1) are XOR masks on the bf16 sign bits of X and of the
 // output; they are per position within the row, the same for every row, and sit
 // in LDS in the lanes' own layout.
-template <int A, int B, bool HALF>
+template <int A, int B, bool HALF, bool MANY>
 __global__ void __launch_bounds__(kKronThreads) __attribute__((amdgpu_waves_per_eu(CTMI_HAD_KRON_WAVES)))
-hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
-                     const uint16_t* __restrict__ mbt, const uint16_t* __restrict__ mat,
-                     const float* __restrict__ s_in, const float* __restrict__ s_out,
-                     int64_t n_rows, float inv_sqrt_n) {
+hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ mbt,
+                     const uint16_t* __restrict__ mat, const float* __restrict__ s_in,
+                     const float* __restrict__ s_out, float inv_sqrt_n) {
   constexpr int N = A * B;
   constexpr int KS = B / 32;   // k steps of stage 1
   constexpr int MT = A / 16;   // sub-row tiles
@@ -643,8 +702,10 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
 
   const int64_t stride = (int64_t)gridDim.x * kKronWaves;
   for (int64_t row = (int64_t)blockIdx.x * kKronWaves + wave; row < n_rows; row += stride) {
-    const uint16_t* src = x + row * N;
-    uint16_t* dst = out + row * N;
+    int64_t local;
+    const int j = had_job<MANY>(jobs, row, &local);  // n_rows: data rows over all jobs
+    const uint16_t* src = static_cast<const uint16_t*>(jobs.x[j]) + local * N;
+    uint16_t* dst = static_cast<uint16_t*>(jobs.out[j]) + local * N;
     xfrag_t xf[MT][KS];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
@@ -730,15 +791,20 @@ hadamard_kron_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ out,
   }
 }
 
+// jobs: units are data rows of A * B elements
 template <int A, int B, bool HALF>
-static int launch_had_kron(const HadArgs& a, hipStream_t st) {
-  const int64_t n_rows = a.n_sub / A;
+static int launch_had_kron_jobs(const HadJobs& jobs, int n_jobs, const HadArgs& a, hipStream_t st) {
+  const int64_t n_rows = jobs.end[n_jobs - 1];
   const int64_t wgs = cdiv(n_rows, kKronWaves);
   // as many workgroups as are resident at once (register-limited)
   const int64_t cap = 256 * 4 * (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES)) / kKronWaves;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
-  hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF>), grid, kKronThreads, 0, st, (const uint16_t*)a.x,
-                     (uint16_t*)a.out, a.mbt, a.mat, a.s_in, a.s_out, n_rows, 1.0f / a.sqrt_n);
+  if (n_jobs == 1)
+    hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF, false>), grid, kKronThreads, 0, st, jobs, n_rows,
+                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n);
+  else
+    hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF, true>), grid, kKronThreads, 0, st, jobs, n_rows,
+                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n);
   return CTMI_OK;
 }
 
@@ -794,6 +860,27 @@ static int dispatch_had(int a_dim, int b_dim, const HadArgs& a, hipStream_t st) 
                    b_dim);
 }
 
+// the kernels that keep their operands in registers (and take several tensors per launch)
+static bool had_in_registers(int io_dtype, int a_dim, int b_dim) {
+  if (io_dtype != CTMI_BF16 && io_dtype != CTMI_F16) return false;
+  if (a_dim == 1) return b_dim == 32 || b_dim == 64 || b_dim == 128;
+  return (a_dim == 32 && (b_dim == 32 || b_dim == 64)) || (a_dim == 64 && b_dim == 64);
+}
+
+static int launch_had_jobs(const HadJobs& jobs, int n_jobs, int io_dtype, int a_dim, int b_dim,
+                           const HadArgs& a, hipStream_t st) {
+  const bool half = io_dtype == CTMI_F16;
+#define CTMI_ROWS(BB) (half ? launch_had_rows_jobs<BB, true>(jobs, n_jobs, a, st) \
+                            : launch_had_rows_jobs<BB, false>(jobs, n_jobs, a, st))
+#define CTMI_KRON(AA, BB) (half ? launch_had_kron_jobs<AA, BB, true>(jobs, n_jobs, a, st) \
+                                : launch_had_kron_jobs<AA, BB, false>(jobs, n_jobs, a, st))
+  if (a_dim == 1) return b_dim == 32 ? CTMI_ROWS(32) : (b_dim == 64 ? CTMI_ROWS(64) : CTMI_ROWS(128));
+  if (a_dim == 32) return b_dim == 32 ? CTMI_KRON(32, 32) : CTMI_KRON(32, 64);
+  return CTMI_KRON(64, 64);
+#undef CTMI_ROWS
+#undef CTMI_KRON
+}
+
 }  // namespace ctmi
 
 using namespace ctmi;
@@ -839,31 +926,88 @@ extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, i
   a.sqrt_n = sqrtf((float)n);
   hipStream_t st = (hipStream_t)stream;
   int rc;
-  if (io_dtype == CTMI_BF16 && a_dim == 1) {
-    rc = b_dim == 32 ? launch_had_rows<32, false>(a, st)
-                     : (b_dim == 64 ? launch_had_rows<64, false>(a, st)
-                                    : launch_had_rows<128, false>(a, st));
-  } else if (io_dtype == CTMI_F16 && a_dim == 1) {
-    rc = b_dim == 32 ? launch_had_rows<32, true>(a, st)
-                     : (b_dim == 64 ? launch_had_rows<64, true>(a, st)
-                                    : launch_had_rows<128, true>(a, st));
-  } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 32) {
-    rc = launch_had_kron<32, 32, false>(a, st);
-  } else if (io_dtype == CTMI_BF16 && a_dim == 32 && b_dim == 64) {
-    rc = launch_had_kron<32, 64, false>(a, st);
-  } else if (io_dtype == CTMI_BF16 && a_dim == 64 && b_dim == 64) {
-    rc = launch_had_kron<64, 64, false>(a, st);
-  } else if (io_dtype == CTMI_F16 && a_dim == 32 && b_dim == 32) {
-    rc = launch_had_kron<32, 32, true>(a, st);
-  } else if (io_dtype == CTMI_F16 && a_dim == 32 && b_dim == 64) {
-    rc = launch_had_kron<32, 64, true>(a, st);
-  } else if (io_dtype == CTMI_F16 && a_dim == 64 && b_dim == 64) {
-    rc = launch_had_kron<64, 64, true>(a, st);
+  if (had_in_registers(io_dtype, a_dim, b_dim)) {
+    HadJobs jobs;
+    clear_jobs(&jobs);
+    jobs.x[0] = x;
+    jobs.out[0] = out;
+    jobs.n_sub[0] = a.n_sub;
+    jobs.end[0] = a_dim == 1 ? a.n_sub / 16 : a.n_sub / a_dim;
+    rc = launch_had_jobs(jobs, 1, io_dtype, a_dim, b_dim, a, st);
   } else if (io_dtype == CTMI_BF16) rc = dispatch_had<BF16>(a_dim, b_dim, a, st);
   else if (io_dtype == CTMI_F16) rc = dispatch_had<F16>(a_dim, b_dim, a, st);
   else rc = dispatch_had<F32>(a_dim, b_dim, a, st);
   if (rc) return rc;
   return check_launch("ctmi_hadamard_apply");
+}
+
+extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n_jobs,
+                                        int32_t io_dtype, int32_t a_dim, int32_t b_dim,
+                                        const void* ma_t, const void* mb_t, const float* sign_in,
+                                        const float* sign_out, void* stream) {
+  CTMI_REQUIRE(n_jobs >= 0 && (jobs || n_jobs == 0), CTMI_ERR_VALUE, "bad job list");
+  CTMI_REQUIRE(a_dim >= 1 && b_dim >= 1, CTMI_ERR_VALUE, "bad factor sizes");
+  CTMI_REQUIRE(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32,
+               CTMI_ERR_UNSUPPORTED, "transforms take float16/bfloat16/float32 tensors");
+  CTMI_REQUIRE(ctmi_hadamard_supported(a_dim, b_dim, io_dtype), CTMI_ERR_UNSUPPORTED,
+               "no MFMA kernel for the factorisation %d x %d with this dtype", a_dim, b_dim);
+  const int64_t n = (int64_t)a_dim * b_dim;
+  // validate everything before anything is enqueued
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_hadamard_job& j = jobs[i];
+    CTMI_REQUIRE(j.numel >= 0 && j.numel % n == 0, CTMI_ERR_VALUE,
+                 "job %lld: tensor size %lld is not a multiple of the transform size %lld",
+                 (long long)i, (long long)j.numel, (long long)n);
+    CTMI_REQUIRE(j.numel == 0 || (j.x && j.out), CTMI_ERR_VALUE, "job %lld: NULL tensor pointer",
+                 (long long)i);
+    CTMI_REQUIRE((uintptr_t)j.x % 16 == 0 && (uintptr_t)j.out % 16 == 0, CTMI_ERR_VALUE,
+                 "tensors must be 16-byte aligned");
+  }
+  CTMI_REQUIRE(n_jobs == 0 || (mb_t && (a_dim == 1 || ma_t)), CTMI_ERR_VALUE, "NULL matrix pointer");
+  CTMI_REQUIRE((uintptr_t)mb_t % 16 == 0 && (uintptr_t)ma_t % 16 == 0, CTMI_ERR_VALUE,
+               "tensors must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  HadArgs a;
+  a.x = nullptr;
+  a.out = nullptr;
+  a.mbt = (const uint16_t*)mb_t;
+  a.mat = (const uint16_t*)ma_t;
+  a.s_in = sign_in;
+  a.s_out = sign_out;
+  a.n_sub = 0;
+  a.sqrt_n = sqrtf((float)n);
+  // tensors made of whole units share launches, kHadMaxJobs at a time; the others
+  // (a ragged last group, dtypes on the LDS-staged kernel) get a call of their own
+  const int64_t unit = a_dim == 1 ? 16 * (int64_t)b_dim : n;
+  const bool shared = had_in_registers(io_dtype, a_dim, b_dim);
+  HadJobs t;
+  clear_jobs(&t);
+  int filled = 0;
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_hadamard_job& j = jobs[i];
+    if (j.numel == 0) continue;
+    if (!shared || j.numel % unit != 0) {
+      int rc = ctmi_hadamard_apply(j.x, j.out, io_dtype, j.numel, a_dim, b_dim, ma_t, mb_t, sign_in,
+                                   sign_out, stream);
+      if (rc) return rc;
+      continue;
+    }
+    t.x[filled] = j.x;
+    t.out[filled] = j.out;
+    t.n_sub[filled] = j.numel / b_dim;
+    t.end[filled] = (filled ? t.end[filled - 1] : 0) + j.numel / unit;
+    if (++filled == kHadMaxJobs) {
+      int rc = launch_had_jobs(t, filled, io_dtype, a_dim, b_dim, a, st);
+      if (rc) return rc;
+      clear_jobs(&t);
+      filled = 0;
+    }
+  }
+  if (filled) {
+    int rc = launch_had_jobs(t, filled, io_dtype, a_dim, b_dim, a, st);
+    if (rc) return rc;
+  }
+  return check_launch("ctmi_hadamard_apply_many");
 }
 
 extern "C" int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel,
@@ -893,24 +1037,31 @@ extern "C" int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int
   return check_launch("ctmi_block_matmul");
 }
 
-extern "C" int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t numel, int32_t b_dim,
-                                        const void* mb_t, const float* sign_in,
-                                        const float* sign_out, int32_t num_bits, int32_t symmetric,
-                                        int32_t* packed, void* scale, void* rotated, void* stream) {
-  CTMI_REQUIRE(numel >= 0, CTMI_ERR_VALUE, "negative size");
+static int hqp_check(int32_t io_dtype, int32_t b_dim, int32_t num_bits, int32_t symmetric) {
   CTMI_REQUIRE(io_dtype == CTMI_BF16, CTMI_ERR_UNSUPPORTED,
                "the fused rotation + quantization takes bfloat16 tensors");
   CTMI_REQUIRE(b_dim == 32 || b_dim == 64 || b_dim == 128, CTMI_ERR_UNSUPPORTED,
                "block (= group) size must be 32, 64 or 128, got %d", b_dim);
   CTMI_REQUIRE(num_bits == 4 && symmetric, CTMI_ERR_UNSUPPORTED,
                "only symmetric 4-bit integer quantization is fused");
-  CTMI_REQUIRE(numel % b_dim == 0, CTMI_ERR_VALUE,
-               "tensor size %lld is not a multiple of the block size %d", (long long)numel, b_dim);
-  if (numel == 0) return CTMI_OK;
-  CTMI_REQUIRE(x && mb_t && packed && scale, CTMI_ERR_VALUE, "NULL tensor pointer");
-  CTMI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)mb_t % 16 == 0 && (uintptr_t)rotated % 16 == 0 &&
-                   (uintptr_t)packed % 4 == 0 && (uintptr_t)scale % 2 == 0,
+  return CTMI_OK;
+}
+
+static int hqp_check_job(const ctmi_hadamard_pack_job& j, int32_t b_dim) {
+  CTMI_REQUIRE(j.numel >= 0, CTMI_ERR_VALUE, "negative size");
+  CTMI_REQUIRE(j.numel % b_dim == 0, CTMI_ERR_VALUE,
+               "tensor size %lld is not a multiple of the block size %d", (long long)j.numel, b_dim);
+  if (j.numel == 0) return CTMI_OK;
+  CTMI_REQUIRE(j.x && j.packed && j.scale, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE((uintptr_t)j.x % 16 == 0 && (uintptr_t)j.rotated % 16 == 0 &&
+                   (uintptr_t)j.packed % 4 == 0 && (uintptr_t)j.scale % 2 == 0,
                CTMI_ERR_VALUE, "tensors must be 16-byte aligned");
+  return CTMI_OK;
+}
+
+static void hqp_launch(const HadJobs& t, int filled, int32_t b_dim, const void* mb_t,
+                       const float* sign_in, const float* sign_out, int32_t num_bits,
+                       hipStream_t st) {
   QpCfg c{};
   quant_range(CTMI_QTYPE_INT, num_bits, &c.bit_min, &c.bit_max);
   c.range = c.bit_max - c.bit_min;
@@ -920,19 +1071,71 @@ extern "C" int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t
   c.symmetric = 1;
   c.mt = c.zp_sub_dtype = c.scale_dtype = CTMI_BF16;
   c.zp_dtype = CTMI_I8;
-  const int64_t n_sub = numel / b_dim;
-  const int64_t wgs = cdiv(cdiv(n_sub, 16), kHqpWaves);
+  const int64_t n_groups = t.end[filled - 1];
+  const int64_t wgs = cdiv(n_groups, kHqpWaves);
   const int64_t cap = 256 * CTMI_HQP_WG_PER_CU;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
   const float inv = 1.0f / sqrtf((float)b_dim);
-  hipStream_t st = (hipStream_t)stream;
-#define CTMI_HQP(BB)                                                                              \
-  hipLaunchKernelGGL(hadamard_quant_pack_kernel<BB>, grid, kHqpThreads, 0, st, (const uint16_t*)x, \
-                     (const uint16_t*)mb_t, sign_in, sign_out, packed, (uint16_t*)scale,          \
-                     (uint16_t*)rotated, n_sub, inv, c)
-  if (b_dim == 32) CTMI_HQP(32);
-  else if (b_dim == 64) CTMI_HQP(64);
-  else CTMI_HQP(128);
+#define CTMI_HQP(BB)                                                                             \
+  if (filled == 1)                                                                               \
+    hipLaunchKernelGGL((hadamard_quant_pack_kernel<BB, false>), grid, kHqpThreads, 0, st, t,     \
+                       n_groups, (const uint16_t*)mb_t, sign_in, sign_out, inv, c);              \
+  else                                                                                           \
+    hipLaunchKernelGGL((hadamard_quant_pack_kernel<BB, true>), grid, kHqpThreads, 0, st, t,      \
+                       n_groups, (const uint16_t*)mb_t, sign_in, sign_out, inv, c)
+  if (b_dim == 32) { CTMI_HQP(32); }
+  else if (b_dim == 64) { CTMI_HQP(64); }
+  else { CTMI_HQP(128); }
 #undef CTMI_HQP
-  return check_launch("ctmi_hadamard_quant_pack");
+}
+
+extern "C" int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_jobs,
+                                             int32_t io_dtype, int32_t b_dim, const void* mb_t,
+                                             const float* sign_in, const float* sign_out,
+                                             int32_t num_bits, int32_t symmetric, void* stream) {
+  CTMI_REQUIRE(n_jobs >= 0 && (jobs || n_jobs == 0), CTMI_ERR_VALUE, "bad job list");
+  int rc = hqp_check(io_dtype, b_dim, num_bits, symmetric);
+  if (rc) return rc;
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    rc = hqp_check_job(jobs[i], b_dim);
+    if (rc) return rc;
+  }
+  CTMI_REQUIRE(n_jobs == 0 || (mb_t && (uintptr_t)mb_t % 16 == 0), CTMI_ERR_VALUE,
+               "the matrix must be given, 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  HadJobs t;
+  clear_jobs(&t);
+  int filled = 0;
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_hadamard_pack_job& j = jobs[i];
+    if (j.numel == 0) continue;
+    t.x[filled] = j.x;
+    t.out[filled] = j.packed;
+    t.scale[filled] = j.scale;
+    t.rotated[filled] = j.rotated;
+    t.n_sub[filled] = j.numel / b_dim;
+    t.end[filled] = (filled ? t.end[filled - 1] : 0) + cdiv(j.numel / b_dim, 16);
+    if (++filled == kHadMaxJobs) {
+      hqp_launch(t, filled, b_dim, mb_t, sign_in, sign_out, num_bits, st);
+      clear_jobs(&t);
+      filled = 0;
+    }
+  }
+  if (filled) hqp_launch(t, filled, b_dim, mb_t, sign_in, sign_out, num_bits, st);
+  return check_launch("ctmi_hadamard_quant_pack_many");
+}
+
+extern "C" int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t numel, int32_t b_dim,
+                                        const void* mb_t, const float* sign_in,
+                                        const float* sign_out, int32_t num_bits, int32_t symmetric,
+                                        int32_t* packed, void* scale, void* rotated, void* stream) {
+  ctmi_hadamard_pack_job job;
+  job.x = x;
+  job.packed = packed;
+  job.scale = scale;
+  job.rotated = rotated;
+  job.numel = numel;
+  int rc = ctmi_hadamard_quant_pack_many(&job, 1, io_dtype, b_dim, mb_t, sign_in, sign_out, num_bits,
+                                         symmetric, stream);
+  return rc;
 }

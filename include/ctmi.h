@@ -376,6 +376,19 @@ int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t nume
                         int32_t b_dim, const void* ma_t, const void* mb_t, const float* sign_in,
                         const float* sign_out, void* stream);
 
+/* The same transform on several tensors (the weights of a model that share a
+ * rotation, transform/factory/hadamard.py:46-67 hands one matrix to every module of
+ * a scheme) from one call: tensors share launches, 8 at a time, so that the set-up
+ * of the matrix is paid once per launch and not once per tensor. */
+typedef struct ctmi_hadamard_job {
+  const void* x;
+  void* out;
+  int64_t numel;
+} ctmi_hadamard_job;
+int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n_jobs, int32_t io_dtype,
+                             int32_t a_dim, int32_t b_dim, const void* ma_t, const void* mb_t,
+                             const float* sign_in, const float* sign_out, void* stream);
+
 /* A24 / A25 + A2 + A1 + A11 in one pass, for bf16 tensors, block size b_dim (32,
  * 64 or 128) equal to the quantization group size, symmetric 4-bit integers:
  * the rotation of ctmi_hadamard_apply (a_dim == 1) followed, per rotated block,
@@ -387,6 +400,19 @@ int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t numel, int
                              const void* mb_t, const float* sign_in, const float* sign_out,
                              int32_t num_bits, int32_t symmetric, int32_t* packed, void* scale,
                              void* rotated, void* stream);
+
+/* ctmi_hadamard_quant_pack for several tensors from one call, 8 per launch. */
+typedef struct ctmi_hadamard_pack_job {
+  const void* x;
+  int32_t* packed;
+  void* scale;
+  void* rotated; /* or NULL */
+  int64_t numel;
+} ctmi_hadamard_pack_job;
+int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_jobs,
+                                  int32_t io_dtype, int32_t b_dim, const void* mb_t,
+                                  const float* sign_in, const float* sign_out, int32_t num_bits,
+                                  int32_t symmetric, void* stream);
 
 /* A24 for an arbitrary explicit fp32 matrix w [h,h] (small h, or matrices that
  * are not +-1): every run of h consecutive elements x becomes x * w / sqrt(h).

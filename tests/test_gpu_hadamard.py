@@ -3,7 +3,7 @@ explicit matrix): within one ulp of the output dtype."""
 import pytest
 import torch
 
-from gpu_util import announce
+from gpu_util import announce, assert_bit_equal
 from oracle import hadamard as oh
 
 pytestmark = pytest.mark.gpu
@@ -202,3 +202,49 @@ def test_fused_rotation_quantization_packing(n, shape, gpu):
         o_packed = op.pack_quantized_compress(yc, o_scale, oargs, zero_point=o_zp)["weight_packed"]
         assert torch.equal(fused["weight_scale"].cpu().view(torch.int16), o_scale.view(torch.int16))
         assert torch.equal(fused["weight_packed"].cpu(), o_packed)
+
+
+@pytest.mark.parametrize("n,dtype", [(128, torch.bfloat16), (64, torch.float16), (32, torch.bfloat16),
+                                     (4096, torch.bfloat16), (1024, torch.float16), (2048, torch.bfloat16),
+                                     (128, torch.float32)])
+def test_many_tensors_in_one_call(n, dtype, gpu):
+    """hadamard_apply_many == hadamard_apply tensor by tensor, bit for bit: more tensors than
+    one launch takes (8), sizes that differ, a tensor that ends in a ragged group of
+    sub-rows (it gets a call of its own), an empty one; fp32 goes tensor by tensor"""
+    from compressed_tensors_amd.transform import hadamard_apply, hadamard_apply_many
+
+    announce("hadamard many", n, dtype)
+    g = torch.Generator().manual_seed(n)
+    q_in = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    q_out = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    rows = [16, 48, 5, 64, 1, 32, 16, 80, 16, 33, 0]
+    xs = [(torch.randn(r, 2 * n if n <= 128 else n, generator=g) * 0.05).to(dtype).to(gpu) for r in rows]
+    for signs in (dict(), dict(sign_in=q_in, sign_out=q_out)):
+        got = hadamard_apply_many(xs, n, **signs)
+        assert len(got) == len(xs)
+        for i, (x, y) in enumerate(zip(xs, got)):
+            assert y.shape == x.shape
+            if x.numel():
+                assert_bit_equal(y, hadamard_apply(x, n, **signs), f"tensor {i} ({rows[i]} rows)")
+
+
+def test_fused_many_tensors_in_one_call(gpu):
+    """hadamard_quantize_pack_many == hadamard_quantize_pack tensor by tensor"""
+    from compressed_tensors_amd.quantization import QuantizationArgs
+    from compressed_tensors_amd.transform import hadamard_quantize_pack, hadamard_quantize_pack_many
+
+    announce("fused hadamard many")
+    n = 128
+    g = torch.Generator().manual_seed(77)
+    q = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=n)
+    shapes = [(64, 512), (37, 256), (16, 128), (5, 1024), (128, 256), (1, 128), (48, 384), (33, 128), (96, 640),
+              (7, 256)]
+    xs = [(torch.randn(s, generator=g) * 0.02).bfloat16().to(gpu) for s in shapes]
+    for signs in (dict(), dict(sign_in=q)):
+        got = hadamard_quantize_pack_many(xs, n, args, **signs)
+        for i, (x, out) in enumerate(zip(xs, got)):
+            want = hadamard_quantize_pack(x, n, args, **signs)
+            assert_bit_equal(out["weight_packed"], want["weight_packed"], f"packed {i}")
+            assert_bit_equal(out["weight_scale"], want["weight_scale"], f"scale {i}")
+            assert out["weight_shape"].tolist() == list(shapes[i])
