@@ -200,11 +200,22 @@ def other_workload(torch, name, seed):
             hot = torch.rand(r, c, generator=gen, device=dev) < 1e-3
             w = torch.where(hot, w * 20, w)
             scale, zp = observe_weight_qparams(w, args)
-            entries.append(dict(weight=w, scale=scale, zero_point=None, quantization_args=args))
+            entries.append(dict(weight=w, scale=scale, zero_point=None, quantization_args=args, observed_zp=zp))
             n += r * c
         batch = QuantizedWeightBatch(entries)   # one ctmi_qdq_many call per direction
         keep.append(batch)
         q_calls, d_calls = [batch.compress], [batch.decompress]
+        # one-shot: scales + fp8 codes from one pass over weights that have no scales yet,
+        # against the observer and the quantizer one after the other (one call per weight each)
+        w_obs, w_q, w_one = [], [], []
+        for e, codes in zip(entries, batch.codes):
+            w, sc = e["weight"], e["scale"]
+            r, c = w.shape
+            w_obs.append(observe(w, c, args, sc, e["observed_zp"]))
+            w_q.append(qdq(w, codes, build_qparams(w, sc, None, args), 1, 0))
+            oa = (w.data_ptr(), code(w.dtype), codes.data_ptr(), r, c, c, 1, 8, 1, sc.data_ptr(), code(sc.dtype),
+                  None, code(FP8), st)
+            w_one.append(lambda oa=oa: _lib.check(lib.ctmi_observe_quantize(*oa)))
         acts, a_obs, a_fq, a_dyn = [], [], [], []
         targs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="token",
                                  dynamic=True)
@@ -221,6 +232,9 @@ def other_workload(torch, name, seed):
         na = 8 * 8192 * 4096
         ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_kernel"),
                Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_kernel"),
+               Op("weights one-shot: per-channel observer (224 calls)", w_obs, 2 * n, "observe_wide_kernel"),
+               Op("weights one-shot: quantize with those scales (224 calls)", w_q, 3 * n, "qdq_vec_kernel"),
+               Op("weights one-shot: scales + fp8 codes in one pass (224 calls)", w_one, 3 * n, "dynamic_rows_kernel"),
                Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
                Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel"),
                Op("activations: scales + fake-quantize in one pass (8 x 8192x4096)", a_dyn, 4 * na, "dynamic_rows_kernel")]

@@ -248,6 +248,12 @@ SIGNATURES = {
     "ctmi_dynamic_qdq_supported": (
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32],
     ),
+    "ctmi_observe_quantize_supported": (c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32]),
+    "ctmi_observe_quantize": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32, c_void_p,
+         c_int32, c_void_p, c_int32, c_void_p],
+    ),
     "ctmi_dynamic_qdq": (
         c_int32,
         [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32,

@@ -114,6 +114,66 @@ class NaiveQuantizationCompressor(BaseQuantizationCompressor):
             quantized = quantized.to(device)
         return {"weight": quantized}
 
+    def observe_and_compress_weight(
+        self, weight: Tensor, quantization_args: QuantizationArgs,
+        device: Optional[torch.device] = None,
+    ) -> Dict[str, Tensor]:
+        """One-shot (round-to-nearest) compression of a weight that has no scales yet: the
+        min-max observer (tests/mock_observer.py:38-113), calculate_qparams
+        (quantization/utils/helpers.py:67-146) and compress_weight in one pass over the
+        weight for channel and group strategies.  Returns compress_weight's dict plus
+        "weight_scale" (and "weight_zero_point" for an asymmetric scheme)."""
+        from compressed_tensors_amd.quantization.helpers import _zp_dtype, observe_weight_qparams
+        from compressed_tensors_amd.quantization.quant_args import QuantizationStrategy
+
+        args = quantization_args
+        weight = to_gpu(weight)
+        if weight.ndim != 2:
+            raise ValueError(f"expected a 2-D weight, got shape {tuple(weight.shape)}")
+        rows, cols = weight.shape
+        if args.strategy == QuantizationStrategy.GROUP.value:
+            blk_cols = args.group_size
+        elif args.strategy == QuantizationStrategy.CHANNEL.value:
+            blk_cols = cols
+        else:
+            blk_cols = 0
+        lib = _lib.load()
+        w = weight.contiguous()
+        qtype = _lib.QTYPE_INT if args.type == "int" else _lib.QTYPE_FLOAT
+        fused = (
+            blk_cols > 0 and can_quantize(weight, args) and rows > 0 and cols > 0
+            and w.data_ptr() % (8 * w.element_size()) == 0
+            and lib.ctmi_observe_quantize_supported(_lib.dtype_code(w.dtype), rows, cols, blk_cols,
+                                                    qtype, args.num_bits)
+        )
+        if not fused:
+            scale, zero_point = observe_weight_qparams(weight, args)
+            out = self.compress_weight(weight, scale, args, zero_point=zero_point, device=device)
+            out["weight_scale"] = scale if device is None else scale.to(device)
+            if not args.symmetric:
+                out["weight_zero_point"] = zero_point if device is None else zero_point.to(device)
+            return out
+        n_cells = cols // min(blk_cols, cols)
+        codes = torch.empty((rows, cols), dtype=args.pytorch_dtype(), device=w.device)
+        scale = torch.empty((rows, n_cells), dtype=w.dtype, device=w.device)
+        zero_point = None
+        if not args.symmetric:
+            zero_point = torch.empty((rows, n_cells), dtype=_zp_dtype(args), device=w.device)
+        zp_code = _lib.dtype_code(_zp_dtype(args))
+        _lib.check(
+            lib.ctmi_observe_quantize(
+                w.data_ptr(), _lib.dtype_code(w.dtype), codes.data_ptr(), rows, cols, blk_cols, qtype,
+                args.num_bits, int(args.symmetric), scale.data_ptr(), _lib.dtype_code(scale.dtype),
+                _lib.ptr(zero_point), zp_code, _lib.stream_of(w.device),
+            )
+        )
+        out = {"weight": codes, "weight_scale": scale}
+        if zero_point is not None:
+            out["weight_zero_point"] = zero_point
+        if device is not None:
+            out = {k: v.to(device) for k, v in out.items()}
+        return out
+
     def decompress_weight(
         self,
         compressed_data: Dict[str, Tensor],

@@ -10,6 +10,12 @@
 // min / max, read again and written by fake_quantize); the arithmetic here is the
 // same, step for step, on data that is read once: 4 bytes per bf16 element
 // instead of 6.
+//
+// The same kernels with codes for output (int8 or fp8 instead of the fake-quantized
+// tensor) are the one-shot form of the naive-quantized compressors: min-max
+// observer (tests/mock_observer.py:38-113), calculate_qparams and
+// NaiveQuantizationCompressor.compress_weight (naive_quantized.py:79-114) over a
+// weight that is read once.
 #include <type_traits>
 
 #include "ctmi_device.h"
@@ -53,12 +59,31 @@ __device__ __forceinline__ void store_cell(const DynOut& o, int64_t cell, float 
   if (o.zp) store_from_f32(o.zp, zp_dtype, cell, zv);
 }
 
+// Item `v` of the output: the fake-quantized values, or (CODES) the int8 / fp8 codes
+// that quantize(dtype=args.pytorch_dtype()) returns
+template <typename FT, int QK, bool CODES>
+__device__ __forceinline__ void store_result(void* out_any, int64_t v, bool keep,
+                                             const Vec<typename FT::raw, 8>& a, float sv, float zv,
+                                             const QpCfg& c) {
+  using FR = typename FT::raw;
+  Vec<FR, 8> of;
+  Vec<uint8_t, 8> oc;
+  if constexpr (CODES) {
+    constexpr int kOut = QK == 0 ? kKindI8 : kKindF8;
+    qdq_vec8<FT, kKindFloat, kOut, QK, true>(a, oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
+    if (keep) stg_nt<uint8_t, 8>(static_cast<uint8_t*>(out_any) + v * 8, oc);
+  } else {
+    qdq_vec8<FT, kKindFloat, kKindFloat, QK, true>(a, oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
+    if (keep) stg_nt<FR, 8>(static_cast<FR*>(out_any) + v * 8, of);
+  }
+}
+
 // One workgroup of 256 threads per row-long segment (token / channel) of up to
 // 256 * U vectors of 8 elements: every vector is loaded before anything is looked
 // at; the four wavefronts meet once, over a few words in LDS.
-template <typename FT, int QK, bool SYM, int U>
+template <typename FT, int QK, bool SYM, int U, bool CODES>
 __global__ void __launch_bounds__(256)
-dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __restrict__ out,
+dynamic_rows_kernel(const typename FT::raw* __restrict__ x, void* __restrict__ out_any,
                     DynOut o, int items, QpCfg c) {
   using FR = typename FT::raw;
   __shared__ float part_lo[4], part_hi[4];
@@ -107,22 +132,18 @@ dynamic_rows_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
     cell_qparams<FT, QK, SYM>(lo, hi, unordered, c.bit_min, c.bit_max, &sv, &zv);
   }
   if (threadIdx.x == 0) store_cell(o, s, sv, zv, c.scale_dtype, c.zp_dtype);
-  FR* q = out + s * (int64_t)items * 8;
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int i = k * 256 + threadIdx.x;
-    Vec<FR, 8> of;
-    Vec<uint8_t, 8> oc;
-    qdq_vec8<FT, kKindFloat, kKindFloat, QK, true>(a[k], oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
-    if (i < items) stg_nt<FR, 8>(q + (int64_t)i * 8, of);
+    store_result<FT, QK, CODES>(out_any, s * (int64_t)items + i, i < items, a[k], sv, zv, c);
   }
 }
 
 // Segments of L vectors, L a power of two <= 64 (group strategies): L neighbouring
 // lanes own a segment; memory is one run of vectors numbered like the segments.
-template <typename FT, int QK, bool SYM>
+template <typename FT, int QK, bool SYM, bool CODES>
 __global__ void __launch_bounds__(256)
-dynamic_flat_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __restrict__ out,
+dynamic_flat_kernel(const typename FT::raw* __restrict__ x, void* __restrict__ out_any,
                     DynOut o, int64_t nvec, int L, QpCfg c) {
   using FR = typename FT::raw;
   constexpr int U = 2;
@@ -150,14 +171,11 @@ dynamic_flat_kernel(const typename FT::raw* __restrict__ x, typename FT::raw* __
       cell_qparams<FT, QK, SYM>(lo, hi, group_any(L, unordered), c.bit_min, c.bit_max, &sv, &zv);
     }
     if (v < nvec && (threadIdx.x & (L - 1)) == 0) store_cell(o, v / L, sv, zv, c.scale_dtype, c.zp_dtype);
-    Vec<FR, 8> of;
-    Vec<uint8_t, 8> oc;
-    qdq_vec8<FT, kKindFloat, kKindFloat, QK, true>(a[k], oc, sv, zv, c.bit_min, c.bit_max, &of, &oc);
-    if (v < nvec) stg_nt<FR, 8>(out + v * 8, of);
+    store_result<FT, QK, CODES>(out_any, v, v < nvec, a[k], sv, zv, c);
   }
 }
 
-template <typename FT, int QK, bool SYM>
+template <typename FT, int QK, bool SYM, bool CODES>
 static bool launch_dynamic(const void* x, void* out, const DynOut& o, int64_t rows, int64_t cols,
                            int64_t blk_cols, const QpCfg& c, hipStream_t st) {
   using FR = typename FT::raw;
@@ -167,17 +185,18 @@ static bool launch_dynamic(const void* x, void* out, const DynOut& o, int64_t ro
   if (items <= 64 && (items & (items - 1)) == 0) {
     const int64_t blocks = cdiv(nvec, 256 * 2);
     if (blocks >= (1ll << 31)) return false;
-    hipLaunchKernelGGL((dynamic_flat_kernel<FT, QK, SYM>), (unsigned)blocks, 256, 0, st, (const FR*)x,
-                       (FR*)out, o, nvec, (int)items, c);
+    hipLaunchKernelGGL((dynamic_flat_kernel<FT, QK, SYM, CODES>), (unsigned)blocks, 256, 0, st,
+                       (const FR*)x, out, o, nvec, (int)items, c);
     return true;
   }
   if (n_segments >= (1ll << 31)) return false;
 #define CTMI_DYN(UU)                                                                    \
-  hipLaunchKernelGGL((dynamic_rows_kernel<FT, QK, SYM, UU>), (unsigned)n_segments, 256, 0, st, \
-                     (const FR*)x, (FR*)out, o, (int)items, c)
+  hipLaunchKernelGGL((dynamic_rows_kernel<FT, QK, SYM, UU, CODES>), (unsigned)n_segments, 256, 0, st, \
+                     (const FR*)x, out, o, (int)items, c)
   if (items <= 256) CTMI_DYN(1);
   else if (items <= 256 * 2) CTMI_DYN(2);
   else if (items <= 256 * 4) CTMI_DYN(4);
+  else if (items <= 256 * 8) CTMI_DYN(8);
   else return false;
 #undef CTMI_DYN
   return true;
@@ -200,7 +219,7 @@ extern "C" int ctmi_dynamic_qdq_supported(int32_t x_dtype, int64_t rows, int64_t
   if (has_global_scale) return 0;
   if (!((qtype == CTMI_QTYPE_INT && num_bits <= 8) || (qtype == CTMI_QTYPE_FLOAT && num_bits == 8)))
     return 0;
-  return items <= 1024;
+  return items <= 2048;
 }
 
 extern "C" int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64_t rows,
@@ -230,8 +249,8 @@ extern "C" int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64
   } else {
     const int qk = qtype == CTMI_QTYPE_INT ? 0 : 1;
 #define CTMI_DYN_SYM(FT, QK)                                                               \
-  (symmetric ? launch_dynamic<FT, QK, true>(x, out, o, rows, cols, blk_cols, c, st)        \
-             : launch_dynamic<FT, QK, false>(x, out, o, rows, cols, blk_cols, c, st))
+  (symmetric ? launch_dynamic<FT, QK, true, false>(x, out, o, rows, cols, blk_cols, c, st) \
+             : launch_dynamic<FT, QK, false, false>(x, out, o, rows, cols, blk_cols, c, st))
 #define CTMI_DYN_FT(FT) (qk == 0 ? CTMI_DYN_SYM(FT, 0) : CTMI_DYN_SYM(FT, 1))
     ok = x_dtype == CTMI_BF16 ? CTMI_DYN_FT(BF16)
                               : (x_dtype == CTMI_F16 ? CTMI_DYN_FT(F16) : CTMI_DYN_FT(F32));
@@ -240,4 +259,41 @@ extern "C" int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64
   }
   CTMI_REQUIRE(ok, CTMI_ERR_UNSUPPORTED, "no fused kernel for this layout");
   return check_launch("ctmi_dynamic_qdq");
+}
+
+extern "C" int ctmi_observe_quantize_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                               int64_t blk_cols, int32_t qtype, int32_t num_bits) {
+  if (qtype == CTMI_QTYPE_FLOAT && num_bits != 8) return 0;
+  return ctmi_dynamic_qdq_supported(x_dtype, rows, cols, blk_cols, qtype, num_bits, 0);
+}
+
+extern "C" int ctmi_observe_quantize(const void* x, int32_t x_dtype, void* codes, int64_t rows,
+                                     int64_t cols, int64_t blk_cols, int32_t qtype,
+                                     int32_t num_bits, int32_t symmetric, void* scale_out,
+                                     int32_t scale_dtype, void* zp_out, int32_t zp_dtype,
+                                     void* stream) {
+  CTMI_REQUIRE(rows >= 1 && cols >= 1, CTMI_ERR_VALUE, "cannot observe an empty tensor");
+  CTMI_REQUIRE(blk_cols >= 1, CTMI_ERR_VALUE, "empty cell");
+  QpCfg c;
+  int rc = fill_qpcfg(&c, qtype, num_bits, symmetric, x_dtype, 0, false, scale_dtype, zp_dtype);
+  if (rc) return rc;
+  CTMI_REQUIRE(x && codes && scale_out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE(ctmi_observe_quantize_supported(x_dtype, rows, cols, blk_cols, qtype, num_bits),
+               CTMI_ERR_UNSUPPORTED,
+               "no fused kernel for this layout: compute the scales and quantize separately");
+  CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)codes % 8 == 0,
+               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+  hipStream_t st = (hipStream_t)stream;
+  const DynOut o{scale_out, zp_out};
+  const int qk = qtype == CTMI_QTYPE_INT ? 0 : 1;
+#define CTMI_OQ_SYM(FT, QK)                                                                  \
+  (symmetric ? launch_dynamic<FT, QK, true, true>(x, codes, o, rows, cols, blk_cols, c, st)  \
+             : launch_dynamic<FT, QK, false, true>(x, codes, o, rows, cols, blk_cols, c, st))
+#define CTMI_OQ_FT(FT) (qk == 0 ? CTMI_OQ_SYM(FT, 0) : CTMI_OQ_SYM(FT, 1))
+  const bool ok = x_dtype == CTMI_BF16 ? CTMI_OQ_FT(BF16)
+                                       : (x_dtype == CTMI_F16 ? CTMI_OQ_FT(F16) : CTMI_OQ_FT(F32));
+#undef CTMI_OQ_SYM
+#undef CTMI_OQ_FT
+  CTMI_REQUIRE(ok, CTMI_ERR_UNSUPPORTED, "no fused kernel for this layout");
+  return check_launch("ctmi_observe_quantize");
 }

@@ -332,7 +332,7 @@ int ctmi_observe_nvfp4_compress(const void* x, int32_t x_dtype, int64_t rows, in
  * [rows, cols / blk_cols] outputs with the dtypes ctmi_observe_qparams documents.
  * global_scale: the fp32 scalar of a tensor_group (nvfp4) scheme, else NULL.
  * ctmi_dynamic_qdq_supported() says whether a layout has a fused kernel (int
- * <= 8 bits and fp8: cells of up to 8192 elements in multiples of 8; fp4 with
+ * <= 8 bits and fp8: cells of up to 16384 elements in multiples of 8; fp4 with
  * a global scale: cells of 16); CTMI_ERR_UNSUPPORTED otherwise,
  * and the caller runs ctmi_observe_qparams + ctmi_qdq. */
 int ctmi_dynamic_qdq_supported(int32_t x_dtype, int64_t rows, int64_t cols, int64_t blk_cols,
@@ -341,6 +341,22 @@ int ctmi_dynamic_qdq(const void* x, int32_t x_dtype, void* out, int64_t rows, in
                      int64_t blk_cols, int32_t qtype, int32_t num_bits, int32_t symmetric,
                      const float* global_scale, void* scale_out, int32_t scale_dtype,
                      void* zp_out, int32_t zp_dtype, void* stream);
+
+/* N1 for the naive-quantized formats: one-shot compression of a weight that has no
+ * scales yet.  The min-max observer (tests/mock_observer.py:38-113), calculate_qparams
+ * (quantization/utils/helpers.py:67-146) and NaiveQuantizationCompressor.compress_weight
+ * (naive_quantized.py:79-114: quantize with dtype = args.pytorch_dtype()) for cells of
+ * 1 x blk_cols elements (channel: blk_cols = cols; group: blk_cols = group_size) from
+ * one pass over x.  codes: int8 (integer grids of up to 8 bits) or float8_e4m3fn
+ * [rows, cols]; scale_out [rows, cols / blk_cols] in scale_dtype; zp_out optional.
+ * Same bits as ctmi_observe_qparams followed by ctmi_qdq.  _supported() as for
+ * ctmi_dynamic_qdq. */
+int ctmi_observe_quantize_supported(int32_t x_dtype, int64_t rows, int64_t cols, int64_t blk_cols,
+                                    int32_t qtype, int32_t num_bits);
+int ctmi_observe_quantize(const void* x, int32_t x_dtype, void* codes, int64_t rows, int64_t cols,
+                          int64_t blk_cols, int32_t qtype, int32_t num_bits, int32_t symmetric,
+                          void* scale_out, int32_t scale_dtype, void* zp_out, int32_t zp_dtype,
+                          void* stream);
 
 /* MXFP4 group scales (quantization/utils/mxfp4_utils.py): powers of two held as
  * uint8 exponents.  x / out of the first two are bfloat16 group maxima, n values.

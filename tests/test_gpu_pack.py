@@ -640,3 +640,45 @@ def test_nvfp4_weight_batch_and_state_dict(gpu):
     restored = dict(comp.decompress_from_state_dict(out, names_to_scheme=schemes))
     for i in range(len(shapes)):
         assert_bit_equal(restored[f"m{i}"]["weight"], dense[i], f"state dict decompress {i}")
+
+
+OQ = [
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (96, 512), torch.bfloat16),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (40, 14336), torch.bfloat16),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (33, 4104), torch.float16),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=128), (24, 1024), torch.bfloat16),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (96, 512), torch.bfloat16),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=False, strategy="channel"), (17, 2048), torch.bfloat16),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=128), (16, 256), torch.float16),
+    ("naive-quantized", dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (16, 64), torch.float32),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=False, strategy="channel"), (12, 640), torch.bfloat16),
+    # no fused kernel: rows longer than 16384, one scale for the whole tensor
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (3, 16392), torch.bfloat16),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=True, strategy="tensor"), (31, 64), torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("fmt,spec,shape,dtype", OQ, ids=[f"{c[0]}-{i}" for i, c in enumerate(OQ)])
+def test_naive_observe_and_compress_in_one_pass(fmt, spec, shape, dtype, gpu):
+    """scales + codes from one kernel: the oracle's observer, calculate_qparams and naive
+    compression, bit for bit; shapes without a fused kernel take the two steps"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("one-shot", fmt, spec, shape, dtype)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(43)
+    w = torch.randn(shape, generator=g) * 0.02
+    w[torch.rand(shape, generator=g) < 0.001] *= 20
+    w = w.to(dtype)
+    w.view(-1)[1] = -0.0
+    w[-1] = 0  # an all-zero row: the scale is clamped from below
+    scale, zp = oq.observe_weight(w, oargs)
+    want = op.naive_compress(w, scale, oargs, zero_point=zp)
+    comp = BaseCompressor.load_from_registry(fmt)
+    got = comp.observe_and_compress_weight(w.to(gpu), args)
+    assert set(got) == ({"weight", "weight_scale"} | (set() if spec["symmetric"] else {"weight_zero_point"}))
+    assert_bit_equal(got["weight_scale"], scale, "scale")
+    if not spec["symmetric"]:
+        assert_bit_equal(got["weight_zero_point"], zp, "zero point")
+    assert_bit_equal(got["weight"], want, "codes")
+    assert got["weight"].dtype == args.pytorch_dtype()
