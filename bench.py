@@ -242,7 +242,7 @@ def other_workload(torch, name, seed):
 
     if name == "sparse":
         copies = 6
-        c_calls, d_calls, s_calls, t_calls = [], [], [], []
+        c_calls, d_calls, s_calls, t_calls, two_step, one_step = [], [], [], [], [], []
         nb = 8192 * 8192
         nnz_total = 0
         for _ in range(copies):
@@ -284,13 +284,23 @@ def other_workload(torch, name, seed):
             _lib.check(lib.ctmi_sparse24_compress(*a))
             keep.extend([q, values, bitmask, dense, tmp])
             s_calls.append(lambda a=a: _lib.check(lib.ctmi_sparse24_compress(*a)))
+            # the stacked case: bf16 -> fp8 codes -> 2:4, two steps against one
+            plan = build_qparams(w, scale, None, cargs)
+            keep.extend([w, scale, plan])
+            qa = (w.data_ptr(), code(w.dtype), q.data_ptr(), code(q.dtype), rows, cols, ctypes.byref(plan.qp), 1, 0, st)
+            fa = (w.data_ptr(), code(w.dtype), values.data_ptr(), bitmask.data_ptr(), rows, cols, ctypes.byref(plan.qp), st)
+            two_step.append(lambda qa=qa, a=a: (_lib.check(lib.ctmi_qdq(*qa)), _lib.check(lib.ctmi_sparse24_compress(*a))))
+            one_step.append(lambda fa=fa: _lib.check(lib.ctmi_quantize_sparse24_compress(*fa)))
             t_calls.append(lambda d=d: _lib.check(lib.ctmi_sparse24_decompress(*d)))
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies * (n24 + n24 // 2 + n24 // 8)
+        fused24_bytes = copies * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
         ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_kernel"),
                Op("sparse-bitmask decompress (positions from the bitmask alone)", d_calls, bm_bytes, "bitmask_scatter_tiles_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
-               Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel")]
+               Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
+               Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel"),
+               Op("bf16 -> fp8 codes -> 2:4 compress, one pass", one_step, fused24_bytes, "quant_sparse24_compress_kernel")]
         return "sparse-bitmask / sparse-24-bitmask compress+decompress GB/s", ops, keep
 
     if name == "nvfp4":

@@ -166,6 +166,11 @@ SIGNATURES = {
     ),
     "ctmi_pack_bitmasks": (c_int32, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "ctmi_unpack_bitmasks": (c_int32, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "ctmi_quantize_sparse24_compress_supported": (c_int32, [c_int32, c_int64, c_int64, POINTER(QParams)]),
+    "ctmi_quantize_sparse24_compress": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, POINTER(QParams), c_void_p],
+    ),
     "ctmi_bitmask_tmp_bytes": (c_int64, [c_int64, c_int64]),
     "ctmi_bitmask_count": (
         c_int32,

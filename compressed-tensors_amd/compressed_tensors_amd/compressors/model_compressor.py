@@ -120,6 +120,11 @@ class ModelCompressor:
                  show_progress: bool = False) -> Dict[str, Tensor]:
         if state_dict is None:
             state_dict = model.state_dict()
+        stacked = self._compress_quantized_24(model, state_dict)
+        if stacked:
+            # those weights are done: what is left of them (scales, zero points) goes
+            # through the quantization compressor's own rules below
+            state_dict = {k: v for k, v in state_dict.items() if k not in stacked}
         if self.quantization_compressor is not None:
             module_to_scheme = map_module_to_scheme(model)
             quant_compressor = next(iter(self.quantization_compressor.values()))
@@ -133,7 +138,52 @@ class ModelCompressor:
                 state_dict, compression_targets=self._sparse_targets(model),
                 show_progress=show_progress,
             )
+        for entries in stacked.values():
+            state_dict.update(entries)
         return state_dict
+
+    def _compress_quantized_24(self, model: Module, state_dict: Dict[str, Tensor]) -> Dict[str, Dict[str, Tensor]]:
+        """Weights that get int8 / fp8 codes AND 2:4 compression (quantization first, then
+        the sparse compressor on the codes, model_compressor.py:638-667): both from one pass
+        over the dense weight where a fused kernel exists.  Returns, per dense weight name,
+        the entries the two compressors would have left for it."""
+        from compressed_tensors_amd.compressors.naive_quantized import NaiveQuantizationCompressor
+        from compressed_tensors_amd.compressors.sparse_24_bitmask import (
+            Sparse24BitMaskCompressor, Sparse24BitMaskTensor, quantize_sparse24_compress,
+        )
+
+        if (self.quantization_compressor is None or self.sparsity_compressor is None
+                or not isinstance(self.sparsity_compressor, Sparse24BitMaskCompressor)):
+            return {}
+        quant_compressor = next(iter(self.quantization_compressor.values()))
+        if not isinstance(quant_compressor, NaiveQuantizationCompressor):
+            return {}
+        structure = getattr(self.sparsity_compressor.config, "sparsity_structure", "2:4")
+        if str(getattr(structure, "value", structure)) != "2:4":
+            return {}
+        targets = self._sparse_targets(model)
+        module_to_scheme = map_module_to_scheme(model)
+        done = {}
+        for name in list(state_dict.keys()):
+            if not name.endswith(".weight") or name[: -len(".weight")] not in targets:
+                continue
+            prefix = name[: -len("weight")]
+            scale = state_dict.get(prefix + "weight_scale", None)
+            scheme = module_to_scheme.get(prefix[:-1], None)
+            if scale is None or scheme is None or scheme.weights is None:
+                continue
+            if state_dict.get(prefix + "weight_global_scale", None) is not None:
+                continue
+            pair = quantize_sparse24_compress(
+                state_dict[name], scale, scheme.weights,
+                zero_point=state_dict.get(prefix + "weight_zero_point", None),
+                g_idx=state_dict.get(prefix + "weight_g_idx", None))
+            if pair is None:
+                continue
+            tensor = Sparse24BitMaskTensor(shape=list(state_dict[name].shape), compressed=pair[0],
+                                           bitmask=pair[1])
+            done[name] = tensor.dict(name_prefix=name, device=self.sparsity_compressor.output_device)
+        return done
 
     def decompress(self, model_path, model: Module) -> None:
         """overwrite the weights of `model` with the ones decompressed from a

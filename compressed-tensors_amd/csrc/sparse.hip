@@ -12,6 +12,7 @@
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "qdq_core.h"
 #include "quant_fast.h"
 #include "topk24_lut.h"
 #include "vec_geom.h"
@@ -874,6 +875,32 @@ bytemask24_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64_t n
 // Fused 2:4 compress, cols % 8 == 0.  Work item = N elements (N/4 groups):
 // one 16-byte load, N/2 survivors stored as one vector, N/8 bitmask bytes.
 // One workgroup per chunk of items, every load issued before the first use.
+// item i (N neighbouring elements): the 2 survivors of every group of 4, in column
+// order, and the item's bitmask bytes
+template <typename R, int DT, int N>
+__device__ __forceinline__ void store_survivors24(const Vec<R, N>& a, R* __restrict__ values,
+                                                  uint8_t* __restrict__ bitmask, int64_t i,
+                                                  bool keep_item) {
+  const uint32_t keep_all = keep_masks24<R, DT, N>(a);
+  Vec<R, N / 2> o;
+  Vec<uint8_t, N / 8> m;
+#pragma unroll
+  for (int q = 0; q < N / 4; ++q) {
+    const uint32_t keep = (keep_all >> (4 * q)) & 15u;
+    // the two survivors in column order: the lower one is element 0, 1 or 2,
+    // the upper one element 1, 2 or 3
+    const R e0 = a.v[4 * q], e1 = a.v[4 * q + 1], e2 = a.v[4 * q + 2], e3 = a.v[4 * q + 3];
+    o.v[2 * q] = (keep & 1u) ? e0 : ((keep & 2u) ? e1 : e2);
+    o.v[2 * q + 1] = (keep & 8u) ? e3 : ((keep & 4u) ? e2 : e1);
+  }
+#pragma unroll
+  for (int bq = 0; bq < N / 8; ++bq) m.v[bq] = (uint8_t)((keep_all >> (8 * bq)) & 0xffu);
+  if (keep_item) {
+    stg<R, N / 2>(values + i * (N / 2), o);
+    stg<uint8_t, N / 8>(bitmask + i * (N / 8), m);
+  }
+}
+
 template <typename R, int DT, int N>
 __global__ void __launch_bounds__(kBlock)
 sparse24_compress_kernel(const R* __restrict__ x, R* __restrict__ values,
@@ -889,25 +916,59 @@ sparse24_compress_kernel(const R* __restrict__ x, R* __restrict__ values,
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int64_t i = i0 + k * kBlock;
-    const uint32_t keep_all = keep_masks24<R, DT, N>(a[k]);
-    Vec<R, N / 2> o;
-    Vec<uint8_t, N / 8> m;
+    store_survivors24<R, DT, N>(a[k], values, bitmask, i, i < nitems);
+  }
+}
+
+// Quantization to fp8 / int8 codes and 2:4 compression of the codes in one pass: what
+// ModelCompressor.compress does to a weight that is both quantized (float- / int- /
+// naive-quantized, naive_quantized.py:79-114) and 2:4 sparse (sparse_24_bitmask.py:
+// 162-203), without the dense code tensor in between: 2 + 1/2 + 1/8 bytes per element
+// instead of 3 + 1 5/8.  A lane quantizes 16 neighbouring elements (two vectors of 8,
+// each with its scale: rows are multiples of 16 elements) and keeps 2 of every 4 codes
+// by the rule of get_24_bytemasks on the codes' int8 view.
+template <typename FT, int QK, bool HAS_ZP>
+__global__ void __launch_bounds__(kBlock)
+quant_sparse24_compress_kernel(const typename FT::raw* __restrict__ x,
+                               const typename FT::raw* __restrict__ scale,
+                               const uint8_t* __restrict__ zp, uint8_t* __restrict__ values,
+                               uint8_t* __restrict__ bitmask, int64_t nitems, VecGeom g, float qmin,
+                               float qmax) {
+  using FR = typename FT::raw;
+  constexpr int U = 2;
+  constexpr int kOut = QK == 0 ? kKindI8 : kKindF8;
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  Vec<FR, 8> a[U][2];
+  FR sraw[U][2];
+  uint8_t zraw[U][2];
 #pragma unroll
-    for (int q = 0; q < N / 4; ++q) {
-      const uint32_t keep = (keep_all >> (4 * q)) & 15u;
-      // the two survivors in column order: the lower one is element 0, 1 or 2,
-      // the upper one element 1, 2 or 3
-      const R e0 = a[k].v[4 * q], e1 = a[k].v[4 * q + 1], e2 = a[k].v[4 * q + 2],
-              e3 = a[k].v[4 * q + 3];
-      o.v[2 * q] = (keep & 1u) ? e0 : ((keep & 2u) ? e1 : e2);
-      o.v[2 * q + 1] = (keep & 8u) ? e3 : ((keep & 4u) ? e2 : e1);
-    }
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    const int64_t at = i < nitems ? i : nitems - 1;  // past the end: re-read, not stored
 #pragma unroll
-    for (int bq = 0; bq < N / 8; ++bq) m.v[bq] = (uint8_t)((keep_all >> (8 * bq)) & 0xffu);
-    if (i < nitems) {
-      stg<R, N / 2>(values + i * (N / 2), o);
-      stg<uint8_t, N / 8>(bitmask + i * (N / 8), m);
+    for (int h = 0; h < 2; ++h) {
+      const uint32_t si = scale_index((uint32_t)(at * 2 + h), g);
+      a[k][h] = ldg_nt<FR, 8>(x + (at * 2 + h) * 8);
+      sraw[k][h] = scale[si];
+      if constexpr (HAS_ZP) zraw[k][h] = zp[si];
     }
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    Vec<uint8_t, 16> q;
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      Vec<FR, 8> unused_f;
+      Vec<uint8_t, 8> codes, unused_c;
+      float z = 0.0f;  // the zero point as the reference adds it (zero_point.to(x.dtype))
+      if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw[k][h] : f8e4m3_to_f32(zraw[k][h]);
+      qdq_vec8<FT, kKindFloat, kOut, QK, HAS_ZP>(a[k][h], unused_c, FT::to_f32(sraw[k][h]), z, qmin,
+                                                 qmax, &unused_f, &codes);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) q.v[8 * h + j] = codes.v[j];
+    }
+    store_survivors24<uint8_t, CTMI_I8, 16>(q, values, bitmask, i, i < nitems);
   }
 }
 
@@ -1280,4 +1341,60 @@ extern "C" int ctmi_sparse24_compress(const void* x, int32_t x_dtype, void* valu
                                                 grid_for(rows * pc, kBlock), kBlock, 0, st,
                                                 (const R*)x, bitmask, rows, cols, pc));
   return check_launch("ctmi_sparse24_compress");
+}
+
+extern "C" int ctmi_quantize_sparse24_compress_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                                         const ctmi_qparams* qp) {
+  if (!qp || rows < 1 || cols < 1 || cols % 16) return 0;
+  if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16 && x_dtype != CTMI_F32) return 0;
+  if (qp->scale_dtype != x_dtype || qp->global_scale || qp->col_group) return 0;
+  if (qp->zero_point &&
+      qp->zp_dtype != (qp->qtype == CTMI_QTYPE_FLOAT ? CTMI_F8E4M3 : CTMI_I8))
+    return 0;
+  const bool codes8 = (qp->qtype == CTMI_QTYPE_FLOAT && qp->num_bits == 8) ||
+                      (qp->qtype == CTMI_QTYPE_INT && qp->num_bits <= 8);
+  if (!codes8) return 0;
+  VecGeom g;
+  return vec_geometry(qp, rows, cols, &g) ? 1 : 0;
+}
+
+extern "C" int ctmi_quantize_sparse24_compress(const void* x, int32_t x_dtype, void* values,
+                                               uint8_t* bitmask, int64_t rows, int64_t cols,
+                                               const ctmi_qparams* qp, void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  int rc = check_qparams(qp, rows, cols);
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(ctmi_quantize_sparse24_compress_supported(x_dtype, rows, cols, qp),
+               CTMI_ERR_UNSUPPORTED,
+               "no fused kernel for this layout: quantize, then compress the codes");
+  CTMI_REQUIRE(x && values && bitmask, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)values % 8 == 0 &&
+                   (uintptr_t)bitmask % 2 == 0,
+               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+  VecGeom g;
+  vec_geometry(qp, rows, cols, &g);
+  float qmin, qmax;
+  rc = quant_range(qp->qtype, qp->num_bits, &qmin, &qmax);
+  if (rc) return rc;
+  const int64_t items = rows * cols / 16;
+  const unsigned grid = (unsigned)cdiv(items, kBlock * 2);
+  hipStream_t st = (hipStream_t)stream;
+  const uint8_t* zp = (const uint8_t*)qp->zero_point;
+#define CTMI_QS24_K(FT, RAW, QK, HZ)                                                             \
+  hipLaunchKernelGGL((quant_sparse24_compress_kernel<FT, QK, HZ>), grid, kBlock, 0, st,           \
+                     (const RAW*)x, (const RAW*)qp->scale, zp, (uint8_t*)values, bitmask, items,  \
+                     g, qmin, qmax)
+#define CTMI_QS24(FT, RAW)                                                       \
+  if (qp->qtype == CTMI_QTYPE_INT) {                                             \
+    if (zp) CTMI_QS24_K(FT, RAW, 0, true); else CTMI_QS24_K(FT, RAW, 0, false);  \
+  } else {                                                                       \
+    if (zp) CTMI_QS24_K(FT, RAW, 1, true); else CTMI_QS24_K(FT, RAW, 1, false);  \
+  }
+  if (x_dtype == CTMI_BF16) { CTMI_QS24(BF16, uint16_t); }
+  else if (x_dtype == CTMI_F16) { CTMI_QS24(F16, uint16_t); }
+  else { CTMI_QS24(F32, float); }
+#undef CTMI_QS24_K
+#undef CTMI_QS24
+  return check_launch("ctmi_quantize_sparse24_compress");
 }

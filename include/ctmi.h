@@ -247,6 +247,20 @@ int ctmi_get_24_bytemasks(const void* x, int32_t x_dtype, uint8_t* mask, int64_t
 int ctmi_sparse24_compress(const void* x, int32_t x_dtype, void* values, uint8_t* bitmask,
                            int64_t rows, int64_t cols, void* stream);
 
+/* A12 + A21 in one pass: the stacked case of ModelCompressor.compress
+ * (model_compressors/model_compressor.py:638-667), a weight that is quantized to
+ * fp8 / int8 codes (naive_quantized.py:79-114) and whose codes are then compressed
+ * as 2:4 (sparse_24_bitmask.py:162-203), without the dense code tensor in between.
+ * values: [rows, cols / 2] codes (float8_e4m3fn or int8); bitmask as in
+ * ctmi_sparse24_compress.  Same bits as ctmi_qdq followed by ctmi_sparse24_compress.
+ * _supported(): cols % 16 == 0, scales in x's dtype on a tensor / channel / group
+ * grid, zero point (if any) in the codes' dtype, codes of 8 bits or fewer. */
+int ctmi_quantize_sparse24_compress_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                              const ctmi_qparams* qp);
+int ctmi_quantize_sparse24_compress(const void* x, int32_t x_dtype, void* values, uint8_t* bitmask,
+                                    int64_t rows, int64_t cols, const ctmi_qparams* qp,
+                                    void* stream);
+
 /* A1.  calculate_qparams (quantization/utils/helpers.py:67-146), elementwise
  * over n (min, max) pairs of dtype mm_dtype.  mm_is_0d != 0 when the reference
  * would see 0-d min/max tensors (their zero-point subtraction then promotes to

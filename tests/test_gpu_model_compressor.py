@@ -120,6 +120,8 @@ def test_fp8_plus_sparse24_stack(gpu):
     apply_quantization_scheme(model, qcfg)
     cpu = _prepare(model, args, oargs, gpu)
     mc = ModelCompressor(sparsity_config=scfg, quantization_config=qcfg)
+    # every targeted Linear goes through the kernel that quantizes and compresses in one pass
+    assert set(mc._compress_quantized_24(model, model.state_dict())) == {f"{n}.weight" for n in cpu}
     state = mc.compress(model)
     for name, (w, s, z) in cpu.items():
         codes = op.naive_compress(w, s, oargs, zero_point=z)

@@ -351,3 +351,56 @@ def test_sparse24_repair_over_many_rows(gpu):
     values = x[keep].reshape(rows, cols // 2)
     dense = sparse24_bitmask_decompress(values.to(gpu), pack_bitmasks(keep.to(gpu)), torch.Size((rows, cols)))
     assert_bit_equal(dense, x, "repaired")
+
+
+QS24 = [
+    (dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (64, 512), torch.bfloat16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (33, 4112), torch.float16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="tensor"), (16, 64), torch.bfloat16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=128), (24, 1024), torch.bfloat16),
+    (dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (40, 256), torch.bfloat16),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="channel"), (40, 256), torch.float32),
+    (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (8, 128), torch.bfloat16),
+]
+
+
+@pytest.mark.parametrize("spec,shape,dtype", QS24, ids=[f"qs24-{i}" for i in range(len(QS24))])
+def test_quantization_and_2_4_compression_in_one_pass(spec, shape, dtype, gpu):
+    """codes + 2:4 compression of the codes from one kernel == the oracle's quantize followed
+    by its sparse24_bitmask_compress, with and without the zero point the observer leaves
+    (it decides whether a value that quantizes to -0 keeps its sign bit)"""
+    from compressed_tensors_amd.compressors import quantize_sparse24_compress
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    announce("quantize + 2:4", spec, shape, dtype)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    g = torch.Generator().manual_seed(shape[1])
+    w = torch.randn(shape, generator=g) * 0.02
+    w[torch.rand(shape, generator=g) < 0.002] *= 30
+    w = _prune24(w).to(dtype)
+    w.view(-1)[0:4] = torch.tensor([-1e-7, 0.0, 3e-3, 0.0]).to(dtype)   # a code of -0 among the survivors
+    scale, zp = oq.observe_weight(w, oargs)
+    for zero_point in ((zp,) if not spec["symmetric"] else (zp, None)):
+        codes = oq.quantize(w, scale, zero_point, oargs, dtype=args.pytorch_dtype())
+        want_values, want_bitmask = osp.sparse24_bitmask_compress(codes)
+        got = quantize_sparse24_compress(w.to(gpu), scale.to(gpu), args,
+                                         zero_point=None if zero_point is None else zero_point.to(gpu))
+        assert got is not None, "expected a fused kernel for this layout"
+        assert_bit_equal(got[0], want_values, "values")
+        assert_bit_equal(got[1], want_bitmask, "bitmask")
+
+
+def test_quantization_and_2_4_without_a_fused_kernel(gpu):
+    """rows that are not whole 16-element items, an act-order g_idx: None, and the caller takes
+    the two steps"""
+    from compressed_tensors_amd.compressors import quantize_sparse24_compress
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    announce("quantize + 2:4, unsupported")
+    args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
+    w = torch.randn(8, 24).bfloat16().to(gpu)
+    scale = torch.full((8, 1), 0.01, dtype=torch.bfloat16, device=gpu)
+    assert quantize_sparse24_compress(w, scale, args) is None
+    w = torch.randn(8, 32).bfloat16().to(gpu)
+    assert quantize_sparse24_compress(w, scale, args, g_idx=torch.zeros(32, dtype=torch.int32, device=gpu)) is None
+    assert quantize_sparse24_compress(w, scale, args) is not None
