@@ -924,9 +924,9 @@ sparse24_compress_kernel(const R* __restrict__ x, R* __restrict__ values,
 // ModelCompressor.compress does to a weight that is both quantized (float- / int- /
 // naive-quantized, naive_quantized.py:79-114) and 2:4 sparse (sparse_24_bitmask.py:
 // 162-203), without the dense code tensor in between: 2 + 1/2 + 1/8 bytes per element
-// instead of 3 + 1 5/8.  A lane quantizes 16 neighbouring elements (two vectors of 8,
-// each with its scale: rows are multiples of 16 elements) and keeps 2 of every 4 codes
-// by the rule of get_24_bytemasks on the codes' int8 view.
+// instead of 3 + 1 5/8.  A lane quantizes 8 neighbouring elements (one 16-byte load,
+// one scale: rows are multiples of 8 elements) and keeps 2 of every 4 codes by the rule
+// of get_24_bytemasks on the codes' int8 view.
 template <typename FT, int QK, bool HAS_ZP>
 __global__ void __launch_bounds__(kBlock)
 quant_sparse24_compress_kernel(const typename FT::raw* __restrict__ x,
@@ -935,40 +935,31 @@ quant_sparse24_compress_kernel(const typename FT::raw* __restrict__ x,
                                uint8_t* __restrict__ bitmask, int64_t nitems, VecGeom g, float qmin,
                                float qmax) {
   using FR = typename FT::raw;
-  constexpr int U = 2;
+  constexpr int U = 4;
   constexpr int kOut = QK == 0 ? kKindI8 : kKindF8;
   const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
-  Vec<FR, 8> a[U][2];
-  FR sraw[U][2];
-  uint8_t zraw[U][2];
+  Vec<FR, 8> a[U];
+  FR sraw[U];
+  uint8_t zraw[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int64_t i = i0 + k * kBlock;
     const int64_t at = i < nitems ? i : nitems - 1;  // past the end: re-read, not stored
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const uint32_t si = scale_index((uint32_t)(at * 2 + h), g);
-      a[k][h] = ldg_nt<FR, 8>(x + (at * 2 + h) * 8);
-      sraw[k][h] = scale[si];
-      if constexpr (HAS_ZP) zraw[k][h] = zp[si];
-    }
+    const uint32_t si = scale_index((uint32_t)at, g);
+    a[k] = ldg_nt<FR, 8>(x + at * 8);
+    sraw[k] = scale[si];
+    if constexpr (HAS_ZP) zraw[k] = zp[si];
   }
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int64_t i = i0 + k * kBlock;
-    Vec<uint8_t, 16> q;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      Vec<FR, 8> unused_f;
-      Vec<uint8_t, 8> codes, unused_c;
-      float z = 0.0f;  // the zero point as the reference adds it (zero_point.to(x.dtype))
-      if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw[k][h] : f8e4m3_to_f32(zraw[k][h]);
-      qdq_vec8<FT, kKindFloat, kOut, QK, HAS_ZP>(a[k][h], unused_c, FT::to_f32(sraw[k][h]), z, qmin,
-                                                 qmax, &unused_f, &codes);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) q.v[8 * h + j] = codes.v[j];
-    }
-    store_survivors24<uint8_t, CTMI_I8, 16>(q, values, bitmask, i, i < nitems);
+    Vec<FR, 8> unused_f;
+    Vec<uint8_t, 8> codes, unused_c;
+    float z = 0.0f;  // the zero point as the reference adds it (zero_point.to(x.dtype))
+    if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw[k] : f8e4m3_to_f32(zraw[k]);
+    qdq_vec8<FT, kKindFloat, kOut, QK, HAS_ZP>(a[k], unused_c, FT::to_f32(sraw[k]), z, qmin, qmax,
+                                               &unused_f, &codes);
+    store_survivors24<uint8_t, CTMI_I8, 8>(codes, values, bitmask, i, i < nitems);
   }
 }
 
@@ -1345,7 +1336,7 @@ extern "C" int ctmi_sparse24_compress(const void* x, int32_t x_dtype, void* valu
 
 extern "C" int ctmi_quantize_sparse24_compress_supported(int32_t x_dtype, int64_t rows, int64_t cols,
                                                          const ctmi_qparams* qp) {
-  if (!qp || rows < 1 || cols < 1 || cols % 16) return 0;
+  if (!qp || rows < 1 || cols < 1 || cols % 8) return 0;
   if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16 && x_dtype != CTMI_F32) return 0;
   if (qp->scale_dtype != x_dtype || qp->global_scale || qp->col_group) return 0;
   if (qp->zero_point &&
@@ -1369,16 +1360,15 @@ extern "C" int ctmi_quantize_sparse24_compress(const void* x, int32_t x_dtype, v
                CTMI_ERR_UNSUPPORTED,
                "no fused kernel for this layout: quantize, then compress the codes");
   CTMI_REQUIRE(x && values && bitmask, CTMI_ERR_VALUE, "NULL tensor pointer");
-  CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)values % 8 == 0 &&
-                   (uintptr_t)bitmask % 2 == 0,
+  CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)values % 4 == 0,
                CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
   VecGeom g;
   vec_geometry(qp, rows, cols, &g);
   float qmin, qmax;
   rc = quant_range(qp->qtype, qp->num_bits, &qmin, &qmax);
   if (rc) return rc;
-  const int64_t items = rows * cols / 16;
-  const unsigned grid = (unsigned)cdiv(items, kBlock * 2);
+  const int64_t items = rows * cols / 8;
+  const unsigned grid = (unsigned)cdiv(items, kBlock * 4);
   hipStream_t st = (hipStream_t)stream;
   const uint8_t* zp = (const uint8_t*)qp->zero_point;
 #define CTMI_QS24_K(FT, RAW, QK, HZ)                                                             \

@@ -253,7 +253,7 @@ int ctmi_sparse24_compress(const void* x, int32_t x_dtype, void* values, uint8_t
  * as 2:4 (sparse_24_bitmask.py:162-203), without the dense code tensor in between.
  * values: [rows, cols / 2] codes (float8_e4m3fn or int8); bitmask as in
  * ctmi_sparse24_compress.  Same bits as ctmi_qdq followed by ctmi_sparse24_compress.
- * _supported(): cols % 16 == 0, scales in x's dtype on a tensor / channel / group
+ * _supported(): cols % 8 == 0, scales in x's dtype on a tensor / channel / group
  * grid, zero point (if any) in the codes' dtype, codes of 8 bits or fewer. */
 int ctmi_quantize_sparse24_compress_supported(int32_t x_dtype, int64_t rows, int64_t cols,
                                               const ctmi_qparams* qp);

@@ -357,6 +357,7 @@ QS24 = [
     (dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (64, 512), torch.bfloat16),
     (dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (33, 4112), torch.float16),
     (dict(num_bits=8, type="float", symmetric=True, strategy="tensor"), (16, 64), torch.bfloat16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (19, 24), torch.bfloat16),
     (dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=128), (24, 1024), torch.bfloat16),
     (dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (40, 256), torch.bfloat16),
     (dict(num_bits=8, type="int", symmetric=False, strategy="channel"), (40, 256), torch.float32),
@@ -391,14 +392,14 @@ def test_quantization_and_2_4_compression_in_one_pass(spec, shape, dtype, gpu):
 
 
 def test_quantization_and_2_4_without_a_fused_kernel(gpu):
-    """rows that are not whole 16-element items, an act-order g_idx: None, and the caller takes
+    """rows that are not whole 8-element items, an act-order g_idx: None, and the caller takes
     the two steps"""
     from compressed_tensors_amd.compressors import quantize_sparse24_compress
     from compressed_tensors_amd.quantization import QuantizationArgs
 
     announce("quantize + 2:4, unsupported")
     args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
-    w = torch.randn(8, 24).bfloat16().to(gpu)
+    w = torch.randn(8, 12).bfloat16().to(gpu)
     scale = torch.full((8, 1), 0.01, dtype=torch.bfloat16, device=gpu)
     assert quantize_sparse24_compress(w, scale, args) is None
     w = torch.randn(8, 32).bfloat16().to(gpu)
