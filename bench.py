@@ -462,6 +462,82 @@ def other_workload(torch, name, seed):
     raise SystemExit(f"unknown workload {name}")
 
 
+def cpu_baseline_other(torch, workload, seed):
+    """the oracle's restatement of one representative operation pair of the workload, timed on
+    this host's cores on a bounded sample (same definition of algorithmic bytes as the GPU line)"""
+    from oracle import hadamard as ohad
+    from oracle import pack as opack
+    from oracle import quant as oquant
+    from oracle import sparse as osparse
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(seed)
+    if workload == "fp8-w8a8":
+        spec = dict(num_bits=8, type="float", symmetric=True, strategy="channel")
+        oargs = oquant._Args(**spec)
+        w = (torch.randn(4096, 4096, generator=g) * 0.02).bfloat16()
+        s, z = oquant.observe_weight(w, oargs)
+        nbytes, what = 6 * w.numel(), "fp8 per-channel quantize + dequantize of a 4096x4096 bf16 weight"
+
+        def run():
+            codes = opack.naive_compress(w, s, oargs, zero_point=z)
+            opack.naive_decompress({"weight": codes, "weight_scale": s})
+    elif workload == "sparse":
+        w = (torch.randn(4096, 4096, generator=g) * 0.02).bfloat16()
+        w[torch.rand(4096, 4096, generator=g) < 0.5] = 0
+        nnz = int((w != 0).sum())
+        nbytes = 2 * (2 * w.numel() + w.numel() // 8 + 2 * nnz) + 8 * 4096
+        what = "sparse-bitmask compress + decompress of a 4096x4096 bf16 tensor, half zeros"
+
+        def run():
+            values, bitmask, _ = osparse.bitmask_compress(w)
+            osparse.bitmask_decompress(values, bitmask, list(w.shape))
+    elif workload == "nvfp4":
+        spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+        oargs = oquant._Args(**spec)
+        w = (torch.randn(2048, 4096, generator=g) * 0.02).bfloat16()
+        gs = oquant.generate_gparam(*[t.reshape(1) for t in torch.aminmax(w)])
+        s, z = oquant.observe_weight(w, oargs, global_scale=gs)
+        n = w.numel()
+        nbytes, what = 2 * (2 * n + n // 16 + n // 2), "nvfp4 compress + decompress of a 2048x4096 bf16 weight"
+
+        def run():
+            packed = opack.nvfp4_compress(w, s, gs, oargs)
+            opack.nvfp4_decompress(packed, s, gs)
+    elif workload == "hadamard":
+        x = torch.randn(2048, 4096, generator=g).bfloat16()
+        q = (torch.randint(0, 2, (128,), generator=g) * 2 - 1).double()
+        weight = q[:, None] * ohad.deterministic_hadamard_matrix(128, torch.float64)
+        nbytes, what = 4 * x.numel(), "random-sign Hadamard of size 128 on a 2048x4096 bf16 activation (fp64 matmul, as the reference's offline precision)"
+
+        def run():
+            ohad.hadamard_forward(weight, x, "input")
+    elif workload == "one-shot":
+        spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
+        oargs = oquant._Args(**spec)
+        w = (torch.randn(4096, 4096, generator=g) * 0.02).bfloat16()
+        n = w.numel()
+        nbytes, what = 2 * n + 2 * n // GROUP + n // 2, "observer + qparams + quantize + pack of a 4096x4096 bf16 weight (W4A16 g128)"
+
+        def run():
+            s, z = oquant.observe_weight(w, oargs)
+            opack.pack_quantized_compress(w, s, oargs, zero_point=z)
+    else:
+        return None
+    times = []
+    for it in range(4):
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        if it:
+            times.append(dt)
+    med = statistics.median(times)
+    return {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": what + f", median of 3 after 1 warm-up, torch {torch.__version__} CPU",
+            "seconds": med}
+
+
 def run_other(torch, a):
     metric, ops, keep = other_workload(torch, a.workload, a.seed)
     step_s = time_ops(torch, ops, a.steps, a.warmup)
@@ -490,6 +566,12 @@ def run_other(torch, a):
                         "ms": op.ms, "algorithmic_bytes": op.nbytes} for op in ops],
         "ms_per_step_gpu": gpu_ms,
     }
+    if not a.no_cpu_baseline:
+        del keep, ops
+        torch.cuda.empty_cache()
+        base = cpu_baseline_other(torch, a.workload, a.seed)
+        if base is not None:
+            out["cpu_baseline"] = base
     print(json.dumps(out))
 
 
