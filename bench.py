@@ -220,6 +220,14 @@ def other_workload(torch, name, seed):
             oa = (w.data_ptr(), code(w.dtype), codes.data_ptr(), r, c, c, 1, 8, 1, sc.data_ptr(), code(sc.dtype),
                   None, code(FP8), st)
             w_one.append(lambda oa=oa: _lib.check(lib.ctmi_observe_quantize(*oa)))
+        oq_jobs = (_lib.ObserveQuantizeJob * len(entries))()
+        for job, e, codes in zip(oq_jobs, entries, batch.codes):
+            w, sc = e["weight"], e["scale"]
+            job.x, job.codes, job.scale, job.zero_point = w.data_ptr(), codes.data_ptr(), sc.data_ptr(), None
+            job.rows, job.cols, job.blk_cols, job.x_dtype = w.shape[0], w.shape[1], w.shape[1], code(w.dtype)
+        keep.append(oq_jobs)
+        om = (oq_jobs, len(entries), 1, 8, 1, -1, code(FP8), st)
+        w_many = [lambda om=om: _lib.check(lib.ctmi_observe_quantize_many(*om))]
         acts, a_obs, a_fq, a_dyn = [], [], [], []
         targs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="token",
                                  dynamic=True)
@@ -238,7 +246,8 @@ def other_workload(torch, name, seed):
                Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_kernel"),
                Op("weights one-shot: per-channel observer (224 calls)", w_obs, 2 * n, "observe_wide_kernel", primary=False),
                Op("weights one-shot: quantize with those scales (224 calls)", w_q, 3 * n, "qdq_vec_kernel", primary=False),
-               Op("weights one-shot: scales + fp8 codes in one pass (224 calls)", w_one, 3 * n, "dynamic_rows_kernel"),
+               Op("weights one-shot: scales + fp8 codes in one pass (224 calls)", w_one, 3 * n, "dynamic_rows_kernel", primary=False),
+               Op("weights one-shot: scales + fp8 codes in one pass, one call (8 per launch)", w_many, 3 * n, "dynamic_rows_many_kernel"),
                Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
                Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel"),
                Op("activations: scales + fake-quantize in one pass (8 x 8192x4096)", a_dyn, 4 * na, "dynamic_rows_kernel")]

@@ -20,6 +20,7 @@ from compressed_tensors_amd.quantization.quant_args import QuantizationArgs
 
 __all__ = [
     "QuantizedWeightBatch",
+    "observe_and_compress_weights",
     "NaiveQuantizationCompressor",
     "IntQuantizationCompressor",
     "FloatQuantizationCompressor",
@@ -73,6 +74,60 @@ class QuantizedWeightBatch:
         """enqueue the dequantization of every code tensor; returns the dense tensors"""
         _lib.check(_lib.load().ctmi_qdq_many(self._djobs, self.n, 0, 1, _lib.stream_of(self.device)))
         return self.dense
+
+
+def observe_and_compress_weights(weights, quantization_args: QuantizationArgs):
+    """observe_and_compress_weight for a list of 2-D weights that have no scales yet, from
+    one call (ctmi_observe_quantize_many: rows of one length class share launches, eight
+    weights at a time).  Returns one dict per weight; weights without a fused kernel take
+    the single-weight path."""
+    from compressed_tensors_amd.quantization.helpers import _zp_dtype
+    from compressed_tensors_amd.quantization.quant_args import QuantizationStrategy
+
+    args = quantization_args
+    lib = _lib.load()
+    qtype = _lib.QTYPE_INT if args.type == "int" else _lib.QTYPE_FLOAT
+    results = [None] * len(weights)
+    batch = []
+    for i, weight in enumerate(weights):
+        w = to_gpu(weight)
+        blk_cols = 0
+        if w.ndim == 2:
+            if args.strategy == QuantizationStrategy.GROUP.value:
+                blk_cols = args.group_size
+            elif args.strategy == QuantizationStrategy.CHANNEL.value:
+                blk_cols = w.shape[1]
+        w = w.contiguous()
+        fused = (
+            blk_cols > 0 and w.numel() > 0 and can_quantize(w, args)
+            and w.data_ptr() % (8 * w.element_size()) == 0
+            and lib.ctmi_observe_quantize_supported(_lib.dtype_code(w.dtype), w.shape[0], w.shape[1],
+                                                    blk_cols, qtype, args.num_bits)
+        )
+        if not fused:
+            comp = BaseCompressor.load_from_registry(CompressionFormat.naive_quantized.value)
+            results[i] = comp.observe_and_compress_weight(weight, args)
+            continue
+        rows, cols = w.shape
+        n_cells = cols // min(blk_cols, cols)
+        out = {"weight": torch.empty((rows, cols), dtype=args.pytorch_dtype(), device=w.device),
+               "weight_scale": torch.empty((rows, n_cells), dtype=w.dtype, device=w.device)}
+        if not args.symmetric:
+            out["weight_zero_point"] = torch.empty((rows, n_cells), dtype=_zp_dtype(args), device=w.device)
+        results[i] = out
+        batch.append((w, out, blk_cols))
+    if batch:
+        jobs = (_lib.ObserveQuantizeJob * len(batch))()
+        for job, (w, out, blk_cols) in zip(jobs, batch):
+            job.x, job.codes, job.scale = w.data_ptr(), out["weight"].data_ptr(), out["weight_scale"].data_ptr()
+            job.zero_point = _lib.ptr(out.get("weight_zero_point"))
+            job.rows, job.cols, job.blk_cols = w.shape[0], w.shape[1], blk_cols
+            job.x_dtype = _lib.dtype_code(w.dtype)
+        dev = batch[0][0].device
+        _lib.check(lib.ctmi_observe_quantize_many(
+            jobs, len(batch), qtype, args.num_bits, int(args.symmetric), -1,
+            _lib.dtype_code(_zp_dtype(args)), _lib.stream_of(dev)))
+    return results
 
 
 @BaseCompressor.register(name=CompressionFormat.naive_quantized.value)

@@ -82,13 +82,12 @@ __device__ __forceinline__ void store_result(void* out_any, int64_t v, bool keep
 // 256 * U vectors of 8 elements: every vector is loaded before anything is looked
 // at; the four wavefronts meet once, over a few words in LDS.
 template <typename FT, int QK, bool SYM, int U, bool CODES>
-__global__ void __launch_bounds__(256)
-dynamic_rows_kernel(const typename FT::raw* __restrict__ x, void* __restrict__ out_any,
-                    DynOut o, int items, QpCfg c) {
+__device__ __forceinline__ void rows_segment(const typename FT::raw* __restrict__ x,
+                                             void* __restrict__ out_any, const DynOut& o, int items,
+                                             int64_t s, const QpCfg& c) {
   using FR = typename FT::raw;
   __shared__ float part_lo[4], part_hi[4];
   __shared__ int part_word[4];
-  const int64_t s = blockIdx.x;
   const FR* p = x + s * (int64_t)items * 8;
   Vec<FR, 8> a[U];
 #pragma unroll
@@ -137,6 +136,39 @@ dynamic_rows_kernel(const typename FT::raw* __restrict__ x, void* __restrict__ o
     const int i = k * 256 + threadIdx.x;
     store_result<FT, QK, CODES>(out_any, s * (int64_t)items + i, i < items, a[k], sv, zv, c);
   }
+}
+
+template <typename FT, int QK, bool SYM, int U, bool CODES>
+__global__ void __launch_bounds__(256)
+dynamic_rows_kernel(const typename FT::raw* __restrict__ x, void* __restrict__ out_any,
+                    DynOut o, int items, QpCfg c) {
+  rows_segment<FT, QK, SYM, U, CODES>(x, out_any, o, items, blockIdx.x, c);
+}
+
+// The same for up to kDynMaxJobs tensors per launch: a workgroup finds its tensor by the
+// running totals of segments (all wave-uniform).
+constexpr int kDynMaxJobs = 8;
+struct DynJobs {
+  const void* x[kDynMaxJobs];
+  void* out[kDynMaxJobs];
+  DynOut o[kDynMaxJobs];
+  int64_t end[kDynMaxJobs];  // running total of segments, job 0 .. j (unused: INT64_MAX)
+  int items[kDynMaxJobs];
+};
+
+template <typename FT, int QK, bool SYM, int U, bool CODES>
+__global__ void __launch_bounds__(256) dynamic_rows_many_kernel(DynJobs t, QpCfg c) {
+  const int64_t s = blockIdx.x;
+  int j = 0;
+  int64_t first = 0;
+#pragma unroll
+  for (int i = 0; i < kDynMaxJobs - 1; ++i) {
+    const bool past = s >= t.end[i];
+    j = past ? i + 1 : j;
+    first = past ? t.end[i] : first;
+  }
+  rows_segment<FT, QK, SYM, U, CODES>(static_cast<const typename FT::raw*>(t.x[j]), t.out[j], t.o[j],
+                                      t.items[j], s - first, c);
 }
 
 // Segments of L vectors, L a power of two <= 64 (group strategies): L neighbouring
@@ -296,4 +328,118 @@ extern "C" int ctmi_observe_quantize(const void* x, int32_t x_dtype, void* codes
 #undef CTMI_OQ_FT
   CTMI_REQUIRE(ok, CTMI_ERR_UNSUPPORTED, "no fused kernel for this layout");
   return check_launch("ctmi_observe_quantize");
+}
+
+// rows-per-workgroup class of a job (0: not a row-kernel layout)
+static int rows_class(int64_t cols, int64_t blk_cols) {
+  const int64_t seg = blk_cols < cols ? blk_cols : cols;
+  if (seg % 8 || cols % seg) return 0;
+  const int64_t items = seg / 8;
+  if (items <= 64 && (items & (items - 1)) == 0) return 0;  // the flat kernel's layouts
+  if (items <= 256) return 1;
+  if (items <= 512) return 2;
+  if (items <= 1024) return 4;
+  if (items <= 2048) return 8;
+  return 0;
+}
+
+template <typename FT, int QK, bool SYM>
+static void launch_rows_many(const DynJobs& t, int filled, int u, const QpCfg& c, hipStream_t st) {
+  const unsigned grid = (unsigned)t.end[filled - 1];
+#define CTMI_DM(UU) \
+  hipLaunchKernelGGL((dynamic_rows_many_kernel<FT, QK, SYM, UU, true>), grid, 256, 0, st, t, c)
+  if (u == 1) CTMI_DM(1);
+  else if (u == 2) CTMI_DM(2);
+  else if (u == 4) CTMI_DM(4);
+  else CTMI_DM(8);
+#undef CTMI_DM
+}
+
+extern "C" int ctmi_observe_quantize_many(const ctmi_observe_quantize_job* jobs, int64_t n,
+                                          int32_t qtype, int32_t num_bits, int32_t symmetric,
+                                          int32_t scale_dtype, int32_t zp_dtype, void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  // validate everything before anything is enqueued
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_observe_quantize_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 1 && j.cols >= 1 && j.blk_cols >= 1, CTMI_ERR_VALUE,
+                 "job %lld: cannot observe an empty tensor", (long long)i);
+    QpCfg c;
+    int rc = fill_qpcfg(&c, qtype, num_bits, symmetric, j.x_dtype, 0, false,
+                        scale_dtype < 0 ? j.x_dtype : scale_dtype, zp_dtype);
+    if (rc) return rc;
+    CTMI_REQUIRE(j.x && j.codes && j.scale, CTMI_ERR_VALUE, "job %lld: NULL tensor pointer", (long long)i);
+    CTMI_REQUIRE(ctmi_observe_quantize_supported(j.x_dtype, j.rows, j.cols, j.blk_cols, qtype, num_bits),
+                 CTMI_ERR_UNSUPPORTED,
+                 "job %lld: no fused kernel for this layout: compute the scales and quantize separately",
+                 (long long)i);
+    CTMI_REQUIRE((uintptr_t)j.x % (8 * dtype_size(j.x_dtype)) == 0 && (uintptr_t)j.codes % 8 == 0,
+                 CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const int qk = qtype == CTMI_QTYPE_INT ? 0 : 1;
+  // rows of one length class and dtype share launches, kDynMaxJobs tensors at a time
+  const int dts[3] = {CTMI_BF16, CTMI_F16, CTMI_F32};
+  const int classes[4] = {1, 2, 4, 8};
+  for (int d = 0; d < 3; ++d) {
+    QpCfg c;
+    fill_qpcfg(&c, qtype, num_bits, symmetric, dts[d], 0, false,
+               scale_dtype < 0 ? dts[d] : scale_dtype, zp_dtype);
+    for (int k = 0; k < 4; ++k) {
+      DynJobs t;
+      int filled = 0;
+      auto reset = [&]() {
+        filled = 0;
+        for (int q = 0; q < kDynMaxJobs; ++q) {
+          t.x[q] = nullptr;
+          t.out[q] = nullptr;
+          t.o[q] = DynOut{nullptr, nullptr};
+          t.end[q] = INT64_MAX;
+          t.items[q] = 1;
+        }
+      };
+      auto flush = [&]() {
+        if (!filled) return;
+#define CTMI_DM_SYM(FT, QK)                                                  \
+  (symmetric ? launch_rows_many<FT, QK, true>(t, filled, classes[k], c, st)  \
+             : launch_rows_many<FT, QK, false>(t, filled, classes[k], c, st))
+#define CTMI_DM_FT(FT) (qk == 0 ? CTMI_DM_SYM(FT, 0) : CTMI_DM_SYM(FT, 1))
+        if (dts[d] == CTMI_BF16) CTMI_DM_FT(BF16);
+        else if (dts[d] == CTMI_F16) CTMI_DM_FT(F16);
+        else CTMI_DM_FT(F32);
+#undef CTMI_DM_SYM
+#undef CTMI_DM_FT
+        reset();
+      };
+      reset();
+      for (int64_t i = 0; i < n; ++i) {
+        const ctmi_observe_quantize_job& j = jobs[i];
+        if (j.x_dtype != dts[d] || rows_class(j.cols, j.blk_cols) != classes[k]) continue;
+        const int64_t seg = j.blk_cols < j.cols ? j.blk_cols : j.cols;
+        const int64_t segments = j.rows * (j.cols / seg);
+        const int64_t before = filled ? t.end[filled - 1] : 0;
+        if (filled == kDynMaxJobs || before + segments >= (1ll << 31)) flush();
+        if (segments >= (1ll << 31)) continue;  // taken by the single call below
+        t.x[filled] = j.x;
+        t.out[filled] = j.codes;
+        t.o[filled] = DynOut{j.scale, j.zero_point};
+        t.items[filled] = (int)(seg / 8);
+        t.end[filled] = (filled ? t.end[filled - 1] : 0) + segments;
+        ++filled;
+      }
+      flush();
+    }
+  }
+  int rc = check_launch("ctmi_observe_quantize_many");
+  if (rc) return rc;
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_observe_quantize_job& j = jobs[i];
+    const int64_t seg = j.blk_cols < j.cols ? j.blk_cols : j.cols;
+    if (rows_class(j.cols, j.blk_cols) != 0 && j.rows * (j.cols / seg) < (1ll << 31)) continue;
+    rc = ctmi_observe_quantize(j.x, j.x_dtype, j.codes, j.rows, j.cols, j.blk_cols, qtype, num_bits,
+                               symmetric, j.scale, scale_dtype < 0 ? j.x_dtype : scale_dtype,
+                               j.zero_point, zp_dtype, stream);
+    if (rc) return rc;
+  }
+  return CTMI_OK;
 }

@@ -372,6 +372,20 @@ int ctmi_observe_quantize(const void* x, int32_t x_dtype, void* codes, int64_t r
                           void* scale_out, int32_t scale_dtype, void* zp_out, int32_t zp_dtype,
                           void* stream);
 
+/* every weight of a state dict in one call: rows of one length class share launches,
+ * eight weights at a time; scale_dtype < 0: every weight's scales in its own dtype */
+typedef struct ctmi_observe_quantize_job {
+  const void* x;
+  void* codes;
+  void* scale;
+  void* zero_point; /* optional */
+  int64_t rows, cols, blk_cols;
+  int32_t x_dtype, reserved;
+} ctmi_observe_quantize_job;
+int ctmi_observe_quantize_many(const ctmi_observe_quantize_job* jobs, int64_t n, int32_t qtype,
+                               int32_t num_bits, int32_t symmetric, int32_t scale_dtype,
+                               int32_t zp_dtype, void* stream);
+
 /* MXFP4 group scales (quantization/utils/mxfp4_utils.py): powers of two held as
  * uint8 exponents.  x / out of the first two are bfloat16 group maxima, n values.
  *   ctmi_mxfp4_round_to_power_2   :41-73  (x + 32) & 0xFF80 on the bf16 bits

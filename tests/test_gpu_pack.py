@@ -682,3 +682,29 @@ def test_naive_observe_and_compress_in_one_pass(fmt, spec, shape, dtype, gpu):
         assert_bit_equal(got["weight_zero_point"], zp, "zero point")
     assert_bit_equal(got["weight"], want, "codes")
     assert got["weight"].dtype == args.pytorch_dtype()
+
+
+def test_naive_observe_and_compress_many_weights(gpu):
+    """observe_and_compress_weights == observe_and_compress_weight weight by weight: more
+    weights than a launch takes, rows of every length class, two dtypes, a weight whose
+    rows have no fused kernel"""
+    from compressed_tensors_amd.compressors import BaseCompressor, observe_and_compress_weights
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    announce("one-shot fp8, many weights")
+    shapes = [(64, 512, torch.bfloat16), (8, 4096, torch.bfloat16), (40, 14336, torch.bfloat16), (33, 2048, torch.float16),
+              (16, 1032, torch.bfloat16), (5, 8192, torch.bfloat16), (128, 512, torch.bfloat16), (7, 4104, torch.float16),
+              (96, 1024, torch.bfloat16), (3, 16392, torch.bfloat16), (24, 768, torch.bfloat16), (12, 3072, torch.bfloat16)]
+    g = torch.Generator().manual_seed(91)
+    ws = [(torch.randn(r, c, generator=g) * 0.02).to(dt).to(gpu) for r, c, dt in shapes]
+    for spec in (dict(num_bits=8, type="float", symmetric=True, strategy="channel"),
+                 dict(num_bits=8, type="int", symmetric=False, strategy="channel")):
+        args = QuantizationArgs(**spec)
+        comp = BaseCompressor.load_from_registry("naive-quantized")
+        got = observe_and_compress_weights(ws, args)
+        assert len(got) == len(ws)
+        for i, (w, out) in enumerate(zip(ws, got)):
+            want = comp.observe_and_compress_weight(w, args)
+            assert set(out) == set(want)
+            for key in want:
+                assert_bit_equal(out[key], want[key], f"weight {i} {key}")
