@@ -428,7 +428,8 @@ def other_workload(torch, name, seed):
                     calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
                 nb = sum(4 * x.numel() for x in xs)
                 ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb,
-                              "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel"))
+                              "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
+                              primary=not label.startswith("weights 4096x4096")))
                 if label.startswith("weights 4096x4096"):
                     jobs = (_lib.HadamardJob * len(xs))()
                     outs = [torch.empty_like(x) for x in xs]
@@ -455,7 +456,7 @@ def other_workload(torch, name, seed):
                 calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_quant_pack(*a)))
             nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in tensors[label])
             ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}", calls, nb,
-                          "hadamard_quant_pack_kernel"))
+                          "hadamard_quant_pack_kernel", primary=not label.startswith("weights 4096x4096")))
             if label.startswith("weights 4096x4096"):
                 xs = tensors[label]
                 jobs = (_lib.HadamardPackJob * len(xs))()
