@@ -149,7 +149,7 @@ def test_transform_algebra_on_gpu(gpu):
 
 
 def test_large_activation_properties(gpu):
-    """BASELINE-sized: 8192 x 4096 bf16 activations, block 128 and full 4096: sampled
+    """full-size: 8192 x 4096 bf16 activations, block 128 and full 4096: sampled
     rows against fp64, and an involution check (H H^T / n = I) on the whole tensor"""
     from compressed_tensors_amd.transform import hadamard_apply
 

@@ -316,7 +316,7 @@ def test_attn_head_and_errors(gpu):
 
 
 def test_large_w4a16_properties(gpu):
-    """BASELINE-sized weight: sampled-row parity plus size-independent properties"""
+    """full-size weight (4096 x 14336): sampled-row parity plus size-independent properties"""
     from compressed_tensors_amd.quantization import (
         QuantizationArgs, dequantize, observe_weight_qparams, quantize,
     )
@@ -375,7 +375,7 @@ def test_fp8_codes_on_every_bf16_pattern(gpu):
 
 
 def test_large_fp8_channel_and_token(gpu):
-    """BASELINE-sized fp8 paths: per-channel weight codes and per-token activation QDQ,
+    """full-size fp8 paths: per-channel weight codes and per-token activation QDQ,
     sampled rows against the oracle"""
     from compressed_tensors_amd.quantization import (
         QuantizationArgs, compute_dynamic_scales_and_zp, dequantize, fake_quantize,

@@ -162,7 +162,7 @@ def test_sparse24_errors(gpu):
 
 
 def test_large_bitmask_roundtrip_properties(gpu):
-    """BASELINE-sized (8192 x 8192, 50 % magnitude pruned): sampled parity and a lossless round trip"""
+    """full-size (8192 x 8192, 50 % magnitude pruned): sampled parity and a lossless round trip"""
     from compressed_tensors_amd.compressors import bitmask_compress, bitmask_decompress
 
     announce("large bitmask")
