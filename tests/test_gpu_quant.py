@@ -316,7 +316,7 @@ def test_attn_head_and_errors(gpu):
 
 
 def test_large_w4a16_properties(gpu):
-    """full-size weight (4096 x 14336): sampled-row parity plus size-independent properties"""
+    """full-size weight (4096 x 4096): sampled-row parity plus size-independent properties"""
     from compressed_tensors_amd.quantization import (
         QuantizationArgs, dequantize, observe_weight_qparams, quantize,
     )
