@@ -359,6 +359,7 @@ extern "C" int ctmi_observe_quantize_many(const ctmi_observe_quantize_job* jobs,
                                           int32_t qtype, int32_t num_bits, int32_t symmetric,
                                           int32_t scale_dtype, int32_t zp_dtype, void* stream) {
   CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  if (n == 0) return CTMI_OK;
   // validate everything before anything is enqueued
   for (int64_t i = 0; i < n; ++i) {
     const ctmi_observe_quantize_job& j = jobs[i];

@@ -793,6 +793,7 @@ static bool fp4_chainable(const ctmi_weight_job& j, bool compress, VecGeom* g) {
 static int fp4_many(const ctmi_weight_job* jobs, int64_t n, bool compress, void* stream,
                     const char* what) {
   CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  if (n == 0) return CTMI_OK;
   hipStream_t st = (hipStream_t)stream;
   constexpr uint32_t per = kFp4Block * kFp4Unroll;
   // validate everything before anything is enqueued

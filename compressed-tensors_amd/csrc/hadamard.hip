@@ -946,6 +946,7 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
                                         const void* ma_t, const void* mb_t, const float* sign_in,
                                         const float* sign_out, void* stream) {
   CTMI_REQUIRE(n_jobs >= 0 && (jobs || n_jobs == 0), CTMI_ERR_VALUE, "bad job list");
+  if (n_jobs == 0) return CTMI_OK;
   CTMI_REQUIRE(a_dim >= 1 && b_dim >= 1, CTMI_ERR_VALUE, "bad factor sizes");
   CTMI_REQUIRE(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32,
                CTMI_ERR_UNSUPPORTED, "transforms take float16/bfloat16/float32 tensors");
@@ -1003,6 +1004,9 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
       filled = 0;
     }
   }
+  bool any = false;
+  for (int64_t i = 0; i < n_jobs; ++i) any |= jobs[i].numel != 0;
+  if (!any) return CTMI_OK;
   if (filled) {
     int rc = launch_had_jobs(t, filled, io_dtype, a_dim, b_dim, a, st);
     if (rc) return rc;
@@ -1096,6 +1100,7 @@ extern "C" int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs,
   CTMI_REQUIRE(n_jobs >= 0 && (jobs || n_jobs == 0), CTMI_ERR_VALUE, "bad job list");
   int rc = hqp_check(io_dtype, b_dim, num_bits, symmetric);
   if (rc) return rc;
+  if (n_jobs == 0) return CTMI_OK;
   for (int64_t i = 0; i < n_jobs; ++i) {
     rc = hqp_check_job(jobs[i], b_dim);
     if (rc) return rc;
@@ -1121,6 +1126,9 @@ extern "C" int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs,
       filled = 0;
     }
   }
+  bool any = false;
+  for (int64_t i = 0; i < n_jobs; ++i) any |= jobs[i].numel != 0;
+  if (!any) return CTMI_OK;
   if (filled) hqp_launch(t, filled, b_dim, mb_t, sign_in, sign_out, num_bits, st);
   return check_launch("ctmi_hadamard_quant_pack_many");
 }

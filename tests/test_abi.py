@@ -98,6 +98,58 @@ def test_fp4_and_sparse_argument_errors(ctmi):
     assert "Asymmetric Quantization is not supported for FP4" in _err(ctmi)
 
 
+def test_one_pass_and_many_argument_errors(ctmi):
+    """entry points that take lists of tensors or fuse several steps: everything is checked on
+    the host, for every job, before anything could be enqueued"""
+    # scratch sizes grow with the tensor
+    assert ctmi.ctmi_bitmask_tmp_bytes(8192, 8192) > ctmi.ctmi_bitmask_tmp_bytes(8, 8) > 0
+    assert ctmi.ctmi_sparse24_tmp_bytes(14336, 4096, 1) >= ctmi.ctmi_bitmask_tmp_bytes(14336, 4096)
+    # nvfp4 lists: an odd column count in the second job stops the whole call
+    jobs = (_lib.WeightJob * 2)()
+    for j, cols in zip(jobs, (32, 31)):
+        j.src, j.dst, j.rows, j.cols, j.dense_dtype = 0x1000, 0x2000, 4, cols, _lib.BF16
+        j.qp = _qp(scale_dtype=_lib.F8E4M3, global_scale=0x3000, qtype=_lib.QTYPE_FLOAT, num_bits=4,
+                   s_rows=4, s_cols=2, blk_rows=1, blk_cols=16)
+    assert ctmi.ctmi_nvfp4_compress_many(jobs, 2, None) == _lib.CTMI_ERR_VALUE
+    assert ctmi.ctmi_nvfp4_compress_many(None, 0, None) == _lib.CTMI_OK
+    assert ctmi.ctmi_nvfp4_decompress_many(None, 3, None) == _lib.CTMI_ERR_VALUE
+    # Hadamard lists: sizes must be multiples of the transform size, factorisations built
+    hj = (_lib.HadamardJob * 2)()
+    hj[0].x, hj[0].out, hj[0].numel = 0x1000, 0x2000, 256
+    hj[1].x, hj[1].out, hj[1].numel = 0x1000, 0x2000, 200
+    rc = ctmi.ctmi_hadamard_apply_many(hj, 2, _lib.BF16, 1, 128, None, 0x3000, None, None, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "not a multiple of the transform size" in _err(ctmi)
+    rc = ctmi.ctmi_hadamard_apply_many(hj, 1, _lib.BF16, 3, 5, None, 0x3000, None, None, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED
+    assert ctmi.ctmi_hadamard_apply_many(None, 0, _lib.BF16, 1, 128, None, None, None, None, None) == _lib.CTMI_OK
+    pj = (_lib.HadamardPackJob * 1)()
+    pj[0].x, pj[0].packed, pj[0].scale, pj[0].numel = 0x1000, 0x2000, 0x3000, 256
+    rc = ctmi.ctmi_hadamard_quant_pack_many(pj, 1, _lib.F16, 128, 0x4000, None, None, 4, 1, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "bfloat16" in _err(ctmi)
+    rc = ctmi.ctmi_hadamard_quant_pack_many(pj, 1, _lib.BF16, 128, 0x4000, None, None, 8, 1, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "4-bit" in _err(ctmi)
+    # one-shot codes: layouts without a fused kernel say so
+    assert ctmi.ctmi_observe_quantize_supported(_lib.BF16, 64, 4096, 4096, _lib.QTYPE_FLOAT, 8) == 1
+    assert ctmi.ctmi_observe_quantize_supported(_lib.BF16, 64, 16392, 16392, _lib.QTYPE_FLOAT, 8) == 0
+    assert ctmi.ctmi_observe_quantize_supported(_lib.BF16, 64, 4096, 4096, _lib.QTYPE_FLOAT, 4) == 0
+    rc = ctmi.ctmi_observe_quantize(0x1000, _lib.BF16, 0x2000, 4, 100, 100, _lib.QTYPE_INT, 8, 1, 0x3000,
+                                    _lib.BF16, None, _lib.I8, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "separately" in _err(ctmi)
+    oj = (_lib.ObserveQuantizeJob * 1)()
+    oj[0].x, oj[0].codes, oj[0].scale = 0x1000, 0x2000, 0
+    oj[0].rows, oj[0].cols, oj[0].blk_cols, oj[0].x_dtype = 4, 4096, 4096, _lib.BF16
+    rc = ctmi.ctmi_observe_quantize_many(oj, 1, _lib.QTYPE_FLOAT, 8, 1, -1, _lib.F8E4M3, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "NULL tensor pointer" in _err(ctmi)
+    # quantization + 2:4: rows of whole bitmask bytes, scales in the tensor's dtype
+    qp = _qp(s_rows=4, s_cols=1, blk_rows=1, blk_cols=64, qtype=_lib.QTYPE_FLOAT, num_bits=8)
+    assert ctmi.ctmi_quantize_sparse24_compress_supported(_lib.BF16, 4, 64, ctypes.byref(qp)) == 1
+    assert ctmi.ctmi_quantize_sparse24_compress_supported(_lib.F16, 4, 64, ctypes.byref(qp)) == 0
+    qp = _qp(s_rows=4, s_cols=1, blk_rows=1, blk_cols=12, qtype=_lib.QTYPE_FLOAT, num_bits=8)
+    assert ctmi.ctmi_quantize_sparse24_compress_supported(_lib.BF16, 4, 12, ctypes.byref(qp)) == 0
+    rc = ctmi.ctmi_quantize_sparse24_compress(0x1000, _lib.BF16, 0x2000, 0x3000, 4, 12, ctypes.byref(qp), None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED
+
+
 def test_topk24_table_matches_installed_torch(ctmi):
     """the 2:4 keep table compiled into the library against torch.topk on every
     weak ordering of four keys"""
