@@ -256,6 +256,7 @@ def other_workload(torch, name, seed):
     if name == "sparse":
         copies = 6
         c_calls, d_calls, s_calls, t_calls, two_step, one_step = [], [], [], [], [], []
+        back_two, back_one = [], []
         nb = 8192 * 8192
         nnz_total = 0
         for _ in range(copies):
@@ -305,6 +306,15 @@ def other_workload(torch, name, seed):
             two_step.append(lambda qa=qa, a=a: (_lib.check(lib.ctmi_qdq(*qa)), _lib.check(lib.ctmi_sparse24_compress(*a))))
             one_step.append(lambda fa=fa: _lib.check(lib.ctmi_quantize_sparse24_compress(*fa)))
             t_calls.append(lambda d=d: _lib.check(lib.ctmi_sparse24_decompress(*d)))
+            # ... and the way back: 2:4 -> fp8 codes -> bf16
+            back = torch.empty_like(w)
+            tmp_dq = torch.empty(lib.ctmi_sparse24_dequantize_tmp_bytes(rows, cols), dtype=torch.uint8, device=dev)
+            keep.extend([back, tmp_dq])
+            dq = (dense.data_ptr(), code(dense.dtype), back.data_ptr(), code(back.dtype), rows, cols, ctypes.byref(plan.qp), 0, 1, st)
+            fd = (values.data_ptr(), values.numel(), code(FP8), bitmask.data_ptr(), back.data_ptr(), code(back.dtype),
+                  tmp_dq.data_ptr(), rows, cols, ctypes.byref(plan.qp), st)
+            back_two.append(lambda d=d, dq=dq: (_lib.check(lib.ctmi_sparse24_decompress(*d)), _lib.check(lib.ctmi_qdq(*dq))))
+            back_one.append(lambda fd=fd: _lib.check(lib.ctmi_sparse24_decompress_dequantize(*fd)))
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies * (n24 + n24 // 2 + n24 // 8)
         fused24_bytes = copies * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
@@ -313,7 +323,9 @@ def other_workload(torch, name, seed):
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
-               Op("bf16 -> fp8 codes -> 2:4 compress, one pass", one_step, fused24_bytes, "quant_sparse24_compress_kernel")]
+               Op("bf16 -> fp8 codes -> 2:4 compress, one pass", one_step, fused24_bytes, "quant_sparse24_compress_kernel"),
+               Op("2:4 decompress -> fp8 codes -> bf16, two steps", back_two, fused24_bytes, "qdq_vec_kernel", primary=False),
+               Op("2:4 decompress -> fp8 codes -> bf16, one pass", back_one, fused24_bytes, "sparse24_scatter_dequant_kernel")]
         return "sparse-bitmask / sparse-24-bitmask compress+decompress GB/s", ops, keep
 
     if name == "nvfp4":

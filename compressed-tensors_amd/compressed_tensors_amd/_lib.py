@@ -179,6 +179,14 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_int32, c_void_p, c_void_p, c_int64, c_int64, POINTER(QParams), c_void_p],
     ),
+    "ctmi_sparse24_decompress_dequantize_supported": (
+        c_int32, [c_int32, c_int32, c_int64, c_int64, POINTER(QParams)]),
+    "ctmi_sparse24_dequantize_tmp_bytes": (c_int64, [c_int64, c_int64]),
+    "ctmi_sparse24_decompress_dequantize": (
+        c_int32,
+        [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_int64,
+         POINTER(QParams), c_void_p],
+    ),
     "ctmi_bitmask_tmp_bytes": (c_int64, [c_int64, c_int64]),
     "ctmi_bitmask_count": (
         c_int32,

@@ -24,7 +24,7 @@ from compressed_tensors_amd.config import (
     SparsityCompressionConfig,
 )
 from compressed_tensors_amd.quantization.quant_scheme import QuantizationConfig, QuantizationScheme
-from compressed_tensors_amd.utils.helpers import load_safetensors_state_dict
+from compressed_tensors_amd.utils.helpers import load_safetensors_state_dict, nest_state_dict
 
 __all__ = ["ModelCompressor", "map_module_to_scheme", "match_named_modules",
            "apply_quantization_scheme"]
@@ -142,7 +142,10 @@ class ModelCompressor:
             state_dict.update(entries)
         return state_dict
 
-    def _compress_quantized_24(self, model: Module, state_dict: Dict[str, Tensor]) -> Dict[str, Dict[str, Tensor]]:
+    def _compress_quantized_24(self, model: Module, state_dict: Dict[str, Tensor],
+                               targets: Optional[Set[str]] = None,
+                               module_to_scheme: Optional[Dict[str, QuantizationScheme]] = None,
+                               ) -> Dict[str, Dict[str, Tensor]]:
         """Weights that get int8 / fp8 codes AND 2:4 compression (quantization first, then
         the sparse compressor on the codes, model_compressor.py:638-667): both from one pass
         over the dense weight where a fused kernel exists.  Returns, per dense weight name,
@@ -161,8 +164,10 @@ class ModelCompressor:
         structure = getattr(self.sparsity_compressor.config, "sparsity_structure", "2:4")
         if str(getattr(structure, "value", structure)) != "2:4":
             return {}
-        targets = self._sparse_targets(model)
-        module_to_scheme = map_module_to_scheme(model)
+        if targets is None:
+            targets = self._sparse_targets(model)
+        if module_to_scheme is None:
+            module_to_scheme = map_module_to_scheme(model)
         done = {}
         for name in list(state_dict.keys()):
             if not name.endswith(".weight") or name[: -len(".weight")] not in targets:
@@ -184,6 +189,35 @@ class ModelCompressor:
                                            bitmask=pair[1])
             done[name] = tensor.dict(name_prefix=name, device=self.sparsity_compressor.output_device)
         return done
+
+    def _decompress_quantized_24(self, prefix: str, state: Dict[str, Tensor],
+                                 quant_compressor) -> Optional[Dict[str, Tensor]]:
+        """The way back for one module whose entries are in `state` (full names): 2:4
+        decompression of the codes and their dequantization (sparsity first, quantization
+        second, model_compressor.py:572-604) from one pass where a fused kernel exists.
+        Returns what the two decompressors would have left, or None."""
+        from compressed_tensors_amd.compressors.naive_quantized import NaiveQuantizationCompressor
+        from compressed_tensors_amd.compressors.sparse_24_bitmask import (
+            Sparse24BitMaskCompressor, sparse24_decompress_dequantize,
+        )
+
+        if (not isinstance(self.sparsity_compressor, Sparse24BitMaskCompressor)
+                or not isinstance(quant_compressor, NaiveQuantizationCompressor)):
+            return None
+        names = [f"{prefix}.{n}" for n in self.sparsity_compressor.compression_param_names]
+        scale = state.get(f"{prefix}.weight_scale", None)
+        if scale is None or any(n not in state for n in names):
+            return None
+        if state.get(f"{prefix}.weight_global_scale", None) is not None:
+            return None
+        weight = sparse24_decompress_dequantize(
+            state[f"{prefix}.compressed"], state[f"{prefix}.bitmask"], state[f"{prefix}.shape"], scale,
+            zero_point=state.get(f"{prefix}.weight_zero_point", None),
+            g_idx=state.get(f"{prefix}.weight_g_idx", None))
+        if weight is None:
+            return None
+        rest = {k: v for k, v in state.items() if k not in names}
+        return {f"{prefix}.weight": weight, **rest}
 
     def decompress(self, model_path, model: Module) -> None:
         """overwrite the weights of `model` with the ones decompressed from a
@@ -209,6 +243,22 @@ class ModelCompressor:
                 return
             model_path = load_safetensors_state_dict(model_path, device=device)
         state = model_path
+        if has_sparsity and quant_compressor is not None:
+            # weights that are 2:4 compressed codes: both steps in one pass where possible
+            names_to_scheme = map_module_to_scheme(model)
+            for mod_path in nest_state_dict(state, self.sparsity_compressor.compression_param_names):
+                if mod_path not in names_to_scheme:
+                    continue
+                own = {k: v for k, v in state.items() if k.startswith(mod_path + ".")}
+                dense = self._decompress_quantized_24(mod_path, own, quant_compressor)
+                if dense is None:
+                    continue
+                module = self._module(model, mod_path)
+                for full_name, data in dense.items():
+                    param_name = full_name[len(mod_path) + 1:]
+                    if param_name == "weight" or hasattr(module, param_name):
+                        self._assign(model, full_name, data)
+                state = {k: v for k, v in state.items() if k not in own}
         if (self.sparsity_compressor is not None
                 and self.sparsity_config.format != CompressionFormat.dense.value):
             skip = quant_compressor.compression_param_names if quant_compressor else None
@@ -287,6 +337,10 @@ class ModelCompressor:
             if prefix not in module_to_scheme and prefix not in sparse_targets:
                 continue
             state = {f"{prefix}.{n}": p.data for n, p in module.named_parameters(recurse=False)}
+            stacked = {}
+            if prefix in module_to_scheme and prefix in sparse_targets:
+                stacked = self._compress_quantized_24(model, state, sparse_targets, module_to_scheme)
+                state = {k: v for k, v in state.items() if k not in stacked}
             if prefix in module_to_scheme:
                 compressor = self.quantization_compressor.get(self._format_of(module))
                 state = compressor.compress(state, names_to_scheme=module_to_scheme,
@@ -294,6 +348,8 @@ class ModelCompressor:
             if prefix in sparse_targets:
                 state = self.sparsity_compressor.compress(
                     state, compression_targets=sparse_targets, show_progress=False)
+            for entries in stacked.values():
+                state.update(entries)
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.COMPRESSED
         if (self.quantization_config is not None
@@ -307,12 +363,19 @@ class ModelCompressor:
             if prefix not in module_to_scheme and prefix not in sparse_targets:
                 continue
             state = {f"{prefix}.{n}": p.data for n, p in module.named_parameters(recurse=False)}
-            if prefix in sparse_targets:  # sparsity first
-                state = dict(self.sparsity_compressor.decompress_from_state_dict(state))
-            if prefix in module_to_scheme:  # quantization second
-                compressor = self.quantization_compressor.get(self._format_of(module))
-                state = compressor.decompress_module_from_state_dict(
-                    prefix, state, scheme=module_to_scheme[prefix])
+            dense = None
+            if prefix in sparse_targets and prefix in module_to_scheme:  # both in one pass
+                dense = self._decompress_quantized_24(
+                    prefix, state, self.quantization_compressor.get(self._format_of(module)))
+            if dense is not None:
+                state = dense
+            else:
+                if prefix in sparse_targets:  # sparsity first
+                    state = dict(self.sparsity_compressor.decompress_from_state_dict(state))
+                if prefix in module_to_scheme:  # quantization second
+                    compressor = self.quantization_compressor.get(self._format_of(module))
+                    state = compressor.decompress_module_from_state_dict(
+                        prefix, state, scheme=module_to_scheme[prefix])
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.FROZEN
 

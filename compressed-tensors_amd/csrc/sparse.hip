@@ -27,7 +27,10 @@ constexpr int kWaves = kBlock / kWave;
 // work items per lane of the 2:4 streaming kernels (measured: compress 1 / 2 / 4 items
 // 4.27 / 4.16 / 3.94 TB/s, decompress 3.1 / 4.0 / 4.2)
 constexpr int kS24U = 2;         // compress
-constexpr int kS24ScatterU = 4;  // decompress
+#ifndef CTMI_S24_SCATTER_U
+#define CTMI_S24_SCATTER_U 4
+#endif
+constexpr int kS24ScatterU = CTMI_S24_SCATTER_U;  // decompress
 
 // ------------------------------------------------------------------ block scan
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
@@ -312,11 +315,12 @@ bitmask_compact_kernel(const R* __restrict__ x, const uint8_t* __restrict__ bitm
 // LDS, every thread picks its own 8.  `src` is where the row's values start and is
 // moved past them.  A bitmask with more set bits than there are values reads
 // zeros, never past the end.
-template <typename R>
-__device__ __forceinline__ void scatter_row(const R* __restrict__ values, int64_t nvalues,
-                                            const uint8_t* __restrict__ mask_row, int64_t& src,
-                                            R* __restrict__ row, int64_t cols, int64_t pc, bool vec,
-                                            uint32_t tail, int* scan_s, R* stage) {
+// `store(b, o)` takes the 8 elements that bitmask byte b of the row stands for.
+template <typename R, typename Store>
+__device__ __forceinline__ void scatter_row_to(const R* __restrict__ values, int64_t nvalues,
+                                               const uint8_t* __restrict__ mask_row, int64_t& src,
+                                               int64_t pc, uint32_t tail, int* scan_s, R* stage,
+                                               Store store) {
   for (int64_t b0 = 0; b0 < pc; b0 += kBlock) {
     const int64_t b = b0 + threadIdx.x;
     uint32_t bits = 0;
@@ -334,17 +338,29 @@ __device__ __forceinline__ void scatter_row(const R* __restrict__ values, int64_
       Vec<R, 8> o;
 #pragma unroll
       for (int j = 0; j < 8; ++j) o.v[j] = ((bits >> j) & 1u) ? stage[pre++] : (R)0;
-      if (vec) {
-        stg<R, 8>(row + b * 8, o);
-      } else {
-        for (int j = 0; j < 8; ++j) {
-          const int64_t c = b * 8 + j;
-          if (c < cols) row[c] = o.v[j];
-        }
-      }
+      store(b, o);
     }
     __syncthreads();
   }
+}
+
+// ... into a dense row of the same element type
+template <typename R>
+__device__ __forceinline__ void scatter_row(const R* __restrict__ values, int64_t nvalues,
+                                            const uint8_t* __restrict__ mask_row, int64_t& src,
+                                            R* __restrict__ row, int64_t cols, int64_t pc, bool vec,
+                                            uint32_t tail, int* scan_s, R* stage) {
+  scatter_row_to<R>(values, nvalues, mask_row, src, pc, tail, scan_s, stage,
+                    [&](int64_t b, const Vec<R, 8>& o) {
+                      if (vec) {
+                        stg<R, 8>(row + b * 8, o);
+                      } else {
+                        for (int j = 0; j < 8; ++j) {
+                          const int64_t c = b * 8 + j;
+                          if (c < cols) row[c] = o.v[j];
+                        }
+                      }
+                    });
 }
 
 template <typename R>
@@ -721,6 +737,21 @@ sparse24_scatter_kernel(const R* __restrict__ values, const uint8_t* __restrict_
   if (threadIdx.x == 0) verdicts[blockIdx.x] = any_bad ? 1 : 0;
 }
 
+// Did any streaming workgroup meet a bitmask that is not 2:4?  The same answer in every
+// thread of the workgroup.  `verdicts` is 16-byte aligned.
+__device__ __forceinline__ bool any_bad_verdict(const int* __restrict__ verdicts,
+                                                int64_t n_verdicts) {
+  uint32_t bad = 0;
+  const int64_t quads = n_verdicts / 4;  // 16 bytes per load
+  const u32x4_t* v4 = reinterpret_cast<const u32x4_t*>(verdicts);
+  for (int64_t i = threadIdx.x; i < quads; i += kBlock) {
+    const u32x4_t q = v4[i];
+    bad |= q.x | q.y | q.z | q.w;
+  }
+  for (int64_t i = quads * 4 + threadIdx.x; i < n_verdicts; i += kBlock) bad |= (uint32_t)verdicts[i];
+  return __syncthreads_or((int)bad) != 0;
+}
+
 // What follows the streaming pass: every workgroup looks at all the verdicts (a few
 // KB, from L2) and is done if none is up.  Otherwise the bitmask is not 2:4 and the
 // workgroups redo the tensor as a general scatter, rows dealt round-robin; where a
@@ -737,15 +768,7 @@ sparse24_repair_kernel(const R* __restrict__ values, int64_t nvalues,
   __shared__ int scan_s[kWaves];
   __shared__ int64_t red[kWaves];
   __shared__ R stage[kBlock * 8];
-  uint32_t bad = 0;
-  const int64_t quads = n_verdicts / 4;  // 16 bytes per load; verdicts is 16-byte aligned
-  const u32x4_t* v4 = reinterpret_cast<const u32x4_t*>(verdicts);
-  for (int64_t i = threadIdx.x; i < quads; i += kBlock) {
-    const u32x4_t q = v4[i];
-    bad |= q.x | q.y | q.z | q.w;
-  }
-  for (int64_t i = quads * 4 + threadIdx.x; i < n_verdicts; i += kBlock) bad |= (uint32_t)verdicts[i];
-  if (!__syncthreads_or((int)bad)) return;
+  if (!any_bad_verdict(verdicts, n_verdicts)) return;
   const bool vec = (uintptr_t)out % (8 * sizeof(R)) == 0;
   int64_t src = 0, counted = 0;  // set bits in rows [0, counted)
   for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
@@ -754,6 +777,116 @@ sparse24_repair_kernel(const R* __restrict__ values, int64_t nvalues,
     src += block_sum(c, red);
     scatter_row<R>(values, nvalues, bitmask + r * pc, src, out + r * cols, cols, pc, vec, 0xffu, scan_s,
                    stage);
+    counted = r + 1;
+  }
+}
+
+// 2:4 decompression of int8 / fp8 codes and their dequantization in one pass: what
+// ModelCompressor.decompress does to a weight that is both 2:4 sparse and quantized
+// (the sparse compressor first, sparse_24_bitmask.py:206-224, then dequantize on the
+// dense codes, naive_quantized.py:116-140), without the dense code tensor in between:
+// 1/2 + 1/8 + 2 bytes per element of a bf16 weight instead of 1 5/8 + 3.  A lane takes
+// one bitmask byte and its 4 codes and stores 8 dequantized elements (one scale: rows
+// are multiples of 8 elements); a pruned position holds code 0, as it does in the dense
+// code tensor.  Verdicts as in sparse24_scatter_kernel.
+#ifndef CTMI_S24_DQ_U
+#define CTMI_S24_DQ_U 8
+#endif
+constexpr int kS24DqU = CTMI_S24_DQ_U;
+
+template <typename FT, int QK, bool HAS_ZP>
+__device__ __forceinline__ Vec<typename FT::raw, 8> dequant_codes8(const Vec<uint8_t, 8>& codes,
+                                                                   typename FT::raw sraw,
+                                                                   uint8_t zraw) {
+  constexpr int kIn = QK == 0 ? kKindI8 : kKindF8;
+  Vec<typename FT::raw, 8> unused_f, o;
+  Vec<uint8_t, 8> unused_c;
+  float z = 0.0f;
+  if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw : f8e4m3_to_f32(zraw);
+  qdq_vec8<FT, kIn, kKindFloat, QK, HAS_ZP>(unused_f, codes, FT::to_f32(sraw), z, 0.0f, 0.0f, &o,
+                                            &unused_c);
+  return o;
+}
+
+template <typename FT, int QK, bool HAS_ZP>
+__global__ void __launch_bounds__(kBlock)
+sparse24_scatter_dequant_kernel(const uint8_t* __restrict__ values,
+                                const uint8_t* __restrict__ bitmask,
+                                const typename FT::raw* __restrict__ scale,
+                                const uint8_t* __restrict__ zp, typename FT::raw* __restrict__ out,
+                                int64_t n_items, VecGeom g, int* __restrict__ verdicts) {
+  using FR = typename FT::raw;
+  constexpr int U = kS24DqU;
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  uint8_t m[U], zraw[U];
+  uint32_t v[U];
+  FR sraw[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    int64_t i = i0 + k * kBlock;
+    if (i >= n_items) i = n_items - 1;  // past the end: re-read the last item (not stored)
+    const uint32_t si = scale_index((uint32_t)i, g);
+    m[k] = bitmask[i];
+    v[k] = reinterpret_cast<const uint32_t*>(values)[i];
+    sraw[k] = scale[si];
+    zraw[k] = 0;
+    if constexpr (HAS_ZP) zraw[k] = zp[si];
+  }
+  bool bad = false;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    const uint32_t bits = m[k];
+    uint32_t n = bits - ((bits >> 1) & 0x55u);
+    n = (n & 0x33u) + ((n >> 2) & 0x33u);  // set bits per group of 4
+    bad |= i < n_items && n != 0x22u;
+    Vec<uint8_t, 8> codes;
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const uint32_t gm = (bits >> (4 * q)) & 15u;
+      const uint8_t a = (uint8_t)(v[k] >> (16 * q)), b = (uint8_t)(v[k] >> (16 * q + 8));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const bool keep = (gm >> j) & 1u, second = (gm & ((1u << j) - 1u)) != 0;
+        codes.v[4 * q + j] = keep ? (second ? b : a) : (uint8_t)0;
+      }
+    }
+    const Vec<FR, 8> o = dequant_codes8<FT, QK, HAS_ZP>(codes, sraw[k], zraw[k]);
+    if (i < n_items) stg_nt<FR, 8>(out + i * 8, o);
+  }
+  const int any_bad = __syncthreads_or(bad);
+  if (threadIdx.x == 0) verdicts[blockIdx.x] = any_bad ? 1 : 0;
+}
+
+// ... and what sparse24_repair_kernel is to sparse24_scatter_kernel: nothing for a 2:4
+// bitmask, otherwise the general scatter of the codes, dequantized as they are placed.
+template <typename FT, int QK, bool HAS_ZP>
+__global__ void __launch_bounds__(kBlock)
+sparse24_repair_dequant_kernel(const uint8_t* __restrict__ values, int64_t nvalues,
+                               const uint8_t* __restrict__ bitmask,
+                               const typename FT::raw* __restrict__ scale,
+                               const uint8_t* __restrict__ zp, typename FT::raw* __restrict__ out,
+                               int64_t rows, int64_t pc, VecGeom g,
+                               const int* __restrict__ verdicts, int64_t n_verdicts) {
+  using FR = typename FT::raw;
+  __shared__ int scan_s[kWaves];
+  __shared__ int64_t red[kWaves];
+  __shared__ uint8_t stage[kBlock * 8];
+  if (!any_bad_verdict(verdicts, n_verdicts)) return;
+  int64_t src = 0, counted = 0;  // set bits in rows [0, counted)
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    int64_t c = 0;
+    for (int64_t b = counted * pc + threadIdx.x; b < r * pc; b += kBlock) c += __popc((uint32_t)bitmask[b]);
+    src += block_sum(c, red);
+    scatter_row_to<uint8_t>(values, nvalues, bitmask + r * pc, src, pc, 0xffu, scan_s, stage,
+                            [&](int64_t b, const Vec<uint8_t, 8>& codes) {
+                              const int64_t i = r * pc + b;
+                              const uint32_t si = scale_index((uint32_t)i, g);
+                              uint8_t zraw = 0;
+                              if constexpr (HAS_ZP) zraw = zp[si];
+                              stg<FR, 8>(out + i * 8,
+                                         dequant_codes8<FT, QK, HAS_ZP>(codes, scale[si], zraw));
+                            });
     counted = r + 1;
   }
 }
@@ -1391,4 +1524,74 @@ extern "C" int ctmi_quantize_sparse24_compress(const void* x, int32_t x_dtype, v
 #undef CTMI_QS24_K
 #undef CTMI_QS24
   return check_launch("ctmi_quantize_sparse24_compress");
+}
+
+// the layouts of ctmi_quantize_sparse24_compress, read the other way; how the codes are
+// decoded follows from their dtype, not from the quantization arguments (dequantize
+// infers those from the scale's shape, forward.py:107-138)
+extern "C" int ctmi_sparse24_decompress_dequantize_supported(int32_t values_dtype,
+                                                             int32_t out_dtype, int64_t rows,
+                                                             int64_t cols, const ctmi_qparams* qp) {
+  if (!qp || rows < 1 || cols < 1 || cols % 8) return 0;
+  if (values_dtype != CTMI_I8 && values_dtype != CTMI_F8E4M3) return 0;
+  if (out_dtype != CTMI_BF16 && out_dtype != CTMI_F16 && out_dtype != CTMI_F32) return 0;
+  if (qp->scale_dtype != out_dtype || qp->global_scale || qp->col_group) return 0;
+  if (qp->zero_point && qp->zp_dtype != values_dtype) return 0;
+  VecGeom g;
+  return vec_geometry(qp, rows, cols, &g) ? 1 : 0;
+}
+
+extern "C" int64_t ctmi_sparse24_dequantize_tmp_bytes(int64_t rows, int64_t cols) {
+  const int64_t r = rows < 1 ? 1 : rows, c = cols < 1 ? 1 : cols;
+  return 4 * cdiv(cdiv(r * c, 8), kBlock * kS24DqU) + 16;
+}
+
+extern "C" int ctmi_sparse24_decompress_dequantize(const void* values, int64_t nvalues,
+                                                   int32_t values_dtype, const uint8_t* bitmask,
+                                                   void* out,
+                                                   int32_t out_dtype, void* tmp, int64_t rows,
+                                                   int64_t cols, const ctmi_qparams* qp,
+                                                   void* stream) {
+  CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
+  int rc = check_qparams(qp, rows, cols);
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  CTMI_REQUIRE(ctmi_sparse24_decompress_dequantize_supported(values_dtype, out_dtype, rows, cols, qp),
+               CTMI_ERR_UNSUPPORTED,
+               "no fused kernel for this layout: decompress the codes, then dequantize");
+  CTMI_REQUIRE(values && bitmask && out && tmp, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE(nvalues * 2 == rows * cols, CTMI_ERR_VALUE,
+               "a 2:4 tensor of %lld x %lld elements has %lld values, got %lld", (long long)rows,
+               (long long)cols, (long long)(rows * cols / 2), (long long)nvalues);
+  CTMI_REQUIRE((uintptr_t)out % (8 * dtype_size(out_dtype)) == 0 && (uintptr_t)values % 4 == 0 &&
+                   (uintptr_t)tmp % 16 == 0,
+               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements, tmp to 16 bytes");
+  VecGeom g;
+  vec_geometry(qp, rows, cols, &g);
+  const int64_t items = rows * cols / 8;
+  const int64_t pc = cols / 8;
+  const unsigned grid = (unsigned)cdiv(items, kBlock * kS24DqU);
+  const unsigned repair_grid = (unsigned)(rows < 32 ? rows : 32);
+  int* verdicts = (int*)tmp;
+  hipStream_t st = (hipStream_t)stream;
+  const uint8_t* zp = (const uint8_t*)qp->zero_point;
+#define CTMI_S24DQ_K(FT, RAW, QK, HZ)                                                             \
+  hipLaunchKernelGGL((sparse24_scatter_dequant_kernel<FT, QK, HZ>), grid, kBlock, 0, st,          \
+                     (const uint8_t*)values, bitmask, (const RAW*)qp->scale, zp, (RAW*)out, items, \
+                     g, verdicts);                                                                 \
+  hipLaunchKernelGGL((sparse24_repair_dequant_kernel<FT, QK, HZ>), repair_grid, kBlock, 0, st,    \
+                     (const uint8_t*)values, nvalues, bitmask, (const RAW*)qp->scale, zp,          \
+                     (RAW*)out, rows, pc, g, verdicts, (int64_t)grid)
+#define CTMI_S24DQ(FT, RAW)                                                          \
+  if (values_dtype == CTMI_I8) {                                                     \
+    if (zp) { CTMI_S24DQ_K(FT, RAW, 0, true); } else { CTMI_S24DQ_K(FT, RAW, 0, false); } \
+  } else {                                                                           \
+    if (zp) { CTMI_S24DQ_K(FT, RAW, 1, true); } else { CTMI_S24DQ_K(FT, RAW, 1, false); } \
+  }
+  if (out_dtype == CTMI_BF16) { CTMI_S24DQ(BF16, uint16_t); }
+  else if (out_dtype == CTMI_F16) { CTMI_S24DQ(F16, uint16_t); }
+  else { CTMI_S24DQ(F32, float); }
+#undef CTMI_S24DQ_K
+#undef CTMI_S24DQ
+  return check_launch("ctmi_sparse24_decompress_dequantize");
 }

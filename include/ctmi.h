@@ -261,6 +261,27 @@ int ctmi_quantize_sparse24_compress(const void* x, int32_t x_dtype, void* values
                                     int64_t rows, int64_t cols, const ctmi_qparams* qp,
                                     void* stream);
 
+/* A22 + A13 in one pass: the stacked case of ModelCompressor.decompress
+ * (model_compressors/model_compressor.py:572-604, :694-760): the 2:4 values and bitmask of a
+ * quantized weight are expanded (sparse_24_bitmask.py:206-224) and the codes
+ * dequantized (naive_quantized.py:116-140) without the dense code tensor in between.
+ * values: [rows, cols / 2] codes (float8_e4m3fn or int8), nvalues of them; out:
+ * [rows, cols] of out_dtype, the dtype of the scales.  Same bits as
+ * ctmi_sparse24_decompress followed by ctmi_qdq, also for a bitmask that is not 2:4
+ * (set bits are then filled from `values` in order, as in ctmi_bitmask_decompress).
+ * The codes are decoded by values_dtype (CTMI_I8 or CTMI_F8E4M3), whatever qp's type
+ * says: dequantize() infers its arguments from the scale's shape alone.
+ * _supported(): as for ctmi_quantize_sparse24_compress.  tmp:
+ * ctmi_sparse24_dequantize_tmp_bytes() bytes of device scratch, 16-byte aligned. */
+int ctmi_sparse24_decompress_dequantize_supported(int32_t values_dtype, int32_t out_dtype,
+                                                  int64_t rows, int64_t cols,
+                                                  const ctmi_qparams* qp);
+int64_t ctmi_sparse24_dequantize_tmp_bytes(int64_t rows, int64_t cols);
+int ctmi_sparse24_decompress_dequantize(const void* values, int64_t nvalues, int32_t values_dtype,
+                                        const uint8_t* bitmask, void* out, int32_t out_dtype,
+                                        void* tmp, int64_t rows, int64_t cols,
+                                        const ctmi_qparams* qp, void* stream);
+
 /* A1.  calculate_qparams (quantization/utils/helpers.py:67-146), elementwise
  * over n (min, max) pairs of dtype mm_dtype.  mm_is_0d != 0 when the reference
  * would see 0-d min/max tensors (their zero-point subtraction then promotes to

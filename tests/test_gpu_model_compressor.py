@@ -130,12 +130,36 @@ def test_fp8_plus_sparse24_stack(gpu):
         assert_bit_equal(state[f"{name}.bitmask"], bm, f"{name}.bitmask")
         assert state[f"{name}.shape"].flatten().tolist() == list(w.shape)
         assert f"{name}.weight" not in state and f"{name}.weight_scale" in state
-    mc.compress_model(model)
-    mc.decompress_model(model)
+    # the way back, from the state dict: every such module through the kernel that decompresses
+    # and dequantizes in one pass
+    import copy
+    from unittest import mock
+
+    want = {}
     for name, (w, s, z) in cpu.items():
         codes = op.naive_compress(w, s, oargs, zero_point=z)
-        dense = op.naive_decompress({"weight": codes, "weight_scale": s})
-        assert_bit_equal(model.get_submodule(name).weight.data, dense, f"{name} decompressed")
+        want[name] = op.naive_decompress({"weight": codes, "weight_scale": s})
+    other = copy.deepcopy(model)
+    for name in cpu:
+        other.get_submodule(name).weight.data.zero_()
+    with mock.patch.object(mc, "_decompress_quantized_24", wraps=mc._decompress_quantized_24) as fused:
+        mc.decompress(dict(state), other)
+    assert fused.call_count == len(cpu)
+    for name in cpu:
+        assert_bit_equal(other.get_submodule(name).weight.data, want[name], f"{name} from the state dict")
+        assert_bit_equal(other.get_submodule(name).weight_scale.data, cpu[name][1], f"{name}.weight_scale")
+    # ... and in memory
+    mc.compress_model(model)
+    for name, (w, s, z) in cpu.items():
+        module = model.get_submodule(name)
+        assert_bit_equal(module.compressed.data, state[f"{name}.compressed"], f"{name}.compressed in memory")
+        assert_bit_equal(module.bitmask.data, state[f"{name}.bitmask"], f"{name}.bitmask in memory")
+        assert not hasattr(module, "weight")
+    with mock.patch.object(mc, "_decompress_quantized_24", wraps=mc._decompress_quantized_24) as fused:
+        mc.decompress_model(model)
+    assert fused.call_count == len(cpu)
+    for name in cpu:
+        assert_bit_equal(model.get_submodule(name).weight.data, want[name], f"{name} decompressed")
 
 
 @pytest.mark.parametrize("fmt,spec,dtype", [

@@ -405,3 +405,83 @@ def test_quantization_and_2_4_without_a_fused_kernel(gpu):
     w = torch.randn(8, 32).bfloat16().to(gpu)
     assert quantize_sparse24_compress(w, scale, args, g_idx=torch.zeros(32, dtype=torch.int32, device=gpu)) is None
     assert quantize_sparse24_compress(w, scale, args) is not None
+
+
+@pytest.mark.parametrize("spec,shape,dtype", QS24, ids=[f"s24dq-{i}" for i in range(len(QS24))])
+def test_2_4_decompression_and_dequantization_in_one_pass(spec, shape, dtype, gpu):
+    """2:4 values + bitmask of a quantized weight -> the dense dequantized weight from one
+    kernel == the oracle's sparse24_bitmask_decompress followed by its dequantize (arguments
+    inferred from the scale's shape, as the naive compressor's decompress_weight calls it),
+    and == this library's own two steps"""
+    from compressed_tensors_amd.compressors import (
+        sparse24_bitmask_decompress, sparse24_decompress_dequantize,
+    )
+    from compressed_tensors_amd.quantization import dequantize
+
+    announce("2:4 decompress + dequantize", spec, shape, dtype)
+    oargs = oq._Args(**spec)
+    code_dtype = torch.float8_e4m3fn if spec["type"] == "float" else torch.int8
+    g = torch.Generator().manual_seed(shape[1] + 1)
+    w = torch.randn(shape, generator=g) * 0.02
+    w[torch.rand(shape, generator=g) < 0.002] *= 30
+    w = _prune24(w).to(dtype)
+    scale, zp = oq.observe_weight(w, oargs)
+    for zero_point in ((zp,) if not spec["symmetric"] else (zp, None)):
+        codes = oq.quantize(w, scale, zero_point, oargs, dtype=code_dtype)
+        values, bitmask = osp.sparse24_bitmask_compress(codes)
+        want = oq.dequantize(osp.sparse24_bitmask_decompress(values, bitmask, shape), scale, zero_point)
+        zp_gpu = None if zero_point is None else zero_point.to(gpu)
+        got = sparse24_decompress_dequantize(values.to(gpu), bitmask.to(gpu), shape, scale.to(gpu), zp_gpu)
+        assert got is not None, "expected a fused kernel for this layout"
+        assert got.dtype == dtype and tuple(got.shape) == tuple(shape)
+        assert_bit_equal(got, want, "dequantized weight")
+        two_steps = dequantize(sparse24_bitmask_decompress(values.to(gpu), bitmask.to(gpu), shape),
+                               scale.to(gpu), zp_gpu)
+        assert_bit_equal(got, two_steps, "one pass against two steps")
+
+
+@pytest.mark.parametrize("rows,cols", [(48, 256), (3000, 64)], ids=["48x256", "3000x64"])
+def test_2_4_decompression_and_dequantization_of_a_bitmask_that_is_not_2_4(rows, cols, gpu):
+    """half of the positions set, but not two in every four: the kernel behind the streaming
+    one redoes the tensor as a general scatter, dequantizing as it places the codes"""
+    from compressed_tensors_amd.compressors import sparse24_decompress_dequantize
+
+    announce("2:4 decompress + dequantize, bitmask not 2:4", rows, cols)
+    g = torch.Generator().manual_seed(rows)
+    mask = torch.zeros(rows * cols, dtype=torch.bool)
+    mask[torch.randperm(rows * cols, generator=g)[: rows * cols // 2]] = True
+    mask = mask.view(rows, cols)
+    values = torch.randint(-127, 128, (rows, cols // 2), generator=g, dtype=torch.int8)
+    bitmask = osp.pack_bitmasks(mask)
+    scale = (torch.rand(rows, 1, generator=g) * 0.01 + 0.001).bfloat16()
+    zp = torch.randint(-5, 6, (rows, 1), generator=g, dtype=torch.int8)
+    for code_dtype in (torch.int8, torch.float8_e4m3fn):
+        vals = values.view(code_dtype)
+        zero_point = zp if code_dtype == torch.int8 else None
+        if code_dtype == torch.float8_e4m3fn:  # no NaN codes: their payload bits are not part of the contract
+            vals = torch.where((values & 0x7F) == 0x7F, torch.zeros_like(values), values).view(code_dtype)
+        want = oq.dequantize(osp.bitmask_decompress(vals.flatten(), bitmask, (rows, cols)), scale, zero_point)
+        got = sparse24_decompress_dequantize(vals.to(gpu), bitmask.to(gpu), (rows, cols), scale.to(gpu),
+                                             None if zero_point is None else zero_point.to(gpu))
+        assert got is not None
+        assert_bit_equal(got, want, f"dequantized weight ({code_dtype})")
+
+
+def test_2_4_decompression_and_dequantization_without_a_fused_kernel(gpu):
+    """rows that are not whole 8-element items, scales in another dtype than asked for, codes
+    that are not 8-bit: None, and the caller takes the two steps"""
+    from compressed_tensors_amd.compressors import sparse24_decompress_dequantize
+
+    announce("2:4 decompress + dequantize, unsupported")
+    scale = torch.full((8, 1), 0.01, dtype=torch.bfloat16, device=gpu)
+    values = torch.zeros(8, 6, dtype=torch.int8, device=gpu)
+    bitmask = torch.zeros(8, 2, dtype=torch.uint8, device=gpu)
+    assert sparse24_decompress_dequantize(values, bitmask, (8, 12), scale) is None
+    values = torch.zeros(8, 16, dtype=torch.int8, device=gpu)
+    bitmask = torch.full((8, 4), 0x33, dtype=torch.uint8, device=gpu)
+    assert sparse24_decompress_dequantize(values.to(torch.int16), bitmask, (8, 32), scale) is None
+    assert sparse24_decompress_dequantize(values, bitmask, (8, 32), scale.double()) is None
+    assert sparse24_decompress_dequantize(
+        values, bitmask, (8, 32), scale, g_idx=torch.zeros(32, dtype=torch.int32, device=gpu)) is None
+    out = sparse24_decompress_dequantize(values, bitmask, (8, 32), scale)
+    assert out is not None and out.dtype == torch.bfloat16 and not out.any()
