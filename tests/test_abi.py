@@ -148,6 +148,23 @@ def test_one_pass_and_many_argument_errors(ctmi):
     assert ctmi.ctmi_quantize_sparse24_compress_supported(_lib.BF16, 4, 12, ctypes.byref(qp)) == 0
     rc = ctmi.ctmi_quantize_sparse24_compress(0x1000, _lib.BF16, 0x2000, 0x3000, 4, 12, ctypes.byref(qp), None)
     assert rc == _lib.CTMI_ERR_UNSUPPORTED
+    # ... and the way back: codes are int8 or fp8, as many values as half the elements
+    qp = _qp(s_rows=4, s_cols=1, blk_rows=1, blk_cols=64, qtype=_lib.QTYPE_INT, num_bits=8)
+    ok = ctmi.ctmi_sparse24_decompress_dequantize_supported
+    assert ok(_lib.F8E4M3, _lib.BF16, 4, 64, ctypes.byref(qp)) == 1
+    assert ok(_lib.I8, _lib.BF16, 4, 64, ctypes.byref(qp)) == 1
+    assert ok(_lib.BF16, _lib.BF16, 4, 64, ctypes.byref(qp)) == 0
+    assert ok(_lib.I8, _lib.F32, 4, 64, ctypes.byref(qp)) == 0   # scales are bf16
+    assert ctmi.ctmi_sparse24_dequantize_tmp_bytes(14336, 4096) > ctmi.ctmi_sparse24_dequantize_tmp_bytes(8, 8) > 0
+    rc = ctmi.ctmi_sparse24_decompress_dequantize(0x1000, 100, _lib.I8, 0x2000, 0x3000, _lib.BF16, 0x4000,
+                                                  4, 64, ctypes.byref(qp), None)
+    assert rc == _lib.CTMI_ERR_VALUE and "128 values" in _err(ctmi)
+    rc = ctmi.ctmi_sparse24_decompress_dequantize(0x1000, 128, _lib.I8, 0x2000, 0x3000, _lib.BF16, None,
+                                                  4, 64, ctypes.byref(qp), None)
+    assert rc == _lib.CTMI_ERR_VALUE and "NULL tensor pointer" in _err(ctmi)
+    rc = ctmi.ctmi_sparse24_decompress_dequantize(0x1000, 128, _lib.I16, 0x2000, 0x3000, _lib.BF16, 0x4000,
+                                                  4, 64, ctypes.byref(qp), None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED
 
 
 def test_topk24_table_matches_installed_torch(ctmi):
