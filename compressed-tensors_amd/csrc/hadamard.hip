@@ -20,6 +20,7 @@
 // Tile = S sub-rows of b elements = one contiguous span of memory, staged
 // through LDS in both directions so that every HBM access is a full 16-byte
 // lane access on consecutive addresses.
+#include <atomic>
 #include "ctmi_device.h"
 #include "ctmi_host.h"
 #include "qparams.h"
@@ -832,15 +833,22 @@ block_matmul_kernel(const typename IO::raw* __restrict__ x, const float* __restr
 template <int A, int B, typename IO>
 static int launch_had(const HadArgs& a, hipStream_t st) {
   using C = HadCfg<A, B, IO>;
-  static bool configured = false;
+  // the attribute belongs to the kernel as loaded on one device: once per device
+  constexpr int kMaxDevices = 64;
+  static std::atomic<bool> configured[kMaxDevices];
   auto kern = hadamard_mfma_kernel<A, B, IO>;
-  if (!configured && C::lds_bytes > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)C::lds_bytes);
-    if (e != hipSuccess)
-      return set_error(CTMI_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    configured = true;
+  if (C::lds_bytes > 48 * 1024) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+    const bool tracked = dev >= 0 && dev < kMaxDevices;
+    if (!tracked || !configured[dev].load(std::memory_order_acquire)) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize,
+                                         (int)C::lds_bytes);
+      if (e != hipSuccess)
+        return set_error(CTMI_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+      if (tracked) configured[dev].store(true, std::memory_order_release);
+    }
   }
   const int64_t tiles = cdiv(a.n_sub, C::S);
   const int64_t cap = 256 * 8;
