@@ -1015,9 +1015,9 @@ bytemask24_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64_t n
 // item i (N neighbouring elements): the 2 survivors of every group of 4, in column
 // order, and the item's bitmask bytes
 template <typename R, int DT, int N>
-__device__ __forceinline__ void store_survivors24(const Vec<R, N>& a, R* __restrict__ values,
-                                                  uint8_t* __restrict__ bitmask, int64_t i,
-                                                  bool keep_item) {
+__device__ __forceinline__ void store_survivors24_any(const Vec<R, N>& a, R* __restrict__ values,
+                                                      uint8_t* __restrict__ bitmask, int64_t i,
+                                                      bool keep_item) {
   const uint32_t keep_all = keep_masks24<R, DT, N>(a);
   Vec<R, N / 2> o;
   Vec<uint8_t, N / 8> m;
@@ -1036,6 +1036,64 @@ __device__ __forceinline__ void store_survivors24(const Vec<R, N>& a, R* __restr
     stg<R, N / 2>(values + i * (N / 2), o);
     stg<uint8_t, N / 8>(bitmask + i * (N / 8), m);
   }
+}
+
+// One-byte elements ranked through their int8 view (int8 and float8 tensors), four
+// groups or two to a lane: a group is one 32-bit word, and as long as every group of
+// the wavefront already has exactly two elements that rank above zero (a tensor that
+// was pruned to 2:4, the usual input) everything is done on whole words: which bytes
+// are neither 0x00 nor 0x80 (abs(-128) stays -128 in int8 and ranks below zero), the
+// four flags gathered into the group's bits, the survivors of two groups picked by one
+// byte permute.  Any other wavefront takes the element-wise path.
+template <int N>
+__device__ __forceinline__ void store_survivors24_bytes(const Vec<uint8_t, N>& a,
+                                                        uint8_t* __restrict__ values,
+                                                        uint8_t* __restrict__ bitmask, int64_t i,
+                                                        bool keep_item) {
+  constexpr int G = N / 4;
+  static_assert(G % 2 == 0, "pairs of groups");
+  const Vec<uint32_t, G> w = __builtin_bit_cast(Vec<uint32_t, G>, a);
+  uint32_t keep_all = 0;
+  bool clear = true;
+#pragma unroll
+  for (int q = 0; q < G; ++q) {
+    const uint32_t t = w.v[q] & 0x7F7F7F7Fu;
+    const uint32_t nz = ((t + 0x7F7F7F7Fu) >> 7) & 0x01010101u;  // bit 0 of every byte that ranks above zero
+    clear &= __popc(nz) == 2;
+    keep_all |= ((nz | (nz >> 7) | (nz >> 14) | (nz >> 21)) & 15u) << (4 * q);
+  }
+  if (!wave_all(clear)) {
+    store_survivors24_any<uint8_t, CTMI_I8, N>(a, values, bitmask, i, keep_item);
+    return;
+  }
+  Vec<uint32_t, G / 2> o;
+#pragma unroll
+  for (int p = 0; p < G / 2; ++p) {
+    const uint32_t k0 = (keep_all >> (8 * p)) & 15u, k1 = (keep_all >> (8 * p + 4)) & 15u;
+    // byte numbers of the lower and the upper survivor of either group, in the 8 bytes
+    // {second word, first word}
+    const uint32_t sel = (uint32_t)__builtin_ctz(k0) | ((31u - (uint32_t)__clz(k0)) << 8) |
+                         ((4u + (uint32_t)__builtin_ctz(k1)) << 16) |
+                         ((35u - (uint32_t)__clz(k1)) << 24);
+    o.v[p] = __builtin_amdgcn_perm(w.v[2 * p + 1], w.v[2 * p], sel);
+  }
+  Vec<uint8_t, N / 8> m;
+#pragma unroll
+  for (int bq = 0; bq < N / 8; ++bq) m.v[bq] = (uint8_t)((keep_all >> (8 * bq)) & 0xffu);
+  if (keep_item) {
+    stg<uint32_t, G / 2>(reinterpret_cast<uint32_t*>(values + i * (N / 2)), o);
+    stg<uint8_t, N / 8>(bitmask + i * (N / 8), m);
+  }
+}
+
+template <typename R, int DT, int N>
+__device__ __forceinline__ void store_survivors24(const Vec<R, N>& a, R* __restrict__ values,
+                                                  uint8_t* __restrict__ bitmask, int64_t i,
+                                                  bool keep_item) {
+  if constexpr (sizeof(R) == 1 && DT == CTMI_I8 && N % 8 == 0)
+    store_survivors24_bytes<N>(a, values, bitmask, i, keep_item);
+  else
+    store_survivors24_any<R, DT, N>(a, values, bitmask, i, keep_item);
 }
 
 template <typename R, int DT, int N>
