@@ -256,7 +256,7 @@ def other_workload(torch, name, seed):
     if name == "sparse":
         copies = 6
         c_calls, d_calls, s_calls, t_calls, two_step, one_step = [], [], [], [], [], []
-        back_two, back_one = [], []
+        back_two, back_one, s16_calls, t16_calls = [], [], [], []
         nb = 8192 * 8192
         nnz_total = 0
         for _ in range(copies):
@@ -306,6 +306,17 @@ def other_workload(torch, name, seed):
             two_step.append(lambda qa=qa, a=a: (_lib.check(lib.ctmi_qdq(*qa)), _lib.check(lib.ctmi_sparse24_compress(*a))))
             one_step.append(lambda fa=fa: _lib.check(lib.ctmi_quantize_sparse24_compress(*fa)))
             t_calls.append(lambda d=d: _lib.check(lib.ctmi_sparse24_decompress(*d)))
+            # the same format on the bf16 weight itself (a sparse-only checkpoint)
+            values16 = torch.empty(rows, cols // 2, dtype=w.dtype, device=dev)
+            dense16 = torch.empty_like(w)
+            tmp16 = torch.empty(lib.ctmi_sparse24_tmp_bytes(rows, cols, 2), dtype=torch.uint8, device=dev)
+            bitmask16 = torch.empty_like(bitmask)
+            keep.extend([values16, dense16, tmp16, bitmask16])
+            a16 = (w.data_ptr(), code(w.dtype), values16.data_ptr(), bitmask16.data_ptr(), rows, cols, st)
+            d16 = (values16.data_ptr(), values16.numel(), 2, bitmask16.data_ptr(), dense16.data_ptr(), tmp16.data_ptr(), rows, cols, st)
+            _lib.check(lib.ctmi_sparse24_compress(*a16))
+            s16_calls.append(lambda a16=a16: _lib.check(lib.ctmi_sparse24_compress(*a16)))
+            t16_calls.append(lambda d16=d16: _lib.check(lib.ctmi_sparse24_decompress(*d16)))
             # ... and the way back: 2:4 -> fp8 codes -> bf16
             back = torch.empty_like(w)
             tmp_dq = torch.empty(lib.ctmi_sparse24_dequantize_tmp_bytes(rows, cols), dtype=torch.uint8, device=dev)
@@ -322,6 +333,8 @@ def other_workload(torch, name, seed):
                Op("sparse-bitmask decompress (positions from the bitmask alone)", d_calls, bm_bytes, "bitmask_scatter_tiles_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
+               Op("sparse-24-bitmask compress, 14336x4096 bf16", s16_calls, 2 * s24_bytes - copies * (n24 // 8), "sparse24_compress_kernel"),
+               Op("sparse-24-bitmask decompress, bf16", t16_calls, 2 * s24_bytes - copies * (n24 // 8), "sparse24_scatter_kernel"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
                Op("bf16 -> fp8 codes -> 2:4 compress, one pass", one_step, fused24_bytes, "quant_sparse24_compress_kernel"),
                Op("2:4 decompress -> fp8 codes -> bf16, two steps", back_two, fused24_bytes, "qdq_vec_kernel", primary=False),
