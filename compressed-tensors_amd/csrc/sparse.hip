@@ -933,25 +933,37 @@ __device__ __forceinline__ uint32_t keep24(uint32_t k0, uint32_t k1, uint32_t k2
 // copy of it for the common case).
 template <typename R, int DT, int N>
 __device__ __forceinline__ uint32_t keep_masks24(const Vec<R, N>& a) {
+  constexpr bool kBytes = sizeof(R) == 1;  // int8 and float8 tensors, ranked through their int8 view
+  static_assert(kBytes == (DT == CTMI_I8), "one-byte elements are ranked as int8");
+  uint32_t keep = 0;
+  bool clear = true;
+  if constexpr (kBytes) {
+    // a group is one 32-bit word: which of its bytes are neither 0x00 nor 0x80 (abs(-128)
+    // stays -128 in int8 and ranks below zero), and the four flags gathered into four bits
+    const Vec<uint32_t, N / 4> w = __builtin_bit_cast(Vec<uint32_t, N / 4>, a);
+#pragma unroll
+    for (int q = 0; q < N / 4; ++q) {
+      const uint32_t t = w.v[q] & 0x7F7F7F7Fu;
+      const uint32_t nz = ((t + 0x7F7F7F7Fu) >> 7) & 0x01010101u;
+      clear &= __popc(nz) == 2;
+      keep |= ((nz | (nz >> 7) | (nz >> 14) | (nz >> 21)) & 15u) << (4 * q);
+    }
+    if (wave_all(clear)) return keep;
+  }
   uint32_t keys[N];
 #pragma unroll
   for (int i = 0; i < N; ++i) keys[i] = key24<DT>(a.v[i]);
-  uint32_t keep = 0;
-  bool clear = true;
+  if constexpr (!kBytes) {
 #pragma unroll
-  for (int q = 0; q < N / 4; ++q) {
-    uint32_t pos = 0;
+    for (int q = 0; q < N / 4; ++q) {
+      uint32_t pos = 0;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      // above zero as the ranking sees it (int8-view keys are biased by 128, and
-      // -128, whose abs() stays -128, ranks below zero)
-      const bool gt = DT == CTMI_I8 ? keys[4 * q + j] > 128u : keys[4 * q + j] != 0;
-      pos |= (gt ? 1u : 0u) << j;
+      for (int j = 0; j < 4; ++j) pos |= (keys[4 * q + j] != 0 ? 1u : 0u) << j;
+      clear &= __popc(pos) == 2;
+      keep |= pos << (4 * q);
     }
-    clear &= __popc(pos) == 2;
-    keep |= pos << (4 * q);
+    if (wave_all(clear)) return keep;
   }
-  if (wave_all(clear)) return keep;
   keep = 0;
 #pragma unroll
   for (int q = 0; q < N / 4; ++q)
@@ -987,10 +999,13 @@ bytemask24_vec_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64
   for (int k = 0; k < U; ++k) {
     const int64_t i = i0 + k * kBlock;
     const uint32_t keep = keep_masks24<R, DT, N>(a[k]);
-    Vec<uint8_t, N> o;
+    Vec<uint32_t, N / 4> o;  // four bool bytes per group
 #pragma unroll
-    for (int j = 0; j < N; ++j) o.v[j] = (uint8_t)((keep >> j) & 1u);
-    if (i < nitems) stg<uint8_t, N>(mask + i * N, o);
+    for (int q = 0; q < N / 4; ++q) {
+      const uint32_t kq = (keep >> (4 * q)) & 15u;
+      o.v[q] = (kq | (kq << 7) | (kq << 14) | (kq << 21)) & 0x01010101u;
+    }
+    if (i < nitems) stg<uint32_t, N / 4>(reinterpret_cast<uint32_t*>(mask + i * N), o);
   }
 }
 
@@ -1038,13 +1053,8 @@ __device__ __forceinline__ void store_survivors24_any(const Vec<R, N>& a, R* __r
   }
 }
 
-// One-byte elements ranked through their int8 view (int8 and float8 tensors), four
-// groups or two to a lane: a group is one 32-bit word, and as long as every group of
-// the wavefront already has exactly two elements that rank above zero (a tensor that
-// was pruned to 2:4, the usual input) everything is done on whole words: which bytes
-// are neither 0x00 nor 0x80 (abs(-128) stays -128 in int8 and ranks below zero), the
-// four flags gathered into the group's bits, the survivors of two groups picked by one
-// byte permute.  Any other wavefront takes the element-wise path.
+// One-byte elements (int8 and float8 tensors), four groups or two to a lane: a group is
+// one 32-bit word, and the survivors of two groups are picked by one byte permute.
 template <int N>
 __device__ __forceinline__ void store_survivors24_bytes(const Vec<uint8_t, N>& a,
                                                         uint8_t* __restrict__ values,
@@ -1052,20 +1062,8 @@ __device__ __forceinline__ void store_survivors24_bytes(const Vec<uint8_t, N>& a
                                                         bool keep_item) {
   constexpr int G = N / 4;
   static_assert(G % 2 == 0, "pairs of groups");
+  const uint32_t keep_all = keep_masks24<uint8_t, CTMI_I8, N>(a);  // two bits set in every group
   const Vec<uint32_t, G> w = __builtin_bit_cast(Vec<uint32_t, G>, a);
-  uint32_t keep_all = 0;
-  bool clear = true;
-#pragma unroll
-  for (int q = 0; q < G; ++q) {
-    const uint32_t t = w.v[q] & 0x7F7F7F7Fu;
-    const uint32_t nz = ((t + 0x7F7F7F7Fu) >> 7) & 0x01010101u;  // bit 0 of every byte that ranks above zero
-    clear &= __popc(nz) == 2;
-    keep_all |= ((nz | (nz >> 7) | (nz >> 14) | (nz >> 21)) & 15u) << (4 * q);
-  }
-  if (!wave_all(clear)) {
-    store_survivors24_any<uint8_t, CTMI_I8, N>(a, values, bitmask, i, keep_item);
-    return;
-  }
   Vec<uint32_t, G / 2> o;
 #pragma unroll
   for (int p = 0; p < G / 2; ++p) {
