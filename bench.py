@@ -256,7 +256,7 @@ def other_workload(torch, name, seed):
     if name == "sparse":
         copies = 6
         c_calls, d_calls, s_calls, t_calls, two_step, one_step = [], [], [], [], [], []
-        back_two, back_one, s16_calls, t16_calls = [], [], [], []
+        back_two, back_one, s16_calls, t16_calls, pk_calls, up_calls = [], [], [], [], [], []
         nb = 8192 * 8192
         nnz_total = 0
         for _ in range(copies):
@@ -306,6 +306,16 @@ def other_workload(torch, name, seed):
             two_step.append(lambda qa=qa, a=a: (_lib.check(lib.ctmi_qdq(*qa)), _lib.check(lib.ctmi_sparse24_compress(*a))))
             one_step.append(lambda fa=fa: _lib.check(lib.ctmi_quantize_sparse24_compress(*fa)))
             t_calls.append(lambda d=d: _lib.check(lib.ctmi_sparse24_decompress(*d)))
+            # the bool mask of the weight <-> its packed form
+            bools = get_24_bytemasks(w)
+            bools_back = torch.empty_like(bools)
+            packed = torch.empty(rows, cols // 8, dtype=torch.uint8, device=dev)
+            keep.extend([bools, bools_back, packed])
+            pk = (bools.data_ptr(), packed.data_ptr(), rows, cols, st)
+            up = (packed.data_ptr(), bools_back.data_ptr(), rows, cols, st)
+            _lib.check(lib.ctmi_pack_bitmasks(*pk))
+            pk_calls.append(lambda pk=pk: _lib.check(lib.ctmi_pack_bitmasks(*pk)))
+            up_calls.append(lambda up=up: _lib.check(lib.ctmi_unpack_bitmasks(*up)))
             # the same format on the bf16 weight itself (a sparse-only checkpoint)
             values16 = torch.empty(rows, cols // 2, dtype=w.dtype, device=dev)
             dense16 = torch.empty_like(w)
@@ -335,6 +345,8 @@ def other_workload(torch, name, seed):
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 bf16", s16_calls, 2 * s24_bytes - copies * (n24 // 8), "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress, bf16", t16_calls, 2 * s24_bytes - copies * (n24 // 8), "sparse24_scatter_kernel"),
+               Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies * (n24 + n24 // 8), "pack_bitmasks"),
+               Op("unpack_bitmasks", up_calls, copies * (n24 + n24 // 8), "unpack_bitmasks"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
                Op("bf16 -> fp8 codes -> 2:4 compress, one pass", one_step, fused24_bytes, "quant_sparse24_compress_kernel"),
                Op("2:4 decompress -> fp8 codes -> bf16, two steps", back_two, fused24_bytes, "qdq_vec_kernel", primary=False),

@@ -74,6 +74,62 @@ __device__ __forceinline__ int64_t block_sum(int64_t v, int64_t* smem) {
 }
 
 // ------------------------------------------------------------------ pack / unpack bitmasks
+// Rows of whole bitmask bytes make mask and bitmask flat runs: a lane turns 16 bool
+// bytes (one 16-byte load) into 2 bitmask bytes and back, all loads of a workgroup
+// first, whole 32-bit words at a time: a byte is set if its low 7 bits or its top bit
+// are; four flags gather into four bits by shifts.
+constexpr int kPackU = 4;
+
+__global__ void __launch_bounds__(kBlock)
+pack_bitmasks_flat_kernel(const uint8_t* __restrict__ mask, uint16_t* __restrict__ packed,
+                          int64_t n_items) {
+  constexpr int U = kPackU;
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  Vec<uint32_t, 4> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    int64_t i = i0 + k * kBlock;
+    if (i >= n_items) i = n_items - 1;  // past the end: re-read, not stored
+    a[k] = ldg_nt<uint32_t, 4>(reinterpret_cast<const uint32_t*>(mask) + i * 4);
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    uint32_t bits = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t w = a[k].v[q];
+      const uint32_t nz = ((((w & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | w) >> 7) & 0x01010101u;
+      bits |= ((nz | (nz >> 7) | (nz >> 14) | (nz >> 21)) & 15u) << (4 * q);
+    }
+    if (i < n_items) packed[i] = (uint16_t)bits;
+  }
+}
+
+__global__ void __launch_bounds__(kBlock)
+unpack_bitmasks_flat_kernel(const uint16_t* __restrict__ packed, uint8_t* __restrict__ mask,
+                            int64_t n_items) {
+  constexpr int U = kPackU;
+  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  uint32_t bits[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    bits[k] = packed[i < n_items ? i : n_items - 1];
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    Vec<uint32_t, 4> o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t kq = (bits[k] >> (4 * q)) & 15u;
+      o.v[q] = (kq | (kq << 7) | (kq << 14) | (kq << 21)) & 0x01010101u;
+    }
+    if (i < n_items) stg_nt<uint32_t, 4>(reinterpret_cast<uint32_t*>(mask) + i * 4, o);
+  }
+}
+
 __global__ void __launch_bounds__(kBlock)
 pack_bitmasks_kernel(const uint8_t* __restrict__ mask, uint8_t* __restrict__ packed, int64_t rows,
                      int64_t cols, int64_t pc) {
@@ -1218,6 +1274,14 @@ extern "C" int ctmi_pack_bitmasks(const uint8_t* mask, uint8_t* packed, int64_t 
   if (rows == 0 || cols == 0) return CTMI_OK;
   CTMI_REQUIRE(mask && packed, CTMI_ERR_VALUE, "NULL tensor pointer");
   const int64_t pc = cdiv(cols, 8);
+  const int64_t numel = rows * cols;
+  if (cols % 8 == 0 && numel % 16 == 0 && (uintptr_t)mask % 16 == 0 && (uintptr_t)packed % 2 == 0 &&
+      numel / 16 < (1ll << 40)) {
+    const int64_t n_items = numel / 16;
+    hipLaunchKernelGGL(pack_bitmasks_flat_kernel, (unsigned)cdiv(n_items, kBlock * kPackU), kBlock, 0,
+                       (hipStream_t)stream, mask, (uint16_t*)packed, n_items);
+    return check_launch("ctmi_pack_bitmasks");
+  }
   hipLaunchKernelGGL(pack_bitmasks_kernel, grid_for(rows * pc, kBlock), kBlock, 0,
                      (hipStream_t)stream, mask, packed, rows, cols, pc);
   return check_launch("ctmi_pack_bitmasks");
@@ -1229,6 +1293,14 @@ extern "C" int ctmi_unpack_bitmasks(const uint8_t* packed, uint8_t* mask, int64_
   if (rows == 0 || cols == 0) return CTMI_OK;
   CTMI_REQUIRE(mask && packed, CTMI_ERR_VALUE, "NULL tensor pointer");
   const int64_t pc = cdiv(cols, 8);
+  const int64_t numel = rows * cols;
+  if (cols % 8 == 0 && numel % 16 == 0 && (uintptr_t)mask % 16 == 0 && (uintptr_t)packed % 2 == 0 &&
+      numel / 16 < (1ll << 40)) {
+    const int64_t n_items = numel / 16;
+    hipLaunchKernelGGL(unpack_bitmasks_flat_kernel, (unsigned)cdiv(n_items, kBlock * kPackU), kBlock,
+                       0, (hipStream_t)stream, (const uint16_t*)packed, mask, n_items);
+    return check_launch("ctmi_unpack_bitmasks");
+  }
   hipLaunchKernelGGL(unpack_bitmasks_kernel, grid_for(rows * pc, kBlock), kBlock, 0,
                      (hipStream_t)stream, packed, mask, rows, cols, pc);
   return check_launch("ctmi_unpack_bitmasks");

@@ -10,7 +10,8 @@ pytestmark = pytest.mark.gpu
 FP8 = torch.float8_e4m3fn
 
 
-@pytest.mark.parametrize("shape", [(1, 1), (3, 7), (4, 8), (5, 17), (64, 4096), (2, 3, 20)])
+@pytest.mark.parametrize("shape", [(1, 1), (3, 7), (4, 8), (5, 17), (64, 4096), (2, 3, 20), (33, 4112),
+                                   (14336, 4096)])
 def test_pack_unpack_bitmasks(shape, gpu):
     from compressed_tensors_amd.utils import pack_bitmasks, unpack_bitmasks
 
@@ -20,6 +21,21 @@ def test_pack_unpack_bitmasks(shape, gpu):
     packed = pack_bitmasks(mask.to(gpu))
     assert_bit_equal(packed, osp.pack_bitmasks(mask), "pack_bitmasks")
     assert_bit_equal(unpack_bitmasks(packed, list(shape)), mask, "unpack_bitmasks")
+
+
+@pytest.mark.parametrize("shape", [(6, 40), (5, 17)], ids=["whole-words", "ragged"])
+def test_pack_bitmasks_of_bytes_that_are_not_0_or_1(shape, gpu):
+    """uint8 / int8 masks count as set wherever they are non-zero (numpy.packbits does the
+    same): single high bits, single low bits, 0xff"""
+    from compressed_tensors_amd.utils import pack_bitmasks
+
+    announce("bitmasks of arbitrary bytes", shape)
+    g = torch.Generator().manual_seed(3)
+    picks = torch.tensor([0, 0, 0, 1, 2, 0x40, 0x80, 0xFF, 0x7F, 0x81], dtype=torch.uint8)
+    mask = picks[torch.randint(0, len(picks), shape, generator=g)]
+    want = osp.pack_bitmasks(mask != 0)
+    assert_bit_equal(pack_bitmasks(mask.to(gpu)), want, "uint8")
+    assert_bit_equal(pack_bitmasks(mask.view(torch.int8).to(gpu)), want, "int8")
 
 
 def _sparse_tensor(shape, dtype, sparsity, seed):
