@@ -378,6 +378,8 @@ QS24 = [
     (dict(num_bits=8, type="int", symmetric=True, strategy="channel"), (40, 256), torch.bfloat16),
     (dict(num_bits=8, type="int", symmetric=False, strategy="channel"), (40, 256), torch.float32),
     (dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (8, 128), torch.bfloat16),
+    (dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[16, 64]), (48, 256), torch.bfloat16),
+    (dict(num_bits=8, type="int", symmetric=False, strategy="tensor"), (24, 64), torch.float16),
 ]
 
 
