@@ -4,6 +4,8 @@
 //   bitmask_compress / decompress       compressors/sparse_compressors/sparse_bitmask.py:131-169
 //   get_24_bytemasks                    compressors/sparse_compressors/sparse_24_bitmask.py:227-260
 //   sparse24_bitmask_compress / decompress   sparse_24_bitmask.py:162-224
+//   ... of a weight's int8 / fp8 codes, fused with quantize / dequantize
+//                                       model_compressors/model_compressor.py:572-604, 638-667
 //
 // Bit j of bitmask byte k of a row flags column 8k+j (numpy packbits,
 // bitorder="little"); the last byte of a row is zero padded.  Compacted values
@@ -24,9 +26,12 @@ __constant__ uint8_t kTopk24LutDev[4096] = CTMI_TOPK24_LUT_INIT;
 
 constexpr int kBlock = 256;
 constexpr int kWaves = kBlock / kWave;
-// work items per lane of the 2:4 streaming kernels (measured: compress 1 / 2 / 4 items
-// 4.27 / 4.16 / 3.94 TB/s, decompress 3.1 / 4.0 / 4.2)
-constexpr int kS24U = 2;         // compress
+// work items per lane of the 2:4 streaming kernels (measured on fp8 codes: compress
+// 1 / 2 / 4 / 8 items 5.3 / 5.4 / 5.0 / 4.7 TB/s, decompress 1 / 2 / 4 items 3.1 / 4.0 / 4.2)
+#ifndef CTMI_S24_U
+#define CTMI_S24_U 2
+#endif
+constexpr int kS24U = CTMI_S24_U;  // compress
 #ifndef CTMI_S24_SCATTER_U
 #define CTMI_S24_SCATTER_U 4
 #endif
