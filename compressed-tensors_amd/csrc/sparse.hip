@@ -329,6 +329,86 @@ row_offsets_kernel(const int64_t* __restrict__ counts, int64_t* __restrict__ off
 // gathered into LDS at their rank within the iteration, then the contiguous
 // run is written to HBM by the whole workgroup, so global stores are dense
 // regardless of where the non-zeros sit.
+// Rows of whole bitmask bytes, x aligned to 8 elements: 8192 columns per step.  A lane
+// issues its four bitmask bytes and four 16-byte loads before anything else; the four
+// counts ride through one workgroup scan as 16-bit fields of two words; the survivors
+// are laid out in LDS with the misalignment of their destination, so that what leaves
+// are aligned 16-byte stores (single elements only at the two ends).
+template <typename R>
+__global__ void __launch_bounds__(kBlock)
+bitmask_compact_rows_kernel(const R* __restrict__ x, const uint8_t* __restrict__ bitmask,
+                            const int64_t* __restrict__ row_offsets, R* __restrict__ values,
+                            int64_t rows, int64_t cols, int64_t pc) {
+  constexpr int U = 4;
+  constexpr int VE = 16 / (int)sizeof(R);
+  __shared__ uint32_t w01[kWaves], w23[kWaves];
+  __shared__ __align__(16) R stage[kBlock * 8 * U + VE];
+  const int tid = threadIdx.x, lane = lane_id(), wave = tid / kWave;
+  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+    const R* row = x + r * cols;
+    const uint8_t* mrow = bitmask + r * pc;
+    R* dst = values + row_offsets[r];
+    for (int64_t b0 = 0; b0 < pc; b0 += kBlock * U) {
+      uint32_t bits[U];
+      Vec<R, 8> a[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const int64_t b = b0 + k * kBlock + tid;
+        bits[k] = 0;
+        if (b < pc) {
+          bits[k] = mrow[b];
+          a[k] = ldg<R, 8>(row + b * 8);
+        }
+      }
+      const uint32_t c01 = (uint32_t)__popc(bits[0]) | ((uint32_t)__popc(bits[1]) << 16);
+      const uint32_t c23 = (uint32_t)__popc(bits[2]) | ((uint32_t)__popc(bits[3]) << 16);
+      const uint32_t inc01 = (uint32_t)wave_inclusive_scan((int)c01);
+      const uint32_t inc23 = (uint32_t)wave_inclusive_scan((int)c23);
+      if (lane == kWave - 1) {
+        w01[wave] = inc01;
+        w23[wave] = inc23;
+      }
+      __syncthreads();
+      uint32_t off01 = 0, off23 = 0, tot01 = 0, tot23 = 0;
+#pragma unroll
+      for (int w = 0; w < kWaves; ++w) {
+        const uint32_t s01 = w01[w], s23 = w23[w];
+        if (w < wave) { off01 += s01; off23 += s23; }
+        tot01 += s01;
+        tot23 += s23;
+      }
+      const uint32_t pre01 = off01 + inc01 - c01, pre23 = off23 + inc23 - c23;
+      const int tot[U] = {(int)(tot01 & 0xffffu), (int)(tot01 >> 16), (int)(tot23 & 0xffffu),
+                          (int)(tot23 >> 16)};
+      const int pre[U] = {(int)(pre01 & 0xffffu), (int)(pre01 >> 16), (int)(pre23 & 0xffffu),
+                          (int)(pre23 >> 16)};
+      const int mis = (int)(((uintptr_t)dst % 16) / sizeof(R));
+      int base = mis;
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        int at = base + pre[k];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+          if ((bits[k] >> j) & 1u) stage[at++] = a[k].v[j];
+        base += tot[k];
+      }
+      __syncthreads();
+      const int end = base;         // stage[mis, end) -> dst[0, end - mis)
+      R* dst_al = dst - mis;        // 16-byte aligned
+      for (int e0 = tid * VE; e0 < end; e0 += kBlock * VE) {
+        if (e0 >= mis && e0 + VE <= end) {
+          stg<R, VE>(dst_al + e0, *reinterpret_cast<const Vec<R, VE>*>(stage + e0));
+        } else {
+          for (int e = e0; e < e0 + VE; ++e)
+            if (e >= mis && e < end) dst_al[e] = stage[e];
+        }
+      }
+      dst += end - mis;
+      __syncthreads();
+    }
+  }
+}
+
 template <typename R>
 __global__ void __launch_bounds__(kBlock)
 bitmask_compact_kernel(const R* __restrict__ x, const uint8_t* __restrict__ bitmask,
@@ -1377,15 +1457,19 @@ extern "C" int ctmi_bitmask_compact(const void* x, int32_t elem_size, const uint
   hipStream_t st = (hipStream_t)stream;
   const int64_t pc = cdiv(cols, 8);
   const int grid = rows_grid(rows);
-  if (elem_size == 1)
-    hipLaunchKernelGGL(bitmask_compact_kernel<uint8_t>, grid, kBlock, 0, st, (const uint8_t*)x,
-                       bitmask, row_offsets, (uint8_t*)values, rows, cols, pc);
-  else if (elem_size == 2)
-    hipLaunchKernelGGL(bitmask_compact_kernel<uint16_t>, grid, kBlock, 0, st, (const uint16_t*)x,
-                       bitmask, row_offsets, (uint16_t*)values, rows, cols, pc);
-  else
-    hipLaunchKernelGGL(bitmask_compact_kernel<uint32_t>, grid, kBlock, 0, st, (const uint32_t*)x,
-                       bitmask, row_offsets, (uint32_t*)values, rows, cols, pc);
+  const bool whole = cols % 8 == 0 && (uintptr_t)x % (8 * (size_t)elem_size) == 0 &&
+                     (uintptr_t)values % (size_t)elem_size == 0;
+#define CTMI_COMPACT(R)                                                                          \
+  if (whole)                                                                                     \
+    hipLaunchKernelGGL(bitmask_compact_rows_kernel<R>, grid, kBlock, 0, st, (const R*)x, bitmask, \
+                       row_offsets, (R*)values, rows, cols, pc);                                 \
+  else                                                                                           \
+    hipLaunchKernelGGL(bitmask_compact_kernel<R>, grid, kBlock, 0, st, (const R*)x, bitmask,     \
+                       row_offsets, (R*)values, rows, cols, pc)
+  if (elem_size == 1) { CTMI_COMPACT(uint8_t); }
+  else if (elem_size == 2) { CTMI_COMPACT(uint16_t); }
+  else { CTMI_COMPACT(uint32_t); }
+#undef CTMI_COMPACT
   return check_launch("ctmi_bitmask_compact");
 }
 
