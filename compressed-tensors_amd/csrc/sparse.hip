@@ -191,6 +191,7 @@ bitmask_count_kernel(const R* __restrict__ x, uint32_t nz_mask, uint8_t* __restr
                      int64_t* __restrict__ counts, int64_t rows, int64_t cols, int64_t pc) {
   __shared__ int64_t red[kWaves];
   const bool vec = (cols % 8 == 0) && ((uintptr_t)x % (8 * sizeof(R)) == 0);
+  const bool words = vec && pc % 4 == 0 && (uintptr_t)bitmask % 4 == 0;
   for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
     const R* row = x + r * cols;
     int64_t cnt = 0;
@@ -204,6 +205,7 @@ bitmask_count_kernel(const R* __restrict__ x, uint32_t nz_mask, uint8_t* __restr
           const int64_t b = b0 + k * kBlock;
           a[k] = ldg<R, 8>(row + (b < pc ? b : pc - 1) * 8);  // past the end: re-read, not used
         }
+        uint32_t mine = 0;  // the lane's four bitmask bytes, byte k for vector k
 #pragma unroll
         for (int k = 0; k < U; ++k) {
           const int64_t b = b0 + k * kBlock;
@@ -211,9 +213,22 @@ bitmask_count_kernel(const R* __restrict__ x, uint32_t nz_mask, uint8_t* __restr
             uint32_t bits = 0;
 #pragma unroll
             for (int j = 0; j < 8; ++j) bits |= (uint32_t)(((uint32_t)a[k].v[j] & nz_mask) != 0) << j;
-            bitmask[r * pc + b] = (uint8_t)bits;
+            if (!words) bitmask[r * pc + b] = (uint8_t)bits;
+            mine |= bits << (8 * k);
             cnt += __popc(bits);
           }
+        }
+        if (words) {
+          // four neighbouring lanes hold four neighbouring bytes of each of the four
+          // vectors: lane q of the four collects vector q's and stores one 32-bit word
+          // (rows of whole words: the four lanes are inside the row together or not at all)
+          const int q = threadIdx.x & 3, base = lane_id() & ~3;
+          uint32_t word = 0;
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            word |= ((__shfl(mine, base + j, kWave) >> (8 * q)) & 0xffu) << (8 * j);
+          const int64_t at = b0 - q + (int64_t)q * kBlock;
+          if (at < pc) *reinterpret_cast<uint32_t*>(bitmask + r * pc + at) = word;
         }
       }
     } else {
