@@ -339,7 +339,7 @@ def other_workload(torch, name, seed):
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies * (n24 + n24 // 2 + n24 // 8)
         fused24_bytes = copies * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
-        ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_kernel"),
+        ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_rows_kernel"),
                Op("sparse-bitmask decompress (positions from the bitmask alone)", d_calls, bm_bytes, "bitmask_scatter_tiles_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),

@@ -203,7 +203,7 @@ bitmask_count_kernel(const R* __restrict__ x, uint32_t nz_mask, uint8_t* __restr
 #pragma unroll
         for (int k = 0; k < U; ++k) {
           const int64_t b = b0 + k * kBlock;
-          a[k] = ldg<R, 8>(row + (b < pc ? b : pc - 1) * 8);  // past the end: re-read, not used
+          a[k] = ldg_nt<R, 8>(row + (b < pc ? b : pc - 1) * 8);  // past the end: re-read, not used
         }
         uint32_t mine = 0;  // the lane's four bitmask bytes, byte k for vector k
 #pragma unroll
