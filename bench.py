@@ -283,7 +283,8 @@ def other_workload(torch, name, seed):
         cargs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="channel")
         from compressed_tensors_amd.compressors import get_24_bytemasks
         from compressed_tensors_amd.quantization import quantize
-        for _ in range(copies):
+        copies24 = 16  # values + bitmask of the codes are 37 MB a copy: well beyond the 256 MB last-level cache
+        for _ in range(copies24):
             w = randn(14336, 4096, 0.02)
             w = torch.where(get_24_bytemasks(w), w, torch.zeros_like(w))
             scale, _ = observe_weight_qparams(w, cargs)
@@ -337,16 +338,16 @@ def other_workload(torch, name, seed):
             back_two.append(lambda d=d, dq=dq: (_lib.check(lib.ctmi_sparse24_decompress(*d)), _lib.check(lib.ctmi_qdq(*dq))))
             back_one.append(lambda fd=fd: _lib.check(lib.ctmi_sparse24_decompress_dequantize(*fd)))
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
-        s24_bytes = copies * (n24 + n24 // 2 + n24 // 8)
-        fused24_bytes = copies * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
+        s24_bytes = copies24 * (n24 + n24 // 2 + n24 // 8)
+        fused24_bytes = copies24 * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
         ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_rows_kernel"),
                Op("sparse-bitmask decompress (positions from the bitmask alone)", d_calls, bm_bytes, "bitmask_scatter_tiles_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
-               Op("sparse-24-bitmask compress, 14336x4096 bf16", s16_calls, 2 * s24_bytes - copies * (n24 // 8), "sparse24_compress_kernel"),
-               Op("sparse-24-bitmask decompress, bf16", t16_calls, 2 * s24_bytes - copies * (n24 // 8), "sparse24_scatter_kernel"),
-               Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies * (n24 + n24 // 8), "pack_bitmasks"),
-               Op("unpack_bitmasks", up_calls, copies * (n24 + n24 // 8), "unpack_bitmasks"),
+               Op("sparse-24-bitmask compress, 14336x4096 bf16", s16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_compress_kernel"),
+               Op("sparse-24-bitmask decompress, bf16", t16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel"),
+               Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies24 * (n24 + n24 // 8), "pack_bitmasks"),
+               Op("unpack_bitmasks", up_calls, copies24 * (n24 + n24 // 8), "unpack_bitmasks"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
                Op("bf16 -> fp8 codes -> 2:4 compress, one pass", one_step, fused24_bytes, "quant_sparse24_compress_kernel"),
                Op("2:4 decompress -> fp8 codes -> bf16, two steps", back_two, fused24_bytes, "qdq_vec_kernel", primary=False),
@@ -359,7 +360,8 @@ def other_workload(torch, name, seed):
         ops = []
         for r, c in ((14336, 4096), (4096, 14336)):
             c_calls, d_calls = [], []
-            for _ in range(5):
+            n_copies = 16  # the packed side (33 MB a copy) has to exceed the 256 MB last-level cache too
+            for _ in range(n_copies):
                 w = randn(r, c, 0.02)
                 gs = generate_gparam(w.min().reshape(1), w.max().reshape(1))
                 scale, zp = observe_weight_qparams(w, args, global_scale=gs)
@@ -372,9 +374,9 @@ def other_workload(torch, name, seed):
                 da = (packed.data_ptr(), dense.data_ptr(), code(dense.dtype), r, c, ctypes.byref(dp.qp), st)
                 c_calls.append(lambda ca=ca: _lib.check(lib.ctmi_nvfp4_compress(*ca)))
                 d_calls.append(lambda da=da: _lib.check(lib.ctmi_nvfp4_decompress(*da)))
-            nbytes = 5 * (2 * r * c + r * c // 16 + r * c // 2)
-            ops += [Op(f"nvfp4 compress {r}x{c} (x5)", c_calls, nbytes, "nvfp4_compress_vec_kernel"),
-                    Op(f"nvfp4 decompress {r}x{c} (x5)", d_calls, nbytes, "nvfp4_decompress_vec_kernel")]
+            nbytes = n_copies * (2 * r * c + r * c // 16 + r * c // 2)
+            ops += [Op(f"nvfp4 compress {r}x{c} (x{n_copies})", c_calls, nbytes, "nvfp4_compress_vec_kernel"),
+                    Op(f"nvfp4 decompress {r}x{c} (x{n_copies})", d_calls, nbytes, "nvfp4_decompress_vec_kernel")]
         # the Llama-3-8B-shaped set: one call per weight against all 224 in one call
         from compressed_tensors_amd.compressors import Fp4WeightBatch
         entries, single_c, single_d, n_set = [], [], [], 0

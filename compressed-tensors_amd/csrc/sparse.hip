@@ -372,7 +372,7 @@ bitmask_compact_rows_kernel(const R* __restrict__ x, const uint8_t* __restrict__
         bits[k] = 0;
         if (b < pc) {
           bits[k] = mrow[b];
-          a[k] = ldg<R, 8>(row + b * 8);
+          a[k] = ldg_nt<R, 8>(row + b * 8);
         }
       }
       const uint32_t c01 = (uint32_t)__popc(bits[0]) | ((uint32_t)__popc(bits[1]) << 16);
