@@ -201,6 +201,11 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
     ),
+    "ctmi_bitmask_decompress_static_max_bytes": (c_int64, []),
+    "ctmi_bitmask_decompress_static": (
+        c_int32,
+        [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int64, c_int64, c_void_p],
+    ),
     "ctmi_hadamard_quant_pack": (
         c_int32,
         [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int32,

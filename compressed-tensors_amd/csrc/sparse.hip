@@ -10,6 +10,7 @@
 // Bit j of bitmask byte k of a row flags column 8k+j (numpy packbits,
 // bitorder="little"); the last byte of a row is zero padded.  Compacted values
 // are stored in row-major order of the set bits.
+#include <mutex>
 #include <type_traits>
 
 #include "ctmi_device.h"
@@ -1488,15 +1489,24 @@ extern "C" int ctmi_bitmask_compact(const void* x, int32_t elem_size, const uint
   return check_launch("ctmi_bitmask_compact");
 }
 
-static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
-                         const uint8_t* bitmask, const int64_t* row_offsets, void* out, void* tmp,
-                         int64_t rows, int64_t cols, void* stream, bool try_24, const char* what) {
+// argument checks of the scatter entry points (no HIP call)
+static int scatter_check(const void* values, int64_t nvalues, int32_t elem_size,
+                         const uint8_t* bitmask, void* out, int64_t rows, int64_t cols) {
   CTMI_REQUIRE(rows >= 0 && cols >= 0, CTMI_ERR_VALUE, "negative shape");
   int rc = check_elem(elem_size);
   if (rc) return rc;
   if (rows == 0 || cols == 0) return CTMI_OK;
   CTMI_REQUIRE(bitmask && out, CTMI_ERR_VALUE, "NULL tensor pointer");
   CTMI_REQUIRE(nvalues >= 0 && (values || nvalues == 0), CTMI_ERR_VALUE, "bad values buffer");
+  return CTMI_OK;
+}
+
+static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
+                         const uint8_t* bitmask, const int64_t* row_offsets, void* out, void* tmp,
+                         int64_t rows, int64_t cols, void* stream, bool try_24, const char* what) {
+  int rc = scatter_check(values, nvalues, elem_size, bitmask, out, rows, cols);
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
   CTMI_REQUIRE(row_offsets || tmp, CTMI_ERR_VALUE, "row_offsets and tmp are both NULL");
   hipStream_t st = (hipStream_t)stream;
   const int64_t pc = cdiv(cols, 8);
@@ -1599,6 +1609,60 @@ extern "C" int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int3
                                        void* stream) {
   return scatter_entry(values, nvalues, elem_size, bitmask, row_offsets, out, tmp, rows, cols,
                        stream, false, "ctmi_bitmask_decompress");
+}
+
+// ---- ctmi_bitmask_decompress for callers that cannot allocate: the scratch of the
+// scatter kernels (per-tile set-bit counts and group totals, or per-row counts and
+// offsets) lives in this file-scope device array instead of a caller's buffer.
+// Every GPU holds its own copy at its own address; host code reaches it only
+// through the address hipGetSymbolAddress returns for the current device.
+constexpr int64_t kStaticScratchBytes = 4ll << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+constexpr int kMaxScratchDevices = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[kMaxScratchDevices];  // per device, filled on first use
+
+// device address of `scratch` on the current device
+static int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "hipGetDevice: %s", hipGetErrorString(e));
+  CTMI_REQUIRE(dev >= 0 && dev < kMaxScratchDevices, CTMI_ERR_UNSUPPORTED,
+               "device index %d is beyond the %d devices the static scratch table holds", dev,
+               kMaxScratchDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr)
+      return set_error(CTMI_ERR_HIP, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return CTMI_OK;
+}
+
+extern "C" int64_t ctmi_bitmask_decompress_static_max_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int ctmi_bitmask_decompress_static(const void* values, int64_t nvalues,
+                                              int32_t elem_size, const uint8_t* bitmask, void* out,
+                                              int64_t rows, int64_t cols, void* stream) {
+  int rc = scatter_check(values, nvalues, elem_size, bitmask, out, rows, cols);
+  if (rc) return rc;
+  if (rows == 0 || cols == 0) return CTMI_OK;
+  const int64_t need = ctmi_bitmask_tmp_bytes(rows, cols);
+  CTMI_REQUIRE(need <= kStaticScratchBytes, CTMI_ERR_VALUE,
+               "a [%lld, %lld] tensor needs %lld bytes of scratch, the static buffer holds %lld: "
+               "use ctmi_bitmask_decompress with a caller-owned buffer",
+               (long long)rows, (long long)cols, (long long)need, (long long)kStaticScratchBytes);
+  void* tmp = nullptr;
+  rc = static_scratch(&tmp);
+  if (rc) return rc;
+  // the kernels write every scratch word they later read (counts of all tiles or rows
+  // of THIS call), so what an earlier call left behind needs no clearing
+  return scatter_entry(values, nvalues, elem_size, bitmask, nullptr, out, tmp, rows, cols, stream,
+                       false, "ctmi_bitmask_decompress_static");
 }
 
 extern "C" int ctmi_sparse24_decompress(const void* values, int64_t nvalues, int32_t elem_size,

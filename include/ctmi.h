@@ -222,6 +222,22 @@ int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_si
                             const int64_t* row_offsets, void* out, void* tmp, int64_t rows,
                             int64_t cols, void* stream);
 
+/* ctmi_bitmask_decompress without a scratch argument.  No counterpart in the
+ * reference: it exists for callers that cannot allocate device memory (code under
+ * HIP graph capture, serving loops and harnesses that forbid hipMalloc).  The
+ * scratch of the scatter kernels lives in a device array inside the library,
+ * ctmi_bitmask_decompress_static_max_bytes() bytes (4 MiB) per GPU, held until the
+ * process ends; a shape with ctmi_bitmask_tmp_bytes(rows, cols) above that is
+ * refused with CTMI_ERR_VALUE.  The entry point calls no allocating routine.
+ * Positions come from the bitmask alone (the `tmp` mode of
+ * ctmi_bitmask_decompress); same bits.  All calls on one GPU share that GPU's
+ * array: calls that overlap on one GPU (two streams, two threads) race; calls
+ * enqueued on one stream do not, and nothing needs clearing between them. */
+int64_t ctmi_bitmask_decompress_static_max_bytes(void);
+int ctmi_bitmask_decompress_static(const void* values, int64_t nvalues, int32_t elem_size,
+                                   const uint8_t* bitmask, void* out, int64_t rows, int64_t cols,
+                                   void* stream);
+
 /* A22.  sparse24_bitmask_decompress (sparse_24_bitmask.py:206-224): the same
  * scatter, `out[mask] = values`, for any bitmask.  A bitmask that keeps exactly 2
  * of every 4 columns (what the format holds) needs no prefix sums and is
