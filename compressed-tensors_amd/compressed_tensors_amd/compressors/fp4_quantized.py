@@ -12,7 +12,9 @@ from torch import Tensor
 
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
-from compressed_tensors_amd.compressors.quantized_base import BaseQuantizationCompressor
+from compressed_tensors_amd.compressors.quantized_base import (
+    BaseQuantizationCompressor, LazyDenseOutputs,
+)
 from compressed_tensors_amd.config import CompressionFormat
 from compressed_tensors_amd.quantization.forward import (
     _ShapeOnly,
@@ -179,7 +181,7 @@ class NVFP4PackedCompressor(BaseQuantizationCompressor):
         return out
 
 
-class Fp4WeightBatch:
+class Fp4WeightBatch(LazyDenseOutputs):
     """Every nvfp4 weight of a state dict prepared for one-call compress / decompress
     (ctmi_nvfp4_{compress,decompress}_many).  Buffers are allocated once; `compress()`
     and `decompress()` only enqueue kernels."""
@@ -189,7 +191,7 @@ class Fp4WeightBatch:
         quantization_args, optionally zero_point"""
         self.n = len(entries)
         self._keep = []
-        self.weights, self.packed, self.dense = [], [], []
+        self.weights, self.packed = [], []
         self._cjobs = (_lib.WeightJob * max(self.n, 1))()
         self._djobs = (_lib.WeightJob * max(self.n, 1))()
         self.device = None
@@ -211,16 +213,15 @@ class Fp4WeightBatch:
             dplan = build_qparams(carrier, scale, None, dq_args, None, gs)
             dplan.qp.qtype, dplan.qp.num_bits = _lib.QTYPE_FLOAT, 4
             out_dtype = torch.bfloat16 if dplan.grouped else dplan.dequant_dtype
-            dense = torch.empty((rows, cols), dtype=out_dtype, device=w.device)
+            self._plan_dense((rows, cols), out_dtype, w.device)
             self._keep += [cplan, dplan]
             cj, dj = self._cjobs[i], self._djobs[i]
             cj.src, cj.dst, cj.rows, cj.cols = w.data_ptr(), packed.data_ptr(), rows, cols
             cj.dense_dtype, cj.qp = _lib.dtype_code(w.dtype), cplan.qp
-            dj.src, dj.dst, dj.rows, dj.cols = packed.data_ptr(), dense.data_ptr(), rows, cols
+            dj.src, dj.rows, dj.cols = packed.data_ptr(), rows, cols  # dst: _ensure_dense
             dj.dense_dtype, dj.qp = _lib.dtype_code(out_dtype), dplan.qp
             self.weights.append(w)
             self.packed.append(packed)
-            self.dense.append(dense)
 
     def compress(self):
         """enqueue quantize + pack of every weight; returns the packed tensors"""
@@ -229,10 +230,12 @@ class Fp4WeightBatch:
         return self.packed
 
     def decompress(self):
-        """enqueue unpack + dequantize of every packed weight; returns the dense tensors"""
+        """enqueue unpack + dequantize of every packed weight; returns the dense tensors
+        (allocated at the first call)"""
+        dense = self._ensure_dense()
         if self.n:
             _lib.check(_lib.load().ctmi_nvfp4_decompress_many(self._djobs, self.n, _lib.stream_of(self.device)))
-        return self.dense
+        return dense
 
 
 def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,

@@ -10,7 +10,9 @@ from torch import Tensor
 
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
-from compressed_tensors_amd.compressors.quantized_base import BaseQuantizationCompressor
+from compressed_tensors_amd.compressors.quantized_base import (
+    BaseQuantizationCompressor, LazyDenseOutputs,
+)
 from compressed_tensors_amd.config import CompressionFormat
 from compressed_tensors_amd.quantization.forward import (
     _rows_cols, _ShapeOnly, build_qparams, dequantize, infer_dequant_args, quantize,
@@ -27,10 +29,12 @@ __all__ = [
 ]
 
 
-class QuantizedWeightBatch:
+class QuantizedWeightBatch(LazyDenseOutputs):
     """Every weight of a state dict prepared for one-call quantize / dequantize
     (ctmi_qdq_many): codes in int8 or float8_e4m3fn as the scheme says, buffers
     allocated once, `compress()` / `decompress()` only enqueue kernels."""
+
+    _dense_field = "out"
 
     def __init__(self, entries, device=None):
         """entries: dicts with weight, scale, quantization_args and optionally
@@ -38,7 +42,7 @@ class QuantizedWeightBatch:
         self.n = len(entries)
         self.device = device
         self._keep = []
-        self.weights, self.codes, self.dense = [], [], []
+        self.weights, self.codes = [], []
         self._cjobs = (_lib.QdqJob * max(self.n, 1))()
         self._djobs = (_lib.QdqJob * max(self.n, 1))()
         for i, e in enumerate(entries):
@@ -49,7 +53,7 @@ class QuantizedWeightBatch:
             w = w.contiguous()
             rows, cols = _rows_cols(w)
             codes = torch.empty(w.shape, dtype=args.pytorch_dtype(), device=w.device)
-            dense = torch.empty(w.shape, dtype=scale.dtype, device=w.device)
+            self._plan_dense(w.shape, scale.dtype, w.device)
             cplan = build_qparams(w, scale, zp, args, g_idx, None)
             dq_args = infer_dequant_args(_ShapeOnly(w.shape, codes.dtype), scale)
             # a symmetric scheme stores no zero points: its decompression sees none
@@ -59,11 +63,10 @@ class QuantizedWeightBatch:
             cj, dj = self._cjobs[i], self._djobs[i]
             cj.x, cj.out, cj.rows, cj.cols = w.data_ptr(), codes.data_ptr(), rows, cols
             cj.x_dtype, cj.out_dtype, cj.qp = _lib.dtype_code(w.dtype), _lib.dtype_code(codes.dtype), cplan.qp
-            dj.x, dj.out, dj.rows, dj.cols = codes.data_ptr(), dense.data_ptr(), rows, cols
-            dj.x_dtype, dj.out_dtype, dj.qp = _lib.dtype_code(codes.dtype), _lib.dtype_code(dense.dtype), dplan.qp
+            dj.x, dj.rows, dj.cols = codes.data_ptr(), rows, cols  # out: _ensure_dense
+            dj.x_dtype, dj.out_dtype, dj.qp = _lib.dtype_code(codes.dtype), _lib.dtype_code(scale.dtype), dplan.qp
             self.weights.append(w)
             self.codes.append(codes)
-            self.dense.append(dense)
 
     def compress(self):
         """enqueue the quantization of every weight; returns the code tensors"""
@@ -71,9 +74,11 @@ class QuantizedWeightBatch:
         return self.codes
 
     def decompress(self):
-        """enqueue the dequantization of every code tensor; returns the dense tensors"""
+        """enqueue the dequantization of every code tensor; returns the dense tensors
+        (allocated at the first call)"""
+        dense = self._ensure_dense()
         _lib.check(_lib.load().ctmi_qdq_many(self._djobs, self.n, 0, 1, _lib.stream_of(self.device)))
-        return self.dense
+        return dense
 
 
 def observe_and_compress_weights(weights, quantization_args: QuantizationArgs):

@@ -15,7 +15,9 @@ from torch import Tensor
 
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
-from compressed_tensors_amd.compressors.quantized_base import BaseQuantizationCompressor
+from compressed_tensors_amd.compressors.quantized_base import (
+    BaseQuantizationCompressor, LazyDenseOutputs,
+)
 from compressed_tensors_amd.config import CompressionFormat
 from compressed_tensors_amd.quantization.forward import (
     _ShapeOnly,
@@ -271,7 +273,7 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         return out
 
 
-class PackedWeightBatch:
+class PackedWeightBatch(LazyDenseOutputs):
     """Every weight of a state dict prepared for one-call compress / decompress.
 
     Holds the dense weights, their qparams, the packed outputs and the job
@@ -288,7 +290,7 @@ class PackedWeightBatch:
         self.n = len(entries)
         self.names = [e.get("name", str(i)) for i, e in enumerate(entries)]
         self._keep = []
-        self.weights, self.packed, self.dense, self.scales = [], [], [], []
+        self.weights, self.packed, self.scales = [], [], []
         self._cjobs = (_lib.WeightJob * max(self.n, 1))()
         self._djobs = (_lib.WeightJob * max(self.n, 1))()
         self.device = device
@@ -305,7 +307,7 @@ class PackedWeightBatch:
                 raise ValueError("Packing is only supported for less than 8 bits")
             pf = 32 // args.num_bits
             packed = torch.empty((rows, math.ceil(cols / pf)), dtype=torch.int32, device=w.device)
-            dense = torch.empty((rows, cols), dtype=scale.dtype, device=w.device)
+            self._plan_dense((rows, cols), scale.dtype, w.device)
             cplan = build_qparams(w, scale, zp, args, g_idx, None)
             dq_args = infer_dequant_args(_ShapeOnly(w.shape, torch.int8), scale)
             use_zp = (not args.symmetric) if decompress_zero_points is None else decompress_zero_points
@@ -316,11 +318,10 @@ class PackedWeightBatch:
             cj, dj = self._cjobs[i], self._djobs[i]
             cj.src, cj.dst, cj.rows, cj.cols = w.data_ptr(), packed.data_ptr(), rows, cols
             cj.dense_dtype, cj.qp = _lib.dtype_code(w.dtype), cplan.qp
-            dj.src, dj.dst, dj.rows, dj.cols = packed.data_ptr(), dense.data_ptr(), rows, cols
+            dj.src, dj.rows, dj.cols = packed.data_ptr(), rows, cols  # dst: _ensure_dense
             dj.dense_dtype, dj.qp = _lib.dtype_code(scale.dtype), dplan.qp
             self.weights.append(w)
             self.packed.append(packed)
-            self.dense.append(dense)
             self.scales.append(scale)
 
     def compress(self):
@@ -333,6 +334,8 @@ class PackedWeightBatch:
 
     def launches(self, compress=True):
         """number of kernel launches one compress() (or decompress()) pass enqueues"""
+        if not compress:
+            self._ensure_dense()
         jobs = self._cjobs if compress else self._djobs
         count = _lib.load().ctmi_pack_quantized_launches(jobs, self.n, 1 if compress else 0)
         if count < 0:
@@ -340,12 +343,14 @@ class PackedWeightBatch:
         return int(count)
 
     def decompress(self):
-        """enqueue unpack+dequantize of every packed weight; returns the dense tensors"""
+        """enqueue unpack+dequantize of every packed weight; returns the dense tensors
+        (allocated at the first call)"""
+        dense = self._ensure_dense()
         _lib.check(
             _lib.load().ctmi_pack_quantized_decompress_many(self._djobs, self.n,
                                                             _lib.stream_of(self.device))
         )
-        return self.dense
+        return dense
 
 
 class ObservedWeightBatch:
