@@ -302,17 +302,18 @@ column_rank_zero_kernel(int32_t* __restrict__ rank, int cols) {
 
 __global__ void __launch_bounds__(256)
 column_rank_kernel(const int32_t* __restrict__ g, int32_t* __restrict__ rank, int cols) {
-  __shared__ uint32_t key[kRankTile];
+  __shared__ uint64_t key[kRankTile];
   const int c = blockIdx.x * 256 + threadIdx.x;
   const int base = blockIdx.y * kRankTile;
-  // (g, column) as one unsigned key: cols < 2^16 and g < 2^15 (checked on the host)
+  // (g, column) as one unsigned key that orders like the signed pair: any int32 g
   for (int i = threadIdx.x; i < kRankTile; i += 256) {
     const int c2 = base + i;
-    key[i] = c2 < cols ? (((uint32_t)g[c2] & 0x7fffu) << 16) | (uint32_t)c2 : 0xffffffffu;
+    key[i] = c2 < cols ? ((uint64_t)((uint32_t)g[c2] ^ 0x80000000u) << 32) | (uint32_t)c2
+                       : ~0ull;
   }
   __syncthreads();
   if (c >= cols) return;
-  const uint32_t mine = (((uint32_t)g[c] & 0x7fffu) << 16) | (uint32_t)c;
+  const uint64_t mine = ((uint64_t)((uint32_t)g[c] ^ 0x80000000u) << 32) | (uint32_t)c;
   int below = 0;
 #pragma unroll 8
   for (int i = 0; i < kRankTile; ++i) below += key[i] < mine ? 1 : 0;

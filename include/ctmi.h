@@ -439,7 +439,8 @@ int ctmi_mxfp4_convert_exp_scale(const uint8_t* exps, void* out, int32_t out_dty
  * group_size.  col_group[c] = (place of column c in a stable sort by g_idx) /
  * group_size is that rule as a per-column group index, the form ctmi_qparams
  * takes; a g_idx that holds a -1 is unset and gives column order (c / group_size).
- * g_idx values must lie in [-1, 32767], cols < 65536.  No scratch, no host sync. */
+ * g_idx may hold any int32 values (they are ordered as signed integers, like
+ * torch.argsort orders them); cols < 65536.  No scratch, no host sync. */
 int ctmi_column_groups(const int32_t* g_idx, int64_t cols, int64_t group_size,
                        int32_t* col_group, void* stream);
 

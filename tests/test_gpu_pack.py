@@ -291,6 +291,36 @@ def test_pack_quantized_with_activation_ordering(spec, shape, dtype, sdt, gpu):
     assert_bit_equal(dense, dense_want, "decompress")
 
 
+def test_activation_ordering_with_any_int32_group_labels(gpu):
+    """g_idx values are only ever sorted (forward.py:286-289), so labels beyond 32767 and
+    negative ones other than -1 must group the columns like small ones; a -1 anywhere
+    means the ordering is unset"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=64)
+    args, oargs = _pair(spec)
+    announce("pack-quantized g_idx with wide labels")
+    g = torch.Generator().manual_seed(35)
+    rows, cols = 24, 512
+    w = (torch.randn(rows, cols, generator=g) * 0.02).bfloat16()
+    small = (torch.randperm(cols, generator=g) // 64).to(torch.int32)
+    scale, _ = oq.observe_weight(w.index_select(-1, torch.argsort(small)), oargs)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    want = op.pack_quantized_compress(w, scale, oargs, g_idx=small)["weight_packed"]
+    for name, labels in [("wide", small.long() * 70001 - 200000),
+                         ("int32 extremes", small.long() * 613566756 - 2147483647)]:
+        labels = labels.to(torch.int32)
+        assert_bit_equal(op.pack_quantized_compress(w, scale, oargs, g_idx=labels)["weight_packed"], want, name)
+        got = comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+                                   g_idx=labels.to(gpu))["weight_packed"]
+        assert_bit_equal(got, want, name)
+    unset = small.clone()
+    unset[5] = -1
+    got = comp.compress_weight(weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+                               g_idx=unset.to(gpu))["weight_packed"]
+    assert_bit_equal(got, op.pack_quantized_compress(w, scale, oargs)["weight_packed"], "unset")
+
+
 NQ = [
     ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (96, 512), torch.bfloat16),
     ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="tensor"), (31, 65), torch.float16),

@@ -182,7 +182,7 @@ def test_static_weight_golden(case):
     scale, zp = quant.observe_weight(w, args, global_scale=gs)
     out = quant.fake_quantize(w, scale, zp, args, global_scale=gs)
     want = torch.tensor(case["qdq"]).to(out.dtype)
-    assert torch.allclose(out, want)
+    assert torch.equal(out, want)
     assert torch.nn.functional.mse_loss(out.float(), w.float()) <= case["max_mse"]
 
 
@@ -202,7 +202,7 @@ def test_static_activation_golden(case):
         assert float(mn) == case["min"][0] and float(mx) == case["max"][0]
         scale, zp = quant.calculate_qparams(mn.reshape(1), mx.reshape(1), args)
     out = quant.fake_quantize(x, scale, zp, args, global_scale=gs)
-    assert torch.allclose(out, torch.tensor(case["qdq"]).to(out.dtype))
+    assert torch.equal(out, torch.tensor(case["qdq"]).to(out.dtype))
     assert torch.nn.functional.mse_loss(out.float(), x.float()) <= case["max_mse"]
 
 
@@ -440,5 +440,5 @@ def test_static_attention_golden(case):
     assert torch.equal(mx.float(), torch.tensor(case["max"]))
     scale, zp = quant.calculate_qparams(mn, mx, args)
     out = quant.fake_quantize(x, scale, zp, args)
-    assert torch.allclose(out, torch.tensor(case["qdq"]).to(out.dtype))
+    assert torch.equal(out, torch.tensor(case["qdq"]).to(out.dtype))
     assert torch.nn.functional.mse_loss(out.float(), x.float()) <= case["max_mse"]
