@@ -8,6 +8,13 @@ dequantized (decompress).  Inputs, scales and output buffers are resident in
 HBM before the timed region; scales are computed beforehand by the fused
 min-max observer (not timed).  Prints ONE JSON line.
 
+With no --workload the line is the headline (llama3-8b-w4a16) and carries, under
+"configs", a short run of every other configuration below (its operations, the
+roofline fraction of its dominant kernel, MFMA utilisation for the Hadamard
+kernels, its own CPU baseline) and, under "api_level", ModelCompressor.compress_model
+/ decompress_model timed on a 224-Linear module tree of the same shapes.
+--only-headline leaves those out.
+
 Workloads
   llama3-8b-w4a16   (default) 32 x {q,o 4096x4096; k,v 1024x4096; gate,up 14336x4096;
                     down 4096x14336} bf16 N(0, 0.02), symmetric int4, group 128
@@ -25,6 +32,8 @@ that no pass finds its input in the last-level cache:
                     quantize and pack, as separate passes and as one
   hadamard          block-128 and full 4096 rotations of 8192 x 4096 activations and of
                     4096 x 4096 / 14336 x 4096 weights
+  api               ModelCompressor.compress_model / decompress_model on a module tree of the
+                    default set's 224 weights (wall time of the host mirror above the C ABI)
 """
 import argparse
 import json
@@ -51,14 +60,43 @@ LLAMA3_8B_LAYER = [
 ]
 GROUP = 128
 
-# HBM bytes per launch of the two fused kernels, averaged over the launches of one
-# pass: rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch), each scaled
-# by what the same counter reads for a plain 1 GiB copy (FETCH_SIZE reads 0.5000 of the
-# bytes copied, WRITE_SIZE 1.0000).  The summaries are profiles/pmc_traffic_*.txt.
-MEASURED_TRAFFIC = {
-    ("llama3-8b-w4a16", "pq_compress_vec_kernel"): 631.0e6,
-    ("llama3-8b-w4a16", "pq_decompress_vec_kernel"): 627.2e6,
-}
+PROFILES = ROOT / "profiles"
+MFMA_BF16_PEAK = 2.5e15  # dense bf16 MFMA, published peak
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch from the committed counter summaries: lines of the form
+    `traffic_bytes_per_launch <workload> <kernel> <bytes>` in profiles/*pmc_traffic*.txt
+    (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, KiB per dispatch, each scaled by what
+    the same counter reads for a plain 1 GiB copy).  -> (bytes or None, file name or None)"""
+    for path in sorted(PROFILES.glob("*pmc_traffic*.txt")):
+        for line in path.read_text().splitlines():
+            f = line.split()
+            if len(f) == 4 and f[0] == "traffic_bytes_per_launch" and f[1] == workload and f[2] == kernel:
+                return float(f[3]), f"profiles/{path.name}"
+    return None, None
+
+
+def cpu_threads():
+    """threads the CPU baseline runs on: every core this process may use (its affinity
+    mask, capped by OMP_NUM_THREADS where the host sets one for its share of the machine)"""
+    n = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else (os.cpu_count() or 1)
+    cap = os.environ.get("OMP_NUM_THREADS", "")
+    if cap.isdigit() and int(cap) > 0:
+        n = min(n, int(cap))
+    return max(n, 1)
+
+
+def median_time(run, repeats=5):
+    """median of `repeats` timed runs after one warm-up"""
+    times = []
+    for it in range(repeats + 1):
+        t0 = time.perf_counter()
+        run()
+        dt = time.perf_counter() - t0
+        if it:
+            times.append(dt)
+    return statistics.median(times)
 
 
 def shapes_for(workload: str):
@@ -82,32 +120,29 @@ def cpu_baseline(torch, sample_shapes, seed):
     from oracle import pack as opack
     from oracle import quant as oquant
 
-    threads = os.cpu_count() or 1
-    threads = min(threads, 16)
+    threads = cpu_threads()
     torch.set_num_threads(threads)
     oargs = oquant._Args(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
     g = torch.Generator().manual_seed(seed)
     ws = [(torch.randn(r, c, generator=g) * 0.02).bfloat16() for _, r, c in sample_shapes]
     qps = [oquant.observe_weight(w, oargs) for w in ws]
     per_dir, _ = algorithmic_bytes(sample_shapes)
-    times = []
-    for it in range(4):
-        t0 = time.perf_counter()
+
+    def run():
         for w, (s, z) in zip(ws, qps):
             data = opack.pack_quantized_compress(w, s, oargs, zero_point=z)
             data["weight_scale"] = s
             opack.pack_quantized_decompress(data, oargs)
-        dt = time.perf_counter() - t0
-        if it:  # first pass is the warm-up
-            times.append(dt)
-    med = statistics.median(times)
+
+    med = median_time(run)
     return {
         "value": 2 * per_dir / med / 1e9,
         "unit": "GB/s",
         "cores": threads,
+        "host_cpu_count": os.cpu_count(),
         "kind": "port",
         "sample": "compress+decompress of " + " + ".join(f"{r}x{c}" for _, r, c in sample_shapes)
-        + f" bf16 (W4A16 g128), median of 3 after 1 warm-up, torch {torch.__version__} CPU",
+        + f" bf16 (W4A16 g128), median of 5 after 1 warm-up, torch {torch.__version__} CPU",
         "seconds": med,
     }
 
@@ -118,9 +153,10 @@ class Op:
     """primary=False: an operation that is only there to be compared with (the separate steps a
     fused operation replaces, one call per weight against one call for all)"""
 
-    def __init__(self, name, calls, nbytes, kernel, primary=True):
+    def __init__(self, name, calls, nbytes, kernel, primary=True, mfma_flops=None):
         self.name, self.calls, self.nbytes, self.kernel = name, calls, nbytes, kernel
         self.primary = primary
+        self.mfma_flops = mfma_flops  # flops the kernel issues on the matrix cores, per pass
         self.ms = 0.0
 
 
@@ -387,6 +423,7 @@ def other_workload(torch, name, seed):
             entries.append(dict(weight=w, scale=scale, global_scale=gs, quantization_args=args))
             n_set += r * c
         batch = Fp4WeightBatch(entries)
+        batch.dense  # allocate the decompress side now: its addresses go into the per-weight calls
         keep.append(batch)
         for i in range(batch.n):
             cj, dj = batch._cjobs[i], batch._djobs[i]
@@ -466,9 +503,14 @@ def other_workload(torch, name, seed):
                          _lib.ptr(ma), mb.data_ptr(), q.data_ptr(), None, st)
                     calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
                 nb = sum(4 * x.numel() for x in xs)
+                # matrix-core flops per element: 2 b for the one product of a block-b rotation;
+                # 2 b + 3 * 2 a for a Kronecker pair (the fp32 result of the first product goes
+                # into the second as three bf16 terms)
+                per_elem = 2 * b_dim if a_dim == 1 else 2 * b_dim + 6 * a_dim
+                flops = sum(per_elem * x.numel() for x in xs)
                 ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb,
                               "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
-                              primary=not label.startswith("weights 4096x4096")))
+                              primary=not label.startswith("weights 4096x4096"), mfma_flops=flops))
                 if label.startswith("weights 4096x4096"):
                     jobs = (_lib.HadamardJob * len(xs))()
                     outs = [torch.empty_like(x) for x in xs]
@@ -479,7 +521,8 @@ def other_workload(torch, name, seed):
                          q.data_ptr(), None, st)
                     ops.append(Op(f"random-sign Hadamard, size {n}: {label}, one call (8 per launch)",
                                   [lambda m=m: _lib.check(lib.ctmi_hadamard_apply_many(*m))], nb,
-                                  "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel"))
+                                  "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
+                                  mfma_flops=flops))
         # rotation (block 128) + symmetric int4 group-128 quantization + pack_to_int32, one pass
         mb = deterministic_hadamard_matrix(128, torch.bfloat16, dev).contiguous()
         q = (torch.randint(0, 2, (128,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
@@ -494,8 +537,10 @@ def other_workload(torch, name, seed):
                      4, 1, packed.data_ptr(), scale.data_ptr(), None, st)
                 calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_quant_pack(*a)))
             nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in tensors[label])
+            flops = sum(2 * 128 * x.numel() for x in tensors[label])
             ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}", calls, nb,
-                          "hadamard_quant_pack_kernel", primary=not label.startswith("weights 4096x4096")))
+                          "hadamard_quant_pack_kernel", primary=not label.startswith("weights 4096x4096"),
+                          mfma_flops=flops))
             if label.startswith("weights 4096x4096"):
                 xs = tensors[label]
                 jobs = (_lib.HadamardPackJob * len(xs))()
@@ -509,7 +554,7 @@ def other_workload(torch, name, seed):
                 m = (jobs, len(xs), code(xs[0].dtype), 128, mb.data_ptr(), q.data_ptr(), None, 4, 1, st)
                 ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
                               [lambda m=m: _lib.check(lib.ctmi_hadamard_quant_pack_many(*m))], nb,
-                              "hadamard_quant_pack_kernel"))
+                              "hadamard_quant_pack_kernel", mfma_flops=flops))
         return "Hadamard rotation GB/s (bf16 MFMA), block 128 and full 4096, and fused with int4 packing", ops, keep
 
     raise SystemExit(f"unknown workload {name}")
@@ -523,25 +568,25 @@ def cpu_baseline_other(torch, workload, seed):
     from oracle import quant as oquant
     from oracle import sparse as osparse
 
-    threads = min(os.cpu_count() or 1, 16)
+    threads = cpu_threads()
     torch.set_num_threads(threads)
     g = torch.Generator().manual_seed(seed)
     if workload == "fp8-w8a8":
         spec = dict(num_bits=8, type="float", symmetric=True, strategy="channel")
         oargs = oquant._Args(**spec)
-        w = (torch.randn(4096, 4096, generator=g) * 0.02).bfloat16()
+        w = (torch.randn(14336, 4096, generator=g) * 0.02).bfloat16()
         s, z = oquant.observe_weight(w, oargs)
-        nbytes, what = 6 * w.numel(), "fp8 per-channel quantize + dequantize of a 4096x4096 bf16 weight"
+        nbytes, what = 6 * w.numel(), "fp8 per-channel quantize + dequantize of a 14336x4096 bf16 weight"
 
         def run():
             codes = opack.naive_compress(w, s, oargs, zero_point=z)
             opack.naive_decompress({"weight": codes, "weight_scale": s})
     elif workload == "sparse":
-        w = (torch.randn(4096, 4096, generator=g) * 0.02).bfloat16()
-        w[torch.rand(4096, 4096, generator=g) < 0.5] = 0
+        w = (torch.randn(8192, 8192, generator=g) * 0.02).bfloat16()
+        w[torch.rand(8192, 8192, generator=g) < 0.5] = 0
         nnz = int((w != 0).sum())
-        nbytes = 2 * (2 * w.numel() + w.numel() // 8 + 2 * nnz) + 8 * 4096
-        what = "sparse-bitmask compress + decompress of a 4096x4096 bf16 tensor, half zeros"
+        nbytes = 2 * (2 * w.numel() + w.numel() // 8 + 2 * nnz) + 8 * 8192
+        what = "sparse-bitmask compress + decompress of a 8192x8192 bf16 tensor, half zeros"
 
         def run():
             values, bitmask, _ = osparse.bitmask_compress(w)
@@ -549,116 +594,176 @@ def cpu_baseline_other(torch, workload, seed):
     elif workload == "nvfp4":
         spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
         oargs = oquant._Args(**spec)
-        w = (torch.randn(2048, 4096, generator=g) * 0.02).bfloat16()
+        w = (torch.randn(14336, 4096, generator=g) * 0.02).bfloat16()
         gs = oquant.generate_gparam(*[t.reshape(1) for t in torch.aminmax(w)])
         s, z = oquant.observe_weight(w, oargs, global_scale=gs)
         n = w.numel()
-        nbytes, what = 2 * (2 * n + n // 16 + n // 2), "nvfp4 compress + decompress of a 2048x4096 bf16 weight"
+        nbytes, what = 2 * (2 * n + n // 16 + n // 2), "nvfp4 compress + decompress of a 14336x4096 bf16 weight"
 
         def run():
             packed = opack.nvfp4_compress(w, s, gs, oargs)
             opack.nvfp4_decompress(packed, s, gs)
     elif workload == "hadamard":
-        x = torch.randn(2048, 4096, generator=g).bfloat16()
+        x = torch.randn(8192, 4096, generator=g).bfloat16()
         q = (torch.randint(0, 2, (128,), generator=g) * 2 - 1).double()
         weight = q[:, None] * ohad.deterministic_hadamard_matrix(128, torch.float64)
-        nbytes, what = 4 * x.numel(), "random-sign Hadamard of size 128 on a 2048x4096 bf16 activation (fp64 matmul, as the reference's offline precision)"
+        nbytes, what = 4 * x.numel(), "random-sign Hadamard of size 128 on a 8192x4096 bf16 activation (fp64 matmul, as the reference's offline precision)"
 
         def run():
             ohad.hadamard_forward(weight, x, "input")
     elif workload == "one-shot":
         spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
         oargs = oquant._Args(**spec)
-        w = (torch.randn(4096, 4096, generator=g) * 0.02).bfloat16()
+        w = (torch.randn(14336, 4096, generator=g) * 0.02).bfloat16()
         n = w.numel()
-        nbytes, what = 2 * n + 2 * n // GROUP + n // 2, "observer + qparams + quantize + pack of a 4096x4096 bf16 weight (W4A16 g128)"
+        nbytes, what = 2 * n + 2 * n // GROUP + n // 2, "observer + qparams + quantize + pack of a 14336x4096 bf16 weight (W4A16 g128)"
 
         def run():
             s, z = oquant.observe_weight(w, oargs)
             opack.pack_quantized_compress(w, s, oargs, zero_point=z)
     else:
         return None
-    times = []
-    for it in range(4):
-        t0 = time.perf_counter()
-        run()
-        dt = time.perf_counter() - t0
-        if it:
-            times.append(dt)
-    med = statistics.median(times)
-    return {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-            "sample": what + f", median of 3 after 1 warm-up, torch {torch.__version__} CPU",
+    med = median_time(run)
+    return {"value": nbytes / med / 1e9, "unit": "GB/s", "cores": threads,
+            "host_cpu_count": os.cpu_count(), "kind": "port",
+            "sample": what + f", median of 5 after 1 warm-up, torch {torch.__version__} CPU",
             "seconds": med}
 
 
-def run_other(torch, a):
-    metric, ops, keep = other_workload(torch, a.workload, a.seed)
-    step_s = time_ops(torch, ops, a.steps, a.warmup)
+def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True):
+    """one of the other configurations -> its result object (same fields as the headline
+    line, plus the per-operation table)"""
+    metric, ops, keep = other_workload(torch, workload, seed)
+    step_s = time_ops(torch, ops, steps, warmup)
     total_bytes = sum(op.nbytes for op in ops)
     gpu_ms = sum(op.ms for op in ops)
     # the roofline object describes the operation most of the time goes to (comparison-only
     # operations aside); every operation's own rate is in `operations`
     slow = max((op for op in ops if op.primary), key=lambda op: op.ms)
     n_launch = len(slow.calls)
+    traffic, traffic_source = measured_traffic(workload, slow.kernel)
+
+    def op_row(op):
+        row = {"name": op.name, "kernel": op.kernel, "GBs": op.nbytes / (op.ms * 1e-3) / 1e9,
+               "frac_of_hbm_peak": op.nbytes / (op.ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
+               "ms": op.ms, "algorithmic_bytes": op.nbytes,
+               "for_comparison_only": not op.primary}
+        if op.mfma_flops is not None:
+            row["mfma_TFLOPs"] = op.mfma_flops / (op.ms * 1e-3) / 1e12
+            row["mfma_utilisation"] = op.mfma_flops / (op.ms * 1e-3) / MFMA_BF16_PEAK
+        return row
+
     out = {
         "metric": metric,
         "value": total_bytes / (gpu_ms * 1e-3) / 1e9,
         "unit": "GB/s",
-        "n_gpus": 1, "steps": a.steps, "warmup": a.warmup,
+        "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": step_s * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16 in, codes as the format says (arithmetic in the reference's promoted dtype)",
         "data": "synthetic",
-        "config": {"workload": a.workload, "seed": a.seed,
+        "config": {"workload": workload, "seed": seed,
                    "value_is": "algorithmic bytes of all operations / sum of their GPU times"},
         "roofline": {"bound": "hbm", "kernel": slow.kernel, "operation": slow.name,
                      "achieved": slow.nbytes / (slow.ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": slow.nbytes / (slow.ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                     "traffic": None, "avg_launch_ms": slow.ms / n_launch,
-                     "launches_per_step": n_launch},
-        "operations": [{"name": op.name, "GBs": op.nbytes / (op.ms * 1e-3) / 1e9,
-                        "frac_of_hbm_peak": op.nbytes / (op.ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
-                        "ms": op.ms, "algorithmic_bytes": op.nbytes,
-                        "for_comparison_only": not op.primary} for op in ops],
+                     "achieved_bytes_per_launch": slow.nbytes / n_launch,
+                     "traffic": traffic, "traffic_source": traffic_source,
+                     "avg_launch_ms": slow.ms / n_launch, "launches_per_step": n_launch},
+        "operations": [op_row(op) for op in ops],
         "ms_per_step_gpu": gpu_ms,
     }
-    if not a.no_cpu_baseline:
-        del keep, ops
-        torch.cuda.empty_cache()
-        base = cpu_baseline_other(torch, a.workload, a.seed)
+    mfma = [op for op in ops if op.mfma_flops is not None and op.primary]
+    if mfma:
+        best = max(mfma, key=lambda op: op.mfma_flops / op.ms)
+        out["mfma_utilisation"] = {
+            "peak": "2.5 PFLOP/s dense bf16", "kernel": best.kernel, "operation": best.name,
+            "achieved_TFLOPs": best.mfma_flops / (best.ms * 1e-3) / 1e12,
+            "frac": best.mfma_flops / (best.ms * 1e-3) / MFMA_BF16_PEAK,
+            "counts": "matrix-core flops the kernel issues (an fp32 operand that goes in as three "
+                      "bf16 terms counts three times)"}
+    del keep, ops
+    torch.cuda.empty_cache()
+    if with_cpu_baseline:
+        base = cpu_baseline_other(torch, workload, seed)
         if base is not None:
             out["cpu_baseline"] = base
-    print(json.dumps(out))
+    return out
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="llama3-8b-w4a16")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--seed", type=int, default=0)
-    ap.add_argument("--calib-copies", type=int, default=0,
-                    help="launch N plain 1 GiB copies first (byte-counter calibration when profiling)")
-    a = ap.parse_args()
-    if a.gpus != 1:
-        raise SystemExit(
-            "bench.py measures one GPU: this path shards by whole tensors with no exchange "
-            "step, and no multi-GPU figure is produced (run with --gpus 1)"
-        )
+def api_level(torch, seed, steps):
+    """ModelCompressor.compress_model + decompress_model on a module tree of 224 bf16 Linear
+    layers with the Llama-3-8B shapes (scales attached beforehand by the observer): the cost
+    of the host mirror above the C ABI, next to the kernel-level headline"""
+    from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme, observe_weight_qparams,
+    )
 
-    import torch
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
 
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            for name, r, c in LLAMA3_8B_LAYER:
+                lin = torch.nn.Linear(c, r, bias=False, device="meta", dtype=torch.bfloat16)
+                lin.to_empty(device=dev)
+                lin.weight.data = (torch.randn(r, c, generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+                lin.weight.requires_grad_(False)
+                setattr(self, name, lin)
+
+    model = torch.nn.Module()
+    model.layers = torch.nn.ModuleList([Layer() for _ in range(32)])
+    config = QuantizationConfig(
+        config_groups={"group_0": QuantizationScheme(targets=["Linear"], weights=args)},
+        format="pack-quantized")
+    apply_quantization_scheme(model, config)
+    n = 0
+    for m in model.modules():
+        if isinstance(m, torch.nn.Linear):
+            scale, zp = observe_weight_qparams(m.weight.data, args)
+            m.register_parameter("weight_scale", torch.nn.Parameter(scale, requires_grad=False))
+            m.register_parameter("weight_zero_point", torch.nn.Parameter(zp, requires_grad=False))
+            n += m.weight.numel()
+    mc = ModelCompressor(quantization_config=config)
+    per_dir = 2 * n + 2 * (n // GROUP) + n // 2
+    comp, deco = [], []
+    for it in range(steps + 1):  # first pass is the warm-up
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        mc.compress_model(model)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        mc.decompress_model(model)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        if it:
+            comp.append(t1 - t0)
+            deco.append(t2 - t1)
+    c_s, d_s = statistics.median(comp), statistics.median(deco)
+    return {
+        "what": "ModelCompressor.compress_model + decompress_model, 224 torch.nn.Linear (bf16, on the "
+                "GPU) of the Llama-3-8B shapes, pack-quantized W4A16 g128, wall time incl. the Python "
+                "harness, parameter swaps and allocation of the outputs",
+        "compress_model_ms": c_s * 1e3, "decompress_model_ms": d_s * 1e3,
+        "compress_GBs": per_dir / c_s / 1e9, "decompress_GBs": per_dir / d_s / 1e9,
+        "roundtrip_GBs": 2 * per_dir / (c_s + d_s) / 1e9,
+        "frac_of_hbm_peak": 2 * per_dir / (c_s + d_s) / 1e9 / HBM_PEAK_GBS,
+        "passes": steps, "statistic": "median",
+    }
+
+
+OTHER_WORKLOADS = ("fp8-w8a8", "sparse", "nvfp4", "hadamard", "one-shot")
+
+
+def headline(torch, a):
     from compressed_tensors_amd import _lib
     from compressed_tensors_amd.compressors.pack_quantized import PackedWeightBatch
     from compressed_tensors_amd.quantization import QuantizationArgs, observe_weight_qparams
 
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    _lib.load()
     dev = torch.device("cuda:0")
-    if a.workload in ("fp8-w8a8", "sparse", "nvfp4", "hadamard", "one-shot"):
-        return run_other(torch, a)
     shapes = shapes_for(a.workload)
     args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group",
                             group_size=GROUP)
@@ -687,7 +792,8 @@ def main():
     per_dir, n_elems = algorithmic_bytes(shapes)
     torch.cuda.synchronize()
 
-    # ---- parity spot check against the oracle (outside the timed region)
+    # ---- parity spot check against the oracle (outside the timed region): the first, a
+    # middle and the last rows of three tensors, the last tensor of the set among them
     from oracle import pack as opack
     from oracle import quant as oquant
 
@@ -695,13 +801,17 @@ def main():
     batch.compress()
     batch.decompress()
     torch.cuda.synchronize()
-    rows = slice(0, 64)
-    w0, s0, z0 = (entries[0][k][rows].cpu() for k in ("weight", "scale", "zero_point"))
-    want = opack.pack_quantized_compress(w0, s0, oargs, zero_point=z0)
-    assert torch.equal(batch.packed[0][rows].cpu(), want["weight_packed"]), "compress parity"
-    want_d = opack.pack_quantized_decompress(dict(want, weight_scale=s0), oargs)
-    assert torch.equal(batch.dense[0][rows].cpu().view(torch.int16), want_d.view(torch.int16)), \
-        "decompress parity"
+    checked = []
+    for t in sorted({0, len(entries) // 2, len(entries) - 1}):
+        n_rows = entries[t]["weight"].shape[0]
+        for rows in (slice(0, 32), slice(n_rows // 2, n_rows // 2 + 32), slice(n_rows - 32, n_rows)):
+            w0, s0, z0 = (entries[t][k][rows].cpu() for k in ("weight", "scale", "zero_point"))
+            want = opack.pack_quantized_compress(w0, s0, oargs, zero_point=z0)
+            assert torch.equal(batch.packed[t][rows].cpu(), want["weight_packed"]), "compress parity"
+            want_d = opack.pack_quantized_decompress(dict(want, weight_scale=s0), oargs)
+            assert torch.equal(batch.dense[t][rows].cpu().view(torch.int16), want_d.view(torch.int16)), \
+                "decompress parity"
+        checked.append(entries[t]["name"])
 
     # ---- timed region
     for _ in range(a.warmup):
@@ -731,7 +841,7 @@ def main():
     if deco_ms > comp_ms:
         dom, dom_gbs, dom_ms, n_launch = ("pq_decompress_vec_kernel", deco_gbs, deco_ms,
                                           batch.launches(compress=False))
-    traffic = MEASURED_TRAFFIC.get((a.workload, dom))
+    traffic, traffic_source = measured_traffic(a.workload, dom)
 
     out = {
         "metric": "compress+decompress GB/s & % HBM roofline, Llama-3-8B-shaped W4A16 g128",
@@ -766,6 +876,7 @@ def main():
             "achieved_bytes_per_launch": per_dir / n_launch,
             "traffic": traffic,
             "traffic_unit": "HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, copy-calibrated)",
+            "traffic_source": traffic_source,
             "avg_launch_ms": dom_ms / n_launch,
             "launches_per_step": n_launch,
             "compress_GBs": comp_gbs,
@@ -773,13 +884,65 @@ def main():
             "compress_ms": comp_ms,
             "decompress_ms": deco_ms,
         },
-        "parity": "bit-exact vs oracle on the first 64 rows of tensor 0 (checked before timing)",
+        "parity": "bit-exact vs oracle on the first, middle and last 32 rows of " + ", ".join(checked)
+                  + " (checked before timing)",
     }
+    del batch, entries
+    torch.cuda.empty_cache()
     if not a.no_cpu_baseline:
         sample = LLAMA3_8B_LAYER  # one layer of 32; the other 31 are identical work
         if a.workload == "w4a16-4096":
             sample = [("w", 4096, 4096)]
         out["cpu_baseline"] = cpu_baseline(torch, sample, a.seed)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default=None)
+    ap.add_argument("--only-headline", action="store_true",
+                    help="the default workload without the short runs of the other configurations")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--calib-copies", type=int, default=0,
+                    help="launch N plain 1 GiB copies first (byte-counter calibration when profiling)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        raise SystemExit(
+            "bench.py measures one GPU: this path shards by whole tensors with no exchange "
+            "step, and no multi-GPU figure is produced (run with --gpus 1)"
+        )
+
+    import torch
+
+    from compressed_tensors_amd import _lib
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    _lib.load()
+    everything = a.workload is None and not a.only_headline
+    if a.workload is None:
+        a.workload = "llama3-8b-w4a16"
+    if a.workload == "api":
+        print(json.dumps(api_level(torch, a.seed, a.steps)))
+        return
+    if a.workload in OTHER_WORKLOADS:
+        print(json.dumps(run_other(torch, a.workload, a.seed, a.steps, a.warmup,
+                                   not a.no_cpu_baseline)))
+        return
+    out = headline(torch, a)
+    if everything:
+        # the other configurations of the path, a few steps each
+        steps, warmup = min(a.steps, 5), min(a.warmup, 2)
+        out["configs"] = {}
+        for w in OTHER_WORKLOADS:
+            r = run_other(torch, w, a.seed, steps, warmup, not a.no_cpu_baseline)
+            out["configs"][w] = {k: r[k] for k in ("metric", "value", "unit", "steps", "ms_per_step_gpu",
+                                                   "roofline", "mfma_utilisation", "operations",
+                                                   "cpu_baseline") if k in r}
+        out["api_level"] = api_level(torch, a.seed, min(a.steps, 5))
     print(json.dumps(out))
 
 

@@ -333,10 +333,16 @@ class ModelCompressor:
     def compress_model(self, model: Module) -> None:
         module_to_scheme = map_module_to_scheme(model)
         sparse_targets = self._sparse_targets(model)
+        # modules that are only quantized: all modules of one format go through one
+        # state-dict call of their compressor (one multi-weight call of the C ABI)
+        by_format: Dict[str, List] = {}
         for prefix, module in list(model.named_modules()):
             if prefix not in module_to_scheme and prefix not in sparse_targets:
                 continue
-            state = {f"{prefix}.{n}": p.data for n, p in module.named_parameters(recurse=False)}
+            if prefix in module_to_scheme and prefix not in sparse_targets:
+                by_format.setdefault(self._format_of(module), []).append((prefix, module))
+                continue
+            state = self._own_parameters(module, prefix)
             stacked = {}
             if prefix in module_to_scheme and prefix in sparse_targets:
                 stacked = self._compress_quantized_24(model, state, sparse_targets, module_to_scheme)
@@ -352,6 +358,18 @@ class ModelCompressor:
                 state.update(entries)
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.COMPRESSED
+        for fmt, members in by_format.items():
+            state = {}
+            for prefix, module in members:
+                state.update(self._own_parameters(module, prefix))
+            state = self.quantization_compressor.get(fmt).compress(
+                state, names_to_scheme=module_to_scheme, show_progress=False)
+            per_module: Dict[str, Dict[str, Tensor]] = {prefix: {} for prefix, _ in members}
+            for name, value in state.items():
+                per_module[name.rpartition(".")[0]][name] = value
+            for prefix, module in members:
+                self._swap_parameters(module, prefix, per_module[prefix])
+                module.quantization_status = QuantizationStatus.COMPRESSED
         if (self.quantization_config is not None
                 and self.quantization_config.format != CompressionFormat.dense.value):
             self.quantization_config.quantization_status = QuantizationStatus.COMPRESSED.value
@@ -359,10 +377,15 @@ class ModelCompressor:
     def decompress_model(self, model: Module) -> None:
         module_to_scheme = map_module_to_scheme(model)
         sparse_targets = self._sparse_targets(model)
+        by_format: Dict[str, List] = {}
         for prefix, module in list(model.named_modules()):
             if prefix not in module_to_scheme and prefix not in sparse_targets:
                 continue
-            state = {f"{prefix}.{n}": p.data for n, p in module.named_parameters(recurse=False)}
+            state = self._own_parameters(module, prefix)
+            if prefix in module_to_scheme and prefix not in sparse_targets:
+                # only quantized: decompressed below, all modules of one format from one call
+                by_format.setdefault(self._format_of(module), []).append((prefix, module, state))
+                continue
             dense = None
             if prefix in sparse_targets and prefix in module_to_scheme:  # both in one pass
                 dense = self._decompress_quantized_24(
@@ -378,6 +401,17 @@ class ModelCompressor:
                         prefix, state, scheme=module_to_scheme[prefix])
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.FROZEN
+        for fmt, members in by_format.items():
+            compressor = self.quantization_compressor.get(fmt)
+            local = [{k[len(prefix) + 1:]: v for k, v in state.items()} for prefix, _, state in members]
+            todo = [i for i, data in enumerate(local) if "weight_scale" in data]
+            dense = compressor.decompress_weights(
+                [(local[i], module_to_scheme[members[i][0]].weights) for i in todo])
+            for i, weight in zip(todo, dense):
+                local[i]["weight"] = weight
+            for (prefix, module, _), data in zip(members, local):
+                self._swap_parameters(module, prefix, {f"{prefix}.{k}": v for k, v in data.items()})
+                module.quantization_status = QuantizationStatus.FROZEN
 
     # ----- helpers ----- #
     @staticmethod
@@ -385,12 +419,19 @@ class ModelCompressor:
         return model.get_submodule(path) if path else model
 
     @staticmethod
+    def _own_parameters(module: Module, prefix: str) -> Dict[str, Tensor]:
+        """the module's own parameters under their state-dict names"""
+        return {f"{prefix}.{n}": p.data for n, p in module._parameters.items() if p is not None}
+
+    @staticmethod
     def _swap_parameters(module: Module, prefix: str, state: Dict[str, Tensor]) -> None:
-        for name, _ in list(module.named_parameters(recurse=False)):
-            delattr(module, name)
+        """replace the module's own parameters by the entries of `state` (full names)"""
+        params = module._parameters
+        params.clear()
+        cut = len(prefix) + 1
         for name, value in state.items():
-            local = name[len(prefix) + 1:] if name.startswith(prefix + ".") else name
-            module.register_parameter(local, torch.nn.Parameter(value, requires_grad=False))
+            local = name[cut:] if name.startswith(prefix + ".") else name
+            params[local] = torch.nn.Parameter(value, requires_grad=False)
 
     def _assign(self, model: Module, full_name: str, data: Tensor) -> None:
         prefix, _, param_name = full_name.rpartition(".")

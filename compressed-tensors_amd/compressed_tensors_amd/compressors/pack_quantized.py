@@ -31,6 +31,7 @@ __all__ = ["PackedQuantizationCompressor", "PackedWeightBatch", "ObservedWeightB
            "pack_to_int32", "unpack_from_int32"]
 
 _PACKABLE = (QuantizationStrategy.GROUP.value, QuantizationStrategy.CHANNEL.value)
+_CHUNK = 32  # weights per multi-weight call of the state-dict paths (4 launches of 8)
 
 
 def pack_to_int32(value: Tensor, num_bits: int, packed_dim: int = 1) -> Tensor:
@@ -273,6 +274,58 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         return out
 
 
+def _decompress_weights_batched(self, items) -> list:
+    """PackedQuantizationCompressor.decompress_weight (pack_quantized.py:147-183) for a list
+    of (compressed_data, quantization_args) pairs from one ctmi_pack_quantized_decompress_many
+    call; same tensors as the per-weight calls"""
+    if len(items) > _CHUNK:  # the GPU starts on the first chunk while the rest is prepared
+        outs = []
+        for at in range(0, len(items), _CHUNK):
+            outs += _decompress_weights_batched(self, items[at:at + _CHUNK])
+        return outs
+    n = len(items)
+    if n == 0:
+        return []
+    jobs = (_lib.WeightJob * n)()
+    outs, keep, device = [], [], None
+    for i, (data, args) in enumerate(items):
+        packed = to_gpu(data["weight_packed"])
+        scale = to_gpu(data["weight_scale"])
+        zero_point = to_gpu(data.get("weight_zero_point", None))
+        g_idx = to_gpu(data.get("weight_g_idx", None))
+        shape = torch.Size(int(d) for d in data["weight_shape"])
+        if packed.dtype is not torch.int32:
+            raise ValueError(f"Expected {torch.int32} but got {packed.dtype}, Aborting unpack.")
+        if args.num_bits > 8:
+            raise ValueError("Unpacking is only supported for less than 8 bits")
+        if len(shape) != 2:
+            raise ValueError(f"expected a 2-D weight, got shape {tuple(shape)}")
+        if not args.symmetric and args.strategy in _PACKABLE:
+            assert zero_point is not None, "Asymmetric quantization requires zero-point values"
+            zero_point = unpack_from_int32(zero_point, args.num_bits, (shape[0], scale.shape[-1]),
+                                           packed_dim=0)
+        carrier = _ShapeOnly(shape, torch.int8)
+        plan = build_qparams(carrier, scale, zero_point, infer_dequant_args(carrier, scale), g_idx, None)
+        plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_INT, args.num_bits
+        rows, cols = shape
+        need = math.ceil(cols / (32 // args.num_bits))
+        if packed.shape[1] != need:
+            packed = packed[:, :need]
+        packed = packed.contiguous()
+        out = torch.empty(shape, dtype=scale.dtype, device=packed.device)
+        j = jobs[i]
+        j.src, j.dst, j.rows, j.cols = packed.data_ptr(), out.data_ptr(), rows, cols
+        j.dense_dtype, j.qp = _lib.dtype_code(scale.dtype), plan.qp
+        keep += [packed, plan]
+        outs.append(out)
+        device = device or packed.device
+    _lib.check(_lib.load().ctmi_pack_quantized_decompress_many(jobs, n, _lib.stream_of(device)))
+    return outs
+
+
+PackedQuantizationCompressor.decompress_weights = _decompress_weights_batched
+
+
 class PackedWeightBatch(LazyDenseOutputs):
     """Every weight of a state dict prepared for one-call compress / decompress.
 
@@ -290,7 +343,7 @@ class PackedWeightBatch(LazyDenseOutputs):
         self.n = len(entries)
         self.names = [e.get("name", str(i)) for i, e in enumerate(entries)]
         self._keep = []
-        self.weights, self.packed, self.scales = [], [], []
+        self.weights, self.packed, self.scales, self._dspecs = [], [], [], []
         self._cjobs = (_lib.WeightJob * max(self.n, 1))()
         self._djobs = (_lib.WeightJob * max(self.n, 1))()
         self.device = device
@@ -309,20 +362,26 @@ class PackedWeightBatch(LazyDenseOutputs):
             packed = torch.empty((rows, math.ceil(cols / pf)), dtype=torch.int32, device=w.device)
             self._plan_dense((rows, cols), scale.dtype, w.device)
             cplan = build_qparams(w, scale, zp, args, g_idx, None)
-            dq_args = infer_dequant_args(_ShapeOnly(w.shape, torch.int8), scale)
             use_zp = (not args.symmetric) if decompress_zero_points is None else decompress_zero_points
-            dplan = build_qparams(_ShapeOnly(w.shape, torch.int8), scale, zp if use_zp else None,
-                                  dq_args, g_idx, None)
-            dplan.qp.qtype, dplan.qp.num_bits = _lib.QTYPE_INT, args.num_bits
-            self._keep += [cplan, dplan]
+            # the decompress side (its qparams, its dense output) waits for the first decompress()
+            self._dspecs.append((w.shape, scale, zp if use_zp else None, g_idx, args.num_bits))
+            self._keep.append(cplan)
             cj, dj = self._cjobs[i], self._djobs[i]
             cj.src, cj.dst, cj.rows, cj.cols = w.data_ptr(), packed.data_ptr(), rows, cols
             cj.dense_dtype, cj.qp = _lib.dtype_code(w.dtype), cplan.qp
-            dj.src, dj.rows, dj.cols = packed.data_ptr(), rows, cols  # dst: _ensure_dense
-            dj.dense_dtype, dj.qp = _lib.dtype_code(scale.dtype), dplan.qp
+            dj.src, dj.rows, dj.cols = packed.data_ptr(), rows, cols
+            dj.dense_dtype = _lib.dtype_code(scale.dtype)
             self.weights.append(w)
             self.packed.append(packed)
             self.scales.append(scale)
+
+    def _finish_decompress_job(self, i):
+        shape, scale, zp, g_idx, num_bits = self._dspecs[i]
+        carrier = _ShapeOnly(shape, torch.int8)
+        dplan = build_qparams(carrier, scale, zp, infer_dequant_args(carrier, scale), g_idx, None)
+        dplan.qp.qtype, dplan.qp.num_bits = _lib.QTYPE_INT, num_bits
+        self._keep.append(dplan)
+        self._djobs[i].qp = dplan.qp
 
     def compress(self):
         """enqueue quantize+pack of every weight; returns the packed tensors"""
@@ -436,9 +495,11 @@ def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progre
                          quantization_args=args))
         order.append((name, prefix, args))
     packed_by_name = {}
-    if jobs:
-        batch = PackedWeightBatch(jobs)
-        for (name, prefix, args), packed in zip(order, batch.compress()):
+    # a few launches' worth of weights per call: the GPU works on one chunk while the
+    # host prepares the job table of the next
+    for at in range(0, len(jobs), _CHUNK):
+        batch = PackedWeightBatch(jobs[at:at + _CHUNK])
+        for (name, prefix, args), packed in zip(order[at:at + _CHUNK], batch.compress()):
             packed_by_name[name] = packed
 
     def move(t):

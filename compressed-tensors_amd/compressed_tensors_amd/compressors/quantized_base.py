@@ -49,8 +49,12 @@ class LazyDenseOutputs:
             self._dense = [torch.empty(shape, dtype=dtype, device=device)
                            for shape, dtype, device in specs]
             for i, t in enumerate(self._dense):
+                self._finish_decompress_job(i)
                 setattr(self._djobs[i], self._dense_field, t.data_ptr())
         return self._dense
+
+    def _finish_decompress_job(self, i):
+        """hook: whatever else of decompress job i was left for the first decompress()"""
 
     @property
     def dense(self):
@@ -144,6 +148,12 @@ class BaseQuantizationCompressor(BaseCompressor):
                     compressed_data=weight_data, quantization_args=quant_args
                 )
                 yield module_path, weight_data
+
+    def decompress_weights(self, items) -> list:
+        """decompress_weight for a list of (compressed_data, quantization_args) pairs;
+        formats with a multi-weight entry point in the C ABI override this with one call"""
+        return [self.decompress_weight(compressed_data=data, quantization_args=args)
+                for data, args in items]
 
     def decompress_module_from_state_dict(
         self, prefix: str, state_dict: Dict[str, Tensor], scheme: Any
