@@ -220,36 +220,116 @@ __device__ __forceinline__ uint32_t nvfp4_codes_exact(const Vec<typename XT::raw
   return acc;
 }
 
-// Same codes without the divisions.  The exact quotient q = x / s lies between
-// x * r_lo and x * r_hi, r = rcp(s) widened by 2^-20 either way (rcp and the
-// product are each good to 2^-23); rounding to e2m1 is monotonic, so when both
-// ends convert to the same code that is q's code.  Otherwise (about one value in
-// 10^5 sits that close to a boundary) the wavefront redoes the vector exactly.
-// fma(x, r, +0) instead of x * r turns a -0 quotient into +0, as the reference's
-// sign(0) = 0 does.  NaNs take the exact path.
-template <typename XT, bool HAS_ZP>
-__device__ __forceinline__ uint32_t nvfp4_codes(const Vec<typename XT::raw, 8>& xv, float s,
-                                                float z) {
-  const float r = __builtin_amdgcn_rcpf(s);
-  const float r_lo = r * 0.99999904632568359375f, r_hi = r * 1.00000095367431640625f;
-  float lo[8], hi[8];
-  bool ok = s >= 7.888609052210118e-31f && s <= 1.2676506002282294e30f;
-  // a zero point of zero (what symmetric schemes carry) only turns -0 into +0,
-  // which the fma below does as well; any other takes the exact path
-  if constexpr (HAS_ZP) ok &= z == 0.0f;
+// The effective scale of a group is fp32(fp8 code) / global_scale: only 256 values
+// per weight.  A workgroup works them out once (the exact division, the reciprocal
+// and whether the scale is in the range where the fast path holds) while its loads
+// are in flight, and a group's arithmetic starts from one 16-byte LDS read instead
+// of a division and a reciprocal.
+struct alignas(16) Fp4Scale {
+  float s;   // fp32(fp8 code) / global_scale, the exact quotient
+  float r;   // rcp(s) for the fast path, or NaN where only the division is safe
+  float y;   // rcp(s) after one Newton step: what an IEEE division multiplies by
+  float pad;
+};
+
+__device__ __forceinline__ void build_scale_lut(Fp4Scale* lut, float gs) {
+  const int t = threadIdx.x;
+  if (t < 256) {
+    const float s = __builtin_amdgcn_cvt_f32_fp8(t, 0) / gs;
+    // below 2^12 a quotient of the smallest bfloat16 / float16 magnitude stays above
+    // the addend of nvfp4_codes_fast; above 2^-60 the residuals of nvfp4_codes_divided
+    // stay in the normal range for every input that can reach a code other than zero
+    const bool tame = s >= 8.673617379884035e-19f && s < 4096.0f;
+    const float y0 = __builtin_amdgcn_rcpf(s);
+    Fp4Scale e;
+    e.s = s;
+    e.r = tame ? y0 : __uint_as_float(0x7fc00000u);
+    e.y = __builtin_fmaf(__builtin_fmaf(-s, y0, 1.0f), y0, y0);
+    e.pad = 0.0f;
+    lut[t] = e;
+  }
+  __syncthreads();
+}
+
+// The codes of 8 elements without divisions and with ONE conversion per pair (the
+// hardware's e2m1 converter is several times slower than an fma; converting a lower and
+// an upper bracket of every quotient made it the bottleneck).
+// q = x * rcp(s) is within 3 ulp of the reference's quotient x / s (rcp: 1 ulp, the
+// product: 1/2, the reference's own rounding: 1/2, a tie broken by the addend: 1).
+// Every rounding boundary of the e2m1 grid (0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5) has a
+// significand of 1, 1.25, 1.5 or 1.75: its low 21 bits are zero.  So if the low 21 bits
+// of q are not within 8 of zero (mod 2^21), no boundary lies between q and the exact
+// quotient, both convert to the same code, and the converter's round-to-nearest-even
+// is the reference's bucket rule.  Otherwise (8 values in a million, an infinity, a
+// scale outside the tame range, whose reciprocal is a NaN with those bits zero, and
+// whatever sits near a power of two) the wavefront redoes the vector with exact
+// divisions.  The addend, 16 ulp of the smallest denormal, is absorbed by every
+// quotient that matters; it keeps exact zeros (which have no bits set) out of the
+// slow path and turns a -0 quotient into +0 as the reference's sign(0) = 0 does,
+// while a negative quotient that rounds to zero keeps its sign (code 8).  A NaN
+// element has no defined code in the reference (the sign of a NaN product); it gets
+// whatever the converter gives and touches no other element.
+// *ok is cleared when the codes returned may differ from the reference's; the caller
+// then redoes the vector with nvfp4_codes_exact.  No branch in here, on purpose: a
+// wave-level branch after every vector (skip the exact path if all lanes are fine)
+// cost this kernel a fifth of its speed.  Callers store what the fast path gives for
+// all their vectors, test once, and overwrite in the rare case.
+template <typename XT>
+__device__ __forceinline__ uint32_t nvfp4_codes_fast(const Vec<typename XT::raw, 8>& xv,
+                                                     const Fp4Scale& e, bool* ok) {
+  const float c0 = __uint_as_float(0x10u);
+  float q[8];
+  uint32_t nearest = 0xffffffffu;
 #pragma unroll
   for (int i = 0; i < 8; i += 2) {
     const float x0 = XT::to_f32(xv.v[i]), x1 = XT::to_f32(xv.v[i + 1]);
-    ok &= !__builtin_isunordered(x0, x1);
-    lo[i] = __builtin_fmaf(x0, r_lo, 0.0f);
-    hi[i] = __builtin_fmaf(x0, r_hi, 0.0f);
-    lo[i + 1] = __builtin_fmaf(x1, r_lo, 0.0f);
-    hi[i + 1] = __builtin_fmaf(x1, r_hi, 0.0f);
+    q[i] = __builtin_fmaf(x0, e.r, c0);
+    q[i + 1] = __builtin_fmaf(x1, e.r, c0);
+    // the low 21 bits, moved to the top, of the bit pattern + 8
+    const uint32_t t0 = (__float_as_uint(q[i]) + 8u) << 11, t1 = (__float_as_uint(q[i + 1]) + 8u) << 11;
+    nearest = min(nearest, min(t0, t1));
+    if constexpr (XT::id == CTMI_F32) {
+      // float32 inputs reach below the addend: a quotient in the denormal range that is
+      // not the addend itself (x == 0) takes the exact path
+      const uint32_t a0 = __float_as_uint(q[i]) & 0x7fffffffu, a1 = __float_as_uint(q[i + 1]) & 0x7fffffffu;
+      if ((a0 < 0x00800000u && a0 != 0x10u) || (a1 < 0x00800000u && a1 != 0x10u)) nearest = 0;
+    }
   }
-  const uint32_t c_lo = fp4_pack8_hw(lo), c_hi = fp4_pack8_hw(hi);
-  ok &= c_lo == c_hi;
-  if (__builtin_expect(wave_all(ok), 1)) return c_lo;
-  return nvfp4_codes_exact<XT, HAS_ZP>(xv, s, z);
+  *ok &= nearest >= (16u << 11);
+  return fp4_pack8_hw(q);
+}
+
+// Second tier, for the vectors the fast path is not sure of.  Weights of one tensor
+// share few distinct quotient significands (a bfloat16 has 128, the scales of a tensor 8,
+// and a global scale computed in bfloat16 has 8 bits itself), so quotients that ROUND to
+// a boundary such as 1.25, or sit on a grid value such as 1.5, are systematic: in one
+// tensor of three every wavefront meets one.  What settles them is the correctly rounded
+// quotient, and that is five multiply-adds away: with y the Newton-refined reciprocal
+// from the table,
+//     q0 = x y;  q1 = q0 + (x - s q0) y;  q2 = q1 + (x - s q1) y
+// is, instruction for instruction, what an IEEE float division x / s executes between
+// its pre-scaling and its fix-up, and those two only act when the exponents of x and s
+// lie 96 or more apart or an operand, a reciprocal or the quotient leaves the normal
+// range.  So for a tame scale (2^-60 <= s < 2^12) and 2^-30 <= |x| < 2^30 (or x == 0)
+// q2 is bit for bit the reference's x / s, at a third of the cost of the general
+// division; anything else clears *ok and takes nvfp4_codes_exact.
+template <typename XT>
+__device__ __forceinline__ uint32_t nvfp4_codes_divided(const Vec<typename XT::raw, 8>& xv,
+                                                        const Fp4Scale& e, bool* ok) {
+  float q[8];
+  bool fine = e.r == e.r;  // a tame scale
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float x = XT::to_f32(xv.v[i]);
+    const uint32_t mag = __float_as_uint(x) & 0x7fffffffu;
+    fine &= (mag - 0x30800000u) < (0x4e800000u - 0x30800000u) || mag == 0;
+    const float q0 = x * e.y;
+    const float q1 = __builtin_fmaf(__builtin_fmaf(-e.s, q0, x), e.y, q0);
+    const float q2 = __builtin_fmaf(__builtin_fmaf(-e.s, q1, x), e.y, q1);
+    q[i] = q2 + 0.0f;  // an exact zero loses its sign, as in the reference's sign(0) = 0
+  }
+  *ok &= fine;
+  return fp4_pack8_hw(q);
 }
 
 template <typename XT, bool HAS_ZP>
@@ -258,6 +338,7 @@ nvfp4_compress_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t*
                           const uint8_t* __restrict__ zp, const float* __restrict__ gscale,
                           uint32_t* __restrict__ out, VecGeom g) {
   constexpr int B = kFp4Block, U = kFp4Unroll;
+  __shared__ Fp4Scale lut[256];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
@@ -275,16 +356,40 @@ nvfp4_compress_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t*
         xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
         sraw[k] = scale[si[k]];
         if constexpr (HAS_ZP) zraw[k] = zp[si[k]];
+      } else {
+        sraw[k] = 0;
       }
     }
+    build_scale_lut(lut, gs);
+    bool ok = true;
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < g.nvec) {
-        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
+        // a zero point of zero (what symmetric schemes carry) only turns -0 into +0, which
+        // the fast path does as well; any other takes the exact path
+        if constexpr (HAS_ZP) ok &= (zraw[k] & 0x7f) == 0;
+        __builtin_nontemporal_store(nvfp4_codes_fast<XT>(xv[k], lut[sraw[k]], &ok), out + v);
+      }
+    }
+    if (__builtin_expect(wave_all(ok), 1)) return;
+    ok = true;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
+        if constexpr (HAS_ZP) ok &= (zraw[k] & 0x7f) == 0;
+        out[v] = nvfp4_codes_divided<XT>(xv[k], lut[sraw[k]], &ok);
+      }
+    }
+    if (wave_all(ok)) return;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < g.nvec) {
         // zero_point.to(x.dtype): an fp8 value is exact in every wider float type
         const float z = HAS_ZP ? __builtin_amdgcn_cvt_f32_fp8((int)zraw[k], 0) : 0.0f;
-        __builtin_nontemporal_store(nvfp4_codes<XT, HAS_ZP>(xv[k], s, z), out + v);
+        out[v] = nvfp4_codes_exact<XT, HAS_ZP>(xv[k], lut[sraw[k]].s, z);
       }
     }
   };
@@ -298,6 +403,7 @@ nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* 
                             const float* __restrict__ gscale, typename OT::raw* __restrict__ out,
                             VecGeom g) {
   constexpr int B = kFp4Block, U = kFp4Unroll;
+  __shared__ Fp4Scale lut[256];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
@@ -314,13 +420,16 @@ nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* 
       if (!GUARD || v < g.nvec) {
         pv[k] = packed[v];
         sraw[k] = scale[si[k]];
+      } else {
+        sraw[k] = 0;
       }
     }
+    build_scale_lut(lut, gs);
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < g.nvec) {
-        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
+        const float s = lut[sraw[k]].s;
         float t[8];
         fp4_unpack8_hw(pv[k], t);
         Vec<typename OT::raw, 8> o;
@@ -349,6 +458,7 @@ __global__ void __launch_bounds__(kFp4Block) nvfp4_compress_chain_kernel(ChainTa
   const float gs = reinterpret_cast<const float*>(job.zp)[0];
   const uint32_t v0 = local * (B * U) + threadIdx.x;
   const bool full = (local + 1) * (uint32_t)(B * U) <= nvec;
+  __shared__ Fp4Scale lut[256];
   auto body = [&](auto guard) {
     constexpr bool GUARD = decltype(guard)::value;
     Vec<typename XT::raw, 8> xv[U];
@@ -359,15 +469,30 @@ __global__ void __launch_bounds__(kFp4Block) nvfp4_compress_chain_kernel(ChainTa
       if (!GUARD || v < nvec) {
         xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
         sraw[k] = scale[v >> job.shift];
+      } else {
+        sraw[k] = 0;
       }
     }
+    build_scale_lut(lut, gs);
+    bool ok = true;
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
-      if (!GUARD || v < nvec) {
-        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
-        __builtin_nontemporal_store(nvfp4_codes<XT, false>(xv[k], s, 0.0f), out + v);
-      }
+      if (!GUARD || v < nvec)
+        __builtin_nontemporal_store(nvfp4_codes_fast<XT>(xv[k], lut[sraw[k]], &ok), out + v);
+    }
+    if (__builtin_expect(wave_all(ok), 1)) return;
+    ok = true;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) out[v] = nvfp4_codes_divided<XT>(xv[k], lut[sraw[k]], &ok);
+    }
+    if (wave_all(ok)) return;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const uint32_t v = v0 + k * B;
+      if (!GUARD || v < nvec) out[v] = nvfp4_codes_exact<XT, false>(xv[k], lut[sraw[k]].s, 0.0f);
     }
   };
   if (full) body(std::false_type{});
@@ -385,6 +510,7 @@ __global__ void __launch_bounds__(kFp4Block) nvfp4_decompress_chain_kernel(Chain
   const float gs = reinterpret_cast<const float*>(job.zp)[0];
   const uint32_t v0 = local * (B * U) + threadIdx.x;
   const bool full = (local + 1) * (uint32_t)(B * U) <= nvec;
+  __shared__ Fp4Scale lut[256];
   auto body = [&](auto guard) {
     constexpr bool GUARD = decltype(guard)::value;
     uint32_t pv[U];
@@ -395,13 +521,16 @@ __global__ void __launch_bounds__(kFp4Block) nvfp4_decompress_chain_kernel(Chain
       if (!GUARD || v < nvec) {
         pv[k] = packed[v];
         sraw[k] = scale[v >> job.shift];
+      } else {
+        sraw[k] = 0;
       }
     }
+    build_scale_lut(lut, gs);
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
       if (!GUARD || v < nvec) {
-        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
+        const float s = lut[sraw[k]].s;
         float f[8];
         fp4_unpack8_hw(pv[k], f);
         Vec<typename OT::raw, 8> o;
@@ -425,6 +554,8 @@ nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __re
                      const float* __restrict__ gscale, typename XT::raw* __restrict__ out,
                      VecGeom g) {
   constexpr int B = kFp4QdqBlock, U = kFp4QdqUnroll;
+  static_assert(B >= 256, "the scale table is built by 256 threads");
+  __shared__ Fp4Scale lut[256];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
@@ -441,22 +572,45 @@ nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __re
       if (!GUARD || v < g.nvec) {
         xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
         sraw[k] = scale[si[k]];
+      } else {
+        sraw[k] = 0;
       }
     }
+    build_scale_lut(lut, gs);
+    auto emit = [&](int k, uint32_t codes, float s) {
+      float t[8];
+      fp4_unpack8_hw(codes, t);
+      Vec<typename XT::raw, 8> o;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float xi = XT::to_f32(xv[k].v[i]);
+        o.v[i] = XT::from_f32(xi != xi ? xi : t[i] * s);  // a NaN stays one (no code stands for it)
+      }
+      stg_nt<typename XT::raw, 8>(out + (size_t)(v0 + k * B) * 8, o);
+    };
+    bool ok = true;
 #pragma unroll
     for (int k = 0; k < U; ++k) {
-      const uint32_t v = v0 + k * B;
-      if (!GUARD || v < g.nvec) {
-        const float s = __builtin_amdgcn_cvt_f32_fp8((int)sraw[k], 0) / gs;
-        float t[8];
-        fp4_unpack8_hw(nvfp4_codes<XT, false>(xv[k], s, 0.0f), t);
-        Vec<typename XT::raw, 8> o;
+      if (!GUARD || v0 + k * B < g.nvec) {
+        const Fp4Scale e = lut[sraw[k]];
+        emit(k, nvfp4_codes_fast<XT>(xv[k], e, &ok), e.s);
+      }
+    }
+    if (__builtin_expect(wave_all(ok), 1)) return;
+    ok = true;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const float xi = XT::to_f32(xv[k].v[i]);
-          o.v[i] = XT::from_f32(xi != xi ? xi : t[i] * s);  // a NaN stays one (no code stands for it)
-        }
-        stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
+    for (int k = 0; k < U; ++k) {
+      if (!GUARD || v0 + k * B < g.nvec) {
+        const Fp4Scale e = lut[sraw[k]];
+        emit(k, nvfp4_codes_divided<XT>(xv[k], e, &ok), e.s);
+      }
+    }
+    if (wave_all(ok)) return;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      if (!GUARD || v0 + k * B < g.nvec) {
+        const float s = lut[sraw[k]].s;
+        emit(k, nvfp4_codes_exact<XT, false>(xv[k], s, 0.0f), s);
       }
     }
   };
@@ -524,6 +678,7 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
                      typename XT::raw* __restrict__ out, uint8_t* __restrict__ scale_out,
                      uint8_t* __restrict__ zp_out, uint32_t nvec) {
   constexpr int B = kFp4Block, U = 2;
+  __shared__ Fp4Scale lut[256];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   Vec<typename XT::raw, 8> xv[U];
@@ -532,6 +687,18 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
     const uint32_t v = v0 + k * B;
     xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)(v < nvec ? v : nvec - 1) * 8);
   }
+  build_scale_lut(lut, gs);
+  auto emit = [&](int k, uint32_t c, float s) {
+    const uint32_t v = v0 + k * B;
+    float t[8];
+    fp4_unpack8_hw(c, t);
+    Vec<typename XT::raw, 8> o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o.v[i] = XT::from_f32(t[i] * s);  // a NaN in the group made s NaN
+    if (v < nvec) stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
+  };
+  bool ok = true;
+  uint8_t codes[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
@@ -554,13 +721,21 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
       if (scale_out) scale_out[v >> 1] = code;
       if (zp_out) zp_out[v >> 1] = 0;  // fp8 zero
     }
-    const float s = sv / gs;
-    float t[8];
-    fp4_unpack8_hw(nvfp4_codes<XT, true>(xv[k], s, 0.0f), t);
-    Vec<typename XT::raw, 8> o;
+    codes[k] = code;
+    emit(k, nvfp4_codes_fast<XT>(xv[k], lut[code], &ok), lut[code].s);
+  }
+  if (__builtin_expect(wave_all(ok), 1)) return;
+  ok = true;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o.v[i] = XT::from_f32(t[i] * s);  // a NaN in the group made s NaN
-    if (v < nvec) stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
+  for (int k = 0; k < U; ++k) {
+    const Fp4Scale e = lut[codes[k]];
+    emit(k, nvfp4_codes_divided<XT>(xv[k], e, &ok), e.s);
+  }
+  if (wave_all(ok)) return;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const float s = lut[codes[k]].s;
+    emit(k, nvfp4_codes_exact<XT, true>(xv[k], s, 0.0f), s);
   }
 }
 
@@ -575,6 +750,7 @@ nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
                               const float* __restrict__ gscale, uint32_t* __restrict__ packed,
                               uint8_t* __restrict__ scale_out, uint32_t nvec) {
   constexpr int B = kFp4Block, U = 2;
+  __shared__ Fp4Scale lut[256];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   Vec<typename XT::raw, 8> xv[U];
@@ -583,6 +759,9 @@ nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
     const uint32_t v = v0 + k * B;
     xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)(v < nvec ? v : nvec - 1) * 8);
   }
+  build_scale_lut(lut, gs);
+  bool ok = true;
+  uint8_t codes[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
@@ -600,10 +779,26 @@ nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
       code = nvfp4_group_scale<XT>(__builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f),
                                    group_any(2, unordered), gs, &sv);
     }
+    codes[k] = code;
+    const uint32_t c = nvfp4_codes_fast<XT>(xv[k], lut[code], &ok);
     if (v < nvec) {
       if ((threadIdx.x & 1) == 0) scale_out[v >> 1] = code;
-      __builtin_nontemporal_store(nvfp4_codes<XT, true>(xv[k], sv / gs, 0.0f), packed + v);
+      __builtin_nontemporal_store(c, packed + v);
     }
+  }
+  if (__builtin_expect(wave_all(ok), 1)) return;
+  ok = true;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    const uint32_t c = nvfp4_codes_divided<XT>(xv[k], lut[codes[k]], &ok);
+    if (v < nvec) packed[v] = c;
+  }
+  if (wave_all(ok)) return;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    if (v < nvec) packed[v] = nvfp4_codes_exact<XT, true>(xv[k], lut[codes[k]].s, 0.0f);
   }
 }
 
