@@ -802,6 +802,54 @@ nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
   }
 }
 
+// The observer on its own for the same scheme (tests/mock_observer.py:38-113 +
+// helpers.py:101-120): group-16 fp8 scales (and their all-zero zero points) of a 16-bit
+// tensor, with the arithmetic of the fused kernels above (absmax on the raw bits, one
+// scale per pair of lanes) instead of the general min / max observer.
+template <typename XT>
+__global__ void __launch_bounds__(kFp4Block)
+nvfp4_observe_kernel(const typename XT::raw* __restrict__ x, const float* __restrict__ gscale,
+                     uint8_t* __restrict__ scale_out, uint8_t* __restrict__ zp_out, uint32_t nvec) {
+  static_assert(sizeof(typename XT::raw) == 2, "16-bit inputs");
+  constexpr int B = kFp4Block, U = 4;
+  const float gs = gscale[0];
+  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+  Vec<typename XT::raw, 8> xv[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)(v < nvec ? v : nvec - 1) * 8);
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * B;
+    const uint32_t m = group_umax(2, absmax8_bits<XT>(xv[k]));
+    constexpr uint32_t kInf = XT::id == CTMI_BF16 ? 0x7f80u : 0x7c00u;
+    float sv;
+    const uint8_t code = nvfp4_group_scale<XT>(XT::to_f32((typename XT::raw)m), m > kInf, gs, &sv);
+    if (v < nvec && (threadIdx.x & 1) == 0) {
+      scale_out[v >> 1] = code;
+      if (zp_out) zp_out[v >> 1] = 0;  // fp8 zero
+    }
+  }
+}
+
+// scales-only entry for ctmi_observe_qparams; false = not this kernel's case
+bool nvfp4_observe_try(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t blk_cols,
+                       const float* gscale, void* scale_out, void* zp_out, const QpCfg& c,
+                       hipStream_t st) {
+  if (!gscale || blk_cols != 16 || cols % 16 || !c.fp4_global || (uintptr_t)x % 16) return false;
+  if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16) return false;
+  const int64_t nvec = rows * cols / 8;
+  const int64_t grid = cdiv(nvec, kFp4Block * 4);
+  if (nvec >= (1ll << 32) || grid >= (1ll << 31)) return false;
+  auto* so = (uint8_t*)scale_out;
+  auto* zo = (uint8_t*)zp_out;
+  if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(nvfp4_observe_kernel<BF16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, so, zo, (uint32_t)nvec);
+  else hipLaunchKernelGGL(nvfp4_observe_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, gscale, so, zo, (uint32_t)nvec);
+  return true;
+}
+
 bool nvfp4_dynamic_try(const void* x, int x_dtype, void* out, int64_t rows, int64_t cols,
                        int64_t blk_cols, const float* gscale, void* scale_out, void* zp_out,
                        const QpCfg& c, hipStream_t st) {

@@ -14,6 +14,12 @@
 
 namespace ctmi {
 
+// fp4.hip: group-16 fp8 scales of a 16-bit tensor; false = not its case, nothing launched
+bool nvfp4_observe_try(const void* x, int x_dtype, int64_t rows, int64_t cols, int64_t blk_cols,
+                       const float* gscale, void* scale_out, void* zp_out, const QpCfg& c,
+                       hipStream_t st);
+
+
 __global__ void __launch_bounds__(256)
 qparams_kernel(const void* __restrict__ mn, const void* __restrict__ mx, const float* gscale,
                void* __restrict__ scale, void* __restrict__ zp, int64_t n, QpCfg c) {
@@ -453,6 +459,11 @@ extern "C" int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows
   SegGeom g;
   seg_geometry(&g, x, dtype_size(x_dtype), rows, cols, blk_cols);
   const ObserveOut o{scale, zero_point, min_out, max_out};
+  // nvfp4 group-16 scales of a 16-bit tensor have a kernel of their own
+  if (!min_out && !max_out && (!zero_point || zp_dtype == CTMI_F8E4M3) &&
+      nvfp4_observe_try(x, x_dtype, rows, cols, blk_cols, global_scale, scale, zero_point, c,
+                        (hipStream_t)stream))
+    return check_launch("ctmi_observe_qparams");
   CTMI_DISPATCH_XT(x_dtype, {
     if (!observe_streaming<XT>(x, global_scale, o, g, c, (hipStream_t)stream))
       hipLaunchKernelGGL(observe_rows_kernel<XT>, seg_grid(g), 256, 0, (hipStream_t)stream,
