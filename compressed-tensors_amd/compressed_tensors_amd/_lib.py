@@ -238,6 +238,12 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
          c_void_p, c_void_p],
     ),
+    "ctmi_kron_matmul_supported": (c_int32, [c_int32, c_int32, c_int32]),
+    "ctmi_kron_matmul": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+         c_int32, c_float, c_void_p],
+    ),
     "ctmi_block_matmul": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p],

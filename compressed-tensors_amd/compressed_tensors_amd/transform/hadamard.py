@@ -11,15 +11,23 @@ Reference surface mirrored here:
       transform/transform_args.py:24-85, transform/transform_scheme.py:26-55
 
 A Hadamard transform object remembers how its matrix was built,
-    W = diag(signs) * Sylvester(n)          (signs = 1 for the deterministic kind),
+    W = diag(signs) * Sylvester(n)                  (signs = 1 for the deterministic kind)
+    W = diag(signs) * (H_K^T (x) Sylvester(n / K))  (random kind, n not a power of two)
 so `forward` never touches the n x n matrix: the signs are applied on the way
 in or out and Sylvester(n) = Sylvester(a) (x) Sylvester(b) runs as two small
-products on the matrix cores (ctmi_hadamard_apply).  `weight` materialises the
-dense matrix on demand for callers that want to look at it.  Explicit dense
-matrices (anything that is not such a product) go through torch.matmul on the
-GPU, as in the reference.
+products on the matrix cores (ctmi_hadamard_apply); sizes K * 2^m with K from the
+table of known Hadamard matrices (12, 20, 28 ... 224: 14336 = 224 * 64) run through
+ctmi_kron_matmul.  `weight` materialises the dense matrix on demand for callers that
+want to look at it.  Explicit dense matrices go through ctmi_kron_matmul too when a
+run fits its LDS tile, else (and for float64) through torch.matmul on the GPU.
+
+The table of known matrices is data, not code: `hadamards.safetensors` as the reference
+ships it (keys "12", "20", ...: int8 K x K).  It is looked for at the path given to
+`load_hadamard_table`, in $CTMI_HADAMARD_TABLE, and next to an installed
+`compressed_tensors` package (found without importing it).
 """
 import math
+import os
 from enum import Enum
 from typing import Dict, List, Optional, Tuple
 
@@ -35,6 +43,9 @@ __all__ = [
     "deterministic_hadamard_matrix",
     "random_hadamard_matrix",
     "random_hadamard_signs",
+    "load_hadamard_table",
+    "known_hadamard_block",
+    "kron_apply",
     "hadamard_factors",
     "hadamard_apply",
     "hadamard_quantize_pack",
@@ -80,21 +91,87 @@ def random_hadamard_signs(size: int, gen: Optional[torch.Generator] = None) -> T
     return q * 2 - 1
 
 
+_TABLE_ENV = "CTMI_HADAMARD_TABLE"
+_table_cache: Dict[str, Dict[int, Tensor]] = {}
+
+
+def _default_table_path() -> Optional[str]:
+    path = os.environ.get(_TABLE_ENV)
+    if path:
+        return path
+    import importlib.util
+
+    try:
+        spec = importlib.util.find_spec("compressed_tensors")
+    except (ImportError, ValueError):
+        spec = None
+    for root in (spec.submodule_search_locations or []) if spec else []:
+        candidate = os.path.join(root, "transform", "utils", "hadamards.safetensors")
+        if os.path.exists(candidate):
+            return candidate
+    return None
+
+
+def load_hadamard_table(path: Optional[str] = None) -> Dict[int, Tensor]:
+    """{K: int8 K x K Hadamard matrix} from a safetensors file laid out like the
+    reference's hadamards.safetensors (transform/utils/hadamard.py:28, :102-129).  The file
+    is read with safetensors (nothing in it is executed) and every matrix is checked:
+    entries +-1 and H H^T = K I."""
+    path = path or _default_table_path()
+    if path is None:
+        raise FileNotFoundError(
+            "no table of known Hadamard matrices: pass its path, set $" + _TABLE_ENV +
+            ", or install compressed_tensors (its transform/utils/hadamards.safetensors is used)")
+    path = os.path.abspath(path)
+    if path not in _table_cache:
+        from safetensors import safe_open
+
+        table = {}
+        with safe_open(path, framework="pt", device="cpu") as f:
+            for key in f.keys():
+                h = f.get_tensor(key)
+                k = int(key)
+                hd = h.to(torch.float64)
+                if tuple(h.shape) != (k, k) or not bool((hd.abs() == 1).all()) or not torch.equal(
+                        hd @ hd.T, k * torch.eye(k, dtype=torch.float64)):
+                    raise ValueError(f"entry {key!r} of {path} is not a {k} x {k} Hadamard matrix")
+                table[k] = h.to(torch.int8)
+        _table_cache[path] = table
+    return _table_cache[path]
+
+
+def known_hadamard_block(n: int, table_path: Optional[str] = None) -> Tuple[int, Optional[Tensor]]:
+    """(K, H_K) as the reference's _fetch_hadamard_divisor picks it (hadamard.py:102-129):
+    the largest K of the table with n / K a power of two.  For a power of two n other than
+    32 that block is Sylvester's matrix of order min(n, 256) - true of the reference's
+    table - and no table is needed: returns (K, None)."""
+    if is_pow2(n) and n != 32:
+        return min(n, 256), None
+    table = load_hadamard_table(table_path)
+    for k in sorted(table, reverse=True):
+        if n % k == 0 and is_pow2(n // k):
+            return k, table[k]
+    raise ValueError(f"Cannot construct random hadamard matrix of size {n}")
+
+
 def random_hadamard_matrix(
     size: int,
     dtype: torch.dtype = torch.bfloat16,
     device=torch.device("cpu"),
     gen: Optional[torch.Generator] = None,
+    table_path: Optional[str] = None,
 ) -> Tensor:
-    """diag(Q) * H.  For a power of two of at least 64 the reference's butterfly
-    stages end in a stored Sylvester block, so H = Sylvester(size); other sizes
-    need the reference's table of known Hadamard matrices and are not built."""
-    if not (is_pow2(size) and size >= 64):
-        raise NotImplementedError(
-            f"random Hadamard matrices are built for powers of two >= 64, got {size}"
-        )
+    """The reference's random Hadamard matrix (hadamard.py:65-89, :132-163): diag(Q)
+    pushed through log2(size / K) butterfly stages and the known K x K block, which is
+    diag(Q) * (H_K^T (x) Sylvester(size / K)); for a power of two >= 64 that is
+    diag(Q) * Sylvester(size)."""
+    k, block = known_hadamard_block(size, table_path)
     q = random_hadamard_signs(size, gen).to(device=device)
-    h = deterministic_hadamard_matrix(size, torch.float32, device)
+    if block is None:
+        h = deterministic_hadamard_matrix(size, torch.float32, device)
+    else:
+        s = deterministic_hadamard_matrix(size // k, torch.float32, device)
+        h = torch.kron(block.to(device=device, dtype=torch.float32).T.contiguous(), s)
     return (q.unsqueeze(1) * h).to(dtype)
 
 
@@ -154,6 +231,50 @@ def hadamard_apply(
             x.data_ptr(), out.data_ptr(), code, x.numel(), a, b, _lib.ptr(ma_t), mb_t.data_ptr(),
             _lib.ptr(s_in), _lib.ptr(s_out), _lib.stream_of(dev),
         )
+    )
+    return out
+
+
+def kron_apply(
+    value: Tensor,
+    w: Tensor,
+    inner: int = 1,
+    sign_in: Optional[Tensor] = None,
+    sign_out: Optional[Tensor] = None,
+    sylvester: bool = False,
+    scale: Optional[float] = None,
+) -> Tensor:
+    """every run of h * inner elements x of the last dim, as X[h, inner] after sign_in,
+    becomes vec(w^T X S) * sign_out * scale, S = Sylvester(inner) or the identity: the
+    product x * diag(sign_in) * (w (x) S) * diag(sign_out) * scale (ctmi_kron_matmul).
+    scale defaults to 1 / sqrt(h * inner) with the Sylvester factor, 1 without."""
+    x = to_gpu(value).contiguous()
+    if x.dtype not in _FLOATS:
+        raise NotImplementedError(f"transforms of dtype {x.dtype} are not supported")
+    h = int(w.shape[0])
+    if w.ndim != 2 or w.shape[1] != h:
+        raise ValueError("the explicit factor must be square")
+    n = h * inner
+    if x.shape[-1] % n != 0:
+        raise ValueError(f"{n} must divide the last dimension {x.shape[-1]}")
+    lib = _lib.load()
+    code = _lib.dtype_code(x.dtype)
+    if not lib.ctmi_kron_matmul_supported(h, inner, code):
+        raise NotImplementedError(f"no kernel for a {h} x {inner} run of {x.dtype}")
+    dev = x.device
+    wf = w.to(device=dev, dtype=torch.float32).contiguous()
+    s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
+    s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
+    for sgn in (s_in, s_out):
+        if sgn is not None and sgn.numel() != n:
+            raise ValueError(f"sign vectors hold {n} values")
+    if scale is None:
+        scale = 1.0 / math.sqrt(n) if sylvester else 1.0
+    out = torch.empty_like(x)
+    _lib.check(
+        lib.ctmi_kron_matmul(x.data_ptr(), out.data_ptr(), code, x.numel(), h, inner, wf.data_ptr(),
+                             _lib.ptr(s_in), _lib.ptr(s_out), int(bool(sylvester)), float(scale),
+                             _lib.stream_of(dev))
     )
     return out
 
@@ -339,37 +460,61 @@ class TransformScheme:
         self.precision = precision
 
 
-def _matmul_blocks(a: Tensor, b: Tensor) -> Tensor:
-    """A @ B where the smaller square operand acts block-diagonally (matrix.py:137-171)"""
-    if a.shape[-1] > b.shape[-2]:
-        h = b.shape[-2]
-        return (a.unflatten(-1, (a.shape[-1] // h, h)) @ b).flatten(-2, -1)
-    if a.shape[-1] < b.shape[-2]:
-        h = a.shape[-1]
-        return (a @ b.unflatten(-2, (b.shape[-2] // h, h))).flatten(-3, -2)
-    return a @ b
+def _kernel_takes(value: Tensor, matrix: Tensor) -> bool:
+    if value.dtype != matrix.dtype or value.dtype not in _FLOATS or value.numel() == 0:
+        return False
+    return bool(_lib.load().ctmi_kron_matmul_supported(int(matrix.shape[0]), 1,
+                                                       _lib.dtype_code(value.dtype)))
+
+
+def _times_blocks(value: Tensor, w: Tensor) -> Tensor:
+    """value @ blockdiag(w, w, ...): w acts on every run of w.shape[0] values of the last
+    dim (matrix.py:137-171, first branch).  ctmi_kron_matmul where a tile of runs fits in
+    LDS and the dtypes agree (float16 / bfloat16 / float32); else a library GEMM."""
+    h = w.shape[0]
+    if value.shape[-1] % h != 0:
+        raise ValueError(f"a {h} x {h} transform does not divide a dimension of {value.shape[-1]}")
+    if _kernel_takes(value, w):
+        return kron_apply(value, w, scale=1.0)
+    if value.shape[-1] == h:
+        return value @ w
+    return (value.unflatten(-1, (value.shape[-1] // h, h)) @ w).flatten(-2, -1)
+
+
+def _blocks_times(w: Tensor, value: Tensor) -> Tensor:
+    """blockdiag(w, w, ...) @ value (matrix.py:137-171, second branch)
+    = (value^T @ blockdiag(w^T, ...))^T"""
+    h = w.shape[0]
+    if value.shape[-2] % h != 0:
+        raise ValueError(f"a {h} x {h} transform does not divide a dimension of {value.shape[-2]}")
+    if value.ndim == 2 and _kernel_takes(value, w):
+        return kron_apply(value.T.contiguous(), w.T, scale=1.0).T.contiguous()
+    if value.shape[-2] == h:
+        return w @ value
+    return (w @ value.unflatten(-2, (value.shape[-2] // h, h))).flatten(-3, -2)
 
 
 def apply_transform_weight(
     transform_weight: Tensor, value: Tensor, location, module_type: type
 ) -> Tensor:
-    """Explicit-matrix form (matrix.py:65-134): a library GEMM on the GPU.  The
-    structured, matrix-free path is HadamardTransform.forward."""
+    """Explicit-matrix form (matrix.py:65-134), unscaled: ctmi_kron_matmul on the GPU
+    where the matrix fits its tile, a library GEMM otherwise.  The structured, matrix-free
+    path is HadamardTransform.forward."""
     assert transform_weight.shape[0] == transform_weight.shape[1]
     w, v = to_gpu(transform_weight), to_gpu(value)
     location = TransformLocation(location)
     if location.is_online():
-        return _matmul_blocks(v, w)
+        return _times_blocks(v, w)
     if module_type == torch.nn.Linear:
         if location == TransformLocation.WEIGHT_INPUT:
-            return _matmul_blocks(v, w.T)
+            return _times_blocks(v, w.T)
         if location == TransformLocation.WEIGHT_OUTPUT:
-            return _matmul_blocks(w.T, v)
+            return _blocks_times(w.T, v)
     elif module_type == torch.nn.Embedding:
         if location == TransformLocation.WEIGHT_INPUT:
-            return _matmul_blocks(w, v)
+            return _blocks_times(w, v)
         if location == TransformLocation.WEIGHT_OUTPUT:
-            return _matmul_blocks(v, w)
+            return _times_blocks(v, w)
     raise NotImplementedError(f"Applying transforms to {module_type} {location} is not supported")
 
 
@@ -391,33 +536,71 @@ def _orientation(location: TransformLocation, module_type: type) -> Tuple[bool, 
     raise NotImplementedError(f"Applying transforms to {module_type} {location} is not supported")
 
 
+def _kron_plan(n: int, block: Optional[Tensor]) -> Optional[Tuple[int, int]]:
+    """(h, b) of the run layout ctmi_kron_matmul gets for a transform of size n: the known
+    block times Sylvester(n / K), or for a power of two without an MFMA kernel (256, 512,
+    anything below 32) Sylvester(n / b) as the explicit factor beside Sylvester(b)."""
+    if block is not None:
+        return int(block.shape[0]), n // int(block.shape[0])
+    if is_pow2(n):
+        b = min(n, 64)
+        return n // b, b
+    return None
+
+
 class HadamardTransform(torch.nn.Module):
-    """W = diag(signs) * Sylvester(size), optionally row/column permuted by `perm`
-    (W[perm][:, perm]); forward(value) applies it at `args.location`, divides by
-    sqrt(size) and returns value.dtype (hadamard.py:85-121)."""
+    """W = diag(signs) * H, optionally row/column permuted by `perm` (W[perm][:, perm]),
+    where H = Sylvester(size) or, with `block` = a known K x K Hadamard matrix,
+    H = block^T (x) Sylvester(size / K) as the reference builds it for sizes that are not
+    powers of two (transform/utils/hadamard.py:65-89, :132-163); forward(value) applies it
+    at `args.location`, divides by sqrt(size) and returns value.dtype
+    (transform/factory/hadamard.py:85-121)."""
 
     def __init__(self, size: int, signs: Optional[Tensor], perm: Optional[Tensor],
                  scheme: TransformScheme, args: TransformArgs, module_type: type,
-                 precision: torch.dtype = torch.float32):
+                 precision: torch.dtype = torch.float32, block: Optional[Tensor] = None):
         super().__init__()
-        if not is_pow2(size):
+        if block is None and not is_pow2(size):
             raise ValueError("Cannot construct deterministic hadamard of size != 2^n")
+        if block is not None:
+            k = int(block.shape[0])
+            if block.ndim != 2 or block.shape[1] != k or size % k != 0 or not is_pow2(size // k):
+                raise ValueError(f"a {tuple(block.shape)} block does not build a matrix of size {size}")
         self.size = size
         self.signs = signs
         self.perm = perm
+        self.block = block
         self.scheme = scheme
         self.args = args
         self.module_type = module_type
         self.precision = precision
         self._scale = torch.tensor(size, dtype=torch.float64).sqrt()
+        self._factor: Dict[Tuple[str, bool], Tensor] = {}
 
     @property
     def weight(self) -> Tensor:
         """the dense matrix the reference would hold (before `perm`)"""
-        h = deterministic_hadamard_matrix(self.size, self.precision, torch.device("cpu"))
+        if self.block is None:
+            h = deterministic_hadamard_matrix(self.size, self.precision, torch.device("cpu"))
+        else:
+            k = int(self.block.shape[0])
+            s = deterministic_hadamard_matrix(self.size // k, self.precision, torch.device("cpu"))
+            h = torch.kron(self.block.to(self.precision).cpu().T.contiguous(), s)
         if self.signs is not None:
             h = self.signs.to(self.precision).cpu().unsqueeze(1) * h
         return h
+
+    def _explicit_factor(self, h: int, transposed: bool, device) -> Tensor:
+        """fp32 [h, h] factor w of W = diag(q) (w (x) S) for x W, of W^T for x W^T"""
+        key = (str(device), transposed)
+        if key not in self._factor:
+            if self.block is None:
+                w = deterministic_hadamard_matrix(h, torch.float32, device)  # symmetric
+            else:
+                w = self.block.to(device=device, dtype=torch.float32)
+                w = w.contiguous() if transposed else w.T.contiguous()
+            self._factor[key] = w
+        return self._factor[key]
 
     def forward(self, value: Tensor) -> Tensor:
         left, transposed = _orientation(self.args.location, self.module_type)
@@ -428,10 +611,16 @@ class HadamardTransform(torch.nn.Module):
             transposed = not transposed
         value = to_gpu(value)
         n = self.size
-        fast = hadamard_factors(n) is not None and value.dtype in _FLOATS and bool(
-            _lib.load().ctmi_hadamard_supported(*hadamard_factors(n), _lib.dtype_code(value.dtype))
-        )
-        if not fast:
+        lib = _lib.load()
+        mfma = (self.block is None and hadamard_factors(n) is not None and value.dtype in _FLOATS
+                and bool(lib.ctmi_hadamard_supported(*hadamard_factors(n),
+                                                     _lib.dtype_code(value.dtype))))
+        plan = None if mfma else _kron_plan(n, self.block)
+        if plan is not None and not (value.dtype in _FLOATS and bool(
+                lib.ctmi_kron_matmul_supported(plan[0], plan[1], _lib.dtype_code(value.dtype)))):
+            plan = None
+        if not mfma and plan is None:
+            # float64 values, or a run too long for LDS: the dense matrix and a library GEMM
             w = self.weight.to(value.device)
             if self.perm is not None:
                 w = w[self.perm.to(w.device)][:, self.perm.to(w.device)]
@@ -454,7 +643,13 @@ class HadamardTransform(torch.nn.Module):
             p = self.perm.to(x.device)
             blocks = x.unflatten(-1, (x.shape[-1] // n, n))
             x = blocks.index_select(-1, torch.argsort(p)).flatten(-2, -1)
-        y = hadamard_apply(x, n, sign_in=s_in, sign_out=s_out)
+        if mfma:
+            y = hadamard_apply(x, n, sign_in=s_in, sign_out=s_out)
+        else:
+            # W = diag(q) (B^T (x) S):  x W = (x * q) (B^T (x) S);  x W^T = (x (B (x) S)) * q
+            h, b = plan
+            y = kron_apply(x.contiguous(), self._explicit_factor(h, transposed, x.device), inner=b,
+                           sign_in=s_in, sign_out=s_out, sylvester=True)
         if self.perm is not None:
             y = y.unflatten(-1, (y.shape[-1] // n, n)).index_select(-1, p).flatten(-2, -1)
         return y.transpose(0, -1).contiguous() if left else y
@@ -503,14 +698,19 @@ class HadamardFactory(TransformFactory):
     def __init__(self, name: str, scheme: TransformScheme, seed: Optional[int] = None):
         super().__init__(name, scheme, seed)
         self._signs: Dict[int, Optional[Tensor]] = {}
+        self._blocks: Dict[int, Optional[Tensor]] = {}
         self._perms: Dict[int, Tensor] = {}
 
     def _create_signs(self, size: int) -> Optional[Tensor]:
         return None
 
+    def _create_block(self, size: int) -> Optional[Tensor]:
+        return None
+
     def create_transform(self, module: torch.nn.Module, args: TransformArgs) -> HadamardTransform:
         size = _transform_size(module, args.location, self.scheme.head_dim)
         if size not in self._signs:  # one draw per size, as the reference's weight cache
+            self._blocks[size] = self._create_block(size)
             self._signs[size] = self._create_signs(size)
         perm = None
         if self.scheme.randomize:
@@ -519,14 +719,21 @@ class HadamardFactory(TransformFactory):
             perm = self._perms[size]
         precision = self.scheme.precision if args.is_online() else torch.float64
         return HadamardTransform(size, self._signs[size], perm, self.scheme, args, type(module),
-                                 precision=precision)
+                                 precision=precision, block=self._blocks[size])
 
 
 @TransformFactory.register("random-hadamard")
 class RandomHadamardFactory(HadamardFactory):
+    """`table_path`: the file of known Hadamard matrices that sizes other than powers of two
+    (and 32) end in; by default looked up as `load_hadamard_table` describes."""
+
+    def __init__(self, name: str, scheme: TransformScheme, seed: Optional[int] = None,
+                 table_path: Optional[str] = None):
+        super().__init__(name, scheme, seed)
+        self.table_path = table_path
+
+    def _create_block(self, size: int) -> Optional[Tensor]:
+        return known_hadamard_block(size, self.table_path)[1]
+
     def _create_signs(self, size: int) -> Optional[Tensor]:
-        if not (is_pow2(size) and size >= 64):
-            raise NotImplementedError(
-                f"random Hadamard matrices are built for powers of two >= 64, got {size}"
-            )
         return random_hadamard_signs(size, self.generator)

@@ -809,27 +809,6 @@ static int launch_had_kron_jobs(const HadJobs& jobs, int n_jobs, const HadArgs& 
   return CTMI_OK;
 }
 
-// ---------------------------------------------------------------- any small dense matrix (VALU)
-// y[r, g*h + j] = sum_k x[r, g*h + k] * w[k, j] / sqrt_n for an explicit fp32
-// h x h matrix: covers sizes and matrices the MFMA path does not (h < 32,
-// non-Kronecker sizes, matrices that are not +-1).  One workgroup per h-chunk.
-template <typename IO>
-__global__ void __launch_bounds__(256)
-block_matmul_kernel(const typename IO::raw* __restrict__ x, const float* __restrict__ w,
-                    typename IO::raw* __restrict__ out, int64_t n_chunks, int h, float sqrt_n) {
-  extern __shared__ float xrow[];
-  for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-    __syncthreads();
-    for (int k = threadIdx.x; k < h; k += blockDim.x) xrow[k] = IO::to_f32(x[c * h + k]);
-    __syncthreads();
-    for (int j = threadIdx.x; j < h; j += blockDim.x) {
-      float acc = 0.0f;
-      for (int k = 0; k < h; ++k) acc = fmaf(xrow[k], w[(int64_t)k * h + j], acc);
-      out[c * h + j] = IO::from_f32(acc / sqrt_n);
-    }
-  }
-}
-
 template <int A, int B, typename IO>
 static int launch_had(const HadArgs& a, hipStream_t st) {
   using C = HadCfg<A, B, IO>;
@@ -1020,33 +999,6 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
     if (rc) return rc;
   }
   return check_launch("ctmi_hadamard_apply_many");
-}
-
-extern "C" int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel,
-                                 int32_t h, const float* w, void* stream) {
-  CTMI_REQUIRE(numel >= 0, CTMI_ERR_VALUE, "negative size");
-  CTMI_REQUIRE(h >= 1 && h <= 8192, CTMI_ERR_UNSUPPORTED, "block size must be in 1..8192");
-  CTMI_REQUIRE(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32,
-               CTMI_ERR_UNSUPPORTED, "transforms take float16/bfloat16/float32 tensors");
-  CTMI_REQUIRE(numel % h == 0, CTMI_ERR_VALUE,
-               "tensor size %lld is not a multiple of the transform size %d", (long long)numel, h);
-  if (numel == 0) return CTMI_OK;
-  CTMI_REQUIRE(x && out && w, CTMI_ERR_VALUE, "NULL tensor pointer");
-  const int64_t chunks = numel / h;
-  const unsigned grid = (unsigned)(chunks < 256 * 32 ? chunks : 256 * 32);
-  const float sqrt_n = sqrtf((float)h);
-  hipStream_t st = (hipStream_t)stream;
-  const size_t lds = (size_t)h * sizeof(float);
-  if (io_dtype == CTMI_BF16)
-    hipLaunchKernelGGL(block_matmul_kernel<BF16>, grid, 256, lds, st, (const uint16_t*)x, w,
-                       (uint16_t*)out, chunks, h, sqrt_n);
-  else if (io_dtype == CTMI_F16)
-    hipLaunchKernelGGL(block_matmul_kernel<F16>, grid, 256, lds, st, (const uint16_t*)x, w,
-                       (uint16_t*)out, chunks, h, sqrt_n);
-  else
-    hipLaunchKernelGGL(block_matmul_kernel<F32>, grid, 256, lds, st, (const float*)x, w,
-                       (float*)out, chunks, h, sqrt_n);
-  return check_launch("ctmi_block_matmul");
 }
 
 static int hqp_check(int32_t io_dtype, int32_t b_dim, int32_t num_bits, int32_t symmetric) {

@@ -496,9 +496,27 @@ int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_
                                   const float* sign_in, const float* sign_out, int32_t num_bits,
                                   int32_t symmetric, void* stream);
 
-/* A24 for an arbitrary explicit fp32 matrix w [h,h] (small h, or matrices that
- * are not +-1): every run of h consecutive elements x becomes x * w / sqrt(h).
- * fp32 accumulation on the vector ALUs. */
+/* A23 / A24 for matrices with an explicit factor (transform/utils/matrix.py:137-171 for
+ * a small explicit matrix; transform/utils/hadamard.py:102-163 for the reference's
+ * Hadamard matrices of size K * 2^m built from its table of known K x K matrices,
+ * diag(Q) * (H_K^T (x) Sylvester(2^m)), e.g. 14336 = 224 * 64).  Every run of h * b
+ * consecutive elements x, viewed as X[h, b] after the optional sign_in, becomes
+ *     vec(w^T X S_b) * sign_out * scale        (sylvester != 0, S_b = Sylvester(b))
+ *     vec(w^T X)     * sign_out * scale        (sylvester == 0)
+ * i.e. x * diag(sign_in) * (w (x) S_b) * diag(sign_out) * scale, rounded once to
+ * io_dtype (scale = 1 / sqrt(h * b) makes a Hadamard rotation orthonormal).  w: fp32
+ * [h, h] row-major (any values); sign_in / sign_out: fp32 [h * b] or NULL; b a power of
+ * two up to 256 and h * b * 4 bytes within 159 KB; for b = 1, 64 runs share a workgroup
+ * and h may be at most 313 (ctmi_kron_matmul_supported).  fp32 accumulation on the vector
+ * ALUs. */
+int ctmi_kron_matmul_supported(int32_t h, int32_t b, int32_t io_dtype);
+int ctmi_kron_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t h,
+                     int32_t b, const float* w, const float* sign_in, const float* sign_out,
+                     int32_t sylvester, float scale, void* stream);
+
+/* A24 for an arbitrary explicit fp32 matrix w [h,h] (h up to 313; matrices that are not
+ * +-1 included): every run of h consecutive elements x becomes x * w / sqrt(h).  The case
+ * b = 1, scale = 1 / sqrt(h) of ctmi_kron_matmul. */
 int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t h,
                       const float* w, void* stream);
 

@@ -5,10 +5,13 @@ transform/factory/hadamard.py:46-121 of the reference on CPU tensors.
 
 The reference ends its butterfly recursion in a table of known Hadamard
 matrices (hadamards.safetensors) that does not travel with this repository.
-For a power of two n >= 64 the table entry it picks (the largest K in
-{256, 128, 64} with n / K a power of two) is Sylvester's matrix of that order —
-tests/test_oracle_hadamard.py checks this against the reference's file when it
-is present — so `known_block` rebuilds it; other sizes are not covered.
+For a power of two n other than 32 the table entry it picks (the largest K in
+{256, 128, 64, 16, 8, 4, 2, 1} with n / K a power of two) is Sylvester's matrix of
+that order - tests/test_oracle_hadamard.py checks this against the reference's file
+when it is present - so `known_block` rebuilds it.  Other sizes take the table as an
+argument ({K: K x K matrix}); the tests pass the blocks of
+tests/golden/hadamard_blocks.safetensors, which cover the sizes of the reference's
+own Hadamard tests.
 """
 import math
 from typing import Optional
@@ -29,18 +32,23 @@ def deterministic_hadamard_matrix(size, dtype=torch.bfloat16, device=torch.devic
     return h
 
 
-def known_block(n: int, dtype) -> torch.Tensor:
-    """stand-in for _fetch_hadamard_divisor (hadamard.py:102-129) on powers of two >= 64"""
-    for k in (256, 128, 64):
-        if n % k == 0 and (n // k) & (n // k - 1) == 0:
-            return deterministic_hadamard_matrix(k, dtype)
+def known_block(n: int, dtype, table=None) -> torch.Tensor:
+    """_fetch_hadamard_divisor (hadamard.py:102-129): the largest K of the table with n / K
+    a power of two.  Without a table: powers of two other than 32, whose entries are
+    Sylvester's matrices."""
+    if table is not None:
+        for k in sorted(table, reverse=True):
+            if n % k == 0 and (n // k) & (n // k - 1) == 0:
+                return table[k].to(dtype)
+    elif n & (n - 1) == 0 and n != 32:
+        return deterministic_hadamard_matrix(min(n, 256), dtype)
     raise ValueError(f"Cannot construct random hadamard matrix of size {n}")
 
 
-def matmul_hadU(x: torch.Tensor) -> torch.Tensor:
+def matmul_hadU(x: torch.Tensor, table=None) -> torch.Tensor:
     # hadamard.py:132-163: butterfly stages down to the known block, then the block
     size = x.size(0)
-    had_k = known_block(size, x.dtype)
+    had_k = known_block(size, x.dtype, table)
     k = had_k.size(0)
     inp = x.clone().view(-1, size, 1)
     out = inp.clone()
@@ -56,11 +64,12 @@ def matmul_hadU(x: torch.Tensor) -> torch.Tensor:
     return inp.view(x.shape)
 
 
-def random_hadamard_matrix(size, dtype=torch.bfloat16, gen: Optional[torch.Generator] = None):
+def random_hadamard_matrix(size, dtype=torch.bfloat16, gen: Optional[torch.Generator] = None,
+                           table=None):
     # hadamard.py:65-89
     q = torch.randint(low=0, high=2, size=(size,), generator=gen, dtype=dtype)
     q = q * 2 - 1
-    return matmul_hadU(torch.diag(q))
+    return matmul_hadU(torch.diag(q), table)
 
 
 def multihead_matmul(a, b):

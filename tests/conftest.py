@@ -72,3 +72,42 @@ def gpu():
 
     assert torch.cuda.is_available(), "GPU tests need a GPU"
     return torch.device("cuda:0")
+
+
+def unpack_hadamard_blocks(path=None):
+    """{K: int8 K x K} from tests/golden/hadamard_blocks.safetensors (bit-packed rows)"""
+    import numpy as np
+    import torch
+    from safetensors import safe_open
+
+    path = path or ROOT / "tests" / "golden" / "hadamard_blocks.safetensors"
+    blocks = {}
+    with safe_open(str(path), framework="pt", device="cpu") as f:
+        for key in f.keys():
+            k = int(key)
+            bits = np.unpackbits(f.get_tensor(key).numpy(), axis=1)[:, :k]
+            blocks[k] = torch.from_numpy(bits.astype(np.int8) * 2 - 1)
+    return blocks
+
+
+@pytest.fixture(scope="session")
+def hadamard_blocks():
+    return unpack_hadamard_blocks()
+
+
+@pytest.fixture(scope="session")
+def hadamard_table_path(tmp_path_factory, hadamard_blocks):
+    """the golden blocks (and Sylvester's matrices for the powers of two the reference's
+    table holds) written out in the layout of the reference's hadamards.safetensors"""
+    import torch
+    from safetensors.torch import save_file
+
+    table = {str(k): h.clone() for k, h in hadamard_blocks.items()}
+    for k in (1, 2, 4, 8, 16, 64, 128, 256):
+        h = torch.ones(1, 1, dtype=torch.int8)
+        while h.shape[0] < k:
+            h = torch.cat([torch.cat([h, h], 1), torch.cat([h, -h], 1)], 0)
+        table[str(k)] = h.contiguous()
+    path = tmp_path_factory.mktemp("hadamard") / "hadamards.safetensors"
+    save_file(table, str(path))
+    return str(path)

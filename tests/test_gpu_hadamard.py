@@ -248,3 +248,138 @@ def test_fused_many_tensors_in_one_call(gpu):
             assert_bit_equal(out["weight_packed"], want["weight_packed"], f"packed {i}")
             assert_bit_equal(out["weight_scale"], want["weight_scale"], f"scale {i}")
             assert out["weight_shape"].tolist() == list(shapes[i])
+
+
+# ---------------------------------------------------------------- explicit factors (ctmi_kron_matmul)
+
+
+def _sylvester64(n):
+    return oh.deterministic_hadamard_matrix(n, torch.float64)
+
+
+@pytest.mark.parametrize("h,b", [(12, 2), (12, 64), (20, 8), (28, 128), (224, 64), (1, 256), (4, 64),
+                                 (8, 64), (1, 8), (3, 1), (148, 128)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_kron_matmul(h, b, dtype, gpu):
+    """x * diag(s_in) * (w (x) Sylvester(b)) * diag(s_out) / sqrt(h b) against fp64, for
+    factors w that are not Hadamard matrices either; the run count is odd, so the last
+    workgroup of the several-runs-per-workgroup layout is partly empty"""
+    from compressed_tensors_amd.transform import kron_apply
+
+    announce("kron_matmul", h, b, dtype)
+    n = h * b
+    g = torch.Generator().manual_seed(1000 * h + b)
+    runs = 37 if n <= 4096 else 5
+    x = torch.randn(runs, n, generator=g).to(dtype)
+    w = torch.randn(h, h, generator=g).float() if h != 224 else (
+        torch.randint(0, 2, (h, h), generator=g) * 2 - 1).float()
+    s_in = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    s_out = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    dense = torch.kron(w.double(), _sylvester64(b))
+    y = kron_apply(x.to(gpu), w, inner=b, sylvester=True)
+    _assert_within_ulp(y, (x.double() @ dense / n ** 0.5).to(dtype), "plain")
+    y = kron_apply(x.to(gpu), w, inner=b, sign_in=s_in, sign_out=s_out, sylvester=True)
+    want = ((x.double() * s_in.double()) @ dense * s_out.double() / n ** 0.5).to(dtype)
+    _assert_within_ulp(y, want, "signs")
+    # without the Sylvester factor: w (x) I, unscaled
+    y = kron_apply(x.to(gpu), w, inner=b, sylvester=False)
+    want = (x.double() @ torch.kron(w.double(), torch.eye(b, dtype=torch.float64))).to(dtype)
+    _assert_within_ulp(y, want, "identity inner factor")
+
+
+@pytest.mark.parametrize("h", [1, 3, 16, 100, 128, 313])
+def test_block_matmul_entry_point(h, ctmi, gpu):
+    """ctmi_block_matmul straight through the C ABI: every run of h values times an
+    arbitrary matrix / sqrt(h); 70 runs = one full tile of 64 and a ragged one"""
+    from compressed_tensors_amd import _lib
+
+    announce("ctmi_block_matmul", h)
+    g = torch.Generator().manual_seed(h)
+    x = torch.randn(70, h, generator=g).bfloat16()
+    w = torch.randn(h, h, generator=g)
+    xg, wg = x.to(gpu), w.to(gpu)
+    out = torch.empty_like(xg)
+    _lib.check(ctmi.ctmi_block_matmul(xg.data_ptr(), out.data_ptr(), _lib.dtype_code(x.dtype),
+                                      x.numel(), h, wg.data_ptr(), _lib.stream_of(gpu)))
+    torch.cuda.synchronize()
+    _assert_within_ulp(out, (x.double() @ w.double() / h ** 0.5).bfloat16(), f"h={h}")
+
+
+def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
+    from compressed_tensors_amd import _lib
+
+    code = _lib.dtype_code(torch.bfloat16)
+    assert ctmi.ctmi_kron_matmul_supported(224, 64, code) == 1
+    assert ctmi.ctmi_kron_matmul_supported(313, 1, code) == 1
+    assert ctmi.ctmi_kron_matmul_supported(314, 1, code) == 0
+    assert ctmi.ctmi_kron_matmul_supported(12, 3, code) == 0      # inner size not a power of two
+    assert ctmi.ctmi_kron_matmul_supported(12, 512, code) == 0    # more than 256 lanes
+    assert ctmi.ctmi_kron_matmul_supported(256, 256, code) == 0   # 256 KB of LDS
+    x = torch.zeros(314 * 4, dtype=torch.bfloat16, device=gpu)
+    w = torch.zeros(314, 314, device=gpu)
+    rc = ctmi.ctmi_block_matmul(x.data_ptr(), x.data_ptr(), code, x.numel(), 314, w.data_ptr(), None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED
+    rc = ctmi.ctmi_kron_matmul(x.data_ptr(), x.data_ptr(), code, 100, 12, 2, w.data_ptr(), None, None,
+                               1, 1.0, None)
+    assert rc == _lib.CTMI_ERR_VALUE  # 100 is not a multiple of 24
+
+
+@pytest.mark.parametrize("size", [768, 1600, 14336, 32, 256, 512, 16])
+@pytest.mark.parametrize("location,inverse", [("input", False), ("weight_input", True),
+                                              ("weight_output", False), ("output", True)])
+def test_random_hadamard_of_any_table_size(size, location, inverse, gpu, hadamard_table_path):
+    """sizes K * 2^m from the table of known matrices (14336 = 224 * 64: Llama-3's
+    intermediate size), 32 (whose table entry is not Sylvester's) and the powers of two
+    that have no matrix-core kernel: forward against the dense fp64 matrix the oracle
+    builds with the reference's butterfly stages"""
+    from compressed_tensors_amd.transform import (
+        TransformArgs, TransformFactory, TransformScheme, load_hadamard_table,
+    )
+
+    announce("random hadamard", size, location, inverse)
+    scheme = TransformScheme(type="random-hadamard")
+    factory = TransformFactory.from_scheme(scheme, name="t", seed=size, table_path=hadamard_table_path)
+    other = 48
+    if location in ("input", "weight_input"):
+        linear = torch.nn.Linear(size, other, bias=False, device="meta")
+    else:
+        linear = torch.nn.Linear(other, size, bias=False, device="meta")
+    tfm = factory.create_transform(linear, TransformArgs(["Linear"], location, inverse=inverse))
+    assert tfm.size == size
+    table = {k: v for k, v in load_hadamard_table(hadamard_table_path).items()}
+    gen = torch.Generator().manual_seed(size)
+    weight64 = oh.random_hadamard_matrix(size, dtype=torch.float64, gen=gen, table=table)
+    g = torch.Generator().manual_seed(5)
+    if location in ("weight_input", "weight_output"):
+        value = (torch.randn(linear.out_features, linear.in_features, generator=g) * 0.02).bfloat16()
+    else:
+        value = torch.randn(3, 5, size, generator=g).bfloat16()
+    got = tfm(value.to(gpu))
+    _assert_within_ulp(got, _reference(weight64, value, location, inverse), f"{size} {location}")
+    if size == 768:
+        assert torch.equal(tfm.weight.double(), weight64)
+
+
+@pytest.mark.parametrize("location", ["input", "weight_input", "weight_output", "output"])
+@pytest.mark.parametrize("module_type", [torch.nn.Linear, torch.nn.Embedding])
+def test_apply_transform_weight_runs_the_kernel(location, module_type, gpu, monkeypatch):
+    """explicit 128 x 128 blocks (a head dimension) on a 512-wide value: every location
+    and module kind against the oracle in fp64; torch.matmul must not be what ran"""
+    from compressed_tensors_amd.transform import apply_transform_weight
+    from compressed_tensors_amd.transform import hadamard as product
+
+    announce("apply_transform_weight", location, module_type.__name__)
+    if module_type is torch.nn.Embedding and location in ("input", "output"):
+        pytest.skip("online locations do not depend on the module kind")
+    g = torch.Generator().manual_seed(17)
+    w = torch.randn(128, 128, generator=g).bfloat16()
+    left = (module_type is torch.nn.Linear and location == "weight_output") or (
+        module_type is torch.nn.Embedding and location == "weight_input")
+    value = (torch.randn(512, 96, generator=g) if left else torch.randn(96, 512, generator=g)).bfloat16()
+    calls = []
+    real = product.kron_apply
+    monkeypatch.setattr(product, "kron_apply", lambda *a, **k: calls.append(1) or real(*a, **k))
+    got = apply_transform_weight(w.to(gpu), value.to(gpu), location, module_type)
+    assert calls, "the HIP kernel was not used"
+    want = oh.apply_transform_weight(w.double(), value.double(), location, module_type).bfloat16()
+    _assert_within_ulp(got, want, f"{location} {module_type.__name__}")

@@ -102,3 +102,95 @@ def test_product_host_construction_matches_oracle():
         hb = oh.deterministic_hadamard_matrix(b, torch.float32)
         if n <= 4096:
             assert torch.equal(torch.kron(ha, hb), oh.deterministic_hadamard_matrix(n, torch.float32))
+
+
+# ---------------------------------------------------------------- sizes that are not powers of two
+
+
+def _table(hadamard_blocks):
+    """the golden blocks plus Sylvester's matrices where the reference's table holds them"""
+    table = dict(hadamard_blocks)
+    for k in (1, 2, 4, 8, 16, 64, 128, 256):
+        table[k] = oh.deterministic_hadamard_matrix(k, torch.int8)
+    return table
+
+
+def test_golden_blocks_are_hadamard(hadamard_blocks):
+    assert set(hadamard_blocks) == {12, 20, 28, 32, 144, 148, 160, 192, 200, 224, 240}
+    for k, h in hadamard_blocks.items():
+        hd = h.to(torch.int64)
+        assert tuple(h.shape) == (k, k) and bool((hd.abs() == 1).all())
+        assert torch.equal(hd @ hd.T, k * torch.eye(k, dtype=torch.int64)), k
+    # 32 is the power of two whose entry is not Sylvester's matrix
+    assert not torch.equal(hadamard_blocks[32], oh.deterministic_hadamard_matrix(32, torch.int8))
+
+
+@pytest.mark.skipif(not REF_TABLE.exists(), reason="reference tree not present on this machine")
+def test_golden_blocks_equal_the_reference_table(hadamard_blocks):
+    from safetensors import safe_open
+
+    with safe_open(str(REF_TABLE), framework="pt", device="cpu") as f:
+        for k, h in hadamard_blocks.items():
+            assert torch.equal(f.get_tensor(str(k)).to(torch.int8), h), k
+        # every power of two but 32 is Sylvester's matrix there
+        for k in (1, 2, 4, 8, 16, 64, 128, 256):
+            assert torch.equal(f.get_tensor(str(k)).to(torch.int8),
+                               oh.deterministic_hadamard_matrix(k, torch.int8)), k
+        keys = sorted(int(k) for k in f.keys())
+    # the sizes of the reference's own tests end in blocks the fixture holds
+    for n, want in {768: 192, 1280: 160, 1600: 200, 3584: 224, 3840: 240, 7168: 224,
+                    14336: 224, 18432: 144, 18944: 148}.items():
+        pick = next(k for k in sorted(keys, reverse=True) if n % k == 0 and (n // k) & (n // k - 1) == 0)
+        assert pick == want, n
+
+
+@pytest.mark.parametrize("size", [768, 1280, 1600, 3584, 3840])
+def test_butterfly_construction_is_orthogonal(size, hadamard_blocks):
+    """the reference's own criterion (test_hadamard.py:44-52): H H^T / n == I"""
+    gen = torch.Generator().manual_seed(size)
+    r = oh.random_hadamard_matrix(size, dtype=torch.float32, gen=gen, table=_table(hadamard_blocks))
+    assert set(r.unique().tolist()) == {-1.0, 1.0}
+    assert torch.equal(r @ r.T, size * torch.eye(size, dtype=torch.float32))
+
+
+@pytest.mark.parametrize("size", [24, 40, 56, 32, 96, 448, 768, 1600, 3584])
+def test_closed_form_equals_butterflies(size, hadamard_blocks, hadamard_table_path):
+    """product: diag(Q) (H_K^T (x) Sylvester(n / K)); oracle: the reference's butterfly
+    stages followed by the block - and a brute-force entry formula for three of them"""
+    from compressed_tensors_amd.transform import known_hadamard_block, random_hadamard_matrix
+
+    table = _table(hadamard_blocks)
+    g1, g2 = torch.Generator().manual_seed(size), torch.Generator().manual_seed(size)
+    want = oh.random_hadamard_matrix(size, dtype=torch.float32, gen=g1, table=table)
+    got = random_hadamard_matrix(size, torch.float32, gen=g2, table_path=hadamard_table_path)
+    assert torch.equal(got, want)
+    k, block = known_hadamard_block(size, hadamard_table_path)
+    assert k == oh.known_block(size, torch.int8, table).shape[0]
+    assert torch.equal(block, oh.known_block(size, torch.int8, table))
+    if size <= 96:
+        g3 = torch.Generator().manual_seed(size)
+        q = torch.randint(0, 2, (size,), generator=g3, dtype=torch.float32) * 2 - 1
+        m = size // k
+        for i in range(size):
+            for j in range(0, size, 7):
+                # W[i, j] = Q[i] * H_K[j // m, i // m] * (-1)^popcount((i % m) & (j % m))
+                s = -1.0 if bin((i % m) & (j % m)).count("1") & 1 else 1.0
+                assert got[i, j] == q[i] * float(block[j // m, i // m]) * s
+
+
+def test_table_loader_rejects_what_is_not_hadamard(tmp_path, hadamard_table_path):
+    from safetensors.torch import save_file
+
+    from compressed_tensors_amd.transform import known_hadamard_block, load_hadamard_table
+
+    table = load_hadamard_table(hadamard_table_path)
+    assert table[224].dtype == torch.int8 and 12 in table and 256 in table
+    bad = table[12].clone()
+    bad[0, 0] = -bad[0, 0]
+    path = tmp_path / "bad.safetensors"
+    save_file({"12": bad}, str(path))
+    with pytest.raises(ValueError):
+        load_hadamard_table(str(path))
+    with pytest.raises(ValueError):
+        known_hadamard_block(14336 + 4, hadamard_table_path)  # 3585 * 4: no entry fits
+    assert known_hadamard_block(4096) == (256, None) and known_hadamard_block(16) == (16, None)
