@@ -543,7 +543,7 @@ def _kron_plan(n: int, block: Optional[Tensor]) -> Optional[Tuple[int, int]]:
     if block is not None:
         return int(block.shape[0]), n // int(block.shape[0])
     if is_pow2(n):
-        b = min(n, 64)
+        b = n if n <= 512 else 64  # up to 512 the butterflies stay inside a wavefront
         return n // b, b
     return None
 

@@ -10,7 +10,8 @@
 //     W = diag(sign_in) * (w (x) S_b) * diag(sign_out) * scale
 // to every run of n = h * b elements x: with X = reshape(x * sign_in, [h, b]),
 //     y = vec(w^T X S_b) * scale,    S_b = Sylvester(b) or, without it, the identity.
-// A workgroup holds one run in LDS as fp32, runs the butterflies of S_b in place and
+// Plain Sylvester transforms up to 512 (h = 1) stay inside a wavefront's registers
+// (fwht_wave_kernel).  Otherwise a workgroup holds one run in LDS as fp32, runs the butterflies of S_b in place and
 // then the product with w on the vector ALUs: a lane owns an inner index j, a wavefront
 // a range of output rows, so that the entries of w it needs are wave-uniform and come
 // through the scalar cache.  One rounding, at the end.  h = 224, b = 64: 3.2 M
@@ -188,6 +189,105 @@ __global__ void __launch_bounds__(kKmThreads) block_tile_kernel(KronArgs a) {
   }
 }
 
+// h = 1 with the Sylvester factor, b <= 512: the butterflies never leave a wavefront.  A lane
+// holds 8 neighbouring elements (three stages in registers), the strides 8 ... 256 pair it
+// with the lanes xor 1 ... 32; a wavefront covers 512 elements = 512 / b runs.  No LDS, one
+// 16-byte access per lane each way (two for float32).
+constexpr int kFwhtPer = 8;
+constexpr int kFwhtChunk = kWave * kFwhtPer;
+
+// the value of lane (l ^ m): a data-parallel-primitive move where one exists (neighbours in
+// a quad, the other half of a row of 16), the LDS crossbar otherwise.  m is a constant after
+// unrolling.
+__device__ __forceinline__ float lane_xor(float v, int m) {
+  const int bits = __builtin_bit_cast(int, v);
+  int r;
+  if (m == 1) r = __builtin_amdgcn_update_dpp(bits, bits, 0xB1, 0xF, 0xF, false);        // quad_perm [1,0,3,2]
+  else if (m == 2) r = __builtin_amdgcn_update_dpp(bits, bits, 0x4E, 0xF, 0xF, false);   // quad_perm [2,3,0,1]
+  else if (m == 8) r = __builtin_amdgcn_update_dpp(bits, bits, 0x128, 0xF, 0xF, false);  // row_ror:8
+  else r = wave_shfl_xor(bits, m);
+  return __builtin_bit_cast(float, r);
+}
+
+template <typename IO>
+__global__ void __launch_bounds__(kKmThreads) fwht_wave_kernel(KronArgs a, int64_t numel,
+                                                                int vector_ok) {
+  using R = typename IO::raw;
+  constexpr int VE = 16 / (int)sizeof(R);
+  const auto* __restrict__ x = static_cast<const R*>(a.x);
+  auto* __restrict__ out = static_cast<R*>(a.out);
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = ((int64_t)blockIdx.x * kKmThreads + threadIdx.x) / kWave;
+  const int64_t n_waves = (int64_t)gridDim.x * (kKmThreads / kWave);
+  const int64_t n_chunks = (numel + kFwhtChunk - 1) / kFwhtChunk;
+  const float factor = a.w[0] * a.scale;
+  for (int64_t chunk = wave; chunk < n_chunks; chunk += n_waves) {
+    const int64_t e0 = chunk * kFwhtChunk + (int64_t)lane * kFwhtPer;
+    const bool full = vector_ok && e0 + kFwhtPer <= numel;
+    float v[kFwhtPer];
+    if (full) {
+#pragma unroll
+      for (int q = 0; q < kFwhtPer / VE; ++q) {
+        const Vec<R, VE> r = ldg_nt<R, VE>(x + e0 + q * VE);
+#pragma unroll
+        for (int i = 0; i < VE; ++i) v[q * VE + i] = IO::to_f32(r.v[i]);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kFwhtPer; ++i) v[i] = e0 + i < numel ? IO::to_f32(x[e0 + i]) : 0.0f;
+    }
+    const int pos = (int)(e0 & (a.b - 1));  // b divides the chunk size or is a multiple of 8
+    if (a.sign_in) {
+#pragma unroll
+      for (int i = 0; i < kFwhtPer; ++i) v[i] *= a.sign_in[(pos + i) & (a.b - 1)];
+    }
+    // strides 1, 2, 4: inside the lane (runs shorter than 8 stop early)
+#pragma unroll
+    for (int st = 1; st < kFwhtPer; st <<= 1) {
+      if (st < a.b) {
+#pragma unroll
+        for (int i = 0; i < kFwhtPer; ++i) {
+          if ((i & st) == 0) {
+            const float u = v[i], w = v[i + st];
+            v[i] = u + w;
+            v[i + st] = u - w;
+          }
+        }
+      }
+    }
+    // strides 8 ... b / 2: between lanes
+#pragma unroll
+    for (int m = 1; m < kWave; m <<= 1) {
+      if (m * kFwhtPer < a.b) {
+        const bool upper = (lane & m) != 0;
+#pragma unroll
+        for (int i = 0; i < kFwhtPer; ++i) {
+          const float other = lane_xor(v[i], m);
+          v[i] = upper ? other - v[i] : v[i] + other;
+        }
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kFwhtPer; ++i) {
+      v[i] *= factor;
+      if (a.sign_out) v[i] *= a.sign_out[(pos + i) & (a.b - 1)];
+    }
+    if (full) {
+#pragma unroll
+      for (int q = 0; q < kFwhtPer / VE; ++q) {
+        Vec<R, VE> r;
+#pragma unroll
+        for (int i = 0; i < VE; ++i) r.v[i] = IO::from_f32(v[q * VE + i]);
+        stg_nt<R, VE>(out + e0 + q * VE, r);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < kFwhtPer; ++i)
+        if (e0 + i < numel) out[e0 + i] = IO::from_f32(v[i]);
+    }
+  }
+}
+
 constexpr size_t kKmLdsMax = 160 * 1024 - 1024;
 
 size_t kron_lds_bytes(int h, int b) {
@@ -196,6 +296,15 @@ size_t kron_lds_bytes(int h, int b) {
 
 template <typename IO>
 int launch_kron(const KronArgs& a, hipStream_t st) {
+  if (a.h == 1 && a.sylvester && a.b <= kFwhtChunk) {
+    const int64_t numel = a.n_runs * a.b;
+    const int64_t n_chunks = (numel + kFwhtChunk - 1) / kFwhtChunk;
+    const int64_t n_wg = (n_chunks + kKmThreads / kWave - 1) / (kKmThreads / kWave);
+    const unsigned grid = (unsigned)(n_wg < 256 * 16 ? n_wg : 256 * 16);
+    const int vector_ok = (uintptr_t)a.x % 16 == 0 && (uintptr_t)a.out % 16 == 0;
+    hipLaunchKernelGGL(fwht_wave_kernel<IO>, grid, kKmThreads, 0, st, a, numel, vector_ok);
+    return CTMI_OK;
+  }
   if (a.b == 1) {
     const size_t lds = kron_lds_bytes(a.h, 1);
     auto kern = block_tile_kernel<IO>;
@@ -240,7 +349,9 @@ using namespace ctmi;
 
 extern "C" int ctmi_kron_matmul_supported(int32_t h, int32_t b, int32_t io_dtype) {
   if (!(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32)) return 0;
-  if (h < 1 || b < 1 || b > 256 || (b & (b - 1)) != 0) return 0;
+  if (h < 1 || b < 1 || (b & (b - 1)) != 0) return 0;
+  if (h == 1 && b <= 512) return 1;  // butterflies inside a wavefront
+  if (b > 256) return 0;
   return kron_lds_bytes(h, b) <= kKmLdsMax ? 1 : 0;  // a run (b = 1: a tile of 64) as fp32 in LDS
 }
 
@@ -256,6 +367,8 @@ extern "C" int ctmi_kron_matmul(const void* x, void* out, int32_t io_dtype, int6
                "a run of %d x %d elements does not fit the kernel (inner size a power of two up "
                "to 256 and %d x %d x 4 bytes within 159 KB; for inner size 1, h up to 313)",
                h, b, h, b);
+  CTMI_REQUIRE(b <= 256 || (h == 1 && sylvester), CTMI_ERR_UNSUPPORTED,
+               "an inner size of %d runs only as a plain Sylvester transform (h = 1)", b);
   CTMI_REQUIRE(numel % ((int64_t)h * b) == 0, CTMI_ERR_VALUE,
                "tensor size %lld is not a multiple of the transform size %lld", (long long)numel,
                (long long)h * b);

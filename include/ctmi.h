@@ -507,7 +507,8 @@ int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_
  * io_dtype (scale = 1 / sqrt(h * b) makes a Hadamard rotation orthonormal).  w: fp32
  * [h, h] row-major (any values); sign_in / sign_out: fp32 [h * b] or NULL; b a power of
  * two up to 256 and h * b * 4 bytes within 159 KB; for b = 1, 64 runs share a workgroup
- * and h may be at most 313 (ctmi_kron_matmul_supported).  fp32 accumulation on the vector
+ * and h may be at most 313; for h = 1 with the Sylvester factor b may be 512, and the
+ * butterflies stay in a wavefront's registers (ctmi_kron_matmul_supported).  fp32 accumulation on the vector
  * ALUs. */
 int ctmi_kron_matmul_supported(int32_t h, int32_t b, int32_t io_dtype);
 int ctmi_kron_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t h,

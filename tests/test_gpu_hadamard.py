@@ -258,7 +258,8 @@ def _sylvester64(n):
 
 
 @pytest.mark.parametrize("h,b", [(12, 2), (12, 64), (20, 8), (28, 128), (224, 64), (1, 256), (4, 64),
-                                 (8, 64), (1, 8), (3, 1), (148, 128)])
+                                 (8, 64), (1, 8), (3, 1), (148, 128), (1, 512), (1, 2), (1, 16),
+                                 (1, 1)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_kron_matmul(h, b, dtype, gpu):
     """x * diag(s_in) * (w (x) Sylvester(b)) * diag(s_out) / sqrt(h b) against fp64, for
@@ -281,6 +282,8 @@ def test_kron_matmul(h, b, dtype, gpu):
     y = kron_apply(x.to(gpu), w, inner=b, sign_in=s_in, sign_out=s_out, sylvester=True)
     want = ((x.double() * s_in.double()) @ dense * s_out.double() / n ** 0.5).to(dtype)
     _assert_within_ulp(y, want, "signs")
+    if b > 256:
+        return
     # without the Sylvester factor: w (x) I, unscaled
     y = kron_apply(x.to(gpu), w, inner=b, sylvester=False)
     want = (x.double() @ torch.kron(w.double(), torch.eye(b, dtype=torch.float64))).to(dtype)
@@ -314,6 +317,8 @@ def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
     assert ctmi.ctmi_kron_matmul_supported(314, 1, code) == 0
     assert ctmi.ctmi_kron_matmul_supported(12, 3, code) == 0      # inner size not a power of two
     assert ctmi.ctmi_kron_matmul_supported(12, 512, code) == 0    # more than 256 lanes
+    assert ctmi.ctmi_kron_matmul_supported(1, 512, code) == 1     # plain Sylvester: in registers
+    assert ctmi.ctmi_kron_matmul_supported(1, 1024, code) == 0
     assert ctmi.ctmi_kron_matmul_supported(256, 256, code) == 0   # 256 KB of LDS
     x = torch.zeros(314 * 4, dtype=torch.bfloat16, device=gpu)
     w = torch.zeros(314, 314, device=gpu)
@@ -322,6 +327,9 @@ def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
     rc = ctmi.ctmi_kron_matmul(x.data_ptr(), x.data_ptr(), code, 100, 12, 2, w.data_ptr(), None, None,
                                1, 1.0, None)
     assert rc == _lib.CTMI_ERR_VALUE  # 100 is not a multiple of 24
+    rc = ctmi.ctmi_kron_matmul(x.data_ptr(), x.data_ptr(), code, 1024, 1, 512, w.data_ptr(), None,
+                               None, 0, 1.0, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED  # 512 lanes only for the Sylvester factor
 
 
 @pytest.mark.parametrize("size", [768, 1600, 14336, 32, 256, 512, 16])
