@@ -555,6 +555,38 @@ def other_workload(torch, name, seed):
                 ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
                               [lambda m=m: _lib.check(lib.ctmi_hadamard_quant_pack_many(*m))], nb,
                               "hadamard_quant_pack_kernel", mfma_flops=flops))
+        # the full 4096-wide rotation (64 x 64) with the same quantization in its epilogue
+        mb64 = deterministic_hadamard_matrix(64, torch.bfloat16, dev).contiguous()
+        q4k = (torch.randint(0, 2, (4096,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
+        keep.extend([mb64, q4k])
+        for label in ("weights 4096x4096 (x16)", "weights 14336x4096 (x5)"):
+            xs = tensors[label]
+            calls = []
+            many = (_lib.HadamardPackJob * len(xs))()
+            for i, x in enumerate(xs):
+                one = (_lib.HadamardPackJob * 1)()
+                for job in (one[0], many[i]):
+                    packed = torch.empty(x.shape[0], x.shape[1] // 8, dtype=torch.int32, device=dev)
+                    scale = torch.empty(x.shape[0], x.shape[1] // 128, dtype=torch.bfloat16, device=dev)
+                    keep.extend([packed, scale])
+                    job.x, job.packed, job.scale, job.rotated, job.numel = (
+                        x.data_ptr(), packed.data_ptr(), scale.data_ptr(), None, x.numel())
+                keep.append(one)
+                a = (one, 1, code(x.dtype), 64, 64, mb64.data_ptr(), mb64.data_ptr(), q4k.data_ptr(), None,
+                     128, 4, 1, st)
+                calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_kron_quant_pack_many(*a)))
+            keep.append(many)
+            nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in xs)
+            flops = sum((2 * 64 + 6 * 64) * x.numel() for x in xs)
+            ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}", calls, nb,
+                          "hadamard_kron_kernel", primary=not label.startswith("weights 4096x4096"),
+                          mfma_flops=flops))
+            if label.startswith("weights 4096x4096"):
+                m = (many, len(xs), code(xs[0].dtype), 64, 64, mb64.data_ptr(), mb64.data_ptr(),
+                     q4k.data_ptr(), None, 128, 4, 1, st)
+                ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
+                              [lambda m=m: _lib.check(lib.ctmi_hadamard_kron_quant_pack_many(*m))], nb,
+                              "hadamard_kron_kernel", mfma_flops=flops))
         return "Hadamard rotation GB/s (bf16 MFMA), block 128 and full 4096, and fused with int4 packing", ops, keep
 
     raise SystemExit(f"unknown workload {name}")

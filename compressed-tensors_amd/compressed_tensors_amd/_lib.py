@@ -233,6 +233,11 @@ SIGNATURES = {
         [POINTER(HadamardPackJob), c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
          c_int32, c_void_p],
     ),
+    "ctmi_hadamard_kron_quant_pack_many": (
+        c_int32,
+        [POINTER(HadamardPackJob), c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_int32, c_int32, c_int32, c_void_p],
+    ),
     "ctmi_hadamard_apply": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p,

@@ -279,6 +279,25 @@ def kron_apply(
     return out
 
 
+_FUSED_KRON = {2048: (32, 64), 4096: (64, 64)}  # transform sizes fused with group size 128
+
+
+def _fused_plan(n: int, args) -> Optional[Tuple[int, int]]:
+    """None: block size n = group size (32, 64, 128); (a, b): transform size n = a * b with
+    groups of 128"""
+    kind = str(getattr(args.type, "value", args.type))
+    strategy = str(getattr(args.strategy, "value", args.strategy))
+    if not (args.num_bits == 4 and kind == "int" and args.symmetric and strategy == "group"):
+        raise NotImplementedError("the fused path covers symmetric int4 group quantization")
+    if n in (32, 64, 128) and args.group_size == n:
+        return None
+    if n in _FUSED_KRON and args.group_size == 128:
+        return _FUSED_KRON[n]
+    raise NotImplementedError(
+        "the fused path covers block sizes 32, 64 and 128 with group_size == block size, and "
+        "transform sizes 2048 and 4096 with group_size 128")
+
+
 def hadamard_quantize_pack(
     value: Tensor,
     n: int,
@@ -289,43 +308,54 @@ def hadamard_quantize_pack(
     return_rotated: bool = False,
 ) -> Dict[str, Tensor]:
     """hadamard_apply, the min-max observer and pack-quantized compression in one
-    pass over a bf16 [rows, cols] tensor, for block size n (32, 64 or 128) equal
-    to the group size of a symmetric 4-bit integer scheme.  Returns what the
-    three steps return, bit for bit: weight_packed int32 [rows, cols / 8],
-    weight_scale bf16 [rows, cols / n], weight_shape int64 [2] (and the rotated
-    tensor under "rotated" if asked for)."""
-    x = to_gpu(value).contiguous()
-    args = quantization_args
-    if x.ndim != 2 or x.dtype != torch.bfloat16:
-        raise NotImplementedError("the fused path takes 2-D bfloat16 tensors")
-    if not (args.num_bits == 4 and str(getattr(args.type, "value", args.type)) == "int" and args.symmetric
-            and str(getattr(args.strategy, "value", args.strategy)) == "group" and args.group_size == n):
-        raise NotImplementedError(
-            "the fused path covers symmetric int4 group quantization with group_size == block size")
-    if n not in (32, 64, 128):
-        raise NotImplementedError("block size must be 32, 64 or 128")
-    rows, cols = x.shape
-    if cols % n != 0:
-        raise ValueError(f"{n} must divide the last dimension {cols}")
-    dev = x.device
-    mb_t = (_sylvester_bf16(n, dev) if matrix_t is None
-            else matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous())
+    pass over a bf16 [rows, cols] tensor of a symmetric 4-bit integer group scheme:
+    block size n (32, 64 or 128) equal to the group size, or a transform of size 2048 or
+    4096 with groups of 128.  Returns what the three steps return, bit for bit:
+    weight_packed int32 [rows, cols / 8], weight_scale bf16 [rows, cols / group_size],
+    weight_shape int64 [2] (and the rotated tensor under "rotated" if asked for)."""
+    return _quantize_pack([value], n, quantization_args, sign_in, sign_out, matrix_t,
+                          return_rotated)[0]
+
+
+def _quantize_pack(values, n, args, sign_in, sign_out, matrix_t, return_rotated):
+    xs = [to_gpu(v).contiguous() for v in values]
+    plan = _fused_plan(n, args)
+    if plan is not None and matrix_t is not None:
+        raise NotImplementedError("explicit matrices are supported for sizes 32, 64 and 128")
+    dev = xs[0].device
+    for x in xs:
+        if x.ndim != 2 or x.dtype != torch.bfloat16 or x.device != dev:
+            raise NotImplementedError("the fused path takes 2-D bfloat16 tensors on one device")
+        if x.shape[1] % n != 0:
+            raise ValueError(f"{n} must divide the last dimension {x.shape[1]}")
     s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
     s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
-    packed = torch.empty((rows, cols // 8), dtype=torch.int32, device=dev)
-    scale = torch.empty((rows, cols // n), dtype=torch.bfloat16, device=dev)
-    rotated = torch.empty_like(x) if return_rotated else None
-    _lib.check(
-        _lib.load().ctmi_hadamard_quant_pack(
-            x.data_ptr(), _lib.dtype_code(x.dtype), x.numel(), n, mb_t.data_ptr(), _lib.ptr(s_in),
-            _lib.ptr(s_out), 4, 1, packed.data_ptr(), scale.data_ptr(), _lib.ptr(rotated),
-            _lib.stream_of(dev),
-        )
-    )
-    out = {"weight_packed": packed, "weight_scale": scale, "weight_shape": torch.tensor(x.shape)}
-    if return_rotated:
-        out["rotated"] = rotated
-    return out
+    group = args.group_size
+    jobs = (_lib.HadamardPackJob * len(xs))()
+    results = []
+    for job, x in zip(jobs, xs):
+        rows, cols = x.shape
+        packed = torch.empty((rows, cols // 8), dtype=torch.int32, device=dev)
+        scale = torch.empty((rows, cols // group), dtype=torch.bfloat16, device=dev)
+        rotated = torch.empty_like(x) if return_rotated else None
+        job.x, job.packed, job.scale, job.rotated, job.numel = (
+            x.data_ptr(), packed.data_ptr(), scale.data_ptr(), _lib.ptr(rotated), x.numel())
+        out = {"weight_packed": packed, "weight_scale": scale, "weight_shape": torch.tensor(x.shape)}
+        if return_rotated:
+            out["rotated"] = rotated
+        results.append(out)
+    lib, code, stream = _lib.load(), _lib.dtype_code(torch.bfloat16), _lib.stream_of(dev)
+    if plan is None:
+        mb_t = (_sylvester_bf16(n, dev) if matrix_t is None
+                else matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous())
+        _lib.check(lib.ctmi_hadamard_quant_pack_many(
+            jobs, len(xs), code, n, mb_t.data_ptr(), _lib.ptr(s_in), _lib.ptr(s_out), 4, 1, stream))
+    else:
+        a, b = plan
+        _lib.check(lib.ctmi_hadamard_kron_quant_pack_many(
+            jobs, len(xs), code, a, b, _sylvester_bf16(a, dev).data_ptr(),
+            _sylvester_bf16(b, dev).data_ptr(), _lib.ptr(s_in), _lib.ptr(s_out), group, 4, 1, stream))
+    return results
 
 
 def hadamard_apply_many(
@@ -387,40 +417,7 @@ def hadamard_quantize_pack_many(
     launch); one dict per tensor, as hadamard_quantize_pack returns it"""
     if not values:
         return []
-    xs = [to_gpu(v).contiguous() for v in values]
-    args = quantization_args
-    if not (args.num_bits == 4 and str(getattr(args.type, "value", args.type)) == "int" and args.symmetric
-            and str(getattr(args.strategy, "value", args.strategy)) == "group" and args.group_size == n):
-        raise NotImplementedError(
-            "the fused path covers symmetric int4 group quantization with group_size == block size")
-    if n not in (32, 64, 128):
-        raise NotImplementedError("block size must be 32, 64 or 128")
-    dev = xs[0].device
-    for x in xs:
-        if x.ndim != 2 or x.dtype != torch.bfloat16 or x.device != dev:
-            raise NotImplementedError("the fused path takes 2-D bfloat16 tensors on one device")
-        if x.shape[1] % n != 0:
-            raise ValueError(f"{n} must divide the last dimension {x.shape[1]}")
-    mb_t = (_sylvester_bf16(n, dev) if matrix_t is None
-            else matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous())
-    s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
-    s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
-    jobs = (_lib.HadamardPackJob * len(xs))()
-    results = []
-    for job, x in zip(jobs, xs):
-        rows, cols = x.shape
-        packed = torch.empty((rows, cols // 8), dtype=torch.int32, device=dev)
-        scale = torch.empty((rows, cols // n), dtype=torch.bfloat16, device=dev)
-        job.x, job.packed, job.scale, job.rotated, job.numel = (
-            x.data_ptr(), packed.data_ptr(), scale.data_ptr(), None, x.numel())
-        results.append({"weight_packed": packed, "weight_scale": scale,
-                        "weight_shape": torch.tensor(x.shape)})
-    _lib.check(
-        _lib.load().ctmi_hadamard_quant_pack_many(
-            jobs, len(xs), _lib.dtype_code(torch.bfloat16), n, mb_t.data_ptr(), _lib.ptr(s_in),
-            _lib.ptr(s_out), 4, 1, _lib.stream_of(dev))
-    )
-    return results
+    return _quantize_pack(values, n, quantization_args, sign_in, sign_out, matrix_t, False)
 
 
 # ------------------------------------------------------------------ vocabulary

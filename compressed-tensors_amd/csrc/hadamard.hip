@@ -629,11 +629,23 @@ hadamard_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const uint16_t* __res
 // Signs (entries +1 / -1) are XOR masks on the bf16 sign bits of X and of the
 // output; they are per position within the row, the same for every row, and sit
 // in LDS in the lanes' own layout.
-template <int A, int B, bool HALF, bool MANY>
+//
+// B = 64: a sub-row is one 128-byte line.  Its two halves (column pairs p = 0, 1) come out
+// of stage 2 one after the other; the first is held back so that both stores leave
+// together and meet in the cache as a whole line.
+//
+// QUANT (B = 64, bfloat16): the W4A16 pipeline for group size 128 in the epilogue, as in
+// hadamard_quant_pack_kernel.  A group is two neighbouring output sub-rows, i.e. the 8
+// lanes (l16 ^ 1, every lq) with both halves: they agree on max |x| through three lane
+// exchanges, then each lane quantizes and packs its 2 x 8 values into two words.  jobs.out
+// is then the packed tensor, jobs.scale the group scales, jobs.rotated (optional) the
+// rotated tensor.
+template <int A, int B, bool HALF, bool MANY, bool QUANT = false>
 __global__ void __launch_bounds__(kKronThreads) __attribute__((amdgpu_waves_per_eu(CTMI_HAD_KRON_WAVES)))
 hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ mbt,
                      const uint16_t* __restrict__ mat, const float* __restrict__ s_in,
-                     const float* __restrict__ s_out, float inv_sqrt_n) {
+                     const float* __restrict__ s_out, float inv_sqrt_n, QpCfg cfg) {
+  static_assert(!QUANT || (B == 64 && !HALF), "the fused epilogue is written for 64-wide bf16 sub-rows");
   constexpr int N = A * B;
   constexpr int KS = B / 32;   // k steps of stage 1
   constexpr int MT = A / 16;   // sub-row tiles
@@ -706,7 +718,16 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
     int64_t local;
     const int j = had_job<MANY>(jobs, row, &local);  // n_rows: data rows over all jobs
     const uint16_t* src = static_cast<const uint16_t*>(jobs.x[j]) + local * N;
-    uint16_t* dst = static_cast<uint16_t*>(jobs.out[j]) + local * N;
+    uint16_t* dst = QUANT ? static_cast<uint16_t*>(jobs.rotated[j])
+                          : static_cast<uint16_t*>(jobs.out[j]);
+    if (!QUANT || dst) dst += local * N;
+    int32_t* packed = nullptr;
+    uint16_t* scale = nullptr;
+    if constexpr (QUANT) {
+      packed = static_cast<int32_t*>(jobs.out[j]) + local * (N / 8);
+      scale = static_cast<uint16_t*>(jobs.scale[j]) + local * (N / 128);
+    }
+    u32x4_t held[B == 64 ? AT : 1];  // first halves of the output sub-rows
     xfrag_t xf[MT][KS];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
@@ -786,7 +807,46 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
           o[3] = pack_bf16x2(y1[2] * inv_sqrt_n, y1[3] * inv_sqrt_n);
         }
         if (signed_io) o ^= sign_out_lds[at * (NT / 2) + p][lane];
-        stg<uint16_t, 8>(dst + (16 * at + l16) * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o));
+        uint16_t* at_dst = dst + (16 * at + l16) * B + 8 * lq;
+        if constexpr (B != 64) {
+          stg<uint16_t, 8>(at_dst + 32 * p, __builtin_bit_cast(Vec<uint16_t, 8>, o));
+        } else if (p == 0) {
+          held[at] = o;
+        } else if constexpr (!QUANT) {
+          stg<uint16_t, 8>(at_dst, __builtin_bit_cast(Vec<uint16_t, 8>, held[at]));
+          stg<uint16_t, 8>(at_dst + 32, __builtin_bit_cast(Vec<uint16_t, 8>, o));
+        } else {
+          // max |x| of the group on the packed 16-bit halves (bf16 magnitudes order like
+          // their bit patterns, a NaN above everything), then over the group's 8 lanes
+          typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+          u16x2_t top = {0, 0};
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2_t, held[at][w] & 0x7FFF7FFFu));
+            top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2_t, o[w] & 0x7FFF7FFFu));
+          }
+          uint32_t mag = top.x > top.y ? top.x : top.y;
+#pragma unroll
+          for (int d = 1; d < 64; d = d == 1 ? 16 : d << 1) {
+            const uint32_t other = (uint32_t)__shfl_xor((int)mag, d, kWave);
+            mag = other > mag ? other : mag;
+          }
+          // calculate_qparams, symmetric, in bf16 (helpers.py:101-122)
+          float sv = bf16_to_f32(f32_to_bf16(bf16_to_f32((uint16_t)mag) / cfg.sym_div));
+          sv = (sv != sv) ? sv : fmaxf(sv, 1.1920928955078125e-07f);
+          const Vec<int32_t, 1> w0 = quant_pack8<BF16, BF16, 4, false>(
+              __builtin_bit_cast(Vec<uint16_t, 8>, held[at]), sv, 0.0f, cfg.bit_min, cfg.bit_max);
+          const Vec<int32_t, 1> w1 = quant_pack8<BF16, BF16, 4, false>(
+              __builtin_bit_cast(Vec<uint16_t, 8>, o), sv, 0.0f, cfg.bit_min, cfg.bit_max);
+          const int sub = 16 * at + l16;
+          packed[sub * (B / 8) + lq] = w0.v[0];
+          packed[sub * (B / 8) + 4 + lq] = w1.v[0];
+          if (lq == 0 && (l16 & 1) == 0) scale[sub / 2] = f32_to_bf16(sv);
+          if (dst) {
+            stg<uint16_t, 8>(at_dst, __builtin_bit_cast(Vec<uint16_t, 8>, held[at]));
+            stg<uint16_t, 8>(at_dst + 32, __builtin_bit_cast(Vec<uint16_t, 8>, o));
+          }
+        }
       }
     }
   }
@@ -800,12 +860,30 @@ static int launch_had_kron_jobs(const HadJobs& jobs, int n_jobs, const HadArgs& 
   // as many workgroups as are resident at once (register-limited)
   const int64_t cap = 256 * 4 * (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES)) / kKronWaves;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
+  const QpCfg none{};
   if (n_jobs == 1)
     hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF, false>), grid, kKronThreads, 0, st, jobs, n_rows,
-                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n);
+                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, none);
   else
     hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF, true>), grid, kKronThreads, 0, st, jobs, n_rows,
-                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n);
+                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, none);
+  return CTMI_OK;
+}
+
+// the same with the quantization epilogue (bf16, B = 64, group size 128)
+template <int A>
+static int launch_had_kron_quant_jobs(const HadJobs& jobs, int n_jobs, const HadArgs& a,
+                                      const QpCfg& cfg, hipStream_t st) {
+  const int64_t n_rows = jobs.end[n_jobs - 1];
+  const int64_t wgs = cdiv(n_rows, kKronWaves);
+  const int64_t cap = 256 * 4 * (A * 64 <= 2048 ? 4 : CTMI_HAD_KRON_WAVES) / kKronWaves;
+  const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
+  if (n_jobs == 1)
+    hipLaunchKernelGGL((hadamard_kron_kernel<A, 64, false, false, true>), grid, kKronThreads, 0, st,
+                       jobs, n_rows, a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, cfg);
+  else
+    hipLaunchKernelGGL((hadamard_kron_kernel<A, 64, false, true, true>), grid, kKronThreads, 0, st,
+                       jobs, n_rows, a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, cfg);
   return CTMI_OK;
 }
 
@@ -1091,6 +1169,83 @@ extern "C" int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs,
   if (!any) return CTMI_OK;
   if (filled) hqp_launch(t, filled, b_dim, mb_t, sign_in, sign_out, num_bits, st);
   return check_launch("ctmi_hadamard_quant_pack_many");
+}
+
+extern "C" int ctmi_hadamard_kron_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_jobs,
+                                                  int32_t io_dtype, int32_t a_dim, int32_t b_dim,
+                                                  const void* ma_t, const void* mb_t,
+                                                  const float* sign_in, const float* sign_out,
+                                                  int32_t group_size, int32_t num_bits,
+                                                  int32_t symmetric, void* stream) {
+  CTMI_REQUIRE(n_jobs >= 0 && (jobs || n_jobs == 0), CTMI_ERR_VALUE, "bad job list");
+  CTMI_REQUIRE(io_dtype == CTMI_BF16, CTMI_ERR_UNSUPPORTED,
+               "the fused rotation + quantization takes bfloat16 tensors");
+  CTMI_REQUIRE((a_dim == 32 || a_dim == 64) && b_dim == 64, CTMI_ERR_UNSUPPORTED,
+               "the fused rotation + quantization covers the factorisations 32 x 64 and 64 x 64, "
+               "got %d x %d", a_dim, b_dim);
+  CTMI_REQUIRE(group_size == 128, CTMI_ERR_UNSUPPORTED, "group size must be 128, got %d", group_size);
+  CTMI_REQUIRE(num_bits == 4 && symmetric, CTMI_ERR_UNSUPPORTED,
+               "only symmetric 4-bit integer quantization is fused");
+  if (n_jobs == 0) return CTMI_OK;
+  const int64_t n = (int64_t)a_dim * b_dim;
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_hadamard_pack_job& j = jobs[i];
+    CTMI_REQUIRE(j.numel >= 0 && j.numel % n == 0, CTMI_ERR_VALUE,
+                 "job %lld: tensor size %lld is not a multiple of the transform size %lld",
+                 (long long)i, (long long)j.numel, (long long)n);
+    if (j.numel == 0) continue;
+    CTMI_REQUIRE(j.x && j.packed && j.scale, CTMI_ERR_VALUE, "job %lld: NULL tensor pointer",
+                 (long long)i);
+    CTMI_REQUIRE((uintptr_t)j.x % 16 == 0 && (uintptr_t)j.rotated % 16 == 0 &&
+                     (uintptr_t)j.packed % 4 == 0 && (uintptr_t)j.scale % 2 == 0,
+                 CTMI_ERR_VALUE, "tensors must be 16-byte aligned");
+  }
+  CTMI_REQUIRE(mb_t && ma_t && (uintptr_t)mb_t % 16 == 0 && (uintptr_t)ma_t % 16 == 0, CTMI_ERR_VALUE,
+               "the matrices must be given, 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  QpCfg c{};
+  quant_range(CTMI_QTYPE_INT, num_bits, &c.bit_min, &c.bit_max);
+  c.range = c.bit_max - c.bit_min;
+  c.sym_div = (float)((double)c.range / 2.0);
+  c.qtype = CTMI_QTYPE_INT;
+  c.num_bits = num_bits;
+  c.symmetric = 1;
+  c.mt = c.zp_sub_dtype = c.scale_dtype = CTMI_BF16;
+  c.zp_dtype = CTMI_I8;
+  HadArgs a;
+  a.x = nullptr;
+  a.out = nullptr;
+  a.mbt = (const uint16_t*)mb_t;
+  a.mat = (const uint16_t*)ma_t;
+  a.s_in = sign_in;
+  a.s_out = sign_out;
+  a.n_sub = 0;
+  a.sqrt_n = sqrtf((float)n);
+  HadJobs t;
+  clear_jobs(&t);
+  int filled = 0;
+  bool any = false;
+  auto flush = [&]() {
+    if (a_dim == 32) launch_had_kron_quant_jobs<32>(t, filled, a, c, st);
+    else launch_had_kron_quant_jobs<64>(t, filled, a, c, st);
+    clear_jobs(&t);
+    filled = 0;
+  };
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_hadamard_pack_job& j = jobs[i];
+    if (j.numel == 0) continue;
+    any = true;
+    t.x[filled] = j.x;
+    t.out[filled] = j.packed;
+    t.scale[filled] = j.scale;
+    t.rotated[filled] = j.rotated;
+    t.n_sub[filled] = j.numel / b_dim;
+    t.end[filled] = (filled ? t.end[filled - 1] : 0) + j.numel / n;
+    if (++filled == kHadMaxJobs) flush();
+  }
+  if (!any) return CTMI_OK;
+  if (filled) flush();
+  return check_launch("ctmi_hadamard_kron_quant_pack_many");
 }
 
 extern "C" int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t numel, int32_t b_dim,

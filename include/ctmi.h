@@ -496,6 +496,17 @@ int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_
                                   const float* sign_in, const float* sign_out, int32_t num_bits,
                                   int32_t symmetric, void* stream);
 
+/* The same pipeline for transforms of size a_dim * b_dim = 32 x 64 or 64 x 64 (2048, 4096)
+ * with group size 128: ctmi_hadamard_apply (factored form, ma_t / mb_t as there), the
+ * symmetric int4 min-max observer over groups of 128 and ctmi_pack_quantized_compress in
+ * one pass; same bits as those calls in sequence.  packed: int32 [numel / 8]; scale: bf16
+ * [numel / 128]; rotated optional. */
+int ctmi_hadamard_kron_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_jobs,
+                                       int32_t io_dtype, int32_t a_dim, int32_t b_dim,
+                                       const void* ma_t, const void* mb_t, const float* sign_in,
+                                       const float* sign_out, int32_t group_size, int32_t num_bits,
+                                       int32_t symmetric, void* stream);
+
 /* A23 / A24 for matrices with an explicit factor (transform/utils/matrix.py:137-171 for
  * a small explicit matrix; transform/utils/hadamard.py:102-163 for the reference's
  * Hadamard matrices of size K * 2^m built from its table of known K x K matrices,

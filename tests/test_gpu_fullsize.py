@@ -239,19 +239,21 @@ def test_hadamard_weight_rotation_at_full_size(n, shape, gpu):
         assert not bool((err > tol).any()), f"rows {sl}: max ratio {(err / tol).max():.2f}"
 
 
-def test_fused_rotation_quantization_packing_at_full_size(gpu):
-    """hadamard_quantize_pack on a 14336 x 4096 weight (block 128 = group 128): the rotated
-    tensor equals hadamard_apply's, and scales / packed words equal the oracle's observer
-    and pack-quantized compressor on the rotated rows"""
+@pytest.mark.parametrize("n", [128, 4096])
+def test_fused_rotation_quantization_packing_at_full_size(n, gpu):
+    """hadamard_quantize_pack on a 14336 x 4096 weight (block 128 = group 128, and the full
+    4096-wide rotation with groups of 128): the rotated tensor equals hadamard_apply's, and
+    scales / packed words equal the oracle's observer and pack-quantized compressor on the
+    rotated rows"""
     from compressed_tensors_amd.quantization import QuantizationArgs
     from compressed_tensors_amd.transform import hadamard_apply, hadamard_quantize_pack
 
-    n, shape = 128, (14336, 4096)
+    shape = (14336, 4096)
     announce("fused hadamard + int4 + pack", n, shape)
     g = torch.Generator(device=gpu).manual_seed(9)
     w = (torch.randn(shape, generator=g, device=gpu) * 0.02).bfloat16()
     q = (torch.randint(0, 2, (n,), generator=torch.Generator().manual_seed(5)) * 2 - 1).float()
-    spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=n)
+    spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
     args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
     fused = hadamard_quantize_pack(w, n, args, return_rotated=True, sign_out=q)
     y = hadamard_apply(w, n, sign_out=q)

@@ -168,7 +168,8 @@ def test_large_activation_properties(gpu):
         assert float(rel) < 2e-2
 
 
-@pytest.mark.parametrize("n,shape", [(128, (64, 512)), (128, (37, 256)), (64, (33, 192)), (32, (19, 96))])
+@pytest.mark.parametrize("n,shape", [(128, (64, 512)), (128, (37, 256)), (64, (33, 192)), (32, (19, 96)),
+                                     (4096, (37, 4096)), (4096, (5, 8192)), (2048, (21, 4096))])
 def test_fused_rotation_quantization_packing(n, shape, gpu):
     """ctmi_hadamard_quant_pack == hadamard_apply -> min-max observer -> pack-quantized
     compress, bit for bit (each of which is checked against the oracle on its own), and
@@ -182,9 +183,13 @@ def test_fused_rotation_quantization_packing(n, shape, gpu):
     announce("fused hadamard + int4 + pack", n, shape)
     g = torch.Generator().manual_seed(3 * n + shape[0])
     x = (torch.randn(shape, generator=g) * 0.02).bfloat16()
-    x[0, :n] = 0  # an all-zero group: scale clamps to eps
+    group = min(n, 128)  # transforms of 2048 / 4096 elements feed groups of 128
+    if n <= 128:
+        x[0, :n] = 0  # an all-zero group: scale clamps to eps
+    else:
+        x[1] = 0      # a rotated row of zeros: every group of it
     q = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
-    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=n)
+    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=group)
     for signs in (dict(), dict(sign_in=q), dict(sign_out=q)):
         fused = hadamard_quantize_pack(x.to(gpu), n, args, return_rotated=True, **signs)
         y = hadamard_apply(x.to(gpu), n, **signs)
@@ -196,7 +201,7 @@ def test_fused_rotation_quantization_packing(n, shape, gpu):
         assert torch.equal(fused["weight_packed"], want["weight_packed"]), "packed codes"
         assert fused["weight_shape"].tolist() == list(shape)
         # the oracle's chain on the same rotated tensor
-        oargs = oq._Args(num_bits=4, type="int", symmetric=True, strategy="group", group_size=n)
+        oargs = oq._Args(num_bits=4, type="int", symmetric=True, strategy="group", group_size=group)
         yc = y.cpu()
         o_scale, o_zp = oq.observe_weight(yc, oargs)
         o_packed = op.pack_quantized_compress(yc, o_scale, oargs, zero_point=o_zp)["weight_packed"]
@@ -228,18 +233,20 @@ def test_many_tensors_in_one_call(n, dtype, gpu):
                 assert_bit_equal(y, hadamard_apply(x, n, **signs), f"tensor {i} ({rows[i]} rows)")
 
 
-def test_fused_many_tensors_in_one_call(gpu):
+@pytest.mark.parametrize("n", [128, 4096])
+def test_fused_many_tensors_in_one_call(n, gpu):
     """hadamard_quantize_pack_many == hadamard_quantize_pack tensor by tensor"""
     from compressed_tensors_amd.quantization import QuantizationArgs
     from compressed_tensors_amd.transform import hadamard_quantize_pack, hadamard_quantize_pack_many
 
-    announce("fused hadamard many")
-    n = 128
+    announce("fused hadamard many", n)
     g = torch.Generator().manual_seed(77)
     q = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
-    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=n)
+    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
     shapes = [(64, 512), (37, 256), (16, 128), (5, 1024), (128, 256), (1, 128), (48, 384), (33, 128), (96, 640),
               (7, 256)]
+    if n > 128:
+        shapes = [(r, n * (1 + i % 2)) for i, (r, _) in enumerate(shapes)]
     xs = [(torch.randn(s, generator=g) * 0.02).bfloat16().to(gpu) for s in shapes]
     for signs in (dict(), dict(sign_in=q)):
         got = hadamard_quantize_pack_many(xs, n, args, **signs)
