@@ -320,6 +320,7 @@ def other_workload(torch, name, seed):
         from compressed_tensors_amd.compressors import get_24_bytemasks
         from compressed_tensors_amd.quantization import quantize
         copies24 = 16  # values + bitmask of the codes are 37 MB a copy: well beyond the 256 MB last-level cache
+        s24_jobs = []
         for _ in range(copies24):
             w = randn(14336, 4096, 0.02)
             w = torch.where(get_24_bytemasks(w), w, torch.zeros_like(w))
@@ -343,6 +344,7 @@ def other_workload(torch, name, seed):
             two_step.append(lambda qa=qa, a=a: (_lib.check(lib.ctmi_qdq(*qa)), _lib.check(lib.ctmi_sparse24_compress(*a))))
             one_step.append(lambda fa=fa: _lib.check(lib.ctmi_quantize_sparse24_compress(*fa)))
             t_calls.append(lambda d=d: _lib.check(lib.ctmi_sparse24_decompress(*d)))
+            s24_jobs.append((q, values, bitmask, dense, rows, cols))
             # the bool mask of the weight <-> its packed form
             bools = get_24_bytemasks(w)
             bools_back = torch.empty_like(bools)
@@ -373,6 +375,14 @@ def other_workload(torch, name, seed):
                   tmp_dq.data_ptr(), rows, cols, ctypes.byref(plan.qp), st)
             back_two.append(lambda d=d, dq=dq: (_lib.check(lib.ctmi_sparse24_decompress(*d)), _lib.check(lib.ctmi_qdq(*dq))))
             back_one.append(lambda fd=fd: _lib.check(lib.ctmi_sparse24_decompress_dequantize(*fd)))
+        cj, dj = (_lib.Sparse24Job * copies24)(), (_lib.Sparse24Job * copies24)()
+        for k, (q, values, bitmask, dense, rows, cols) in enumerate(s24_jobs):
+            for job, full in ((cj[k], q), (dj[k], dense)):
+                job.dense, job.values, job.bitmask = full.data_ptr(), values.data_ptr(), bitmask.data_ptr()
+                job.nvalues, job.rows, job.cols = values.numel(), rows, cols
+        keep.extend([cj, dj])
+        cm = (cj, copies24, code(FP8), st)
+        dm = (dj, copies24, 1, st)
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies24 * (n24 + n24 // 2 + n24 // 8)
         fused24_bytes = copies24 * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
@@ -380,6 +390,10 @@ def other_workload(torch, name, seed):
                Op("sparse-bitmask decompress (positions from the bitmask alone)", d_calls, bm_bytes, "bitmask_scatter_tiles_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
+               Op("sparse-24-bitmask compress, fp8, all 16 in one call (8 per launch)",
+                  [lambda: _lib.check(lib.ctmi_sparse24_compress_many(*cm))], s24_bytes, "sparse24_compress_chain_kernel"),
+               Op("sparse-24-bitmask decompress, fp8, all 16 in one call (8 per launch)",
+                  [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm))], s24_bytes, "sparse24_scatter_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 bf16", s16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress, bf16", t16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel"),
                Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies24 * (n24 + n24 // 8), "pack_bitmasks"),

@@ -98,6 +98,13 @@ class HadamardPackJob(ctypes.Structure):
                 ("numel", c_int64)]
 
 
+class Sparse24Job(ctypes.Structure):
+    """mirror of `struct ctmi_sparse24_job`"""
+
+    _fields_ = [("dense", c_void_p), ("values", c_void_p), ("bitmask", c_void_p),
+                ("nvalues", c_int64), ("rows", c_int64), ("cols", c_int64)]
+
+
 class ObserveQuantizeJob(ctypes.Structure):
     """mirror of `struct ctmi_observe_quantize_job`"""
 
@@ -228,6 +235,8 @@ SIGNATURES = {
         [POINTER(HadamardJob), c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
          c_void_p, c_void_p],
     ),
+    "ctmi_sparse24_compress_many": (c_int32, [POINTER(Sparse24Job), c_int64, c_int32, c_void_p]),
+    "ctmi_sparse24_decompress_many": (c_int32, [POINTER(Sparse24Job), c_int64, c_int32, c_void_p]),
     "ctmi_hadamard_quant_pack_many": (
         c_int32,
         [POINTER(HadamardPackJob), c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,

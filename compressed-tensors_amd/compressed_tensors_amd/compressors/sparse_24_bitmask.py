@@ -23,6 +23,8 @@ __all__ = [
     "Sparse24BitMaskTensor",
     "sparse24_bitmask_compress",
     "sparse24_bitmask_decompress",
+    "sparse24_bitmask_compress_many",
+    "sparse24_bitmask_decompress_many",
     "quantize_sparse24_compress",
     "sparse24_decompress_dequantize",
     "get_24_bytemasks",
@@ -81,6 +83,84 @@ def sparse24_bitmask_compress(
         )
     )
     return values, bitmask
+
+
+def _streams(rows: int, cols: int, esize: int, decompress: bool) -> bool:
+    """the shapes the multi-tensor entry points take: rows of whole bitmask bytes and a
+    whole number of work items"""
+    per = 16 if esize == 1 else 8
+    return rows > 0 and cols > 0 and cols % 8 == 0 and (rows * cols) % per == 0
+
+
+def sparse24_bitmask_compress_many(tensors: List[Tensor]) -> List[Tuple[Tensor, Tensor]]:
+    """sparse24_bitmask_compress on several 2-D tensors: those of one dtype go to the GPU
+    in one call (ctmi_sparse24_compress_many, 8 tensors per launch); shapes it does not
+    take get a call of their own.  Same bits either way."""
+    results: List[Optional[Tuple[Tensor, Tensor]]] = [None] * len(tensors)
+    by_dtype: Dict[torch.dtype, List[int]] = {}
+    xs: List[Optional[Tensor]] = [None] * len(tensors)
+    for i, t in enumerate(tensors):
+        if t.is_meta or t.ndim != 2 or t.dtype not in _RANKABLE or not _streams(
+                t.shape[0], t.shape[1], t.element_size(), False):
+            results[i] = sparse24_bitmask_compress(t)
+            continue
+        xs[i] = to_gpu(t).contiguous()
+        by_dtype.setdefault(t.dtype, []).append(i)
+    lib = _lib.load()
+    for dtype, idx in by_dtype.items():
+        dev = xs[idx[0]].device
+        idx_here = [i for i in idx if xs[i].device == dev]
+        for i in idx:
+            if xs[i].device != dev:
+                results[i] = sparse24_bitmask_compress(xs[i])
+        jobs = (_lib.Sparse24Job * len(idx_here))()
+        for job, i in zip(jobs, idx_here):
+            x = xs[i]
+            rows, cols = x.shape
+            values = torch.empty((rows, cols // 2), dtype=dtype, device=dev)
+            bitmask = torch.empty((rows, cols // 8), dtype=torch.uint8, device=dev)
+            job.dense, job.values, job.bitmask = x.data_ptr(), values.data_ptr(), bitmask.data_ptr()
+            job.nvalues, job.rows, job.cols = values.numel(), rows, cols
+            results[i] = (values, bitmask)
+        _lib.check(lib.ctmi_sparse24_compress_many(jobs, len(idx_here), _lib.dtype_code(dtype),
+                                                   _lib.stream_of(dev)))
+    return results
+
+
+def sparse24_bitmask_decompress_many(items: List[Tuple[Tensor, Tensor, List[int]]]) -> List[Tensor]:
+    """sparse24_bitmask_decompress on several (values, bitmask, shape) triples: those of one
+    element size go to the GPU in one call (ctmi_sparse24_decompress_many)"""
+    results: List[Optional[Tensor]] = [None] * len(items)
+    groups: Dict[Tuple[torch.dtype, str], List[int]] = {}
+    prepared = {}
+    for i, (values, bitmask, shape) in enumerate(items):
+        shape = [int(d) for d in (shape.flatten().tolist() if isinstance(shape, Tensor) else shape)]
+        rows = 1
+        for d in shape[:-1]:
+            rows *= d
+        cols = shape[-1] if shape else 0
+        ok = (not values.is_meta and len(shape) >= 1 and _streams(rows, cols, values.element_size(), True)
+              and values.numel() * 2 == rows * cols and bitmask.numel() * 8 == rows * cols
+              and values.element_size() in (1, 2, 4))
+        if not ok:
+            results[i] = sparse24_bitmask_decompress(values, bitmask, shape)
+            continue
+        v, b = to_gpu(values).contiguous().reshape(-1), to_gpu(bitmask).contiguous()
+        prepared[i] = (v, b, shape, rows, cols)
+        groups.setdefault((v.dtype, str(v.device)), []).append(i)
+    lib = _lib.load()
+    for (dtype, _), idx in groups.items():
+        dev = prepared[idx[0]][0].device
+        jobs = (_lib.Sparse24Job * len(idx))()
+        for job, i in zip(jobs, idx):
+            v, b, shape, rows, cols = prepared[i]
+            out = torch.empty(shape, dtype=dtype, device=dev)
+            job.dense, job.values, job.bitmask = out.data_ptr(), v.data_ptr(), b.data_ptr()
+            job.nvalues, job.rows, job.cols = v.numel(), rows, cols
+            results[i] = out
+        _lib.check(lib.ctmi_sparse24_decompress_many(jobs, len(idx), v.element_size(),
+                                                     _lib.stream_of(dev)))
+    return results
 
 
 def quantize_sparse24_compress(weight: Tensor, scale: Tensor, quantization_args,
@@ -229,3 +309,35 @@ class Sparse24BitMaskCompressor(BaseSparseCompressor):
 
     def decompress_weight(self, weight_data):
         return Sparse24BitMaskTensor.from_compressed_data(**weight_data).decompress()
+
+    # the whole state dict in a few calls: the weights of one dtype share launches
+    def compress(self, model_state, compression_targets=None, show_progress: bool = False):
+        names = [n for n in model_state if self.should_compress(n, compression_targets)]
+        structure = getattr(self.config, "sparsity_structure", SparsityStructure.TWO_FOUR.value)
+        assert SparsityStructure(structure) == SparsityStructure.TWO_FOUR, "Only 2:4 sparsity is supported"
+        for n in names:
+            assert len(model_state[n].shape) == 2, "Only 2D tensors are supported"
+        compressed = dict(zip(names, sparse24_bitmask_compress_many([model_state[n] for n in names])))
+        out: Dict[str, Tensor] = {}
+        for name, value in model_state.items():
+            if name not in compressed:
+                out[name] = value
+                continue
+            values, bitmask = compressed[name]
+            tensor = Sparse24BitMaskTensor(shape=list(value.shape), compressed=values, bitmask=bitmask)
+            out.update(tensor.dict(name_prefix=name,
+                                   device="meta" if value.is_meta else self.output_device))
+        return out
+
+    def decompress_from_state_dict(self, state_dict):
+        from compressed_tensors_amd.utils.helpers import nest_state_dict
+
+        nested, ignored = nest_state_dict(state_dict, self.compression_param_names,
+                                          return_unmatched_params=True)
+        paths = list(nested)
+        dense = sparse24_bitmask_decompress_many(
+            [(nested[p]["compressed"], nested[p]["bitmask"], nested[p]["shape"]) for p in paths])
+        for path, weight in zip(paths, dense):
+            yield merge_names(path, "weight"), weight
+        for name, value in ignored.items():
+            yield name, value

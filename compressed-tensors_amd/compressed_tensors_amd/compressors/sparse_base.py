@@ -44,13 +44,14 @@ class BaseSparseCompressor(BaseCompressor):
         **kwargs,
     ) -> Generator[Tuple[str, Tensor], None, None]:
         if isinstance(path_to_model_or_tensors, dict):
-            nested, ignored = nest_state_dict(
+            _, ignored = nest_state_dict(
                 path_to_model_or_tensors, self.compression_param_names, return_unmatched_params=True
             )
-            for module_path, weight_data in nested.items():
-                yield merge_names(module_path, "weight"), self.decompress_weight(dict(weight_data))
-            for name, value in ignored.items():
-                if params_to_skip_load is not None and any(p in name for p in params_to_skip_load):
+            # through decompress_from_state_dict, which formats with a multi-tensor entry
+            # point in the C ABI override
+            for name, value in self.decompress_from_state_dict(path_to_model_or_tensors):
+                if (name in ignored and params_to_skip_load is not None
+                        and any(p in name for p in params_to_skip_load)):
                     continue
                 yield name, value
             return

@@ -75,15 +75,13 @@ static_assert(kMaxJobs == 8 && offsetof(ChainTable, chunk_end) == 0 &&
                   offsetof(ChainTable, nvec) == 32,
               "find_job reads chunk_end and nvec as the first 16 dwords of the kernel argument");
 
-// The job of workgroup `chunk`, the chunk's number within that job and the job's
-// item count.  The table must be the kernel's only argument.  Its head (chunk_end
-// and nvec) is fetched with one 64-byte scalar load written out by hand: left to
-// itself the compiler turns the search into a chain of dependent loads, and a
-// wave of these kernels lives too short to hide several scalar round trips.
-// The search itself is then compares and selects on registers, and the job's 64
-// bytes follow as one more batch of scalar loads.
-__device__ __forceinline__ ChainJob find_job(const ChainTable& t, uint32_t chunk, uint32_t* local,
-                                          uint32_t* nvec) {
+// The job of workgroup `chunk` (its index), the chunk's number within that job and the
+// job's item count, for any table that is the kernel's only argument and starts with
+// chunk_end[8] and the item counts [8].  This head is fetched with one 64-byte scalar
+// load written out by hand: left to itself the compiler turns the search into a chain of
+// dependent loads, and a wave of these kernels lives too short to hide several scalar
+// round trips.  The search itself is then compares and selects on registers.
+__device__ __forceinline__ uint32_t find_job_index(uint32_t chunk, uint32_t* local, uint32_t* nvec) {
   typedef uint32_t u32x16 __attribute__((ext_vector_type(16)));
   u32x16 head;
   asm volatile("s_load_dwordx16 %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)"
@@ -100,7 +98,13 @@ __device__ __forceinline__ ChainJob find_job(const ChainTable& t, uint32_t chunk
   }
   *local = chunk - first;
   *nvec = nv;
-  return t.job[j];
+  return j;
+}
+
+// ... and the job's 64 bytes, one more batch of scalar loads
+__device__ __forceinline__ ChainJob find_job(const ChainTable& t, uint32_t chunk, uint32_t* local,
+                                          uint32_t* nvec) {
+  return t.job[find_job_index(chunk, local, nvec)];
 }
 
 template <bool FLAT>

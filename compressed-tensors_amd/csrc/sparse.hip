@@ -10,11 +10,14 @@
 // Bit j of bitmask byte k of a row flags column 8k+j (numpy packbits,
 // bitorder="little"); the last byte of a row is zero padded.  Compacted values
 // are stored in row-major order of the set bits.
+#include <atomic>
+#include <cstddef>
 #include <mutex>
 #include <type_traits>
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "job_table.h"
 #include "qdq_core.h"
 #include "quant_fast.h"
 #include "topk24_lut.h"
@@ -830,112 +833,217 @@ bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
 // In a well-formed 2:4 bitmask every group of 4 columns keeps exactly 2, so the
 // values of group g are values[2g], values[2g+1] and no prefix sum over the
 // bitmask is needed: a lane turns E columns' worth of mask bits and E/2 values
-// into one 16-byte store.  Whether the bitmask IS well formed is only known once
-// all of it has been looked at: every lane checks its own bits and raises
-// a verdict for its workgroup otherwise, and sparse24_repair_kernel, enqueued behind
-// this one, does the general scatter (and overwrites the output) only if a verdict
-// went up.
+// into 16-byte stores.  Whether the bitmask IS well formed is only known once
+// all of it has been looked at.  Every lane checks its own bits, and a workgroup
+// that met a group which does not keep exactly 2 says so in a word of the launch.
+// sparse24_repair_kernel, enqueued behind the streaming kernel, reads that one
+// word and is done if it is zero; otherwise (a bitmask no 2:4 compressor wrote) it
+// redoes the tensors named there as a general scatter.  The second kernel has to be
+// a kernel of its own: its stores replace those of the first, and only the end of a
+// kernel puts the first kernel's stores, which may still sit in the L2 of another
+// XCD, in front of them.  (A fence per workgroup that would order them inside one
+// kernel writes that L2 back every time: measured 20 times slower.)
+//
+// The words: kS24Slots pairs {jobs with a bad group, repair workgroups done} in
+// device memory of the library, all zero between launches (a repair that found
+// something puts its pair back to zero when its last workgroup is done).  Launches
+// take the pairs in turn, so launches in flight at the same time (other streams) do
+// not share one unless there are kS24Slots of them.
+constexpr int kS24Slots = 256;
+__device__ unsigned int s24_slot_state[kS24Slots][2];
+
+static uint32_t next_s24_slot() {
+  static std::atomic<uint32_t> ticket{0};
+  return ticket.fetch_add(1, std::memory_order_relaxed) % kS24Slots;
+}
+
+// called by every thread of a streaming workgroup: `bad` goes up for job `job`
+__device__ __forceinline__ void s24_report(uint32_t slot, uint32_t job, bool bad) {
+  if (__syncthreads_or(bad) && threadIdx.x == 0) atomicOr(&s24_slot_state[slot][0], 1u << job);
+}
+
+// In the kernel behind: the set of jobs to redo (the same in every thread), 0 for
+// well-formed bitmasks.
+__device__ __forceinline__ uint32_t s24_bad_jobs(uint32_t slot) {
+  return __hip_atomic_load(&s24_slot_state[slot][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// ... and once a repair workgroup is done with them: the last one clears the pair
+__device__ __forceinline__ void s24_repair_done(uint32_t slot) {
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    unsigned int* st = s24_slot_state[slot];
+    if (atomicAdd(&st[1], 1u) == gridDim.x - 1) {
+      atomicExch(&st[0], 0u);
+      atomicExch(&st[1], 0u);
+    }
+  }
+}
+
 template <typename R>
 struct Scatter24 {
   static constexpr int E = sizeof(R) == 1 ? 16 : 8;  // columns per lane
   using MaskT = typename std::conditional<E == 16, uint16_t, uint8_t>::type;
 };
 
+// Byte selectors for v_perm_b32, 32 per element size, in LDS: entry (m, h) places the two
+// survivors of a group with mask nibble m.  One-byte elements: the group's 4 output bytes
+// from the pair (a, b) in the low (h = 0) or high (h = 1) half of a word of values.
+// Two-byte elements: output elements 2h and 2h + 1 from the word (a, b).  The first kept
+// position takes a, every later one b, a dropped one the constant zero (selector 0x0c).
+template <int ES>
+__device__ __forceinline__ uint32_t s24_selector(int idx) {
+  const uint32_t m = (uint32_t)idx & 15u, h = (uint32_t)idx >> 4;
+  uint32_t sel = 0;
+  if constexpr (ES == 1) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const bool keep = (m >> q) & 1u, second = (m & ((1u << q) - 1u)) != 0;
+      sel |= (keep ? 2u * h + (second ? 1u : 0u) : 0x0cu) << (8 * q);
+    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const uint32_t q = 2u * h + (uint32_t)e;
+      const bool keep = (m >> q) & 1u, second = (m & ((1u << q) - 1u)) != 0;
+      sel |= (keep ? (second ? 0x0302u : 0x0100u) : 0x0c0cu) << (16 * e);
+    }
+  }
+  return sel;
+}
+
+struct S24Job {
+  const void* values;
+  const uint8_t* bitmask;
+  void* out;
+  int64_t nvalues, rows, cols;
+};
+
+// kernel argument (the only one: find_job_index reads its head)
+struct S24Table {
+  uint32_t chunk_end[kMaxJobs];  // running total of workgroups, job 0 .. j (unused: 0xFFFFFFFF)
+  uint32_t n_items[kMaxJobs];
+  S24Job job[kMaxJobs];
+  uint32_t slot;
+};
+static_assert(offsetof(S24Table, chunk_end) == 0 && offsetof(S24Table, n_items) == 32, "find_job_index");
+
+// The general scatter of a whole tensor, rows dealt round-robin to the workgroups of the
+// launch; where a row's values start is the number of set bits before it, which each
+// workgroup counts by itself as it moves from one of its rows to the next (rows are whole
+// bitmask bytes here, so the rows in between are one run of bytes).
 template <typename R>
-__global__ void __launch_bounds__(kBlock)
-sparse24_scatter_kernel(const R* __restrict__ values, const uint8_t* __restrict__ bitmask,
-                        R* __restrict__ out, int64_t n_items, int* __restrict__ verdicts) {
+__device__ void s24_redo_job(const S24Job& job, int* scan_s, int64_t* red, R* stage) {
+  const R* values = static_cast<const R*>(job.values);
+  R* out = static_cast<R*>(job.out);
+  const int64_t pc = job.cols / 8;
+  const bool vec = (uintptr_t)out % (8 * sizeof(R)) == 0;
+  int64_t src = 0, counted = 0;  // set bits in rows [0, counted)
+  for (int64_t r = blockIdx.x; r < job.rows; r += gridDim.x) {
+    int64_t c = 0;
+    for (int64_t b = counted * pc + threadIdx.x; b < r * pc; b += kBlock)
+      c += __popc((uint32_t)job.bitmask[b]);
+    src += block_sum(c, red);
+    scatter_row<R>(values, job.nvalues, job.bitmask + r * pc, src, out + r * job.cols, job.cols, pc,
+                   vec, 0xffu, scan_s, stage);
+    counted = r + 1;
+  }
+}
+
+template <typename R>
+__global__ void __launch_bounds__(kBlock) sparse24_scatter_kernel(S24Table t) {
   constexpr int E = Scatter24<R>::E, U = kS24ScatterU;
+  constexpr int VE = 16 / (int)sizeof(R);  // elements per 16-byte access
   using MaskT = typename Scatter24<R>::MaskT;
-  const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
+  constexpr uint32_t kAll = E == 16 ? 0xFFFFu : 0xFFu;
+  __shared__ uint32_t lut[32];
+  if constexpr (sizeof(R) < 4) {
+    if (threadIdx.x < 32) lut[threadIdx.x] = s24_selector<(int)sizeof(R)>((int)threadIdx.x);
+    __syncthreads();
+  }
+  uint32_t local, n_items;
+  const uint32_t j = find_job_index(blockIdx.x, &local, &n_items);
+  const S24Job job = t.job[j];
+  const R* __restrict__ values = static_cast<const R*>(job.values);
+  R* __restrict__ out = static_cast<R*>(job.out);
+  const uint32_t i0 = local * (kBlock * U) + threadIdx.x;
   MaskT m[U];
   Vec<R, E / 2> v[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     // past the end: re-read the last item (not stored)
-    int64_t i = i0 + k * kBlock;
+    uint32_t i = i0 + k * kBlock;
     if (i >= n_items) i = n_items - 1;
-    m[k] = reinterpret_cast<const MaskT*>(bitmask)[i];
-    v[k] = ldg<R, E / 2>(values + i * (E / 2));
+    m[k] = reinterpret_cast<const MaskT*>(job.bitmask)[i];
+    if constexpr (sizeof(R) * (E / 2) <= 16) {
+      v[k] = ldg<R, E / 2>(values + (int64_t)i * (E / 2));
+    } else {
+#pragma unroll
+      for (int h = 0; h < E / 2 / VE; ++h) {
+        const Vec<R, VE> part = ldg<R, VE>(values + (int64_t)i * (E / 2) + h * VE);
+#pragma unroll
+        for (int e = 0; e < VE; ++e) v[k].v[h * VE + e] = part.v[e];
+      }
+    }
   }
   bool bad = false;
 #pragma unroll
   for (int k = 0; k < U; ++k) {
-    const int64_t i = i0 + k * kBlock;
+    const uint32_t i = i0 + k * kBlock;
     const uint32_t bits = m[k];
-    uint32_t n = bits - ((bits >> 1) & 0x5555u);
-    n = (n & 0x3333u) + ((n >> 2) & 0x3333u);  // set bits per group of 4
-    bad |= i < n_items && n != (E == 16 ? 0x2222u : 0x22u);
+    uint32_t n = bits - ((bits >> 1) & 0x55555555u);
+    n = (n & 0x33333333u) + ((n >> 2) & 0x33333333u);  // set bits per group of 4
+    bad |= i < n_items && n != (0x22222222u & kAll);
     Vec<R, E> o;
+    if constexpr (sizeof(R) == 4) {
 #pragma unroll
-    for (int g = 0; g < E / 4; ++g) {
-      const uint32_t gm = (bits >> (4 * g)) & 15u;
-      const R a = v[k].v[2 * g], b = v[k].v[2 * g + 1];
+      for (int g = 0; g < E / 4; ++g) {
+        const uint32_t gm = (bits >> (4 * g)) & 15u;
+        const R a = v[k].v[2 * g], b = v[k].v[2 * g + 1];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const bool keep = (gm >> j) & 1u, second = (gm & ((1u << j) - 1u)) != 0;
-        o.v[4 * g + j] = keep ? (second ? b : a) : (R)0;
+        for (int q = 0; q < 4; ++q) {
+          const bool keep = (gm >> q) & 1u, second = (gm & ((1u << q) - 1u)) != 0;
+          o.v[4 * g + q] = keep ? (second ? b : a) : (R)0;
+        }
       }
+    } else {
+      // 16 bytes out of 8: one v_perm_b32 per output word
+      const Vec<uint32_t, 2> vw = __builtin_bit_cast(Vec<uint32_t, 2>, v[k]);
+      Vec<uint32_t, 4> ow;
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        // one-byte elements: word w is group w, its pair in half (w & 1) of values word w / 2;
+        // two-byte elements: word w is half (w & 1) of group w / 2, whose pair is values word w / 2
+        const uint32_t gm = (bits >> (sizeof(R) == 1 ? 4 * w : 4 * (w / 2))) & 15u;
+        ow.v[w] = __builtin_amdgcn_perm(0u, vw.v[w / 2], lut[gm + 16 * (w & 1)]);
+      }
+      o = __builtin_bit_cast(Vec<R, E>, ow);
     }
     if (i < n_items) {
-      if constexpr (sizeof(R) * E == 16) {
-        stg_nt<R, E>(out + i * E, o);
-      } else {  // 4-byte elements: two 16-byte halves
-        Vec<R, 4> lo, hi;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) { lo.v[j] = o.v[j]; hi.v[j] = o.v[4 + j]; }
-        stg<R, 4>(out + i * E, lo);
-        stg<R, 4>(out + i * E + 4, hi);
+      for (int h = 0; h < E / VE; ++h) {
+        Vec<R, VE> part;
+#pragma unroll
+        for (int e = 0; e < VE; ++e) part.v[e] = o.v[h * VE + e];
+        stg_nt<R, VE>(out + (int64_t)i * E + h * VE, part);
       }
     }
   }
-  // every workgroup leaves its verdict, good or bad: nothing has to be cleared beforehand
-  const int any_bad = __syncthreads_or(bad);
-  if (threadIdx.x == 0) verdicts[blockIdx.x] = any_bad ? 1 : 0;
+  s24_report(t.slot, j, bad);
 }
 
-// Did any streaming workgroup meet a bitmask that is not 2:4?  The same answer in every
-// thread of the workgroup.  `verdicts` is 16-byte aligned.
-__device__ __forceinline__ bool any_bad_verdict(const int* __restrict__ verdicts,
-                                                int64_t n_verdicts) {
-  uint32_t bad = 0;
-  const int64_t quads = n_verdicts / 4;  // 16 bytes per load
-  const u32x4_t* v4 = reinterpret_cast<const u32x4_t*>(verdicts);
-  for (int64_t i = threadIdx.x; i < quads; i += kBlock) {
-    const u32x4_t q = v4[i];
-    bad |= q.x | q.y | q.z | q.w;
-  }
-  for (int64_t i = quads * 4 + threadIdx.x; i < n_verdicts; i += kBlock) bad |= (uint32_t)verdicts[i];
-  return __syncthreads_or((int)bad) != 0;
-}
+constexpr int kS24RepairGrid = 32;
 
-// What follows the streaming pass: every workgroup looks at all the verdicts (a few
-// KB, from L2) and is done if none is up.  Otherwise the bitmask is not 2:4 and the
-// workgroups redo the tensor as a general scatter, rows dealt round-robin; where a
-// row's values start is the number of set bits before it, which each workgroup
-// counts by itself as it moves from one of its rows to the next (rows are whole
-// bitmask bytes here, so the rows in between are one run of bytes).  Slow next to
-// the streaming pass, but it only runs for a bitmask that no 2:4 compressor wrote.
 template <typename R>
-__global__ void __launch_bounds__(kBlock)
-sparse24_repair_kernel(const R* __restrict__ values, int64_t nvalues,
-                       const uint8_t* __restrict__ bitmask, R* __restrict__ out, int64_t rows,
-                       int64_t cols, int64_t pc, const int* __restrict__ verdicts,
-                       int64_t n_verdicts) {
+__global__ void __launch_bounds__(kBlock) sparse24_repair_kernel(S24Table t) {
+  const uint32_t todo = s24_bad_jobs(t.slot);
+  if (todo == 0) return;
   __shared__ int scan_s[kWaves];
   __shared__ int64_t red[kWaves];
   __shared__ R stage[kBlock * 8];
-  if (!any_bad_verdict(verdicts, n_verdicts)) return;
-  const bool vec = (uintptr_t)out % (8 * sizeof(R)) == 0;
-  int64_t src = 0, counted = 0;  // set bits in rows [0, counted)
-  for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
-    int64_t c = 0;
-    for (int64_t b = counted * pc + threadIdx.x; b < r * pc; b += kBlock) c += __popc((uint32_t)bitmask[b]);
-    src += block_sum(c, red);
-    scatter_row<R>(values, nvalues, bitmask + r * pc, src, out + r * cols, cols, pc, vec, 0xffu, scan_s,
-                   stage);
-    counted = r + 1;
-  }
+  for (int q = 0; q < kMaxJobs; ++q)
+    if ((todo >> q) & 1u) s24_redo_job<R>(t.job[q], scan_s, red, stage);
+  s24_repair_done(t.slot);
 }
 
 // 2:4 decompression of int8 / fp8 codes and their dequantization in one pass: what
@@ -971,9 +1079,12 @@ sparse24_scatter_dequant_kernel(const uint8_t* __restrict__ values,
                                 const uint8_t* __restrict__ bitmask,
                                 const typename FT::raw* __restrict__ scale,
                                 const uint8_t* __restrict__ zp, typename FT::raw* __restrict__ out,
-                                int64_t n_items, VecGeom g, int* __restrict__ verdicts) {
+                                int64_t n_items, VecGeom g, uint32_t slot) {
   using FR = typename FT::raw;
   constexpr int U = kS24DqU;
+  __shared__ uint32_t lut[32];
+  if (threadIdx.x < 32) lut[threadIdx.x] = s24_selector<1>((int)threadIdx.x);
+  __syncthreads();
   const int64_t i0 = (int64_t)blockIdx.x * (kBlock * U) + threadIdx.x;
   uint8_t m[U], zraw[U];
   uint32_t v[U];
@@ -997,22 +1108,15 @@ sparse24_scatter_dequant_kernel(const uint8_t* __restrict__ values,
     uint32_t n = bits - ((bits >> 1) & 0x55u);
     n = (n & 0x33u) + ((n >> 2) & 0x33u);  // set bits per group of 4
     bad |= i < n_items && n != 0x22u;
-    Vec<uint8_t, 8> codes;
+    Vec<uint32_t, 2> cw;  // 8 codes out of 4: one v_perm_b32 per group
 #pragma unroll
-    for (int q = 0; q < 2; ++q) {
-      const uint32_t gm = (bits >> (4 * q)) & 15u;
-      const uint8_t a = (uint8_t)(v[k] >> (16 * q)), b = (uint8_t)(v[k] >> (16 * q + 8));
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const bool keep = (gm >> j) & 1u, second = (gm & ((1u << j) - 1u)) != 0;
-        codes.v[4 * q + j] = keep ? (second ? b : a) : (uint8_t)0;
-      }
-    }
+    for (int q = 0; q < 2; ++q)
+      cw.v[q] = __builtin_amdgcn_perm(0u, v[k], lut[((bits >> (4 * q)) & 15u) + 16 * q]);
+    const Vec<uint8_t, 8> codes = __builtin_bit_cast(Vec<uint8_t, 8>, cw);
     const Vec<FR, 8> o = dequant_codes8<FT, QK, HAS_ZP>(codes, sraw[k], zraw[k]);
     if (i < n_items) stg_nt<FR, 8>(out + i * 8, o);
   }
-  const int any_bad = __syncthreads_or(bad);
-  if (threadIdx.x == 0) verdicts[blockIdx.x] = any_bad ? 1 : 0;
+  s24_report(slot, 0, bad);
 }
 
 // ... and what sparse24_repair_kernel is to sparse24_scatter_kernel: nothing for a 2:4
@@ -1023,13 +1127,12 @@ sparse24_repair_dequant_kernel(const uint8_t* __restrict__ values, int64_t nvalu
                                const uint8_t* __restrict__ bitmask,
                                const typename FT::raw* __restrict__ scale,
                                const uint8_t* __restrict__ zp, typename FT::raw* __restrict__ out,
-                               int64_t rows, int64_t pc, VecGeom g,
-                               const int* __restrict__ verdicts, int64_t n_verdicts) {
+                               int64_t rows, int64_t pc, VecGeom g, uint32_t slot) {
   using FR = typename FT::raw;
+  if (s24_bad_jobs(slot) == 0) return;
   __shared__ int scan_s[kWaves];
   __shared__ int64_t red[kWaves];
   __shared__ uint8_t stage[kBlock * 8];
-  if (!any_bad_verdict(verdicts, n_verdicts)) return;
   int64_t src = 0, counted = 0;  // set bits in rows [0, counted)
   for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
     int64_t c = 0;
@@ -1046,6 +1149,7 @@ sparse24_repair_dequant_kernel(const uint8_t* __restrict__ values, int64_t nvalu
                             });
     counted = r + 1;
   }
+  s24_repair_done(slot);
 }
 
 // ------------------------------------------------------------------ 2:4 selection
@@ -1270,6 +1374,39 @@ sparse24_compress_kernel(const R* __restrict__ x, R* __restrict__ values,
   }
 }
 
+// the same for up to kMaxJobs tensors of one dtype
+struct S24CompressJob {
+  const void* x;
+  void* values;
+  uint8_t* bitmask;
+};
+struct S24CompressTable {  // the kernel's only argument: find_job_index reads its head
+  uint32_t chunk_end[kMaxJobs];
+  uint32_t n_items[kMaxJobs];
+  S24CompressJob job[kMaxJobs];
+};
+static_assert(offsetof(S24CompressTable, n_items) == 32, "find_job_index");
+
+template <typename R, int DT, int N>
+__global__ void __launch_bounds__(kBlock) sparse24_compress_chain_kernel(S24CompressTable t) {
+  constexpr int U = kS24U;
+  uint32_t local, nitems;
+  const S24CompressJob job = t.job[find_job_index(blockIdx.x, &local, &nitems)];
+  const R* __restrict__ x = static_cast<const R*>(job.x);
+  const int64_t i0 = (int64_t)local * (kBlock * U) + threadIdx.x;
+  Vec<R, N> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    a[k] = ldg<R, N>(x + (i < nitems ? i : nitems - 1) * N);  // past the end: re-read, not stored
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t i = i0 + k * kBlock;
+    store_survivors24<R, DT, N>(a[k], static_cast<R*>(job.values), job.bitmask, i, i < nitems);
+  }
+}
+
 // Quantization to fp8 / int8 codes and 2:4 compression of the codes in one pass: what
 // ModelCompressor.compress does to a weight that is both quantized (float- / int- /
 // naive-quantized, naive_quantized.py:79-114) and 2:4 sparse (sparse_24_bitmask.py:
@@ -1413,13 +1550,10 @@ extern "C" int64_t ctmi_bitmask_tmp_bytes(int64_t rows, int64_t cols) {
   return 16 * r + 16 * cdiv(r * c, kTileElems) + 32;
 }
 
-// one verdict per streaming workgroup, or what the general kernels need
+// what the general kernels need (the 2:4 streaming kernel needs none)
 extern "C" int64_t ctmi_sparse24_tmp_bytes(int64_t rows, int64_t cols, int32_t elem_size) {
-  const int64_t r = rows < 1 ? 1 : rows, c = cols < 1 ? 1 : cols;
-  const int64_t items = cdiv(r * c, elem_size == 1 ? 16 : 8);
-  const int64_t verdicts = 4 * cdiv(items, kBlock * kS24ScatterU) + 8;
-  const int64_t general = ctmi_bitmask_tmp_bytes(rows, cols);
-  return verdicts > general ? verdicts : general;
+  (void)elem_size;
+  return ctmi_bitmask_tmp_bytes(rows, cols);
 }
 
 static int check_elem(int32_t elem_size) {
@@ -1501,6 +1635,44 @@ static int scatter_check(const void* values, int64_t nvalues, int32_t elem_size,
   return CTMI_OK;
 }
 
+// what sparse24_scatter_kernel needs of a tensor: half as many values as elements, rows of
+// whole bitmask bytes, whole work items, aligned accesses
+static bool s24_streamable(const void* values, int64_t nvalues, int32_t elem_size,
+                           const uint8_t* bitmask, const void* out, int64_t rows, int64_t cols) {
+  const int64_t numel = rows * cols;
+  const int e24 = elem_size == 1 ? 16 : 8;
+  return nvalues * 2 == numel && cols % 8 == 0 && numel % e24 == 0 && (uintptr_t)out % 16 == 0 &&
+         (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % (e24 / 8) == 0 &&
+         numel / e24 < (1ll << 31);
+}
+
+// up to kMaxJobs streamable tensors of one element size in one launch
+static void s24_launch(const S24Job* jobs, int n, int32_t elem_size, hipStream_t st) {
+  S24Table t;
+  const int e24 = elem_size == 1 ? 16 : 8;
+  uint32_t total = 0;
+  for (int k = 0; k < kMaxJobs; ++k) {
+    if (k < n) {
+      t.job[k] = jobs[k];
+      t.n_items[k] = (uint32_t)(jobs[k].rows * jobs[k].cols / e24);
+      total += (uint32_t)cdiv((int64_t)t.n_items[k], kBlock * kS24ScatterU);
+      t.chunk_end[k] = total;
+    } else {
+      t.job[k] = S24Job{nullptr, nullptr, nullptr, 0, 0, 0};
+      t.n_items[k] = 0;
+      t.chunk_end[k] = 0xFFFFFFFFu;
+    }
+  }
+  t.slot = next_s24_slot();
+#define CTMI_24(R)                                                                \
+  hipLaunchKernelGGL(sparse24_scatter_kernel<R>, total, kBlock, 0, st, t);        \
+  hipLaunchKernelGGL(sparse24_repair_kernel<R>, kS24RepairGrid, kBlock, 0, st, t)
+  if (elem_size == 1) { CTMI_24(uint8_t); }
+  else if (elem_size == 2) { CTMI_24(uint16_t); }
+  else { CTMI_24(uint32_t); }
+#undef CTMI_24
+}
+
 static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
                          const uint8_t* bitmask, const int64_t* row_offsets, void* out, void* tmp,
                          int64_t rows, int64_t cols, void* stream, bool try_24, const char* what) {
@@ -1512,25 +1684,10 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
   const int64_t pc = cdiv(cols, 8);
   const int64_t numel = rows * cols;
   // exactly half as many values as elements, rows of whole bitmask bytes: the 2:4
-  // streaming kernel, and behind it the kernel that redoes the work if the bitmask
-  // turns out not to be 2:4 (see sparse24_scatter_kernel)
-  const int e24 = elem_size == 1 ? 16 : 8;
-  if (try_24 && tmp && nvalues * 2 == numel && cols % 8 == 0 && numel % e24 == 0 &&
-      (uintptr_t)out % 16 == 0 && (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 2 == 0 &&
-      (uintptr_t)tmp % 16 == 0 && numel / e24 < (1ll << 40)) {
-    int* verdicts = (int*)tmp;
-    const int64_t n_items = numel / e24;
-    const unsigned g24 = (unsigned)cdiv(n_items, kBlock * kS24ScatterU);
-    const unsigned repair_grid = (unsigned)(rows < 32 ? rows : 32);
-#define CTMI_24(R)                                                                               \
-  hipLaunchKernelGGL(sparse24_scatter_kernel<R>, g24, kBlock, 0, st, (const R*)values, bitmask,  \
-                     (R*)out, n_items, verdicts);                                                \
-  hipLaunchKernelGGL(sparse24_repair_kernel<R>, repair_grid, kBlock, 0, st, (const R*)values,    \
-                     nvalues, bitmask, (R*)out, rows, cols, pc, verdicts, (int64_t)g24)
-    if (elem_size == 1) { CTMI_24(uint8_t); }
-    else if (elem_size == 2) { CTMI_24(uint16_t); }
-    else { CTMI_24(uint32_t); }
-#undef CTMI_24
+  // streaming kernel (which also copes with a bitmask that turns out not to be 2:4)
+  if (try_24 && s24_streamable(values, nvalues, elem_size, bitmask, out, rows, cols)) {
+    S24Job job{values, bitmask, out, nvalues, rows, cols};
+    s24_launch(&job, 1, elem_size, st);
     return check_launch(what);
   }
   if (tmp && cols % 8 == 0 && numel % 16 == 0 && (uintptr_t)out % 16 == 0 &&
@@ -1767,6 +1924,99 @@ extern "C" int ctmi_sparse24_compress(const void* x, int32_t x_dtype, void* valu
   return check_launch("ctmi_sparse24_compress");
 }
 
+extern "C" int ctmi_sparse24_compress_many(const ctmi_sparse24_job* jobs, int64_t n_jobs,
+                                           int32_t x_dtype, void* stream) {
+  CTMI_REQUIRE(n_jobs >= 0 && (jobs || n_jobs == 0), CTMI_ERR_VALUE, "bad job list");
+  int rc = check_24_dtype(x_dtype);
+  if (rc) return rc;
+  const int es = dtype_size(x_dtype);
+  const int per = es == 1 ? 16 : 8;  // elements per work item
+  // everything is checked before anything is enqueued
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_sparse24_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 0 && j.cols >= 0, CTMI_ERR_VALUE, "job %lld: negative shape", (long long)i);
+    if (j.rows == 0 || j.cols == 0) continue;
+    CTMI_REQUIRE(j.dense && j.values && j.bitmask, CTMI_ERR_VALUE, "job %lld: NULL tensor pointer",
+                 (long long)i);
+    const int64_t n = j.rows * j.cols;
+    CTMI_REQUIRE(j.cols % 8 == 0 && n % per == 0 && (uintptr_t)j.dense % (per * es) == 0 &&
+                     (uintptr_t)j.values % (per * es / 2) == 0 && n / per < (1ll << 31),
+                 CTMI_ERR_UNSUPPORTED,
+                 "job %lld: the multi-tensor call takes rows of whole bitmask bytes and aligned "
+                 "tensors; use ctmi_sparse24_compress for this one", (long long)i);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  S24CompressTable t;
+  int filled = 0;
+  uint32_t total = 0;
+  bool any = false;
+  auto flush = [&]() {
+    for (int k = filled; k < kMaxJobs; ++k) {
+      t.chunk_end[k] = 0xFFFFFFFFu;
+      t.n_items[k] = 0;
+      t.job[k] = S24CompressJob{nullptr, nullptr, nullptr};
+    }
+    if (es == 1)
+      hipLaunchKernelGGL((sparse24_compress_chain_kernel<uint8_t, CTMI_I8, 16>), total, kBlock, 0, st, t);
+    else if (x_dtype == CTMI_BF16)
+      hipLaunchKernelGGL((sparse24_compress_chain_kernel<uint16_t, CTMI_BF16, 8>), total, kBlock, 0, st, t);
+    else if (es == 2)
+      hipLaunchKernelGGL((sparse24_compress_chain_kernel<uint16_t, CTMI_F16, 8>), total, kBlock, 0, st, t);
+    else
+      hipLaunchKernelGGL((sparse24_compress_chain_kernel<uint32_t, CTMI_F32, 8>), total, kBlock, 0, st, t);
+    filled = 0;
+    total = 0;
+  };
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_sparse24_job& j = jobs[i];
+    if (j.rows == 0 || j.cols == 0) continue;
+    any = true;
+    t.job[filled] = S24CompressJob{j.dense, j.values, j.bitmask};
+    t.n_items[filled] = (uint32_t)(j.rows * j.cols / per);
+    total += (uint32_t)cdiv((int64_t)t.n_items[filled], kBlock * kS24U);
+    t.chunk_end[filled] = total;
+    if (++filled == kMaxJobs) flush();
+  }
+  if (!any) return CTMI_OK;
+  if (filled) flush();
+  return check_launch("ctmi_sparse24_compress_many");
+}
+
+extern "C" int ctmi_sparse24_decompress_many(const ctmi_sparse24_job* jobs, int64_t n_jobs,
+                                             int32_t elem_size, void* stream) {
+  CTMI_REQUIRE(n_jobs >= 0 && (jobs || n_jobs == 0), CTMI_ERR_VALUE, "bad job list");
+  int rc = check_elem(elem_size);
+  if (rc) return rc;
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_sparse24_job& j = jobs[i];
+    rc = scatter_check(j.values, j.nvalues, elem_size, j.bitmask, j.dense, j.rows, j.cols);
+    if (rc) return rc;
+    if (j.rows == 0 || j.cols == 0) continue;
+    CTMI_REQUIRE(s24_streamable(j.values, j.nvalues, elem_size, j.bitmask, j.dense, j.rows, j.cols),
+                 CTMI_ERR_UNSUPPORTED,
+                 "job %lld: the multi-tensor call takes tensors with rows * cols / 2 values, rows "
+                 "of whole bitmask bytes and aligned buffers; use ctmi_sparse24_decompress for "
+                 "this one", (long long)i);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  S24Job batch[kMaxJobs];
+  int filled = 0;
+  bool any = false;
+  for (int64_t i = 0; i < n_jobs; ++i) {
+    const ctmi_sparse24_job& j = jobs[i];
+    if (j.rows == 0 || j.cols == 0) continue;
+    any = true;
+    batch[filled] = S24Job{j.values, j.bitmask, j.dense, j.nvalues, j.rows, j.cols};
+    if (++filled == kMaxJobs) {
+      s24_launch(batch, filled, elem_size, st);
+      filled = 0;
+    }
+  }
+  if (!any) return CTMI_OK;
+  if (filled) s24_launch(batch, filled, elem_size, st);
+  return check_launch("ctmi_sparse24_decompress_many");
+}
+
 extern "C" int ctmi_quantize_sparse24_compress_supported(int32_t x_dtype, int64_t rows, int64_t cols,
                                                          const ctmi_qparams* qp) {
   if (!qp || rows < 1 || cols < 1 || cols % 8) return 0;
@@ -1838,8 +2088,9 @@ extern "C" int ctmi_sparse24_decompress_dequantize_supported(int32_t values_dtyp
 }
 
 extern "C" int64_t ctmi_sparse24_dequantize_tmp_bytes(int64_t rows, int64_t cols) {
-  const int64_t r = rows < 1 ? 1 : rows, c = cols < 1 ? 1 : cols;
-  return 4 * cdiv(cdiv(r * c, 8), kBlock * kS24DqU) + 16;
+  (void)rows;
+  (void)cols;
+  return 0;  // the verdicts of the streaming workgroups live in the library's own counters
 }
 
 extern "C" int ctmi_sparse24_decompress_dequantize(const void* values, int64_t nvalues,
@@ -1855,29 +2106,27 @@ extern "C" int ctmi_sparse24_decompress_dequantize(const void* values, int64_t n
   CTMI_REQUIRE(ctmi_sparse24_decompress_dequantize_supported(values_dtype, out_dtype, rows, cols, qp),
                CTMI_ERR_UNSUPPORTED,
                "no fused kernel for this layout: decompress the codes, then dequantize");
-  CTMI_REQUIRE(values && bitmask && out && tmp, CTMI_ERR_VALUE, "NULL tensor pointer");
+  (void)tmp;  // no scratch is used any more; the argument stays for callers built against it
+  CTMI_REQUIRE(values && bitmask && out, CTMI_ERR_VALUE, "NULL tensor pointer");
   CTMI_REQUIRE(nvalues * 2 == rows * cols, CTMI_ERR_VALUE,
                "a 2:4 tensor of %lld x %lld elements has %lld values, got %lld", (long long)rows,
                (long long)cols, (long long)(rows * cols / 2), (long long)nvalues);
-  CTMI_REQUIRE((uintptr_t)out % (8 * dtype_size(out_dtype)) == 0 && (uintptr_t)values % 4 == 0 &&
-                   (uintptr_t)tmp % 16 == 0,
-               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements, tmp to 16 bytes");
+  CTMI_REQUIRE((uintptr_t)out % (8 * dtype_size(out_dtype)) == 0 && (uintptr_t)values % 4 == 0,
+               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
   VecGeom g;
   vec_geometry(qp, rows, cols, &g);
   const int64_t items = rows * cols / 8;
-  const int64_t pc = cols / 8;
   const unsigned grid = (unsigned)cdiv(items, kBlock * kS24DqU);
-  const unsigned repair_grid = (unsigned)(rows < 32 ? rows : 32);
-  int* verdicts = (int*)tmp;
   hipStream_t st = (hipStream_t)stream;
   const uint8_t* zp = (const uint8_t*)qp->zero_point;
+  const uint32_t slot = next_s24_slot();
 #define CTMI_S24DQ_K(FT, RAW, QK, HZ)                                                             \
   hipLaunchKernelGGL((sparse24_scatter_dequant_kernel<FT, QK, HZ>), grid, kBlock, 0, st,          \
                      (const uint8_t*)values, bitmask, (const RAW*)qp->scale, zp, (RAW*)out, items, \
-                     g, verdicts);                                                                 \
-  hipLaunchKernelGGL((sparse24_repair_dequant_kernel<FT, QK, HZ>), repair_grid, kBlock, 0, st,    \
+                     g, slot);                                                                     \
+  hipLaunchKernelGGL((sparse24_repair_dequant_kernel<FT, QK, HZ>), kS24RepairGrid, kBlock, 0, st, \
                      (const uint8_t*)values, nvalues, bitmask, (const RAW*)qp->scale, zp,          \
-                     (RAW*)out, rows, pc, g, verdicts, (int64_t)grid)
+                     (RAW*)out, rows, cols / 8, g, slot)
 #define CTMI_S24DQ(FT, RAW)                                                          \
   if (values_dtype == CTMI_I8) {                                                     \
     if (zp) { CTMI_S24DQ_K(FT, RAW, 0, true); } else { CTMI_S24DQ_K(FT, RAW, 0, false); } \

@@ -241,14 +241,37 @@ int ctmi_bitmask_decompress_static(const void* values, int64_t nvalues, int32_t 
 /* A22.  sparse24_bitmask_decompress (sparse_24_bitmask.py:206-224): the same
  * scatter, `out[mask] = values`, for any bitmask.  A bitmask that keeps exactly 2
  * of every 4 columns (what the format holds) needs no prefix sums and is
- * expanded in one streaming pass; the general path of ctmi_bitmask_decompress is
- * enqueued behind it and does its work only if some group turned out not to
- * keep exactly 2.  tmp: ctmi_sparse24_tmp_bytes(rows, cols, elem_size) bytes of
- * device scratch; it needs no initialisation. */
+ * expanded in one streaming pass.  Every workgroup checks the groups it
+ * expands; a small kernel enqueued behind reads one word and, only if some group
+ * did not keep exactly 2 (a bitmask no 2:4 compressor wrote), redoes the tensor
+ * as a general scatter.  Other shapes (values that are not half the elements,
+ * rows that are not whole bitmask bytes) take the path of ctmi_bitmask_decompress
+ * and use tmp: ctmi_sparse24_tmp_bytes(rows, cols, elem_size) bytes of device
+ * scratch; it needs no initialisation. */
 int64_t ctmi_sparse24_tmp_bytes(int64_t rows, int64_t cols, int32_t elem_size);
 int ctmi_sparse24_decompress(const void* values, int64_t nvalues, int32_t elem_size,
                              const uint8_t* bitmask, void* out, void* tmp, int64_t rows,
                              int64_t cols, void* stream);
+
+/* ctmi_sparse24_compress / ctmi_sparse24_decompress for several tensors of one dtype
+ * from one call, 8 per launch.  Every tensor must have rows of whole bitmask bytes
+ * (cols % 8 == 0), a whole number of work items (rows * cols a multiple of 16 for
+ * 1-byte elements, of 8 otherwise) and 16-byte aligned
+ * buffers; for decompression also nvalues * 2 == rows * cols.  A job that does not
+ * is refused with CTMI_ERR_UNSUPPORTED before anything is enqueued: give it a call
+ * of its own.  `dense` is read by compress_many and written by decompress_many;
+ * nvalues is ignored by compress_many. */
+typedef struct ctmi_sparse24_job {
+  void* dense;      /* [rows, cols] */
+  void* values;     /* [rows, cols / 2] */
+  uint8_t* bitmask; /* [rows, cols / 8] */
+  int64_t nvalues;
+  int64_t rows, cols;
+} ctmi_sparse24_job;
+int ctmi_sparse24_compress_many(const ctmi_sparse24_job* jobs, int64_t n_jobs, int32_t x_dtype,
+                                void* stream);
+int ctmi_sparse24_decompress_many(const ctmi_sparse24_job* jobs, int64_t n_jobs,
+                                  int32_t elem_size, void* stream);
 
 /* A20.  get_24_bytemasks (sparse_24_bitmask.py:227-260): top-2-of-4 by
  * |value| with torch.topk's tie order.  x_dtype: a float type (ranked on the
@@ -287,8 +310,9 @@ int ctmi_quantize_sparse24_compress(const void* x, int32_t x_dtype, void* values
  * (set bits are then filled from `values` in order, as in ctmi_bitmask_decompress).
  * The codes are decoded by values_dtype (CTMI_I8 or CTMI_F8E4M3), whatever qp's type
  * says: dequantize() infers its arguments from the scale's shape alone.
- * _supported(): as for ctmi_quantize_sparse24_compress.  tmp:
- * ctmi_sparse24_dequantize_tmp_bytes() bytes of device scratch, 16-byte aligned. */
+ * _supported(): as for ctmi_quantize_sparse24_compress.  tmp is no longer used (what the
+ * check for a bitmask that is not 2:4 needs lives inside the library, as for
+ * ctmi_sparse24_decompress) and may be NULL; ctmi_sparse24_dequantize_tmp_bytes() is 0. */
 int ctmi_sparse24_decompress_dequantize_supported(int32_t values_dtype, int32_t out_dtype,
                                                   int64_t rows, int64_t cols,
                                                   const ctmi_qparams* qp);

@@ -155,11 +155,24 @@ def test_one_pass_and_many_argument_errors(ctmi):
     assert ok(_lib.I8, _lib.BF16, 4, 64, ctypes.byref(qp)) == 1
     assert ok(_lib.BF16, _lib.BF16, 4, 64, ctypes.byref(qp)) == 0
     assert ok(_lib.I8, _lib.F32, 4, 64, ctypes.byref(qp)) == 0   # scales are bf16
-    assert ctmi.ctmi_sparse24_dequantize_tmp_bytes(14336, 4096) > ctmi.ctmi_sparse24_dequantize_tmp_bytes(8, 8) > 0
+    assert ctmi.ctmi_sparse24_dequantize_tmp_bytes(14336, 4096) == 0  # the check needs no caller scratch
+    # several 2:4 tensors per call: shapes the streaming kernels do not take are refused up front
+    sj = (_lib.Sparse24Job * 2)()
+    for j, (rows, cols) in zip(sj, ((4, 64), (4, 12))):
+        j.dense, j.values, j.bitmask, j.nvalues, j.rows, j.cols = 0x1000, 0x2000, 0x3000, rows * cols // 2, rows, cols
+    rc = ctmi.ctmi_sparse24_compress_many(sj, 2, _lib.BF16, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "job 1" in _err(ctmi)
+    rc = ctmi.ctmi_sparse24_decompress_many(sj, 2, 2, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "job 1" in _err(ctmi)
+    sj[0].nvalues = 5
+    rc = ctmi.ctmi_sparse24_decompress_many(sj, 1, 2, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "job 0" in _err(ctmi)
+    assert ctmi.ctmi_sparse24_compress_many(sj, 0, _lib.BF16, None) == 0
+    assert ctmi.ctmi_sparse24_compress_many(sj, 1, _lib.I32, None) != 0
     rc = ctmi.ctmi_sparse24_decompress_dequantize(0x1000, 100, _lib.I8, 0x2000, 0x3000, _lib.BF16, 0x4000,
                                                   4, 64, ctypes.byref(qp), None)
     assert rc == _lib.CTMI_ERR_VALUE and "128 values" in _err(ctmi)
-    rc = ctmi.ctmi_sparse24_decompress_dequantize(0x1000, 128, _lib.I8, 0x2000, 0x3000, _lib.BF16, None,
+    rc = ctmi.ctmi_sparse24_decompress_dequantize(0x1000, 128, _lib.I8, 0x2000, None, _lib.BF16, None,
                                                   4, 64, ctypes.byref(qp), None)
     assert rc == _lib.CTMI_ERR_VALUE and "NULL tensor pointer" in _err(ctmi)
     rc = ctmi.ctmi_sparse24_decompress_dequantize(0x1000, 128, _lib.I16, 0x2000, 0x3000, _lib.BF16, 0x4000,

@@ -535,3 +535,98 @@ def test_stacked_round_trip_at_full_size(gpu):
     again = quantize_sparse24_compress(back, scale, args)
     assert_bit_equal(again[1], bitmask, "bitmask of the round trip")
     assert_bit_equal(again[0], values, "values of the round trip")
+
+
+# ---------------------------------------------------------------- several 2:4 tensors per call
+
+
+def _prune24(x):
+    """zero the two smallest magnitudes of every group of 4 (ties do not matter here)"""
+    g = x.float().abs().reshape(-1, 4)
+    keep = torch.zeros_like(g, dtype=torch.bool)
+    keep.scatter_(1, g.topk(2, dim=1).indices, True)
+    return torch.where(keep.reshape(x.shape), x, torch.zeros_like(x))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float8_e4m3fn, torch.float32, torch.float16])
+def test_sparse24_many_tensors_in_one_call(dtype, gpu):
+    """sparse24_bitmask_compress_many / _decompress_many == the single-tensor calls, bit for
+    bit, and the oracle: more tensors than one launch takes (8), sizes that differ, a shape
+    the chained kernels do not take (it gets a call of its own), and among the tensors to
+    decompress one whose bitmask is not 2:4 (the last workgroup of the launch redoes it)"""
+    from compressed_tensors_amd.compressors import (
+        sparse24_bitmask_compress, sparse24_bitmask_compress_many, sparse24_bitmask_decompress,
+        sparse24_bitmask_decompress_many,
+    )
+    from compressed_tensors_amd.utils.helpers import pack_bitmasks
+
+    announce("sparse24 many", dtype)
+    g = torch.Generator().manual_seed(31)
+    shapes = [(64, 512), (37, 256), (16, 128), (5, 1024), (128, 256), (1, 64), (48, 384), (3, 12), (96, 640),
+              (7, 256), (300, 4096)]
+    xs = [torch.randn(s, generator=g).clamp(-3, 3).to(dtype) for s in shapes]
+    got = sparse24_bitmask_compress_many([x.to(gpu) for x in xs])
+    assert len(got) == len(xs)
+    for i, (x, (values, bitmask)) in enumerate(zip(xs, got)):
+        want_v, want_b = sparse24_bitmask_compress(x.to(gpu))
+        assert_bit_equal(values, want_v, f"values {i}")
+        assert_bit_equal(bitmask, want_b, f"bitmask {i}")
+        o_v, o_b = osp.sparse24_bitmask_compress(x)
+        assert_bit_equal(values, o_v, f"values {i} vs oracle")
+        assert_bit_equal(bitmask, o_b, f"bitmask {i} vs oracle")
+    items = [(v, b, list(s)) for (v, b), s in zip(got, shapes)]
+    # a tensor whose bitmask keeps half of the elements but not 2 per group
+    rows, cols = 40, 256
+    keep = torch.zeros(rows, cols, dtype=torch.bool)
+    keep.scatter_(1, torch.rand(rows, cols, generator=g).argsort(dim=1)[:, : cols // 2], True)
+    odd = torch.randn(rows, cols, generator=g).clamp(-3, 3)
+    odd[odd == 0] = 1.0
+    odd = torch.where(keep, odd, torch.zeros_like(odd)).to(dtype)
+    raw = odd.view(torch.int8) if dtype == torch.float8_e4m3fn else odd
+    odd_values = raw[keep].reshape(rows, cols // 2)
+    if dtype == torch.float8_e4m3fn:
+        odd_values = odd_values.view(torch.float8_e4m3fn)
+    items.insert(4, (odd_values.to(gpu), pack_bitmasks(keep.to(gpu)), [rows, cols]))
+    dense = sparse24_bitmask_decompress_many(items)
+    assert len(dense) == len(items)
+    for i, ((v, b, s), d) in enumerate(zip(items, dense)):
+        assert_bit_equal(d, sparse24_bitmask_decompress(v, b, torch.Size(s)), f"dense {i}")
+    assert_bit_equal(dense[4], odd, "tensor with a bitmask that is not 2:4")
+    for i, x in enumerate(xs):
+        k = i if i < 4 else i + 1
+        assert_bit_equal(dense[k], osp.sparse24_bitmask_decompress(*osp.sparse24_bitmask_compress(x), shapes[i]),
+                         f"dense {k} vs oracle")
+    # the calls after a repair find the launch counters back at zero: once more, all 2:4
+    again = sparse24_bitmask_decompress_many([it for k, it in enumerate(items) if k != 4])
+    for i, d in enumerate(again):
+        assert_bit_equal(d, dense[i if i < 4 else i + 1], f"second call {i}")
+
+
+def test_sparse24_compressor_state_dict_in_few_calls(gpu):
+    """Sparse24BitMaskCompressor.compress / decompress on a state dict (one multi-tensor
+    call per dtype) against the oracle tensor by tensor"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("sparse24 state dict")
+    g = torch.Generator().manual_seed(2)
+    state = {f"layers.{i}.proj.weight": _prune24(torch.randn(64 + 32 * i, 256, generator=g)).bfloat16().to(gpu)
+             for i in range(10)}
+    state["layers.0.proj.bias"] = torch.randn(64, generator=g).to(gpu)
+    state["norm.weight"] = torch.randn(256, 4, generator=g).to(gpu)  # rows of half a bitmask byte
+    comp = BaseCompressor.load_from_registry("sparse-24-bitmask")
+    packed = comp.compress(state, compression_targets={n[: -len(".weight")] for n in state if n.endswith("weight")})
+    for name, w in state.items():
+        if not name.endswith(".weight"):
+            assert packed[name] is w
+            continue
+        prefix = name[: -len(".weight")]
+        o_v, o_b = osp.sparse24_bitmask_compress(w.cpu())
+        assert_bit_equal(packed[prefix + ".compressed"], o_v, name)
+        assert_bit_equal(packed[prefix + ".bitmask"], o_b, name)
+        assert packed[prefix + ".shape"].flatten().tolist() == list(w.shape)
+    back = dict(comp.decompress(packed))
+    assert set(back) == set(state)
+    for name, w in state.items():
+        want = w if not name.endswith(".weight") else osp.sparse24_bitmask_decompress(
+            *osp.sparse24_bitmask_compress(w.cpu()), tuple(w.shape))
+        assert_bit_equal(back[name], want, name)
