@@ -295,6 +295,13 @@ SIGNATURES = {
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32],
     ),
     "ctmi_observe_quantize_supported": (c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32]),
+    "ctmi_observe_quantize_blocks_supported": (
+        c_int32, [c_int32, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32]),
+    "ctmi_observe_quantize_blocks": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32,
+         c_void_p, c_int32, c_void_p, c_int32, c_void_p],
+    ),
     "ctmi_observe_quantize_many": (
         c_int32,
         [POINTER(ObserveQuantizeJob), c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p],

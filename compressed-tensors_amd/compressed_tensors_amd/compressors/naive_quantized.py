@@ -200,6 +200,10 @@ class NaiveQuantizationCompressor(BaseQuantizationCompressor):
         lib = _lib.load()
         w = weight.contiguous()
         qtype = _lib.QTYPE_INT if args.type == "int" else _lib.QTYPE_FLOAT
+        if args.strategy == QuantizationStrategy.BLOCK.value and rows > 0 and cols > 0:
+            out = self._observe_and_compress_blocks(w, args, qtype)
+            if out is not None:
+                return out if device is None else {k: v.to(device) for k, v in out.items()}
         fused = (
             blk_cols > 0 and can_quantize(weight, args) and rows > 0 and cols > 0
             and w.data_ptr() % (8 * w.element_size()) == 0
@@ -232,6 +236,35 @@ class NaiveQuantizationCompressor(BaseQuantizationCompressor):
             out["weight_zero_point"] = zero_point
         if device is not None:
             out = {k: v.to(device) for k, v in out.items()}
+        return out
+
+    def _observe_and_compress_blocks(self, w: Tensor, args: QuantizationArgs, qtype: int):
+        """block strategy: one workgroup per block, the weight read once
+        (ctmi_observe_quantize_blocks); None where the layout has no such kernel"""
+        from compressed_tensors_amd.quantization.helpers import _zp_dtype
+
+        lib = _lib.load()
+        rows, cols = w.shape
+        bh, bw = args.block_structure
+        if not (can_quantize(w, args) and w.data_ptr() % (8 * w.element_size()) == 0
+                and lib.ctmi_observe_quantize_blocks_supported(
+                    _lib.dtype_code(w.dtype), rows, cols, bh, bw, qtype, args.num_bits)):
+            return None
+        codes = torch.empty((rows, cols), dtype=args.pytorch_dtype(), device=w.device)
+        scale = torch.empty((rows // bh, cols // bw), dtype=w.dtype, device=w.device)
+        zero_point = None
+        if not args.symmetric:
+            zero_point = torch.empty((rows // bh, cols // bw), dtype=_zp_dtype(args), device=w.device)
+        _lib.check(
+            lib.ctmi_observe_quantize_blocks(
+                w.data_ptr(), _lib.dtype_code(w.dtype), codes.data_ptr(), rows, cols, bh, bw, qtype,
+                args.num_bits, int(args.symmetric), scale.data_ptr(), _lib.dtype_code(scale.dtype),
+                _lib.ptr(zero_point), _lib.dtype_code(_zp_dtype(args)), _lib.stream_of(w.device),
+            )
+        )
+        out = {"weight": codes, "weight_scale": scale}
+        if zero_point is not None:
+            out["weight_zero_point"] = zero_point
         return out
 
     def decompress_weight(

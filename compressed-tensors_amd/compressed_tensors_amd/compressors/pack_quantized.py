@@ -173,14 +173,17 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
 
     def observe_and_compress_weight(
         self, weight: Tensor, quantization_args: QuantizationArgs,
-        device: Optional[torch.device] = None,
+        device: Optional[torch.device] = None, g_idx: Optional[Tensor] = None,
     ) -> Dict[str, Tensor]:
         """One-shot (round-to-nearest) compression of a weight that has no scales yet:
         the min-max observer (tests/mock_observer.py:38-113), calculate_qparams
         (quantization/utils/helpers.py:67-146) and compress_weight
-        (pack_quantized.py:88-146) in one pass over the weight.  Returns
-        compress_weight's dict plus "weight_scale" (and the packed
-        "weight_zero_point" of an asymmetric scheme)."""
+        (pack_quantized.py:88-146) in one pass over the weight for group and channel
+        strategies; the other strategies (one scale per tensor, blocks) and activation
+        ordering run the observer and the compressor one after the other.  With g_idx the
+        observer sees the columns in the order quantize groups them (sorted by g_idx,
+        forward.py:286-303).  Returns compress_weight's dict plus "weight_scale" (and the
+        packed "weight_zero_point" of an asymmetric scheme)."""
         args = quantization_args
         weight = to_gpu(weight)
         if weight.ndim != 2:
@@ -195,7 +198,7 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         lib = _lib.load()
         w = weight.contiguous()
         fused = (
-            blk_cols > 0 and args.type == "int" and can_quantize(weight, args)
+            g_idx is None and blk_cols > 0 and args.type == "int" and can_quantize(weight, args)
             and w.data_ptr() % (8 * w.element_size()) == 0
             and lib.ctmi_observe_pack_quantized_supported(
                 _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits)
@@ -203,8 +206,12 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         if not fused:
             from compressed_tensors_amd.quantization.helpers import observe_weight_qparams
 
-            scale, zero_point = observe_weight_qparams(weight, args)
-            out = self.compress_weight(weight, scale, args, zero_point=zero_point, device=device)
+            seen = weight
+            if g_idx is not None and not bool((g_idx == -1).any()):
+                seen = weight.index_select(1, torch.argsort(to_gpu(g_idx).long()))
+            scale, zero_point = observe_weight_qparams(seen, args)
+            out = self.compress_weight(weight, scale, args, zero_point=zero_point, g_idx=g_idx,
+                                       device=device)
             out["weight_scale"] = scale if device is None else scale.to(device)
             return out
         n_cells = cols // min(blk_cols, cols)
@@ -420,14 +427,16 @@ class ObservedWeightBatch:
     PackedQuantizationCompressor.observe_and_compress_weight returns."""
 
     def __init__(self, entries, device=None):
-        """entries: dicts with weight (2-D float tensor) and quantization_args
-        (int, 4 or 8 bits, group or channel strategy)"""
+        """entries: dicts with weight (2-D float tensor), quantization_args and, for
+        activation ordering, g_idx.  Integer group / channel schemes of 4 or 8 bits share the
+        one-pass launches; anything else (one scale per tensor, blocks, other group sizes,
+        g_idx) is compressed weight by weight when compress() runs, observer first."""
         lib = _lib.load()
-        self.n = len(entries)
         self.device = device
         self.weights, self.packed, self.scales, self.zero_points, self.args = [], [], [], [], []
-        self._jobs = (_lib.ObservePackJob * max(self.n, 1))()
-        for i, e in enumerate(entries):
+        self._slots = []   # per entry: ("fused", index into the job table) or ("single", entry)
+        jobs = []
+        for e in entries:
             args = e["quantization_args"]
             w = to_gpu(e["weight"]).contiguous()
             if w.ndim != 2:
@@ -437,31 +446,44 @@ class ObservedWeightBatch:
             rows, cols = w.shape
             blk_cols = {QuantizationStrategy.GROUP.value: args.group_size,
                         QuantizationStrategy.CHANNEL.value: cols}.get(args.strategy, 0)
-            if not (blk_cols and args.type == "int" and lib.ctmi_observe_pack_quantized_supported(
-                    _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits)):
-                raise NotImplementedError(
-                    f"no one-pass kernel for {args.strategy} / {args.num_bits} bits on a "
-                    f"{tuple(w.shape)} {w.dtype} weight: use observe_and_compress_weight")
+            if not (e.get("g_idx") is None and blk_cols and args.type == "int"
+                    and lib.ctmi_observe_pack_quantized_supported(
+                        _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits)):
+                self._slots.append(("single", dict(weight=w, quantization_args=args,
+                                                   g_idx=e.get("g_idx"))))
+                continue
+            self._slots.append(("fused", len(jobs)))
             n_cells = cols // min(blk_cols, cols)
             packed = torch.empty((rows, cols * args.num_bits // 32), dtype=torch.int32, device=w.device)
             scale = torch.empty((rows, n_cells), dtype=w.dtype, device=w.device)
             zp = None if args.symmetric else torch.empty((rows, n_cells), dtype=torch.int8, device=w.device)
-            j = self._jobs[i]
-            j.x, j.packed, j.scale, j.zero_point = w.data_ptr(), packed.data_ptr(), scale.data_ptr(), _lib.ptr(zp)
-            j.rows, j.cols, j.blk_cols = rows, cols, blk_cols
-            j.x_dtype, j.num_bits, j.symmetric = _lib.dtype_code(w.dtype), args.num_bits, int(args.symmetric)
+            jobs.append((w.data_ptr(), packed.data_ptr(), scale.data_ptr(), _lib.ptr(zp), rows, cols,
+                         blk_cols, _lib.dtype_code(w.dtype), args.num_bits, int(args.symmetric)))
             self.weights.append(w)
             self.packed.append(packed)
             self.scales.append(scale)
             self.zero_points.append(zp)
             self.args.append(args)
+        self.n = len(jobs)
+        self._jobs = (_lib.ObservePackJob * max(self.n, 1))()
+        for j, f in zip(self._jobs, jobs):
+            (j.x, j.packed, j.scale, j.zero_point, j.rows, j.cols, j.blk_cols, j.x_dtype, j.num_bits,
+             j.symmetric) = f
 
     def compress(self):
-        _lib.check(_lib.load().ctmi_observe_pack_quantized_many(self._jobs, self.n,
-                                                                _lib.stream_of(self.device)))
+        if self.n:
+            _lib.check(_lib.load().ctmi_observe_pack_quantized_many(self._jobs, self.n,
+                                                                    _lib.stream_of(self.device)))
+        comp = None
         out = []
-        for w, packed, scale, zp, args in zip(self.weights, self.packed, self.scales,
-                                              self.zero_points, self.args):
+        for kind, what in self._slots:
+            if kind == "single":
+                comp = comp or BaseCompressor.load_from_registry(CompressionFormat.pack_quantized.value)
+                out.append(comp.observe_and_compress_weight(
+                    what["weight"], what["quantization_args"], g_idx=what["g_idx"]))
+                continue
+            w, packed, scale, zp, args = (self.weights[what], self.packed[what], self.scales[what],
+                                          self.zero_points[what], self.args[what])
             d = {"weight_shape": torch.tensor(w.shape), "weight_packed": packed, "weight_scale": scale}
             if zp is not None:
                 d["weight_zero_point"] = pack_to_int32(zp, args.num_bits, packed_dim=0)

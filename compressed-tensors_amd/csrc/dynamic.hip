@@ -81,19 +81,41 @@ __device__ __forceinline__ void store_result(void* out_any, int64_t v, bool keep
 // One workgroup of 256 threads per row-long segment (token / channel) of up to
 // 256 * U vectors of 8 elements: every vector is loaded before anything is looked
 // at; the four wavefronts meet once, over a few words in LDS.
-template <typename FT, int QK, bool SYM, int U, bool CODES>
+// Where the vectors of a cell lie.  A row-long segment is one run of vectors; a block of
+// the block strategy (observer reshape of tests/mock_observer.py:95-113: cells of
+// block_height x block_width elements) is `ipr` vectors in each of its rows.
+struct CellLayout {
+  int ipr;          // vectors per row of the cell (0: the cell is one run of vectors)
+  int row_pitch;    // vectors per row of the tensor
+  int cells_per_row;
+  int cell_rows;
+};
+
+template <bool BLOCK>
+__device__ __forceinline__ int64_t cell_vector(const CellLayout& g, int64_t s, int items, int i) {
+  if constexpr (!BLOCK) {
+    return s * (int64_t)items + i;
+  } else {
+    const int64_t br = s / g.cells_per_row, bc = s - br * g.cells_per_row;
+    const int r = i / g.ipr, ci = i - r * g.ipr;
+    return (br * g.cell_rows + r) * (int64_t)g.row_pitch + bc * g.ipr + ci;
+  }
+}
+
+template <typename FT, int QK, bool SYM, int U, bool CODES, bool BLOCK = false>
 __device__ __forceinline__ void rows_segment(const typename FT::raw* __restrict__ x,
                                              void* __restrict__ out_any, const DynOut& o, int items,
-                                             int64_t s, const QpCfg& c) {
+                                             int64_t s, const QpCfg& c,
+                                             const CellLayout& g = CellLayout{0, 0, 0, 0}) {
   using FR = typename FT::raw;
   __shared__ float part_lo[4], part_hi[4];
   __shared__ int part_word[4];
-  const FR* p = x + s * (int64_t)items * 8;
   Vec<FR, 8> a[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int i = k * 256 + threadIdx.x;
-    a[k] = ldg_nt<FR, 8>(p + (int64_t)(i < items ? i : items - 1) * 8);  // re-reads do not change min / max
+    // past the end: re-reads do not change min / max
+    a[k] = ldg_nt<FR, 8>(x + cell_vector<BLOCK>(g, s, items, i < items ? i : items - 1) * 8);
   }
   float sv, zv;
   if constexpr (SYM && sizeof(FR) == 2) {
@@ -134,8 +156,17 @@ __device__ __forceinline__ void rows_segment(const typename FT::raw* __restrict_
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const int i = k * 256 + threadIdx.x;
-    store_result<FT, QK, CODES>(out_any, s * (int64_t)items + i, i < items, a[k], sv, zv, c);
+    store_result<FT, QK, CODES>(out_any, cell_vector<BLOCK>(g, s, items, i < items ? i : 0), i < items,
+                                a[k], sv, zv, c);
   }
+}
+
+// one workgroup per block of the block strategy, the whole block in registers
+template <typename FT, int QK, bool SYM, int U>
+__global__ void __launch_bounds__(256)
+observe_quantize_blocks_kernel(const typename FT::raw* __restrict__ x, void* __restrict__ codes,
+                               DynOut o, int items, CellLayout g, QpCfg c) {
+  rows_segment<FT, QK, SYM, U, true, true>(x, codes, o, items, blockIdx.x, c, g);
 }
 
 template <typename FT, int QK, bool SYM, int U, bool CODES>
@@ -328,6 +359,64 @@ extern "C" int ctmi_observe_quantize(const void* x, int32_t x_dtype, void* codes
 #undef CTMI_OQ_FT
   CTMI_REQUIRE(ok, CTMI_ERR_UNSUPPORTED, "no fused kernel for this layout");
   return check_launch("ctmi_observe_quantize");
+}
+
+extern "C" int ctmi_observe_quantize_blocks_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                                      int64_t blk_rows, int64_t blk_cols,
+                                                      int32_t qtype, int32_t num_bits) {
+  if (x_dtype != CTMI_BF16 && x_dtype != CTMI_F16 && x_dtype != CTMI_F32) return 0;
+  if (rows < 1 || cols < 1 || blk_rows < 1 || blk_cols < 1) return 0;
+  if (!((qtype == CTMI_QTYPE_INT && num_bits <= 8) || (qtype == CTMI_QTYPE_FLOAT && num_bits == 8)))
+    return 0;
+  if (rows % blk_rows || cols % blk_cols || blk_cols % 8) return 0;
+  if (cols / 8 >= (1ll << 31) || (rows / blk_rows) * (cols / blk_cols) >= (1ll << 31)) return 0;
+  return blk_rows * blk_cols / 8 <= 2048;  // a block lives in the registers of one workgroup
+}
+
+extern "C" int ctmi_observe_quantize_blocks(const void* x, int32_t x_dtype, void* codes, int64_t rows,
+                                            int64_t cols, int64_t blk_rows, int64_t blk_cols,
+                                            int32_t qtype, int32_t num_bits, int32_t symmetric,
+                                            void* scale_out, int32_t scale_dtype, void* zp_out,
+                                            int32_t zp_dtype, void* stream) {
+  CTMI_REQUIRE(rows >= 1 && cols >= 1, CTMI_ERR_VALUE, "cannot observe an empty tensor");
+  CTMI_REQUIRE(blk_rows >= 1 && blk_cols >= 1, CTMI_ERR_VALUE, "empty cell");
+  QpCfg c;
+  // min / max of a block are not 0-d tensors: the zero-point arithmetic stays in x's dtype
+  int rc = fill_qpcfg(&c, qtype, num_bits, symmetric, x_dtype, 0, false, scale_dtype, zp_dtype);
+  if (rc) return rc;
+  CTMI_REQUIRE(x && codes && scale_out, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE(ctmi_observe_quantize_blocks_supported(x_dtype, rows, cols, blk_rows, blk_cols, qtype,
+                                                      num_bits),
+               CTMI_ERR_UNSUPPORTED,
+               "no fused kernel for this layout (blocks must tile the tensor, be a multiple of 8 "
+               "wide and hold at most 16384 elements): compute the scales and quantize separately");
+  CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)codes % 8 == 0,
+               CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+  hipStream_t st = (hipStream_t)stream;
+  const DynOut o{scale_out, zp_out};
+  const int items = (int)(blk_rows * blk_cols / 8);
+  const CellLayout g{(int)(blk_cols / 8), (int)(cols / 8), (int)(cols / blk_cols), (int)blk_rows};
+  const unsigned grid = (unsigned)((rows / blk_rows) * (cols / blk_cols));
+#define CTMI_OQB_U(FT, QK, SYM, UU)                                                               \
+  hipLaunchKernelGGL((observe_quantize_blocks_kernel<FT, QK, SYM, UU>), grid, 256, 0, st,         \
+                     (const typename FT::raw*)x, codes, o, items, g, c)
+#define CTMI_OQB(FT, QK, SYM)                    \
+  if (items <= 256) CTMI_OQB_U(FT, QK, SYM, 1);  \
+  else if (items <= 512) CTMI_OQB_U(FT, QK, SYM, 2);  \
+  else if (items <= 1024) CTMI_OQB_U(FT, QK, SYM, 4); \
+  else CTMI_OQB_U(FT, QK, SYM, 8)
+#define CTMI_OQB_SYM(FT, QK) \
+  if (symmetric) { CTMI_OQB(FT, QK, true); } else { CTMI_OQB(FT, QK, false); }
+#define CTMI_OQB_FT(FT) \
+  if (qtype == CTMI_QTYPE_INT) { CTMI_OQB_SYM(FT, 0) } else { CTMI_OQB_SYM(FT, 1) }
+  if (x_dtype == CTMI_BF16) { CTMI_OQB_FT(BF16) }
+  else if (x_dtype == CTMI_F16) { CTMI_OQB_FT(F16) }
+  else { CTMI_OQB_FT(F32) }
+#undef CTMI_OQB_U
+#undef CTMI_OQB
+#undef CTMI_OQB_SYM
+#undef CTMI_OQB_FT
+  return check_launch("ctmi_observe_quantize_blocks");
 }
 
 // rows-per-workgroup class of a job (0: not a row-kernel layout)

@@ -433,6 +433,20 @@ int ctmi_observe_quantize(const void* x, int32_t x_dtype, void* codes, int64_t r
                           void* scale_out, int32_t scale_dtype, void* zp_out, int32_t zp_dtype,
                           void* stream);
 
+/* The same for the block strategy (cells of blk_rows x blk_cols elements, the observer's
+ * reshape in tests/mock_observer.py:95-113; e.g. 128 x 128 fp8 blocks): one workgroup holds
+ * a block in registers, so the weight is still read once.  scale_out / zp_out:
+ * [rows / blk_rows, cols / blk_cols].  Blocks must tile the tensor, be a multiple of 8
+ * wide and hold at most 16384 elements.  Same bits as ctmi_minmax + ctmi_calculate_qparams
+ * + ctmi_qdq. */
+int ctmi_observe_quantize_blocks_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                           int64_t blk_rows, int64_t blk_cols, int32_t qtype,
+                                           int32_t num_bits);
+int ctmi_observe_quantize_blocks(const void* x, int32_t x_dtype, void* codes, int64_t rows,
+                                 int64_t cols, int64_t blk_rows, int64_t blk_cols, int32_t qtype,
+                                 int32_t num_bits, int32_t symmetric, void* scale_out,
+                                 int32_t scale_dtype, void* zp_out, int32_t zp_dtype, void* stream);
+
 /* every weight of a state dict in one call: rows of one length class share launches,
  * eight weights at a time; scale_dtype < 0: every weight's scales in its own dtype */
 typedef struct ctmi_observe_quantize_job {

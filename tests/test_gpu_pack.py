@@ -211,9 +211,38 @@ def test_observed_weight_batch_matches_single_calls(gpu):
         assert set(d) == set(want)
         for k in want:
             assert_bit_equal(d[k], want[k], k)
-    with pytest.raises(NotImplementedError):
-        ObservedWeightBatch([dict(weight=entries[0]["weight"], quantization_args=QuantizationArgs(
-            num_bits=4, type="int", symmetric=True, strategy="tensor"))])
+
+
+def test_observed_weight_batch_takes_every_strategy(gpu):
+    """weights without a one-pass kernel (one scale per tensor, blocks, a group size that is
+    not a power of two, activation ordering) go through the batch as well: the observer and
+    the compressor run one after the other for them.  Against the oracle's observer (on the
+    columns sorted by g_idx where there is one, forward.py:286-303) and compressor."""
+    from compressed_tensors_amd.compressors import ObservedWeightBatch
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    announce("observed weight batch, every strategy")
+    g = torch.Generator().manual_seed(18)
+    specs = [dict(num_bits=4, type="int", symmetric=True, strategy="tensor"),
+             dict(num_bits=4, type="int", symmetric=False, strategy="block", block_structure=[16, 64]),
+             dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=24),
+             dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128),
+             dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=32)]
+    shapes = [(32, 128), (48, 192), (16, 48), (64, 512), (24, 256)]
+    ws = [(torch.randn(s, generator=g) * 0.02).bfloat16() for s in shapes]
+    g_idx = [None, None, None, None, torch.randperm(256, generator=g).to(torch.int32) // 32]
+    entries = [dict(weight=w.to(gpu), quantization_args=QuantizationArgs(**spec),
+                    **({} if gi is None else {"g_idx": gi.to(gpu)}))
+               for w, spec, gi in zip(ws, specs, g_idx)]
+    got = ObservedWeightBatch(entries).compress()
+    for i, (w, spec, gi, d) in enumerate(zip(ws, specs, g_idx, got)):
+        oargs = oq._Args(**spec)
+        seen = w if gi is None else w.index_select(1, torch.argsort(gi.long()))
+        scale, zp = oq.observe_weight(seen, oargs)
+        want = op.pack_quantized_compress(w, scale, oargs, zero_point=zp, g_idx=gi)
+        assert_bit_equal(d["weight_scale"], scale, f"scale {i}")
+        for k in want:
+            assert_bit_equal(d[k], want[k], f"{k} {i}")
 
 
 def test_pack_quantized_state_dict_and_g_idx(gpu):
@@ -682,7 +711,14 @@ OQ = [
     ("int-quantized", dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=128), (16, 256), torch.float16),
     ("naive-quantized", dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32), (16, 64), torch.float32),
     ("float-quantized", dict(num_bits=8, type="float", symmetric=False, strategy="channel"), (12, 640), torch.bfloat16),
-    # no fused kernel: rows longer than 16384, one scale for the whole tensor
+    # block strategy: one workgroup per block, the block in registers
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[128, 128]), (256, 512), torch.bfloat16),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[128, 128]), (128, 4096), torch.float16),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=False, strategy="block", block_structure=[16, 64]), (48, 192), torch.float32),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=False, strategy="block", block_structure=[3, 8]), (9, 40), torch.bfloat16),
+    # no fused kernel: a block of more than 16384 elements, rows longer than 16384, one scale
+    # for the whole tensor
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[256, 128]), (256, 256), torch.bfloat16),
     ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), (3, 16392), torch.bfloat16),
     ("int-quantized", dict(num_bits=8, type="int", symmetric=True, strategy="tensor"), (31, 64), torch.bfloat16),
 ]
