@@ -462,6 +462,26 @@ def other_workload(torch, name, seed):
                 Op("nvfp4 compress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.compress], set_bytes, "nvfp4_compress_chain_kernel"),
                 Op("nvfp4 decompress, Llama-3-8B set, one call per weight (224)", single_d, set_bytes, "nvfp4_decompress_vec_kernel", primary=False),
                 Op("nvfp4 decompress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.decompress], set_bytes, "nvfp4_decompress_chain_kernel")]
+        # one-shot: group scales + codes from one pass over weights whose global scale is known
+        oj = (_lib.ObserveNvfp4Job * batch.n)()
+        one_calls = []
+        for i, e in enumerate(entries):
+            w, gs = e["weight"], e["global_scale"]
+            r, c = w.shape
+            sc_out = torch.empty(r, c // 16, dtype=FP8, device=dev)
+            keep.append(sc_out)
+            cj = batch._cjobs[i]
+            oj[i].x, oj[i].global_scale, oj[i].packed, oj[i].scale = w.data_ptr(), gs.data_ptr(), cj.dst, sc_out.data_ptr()
+            oj[i].rows, oj[i].cols, oj[i].x_dtype = r, c, code(w.dtype)
+            oa = (w.data_ptr(), code(w.dtype), r, c, gs.data_ptr(), cj.dst, sc_out.data_ptr(), st)
+            one_calls.append(lambda oa=oa: _lib.check(lib.ctmi_observe_nvfp4_compress(*oa)))
+        keep.append(oj)
+        om = (oj, batch.n, st)
+        ops += [Op("nvfp4 one-shot (scales + codes), Llama-3-8B set, one call per weight (224)", one_calls, set_bytes,
+                   "nvfp4_observe_compress_kernel", primary=False),
+                Op("nvfp4 one-shot (scales + codes), Llama-3-8B set, all weights in one call (8 per launch)",
+                   [lambda: _lib.check(lib.ctmi_observe_nvfp4_compress_many(*om))], set_bytes,
+                   "nvfp4_observe_compress_chain_kernel")]
         aargs = QuantizationArgs(num_bits=4, type="float", symmetric=True, strategy="tensor_group",
                                  group_size=16, dynamic="local")
         o_calls, f_calls, y_calls = [], [], []

@@ -105,6 +105,13 @@ class Sparse24Job(ctypes.Structure):
                 ("nvalues", c_int64), ("rows", c_int64), ("cols", c_int64)]
 
 
+class ObserveNvfp4Job(ctypes.Structure):
+    """mirror of `struct ctmi_observe_nvfp4_job`"""
+
+    _fields_ = [("x", c_void_p), ("global_scale", c_void_p), ("packed", c_void_p), ("scale", c_void_p),
+                ("rows", c_int64), ("cols", c_int64), ("x_dtype", c_int32), ("reserved", c_int32)]
+
+
 class ObserveQuantizeJob(ctypes.Structure):
     """mirror of `struct ctmi_observe_quantize_job`"""
 
@@ -295,6 +302,7 @@ SIGNATURES = {
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32],
     ),
     "ctmi_observe_quantize_supported": (c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32, c_int32]),
+    "ctmi_observe_nvfp4_compress_many": (c_int32, [POINTER(ObserveNvfp4Job), c_int64, c_void_p]),
     "ctmi_observe_quantize_blocks_supported": (
         c_int32, [c_int32, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32]),
     "ctmi_observe_quantize_blocks": (

@@ -24,6 +24,7 @@ from compressed_tensors_amd.quantization.forward import (
 from compressed_tensors_amd.quantization.quant_args import QuantizationArgs
 
 __all__ = [
+    "nvfp4_observe_and_compress_weights",
     "Fp4WeightBatch",
     "NVFP4PackedCompressor",
     "MXFP4PackedCompressor",
@@ -179,6 +180,42 @@ class NVFP4PackedCompressor(BaseQuantizationCompressor):
             )
         )
         return out
+
+
+def nvfp4_observe_and_compress_weights(weights, quantization_args: QuantizationArgs,
+                                       global_scales=None):
+    """NVFP4PackedCompressor.observe_and_compress_weight for a list of 2-D weights from one
+    call (ctmi_observe_nvfp4_compress_many: weights of one dtype share launches, eight at a
+    time).  global_scales: one per weight, or None (then each is generate_gparam of its
+    weight's min / max).  Returns one dict per weight."""
+    from compressed_tensors_amd.quantization.helpers import generate_gparam, minmax
+
+    args = quantization_args
+    if args.group_size != 16:
+        raise NotImplementedError("one-pass nvfp4 compression needs groups of 16 columns")
+    ws = [to_gpu(w).contiguous() for w in weights]
+    jobs = (_lib.ObserveNvfp4Job * max(len(ws), 1))()
+    results = []
+    for i, (job, w) in enumerate(zip(jobs, ws)):
+        if w.ndim != 2:
+            raise ValueError(f"expected a 2-D weight, got shape {tuple(w.shape)}")
+        rows, cols = w.shape
+        if cols % 16 or w.data_ptr() % (8 * w.element_size()):
+            raise NotImplementedError("one-pass nvfp4 compression needs groups of 16 columns")
+        gs = None if global_scales is None else global_scales[i]
+        if gs is None:
+            mn, mx = minmax(w, rows, cols)
+            gs = generate_gparam(mn.reshape(1), mx.reshape(1))
+        gs = to_gpu(gs).to(torch.float32).reshape(-1).contiguous()
+        packed = torch.empty((rows, cols // 2), dtype=torch.uint8, device=w.device)
+        scale = torch.empty((rows, cols // 16), dtype=torch.float8_e4m3fn, device=w.device)
+        job.x, job.global_scale, job.packed, job.scale = (
+            w.data_ptr(), gs.data_ptr(), packed.data_ptr(), scale.data_ptr())
+        job.rows, job.cols, job.x_dtype = rows, cols, _lib.dtype_code(w.dtype)
+        results.append({"weight_packed": packed, "weight_scale": scale, "weight_global_scale": gs})
+    if ws:
+        _lib.check(_lib.load().ctmi_observe_nvfp4_compress_many(jobs, len(ws), _lib.stream_of(ws[0].device)))
+    return results
 
 
 class Fp4WeightBatch(LazyDenseOutputs):

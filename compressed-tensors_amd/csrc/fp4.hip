@@ -744,15 +744,16 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
 // helpers.py:101-120) and NVFP4PackedCompressor.compress_weight
 // (fp4_quantized.py:84-107) with those scales and their all-zero zero points, the
 // weight read once.
+constexpr int kFp4ObserveU = 2;
+
 template <typename XT>
-__global__ void __launch_bounds__(kFp4Block)
-nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
-                              const float* __restrict__ gscale, uint32_t* __restrict__ packed,
-                              uint8_t* __restrict__ scale_out, uint32_t nvec) {
-  constexpr int B = kFp4Block, U = 2;
-  __shared__ Fp4Scale lut[256];
-  const float gs = gscale[0];
-  const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
+__device__ __forceinline__ void nvfp4_observe_compress_chunk(const typename XT::raw* __restrict__ x,
+                                                             float gs, uint32_t* __restrict__ packed,
+                                                             uint8_t* __restrict__ scale_out,
+                                                             uint32_t nvec, uint32_t chunk,
+                                                             Fp4Scale* lut) {
+  constexpr int B = kFp4Block, U = kFp4ObserveU;
+  const uint32_t v0 = chunk * (B * U) + threadIdx.x;
   Vec<typename XT::raw, 8> xv[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
@@ -800,6 +801,28 @@ nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
     const uint32_t v = v0 + k * B;
     if (v < nvec) packed[v] = nvfp4_codes_exact<XT, true>(xv[k], lut[codes[k]].s, 0.0f);
   }
+}
+
+template <typename XT>
+__global__ void __launch_bounds__(kFp4Block)
+nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
+                              const float* __restrict__ gscale, uint32_t* __restrict__ packed,
+                              uint8_t* __restrict__ scale_out, uint32_t nvec) {
+  __shared__ Fp4Scale lut[256];
+  nvfp4_observe_compress_chunk<XT>(x, gscale[0], packed, scale_out, nvec, blockIdx.x, lut);
+}
+
+// ... for up to kMaxJobs weights per launch: job.scale is written, the zero-point slot
+// carries the global scale (as in nvfp4_compress_chain_kernel)
+template <typename XT>
+__global__ void __launch_bounds__(kFp4Block) nvfp4_observe_compress_chain_kernel(ChainTable t) {
+  __shared__ Fp4Scale lut[256];
+  uint32_t local, nvec;
+  const ChainJob job = find_job(t, blockIdx.x, &local, &nvec);
+  nvfp4_observe_compress_chunk<XT>(static_cast<const typename XT::raw*>(job.src),
+                                   reinterpret_cast<const float*>(job.zp)[0],
+                                   static_cast<uint32_t*>(job.dst),
+                                   static_cast<uint8_t*>(const_cast<void*>(job.scale)), nvec, local, lut);
 }
 
 // The observer on its own for the same scheme (tests/mock_observer.py:38-113 +
@@ -1130,7 +1153,7 @@ extern "C" int ctmi_observe_nvfp4_compress(const void* x, int32_t x_dtype, int64
   CTMI_REQUIRE((uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)packed % 4 == 0,
                CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
   const int64_t nvec = rows * cols / 8;
-  const int64_t grid = cdiv(nvec, kFp4Block * 2);
+  const int64_t grid = cdiv(nvec, kFp4Block * kFp4ObserveU);
   CTMI_REQUIRE(nvec < (1ll << 32) && grid < (1ll << 31), CTMI_ERR_UNSUPPORTED, "tensor too large");
   hipStream_t st = (hipStream_t)stream;
   auto* out = (uint32_t*)packed;
@@ -1138,4 +1161,68 @@ extern "C" int ctmi_observe_nvfp4_compress(const void* x, int32_t x_dtype, int64
   else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(nvfp4_observe_compress_kernel<F16>, (unsigned)grid, kFp4Block, 0, st, (const uint16_t*)x, global_scale, out, scale, (uint32_t)nvec);
   else hipLaunchKernelGGL(nvfp4_observe_compress_kernel<F32>, (unsigned)grid, kFp4Block, 0, st, (const float*)x, global_scale, out, scale, (uint32_t)nvec);
   return check_launch("ctmi_observe_nvfp4_compress");
+}
+
+extern "C" int ctmi_observe_nvfp4_compress_many(const ctmi_observe_nvfp4_job* jobs, int64_t n,
+                                                void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  // everything is checked before anything is enqueued
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_observe_nvfp4_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 1 && j.cols >= 1, CTMI_ERR_VALUE, "job %lld: cannot observe an empty tensor",
+                 (long long)i);
+    int rc = check_float3(j.x_dtype, "nvfp4 input");
+    if (rc) return rc;
+    CTMI_REQUIRE(j.cols % 16 == 0, CTMI_ERR_UNSUPPORTED, "job %lld: columns must come in groups of 16",
+                 (long long)i);
+    CTMI_REQUIRE(j.x && j.global_scale && j.packed && j.scale, CTMI_ERR_VALUE,
+                 "job %lld: NULL tensor pointer", (long long)i);
+    CTMI_REQUIRE((uintptr_t)j.x % (8 * dtype_size(j.x_dtype)) == 0 && (uintptr_t)j.packed % 4 == 0,
+                 CTMI_ERR_VALUE, "job %lld: tensors must be aligned to 8 elements", (long long)i);
+    CTMI_REQUIRE(j.rows * j.cols / 8 < (1ll << 31), CTMI_ERR_UNSUPPORTED, "job %lld: tensor too large",
+                 (long long)i);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const int dts[3] = {CTMI_BF16, CTMI_F16, CTMI_F32};
+  for (int d = 0; d < 3; ++d) {
+    ChainTable t;
+    int filled = 0;
+    uint32_t total = 0;
+    auto flush = [&]() {
+      for (int k = filled; k < kMaxJobs; ++k) {
+        t.chunk_end[k] = 0xFFFFFFFFu;
+        t.nvec[k] = 0;
+        t.job[k] = ChainJob{};
+      }
+      t.n = filled;
+      t.qmin = t.qmax = 0.0f;
+      if (dts[d] == CTMI_BF16)
+        hipLaunchKernelGGL(nvfp4_observe_compress_chain_kernel<BF16>, total, kFp4Block, 0, st, t);
+      else if (dts[d] == CTMI_F16)
+        hipLaunchKernelGGL(nvfp4_observe_compress_chain_kernel<F16>, total, kFp4Block, 0, st, t);
+      else
+        hipLaunchKernelGGL(nvfp4_observe_compress_chain_kernel<F32>, total, kFp4Block, 0, st, t);
+      filled = 0;
+      total = 0;
+    };
+    for (int64_t i = 0; i < n; ++i) {
+      const ctmi_observe_nvfp4_job& j = jobs[i];
+      if (j.x_dtype != dts[d]) continue;
+      const uint32_t nvec = (uint32_t)(j.rows * j.cols / 8);
+      const uint32_t chunks = (uint32_t)cdiv((int64_t)nvec, kFp4Block * kFp4ObserveU);
+      if (filled && (uint64_t)total + chunks >= (1ull << 31)) flush();
+      ChainJob cj{};
+      cj.src = j.x;
+      cj.dst = j.packed;
+      cj.scale = j.scale;
+      cj.zp = reinterpret_cast<const int8_t*>(j.global_scale);
+      t.job[filled] = cj;
+      t.nvec[filled] = nvec;
+      total += chunks;
+      t.chunk_end[filled] = total;
+      if (++filled == kMaxJobs) flush();
+    }
+    if (filled) flush();
+  }
+  return n ? check_launch("ctmi_observe_nvfp4_compress_many") : CTMI_OK;
 }

@@ -397,6 +397,18 @@ int ctmi_observe_nvfp4_compress(const void* x, int32_t x_dtype, int64_t rows, in
                                 const float* global_scale, uint8_t* packed, uint8_t* scale,
                                 void* stream);
 
+/* every weight of a state dict in one call: weights of one dtype share launches, eight at
+ * a time */
+typedef struct ctmi_observe_nvfp4_job {
+  const void* x;
+  const float* global_scale;
+  uint8_t* packed;
+  uint8_t* scale;
+  int64_t rows, cols;
+  int32_t x_dtype, reserved;
+} ctmi_observe_nvfp4_job;
+int ctmi_observe_nvfp4_compress_many(const ctmi_observe_nvfp4_job* jobs, int64_t n, void* stream);
+
 /* A26.  Dynamic activation quantization in one pass (forward_quantize with
  * args.dynamic, quantization/lifecycle/forward.py:414-451): the scales of
  * compute_dynamic_scales_and_zp (quantization/utils/helpers.py:149-205, via

@@ -478,6 +478,38 @@ def test_nvfp4_observe_and_compress_in_one_pass(shape, dtype, gpu):
         comp.observe_and_compress_weight(w.to(gpu)[:, :24].contiguous(), args)
 
 
+def test_nvfp4_observe_and_compress_many_weights(gpu):
+    """nvfp4_observe_and_compress_weights == observe_and_compress_weight weight by weight and
+    the oracle: more weights than a launch takes, three dtypes, a chunk that ends ragged"""
+    from compressed_tensors_amd.compressors import BaseCompressor, nvfp4_observe_and_compress_weights
+
+    announce("one-shot nvfp4, many weights")
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+    args, oargs = _pair(spec)
+    shapes = [(64, 256, torch.bfloat16), (37, 48, torch.bfloat16), (32, 4112, torch.float16), (8, 64, torch.float32),
+              (128, 512, torch.bfloat16), (5, 16, torch.bfloat16), (96, 1024, torch.bfloat16), (40, 2048, torch.bfloat16),
+              (16, 4096, torch.bfloat16), (300, 64, torch.bfloat16), (24, 768, torch.float16), (12, 3072, torch.bfloat16)]
+    g = torch.Generator().manual_seed(66)
+    ws = [(torch.randn(r, c, generator=g) * 0.02).to(dt) for r, c, dt in shapes]
+    comp = BaseCompressor.load_from_registry("nvfp4-pack-quantized")
+    got = nvfp4_observe_and_compress_weights([w.to(gpu) for w in ws], args)
+    assert len(got) == len(ws)
+    for i, (w, out) in enumerate(zip(ws, got)):
+        single = comp.observe_and_compress_weight(w.to(gpu), args)
+        assert set(out) == set(single)
+        for key in single:
+            assert_bit_equal(out[key], single[key], f"weight {i} {key}")
+        gs = oq.generate_gparam(*[t.reshape(1) for t in torch.aminmax(w)])
+        scale, zp = oq.observe_weight(w, oargs, global_scale=gs)
+        assert_bit_equal(out["weight_scale"], scale, f"weight {i} scales vs oracle")
+        assert_bit_equal(out["weight_packed"], op.nvfp4_compress(w, scale, gs, oargs, zero_point=zp),
+                         f"weight {i} codes vs oracle")
+    given = nvfp4_observe_and_compress_weights([w.to(gpu) for w in ws[:3]], args,
+                                               global_scales=[o["weight_global_scale"] for o in got[:3]])
+    for i in range(3):
+        assert_bit_equal(given[i]["weight_packed"], got[i]["weight_packed"], f"global scale given {i}")
+
+
 @pytest.mark.parametrize("scale_value,global_scale", [(1.0, 1.0), (0.75, 3.0), (448.0, 1234.5),
                                                       (2.0 ** -9, 0.37)])
 def test_nvfp4_every_bf16_pattern(scale_value, global_scale, gpu):
