@@ -572,7 +572,7 @@ class HadamardTransform(torch.nn.Module):
         self.module_type = module_type
         self.precision = precision
         self._scale = torch.tensor(size, dtype=torch.float64).sqrt()
-        self._factor: Dict[Tuple[str, bool], Tensor] = {}
+        self._factor: Dict[tuple, Tensor] = {}
 
     @property
     def weight(self) -> Tensor:
@@ -612,11 +612,16 @@ class HadamardTransform(torch.nn.Module):
         mfma = (self.block is None and hadamard_factors(n) is not None and value.dtype in _FLOATS
                 and bool(lib.ctmi_hadamard_supported(*hadamard_factors(n),
                                                      _lib.dtype_code(value.dtype))))
-        plan = None if mfma else _kron_plan(n, self.block)
+        big = None  # (a, b): a known block times Sylvester(b) on the matrix cores
+        if (not mfma and self.block is not None and value.dtype in _FLOATS and bool(
+                lib.ctmi_hadamard_supported(int(self.block.shape[0]), n // int(self.block.shape[0]),
+                                            _lib.dtype_code(value.dtype)))):
+            big = (int(self.block.shape[0]), n // int(self.block.shape[0]))
+        plan = None if (mfma or big) else _kron_plan(n, self.block)
         if plan is not None and not (value.dtype in _FLOATS and bool(
                 lib.ctmi_kron_matmul_supported(plan[0], plan[1], _lib.dtype_code(value.dtype)))):
             plan = None
-        if not mfma and plan is None:
+        if not mfma and big is None and plan is None:
             # float64 values, or a run too long for LDS: the dense matrix and a library GEMM
             w = self.weight.to(value.device)
             if self.perm is not None:
@@ -642,6 +647,22 @@ class HadamardTransform(torch.nn.Module):
             x = blocks.index_select(-1, torch.argsort(p)).flatten(-2, -1)
         if mfma:
             y = hadamard_apply(x, n, sign_in=s_in, sign_out=s_out)
+        elif big is not None:
+            # x (Ma (x) S) with Ma = B^T for x W, B for x W^T; the kernel takes Ma^T
+            a, b = big
+            key = ("bf16", str(x.device), transposed)
+            if key not in self._factor:
+                m = self.block.to(device=x.device, dtype=torch.bfloat16)
+                self._factor[key] = (m.T if transposed else m).contiguous()
+            x = x.contiguous()
+            y = torch.empty_like(x)
+            sign = (lambda t: None if t is None else
+                    t.to(device=x.device, dtype=torch.float32).contiguous())
+            si, so = sign(s_in), sign(s_out)
+            _lib.check(lib.ctmi_hadamard_apply(
+                x.data_ptr(), y.data_ptr(), _lib.dtype_code(x.dtype), x.numel(), a, b,
+                self._factor[key].data_ptr(), _sylvester_bf16(b, x.device).data_ptr(),
+                _lib.ptr(si), _lib.ptr(so), _lib.stream_of(x.device)))
         else:
             # W = diag(q) (B^T (x) S):  x W = (x * q) (B^T (x) S);  x W^T = (x (B (x) S)) * q
             h, b = plan

@@ -640,12 +640,32 @@ hadamard_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const uint16_t* __res
 // exchanges, then each lane quantizes and packs its 2 x 8 values into two words.  jobs.out
 // is then the packed tensor, jobs.scale the group scales, jobs.rotated (optional) the
 // rotated tensor.
+//
+// A > 64 (224 x 64 = 14336, 224 x 32 = 7168: the reference's Hadamard matrices of size
+// K * 2^m with its known 224 x 224 block as Ma): a row is 112 registers a lane, so one wave
+// per SIMD, and Ma (100 KB in bf16) does not fit in registers: its fragments sit in LDS, in
+// the lanes' own layout, and are read at each use (one read serves the three products of
+// the split intermediate).
+template <int A, int B>
+struct KronLds {
+  static constexpr bool kBig = A > 64;
+  static constexpr int KS = B / 32, MT = A / 16, NT = B / 16, PS = A / 32, AT = A / 16;
+  static constexpr size_t sign_in = (size_t)MT * KS * kWave * 16;
+  static constexpr size_t sign_out = (size_t)AT * (NT / 2) * kWave * 16;
+  static constexpr size_t ma = kBig ? (size_t)AT * PS * kWave * 16 : 0;
+  static constexpr size_t bytes = sign_in + sign_out + ma;
+};
+
 template <int A, int B, bool HALF, bool MANY, bool QUANT = false>
-__global__ void __launch_bounds__(kKronThreads) __attribute__((amdgpu_waves_per_eu(CTMI_HAD_KRON_WAVES)))
+__global__ void __launch_bounds__(kKronThreads)
+__attribute__((amdgpu_waves_per_eu(A > 64 ? 1 : CTMI_HAD_KRON_WAVES)))
 hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ mbt,
                      const uint16_t* __restrict__ mat, const float* __restrict__ s_in,
                      const float* __restrict__ s_out, float inv_sqrt_n, QpCfg cfg) {
   static_assert(!QUANT || (B == 64 && !HALF), "the fused epilogue is written for 64-wide bf16 sub-rows");
+  static_assert(A % 32 == 0 && B % 32 == 0, "whole k steps");
+  constexpr bool BIG = KronLds<A, B>::kBig;
+  static_assert(!(BIG && QUANT), "the fused epilogue holds half rows back: not with A > 64");
   constexpr int N = A * B;
   constexpr int KS = B / 32;   // k steps of stage 1
   constexpr int MT = A / 16;   // sub-row tiles
@@ -661,8 +681,12 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
   // bfloat16 to float16 exactly); stage 2 works on the fp32 intermediate as before.
   using xfrag_t = typename std::conditional<HALF, f16x8_t, bf16x8_t>::type;
 
-  __shared__ u32x4_t sign_in_lds[MT * KS][kWave];
-  __shared__ u32x4_t sign_out_lds[AT * (NT / 2)][kWave];
+  extern __shared__ __align__(16) unsigned char kron_lds[];
+  typedef u32x4_t lane_row_t[kWave];
+  lane_row_t* sign_in_lds = reinterpret_cast<lane_row_t*>(kron_lds);
+  lane_row_t* sign_out_lds = reinterpret_cast<lane_row_t*>(kron_lds + KronLds<A, B>::sign_in);
+  lane_row_t* ma_lds = reinterpret_cast<lane_row_t*>(kron_lds + KronLds<A, B>::sign_in +
+                                                     KronLds<A, B>::sign_out);
   const bool signed_io = s_in || s_out;
   if (signed_io) {
     const uint32_t* pin = reinterpret_cast<const uint32_t*>(s_in ? (const void*)s_in : (const void*)mbt);
@@ -686,12 +710,18 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
         w[d] = (((pout[pos + 2 * d] >> 31) & use_out) << 15) | (((pout[pos + 2 * d + 1] >> 31) & use_out) << 31);
       sign_out_lds[f][lane] = w;
     }
-    __syncthreads();
   }
+  if constexpr (BIG) {
+    for (int f = wave; f < AT * PS; f += kKronWaves) {
+      const int at = f / PS, ps = f % PS;
+      ma_lds[f][lane] = *reinterpret_cast<const u32x4_t*>(mat + (16 * at + l16) * A + 32 * ps + 8 * lq);
+    }
+  }
+  if (signed_io || BIG) __syncthreads();
 
   // the two small matrices, as B operands
   xfrag_t mbf[NT][KS];
-  bf16x8_t maf[AT][PS];
+  bf16x8_t maf[BIG ? 1 : AT][BIG ? 1 : PS];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -706,12 +736,14 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
       }
       mbf[nt][ks] = __builtin_bit_cast(xfrag_t, m);
     }
+  if constexpr (!BIG) {
 #pragma unroll
-  for (int at = 0; at < AT; ++at)
+    for (int at = 0; at < AT; ++at)
 #pragma unroll
-    for (int ps = 0; ps < PS; ++ps)
-      maf[at][ps] = __builtin_bit_cast(
-          bf16x8_t, ldg<uint16_t, 8>(mat + (16 * at + l16) * A + 32 * ps + 8 * lq));
+      for (int ps = 0; ps < PS; ++ps)
+        maf[at][ps] = __builtin_bit_cast(
+            bf16x8_t, ldg<uint16_t, 8>(mat + (16 * at + l16) * A + 32 * ps + 8 * lq));
+  }
 
   const int64_t stride = (int64_t)gridDim.x * kKronWaves;
   for (int64_t row = (int64_t)blockIdx.x * kKronWaves + wave; row < n_rows; row += stride) {
@@ -727,7 +759,7 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
       packed = static_cast<int32_t*>(jobs.out[j]) + local * (N / 8);
       scale = static_cast<uint16_t*>(jobs.scale[j]) + local * (N / 128);
     }
-    u32x4_t held[B == 64 ? AT : 1];  // first halves of the output sub-rows
+    u32x4_t held[B == 64 && !BIG ? AT : 1];  // first halves of the output sub-rows
     xfrag_t xf[MT][KS];
 #pragma unroll
     for (int m = 0; m < MT; ++m)
@@ -785,12 +817,22 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
       for (int at = 0; at < AT; ++at) {
         f32x4_t y0 = {0.0f, 0.0f, 0.0f, 0.0f}, y1 = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int ps = 0; ps < PS; ++ps)
+        for (int ps = 0; ps < PS; ++ps) {
+          bf16x8_t mf;
+          if constexpr (BIG) {
+            // keeps the compiler from hoisting these (loop-invariant) LDS reads out of the
+            // row loop, back into hundreds of registers
+            asm volatile("" ::: "memory");
+            mf = __builtin_bit_cast(bf16x8_t, ma_lds[at * PS + ps][lane]);
+          } else {
+            mf = maf[at][ps];
+          }
 #pragma unroll
           for (int sp = NSPLIT - 1; sp >= 0; --sp) {  // small terms first
-            y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf[0][ps][sp], maf[at][ps], y0, 0, 0, 0);
-            y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf[1][ps][sp], maf[at][ps], y1, 0, 0, 0);
+            y0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf[0][ps][sp], mf, y0, 0, 0, 0);
+            y1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tf[1][ps][sp], mf, y1, 0, 0, 0);
           }
+        }
         u32x4_t o;
         if constexpr (HALF) {
 #pragma unroll
@@ -808,7 +850,7 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
         }
         if (signed_io) o ^= sign_out_lds[at * (NT / 2) + p][lane];
         uint16_t* at_dst = dst + (16 * at + l16) * B + 8 * lq;
-        if constexpr (B != 64) {
+        if constexpr (B != 64 || BIG) {
           stg<uint16_t, 8>(at_dst + 32 * p, __builtin_bit_cast(Vec<uint16_t, 8>, o));
         } else if (p == 0) {
           held[at] = o;
@@ -857,16 +899,24 @@ template <int A, int B, bool HALF>
 static int launch_had_kron_jobs(const HadJobs& jobs, int n_jobs, const HadArgs& a, hipStream_t st) {
   const int64_t n_rows = jobs.end[n_jobs - 1];
   const int64_t wgs = cdiv(n_rows, kKronWaves);
-  // as many workgroups as are resident at once (register-limited)
-  const int64_t cap = 256 * 4 * (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES)) / kKronWaves;
+  // as many workgroups as are resident at once (register-limited; one wave per SIMD for A > 64)
+  const int waves = A > 64 ? 1 : (A * B <= 1024 ? 8 : (A * B <= 2048 ? 4 : CTMI_HAD_KRON_WAVES));
+  const int64_t cap = 256 * 4 * waves / kKronWaves;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
   const QpCfg none{};
-  if (n_jobs == 1)
-    hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF, false>), grid, kKronThreads, 0, st, jobs, n_rows,
-                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, none);
-  else
-    hipLaunchKernelGGL((hadamard_kron_kernel<A, B, HALF, true>), grid, kKronThreads, 0, st, jobs, n_rows,
-                       a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, none);
+  constexpr size_t lds = KronLds<A, B>::bytes;
+  auto one = hadamard_kron_kernel<A, B, HALF, false>;
+  auto many = hadamard_kron_kernel<A, B, HALF, true>;
+  auto kern = n_jobs == 1 ? one : many;
+  if (lds > 48 * 1024) {
+    // the attribute belongs to the kernel as loaded on one device; setting it again is cheap
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess)
+      return set_error(CTMI_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  hipLaunchKernelGGL(kern, grid, kKronThreads, lds, st, jobs, n_rows, a.mbt, a.mat, a.s_in, a.s_out,
+                     1.0f / a.sqrt_n, none);
   return CTMI_OK;
 }
 
@@ -878,11 +928,12 @@ static int launch_had_kron_quant_jobs(const HadJobs& jobs, int n_jobs, const Had
   const int64_t wgs = cdiv(n_rows, kKronWaves);
   const int64_t cap = 256 * 4 * (A * 64 <= 2048 ? 4 : CTMI_HAD_KRON_WAVES) / kKronWaves;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
+  constexpr size_t lds = KronLds<A, 64>::bytes;
   if (n_jobs == 1)
-    hipLaunchKernelGGL((hadamard_kron_kernel<A, 64, false, false, true>), grid, kKronThreads, 0, st,
+    hipLaunchKernelGGL((hadamard_kron_kernel<A, 64, false, false, true>), grid, kKronThreads, lds, st,
                        jobs, n_rows, a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, cfg);
   else
-    hipLaunchKernelGGL((hadamard_kron_kernel<A, 64, false, true, true>), grid, kKronThreads, 0, st,
+    hipLaunchKernelGGL((hadamard_kron_kernel<A, 64, false, true, true>), grid, kKronThreads, lds, st,
                        jobs, n_rows, a.mbt, a.mat, a.s_in, a.s_out, 1.0f / a.sqrt_n, cfg);
   return CTMI_OK;
 }
@@ -929,7 +980,8 @@ static int dispatch_had(int a_dim, int b_dim, const HadArgs& a, hipStream_t st) 
 static bool had_in_registers(int io_dtype, int a_dim, int b_dim) {
   if (io_dtype != CTMI_BF16 && io_dtype != CTMI_F16) return false;
   if (a_dim == 1) return b_dim == 32 || b_dim == 64 || b_dim == 128;
-  return (a_dim == 32 && (b_dim == 32 || b_dim == 64)) || (a_dim == 64 && b_dim == 64);
+  return (a_dim == 32 && (b_dim == 32 || b_dim == 64)) || (a_dim == 64 && b_dim == 64) ||
+         (a_dim == 224 && (b_dim == 32 || b_dim == 64));
 }
 
 static int launch_had_jobs(const HadJobs& jobs, int n_jobs, int io_dtype, int a_dim, int b_dim,
@@ -941,6 +993,7 @@ static int launch_had_jobs(const HadJobs& jobs, int n_jobs, int io_dtype, int a_
                                 : launch_had_kron_jobs<AA, BB, false>(jobs, n_jobs, a, st))
   if (a_dim == 1) return b_dim == 32 ? CTMI_ROWS(32) : (b_dim == 64 ? CTMI_ROWS(64) : CTMI_ROWS(128));
   if (a_dim == 32) return b_dim == 32 ? CTMI_KRON(32, 32) : CTMI_KRON(32, 64);
+  if (a_dim == 224) return b_dim == 32 ? CTMI_KRON(224, 32) : CTMI_KRON(224, 64);
   return CTMI_KRON(64, 64);
 #undef CTMI_ROWS
 #undef CTMI_KRON
@@ -951,6 +1004,8 @@ static int launch_had_jobs(const HadJobs& jobs, int n_jobs, int io_dtype, int a_
 using namespace ctmi;
 
 extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
+  // 224 x 32 and 224 x 64 (7168 and 14336, Ma any +-1 matrix of order 224): 16-bit tensors
+  if (a_dim == 224 && (b_dim == 32 || b_dim == 64)) return io_dtype == CTMI_BF16 || io_dtype == CTMI_F16;
   const bool pair = (a_dim == 1 && (b_dim == 32 || b_dim == 64 || b_dim == 128)) ||
                     (a_dim == 32 && (b_dim == 32 || b_dim == 64)) ||
                     (a_dim == 64 && (b_dim == 64 || b_dim == 128));

@@ -339,7 +339,7 @@ def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
     assert rc == _lib.CTMI_ERR_UNSUPPORTED  # 512 lanes only for the Sylvester factor
 
 
-@pytest.mark.parametrize("size", [768, 1600, 14336, 32, 256, 512, 16])
+@pytest.mark.parametrize("size", [768, 1600, 7168, 14336, 32, 256, 512, 16])
 @pytest.mark.parametrize("location,inverse", [("input", False), ("weight_input", True),
                                               ("weight_output", False), ("output", True)])
 def test_random_hadamard_of_any_table_size(size, location, inverse, gpu, hadamard_table_path):
@@ -398,3 +398,38 @@ def test_apply_transform_weight_runs_the_kernel(location, module_type, gpu, monk
     assert calls, "the HIP kernel was not used"
     want = oh.apply_transform_weight(w.double(), value.double(), location, module_type).bfloat16()
     _assert_within_ulp(got, want, f"{location} {module_type.__name__}")
+
+
+@pytest.mark.parametrize("b", [32, 64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_blocks):
+    """ctmi_hadamard_apply for 224 x 32 and 224 x 64 (7168, 14336) straight through the C ABI:
+    x diag(s_in) (Ma (x) Sylvester(b)) diag(s_out) / sqrt(n) against fp64, Ma the known
+    Hadamard matrix of order 224 and a random +-1 matrix; more rows than workgroups hold at
+    a time, and a count that leaves the last workgroup's waves without a row"""
+    from compressed_tensors_amd import _lib
+
+    announce("hadamard_apply 224 x", b, dtype)
+    n = 224 * b
+    g = torch.Generator().manual_seed(b)
+    rows = 1027
+    x = torch.randn(rows, n, generator=g).to(dtype)
+    s_in = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    s_out = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
+    mb = oh.deterministic_hadamard_matrix(b, torch.bfloat16).to(gpu)
+    sample = torch.tensor([0, 1, 255, 256, 511, 1023, 1024, 1026])
+    for ma in (hadamard_blocks[224].double(), (torch.randint(0, 2, (224, 224), generator=g) * 2 - 1).double()):
+        dense = torch.kron(ma, oh.deterministic_hadamard_matrix(b, torch.float64))
+        ma_t = ma.T.contiguous().bfloat16().to(gpu)
+        xg = x.to(gpu)
+        for si, so in ((None, None), (s_in, None), (None, s_out)):
+            out = torch.empty_like(xg)
+            sig, sog = (None if t is None else t.to(gpu) for t in (si, so))
+            _lib.check(ctmi.ctmi_hadamard_apply(xg.data_ptr(), out.data_ptr(), _lib.dtype_code(dtype), xg.numel(),
+                                                224, b, ma_t.data_ptr(), mb.data_ptr(), _lib.ptr(sig),
+                                                _lib.ptr(sog), _lib.stream_of(gpu)))
+            xs = x[sample].double() * (1.0 if si is None else si.double())
+            want = xs @ dense * (1.0 if so is None else so.double()) / n ** 0.5
+            _assert_within_ulp(out[sample.to(gpu)], want.to(dtype), f"signs in={si is not None} out={so is not None}")
+    assert ctmi.ctmi_hadamard_supported(224, 64, _lib.dtype_code(torch.float32)) == 0
+    assert ctmi.ctmi_hadamard_supported(224, 128, _lib.dtype_code(torch.bfloat16)) == 0
