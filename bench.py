@@ -569,6 +569,25 @@ def other_workload(torch, name, seed):
                                   [lambda m=m: _lib.check(lib.ctmi_hadamard_apply_many(*m))], nb,
                                   "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
                                   mfma_flops=flops))
+        # 14336 = 224 x 64: a known Hadamard matrix of order 224 (here: any +-1 matrix, the kernel's
+        # work does not depend on the entries) times Sylvester(64), as the reference builds the
+        # rotation in front of Llama-3's down projections
+        xs14 = [randn(4096, 14336) for _ in range(5)]
+        ma224 = (torch.randint(0, 2, (224, 224), generator=torch.Generator().manual_seed(seed)) * 2 - 1
+                 ).bfloat16().to(dev).contiguous()
+        mb64 = deterministic_hadamard_matrix(64, torch.bfloat16, dev).contiguous()
+        q14 = (torch.randint(0, 2, (14336,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
+        keep.extend([ma224, mb64, q14])
+        calls = []
+        for x in xs14:
+            out = torch.empty_like(x)
+            keep.extend([x, out])
+            a = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), 224, 64, ma224.data_ptr(),
+                 mb64.data_ptr(), q14.data_ptr(), None, st)
+            calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
+        ops.append(Op("random-sign Hadamard, size 14336 = 224 x 64: activations 4096x14336 (x5)", calls,
+                      sum(4 * x.numel() for x in xs14), "hadamard_kron_kernel", primary=False,
+                      mfma_flops=sum((2 * 64 + 6 * 224) * x.numel() for x in xs14)))
         # rotation (block 128) + symmetric int4 group-128 quantization + pack_to_int32, one pass
         mb = deterministic_hadamard_matrix(128, torch.bfloat16, dev).contiguous()
         q = (torch.randint(0, 2, (128,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
@@ -720,6 +739,10 @@ def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True):
     slow = max((op for op in ops if op.primary), key=lambda op: op.ms)
     n_launch = len(slow.calls)
     traffic, traffic_source = measured_traffic(workload, slow.kernel)
+    if traffic is None and (PROFILES / "all_workloads_pmc_traffic.txt").exists():
+        # one kernel serves launches of many sizes here: the counters are listed per kernel and
+        # grid size in that file instead of as one figure per launch
+        traffic_source = "profiles/all_workloads_pmc_traffic.txt (FETCH_SIZE / WRITE_SIZE per kernel and grid size)"
 
     def op_row(op):
         row = {"name": op.name, "kernel": op.kernel, "GBs": op.nbytes / (op.ms * 1e-3) / 1e9,
