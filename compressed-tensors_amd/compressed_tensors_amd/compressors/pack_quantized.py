@@ -245,7 +245,8 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         scale = to_gpu(compressed_data["weight_scale"])
         zero_point = to_gpu(compressed_data.get("weight_zero_point", None))
         g_idx = to_gpu(compressed_data.get("weight_g_idx", None))
-        shape = torch.Size(int(d) for d in compressed_data["weight_shape"])
+        ws = compressed_data["weight_shape"]
+        shape = torch.Size(ws.flatten().tolist() if isinstance(ws, Tensor) else [int(d) for d in ws])
         num_bits = args.num_bits
         if packed.dtype is not torch.int32:
             raise ValueError(f"Expected {torch.int32} but got {packed.dtype}, Aborting unpack.")
@@ -300,7 +301,8 @@ def _decompress_weights_batched(self, items) -> list:
         scale = to_gpu(data["weight_scale"])
         zero_point = to_gpu(data.get("weight_zero_point", None))
         g_idx = to_gpu(data.get("weight_g_idx", None))
-        shape = torch.Size(int(d) for d in data["weight_shape"])
+        ws = data["weight_shape"]
+        shape = torch.Size(ws.flatten().tolist() if isinstance(ws, Tensor) else [int(d) for d in ws])
         if packed.dtype is not torch.int32:
             raise ValueError(f"Expected {torch.int32} but got {packed.dtype}, Aborting unpack.")
         if args.num_bits > 8:

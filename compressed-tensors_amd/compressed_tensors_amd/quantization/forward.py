@@ -8,6 +8,7 @@ separate torch ops; here the strategy is reduced to a scale-grid description
 (`QParams`) and one HIP kernel replays the whole chain per element.
 """
 import ctypes
+import functools
 import math
 from typing import Optional, Tuple
 
@@ -46,6 +47,11 @@ def _rows_cols(x) -> Tuple[int, int]:
 def _leading_grid(x_shape, s_shape) -> Tuple[int, int]:
     """Map the broadcast of scale dims over x's leading dims to
     (s_rows, blk_rows): scale row of flattened x row r = (r // blk_rows) % s_rows."""
+    return _leading_grid_of(tuple(x_shape), tuple(s_shape))
+
+
+@functools.lru_cache(maxsize=4096)
+def _leading_grid_of(x_shape: tuple, s_shape: tuple) -> Tuple[int, int]:
     lead = list(x_shape[:-1])
     s_lead = list(s_shape)
     if len(s_lead) > len(lead):
@@ -296,8 +302,23 @@ def quantize(
     return _run(x, scale, zero_point, args, True, False, dtype, g_idx, global_scale)
 
 
+_inferred: dict = {}
+
+
 def infer_dequant_args(x_q: torch.Tensor, scale: torch.Tensor) -> QuantizationArgs:
-    """strategy inference of `dequantize(args=None)`, forward.py:107-138"""
+    """strategy inference of `dequantize(args=None)`, forward.py:107-138.  The result
+    depends on the two shapes only and is read, never changed: one object per pair of
+    shapes (a model has a handful of them and hundreds of weights)."""
+    key = (tuple(x_q.shape), tuple(scale.shape))
+    args = _inferred.get(key)
+    if args is None:
+        if len(_inferred) > 4096:
+            _inferred.clear()
+        args = _inferred[key] = _infer_dequant_args(x_q, scale)
+    return args
+
+
+def _infer_dequant_args(x_q, scale) -> QuantizationArgs:
     if scale.ndim in (0, 1):
         return QuantizationArgs(strategy=QuantizationStrategy.TENSOR)
     if scale.ndim == 2:
