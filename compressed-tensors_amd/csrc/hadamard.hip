@@ -649,10 +649,14 @@ hadamard_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const uint16_t* __res
 template <int A, int B>
 struct KronLds {
   static constexpr bool kBig = A > 64;
+#ifndef CTMI_HAD_KRON_MA_LDS_FROM
+#define CTMI_HAD_KRON_MA_LDS_FROM 65  // smallest A whose Ma is read from LDS instead of registers
+#endif
+  static constexpr bool kMaLds = A >= CTMI_HAD_KRON_MA_LDS_FROM;
   static constexpr int KS = B / 32, MT = A / 16, NT = B / 16, PS = A / 32, AT = A / 16;
   static constexpr size_t sign_in = (size_t)MT * KS * kWave * 16;
   static constexpr size_t sign_out = (size_t)AT * (NT / 2) * kWave * 16;
-  static constexpr size_t ma = kBig ? (size_t)AT * PS * kWave * 16 : 0;
+  static constexpr size_t ma = kMaLds ? (size_t)AT * PS * kWave * 16 : 0;
   static constexpr size_t bytes = sign_in + sign_out + ma;
 };
 
@@ -665,6 +669,7 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
   static_assert(!QUANT || (B == 64 && !HALF), "the fused epilogue is written for 64-wide bf16 sub-rows");
   static_assert(A % 32 == 0 && B % 32 == 0, "whole k steps");
   constexpr bool BIG = KronLds<A, B>::kBig;
+  constexpr bool MA_LDS = KronLds<A, B>::kMaLds;
   static_assert(!(BIG && QUANT), "the fused epilogue holds half rows back: not with A > 64");
   constexpr int N = A * B;
   constexpr int KS = B / 32;   // k steps of stage 1
@@ -711,17 +716,17 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
       sign_out_lds[f][lane] = w;
     }
   }
-  if constexpr (BIG) {
+  if constexpr (MA_LDS) {
     for (int f = wave; f < AT * PS; f += kKronWaves) {
       const int at = f / PS, ps = f % PS;
       ma_lds[f][lane] = *reinterpret_cast<const u32x4_t*>(mat + (16 * at + l16) * A + 32 * ps + 8 * lq);
     }
   }
-  if (signed_io || BIG) __syncthreads();
+  if (signed_io || MA_LDS) __syncthreads();
 
   // the two small matrices, as B operands
   xfrag_t mbf[NT][KS];
-  bf16x8_t maf[BIG ? 1 : AT][BIG ? 1 : PS];
+  bf16x8_t maf[MA_LDS ? 1 : AT][MA_LDS ? 1 : PS];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -736,7 +741,7 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
       }
       mbf[nt][ks] = __builtin_bit_cast(xfrag_t, m);
     }
-  if constexpr (!BIG) {
+  if constexpr (!MA_LDS) {
 #pragma unroll
     for (int at = 0; at < AT; ++at)
 #pragma unroll
@@ -819,7 +824,7 @@ hadamard_kron_kernel(HadJobs jobs, int64_t n_rows, const uint16_t* __restrict__ 
 #pragma unroll
         for (int ps = 0; ps < PS; ++ps) {
           bf16x8_t mf;
-          if constexpr (BIG) {
+          if constexpr (MA_LDS) {
             // keeps the compiler from hoisting these (loop-invariant) LDS reads out of the
             // row loop, back into hundreds of registers
             asm volatile("" ::: "memory");
