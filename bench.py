@@ -421,7 +421,7 @@ def other_workload(torch, name, seed):
                                 group_size=16)
         ops = []
         for r, c in ((14336, 4096), (4096, 14336)):
-            c_calls, d_calls = [], []
+            c_calls, d_calls, many_c, many_d = [], [], [], []
             n_copies = 16  # the packed side (33 MB a copy) has to exceed the 256 MB last-level cache too
             for _ in range(n_copies):
                 w = randn(r, c, 0.02)
@@ -436,9 +436,22 @@ def other_workload(torch, name, seed):
                 da = (packed.data_ptr(), dense.data_ptr(), code(dense.dtype), r, c, ctypes.byref(dp.qp), st)
                 c_calls.append(lambda ca=ca: _lib.check(lib.ctmi_nvfp4_compress(*ca)))
                 d_calls.append(lambda da=da: _lib.check(lib.ctmi_nvfp4_decompress(*da)))
+                many_c.append((w.data_ptr(), packed.data_ptr(), code(w.dtype), cp))
+                many_d.append((packed.data_ptr(), dense.data_ptr(), code(dense.dtype), dp))
             nbytes = n_copies * (2 * r * c + r * c // 16 + r * c // 2)
             ops += [Op(f"nvfp4 compress {r}x{c} (x{n_copies})", c_calls, nbytes, "nvfp4_compress_vec_kernel"),
                     Op(f"nvfp4 decompress {r}x{c} (x{n_copies})", d_calls, nbytes, "nvfp4_decompress_vec_kernel")]
+            # the same tensors through the multi-weight entry points (what the compressor's
+            # state-dict path calls): 8 per launch
+            for many, entry, kernel, what in ((many_c, lib.ctmi_nvfp4_compress_many, "nvfp4_compress_chain_kernel", "compress"),
+                                              (many_d, lib.ctmi_nvfp4_decompress_many, "nvfp4_decompress_chain_kernel", "decompress")):
+                jobs = (_lib.WeightJob * len(many))()
+                for job, (src, dst, dt, plan) in zip(jobs, many):
+                    job.src, job.dst, job.rows, job.cols, job.dense_dtype, job.qp = src, dst, r, c, dt, plan.qp
+                keep.append(jobs)
+                m = (jobs, len(many), st)
+                ops.append(Op(f"nvfp4 {what} {r}x{c} (x{n_copies}), one call (8 per launch)",
+                              [lambda m=m, entry=entry: _lib.check(entry(*m))], nbytes, kernel))
         # the Llama-3-8B-shaped set: one call per weight against all 224 in one call
         from compressed_tensors_amd.compressors import Fp4WeightBatch
         entries, single_c, single_d, n_set = [], [], [], 0
