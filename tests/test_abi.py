@@ -215,3 +215,66 @@ def test_product_refuses_cpu_tensors():
     s = torch.ones(1, dtype=torch.bfloat16)
     with pytest.raises(RuntimeError, match="GPU"):
         quantize(x, s, None, QuantizationArgs(num_bits=4))
+
+
+def test_transform_and_block_entry_point_errors(ctmi):
+    """the entry points for explicit transform factors, the fused full-width rotation and the
+    block-strategy one-shot: refused on the host, whatever device there is"""
+    # ctmi_kron_matmul: what fits, and sizes that do not divide the tensor
+    assert ctmi.ctmi_kron_matmul_supported(224, 64, _lib.BF16) == 1
+    assert ctmi.ctmi_kron_matmul_supported(1, 512, _lib.F32) == 1
+    assert ctmi.ctmi_kron_matmul_supported(12, 3, _lib.BF16) == 0
+    assert ctmi.ctmi_kron_matmul_supported(12, 64, _lib.I8) == 0
+    rc = ctmi.ctmi_kron_matmul(0x1000, 0x2000, _lib.BF16, 100, 12, 2, 0x3000, None, None, 1, 1.0, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "multiple of the transform size" in _err(ctmi)
+    rc = ctmi.ctmi_kron_matmul(0x1000, 0x2000, _lib.BF16, 1024, 1, 512, 0x3000, None, None, 0, 1.0, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "Sylvester" in _err(ctmi)
+    rc = ctmi.ctmi_kron_matmul(0x1000, 0x2000, _lib.BF16, 24, 12, 2, None, None, None, 1, 1.0, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "NULL tensor pointer" in _err(ctmi)
+    assert ctmi.ctmi_kron_matmul(None, None, _lib.BF16, 0, 12, 2, None, None, None, 1, 1.0, None) == _lib.CTMI_OK
+    rc = ctmi.ctmi_block_matmul(0x1000, 0x2000, _lib.BF16, 400 * 4, 400, 0x3000, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED
+    # matrix-core factorisations: 224 x 32 / 64 for 16-bit tensors only
+    assert ctmi.ctmi_hadamard_supported(224, 64, _lib.BF16) == 1
+    assert ctmi.ctmi_hadamard_supported(224, 32, _lib.F16) == 1
+    assert ctmi.ctmi_hadamard_supported(224, 64, _lib.F32) == 0
+    assert ctmi.ctmi_hadamard_supported(224, 128, _lib.BF16) == 0
+    # fused rotation of 2048 / 4096 + groups of 128
+    pj = (_lib.HadamardPackJob * 1)()
+    pj[0].x, pj[0].packed, pj[0].scale, pj[0].numel = 0x1000, 0x2000, 0x3000, 4096
+    call = ctmi.ctmi_hadamard_kron_quant_pack_many
+    assert call(pj, 1, _lib.BF16, 64, 128, 0x4000, 0x5000, None, None, 128, 4, 1, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert call(pj, 1, _lib.BF16, 64, 64, 0x4000, 0x5000, None, None, 64, 4, 1, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert "group size" in _err(ctmi)
+    assert call(pj, 1, _lib.F16, 64, 64, 0x4000, 0x5000, None, None, 128, 4, 1, None) == _lib.CTMI_ERR_UNSUPPORTED
+    pj[0].numel = 4000
+    rc = call(pj, 1, _lib.BF16, 64, 64, 0x4000, 0x5000, None, None, 128, 4, 1, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "not a multiple of the transform size" in _err(ctmi)
+    pj[0].numel = 4096
+    rc = call(pj, 1, _lib.BF16, 64, 64, None, 0x5000, None, None, 128, 4, 1, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "matrices" in _err(ctmi)
+    assert call(None, 0, _lib.BF16, 64, 64, None, None, None, None, 128, 4, 1, None) == _lib.CTMI_OK
+    # one-shot block strategy
+    ok = ctmi.ctmi_observe_quantize_blocks_supported
+    assert ok(_lib.BF16, 256, 512, 128, 128, _lib.QTYPE_FLOAT, 8) == 1
+    assert ok(_lib.BF16, 256, 512, 256, 128, _lib.QTYPE_FLOAT, 8) == 0   # 32768 elements a block
+    assert ok(_lib.BF16, 250, 512, 128, 128, _lib.QTYPE_FLOAT, 8) == 0   # blocks must tile the tensor
+    assert ok(_lib.BF16, 256, 512, 128, 12, _lib.QTYPE_FLOAT, 8) == 0    # 8 columns at a time
+    assert ok(_lib.BF16, 256, 512, 128, 128, _lib.QTYPE_FLOAT, 4) == 0
+    rc = ctmi.ctmi_observe_quantize_blocks(0x1000, _lib.BF16, 0x2000, 250, 512, 128, 128, _lib.QTYPE_FLOAT, 8, 1,
+                                           0x3000, _lib.BF16, None, _lib.F8E4M3, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "tile the tensor" in _err(ctmi)
+    rc = ctmi.ctmi_observe_quantize_blocks(0x1000, _lib.BF16, None, 256, 512, 128, 128, _lib.QTYPE_FLOAT, 8, 1,
+                                           0x3000, _lib.BF16, None, _lib.F8E4M3, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "NULL tensor pointer" in _err(ctmi)
+    # nvfp4 one-shot, several weights: groups of 16 columns, every job checked first
+    oj = (_lib.ObserveNvfp4Job * 2)()
+    for j, cols in zip(oj, (64, 40)):
+        j.x, j.global_scale, j.packed, j.scale = 0x1000, 0x2000, 0x3000, 0x4000
+        j.rows, j.cols, j.x_dtype = 4, cols, _lib.BF16
+    rc = ctmi.ctmi_observe_nvfp4_compress_many(oj, 2, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "job 1" in _err(ctmi)
+    oj[1].cols, oj[1].scale = 64, None
+    rc = ctmi.ctmi_observe_nvfp4_compress_many(oj, 2, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "job 1" in _err(ctmi)
+    assert ctmi.ctmi_observe_nvfp4_compress_many(None, 0, None) == _lib.CTMI_OK
