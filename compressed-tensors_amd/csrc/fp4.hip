@@ -313,23 +313,107 @@ __device__ __forceinline__ uint32_t nvfp4_codes_fast(const Vec<typename XT::raw,
 // range.  So for a tame scale (2^-60 <= s < 2^12) and 2^-30 <= |x| < 2^30 (or x == 0)
 // q2 is bit for bit the reference's x / s, at a third of the cost of the general
 // division; anything else clears *ok and takes nvfp4_codes_exact.
+__device__ __forceinline__ float nvfp4_quotient_divided(float x, const Fp4Scale& e, bool* fine) {
+  const uint32_t mag = __float_as_uint(x) & 0x7fffffffu;
+  *fine &= (mag - 0x30800000u) < (0x4e800000u - 0x30800000u) || mag == 0;
+  const float q0 = x * e.y;
+  const float q1 = __builtin_fmaf(__builtin_fmaf(-e.s, q0, x), e.y, q0);
+  const float q2 = __builtin_fmaf(__builtin_fmaf(-e.s, q1, x), e.y, q1);
+  return q2 + 0.0f;  // an exact zero loses its sign, as in the reference's sign(0) = 0
+}
+
 template <typename XT>
 __device__ __forceinline__ uint32_t nvfp4_codes_divided(const Vec<typename XT::raw, 8>& xv,
                                                         const Fp4Scale& e, bool* ok) {
   float q[8];
   bool fine = e.r == e.r;  // a tame scale
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float x = XT::to_f32(xv.v[i]);
-    const uint32_t mag = __float_as_uint(x) & 0x7fffffffu;
-    fine &= (mag - 0x30800000u) < (0x4e800000u - 0x30800000u) || mag == 0;
-    const float q0 = x * e.y;
-    const float q1 = __builtin_fmaf(__builtin_fmaf(-e.s, q0, x), e.y, q0);
-    const float q2 = __builtin_fmaf(__builtin_fmaf(-e.s, q1, x), e.y, q1);
-    q[i] = q2 + 0.0f;  // an exact zero loses its sign, as in the reference's sign(0) = 0
-  }
+  for (int i = 0; i < 8; ++i) q[i] = nvfp4_quotient_divided(XT::to_f32(xv.v[i]), e, &fine);
   *ok &= fine;
   return fp4_pack8_hw(q);
+}
+
+// Who does the second tier.  In a tensor whose quotients hit boundaries systematically
+// three elements in two thousand are in doubt, but that is one or two in nearly every
+// wavefront, and a wavefront that redoes all its vectors for them doubles its arithmetic.
+// So the lanes that hold a doubtful vector put it into a queue of their wavefront in
+// LDS, and the queue is worked through four lanes to a vector (a lane takes two elements
+// and produces one byte of codes): sixteen vectors cost what one cost before.  The
+// owners then take their four bytes back.  Nothing here leaves the wavefront: LDS
+// instructions of one wavefront execute in order, so all it needs is that the compiler
+// keeps the order as well.
+constexpr int kFp4RedoCap = 32;  // vectors per wavefront; beyond that every lane redoes its own
+
+template <typename XT>
+struct Fp4Redo {
+  Vec<typename XT::raw, 8> x[kFp4RedoCap];
+  uint32_t sraw[kFp4RedoCap];
+  uint32_t codes[kFp4RedoCap];
+};
+
+__device__ __forceinline__ void lds_in_order() { asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory"); }
+
+// false: not done here (too many doubtful vectors, or one outside the range the
+// division-free sequence covers); codes[] is then untouched or partly replaced by
+// equally valid codes of vectors that were fine
+template <typename XT, int U>
+__device__ __forceinline__ bool nvfp4_redo_doubtful(const Vec<typename XT::raw, 8>* xv,
+                                                    const uint8_t* sraw, const bool* okk,
+                                                    uint32_t* codes, const Fp4Scale* lut,
+                                                    Fp4Redo<XT>& q) {
+  const uint32_t lane = threadIdx.x & 63u;
+  uint32_t count = 0, slot[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint64_t m = __builtin_amdgcn_ballot_w64(!okk[k]);
+    slot[k] = count + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u));
+    count += (uint32_t)__builtin_popcountll(m);
+  }
+  if (count > (uint32_t)kFp4RedoCap) return false;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    if (!okk[k]) {
+      q.x[slot[k]] = xv[k];
+      q.sraw[slot[k]] = sraw[k];
+    }
+  }
+  lds_in_order();
+  bool fine = true;
+  for (uint32_t base = 0; base < count; base += 16) {
+    const uint32_t e = base + (lane >> 2), pair = lane & 3u;
+    if (e < count) {
+      const Fp4Scale sc = lut[q.sraw[e]];
+      fine &= sc.r == sc.r;
+      const typename XT::raw* px = reinterpret_cast<const typename XT::raw*>(&q.x[e]) + 2 * pair;
+      const float qa = nvfp4_quotient_divided(XT::to_f32(px[0]), sc, &fine);
+      const float qb = nvfp4_quotient_divided(XT::to_f32(px[1]), sc, &fine);
+      reinterpret_cast<uint8_t*>(&q.codes[e])[pair] =
+          (uint8_t)__builtin_amdgcn_cvt_scalef32_pk_fp4_f32(0u, qa, qb, 1.0f, 0);
+    }
+  }
+  lds_in_order();
+  if (!wave_all(fine)) return false;
+#pragma unroll
+  for (int k = 0; k < U; ++k)
+    if (!okk[k]) codes[k] = q.codes[slot[k]];
+  return true;
+}
+
+// The codes of a wavefront's U vectors once the fast path has flagged some of them
+// (okk[k] false): the queue above, else the division-free sequence for every vector,
+// else exact divisions.
+template <typename XT, int U>
+__device__ __forceinline__ void nvfp4_settle_codes(const Vec<typename XT::raw, 8>* xv,
+                                                   const uint8_t* sraw, const bool* okk,
+                                                   uint32_t* codes, const Fp4Scale* lut,
+                                                   Fp4Redo<XT>* redo) {
+  if (nvfp4_redo_doubtful<XT, U>(xv, sraw, okk, codes, lut, redo[threadIdx.x >> 6])) return;
+  bool ok = true;
+#pragma unroll
+  for (int k = 0; k < U; ++k) codes[k] = nvfp4_codes_divided<XT>(xv[k], lut[sraw[k]], &ok);
+  if (wave_all(ok)) return;
+#pragma unroll
+  for (int k = 0; k < U; ++k) codes[k] = nvfp4_codes_exact<XT, false>(xv[k], lut[sraw[k]].s, 0.0f);
 }
 
 template <typename XT, bool HAS_ZP>
@@ -339,6 +423,7 @@ nvfp4_compress_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t*
                           uint32_t* __restrict__ out, VecGeom g) {
   constexpr int B = kFp4Block, U = kFp4Unroll;
   __shared__ Fp4Scale lut[256];
+  __shared__ Fp4Redo<XT> redo[B / 64];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
@@ -357,40 +442,43 @@ nvfp4_compress_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t*
         sraw[k] = scale[si[k]];
         if constexpr (HAS_ZP) zraw[k] = zp[si[k]];
       } else {
+        xv[k] = {};
         sraw[k] = 0;
+        if constexpr (HAS_ZP) zraw[k] = 0;
       }
     }
     build_scale_lut(lut, gs);
-    bool ok = true;
+    bool okk[U], plain = true;
+    uint32_t codes[U];
 #pragma unroll
     for (int k = 0; k < U; ++k) {
-      const uint32_t v = v0 + k * B;
-      if (!GUARD || v < g.nvec) {
+      okk[k] = true;
+      if (!GUARD || v0 + k * B < g.nvec) {
         // a zero point of zero (what symmetric schemes carry) only turns -0 into +0, which
         // the fast path does as well; any other takes the exact path
-        if constexpr (HAS_ZP) ok &= (zraw[k] & 0x7f) == 0;
-        __builtin_nontemporal_store(nvfp4_codes_fast<XT>(xv[k], lut[sraw[k]], &ok), out + v);
+        if constexpr (HAS_ZP) plain &= (zraw[k] & 0x7f) == 0;
+        codes[k] = nvfp4_codes_fast<XT>(xv[k], lut[sraw[k]], &okk[k]);
       }
     }
-    if (__builtin_expect(wave_all(ok), 1)) return;
-    ok = true;
+    bool ok = plain;
+#pragma unroll
+    for (int k = 0; k < U; ++k) ok &= okk[k];
+    if (__builtin_expect(!wave_all(ok), 0)) {
+      if (!HAS_ZP || wave_all(plain)) {
+        nvfp4_settle_codes<XT, U>(xv, sraw, okk, codes, lut, redo);
+      } else {
+#pragma unroll
+        for (int k = 0; k < U; ++k) {
+          // zero_point.to(x.dtype): an fp8 value is exact in every wider float type
+          const float z = HAS_ZP ? __builtin_amdgcn_cvt_f32_fp8((int)zraw[k], 0) : 0.0f;
+          codes[k] = nvfp4_codes_exact<XT, HAS_ZP>(xv[k], lut[sraw[k]].s, z);
+        }
+      }
+    }
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
-      if (!GUARD || v < g.nvec) {
-        if constexpr (HAS_ZP) ok &= (zraw[k] & 0x7f) == 0;
-        out[v] = nvfp4_codes_divided<XT>(xv[k], lut[sraw[k]], &ok);
-      }
-    }
-    if (wave_all(ok)) return;
-#pragma unroll
-    for (int k = 0; k < U; ++k) {
-      const uint32_t v = v0 + k * B;
-      if (!GUARD || v < g.nvec) {
-        // zero_point.to(x.dtype): an fp8 value is exact in every wider float type
-        const float z = HAS_ZP ? __builtin_amdgcn_cvt_f32_fp8((int)zraw[k], 0) : 0.0f;
-        out[v] = nvfp4_codes_exact<XT, HAS_ZP>(xv[k], lut[sraw[k]].s, z);
-      }
+      if (!GUARD || v < g.nvec) __builtin_nontemporal_store(codes[k], out + v);
     }
   };
   if (full) body(std::false_type{});
@@ -459,6 +547,7 @@ __global__ void __launch_bounds__(kFp4Block) nvfp4_compress_chain_kernel(ChainTa
   const uint32_t v0 = local * (B * U) + threadIdx.x;
   const bool full = (local + 1) * (uint32_t)(B * U) <= nvec;
   __shared__ Fp4Scale lut[256];
+  __shared__ Fp4Redo<XT> redo[B / 64];
   auto body = [&](auto guard) {
     constexpr bool GUARD = decltype(guard)::value;
     Vec<typename XT::raw, 8> xv[U];
@@ -470,29 +559,24 @@ __global__ void __launch_bounds__(kFp4Block) nvfp4_compress_chain_kernel(ChainTa
         xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
         sraw[k] = scale[v >> job.shift];
       } else {
+        xv[k] = {};
         sraw[k] = 0;
       }
     }
     build_scale_lut(lut, gs);
-    bool ok = true;
+    bool okk[U], ok = true;
+    uint32_t codes[U];
 #pragma unroll
     for (int k = 0; k < U; ++k) {
-      const uint32_t v = v0 + k * B;
-      if (!GUARD || v < nvec)
-        __builtin_nontemporal_store(nvfp4_codes_fast<XT>(xv[k], lut[sraw[k]], &ok), out + v);
+      okk[k] = true;
+      if (!GUARD || v0 + k * B < nvec) codes[k] = nvfp4_codes_fast<XT>(xv[k], lut[sraw[k]], &okk[k]);
+      ok &= okk[k];
     }
-    if (__builtin_expect(wave_all(ok), 1)) return;
-    ok = true;
+    if (__builtin_expect(!wave_all(ok), 0)) nvfp4_settle_codes<XT, U>(xv, sraw, okk, codes, lut, redo);
 #pragma unroll
     for (int k = 0; k < U; ++k) {
       const uint32_t v = v0 + k * B;
-      if (!GUARD || v < nvec) out[v] = nvfp4_codes_divided<XT>(xv[k], lut[sraw[k]], &ok);
-    }
-    if (wave_all(ok)) return;
-#pragma unroll
-    for (int k = 0; k < U; ++k) {
-      const uint32_t v = v0 + k * B;
-      if (!GUARD || v < nvec) out[v] = nvfp4_codes_exact<XT, false>(xv[k], lut[sraw[k]].s, 0.0f);
+      if (!GUARD || v < nvec) __builtin_nontemporal_store(codes[k], out + v);
     }
   };
   if (full) body(std::false_type{});
@@ -556,6 +640,7 @@ nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __re
   constexpr int B = kFp4QdqBlock, U = kFp4QdqUnroll;
   static_assert(B >= 256, "the scale table is built by 256 threads");
   __shared__ Fp4Scale lut[256];
+  __shared__ Fp4Redo<XT> redo[B / 64];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   const bool full = (blockIdx.x + 1) * (uint32_t)(B * U) <= g.nvec;
@@ -573,6 +658,7 @@ nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __re
         xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)v * 8);
         sraw[k] = scale[si[k]];
       } else {
+        xv[k] = {};
         sraw[k] = 0;
       }
     }
@@ -588,31 +674,18 @@ nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __re
       }
       stg_nt<typename XT::raw, 8>(out + (size_t)(v0 + k * B) * 8, o);
     };
-    bool ok = true;
+    bool okk[U], ok = true;
+    uint32_t codes[U];
 #pragma unroll
     for (int k = 0; k < U; ++k) {
-      if (!GUARD || v0 + k * B < g.nvec) {
-        const Fp4Scale e = lut[sraw[k]];
-        emit(k, nvfp4_codes_fast<XT>(xv[k], e, &ok), e.s);
-      }
+      okk[k] = true;
+      if (!GUARD || v0 + k * B < g.nvec) codes[k] = nvfp4_codes_fast<XT>(xv[k], lut[sraw[k]], &okk[k]);
+      ok &= okk[k];
     }
-    if (__builtin_expect(wave_all(ok), 1)) return;
-    ok = true;
+    if (__builtin_expect(!wave_all(ok), 0)) nvfp4_settle_codes<XT, U>(xv, sraw, okk, codes, lut, redo);
 #pragma unroll
-    for (int k = 0; k < U; ++k) {
-      if (!GUARD || v0 + k * B < g.nvec) {
-        const Fp4Scale e = lut[sraw[k]];
-        emit(k, nvfp4_codes_divided<XT>(xv[k], e, &ok), e.s);
-      }
-    }
-    if (wave_all(ok)) return;
-#pragma unroll
-    for (int k = 0; k < U; ++k) {
-      if (!GUARD || v0 + k * B < g.nvec) {
-        const float s = lut[sraw[k]].s;
-        emit(k, nvfp4_codes_exact<XT, false>(xv[k], s, 0.0f), s);
-      }
-    }
+    for (int k = 0; k < U; ++k)
+      if (!GUARD || v0 + k * B < g.nvec) emit(k, codes[k], lut[sraw[k]].s);
   };
   if (full) body(std::false_type{});
   else body(std::true_type{});
@@ -679,6 +752,7 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
                      uint8_t* __restrict__ zp_out, uint32_t nvec) {
   constexpr int B = kFp4Block, U = 2;
   __shared__ Fp4Scale lut[256];
+  __shared__ Fp4Redo<XT> redo[B / 64];
   const float gs = gscale[0];
   const uint32_t v0 = blockIdx.x * (B * U) + threadIdx.x;
   Vec<typename XT::raw, 8> xv[U];
@@ -697,8 +771,9 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
     for (int i = 0; i < 8; ++i) o.v[i] = XT::from_f32(t[i] * s);  // a NaN in the group made s NaN
     if (v < nvec) stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
   };
-  bool ok = true;
-  uint8_t codes[U];
+  bool okk[U], ok = true;
+  uint8_t sraw[U];
+  uint32_t codes[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
@@ -721,22 +796,14 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
       if (scale_out) scale_out[v >> 1] = code;
       if (zp_out) zp_out[v >> 1] = 0;  // fp8 zero
     }
-    codes[k] = code;
-    emit(k, nvfp4_codes_fast<XT>(xv[k], lut[code], &ok), lut[code].s);
+    sraw[k] = code;
+    okk[k] = true;
+    codes[k] = nvfp4_codes_fast<XT>(xv[k], lut[code], &okk[k]);
+    ok &= okk[k];
   }
-  if (__builtin_expect(wave_all(ok), 1)) return;
-  ok = true;
+  if (__builtin_expect(!wave_all(ok), 0)) nvfp4_settle_codes<XT, U>(xv, sraw, okk, codes, lut, redo);
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const Fp4Scale e = lut[codes[k]];
-    emit(k, nvfp4_codes_divided<XT>(xv[k], e, &ok), e.s);
-  }
-  if (wave_all(ok)) return;
-#pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const float s = lut[codes[k]].s;
-    emit(k, nvfp4_codes_exact<XT, true>(xv[k], s, 0.0f), s);
-  }
+  for (int k = 0; k < U; ++k) emit(k, codes[k], lut[sraw[k]].s);
 }
 
 // One-shot nvfp4 compression of a weight whose global scale is known: group scales
@@ -751,7 +818,7 @@ __device__ __forceinline__ void nvfp4_observe_compress_chunk(const typename XT::
                                                              float gs, uint32_t* __restrict__ packed,
                                                              uint8_t* __restrict__ scale_out,
                                                              uint32_t nvec, uint32_t chunk,
-                                                             Fp4Scale* lut) {
+                                                             Fp4Scale* lut, Fp4Redo<XT>* redo) {
   constexpr int B = kFp4Block, U = kFp4ObserveU;
   const uint32_t v0 = chunk * (B * U) + threadIdx.x;
   Vec<typename XT::raw, 8> xv[U];
@@ -761,8 +828,9 @@ __device__ __forceinline__ void nvfp4_observe_compress_chunk(const typename XT::
     xv[k] = ldg_nt<typename XT::raw, 8>(x + (size_t)(v < nvec ? v : nvec - 1) * 8);
   }
   build_scale_lut(lut, gs);
-  bool ok = true;
-  uint8_t codes[U];
+  bool okk[U], ok = true;
+  uint8_t sraw[U];
+  uint32_t codes[U];
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
@@ -780,26 +848,17 @@ __device__ __forceinline__ void nvfp4_observe_compress_chunk(const typename XT::
       code = nvfp4_group_scale<XT>(__builtin_fmaxf(__builtin_fmaxf(-lo, hi), 0.0f),
                                    group_any(2, unordered), gs, &sv);
     }
-    codes[k] = code;
-    const uint32_t c = nvfp4_codes_fast<XT>(xv[k], lut[code], &ok);
-    if (v < nvec) {
-      if ((threadIdx.x & 1) == 0) scale_out[v >> 1] = code;
-      __builtin_nontemporal_store(c, packed + v);
-    }
+    sraw[k] = code;
+    okk[k] = true;
+    codes[k] = nvfp4_codes_fast<XT>(xv[k], lut[code], &okk[k]);
+    ok &= okk[k];
+    if (v < nvec && (threadIdx.x & 1) == 0) scale_out[v >> 1] = code;
   }
-  if (__builtin_expect(wave_all(ok), 1)) return;
-  ok = true;
+  if (__builtin_expect(!wave_all(ok), 0)) nvfp4_settle_codes<XT, U>(xv, sraw, okk, codes, lut, redo);
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * B;
-    const uint32_t c = nvfp4_codes_divided<XT>(xv[k], lut[codes[k]], &ok);
-    if (v < nvec) packed[v] = c;
-  }
-  if (wave_all(ok)) return;
-#pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const uint32_t v = v0 + k * B;
-    if (v < nvec) packed[v] = nvfp4_codes_exact<XT, true>(xv[k], lut[codes[k]].s, 0.0f);
+    if (v < nvec) __builtin_nontemporal_store(codes[k], packed + v);
   }
 }
 
@@ -809,7 +868,8 @@ nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
                               const float* __restrict__ gscale, uint32_t* __restrict__ packed,
                               uint8_t* __restrict__ scale_out, uint32_t nvec) {
   __shared__ Fp4Scale lut[256];
-  nvfp4_observe_compress_chunk<XT>(x, gscale[0], packed, scale_out, nvec, blockIdx.x, lut);
+  __shared__ Fp4Redo<XT> redo[kFp4Block / 64];
+  nvfp4_observe_compress_chunk<XT>(x, gscale[0], packed, scale_out, nvec, blockIdx.x, lut, redo);
 }
 
 // ... for up to kMaxJobs weights per launch: job.scale is written, the zero-point slot
@@ -817,12 +877,13 @@ nvfp4_observe_compress_kernel(const typename XT::raw* __restrict__ x,
 template <typename XT>
 __global__ void __launch_bounds__(kFp4Block) nvfp4_observe_compress_chain_kernel(ChainTable t) {
   __shared__ Fp4Scale lut[256];
+  __shared__ Fp4Redo<XT> redo[kFp4Block / 64];
   uint32_t local, nvec;
   const ChainJob job = find_job(t, blockIdx.x, &local, &nvec);
   nvfp4_observe_compress_chunk<XT>(static_cast<const typename XT::raw*>(job.src),
                                    reinterpret_cast<const float*>(job.zp)[0],
                                    static_cast<uint32_t*>(job.dst),
-                                   static_cast<uint8_t*>(const_cast<void*>(job.scale)), nvec, local, lut);
+                                   static_cast<uint8_t*>(const_cast<void*>(job.scale)), nvec, local, lut, redo);
 }
 
 // The observer on its own for the same scheme (tests/mock_observer.py:38-113 +

@@ -545,6 +545,65 @@ def test_nvfp4_every_bf16_pattern(scale_value, global_scale, gpu):
     assert bool(torch.isnan(fq[~finite].float()).all() == torch.isnan(want_fq[~finite].float()).all())
 
 
+@pytest.mark.parametrize("global_scale", [23040.0, 24576.0, 24064.0])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_nvfp4_quotients_on_rounding_boundaries(global_scale, dtype, gpu):
+    """Global scales with few significant bits (23040 = 45 * 2^9, 24576 = 3 * 2^13: what
+    448 * 6 / amax gives when it is rounded to bfloat16) put a few quotients of nearly every
+    wavefront exactly on a rounding boundary of the e2m1 grid, where only the correctly
+    rounded division settles the code: every entry point that computes codes, against the
+    oracle, plus a tensor where whole rows sit on boundaries (more doubtful vectors than
+    the wavefront's queue takes)."""
+    from compressed_tensors_amd.compressors import BaseCompressor, nvfp4_observe_and_compress_weights
+    from compressed_tensors_amd.quantization import compute_dynamic_scales_and_zp, fake_quantize
+
+    announce("nvfp4 boundaries", global_scale, dtype)
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(int(global_scale))
+    w = (torch.randn(520, 2048, generator=g) * 0.02).to(dtype)
+    gs = torch.tensor([global_scale], dtype=torch.float32)
+    scale, zp = oq.observe_weight(w, oargs, global_scale=gs)
+    # rows 8..15: every element a boundary or a grid value times its group's effective scale
+    # (exact in every dtype when the scale has few bits; elsewhere just more inputs)
+    eff = (scale[8:16].float() / gs).repeat_interleave(16, dim=1)
+    marks = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, -2.5, -0.25])
+    w[8:16] = (eff * marks.repeat(8, 2048 // 16)).to(dtype)
+    scale, zp = oq.observe_weight(w, oargs, global_scale=gs)
+    want = op.nvfp4_compress(w, scale, gs, oargs, zero_point=zp)
+    on_boundary = ((w.float() / (scale.float() / gs).repeat_interleave(16, dim=1)).abs().unsqueeze(-1)
+                   == marks[:7]).any(-1)
+    if dtype == torch.float32:
+        assert int(on_boundary[8:16].sum()) > 8000  # the products above are exact
+    elif global_scale != 24064.0:
+        assert int(on_boundary[16:].sum()) > 100  # here and there in the random rows
+    comp = BaseCompressor.load_from_registry("nvfp4-pack-quantized")
+    dev = dict(weight=w.to(gpu), scale=scale.to(gpu), global_scale=gs.to(gpu), quantization_args=args)
+    assert_bit_equal(comp.compress_weight(**dev)["weight_packed"], want, "compress_weight")
+    assert_bit_equal(comp.compress_weight(**dev, zero_point=zp.to(gpu))["weight_packed"], want, "with zero points")
+    from compressed_tensors_amd.compressors import Fp4WeightBatch
+    batch = Fp4WeightBatch([dev, dict(dev, weight=w.to(gpu).flip(0).contiguous(), scale=scale.to(gpu).flip(0).contiguous())])
+    batch.compress()
+    assert_bit_equal(batch.packed[0], want, "multi-weight compress")
+    assert_bit_equal(batch.packed[1], want.flip(0), "multi-weight compress, second weight")
+    one = comp.observe_and_compress_weight(w.to(gpu), args, global_scale=gs.to(gpu))
+    assert_bit_equal(one["weight_scale"], scale, "one-shot scales")
+    assert_bit_equal(one["weight_packed"], want, "one-shot codes")
+    many = nvfp4_observe_and_compress_weights([w.to(gpu), w.to(gpu)[:100].contiguous()], args,
+                                              global_scales=[gs.to(gpu), gs.to(gpu)])
+    assert_bit_equal(many[0]["weight_packed"], want, "one-shot codes, several weights")
+    assert_bit_equal(many[1]["weight_packed"], want[:100], "one-shot codes, several weights (second)")
+    fq = fake_quantize(w.to(gpu), scale.to(gpu), None, args, global_scale=gs.to(gpu))
+    assert_bit_equal(fq, oq.fake_quantize(w, scale, None, oargs, global_scale=gs), "fake-quantize")
+    aspec = dict(spec, dynamic="local")
+    aargs, oaargs = _pair(aspec)
+    from compressed_tensors_amd.quantization import dynamic_fake_quantize
+    dyn = dynamic_fake_quantize(w.to(gpu), aargs, global_scale=gs.to(gpu))
+    assert dyn is not None
+    s_d, z_d = oq.compute_dynamic_scales_and_zp(w, oaargs, global_scale=gs)
+    assert_bit_equal(dyn, oq.fake_quantize(w, s_d, z_d, oaargs, global_scale=gs), "dynamic fake-quantize")
+
+
 def test_weight_larger_than_4_gib(gpu):
     """a 140 000 x 16 384 bf16 weight (4.6 GB: byte offsets beyond 32 bits, an lm_head of
     a large model): slices at both ends and in the middle against the oracle, and the
