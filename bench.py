@@ -567,9 +567,11 @@ def other_workload(torch, name, seed):
                 # into the second as three bf16 terms)
                 per_elem = 2 * b_dim if a_dim == 1 else 2 * b_dim + 6 * a_dim
                 flops = sum(per_elem * x.numel() for x in xs)
-                ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb,
-                              "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
-                              primary=not label.startswith("weights 4096x4096"), mfma_flops=flops))
+                # size 4096 on the matrix cores: kept to compare with the butterfly kernel below,
+                # which is what hadamard_apply picks for this size
+                ops.append(Op(f"random-sign Hadamard, size {n}{' (matrix cores)' if a_dim > 1 else ''}: {label}",
+                              calls, nb, "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
+                              primary=a_dim == 1 and not label.startswith("weights 4096x4096"), mfma_flops=flops))
                 if label.startswith("weights 4096x4096"):
                     jobs = (_lib.HadamardJob * len(xs))()
                     outs = [torch.empty_like(x) for x in xs]
@@ -578,10 +580,38 @@ def other_workload(torch, name, seed):
                     keep.extend([jobs, outs])
                     m = (jobs, len(xs), code(xs[0].dtype), a_dim, b_dim, _lib.ptr(ma), mb.data_ptr(),
                          q.data_ptr(), None, st)
-                    ops.append(Op(f"random-sign Hadamard, size {n}: {label}, one call (8 per launch)",
+                    ops.append(Op(f"random-sign Hadamard, size {n}{' (matrix cores)' if a_dim > 1 else ''}: {label}, "
+                                  "one call (8 per launch)",
                                   [lambda m=m: _lib.check(lib.ctmi_hadamard_apply_many(*m))], nb,
                                   "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
-                                  mfma_flops=flops))
+                                  primary=a_dim == 1, mfma_flops=flops))
+        # sizes 4096 and 8192 as butterflies in registers (ctmi_sylvester_apply_many): what
+        # hadamard_apply and HadamardTransform.forward run for these sizes
+        tensors["activations 4096x8192 (x8)"] = [randn(4096, 8192) for _ in range(8)]
+        for n, labels in ((4096, ("activations 8192x4096 (x8)", "weights 4096x4096 (x16)", "weights 14336x4096 (x5)")),
+                          (8192, ("activations 4096x8192 (x8)",))):
+            q = (torch.randint(0, 2, (n,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
+            keep.append(q)
+            for label in labels:
+                xs = tensors[label]
+                calls = []
+                many = (_lib.HadamardJob * len(xs))()
+                for i, x in enumerate(xs):
+                    out = torch.empty_like(x)
+                    one = (_lib.HadamardJob * 1)()
+                    for job in (one[0], many[i]):
+                        job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()
+                    keep.extend([x, out, one])
+                    a = (one, 1, code(x.dtype), n, q.data_ptr(), None, st)
+                    calls.append(lambda a=a: _lib.check(lib.ctmi_sylvester_apply_many(*a)))
+                keep.append(many)
+                nb = sum(4 * x.numel() for x in xs)
+                ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb, "fwht_lds_kernel",
+                              primary=not label.startswith("weights 4096x4096")))
+                if label.startswith("weights 4096x4096"):
+                    m = (many, len(xs), code(xs[0].dtype), n, q.data_ptr(), None, st)
+                    ops.append(Op(f"random-sign Hadamard, size {n}: {label}, one call (8 per launch)",
+                                  [lambda m=m: _lib.check(lib.ctmi_sylvester_apply_many(*m))], nb, "fwht_lds_kernel"))
         # 14336 = 224 x 64: a known Hadamard matrix of order 224 (here: any +-1 matrix, the kernel's
         # work does not depend on the entries) times Sylvester(64), as the reference builds the
         # rotation in front of Llama-3's down projections
@@ -656,16 +686,31 @@ def other_workload(torch, name, seed):
             keep.append(many)
             nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in xs)
             flops = sum((2 * 64 + 6 * 64) * x.numel() for x in xs)
-            ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}", calls, nb,
-                          "hadamard_kron_kernel", primary=not label.startswith("weights 4096x4096"),
-                          mfma_flops=flops))
+            ops.append(Op(f"fused: Hadamard 4096 (matrix cores) + int4 g128 quantize + pack, {label}", calls, nb,
+                          "hadamard_kron_kernel", primary=False, mfma_flops=flops))
             if label.startswith("weights 4096x4096"):
                 m = (many, len(xs), code(xs[0].dtype), 64, 64, mb64.data_ptr(), mb64.data_ptr(),
                      q4k.data_ptr(), None, 128, 4, 1, st)
-                ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
+                ops.append(Op(f"fused: Hadamard 4096 (matrix cores) + int4 g128 quantize + pack, {label}, "
+                              "one call (8 per launch)",
                               [lambda m=m: _lib.check(lib.ctmi_hadamard_kron_quant_pack_many(*m))], nb,
-                              "hadamard_kron_kernel", mfma_flops=flops))
-        return "Hadamard rotation GB/s (bf16 MFMA), block 128 and full 4096, and fused with int4 packing", ops, keep
+                              "hadamard_kron_kernel", primary=False, mfma_flops=flops))
+            # the same through the butterfly kernel (what hadamard_quantize_pack picks)
+            calls = []
+            for i in range(len(xs)):
+                one = (_lib.HadamardPackJob * 1)()
+                one[0] = many[i]
+                keep.append(one)
+                a = (one, 1, code(xs[i].dtype), 4096, q4k.data_ptr(), None, 128, 4, 1, st)
+                calls.append(lambda a=a: _lib.check(lib.ctmi_sylvester_quant_pack_many(*a)))
+            ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}", calls, nb,
+                          "fwht_lds_kernel", primary=not label.startswith("weights 4096x4096")))
+            if label.startswith("weights 4096x4096"):
+                m = (many, len(xs), code(xs[0].dtype), 4096, q4k.data_ptr(), None, 128, 4, 1, st)
+                ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
+                              [lambda m=m: _lib.check(lib.ctmi_sylvester_quant_pack_many(*m))], nb,
+                              "fwht_lds_kernel"))
+        return "Hadamard rotation GB/s, block 128 (bf16 MFMA) and full 4096 / 8192 (butterflies), and fused with int4 packing", ops, keep
 
     raise SystemExit(f"unknown workload {name}")
 

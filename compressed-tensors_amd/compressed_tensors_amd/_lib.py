@@ -249,6 +249,16 @@ SIGNATURES = {
         [POINTER(HadamardPackJob), c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32,
          c_int32, c_void_p],
     ),
+    "ctmi_sylvester_supported": (c_int32, [c_int32, c_int32]),
+    "ctmi_sylvester_apply_many": (
+        c_int32,
+        [POINTER(HadamardJob), c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],
+    ),
+    "ctmi_sylvester_quant_pack_many": (
+        c_int32,
+        [POINTER(HadamardPackJob), c_int64, c_int32, c_int32, c_void_p, c_void_p, c_int32, c_int32,
+         c_int32, c_void_p],
+    ),
     "ctmi_hadamard_kron_quant_pack_many": (
         c_int32,
         [POINTER(HadamardPackJob), c_int64, c_int32, c_int32, c_int32, c_void_p, c_void_p, c_void_p,

@@ -193,21 +193,65 @@ def _sylvester_bf16(size: int, device) -> Tensor:
     return _factor_cache[key]
 
 
+# Sylvester sizes with a butterfly kernel (ctmi_sylvester_*), and those where it is the faster
+# one (measured on 14336 x 4096 bf16 weights: 4096: 5.1-5.4 TB/s against 4.4-4.5 on the matrix
+# cores, 8192: 4.4 against 0.8; 1024 and 2048 are level)
+_BUTTERFLY = (1024, 2048, 4096, 8192)
+_BUTTERFLY_FIRST = (4096, 8192)
+
+
+def _butterfly(n: int, dtype, kernel: Optional[str], matrix_t=None) -> bool:
+    """does a Sylvester transform of size n go to the butterfly kernel?  kernel: None (the
+    faster one), "butterfly" or "mfma"."""
+    if kernel not in (None, "butterfly", "mfma"):
+        raise ValueError(f"unknown kernel {kernel!r}")
+    if matrix_t is not None or n not in _BUTTERFLY or kernel == "mfma" or dtype not in _FLOATS:
+        if kernel == "butterfly":
+            raise NotImplementedError(f"no butterfly kernel for size {n}, dtype {dtype} or an explicit matrix")
+        return False
+    if kernel == "butterfly" or n in _BUTTERFLY_FIRST:
+        return True
+    fac = _KRON.get(n)
+    return fac is None or not _lib.load().ctmi_hadamard_supported(fac[0], fac[1], _lib.dtype_code(dtype))
+
+
+def hadamard_kernel_exists(n: int, dtype) -> bool:
+    """is there a kernel for x -> x Sylvester(n) on tensors of this dtype?"""
+    if dtype not in _FLOATS:
+        return False
+    fac = _KRON.get(n)
+    return n in _BUTTERFLY or (fac is not None and bool(
+        _lib.load().ctmi_hadamard_supported(fac[0], fac[1], _lib.dtype_code(dtype))))
+
+
+def _sign(t: Optional[Tensor], dev) -> Optional[Tensor]:
+    return None if t is None else t.to(device=dev, dtype=torch.float32).contiguous()
+
+
+def _aligned(*tensors) -> bool:
+    return all(t is None or t.data_ptr() % 16 == 0 for t in tensors)
+
+
 def hadamard_apply(
     value: Tensor,
     n: int,
     sign_in: Optional[Tensor] = None,
     sign_out: Optional[Tensor] = None,
     matrix_t: Optional[Tensor] = None,
+    kernel: Optional[str] = None,
 ) -> Tensor:
     """every run of n elements x of the last dim becomes
     (x * sign_in) @ M * sign_out / sqrt(n), M = Sylvester(n) or, for n <= 128,
-    the explicit matrix whose transpose is `matrix_t` (bf16, entries exact in bf16)."""
+    the explicit matrix whose transpose is `matrix_t` (bf16, entries exact in bf16).
+    kernel: "mfma" / "butterfly" to pick between the two implementations of the Sylvester
+    sizes 1024 ... 8192 (default: the faster one)."""
     x = to_gpu(value).contiguous()
     if x.dtype not in _FLOATS:
         raise NotImplementedError(f"transforms of dtype {x.dtype} are not supported")
     if x.shape[-1] % n != 0:
         raise ValueError(f"{n} must divide the last dimension {x.shape[-1]}")
+    if _butterfly(n, x.dtype, kernel, matrix_t) and (kernel == "butterfly" or _aligned(x)):
+        return hadamard_apply_many([x], n, sign_in, sign_out, kernel="butterfly")[0]
     fac = hadamard_factors(n)
     lib = _lib.load()
     code = _lib.dtype_code(x.dtype)
@@ -279,23 +323,27 @@ def kron_apply(
     return out
 
 
-_FUSED_KRON = {2048: (32, 64), 4096: (64, 64)}  # transform sizes fused with group size 128
+_FUSED_KRON = {2048: (32, 64), 4096: (64, 64)}  # transform sizes fused with group size 128 (MFMA)
 
 
-def _fused_plan(n: int, args) -> Optional[Tuple[int, int]]:
+def _fused_plan(n: int, args, kernel: Optional[str] = None):
     """None: block size n = group size (32, 64, 128); (a, b): transform size n = a * b with
-    groups of 128"""
+    groups of 128 on the matrix cores; "butterfly": the same on the butterfly kernel"""
     kind = str(getattr(args.type, "value", args.type))
     strategy = str(getattr(args.strategy, "value", args.strategy))
     if not (args.num_bits == 4 and kind == "int" and args.symmetric and strategy == "group"):
         raise NotImplementedError("the fused path covers symmetric int4 group quantization")
     if n in (32, 64, 128) and args.group_size == n:
         return None
-    if n in _FUSED_KRON and args.group_size == 128:
-        return _FUSED_KRON[n]
+    if args.group_size == 128:
+        if n in _BUTTERFLY and kernel != "mfma" and (kernel == "butterfly" or n in _BUTTERFLY_FIRST
+                                                      or n not in _FUSED_KRON):
+            return "butterfly"
+        if n in _FUSED_KRON and kernel != "butterfly":
+            return _FUSED_KRON[n]
     raise NotImplementedError(
         "the fused path covers block sizes 32, 64 and 128 with group_size == block size, and "
-        "transform sizes 2048 and 4096 with group_size 128")
+        "transform sizes 1024, 2048, 4096 and 8192 with group_size 128")
 
 
 def hadamard_quantize_pack(
@@ -306,20 +354,22 @@ def hadamard_quantize_pack(
     sign_out: Optional[Tensor] = None,
     matrix_t: Optional[Tensor] = None,
     return_rotated: bool = False,
+    kernel: Optional[str] = None,
 ) -> Dict[str, Tensor]:
     """hadamard_apply, the min-max observer and pack-quantized compression in one
     pass over a bf16 [rows, cols] tensor of a symmetric 4-bit integer group scheme:
-    block size n (32, 64 or 128) equal to the group size, or a transform of size 2048 or
-    4096 with groups of 128.  Returns what the three steps return, bit for bit:
+    block size n (32, 64 or 128) equal to the group size, or a transform of size 1024,
+    2048, 4096 or 8192 with groups of 128.  Returns what the three steps return, bit for
+    bit (with the same `kernel` in hadamard_apply):
     weight_packed int32 [rows, cols / 8], weight_scale bf16 [rows, cols / group_size],
     weight_shape int64 [2] (and the rotated tensor under "rotated" if asked for)."""
     return _quantize_pack([value], n, quantization_args, sign_in, sign_out, matrix_t,
-                          return_rotated)[0]
+                          return_rotated, kernel)[0]
 
 
-def _quantize_pack(values, n, args, sign_in, sign_out, matrix_t, return_rotated):
+def _quantize_pack(values, n, args, sign_in, sign_out, matrix_t, return_rotated, kernel=None):
     xs = [to_gpu(v).contiguous() for v in values]
-    plan = _fused_plan(n, args)
+    plan = _fused_plan(n, args, kernel)
     if plan is not None and matrix_t is not None:
         raise NotImplementedError("explicit matrices are supported for sizes 32, 64 and 128")
     dev = xs[0].device
@@ -350,6 +400,9 @@ def _quantize_pack(values, n, args, sign_in, sign_out, matrix_t, return_rotated)
                 else matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous())
         _lib.check(lib.ctmi_hadamard_quant_pack_many(
             jobs, len(xs), code, n, mb_t.data_ptr(), _lib.ptr(s_in), _lib.ptr(s_out), 4, 1, stream))
+    elif plan == "butterfly":
+        _lib.check(lib.ctmi_sylvester_quant_pack_many(
+            jobs, len(xs), code, n, _lib.ptr(s_in), _lib.ptr(s_out), group, 4, 1, stream))
     else:
         a, b = plan
         _lib.check(lib.ctmi_hadamard_kron_quant_pack_many(
@@ -364,6 +417,7 @@ def hadamard_apply_many(
     sign_in: Optional[Tensor] = None,
     sign_out: Optional[Tensor] = None,
     matrix_t: Optional[Tensor] = None,
+    kernel: Optional[str] = None,
 ) -> List[Tensor]:
     """hadamard_apply on several tensors of one dtype that share the matrix and the
     signs (the weights of a model under one transform scheme), from one call: the
@@ -379,9 +433,19 @@ def hadamard_apply_many(
             raise ValueError("tensors of one call share dtype and device")
         if x.shape[-1] % n != 0:
             raise ValueError(f"{n} must divide the last dimension {x.shape[-1]}")
-    fac = hadamard_factors(n)
     lib = _lib.load()
     code = _lib.dtype_code(dtype)
+    if _butterfly(n, dtype, kernel, matrix_t):
+        s_in, s_out = _sign(sign_in, dev), _sign(sign_out, dev)
+        if _aligned(s_in, s_out, *xs) or kernel == "butterfly":
+            outs = [torch.empty_like(x) for x in xs]
+            jobs = (_lib.HadamardJob * len(xs))()
+            for job, x, out in zip(jobs, xs, outs):
+                job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()
+            _lib.check(lib.ctmi_sylvester_apply_many(jobs, len(xs), code, n, _lib.ptr(s_in), _lib.ptr(s_out),
+                                                     _lib.stream_of(dev)))
+            return outs
+    fac = hadamard_factors(n)
     if fac is None or not lib.ctmi_hadamard_supported(fac[0], fac[1], code):
         raise NotImplementedError(f"no MFMA Hadamard kernel for size {n} and dtype {dtype}")
     a, b = fac
@@ -412,12 +476,13 @@ def hadamard_quantize_pack_many(
     sign_in: Optional[Tensor] = None,
     sign_out: Optional[Tensor] = None,
     matrix_t: Optional[Tensor] = None,
+    kernel: Optional[str] = None,
 ) -> List[Dict[str, Tensor]]:
     """hadamard_quantize_pack on several bf16 [rows, cols] tensors from one call (8 per
     launch); one dict per tensor, as hadamard_quantize_pack returns it"""
     if not values:
         return []
-    return _quantize_pack(values, n, quantization_args, sign_in, sign_out, matrix_t, False)
+    return _quantize_pack(values, n, quantization_args, sign_in, sign_out, matrix_t, False, kernel)
 
 
 # ------------------------------------------------------------------ vocabulary
@@ -609,9 +674,7 @@ class HadamardTransform(torch.nn.Module):
         value = to_gpu(value)
         n = self.size
         lib = _lib.load()
-        mfma = (self.block is None and hadamard_factors(n) is not None and value.dtype in _FLOATS
-                and bool(lib.ctmi_hadamard_supported(*hadamard_factors(n),
-                                                     _lib.dtype_code(value.dtype))))
+        mfma = self.block is None and hadamard_kernel_exists(n, value.dtype)  # or the butterfly kernel
         big = None  # (a, b): a known block times Sylvester(b) on the matrix cores
         if (not mfma and self.block is not None and value.dtype in _FLOATS and bool(
                 lib.ctmi_hadamard_supported(int(self.block.shape[0]), n // int(self.block.shape[0]),

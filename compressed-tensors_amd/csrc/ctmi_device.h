@@ -187,6 +187,62 @@ struct alignas(sizeof(R) * N) Vec {
   R v[N];
 };
 
+// two fp32 -> two bf16 (round to nearest even) in one dword, by v_cvt_pk_bf16_f32: low
+// half = a, high half = b.  Which NaN a NaN becomes is the instruction's choice
+// (f32_to_bf16 makes every NaN 0x7FC0).
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+  const f32x2 f = {a, b};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
+// 8 fp32 -> 8 elements of T with the bits T::from_f32 gives.  bfloat16 goes through the packed
+// conversion; a lane whose vector holds a NaN (seen on the packed halves: magnitude above
+// 0x7F80) redoes it element by element, which puts the canonical 0x7FC0 there.
+template <typename T>
+__device__ __forceinline__ Vec<typename T::raw, 8> pack8_exact_from_f32(const float* f) {
+  if constexpr (T::id == CTMI_BF16) {
+    typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+    Vec<uint32_t, 4> w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w.v[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
+    u16x2 top = __builtin_bit_cast(u16x2, w.v[0] & 0x7FFF7FFFu);
+#pragma unroll
+    for (int j = 1; j < 4; ++j)
+      top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2, w.v[j] & 0x7FFF7FFFu));
+    // + 0x7F carries into bit 15 exactly for the magnitudes above 0x7F80
+    if (__builtin_expect(((__builtin_bit_cast(uint32_t, top) + 0x007F007Fu) & 0x80008000u) != 0, 0)) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        w.v[j] = (uint32_t)f32_to_bf16(f[2 * j]) | ((uint32_t)f32_to_bf16(f[2 * j + 1]) << 16);
+    }
+    return __builtin_bit_cast(Vec<uint16_t, 8>, w);
+  } else {
+    Vec<typename T::raw, 8> o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o.v[i] = T::from_f32(f[i]);
+    return o;
+  }
+}
+
+// 8 fp32 -> 8 elements of T; bfloat16 through the packed conversion above, so for values
+// that are not NaN or whose NaN bits nothing pins
+template <typename T>
+__device__ __forceinline__ Vec<typename T::raw, 8> pack8_from_f32(const float* f) {
+  if constexpr (T::id == CTMI_BF16) {
+    Vec<uint32_t, 4> w;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) w.v[j] = pack_bf16x2(f[2 * j], f[2 * j + 1]);
+    return __builtin_bit_cast(Vec<uint16_t, 8>, w);
+  } else {
+    Vec<typename T::raw, 8> o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o.v[i] = T::from_f32(f[i]);
+    return o;
+  }
+}
+
 template <typename R, int N>
 __device__ __forceinline__ Vec<R, N> ldg(const R* p) {
   return *reinterpret_cast<const Vec<R, N>*>(p);

@@ -85,10 +85,10 @@ fp4_unpack_vec_kernel(const uint32_t* __restrict__ in, typename OT::raw* __restr
   for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
        v += (int64_t)gridDim.x * blockDim.x) {
     const uint32_t w = in[v];
-    Vec<typename OT::raw, 8> o;
+    float f[8];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o.v[i] = OT::from_f32(fp4_decode((int)((w >> (4 * i)) & 15u)));
-    stg<typename OT::raw, 8>(out + v * 8, o);
+    for (int i = 0; i < 8; ++i) f[i] = fp4_decode((int)((w >> (4 * i)) & 15u));
+    stg<typename OT::raw, 8>(out + v * 8, pack8_from_f32<OT>(f));  // sixteen values, none a NaN
   }
 }
 
@@ -520,10 +520,9 @@ nvfp4_decompress_vec_kernel(const uint32_t* __restrict__ packed, const uint8_t* 
         const float s = lut[sraw[k]].s;
         float t[8];
         fp4_unpack8_hw(pv[k], t);
-        Vec<typename OT::raw, 8> o;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o.v[i] = OT::from_f32(t[i] * s);
-        stg_nt<typename OT::raw, 8>(out + (size_t)v * 8, o);
+        for (int i = 0; i < 8; ++i) t[i] *= s;
+        stg_nt<typename OT::raw, 8>(out + (size_t)v * 8, pack8_exact_from_f32<OT>(t));
       }
     }
   };
@@ -617,10 +616,9 @@ __global__ void __launch_bounds__(kFp4Block) nvfp4_decompress_chain_kernel(Chain
         const float s = lut[sraw[k]].s;
         float f[8];
         fp4_unpack8_hw(pv[k], f);
-        Vec<typename OT::raw, 8> o;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) o.v[i] = OT::from_f32(f[i] * s);
-        stg_nt<typename OT::raw, 8>(out + (size_t)v * 8, o);
+        for (int i = 0; i < 8; ++i) f[i] *= s;
+        stg_nt<typename OT::raw, 8>(out + (size_t)v * 8, pack8_exact_from_f32<OT>(f));
       }
     }
   };
@@ -666,13 +664,12 @@ nvfp4_qdq_vec_kernel(const typename XT::raw* __restrict__ x, const uint8_t* __re
     auto emit = [&](int k, uint32_t codes, float s) {
       float t[8];
       fp4_unpack8_hw(codes, t);
-      Vec<typename XT::raw, 8> o;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const float xi = XT::to_f32(xv[k].v[i]);
-        o.v[i] = XT::from_f32(xi != xi ? xi : t[i] * s);  // a NaN stays one (no code stands for it)
+        t[i] = xi != xi ? xi : t[i] * s;  // a NaN stays one (no code stands for it)
       }
-      stg_nt<typename XT::raw, 8>(out + (size_t)(v0 + k * B) * 8, o);
+      stg_nt<typename XT::raw, 8>(out + (size_t)(v0 + k * B) * 8, pack8_exact_from_f32<XT>(t));
     };
     bool okk[U], ok = true;
     uint32_t codes[U];
@@ -766,10 +763,9 @@ nvfp4_dynamic_kernel(const typename XT::raw* __restrict__ x, const float* __rest
     const uint32_t v = v0 + k * B;
     float t[8];
     fp4_unpack8_hw(c, t);
-    Vec<typename XT::raw, 8> o;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) o.v[i] = XT::from_f32(t[i] * s);  // a NaN in the group made s NaN
-    if (v < nvec) stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, o);
+    for (int i = 0; i < 8; ++i) t[i] *= s;  // a NaN in the group made s NaN
+    if (v < nvec) stg_nt<typename XT::raw, 8>(out + (size_t)v * 8, pack8_exact_from_f32<XT>(t));
   };
   bool okk[U], ok = true;
   uint8_t sraw[U];

@@ -19,6 +19,7 @@
 // takes a fraction of a millisecond, once per weight.
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "fwht.h"
 
 namespace ctmi {
 namespace {
@@ -273,12 +274,16 @@ __global__ void __launch_bounds__(kKmThreads) fwht_wave_kernel(KronArgs a, int64
       if (a.sign_out) v[i] *= a.sign_out[(pos + i) & (a.b - 1)];
     }
     if (full) {
+      if constexpr (VE == 8) {
+        stg_nt<R, 8>(out + e0, pack8_from_f32<IO>(v));
+      } else {
 #pragma unroll
-      for (int q = 0; q < kFwhtPer / VE; ++q) {
-        Vec<R, VE> r;
+        for (int q = 0; q < kFwhtPer / VE; ++q) {
+          Vec<R, VE> r;
 #pragma unroll
-        for (int i = 0; i < VE; ++i) r.v[i] = IO::from_f32(v[q * VE + i]);
-        stg_nt<R, VE>(out + e0 + q * VE, r);
+          for (int i = 0; i < VE; ++i) r.v[i] = IO::from_f32(v[q * VE + i]);
+          stg_nt<R, VE>(out + e0 + q * VE, r);
+        }
       }
     } else {
 #pragma unroll
@@ -296,6 +301,15 @@ size_t kron_lds_bytes(int h, int b) {
 
 template <typename IO>
 int launch_kron(const KronArgs& a, hipStream_t st) {
+  if (a.h == 1 && a.sylvester && fwht_size_supported(a.b)) {
+    FwhtJob job;
+    job.x = a.x;
+    job.out = a.out;
+    job.packed = nullptr;
+    job.scale = nullptr;
+    job.rows = a.n_runs;
+    return fwht_launch(&job, 1, IO::id, a.b, a.sign_in, a.sign_out, a.w, a.scale, nullptr, st);
+  }
   if (a.h == 1 && a.sylvester && a.b <= kFwhtChunk) {
     const int64_t numel = a.n_runs * a.b;
     const int64_t n_chunks = (numel + kFwhtChunk - 1) / kFwhtChunk;
@@ -350,7 +364,7 @@ using namespace ctmi;
 extern "C" int ctmi_kron_matmul_supported(int32_t h, int32_t b, int32_t io_dtype) {
   if (!(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32)) return 0;
   if (h < 1 || b < 1 || (b & (b - 1)) != 0) return 0;
-  if (h == 1 && b <= 512) return 1;  // butterflies inside a wavefront
+  if (h == 1 && (b <= 512 || fwht_size_supported(b))) return 1;  // butterflies in registers
   if (b > 256) return 0;
   return kron_lds_bytes(h, b) <= kKmLdsMax ? 1 : 0;  // a run (b = 1: a tile of 64) as fp32 in LDS
 }

@@ -78,16 +78,16 @@ __device__ __forceinline__ Vec<typename ST::raw, 8> unpack_dequant8_each(
     const Vec<int32_t, BITS / 4>& pv, const float* s, const float* z) {
   constexpr int PF = 32 / BITS;
   constexpr int OFF = 1 << (BITS - 1);
-  Vec<typename ST::raw, 8> o;
+  float f[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
     const uint32_t word = (uint32_t)pv.v[e / PF];
     const int q = (int)((word >> (BITS * (e % PF))) & ((1u << BITS) - 1u)) - OFF;
     float t = (float)q;
     if (HAS_ZP) t -= z[e];
-    o.v[e] = ST::from_f32(t * s[e]);
+    f[e] = t * s[e];
   }
-  return o;
+  return pack8_exact_from_f32<ST>(f);
 }
 
 template <typename XT, typename ST, int BITS, bool HAS_ZP, int RB>

@@ -25,13 +25,6 @@
 namespace ctmi {
 
 typedef float f32x2_t __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
-
-// two fp32 -> two bf16 (RNE) in one dword: low half = a, high half = b
-__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
-  f32x2_t f = {a, b};
-  return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2_t));
-}
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return u2f(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return u2f(w & 0xffff0000u); }
 

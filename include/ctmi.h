@@ -557,6 +557,28 @@ int ctmi_hadamard_kron_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64
                                        const float* sign_out, int32_t group_size, int32_t num_bits,
                                        int32_t symmetric, void* stream);
 
+/* A23 / A24 for the reference's own matrices of a power-of-two size n = 1024, 2048, 4096 or
+ * 8192: Sylvester's H_n (deterministic_hadamard_matrix, transform/utils/hadamard.py:33-62)
+ * and diag(signs) * H_n (random_hadamard_matrix, :65-89, whose table of known blocks holds
+ * Sylvester's matrices for these sizes).  Every run of n elements x becomes
+ *     x * diag(sign_in) * H_n * diag(sign_out) / sqrt(n)
+ * (transform/factory/hadamard.py:104-121) rounded to io_dtype (bf16 / f16 / f32), computed
+ * as log2(n) butterfly stages in fp32 registers: no matrix is read and nothing is rounded
+ * before the end.  sign_in / sign_out: fp32 [n] or NULL, 16-byte aligned like the tensors.
+ * Several tensors share a launch, 8 at a time. */
+int ctmi_sylvester_supported(int32_t n, int32_t io_dtype);
+int ctmi_sylvester_apply_many(const ctmi_hadamard_job* jobs, int64_t n_jobs, int32_t io_dtype,
+                              int32_t n, const float* sign_in, const float* sign_out, void* stream);
+
+/* ... followed in the same pass by the W4A16 pipeline of ctmi_hadamard_kron_quant_pack_many
+ * (bf16 tensors, symmetric int4, group size 128): same bits as ctmi_sylvester_apply_many and
+ * ctmi_observe_pack_quantized in sequence.  packed: int32 [numel / 8]; scale: bf16
+ * [numel / 128]; rotated optional. */
+int ctmi_sylvester_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64_t n_jobs,
+                                   int32_t io_dtype, int32_t n, const float* sign_in,
+                                   const float* sign_out, int32_t group_size, int32_t num_bits,
+                                   int32_t symmetric, void* stream);
+
 /* A23 / A24 for matrices with an explicit factor (transform/utils/matrix.py:137-171 for
  * a small explicit matrix; transform/utils/hadamard.py:102-163 for the reference's
  * Hadamard matrices of size K * 2^m built from its table of known K x K matrices,
@@ -568,9 +590,10 @@ int ctmi_hadamard_kron_quant_pack_many(const ctmi_hadamard_pack_job* jobs, int64
  * io_dtype (scale = 1 / sqrt(h * b) makes a Hadamard rotation orthonormal).  w: fp32
  * [h, h] row-major (any values); sign_in / sign_out: fp32 [h * b] or NULL; b a power of
  * two up to 256 and h * b * 4 bytes within 159 KB; for b = 1, 64 runs share a workgroup
- * and h may be at most 313; for h = 1 with the Sylvester factor b may be 512, and the
- * butterflies stay in a wavefront's registers (ctmi_kron_matmul_supported).  fp32 accumulation on the vector
- * ALUs. */
+ * and h may be at most 313; for h = 1 with the Sylvester factor b may be 512 (the
+ * butterflies stay in a wavefront's registers) or 1024, 2048, 4096, 8192 (the kernel of
+ * ctmi_sylvester_apply_many; tensors and sign vectors 16-byte aligned);
+ * ctmi_kron_matmul_supported tells.  fp32 accumulation on the vector ALUs. */
 int ctmi_kron_matmul_supported(int32_t h, int32_t b, int32_t io_dtype);
 int ctmi_kron_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t h,
                      int32_t b, const float* w, const float* sign_in, const float* sign_out,

@@ -278,3 +278,47 @@ def test_transform_and_block_entry_point_errors(ctmi):
     rc = ctmi.ctmi_observe_nvfp4_compress_many(oj, 2, None)
     assert rc == _lib.CTMI_ERR_VALUE and "job 1" in _err(ctmi)
     assert ctmi.ctmi_observe_nvfp4_compress_many(None, 0, None) == _lib.CTMI_OK
+
+
+def test_sylvester_entry_point_errors(ctmi):
+    """the butterfly kernels' entry points: sizes, dtypes, alignment and job lists, refused on the host"""
+    assert ctmi.ctmi_sylvester_supported(4096, _lib.BF16) == 1
+    assert ctmi.ctmi_sylvester_supported(8192, _lib.F32) == 1
+    assert ctmi.ctmi_sylvester_supported(512, _lib.BF16) == 0
+    assert ctmi.ctmi_sylvester_supported(16384, _lib.BF16) == 0
+    assert ctmi.ctmi_sylvester_supported(4096, _lib.I8) == 0
+    assert ctmi.ctmi_kron_matmul_supported(1, 4096, _lib.F16) == 1
+    jobs = (_lib.HadamardJob * 2)()
+    jobs[0].x, jobs[0].out, jobs[0].numel = 0x1000, 0x2000, 8192
+    jobs[1].x, jobs[1].out, jobs[1].numel = 0x3000, 0x4000, 4096 * 3
+    call = ctmi.ctmi_sylvester_apply_many
+    assert call(jobs, 2, _lib.BF16, 512, None, None, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert "1024, 2048, 4096 and 8192" in _err(ctmi)
+    assert call(jobs, 2, _lib.I8, 4096, None, None, None) == _lib.CTMI_ERR_UNSUPPORTED
+    jobs[1].numel = 5000
+    assert call(jobs, 2, _lib.BF16, 4096, None, None, None) == _lib.CTMI_ERR_VALUE
+    assert "job 1" in _err(ctmi) and "multiple of the transform size" in _err(ctmi)
+    jobs[1].numel, jobs[1].out = 4096, None
+    assert call(jobs, 2, _lib.BF16, 4096, None, None, None) == _lib.CTMI_ERR_VALUE and "job 1" in _err(ctmi)
+    jobs[1].out = 0x4008
+    assert call(jobs, 2, _lib.BF16, 4096, None, None, None) == _lib.CTMI_ERR_VALUE and "aligned" in _err(ctmi)
+    jobs[1].out = 0x4000
+    assert call(jobs, 2, _lib.BF16, 4096, 0x5004, None, None) == _lib.CTMI_ERR_VALUE and "sign vectors" in _err(ctmi)
+    assert call(None, 0, _lib.BF16, 4096, None, None, None) == _lib.CTMI_OK
+    jobs[0].numel = jobs[1].numel = 0
+    assert call(jobs, 2, _lib.BF16, 4096, None, None, None) == _lib.CTMI_OK  # nothing to do, nothing launched
+    pj = (_lib.HadamardPackJob * 1)()
+    pj[0].x, pj[0].packed, pj[0].scale, pj[0].numel = 0x1000, 0x2000, 0x3000, 8192
+    fused = ctmi.ctmi_sylvester_quant_pack_many
+    assert fused(pj, 1, _lib.F16, 4096, None, None, 128, 4, 1, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert fused(pj, 1, _lib.BF16, 4096, None, None, 64, 4, 1, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert "group size" in _err(ctmi)
+    assert fused(pj, 1, _lib.BF16, 4096, None, None, 128, 8, 1, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert fused(pj, 1, _lib.BF16, 4096, None, None, 128, 4, 0, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert fused(pj, 1, _lib.BF16, 256, None, None, 128, 4, 1, None) == _lib.CTMI_ERR_UNSUPPORTED
+    pj[0].scale = None
+    assert fused(pj, 1, _lib.BF16, 4096, None, None, 128, 4, 1, None) == _lib.CTMI_ERR_VALUE
+    assert fused(None, 0, _lib.BF16, 4096, None, None, 128, 4, 1, None) == _lib.CTMI_OK
+    # the same kernel behind ctmi_kron_matmul (h = 1, Sylvester inner factor)
+    rc = ctmi.ctmi_kron_matmul(0x1008, 0x2000, _lib.BF16, 4096, 1, 4096, 0x3000, None, None, 1, 1.0, None)
+    assert rc == _lib.CTMI_ERR_VALUE and "aligned" in _err(ctmi)

@@ -41,27 +41,52 @@ def _reference(weight64, value, location, inverse=False, module_type=torch.nn.Li
 SIZES = [32, 64, 128, 1024, 2048, 4096, 8192]
 
 
+@pytest.mark.parametrize("kernel", ["mfma", "butterfly"])
 @pytest.mark.parametrize("n", SIZES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
-def test_sylvester_apply(n, dtype, gpu):
+def test_sylvester_apply(n, dtype, kernel, gpu):
+    """both implementations of x -> x H_n: products with the factors of H_n on the matrix
+    cores, and (n >= 1024) butterflies in registers"""
     from compressed_tensors_amd import _lib
     from compressed_tensors_amd.transform import hadamard_apply, hadamard_factors
 
-    announce("hadamard_apply", n, dtype)
+    announce("hadamard_apply", n, dtype, kernel)
     a, b = hadamard_factors(n)
-    if not _lib.load().ctmi_hadamard_supported(a, b, _lib.dtype_code(dtype)):
+    if kernel == "mfma" and not _lib.load().ctmi_hadamard_supported(a, b, _lib.dtype_code(dtype)):
         pytest.skip("factorisation not built for this dtype")
+    if kernel == "butterfly" and not _lib.load().ctmi_sylvester_supported(n, _lib.dtype_code(dtype)):
+        with pytest.raises(NotImplementedError):
+            hadamard_apply(torch.zeros(1, n, dtype=dtype, device=gpu), n, kernel=kernel)
+        return
     g = torch.Generator().manual_seed(n)
     rows = 37 if n <= 2048 else 9
     x = torch.randn(rows, 2 * n if n <= 1024 else n, generator=g).to(dtype)
     q = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).double()
     h = oh.deterministic_hadamard_matrix(n, torch.float64)
-    y = hadamard_apply(x.to(gpu), n)
+    y = hadamard_apply(x.to(gpu), n, kernel=kernel)
     _assert_within_ulp(y, _reference(h, x, "input"), "plain")
-    y = hadamard_apply(x.to(gpu), n, sign_in=q.float())
+    y = hadamard_apply(x.to(gpu), n, sign_in=q.float(), kernel=kernel)
     _assert_within_ulp(y, _reference(q.unsqueeze(1) * h, x, "input"), "sign_in")
-    y = hadamard_apply(x.to(gpu), n, sign_out=q.float())
+    y = hadamard_apply(x.to(gpu), n, sign_out=q.float(), kernel=kernel)
     _assert_within_ulp(y, _reference((q.unsqueeze(1) * h).T, x, "input"), "sign_out")
+    y = hadamard_apply(x.to(gpu), n, sign_in=q.float(), sign_out=q.flip(0).float(), kernel=kernel)
+    _assert_within_ulp(y, _reference(q.unsqueeze(1) * h * q.flip(0), x, "input"), "both signs")
+
+
+def test_butterfly_kernel_runs_of_many_rows(gpu):
+    """more runs than workgroups are resident (every workgroup takes several, with the next
+    run's loads and first pass under way), for each size: every row against the fp64 product"""
+    from compressed_tensors_amd.transform import hadamard_apply
+
+    for n, rows in ((1024, 40_000), (2048, 20_000), (4096, 5_000), (8192, 4_099)):
+        announce("butterfly rows", n, rows)
+        g = torch.Generator(device=gpu).manual_seed(n)
+        x = torch.randn(rows, n, generator=g, device=gpu).bfloat16()
+        y = hadamard_apply(x, n, kernel="butterfly")
+        h = oh.deterministic_hadamard_matrix(n, torch.float64).to(gpu)
+        for r0 in range(0, rows, 4096):
+            want = (x[r0:r0 + 4096].double() @ h / n ** 0.5).bfloat16()
+            _assert_within_ulp(y[r0:r0 + 4096], want.cpu(), f"n={n} rows {r0}..")
 
 
 def test_explicit_small_matrix(gpu):
@@ -168,9 +193,12 @@ def test_large_activation_properties(gpu):
         assert float(rel) < 2e-2
 
 
-@pytest.mark.parametrize("n,shape", [(128, (64, 512)), (128, (37, 256)), (64, (33, 192)), (32, (19, 96)),
-                                     (4096, (37, 4096)), (4096, (5, 8192)), (2048, (21, 4096))])
-def test_fused_rotation_quantization_packing(n, shape, gpu):
+@pytest.mark.parametrize("n,shape,kernel", [
+    (128, (64, 512), None), (128, (37, 256), None), (64, (33, 192), None), (32, (19, 96), None),
+    (4096, (37, 4096), "mfma"), (4096, (5, 8192), "mfma"), (2048, (21, 4096), "mfma"),
+    (4096, (37, 4096), "butterfly"), (4096, (2100, 8192), "butterfly"), (2048, (21, 4096), "butterfly"),
+    (1024, (300, 3072), "butterfly"), (8192, (11, 8192), "butterfly"), (8192, (3000, 8192), None)])
+def test_fused_rotation_quantization_packing(n, shape, kernel, gpu):
     """ctmi_hadamard_quant_pack == hadamard_apply -> min-max observer -> pack-quantized
     compress, bit for bit (each of which is checked against the oracle on its own), and
     the whole chain against the oracle's."""
@@ -180,7 +208,8 @@ def test_fused_rotation_quantization_packing(n, shape, gpu):
     from compressed_tensors_amd.quantization import QuantizationArgs, observe_weight_qparams
     from compressed_tensors_amd.transform import hadamard_apply, hadamard_quantize_pack
 
-    announce("fused hadamard + int4 + pack", n, shape)
+    announce("fused hadamard + int4 + pack", n, shape, kernel)
+    kern = dict(kernel=kernel) if n > 128 else {}
     g = torch.Generator().manual_seed(3 * n + shape[0])
     x = (torch.randn(shape, generator=g) * 0.02).bfloat16()
     group = min(n, 128)  # transforms of 2048 / 4096 elements feed groups of 128
@@ -191,8 +220,10 @@ def test_fused_rotation_quantization_packing(n, shape, gpu):
     q = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
     args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=group)
     for signs in (dict(), dict(sign_in=q), dict(sign_out=q)):
-        fused = hadamard_quantize_pack(x.to(gpu), n, args, return_rotated=True, **signs)
-        y = hadamard_apply(x.to(gpu), n, **signs)
+        fused = hadamard_quantize_pack(x.to(gpu), n, args, return_rotated=True, **signs, **kern)
+        y = hadamard_apply(x.to(gpu), n, **signs, **kern)
+        no_copy = hadamard_quantize_pack(x.to(gpu), n, args, **signs, **kern)
+        assert torch.equal(no_copy["weight_packed"], fused["weight_packed"]) and "rotated" not in no_copy
         assert torch.equal(fused["rotated"].view(torch.int16), y.view(torch.int16)), "rotated tensor"
         scale, zp = observe_weight_qparams(y, args)
         comp = BaseCompressor.load_from_registry("pack-quantized")
@@ -211,7 +242,7 @@ def test_fused_rotation_quantization_packing(n, shape, gpu):
 
 @pytest.mark.parametrize("n,dtype", [(128, torch.bfloat16), (64, torch.float16), (32, torch.bfloat16),
                                      (4096, torch.bfloat16), (1024, torch.float16), (2048, torch.bfloat16),
-                                     (128, torch.float32)])
+                                     (128, torch.float32), (8192, torch.float16), (4096, torch.float32)])
 def test_many_tensors_in_one_call(n, dtype, gpu):
     """hadamard_apply_many == hadamard_apply tensor by tensor, bit for bit: more tensors than
     one launch takes (8), sizes that differ, a tensor that ends in a ragged group of
@@ -233,7 +264,7 @@ def test_many_tensors_in_one_call(n, dtype, gpu):
                 assert_bit_equal(y, hadamard_apply(x, n, **signs), f"tensor {i} ({rows[i]} rows)")
 
 
-@pytest.mark.parametrize("n", [128, 4096])
+@pytest.mark.parametrize("n", [128, 4096, 2048, 1024])
 def test_fused_many_tensors_in_one_call(n, gpu):
     """hadamard_quantize_pack_many == hadamard_quantize_pack tensor by tensor"""
     from compressed_tensors_amd.quantization import QuantizationArgs
@@ -325,7 +356,9 @@ def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
     assert ctmi.ctmi_kron_matmul_supported(12, 3, code) == 0      # inner size not a power of two
     assert ctmi.ctmi_kron_matmul_supported(12, 512, code) == 0    # more than 256 lanes
     assert ctmi.ctmi_kron_matmul_supported(1, 512, code) == 1     # plain Sylvester: in registers
-    assert ctmi.ctmi_kron_matmul_supported(1, 1024, code) == 0
+    assert ctmi.ctmi_kron_matmul_supported(1, 1024, code) == 1    # ... and up to 8192 with the run in LDS
+    assert ctmi.ctmi_kron_matmul_supported(1, 16384, code) == 0
+    assert ctmi.ctmi_kron_matmul_supported(2, 1024, code) == 0
     assert ctmi.ctmi_kron_matmul_supported(256, 256, code) == 0   # 256 KB of LDS
     x = torch.zeros(314 * 4, dtype=torch.bfloat16, device=gpu)
     w = torch.zeros(314, 314, device=gpu)
