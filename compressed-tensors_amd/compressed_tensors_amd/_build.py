@@ -36,6 +36,12 @@ FLAGS = [
 ]
 
 
+# per source file (by stem): the butterfly kernels chain matrix-core results into vector code,
+# so their accumulators live in ordinary registers (no copies out of a second register class,
+# and the registers are reused once the accumulators are dead)
+EXTRA_FLAGS = {"fwht": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
+
 def sources():
     return sorted(str(p) for p in CSRC_DIR.glob("*.hip"))
 
@@ -65,8 +71,8 @@ def build_library(verbose: bool = False, jobs: int = 0) -> Path:
     jobs = jobs or min(len(srcs), os.cpu_count() or 1, 16)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(
-            lambda so: _run([HIPCC, *compile_flags, f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", "-c", so[0],
-                             "-o", so[1]], verbose),
+            lambda so: _run([HIPCC, *compile_flags, *EXTRA_FLAGS.get(Path(so[0]).stem, []),
+                             f"-I{INCLUDE_DIR}", f"-I{CSRC_DIR}", "-c", so[0], "-o", so[1]], verbose),
             zip(srcs, objs)))
     tmp = LIB_PATH.with_suffix(".so.tmp")
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", str(tmp)], verbose)
