@@ -628,9 +628,22 @@ def other_workload(torch, name, seed):
             a = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), 224, 64, ma224.data_ptr(),
                  mb64.data_ptr(), q14.data_ptr(), None, st)
             calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
-        ops.append(Op("random-sign Hadamard, size 14336 = 224 x 64: activations 4096x14336 (x5)", calls,
+        ops.append(Op("random-sign Hadamard, size 14336 = 224 x 64, both factors as matrix products: "
+                      "activations 4096x14336 (x5)", calls,
                       sum(4 * x.numel() for x in xs14), "hadamard_kron_kernel", primary=False,
                       mfma_flops=sum((2 * 64 + 6 * 224) * x.numel() for x in xs14)))
+        # the same transform as HadamardTransform.forward runs it: the block on the matrix cores,
+        # Sylvester(64) as butterflies (no matrix for it: mb_t = NULL)
+        calls = []
+        for x in xs14:
+            out = torch.empty_like(x)
+            keep.append(out)
+            a = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), 224, 64, ma224.data_ptr(),
+                 None, q14.data_ptr(), None, st)
+            calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
+        ops.append(Op("random-sign Hadamard, size 14336 = 224 x 64: activations 4096x14336 (x5)", calls,
+                      sum(4 * x.numel() for x in xs14), "block_sylvester64_kernel",
+                      mfma_flops=sum(2 * 224 * x.numel() for x in xs14)))
         # rotation (block 128) + symmetric int4 group-128 quantization + pack_to_int32, one pass
         mb = deterministic_hadamard_matrix(128, torch.bfloat16, dev).contiguous()
         q = (torch.randint(0, 2, (128,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)

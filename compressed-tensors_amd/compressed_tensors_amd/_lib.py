@@ -250,6 +250,7 @@ SIGNATURES = {
          c_int32, c_void_p],
     ),
     "ctmi_sylvester_supported": (c_int32, [c_int32, c_int32]),
+    "ctmi_hadamard_sylvester_inner_supported": (c_int32, [c_int32, c_int32, c_int32]),
     "ctmi_sylvester_apply_many": (
         c_int32,
         [POINTER(HadamardJob), c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p],

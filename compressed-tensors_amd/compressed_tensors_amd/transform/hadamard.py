@@ -676,10 +676,13 @@ class HadamardTransform(torch.nn.Module):
         lib = _lib.load()
         mfma = self.block is None and hadamard_kernel_exists(n, value.dtype)  # or the butterfly kernel
         big = None  # (a, b): a known block times Sylvester(b) on the matrix cores
-        if (not mfma and self.block is not None and value.dtype in _FLOATS and bool(
-                lib.ctmi_hadamard_supported(int(self.block.shape[0]), n // int(self.block.shape[0]),
-                                            _lib.dtype_code(value.dtype)))):
-            big = (int(self.block.shape[0]), n // int(self.block.shape[0]))
+        inner_butterflies = False  # ... with Sylvester(b) as butterflies on the block product
+        if not mfma and self.block is not None and value.dtype in _FLOATS:
+            k, code = int(self.block.shape[0]), _lib.dtype_code(value.dtype)
+            if lib.ctmi_hadamard_sylvester_inner_supported(k, n // k, code):
+                big, inner_butterflies = (k, n // k), True
+            elif lib.ctmi_hadamard_supported(k, n // k, code):
+                big = (k, n // k)
         plan = None if (mfma or big) else _kron_plan(n, self.block)
         if plan is not None and not (value.dtype in _FLOATS and bool(
                 lib.ctmi_kron_matmul_supported(plan[0], plan[1], _lib.dtype_code(value.dtype)))):
@@ -722,9 +725,10 @@ class HadamardTransform(torch.nn.Module):
             sign = (lambda t: None if t is None else
                     t.to(device=x.device, dtype=torch.float32).contiguous())
             si, so = sign(s_in), sign(s_out)
+            mb = None if inner_butterflies else _sylvester_bf16(b, x.device)
             _lib.check(lib.ctmi_hadamard_apply(
                 x.data_ptr(), y.data_ptr(), _lib.dtype_code(x.dtype), x.numel(), a, b,
-                self._factor[key].data_ptr(), _sylvester_bf16(b, x.device).data_ptr(),
+                self._factor[key].data_ptr(), _lib.ptr(mb),
                 _lib.ptr(si), _lib.ptr(so), _lib.stream_of(x.device)))
         else:
             # W = diag(q) (B^T (x) S):  x W = (x * q) (B^T (x) S);  x W^T = (x (B (x) S)) * q

@@ -1,0 +1,356 @@
+// Transforms W = diag(sign_in) * (Ma (x) Sylvester(64)) * diag(sign_out) * scale on runs of
+// K * 64 bfloat16 elements, K <= 224: the reference's Hadamard matrices of size K * 2^m
+//
+//   random_hadamard_matrix, _matmul_hadU        transform/utils/hadamard.py:65-163
+//   HadamardTransform.forward                   transform/factory/hadamard.py:104-121
+//
+// (K from its table of known matrices: 12, 20, 28 ... 224; 14336 = 224 * 64 is the size in
+// front of Llama-3's down projections).  A run is a K x 64 matrix X (element 64 i + j) and
+//     y = vec(Ma^T X S),      S = Sylvester(64).
+// The product with Ma takes bfloat16 inputs and a matrix of +-1, so it is exact as ONE product
+// on the matrix cores (v_mfma_f32_32x32x16_bf16, fp32 accumulation); the factor S then needs no
+// matrix at all: it is six butterfly stages on the fp32 accumulators.  Nothing is split into
+// bfloat16 terms, which is what made the two-product kernel three times as expensive.
+//
+// Per run a wavefront computes D[j][i'] = sum_i X[i][j] Ma[i][i'] with j on the M side:
+//   A operand  X^T: lane (c, g) holds X[16 ks + 8 g + e][32 mt + c], e = 0..7: picked as single
+//              16-bit elements out of an image of 32 rows of X in LDS (the run streams through
+//              it, 4.5 KB at a time, loaded as whole 128-byte lines)
+//   B operand  Ma: lane (c, g) holds Ma[16 ks + 8 g + e][32 nt + c] = 16 bytes of row 32 nt + c
+//              of Ma^T; all fragments of Ma sit in LDS in the lanes' own order (K = 224: 98 KB,
+//              shared by the four wavefronts of the workgroup) and one read serves both M tiles
+//   D          acc[mt][nt][4 b + r] = D[32 mt + 8 b + 4 g + r][32 nt + c]
+// The butterflies over j: the stage over mt adds and subtracts whole accumulator tiles; one
+// exchange between the lane halves (v_permlane32_swap) pairs the two values of the stage over
+// g in one lane; the other four stages are within a lane's 16 values.  Afterwards lane (c, h)
+// holds, for every nt, the 32 neighbouring outputs y[64 (32 nt + c) + 32 h ...]: they go
+// through the LDS image once more so that the stores are whole lines again.
+//
+// One wavefront per SIMD for K > 128: the accumulators are 32 NT registers a lane and the next
+// run, prefetched whole, another 16 NT.
+#include <utility>
+
+#include "ctmi_device.h"
+#include "ctmi_host.h"
+#include "fwht.h"
+
+namespace ctmi {
+namespace {
+
+typedef __bf16 bs_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float bs_f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t bs_u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBsWaves = 4;
+constexpr int kBsThreads = kBsWaves * kWave;
+constexpr int kBsPitch = 36;                    // dwords between the rows of an image (64 bf16 + 16 bytes)
+constexpr int kBsImage = 32 * kBsPitch;         // dwords of an image of 32 rows
+constexpr int kBsRing = kBsImage;               // per wavefront
+
+struct BsTable {
+  const void* x[kFwhtMaxJobs];
+  void* out[kFwhtMaxJobs];
+  int64_t end[kFwhtMaxJobs];  // running total of runs, job 0 .. j (unused: INT64_MAX)
+  int64_t total;
+};
+
+// A wavefront's run number is the same in all its lanes, which the compiler cannot see: said
+// outright, the search and the table reads behind it are scalar instructions.  (As vector
+// loads they would also make every prefetch wait for all loads in flight.)
+__device__ __forceinline__ int64_t bs_uniform(int64_t v) {
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+  const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)v >> 32));
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
+__device__ __forceinline__ int bs_job(const BsTable& t, int64_t run, int64_t* local) {
+  run = bs_uniform(run);
+  int j = 0;
+  int64_t first = 0;
+#pragma unroll
+  for (int i = 0; i < kFwhtMaxJobs - 1; ++i) {
+    const bool past = run >= t.end[i];
+    j = past ? i + 1 : j;
+    first = past ? t.end[i] : first;
+  }
+  *local = run - first;
+  return j;
+}
+
+// fragments of Ma, the sign masks (SIGNS != 0), one image per wavefront
+constexpr size_t bs_lds_bytes(int nt, bool signs) {
+  return ((size_t)2 * nt * nt * kWave * 4 + (signs ? (size_t)nt * 4 * kWave * 4 : 0) +
+          (size_t)kBsWaves * kBsRing) * sizeof(uint32_t);
+}
+
+// NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out
+template <int NT, int SIGNS>
+__global__ void __launch_bounds__(kBsThreads, 1)
+block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
+                         const float* __restrict__ signs, float scale) {
+  constexpr int KS = 2 * NT;  // steps of 16 over the contracted index
+  extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
+  bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
+  bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [NT * 4][64] (SIGNS != 0)
+  const uint32_t l = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const uint32_t c = l & 31u, g = l >> 5;
+  uint32_t* image = bs_lds + (KS * NT + (SIGNS ? NT * 4 : 0)) * kWave * 4 + wave * kBsRing;
+  const int64_t n = (int64_t)k_dim * 64;
+
+  // The fragments of Ma, zero beyond K.  Eight at a time per wavefront, loads first: one after
+  // the other they would cost the launch as many memory round trips as there are fragments.
+  const bool ma_vectors = k_dim % 8 == 0 && (uintptr_t)ma_t % 16 == 0;  // 16-byte pieces of whole rows
+  for (int f0 = 0; f0 < KS * NT; f0 += kBsWaves * 8) {
+    bs_u32x4 w[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int f = f0 + u * kBsWaves + (int)wave;
+      const int ks = f / NT, nt = f % NT;
+      const int col = 32 * nt + (int)c, i0 = 16 * ks + 8 * (int)g;  // Ma[i0 + e][col] = ma_t[col][i0 + e]
+      w[u] = bs_u32x4{0u, 0u, 0u, 0u};
+      if (f < KS * NT && col < k_dim) {
+        if (ma_vectors) {
+          if (i0 < k_dim) w[u] = __builtin_bit_cast(bs_u32x4, ldg<uint16_t, 8>(ma_t + (int64_t)col * k_dim + i0));
+        } else {
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const int i = i0 + 2 * d;
+            const uint32_t lo = i < k_dim ? ma_t[(int64_t)col * k_dim + i] : 0u;
+            const uint32_t hi = i + 1 < k_dim ? ma_t[(int64_t)col * k_dim + i + 1] : 0u;
+            w[u][d] = lo | (hi << 16);
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int f = f0 + u * kBsWaves + (int)wave;
+      if (f < KS * NT) ma_frag[f * kWave + l] = w[u];
+    }
+  }
+  // Sign masks of the vectors a lane loads (SIGNS == 1: vector q of chunk ch is row
+  // 32 ch + l / 8 + 8 q, columns 8 (l % 8) ...) or stores (SIGNS == 2: the same positions with
+  // the tile nt in place of the chunk): the same for the four wavefronts, read at each use
+  if constexpr (SIGNS != 0) {
+    for (int f = (int)wave; f < NT * 4; f += kBsWaves) {
+      const int row = 32 * (f >> 2) + (int)(l >> 3) + 8 * (f & 3);
+      bs_u32x4 m = {0u, 0u, 0u, 0u};
+      if (row < k_dim) {
+        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + 64 * row + 8 * (l & 7u));
+#pragma unroll
+        for (int d = 0; d < 4; ++d) m[d] = ((s8.v[2 * d] >> 16) & 0x8000u) | (s8.v[2 * d + 1] & 0x80000000u);
+      }
+      flip[f * kWave + l] = m;
+    }
+  }
+  __syncthreads();
+
+  // selector that puts the 16-bit element of column c out of two dwords (columns c & ~1, c | 1
+  // of two neighbouring rows) side by side
+  const uint32_t pick = (c & 1u) ? 0x07060302u : 0x05040100u;
+
+  // A run is NT chunks of 32 rows of X, 4 vectors a lane each; rows beyond K read as zeros.
+  // All of the next run is in flight while this one is worked on: with one wavefront per SIMD
+  // nothing else hides the latency of memory.
+  // No branch around the loads (a load under a condition makes the compiler wait for it on
+  // the spot): a run beyond the last reads the last again, a row beyond K reads row K - 1 and
+  // is replaced by zeros when it is used.
+  bs_u32x4 in[NT][4];
+  auto fetch = [&](int64_t r, int ch) {
+    r = r < tab.total ? r : tab.total - 1;
+    int64_t local;
+    const int j = bs_job(tab, r, &local);
+    const uint16_t* __restrict__ xr = static_cast<const uint16_t*>(tab.x[j]) + local * n;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int row = 32 * ch + (int)(l >> 3) + 8 * q;
+      in[ch][q] = __builtin_bit_cast(
+          bs_u32x4, ldg_nt<uint16_t, 8>(xr + 64 * (row < k_dim ? row : k_dim - 1) + 8 * (l & 7u)));
+    }
+  };
+
+  const int64_t step = (int64_t)gridDim.x * kBsWaves;
+  int64_t run = (int64_t)blockIdx.x * kBsWaves + wave;
+#pragma unroll
+  for (int ch = 0; ch < NT; ++ch) fetch(run, ch);
+  for (; run < tab.total; run += step) {
+    bs_f32x16_t acc[2][NT];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
+#pragma unroll
+    for (int ch = 0; ch < NT; ++ch) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        bs_u32x4 w = in[ch][q];
+        if (32 * ch + (int)(l >> 3) + 8 * q >= k_dim) w = bs_u32x4{0u, 0u, 0u, 0u};
+        if constexpr (SIGNS == 1) w ^= flip[(ch * 4 + q) * kWave + l];
+        *reinterpret_cast<bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]) = w;
+      }
+      fetch(run + step, ch);
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2; ++ks2) {
+        const int ks = 2 * ch + ks2;
+        // A operands for both M tiles: rows 16 ks2 + 8 g + e of the image, column 32 mt + c
+        bs_u32x4 a[2];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int d = 0; d < 4; ++d) {
+            const uint32_t* p = &image[(16 * ks2 + 8 * g + 2 * d) * kBsPitch + 16 * mt + (c >> 1)];
+            a[mt][d] = __builtin_amdgcn_perm(p[kBsPitch], p[0], pick);
+          }
+        // Up to 4 tiles: all fragments of Ma for this step first, one LDS latency per step
+        // instead of one per pair of tiles (with 7 tiles the registers do not reach)
+        if constexpr (NT <= 4) {
+          bs_u32x4 bq[NT];
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) bq[nt] = ma_frag[(ks * NT + nt) * kWave + l];
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const bs_bf16x8_t b = __builtin_bit_cast(bs_bf16x8_t, bq[nt]);
+            acc[0][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[0]), b,
+                                                                 acc[0][nt], 0, 0, 0);
+            acc[1][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[1]), b,
+                                                                 acc[1][nt], 0, 0, 0);
+          }
+        } else {
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            const bs_bf16x8_t b = __builtin_bit_cast(bs_bf16x8_t, ma_frag[(ks * NT + nt) * kWave + l]);
+            acc[0][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[0]), b,
+                                                                 acc[0][nt], 0, 0, 0);
+            acc[1][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[1]), b,
+                                                                 acc[1][nt], 0, 0, 0);
+          }
+        }
+      }
+    }
+    // butterflies over j = 32 mt + 8 b + 4 g + r
+    int64_t local;
+    const int j = bs_job(tab, run, &local);
+    uint16_t* __restrict__ yr = static_cast<uint16_t*>(tab.out[j]) + local * n;
+    const uint32_t h = g;  // after the exchange: lane half h holds j = 32 h ...
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      float u[2][16];  // u[x][4 b + r] = value at j = 32 h + 8 b + 4 x + r
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const float s = acc[0][nt][v] + acc[1][nt][v], t = acc[0][nt][v] - acc[1][nt][v];  // stage over mt
+        const auto pr = __builtin_amdgcn_permlane32_swap(__float_as_uint(s), __float_as_uint(t), false, false);
+        const float lower = __uint_as_float(pr[0]), upper = __uint_as_float(pr[1]);  // g = 0, g = 1
+        u[0][v] = lower + upper;
+        u[1][v] = lower - upper;
+      }
+#pragma unroll
+      for (int x = 0; x < 2; ++x)
+#pragma unroll
+        for (int st = 1; st < 16; st <<= 1)
+#pragma unroll
+          for (int v = 0; v < 16; ++v)
+            if ((v & st) == 0) {
+              const float p = u[x][v], m = u[x][v + st];
+              u[x][v] = p + m;
+              u[x][v + st] = p - m;
+            }
+      // row c of this tile, 32 outputs from column 32 h: 8 b + 4 x + r -> four vectors of 8
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        bs_u32x4 w;
+        w[0] = pack_bf16x2(u[0][4 * b] * scale, u[0][4 * b + 1] * scale);
+        w[1] = pack_bf16x2(u[0][4 * b + 2] * scale, u[0][4 * b + 3] * scale);
+        w[2] = pack_bf16x2(u[1][4 * b] * scale, u[1][4 * b + 1] * scale);
+        w[3] = pack_bf16x2(u[1][4 * b + 2] * scale, u[1][4 * b + 3] * scale);
+        *reinterpret_cast<bs_u32x4*>(&image[c * kBsPitch + 16 * h + 4 * b]) = w;
+      }
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = 32 * nt + (int)(l >> 3) + 8 * q;
+        bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
+        if constexpr (SIGNS == 2) w ^= flip[(nt * 4 + q) * kWave + l];
+        if (row < k_dim)
+          stg_nt<uint16_t, 8>(yr + 64 * row + 8 * (l & 7u), __builtin_bit_cast(Vec<uint16_t, 8>, w));
+      }
+    }
+  }
+}
+
+template <int NT, int SIGNS>
+int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
+                      hipStream_t st) {
+  auto kern = block_sylvester64_kernel<NT, SIGNS>;
+  constexpr size_t lds = bs_lds_bytes(NT, SIGNS != 0);
+  if (lds > 48 * 1024) {
+    // the attribute belongs to the kernel as loaded on one device; setting it again is cheap
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  // as many workgroups as are resident together (one per compute unit for K > 128, where a
+  // wavefront fills a SIMD's registers); every wavefront takes runs in turn
+  static int per_cu = 0;  // the same on every device of one process (one architecture)
+  int dev = 0, cus = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess && per_cu == 0) {
+    int n = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, kBsThreads, lds);
+    per_cu = n > 0 ? n : 1;
+  }
+  if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "device query: %s", hipGetErrorString(e));
+  const int64_t wgs = cdiv(tab.total, kBsWaves);
+  const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * per_cu;
+  const int64_t each = cdiv(wgs, cap);  // runs per wavefront, the same for all
+  const unsigned grid = (unsigned)cdiv(wgs, each);
+  hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale);
+  return CTMI_OK;
+}
+
+template <int NT>
+int launch_bs(const BsTable& tab, const uint16_t* ma_t, int k, const float* sign_in,
+              const float* sign_out, float scale, hipStream_t st) {
+  if (sign_in) return launch_bs_variant<NT, 1>(tab, ma_t, k, sign_in, scale, st);
+  if (sign_out) return launch_bs_variant<NT, 2>(tab, ma_t, k, sign_out, scale, st);
+  return launch_bs_variant<NT, 0>(tab, ma_t, k, nullptr, scale, st);
+}
+
+}  // namespace
+
+bool block_sylvester64_supported(int k, int io_dtype, bool both_signs) {
+  return io_dtype == CTMI_BF16 && k >= 1 && k <= 224 && !both_signs;
+}
+
+int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int k, const uint16_t* ma_t,
+                             const float* sign_in, const float* sign_out, float scale, hipStream_t st) {
+  CTMI_REQUIRE(block_sylvester64_supported(k, CTMI_BF16, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
+               "blocks of up to 224 x 224 with signs on one side");
+  CTMI_REQUIRE(n_jobs >= 1 && n_jobs <= kFwhtMaxJobs, CTMI_ERR_VALUE, "1 to %d tensors a launch", kFwhtMaxJobs);
+  CTMI_REQUIRE(ma_t && (uintptr_t)sign_in % 16 == 0 && (uintptr_t)sign_out % 16 == 0, CTMI_ERR_VALUE,
+               "the block must be given; sign vectors must be 16-byte aligned");
+  BsTable tab;
+  int64_t total = 0;
+  for (int i = 0; i < kFwhtMaxJobs; ++i) {
+    const bool live = i < n_jobs;
+    tab.x[i] = live ? jobs[i].x : nullptr;
+    tab.out[i] = live ? jobs[i].out : nullptr;
+    if (live) {
+      CTMI_REQUIRE(jobs[i].rows > 0 && jobs[i].x && jobs[i].out, CTMI_ERR_VALUE,
+                   "tensor %d: NULL pointer or no runs", i);
+      CTMI_REQUIRE((uintptr_t)jobs[i].x % 16 == 0 && (uintptr_t)jobs[i].out % 16 == 0, CTMI_ERR_VALUE,
+                   "tensors must be 16-byte aligned");
+      total += jobs[i].rows;
+    }
+    tab.end[i] = live ? total : INT64_MAX;
+  }
+  tab.total = total;
+  if (k <= 32) return launch_bs<1>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 64) return launch_bs<2>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 128) return launch_bs<4>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  return launch_bs<7>(tab, ma_t, k, sign_in, sign_out, scale, st);
+}
+
+}  // namespace ctmi

@@ -141,11 +141,19 @@ struct FwhtTable {
   int64_t total;
 };
 
+// (a run number is the same in all lanes of a workgroup, which the compiler cannot always see:
+// said outright, the search and the table reads behind it are scalar instructions; as vector
+// loads they would make every prefetch wait for all loads in flight)
 template <bool MANY>
 __device__ __forceinline__ int fwht_job(const FwhtTable& t, int64_t run, int64_t* local) {
   if constexpr (!MANY) {
     *local = run;
     return 0;
+  }
+  {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)run);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)run >> 32));
+    run = (int64_t)(((uint64_t)hi << 32) | lo);
   }
   int j = 0;
   int64_t first = 0;

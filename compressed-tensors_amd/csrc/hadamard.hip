@@ -23,6 +23,7 @@
 #include <atomic>
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "fwht.h"
 #include "qparams.h"
 #include "quant_core.h"
 #include "quant_fast.h"
@@ -1021,6 +1022,10 @@ extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_
   return 0;
 }
 
+extern "C" int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
+  return b_dim == 64 && a_dim > 1 && block_sylvester64_supported(a_dim, io_dtype, false);
+}
+
 extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel,
                                    int32_t a_dim, int32_t b_dim, const void* ma_t,
                                    const void* mb_t, const float* sign_in, const float* sign_out,
@@ -1033,6 +1038,14 @@ extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, i
   CTMI_REQUIRE(numel % n == 0, CTMI_ERR_VALUE,
                "tensor size %lld is not a multiple of the transform size %lld", (long long)numel,
                (long long)n);
+  if (!mb_t && a_dim > 1) {
+    // Mb = Sylvester(64): the product with Ma on the matrix cores, butterflies for Mb
+    ctmi_hadamard_job job;
+    job.x = x;
+    job.out = out;
+    job.numel = numel;
+    return ctmi_hadamard_apply_many(&job, 1, io_dtype, a_dim, b_dim, ma_t, mb_t, sign_in, sign_out, stream);
+  }
   CTMI_REQUIRE(ctmi_hadamard_supported(a_dim, b_dim, io_dtype), CTMI_ERR_UNSUPPORTED,
                "no MFMA kernel for the factorisation %d x %d with this dtype", a_dim, b_dim);
   if (numel == 0) return CTMI_OK;
@@ -1075,8 +1088,15 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
   CTMI_REQUIRE(a_dim >= 1 && b_dim >= 1, CTMI_ERR_VALUE, "bad factor sizes");
   CTMI_REQUIRE(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32,
                CTMI_ERR_UNSUPPORTED, "transforms take float16/bfloat16/float32 tensors");
-  CTMI_REQUIRE(ctmi_hadamard_supported(a_dim, b_dim, io_dtype), CTMI_ERR_UNSUPPORTED,
-               "no MFMA kernel for the factorisation %d x %d with this dtype", a_dim, b_dim);
+  const bool sylvester_inner = !mb_t && a_dim > 1;
+  if (sylvester_inner)
+    CTMI_REQUIRE(ctmi_hadamard_sylvester_inner_supported(a_dim, b_dim, io_dtype) && !(sign_in && sign_out),
+                 CTMI_ERR_UNSUPPORTED,
+                 "without mb_t (Mb = Sylvester's matrix): b_dim 64, a_dim up to 224, bfloat16 tensors, "
+                 "signs on one side; got %d x %d", a_dim, b_dim);
+  else
+    CTMI_REQUIRE(ctmi_hadamard_supported(a_dim, b_dim, io_dtype), CTMI_ERR_UNSUPPORTED,
+                 "no MFMA kernel for the factorisation %d x %d with this dtype", a_dim, b_dim);
   const int64_t n = (int64_t)a_dim * b_dim;
   // validate everything before anything is enqueued
   for (int64_t i = 0; i < n_jobs; ++i) {
@@ -1089,10 +1109,34 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
     CTMI_REQUIRE((uintptr_t)j.x % 16 == 0 && (uintptr_t)j.out % 16 == 0, CTMI_ERR_VALUE,
                  "tensors must be 16-byte aligned");
   }
-  CTMI_REQUIRE(n_jobs == 0 || (mb_t && (a_dim == 1 || ma_t)), CTMI_ERR_VALUE, "NULL matrix pointer");
+  CTMI_REQUIRE(n_jobs == 0 || ((mb_t || sylvester_inner) && (a_dim == 1 || ma_t)), CTMI_ERR_VALUE,
+               "NULL matrix pointer");
   CTMI_REQUIRE((uintptr_t)mb_t % 16 == 0 && (uintptr_t)ma_t % 16 == 0, CTMI_ERR_VALUE,
                "tensors must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
+  if (sylvester_inner) {
+    FwhtJob batch[kFwhtMaxJobs];
+    int filled = 0;
+    bool any = false;
+    for (int64_t i = 0; i <= n_jobs; ++i) {
+      if (i < n_jobs && jobs[i].numel > 0) {
+        FwhtJob& b = batch[filled++];
+        b.x = jobs[i].x;
+        b.out = jobs[i].out;
+        b.packed = nullptr;
+        b.scale = nullptr;
+        b.rows = jobs[i].numel / n;
+      }
+      if (filled == kFwhtMaxJobs || (i == n_jobs && filled)) {
+        const int rc = block_sylvester64_launch(batch, filled, a_dim, (const uint16_t*)ma_t, sign_in, sign_out,
+                                                1.0f / sqrtf((float)n), st);
+        if (rc) return rc;
+        filled = 0;
+        any = true;
+      }
+    }
+    return any ? check_launch("ctmi_hadamard_apply_many") : CTMI_OK;
+  }
   HadArgs a;
   a.x = nullptr;
   a.out = nullptr;

@@ -504,6 +504,13 @@ int ctmi_column_groups(const int32_t* g_idx, int64_t cols, int64_t group_size,
  * sign_out: fp32 [n] or NULL.  Runs on bf16 MFMA; ctmi_hadamard_supported says
  * which (a_dim, b_dim, dtype) combinations are built. */
 int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype);
+/* mb_t == NULL (with a_dim > 1) stands for Mb = Sylvester's matrix of order b_dim, the form of
+ * the reference's Hadamard matrices of size K * 2^m (transform/utils/hadamard.py:132-163: a
+ * known K x K block times butterflies).  Then only the product with Ma runs on the matrix
+ * cores (bf16 inputs: exact in one product) and Mb is butterfly stages on its fp32 result:
+ * b_dim 64, a_dim up to 224 (any block: 12 x 64 = 768 ... 224 x 64 = 14336), bfloat16
+ * tensors, signs on one side (ctmi_hadamard_sylvester_inner_supported). */
+int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype);
 int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t a_dim,
                         int32_t b_dim, const void* ma_t, const void* mb_t, const float* sign_in,
                         const float* sign_out, void* stream);
