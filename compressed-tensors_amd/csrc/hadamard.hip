@@ -78,6 +78,14 @@ __device__ __forceinline__ int had_job(const HadJobs& t, int64_t unit, int64_t* 
     *local = unit;
     return 0;
   }
+  {
+    // a wavefront's unit is the same in all its lanes, which the compiler cannot see: said
+    // outright, the search and the table reads behind it are scalar instructions (as vector
+    // loads they make the wavefront wait for every load it has in flight)
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)unit);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)unit >> 32));
+    unit = (int64_t)(((uint64_t)hi << 32) | lo);
+  }
   int j = 0;
   int64_t first = 0;
 #pragma unroll
