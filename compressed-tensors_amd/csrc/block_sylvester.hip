@@ -156,11 +156,13 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   // the spot): a run beyond the last reads the last again, a row beyond K reads row K - 1 and
   // is replaced by zeros when it is used.
   bs_u32x4 in[NT][4];
-  auto fetch = [&](int64_t r, int ch) {
+  auto run_start = [&](int64_t r) {  // where run r begins (table reads: once per run, not per chunk)
     r = r < tab.total ? r : tab.total - 1;
     int64_t local;
     const int j = bs_job(tab, r, &local);
-    const uint16_t* __restrict__ xr = static_cast<const uint16_t*>(tab.x[j]) + local * n;
+    return static_cast<const uint16_t*>(tab.x[j]) + local * n;
+  };
+  auto fetch = [&](const uint16_t* __restrict__ xr, int ch) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int row = 32 * ch + (int)(l >> 3) + 8 * q;
@@ -171,9 +173,13 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
 
   const int64_t step = (int64_t)gridDim.x * kBsWaves;
   int64_t run = (int64_t)blockIdx.x * kBsWaves + wave;
+  {
+    const uint16_t* first = run_start(run);
 #pragma unroll
-  for (int ch = 0; ch < NT; ++ch) fetch(run, ch);
+    for (int ch = 0; ch < NT; ++ch) fetch(first, ch);
+  }
   for (; run < tab.total; run += step) {
+    const uint16_t* next = run_start(run + step);
     bs_f32x16_t acc[2][NT];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -183,26 +189,38 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
 #pragma unroll
     for (int ch = 0; ch < NT; ++ch) {
+      // (LDS reads grouped ahead of the LDS writes they do not depend on: the compiler keeps
+      // accesses of the one shared array in program order, and every read that sits behind
+      // a write costs the wavefront a round trip of its own)
+      bs_u32x4 fl[SIGNS == 1 ? 4 : 1];
+      if constexpr (SIGNS == 1) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) fl[q] = flip[(ch * 4 + q) * kWave + l];
+      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         bs_u32x4 w = in[ch][q];
         if (32 * ch + (int)(l >> 3) + 8 * q >= k_dim) w = bs_u32x4{0u, 0u, 0u, 0u};
-        if constexpr (SIGNS == 1) w ^= flip[(ch * 4 + q) * kWave + l];
+        if constexpr (SIGNS == 1) w ^= fl[q];
         *reinterpret_cast<bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]) = w;
       }
-      fetch(run + step, ch);
+      fetch(next, ch);
+      // A operands of both steps and both M tiles: rows 16 ks2 + 8 g + e of the image,
+      // column 32 mt + c
+      bs_u32x4 a2[2][2];
 #pragma unroll
-      for (int ks2 = 0; ks2 < 2; ++ks2) {
-        const int ks = 2 * ch + ks2;
-        // A operands for both M tiles: rows 16 ks2 + 8 g + e of the image, column 32 mt + c
-        bs_u32x4 a[2];
+      for (int ks2 = 0; ks2 < 2; ++ks2)
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
           for (int d = 0; d < 4; ++d) {
             const uint32_t* p = &image[(16 * ks2 + 8 * g + 2 * d) * kBsPitch + 16 * mt + (c >> 1)];
-            a[mt][d] = __builtin_amdgcn_perm(p[kBsPitch], p[0], pick);
+            a2[ks2][mt][d] = __builtin_amdgcn_perm(p[kBsPitch], p[0], pick);
           }
+#pragma unroll
+      for (int ks2 = 0; ks2 < 2; ++ks2) {
+        const int ks = 2 * ch + ks2;
+        const bs_u32x4* a = a2[ks2];
         // Up to 4 tiles: all fragments of Ma for this step first, one LDS latency per step
         // instead of one per pair of tiles (with 7 tiles the registers do not reach)
         if constexpr (NT <= 4) {
@@ -267,11 +285,16 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         w[3] = pack_bf16x2(u[1][4 * b + 2] * scale, u[1][4 * b + 3] * scale);
         *reinterpret_cast<bs_u32x4*>(&image[c * kBsPitch + 16 * h + 4 * b]) = w;
       }
+      bs_u32x4 fo[SIGNS == 2 ? 4 : 1];
+      if constexpr (SIGNS == 2) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) fo[q] = flip[(nt * 4 + q) * kWave + l];
+      }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const int row = 32 * nt + (int)(l >> 3) + 8 * q;
         bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
-        if constexpr (SIGNS == 2) w ^= flip[(nt * 4 + q) * kWave + l];
+        if constexpr (SIGNS == 2) w ^= fo[q];
         if (row < k_dim)
           stg_nt<uint16_t, 8>(yr + 64 * row + 8 * (l & 7u), __builtin_bit_cast(Vec<uint16_t, 8>, w));
       }
