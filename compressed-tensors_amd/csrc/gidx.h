@@ -27,6 +27,16 @@ struct GidxArgs {
 
 constexpr int kGidxThreads = 256;
 
+// One activation-ordered weight of a pack-quantized launch: dense -> packed
+// (compress) or packed -> dense, `dense_dtype` the dense side's element type.
+struct GidxWeight {
+  const void* src;
+  void* dst;
+  int64_t rows, cols;
+  const ctmi_qparams* qp;
+  int dense_dtype;
+};
+
 // stage RB rows of scales (zero points) as fp32: lds_s[rb * s_cols + j]; with lds_r
 // also their reciprocals.  Returns whether a staged scale is outside the range
 // where the reciprocal path is exact.

@@ -20,6 +20,7 @@
 #include "quant_fast.h"
 #include "vec_geom.h"
 #include "job_table.h"
+#include "gidx.h"
 
 namespace ctmi {
 
@@ -457,10 +458,8 @@ extern "C" int ctmi_unpack_from_int32(const int32_t* in, int8_t* out, int64_t ro
 namespace ctmi {
 bool gidx_geometry(const ctmi_qparams* qp, int64_t rows, int64_t cols, int dense_dtype,
                    const void* dense, const void* packed);
-void gidx_launch_compress(const void* x, int x_dtype, int32_t* out, int64_t rows, int64_t cols,
-                          const ctmi_qparams* qp, hipStream_t st);
-void gidx_launch_decompress(const int32_t* packed, void* out, int64_t rows, int64_t cols,
-                            const ctmi_qparams* qp, hipStream_t st);
+bool gidx_same_launch(const GidxWeight& a, const GidxWeight& b, bool compress);
+void gidx_launch_many(const GidxWeight* w, int n, bool compress, hipStream_t st);
 }  // namespace ctmi
 
 // ---- pack-quantized compress / decompress: validate (no HIP call), then launch.
@@ -597,14 +596,27 @@ static int run_plans(PqPlan* plans, int64_t n, bool compress, hipStream_t st, co
   for (int64_t i = 0; i < n; ++i) {
     if (done[i] || plans[i].empty) continue;
     if (plans[i].gidx) {
-      const PqPlan& g = plans[i];
-      ++launches;
-      if (count_only) {
-      } else if (compress)
-        gidx_launch_compress(g.src, g.dense_dtype, (int32_t*)g.dst, g.rows, g.cols, &g.qp, st);
-      else
-        gidx_launch_decompress((const int32_t*)g.src, g.dst, g.rows, g.cols, &g.qp, st);
-      done[i] = 1;
+      // every remaining activation-ordered weight of the same template instance
+      auto weight = [&](int64_t k) {
+        const PqPlan& g = plans[k];
+        return GidxWeight{g.src, g.dst, g.rows, g.cols, &g.qp, g.dense_dtype};
+      };
+      GidxWeight w[kMaxJobs];
+      int m = 0;
+      auto flush_gidx = [&]() {
+        if (m == 0) return;
+        ++launches;
+        if (!count_only) gidx_launch_many(w, m, compress, st);
+        m = 0;
+      };
+      for (int64_t k = i; k < n; ++k) {
+        if (done[k] || plans[k].empty || !plans[k].gidx) continue;
+        if (k != i && !gidx_same_launch(weight(i), weight(k), compress)) continue;
+        if (m == kMaxJobs) flush_gidx();
+        w[m++] = weight(k);
+        done[k] = 1;
+      }
+      flush_gidx();
       continue;
     }
     if (!plans[i].vec) {

@@ -7,6 +7,7 @@
 // (and zero points) are staged in LDS as fp32 once and gathered from there, so the
 // only per-element global traffic is the dense / packed data itself, in 16-byte
 // pieces as in the column-ordered kernels.
+#include <algorithm>
 #include <type_traits>
 
 #include "ctmi_device.h"
@@ -14,8 +15,20 @@
 #include "quant_core.h"
 #include "quant_fast.h"
 #include "gidx.h"
+#include "job_table.h"
 
 namespace ctmi {
+
+// Kernel argument of a launch over up to kMaxJobs activation-ordered weights: the
+// head find_job_index reads (running totals of workgroups; the second row of
+// counts is not used here), then what each weight's workgroups need.
+struct GidxTable {
+  uint32_t chunk_end[kMaxJobs];
+  uint32_t unused[kMaxJobs];
+  GidxArgs job[kMaxJobs];
+};
+static_assert(offsetof(GidxTable, chunk_end) == 0 && offsetof(GidxTable, job) == 64,
+              "find_job_index reads the first 16 dwords of the kernel argument");
 
 // quantize + pack 8 elements, every element with its own scale / zero point: the
 // reference chain with one IEEE division per element
@@ -91,7 +104,9 @@ __device__ __forceinline__ Vec<typename ST::raw, 8> unpack_dequant8_each(
 }
 
 template <typename XT, typename ST, int BITS, bool HAS_ZP, int RB>
-__global__ void __launch_bounds__(kGidxThreads) pq_gidx_compress_kernel(GidxArgs a) {
+__global__ void __launch_bounds__(kGidxThreads) pq_gidx_compress_kernel(GidxTable t) {
+  uint32_t blk, unused;
+  const GidxArgs a = t.job[find_job_index(blockIdx.x, &blk, &unused)];
   using XR = typename XT::raw;
   constexpr int W = BITS / 4;
   constexpr bool kBf16 = XT::id == CTMI_BF16 && ST::id == CTMI_BF16;
@@ -99,7 +114,7 @@ __global__ void __launch_bounds__(kGidxThreads) pq_gidx_compress_kernel(GidxArgs
   float* lds_s = lds;
   float* lds_r = lds + RB * a.s_cols;
   float* lds_z = lds + 2 * RB * a.s_cols;
-  const uint32_t rowblk = blockIdx.x / a.tiles, tile = blockIdx.x - rowblk * a.tiles;
+  const uint32_t rowblk = blk / a.tiles, tile = blk - rowblk * a.tiles;
   const uint32_t row0 = rowblk * RB;
   const uint32_t cv = tile * kGidxThreads + threadIdx.x;
   const bool lane_ok = cv < a.vpr;
@@ -139,13 +154,15 @@ __global__ void __launch_bounds__(kGidxThreads) pq_gidx_compress_kernel(GidxArgs
 }
 
 template <typename ST, int BITS, bool HAS_ZP, int RB>
-__global__ void __launch_bounds__(kGidxThreads) pq_gidx_decompress_kernel(GidxArgs a) {
+__global__ void __launch_bounds__(kGidxThreads) pq_gidx_decompress_kernel(GidxTable t) {
+  uint32_t blk, unused;
+  const GidxArgs a = t.job[find_job_index(blockIdx.x, &blk, &unused)];
   using SR = typename ST::raw;
   constexpr int W = BITS / 4;
   extern __shared__ float lds[];
   float* lds_s = lds;
   float* lds_z = lds + RB * a.s_cols;
-  const uint32_t rowblk = blockIdx.x / a.tiles, tile = blockIdx.x - rowblk * a.tiles;
+  const uint32_t rowblk = blk / a.tiles, tile = blk - rowblk * a.tiles;
   const uint32_t row0 = rowblk * RB;
   const uint32_t cv = tile * kGidxThreads + threadIdx.x;
   const bool lane_ok = cv < a.vpr;
@@ -175,51 +192,59 @@ __global__ void __launch_bounds__(kGidxThreads) pq_gidx_decompress_kernel(GidxAr
   }
 }
 
+// One launch for the weights of a table; they share the template instance named by `key`.
+struct GidxKey {
+  int dense_dtype, scale_dtype, bits, rb;
+  bool has_zp;
+  bool operator==(const GidxKey& o) const {
+    return dense_dtype == o.dense_dtype && scale_dtype == o.scale_dtype && bits == o.bits &&
+           rb == o.rb && has_zp == o.has_zp;
+  }
+};
+
 template <typename XT, typename ST, int BITS, bool HAS_ZP>
-static void launch_gidx_compress_rb(const GidxArgs& a, int rb, size_t lds, hipStream_t st) {
-  const unsigned grid = (unsigned)(cdiv(a.rows, rb) * a.tiles);
-#define CTMI_G(RB) hipLaunchKernelGGL((pq_gidx_compress_kernel<XT, ST, BITS, HAS_ZP, RB>), grid, kGidxThreads, lds, st, a)
+static void launch_gidx_compress_rb(const GidxTable& t, int rb, unsigned grid, size_t lds, hipStream_t st) {
+#define CTMI_G(RB) hipLaunchKernelGGL((pq_gidx_compress_kernel<XT, ST, BITS, HAS_ZP, RB>), grid, kGidxThreads, lds, st, t)
   if (rb == 8) CTMI_G(8); else if (rb == 4) CTMI_G(4); else if (rb == 2) CTMI_G(2); else CTMI_G(1);
 #undef CTMI_G
 }
 
 template <typename ST, int BITS, bool HAS_ZP>
-static void launch_gidx_decompress_rb(const GidxArgs& a, int rb, size_t lds, hipStream_t st) {
-  const unsigned grid = (unsigned)(cdiv(a.rows, rb) * a.tiles);
-#define CTMI_G(RB) hipLaunchKernelGGL((pq_gidx_decompress_kernel<ST, BITS, HAS_ZP, RB>), grid, kGidxThreads, lds, st, a)
+static void launch_gidx_decompress_rb(const GidxTable& t, int rb, unsigned grid, size_t lds, hipStream_t st) {
+#define CTMI_G(RB) hipLaunchKernelGGL((pq_gidx_decompress_kernel<ST, BITS, HAS_ZP, RB>), grid, kGidxThreads, lds, st, t)
   if (rb == 8) CTMI_G(8); else if (rb == 4) CTMI_G(4); else if (rb == 2) CTMI_G(2); else CTMI_G(1);
 #undef CTMI_G
 }
 
 template <typename XT, typename ST>
-static void launch_gidx_compress_st(const GidxArgs& a, int bits, int rb, size_t lds, hipStream_t st) {
-  const bool has_zp = a.zp != nullptr;
-  if (bits == 4) {
-    if (has_zp) launch_gidx_compress_rb<XT, ST, 4, true>(a, rb, lds, st);
-    else launch_gidx_compress_rb<XT, ST, 4, false>(a, rb, lds, st);
+static void launch_gidx_compress_st(const GidxKey& k, const GidxTable& t, unsigned grid, size_t lds,
+                                    hipStream_t st) {
+  if (k.bits == 4) {
+    if (k.has_zp) launch_gidx_compress_rb<XT, ST, 4, true>(t, k.rb, grid, lds, st);
+    else launch_gidx_compress_rb<XT, ST, 4, false>(t, k.rb, grid, lds, st);
   } else {
-    if (has_zp) launch_gidx_compress_rb<XT, ST, 8, true>(a, rb, lds, st);
-    else launch_gidx_compress_rb<XT, ST, 8, false>(a, rb, lds, st);
+    if (k.has_zp) launch_gidx_compress_rb<XT, ST, 8, true>(t, k.rb, grid, lds, st);
+    else launch_gidx_compress_rb<XT, ST, 8, false>(t, k.rb, grid, lds, st);
   }
 }
 
 template <typename XT>
-static void launch_gidx_compress_xt(const GidxArgs& a, int scale_dtype, int bits, int rb,
-                                    size_t lds, hipStream_t st) {
-  if (scale_dtype == CTMI_BF16) launch_gidx_compress_st<XT, BF16>(a, bits, rb, lds, st);
-  else if (scale_dtype == CTMI_F16) launch_gidx_compress_st<XT, F16>(a, bits, rb, lds, st);
-  else launch_gidx_compress_st<XT, F32>(a, bits, rb, lds, st);
+static void launch_gidx_compress_xt(const GidxKey& k, const GidxTable& t, unsigned grid, size_t lds,
+                                    hipStream_t st) {
+  if (k.scale_dtype == CTMI_BF16) launch_gidx_compress_st<XT, BF16>(k, t, grid, lds, st);
+  else if (k.scale_dtype == CTMI_F16) launch_gidx_compress_st<XT, F16>(k, t, grid, lds, st);
+  else launch_gidx_compress_st<XT, F32>(k, t, grid, lds, st);
 }
 
 template <typename ST>
-static void launch_gidx_decompress_st(const GidxArgs& a, int bits, int rb, size_t lds, hipStream_t st) {
-  const bool has_zp = a.zp != nullptr;
-  if (bits == 4) {
-    if (has_zp) launch_gidx_decompress_rb<ST, 4, true>(a, rb, lds, st);
-    else launch_gidx_decompress_rb<ST, 4, false>(a, rb, lds, st);
+static void launch_gidx_decompress_st(const GidxKey& k, const GidxTable& t, unsigned grid, size_t lds,
+                                      hipStream_t st) {
+  if (k.bits == 4) {
+    if (k.has_zp) launch_gidx_decompress_rb<ST, 4, true>(t, k.rb, grid, lds, st);
+    else launch_gidx_decompress_rb<ST, 4, false>(t, k.rb, grid, lds, st);
   } else {
-    if (has_zp) launch_gidx_decompress_rb<ST, 8, true>(a, rb, lds, st);
-    else launch_gidx_decompress_rb<ST, 8, false>(a, rb, lds, st);
+    if (k.has_zp) launch_gidx_decompress_rb<ST, 8, true>(t, k.rb, grid, lds, st);
+    else launch_gidx_decompress_rb<ST, 8, false>(t, k.rb, grid, lds, st);
   }
 }
 
@@ -260,30 +285,68 @@ static GidxArgs gidx_args(const ctmi_qparams* qp, int64_t rows, int64_t cols) {
   return a;
 }
 
-void gidx_launch_compress(const void* x, int x_dtype, int32_t* out, int64_t rows, int64_t cols,
-                          const ctmi_qparams* qp, hipStream_t st) {
-  GidxArgs a = gidx_args(qp, rows, cols);
-  a.dense = x;
-  a.packed_out = out;
-  const int arrays = qp->zero_point ? 3 : 2;
-  const int rb = gidx_rows_per_block(qp->s_cols, arrays);
-  const size_t lds = (size_t)rb * qp->s_cols * 4 * arrays;
-  if (x_dtype == CTMI_BF16) launch_gidx_compress_xt<BF16>(a, qp->scale_dtype, qp->num_bits, rb, lds, st);
-  else if (x_dtype == CTMI_F16) launch_gidx_compress_xt<F16>(a, qp->scale_dtype, qp->num_bits, rb, lds, st);
-  else launch_gidx_compress_xt<F32>(a, qp->scale_dtype, qp->num_bits, rb, lds, st);
+static GidxKey gidx_key(const GidxWeight& w, bool compress) {
+  const int arrays = (compress ? 2 : 1) + (w.qp->zero_point ? 1 : 0);
+  return GidxKey{w.dense_dtype, w.qp->scale_dtype, w.qp->num_bits,
+                 gidx_rows_per_block(w.qp->s_cols, arrays), w.qp->zero_point != nullptr};
 }
 
-void gidx_launch_decompress(const int32_t* packed, void* out, int64_t rows, int64_t cols,
-                            const ctmi_qparams* qp, hipStream_t st) {
-  GidxArgs a = gidx_args(qp, rows, cols);
-  a.dense = out;
-  a.packed_in = packed;
-  const int arrays = qp->zero_point ? 2 : 1;
-  const int rb = gidx_rows_per_block(qp->s_cols, arrays);
-  const size_t lds = (size_t)rb * qp->s_cols * 4 * arrays;
-  if (qp->scale_dtype == CTMI_BF16) launch_gidx_decompress_st<BF16>(a, qp->num_bits, rb, lds, st);
-  else if (qp->scale_dtype == CTMI_F16) launch_gidx_decompress_st<F16>(a, qp->num_bits, rb, lds, st);
-  else launch_gidx_decompress_st<F32>(a, qp->num_bits, rb, lds, st);
+// Do two weights run in the same template instance (and so may share a launch)?
+bool gidx_same_launch(const GidxWeight& a, const GidxWeight& b, bool compress) {
+  return gidx_key(a, compress) == gidx_key(b, compress);
+}
+
+// Enqueue up to kMaxJobs weights that gidx_geometry accepted and gidx_same_launch
+// groups, as one launch.  Weights are cut so that the grid stays below 2^31 workgroups.
+void gidx_launch_many(const GidxWeight* w, int n, bool compress, hipStream_t st) {
+  const GidxKey key = gidx_key(w[0], compress);
+  const int arrays = (compress ? 2 : 1) + (key.has_zp ? 1 : 0);
+  GidxTable t;
+  auto reset = [&]() {
+    for (int k = 0; k < kMaxJobs; ++k) {
+      t.chunk_end[k] = 0xFFFFFFFFu;
+      t.unused[k] = 0;
+      t.job[k] = GidxArgs{};
+    }
+  };
+  int filled = 0;
+  uint64_t groups = 0;
+  size_t lds = 0;
+  auto flush = [&]() {
+    if (filled == 0) return;
+    if (compress) {
+      if (key.dense_dtype == CTMI_BF16) launch_gidx_compress_xt<BF16>(key, t, (unsigned)groups, lds, st);
+      else if (key.dense_dtype == CTMI_F16) launch_gidx_compress_xt<F16>(key, t, (unsigned)groups, lds, st);
+      else launch_gidx_compress_xt<F32>(key, t, (unsigned)groups, lds, st);
+    } else {
+      if (key.scale_dtype == CTMI_BF16) launch_gidx_decompress_st<BF16>(key, t, (unsigned)groups, lds, st);
+      else if (key.scale_dtype == CTMI_F16) launch_gidx_decompress_st<F16>(key, t, (unsigned)groups, lds, st);
+      else launch_gidx_decompress_st<F32>(key, t, (unsigned)groups, lds, st);
+    }
+    filled = 0;
+    groups = 0;
+    lds = 0;
+    reset();
+  };
+  reset();
+  for (int i = 0; i < n; ++i) {
+    GidxArgs a = gidx_args(w[i].qp, w[i].rows, w[i].cols);
+    if (compress) {
+      a.dense = w[i].src;
+      a.packed_out = (int32_t*)w[i].dst;
+    } else {
+      a.packed_in = (const int32_t*)w[i].src;
+      a.dense = w[i].dst;
+    }
+    const uint64_t mine = (uint64_t)cdiv(w[i].rows, key.rb) * a.tiles;
+    if (filled == kMaxJobs || groups + mine >= (1ull << 31)) flush();
+    t.job[filled] = a;
+    groups += mine;
+    t.chunk_end[filled] = (uint32_t)groups;
+    lds = std::max(lds, (size_t)key.rb * w[i].qp->s_cols * 4 * arrays);
+    ++filled;
+  }
+  flush();
 }
 
 // ------------------------------------------------------------------ g_idx -> group of a column

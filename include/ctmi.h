@@ -147,7 +147,8 @@ typedef struct ctmi_weight_job {
  * decompress_from_state_dict (compressors/quantized_compressors/base.py:91-125,
  * 213-230) for the pack-quantized format: n fused launches from one call.
  * Every job is validated before anything is enqueued; weights that share a
- * dtype / bit-width combination are chained into common launches. */
+ * dtype / bit-width combination are chained into common launches, 8 per launch;
+ * activation-ordered weights (qp.col_group set) likewise, among themselves. */
 int ctmi_pack_quantized_compress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
 int ctmi_pack_quantized_decompress_many(const ctmi_weight_job* jobs, int64_t n, void* stream);
 /* Number of kernel launches the call above (compress != 0) or its inverse

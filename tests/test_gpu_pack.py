@@ -320,6 +320,48 @@ def test_pack_quantized_with_activation_ordering(spec, shape, dtype, sdt, gpu):
     assert_bit_equal(dense, dense_want, "decompress")
 
 
+def test_activation_ordered_weights_share_launches(gpu):
+    """a batch of activation-ordered weights (more than one launch holds, two scale dtypes,
+    with and without zero points, ragged shapes): the shared launches give the bytes of the
+    per-weight calls, for compress and for decompress"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.compressors.pack_quantized import PackedWeightBatch
+
+    announce("pack-quantized g_idx, many weights per launch")
+    sym = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    asym = dict(sym, symmetric=False, group_size=64)
+    eight = dict(sym, num_bits=8, group_size=32)
+    cases = [(sym, (33, 1024), torch.bfloat16)] * 2 + [(asym, (17, 512), torch.bfloat16),
+             (sym, (5, 4096), torch.bfloat16), (eight, (12, 288), torch.bfloat16),
+             (sym, (64, 2048), torch.float16), (asym, (40, 2112), torch.bfloat16)]
+    cases += [(sym, (r, 1280), torch.bfloat16) for r in (1, 2, 3, 7, 8, 9, 31, 64, 65)]
+    g = torch.Generator().manual_seed(35)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    entries, singles = [], []
+    for spec, shape, dtype in cases:
+        args, oargs = _pair(spec)
+        w = (torch.randn(shape, generator=g) * 0.02).to(dtype)
+        g_idx = (torch.randperm(shape[1], generator=g) // spec["group_size"]).to(torch.int32)
+        scale, zp = oq.observe_weight(w.index_select(-1, torch.argsort(g_idx)), oargs)
+        zp = None if spec["symmetric"] else zp
+        entry = dict(weight=w.to(gpu), scale=scale.to(gpu), quantization_args=args,
+                     g_idx=g_idx.to(gpu), **({} if zp is None else {"zero_point": zp.to(gpu)}))
+        entries.append(entry)
+        single = comp.compress_weight(**entry)
+        dense = comp.decompress_weight(dict(single, weight_scale=entry["scale"], weight_g_idx=entry["g_idx"]),
+                                       quantization_args=args)
+        singles.append((single["weight_packed"], dense))
+    batch = PackedWeightBatch(entries)
+    # 12 symmetric bf16 4-bit weights in 2 launches, one launch for each other kind
+    assert batch.launches(True) == 5 and batch.launches(False) == 5
+    for _ in range(2):
+        packed = batch.compress()
+        dense = batch.decompress()
+        for i, (want_packed, want_dense) in enumerate(singles):
+            assert_bit_equal(packed[i], want_packed, f"packed {i}")
+            assert_bit_equal(dense[i], want_dense, f"dense {i}")
+
+
 def test_activation_ordering_with_any_int32_group_labels(gpu):
     """g_idx values are only ever sorted (forward.py:286-289), so labels beyond 32767 and
     negative ones other than -1 must group the columns like small ones; a -1 anywhere
