@@ -42,13 +42,16 @@ constexpr int kS24U = CTMI_S24_U;  // compress
 constexpr int kS24ScatterU = CTMI_S24_SCATTER_U;  // decompress
 
 // ------------------------------------------------------------------ block scan
+// Inclusive prefix sum over the wavefront with data-parallel-primitive moves: shifts
+// inside rows of 16 lanes (lanes without a source add zero), then lane 15 of rows 0
+// and 2 into rows 1 and 3, then lane 31 into rows 2 and 3.  No LDS crossbar trips.
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
-  const int lane = lane_id();
-#pragma unroll
-  for (int d = 1; d < kWave; d <<= 1) {
-    const int t = __shfl_up(v, d, kWave);
-    if (lane >= d) v += t;
-  }
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xf, 0xf, true);   // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xf, 0xf, true);   // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xf, 0xf, true);   // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xf, 0xf, true);   // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false);  // row_bcast:15
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false);  // row_bcast:31
   return v;
 }
 
@@ -638,12 +641,7 @@ static bool scatter_wave_ok(const void* values, const uint8_t* bitmask, const vo
 // where each tile's values start, and the scatter then knows before it has looked
 // at anything which values a tile needs: it fetches them together with the tile's
 // bitmask, stages them in LDS and every lane picks its own.
-#ifndef CTMI_TILE_U
-#define CTMI_TILE_U 1
-#endif
-constexpr int kTileU = CTMI_TILE_U;            // 16-element items per lane
-constexpr int kTileItems = kBlock * kTileU;
-constexpr int kTileElems = kTileItems * 16;
+constexpr int kTileElems = kBlock * 16;        // 16 elements per lane of the scatter
 constexpr int kTileBytes = kTileElems / 8;     // bitmask bytes per tile
 
 __global__ void __launch_bounds__(kBlock)
@@ -671,10 +669,11 @@ tile_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
 }
 
 // The same count for tensors of up to kGroupTiles * kMaxGroups tiles, without the
-// scan in between: a workgroup counts a group of kGroupTiles neighbouring tiles
-// and leaves, per tile, the count of the group's earlier tiles and its own, and per
-// group its total; a scatter workgroup adds up the totals of the groups before its
-// own by itself (at most kMaxGroups words, from L2).
+// scan kernel in between: a workgroup counts a group of kGroupTiles neighbouring
+// tiles and leaves, per tile, the count of the group's earlier tiles and its own, and
+// per group its total; the workgroup that finishes last (a ticket drawn with an
+// atomic, no waiting) turns the totals into the set bits before each group.  A
+// scatter workgroup then finds its place with two scalar loads.
 constexpr int kGroupTiles = 64;
 constexpr int kGroupThreads = 1024;
 constexpr int kMaxGroups = 1024;
@@ -683,12 +682,28 @@ struct TileInfo {
   int32_t count;   // set bits in the tile
 };
 
+// Which workgroup of the count is the last to finish: kTicketSlots counters in device
+// memory of the library, zero between launches (the last workgroup puts its counter
+// back).  Launches take them in turn, so launches in flight at the same time (other
+// streams) do not share one unless there are kTicketSlots of them.
+constexpr int kTicketSlots = 256;
+__device__ unsigned int popcount_ticket[kTicketSlots];
+
+static uint32_t next_ticket_slot() {
+  static std::atomic<uint32_t> ticket{0};
+  return ticket.fetch_add(1, std::memory_order_relaxed) % kTicketSlots;
+}
+
+static_assert(kGroupThreads >= kMaxGroups, "the last workgroup scans one group total per thread");
+
 __global__ void __launch_bounds__(kGroupThreads)
 tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
                             TileInfo* __restrict__ info, int32_t* __restrict__ group_total,
-                            int64_t ntiles) {
+                            int32_t* __restrict__ group_before, int64_t ntiles, uint32_t slot) {
   constexpr int kPerWave = kGroupTiles / (kGroupThreads / kWave);  // tiles per wavefront
   __shared__ int cnt_s[kGroupTiles];
+  __shared__ int wsum_s[kGroupThreads / kWave];
+  __shared__ int last_s;
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int64_t tile0 = (int64_t)blockIdx.x * kGroupTiles;
   int cnt[kPerWave];
@@ -720,111 +735,165 @@ tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
     const int c = cnt_s[lane];
     const int inc = wave_inclusive_scan(c);
     if (tile0 + lane < ntiles) info[tile0 + lane] = TileInfo{inc - c, c};
-    if (lane == kWave - 1) group_total[blockIdx.x] = inc;
+    if (lane == kWave - 1) {
+      // the total goes out for the other workgroups of this launch to read, then the
+      // ticket: whoever draws the last one sees every total
+      __hip_atomic_store(&group_total[blockIdx.x], inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned int drawn = __hip_atomic_fetch_add(&popcount_ticket[slot], 1u, __ATOMIC_ACQ_REL,
+                                                        __HIP_MEMORY_SCOPE_AGENT);
+      last_s = drawn == gridDim.x - 1;
+    }
   }
+  __syncthreads();
+  if (!last_s) return;
+  // the last workgroup: set bits before each group, one group per thread
+  const int g = threadIdx.x;
+  const int t = g < (int)gridDim.x
+                    ? __hip_atomic_load(&group_total[g], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                    : 0;
+  const int inc = wave_inclusive_scan(t);
+  if (lane == kWave - 1) wsum_s[wave] = inc;
+  __syncthreads();
+  int before = inc - t;
+#pragma unroll
+  for (int w = 0; w < kGroupThreads / kWave; ++w) before += w < wave ? wsum_s[w] : 0;
+  if (g < (int)gridDim.x) group_before[g] = before;
+  if (threadIdx.x == 0)
+    __hip_atomic_store(&popcount_ticket[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Set bits beyond nvalues read as zero.  GROUPED: positions from
-// tile_popcount_groups_kernel (info, group_total), else from tile_popcount_kernel
+// tile_popcount_groups_kernel (info, group_before), else from tile_popcount_kernel
 // and the scan behind it (tile_counts, tile_offsets).
+//
+// A wavefront takes 1024 neighbouring elements of the tile, as 16-byte pieces: piece q
+// of lane l is elements [q * 64 * VE + l * VE, + VE) of the stretch, so that every
+// store instruction of the wavefront writes 1 KB without gaps (whole memory lines; with
+// a lane's 16 elements side by side a store would leave every other 16 bytes to the
+// next one, and the device moves such halves noticeably slower).
 template <typename R, bool GROUPED>
 __global__ void __launch_bounds__(kBlock)
 bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
-                             const uint16_t* __restrict__ words,
+                             const uint8_t* __restrict__ bitmask,
                              const int64_t* __restrict__ tile_counts,
                              const int64_t* __restrict__ tile_offsets,
                              const TileInfo* __restrict__ info,
-                             const int32_t* __restrict__ group_total, R* __restrict__ out,
-                             int64_t n_items) {
-  constexpr int E = 16, U = kTileU;
-  constexpr int VE = 16 / (int)sizeof(R);
-  __shared__ int wtot[U][kWaves];
-  __shared__ __align__(16) R stage[kTileElems + 2 * VE];
+                             const int32_t* __restrict__ group_before, R* __restrict__ out,
+                             int64_t numel) {
+  constexpr int VE = 16 / (int)sizeof(R);  // elements of a piece
+  constexpr int NP = 16 / VE;              // pieces of a lane
+  constexpr int P = (NP + 1) / 2;
+  static_assert(kTileElems == kWaves * kWave * 16, "1024 elements per wavefront");
+  __shared__ int wtot[kWaves];
+  // the tile's values, up to VE - 1 before them and room for the reads of unset
+  // elements behind the last one
+  __shared__ __align__(16) R stage[kTileElems + 2 * VE + 16];
   const int tid = threadIdx.x, lane = lane_id(), wave = tid / kWave;
   const int64_t tile = blockIdx.x;
-  const int64_t item0 = tile * kTileItems;
   int64_t excl;
   int total;
   if constexpr (GROUPED) {
-    // every wavefront adds up the earlier groups by itself: no barrier
-    const int group = (int)(tile / kGroupTiles);
-    int64_t before = 0;
-    for (int g = lane; g < group; g += kWave) before += group_total[g];
-#pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) before += __shfl_xor(before, d, kWave);
     const TileInfo ti = info[tile];
-    excl = before + ti.before;
+    excl = (int64_t)group_before[tile / kGroupTiles] + ti.before;
     total = ti.count;
   } else {
     excl = tile_offsets[tile];
     total = (int)tile_counts[tile];
   }
 
-  uint32_t bits[U];
+  // the lane's pieces and their bits (numel is a multiple of 16: a piece is inside
+  // the tensor as a whole or not at all)
+  const int64_t elem0 = tile * kTileElems + wave * (kWave * 16) + lane * VE;
+  uint32_t bits[NP];
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const int64_t item = item0 + k * kBlock + tid;
-    bits[k] = item < n_items ? (uint32_t)words[item] : 0u;
+  for (int q = 0; q < NP; ++q) {
+    const int64_t elem = elem0 + q * (kWave * VE);
+    bits[q] = 0;
+    if (elem < numel) {
+      if constexpr (VE == 16) bits[q] = reinterpret_cast<const uint16_t*>(bitmask)[elem >> 4];
+      else bits[q] = ((uint32_t)bitmask[elem >> 3] >> (elem & 7)) & ((1u << VE) - 1u);
+    }
   }
-  // values [excl, excl + total) -> LDS, from the 16-byte boundary below excl
+  // values [excl, excl + total) -> LDS, from the 16-byte boundary below excl; lanes
+  // count in elements from there, `have` of which exist
   const int64_t base = excl & ~(int64_t)(VE - 1);
   const int off = (int)(excl - base);
   const int nvecs = (off + total + VE - 1) / VE;
+  const int64_t left = nvalues - base;
+  const int have = (int)(left < 0 ? 0 : left > kTileElems + 2 * VE ? kTileElems + 2 * VE : left);
+  const R* from = values + base;
   for (int i = tid; i < nvecs; i += kBlock) {
-    const int64_t e0 = base + (int64_t)i * VE;
+    const int e0 = i * VE;
     Vec<R, VE> v;
-    if (e0 < nvalues) {
+#pragma unroll
+    for (int e = 0; e < VE; ++e) v.v[e] = (R)0;
+    if (e0 < have) {
       // an aligned vector that starts inside the buffer never leaves its page
-      v = ldg<R, VE>(values + e0);
+      v = ldg<R, VE>(from + e0);
+      if (e0 + VE > have) {  // set bits beyond the values read as zero
 #pragma unroll
-      for (int e = 0; e < VE; ++e)
-        if (e0 + e >= nvalues) v.v[e] = (R)0;
-    } else {
-#pragma unroll
-      for (int e = 0; e < VE; ++e) v.v[e] = (R)0;
+        for (int e = 0; e < VE; ++e)
+          if (e0 + e >= have) v.v[e] = (R)0;
+      }
     }
-    *reinterpret_cast<Vec<R, VE>*>(stage + i * VE) = v;
+    *reinterpret_cast<Vec<R, VE>*>(stage + e0) = v;
   }
-  // ranks: item k of a lane comes after every item k' < k and after item k of the lanes below
-  int cnt[U], inc[U], pre[U];
+  // Ranks.  In the tile's order a wavefront's piece q of all lanes comes before its
+  // piece q + 1.  Two pieces' counts ride through one scan as 16-bit fields.
+  int first[NP];
+  int wave_total = 0;
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    cnt[k] = __popc(bits[k]);
-    inc[k] = wave_inclusive_scan(cnt[k]);
-    if (lane == kWave - 1) wtot[k][wave] = inc[k];
+  for (int p = 0; p < P; ++p) {
+    uint32_t cnt2 = (uint32_t)__popc(bits[2 * p]);
+    if (2 * p + 1 < NP) cnt2 |= (uint32_t)__popc(bits[2 * p + 1]) << 16;
+    const uint32_t inc2 = (uint32_t)wave_inclusive_scan((int)cnt2);
+    const uint32_t all2 = (uint32_t)__builtin_amdgcn_readlane((int)inc2, kWave - 1);
+    const uint32_t below2 = inc2 - cnt2;
+    first[2 * p] = wave_total + (int)(below2 & 0xffffu);
+    wave_total += (int)(all2 & 0xffffu);
+    if (2 * p + 1 < NP) {
+      first[2 * p + 1] = wave_total + (int)(below2 >> 16);
+      wave_total += (int)(all2 >> 16);
+    }
   }
+  if (lane == 0) wtot[wave] = wave_total;
   __syncthreads();
-  int before = 0;
+  int before = off;
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    int mine = before;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const int s = wtot[k][w];
-      if (w < wave) mine += s;
-      before += s;
-    }
-    pre[k] = mine + inc[k] - cnt[k];
+  for (int w = 0; w < kWaves; ++w) {
+    const int t = wtot[w];
+    before += w < wave ? t : 0;
   }
+  // Element j of a piece is value number popcount(bits below j) of the piece's if bit j
+  // is set.  Every element is read, set or not (the place is inside the staged image
+  // either way), and cleared by a mask afterwards: no branch per element.
 #pragma unroll
-  for (int k = 0; k < U; ++k) {
-    const int64_t item = item0 + k * kBlock + tid;
-    if (item < n_items) {
-      int idx = off + pre[k];
-      Vec<R, E> o;
+  for (int q = 0; q < NP; ++q) {
+    const int64_t elem = elem0 + q * (kWave * VE);
+    if (elem < numel) {
+      const uint32_t mine = bits[q];
+      const int at = before + first[q];
+      Vec<R, VE> o;
+      if constexpr (sizeof(R) == 2) {
+        uint32_t w2[VE / 2];
 #pragma unroll
-      for (int j = 0; j < E; ++j) {
-        const bool set = (bits[k] >> j) & 1u;
-        o.v[j] = set ? stage[idx] : (R)0;
-        idx += set ? 1 : 0;
+        for (int h = 0; h < VE / 2; ++h) {
+          const uint32_t lo = stage[at + __popc(mine & ((1u << (2 * h)) - 1u))];
+          const uint32_t hi = stage[at + __popc(mine & ((1u << (2 * h + 1)) - 1u))];
+          const uint32_t keep_lo = (uint32_t)((int32_t)(mine << (31 - 2 * h)) >> 31);
+          const uint32_t keep_hi = (uint32_t)((int32_t)(mine << (30 - 2 * h)) >> 31);
+          w2[h] = (lo | (hi << 16)) & ((keep_lo & 0xffffu) | (keep_hi & 0xffff0000u));
+        }
+        o = __builtin_bit_cast(Vec<R, VE>, w2);
+      } else {
+#pragma unroll
+        for (int j = 0; j < VE; ++j) {
+          const R v = stage[at + __popc(mine & ((1u << j) - 1u))];
+          const R keep = (R)(0 - (R)((mine >> j) & 1u));
+          o.v[j] = v & keep;
+        }
       }
-#pragma unroll
-      for (int h = 0; h < E / VE; ++h) {
-        Vec<R, VE> part;
-#pragma unroll
-        for (int e = 0; e < VE; ++e) part.v[e] = o.v[h * VE + e];
-        stg_nt<R, VE>(out + item * E + h * VE, part);
-      }
+      stg_nt<R, VE>(out + elem, o);
     }
   }
 }
@@ -1694,9 +1763,7 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
       (uintptr_t)values % 16 == 0 && (uintptr_t)bitmask % 16 == 0 && (uintptr_t)tmp % 8 == 0 &&
       cdiv(numel, kTileElems) < (1ll << 31)) {
     // positions from the bitmask alone, as in the reference (sparse_bitmask.py:152-169)
-    const int64_t n_items = numel / 16;
-    const int64_t ntiles = cdiv(n_items, kTileItems);
-    const uint16_t* words = reinterpret_cast<const uint16_t*>(bitmask);
+    const int64_t ntiles = cdiv(numel, kTileElems);
     const int64_t ngroups = cdiv(ntiles, kGroupTiles);
     int64_t* counts = nullptr;
     int64_t* offs = nullptr;
@@ -1705,9 +1772,10 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
     const bool grouped = ngroups <= kMaxGroups;
     if (grouped) {
       info = (TileInfo*)tmp;
-      totals = (int32_t*)(info + ntiles);
+      int32_t* group_totals = (int32_t*)(info + ntiles);
+      totals = group_totals + ngroups;  // set bits before each group
       hipLaunchKernelGGL(tile_popcount_groups_kernel, (unsigned)ngroups, kGroupThreads, 0, st,
-                         bitmask, rows * pc, info, totals, ntiles);
+                         bitmask, rows * pc, info, group_totals, totals, ntiles, next_ticket_slot());
     } else {
       counts = (int64_t*)tmp;
       offs = counts + ntiles;
@@ -1719,12 +1787,12 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
 #define CTMI_TILES(R)                                                                              \
   if (grouped)                                                                                     \
     hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, true>), (unsigned)ntiles, kBlock, 0, st,   \
-                       (const R*)values, nvalues, words, counts, offs, info, totals, (R*)out,      \
-                       n_items);                                                                   \
+                       (const R*)values, nvalues, bitmask, counts, offs, info, totals, (R*)out,    \
+                       numel);                                                                     \
   else                                                                                             \
     hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, false>), (unsigned)ntiles, kBlock, 0, st,  \
-                       (const R*)values, nvalues, words, counts, offs, info, totals, (R*)out,      \
-                       n_items)
+                       (const R*)values, nvalues, bitmask, counts, offs, info, totals, (R*)out,    \
+                       numel)
     if (elem_size == 1) { CTMI_TILES(uint8_t); }
     else if (elem_size == 2) { CTMI_TILES(uint16_t); }
     else { CTMI_TILES(uint32_t); }

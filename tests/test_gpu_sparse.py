@@ -299,6 +299,35 @@ def test_bitmask_many_tiles(gpu):
                          osp.bitmask_decompress(o_values, o_bitmask, list(shape)), "decompress")
 
 
+@pytest.mark.parametrize("dtype,shape", [(torch.bfloat16, (8192, 4096)), (FP8, (4096, 8192)),
+                                         (torch.float32, (2048, 4096)), (torch.bfloat16, (2048, 4096))],
+                         ids=["bf16", "fp8", "f32", "bf16-one-tile-per-workgroup"])
+def test_bitmask_decompress_runs_of_tiles(dtype, shape, gpu):
+    """tensors of more scatter tiles than workgroups fit the device at once: a workgroup then
+    walks a run of neighbouring tiles and takes every tile's place from the one before.
+    Row blocks that are empty, full, half and nearly empty; all values, and fewer values
+    than set bits (the rest reads as zero).  Expected tensors are built with torch."""
+    from compressed_tensors_amd.compressors import bitmask_compress, bitmask_decompress
+
+    announce("bitmask decompress, runs of tiles", dtype, shape)
+    rows, cols = shape
+    g = torch.Generator(device=gpu).manual_seed(11)
+    x = torch.randint(1, 120, (rows, cols), generator=g, device=gpu).to(torch.float32)
+    keep_prob = torch.tensor([0.0, 1.0, 0.5, 0.1, 0.97, 0.5, 0.0, 0.5], device=gpu)
+    block = keep_prob[(torch.arange(rows, device=gpu) * 8 // rows)].unsqueeze(1)
+    x = torch.where(torch.rand((rows, cols), generator=g, device=gpu) < block, x, torch.zeros_like(x))
+    x = x.to(dtype)
+    values, bitmask, _ = bitmask_compress(x)
+    nz = (x.float() != 0).flatten()
+    assert values.numel() == int(nz.sum())
+    assert_bit_equal(bitmask_decompress(values, bitmask, list(shape)), x, "all values")
+    rank = torch.cumsum(nz.to(torch.int64), 0) - 1
+    for keep in (values.numel() - 3, values.numel() // 2 + 5, 4097):
+        want = torch.where((nz & (rank < keep)).view(shape), x.float(), torch.zeros((), device=gpu)).to(dtype)
+        got = bitmask_decompress(values[:keep].clone(), bitmask, list(shape))
+        assert_bit_equal(got, want, f"first {keep} values")
+
+
 def test_bitmask_decompress_of_a_very_large_tensor(gpu):
     """more tiles than the grouped count handles (> 65536 tiles of 8192 elements): the scatter
     then takes its positions from a scan over all tiles.  Round trip on the GPU, values and
