@@ -295,9 +295,35 @@ bitmask_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t* __restrict
                 (int64_t)gridDim.x * kWaves);
 }
 
-// exclusive scan of counts[rows] -> offsets[rows], total; single workgroup, 8
-// neighbouring rows per thread and step
+// exclusive scan of counts[rows] -> offsets[rows], total; single workgroup.  A
+// wavefront takes 512 neighbouring rows per step, 64 at a time (lanes side by side:
+// whole memory lines per load and store), and scans them with DPP moves; one barrier
+// per step of 8192 rows puts the wavefronts behind one another.
 constexpr int kScanThreads = 1024, kScanPer = 8;
+
+__device__ __forceinline__ int64_t wave_inclusive_scan64(int64_t v) {
+#define CTMI_SCAN64_STEP(ctrl, rows, bound)                                                      \
+  {                                                                                              \
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, ctrl, rows, 0xf, bound); \
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)((uint64_t)v >> 32), ctrl, rows, 0xf, bound); \
+    v += (int64_t)(((uint64_t)hi << 32) | lo);                                                   \
+  }
+  CTMI_SCAN64_STEP(0x111, 0xf, true)   // row_shr:1
+  CTMI_SCAN64_STEP(0x112, 0xf, true)   // row_shr:2
+  CTMI_SCAN64_STEP(0x114, 0xf, true)   // row_shr:4
+  CTMI_SCAN64_STEP(0x118, 0xf, true)   // row_shr:8
+  CTMI_SCAN64_STEP(0x142, 0xa, false)  // row_bcast:15
+  CTMI_SCAN64_STEP(0x143, 0xc, false)  // row_bcast:31
+#undef CTMI_SCAN64_STEP
+  return v;
+}
+
+__device__ __forceinline__ int64_t wave_last64(int64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, kWave - 1);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)v >> 32), kWave - 1);
+  return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 __device__ __forceinline__ void scan_rows(const int64_t* __restrict__ counts,
                                           int64_t* __restrict__ offsets,
                                           int64_t* __restrict__ total, int64_t rows,
@@ -305,34 +331,34 @@ __device__ __forceinline__ void scan_rows(const int64_t* __restrict__ counts,
   int64_t carry = 0;
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   for (int64_t base = 0; base < rows; base += kScanThreads * kScanPer) {
-    const int64_t i0 = base + (int64_t)threadIdx.x * kScanPer;
-    int64_t c[kScanPer];
+    const int64_t i0 = base + (int64_t)wave * (kWave * kScanPer) + lane;
+    int64_t c[kScanPer], before[kScanPer];
 #pragma unroll
-    for (int k = 0; k < kScanPer; ++k) c[k] = i0 + k < rows ? counts[i0 + k] : 0;
-    int64_t mine = 0;
-#pragma unroll
-    for (int k = 0; k < kScanPer; ++k) mine += c[k];
-    int64_t inc = mine;
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-      const int64_t t = __shfl_up(inc, d, kWave);
-      if (lane >= d) inc += t;
+    for (int k = 0; k < kScanPer; ++k) {  // all loads first: no condition on the load itself
+      const int64_t i = i0 + k * kWave;
+      c[k] = counts[i < rows ? i : rows - 1];
     }
-    if (lane == kWave - 1) wsum[wave] = inc;
+#pragma unroll
+    for (int k = 0; k < kScanPer; ++k) c[k] = i0 + k * kWave < rows ? c[k] : 0;
+    int64_t mine = 0;  // of the wavefront's rows so far
+#pragma unroll
+    for (int k = 0; k < kScanPer; ++k) {
+      const int64_t inc = wave_inclusive_scan64(c[k]);
+      before[k] = mine + inc - c[k];
+      mine += wave_last64(inc);
+    }
+    if (lane == 0) wsum[wave] = mine;
     __syncthreads();
     int64_t woff = 0, tot = 0;
 #pragma unroll
     for (int w = 0; w < kScanThreads / kWave; ++w) {
       const int64_t sv = wsum[w];
-      if (w < wave) woff += sv;
+      woff += w < wave ? sv : 0;
       tot += sv;
     }
-    int64_t run = carry + woff + inc - mine;
 #pragma unroll
-    for (int k = 0; k < kScanPer; ++k) {
-      if (i0 + k < rows) offsets[i0 + k] = run;
-      run += c[k];
-    }
+    for (int k = 0; k < kScanPer; ++k)
+      if (i0 + k * kWave < rows) offsets[i0 + k * kWave] = carry + woff + before[k];
     carry += tot;
     __syncthreads();
   }
@@ -701,34 +727,44 @@ tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
                             TileInfo* __restrict__ info, int32_t* __restrict__ group_total,
                             int32_t* __restrict__ group_before, int64_t ntiles, uint32_t slot) {
   constexpr int kPerWave = kGroupTiles / (kGroupThreads / kWave);  // tiles per wavefront
+  static_assert(kPerWave == 4 && kTileBytes == 32 * 16,
+                "a wavefront reads two tiles per load, half a wavefront each");
   __shared__ int cnt_s[kGroupTiles];
   __shared__ int wsum_s[kGroupThreads / kWave];
   __shared__ int last_s;
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int64_t tile0 = (int64_t)blockIdx.x * kGroupTiles;
-  int cnt[kPerWave];
+  // The wavefront's four tiles are 2 KB in a row: two 16-byte loads per lane, both
+  // issued before anything is counted (an address past the end is replaced, what it
+  // brings is not used).  The counts of the two loads ride through one scan as
+  // 16-bit fields; lanes 31 and 63 then hold what the four tiles add up to.
+  const int64_t b0 = (tile0 + wave * kPerWave) * kTileBytes + lane * 16;
+  u32x4_t q[2];
 #pragma unroll
-  for (int t = 0; t < kPerWave; ++t) {
-    const int64_t tile = tile0 + wave * kPerWave + t;
-    cnt[t] = 0;
-#pragma unroll
-    for (int i = 0; i < kTileBytes; i += kWave * 16) {
-      const int64_t b0 = tile * kTileBytes + i + lane * 16;
-      if (i + lane * 16 >= kTileBytes) {
-        // a tile shorter than one step of the wavefront
-      } else if (b0 + 16 <= nbytes) {
-        const u32x4_t q = *reinterpret_cast<const u32x4_t*>(bitmask + b0);
-        cnt[t] += __popc(q.x) + __popc(q.y) + __popc(q.z) + __popc(q.w);
-      } else {
-        for (int64_t b = b0; b < nbytes; ++b) cnt[t] += __popc((uint32_t)bitmask[b]);
-      }
-    }
+  for (int j = 0; j < 2; ++j) {
+    const int64_t b = b0 + j * (kWave * 16);
+    q[j] = *reinterpret_cast<const u32x4_t*>(bitmask + (b < nbytes ? b : 0));
   }
+  uint32_t cnt2 = 0;
 #pragma unroll
-  for (int t = 0; t < kPerWave; ++t) {
-#pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) cnt[t] += __shfl_xor(cnt[t], d, kWave);
-    if (lane == 0) cnt_s[wave * kPerWave + t] = cnt[t];
+  for (int j = 0; j < 2; ++j) {
+    const int64_t b = b0 + j * (kWave * 16);
+    int c = 0;
+    if (b + 16 <= nbytes) {
+      c = __popc(q[j].x) + __popc(q[j].y) + __popc(q[j].z) + __popc(q[j].w);
+    } else {
+      for (int64_t at = b; at < nbytes; ++at) c += __popc((uint32_t)bitmask[at]);
+    }
+    cnt2 |= (uint32_t)c << (16 * j);
+  }
+  const uint32_t inc2 = (uint32_t)wave_inclusive_scan((int)cnt2);
+  const uint32_t half = (uint32_t)__builtin_amdgcn_readlane((int)inc2, kWave / 2 - 1);
+  const uint32_t all = (uint32_t)__builtin_amdgcn_readlane((int)inc2, kWave - 1);
+  if (lane == 0) {
+    cnt_s[wave * kPerWave + 0] = (int)(half & 0xffffu);
+    cnt_s[wave * kPerWave + 1] = (int)((all & 0xffffu) - (half & 0xffffu));
+    cnt_s[wave * kPerWave + 2] = (int)(half >> 16);
+    cnt_s[wave * kPerWave + 3] = (int)((all >> 16) - (half >> 16));
   }
   __syncthreads();
   if (wave == 0) {
@@ -736,10 +772,14 @@ tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
     const int inc = wave_inclusive_scan(c);
     if (tile0 + lane < ntiles) info[tile0 + lane] = TileInfo{inc - c, c};
     if (lane == kWave - 1) {
-      // the total goes out for the other workgroups of this launch to read, then the
-      // ticket: whoever draws the last one sees every total
+      // The total goes out where every workgroup of the device reads it (a device-scope
+      // atomic store), the lane waits until it has arrived, then draws its ticket:
+      // whoever draws the last one finds every total in place.  A release fence
+      // would order the two as well, but it writes the whole L2 back, in every
+      // workgroup, and doubled the time of this pass.
       __hip_atomic_store(&group_total[blockIdx.x], inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned int drawn = __hip_atomic_fetch_add(&popcount_ticket[slot], 1u, __ATOMIC_ACQ_REL,
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      const unsigned int drawn = __hip_atomic_fetch_add(&popcount_ticket[slot], 1u, __ATOMIC_RELAXED,
                                                         __HIP_MEMORY_SCOPE_AGENT);
       last_s = drawn == gridDim.x - 1;
     }
