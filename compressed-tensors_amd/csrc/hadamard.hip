@@ -291,11 +291,14 @@ __global__ void __launch_bounds__(kHadThreads) hadamard_mfma_kernel(HadArgs a) {
   }
 }
 
-// ---------------------------------------------------------------- block sizes up to 128, bf16, no LDS
-// One wavefront owns 16 sub-rows at a time and never talks to another wave.
-// Accesses are plain (not streaming) ones: a lane group touches half a cache
-// line per instruction and the other half with the next, which the streaming
-// hint turns into two trips to memory.
+// ---------------------------------------------------------------- block sizes up to 128, bf16 / float16
+// One wavefront owns 16 sub-rows at a time and never talks to another wave.  The 16
+// sub-rows are one stretch of memory; the wavefront loads and stores it lanes side by
+// side, whole memory lines per instruction, and passes it through an image in LDS of
+// its own on the way to the operand layout and back (the operand layout itself asks a
+// lane group for half a line per instruction and the other half with the next; read
+// and written that way the kernel was 7 % slower at 128, 20 % at 64).  Accesses are
+// plain ones: streaming loads cost 2 %, streaming stores 5-10 %.
 // With D^T = Mb^T * X^T on v_mfma_f32_16x16x32_bf16 the operand layouts line up
 // with memory on both sides:
 //   B operand (X^T): lane (i + 16 q) holds X[row i][32 ks + 8 q .. + 8], one
@@ -379,22 +382,6 @@ hadamard_rows_kernel(HadJobs jobs, int64_t n_full, int ragged_sub,
   const int64_t stride = (int64_t)gridDim.x * kRowsWaves;
   const int64_t first = (int64_t)blockIdx.x * kRowsWaves + wave;
 
-  // Loads are never conditional (a group past the end re-reads the last whole
-  // one) and the stores of whole groups are not either: with a fixed number of
-  // memory operations per step the waits can say exactly how many newer
-  // operations may still be in flight.  Where the group's outputs go is looked up
-  // together with where its inputs are.
-  auto load_group = [&](int64_t grp, frag_t* xf, uint16_t** dst) {
-    if (grp >= n_full) grp = n_full - 1;
-    int64_t local;
-    const int j = had_job<MANY>(jobs, grp, &local);
-    const int64_t at = (local * 16 + l16) * B + 8 * lq;
-    const uint16_t* src = static_cast<const uint16_t*>(jobs.x[j]) + at;
-    *dst = static_cast<uint16_t*>(jobs.out[j]) + at;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks)
-      xf[ks] = __builtin_bit_cast(frag_t, ldg<uint16_t, 8>(src + 32 * ks));
-  };
   auto pack2 = [&](float lo, float hi) -> uint32_t {
     if constexpr (HALF) return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
     else return pack_bf16x2(lo, hi);
@@ -421,28 +408,82 @@ hadamard_rows_kernel(HadJobs jobs, int64_t n_full, int ragged_sub,
       if (keep) stg<uint16_t, 8>(dst + 32 * p, __builtin_bit_cast(Vec<uint16_t, 8>, o));
     }
   };
+  // A group of 16 sub-rows is one stretch of 32 B bytes in memory.  It is loaded and
+  // stored as such, lanes side by side (every instruction whole memory lines), and
+  // turned into the operand layout and back in an image of the group in LDS that
+  // belongs to the wavefront alone: no barrier.  Sub-rows are 16 bytes further apart
+  // than they are long, so that the 16 lanes that read one column of pieces hit
+  // different banks.
+  constexpr int kPitch = (2 * B + 16) / 4;  // dwords between sub-rows of the image
+  constexpr int kPieces = B / 8;            // 16-byte pieces of a sub-row
+  __shared__ __attribute__((aligned(16))) uint32_t image_lds[kRowsWaves][16 * kPitch];
+  uint32_t* const img = image_lds[wave];
+  // piece j of the stretch, and the piece of sub-row l16 at columns 32 t + 8 lq
+  auto linear_at = [&](int j) { return (j / kPieces) * kPitch + (j % kPieces) * 4; };
+  auto operand_at = [&](int t) { return l16 * kPitch + 16 * t + 4 * lq; };
+  // Loads are never conditional (a group past the end re-reads the last whole one)
+  // and the stores of whole groups are not either: with a fixed number of memory
+  // operations per step the waits can say exactly how many newer operations may
+  // still be in flight.  Where the group's outputs go is looked up together with
+  // where its inputs are.
+  auto load_block = [&](int64_t grp, u32x4_t* raw, uint16_t** dst) {
+    if (grp >= n_full) grp = n_full - 1;
+    int64_t local;
+    const int j = had_job<MANY>(jobs, grp, &local);
+    const int64_t at = local * 16 * B + lane * 8;
+    const uint16_t* src = static_cast<const uint16_t*>(jobs.x[j]) + at;
+    *dst = static_cast<uint16_t*>(jobs.out[j]) + at;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      raw[ks] = __builtin_bit_cast(u32x4_t, ldg<uint16_t, 8>(src + 512 * ks));
+  };
   if (first < n_full) {
-    // Software pipeline one group ahead, two register sets taking turns (no
-    // copies).  The first group is handled ahead of the loop so that the loop is
-    // entered with the same operations in flight as on its back edge (one set's
-    // loads, then a group's stores): a wait for loads then never has to cover
-    // the stores issued after them, which would cost a store latency per group.
-    frag_t xa[KS], xb[KS];
-    uint16_t *da, *db;
+    u32x4_t raw[KS];
+    uint16_t *dst, *dst_next;
     int64_t g = first;
-    load_group(g, xa, &da);
-    load_group(g + stride, xb, &db);
-    transform_rows(xa, da, true);
-    g += stride;
-    while (g < n_full) {  // invariant: group g is in xb
-      load_group(g + stride, xa, &da);
-      transform_rows(xb, db, true);
+    load_block(g, raw, &dst);
+    // The first group is handled ahead of the loop so that the loop is entered with
+    // the same operations in flight as on its back edge (a group's loads, then a
+    // group's stores): the wait for the loads then leaves the stores in flight.
+    auto step = [&]() {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        *reinterpret_cast<u32x4_t*>(&img[linear_at(ks * kWave + lane)]) = raw[ks];
+      load_block(g + stride, raw, &dst_next);
+      frag_t xf[KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        xf[ks] = __builtin_bit_cast(frag_t, *reinterpret_cast<const u32x4_t*>(&img[operand_at(ks)]));
+#pragma unroll
+      for (int p = 0; p < NP; ++p) {
+        f32x4_t a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          if constexpr (HALF) {
+            a0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(mb[2 * p][ks], xf[ks], a0, 0, 0, 0);
+            a1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(mb[2 * p + 1][ks], xf[ks], a1, 0, 0, 0);
+          } else {
+            a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p][ks], xf[ks], a0, 0, 0, 0);
+            a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(mb[2 * p + 1][ks], xf[ks], a1, 0, 0, 0);
+          }
+        }
+        u32x4_t o;
+        o[0] = pack2(a0[0] * inv_sqrt_n, a0[1] * inv_sqrt_n);
+        o[1] = pack2(a0[2] * inv_sqrt_n, a0[3] * inv_sqrt_n);
+        o[2] = pack2(a1[0] * inv_sqrt_n, a1[1] * inv_sqrt_n);
+        o[3] = pack2(a1[2] * inv_sqrt_n, a1[3] * inv_sqrt_n);
+        *reinterpret_cast<u32x4_t*>(&img[operand_at(p)]) = o;
+      }
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4_t r = *reinterpret_cast<const u32x4_t*>(&img[linear_at(ks * kWave + lane)]);
+        stg<uint16_t, 8>(dst + 512 * ks, __builtin_bit_cast(Vec<uint16_t, 8>, r));
+      }
+      dst = dst_next;
       g += stride;
-      if (g >= n_full) break;
-      load_group(g + stride, xb, &db);
-      transform_rows(xa, da, true);
-      g += stride;
-    }
+    };
+    step();
+    while (g < n_full) step();
   }
   // the ragged last group (fewer than 16 sub-rows; single tensors only), by the wave
   // whose turn it is
