@@ -328,6 +328,31 @@ def test_bitmask_decompress_runs_of_tiles(dtype, shape, gpu):
         assert_bit_equal(got, want, f"first {keep} values")
 
 
+def test_bitmask_decompress_on_two_streams_at_once(gpu):
+    """decompressions in flight on two streams at the same time (each launch of the count
+    pass takes its own ticket counter inside the library): the results of the calls made one
+    after the other"""
+    from compressed_tensors_amd.compressors import bitmask_compress, bitmask_decompress
+
+    announce("bitmask decompress, two streams")
+    tensors = [_sparse_tensor((2048, 4096), torch.bfloat16, sp, seed=60 + i).to(gpu)
+               for i, sp in enumerate((0.5, 0.8, 0.2, 0.5))]
+    packed = [bitmask_compress(x) for x in tensors]
+    alone = [bitmask_decompress(values, bitmask, [2048, 4096]) for values, bitmask, _ in packed]
+    for x, back in zip(tensors, alone):
+        assert torch.equal(torch.nan_to_num(back.float()), torch.nan_to_num(x.float()))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(device=gpu), torch.cuda.Stream(device=gpu)]
+    results = []
+    for rep in range(6):
+        for i, (values, bitmask, _) in enumerate(packed):
+            with torch.cuda.stream(streams[(rep + i) % 2]):
+                results.append((i, bitmask_decompress(values, bitmask, [2048, 4096])))
+    torch.cuda.synchronize()
+    for i, got in results:
+        assert_bit_equal(got, alone[i], f"tensor {i}")
+
+
 def test_bitmask_decompress_of_a_very_large_tensor(gpu):
     """more tiles than the grouped count handles (> 65536 tiles of 8192 elements): the scatter
     then takes its positions from a scan over all tiles.  Round trip on the GPU, values and
