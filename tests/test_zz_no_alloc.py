@@ -60,6 +60,54 @@ def test_static_scratch_decompress_matches_the_scratch_argument_one(ctmi, gpu):
         assert torch.equal(_bits(b), _bits(a)), "static-scratch entry point vs scratch-argument one"
 
 
+@pytest.mark.gpu
+def test_static_scratch_decompress_replays_from_a_captured_graph(ctmi, gpu):
+    """the caller the entry point is for: captured once into a HIP graph (nothing is allocated
+    and nothing cleared by a memset node), replayed several times with new inputs copied into
+    the same buffers and eager work in between; every replay equals the eager call"""
+    from compressed_tensors_amd import _lib
+
+    announce("static-scratch decompress in a captured graph")
+    rows, cols = 1024, 4096
+    packed = []
+    for seed, sparsity in ((11, 0.5), (12, 0.9), (13, 0.2), (14, 0.5)):
+        values, bitmask, _ = osp.bitmask_compress(_case(rows, cols, torch.bfloat16, sparsity, seed))
+        packed.append((values.to(gpu), bitmask.to(gpu).contiguous()))
+    room = max(v.numel() for v, _ in packed)
+    d_values = torch.zeros(room, dtype=torch.bfloat16, device=gpu)
+    d_bitmask = torch.zeros_like(packed[0][1])
+    out = torch.empty((rows, cols), dtype=torch.bfloat16, device=gpu)
+    tmp = torch.empty(ctmi.ctmi_bitmask_tmp_bytes(rows, cols), dtype=torch.uint8, device=gpu)
+
+    def load(k):
+        d_values.zero_()
+        d_values[: packed[k][0].numel()].copy_(packed[k][0])
+        d_bitmask.copy_(packed[k][1])
+
+    def call():
+        # nvalues is fixed in the captured call: the buffer's size; what lies behind a
+        # tensor's own values is zero and is never reached by a set bit
+        _lib.check(ctmi.ctmi_bitmask_decompress_static(d_values.data_ptr(), room, 2, d_bitmask.data_ptr(),
+                                                       out.data_ptr(), rows, cols, _lib.stream_of(gpu)))
+
+    load(0)
+    call()  # the per-device set-up of the entry point happens outside the capture
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()
+    for k in (1, 2, 3, 0, 2):
+        load(k)
+        want = torch.empty_like(out)
+        _lib.check(ctmi.ctmi_bitmask_decompress(d_values.data_ptr(), room, 2, d_bitmask.data_ptr(), None,
+                                                want.data_ptr(), tmp.data_ptr(), rows, cols,
+                                                _lib.stream_of(gpu)))
+        out.fill_(3.0)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(_bits(out.cpu()), _bits(want.cpu())), f"replay with tensor {k}"
+
+
 def test_static_scratch_rejects_what_does_not_fit(ctmi):
     """refused on the host, before any HIP call: runs without a GPU"""
     from compressed_tensors_amd import _lib
