@@ -1,5 +1,5 @@
 // Transforms W = diag(sign_in) * (Ma (x) Sylvester(64)) * diag(sign_out) * scale on runs of
-// K * 64 bfloat16 elements, K <= 224: the reference's Hadamard matrices of size K * 2^m
+// K * 64 bfloat16 (or float16) elements, K <= 224: the reference's Hadamard matrices of size K * 2^m
 //
 //   random_hadamard_matrix, _matmul_hadU        transform/utils/hadamard.py:65-163
 //   HadamardTransform.forward                   transform/factory/hadamard.py:104-121
@@ -32,12 +32,14 @@
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "quant_fast.h"
 #include "fwht.h"
 
 namespace ctmi {
 namespace {
 
 typedef __bf16 bs_bf16x8_t __attribute__((ext_vector_type(8)));
+typedef _Float16 bs_f16x8_t __attribute__((ext_vector_type(8)));
 typedef float bs_f32x16_t __attribute__((ext_vector_type(16)));
 typedef uint32_t bs_u32x4 __attribute__((ext_vector_type(4)));
 
@@ -83,8 +85,20 @@ constexpr size_t bs_lds_bytes(int nt, bool signs) {
           (size_t)kBsWaves * kBsRing) * sizeof(uint32_t);
 }
 
-// NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out
-template <int NT, int SIGNS>
+// One product on the matrix cores: bfloat16 operands, or (HALF) float16 ones
+template <bool HALF>
+__device__ __forceinline__ bs_f32x16_t bs_mma(const bs_u32x4& a, const bs_u32x4& b, const bs_f32x16_t& c) {
+  if constexpr (HALF)
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(bs_f16x8_t, a),
+                                                  __builtin_bit_cast(bs_f16x8_t, b), c, 0, 0, 0);
+  else
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a),
+                                                   __builtin_bit_cast(bs_bf16x8_t, b), c, 0, 0, 0);
+}
+
+// NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out;
+// HALF: float16 tensors (the matrix arrives in bfloat16 and converts exactly: entries +-1)
+template <int NT, int SIGNS, bool HALF>
 __global__ void __launch_bounds__(kBsThreads, 1)
 block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
                          const float* __restrict__ signs, float scale) {
@@ -125,6 +139,11 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int f = f0 + u * kBsWaves + (int)wave;
+      if constexpr (HALF) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          w[u][d] = (uint32_t)f32_to_f16(bf16_lo(w[u][d])) | ((uint32_t)f32_to_f16(bf16_hi(w[u][d])) << 16);
+      }
       if (f < KS * NT) ma_frag[f * kWave + l] = w[u];
     }
   }
@@ -171,6 +190,10 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
     }
   };
 
+  auto pack2 = [](float lo, float hi) -> uint32_t {
+    if constexpr (HALF) return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
+    else return pack_bf16x2(lo, hi);
+  };
   const int64_t step = (int64_t)gridDim.x * kBsWaves;
   int64_t run = (int64_t)blockIdx.x * kBsWaves + wave;
   {
@@ -230,20 +253,15 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
           asm volatile("" ::: "memory");
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
-            const bs_bf16x8_t b = __builtin_bit_cast(bs_bf16x8_t, bq[nt]);
-            acc[0][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[0]), b,
-                                                                 acc[0][nt], 0, 0, 0);
-            acc[1][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[1]), b,
-                                                                 acc[1][nt], 0, 0, 0);
+            acc[0][nt] = bs_mma<HALF>(a[0], bq[nt], acc[0][nt]);
+            acc[1][nt] = bs_mma<HALF>(a[1], bq[nt], acc[1][nt]);
           }
         } else {
 #pragma unroll
           for (int nt = 0; nt < NT; ++nt) {
-            const bs_bf16x8_t b = __builtin_bit_cast(bs_bf16x8_t, ma_frag[(ks * NT + nt) * kWave + l]);
-            acc[0][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[0]), b,
-                                                                 acc[0][nt], 0, 0, 0);
-            acc[1][nt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bs_bf16x8_t, a[1]), b,
-                                                                 acc[1][nt], 0, 0, 0);
+            const bs_u32x4 b = ma_frag[(ks * NT + nt) * kWave + l];
+            acc[0][nt] = bs_mma<HALF>(a[0], b, acc[0][nt]);
+            acc[1][nt] = bs_mma<HALF>(a[1], b, acc[1][nt]);
           }
         }
       }
@@ -279,10 +297,10 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
         bs_u32x4 w;
-        w[0] = pack_bf16x2(u[0][4 * b] * scale, u[0][4 * b + 1] * scale);
-        w[1] = pack_bf16x2(u[0][4 * b + 2] * scale, u[0][4 * b + 3] * scale);
-        w[2] = pack_bf16x2(u[1][4 * b] * scale, u[1][4 * b + 1] * scale);
-        w[3] = pack_bf16x2(u[1][4 * b + 2] * scale, u[1][4 * b + 3] * scale);
+        w[0] = pack2(u[0][4 * b] * scale, u[0][4 * b + 1] * scale);
+        w[1] = pack2(u[0][4 * b + 2] * scale, u[0][4 * b + 3] * scale);
+        w[2] = pack2(u[1][4 * b] * scale, u[1][4 * b + 1] * scale);
+        w[3] = pack2(u[1][4 * b + 2] * scale, u[1][4 * b + 3] * scale);
         *reinterpret_cast<bs_u32x4*>(&image[c * kBsPitch + 16 * h + 4 * b]) = w;
       }
       bs_u32x4 fo[SIGNS == 2 ? 4 : 1];
@@ -302,10 +320,10 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   }
 }
 
-template <int NT, int SIGNS>
+template <int NT, int SIGNS, bool HALF>
 int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
                       hipStream_t st) {
-  auto kern = block_sylvester64_kernel<NT, SIGNS>;
+  auto kern = block_sylvester64_kernel<NT, SIGNS, HALF>;
   constexpr size_t lds = bs_lds_bytes(NT, SIGNS != 0);
   if (lds > 48 * 1024) {
     // the attribute belongs to the kernel as loaded on one device; setting it again is cheap
@@ -333,24 +351,31 @@ int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const flo
   return CTMI_OK;
 }
 
+template <int NT, bool HALF>
+int launch_bs_dtype(const BsTable& tab, const uint16_t* ma_t, int k, const float* sign_in,
+                    const float* sign_out, float scale, hipStream_t st) {
+  if (sign_in) return launch_bs_variant<NT, 1, HALF>(tab, ma_t, k, sign_in, scale, st);
+  if (sign_out) return launch_bs_variant<NT, 2, HALF>(tab, ma_t, k, sign_out, scale, st);
+  return launch_bs_variant<NT, 0, HALF>(tab, ma_t, k, nullptr, scale, st);
+}
+
 template <int NT>
-int launch_bs(const BsTable& tab, const uint16_t* ma_t, int k, const float* sign_in,
+int launch_bs(const BsTable& tab, int io_dtype, const uint16_t* ma_t, int k, const float* sign_in,
               const float* sign_out, float scale, hipStream_t st) {
-  if (sign_in) return launch_bs_variant<NT, 1>(tab, ma_t, k, sign_in, scale, st);
-  if (sign_out) return launch_bs_variant<NT, 2>(tab, ma_t, k, sign_out, scale, st);
-  return launch_bs_variant<NT, 0>(tab, ma_t, k, nullptr, scale, st);
+  if (io_dtype == CTMI_F16) return launch_bs_dtype<NT, true>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  return launch_bs_dtype<NT, false>(tab, ma_t, k, sign_in, sign_out, scale, st);
 }
 
 }  // namespace
 
 bool block_sylvester64_supported(int k, int io_dtype, bool both_signs) {
-  return io_dtype == CTMI_BF16 && k >= 1 && k <= 224 && !both_signs;
+  return (io_dtype == CTMI_BF16 || io_dtype == CTMI_F16) && k >= 1 && k <= 224 && !both_signs;
 }
 
-int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int k, const uint16_t* ma_t,
+int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int k, const uint16_t* ma_t,
                              const float* sign_in, const float* sign_out, float scale, hipStream_t st) {
-  CTMI_REQUIRE(block_sylvester64_supported(k, CTMI_BF16, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
-               "blocks of up to 224 x 224 with signs on one side");
+  CTMI_REQUIRE(block_sylvester64_supported(k, io_dtype, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
+               "bfloat16 or float16 tensors, blocks of up to 224 x 224 with signs on one side");
   CTMI_REQUIRE(n_jobs >= 1 && n_jobs <= kFwhtMaxJobs, CTMI_ERR_VALUE, "1 to %d tensors a launch", kFwhtMaxJobs);
   CTMI_REQUIRE(ma_t && (uintptr_t)sign_in % 16 == 0 && (uintptr_t)sign_out % 16 == 0, CTMI_ERR_VALUE,
                "the block must be given; sign vectors must be 16-byte aligned");
@@ -370,10 +395,10 @@ int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int k, const uint1
     tab.end[i] = live ? total : INT64_MAX;
   }
   tab.total = total;
-  if (k <= 32) return launch_bs<1>(tab, ma_t, k, sign_in, sign_out, scale, st);
-  if (k <= 64) return launch_bs<2>(tab, ma_t, k, sign_in, sign_out, scale, st);
-  if (k <= 128) return launch_bs<4>(tab, ma_t, k, sign_in, sign_out, scale, st);
-  return launch_bs<7>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 32) return launch_bs<1>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 64) return launch_bs<2>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 128) return launch_bs<4>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+  return launch_bs<7>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
 }
 
 }  // namespace ctmi

@@ -1177,7 +1177,7 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
         b.rows = jobs[i].numel / n;
       }
       if (filled == kFwhtMaxJobs || (i == n_jobs && filled)) {
-        const int rc = block_sylvester64_launch(batch, filled, a_dim, (const uint16_t*)ma_t, sign_in, sign_out,
+        const int rc = block_sylvester64_launch(batch, filled, io_dtype, a_dim, (const uint16_t*)ma_t, sign_in, sign_out,
                                                 1.0f / sqrtf((float)n), st);
         if (rc) return rc;
         filled = 0;

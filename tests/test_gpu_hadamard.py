@@ -468,22 +468,25 @@ def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_block
     assert ctmi.ctmi_hadamard_supported(224, 128, _lib.dtype_code(torch.bfloat16)) == 0
 
 
-@pytest.mark.parametrize("k", [224, 12, 28, 36, 64, 100, 128, 160])
-def test_block_times_sylvester64_with_butterflies(k, ctmi, gpu, hadamard_blocks):
+@pytest.mark.parametrize("k,dtype", [(k, torch.bfloat16) for k in (224, 12, 28, 36, 64, 100, 128, 160)] +
+                         [(k, torch.float16) for k in (224, 28, 64, 100)],
+                         ids=lambda v: str(v).replace("torch.", ""))
+def test_block_times_sylvester64_with_butterflies(k, dtype, ctmi, gpu, hadamard_blocks):
     """ctmi_hadamard_apply without mb_t (Mb = Sylvester(64)): the product with the block on the
-    matrix cores, the Sylvester factor as butterflies on its fp32 result.  Blocks of every tile
+    matrix cores, the Sylvester factor as butterflies on its fp32 result; bfloat16 and float16
+    tensors (the block is given in bfloat16 either way).  Blocks of every tile
     count (K <= 32, 64, 128, 224) incl. sizes that leave rows of the last tile empty, a random
     +-1 matrix and (where the table has one) the known Hadamard block; more runs than the
     workgroups hold at a time; signs on either side; several tensors in one call."""
     from compressed_tensors_amd import _lib
 
-    announce("block x Sylvester(64), butterflies", k)
-    code = _lib.dtype_code(torch.bfloat16)
+    announce("block x Sylvester(64), butterflies", k, dtype)
+    code = _lib.dtype_code(dtype)
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 64, code) == 1
     n = k * 64
     g = torch.Generator().manual_seed(k)
     rows = 2051 if k <= 64 else 1027
-    x = torch.randn(rows, n, generator=g).bfloat16()
+    x = torch.randn(rows, n, generator=g).to(dtype)
     s = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
     sample = torch.tensor([0, 1, 255, 256, 511, 1023, 1024, rows - 1])
     blocks = [(torch.randint(0, 2, (k, k), generator=g) * 2 - 1).double()]
@@ -502,10 +505,10 @@ def test_block_times_sylvester64_with_butterflies(k, ctmi, gpu, hadamard_blocks)
             assert not bool(torch.isnan(out.float()).any()), "every element written"
             xs = x[sample].double() * (1.0 if si is None else si.double())
             want = xs @ dense * (1.0 if so is None else so.double()) / n ** 0.5
-            _assert_within_ulp(out[sample.to(gpu)], want.bfloat16(), f"signs in={si is not None} out={so is not None}")
+            _assert_within_ulp(out[sample.to(gpu)], want.to(dtype), f"signs in={si is not None} out={so is not None}")
     # several tensors from one call == one by one
     ma_t = blocks[0].T.contiguous().bfloat16().to(gpu)
-    xs = [torch.randn(r, n, generator=g).bfloat16().to(gpu) for r in (3, 70, 1, 16, 5, 9, 33, 2, 40, 7)]
+    xs = [torch.randn(r, n, generator=g).to(dtype).to(gpu) for r in (3, 70, 1, 16, 5, 9, 33, 2, 40, 7)]
     outs = [torch.empty_like(t) for t in xs]
     jobs = (_lib.HadamardJob * len(xs))()
     for job, t, o in zip(jobs, xs, outs):
@@ -521,7 +524,7 @@ def test_block_times_sylvester64_with_butterflies(k, ctmi, gpu, hadamard_blocks)
     # what it does not take
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 32, code) == 0
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(225, 64, code) == 0
-    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 64, _lib.dtype_code(torch.float16)) == 0
+    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 64, _lib.dtype_code(torch.float32)) == 0
     rc = ctmi.ctmi_hadamard_apply(xg.data_ptr(), xg.data_ptr(), code, xg.numel(), k, 64, ma_t.data_ptr(), None,
                                   sg.data_ptr(), sg.data_ptr(), _lib.stream_of(gpu))
     assert rc == _lib.CTMI_ERR_UNSUPPORTED
