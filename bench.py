@@ -835,7 +835,11 @@ def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True):
         "dtype": "bf16 in, codes as the format says (arithmetic in the reference's promoted dtype)",
         "data": "synthetic",
         "config": {"workload": workload, "seed": seed,
-                   "value_is": "algorithmic bytes of all operations / sum of their GPU times"},
+                   "value_is": "algorithmic bytes of all operations / sum of their GPU times",
+                   "value_without_comparison_lines_is": "the same over the operations the library's own "
+                                                        "dispatch runs (for_comparison_only false)"},
+        "value_without_comparison_lines": sum(op.nbytes for op in ops if op.primary) /
+                                          (sum(op.ms for op in ops if op.primary) * 1e-3) / 1e9,
         "roofline": {"bound": "hbm", "kernel": slow.kernel, "operation": slow.name,
                      "achieved": slow.nbytes / (slow.ms * 1e-3) / 1e9, "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": slow.nbytes / (slow.ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
