@@ -332,7 +332,7 @@ def other_workload(torch, name, seed):
         from compressed_tensors_amd.compressors import get_24_bytemasks
         from compressed_tensors_amd.quantization import quantize
         copies24 = 16  # values + bitmask of the codes are 37 MB a copy: well beyond the 256 MB last-level cache
-        s24_jobs = []
+        s24_jobs, s24_jobs16 = [], []
         for _ in range(copies24):
             w = randn(14336, 4096, 0.02)
             w = torch.where(get_24_bytemasks(w), w, torch.zeros_like(w))
@@ -376,6 +376,7 @@ def other_workload(torch, name, seed):
             a16 = (w.data_ptr(), code(w.dtype), values16.data_ptr(), bitmask16.data_ptr(), rows, cols, st)
             d16 = (values16.data_ptr(), values16.numel(), 2, bitmask16.data_ptr(), dense16.data_ptr(), tmp16.data_ptr(), rows, cols, st)
             _lib.check(lib.ctmi_sparse24_compress(*a16))
+            s24_jobs16.append((w, values16, bitmask16, dense16, rows, cols))
             s16_calls.append(lambda a16=a16: _lib.check(lib.ctmi_sparse24_compress(*a16)))
             t16_calls.append(lambda d16=d16: _lib.check(lib.ctmi_sparse24_decompress(*d16)))
             # ... and the way back: 2:4 -> fp8 codes -> bf16
@@ -392,9 +393,16 @@ def other_workload(torch, name, seed):
             for job, full in ((cj[k], q), (dj[k], dense)):
                 job.dense, job.values, job.bitmask = full.data_ptr(), values.data_ptr(), bitmask.data_ptr()
                 job.nvalues, job.rows, job.cols = values.numel(), rows, cols
-        keep.extend([cj, dj])
+        cj16, dj16 = (_lib.Sparse24Job * copies24)(), (_lib.Sparse24Job * copies24)()
+        for k, (w, values, bitmask, dense, rows, cols) in enumerate(s24_jobs16):
+            for job, full in ((cj16[k], w), (dj16[k], dense)):
+                job.dense, job.values, job.bitmask = full.data_ptr(), values.data_ptr(), bitmask.data_ptr()
+                job.nvalues, job.rows, job.cols = values.numel(), rows, cols
+        keep.extend([cj, dj, cj16, dj16])
         cm = (cj, copies24, code(FP8), st)
         dm = (dj, copies24, 1, st)
+        cm16 = (cj16, copies24, code(s24_jobs16[0][0].dtype), st)
+        dm16 = (dj16, copies24, 2, st)
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies24 * (n24 + n24 // 2 + n24 // 8)
         fused24_bytes = copies24 * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
@@ -408,6 +416,12 @@ def other_workload(torch, name, seed):
                   [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm))], s24_bytes, "sparse24_scatter_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 bf16", s16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress, bf16", t16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel"),
+               Op("sparse-24-bitmask compress, bf16, all 16 in one call (8 per launch)",
+                  [lambda: _lib.check(lib.ctmi_sparse24_compress_many(*cm16))],
+                  2 * s24_bytes - copies24 * (n24 // 8), "sparse24_compress_chain_kernel"),
+               Op("sparse-24-bitmask decompress, bf16, all 16 in one call (8 per launch)",
+                  [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm16))],
+                  2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel"),
                Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies24 * (n24 + n24 // 8), "pack_bitmasks"),
                Op("unpack_bitmasks", up_calls, copies24 * (n24 + n24 // 8), "unpack_bitmasks"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
