@@ -97,19 +97,27 @@ __device__ __forceinline__ bs_f32x16_t bs_mma(const bs_u32x4& a, const bs_u32x4&
 }
 
 // NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out;
-// HALF: float16 tensors (the matrix arrives in bfloat16 and converts exactly: entries +-1)
-template <int NT, int SIGNS, bool HALF>
+// HALF: float16 tensors (the matrix arrives in bfloat16 and converts exactly: entries +-1);
+// PAIR: runs of K * 32 elements (Ma (x) Sylvester(32), e.g. 7168 = 224 * 32), two at a time:
+// the 64 columns of the image are 32 of one run and 32 of the next, the two M tiles are the
+// two runs, and the butterfly stage over the M tiles is left out.  Lanes whose piece of a row
+// lies in the left half of the image (l % 8 < 4) load and store the first run, the others
+// the second; a single last run is paired with itself and its second copy is not stored.
+template <int NT, int SIGNS, bool HALF, bool PAIR>
 __global__ void __launch_bounds__(kBsThreads, 1)
 block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
                          const float* __restrict__ signs, float scale) {
   constexpr int KS = 2 * NT;  // steps of 16 over the contracted index
+  constexpr int INNER = PAIR ? 32 : 64;
   extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
   bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
   bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [NT * 4][64] (SIGNS != 0)
   const uint32_t l = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const uint32_t c = l & 31u, g = l >> 5;
   uint32_t* image = bs_lds + (KS * NT + (SIGNS ? NT * 4 : 0)) * kWave * 4 + wave * kBsRing;
-  const int64_t n = (int64_t)k_dim * 64;
+  const int64_t n = (int64_t)k_dim * INNER;
+  const uint32_t piece = 8 * (l & (INNER / 8 - 1));  // the lane's 8 columns inside a row of a run
+  const bool second = PAIR && (l & 4u);              // the lane belongs to the second run of a pair
 
   // The fragments of Ma, zero beyond K.  Eight at a time per wavefront, loads first: one after
   // the other they would cost the launch as many memory round trips as there are fragments.
@@ -155,7 +163,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       const int row = 32 * (f >> 2) + (int)(l >> 3) + 8 * (f & 3);
       bs_u32x4 m = {0u, 0u, 0u, 0u};
       if (row < k_dim) {
-        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + 64 * row + 8 * (l & 7u));
+        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + INNER * row + piece);
 #pragma unroll
         for (int d = 0; d < 4; ++d) m[d] = ((s8.v[2 * d] >> 16) & 0x8000u) | (s8.v[2 * d + 1] & 0x80000000u);
       }
@@ -175,20 +183,32 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   // the spot): a run beyond the last reads the last again, a row beyond K reads row K - 1 and
   // is replaced by zeros when it is used.
   bs_u32x4 in[NT][4];
-  auto run_start = [&](int64_t r) {  // where run r begins (table reads: once per run, not per chunk)
-    r = r < tab.total ? r : tab.total - 1;
-    int64_t local;
-    const int j = bs_job(tab, r, &local);
-    return static_cast<const uint16_t*>(tab.x[j]) + local * n;
+  // where the lane's run of unit u begins (a unit: one run, or PAIR: two neighbouring ones);
+  // table reads once per unit, not per chunk
+  auto run_start = [&](int64_t u) {
+    if constexpr (PAIR) {
+      int64_t la, lb;
+      const int64_t ra = min(2 * u, tab.total - 1), rb = min(2 * u + 1, tab.total - 1);
+      const int ja = bs_job(tab, ra, &la), jb = bs_job(tab, rb, &lb);
+      const uint16_t* a = static_cast<const uint16_t*>(tab.x[ja]) + la * n;
+      const uint16_t* b = static_cast<const uint16_t*>(tab.x[jb]) + lb * n;
+      return second ? b : a;
+    } else {
+      const int64_t r = u < tab.total ? u : tab.total - 1;
+      int64_t local;
+      const int j = bs_job(tab, r, &local);
+      return static_cast<const uint16_t*>(tab.x[j]) + local * n;
+    }
   };
   auto fetch = [&](const uint16_t* __restrict__ xr, int ch) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int row = 32 * ch + (int)(l >> 3) + 8 * q;
       in[ch][q] = __builtin_bit_cast(
-          bs_u32x4, ldg_nt<uint16_t, 8>(xr + 64 * (row < k_dim ? row : k_dim - 1) + 8 * (l & 7u)));
+          bs_u32x4, ldg_nt<uint16_t, 8>(xr + INNER * (row < k_dim ? row : k_dim - 1) + piece));
     }
   };
+  const int64_t units = PAIR ? (tab.total + 1) / 2 : tab.total;
 
   auto pack2 = [](float lo, float hi) -> uint32_t {
     if constexpr (HALF) return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
@@ -201,7 +221,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
 #pragma unroll
     for (int ch = 0; ch < NT; ++ch) fetch(first, ch);
   }
-  for (; run < tab.total; run += step) {
+  for (; run < units; run += step) {
     const uint16_t* next = run_start(run + step);
     bs_f32x16_t acc[2][NT];
 #pragma unroll
@@ -267,16 +287,30 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       }
     }
     // butterflies over j = 32 mt + 8 b + 4 g + r
-    int64_t local;
-    const int j = bs_job(tab, run, &local);
-    uint16_t* __restrict__ yr = static_cast<uint16_t*>(tab.out[j]) + local * n;
-    const uint32_t h = g;  // after the exchange: lane half h holds j = 32 h ...
+    uint16_t* __restrict__ yr;
+    bool stored = true;  // PAIR: the second copy of a single last run is not
+    if constexpr (PAIR) {
+      int64_t la, lb;
+      const int64_t rb = 2 * run + 1 < tab.total ? 2 * run + 1 : 2 * run;
+      const int ja = bs_job(tab, 2 * run, &la), jb = bs_job(tab, rb, &lb);
+      uint16_t* a = static_cast<uint16_t*>(tab.out[ja]) + la * n;
+      uint16_t* b = static_cast<uint16_t*>(tab.out[jb]) + lb * n;
+      yr = second ? b : a;
+      stored = !second || 2 * run + 1 < tab.total;
+    } else {
+      int64_t local;
+      const int j = bs_job(tab, run, &local);
+      yr = static_cast<uint16_t*>(tab.out[j]) + local * n;
+    }
+    const uint32_t h = g;  // after the exchange: lane half h holds j = 32 h ... (PAIR: run h of the two)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       float u[2][16];  // u[x][4 b + r] = value at j = 32 h + 8 b + 4 x + r
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const float s = acc[0][nt][v] + acc[1][nt][v], t = acc[0][nt][v] - acc[1][nt][v];  // stage over mt
+        // stage over mt (PAIR: the two tiles are two runs and stay apart)
+        const float s = PAIR ? acc[0][nt][v] : acc[0][nt][v] + acc[1][nt][v];
+        const float t = PAIR ? acc[1][nt][v] : acc[0][nt][v] - acc[1][nt][v];
         const auto pr = __builtin_amdgcn_permlane32_swap(__float_as_uint(s), __float_as_uint(t), false, false);
         const float lower = __uint_as_float(pr[0]), upper = __uint_as_float(pr[1]);  // g = 0, g = 1
         u[0][v] = lower + upper;
@@ -313,17 +347,17 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         const int row = 32 * nt + (int)(l >> 3) + 8 * q;
         bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
         if constexpr (SIGNS == 2) w ^= fo[q];
-        if (row < k_dim)
-          stg_nt<uint16_t, 8>(yr + 64 * row + 8 * (l & 7u), __builtin_bit_cast(Vec<uint16_t, 8>, w));
+        if (row < k_dim && stored)
+          stg_nt<uint16_t, 8>(yr + INNER * row + piece, __builtin_bit_cast(Vec<uint16_t, 8>, w));
       }
     }
   }
 }
 
-template <int NT, int SIGNS, bool HALF>
+template <int NT, int SIGNS, bool HALF, bool PAIR>
 int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
                       hipStream_t st) {
-  auto kern = block_sylvester64_kernel<NT, SIGNS, HALF>;
+  auto kern = block_sylvester64_kernel<NT, SIGNS, HALF, PAIR>;
   constexpr size_t lds = bs_lds_bytes(NT, SIGNS != 0);
   if (lds > 48 * 1024) {
     // the attribute belongs to the kernel as loaded on one device; setting it again is cheap
@@ -343,7 +377,7 @@ int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const flo
     per_cu = n > 0 ? n : 1;
   }
   if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "device query: %s", hipGetErrorString(e));
-  const int64_t wgs = cdiv(tab.total, kBsWaves);
+  const int64_t wgs = cdiv(PAIR ? (tab.total + 1) / 2 : tab.total, kBsWaves);
   const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * per_cu;
   const int64_t each = cdiv(wgs, cap);  // runs per wavefront, the same for all
   const unsigned grid = (unsigned)cdiv(wgs, each);
@@ -351,19 +385,23 @@ int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const flo
   return CTMI_OK;
 }
 
-template <int NT, bool HALF>
+template <int NT, bool HALF, bool PAIR>
 int launch_bs_dtype(const BsTable& tab, const uint16_t* ma_t, int k, const float* sign_in,
                     const float* sign_out, float scale, hipStream_t st) {
-  if (sign_in) return launch_bs_variant<NT, 1, HALF>(tab, ma_t, k, sign_in, scale, st);
-  if (sign_out) return launch_bs_variant<NT, 2, HALF>(tab, ma_t, k, sign_out, scale, st);
-  return launch_bs_variant<NT, 0, HALF>(tab, ma_t, k, nullptr, scale, st);
+  if (sign_in) return launch_bs_variant<NT, 1, HALF, PAIR>(tab, ma_t, k, sign_in, scale, st);
+  if (sign_out) return launch_bs_variant<NT, 2, HALF, PAIR>(tab, ma_t, k, sign_out, scale, st);
+  return launch_bs_variant<NT, 0, HALF, PAIR>(tab, ma_t, k, nullptr, scale, st);
 }
 
 template <int NT>
-int launch_bs(const BsTable& tab, int io_dtype, const uint16_t* ma_t, int k, const float* sign_in,
-              const float* sign_out, float scale, hipStream_t st) {
-  if (io_dtype == CTMI_F16) return launch_bs_dtype<NT, true>(tab, ma_t, k, sign_in, sign_out, scale, st);
-  return launch_bs_dtype<NT, false>(tab, ma_t, k, sign_in, sign_out, scale, st);
+int launch_bs(const BsTable& tab, int io_dtype, int inner, const uint16_t* ma_t, int k,
+              const float* sign_in, const float* sign_out, float scale, hipStream_t st) {
+  const bool half = io_dtype == CTMI_F16;
+  if (inner == 32)
+    return half ? launch_bs_dtype<NT, true, true>(tab, ma_t, k, sign_in, sign_out, scale, st)
+                : launch_bs_dtype<NT, false, true>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  return half ? launch_bs_dtype<NT, true, false>(tab, ma_t, k, sign_in, sign_out, scale, st)
+              : launch_bs_dtype<NT, false, false>(tab, ma_t, k, sign_in, sign_out, scale, st);
 }
 
 }  // namespace
@@ -372,8 +410,10 @@ bool block_sylvester64_supported(int k, int io_dtype, bool both_signs) {
   return (io_dtype == CTMI_BF16 || io_dtype == CTMI_F16) && k >= 1 && k <= 224 && !both_signs;
 }
 
-int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int k, const uint16_t* ma_t,
-                             const float* sign_in, const float* sign_out, float scale, hipStream_t st) {
+int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int k, int inner,
+                             const uint16_t* ma_t, const float* sign_in, const float* sign_out,
+                             float scale, hipStream_t st) {
+  CTMI_REQUIRE(inner == 64 || inner == 32, CTMI_ERR_UNSUPPORTED, "Sylvester factor of 64 or 32");
   CTMI_REQUIRE(block_sylvester64_supported(k, io_dtype, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
                "bfloat16 or float16 tensors, blocks of up to 224 x 224 with signs on one side");
   CTMI_REQUIRE(n_jobs >= 1 && n_jobs <= kFwhtMaxJobs, CTMI_ERR_VALUE, "1 to %d tensors a launch", kFwhtMaxJobs);
@@ -395,10 +435,10 @@ int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int 
     tab.end[i] = live ? total : INT64_MAX;
   }
   tab.total = total;
-  if (k <= 32) return launch_bs<1>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
-  if (k <= 64) return launch_bs<2>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
-  if (k <= 128) return launch_bs<4>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
-  return launch_bs<7>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 32) return launch_bs<1>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 64) return launch_bs<2>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 128) return launch_bs<4>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
+  return launch_bs<7>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
 }
 
 }  // namespace ctmi

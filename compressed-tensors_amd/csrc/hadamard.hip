@@ -1072,7 +1072,7 @@ extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_
 }
 
 extern "C" int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
-  return b_dim == 64 && a_dim > 1 && block_sylvester64_supported(a_dim, io_dtype, false);
+  return (b_dim == 64 || b_dim == 32) && a_dim > 1 && block_sylvester64_supported(a_dim, io_dtype, false);
 }
 
 extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel,
@@ -1177,7 +1177,7 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
         b.rows = jobs[i].numel / n;
       }
       if (filled == kFwhtMaxJobs || (i == n_jobs && filled)) {
-        const int rc = block_sylvester64_launch(batch, filled, io_dtype, a_dim, (const uint16_t*)ma_t, sign_in, sign_out,
+        const int rc = block_sylvester64_launch(batch, filled, io_dtype, a_dim, b_dim, (const uint16_t*)ma_t, sign_in, sign_out,
                                                 1.0f / sqrtf((float)n), st);
         if (rc) return rc;
         filled = 0;

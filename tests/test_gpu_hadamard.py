@@ -468,22 +468,26 @@ def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_block
     assert ctmi.ctmi_hadamard_supported(224, 128, _lib.dtype_code(torch.bfloat16)) == 0
 
 
-@pytest.mark.parametrize("k,dtype", [(k, torch.bfloat16) for k in (224, 12, 28, 36, 64, 100, 128, 160)] +
-                         [(k, torch.float16) for k in (224, 28, 64, 100)],
+@pytest.mark.parametrize("k,dtype,inner",
+                         [(k, torch.bfloat16, 64) for k in (224, 12, 28, 36, 64, 100, 128, 160)] +
+                         [(k, torch.float16, 64) for k in (224, 28, 64, 100)] +
+                         [(k, torch.bfloat16, 32) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 32)],
                          ids=lambda v: str(v).replace("torch.", ""))
-def test_block_times_sylvester64_with_butterflies(k, dtype, ctmi, gpu, hadamard_blocks):
+def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, hadamard_blocks):
     """ctmi_hadamard_apply without mb_t (Mb = Sylvester(64)): the product with the block on the
     matrix cores, the Sylvester factor as butterflies on its fp32 result; bfloat16 and float16
-    tensors (the block is given in bfloat16 either way).  Blocks of every tile
+    tensors (the block is given in bfloat16 either way); Sylvester(32) in place of Sylvester(64)
+    (two runs share the kernel's 64 columns; odd numbers of runs, pairs that straddle two
+    tensors of one call).  Blocks of every tile
     count (K <= 32, 64, 128, 224) incl. sizes that leave rows of the last tile empty, a random
     +-1 matrix and (where the table has one) the known Hadamard block; more runs than the
     workgroups hold at a time; signs on either side; several tensors in one call."""
     from compressed_tensors_amd import _lib
 
-    announce("block x Sylvester(64), butterflies", k, dtype)
+    announce("block x Sylvester(64 or 32), butterflies", k, dtype, inner)
     code = _lib.dtype_code(dtype)
-    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 64, code) == 1
-    n = k * 64
+    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, inner, code) == 1
+    n = k * inner
     g = torch.Generator().manual_seed(k)
     rows = 2051 if k <= 64 else 1027
     x = torch.randn(rows, n, generator=g).to(dtype)
@@ -494,12 +498,12 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, ctmi, gpu, hadamard_
         blocks.append(hadamard_blocks[k].double())
     xg = x.to(gpu)
     for ma in blocks:
-        dense = torch.kron(ma, oh.deterministic_hadamard_matrix(64, torch.float64))
+        dense = torch.kron(ma, oh.deterministic_hadamard_matrix(inner, torch.float64))
         ma_t = ma.T.contiguous().bfloat16().to(gpu)
         for si, so in ((None, None), (s, None), (None, s)):
             out = torch.full_like(xg, float("nan"))
             sig, sog = (None if t is None else t.to(gpu) for t in (si, so))
-            _lib.check(ctmi.ctmi_hadamard_apply(xg.data_ptr(), out.data_ptr(), code, xg.numel(), k, 64,
+            _lib.check(ctmi.ctmi_hadamard_apply(xg.data_ptr(), out.data_ptr(), code, xg.numel(), k, inner,
                                                 ma_t.data_ptr(), None, _lib.ptr(sig), _lib.ptr(sog),
                                                 _lib.stream_of(gpu)))
             assert not bool(torch.isnan(out.float()).any()), "every element written"
@@ -514,17 +518,17 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, ctmi, gpu, hadamard_
     for job, t, o in zip(jobs, xs, outs):
         job.x, job.out, job.numel = t.data_ptr(), o.data_ptr(), t.numel()
     sg = s.to(gpu)
-    _lib.check(ctmi.ctmi_hadamard_apply_many(jobs, len(xs), code, k, 64, ma_t.data_ptr(), None, sg.data_ptr(), None,
+    _lib.check(ctmi.ctmi_hadamard_apply_many(jobs, len(xs), code, k, inner, ma_t.data_ptr(), None, sg.data_ptr(), None,
                                              _lib.stream_of(gpu)))
     for t, o in zip(xs, outs):
         one = torch.empty_like(t)
-        _lib.check(ctmi.ctmi_hadamard_apply(t.data_ptr(), one.data_ptr(), code, t.numel(), k, 64, ma_t.data_ptr(),
+        _lib.check(ctmi.ctmi_hadamard_apply(t.data_ptr(), one.data_ptr(), code, t.numel(), k, inner, ma_t.data_ptr(),
                                             None, sg.data_ptr(), None, _lib.stream_of(gpu)))
         assert_bit_equal(o, one, f"tensor of {t.shape[0]} runs")
     # what it does not take
-    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 32, code) == 0
+    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 128, code) == 0
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(225, 64, code) == 0
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 64, _lib.dtype_code(torch.float32)) == 0
-    rc = ctmi.ctmi_hadamard_apply(xg.data_ptr(), xg.data_ptr(), code, xg.numel(), k, 64, ma_t.data_ptr(), None,
+    rc = ctmi.ctmi_hadamard_apply(xg.data_ptr(), xg.data_ptr(), code, xg.numel(), k, inner, ma_t.data_ptr(), None,
                                   sg.data_ptr(), sg.data_ptr(), _lib.stream_of(gpu))
     assert rc == _lib.CTMI_ERR_UNSUPPORTED
