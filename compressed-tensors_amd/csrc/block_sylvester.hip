@@ -96,31 +96,15 @@ __device__ __forceinline__ bs_f32x16_t bs_mma(const bs_u32x4& a, const bs_u32x4&
                                                    __builtin_bit_cast(bs_bf16x8_t, b), c, 0, 0, 0);
 }
 
-// NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out;
-// HALF: float16 tensors (the matrix arrives in bfloat16 and converts exactly: entries +-1);
-// PAIR: runs of K * 32 elements (Ma (x) Sylvester(32), e.g. 7168 = 224 * 32), two at a time:
-// the 64 columns of the image are 32 of one run and 32 of the next, the two M tiles are the
-// two runs, and the butterfly stage over the M tiles is left out.  Lanes whose piece of a row
-// lies in the left half of the image (l % 8 < 4) load and store the first run, the others
-// the second; a single last run is paired with itself and its second copy is not stored.
-template <int NT, int SIGNS, bool HALF, bool PAIR>
-__global__ void __launch_bounds__(kBsThreads, 1)
-block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
-                         const float* __restrict__ signs, float scale) {
-  constexpr int KS = 2 * NT;  // steps of 16 over the contracted index
-  constexpr int INNER = PAIR ? 32 : 64;
-  extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
-  bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
-  bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [NT * 4][64] (SIGNS != 0)
-  const uint32_t l = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+// The fragments of Ma into LDS, zero beyond K: fragment (ks, nt), lane (c, g) holds
+// Ma[16 ks + 8 g + e][32 nt + c], e = 0..7.  Eight at a time per wavefront, loads first: one
+// after the other they would cost the launch as many memory round trips as there are
+// fragments.
+template <int NT, bool HALF>
+__device__ __forceinline__ void bs_load_fragments(const uint16_t* __restrict__ ma_t, int k_dim,
+                                                  bs_u32x4* ma_frag, uint32_t wave, uint32_t l) {
+  constexpr int KS = 2 * NT;
   const uint32_t c = l & 31u, g = l >> 5;
-  uint32_t* image = bs_lds + (KS * NT + (SIGNS ? NT * 4 : 0)) * kWave * 4 + wave * kBsRing;
-  const int64_t n = (int64_t)k_dim * INNER;
-  const uint32_t piece = 8 * (l & (INNER / 8 - 1));  // the lane's 8 columns inside a row of a run
-  const bool second = PAIR && (l & 4u);              // the lane belongs to the second run of a pair
-
-  // The fragments of Ma, zero beyond K.  Eight at a time per wavefront, loads first: one after
-  // the other they would cost the launch as many memory round trips as there are fragments.
   const bool ma_vectors = k_dim % 8 == 0 && (uintptr_t)ma_t % 16 == 0;  // 16-byte pieces of whole rows
   for (int f0 = 0; f0 < KS * NT; f0 += kBsWaves * 8) {
     bs_u32x4 w[8];
@@ -155,6 +139,32 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       if (f < KS * NT) ma_frag[f * kWave + l] = w[u];
     }
   }
+}
+
+// NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out;
+// HALF: float16 tensors (the matrix arrives in bfloat16 and converts exactly: entries +-1);
+// PAIR: runs of K * 32 elements (Ma (x) Sylvester(32), e.g. 7168 = 224 * 32), two at a time:
+// the 64 columns of the image are 32 of one run and 32 of the next, the two M tiles are the
+// two runs, and the butterfly stage over the M tiles is left out.  Lanes whose piece of a row
+// lies in the left half of the image (l % 8 < 4) load and store the first run, the others
+// the second; a single last run is paired with itself and its second copy is not stored.
+template <int NT, int SIGNS, bool HALF, bool PAIR>
+__global__ void __launch_bounds__(kBsThreads, 1)
+block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
+                         const float* __restrict__ signs, float scale) {
+  constexpr int KS = 2 * NT;  // steps of 16 over the contracted index
+  constexpr int INNER = PAIR ? 32 : 64;
+  extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
+  bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
+  bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [NT * 4][64] (SIGNS != 0)
+  const uint32_t l = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const uint32_t c = l & 31u, g = l >> 5;
+  uint32_t* image = bs_lds + (KS * NT + (SIGNS ? NT * 4 : 0)) * kWave * 4 + wave * kBsRing;
+  const int64_t n = (int64_t)k_dim * INNER;
+  const uint32_t piece = 8 * (l & (INNER / 8 - 1));  // the lane's 8 columns inside a row of a run
+  const bool second = PAIR && (l & 4u);              // the lane belongs to the second run of a pair
+
+  bs_load_fragments<NT, HALF>(ma_t, k_dim, ma_frag, wave, l);
   // Sign masks of the vectors a lane loads (SIGNS == 1: vector q of chunk ch is row
   // 32 ch + l / 8 + 8 q, columns 8 (l % 8) ...) or stores (SIGNS == 2: the same positions with
   // the tile nt in place of the chunk): the same for the four wavefronts, read at each use
@@ -354,6 +364,208 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   }
 }
 
+// ---------------------------------------------------------------- Ma (x) Sylvester(128)
+// Runs of K * 128 elements (28672 = 224 * 128).  Sylvester(128) = Sylvester(2) (x) Sylvester(64):
+// a row of the run is two halves of 64 columns, each half goes through the product with Ma
+// like a run of the kernel above, and the stage over the halves is one more addition and
+// subtraction of accumulator tiles in front of the other six.  Four M tiles of accumulators
+// for all of Ma's column tiles do not fit a wavefront, so the order is turned round: first
+// all A operands of the run (both halves, 32 NT registers), then one output tile of Ma after
+// the other, each with its four accumulator tiles, its butterflies and its stores; one read
+// of a fragment of Ma serves four products.  No run is held ahead.
+// Sign masks: one word per lane and vector in LDS (bit 15 - d / 31 - d for the two elements
+// of dword d), expanded by a shift and a mask at each use: whole masks would not fit.
+constexpr size_t bs128_lds_bytes(int nt, bool signs) {
+  return ((size_t)2 * nt * nt * kWave * 4 + (signs ? (size_t)2 * nt * 4 * kWave : 0) +
+          (size_t)kBsWaves * kBsRing) * sizeof(uint32_t);
+}
+
+template <int NT, int SIGNS, bool HALF>
+__global__ void __launch_bounds__(kBsThreads, 1)
+block_sylvester128_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
+                          const float* __restrict__ signs, float scale) {
+  constexpr int KS = 2 * NT;
+  extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
+  bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);   // [KS * NT][64]
+  uint32_t* flipc = bs_lds + KS * NT * kWave * 4;            // [2][NT * 4][64] (SIGNS != 0)
+  const uint32_t l = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const uint32_t c = l & 31u, g = l >> 5;
+  uint32_t* image = bs_lds + KS * NT * kWave * 4 + (SIGNS ? 2 * NT * 4 * kWave : 0) + wave * kBsRing;
+  const int64_t n = (int64_t)k_dim * 128;
+  bs_load_fragments<NT, HALF>(ma_t, k_dim, ma_frag, wave, l);
+  if constexpr (SIGNS != 0) {
+    for (int f = (int)wave; f < 2 * NT * 4; f += kBsWaves) {
+      const int hf = f / (NT * 4), rest = f % (NT * 4);
+      const int row = 32 * (rest >> 2) + (int)(l >> 3) + 8 * (rest & 3);
+      uint32_t m = 0;
+      if (row < k_dim) {
+        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + 128 * row +
+                                                     64 * hf + 8 * (l & 7u));
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+          m |= ((s8.v[2 * d] >> 31) << (15 - d)) | ((s8.v[2 * d + 1] >> 31) << (31 - d));
+      }
+      flipc[f * kWave + l] = m;
+    }
+  }
+  __syncthreads();
+  const uint32_t pick = (c & 1u) ? 0x07060302u : 0x05040100u;
+  auto pack2 = [](float lo, float hi) -> uint32_t {
+    if constexpr (HALF) return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
+    else return pack_bf16x2(lo, hi);
+  };
+  auto flip_of = [&](int hf, int tile, int q) {  // the lane's mask for vector q of a chunk / tile
+    const uint32_t m = flipc[((hf * NT + tile) * 4 + q) * kWave + l];
+    bs_u32x4 w;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) w[d] = (m << d) & 0x80008000u;
+    return w;
+  };
+  const int64_t step = (int64_t)gridDim.x * kBsWaves;
+  for (int64_t run = (int64_t)blockIdx.x * kBsWaves + wave; run < tab.total; run += step) {
+    int64_t local;
+    const int j = bs_job(tab, run, &local);
+    const uint16_t* __restrict__ xr = static_cast<const uint16_t*>(tab.x[j]) + local * n;
+    uint16_t* __restrict__ yr = static_cast<uint16_t*>(tab.out[j]) + local * n;
+    // ---- the A operands of both halves: aop[hf][ks][mt]
+    bs_u32x4 aop[2][KS][2];
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      bs_u32x4 in[NT][4];
+#pragma unroll
+      for (int ch = 0; ch < NT; ++ch)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int row = 32 * ch + (int)(l >> 3) + 8 * q;
+          in[ch][q] = __builtin_bit_cast(
+              bs_u32x4, ldg_nt<uint16_t, 8>(xr + 128 * (row < k_dim ? row : k_dim - 1) + 64 * hf + 8 * (l & 7u)));
+        }
+#pragma unroll
+      for (int ch = 0; ch < NT; ++ch) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          bs_u32x4 w = in[ch][q];
+          if (32 * ch + (int)(l >> 3) + 8 * q >= k_dim) w = bs_u32x4{0u, 0u, 0u, 0u};
+          if constexpr (SIGNS == 1) w ^= flip_of(hf, ch, q);
+          *reinterpret_cast<bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]) = w;
+        }
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ++ks2)
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) {
+              const uint32_t* p = &image[(16 * ks2 + 8 * g + 2 * d) * kBsPitch + 16 * mt + (c >> 1)];
+              aop[hf][2 * ch + ks2][mt][d] = __builtin_amdgcn_perm(p[kBsPitch], p[0], pick);
+            }
+      }
+    }
+    // ---- one output tile of Ma after the other
+    const uint32_t h = g;  // after the exchange: lane half h holds columns 32 h ... of its half
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) {
+      bs_f32x16_t acc[2][2];
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[hf][mt][i] = 0.0f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bs_u32x4 b = ma_frag[(ks * NT + nt) * kWave + l];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf)
+#pragma unroll
+          for (int mt = 0; mt < 2; ++mt) acc[hf][mt] = bs_mma<HALF>(aop[hf][ks][mt], b, acc[hf][mt]);
+      }
+#pragma unroll
+      for (int oh = 0; oh < 2; ++oh) {  // output half: sum (0) or difference (1) of the input halves
+        float u[2][16];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const float y0 = oh == 0 ? acc[0][0][v] + acc[1][0][v] : acc[0][0][v] - acc[1][0][v];  // stage over the halves
+          const float y1 = oh == 0 ? acc[0][1][v] + acc[1][1][v] : acc[0][1][v] - acc[1][1][v];
+          const float s = y0 + y1, t = y0 - y1;  // stage over mt
+          const auto pr = __builtin_amdgcn_permlane32_swap(__float_as_uint(s), __float_as_uint(t), false, false);
+          const float lower = __uint_as_float(pr[0]), upper = __uint_as_float(pr[1]);  // g = 0, g = 1
+          u[0][v] = lower + upper;
+          u[1][v] = lower - upper;
+        }
+#pragma unroll
+        for (int x = 0; x < 2; ++x)
+#pragma unroll
+          for (int st = 1; st < 16; st <<= 1)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+              if ((v & st) == 0) {
+                const float p = u[x][v], m = u[x][v + st];
+                u[x][v] = p + m;
+                u[x][v + st] = p - m;
+              }
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          bs_u32x4 w;
+          w[0] = pack2(u[0][4 * b] * scale, u[0][4 * b + 1] * scale);
+          w[1] = pack2(u[0][4 * b + 2] * scale, u[0][4 * b + 3] * scale);
+          w[2] = pack2(u[1][4 * b] * scale, u[1][4 * b + 1] * scale);
+          w[3] = pack2(u[1][4 * b + 2] * scale, u[1][4 * b + 3] * scale);
+          *reinterpret_cast<bs_u32x4*>(&image[c * kBsPitch + 16 * h + 4 * b]) = w;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int row = 32 * nt + (int)(l >> 3) + 8 * q;
+          bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
+          if constexpr (SIGNS == 2) w ^= flip_of(oh, nt, q);
+          if (row < k_dim)
+            stg_nt<uint16_t, 8>(yr + 128 * row + 64 * oh + 8 * (l & 7u), __builtin_bit_cast(Vec<uint16_t, 8>, w));
+        }
+      }
+    }
+  }
+}
+
+template <int NT, int SIGNS, bool HALF>
+int launch_bs128_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
+                         hipStream_t st) {
+  auto kern = block_sylvester128_kernel<NT, SIGNS, HALF>;
+  constexpr size_t lds = bs128_lds_bytes(NT, SIGNS != 0);
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  }
+  static int per_cu = 0;
+  int dev = 0, cus = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e == hipSuccess) e = hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev);
+  if (e == hipSuccess && per_cu == 0) {
+    int n = 0;
+    e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kern, kBsThreads, lds);
+    per_cu = n > 0 ? n : 1;
+  }
+  if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "device query: %s", hipGetErrorString(e));
+  const int64_t wgs = cdiv(tab.total, kBsWaves);
+  const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * per_cu;
+  const int64_t each = cdiv(wgs, cap);
+  const unsigned grid = (unsigned)cdiv(wgs, each);
+  hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale);
+  return CTMI_OK;
+}
+
+template <int NT>
+int launch_bs128(const BsTable& tab, int io_dtype, const uint16_t* ma_t, int k, const float* sign_in,
+                 const float* sign_out, float scale, hipStream_t st) {
+  const bool half = io_dtype == CTMI_F16;
+#define CTMI_BS128(S, signs)                                                                  \
+  (half ? launch_bs128_variant<NT, S, true>(tab, ma_t, k, signs, scale, st)                   \
+        : launch_bs128_variant<NT, S, false>(tab, ma_t, k, signs, scale, st))
+  if (sign_in) return CTMI_BS128(1, sign_in);
+  if (sign_out) return CTMI_BS128(2, sign_out);
+  return CTMI_BS128(0, nullptr);
+#undef CTMI_BS128
+}
+
 template <int NT, int SIGNS, bool HALF, bool PAIR>
 int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
                       hipStream_t st) {
@@ -413,7 +625,8 @@ bool block_sylvester64_supported(int k, int io_dtype, bool both_signs) {
 int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int k, int inner,
                              const uint16_t* ma_t, const float* sign_in, const float* sign_out,
                              float scale, hipStream_t st) {
-  CTMI_REQUIRE(inner == 64 || inner == 32, CTMI_ERR_UNSUPPORTED, "Sylvester factor of 64 or 32");
+  CTMI_REQUIRE(inner == 128 || inner == 64 || inner == 32, CTMI_ERR_UNSUPPORTED,
+               "Sylvester factor of 32, 64 or 128");
   CTMI_REQUIRE(block_sylvester64_supported(k, io_dtype, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
                "bfloat16 or float16 tensors, blocks of up to 224 x 224 with signs on one side");
   CTMI_REQUIRE(n_jobs >= 1 && n_jobs <= kFwhtMaxJobs, CTMI_ERR_VALUE, "1 to %d tensors a launch", kFwhtMaxJobs);
@@ -435,6 +648,12 @@ int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int 
     tab.end[i] = live ? total : INT64_MAX;
   }
   tab.total = total;
+  if (inner == 128) {
+    if (k <= 32) return launch_bs128<1>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+    if (k <= 64) return launch_bs128<2>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+    if (k <= 128) return launch_bs128<4>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+    return launch_bs128<7>(tab, io_dtype, ma_t, k, sign_in, sign_out, scale, st);
+  }
   if (k <= 32) return launch_bs<1>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
   if (k <= 64) return launch_bs<2>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
   if (k <= 128) return launch_bs<4>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);

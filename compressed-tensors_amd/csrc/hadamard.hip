@@ -1072,7 +1072,8 @@ extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_
 }
 
 extern "C" int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
-  return (b_dim == 64 || b_dim == 32) && a_dim > 1 && block_sylvester64_supported(a_dim, io_dtype, false);
+  return (b_dim == 128 || b_dim == 64 || b_dim == 32) && a_dim > 1 &&
+         block_sylvester64_supported(a_dim, io_dtype, false);
 }
 
 extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel,

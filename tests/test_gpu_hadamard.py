@@ -471,20 +471,22 @@ def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_block
 @pytest.mark.parametrize("k,dtype,inner",
                          [(k, torch.bfloat16, 64) for k in (224, 12, 28, 36, 64, 100, 128, 160)] +
                          [(k, torch.float16, 64) for k in (224, 28, 64, 100)] +
-                         [(k, torch.bfloat16, 32) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 32)],
+                         [(k, torch.bfloat16, 32) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 32)] +
+                         [(k, torch.bfloat16, 128) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 128)],
                          ids=lambda v: str(v).replace("torch.", ""))
 def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, hadamard_blocks):
     """ctmi_hadamard_apply without mb_t (Mb = Sylvester(64)): the product with the block on the
     matrix cores, the Sylvester factor as butterflies on its fp32 result; bfloat16 and float16
     tensors (the block is given in bfloat16 either way); Sylvester(32) in place of Sylvester(64)
     (two runs share the kernel's 64 columns; odd numbers of runs, pairs that straddle two
-    tensors of one call).  Blocks of every tile
+    tensors of one call) and Sylvester(128) (28672 = 224 * 128: two halves of 64 columns and a
+    stage over the halves).  Blocks of every tile
     count (K <= 32, 64, 128, 224) incl. sizes that leave rows of the last tile empty, a random
     +-1 matrix and (where the table has one) the known Hadamard block; more runs than the
     workgroups hold at a time; signs on either side; several tensors in one call."""
     from compressed_tensors_amd import _lib
 
-    announce("block x Sylvester(64 or 32), butterflies", k, dtype, inner)
+    announce("block x Sylvester(32 / 64 / 128), butterflies", k, dtype, inner)
     code = _lib.dtype_code(dtype)
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, inner, code) == 1
     n = k * inner
@@ -498,7 +500,7 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, ha
         blocks.append(hadamard_blocks[k].double())
     xg = x.to(gpu)
     for ma in blocks:
-        dense = torch.kron(ma, oh.deterministic_hadamard_matrix(inner, torch.float64))
+        sylvester = oh.deterministic_hadamard_matrix(inner, torch.float64)
         ma_t = ma.T.contiguous().bfloat16().to(gpu)
         for si, so in ((None, None), (s, None), (None, s)):
             out = torch.full_like(xg, float("nan"))
@@ -508,7 +510,9 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, ha
                                                 _lib.stream_of(gpu)))
             assert not bool(torch.isnan(out.float()).any()), "every element written"
             xs = x[sample].double() * (1.0 if si is None else si.double())
-            want = xs @ dense * (1.0 if so is None else so.double()) / n ** 0.5
+            # x (Ma (x) S) for the run seen as a k x inner matrix X: Ma^T X S
+            want = torch.einsum("rki,kj,im->rjm", xs.unflatten(-1, (k, inner)), ma, sylvester).flatten(-2, -1)
+            want = want * (1.0 if so is None else so.double()) / n ** 0.5
             _assert_within_ulp(out[sample.to(gpu)], want.to(dtype), f"signs in={si is not None} out={so is not None}")
     # several tensors from one call == one by one
     ma_t = blocks[0].T.contiguous().bfloat16().to(gpu)
@@ -526,7 +530,7 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, ha
                                             None, sg.data_ptr(), None, _lib.stream_of(gpu)))
         assert_bit_equal(o, one, f"tensor of {t.shape[0]} runs")
     # what it does not take
-    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 128, code) == 0
+    assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 256, code) == 0
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(225, 64, code) == 0
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 64, _lib.dtype_code(torch.float32)) == 0
     rc = ctmi.ctmi_hadamard_apply(xg.data_ptr(), xg.data_ptr(), code, xg.numel(), k, inner, ma_t.data_ptr(), None,
