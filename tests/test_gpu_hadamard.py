@@ -372,12 +372,12 @@ def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
     assert rc == _lib.CTMI_ERR_UNSUPPORTED  # 512 lanes only for the Sylvester factor
 
 
-@pytest.mark.parametrize("size", [768, 1600, 7168, 14336, 32, 256, 512, 16])
+@pytest.mark.parametrize("size", [768, 1600, 3584, 7168, 14336, 32, 256, 512, 16])
 @pytest.mark.parametrize("location,inverse", [("input", False), ("weight_input", True),
                                               ("weight_output", False), ("output", True)])
 def test_random_hadamard_of_any_table_size(size, location, inverse, gpu, hadamard_table_path):
-    """sizes K * 2^m from the table of known matrices (14336 = 224 * 64: Llama-3's
-    intermediate size), 32 (whose table entry is not Sylvester's) and the powers of two
+    """sizes K * 2^m from the table of known matrices (3584 = 28 * 128, 7168 = 224 * 32,
+    14336 = 224 * 64: Llama-3's intermediate size), 32 (whose table entry is not Sylvester's) and the powers of two
     that have no matrix-core kernel: forward against the dense fp64 matrix the oracle
     builds with the reference's butterfly stages"""
     from compressed_tensors_amd.transform import (
