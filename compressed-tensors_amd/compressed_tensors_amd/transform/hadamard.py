@@ -610,6 +610,23 @@ def _kron_plan(n: int, block: Optional[Tensor]) -> Optional[Tuple[int, int]]:
     return None
 
 
+def _matrix_core_split(lib, k: int, b: int, code: int) -> Optional[Tuple[int, int, bool]]:
+    """(a, inner, butterflies) for H = B (x) Sylvester(b) with a k x k block B (k = 1: Sylvester
+    alone) on the matrix cores: an a x a block as the explicit factor and Sylvester(inner) as
+    butterflies on its product, or both as products.  Where b itself is not an inner size of
+    the kernel, the block grows by a Sylvester factor:
+    B (x) S(b) = (B (x) S(b / inner)) (x) S(inner), e.g. 5120 = 20 * 256 = 40 * 128."""
+    if k > 1 and lib.ctmi_hadamard_sylvester_inner_supported(k, b, code):
+        return k, b, True
+    for inner in (128, 64, 32):
+        if b > inner and b % inner == 0 and lib.ctmi_hadamard_sylvester_inner_supported(
+                k * (b // inner), inner, code):
+            return k * (b // inner), inner, True
+    if k > 1 and lib.ctmi_hadamard_supported(k, b, code):
+        return k, b, False
+    return None
+
+
 class HadamardTransform(torch.nn.Module):
     """W = diag(signs) * H, optionally row/column permuted by `perm` (W[perm][:, perm]),
     where H = Sylvester(size) or, with `block` = a known K x K Hadamard matrix,
@@ -675,14 +692,13 @@ class HadamardTransform(torch.nn.Module):
         n = self.size
         lib = _lib.load()
         mfma = self.block is None and hadamard_kernel_exists(n, value.dtype)  # or the butterfly kernel
-        big = None  # (a, b): a known block times Sylvester(b) on the matrix cores
+        big = None  # (a, b): an a x a block times Sylvester(b) on the matrix cores
         inner_butterflies = False  # ... with Sylvester(b) as butterflies on the block product
-        if not mfma and self.block is not None and value.dtype in _FLOATS:
-            k, code = int(self.block.shape[0]), _lib.dtype_code(value.dtype)
-            if lib.ctmi_hadamard_sylvester_inner_supported(k, n // k, code):
-                big, inner_butterflies = (k, n // k), True
-            elif lib.ctmi_hadamard_supported(k, n // k, code):
-                big = (k, n // k)
+        if not mfma and value.dtype in _FLOATS:
+            k = 1 if self.block is None else int(self.block.shape[0])
+            split = _matrix_core_split(lib, k, n // k, _lib.dtype_code(value.dtype))
+            if split is not None:
+                big, inner_butterflies = split[:2], split[2]
         plan = None if (mfma or big) else _kron_plan(n, self.block)
         if plan is not None and not (value.dtype in _FLOATS and bool(
                 lib.ctmi_kron_matmul_supported(plan[0], plan[1], _lib.dtype_code(value.dtype)))):
@@ -718,7 +734,11 @@ class HadamardTransform(torch.nn.Module):
             a, b = big
             key = ("bf16", str(x.device), transposed)
             if key not in self._factor:
-                m = self.block.to(device=x.device, dtype=torch.bfloat16)
+                k = 1 if self.block is None else int(self.block.shape[0])
+                m = (torch.ones(1, 1, dtype=torch.bfloat16, device=x.device) if self.block is None
+                     else self.block.to(device=x.device, dtype=torch.bfloat16))
+                if a > k:  # the block grown by a Sylvester factor (symmetric: transposes with m)
+                    m = torch.kron(m, _sylvester_bf16(a // k, x.device))
                 self._factor[key] = (m.T if transposed else m).contiguous()
             x = x.contiguous()
             y = torch.empty_like(x)

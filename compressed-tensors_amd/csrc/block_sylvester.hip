@@ -143,26 +143,33 @@ __device__ __forceinline__ void bs_load_fragments(const uint16_t* __restrict__ m
 
 // NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out;
 // HALF: float16 tensors (the matrix arrives in bfloat16 and converts exactly: entries +-1);
-// PAIR: runs of K * 32 elements (Ma (x) Sylvester(32), e.g. 7168 = 224 * 32), two at a time:
-// the 64 columns of the image are 32 of one run and 32 of the next, the two M tiles are the
-// two runs, and the butterfly stage over the M tiles is left out.  Lanes whose piece of a row
-// lies in the left half of the image (l % 8 < 4) load and store the first run, the others
-// the second; a single last run is paired with itself and its second copy is not stored.
-template <int NT, int SIGNS, bool HALF, bool PAIR>
+// PAIR (RUNS != 1): runs of K * 2^log_inner elements, 2^log_inner = 32, 16 or 8 (Ma (x) Sylvester(32),
+// e.g. 7168 = 224 * 32, 3584 = 224 * 16, 1792 = 224 * 8), two, four or eight at a time: the
+// 64 columns of the image are 32 (16, 8) of one run beside those of the next, and the
+// butterfly stages over the column bits that tell the runs apart are left out (the stage over
+// the M tiles always; 16: the one 16 columns apart as well; 8: and the one 8 apart).  A lane
+// loads and stores the run its piece of a row lies in; where the tensors end inside a unit
+// the missing runs are read as the last one once more and not stored.
+// RUNS: 1 for Sylvester(64), 2 for Sylvester(32), 0 for 16 and 8 (log_inner read at run time:
+// the two share a kernel).
+template <int NT, int SIGNS, bool HALF, int RUNS>
 __global__ void __launch_bounds__(kBsThreads, 1)
 block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
-                         const float* __restrict__ signs, float scale) {
+                         const float* __restrict__ signs, float scale, int log_inner) {
   constexpr int KS = 2 * NT;  // steps of 16 over the contracted index
-  constexpr int INNER = PAIR ? 32 : 64;
+  constexpr bool PAIR = RUNS != 1;
+  if constexpr (RUNS == 1) log_inner = 6;
+  if constexpr (RUNS == 2) log_inner = 5;
+  const int unit_runs = 64 >> log_inner;  // runs side by side in the image
   extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
   bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
   bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [NT * 4][64] (SIGNS != 0)
   const uint32_t l = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const uint32_t c = l & 31u, g = l >> 5;
   uint32_t* image = bs_lds + (KS * NT + (SIGNS ? NT * 4 : 0)) * kWave * 4 + wave * kBsRing;
-  const int64_t n = (int64_t)k_dim * INNER;
-  const uint32_t piece = 8 * (l & (INNER / 8 - 1));  // the lane's 8 columns inside a row of a run
-  const bool second = PAIR && (l & 4u);              // the lane belongs to the second run of a pair
+  const int64_t n = (int64_t)k_dim << log_inner;
+  const uint32_t piece = 8 * (l & ((1u << (log_inner - 3)) - 1u));  // the lane's 8 columns inside a row of a run
+  const uint32_t my_run = PAIR ? (l & 7u) >> (log_inner - 3) : 0u;  // ... and that run's place in the unit
 
   bs_load_fragments<NT, HALF>(ma_t, k_dim, ma_frag, wave, l);
   // Sign masks of the vectors a lane loads (SIGNS == 1: vector q of chunk ch is row
@@ -173,7 +180,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       const int row = 32 * (f >> 2) + (int)(l >> 3) + 8 * (f & 3);
       bs_u32x4 m = {0u, 0u, 0u, 0u};
       if (row < k_dim) {
-        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + INNER * row + piece);
+        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + ((int64_t)row << log_inner) + piece);
 #pragma unroll
         for (int d = 0; d < 4; ++d) m[d] = ((s8.v[2 * d] >> 16) & 0x8000u) | (s8.v[2 * d + 1] & 0x80000000u);
       }
@@ -193,16 +200,21 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   // the spot): a run beyond the last reads the last again, a row beyond K reads row K - 1 and
   // is replaced by zeros when it is used.
   bs_u32x4 in[NT][4];
-  // where the lane's run of unit u begins (a unit: one run, or PAIR: two neighbouring ones);
+  // where the lane's run of unit u begins (a unit: one run, or PAIR: up to eight neighbouring
+  // ones, each looked up with scalar instructions and kept by the lanes it belongs to);
   // table reads once per unit, not per chunk
   auto run_start = [&](int64_t u) {
     if constexpr (PAIR) {
-      int64_t la, lb;
-      const int64_t ra = min(2 * u, tab.total - 1), rb = min(2 * u + 1, tab.total - 1);
-      const int ja = bs_job(tab, ra, &la), jb = bs_job(tab, rb, &lb);
-      const uint16_t* a = static_cast<const uint16_t*>(tab.x[ja]) + la * n;
-      const uint16_t* b = static_cast<const uint16_t*>(tab.x[jb]) + lb * n;
-      return second ? b : a;
+      const uint16_t* mine = nullptr;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (i < unit_runs) {
+          int64_t local;
+          const int j = bs_job(tab, min(unit_runs * u + i, tab.total - 1), &local);
+          const uint16_t* p = static_cast<const uint16_t*>(tab.x[j]) + local * n;
+          mine = my_run == (uint32_t)i ? p : mine;
+        }
+      return mine;
     } else {
       const int64_t r = u < tab.total ? u : tab.total - 1;
       int64_t local;
@@ -215,10 +227,10 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
     for (int q = 0; q < 4; ++q) {
       const int row = 32 * ch + (int)(l >> 3) + 8 * q;
       in[ch][q] = __builtin_bit_cast(
-          bs_u32x4, ldg_nt<uint16_t, 8>(xr + INNER * (row < k_dim ? row : k_dim - 1) + piece));
+          bs_u32x4, ldg_nt<uint16_t, 8>(xr + ((int64_t)(row < k_dim ? row : k_dim - 1) << log_inner) + piece));
     }
   };
-  const int64_t units = PAIR ? (tab.total + 1) / 2 : tab.total;
+  const int64_t units = (tab.total + unit_runs - 1) >> (6 - log_inner);
 
   auto pack2 = [](float lo, float hi) -> uint32_t {
     if constexpr (HALF) return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
@@ -298,21 +310,24 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
     }
     // butterflies over j = 32 mt + 8 b + 4 g + r
     uint16_t* __restrict__ yr;
-    bool stored = true;  // PAIR: the second copy of a single last run is not
+    bool stored = true;  // PAIR: a run past the last tensor is not
     if constexpr (PAIR) {
-      int64_t la, lb;
-      const int64_t rb = 2 * run + 1 < tab.total ? 2 * run + 1 : 2 * run;
-      const int ja = bs_job(tab, 2 * run, &la), jb = bs_job(tab, rb, &lb);
-      uint16_t* a = static_cast<uint16_t*>(tab.out[ja]) + la * n;
-      uint16_t* b = static_cast<uint16_t*>(tab.out[jb]) + lb * n;
-      yr = second ? b : a;
-      stored = !second || 2 * run + 1 < tab.total;
+      yr = nullptr;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        if (i < unit_runs) {
+          int64_t local;
+          const int j = bs_job(tab, min(unit_runs * run + i, tab.total - 1), &local);
+          uint16_t* p = static_cast<uint16_t*>(tab.out[j]) + local * n;
+          yr = my_run == (uint32_t)i ? p : yr;
+        }
+      stored = unit_runs * run + (int64_t)my_run < tab.total;
     } else {
       int64_t local;
       const int j = bs_job(tab, run, &local);
       yr = static_cast<uint16_t*>(tab.out[j]) + local * n;
     }
-    const uint32_t h = g;  // after the exchange: lane half h holds j = 32 h ... (PAIR: run h of the two)
+    const uint32_t h = g;  // after the exchange: lane half h holds j = 32 h ... (PAIR: other runs than half 1 - h)
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
       float u[2][16];  // u[x][4 b + r] = value at j = 32 h + 8 b + 4 x + r
@@ -329,7 +344,9 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
 #pragma unroll
       for (int x = 0; x < 2; ++x)
 #pragma unroll
-        for (int st = 1; st < 16; st <<= 1)
+        for (int st = 1; st < 16; st <<= 1) {
+          // value 4 b + r sits at column 8 b + 4 x + r: st = 4 pairs columns 8 apart, st = 8 16 apart
+          if (PAIR && ((st == 8 && log_inner < 5) || (st == 4 && log_inner < 4))) continue;
 #pragma unroll
           for (int v = 0; v < 16; ++v)
             if ((v & st) == 0) {
@@ -337,6 +354,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
               u[x][v] = p + m;
               u[x][v + st] = p - m;
             }
+        }
       // row c of this tile, 32 outputs from column 32 h: 8 b + 4 x + r -> four vectors of 8
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
@@ -358,7 +376,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
         if constexpr (SIGNS == 2) w ^= fo[q];
         if (row < k_dim && stored)
-          stg_nt<uint16_t, 8>(yr + INNER * row + piece, __builtin_bit_cast(Vec<uint16_t, 8>, w));
+          stg_nt<uint16_t, 8>(yr + ((int64_t)row << log_inner) + piece, __builtin_bit_cast(Vec<uint16_t, 8>, w));
       }
     }
   }
@@ -566,10 +584,10 @@ int launch_bs128(const BsTable& tab, int io_dtype, const uint16_t* ma_t, int k, 
 #undef CTMI_BS128
 }
 
-template <int NT, int SIGNS, bool HALF, bool PAIR>
+template <int NT, int SIGNS, bool HALF, int RUNS>
 int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
-                      hipStream_t st) {
-  auto kern = block_sylvester64_kernel<NT, SIGNS, HALF, PAIR>;
+                      int log_inner, hipStream_t st) {
+  auto kern = block_sylvester64_kernel<NT, SIGNS, HALF, RUNS>;
   constexpr size_t lds = bs_lds_bytes(NT, SIGNS != 0);
   if (lds > 48 * 1024) {
     // the attribute belongs to the kernel as loaded on one device; setting it again is cheap
@@ -589,31 +607,36 @@ int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const flo
     per_cu = n > 0 ? n : 1;
   }
   if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "device query: %s", hipGetErrorString(e));
-  const int64_t wgs = cdiv(PAIR ? (tab.total + 1) / 2 : tab.total, kBsWaves);
+  const int64_t wgs = cdiv(cdiv(tab.total, (int64_t)(64 >> log_inner)), kBsWaves);
   const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * per_cu;
   const int64_t each = cdiv(wgs, cap);  // runs per wavefront, the same for all
   const unsigned grid = (unsigned)cdiv(wgs, each);
-  hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale);
+  hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale, log_inner);
   return CTMI_OK;
 }
 
-template <int NT, bool HALF, bool PAIR>
+template <int NT, bool HALF, int RUNS>
 int launch_bs_dtype(const BsTable& tab, const uint16_t* ma_t, int k, const float* sign_in,
-                    const float* sign_out, float scale, hipStream_t st) {
-  if (sign_in) return launch_bs_variant<NT, 1, HALF, PAIR>(tab, ma_t, k, sign_in, scale, st);
-  if (sign_out) return launch_bs_variant<NT, 2, HALF, PAIR>(tab, ma_t, k, sign_out, scale, st);
-  return launch_bs_variant<NT, 0, HALF, PAIR>(tab, ma_t, k, nullptr, scale, st);
+                    const float* sign_out, float scale, int log_inner, hipStream_t st) {
+  if (sign_in) return launch_bs_variant<NT, 1, HALF, RUNS>(tab, ma_t, k, sign_in, scale, log_inner, st);
+  if (sign_out) return launch_bs_variant<NT, 2, HALF, RUNS>(tab, ma_t, k, sign_out, scale, log_inner, st);
+  return launch_bs_variant<NT, 0, HALF, RUNS>(tab, ma_t, k, nullptr, scale, log_inner, st);
 }
 
 template <int NT>
 int launch_bs(const BsTable& tab, int io_dtype, int inner, const uint16_t* ma_t, int k,
               const float* sign_in, const float* sign_out, float scale, hipStream_t st) {
   const bool half = io_dtype == CTMI_F16;
+  if (inner < 32) {
+    const int log_inner = inner == 16 ? 4 : 3;
+    return half ? launch_bs_dtype<NT, true, 0>(tab, ma_t, k, sign_in, sign_out, scale, log_inner, st)
+                : launch_bs_dtype<NT, false, 0>(tab, ma_t, k, sign_in, sign_out, scale, log_inner, st);
+  }
   if (inner == 32)
-    return half ? launch_bs_dtype<NT, true, true>(tab, ma_t, k, sign_in, sign_out, scale, st)
-                : launch_bs_dtype<NT, false, true>(tab, ma_t, k, sign_in, sign_out, scale, st);
-  return half ? launch_bs_dtype<NT, true, false>(tab, ma_t, k, sign_in, sign_out, scale, st)
-              : launch_bs_dtype<NT, false, false>(tab, ma_t, k, sign_in, sign_out, scale, st);
+    return half ? launch_bs_dtype<NT, true, 2>(tab, ma_t, k, sign_in, sign_out, scale, 5, st)
+                : launch_bs_dtype<NT, false, 2>(tab, ma_t, k, sign_in, sign_out, scale, 5, st);
+  return half ? launch_bs_dtype<NT, true, 1>(tab, ma_t, k, sign_in, sign_out, scale, 6, st)
+              : launch_bs_dtype<NT, false, 1>(tab, ma_t, k, sign_in, sign_out, scale, 6, st);
 }
 
 }  // namespace
@@ -625,8 +648,8 @@ bool block_sylvester64_supported(int k, int io_dtype, bool both_signs) {
 int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int k, int inner,
                              const uint16_t* ma_t, const float* sign_in, const float* sign_out,
                              float scale, hipStream_t st) {
-  CTMI_REQUIRE(inner == 128 || inner == 64 || inner == 32, CTMI_ERR_UNSUPPORTED,
-               "Sylvester factor of 32, 64 or 128");
+  CTMI_REQUIRE(inner == 128 || inner == 64 || inner == 32 || inner == 16 || inner == 8, CTMI_ERR_UNSUPPORTED,
+               "Sylvester factor of 8, 16, 32, 64 or 128");
   CTMI_REQUIRE(block_sylvester64_supported(k, io_dtype, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
                "bfloat16 or float16 tensors, blocks of up to 224 x 224 with signs on one side");
   CTMI_REQUIRE(n_jobs >= 1 && n_jobs <= kFwhtMaxJobs, CTMI_ERR_VALUE, "1 to %d tensors a launch", kFwhtMaxJobs);

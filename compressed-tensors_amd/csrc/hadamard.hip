@@ -1072,7 +1072,7 @@ extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_
 }
 
 extern "C" int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
-  return (b_dim == 128 || b_dim == 64 || b_dim == 32) && a_dim > 1 &&
+  return (b_dim == 128 || b_dim == 64 || b_dim == 32 || b_dim == 16 || b_dim == 8) && a_dim > 1 &&
          block_sylvester64_supported(a_dim, io_dtype, false);
 }
 
@@ -1142,8 +1142,8 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
   if (sylvester_inner)
     CTMI_REQUIRE(ctmi_hadamard_sylvester_inner_supported(a_dim, b_dim, io_dtype) && !(sign_in && sign_out),
                  CTMI_ERR_UNSUPPORTED,
-                 "without mb_t (Mb = Sylvester's matrix): b_dim 64, a_dim up to 224, bfloat16 tensors, "
-                 "signs on one side; got %d x %d", a_dim, b_dim);
+                 "without mb_t (Mb = Sylvester's matrix): b_dim 8 ... 128, a_dim up to 224, bfloat16 or "
+                 "float16 tensors, signs on one side; got %d x %d", a_dim, b_dim);
   else
     CTMI_REQUIRE(ctmi_hadamard_supported(a_dim, b_dim, io_dtype), CTMI_ERR_UNSUPPORTED,
                  "no MFMA kernel for the factorisation %d x %d with this dtype", a_dim, b_dim);

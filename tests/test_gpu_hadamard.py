@@ -372,17 +372,26 @@ def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
     assert rc == _lib.CTMI_ERR_UNSUPPORTED  # 512 lanes only for the Sylvester factor
 
 
-@pytest.mark.parametrize("size", [768, 1600, 3584, 7168, 14336, 32, 256, 512, 16])
+@pytest.mark.parametrize("size", [768, 1600, 3584, 7168, 14336, 3072, 5120, 16384, 32, 256, 512, 16])
 @pytest.mark.parametrize("location,inverse", [("input", False), ("weight_input", True),
                                               ("weight_output", False), ("output", True)])
-def test_random_hadamard_of_any_table_size(size, location, inverse, gpu, hadamard_table_path):
+def test_random_hadamard_of_any_table_size(size, location, inverse, gpu, hadamard_table_path,
+                                           monkeypatch):
     """sizes K * 2^m from the table of known matrices (3584 = 28 * 128, 7168 = 224 * 32,
-    14336 = 224 * 64: Llama-3's intermediate size), 32 (whose table entry is not Sylvester's) and the powers of two
+    14336 = 224 * 64: Llama-3's intermediate size; 3072 = 12 * 256 and 5120 = 20 * 256, where
+    the block grows by Sylvester(2) to meet the kernel's 128), 16384 = Sylvester(128) as the
+    block of 128 * 128, 32 (whose table entry is not Sylvester's) and the powers of two
     that have no matrix-core kernel: forward against the dense fp64 matrix the oracle
     builds with the reference's butterfly stages"""
     from compressed_tensors_amd.transform import (
         TransformArgs, TransformFactory, TransformScheme, load_hadamard_table,
     )
+    from compressed_tensors_amd.transform import hadamard as product
+
+    if size >= 1024:  # these have a matrix-core kernel: the dense matrix must not be what ran
+        def refuse(*a, **k):
+            raise AssertionError(f"size {size} went through the dense matrix")
+        monkeypatch.setattr(product, "apply_transform_weight", refuse)
 
     announce("random hadamard", size, location, inverse)
     scheme = TransformScheme(type="random-hadamard")
@@ -472,26 +481,31 @@ def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_block
                          [(k, torch.bfloat16, 64) for k in (224, 12, 28, 36, 64, 100, 128, 160)] +
                          [(k, torch.float16, 64) for k in (224, 28, 64, 100)] +
                          [(k, torch.bfloat16, 32) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 32)] +
-                         [(k, torch.bfloat16, 128) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 128)],
+                         [(k, torch.bfloat16, 128) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 128)] +
+                         [(k, torch.bfloat16, 16) for k in (224, 192, 28, 64, 100)] + [(224, torch.float16, 16)] +
+                         [(k, torch.bfloat16, 8) for k in (224, 192, 20, 100)] + [(192, torch.float16, 8)],
                          ids=lambda v: str(v).replace("torch.", ""))
 def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, hadamard_blocks):
     """ctmi_hadamard_apply without mb_t (Mb = Sylvester(64)): the product with the block on the
     matrix cores, the Sylvester factor as butterflies on its fp32 result; bfloat16 and float16
-    tensors (the block is given in bfloat16 either way); Sylvester(32) in place of Sylvester(64)
-    (two runs share the kernel's 64 columns; odd numbers of runs, pairs that straddle two
-    tensors of one call) and Sylvester(128) (28672 = 224 * 128: two halves of 64 columns and a
+    tensors (the block is given in bfloat16 either way); Sylvester(32), (16) and (8) in place of
+    Sylvester(64) (two, four or eight runs share the kernel's 64 columns; numbers of runs that
+    leave the last unit part empty, units that straddle the tensors of one call: 3584 = 224 * 16
+    and 3072 = 192 * 16 are how the reference builds those sizes) and Sylvester(128) (28672 = 224 * 128: two halves of 64 columns and a
     stage over the halves).  Blocks of every tile
     count (K <= 32, 64, 128, 224) incl. sizes that leave rows of the last tile empty, a random
     +-1 matrix and (where the table has one) the known Hadamard block; more runs than the
     workgroups hold at a time; signs on either side; several tensors in one call."""
     from compressed_tensors_amd import _lib
 
-    announce("block x Sylvester(32 / 64 / 128), butterflies", k, dtype, inner)
+    announce("block x Sylvester(8 ... 128), butterflies", k, dtype, inner)
     code = _lib.dtype_code(dtype)
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, inner, code) == 1
     n = k * inner
     g = torch.Generator().manual_seed(k)
     rows = 2051 if k <= 64 else 1027
+    if inner < 32:
+        rows = 4 * rows + 1  # short runs: as many elements, and a last unit with one run
     x = torch.randn(rows, n, generator=g).to(dtype)
     s = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float()
     sample = torch.tensor([0, 1, 255, 256, 511, 1023, 1024, rows - 1])
