@@ -658,6 +658,22 @@ def other_workload(torch, name, seed):
         ops.append(Op("random-sign Hadamard, size 14336 = 224 x 64: activations 4096x14336 (x5)", calls,
                       sum(4 * x.numel() for x in xs14), "block_sylvester64_kernel",
                       mfma_flops=sum(2 * 224 * x.numel() for x in xs14)))
+        # 3584 = 224 x 16 (the reference takes the largest block of its table: hidden sizes such
+        # as 3584 and 3072 come out as a large block times a short Sylvester factor): four runs
+        # share the kernel's 64 columns
+        xs35 = [randn(16384, 3584) for _ in range(5)]
+        q35 = (torch.randint(0, 2, (3584,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
+        keep.append(q35)
+        calls = []
+        for x in xs35:
+            out = torch.empty_like(x)
+            keep.extend([x, out])
+            a = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), 224, 16, ma224.data_ptr(),
+                 None, q35.data_ptr(), None, st)
+            calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
+        ops.append(Op("random-sign Hadamard, size 3584 = 224 x 16: activations 16384x3584 (x5)", calls,
+                      sum(4 * x.numel() for x in xs35), "block_sylvester64_kernel",
+                      mfma_flops=sum(2 * 224 * x.numel() for x in xs35)))
         # rotation (block 128) + symmetric int4 group-128 quantization + pack_to_int32, one pass
         mb = deterministic_hadamard_matrix(128, torch.bfloat16, dev).contiguous()
         q = (torch.randint(0, 2, (128,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)

@@ -79,6 +79,21 @@ __device__ __forceinline__ int bs_job(const BsTable& t, int64_t run, int64_t* lo
   return j;
 }
 
+// Where run number `run` (its own in every lane) of n elements begins, in the inputs or (OUT)
+// the outputs: the table's entries picked by comparisons, no indexed read of the table.
+template <bool OUT>
+__device__ __forceinline__ uint16_t* bs_lane_run(const BsTable& t, int64_t run, int64_t n) {
+  int64_t first = 0;
+  const void* base = OUT ? t.out[0] : t.x[0];
+#pragma unroll
+  for (int i = 0; i < kFwhtMaxJobs - 1; ++i) {
+    const bool past = run >= t.end[i];
+    first = past ? t.end[i] : first;
+    base = past ? (OUT ? t.out[i + 1] : t.x[i + 1]) : base;
+  }
+  return static_cast<uint16_t*>(const_cast<void*>(base)) + (run - first) * n;
+}
+
 // fragments of Ma, the sign masks (SIGNS != 0), one image per wavefront
 constexpr size_t bs_lds_bytes(int nt, bool signs) {
   return ((size_t)2 * nt * nt * kWave * 4 + (signs ? (size_t)nt * 4 * kWave * 4 : 0) +
@@ -143,24 +158,22 @@ __device__ __forceinline__ void bs_load_fragments(const uint16_t* __restrict__ m
 
 // NT: column tiles of 32 that cover K (K <= 32 NT); SIGNS: 0 none, 1 sign_in, 2 sign_out;
 // HALF: float16 tensors (the matrix arrives in bfloat16 and converts exactly: entries +-1);
-// PAIR (RUNS != 1): runs of K * 2^log_inner elements, 2^log_inner = 32, 16 or 8 (Ma (x) Sylvester(32),
+// PAIR (RUNS != 1): runs of K * 2^log_inner elements, 2^log_inner = 64 / RUNS = 32, 16 or 8 (Ma (x) Sylvester(32),
 // e.g. 7168 = 224 * 32, 3584 = 224 * 16, 1792 = 224 * 8), two, four or eight at a time: the
 // 64 columns of the image are 32 (16, 8) of one run beside those of the next, and the
 // butterfly stages over the column bits that tell the runs apart are left out (the stage over
 // the M tiles always; 16: the one 16 columns apart as well; 8: and the one 8 apart).  A lane
 // loads and stores the run its piece of a row lies in; where the tensors end inside a unit
 // the missing runs are read as the last one once more and not stored.
-// RUNS: 1 for Sylvester(64), 2 for Sylvester(32), 0 for 16 and 8 (log_inner read at run time:
-// the two share a kernel).
+// RUNS: runs side by side in the image: 1, 2, 4, 8 for Sylvester(64), (32), (16), (8).
 template <int NT, int SIGNS, bool HALF, int RUNS>
 __global__ void __launch_bounds__(kBsThreads, 1)
 block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
-                         const float* __restrict__ signs, float scale, int log_inner) {
+                         const float* __restrict__ signs, float scale) {
   constexpr int KS = 2 * NT;  // steps of 16 over the contracted index
   constexpr bool PAIR = RUNS != 1;
-  if constexpr (RUNS == 1) log_inner = 6;
-  if constexpr (RUNS == 2) log_inner = 5;
-  const int unit_runs = 64 >> log_inner;  // runs side by side in the image
+  constexpr int log_inner = RUNS == 1 ? 6 : RUNS == 2 ? 5 : RUNS == 4 ? 4 : 3;
+  constexpr int unit_runs = RUNS;
   extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
   bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
   bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [NT * 4][64] (SIGNS != 0)
@@ -180,7 +193,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       const int row = 32 * (f >> 2) + (int)(l >> 3) + 8 * (f & 3);
       bs_u32x4 m = {0u, 0u, 0u, 0u};
       if (row < k_dim) {
-        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + ((int64_t)row << log_inner) + piece);
+        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + (row << log_inner) + piece);
 #pragma unroll
         for (int d = 0; d < 4; ++d) m[d] = ((s8.v[2 * d] >> 16) & 0x8000u) | (s8.v[2 * d + 1] & 0x80000000u);
       }
@@ -200,21 +213,19 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   // the spot): a run beyond the last reads the last again, a row beyond K reads row K - 1 and
   // is replaced by zeros when it is used.
   bs_u32x4 in[NT][4];
-  // where the lane's run of unit u begins (a unit: one run, or PAIR: up to eight neighbouring
-  // ones, each looked up with scalar instructions and kept by the lanes it belongs to);
+  // where the lane's run of unit u begins (a unit: one run, two neighbouring ones looked up
+  // with scalar instructions, or four / eight looked up by every lane for itself);
   // table reads once per unit, not per chunk
   auto run_start = [&](int64_t u) {
-    if constexpr (PAIR) {
-      const uint16_t* mine = nullptr;
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (i < unit_runs) {
-          int64_t local;
-          const int j = bs_job(tab, min(unit_runs * u + i, tab.total - 1), &local);
-          const uint16_t* p = static_cast<const uint16_t*>(tab.x[j]) + local * n;
-          mine = my_run == (uint32_t)i ? p : mine;
-        }
-      return mine;
+    if constexpr (RUNS > 2) {
+      return (const uint16_t*)bs_lane_run<false>(tab, min(unit_runs * u + (int64_t)my_run, tab.total - 1), n);
+    } else if constexpr (PAIR) {
+      int64_t la, lb;
+      const int64_t ra = min(2 * u, tab.total - 1), rb = min(2 * u + 1, tab.total - 1);
+      const int ja = bs_job(tab, ra, &la), jb = bs_job(tab, rb, &lb);
+      const uint16_t* a = static_cast<const uint16_t*>(tab.x[ja]) + la * n;
+      const uint16_t* b = static_cast<const uint16_t*>(tab.x[jb]) + lb * n;
+      return my_run ? b : a;
     } else {
       const int64_t r = u < tab.total ? u : tab.total - 1;
       int64_t local;
@@ -227,10 +238,10 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
     for (int q = 0; q < 4; ++q) {
       const int row = 32 * ch + (int)(l >> 3) + 8 * q;
       in[ch][q] = __builtin_bit_cast(
-          bs_u32x4, ldg_nt<uint16_t, 8>(xr + ((int64_t)(row < k_dim ? row : k_dim - 1) << log_inner) + piece));
+          bs_u32x4, ldg_nt<uint16_t, 8>(xr + ((row < k_dim ? row : k_dim - 1) << log_inner) + piece));
     }
   };
-  const int64_t units = (tab.total + unit_runs - 1) >> (6 - log_inner);
+  const int64_t units = PAIR ? (tab.total + unit_runs - 1) / unit_runs : tab.total;
 
   auto pack2 = [](float lo, float hi) -> uint32_t {
     if constexpr (HALF) return (uint32_t)f32_to_f16(lo) | ((uint32_t)f32_to_f16(hi) << 16);
@@ -311,17 +322,18 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
     // butterflies over j = 32 mt + 8 b + 4 g + r
     uint16_t* __restrict__ yr;
     bool stored = true;  // PAIR: a run past the last tensor is not
-    if constexpr (PAIR) {
-      yr = nullptr;
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
-        if (i < unit_runs) {
-          int64_t local;
-          const int j = bs_job(tab, min(unit_runs * run + i, tab.total - 1), &local);
-          uint16_t* p = static_cast<uint16_t*>(tab.out[j]) + local * n;
-          yr = my_run == (uint32_t)i ? p : yr;
-        }
-      stored = unit_runs * run + (int64_t)my_run < tab.total;
+    if constexpr (RUNS > 2) {
+      const int64_t mine = unit_runs * run + (int64_t)my_run;
+      yr = bs_lane_run<true>(tab, min(mine, tab.total - 1), n);
+      stored = mine < tab.total;
+    } else if constexpr (PAIR) {
+      int64_t la, lb;
+      const int64_t rb = 2 * run + 1 < tab.total ? 2 * run + 1 : 2 * run;
+      const int ja = bs_job(tab, 2 * run, &la), jb = bs_job(tab, rb, &lb);
+      uint16_t* a = static_cast<uint16_t*>(tab.out[ja]) + la * n;
+      uint16_t* b = static_cast<uint16_t*>(tab.out[jb]) + lb * n;
+      yr = my_run ? b : a;
+      stored = !my_run || 2 * run + 1 < tab.total;
     } else {
       int64_t local;
       const int j = bs_job(tab, run, &local);
@@ -376,7 +388,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
         if constexpr (SIGNS == 2) w ^= fo[q];
         if (row < k_dim && stored)
-          stg_nt<uint16_t, 8>(yr + ((int64_t)row << log_inner) + piece, __builtin_bit_cast(Vec<uint16_t, 8>, w));
+          stg_nt<uint16_t, 8>(yr + (row << log_inner) + piece, __builtin_bit_cast(Vec<uint16_t, 8>, w));
       }
     }
   }
@@ -586,7 +598,7 @@ int launch_bs128(const BsTable& tab, int io_dtype, const uint16_t* ma_t, int k, 
 
 template <int NT, int SIGNS, bool HALF, int RUNS>
 int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
-                      int log_inner, hipStream_t st) {
+                      hipStream_t st) {
   auto kern = block_sylvester64_kernel<NT, SIGNS, HALF, RUNS>;
   constexpr size_t lds = bs_lds_bytes(NT, SIGNS != 0);
   if (lds > 48 * 1024) {
@@ -607,36 +619,34 @@ int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const flo
     per_cu = n > 0 ? n : 1;
   }
   if (e != hipSuccess) return set_error(CTMI_ERR_HIP, "device query: %s", hipGetErrorString(e));
-  const int64_t wgs = cdiv(cdiv(tab.total, (int64_t)(64 >> log_inner)), kBsWaves);
+  const int64_t wgs = cdiv(cdiv(tab.total, (int64_t)RUNS), kBsWaves);
   const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * per_cu;
   const int64_t each = cdiv(wgs, cap);  // runs per wavefront, the same for all
   const unsigned grid = (unsigned)cdiv(wgs, each);
-  hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale, log_inner);
+  hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale);
   return CTMI_OK;
 }
 
 template <int NT, bool HALF, int RUNS>
 int launch_bs_dtype(const BsTable& tab, const uint16_t* ma_t, int k, const float* sign_in,
-                    const float* sign_out, float scale, int log_inner, hipStream_t st) {
-  if (sign_in) return launch_bs_variant<NT, 1, HALF, RUNS>(tab, ma_t, k, sign_in, scale, log_inner, st);
-  if (sign_out) return launch_bs_variant<NT, 2, HALF, RUNS>(tab, ma_t, k, sign_out, scale, log_inner, st);
-  return launch_bs_variant<NT, 0, HALF, RUNS>(tab, ma_t, k, nullptr, scale, log_inner, st);
+                    const float* sign_out, float scale, hipStream_t st) {
+  if (sign_in) return launch_bs_variant<NT, 1, HALF, RUNS>(tab, ma_t, k, sign_in, scale, st);
+  if (sign_out) return launch_bs_variant<NT, 2, HALF, RUNS>(tab, ma_t, k, sign_out, scale, st);
+  return launch_bs_variant<NT, 0, HALF, RUNS>(tab, ma_t, k, nullptr, scale, st);
 }
 
 template <int NT>
 int launch_bs(const BsTable& tab, int io_dtype, int inner, const uint16_t* ma_t, int k,
               const float* sign_in, const float* sign_out, float scale, hipStream_t st) {
   const bool half = io_dtype == CTMI_F16;
-  if (inner < 32) {
-    const int log_inner = inner == 16 ? 4 : 3;
-    return half ? launch_bs_dtype<NT, true, 0>(tab, ma_t, k, sign_in, sign_out, scale, log_inner, st)
-                : launch_bs_dtype<NT, false, 0>(tab, ma_t, k, sign_in, sign_out, scale, log_inner, st);
-  }
-  if (inner == 32)
-    return half ? launch_bs_dtype<NT, true, 2>(tab, ma_t, k, sign_in, sign_out, scale, 5, st)
-                : launch_bs_dtype<NT, false, 2>(tab, ma_t, k, sign_in, sign_out, scale, 5, st);
-  return half ? launch_bs_dtype<NT, true, 1>(tab, ma_t, k, sign_in, sign_out, scale, 6, st)
-              : launch_bs_dtype<NT, false, 1>(tab, ma_t, k, sign_in, sign_out, scale, 6, st);
+#define CTMI_BS_RUNS(R)                                                                       \
+  (half ? launch_bs_dtype<NT, true, R>(tab, ma_t, k, sign_in, sign_out, scale, st)            \
+        : launch_bs_dtype<NT, false, R>(tab, ma_t, k, sign_in, sign_out, scale, st))
+  if (inner == 8) return CTMI_BS_RUNS(8);
+  if (inner == 16) return CTMI_BS_RUNS(4);
+  if (inner == 32) return CTMI_BS_RUNS(2);
+  return CTMI_BS_RUNS(1);
+#undef CTMI_BS_RUNS
 }
 
 }  // namespace
