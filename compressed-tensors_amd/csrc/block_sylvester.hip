@@ -95,8 +95,8 @@ __device__ __forceinline__ uint16_t* bs_lane_run(const BsTable& t, int64_t run, 
 }
 
 // fragments of Ma, the sign masks (SIGNS != 0), one image per wavefront
-constexpr size_t bs_lds_bytes(int nt, bool signs) {
-  return ((size_t)2 * nt * nt * kWave * 4 + (signs ? (size_t)nt * 4 * kWave * 4 : 0) +
+constexpr size_t bs_lds_bytes(int nt, int ch, int signs) {
+  return ((size_t)2 * ch * nt * kWave * 4 + (signs ? (size_t)(signs == 1 ? ch : nt) * 4 * kWave * 4 : 0) +
           (size_t)kBsWaves * kBsRing) * sizeof(uint32_t);
 }
 
@@ -112,13 +112,15 @@ __device__ __forceinline__ bs_f32x16_t bs_mma(const bs_u32x4& a, const bs_u32x4&
 }
 
 // The fragments of Ma into LDS, zero beyond K: fragment (ks, nt), lane (c, g) holds
-// Ma[16 ks + 8 g + e][32 nt + c], e = 0..7.  Eight at a time per wavefront, loads first: one
+// Ma[16 ks + 8 g + e][first_col + 32 nt + c], e = 0..7 (CH chunks of 32 rows of Ma, NT tiles of
+// 32 of its columns from first_col on).  Eight at a time per wavefront, loads first: one
 // after the other they would cost the launch as many memory round trips as there are
 // fragments.
-template <int NT, bool HALF>
+template <int NT, bool HALF, int CH = NT>
 __device__ __forceinline__ void bs_load_fragments(const uint16_t* __restrict__ ma_t, int k_dim,
-                                                  bs_u32x4* ma_frag, uint32_t wave, uint32_t l) {
-  constexpr int KS = 2 * NT;
+                                                  bs_u32x4* ma_frag, uint32_t wave, uint32_t l,
+                                                  int first_col = 0) {
+  constexpr int KS = 2 * CH;
   const uint32_t c = l & 31u, g = l >> 5;
   const bool ma_vectors = k_dim % 8 == 0 && (uintptr_t)ma_t % 16 == 0;  // 16-byte pieces of whole rows
   for (int f0 = 0; f0 < KS * NT; f0 += kBsWaves * 8) {
@@ -127,7 +129,7 @@ __device__ __forceinline__ void bs_load_fragments(const uint16_t* __restrict__ m
     for (int u = 0; u < 8; ++u) {
       const int f = f0 + u * kBsWaves + (int)wave;
       const int ks = f / NT, nt = f % NT;
-      const int col = 32 * nt + (int)c, i0 = 16 * ks + 8 * (int)g;  // Ma[i0 + e][col] = ma_t[col][i0 + e]
+      const int col = first_col + 32 * nt + (int)c, i0 = 16 * ks + 8 * (int)g;  // Ma[i0 + e][col] = ma_t[col][i0 + e]
       w[u] = bs_u32x4{0u, 0u, 0u, 0u};
       if (f < KS * NT && col < k_dim) {
         if (ma_vectors) {
@@ -166,31 +168,37 @@ __device__ __forceinline__ void bs_load_fragments(const uint16_t* __restrict__ m
 // loads and stores the run its piece of a row lies in; where the tensors end inside a unit
 // the missing runs are read as the last one once more and not stored.
 // RUNS: runs side by side in the image: 1, 2, 4, 8 for Sylvester(64), (32), (16), (8).
-template <int NT, int SIGNS, bool HALF, int RUNS>
+// CH: chunks of 32 rows of X (= of Ma) a run has; NT tiles of 32 output rows from row out_first
+// on are computed.  CH = NT and out_first = 0 for K <= 224; for K up to 256 the accumulators of
+// all eight tiles do not fit beside a run held ahead, and two launches compute four tiles each
+// (CH = 8, NT = 4, out_first = 0 and 128: the run is read twice).
+template <int NT, int SIGNS, bool HALF, int RUNS, int CH = NT>
 __global__ void __launch_bounds__(kBsThreads, 1)
 block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_dim,
-                         const float* __restrict__ signs, float scale) {
-  constexpr int KS = 2 * NT;  // steps of 16 over the contracted index
+                         const float* __restrict__ signs, float scale, int out_first) {
+  constexpr int KS = 2 * CH;  // steps of 16 over the contracted index
+  if constexpr (CH == NT) out_first = 0;
   constexpr bool PAIR = RUNS != 1;
   constexpr int log_inner = RUNS == 1 ? 6 : RUNS == 2 ? 5 : RUNS == 4 ? 4 : 3;
   constexpr int unit_runs = RUNS;
   extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
   bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
-  bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [NT * 4][64] (SIGNS != 0)
+  bs_u32x4* flip = ma_frag + KS * NT * kWave;                                 // [CH or NT][4][64] (SIGNS 1 or 2)
+  constexpr int SIGN_TILES = SIGNS == 1 ? CH : NT;
   const uint32_t l = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const uint32_t c = l & 31u, g = l >> 5;
-  uint32_t* image = bs_lds + (KS * NT + (SIGNS ? NT * 4 : 0)) * kWave * 4 + wave * kBsRing;
+  uint32_t* image = bs_lds + (KS * NT + (SIGNS ? SIGN_TILES * 4 : 0)) * kWave * 4 + wave * kBsRing;
   const int64_t n = (int64_t)k_dim << log_inner;
   const uint32_t piece = 8 * (l & ((1u << (log_inner - 3)) - 1u));  // the lane's 8 columns inside a row of a run
   const uint32_t my_run = PAIR ? (l & 7u) >> (log_inner - 3) : 0u;  // ... and that run's place in the unit
 
-  bs_load_fragments<NT, HALF>(ma_t, k_dim, ma_frag, wave, l);
+  bs_load_fragments<NT, HALF, CH>(ma_t, k_dim, ma_frag, wave, l, out_first);
   // Sign masks of the vectors a lane loads (SIGNS == 1: vector q of chunk ch is row
   // 32 ch + l / 8 + 8 q, columns 8 (l % 8) ...) or stores (SIGNS == 2: the same positions with
   // the tile nt in place of the chunk): the same for the four wavefronts, read at each use
   if constexpr (SIGNS != 0) {
-    for (int f = (int)wave; f < NT * 4; f += kBsWaves) {
-      const int row = 32 * (f >> 2) + (int)(l >> 3) + 8 * (f & 3);
+    for (int f = (int)wave; f < SIGN_TILES * 4; f += kBsWaves) {
+      const int row = (SIGNS == 2 ? out_first : 0) + 32 * (f >> 2) + (int)(l >> 3) + 8 * (f & 3);
       bs_u32x4 m = {0u, 0u, 0u, 0u};
       if (row < k_dim) {
         const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + (row << log_inner) + piece);
@@ -212,7 +220,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   // No branch around the loads (a load under a condition makes the compiler wait for it on
   // the spot): a run beyond the last reads the last again, a row beyond K reads row K - 1 and
   // is replaced by zeros when it is used.
-  bs_u32x4 in[NT][4];
+  bs_u32x4 in[CH][4];
   // where the lane's run of unit u begins (a unit: one run, two neighbouring ones looked up
   // with scalar instructions, or four / eight looked up by every lane for itself);
   // table reads once per unit, not per chunk
@@ -252,7 +260,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   {
     const uint16_t* first = run_start(run);
 #pragma unroll
-    for (int ch = 0; ch < NT; ++ch) fetch(first, ch);
+    for (int ch = 0; ch < CH; ++ch) fetch(first, ch);
   }
   for (; run < units; run += step) {
     const uint16_t* next = run_start(run + step);
@@ -264,7 +272,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[mt][nt][i] = 0.0f;
 #pragma unroll
-    for (int ch = 0; ch < NT; ++ch) {
+    for (int ch = 0; ch < CH; ++ch) {
       // (LDS reads grouped ahead of the LDS writes they do not depend on: the compiler keeps
       // accesses of the one shared array in program order, and every read that sits behind
       // a write costs the wavefront a round trip of its own)
@@ -384,7 +392,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       }
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int row = 32 * nt + (int)(l >> 3) + 8 * q;
+        const int row = out_first + 32 * nt + (int)(l >> 3) + 8 * q;
         bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
         if constexpr (SIGNS == 2) w ^= fo[q];
         if (row < k_dim && stored)
@@ -596,11 +604,11 @@ int launch_bs128(const BsTable& tab, int io_dtype, const uint16_t* ma_t, int k, 
 #undef CTMI_BS128
 }
 
-template <int NT, int SIGNS, bool HALF, int RUNS>
+template <int NT, int SIGNS, bool HALF, int RUNS, int CH = NT>
 int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const float* signs, float scale,
                       hipStream_t st) {
-  auto kern = block_sylvester64_kernel<NT, SIGNS, HALF, RUNS>;
-  constexpr size_t lds = bs_lds_bytes(NT, SIGNS != 0);
+  auto kern = block_sylvester64_kernel<NT, SIGNS, HALF, RUNS, CH>;
+  constexpr size_t lds = bs_lds_bytes(NT, CH, SIGNS);
   if (lds > 48 * 1024) {
     // the attribute belongs to the kernel as loaded on one device; setting it again is cheap
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -623,25 +631,27 @@ int launch_bs_variant(const BsTable& tab, const uint16_t* ma_t, int k, const flo
   const int64_t cap = (int64_t)(cus > 0 ? cus : 256) * per_cu;
   const int64_t each = cdiv(wgs, cap);  // runs per wavefront, the same for all
   const unsigned grid = (unsigned)cdiv(wgs, each);
-  hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale);
+  // CH > NT: the output tiles in turn, NT at a time
+  for (int first = 0; first < 32 * CH && first < k; first += 32 * NT)
+    hipLaunchKernelGGL(kern, grid, kBsThreads, lds, st, tab, ma_t, k, signs, scale, first);
   return CTMI_OK;
 }
 
-template <int NT, bool HALF, int RUNS>
+template <int NT, bool HALF, int RUNS, int CH = NT>
 int launch_bs_dtype(const BsTable& tab, const uint16_t* ma_t, int k, const float* sign_in,
                     const float* sign_out, float scale, hipStream_t st) {
-  if (sign_in) return launch_bs_variant<NT, 1, HALF, RUNS>(tab, ma_t, k, sign_in, scale, st);
-  if (sign_out) return launch_bs_variant<NT, 2, HALF, RUNS>(tab, ma_t, k, sign_out, scale, st);
-  return launch_bs_variant<NT, 0, HALF, RUNS>(tab, ma_t, k, nullptr, scale, st);
+  if (sign_in) return launch_bs_variant<NT, 1, HALF, RUNS, CH>(tab, ma_t, k, sign_in, scale, st);
+  if (sign_out) return launch_bs_variant<NT, 2, HALF, RUNS, CH>(tab, ma_t, k, sign_out, scale, st);
+  return launch_bs_variant<NT, 0, HALF, RUNS, CH>(tab, ma_t, k, nullptr, scale, st);
 }
 
-template <int NT>
+template <int NT, int CH = NT>
 int launch_bs(const BsTable& tab, int io_dtype, int inner, const uint16_t* ma_t, int k,
               const float* sign_in, const float* sign_out, float scale, hipStream_t st) {
   const bool half = io_dtype == CTMI_F16;
 #define CTMI_BS_RUNS(R)                                                                       \
-  (half ? launch_bs_dtype<NT, true, R>(tab, ma_t, k, sign_in, sign_out, scale, st)            \
-        : launch_bs_dtype<NT, false, R>(tab, ma_t, k, sign_in, sign_out, scale, st))
+  (half ? launch_bs_dtype<NT, true, R, CH>(tab, ma_t, k, sign_in, sign_out, scale, st)        \
+        : launch_bs_dtype<NT, false, R, CH>(tab, ma_t, k, sign_in, sign_out, scale, st))
   if (inner == 8) return CTMI_BS_RUNS(8);
   if (inner == 16) return CTMI_BS_RUNS(4);
   if (inner == 32) return CTMI_BS_RUNS(2);
@@ -651,17 +661,17 @@ int launch_bs(const BsTable& tab, int io_dtype, int inner, const uint16_t* ma_t,
 
 }  // namespace
 
-bool block_sylvester64_supported(int k, int io_dtype, bool both_signs) {
-  return (io_dtype == CTMI_BF16 || io_dtype == CTMI_F16) && k >= 1 && k <= 224 && !both_signs;
+bool block_sylvester64_supported(int k, int inner, int io_dtype, bool both_signs) {
+  const bool size = inner == 128 ? k <= 224 : (inner == 64 || inner == 32 || inner == 16 || inner == 8) && k <= 256;
+  return (io_dtype == CTMI_BF16 || io_dtype == CTMI_F16) && k >= 1 && size && !both_signs;
 }
 
 int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int k, int inner,
                              const uint16_t* ma_t, const float* sign_in, const float* sign_out,
                              float scale, hipStream_t st) {
-  CTMI_REQUIRE(inner == 128 || inner == 64 || inner == 32 || inner == 16 || inner == 8, CTMI_ERR_UNSUPPORTED,
-               "Sylvester factor of 8, 16, 32, 64 or 128");
-  CTMI_REQUIRE(block_sylvester64_supported(k, io_dtype, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
-               "bfloat16 or float16 tensors, blocks of up to 224 x 224 with signs on one side");
+  CTMI_REQUIRE(block_sylvester64_supported(k, inner, io_dtype, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
+               "bfloat16 or float16 tensors, a Sylvester factor of 8 ... 64 with blocks of up to 256 x 256 or of "
+               "128 with blocks of up to 224 x 224, signs on one side");
   CTMI_REQUIRE(n_jobs >= 1 && n_jobs <= kFwhtMaxJobs, CTMI_ERR_VALUE, "1 to %d tensors a launch", kFwhtMaxJobs);
   CTMI_REQUIRE(ma_t && (uintptr_t)sign_in % 16 == 0 && (uintptr_t)sign_out % 16 == 0, CTMI_ERR_VALUE,
                "the block must be given; sign vectors must be 16-byte aligned");
@@ -676,6 +686,9 @@ int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int 
                    "tensor %d: NULL pointer or no runs", i);
       CTMI_REQUIRE((uintptr_t)jobs[i].x % 16 == 0 && (uintptr_t)jobs[i].out % 16 == 0, CTMI_ERR_VALUE,
                    "tensors must be 16-byte aligned");
+      // blocks above 224 take two launches, and the second reads the runs again
+      CTMI_REQUIRE(k <= 224 || jobs[i].x != jobs[i].out, CTMI_ERR_VALUE,
+                   "blocks of more than 224 rows are not transformed in place");
       total += jobs[i].rows;
     }
     tab.end[i] = live ? total : INT64_MAX;
@@ -690,7 +703,8 @@ int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int 
   if (k <= 32) return launch_bs<1>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
   if (k <= 64) return launch_bs<2>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
   if (k <= 128) return launch_bs<4>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
-  return launch_bs<7>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 224) return launch_bs<7>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
+  return launch_bs<4, 8>(tab, io_dtype, inner, ma_t, k, sign_in, sign_out, scale, st);
 }
 
 }  // namespace ctmi

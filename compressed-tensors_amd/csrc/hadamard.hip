@@ -1072,8 +1072,7 @@ extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_
 }
 
 extern "C" int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
-  return (b_dim == 128 || b_dim == 64 || b_dim == 32 || b_dim == 16 || b_dim == 8) && a_dim > 1 &&
-         block_sylvester64_supported(a_dim, io_dtype, false);
+  return a_dim > 1 && block_sylvester64_supported(a_dim, b_dim, io_dtype, false);
 }
 
 extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel,
@@ -1142,8 +1141,9 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
   if (sylvester_inner)
     CTMI_REQUIRE(ctmi_hadamard_sylvester_inner_supported(a_dim, b_dim, io_dtype) && !(sign_in && sign_out),
                  CTMI_ERR_UNSUPPORTED,
-                 "without mb_t (Mb = Sylvester's matrix): b_dim 8 ... 128, a_dim up to 224, bfloat16 or "
-                 "float16 tensors, signs on one side; got %d x %d", a_dim, b_dim);
+                 "without mb_t (Mb = Sylvester's matrix): b_dim 8 ... 64 with a_dim up to 256 or b_dim 128 "
+                 "with a_dim up to 224, bfloat16 or float16 tensors, signs on one side; got %d x %d",
+                 a_dim, b_dim);
   else
     CTMI_REQUIRE(ctmi_hadamard_supported(a_dim, b_dim, io_dtype), CTMI_ERR_UNSUPPORTED,
                  "no MFMA kernel for the factorisation %d x %d with this dtype", a_dim, b_dim);
@@ -1158,6 +1158,9 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
                  (long long)i);
     CTMI_REQUIRE((uintptr_t)j.x % 16 == 0 && (uintptr_t)j.out % 16 == 0, CTMI_ERR_VALUE,
                  "tensors must be 16-byte aligned");
+    // a block above 224 rows takes two launches, and the second reads the runs again
+    CTMI_REQUIRE(!(sylvester_inner && a_dim > 224) || j.numel == 0 || j.x != j.out, CTMI_ERR_VALUE,
+                 "job %lld: blocks of more than 224 rows are not transformed in place", (long long)i);
   }
   CTMI_REQUIRE(n_jobs == 0 || ((mb_t || sylvester_inner) && (a_dim == 1 || ma_t)), CTMI_ERR_VALUE,
                "NULL matrix pointer");

@@ -372,15 +372,14 @@ def test_kron_matmul_refuses_what_does_not_fit(ctmi, gpu):
     assert rc == _lib.CTMI_ERR_UNSUPPORTED  # 512 lanes only for the Sylvester factor
 
 
-@pytest.mark.parametrize("size", [768, 1600, 3584, 7168, 14336, 3072, 5120, 16384, 32, 256, 512, 16])
+@pytest.mark.parametrize("size", [768, 1600, 3584, 7168, 14336, 3072, 5120, 3840, 15360, 16384, 32, 256, 512, 16])
 @pytest.mark.parametrize("location,inverse", [("input", False), ("weight_input", True),
                                               ("weight_output", False), ("output", True)])
 def test_random_hadamard_of_any_table_size(size, location, inverse, gpu, hadamard_table_path,
                                            monkeypatch):
     """sizes K * 2^m from the table of known matrices (3584 = 28 * 128, 7168 = 224 * 32,
-    14336 = 224 * 64: Llama-3's intermediate size; 3072 = 12 * 256 and 5120 = 20 * 256, where
-    the block grows by Sylvester(2) to meet the kernel's 128), 16384 = Sylvester(128) as the
-    block of 128 * 128, 32 (whose table entry is not Sylvester's) and the powers of two
+    14336 = 224 * 64: Llama-3's intermediate size; 3072 = 192 * 16, 5120 = 160 * 32, 3840 = 240 * 16
+    and 15360 = 240 * 64 with this table), 16384 = Sylvester(128) as the block of 128 * 128, 32 (whose table entry is not Sylvester's) and the powers of two
     that have no matrix-core kernel: forward against the dense fp64 matrix the oracle
     builds with the reference's butterfly stages"""
     from compressed_tensors_amd.transform import (
@@ -483,7 +482,9 @@ def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_block
                          [(k, torch.bfloat16, 32) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 32)] +
                          [(k, torch.bfloat16, 128) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 128)] +
                          [(k, torch.bfloat16, 16) for k in (224, 192, 28, 64, 100)] + [(224, torch.float16, 16)] +
-                         [(k, torch.bfloat16, 8) for k in (224, 192, 20, 100)] + [(192, torch.float16, 8)],
+                         [(k, torch.bfloat16, 8) for k in (224, 192, 20, 100)] + [(192, torch.float16, 8)] +
+                         [(256, torch.bfloat16, 64), (240, torch.bfloat16, 64), (228, torch.bfloat16, 32),
+                          (240, torch.bfloat16, 16), (252, torch.bfloat16, 8), (240, torch.float16, 64)],
                          ids=lambda v: str(v).replace("torch.", ""))
 def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, hadamard_blocks):
     """ctmi_hadamard_apply without mb_t (Mb = Sylvester(64)): the product with the block on the
@@ -492,7 +493,8 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, ha
     Sylvester(64) (two, four or eight runs share the kernel's 64 columns; numbers of runs that
     leave the last unit part empty, units that straddle the tensors of one call: 3584 = 224 * 16
     and 3072 = 192 * 16 are how the reference builds those sizes) and Sylvester(128) (28672 = 224 * 128: two halves of 64 columns and a
-    stage over the halves).  Blocks of every tile
+    stage over the halves).  Blocks of 228 ... 256 rows (15360 = 240 * 64, 3840 = 240 * 16) take two
+    launches of four output tiles each and are refused in place.  Blocks of every tile
     count (K <= 32, 64, 128, 224) incl. sizes that leave rows of the last tile empty, a random
     +-1 matrix and (where the table has one) the known Hadamard block; more runs than the
     workgroups hold at a time; signs on either side; several tensors in one call."""
@@ -545,7 +547,12 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, ha
         assert_bit_equal(o, one, f"tensor of {t.shape[0]} runs")
     # what it does not take
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 256, code) == 0
-    assert ctmi.ctmi_hadamard_sylvester_inner_supported(225, 64, code) == 0
+    assert ctmi.ctmi_hadamard_sylvester_inner_supported(257, 64, code) == 0
+    assert ctmi.ctmi_hadamard_sylvester_inner_supported(225, 128, code) == 0
+    if k > 224:
+        rc = ctmi.ctmi_hadamard_apply(xg.data_ptr(), xg.data_ptr(), code, xg.numel(), k, inner, ma_t.data_ptr(), None,
+                                      sg.data_ptr(), None, _lib.stream_of(gpu))
+        assert rc == _lib.CTMI_ERR_VALUE  # the second launch would read what the first wrote
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, 64, _lib.dtype_code(torch.float32)) == 0
     rc = ctmi.ctmi_hadamard_apply(xg.data_ptr(), xg.data_ptr(), code, xg.numel(), k, inner, ma_t.data_ptr(), None,
                                   sg.data_ptr(), sg.data_ptr(), _lib.stream_of(gpu))
