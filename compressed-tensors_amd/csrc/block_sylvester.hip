@@ -167,7 +167,9 @@ __device__ __forceinline__ void bs_load_fragments(const uint16_t* __restrict__ m
 // the M tiles always; 16: the one 16 columns apart as well; 8: and the one 8 apart).  A lane
 // loads and stores the run its piece of a row lies in; where the tensors end inside a unit
 // the missing runs are read as the last one once more and not stored.
-// RUNS: runs side by side in the image: 1, 2, 4, 8 for Sylvester(64), (32), (16), (8).
+// RUNS: runs side by side in the image: 1, 2, 4, 8, 16 for Sylvester(64), (32), (16), (8), (4).
+// With 16 (768 = 192 * 4, 896 = 224 * 4) a lane's 8 columns are the rows of two runs: two
+// 8-byte loads and stores, and the stage between the lane halves only exchanges.
 // CH: chunks of 32 rows of X (= of Ma) a run has; NT tiles of 32 output rows from row out_first
 // on are computed.  CH = NT and out_first = 0 for K <= 224; for K up to 256 the accumulators of
 // all eight tiles do not fit beside a run held ahead, and two launches compute four tiles each
@@ -179,7 +181,8 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   constexpr int KS = 2 * CH;  // steps of 16 over the contracted index
   if constexpr (CH == NT) out_first = 0;
   constexpr bool PAIR = RUNS != 1;
-  constexpr int log_inner = RUNS == 1 ? 6 : RUNS == 2 ? 5 : RUNS == 4 ? 4 : 3;
+  constexpr int log_inner = RUNS == 1 ? 6 : RUNS == 2 ? 5 : RUNS == 4 ? 4 : RUNS == 8 ? 3 : 2;
+  constexpr bool TWO = RUNS == 16;  // a lane's 8 columns are the rows of two runs of 4 columns
   constexpr int unit_runs = RUNS;
   extern __shared__ __attribute__((aligned(16))) uint32_t bs_lds[];
   bs_u32x4* ma_frag = reinterpret_cast<bs_u32x4*>(bs_lds);                    // [KS * NT][64]
@@ -189,8 +192,10 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   const uint32_t c = l & 31u, g = l >> 5;
   uint32_t* image = bs_lds + (KS * NT + (SIGNS ? SIGN_TILES * 4 : 0)) * kWave * 4 + wave * kBsRing;
   const int64_t n = (int64_t)k_dim << log_inner;
-  const uint32_t piece = 8 * (l & ((1u << (log_inner - 3)) - 1u));  // the lane's 8 columns inside a row of a run
-  const uint32_t my_run = PAIR ? (l & 7u) >> (log_inner - 3) : 0u;  // ... and that run's place in the unit
+  // the lane's 8 columns inside a row of a run, and that run's place in the unit (TWO: the
+  // first of its two runs)
+  const uint32_t piece = TWO ? 0u : 8 * (l & ((1u << (TWO ? 0 : log_inner - 3)) - 1u));
+  const uint32_t my_run = TWO ? 2 * (l & 7u) : PAIR ? (l & 7u) >> (TWO ? 0 : log_inner - 3) : 0u;
 
   bs_load_fragments<NT, HALF, CH>(ma_t, k_dim, ma_frag, wave, l, out_first);
   // Sign masks of the vectors a lane loads (SIGNS == 1: vector q of chunk ch is row
@@ -201,9 +206,16 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       const int row = (SIGNS == 2 ? out_first : 0) + 32 * (f >> 2) + (int)(l >> 3) + 8 * (f & 3);
       bs_u32x4 m = {0u, 0u, 0u, 0u};
       if (row < k_dim) {
-        const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + (row << log_inner) + piece);
+        if constexpr (TWO) {  // both runs: the row's four signs
+          const Vec<uint32_t, 4> s4 = ldg<uint32_t, 4>(reinterpret_cast<const uint32_t*>(signs) + 4 * row);
 #pragma unroll
-        for (int d = 0; d < 4; ++d) m[d] = ((s8.v[2 * d] >> 16) & 0x8000u) | (s8.v[2 * d + 1] & 0x80000000u);
+          for (int d = 0; d < 2; ++d)
+            m[d] = m[d + 2] = ((s4.v[2 * d] >> 16) & 0x8000u) | (s4.v[2 * d + 1] & 0x80000000u);
+        } else {
+          const Vec<uint32_t, 8> s8 = ldg<uint32_t, 8>(reinterpret_cast<const uint32_t*>(signs) + (row << log_inner) + piece);
+#pragma unroll
+          for (int d = 0; d < 4; ++d) m[d] = ((s8.v[2 * d] >> 16) & 0x8000u) | (s8.v[2 * d + 1] & 0x80000000u);
+        }
       }
       flip[f * kWave + l] = m;
     }
@@ -224,9 +236,10 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   // where the lane's run of unit u begins (a unit: one run, two neighbouring ones looked up
   // with scalar instructions, or four / eight looked up by every lane for itself);
   // table reads once per unit, not per chunk
-  auto run_start = [&](int64_t u) {
+  auto run_start = [&](int64_t u, int second = 0) {
     if constexpr (RUNS > 2) {
-      return (const uint16_t*)bs_lane_run<false>(tab, min(unit_runs * u + (int64_t)my_run, tab.total - 1), n);
+      return (const uint16_t*)bs_lane_run<false>(
+          tab, min(unit_runs * u + (int64_t)my_run + second, tab.total - 1), n);
     } else if constexpr (PAIR) {
       int64_t la, lb;
       const int64_t ra = min(2 * u, tab.total - 1), rb = min(2 * u + 1, tab.total - 1);
@@ -241,12 +254,18 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
       return static_cast<const uint16_t*>(tab.x[j]) + local * n;
     }
   };
-  auto fetch = [&](const uint16_t* __restrict__ xr, int ch) {
+  auto fetch = [&](const uint16_t* __restrict__ xr, const uint16_t* __restrict__ xr2, int ch) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int row = 32 * ch + (int)(l >> 3) + 8 * q;
-      in[ch][q] = __builtin_bit_cast(
-          bs_u32x4, ldg_nt<uint16_t, 8>(xr + ((row < k_dim ? row : k_dim - 1) << log_inner) + piece));
+      const int at = ((row < k_dim ? row : k_dim - 1) << log_inner) + piece;
+      if constexpr (TWO) {
+        const Vec<uint32_t, 2> a = __builtin_bit_cast(Vec<uint32_t, 2>, ldg_nt<uint16_t, 4>(xr + at));
+        const Vec<uint32_t, 2> b = __builtin_bit_cast(Vec<uint32_t, 2>, ldg_nt<uint16_t, 4>(xr2 + at));
+        in[ch][q] = bs_u32x4{a.v[0], a.v[1], b.v[0], b.v[1]};
+      } else {
+        in[ch][q] = __builtin_bit_cast(bs_u32x4, ldg_nt<uint16_t, 8>(xr + at));
+      }
     }
   };
   const int64_t units = PAIR ? (tab.total + unit_runs - 1) / unit_runs : tab.total;
@@ -259,11 +278,13 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
   int64_t run = (int64_t)blockIdx.x * kBsWaves + wave;
   {
     const uint16_t* first = run_start(run);
+    const uint16_t* first2 = TWO ? run_start(run, 1) : first;
 #pragma unroll
-    for (int ch = 0; ch < CH; ++ch) fetch(first, ch);
+    for (int ch = 0; ch < CH; ++ch) fetch(first, first2, ch);
   }
   for (; run < units; run += step) {
     const uint16_t* next = run_start(run + step);
+    const uint16_t* next2 = TWO ? run_start(run + step, 1) : next;
     bs_f32x16_t acc[2][NT];
 #pragma unroll
     for (int mt = 0; mt < 2; ++mt)
@@ -288,7 +309,7 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         if constexpr (SIGNS == 1) w ^= fl[q];
         *reinterpret_cast<bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]) = w;
       }
-      fetch(next, ch);
+      fetch(next, next2, ch);
       // A operands of both steps and both M tiles: rows 16 ks2 + 8 g + e of the image,
       // column 32 mt + c
       bs_u32x4 a2[2][2];
@@ -330,10 +351,16 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
     // butterflies over j = 32 mt + 8 b + 4 g + r
     uint16_t* __restrict__ yr;
     bool stored = true;  // PAIR: a run past the last tensor is not
+    uint16_t* __restrict__ yr2 = nullptr;  // TWO: the lane's second run
+    bool stored2 = false;
     if constexpr (RUNS > 2) {
       const int64_t mine = unit_runs * run + (int64_t)my_run;
       yr = bs_lane_run<true>(tab, min(mine, tab.total - 1), n);
       stored = mine < tab.total;
+      if constexpr (TWO) {
+        yr2 = bs_lane_run<true>(tab, min(mine + 1, tab.total - 1), n);
+        stored2 = mine + 1 < tab.total;
+      }
     } else if constexpr (PAIR) {
       int64_t la, lb;
       const int64_t rb = 2 * run + 1 < tab.total ? 2 * run + 1 : 2 * run;
@@ -358,8 +385,8 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         const float t = PAIR ? acc[1][nt][v] : acc[0][nt][v] - acc[1][nt][v];
         const auto pr = __builtin_amdgcn_permlane32_swap(__float_as_uint(s), __float_as_uint(t), false, false);
         const float lower = __uint_as_float(pr[0]), upper = __uint_as_float(pr[1]);  // g = 0, g = 1
-        u[0][v] = lower + upper;
-        u[1][v] = lower - upper;
+        u[0][v] = TWO ? lower : lower + upper;  // (TWO: columns 4 apart belong to two runs)
+        u[1][v] = TWO ? upper : lower - upper;
       }
 #pragma unroll
       for (int x = 0; x < 2; ++x)
@@ -395,8 +422,14 @@ block_sylvester64_kernel(BsTable tab, const uint16_t* __restrict__ ma_t, int k_d
         const int row = out_first + 32 * nt + (int)(l >> 3) + 8 * q;
         bs_u32x4 w = *reinterpret_cast<const bs_u32x4*>(&image[((l >> 3) + 8 * q) * kBsPitch + 4 * (l & 7u)]);
         if constexpr (SIGNS == 2) w ^= fo[q];
-        if (row < k_dim && stored)
+        if constexpr (TWO) {
+          if (row < k_dim && stored)
+            stg_nt<uint16_t, 4>(yr + 4 * row, __builtin_bit_cast(Vec<uint16_t, 4>, Vec<uint32_t, 2>{{w[0], w[1]}}));
+          if (row < k_dim && stored2)
+            stg_nt<uint16_t, 4>(yr2 + 4 * row, __builtin_bit_cast(Vec<uint16_t, 4>, Vec<uint32_t, 2>{{w[2], w[3]}}));
+        } else if (row < k_dim && stored) {
           stg_nt<uint16_t, 8>(yr + (row << log_inner) + piece, __builtin_bit_cast(Vec<uint16_t, 8>, w));
+        }
       }
     }
   }
@@ -652,6 +685,7 @@ int launch_bs(const BsTable& tab, int io_dtype, int inner, const uint16_t* ma_t,
 #define CTMI_BS_RUNS(R)                                                                       \
   (half ? launch_bs_dtype<NT, true, R, CH>(tab, ma_t, k, sign_in, sign_out, scale, st)        \
         : launch_bs_dtype<NT, false, R, CH>(tab, ma_t, k, sign_in, sign_out, scale, st))
+  if (inner == 4) return CTMI_BS_RUNS(16);
   if (inner == 8) return CTMI_BS_RUNS(8);
   if (inner == 16) return CTMI_BS_RUNS(4);
   if (inner == 32) return CTMI_BS_RUNS(2);
@@ -662,7 +696,8 @@ int launch_bs(const BsTable& tab, int io_dtype, int inner, const uint16_t* ma_t,
 }  // namespace
 
 bool block_sylvester64_supported(int k, int inner, int io_dtype, bool both_signs) {
-  const bool size = inner == 128 ? k <= 224 : (inner == 64 || inner == 32 || inner == 16 || inner == 8) && k <= 256;
+  const bool size = inner == 128 ? k <= 224
+                                 : (inner == 64 || inner == 32 || inner == 16 || inner == 8 || inner == 4) && k <= 256;
   return (io_dtype == CTMI_BF16 || io_dtype == CTMI_F16) && k >= 1 && size && !both_signs;
 }
 
@@ -670,7 +705,7 @@ int block_sylvester64_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int 
                              const uint16_t* ma_t, const float* sign_in, const float* sign_out,
                              float scale, hipStream_t st) {
   CTMI_REQUIRE(block_sylvester64_supported(k, inner, io_dtype, sign_in && sign_out), CTMI_ERR_UNSUPPORTED,
-               "bfloat16 or float16 tensors, a Sylvester factor of 8 ... 64 with blocks of up to 256 x 256 or of "
+               "bfloat16 or float16 tensors, a Sylvester factor of 4 ... 64 with blocks of up to 256 x 256 or of "
                "128 with blocks of up to 224 x 224, signs on one side");
   CTMI_REQUIRE(n_jobs >= 1 && n_jobs <= kFwhtMaxJobs, CTMI_ERR_VALUE, "1 to %d tensors a launch", kFwhtMaxJobs);
   CTMI_REQUIRE(ma_t && (uintptr_t)sign_in % 16 == 0 && (uintptr_t)sign_out % 16 == 0, CTMI_ERR_VALUE,

@@ -31,7 +31,7 @@ int fwht_launch(const FwhtJob* jobs, int n_jobs, int io_dtype, int n, const floa
                 const float* sign_out, const float* w0, float scale, const QpCfg* quant,
                 hipStream_t st);
 
-// y = x * diag(sign_in) * (Ma (x) Sylvester(inner)) * diag(sign_out) * scale, inner = 8 ... 128,
+// y = x * diag(sign_in) * (Ma (x) Sylvester(inner)) * diag(sign_out) * scale, inner = 4 ... 128,
 // for every run of k * inner bfloat16 or float16 elements (block_sylvester.hip): ma_t = Ma^T,
 // [k, k] bfloat16 with entries exact in bfloat16 (and, for float16 tensors, in float16), k up to
 // 256 (224 for inner = 128; above 224 not in place); signs on at most one side.  job.packed /

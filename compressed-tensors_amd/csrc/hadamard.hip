@@ -1141,7 +1141,7 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
   if (sylvester_inner)
     CTMI_REQUIRE(ctmi_hadamard_sylvester_inner_supported(a_dim, b_dim, io_dtype) && !(sign_in && sign_out),
                  CTMI_ERR_UNSUPPORTED,
-                 "without mb_t (Mb = Sylvester's matrix): b_dim 8 ... 64 with a_dim up to 256 or b_dim 128 "
+                 "without mb_t (Mb = Sylvester's matrix): b_dim 4 ... 64 with a_dim up to 256 or b_dim 128 "
                  "with a_dim up to 224, bfloat16 or float16 tensors, signs on one side; got %d x %d",
                  a_dim, b_dim);
   else

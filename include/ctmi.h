@@ -509,7 +509,7 @@ int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype);
  * the reference's Hadamard matrices of size K * 2^m (transform/utils/hadamard.py:132-163: a
  * known K x K block times butterflies).  Then only the product with Ma runs on the matrix
  * cores (16-bit inputs: exact in one product) and Mb is butterfly stages on its fp32 result:
- * b_dim 8, 16, 32 or 64 with a_dim up to 256 (above 224: two launches, out must not be x), or
+ * b_dim 4, 8, 16, 32 or 64 with a_dim up to 256 (above 224: two launches, out must not be x), or
  * b_dim 128 with a_dim up to 224 (any block; the reference takes the largest
  * block of its table, so the sizes met are 192 x 16 = 3072, 224 x 16 = 3584, 160 x 32 = 5120,
  * 224 x 32 = 7168, 224 x 64 = 14336, 224 x 128 = 28672 ...), bfloat16 or float16 tensors,

@@ -387,7 +387,7 @@ def test_random_hadamard_of_any_table_size(size, location, inverse, gpu, hadamar
     )
     from compressed_tensors_amd.transform import hadamard as product
 
-    if size >= 1024:  # these have a matrix-core kernel: the dense matrix must not be what ran
+    if size >= 768:  # these have a matrix-core kernel: the dense matrix must not be what ran
         def refuse(*a, **k):
             raise AssertionError(f"size {size} went through the dense matrix")
         monkeypatch.setattr(product, "apply_transform_weight", refuse)
@@ -483,14 +483,15 @@ def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_block
                          [(k, torch.bfloat16, 128) for k in (224, 28, 64, 100, 128)] + [(224, torch.float16, 128)] +
                          [(k, torch.bfloat16, 16) for k in (224, 192, 28, 64, 100)] + [(224, torch.float16, 16)] +
                          [(k, torch.bfloat16, 8) for k in (224, 192, 20, 100)] + [(192, torch.float16, 8)] +
+                         [(k, torch.bfloat16, 4) for k in (224, 192, 100, 240)] + [(224, torch.float16, 4)] +
                          [(256, torch.bfloat16, 64), (240, torch.bfloat16, 64), (228, torch.bfloat16, 32),
                           (240, torch.bfloat16, 16), (252, torch.bfloat16, 8), (240, torch.float16, 64)],
                          ids=lambda v: str(v).replace("torch.", ""))
 def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, hadamard_blocks):
     """ctmi_hadamard_apply without mb_t (Mb = Sylvester(64)): the product with the block on the
     matrix cores, the Sylvester factor as butterflies on its fp32 result; bfloat16 and float16
-    tensors (the block is given in bfloat16 either way); Sylvester(32), (16) and (8) in place of
-    Sylvester(64) (two, four or eight runs share the kernel's 64 columns; numbers of runs that
+    tensors (the block is given in bfloat16 either way); Sylvester(32), (16), (8) and (4) in place of
+    Sylvester(64) (two, four, eight or sixteen runs share the kernel's 64 columns; numbers of runs that
     leave the last unit part empty, units that straddle the tensors of one call: 3584 = 224 * 16
     and 3072 = 192 * 16 are how the reference builds those sizes) and Sylvester(128) (28672 = 224 * 128: two halves of 64 columns and a
     stage over the halves).  Blocks of 228 ... 256 rows (15360 = 240 * 64, 3840 = 240 * 16) take two
@@ -500,7 +501,7 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, ha
     workgroups hold at a time; signs on either side; several tensors in one call."""
     from compressed_tensors_amd import _lib
 
-    announce("block x Sylvester(8 ... 128), butterflies", k, dtype, inner)
+    announce("block x Sylvester(4 ... 128), butterflies", k, dtype, inner)
     code = _lib.dtype_code(dtype)
     assert ctmi.ctmi_hadamard_sylvester_inner_supported(k, inner, code) == 1
     n = k * inner
