@@ -194,3 +194,28 @@ def test_table_loader_rejects_what_is_not_hadamard(tmp_path, hadamard_table_path
     with pytest.raises(ValueError):
         known_hadamard_block(14336 + 4, hadamard_table_path)  # 3585 * 4: no entry fits
     assert known_hadamard_block(4096) == (256, None) and known_hadamard_block(16) == (16, None)
+
+
+def test_matrix_core_split_follows_the_largest_block_rule(ctmi, hadamard_table_path):
+    """host logic only (the library's `supported` queries touch no GPU): for the sizes the
+    reference builds from its table - the largest block that leaves a power of two,
+    hadamard.py:102-129 - HadamardTransform finds a block x Sylvester split the one-product
+    kernel takes, and folds a power of two above 128 into the block"""
+    from compressed_tensors_amd import _lib
+    from compressed_tensors_amd.transform import known_hadamard_block
+    from compressed_tensors_amd.transform.hadamard import _matrix_core_split
+
+    code = _lib.dtype_code(torch.bfloat16)
+    # with the fixture's table (blocks 12, 20, 28, 144 ... 240 and the powers of two)
+    for size, block, inner in ((768, 192, 4), (3072, 192, 16), (3584, 224, 16), (3840, 240, 16),
+                               (5120, 160, 32), (7168, 224, 32), (14336, 224, 64), (15360, 240, 64)):
+        k, _ = known_hadamard_block(size, hadamard_table_path)
+        assert (k, size // k) == (block, inner)
+        assert _matrix_core_split(ctmi, k, size // k, code) == (block, inner, True)
+    assert _matrix_core_split(ctmi, 224, 128, code) == (224, 128, True)   # 28672
+    assert _matrix_core_split(ctmi, 240, 128, code) is None               # 30720: no kernel
+    assert _matrix_core_split(ctmi, 20, 256, code) == (40, 128, True)     # a caller's small block: folded
+    assert _matrix_core_split(ctmi, 1, 16384, code) == (128, 128, True)   # Sylvester(16384)
+    assert _matrix_core_split(ctmi, 1, 32768, code) is None
+    assert _matrix_core_split(ctmi, 144, 256, code) is None               # 36864: the folded block has 288 rows
+    assert _matrix_core_split(ctmi, 224, 64, _lib.dtype_code(torch.float32)) is None
