@@ -693,6 +693,9 @@ int bs_by_block(const BsTable& tab, const uint16_t* ma_t, int k, const float* si
   if (k <= 32) return launch_bs_dtype<1, HALF, RUNS>(tab, ma_t, k, sign_in, sign_out, scale, st);
   if (k <= 64) return launch_bs_dtype<2, HALF, RUNS>(tab, ma_t, k, sign_in, sign_out, scale, st);
   if (k <= 128) return launch_bs_dtype<4, HALF, RUNS>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  // (the reference's largest-block rule gives blocks of 132 ... 256 rows: a tile count of their own each)
+  if (k <= 160) return launch_bs_dtype<5, HALF, RUNS>(tab, ma_t, k, sign_in, sign_out, scale, st);
+  if (k <= 192) return launch_bs_dtype<6, HALF, RUNS>(tab, ma_t, k, sign_in, sign_out, scale, st);
   if (k <= 224) return launch_bs_dtype<7, HALF, RUNS>(tab, ma_t, k, sign_in, sign_out, scale, st);
   return launch_bs_dtype<4, HALF, RUNS, 8>(tab, ma_t, k, sign_in, sign_out, scale, st);
 }
@@ -705,6 +708,8 @@ int bs_wide(const BsTable& tab, int inner, const uint16_t* ma_t, int k, const fl
     if (k <= 32) return launch_bs128<1, HALF>(tab, ma_t, k, sign_in, sign_out, scale, st);
     if (k <= 64) return launch_bs128<2, HALF>(tab, ma_t, k, sign_in, sign_out, scale, st);
     if (k <= 128) return launch_bs128<4, HALF>(tab, ma_t, k, sign_in, sign_out, scale, st);
+    if (k <= 160) return launch_bs128<5, HALF>(tab, ma_t, k, sign_in, sign_out, scale, st);
+    if (k <= 192) return launch_bs128<6, HALF>(tab, ma_t, k, sign_in, sign_out, scale, st);
     return launch_bs128<7, HALF>(tab, ma_t, k, sign_in, sign_out, scale, st);
   }
   if (inner == 64) return bs_by_block<HALF, 1>(tab, ma_t, k, sign_in, sign_out, scale, st);

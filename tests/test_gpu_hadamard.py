@@ -484,6 +484,8 @@ def test_matrix_core_kernel_with_a_224_block(b, dtype, ctmi, gpu, hadamard_block
                          [(k, torch.bfloat16, 16) for k in (224, 192, 28, 64, 100)] + [(224, torch.float16, 16)] +
                          [(k, torch.bfloat16, 8) for k in (224, 192, 20, 100)] + [(192, torch.float16, 8)] +
                          [(k, torch.bfloat16, 4) for k in (224, 192, 100, 240)] + [(224, torch.float16, 4)] +
+                         [(160, torch.bfloat16, 128), (192, torch.bfloat16, 128), (148, torch.float16, 128),
+                          (192, torch.bfloat16, 64), (148, torch.bfloat16, 32)] +
                          [(256, torch.bfloat16, 64), (240, torch.bfloat16, 64), (228, torch.bfloat16, 32),
                           (240, torch.bfloat16, 16), (252, torch.bfloat16, 8), (240, torch.float16, 64)],
                          ids=lambda v: str(v).replace("torch.", ""))
