@@ -143,20 +143,34 @@ def cpu_baseline(torch, sample_shapes, seed):
         "kind": "port",
         "sample": "compress+decompress of " + " + ".join(f"{r}x{c}" for _, r, c in sample_shapes)
         + f" bf16 (W4A16 g128), median of 5 after 1 warm-up, torch {torch.__version__} CPU",
+        "sample_short": f"compress+decompress of {len(sample_shapes)} of the workload's tensors "
+                        f"({sum(r * c for _, r, c in sample_shapes)} elements), median of 5",
         "seconds": med,
     }
 
 
 # ---------------------------------------------------------------------------------------------
 # The other configurations: lists of operations on the C ABI, prepared once and timed one by one
+def chained(n_tensors, per_launch=8):
+    """kernel launches of a many-tensor entry point: every chain kernel of the library takes up
+    to 8 tensors a launch"""
+    return -(-n_tensors // per_launch)
+
+
 class Op:
     """primary=False: an operation that is only there to be compared with (the separate steps a
     fused operation replaces, one call per weight against one call for all)"""
 
-    def __init__(self, name, calls, nbytes, kernel, primary=True, mfma_flops=None):
+    def __init__(self, name, calls, nbytes, kernel, primary=True, mfma_flops=None, launches=None,
+                 useful_flops=None):
         self.name, self.calls, self.nbytes, self.kernel = name, calls, nbytes, kernel
         self.primary = primary
         self.mfma_flops = mfma_flops  # flops the kernel issues on the matrix cores, per pass
+        # ... and those of them the transform needs: an fp32 operand that goes into a product as
+        # three bf16 terms is issued three times and needed once
+        self.useful_flops = mfma_flops if useful_flops is None else useful_flops
+        # launches of `kernel` per pass: one per call unless a call chains several
+        self.launches = len(calls) if launches is None else launches
         self.ms = 0.0
 
 
@@ -288,12 +302,12 @@ def other_workload(torch, name, seed):
             a_dyn.append(dynamic(x, out, 4096, targs))
             acts.append(x)
         na = 8 * 8192 * 4096
-        ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_kernel"),
-               Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_kernel"),
+        ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_kernel", launches=chained(len(entries))),
+               Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_kernel", launches=chained(len(entries))),
                Op("weights one-shot: per-channel observer (224 calls)", w_obs, 2 * n, "observe_wide_kernel", primary=False),
                Op("weights one-shot: quantize with those scales (224 calls)", w_q, 3 * n, "qdq_vec_kernel", primary=False),
                Op("weights one-shot: scales + fp8 codes in one pass (224 calls)", w_one, 3 * n, "dynamic_rows_kernel", primary=False),
-               Op("weights one-shot: scales + fp8 codes in one pass, one call (8 per launch)", w_many, 3 * n, "dynamic_rows_many_kernel"),
+               Op("weights one-shot: scales + fp8 codes in one pass, one call (8 per launch)", w_many, 3 * n, "dynamic_rows_many_kernel", launches=chained(len(entries))),
                Op("weights one-shot, 128x128 blocks: scales + fp8 codes in one pass (224 calls)", w_blk, 3 * n,
                   "observe_quantize_blocks_kernel", primary=False),
                Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
@@ -411,17 +425,17 @@ def other_workload(torch, name, seed):
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
                Op("sparse-24-bitmask compress, fp8, all 16 in one call (8 per launch)",
-                  [lambda: _lib.check(lib.ctmi_sparse24_compress_many(*cm))], s24_bytes, "sparse24_compress_chain_kernel"),
+                  [lambda: _lib.check(lib.ctmi_sparse24_compress_many(*cm))], s24_bytes, "sparse24_compress_chain_kernel", launches=chained(copies24)),
                Op("sparse-24-bitmask decompress, fp8, all 16 in one call (8 per launch)",
-                  [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm))], s24_bytes, "sparse24_scatter_kernel"),
+                  [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm))], s24_bytes, "sparse24_scatter_kernel", launches=chained(copies24)),
                Op("sparse-24-bitmask compress, 14336x4096 bf16", s16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress, bf16", t16_calls, 2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel"),
                Op("sparse-24-bitmask compress, bf16, all 16 in one call (8 per launch)",
                   [lambda: _lib.check(lib.ctmi_sparse24_compress_many(*cm16))],
-                  2 * s24_bytes - copies24 * (n24 // 8), "sparse24_compress_chain_kernel"),
+                  2 * s24_bytes - copies24 * (n24 // 8), "sparse24_compress_chain_kernel", launches=chained(copies24)),
                Op("sparse-24-bitmask decompress, bf16, all 16 in one call (8 per launch)",
                   [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm16))],
-                  2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel"),
+                  2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel", launches=chained(copies24)),
                Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies24 * (n24 + n24 // 8), "pack_bitmasks"),
                Op("unpack_bitmasks", up_calls, copies24 * (n24 + n24 // 8), "unpack_bitmasks"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
@@ -465,7 +479,7 @@ def other_workload(torch, name, seed):
                 keep.append(jobs)
                 m = (jobs, len(many), st)
                 ops.append(Op(f"nvfp4 {what} {r}x{c} (x{n_copies}), one call (8 per launch)",
-                              [lambda m=m, entry=entry: _lib.check(entry(*m))], nbytes, kernel))
+                              [lambda m=m, entry=entry: _lib.check(entry(*m))], nbytes, kernel, launches=chained(n_copies)))
         # the Llama-3-8B-shaped set: one call per weight against all 224 in one call
         from compressed_tensors_amd.compressors import Fp4WeightBatch
         entries, single_c, single_d, n_set = [], [], [], 0
@@ -486,9 +500,9 @@ def other_workload(torch, name, seed):
             single_d.append(lambda da=da: _lib.check(lib.ctmi_nvfp4_decompress(*da)))
         set_bytes = 2 * n_set + n_set // 16 + n_set // 2
         ops += [Op("nvfp4 compress, Llama-3-8B set, one call per weight (224)", single_c, set_bytes, "nvfp4_compress_vec_kernel", primary=False),
-                Op("nvfp4 compress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.compress], set_bytes, "nvfp4_compress_chain_kernel"),
+                Op("nvfp4 compress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.compress], set_bytes, "nvfp4_compress_chain_kernel", launches=chained(batch.n)),
                 Op("nvfp4 decompress, Llama-3-8B set, one call per weight (224)", single_d, set_bytes, "nvfp4_decompress_vec_kernel", primary=False),
-                Op("nvfp4 decompress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.decompress], set_bytes, "nvfp4_decompress_chain_kernel")]
+                Op("nvfp4 decompress, Llama-3-8B set, all weights in one call (8 per launch)", [batch.decompress], set_bytes, "nvfp4_decompress_chain_kernel", launches=chained(batch.n))]
         # one-shot: group scales + codes from one pass over weights whose global scale is known
         oj = (_lib.ObserveNvfp4Job * batch.n)()
         one_calls = []
@@ -508,7 +522,7 @@ def other_workload(torch, name, seed):
                    "nvfp4_observe_compress_kernel", primary=False),
                 Op("nvfp4 one-shot (scales + codes), Llama-3-8B set, all weights in one call (8 per launch)",
                    [lambda: _lib.check(lib.ctmi_observe_nvfp4_compress_many(*om))], set_bytes,
-                   "nvfp4_observe_compress_chain_kernel")]
+                   "nvfp4_observe_compress_chain_kernel", launches=chained(batch.n))]
         aargs = QuantizationArgs(num_bits=4, type="float", symmetric=True, strategy="tensor_group",
                                  group_size=16, dynamic="local")
         o_calls, f_calls, y_calls = [], [], []
@@ -554,7 +568,7 @@ def other_workload(torch, name, seed):
         ops = [Op("observer + qparams, group 128 (224 tensors, one call each)", sep_obs, 2 * n + 3 * g, "observe_flat_kernel", primary=False),
                Op("quantize + pack with those scales (one call each)", sep_cmp, 2 * n + 2 * g + n // 2, "pq_compress_vec_kernel", primary=False),
                Op("observer + qparams + quantize + pack in one pass (one call each)", fused, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel", primary=False),
-               Op("the same, all 224 tensors in one call (8 per launch)", many, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel")]
+               Op("the same, all 224 tensors in one call (8 per launch)", many, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel", launches=chained(len(job_fields)))]
         return "one-shot W4A16 g128 compression GB/s (no scales given), Llama-3-8B-shaped weights", ops, keep
 
     if name == "hadamard":
@@ -581,11 +595,13 @@ def other_workload(torch, name, seed):
                 # into the second as three bf16 terms)
                 per_elem = 2 * b_dim if a_dim == 1 else 2 * b_dim + 6 * a_dim
                 flops = sum(per_elem * x.numel() for x in xs)
+                useful = sum(2 * (a_dim + b_dim if a_dim > 1 else b_dim) * x.numel() for x in xs)
                 # size 4096 on the matrix cores: kept to compare with the butterfly kernel below,
                 # which is what hadamard_apply picks for this size
                 ops.append(Op(f"random-sign Hadamard, size {n}{' (matrix cores)' if a_dim > 1 else ''}: {label}",
                               calls, nb, "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
-                              primary=a_dim == 1 and not label.startswith("weights 4096x4096"), mfma_flops=flops))
+                              primary=a_dim == 1 and not label.startswith("weights 4096x4096"), mfma_flops=flops,
+                              useful_flops=useful))
                 if label.startswith("weights 4096x4096"):
                     jobs = (_lib.HadamardJob * len(xs))()
                     outs = [torch.empty_like(x) for x in xs]
@@ -598,7 +614,8 @@ def other_workload(torch, name, seed):
                                   "one call (8 per launch)",
                                   [lambda m=m: _lib.check(lib.ctmi_hadamard_apply_many(*m))], nb,
                                   "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
-                                  primary=a_dim == 1, mfma_flops=flops))
+                                  primary=a_dim == 1, mfma_flops=flops, useful_flops=useful,
+                                  launches=chained(len(xs))))
         # sizes 4096 and 8192 as butterflies in registers (ctmi_sylvester_apply_many): what
         # hadamard_apply and HadamardTransform.forward run for these sizes
         tensors["activations 4096x8192 (x8)"] = [randn(4096, 8192) for _ in range(8)]
@@ -620,12 +637,18 @@ def other_workload(torch, name, seed):
                     calls.append(lambda a=a: _lib.check(lib.ctmi_sylvester_apply_many(*a)))
                 keep.append(many)
                 nb = sum(4 * x.numel() for x in xs)
-                ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb, "fwht_lds_kernel",
-                              primary=not label.startswith("weights 4096x4096")))
+                # bf16 runs of 4096 go to the kernel that does the 64 x 64 factor over the inner
+                # index as ONE exact bf16 product on the matrix cores (2 * 64 flops an element, all
+                # of them needed) and the other factor as butterflies; 8192 is butterflies only
+                kernel = "fwht_mfma_kernel" if n == 4096 else "fwht_lds_kernel"
+                flops = sum(2 * 64 * x.numel() for x in xs) if n == 4096 else None
+                ops.append(Op(f"random-sign Hadamard, size {n}: {label}", calls, nb, kernel,
+                              primary=not label.startswith("weights 4096x4096"), mfma_flops=flops))
                 if label.startswith("weights 4096x4096"):
                     m = (many, len(xs), code(xs[0].dtype), n, q.data_ptr(), None, st)
                     ops.append(Op(f"random-sign Hadamard, size {n}: {label}, one call (8 per launch)",
-                                  [lambda m=m: _lib.check(lib.ctmi_sylvester_apply_many(*m))], nb, "fwht_lds_kernel"))
+                                  [lambda m=m: _lib.check(lib.ctmi_sylvester_apply_many(*m))], nb, kernel,
+                                  mfma_flops=flops, launches=chained(len(xs))))
         # 14336 = 224 x 64: a known Hadamard matrix of order 224 (here: any +-1 matrix, the kernel's
         # work does not depend on the entries) times Sylvester(64), as the reference builds the
         # rotation in front of Llama-3's down projections
@@ -645,7 +668,8 @@ def other_workload(torch, name, seed):
         ops.append(Op("random-sign Hadamard, size 14336 = 224 x 64, both factors as matrix products: "
                       "activations 4096x14336 (x5)", calls,
                       sum(4 * x.numel() for x in xs14), "hadamard_kron_kernel", primary=False,
-                      mfma_flops=sum((2 * 64 + 6 * 224) * x.numel() for x in xs14)))
+                      mfma_flops=sum((2 * 64 + 6 * 224) * x.numel() for x in xs14),
+                      useful_flops=sum(2 * (64 + 224) * x.numel() for x in xs14)))
         # the same transform as HadamardTransform.forward runs it: the block on the matrix cores,
         # Sylvester(64) as butterflies (no matrix for it: mb_t = NULL)
         calls = []
@@ -705,7 +729,7 @@ def other_workload(torch, name, seed):
                 m = (jobs, len(xs), code(xs[0].dtype), 128, mb.data_ptr(), q.data_ptr(), None, 4, 1, st)
                 ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
                               [lambda m=m: _lib.check(lib.ctmi_hadamard_quant_pack_many(*m))], nb,
-                              "hadamard_quant_pack_kernel", mfma_flops=flops))
+                              "hadamard_quant_pack_kernel", mfma_flops=flops, launches=chained(len(xs))))
         # the full 4096-wide rotation (64 x 64) with the same quantization in its epilogue
         mb64 = deterministic_hadamard_matrix(64, torch.bfloat16, dev).contiguous()
         q4k = (torch.randint(0, 2, (4096,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
@@ -729,15 +753,17 @@ def other_workload(torch, name, seed):
             keep.append(many)
             nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in xs)
             flops = sum((2 * 64 + 6 * 64) * x.numel() for x in xs)
+            useful = sum(2 * (64 + 64) * x.numel() for x in xs)
             ops.append(Op(f"fused: Hadamard 4096 (matrix cores) + int4 g128 quantize + pack, {label}", calls, nb,
-                          "hadamard_kron_kernel", primary=False, mfma_flops=flops))
+                          "hadamard_kron_kernel", primary=False, mfma_flops=flops, useful_flops=useful))
             if label.startswith("weights 4096x4096"):
                 m = (many, len(xs), code(xs[0].dtype), 64, 64, mb64.data_ptr(), mb64.data_ptr(),
                      q4k.data_ptr(), None, 128, 4, 1, st)
                 ops.append(Op(f"fused: Hadamard 4096 (matrix cores) + int4 g128 quantize + pack, {label}, "
                               "one call (8 per launch)",
                               [lambda m=m: _lib.check(lib.ctmi_hadamard_kron_quant_pack_many(*m))], nb,
-                              "hadamard_kron_kernel", primary=False, mfma_flops=flops))
+                              "hadamard_kron_kernel", primary=False, mfma_flops=flops, useful_flops=useful,
+                              launches=chained(len(xs))))
             # the same through the butterfly kernel (what hadamard_quantize_pack picks)
             calls = []
             for i in range(len(xs)):
@@ -746,13 +772,14 @@ def other_workload(torch, name, seed):
                 keep.append(one)
                 a = (one, 1, code(xs[i].dtype), 4096, q4k.data_ptr(), None, 128, 4, 1, st)
                 calls.append(lambda a=a: _lib.check(lib.ctmi_sylvester_quant_pack_many(*a)))
+            flops = sum(2 * 64 * x.numel() for x in xs)
             ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}", calls, nb,
-                          "fwht_lds_kernel", primary=not label.startswith("weights 4096x4096")))
+                          "fwht_mfma_kernel", primary=not label.startswith("weights 4096x4096"), mfma_flops=flops))
             if label.startswith("weights 4096x4096"):
                 m = (many, len(xs), code(xs[0].dtype), 4096, q4k.data_ptr(), None, 128, 4, 1, st)
                 ops.append(Op(f"fused: Hadamard 4096 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
                               [lambda m=m: _lib.check(lib.ctmi_sylvester_quant_pack_many(*m))], nb,
-                              "fwht_lds_kernel"))
+                              "fwht_mfma_kernel", mfma_flops=flops, launches=chained(len(xs))))
         return "Hadamard rotation GB/s, block 128 (bf16 MFMA) and full 4096 / 8192 (butterflies), and fused with int4 packing", ops, keep
 
     raise SystemExit(f"unknown workload {name}")
@@ -828,31 +855,36 @@ def cpu_baseline_other(torch, workload, seed):
             "seconds": med}
 
 
-def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True):
+def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True, only_op=None):
     """one of the other configurations -> its result object (same fields as the headline
-    line, plus the per-operation table)"""
+    line, plus the per-operation table).  only_op: time just the operations whose name contains
+    this text (a counter run then sees the launches of that operation and no others)"""
     metric, ops, keep = other_workload(torch, workload, seed)
+    if only_op:
+        ops = [op for op in ops if only_op in op.name]
+        if not ops:
+            raise SystemExit(f"no operation of {workload} is named like {only_op!r}")
+        for op in ops:
+            op.primary = True
     step_s = time_ops(torch, ops, steps, warmup)
     total_bytes = sum(op.nbytes for op in ops)
     gpu_ms = sum(op.ms for op in ops)
     # the roofline object describes the operation most of the time goes to (comparison-only
     # operations aside); every operation's own rate is in `operations`
     slow = max((op for op in ops if op.primary), key=lambda op: op.ms)
-    n_launch = len(slow.calls)
+    n_launch = slow.launches
     traffic, traffic_source = measured_traffic(workload, slow.kernel)
-    if traffic is None and (PROFILES / "all_workloads_pmc_traffic.txt").exists():
-        # one kernel serves launches of many sizes here: the counters are listed per kernel and
-        # grid size in that file instead of as one figure per launch
-        traffic_source = "profiles/all_workloads_pmc_traffic.txt (FETCH_SIZE / WRITE_SIZE per kernel and grid size)"
 
     def op_row(op):
         row = {"name": op.name, "kernel": op.kernel, "GBs": op.nbytes / (op.ms * 1e-3) / 1e9,
                "frac_of_hbm_peak": op.nbytes / (op.ms * 1e-3) / 1e9 / HBM_PEAK_GBS,
                "ms": op.ms, "algorithmic_bytes": op.nbytes,
                "for_comparison_only": not op.primary}
+        row["launches"] = op.launches
         if op.mfma_flops is not None:
             row["mfma_TFLOPs"] = op.mfma_flops / (op.ms * 1e-3) / 1e12
             row["mfma_utilisation"] = op.mfma_flops / (op.ms * 1e-3) / MFMA_BF16_PEAK
+            row["mfma_utilisation_useful_flops"] = op.useful_flops / (op.ms * 1e-3) / MFMA_BF16_PEAK
         return row
 
     out = {
@@ -862,7 +894,7 @@ def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True):
         "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": step_s * 1e3,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16 in, codes as the format says (arithmetic in the reference's promoted dtype)",
+        "dtype": "bf16 (codes as the format says; arithmetic in the dtype the reference's chain promotes to)",
         "data": "synthetic",
         "config": {"workload": workload, "seed": seed,
                    "value_is": "algorithmic bytes of all operations / sum of their GPU times",
@@ -886,8 +918,10 @@ def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True):
             "peak": "2.5 PFLOP/s dense bf16", "kernel": best.kernel, "operation": best.name,
             "achieved_TFLOPs": best.mfma_flops / (best.ms * 1e-3) / 1e12,
             "frac": best.mfma_flops / (best.ms * 1e-3) / MFMA_BF16_PEAK,
-            "counts": "matrix-core flops the kernel issues (an fp32 operand that goes in as three "
-                      "bf16 terms counts three times)"}
+            "frac_useful_flops": best.useful_flops / (best.ms * 1e-3) / MFMA_BF16_PEAK,
+            "counts": "frac: matrix-core flops the kernel issues (an fp32 operand that goes in as three "
+                      "bf16 terms counts three times); frac_useful_flops: 2 x (factor sizes) per element, "
+                      "what the transform needs"}
     del keep, ops
     torch.cuda.empty_cache()
     if with_cpu_baseline:
@@ -962,6 +996,68 @@ def api_level(torch, seed, steps):
 
 
 OTHER_WORKLOADS = ("fp8-w8a8", "sparse", "nvfp4", "hadamard", "one-shot")
+
+MAX_LINE = 1500  # characters of the line on stdout: what reads it keeps a short tail only
+
+
+def _sig(x, digits=4):
+    """floats to a few significant digits (the full figures are in the details file)"""
+    if isinstance(x, float):
+        return float(f"{x:.{digits}g}")
+    return x
+
+
+def short_line(out, details_path=None):
+    """the one line that goes to stdout: the contract's fields, the roofline of the dominant
+    kernel, the CPU baseline, and one number for each other configuration"""
+    def pick(d, keys):
+        return {k: _sig(d[k]) for k in keys if k in d}
+
+    line = {k: _sig(out[k]) for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                                      "higher_is_better", "scaling", "vs_baseline", "dtype", "data")
+            if k in out}
+    line["dtype"] = str(out.get("dtype", "")).split(" ")[0]
+    line["config"] = pick(out.get("config", {}), ("workload", "tensors", "elements", "group_size", "seed"))
+    line["roofline"] = pick(out["roofline"], ("bound", "kernel", "achieved", "peak", "unit", "frac",
+                                              "traffic", "achieved_bytes_per_launch", "avg_launch_ms",
+                                              "launches_per_step"))
+    if "cpu_baseline" in out:
+        base = pick(out["cpu_baseline"], ("value", "unit", "cores", "kind", "seconds"))
+        base["sample"] = str(out["cpu_baseline"].get("sample_short") or out["cpu_baseline"].get("sample", ""))[:120]
+        line["cpu_baseline"] = base
+    if "parity" in out:
+        line["parity"] = "bit-exact vs oracle (row slices, before timing)"
+    if "configs" in out:
+        # per configuration: roofline fraction of the operation most of its time goes to
+        line["configs_frac"] = {w: _sig(r["roofline"]["frac"], 3) for w, r in out["configs"].items()}
+    if "mfma_utilisation" in out:
+        line["mfma_frac"] = _sig(out["mfma_utilisation"]["frac"], 3)
+    if "api_level" in out:
+        line["api_level"] = pick(out["api_level"], ("frac_of_hbm_peak", "compress_model_ms", "decompress_model_ms"))
+    if details_path:
+        line["details"] = os.path.relpath(details_path, ROOT)
+    text = json.dumps(line, separators=(",", ":"))
+    if len(text) > MAX_LINE:  # never happens with the fields above; drop the optional ones if it does
+        for k in ("details", "parity", "configs_frac", "api_level", "mfma_frac"):
+            line.pop(k, None)
+            text = json.dumps(line, separators=(",", ":"))
+            if len(text) <= MAX_LINE:
+                break
+    return text
+
+
+def emit(out, details_path):
+    """full result -> the details file (and stderr if the file cannot be written); short line -> stdout"""
+    full = json.dumps(out, indent=1)
+    written = None
+    try:
+        Path(details_path).parent.mkdir(parents=True, exist_ok=True)
+        Path(details_path).write_text(full + "\n")
+        written = details_path
+    except OSError as e:
+        print(f"bench.py: details not written ({e}); they follow on stderr", file=sys.stderr)
+        print(full, file=sys.stderr)
+    print(short_line(out, written), flush=True)
 
 
 def headline(torch, a):
@@ -1060,7 +1156,7 @@ def headline(torch, a):
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16->int4 (arithmetic in fp32 rounded to bf16 per op)",
+        "dtype": "bf16 (every operation of the chain rounds to bf16, as the reference's does; codes are int4)",
         "data": "synthetic",
         "config": {
             "workload": a.workload,
@@ -1096,7 +1192,7 @@ def headline(torch, a):
     del batch, entries
     torch.cuda.empty_cache()
     if not a.no_cpu_baseline:
-        sample = LLAMA3_8B_LAYER  # one layer of 32; the other 31 are identical work
+        sample = LLAMA3_8B_LAYER * 4  # four layers of 32 (about 10 s of CPU work); the others are identical work
         if a.workload == "w4a16-4096":
             sample = [("w", 4096, 4096)]
         out["cpu_baseline"] = cpu_baseline(torch, sample, a.seed)
@@ -1115,6 +1211,11 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--calib-copies", type=int, default=0,
                     help="launch N plain 1 GiB copies first (byte-counter calibration when profiling)")
+    ap.add_argument("--only-op", default=None,
+                    help="with --workload: time only the operations whose name contains this text")
+    ap.add_argument("--details", default=str(ROOT / "gpurun_out" / "bench_details.json"),
+                    help="file the full result goes to (per-operation tables of every configuration); "
+                         "stdout carries one short line")
     a = ap.parse_args()
     if a.gpus != 1:
         raise SystemExit(
@@ -1132,11 +1233,11 @@ def main():
     if a.workload is None:
         a.workload = "llama3-8b-w4a16"
     if a.workload == "api":
-        print(json.dumps(api_level(torch, a.seed, a.steps)))
+        print(json.dumps({k: _sig(v) for k, v in api_level(torch, a.seed, a.steps).items()}))
         return
     if a.workload in OTHER_WORKLOADS:
-        print(json.dumps(run_other(torch, a.workload, a.seed, a.steps, a.warmup,
-                                   not a.no_cpu_baseline)))
+        emit(run_other(torch, a.workload, a.seed, a.steps, a.warmup, not a.no_cpu_baseline, a.only_op),
+             a.details)
         return
     out = headline(torch, a)
     if everything:
@@ -1149,7 +1250,7 @@ def main():
                                                    "roofline", "mfma_utilisation", "operations",
                                                    "cpu_baseline") if k in r}
         out["api_level"] = api_level(torch, a.seed, min(a.steps, 5))
-    print(json.dumps(out))
+    emit(out, a.details)
 
 
 if __name__ == "__main__":

@@ -23,11 +23,18 @@ from compressed_tensors_amd.config import (
     QuantizationStatus,
     SparsityCompressionConfig,
 )
+from compressed_tensors_amd.compressors.quantized_base import own_parameters, swap_parameters
 from compressed_tensors_amd.quantization.quant_scheme import QuantizationConfig, QuantizationScheme
 from compressed_tensors_amd.utils.helpers import load_safetensors_state_dict, nest_state_dict
 
 __all__ = ["ModelCompressor", "map_module_to_scheme", "match_named_modules",
            "apply_quantization_scheme"]
+
+
+def _set_plain(module: Module, name: str, value) -> None:
+    """module.<name> = value for a value that is no parameter, buffer or module (without the
+    checks Module.__setattr__ makes for those)"""
+    object.__setattr__(module, name, value)
 
 
 def _matches(name: str, module: Module, target: str) -> bool:
@@ -55,13 +62,20 @@ def apply_quantization_scheme(model: Module, config: QuantizationConfig) -> None
             module.quantization_status = QuantizationStatus.INITIALIZED
 
 
+def _scheme_of(module: Module):
+    """module.quantization_scheme or None (an instance attribute where it is set: read from
+    the instance's dict, which spares Module.__getattr__'s search on modules without one)"""
+    scheme = module.__dict__.get("quantization_scheme", None)
+    return scheme if scheme is not None else getattr(type(module), "quantization_scheme", None)
+
+
 def map_module_to_scheme(model: Module) -> Dict[str, QuantizationScheme]:
-    return {
-        name.replace("_fsdp_wrapped_module.", ""): module.quantization_scheme
-        for name, module in model.named_modules()
-        if getattr(module, "quantization_scheme", None) is not None
-        and module.quantization_scheme.weights is not None
-    }
+    out = {}
+    for name, module in model.named_modules():
+        scheme = _scheme_of(module)
+        if scheme is not None and scheme.weights is not None:
+            out[name.replace("_fsdp_wrapped_module.", "")] = scheme
+    return out
 
 
 class ModelCompressor:
@@ -330,13 +344,23 @@ class ModelCompressor:
         return cls(sparsity_config=sparsity_config, quantization_config=quantization_config)
 
     # ----- in-memory pathways ----- #
+    def _walk(self, model: Module):
+        """one pass over the module tree -> (named modules, map_module_to_scheme(model),
+        names of the sparsity targets)"""
+        named = list(model.named_modules())
+        module_to_scheme = {}
+        for name, module in named:
+            scheme = _scheme_of(module)
+            if scheme is not None and scheme.weights is not None:
+                module_to_scheme[name.replace("_fsdp_wrapped_module.", "")] = scheme
+        return named, module_to_scheme, self._sparse_targets(model)
+
     def compress_model(self, model: Module) -> None:
-        module_to_scheme = map_module_to_scheme(model)
-        sparse_targets = self._sparse_targets(model)
+        named, module_to_scheme, sparse_targets = self._walk(model)
         # modules that are only quantized: all modules of one format go through one
-        # state-dict call of their compressor (one multi-weight call of the C ABI)
+        # call of their compressor (many-weight calls of the C ABI)
         by_format: Dict[str, List] = {}
-        for prefix, module in list(model.named_modules()):
+        for prefix, module in named:
             if prefix not in module_to_scheme and prefix not in sparse_targets:
                 continue
             if prefix in module_to_scheme and prefix not in sparse_targets:
@@ -359,33 +383,24 @@ class ModelCompressor:
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.COMPRESSED
         for fmt, members in by_format.items():
-            state = {}
-            for prefix, module in members:
-                state.update(self._own_parameters(module, prefix))
-            state = self.quantization_compressor.get(fmt).compress(
-                state, names_to_scheme=module_to_scheme, show_progress=False)
-            per_module: Dict[str, Dict[str, Tensor]] = {prefix: {} for prefix, _ in members}
-            for name, value in state.items():
-                per_module[name.rpartition(".")[0]][name] = value
-            for prefix, module in members:
-                self._swap_parameters(module, prefix, per_module[prefix])
-                module.quantization_status = QuantizationStatus.COMPRESSED
+            self.quantization_compressor.get(fmt).compress_modules(members, module_to_scheme)
+            for _, module in members:
+                _set_plain(module, "quantization_status", QuantizationStatus.COMPRESSED)
         if (self.quantization_config is not None
                 and self.quantization_config.format != CompressionFormat.dense.value):
             self.quantization_config.quantization_status = QuantizationStatus.COMPRESSED.value
 
     def decompress_model(self, model: Module) -> None:
-        module_to_scheme = map_module_to_scheme(model)
-        sparse_targets = self._sparse_targets(model)
+        named, module_to_scheme, sparse_targets = self._walk(model)
         by_format: Dict[str, List] = {}
-        for prefix, module in list(model.named_modules()):
+        for prefix, module in named:
             if prefix not in module_to_scheme and prefix not in sparse_targets:
                 continue
-            state = self._own_parameters(module, prefix)
             if prefix in module_to_scheme and prefix not in sparse_targets:
                 # only quantized: decompressed below, all modules of one format from one call
-                by_format.setdefault(self._format_of(module), []).append((prefix, module, state))
+                by_format.setdefault(self._format_of(module), []).append((prefix, module))
                 continue
+            state = self._own_parameters(module, prefix)
             dense = None
             if prefix in sparse_targets and prefix in module_to_scheme:  # both in one pass
                 dense = self._decompress_quantized_24(
@@ -402,36 +417,17 @@ class ModelCompressor:
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.FROZEN
         for fmt, members in by_format.items():
-            compressor = self.quantization_compressor.get(fmt)
-            local = [{k[len(prefix) + 1:]: v for k, v in state.items()} for prefix, _, state in members]
-            todo = [i for i, data in enumerate(local) if "weight_scale" in data]
-            dense = compressor.decompress_weights(
-                [(local[i], module_to_scheme[members[i][0]].weights) for i in todo])
-            for i, weight in zip(todo, dense):
-                local[i]["weight"] = weight
-            for (prefix, module, _), data in zip(members, local):
-                self._swap_parameters(module, prefix, {f"{prefix}.{k}": v for k, v in data.items()})
-                module.quantization_status = QuantizationStatus.FROZEN
+            self.quantization_compressor.get(fmt).decompress_modules(members, module_to_scheme)
+            for _, module in members:
+                _set_plain(module, "quantization_status", QuantizationStatus.FROZEN)
 
     # ----- helpers ----- #
     @staticmethod
     def _module(model: Module, path: str) -> Module:
         return model.get_submodule(path) if path else model
 
-    @staticmethod
-    def _own_parameters(module: Module, prefix: str) -> Dict[str, Tensor]:
-        """the module's own parameters under their state-dict names"""
-        return {f"{prefix}.{n}": p.data for n, p in module._parameters.items() if p is not None}
-
-    @staticmethod
-    def _swap_parameters(module: Module, prefix: str, state: Dict[str, Tensor]) -> None:
-        """replace the module's own parameters by the entries of `state` (full names)"""
-        params = module._parameters
-        params.clear()
-        cut = len(prefix) + 1
-        for name, value in state.items():
-            local = name[cut:] if name.startswith(prefix + ".") else name
-            params[local] = torch.nn.Parameter(value, requires_grad=False)
+    _own_parameters = staticmethod(own_parameters)
+    _swap_parameters = staticmethod(swap_parameters)
 
     def _assign(self, model: Module, full_name: str, data: Tensor) -> None:
         prefix, _, param_name = full_name.rpartition(".")

@@ -15,6 +15,7 @@ from torch import Tensor
 
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
+from compressed_tensors_amd.compressors.job_tables import WeightJobTable, slab_outputs
 from compressed_tensors_amd.compressors.quantized_base import (
     BaseQuantizationCompressor, LazyDenseOutputs,
 )
@@ -561,3 +562,144 @@ def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progre
 
 
 PackedQuantizationCompressor.compress = _compress_state_dict_batched
+
+
+# ---------------------------------------------------------------------------------------------
+# Module pathways (ModelCompressor.compress_model / decompress_model): the common case - a 2-D
+# float weight on the GPU with group or channel scales, symmetric, no activation ordering - goes
+# into a job table written by columns; everything else takes the state-dict path above.
+_CHUNKS = (8, 24, 32)   # modules per call: a short first one starts the GPU early; then 64 each
+_FLOAT_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+# what compression takes away from a module or writes anew (a symmetric scheme stores no zero points)
+_REPLACED = ("weight", "weight_zero_point", "weight_packed", "weight_shape")
+
+
+def _chunks(n):
+    at = 0
+    for size in _CHUNKS:
+        if at >= n:
+            return
+        yield at, min(at + size, n)
+        at += size
+    while at < n:
+        yield at, min(at + 64, n)
+        at += 64
+
+
+def _args_key(args: QuantizationArgs):
+    return (args.num_bits, args.type, args.symmetric, args.strategy, args.group_size)
+
+
+def _compress_modules_fast(self, members, names_to_scheme) -> None:
+    """PackedQuantizationCompressor.compress_modules: compress_module
+    (compressors/base.py:125-151, pack_quantized.py:88-146) for every (prefix, module) pair"""
+    entry = _lib.load().ctmi_pack_quantized_compress_many
+    table = WeightJobTable()
+    new_param = torch.nn.Parameter
+    slow, arg_keys = [], {}
+    for lo, hi in _chunks(len(members)):
+        picked, shapes, device = [], [], None
+        for prefix, module in members[lo:hi]:
+            params = module._parameters
+            w, scale, zp = params.get("weight"), params.get("weight_scale"), params.get("weight_zero_point")
+            args = names_to_scheme[prefix].weights
+            key = arg_keys.get(id(args))
+            if key is None:
+                key = arg_keys[id(args)] = _args_key(args)
+            if (w is None or scale is None or w.ndim != 2 or w.dtype not in _FLOAT_DTYPES
+                    or w.device.type != "cuda" or not w.is_contiguous()
+                    or scale.dtype not in _FLOAT_DTYPES or scale.device != w.device
+                    or not scale.is_contiguous()
+                    or (zp is not None and (zp.device != w.device or not zp.is_contiguous()))
+                    or not key[2] or key[3] not in _PACKABLE or key[1] != "int" or not 1 <= key[0] <= 8
+                    or (device is not None and device != w.device)
+                    or params.get("weight_g_idx") is not None
+                    or params.get("weight_global_scale") is not None):
+                slow.append((prefix, module))
+                continue
+            device = w.device
+            rows, cols = w.shape
+            picked.append((params, w, scale, zp, args, key, rows, cols))
+            shapes.append((rows, -(-cols // (32 // key[0]))))
+        if not picked:
+            continue
+        packed = slab_outputs(shapes, torch.int32, device)
+        dims = torch.tensor([(p[6], p[7]) for p in picked]).unbind(0)  # every weight_shape, one host tensor
+        for (params, w, scale, zp, args, key, rows, cols), out in zip(picked, packed):
+            tkey = (rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
+            which = table.template(tkey)
+            if which < 0:
+                # the zero points of a symmetric scheme (all zero) take part in the arithmetic
+                # as they are, as in the reference's compress_weight
+                plan = build_qparams(w, scale, zp, args, None, None)
+                table.keep.append(plan)
+                which = table.add_template(tkey, plan)
+            table.add(w.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(w.dtype), which,
+                      scale.data_ptr(), 0 if zp is None else zp.data_ptr())
+        table.launch(entry, _lib.stream_of(device))
+        # the kernels are enqueued: the modules get their new parameters while the GPU works
+        for (params, w, scale, zp, args, key, rows, cols), out, dim in zip(picked, packed, dims):
+            rest = [(n, p) for n, p in params.items() if n not in _REPLACED]
+            params.clear()
+            params["weight_packed"] = new_param(out, requires_grad=False)
+            params["weight_shape"] = new_param(dim, requires_grad=False)
+            params.update(rest)
+    if slow:
+        BaseQuantizationCompressor.compress_modules(self, slow, names_to_scheme)
+
+
+def _decompress_modules_fast(self, members, names_to_scheme) -> None:
+    """PackedQuantizationCompressor.decompress_modules: decompress_module
+    (compressors/base.py:165-190, pack_quantized.py:147-183) for every (prefix, module) pair"""
+    entry = _lib.load().ctmi_pack_quantized_decompress_many
+    table = WeightJobTable()
+    new_param = torch.nn.Parameter
+    slow = []
+    for lo, hi in _chunks(len(members)):
+        picked, shapes, dtype, device = [], [], None, None
+        for prefix, module in members[lo:hi]:
+            params = module._parameters
+            packed, scale, ws = params.get("weight_packed"), params.get("weight_scale"), params.get("weight_shape")
+            args = names_to_scheme[prefix].weights
+            if (packed is None or scale is None or ws is None or ws.device.type != "cpu"
+                    or packed.dtype is not torch.int32 or packed.ndim != 2 or packed.device.type != "cuda"
+                    or not packed.is_contiguous() or scale.ndim != 2 or scale.dtype not in _FLOAT_DTYPES
+                    or scale.device != packed.device or not scale.is_contiguous()
+                    or not args.symmetric or args.strategy not in _PACKABLE or not 1 <= args.num_bits <= 8
+                    or params.get("weight_zero_point") is not None
+                    or params.get("weight_g_idx") is not None
+                    or (dtype is not None and (dtype, device) != (scale.dtype, packed.device))):
+                slow.append((prefix, module))
+                continue
+            shape = tuple(ws.tolist())
+            if len(shape) != 2 or packed.shape != (shape[0], -(-shape[1] // (32 // args.num_bits))):
+                slow.append((prefix, module))
+                continue
+            dtype, device = scale.dtype, packed.device
+            picked.append((params, packed, scale, args.num_bits, shape))
+            shapes.append(shape)
+        if not picked:
+            continue
+        dense = slab_outputs(shapes, dtype, device)
+        for (params, packed, scale, num_bits, shape), out in zip(picked, dense):
+            tkey = (shape, scale.shape, scale.dtype, num_bits)
+            which = table.template(tkey)
+            if which < 0:
+                # dequantize(x_q, scale, zero_point=None, args=None): the strategy follows from
+                # the two shapes, the output dtype is the scale's (pack_quantized.py:176-181)
+                carrier = _ShapeOnly(shape, torch.int8)
+                plan = build_qparams(carrier, scale, None, infer_dequant_args(carrier, scale), None, None)
+                plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_INT, num_bits
+                table.keep.append(plan)
+                which = table.add_template(tkey, plan)
+            table.add(packed.data_ptr(), out.data_ptr(), shape[0], shape[1], _lib.dtype_code(scale.dtype),
+                      which, scale.data_ptr())
+        table.launch(entry, _lib.stream_of(device))
+        for (params, packed, scale, num_bits, shape), out in zip(picked, dense):
+            params["weight"] = new_param(out, requires_grad=False)
+    if slow:
+        BaseQuantizationCompressor.decompress_modules(self, slow, names_to_scheme)
+
+
+PackedQuantizationCompressor.compress_modules = _compress_modules_fast
+PackedQuantizationCompressor.decompress_modules = _decompress_modules_fast

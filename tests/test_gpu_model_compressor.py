@@ -290,3 +290,110 @@ def test_checkpoint_on_disk_roundtrip(tmp_path, gpu):
         save_compressed({}, sparse_path, "sparse-bitmask")
     with pytest.raises(ValueError, match="Unknown compression format"):
         save_compressed({"a.weight": w}, sparse_path, "no-such-format")
+
+
+def test_forward_runs_after_compress_and_decompress_model(gpu):
+    """Linear(bias=False) keeps its empty `bias` slot through compress_model and
+    decompress_model: forward reads it.  The decompressed model computes with the
+    oracle's weights."""
+    from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme,
+    )
+
+    announce("forward after compress_model + decompress_model")
+    torch.manual_seed(2)
+    model = Tiny().to(torch.bfloat16).to(gpu)
+    spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    config = QuantizationConfig(
+        config_groups={"g0": QuantizationScheme(targets=["Linear"], weights=args)},
+        format="pack-quantized", ignore=["lm_head"])
+    apply_quantization_scheme(model, config)
+    cpu = _prepare(model, args, oargs, gpu)
+    mc = ModelCompressor(quantization_config=config)
+    for _ in range(2):  # the second round starts from modules that still hold the packed words
+        mc.compress_model(model)
+        for name in cpu:
+            m = model.get_submodule(name)
+            assert "bias" in m._parameters and m.bias is None
+            assert set(n for n, p in m._parameters.items() if p is not None) == {
+                "weight_packed", "weight_shape", "weight_scale"}
+        mc.decompress_model(model)
+    x = torch.randn(3, 256, device=gpu).bfloat16()
+    for name, (w, s, z) in cpu.items():
+        m = model.get_submodule(name)
+        assert "bias" in m._parameters and m.bias is None
+        want = op.pack_quantized_compress(w, s, oargs, zero_point=z)
+        dense = op.pack_quantized_decompress(dict(want, weight_scale=s), oargs)
+        assert_bit_equal(m.weight.data, dense, name)
+        xin = x if m.in_features == 256 else torch.randn(3, m.in_features, device=gpu).bfloat16()
+        assert_bit_equal(m(xin), torch.nn.functional.linear(xin, dense.to(gpu)).cpu(), f"{name} forward")
+
+
+def test_module_pathway_equals_state_dict_pathway(gpu):
+    """compress_model (job tables written by columns for the common case) leaves in every
+    module what compress(state_dict) returns for it - for the weights that take the common
+    path and for those that do not (asymmetric, activation ordering, channel strategy, fp32)"""
+    from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme, observe_weight_qparams,
+    )
+
+    announce("compress_model vs compress(state_dict)")
+    torch.manual_seed(3)
+
+    class Mixed(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.ModuleList([torch.nn.Linear(256, 64 + 8 * i, bias=False) for i in range(11)])
+            self.b = torch.nn.ModuleList([torch.nn.Linear(256, 48, bias=True) for _ in range(3)])   # asymmetric
+            self.c = torch.nn.ModuleList([torch.nn.Linear(384, 40, bias=False) for _ in range(2)])  # channel
+            self.d = torch.nn.Linear(256, 24, bias=False)                                           # g_idx
+            self.e = torch.nn.Linear(128, 16, bias=False)                                           # fp32 weight
+
+    model = Mixed().to(torch.bfloat16).to(gpu)
+    model.e.float()
+    sym = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    asym = QuantizationArgs(num_bits=4, type="int", symmetric=False, strategy="group", group_size=64)
+    chan = QuantizationArgs(num_bits=8, type="int", symmetric=True, strategy="channel")
+    config = QuantizationConfig(config_groups={
+        "sym": QuantizationScheme(targets=["re:a\\..*", "d", "e"], weights=sym),
+        "asym": QuantizationScheme(targets=["re:b\\..*"], weights=asym),
+        "chan": QuantizationScheme(targets=["re:c\\..*"], weights=chan)}, format="pack-quantized")
+    apply_quantization_scheme(model, config)
+    for name, m in model.named_modules():
+        scheme = getattr(m, "quantization_scheme", None)
+        if scheme is None:
+            continue
+        w = m.weight.data
+        g_idx = None
+        if name == "d":
+            g_idx = (torch.randperm(256, device=gpu) // 128).to(torch.int32)
+            w = w.index_select(1, torch.argsort(g_idx.long()))
+            m.register_parameter("weight_g_idx", torch.nn.Parameter(g_idx, requires_grad=False))
+        scale, zp = observe_weight_qparams(w, scheme.weights)
+        m.register_parameter("weight_scale", torch.nn.Parameter(scale, requires_grad=False))
+        m.register_parameter("weight_zero_point", torch.nn.Parameter(zp, requires_grad=False))
+    mc = ModelCompressor(quantization_config=config)
+    want = mc.compress(model)
+    dense_before = {n: p.data.clone() for n, p in model.named_parameters() if n.endswith(".weight")}
+    mc.compress_model(model)
+    got = {n: p.data for n, p in model.named_parameters()}
+    assert set(got) == set(want)
+    for name in want:
+        assert_bit_equal(got[name], want[name].to(got[name].device), name)
+    assert model.b[0].bias is not None and model.a[0].bias is None and "bias" in model.a[0]._parameters
+    # ... and back: every weight equals its per-weight decompression
+    packed = {n: p.data for n, p in model.named_parameters()}
+    mc.decompress_model(model)
+    comp = mc.quantization_compressor["pack-quantized"]
+    for name, m in model.named_modules():
+        scheme = getattr(m, "quantization_scheme", None)
+        if scheme is None:
+            continue
+        data = {k[len(name) + 1:]: v for k, v in packed.items() if k.startswith(name + ".")}
+        single = comp.decompress_weight(compressed_data=data, quantization_args=scheme.weights)
+        assert_bit_equal(m.weight.data, single.cpu(), f"{name} decompressed")
+        assert m.weight.dtype == m.weight_scale.dtype
+        assert dense_before[f"{name}.weight"].shape == m.weight.shape
