@@ -29,18 +29,23 @@ _ALIGN = 256            # ... if each of them keeps this alignment inside it
 
 class WeightJobTable:
     """Rows are added with `add`; `launch` writes them into a `ctmi_weight_job` array and
-    hands it to a many-weight entry point.  `template` registers the pointer-free part of a
-    job's qparams (as `build_qparams` made it for one weight of the combination)."""
+    hands it to a many-weight entry point.  `add_template` registers the part of a job's
+    qparams that holds no scale or zero-point address (as `build_qparams` made it for one
+    weight of the combination; its other addresses must be NULL)."""
 
     def __init__(self):
         self._templates: List[np.ndarray] = []
         self._template_of: Dict[Tuple, int] = {}
-        self.keep: list = []   # what the templates' plans keep alive (column-group tables, ...)
-        self._reset()
+        self.clear()
 
-    def _reset(self):
+    def clear(self):
+        """drop the rows added since the last launch"""
         self.src, self.dst, self.rows, self.cols, self.dense_dtype = [], [], [], [], []
         self.scale, self.zero_point, self.which = [], [], []
+
+    @property
+    def n_templates(self) -> int:
+        return len(self._templates)
 
     def template(self, key) -> int:
         """index of the template registered under `key`, or -1"""
@@ -48,9 +53,12 @@ class WeightJobTable:
 
     def add_template(self, key, plan) -> int:
         qp = np.frombuffer(bytes(plan.qp), dtype=_QP).copy()
+        if int(qp["col_group"][0]) or int(qp["global_scale"][0]):
+            raise ValueError("a template cannot hold the address of a column-group table or a global scale")
         qp["scale"] = 0
         qp["zero_point"] = 0
         self._templates.append(qp)
+        self._stacked = np.concatenate(self._templates)
         self._template_of[key] = len(self._templates) - 1
         return len(self._templates) - 1
 
@@ -79,11 +87,11 @@ class WeightJobTable:
         tab["rows"] = self.rows
         tab["cols"] = self.cols
         tab["dense_dtype"] = self.dense_dtype
-        qp = np.concatenate(self._templates)[self.which]
+        qp = self._stacked[self.which]
         qp["scale"] = self.scale
         qp["zero_point"] = self.zero_point
         tab["qp"] = qp
-        self._reset()
+        self.clear()
         # the entry points read the table before they return: it need not outlive the call
         _lib.check(entry(ctypes.cast(tab.ctypes.data, _JOB_PTR), n, stream))
 

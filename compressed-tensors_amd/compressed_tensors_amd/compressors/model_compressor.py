@@ -31,6 +31,13 @@ __all__ = ["ModelCompressor", "map_module_to_scheme", "match_named_modules",
            "apply_quantization_scheme"]
 
 
+# Modules per batch of the in-memory pathways.  The host needs somewhat less time per module
+# than the GPU: batches (multiples of the 8 weights of a launch) grow by about half from one to
+# the next, and the GPU hardly waits after the first.
+_BATCHES = (8, 16, 24, 32, 48)
+_BATCH = 64
+
+
 def _set_plain(module: Module, name: str, value) -> None:
     """module.<name> = value for a value that is no parameter, buffer or module (without the
     checks Module.__setattr__ makes for those)"""
@@ -344,82 +351,87 @@ class ModelCompressor:
         return cls(sparsity_config=sparsity_config, quantization_config=quantization_config)
 
     # ----- in-memory pathways ----- #
-    def _walk(self, model: Module):
-        """one pass over the module tree -> (named modules, map_module_to_scheme(model),
-        names of the sparsity targets)"""
-        named = list(model.named_modules())
-        module_to_scheme = {}
-        for name, module in named:
+    def _stream(self, model: Module, module_to_scheme: Dict[str, QuantizationScheme],
+                sparse_targets: Set[str], run_batch):
+        """One pass over the module tree.  Modules that are only quantized are handed to
+        `run_batch(format, members)` in batches per format - a short first batch, so that the
+        GPU starts while the rest of the tree is still being walked - and every other target
+        is yielded as (prefix, module) for the caller to treat on its own.  `module_to_scheme`
+        is filled on the way (map_module_to_scheme's entries)."""
+        pending: Dict[str, List] = {}
+        sent: Dict[str, int] = {}
+        for prefix, module in model.named_modules():
             scheme = _scheme_of(module)
             if scheme is not None and scheme.weights is not None:
-                module_to_scheme[name.replace("_fsdp_wrapped_module.", "")] = scheme
-        return named, module_to_scheme, self._sparse_targets(model)
+                module_to_scheme[prefix.replace("_fsdp_wrapped_module.", "")] = scheme
+            quantized, sparse = prefix in module_to_scheme, prefix in sparse_targets
+            if quantized and not sparse:
+                fmt = self._format_of(module)
+                batch = pending.setdefault(fmt, [])
+                batch.append((prefix, module))
+                k = sent.get(fmt, 0)
+                if len(batch) >= (_BATCHES[k] if k < len(_BATCHES) else _BATCH):
+                    sent[fmt] = k + 1
+                    run_batch(fmt, pending.pop(fmt))
+            elif quantized or sparse:
+                yield prefix, module
+        for fmt, batch in pending.items():
+            run_batch(fmt, batch)
 
     def compress_model(self, model: Module) -> None:
-        named, module_to_scheme, sparse_targets = self._walk(model)
-        # modules that are only quantized: all modules of one format go through one
-        # call of their compressor (many-weight calls of the C ABI)
-        by_format: Dict[str, List] = {}
-        for prefix, module in named:
-            if prefix not in module_to_scheme and prefix not in sparse_targets:
-                continue
-            if prefix in module_to_scheme and prefix not in sparse_targets:
-                by_format.setdefault(self._format_of(module), []).append((prefix, module))
-                continue
+        module_to_scheme: Dict[str, QuantizationScheme] = {}
+        sparse_targets = self._sparse_targets(model)
+
+        def run_batch(fmt, members):
+            # all modules of a batch in many-weight calls of the C ABI
+            self.quantization_compressor.get(fmt).compress_modules(members, module_to_scheme)
+            for _, module in members:
+                _set_plain(module, "quantization_status", QuantizationStatus.COMPRESSED)
+
+        for prefix, module in self._stream(model, module_to_scheme, sparse_targets, run_batch):
             state = self._own_parameters(module, prefix)
             stacked = {}
-            if prefix in module_to_scheme and prefix in sparse_targets:
+            if prefix in module_to_scheme:  # ... and a sparsity target
                 stacked = self._compress_quantized_24(model, state, sparse_targets, module_to_scheme)
                 state = {k: v for k, v in state.items() if k not in stacked}
-            if prefix in module_to_scheme:
                 compressor = self.quantization_compressor.get(self._format_of(module))
                 state = compressor.compress(state, names_to_scheme=module_to_scheme,
                                             show_progress=False)
-            if prefix in sparse_targets:
-                state = self.sparsity_compressor.compress(
-                    state, compression_targets=sparse_targets, show_progress=False)
+            state = self.sparsity_compressor.compress(
+                state, compression_targets=sparse_targets, show_progress=False)
             for entries in stacked.values():
                 state.update(entries)
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.COMPRESSED
-        for fmt, members in by_format.items():
-            self.quantization_compressor.get(fmt).compress_modules(members, module_to_scheme)
-            for _, module in members:
-                _set_plain(module, "quantization_status", QuantizationStatus.COMPRESSED)
         if (self.quantization_config is not None
                 and self.quantization_config.format != CompressionFormat.dense.value):
             self.quantization_config.quantization_status = QuantizationStatus.COMPRESSED.value
 
     def decompress_model(self, model: Module) -> None:
-        named, module_to_scheme, sparse_targets = self._walk(model)
-        by_format: Dict[str, List] = {}
-        for prefix, module in named:
-            if prefix not in module_to_scheme and prefix not in sparse_targets:
-                continue
-            if prefix in module_to_scheme and prefix not in sparse_targets:
-                # only quantized: decompressed below, all modules of one format from one call
-                by_format.setdefault(self._format_of(module), []).append((prefix, module))
-                continue
+        module_to_scheme: Dict[str, QuantizationScheme] = {}
+        sparse_targets = self._sparse_targets(model)
+
+        def run_batch(fmt, members):
+            self.quantization_compressor.get(fmt).decompress_modules(members, module_to_scheme)
+            for _, module in members:
+                _set_plain(module, "quantization_status", QuantizationStatus.FROZEN)
+
+        for prefix, module in self._stream(model, module_to_scheme, sparse_targets, run_batch):
             state = self._own_parameters(module, prefix)
             dense = None
-            if prefix in sparse_targets and prefix in module_to_scheme:  # both in one pass
+            if prefix in module_to_scheme:  # 2:4 decompression and dequantization in one pass
                 dense = self._decompress_quantized_24(
                     prefix, state, self.quantization_compressor.get(self._format_of(module)))
             if dense is not None:
                 state = dense
             else:
-                if prefix in sparse_targets:  # sparsity first
-                    state = dict(self.sparsity_compressor.decompress_from_state_dict(state))
+                state = dict(self.sparsity_compressor.decompress_from_state_dict(state))  # sparsity first
                 if prefix in module_to_scheme:  # quantization second
                     compressor = self.quantization_compressor.get(self._format_of(module))
                     state = compressor.decompress_module_from_state_dict(
                         prefix, state, scheme=module_to_scheme[prefix])
             self._swap_parameters(module, prefix, state)
             module.quantization_status = QuantizationStatus.FROZEN
-        for fmt, members in by_format.items():
-            self.quantization_compressor.get(fmt).decompress_modules(members, module_to_scheme)
-            for _, module in members:
-                _set_plain(module, "quantization_status", QuantizationStatus.FROZEN)
 
     # ----- helpers ----- #
     @staticmethod

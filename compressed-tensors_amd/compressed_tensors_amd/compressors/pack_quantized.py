@@ -568,22 +568,25 @@ PackedQuantizationCompressor.compress = _compress_state_dict_batched
 # Module pathways (ModelCompressor.compress_model / decompress_model): the common case - a 2-D
 # float weight on the GPU with group or channel scales, symmetric, no activation ordering - goes
 # into a job table written by columns; everything else takes the state-dict path above.
-_CHUNKS = (8, 24, 32)   # modules per call: a short first one starts the GPU early; then 64 each
+_CHUNK_MODULES = 64   # modules per call of the C ABI
 _FLOAT_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
 # what compression takes away from a module or writes anew (a symmetric scheme stores no zero points)
 _REPLACED = ("weight", "weight_zero_point", "weight_packed", "weight_shape")
 
 
 def _chunks(n):
-    at = 0
-    for size in _CHUNKS:
-        if at >= n:
-            return
-        yield at, min(at + size, n)
-        at += size
-    while at < n:
-        yield at, min(at + 64, n)
-        at += 64
+    for at in range(0, n, _CHUNK_MODULES):
+        yield at, min(at + _CHUNK_MODULES, n)
+
+
+def _module_table(self) -> WeightJobTable:
+    """the compressor's job table for the module pathways: its templates (the pointer-free
+    part of a weight's qparams per shape / dtype / scheme) stay valid from call to call"""
+    table = self.__dict__.get("_table")
+    if table is None or table.n_templates > 512:
+        table = self.__dict__["_table"] = WeightJobTable()
+    table.clear()  # rows a failed call may have left behind
+    return table
 
 
 def _args_key(args: QuantizationArgs):
@@ -594,7 +597,7 @@ def _compress_modules_fast(self, members, names_to_scheme) -> None:
     """PackedQuantizationCompressor.compress_modules: compress_module
     (compressors/base.py:125-151, pack_quantized.py:88-146) for every (prefix, module) pair"""
     entry = _lib.load().ctmi_pack_quantized_compress_many
-    table = WeightJobTable()
+    table = _module_table(self)
     new_param = torch.nn.Parameter
     slow, arg_keys = [], {}
     for lo, hi in _chunks(len(members)):
@@ -626,13 +629,12 @@ def _compress_modules_fast(self, members, names_to_scheme) -> None:
         packed = slab_outputs(shapes, torch.int32, device)
         dims = torch.tensor([(p[6], p[7]) for p in picked]).unbind(0)  # every weight_shape, one host tensor
         for (params, w, scale, zp, args, key, rows, cols), out in zip(picked, packed):
-            tkey = (rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
+            tkey = ("c", rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
             which = table.template(tkey)
             if which < 0:
                 # the zero points of a symmetric scheme (all zero) take part in the arithmetic
                 # as they are, as in the reference's compress_weight
                 plan = build_qparams(w, scale, zp, args, None, None)
-                table.keep.append(plan)
                 which = table.add_template(tkey, plan)
             table.add(w.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(w.dtype), which,
                       scale.data_ptr(), 0 if zp is None else zp.data_ptr())
@@ -652,7 +654,7 @@ def _decompress_modules_fast(self, members, names_to_scheme) -> None:
     """PackedQuantizationCompressor.decompress_modules: decompress_module
     (compressors/base.py:165-190, pack_quantized.py:147-183) for every (prefix, module) pair"""
     entry = _lib.load().ctmi_pack_quantized_decompress_many
-    table = WeightJobTable()
+    table = _module_table(self)
     new_param = torch.nn.Parameter
     slow = []
     for lo, hi in _chunks(len(members)):
@@ -682,7 +684,7 @@ def _decompress_modules_fast(self, members, names_to_scheme) -> None:
             continue
         dense = slab_outputs(shapes, dtype, device)
         for (params, packed, scale, num_bits, shape), out in zip(picked, dense):
-            tkey = (shape, scale.shape, scale.dtype, num_bits)
+            tkey = ("d", shape, scale.shape, scale.dtype, num_bits)
             which = table.template(tkey)
             if which < 0:
                 # dequantize(x_q, scale, zero_point=None, args=None): the strategy follows from
@@ -690,7 +692,6 @@ def _decompress_modules_fast(self, members, names_to_scheme) -> None:
                 carrier = _ShapeOnly(shape, torch.int8)
                 plan = build_qparams(carrier, scale, None, infer_dequant_args(carrier, scale), None, None)
                 plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_INT, num_bits
-                table.keep.append(plan)
                 which = table.add_template(tkey, plan)
             table.add(packed.data_ptr(), out.data_ptr(), shape[0], shape[1], _lib.dtype_code(scale.dtype),
                       which, scale.data_ptr())

@@ -9,6 +9,12 @@ from oracle import hadamard as oh
 pytestmark = pytest.mark.gpu
 
 
+# elements (of all 16-bit comparisons of this file) that were more than one ulp off and passed
+# on the fp32-accumulation allowance; printed by the last test
+ALLOWANCE = {"elements": 0, "leaning": 0}
+ALLOWANCE_FRACTION = 1e-3
+
+
 def _ulp(t: torch.Tensor) -> torch.Tensor:
     """spacing of t's dtype at |t| (as float64)"""
     bits = {torch.bfloat16: 8, torch.float16: 11, torch.float32: 24}[t.dtype]
@@ -29,6 +35,13 @@ def _assert_within_ulp(got, exact, what, ulps=1.0):
         # (2^-21 of the row's scale): it only shows where cancellation leaves an output
         # thousands of times smaller than its terms, e.g. in float16's subnormal range
         tol = ulps * _ulp(exact) + 2.0 ** -21 * exact.double().abs().amax(-1, keepdim=True)
+        # how many elements lean on that second term: outputs next to a rounding boundary or far
+        # below the row's scale.  It stays a small fraction (ALLOWANCE_FRACTION) of the tensor.
+        leaning = int((err > ulps * _ulp(exact)).sum())
+        ALLOWANCE["elements"] += err.numel()
+        ALLOWANCE["leaning"] += leaning
+        assert leaning <= max(2, ALLOWANCE_FRACTION * err.numel()), \
+            f"{what}: {leaning} of {err.numel()} elements are more than {ulps} ulp off (within the accumulation allowance)"
     bad = err > tol
     assert not bool(bad.any()), f"{what}: {int(bad.sum())} elements off by more than {ulps} ulp; max ratio {(err / tol).max():.2f}"
 
@@ -560,3 +573,12 @@ def test_block_times_sylvester64_with_butterflies(k, dtype, inner, ctmi, gpu, ha
     rc = ctmi.ctmi_hadamard_apply(xg.data_ptr(), xg.data_ptr(), code, xg.numel(), k, inner, ma_t.data_ptr(), None,
                                   sg.data_ptr(), sg.data_ptr(), _lib.stream_of(gpu))
     assert rc == _lib.CTMI_ERR_UNSUPPORTED
+
+
+def test_zz_report_elements_beyond_one_ulp():
+    """runs last in this file: the share of compared 16-bit outputs that differed from the
+    fp64 result by more than one ulp of the output dtype (and passed on the allowance for
+    fp32 accumulation, 2^-21 of the row's largest magnitude)"""
+    n, k = ALLOWANCE["elements"], ALLOWANCE["leaning"]
+    print(f"[hadamard] {k} of {n} compared 16-bit elements were more than 1 ulp off ({k / max(n, 1):.2e})", flush=True)
+    assert k <= 1e-4 * max(n, 1)

@@ -591,6 +591,50 @@ def test_stacked_round_trip_at_full_size(gpu):
     assert_bit_equal(again[0], values, "values of the round trip")
 
 
+def test_stacked_2_4_of_fp8_at_full_size_against_the_oracle(gpu):
+    """the same 14336 x 4096 weight against the oracle's op chain - quantize (fp8, one scale per
+    output channel), then sparse24_bitmask_compress of the codes (sparse_24_bitmask.py:162-224 on
+    what quantized_compressors/base.py:91-125 produced) and the way back - on row slices at the
+    head, in the middle and at the tail: the one-pass kernels, and the two steps one after the
+    other"""
+    from compressed_tensors_amd.compressors import (
+        get_24_bytemasks, quantize_sparse24_compress, sparse24_bitmask_compress,
+        sparse24_bitmask_decompress, sparse24_decompress_dequantize,
+    )
+    from compressed_tensors_amd.quantization import QuantizationArgs, observe_weight_qparams, quantize
+
+    announce("quantize + 2:4 vs oracle, 14336 x 4096")
+    spec = dict(num_bits=8, type="float", symmetric=True, strategy="channel")
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    g = torch.Generator(device=gpu).manual_seed(11)
+    w = torch.randn(14336, 4096, generator=g, device=gpu) * 0.02
+    # every survivor large enough to keep a non-zero code: which of several zero codes of a
+    # group topk keeps is torch's tie order on the CPU, and not what this test is about
+    w = torch.where(w.abs() < 1e-3, torch.full_like(w, 1e-3), w).bfloat16()
+    w = torch.where(get_24_bytemasks(w), w, torch.zeros_like(w))
+    scale, _ = observe_weight_qparams(w, args)
+    fused_values, fused_bitmask = quantize_sparse24_compress(w, scale, args)
+    codes = quantize(w, scale, None, args, dtype=torch.float8_e4m3fn)
+    values, bitmask = sparse24_bitmask_compress(codes)
+    dense = sparse24_bitmask_decompress(values, bitmask, codes.shape)
+    back = sparse24_decompress_dequantize(fused_values, fused_bitmask, w.shape, scale)
+    rows = w.shape[0]
+    for sl in (slice(0, 48), slice(rows // 2 - 7, rows // 2 + 41), slice(rows - 48, rows)):
+        wc = w[sl].cpu()
+        o_scale, _ = oq.observe_weight(wc, oargs)
+        assert_bit_equal(scale[sl], o_scale, f"scales {sl}")
+        o_codes = oq.quantize(wc, o_scale, None, oargs, dtype=torch.float8_e4m3fn)
+        o_values, o_bitmask = osp.sparse24_bitmask_compress(o_codes)
+        assert_bit_equal(codes[sl], o_codes, f"codes {sl}")
+        assert_bit_equal(values[sl], o_values, f"values, two steps {sl}")
+        assert_bit_equal(bitmask[sl], o_bitmask, f"bitmask, two steps {sl}")
+        assert_bit_equal(fused_values[sl], o_values, f"values, one pass {sl}")
+        assert_bit_equal(fused_bitmask[sl], o_bitmask, f"bitmask, one pass {sl}")
+        o_dense = osp.sparse24_bitmask_decompress(o_values, o_bitmask, o_codes.shape)
+        assert_bit_equal(dense[sl], o_dense, f"decompressed codes {sl}")
+        assert_bit_equal(back[sl], oq.dequantize(o_dense, o_scale), f"decompressed + dequantized {sl}")
+
+
 # ---------------------------------------------------------------- several 2:4 tensors per call
 
 
