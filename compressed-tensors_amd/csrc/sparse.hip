@@ -14,6 +14,7 @@
 #include <cstddef>
 #include <mutex>
 #include <type_traits>
+#include <unordered_map>
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
@@ -697,9 +698,10 @@ tile_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
 // The same count for tensors of up to kGroupTiles * kMaxGroups tiles, without the
 // scan kernel in between: a workgroup counts a group of kGroupTiles neighbouring
 // tiles and leaves, per tile, the count of the group's earlier tiles and its own, and
-// per group its total; the workgroup that finishes last (a ticket drawn with an
-// atomic, no waiting) turns the totals into the set bits before each group.  A
-// scatter workgroup then finds its place with two scalar loads.
+// per group its total.  A scatter workgroup adds up the totals of the groups before
+// its own (at most kMaxGroups numbers, resident in L2) and finds its place.  Nothing
+// is handed from one workgroup to another inside a launch: the end of the count
+// kernel is what makes its stores visible, and the library keeps no state of its own.
 constexpr int kGroupTiles = 64;
 constexpr int kGroupThreads = 1024;
 constexpr int kMaxGroups = 1024;
@@ -708,30 +710,14 @@ struct TileInfo {
   int32_t count;   // set bits in the tile
 };
 
-// Which workgroup of the count is the last to finish: kTicketSlots counters in device
-// memory of the library, zero between launches (the last workgroup puts its counter
-// back).  Launches take them in turn, so launches in flight at the same time (other
-// streams) do not share one unless there are kTicketSlots of them.
-constexpr int kTicketSlots = 256;
-__device__ unsigned int popcount_ticket[kTicketSlots];
-
-static uint32_t next_ticket_slot() {
-  static std::atomic<uint32_t> ticket{0};
-  return ticket.fetch_add(1, std::memory_order_relaxed) % kTicketSlots;
-}
-
-static_assert(kGroupThreads >= kMaxGroups, "the last workgroup scans one group total per thread");
-
 __global__ void __launch_bounds__(kGroupThreads)
 tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
                             TileInfo* __restrict__ info, int32_t* __restrict__ group_total,
-                            int32_t* __restrict__ group_before, int64_t ntiles, uint32_t slot) {
+                            int64_t ntiles) {
   constexpr int kPerWave = kGroupTiles / (kGroupThreads / kWave);  // tiles per wavefront
   static_assert(kPerWave == 4 && kTileBytes == 32 * 16,
                 "a wavefront reads two tiles per load, half a wavefront each");
   __shared__ int cnt_s[kGroupTiles];
-  __shared__ int wsum_s[kGroupThreads / kWave];
-  __shared__ int last_s;
   const int lane = lane_id(), wave = threadIdx.x / kWave;
   const int64_t tile0 = (int64_t)blockIdx.x * kGroupTiles;
   // The wavefront's four tiles are 2 KB in a row: two 16-byte loads per lane, both
@@ -771,39 +757,12 @@ tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
     const int c = cnt_s[lane];
     const int inc = wave_inclusive_scan(c);
     if (tile0 + lane < ntiles) info[tile0 + lane] = TileInfo{inc - c, c};
-    if (lane == kWave - 1) {
-      // The total goes out where every workgroup of the device reads it (a device-scope
-      // atomic store), the lane waits until it has arrived, then draws its ticket:
-      // whoever draws the last one finds every total in place.  A release fence
-      // would order the two as well, but it writes the whole L2 back, in every
-      // workgroup, and doubled the time of this pass.
-      __hip_atomic_store(&group_total[blockIdx.x], inc, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      const unsigned int drawn = __hip_atomic_fetch_add(&popcount_ticket[slot], 1u, __ATOMIC_RELAXED,
-                                                        __HIP_MEMORY_SCOPE_AGENT);
-      last_s = drawn == gridDim.x - 1;
-    }
+    if (lane == kWave - 1) group_total[blockIdx.x] = inc;
   }
-  __syncthreads();
-  if (!last_s) return;
-  // the last workgroup: set bits before each group, one group per thread
-  const int g = threadIdx.x;
-  const int t = g < (int)gridDim.x
-                    ? __hip_atomic_load(&group_total[g], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                    : 0;
-  const int inc = wave_inclusive_scan(t);
-  if (lane == kWave - 1) wsum_s[wave] = inc;
-  __syncthreads();
-  int before = inc - t;
-#pragma unroll
-  for (int w = 0; w < kGroupThreads / kWave; ++w) before += w < wave ? wsum_s[w] : 0;
-  if (g < (int)gridDim.x) group_before[g] = before;
-  if (threadIdx.x == 0)
-    __hip_atomic_store(&popcount_ticket[slot], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Set bits beyond nvalues read as zero.  GROUPED: positions from
-// tile_popcount_groups_kernel (info, group_before), else from tile_popcount_kernel
+// tile_popcount_groups_kernel (info, group_total), else from tile_popcount_kernel
 // and the scan behind it (tile_counts, tile_offsets).
 //
 // A wavefront takes 1024 neighbouring elements of the tile, as 16-byte pieces: piece q
@@ -818,7 +777,7 @@ bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
                              const int64_t* __restrict__ tile_counts,
                              const int64_t* __restrict__ tile_offsets,
                              const TileInfo* __restrict__ info,
-                             const int32_t* __restrict__ group_before, R* __restrict__ out,
+                             const int32_t* __restrict__ group_total, R* __restrict__ out,
                              int64_t numel) {
   constexpr int VE = 16 / (int)sizeof(R);  // elements of a piece
   constexpr int NP = 16 / VE;              // pieces of a lane
@@ -833,8 +792,24 @@ bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
   int64_t excl;
   int total;
   if constexpr (GROUPED) {
+    // set bits before the tile's group: every wavefront adds the totals of the earlier
+    // groups up by itself (no more than kMaxGroups / kWave loads a lane, all in flight
+    // together, and no barrier)
+    const int group = (int)(tile / kGroupTiles);
+    int part[kMaxGroups / kWave];
+#pragma unroll
+    for (int k = 0; k < kMaxGroups / kWave; ++k) {
+      const int g = k * kWave + lane;
+      part[k] = (k * kWave < group && g < group) ? group_total[g] : 0;
+    }
+    // (a tensor on this path has at most kMaxGroups * kGroupTiles * kTileElems = 2^28 elements)
+    int sum = 0;
+#pragma unroll
+    for (int k = 0; k < kMaxGroups / kWave; ++k) sum += part[k];
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) sum += __shfl_xor(sum, d, kWave);
     const TileInfo ti = info[tile];
-    excl = (int64_t)group_before[tile / kGroupTiles] + ti.before;
+    excl = (int64_t)sum + ti.before;
     total = ti.count;
   } else {
     excl = tile_offsets[tile];
@@ -955,15 +930,26 @@ bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
 //
 // The words: kS24Slots pairs {jobs with a bad group, repair workgroups done} in
 // device memory of the library, all zero between launches (a repair that found
-// something puts its pair back to zero when its last workgroup is done).  Launches
-// take the pairs in turn, so launches in flight at the same time (other streams) do
-// not share one unless there are kS24Slots of them.
+// something puts its pair back to zero when its last workgroup is done).  A pair
+// belongs to a launch from the start of its streaming kernel to the end of its repair
+// kernel.  Launches on one stream run one after the other, so a stream keeps one pair
+// for all its launches; every stream gets a pair of its own until kS24Slots streams
+// have been seen, and only then do streams share (two launches that share a pair and
+// overlap in time could take each other's verdict).
 constexpr int kS24Slots = 256;
 __device__ unsigned int s24_slot_state[kS24Slots][2];
 
-static uint32_t next_s24_slot() {
-  static std::atomic<uint32_t> ticket{0};
-  return ticket.fetch_add(1, std::memory_order_relaxed) % kS24Slots;
+static uint32_t s24_slot_of(hipStream_t st) {
+  static std::mutex m;
+  static std::unordered_map<hipStream_t, uint32_t> slots;
+  static uint32_t next = 0;
+  std::lock_guard<std::mutex> lock(m);
+  auto it = slots.find(st);
+  if (it != slots.end()) return it->second;
+  if (slots.size() >= (1u << 16)) slots.clear();  // handles of streams long gone
+  const uint32_t slot = next++ % kS24Slots;
+  slots.emplace(st, slot);
+  return slot;
 }
 
 // called by every thread of a streaming workgroup: `bad` goes up for job `job`
@@ -1772,7 +1758,7 @@ static void s24_launch(const S24Job* jobs, int n, int32_t elem_size, hipStream_t
       t.chunk_end[k] = 0xFFFFFFFFu;
     }
   }
-  t.slot = next_s24_slot();
+  t.slot = s24_slot_of(st);
 #define CTMI_24(R)                                                                \
   hipLaunchKernelGGL(sparse24_scatter_kernel<R>, total, kBlock, 0, st, t);        \
   hipLaunchKernelGGL(sparse24_repair_kernel<R>, kS24RepairGrid, kBlock, 0, st, t)
@@ -1812,10 +1798,9 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
     const bool grouped = ngroups <= kMaxGroups;
     if (grouped) {
       info = (TileInfo*)tmp;
-      int32_t* group_totals = (int32_t*)(info + ntiles);
-      totals = group_totals + ngroups;  // set bits before each group
+      totals = (int32_t*)(info + ntiles);  // set bits of each group
       hipLaunchKernelGGL(tile_popcount_groups_kernel, (unsigned)ngroups, kGroupThreads, 0, st,
-                         bitmask, rows * pc, info, group_totals, totals, ntiles, next_ticket_slot());
+                         bitmask, rows * pc, info, totals, ntiles);
     } else {
       counts = (int64_t*)tmp;
       offs = counts + ntiles;
@@ -2227,7 +2212,7 @@ extern "C" int ctmi_sparse24_decompress_dequantize(const void* values, int64_t n
   const unsigned grid = (unsigned)cdiv(items, kBlock * kS24DqU);
   hipStream_t st = (hipStream_t)stream;
   const uint8_t* zp = (const uint8_t*)qp->zero_point;
-  const uint32_t slot = next_s24_slot();
+  const uint32_t slot = s24_slot_of(st);
 #define CTMI_S24DQ_K(FT, RAW, QK, HZ)                                                             \
   hipLaunchKernelGGL((sparse24_scatter_dequant_kernel<FT, QK, HZ>), grid, kBlock, 0, st,          \
                      (const uint8_t*)values, bitmask, (const RAW*)qp->scale, zp, (RAW*)out, items, \

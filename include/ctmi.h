@@ -233,7 +233,9 @@ int ctmi_bitmask_decompress(const void* values, int64_t nvalues, int32_t elem_si
  * Positions come from the bitmask alone (the `tmp` mode of
  * ctmi_bitmask_decompress); same bits.  All calls on one GPU share that GPU's
  * array: calls that overlap on one GPU (two streams, two threads) race; calls
- * enqueued on one stream do not, and nothing needs clearing between them. */
+ * enqueued on one stream do not, and nothing needs clearing between them.  The first
+ * call on a GPU looks up the array's device address (hipGetSymbolAddress): it must be
+ * made outside stream capture; later calls may be captured. */
 int64_t ctmi_bitmask_decompress_static_max_bytes(void);
 int ctmi_bitmask_decompress_static(const void* values, int64_t nvalues, int32_t elem_size,
                                    const uint8_t* bitmask, void* out, int64_t rows, int64_t cols,
@@ -248,7 +250,10 @@ int ctmi_bitmask_decompress_static(const void* values, int64_t nvalues, int32_t 
  * as a general scatter.  Other shapes (values that are not half the elements,
  * rows that are not whole bitmask bytes) take the path of ctmi_bitmask_decompress
  * and use tmp: ctmi_sparse24_tmp_bytes(rows, cols, elem_size) bytes of device
- * scratch; it needs no initialisation. */
+ * scratch; it needs no initialisation.
+ * The word the streaming workgroups report to is one of 256 pairs of words in device
+ * memory of the library; each stream is given a pair of its own when it is first seen
+ * (streams beyond 256 share).  A captured graph keeps the pair of its capture stream. */
 int64_t ctmi_sparse24_tmp_bytes(int64_t rows, int64_t cols, int32_t elem_size);
 int ctmi_sparse24_decompress(const void* values, int64_t nvalues, int32_t elem_size,
                              const uint8_t* bitmask, void* out, void* tmp, int64_t rows,

@@ -728,3 +728,38 @@ def test_sparse24_compressor_state_dict_in_few_calls(gpu):
         want = w if not name.endswith(".weight") else osp.sparse24_bitmask_decompress(
             *osp.sparse24_bitmask_compress(w.cpu()), tuple(w.shape))
         assert_bit_equal(back[name], want, name)
+
+
+def test_sparse24_decompress_many_launches_back_to_back(gpu):
+    """more launches than the library holds verdict words for (256 pairs, one per stream),
+    enqueued without a wait in between, on one stream and spread over three: every result
+    against the oracle.  Every 50th tensor has a bitmask that is not 2:4, so the repair path
+    runs in between and has to leave its words at zero for the launches behind it."""
+    from compressed_tensors_amd.compressors import sparse24_bitmask_compress, sparse24_bitmask_decompress
+    from compressed_tensors_amd.utils.helpers import pack_bitmasks
+
+    announce("sparse24 decompress x 600")
+    g = torch.Generator().manual_seed(77)
+    rows, cols = 64, 512
+    cases = []
+    for k in range(12):
+        x = _prune24(torch.randn(rows, cols, generator=g)).bfloat16()
+        v, b = osp.sparse24_bitmask_compress(x)
+        cases.append((v.to(gpu), b.to(gpu), osp.sparse24_bitmask_decompress(v, b, (rows, cols))))
+    keep = torch.zeros(rows, cols, dtype=torch.bool)
+    keep.scatter_(1, torch.rand(rows, cols, generator=g).argsort(dim=1)[:, : cols // 2], True)
+    odd = torch.randn(rows, cols, generator=g).bfloat16()
+    odd[odd == 0] = 1.0
+    odd = torch.where(keep, odd, torch.zeros_like(odd))
+    malformed = (odd[keep].reshape(rows, cols // 2).to(gpu), pack_bitmasks(keep.to(gpu)), odd)
+    streams = [torch.cuda.current_stream(gpu)] + [torch.cuda.Stream(gpu) for _ in range(2)]
+    torch.cuda.synchronize()
+    for which in ([0] * 600, [i % 3 for i in range(600)]):
+        outs = []
+        for i, s in enumerate(which):
+            v, b, want = malformed if i % 50 == 49 else cases[i % len(cases)]
+            with torch.cuda.stream(streams[s]):
+                outs.append((sparse24_bitmask_decompress(v, b, torch.Size((rows, cols))), want))
+        torch.cuda.synchronize()
+        for i, (got, want) in enumerate(outs):
+            assert_bit_equal(got, want, f"launch {i} of {len(which)} on {len(set(which))} stream(s)")
