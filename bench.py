@@ -543,13 +543,14 @@ def other_workload(torch, name, seed):
     if name == "one-shot":
         # the Llama-3-8B-shaped set, no scales yet: observer + qparams + quantize + pack
         args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
-        sep_obs, sep_cmp, fused, job_fields, n = [], [], [], [], 0
+        sep_obs, sep_cmp, fused, job_fields, n, keep2 = [], [], [], [], 0, []
         for _, r, c in shapes_for("llama3-8b-w4a16"):
             w = randn(r, c, 0.02)
             scale, zp = observe_weight_qparams(w, args)
             packed = torch.empty(r, c // 8, dtype=torch.int32, device=dev)
             plan = build_qparams(w, scale, None, args, None, None)
             keep.extend([w, scale, zp, packed, plan])
+            keep2.append((w, scale, packed))
             sep_obs.append(observe(w, GROUP, args, scale, zp))
             ca = (w.data_ptr(), code(w.dtype), packed.data_ptr(), r, c, ctypes.byref(plan.qp), st)
             sep_cmp.append(lambda ca=ca: _lib.check(lib.ctmi_pack_quantized_compress(*ca)))
@@ -564,11 +565,34 @@ def other_workload(torch, name, seed):
              j.num_bits, j.symmetric) = f
         keep.append(jobs)
         many = [lambda: _lib.check(lib.ctmi_observe_pack_quantized_many(jobs, len(job_fields), st))]
+        # the same set with activation ordering (one random g_idx per row length): the group of
+        # a column is looked up, min / max meet in LDS
+        from compressed_tensors_amd.quantization.forward import _column_groups
+        col_groups, gidx_one, gidx_cmp = {}, [], []
+        for (w, scale, packed) in list(keep2):
+            r, c = w.shape
+            if c not in col_groups:
+                perm = torch.randperm(c, generator=torch.Generator().manual_seed(seed + c)).to(dev)
+                col_groups[c] = ((perm // GROUP).to(torch.int32), _column_groups((perm // GROUP).to(torch.int32), GROUP))
+            g_idx, cg = col_groups[c]
+            ga = (w.data_ptr(), code(w.dtype), r, c, GROUP, 4, 1, cg.data_ptr(), packed.data_ptr(),
+                  scale.data_ptr(), None, st)
+            gidx_one.append(lambda ga=ga: _lib.check(lib.ctmi_observe_pack_quantized_gidx(*ga)))
+            gplan = build_qparams(w, scale, None, args, g_idx, None)
+            keep2.append(gplan)
+            gc = (w.data_ptr(), code(w.dtype), packed.data_ptr(), r, c, ctypes.byref(gplan.qp), st)
+            gidx_cmp.append(lambda gc=gc: _lib.check(lib.ctmi_pack_quantized_compress(*gc)))
+        keep.extend(keep2)
+        keep.append(col_groups)
         g = n // GROUP
         ops = [Op("observer + qparams, group 128 (224 tensors, one call each)", sep_obs, 2 * n + 3 * g, "observe_flat_kernel", primary=False),
                Op("quantize + pack with those scales (one call each)", sep_cmp, 2 * n + 2 * g + n // 2, "pq_compress_vec_kernel", primary=False),
                Op("observer + qparams + quantize + pack in one pass (one call each)", fused, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel", primary=False),
-               Op("the same, all 224 tensors in one call (8 per launch)", many, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel", launches=chained(len(job_fields)))]
+               Op("the same, all 224 tensors in one call (8 per launch)", many, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel", launches=chained(len(job_fields))),
+               Op("activation ordering (g_idx): quantize + pack with given scales, the second of two passes (one call each)",
+                  gidx_cmp, 2 * n + 2 * g + n // 2, "pq_gidx_compress_kernel", primary=False),
+               Op("activation ordering (g_idx): observer + qparams + quantize + pack in one pass (one call each)",
+                  gidx_one, 2 * n + 2 * g + n // 2, "observe_pack_table_kernel", primary=False)]
         return "one-shot W4A16 g128 compression GB/s (no scales given), Llama-3-8B-shaped weights", ops, keep
 
     if name == "hadamard":

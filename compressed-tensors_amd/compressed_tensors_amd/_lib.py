@@ -301,6 +301,14 @@ SIGNATURES = {
         [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p,
          c_void_p, c_void_p],
     ),
+    "ctmi_observe_pack_quantized_gidx_supported": (
+        c_int32, [c_int32, c_int64, c_int64, c_int64, c_int32],
+    ),
+    "ctmi_observe_pack_quantized_gidx": (
+        c_int32,
+        [c_void_p, c_int32, c_int64, c_int64, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p,
+         c_void_p, c_void_p],
+    ),
     "ctmi_mxfp4_round_to_power_2": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "ctmi_mxfp4_generate_scales": (c_int32, [c_void_p, c_void_p, c_int64, c_void_p]),
     "ctmi_mxfp4_convert_exp_scale": (c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_void_p]),

@@ -22,6 +22,7 @@ from compressed_tensors_amd.compressors.quantized_base import (
 from compressed_tensors_amd.config import CompressionFormat
 from compressed_tensors_amd.quantization.forward import (
     _ShapeOnly,
+    _column_groups,
     build_qparams,
     infer_dequant_args,
 )
@@ -172,6 +173,33 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
             out["weight_zero_point"] = pack_to_int32(zero_point, args.num_bits, packed_dim=0)
         return out
 
+    @staticmethod
+    def one_pass_kernel(weight: Tensor, args: QuantizationArgs, g_idx: Optional[Tensor] = None):
+        """which kernel compresses a weight without scales in one pass: "groups" (groups are
+        runs of neighbouring lanes: column order, 8 ... 512 elements, a power of two; or one
+        cell per row), "table" (the group of a column looked up or divided out: activation
+        ordering, any group size) or None (the observer and the compressor run one after
+        the other)"""
+        if weight.ndim != 2 or args.type != "int" or not can_quantize(weight, args):
+            return None
+        rows, cols = weight.shape
+        if args.strategy == QuantizationStrategy.GROUP.value:
+            blk_cols = args.group_size
+        elif args.strategy == QuantizationStrategy.CHANNEL.value:
+            blk_cols, g_idx = cols, None
+        else:
+            return None
+        if weight.data_ptr() % (8 * weight.element_size()) or weight.dtype not in _FLOAT_DTYPES:
+            return None
+        lib, code = _lib.load(), _lib.dtype_code(weight.dtype)
+        if g_idx is None and lib.ctmi_observe_pack_quantized_supported(code, rows, cols, blk_cols, args.num_bits):
+            return "groups"
+        if g_idx is not None and g_idx.numel() >= 1 << 16:
+            return None
+        if lib.ctmi_observe_pack_quantized_gidx_supported(code, rows, cols, min(blk_cols, cols), args.num_bits):
+            return "table"
+        return None
+
     def observe_and_compress_weight(
         self, weight: Tensor, quantization_args: QuantizationArgs,
         device: Optional[torch.device] = None, g_idx: Optional[Tensor] = None,
@@ -180,9 +208,10 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         the min-max observer (tests/mock_observer.py:38-113), calculate_qparams
         (quantization/utils/helpers.py:67-146) and compress_weight
         (pack_quantized.py:88-146) in one pass over the weight for group and channel
-        strategies; the other strategies (one scale per tensor, blocks) and activation
-        ordering run the observer and the compressor one after the other.  With g_idx the
-        observer sees the columns in the order quantize groups them (sorted by g_idx,
+        strategies, with or without activation ordering (`one_pass_kernel` says which kernel
+        takes a weight); the other strategies (one scale per tensor, blocks) and rows beyond
+        16384 elements run the observer and the compressor one after the other.  With g_idx
+        the observer sees the columns in the order quantize groups them (sorted by g_idx,
         forward.py:286-303).  Returns compress_weight's dict plus "weight_scale" (and the
         packed "weight_zero_point" of an asymmetric scheme)."""
         args = quantization_args
@@ -198,13 +227,8 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
             blk_cols = 0
         lib = _lib.load()
         w = weight.contiguous()
-        fused = (
-            g_idx is None and blk_cols > 0 and args.type == "int" and can_quantize(weight, args)
-            and w.data_ptr() % (8 * w.element_size()) == 0
-            and lib.ctmi_observe_pack_quantized_supported(
-                _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits)
-        )
-        if not fused:
+        kernel = self.one_pass_kernel(w, args, g_idx)
+        if kernel is None:
             from compressed_tensors_amd.quantization.helpers import observe_weight_qparams
 
             seen = weight
@@ -221,13 +245,27 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         zero_point = None
         if not args.symmetric:
             zero_point = torch.empty((rows, n_cells), dtype=torch.int8, device=w.device)
-        _lib.check(
-            lib.ctmi_observe_pack_quantized(
-                w.data_ptr(), _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits,
-                int(args.symmetric), packed.data_ptr(), scale.data_ptr(), _lib.ptr(zero_point),
-                _lib.stream_of(w.device),
+        if kernel == "groups":
+            _lib.check(
+                lib.ctmi_observe_pack_quantized(
+                    w.data_ptr(), _lib.dtype_code(w.dtype), rows, cols, blk_cols, args.num_bits,
+                    int(args.symmetric), packed.data_ptr(), scale.data_ptr(), _lib.ptr(zero_point),
+                    _lib.stream_of(w.device),
+                )
             )
-        )
+        else:
+            # groups that are no runs of neighbouring lanes: the group of every column from a
+            # table (activation ordering) or by division (any group size)
+            col_group = None
+            if g_idx is not None and args.strategy == QuantizationStrategy.GROUP.value:
+                col_group = _column_groups(to_gpu(g_idx), args.group_size)
+            _lib.check(
+                lib.ctmi_observe_pack_quantized_gidx(
+                    w.data_ptr(), _lib.dtype_code(w.dtype), rows, cols, min(blk_cols, cols), args.num_bits,
+                    int(args.symmetric), _lib.ptr(col_group), packed.data_ptr(), scale.data_ptr(),
+                    _lib.ptr(zero_point), _lib.stream_of(w.device),
+                )
+            )
         out = {"weight_shape": torch.tensor(weight.shape), "weight_packed": packed,
                "weight_scale": scale}
         if zero_point is not None:

@@ -30,60 +30,6 @@ struct GidxTable {
 static_assert(offsetof(GidxTable, chunk_end) == 0 && offsetof(GidxTable, job) == 64,
               "find_job_index reads the first 16 dwords of the kernel argument");
 
-// quantize + pack 8 elements, every element with its own scale / zero point: the
-// reference chain with one IEEE division per element
-template <typename XT, typename ST, int BITS, bool HAS_ZP>
-__device__ __forceinline__ Vec<int32_t, BITS / 4> quant_pack8_each_exact(
-    const Vec<typename XT::raw, 8>& xv, const float* s, const float* z, float qmin, float qmax) {
-  constexpr int W = BITS / 4;
-  constexpr int PF = 32 / BITS;
-  constexpr int OFF = 1 << (BITS - 1);
-  constexpr int CT = (XT::id == ST::id) ? XT::id : CTMI_F32;
-  Vec<int32_t, W> o;
-#pragma unroll
-  for (int w = 0; w < W; ++w) {
-    uint32_t acc = 0;
-#pragma unroll
-    for (int i = 0; i < PF; ++i) {
-      const int e = w * PF + i;
-      float t = round_ct<CT>(XT::to_f32(xv.v[e]) / s[e]);
-      if (HAS_ZP) t = round_ct<CT>(t + z[e]);
-      t = rintf(clamp_nan(t, qmin, qmax));
-      acc |= ((uint32_t)(f32_to_int(t) + OFF) & ((1u << BITS) - 1u)) << (BITS * i);
-    }
-    o.v[w] = (int32_t)acc;
-  }
-  return o;
-}
-
-// bf16 input, bf16 scales of ordinary magnitude: products with the staged
-// reciprocals (they round to the same bf16 as the quotients), hardware bf16
-// conversions, integer rounding and packing by the magic-number addition
-template <int BITS, bool HAS_ZP>
-__device__ __forceinline__ Vec<int32_t, BITS / 4> quant_pack8_each_bf16(
-    const Vec<uint16_t, 8>& xv, const float* r, const float* z, float qmin, float qmax) {
-  using PC = PackConst<BITS>;
-  constexpr int W = BITS / 4;
-  const Vec<uint32_t, 4> xw = __builtin_bit_cast(Vec<uint32_t, 4>, xv);
-  uint32_t acc[W];
-#pragma unroll
-  for (int w = 0; w < W; ++w) acc[w] = 0u - PC::bias();
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int e0 = 2 * j, e1 = 2 * j + 1;
-    uint32_t t = pack_bf16x2(bf16_lo(xw.v[j]) * r[e0], bf16_hi(xw.v[j]) * r[e1]);
-    if (HAS_ZP) t = pack_bf16x2(bf16_lo(t) + z[e0], bf16_hi(t) + z[e1]);
-    const float c0 = __builtin_amdgcn_fmed3f(bf16_lo(t), qmin, qmax) + PC::MAGIC;
-    const float c1 = __builtin_amdgcn_fmed3f(bf16_hi(t), qmin, qmax) + PC::MAGIC;
-    acc[e0 / PC::PF] += f2u(c0) << (BITS * (e0 % PC::PF));
-    acc[e1 / PC::PF] += f2u(c1) << (BITS * (e1 % PC::PF));
-  }
-  Vec<int32_t, W> o;
-#pragma unroll
-  for (int w = 0; w < W; ++w) o.v[w] = (int32_t)acc[w];
-  return o;
-}
-
 // unpack + dequantize 8 elements: (q - zp) is an integer of at most 8 bits, exact in
 // every float type here, so the reference's chain rounds once, in the product
 template <typename ST, int BITS, bool HAS_ZP>

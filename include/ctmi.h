@@ -394,6 +394,25 @@ int ctmi_observe_pack_quantized(const void* x, int32_t x_dtype, int64_t rows, in
                                 int64_t blk_cols, int32_t num_bits, int32_t symmetric,
                                 int32_t* packed, void* scale, int8_t* zero_point, void* stream);
 
+/* The same pass for weights whose groups are not runs of neighbouring columns of a
+ * power-of-two length: activation ordering (quantization/lifecycle/forward.py:286-303: the
+ * columns are sorted by g_idx and the sorted order is cut into groups, so the observer
+ * (tests/mock_observer.py:38-113 on the sorted columns) takes min / max over the columns of a
+ * group wherever they sit) and column-ordered groups of any size that divides cols.
+ * col_group: int32 [cols], the group of every column (ctmi_column_groups turns a g_idx into
+ * it), or NULL for column / blk_cols.  scale: [rows, cols / blk_cols] in x_dtype; zero_point:
+ * optional int8 of the same shape; packed: int32 [rows, cols * num_bits / 32].  Same bits as
+ * the min-max observer on the weight with its columns sorted by col_group, followed by
+ * ctmi_pack_quantized_compress with qp.col_group set.
+ * _supported(): cols a multiple of 8 and of blk_cols, at most 16384; at most 256 groups a row;
+ * 4- or 8-bit codes. */
+int ctmi_observe_pack_quantized_gidx_supported(int32_t x_dtype, int64_t rows, int64_t cols,
+                                               int64_t blk_cols, int32_t num_bits);
+int ctmi_observe_pack_quantized_gidx(const void* x, int32_t x_dtype, int64_t rows, int64_t cols,
+                                     int64_t blk_cols, int32_t num_bits, int32_t symmetric,
+                                     const int32_t* col_group, int32_t* packed, void* scale,
+                                     int8_t* zero_point, void* stream);
+
 /* The same for the nvfp4 format with a known global scale: group-16 scales of the
  * observer (tests/mock_observer.py:38-113, helpers.py:101-120: fp8 e4m3, zeros
  * replaced by 0.125) and NVFP4PackedCompressor.compress_weight

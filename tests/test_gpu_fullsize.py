@@ -135,6 +135,32 @@ def test_headline_batch_of_224_weights(gpu):
     check(whole, slice(0, 4096))
 
 
+@pytest.mark.parametrize("shape", [(14336, 4096), (4096, 14336)], ids=["14336x4096", "4096x14336"])
+def test_one_pass_with_activation_ordering_at_full_size(shape, gpu):
+    """W4A16 g128 with a random g_idx on the two largest shapes of the set (every workgroup of
+    the one-pass kernel takes several row blocks): scales and packed words against the oracle's
+    observer on the columns sorted by g_idx and its compressor, on row slices"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.quantization import QuantizationArgs
+
+    announce("one-pass act-order", shape)
+    spec = dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    g = torch.Generator(device=gpu).manual_seed(5)
+    w = (torch.randn(shape, generator=g, device=gpu) * 0.02).bfloat16()
+    g_idx = (torch.randperm(shape[1], generator=torch.Generator().manual_seed(6)) // 128).to(torch.int32)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    assert comp.one_pass_kernel(w, args, g_idx.to(gpu)) == "table"
+    got = comp.observe_and_compress_weight(w, args, g_idx=g_idx.to(gpu))
+    order = torch.argsort(g_idx.long(), stable=True)
+    for sl in _slices(shape[0]):
+        wc = w[sl].cpu()
+        o_scale, o_zp = oq.observe_weight(wc.index_select(1, order), oargs)
+        want = op.pack_quantized_compress(wc, o_scale, oargs, zero_point=o_zp, g_idx=g_idx)
+        assert_bit_equal(got["weight_scale"][sl], o_scale, f"scales {sl}")
+        assert_bit_equal(got["weight_packed"][sl], want["weight_packed"], f"packed {sl}")
+
+
 def test_llama_layer_fp8_batch(gpu):
     """fp8 e4m3 per-channel (the W8A8 weight set, with outliers): QuantizedWeightBatch and
     the one-pass observer + quantizer on the real shapes"""

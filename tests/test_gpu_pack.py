@@ -154,6 +154,10 @@ def test_observe_and_compress_in_one_pass(spec, shape, dtype, fused, gpu):
     blk = {"group": spec.get("group_size", 0), "channel": cols}.get(spec["strategy"], 0)
     assert bool(blk and _lib.load().ctmi_observe_pack_quantized_supported(
         _lib.dtype_code(dtype), rows, cols, blk, spec["num_bits"])) == fused
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    table = bool(blk and _lib.load().ctmi_observe_pack_quantized_gidx_supported(
+        _lib.dtype_code(dtype), rows, cols, blk, spec["num_bits"]))
+    assert comp.one_pass_kernel(w.to(gpu), args) == ("groups" if fused else "table" if table else None)
     scale, zp = oq.observe_weight(w, oargs)
     want = op.pack_quantized_compress(w, scale, oargs, zero_point=zp)
     comp = BaseCompressor.load_from_registry("pack-quantized")
@@ -213,13 +217,19 @@ def test_observed_weight_batch_matches_single_calls(gpu):
             assert_bit_equal(d[k], want[k], k)
 
 
-def test_observed_weight_batch_takes_every_strategy(gpu):
-    """weights without a one-pass kernel (one scale per tensor, blocks, a group size that is
-    not a power of two, activation ordering) go through the batch as well: the observer and
-    the compressor run one after the other for them.  Against the oracle's observer (on the
-    columns sorted by g_idx where there is one, forward.py:286-303) and compressor."""
-    from compressed_tensors_amd.compressors import ObservedWeightBatch
-    from compressed_tensors_amd.quantization import QuantizationArgs
+def test_observed_weight_batch_takes_every_strategy(gpu, monkeypatch):
+    """weights that do not share the batch's launches go through it as well: a group size
+    that is not a power of two and activation ordering in one pass of their own (the group of
+    a column looked up), one scale per tensor and blocks with the observer and the compressor
+    one after the other.  Against the oracle's observer (on the columns sorted by g_idx where
+    there is one, forward.py:286-303) and compressor."""
+    from compressed_tensors_amd.compressors import BaseCompressor, ObservedWeightBatch
+    from compressed_tensors_amd.quantization import QuantizationArgs, helpers
+
+    observed = []
+    real = helpers.observe_weight_qparams
+    monkeypatch.setattr(helpers, "observe_weight_qparams",
+                        lambda w, a, *k, **kw: (observed.append(a.strategy), real(w, a, *k, **kw))[1])
 
     announce("observed weight batch, every strategy")
     g = torch.Generator().manual_seed(18)
@@ -235,6 +245,11 @@ def test_observed_weight_batch_takes_every_strategy(gpu):
                     **({} if gi is None else {"g_idx": gi.to(gpu)}))
                for w, spec, gi in zip(ws, specs, g_idx)]
     got = ObservedWeightBatch(entries).compress()
+    # the separate observer ran for the tensor and the block scheme only
+    assert sorted(observed) == ["block", "tensor"]
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    assert [comp.one_pass_kernel(e["weight"], e["quantization_args"], e.get("g_idx")) for e in entries] == [
+        None, None, "table", "groups", "table"]
     for i, (w, spec, gi, d) in enumerate(zip(ws, specs, g_idx, got)):
         oargs = oq._Args(**spec)
         seen = w if gi is None else w.index_select(1, torch.argsort(gi.long()))
@@ -243,6 +258,53 @@ def test_observed_weight_batch_takes_every_strategy(gpu):
         assert_bit_equal(d["weight_scale"], scale, f"scale {i}")
         for k in want:
             assert_bit_equal(d[k], want[k], f"{k} {i}")
+
+
+ACT_ORDER = [
+    # (rows, cols, group_size, dtype, symmetric, num_bits): items per lane 1, 2, 4, 8; rows that do
+    # not fill the last block of a workgroup; more row blocks than workgroups
+    (37, 1024, 128, torch.bfloat16, True, 4),
+    (300, 4096, 128, torch.bfloat16, True, 4),
+    (21, 4096, 128, torch.bfloat16, False, 4),
+    (19, 8192, 64, torch.float16, True, 8),
+    (4100, 512, 32, torch.bfloat16, True, 4),
+    (9, 14336, 128, torch.bfloat16, True, 4),
+    (5, 14336, 128, torch.float32, False, 8),
+    (16, 1536, 24, torch.bfloat16, True, 4),   # no g_idx: groups of 24 by division
+]
+
+
+@pytest.mark.parametrize("rows,cols,group,dtype,symmetric,bits", ACT_ORDER,
+                         ids=[f"ao{i}-{c[1]}" for i, c in enumerate(ACT_ORDER)])
+def test_one_pass_with_activation_ordering(rows, cols, group, dtype, symmetric, bits, gpu):
+    """ctmi_observe_pack_quantized_gidx: min-max observer on the columns as g_idx sorts them,
+    calculate_qparams, quantize with g_idx and pack, from one kernel; against the oracle's
+    observer on the sorted columns followed by its compressor with g_idx"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+
+    announce("one-shot pack-quantized with g_idx", rows, cols, group, dtype, symmetric, bits)
+    spec = dict(num_bits=bits, type="int", symmetric=symmetric, strategy="group", group_size=group)
+    args, oargs = _pair(spec)
+    g = torch.Generator().manual_seed(rows + cols)
+    w = (torch.randn(rows, cols, generator=g) * 0.02).to(dtype)
+    w[0, :9] = 0.0
+    w[-1] = 0.0
+    if rows > 4:
+        w[1] = w[1].abs()
+        w[2] = -w[2].abs()
+        w[3, 7] = float("inf")
+    gi = None if group == 24 else (torch.randperm(cols, generator=g) // group).to(torch.int32)
+    seen = w if gi is None else w.index_select(1, torch.argsort(gi.long(), stable=True))
+    scale, zp = oq.observe_weight(seen, oargs)
+    want = op.pack_quantized_compress(w, scale, oargs, zero_point=zp, g_idx=gi)
+    comp = BaseCompressor.load_from_registry("pack-quantized")
+    wg, gg = w.to(gpu), None if gi is None else gi.to(gpu)
+    assert comp.one_pass_kernel(wg, args, gg) == "table"
+    got = comp.observe_and_compress_weight(wg, args, g_idx=gg)
+    assert set(got) == set(want) | {"weight_scale"}
+    assert_bit_equal(got["weight_scale"], scale, "scale")
+    for k in want:
+        assert_bit_equal(got[k], want[k], k)
 
 
 def test_pack_quantized_state_dict_and_g_idx(gpu):
