@@ -727,19 +727,26 @@ def other_workload(torch, name, seed):
         q = (torch.randint(0, 2, (128,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)
         keep.extend([mb, q])
         for label in ("weights 4096x4096 (x16)", "weights 14336x4096 (x5)"):
-            calls = []
+            calls, calls_matrix = [], []
             for x in tensors[label]:
                 packed = torch.empty(x.shape[0], x.shape[1] // 8, dtype=torch.int32, device=dev)
                 scale = torch.empty(x.shape[0], x.shape[1] // 128, dtype=torch.bfloat16, device=dev)
                 keep.extend([packed, scale])
-                a = (x.data_ptr(), code(x.dtype), x.numel(), 128, mb.data_ptr(), q.data_ptr(), None,
+                # no matrix argument: Sylvester's matrix of 128, what hadamard_quantize_pack passes
+                # for the reference's own matrices of this size
+                a = (x.data_ptr(), code(x.dtype), x.numel(), 128, None, q.data_ptr(), None,
                      4, 1, packed.data_ptr(), scale.data_ptr(), None, st)
                 calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_quant_pack(*a)))
+                ax = a[:4] + (mb.data_ptr(),) + a[5:]
+                calls_matrix.append(lambda ax=ax: _lib.check(lib.ctmi_hadamard_quant_pack(*ax)))
             nb = sum(2 * x.numel() + x.numel() // 2 + 2 * x.numel() // 128 for x in tensors[label])
             flops = sum(2 * 128 * x.numel() for x in tensors[label])
             ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}", calls, nb,
-                          "hadamard_quant_pack_kernel", primary=not label.startswith("weights 4096x4096"),
+                          "sylvester128_quant_pack_kernel", primary=not label.startswith("weights 4096x4096"),
                           mfma_flops=flops))
+            if not label.startswith("weights 4096x4096"):
+                ops.append(Op(f"fused: any 128 x 128 matrix + int4 g128 quantize + pack, {label}", calls_matrix, nb,
+                              "hadamard_quant_pack_kernel", primary=False, mfma_flops=flops))
             if label.startswith("weights 4096x4096"):
                 xs = tensors[label]
                 jobs = (_lib.HadamardPackJob * len(xs))()
@@ -750,10 +757,10 @@ def other_workload(torch, name, seed):
                     job.x, job.packed, job.scale, job.rotated, job.numel = (
                         x.data_ptr(), packed.data_ptr(), scale.data_ptr(), None, x.numel())
                 keep.append(jobs)
-                m = (jobs, len(xs), code(xs[0].dtype), 128, mb.data_ptr(), q.data_ptr(), None, 4, 1, st)
+                m = (jobs, len(xs), code(xs[0].dtype), 128, None, q.data_ptr(), None, 4, 1, st)
                 ops.append(Op(f"fused: Hadamard 128 + int4 g128 quantize + pack, {label}, one call (8 per launch)",
                               [lambda m=m: _lib.check(lib.ctmi_hadamard_quant_pack_many(*m))], nb,
-                              "hadamard_quant_pack_kernel", mfma_flops=flops, launches=chained(len(xs))))
+                              "sylvester128_quant_pack_kernel", mfma_flops=flops, launches=chained(len(xs))))
         # the full 4096-wide rotation (64 x 64) with the same quantization in its epilogue
         mb64 = deterministic_hadamard_matrix(64, torch.bfloat16, dev).contiguous()
         q4k = (torch.randint(0, 2, (4096,), generator=torch.Generator().manual_seed(seed)) * 2 - 1).float().to(dev)

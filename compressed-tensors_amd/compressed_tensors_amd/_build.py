@@ -36,10 +36,12 @@ FLAGS = [
 ]
 
 
-# per source file (by stem): the butterfly kernels chain matrix-core results into vector code,
-# so their accumulators live in ordinary registers (no copies out of a second register class,
-# and the registers are reused once the accumulators are dead)
-EXTRA_FLAGS = {"fwht": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+# per source file (by stem): the butterfly kernels and the rotations with an epilogue chain
+# matrix-core results into vector code, so their accumulators live in ordinary registers (no
+# copies out of a second register class - one instruction per output element -, and the
+# registers are reused once the accumulators are dead)
+EXTRA_FLAGS = {"fwht": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+               "hadamard": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 
 def sources():

@@ -396,10 +396,14 @@ def _quantize_pack(values, n, args, sign_in, sign_out, matrix_t, return_rotated,
         results.append(out)
     lib, code, stream = _lib.load(), _lib.dtype_code(torch.bfloat16), _lib.stream_of(dev)
     if plan is None:
-        mb_t = (_sylvester_bf16(n, dev) if matrix_t is None
-                else matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous())
+        # no matrix argument stands for Sylvester's matrix of 128: that kernel keeps none in memory
+        mb_t = None
+        if matrix_t is not None:
+            mb_t = matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous()
+        elif n != 128 or not _aligned(s_in, s_out):
+            mb_t = _sylvester_bf16(n, dev)
         _lib.check(lib.ctmi_hadamard_quant_pack_many(
-            jobs, len(xs), code, n, mb_t.data_ptr(), _lib.ptr(s_in), _lib.ptr(s_out), 4, 1, stream))
+            jobs, len(xs), code, n, _lib.ptr(mb_t), _lib.ptr(s_in), _lib.ptr(s_out), 4, 1, stream))
     elif plan == "butterfly":
         _lib.check(lib.ctmi_sylvester_quant_pack_many(
             jobs, len(xs), code, n, _lib.ptr(s_in), _lib.ptr(s_out), group, 4, 1, stream))

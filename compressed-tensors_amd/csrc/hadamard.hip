@@ -46,6 +46,9 @@ constexpr int kRowsWaves = kRowsThreads / kWave;
 #endif
 constexpr int kKronThreads = CTMI_HAD_KRON_THREADS;
 constexpr int kKronWaves = kKronThreads / kWave;
+#ifndef CTMI_HQP_GROUPS
+#define CTMI_HQP_GROUPS 1  // groups of 16 sub-rows a wavefront takes at a time
+#endif
 #ifndef CTMI_HQP_TUNING
 #define CTMI_HQP_TUNING 1024, 1  // fused rotation + quantization kernel: threads, workgroups per CU
 #endif
@@ -541,8 +544,17 @@ static int launch_had_rows_jobs(const HadJobs& jobs, int n_jobs, const HadArgs& 
 // those of the three separate steps; the rotated tensor never goes to memory
 // (unless `rotated` asks for it).  A sub-row's 128 outputs sit in the 4 lanes
 // l16 + 16 q; they agree on min / max through two lane exchanges.
+#ifndef CTMI_HQP_LOAD
+#define CTMI_HQP_LOAD ldg
+#endif
+#ifndef CTMI_HQP_STORE
+#define CTMI_HQP_STORE stg
+#endif
+#ifndef CTMI_HQP_MIN_WAVES
+#define CTMI_HQP_MIN_WAVES 4  // wavefronts per SIMD the kernel is compiled for
+#endif
 template <int B, bool MANY>
-__global__ void __launch_bounds__(kHqpThreads)
+__global__ void __launch_bounds__(kHqpThreads, CTMI_HQP_MIN_WAVES)
 hadamard_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const uint16_t* __restrict__ mbt,
                            const float* __restrict__ s_in, const float* __restrict__ s_out,
                            float inv_sqrt_n, QpCfg cfg) {
@@ -576,32 +588,54 @@ hadamard_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const uint16_t* __res
 
   // n_groups: groups of 16 sub-rows over all jobs (a job's last one may be ragged)
   const int64_t stride = (int64_t)gridDim.x * kHqpWaves;
-  for (int64_t g = (int64_t)blockIdx.x * kHqpWaves + wave; g < n_groups; g += stride) {
+  // where a group's sub-rows are and go, and its loads
+  struct Place {
+    int j;
+    int64_t row;
+    bool keep;
+  };
+  auto place_of = [&](int64_t g) {
+    if (g >= n_groups) g = n_groups - 1;  // past the end: the last group again, nothing stored
     int64_t local;
-    const int j = had_job<MANY>(jobs, g, &local);
-    const int64_t n_sub = jobs.n_sub[j];
-    const uint16_t* x = static_cast<const uint16_t*>(jobs.x[j]);
-    int32_t* packed = static_cast<int32_t*>(jobs.out[j]);
-    uint16_t* scale = static_cast<uint16_t*>(jobs.scale[j]);
-    uint16_t* rotated = static_cast<uint16_t*>(jobs.rotated[j]);
-    int64_t row = local * 16 + l16;
-    const bool keep = row < n_sub;
-    if (!keep) row = n_sub - 1;  // ragged last group: recompute the last sub-row, store nothing
-    const uint16_t* src = x + row * B + 8 * lq;
-    bf16x8_t xf[KS];
+    Place pl;
+    pl.j = had_job<MANY>(jobs, g, &local);
+    pl.row = local * 16 + l16;
+    pl.keep = pl.row < jobs.n_sub[pl.j];
+    if (!pl.keep) pl.row = jobs.n_sub[pl.j] - 1;  // ragged last group: the last sub-row again
+    return pl;
+  };
+  auto fetch = [&](const Place& pl, bf16x8_t* xf) {
+    const uint16_t* src = static_cast<const uint16_t*>(jobs.x[pl.j]) + pl.row * B + 8 * lq;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
-      xf[ks] = __builtin_bit_cast(bf16x8_t, ldg<uint16_t, 8>(src + 32 * ks));
-    Vec<uint32_t, 4> o[NP];  // the rotated sub-row in bf16: columns 32 p + 8 lq .. + 8
+      xf[ks] = __builtin_bit_cast(bf16x8_t, CTMI_HQP_LOAD<uint16_t, 8>(src + 32 * ks));
+  };
+  // A wavefront takes G groups at a time (neighbours in memory): every fragment of the matrix
+  // it reads from LDS then serves G products.
+  constexpr int G = CTMI_HQP_GROUPS;
+  for (int64_t g = ((int64_t)blockIdx.x * kHqpWaves + wave) * G; g < n_groups; g += stride * G) {
+    Place here[G];
+    bf16x8_t xf[G][KS];
+#pragma unroll
+    for (int t = 0; t < G; ++t) {
+      here[t] = place_of(g + t);
+      here[t].keep = here[t].keep && g + t < n_groups;
+      fetch(here[t], xf[t]);
+    }
+    Vec<uint32_t, 4> o[G][NP];  // the rotated sub-rows in bf16: columns 32 p + 8 lq .. + 8
     // A symmetric scale only needs max |x| of the group (min(min,0) and max(max,0)
     // enter through their magnitudes, helpers.py:87-104).  Magnitudes of bf16
     // values order like their bit patterns, a NaN above everything: the maximum is
     // taken on the packed 16-bit halves, two elements per instruction.
     typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
-    u16x2_t top = {0, 0};
+    u16x2_t top[G];
+#pragma unroll
+    for (int t = 0; t < G; ++t) top[t] = u16x2_t{0, 0};
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-      f32x4_t a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = {0.0f, 0.0f, 0.0f, 0.0f};
+      f32x4_t a0[G], a1[G];
+#pragma unroll
+      for (int t = 0; t < G; ++t) a0[t] = a1[t] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
       // keeps the compiler from hoisting these (loop-invariant) LDS reads out of
       // the loop, back into 128 registers
       asm volatile("" ::: "memory");
@@ -609,51 +643,304 @@ hadamard_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const uint16_t* __res
       for (int ks = 0; ks < KS; ++ks) {
         const bf16x8_t m0 = __builtin_bit_cast(bf16x8_t, frag_lds[(2 * p) * KS + ks][lane]);
         const bf16x8_t m1 = __builtin_bit_cast(bf16x8_t, frag_lds[(2 * p + 1) * KS + ks][lane]);
-        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(m0, xf[ks], a0, 0, 0, 0);
-        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(m1, xf[ks], a1, 0, 0, 0);
-      }
-      o[p].v[0] = pack_bf16x2(a0[0] * inv_sqrt_n, a0[1] * inv_sqrt_n);
-      o[p].v[1] = pack_bf16x2(a0[2] * inv_sqrt_n, a0[3] * inv_sqrt_n);
-      o[p].v[2] = pack_bf16x2(a1[0] * inv_sqrt_n, a1[1] * inv_sqrt_n);
-      o[p].v[3] = pack_bf16x2(a1[2] * inv_sqrt_n, a1[3] * inv_sqrt_n);
 #pragma unroll
-      for (int w = 0; w < 4; ++w)
-        top = __builtin_elementwise_max(top, __builtin_bit_cast(u16x2_t, o[p].v[w] & 0x7FFF7FFFu));
+        for (int t = 0; t < G; ++t) {
+          a0[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(m0, xf[t][ks], a0[t], 0, 0, 0);
+          a1[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(m1, xf[t][ks], a1[t], 0, 0, 0);
+        }
+      }
+#ifdef CTMI_HQP_DIAG_NOMFMA
+#pragma unroll
+      for (int t = 0; t < G; ++t) {
+        o[t][p] = __builtin_bit_cast(Vec<uint32_t, 4>, xf[t][p]);
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          top[t] = __builtin_elementwise_max(top[t], __builtin_bit_cast(u16x2_t, o[t][p].v[w] & 0x7FFF7FFFu));
+      }
+      continue;
+#endif
+#pragma unroll
+      for (int t = 0; t < G; ++t) {
+        o[t][p].v[0] = pack_bf16x2(a0[t][0] * inv_sqrt_n, a0[t][1] * inv_sqrt_n);
+        o[t][p].v[1] = pack_bf16x2(a0[t][2] * inv_sqrt_n, a0[t][3] * inv_sqrt_n);
+        o[t][p].v[2] = pack_bf16x2(a1[t][0] * inv_sqrt_n, a1[t][1] * inv_sqrt_n);
+        o[t][p].v[3] = pack_bf16x2(a1[t][2] * inv_sqrt_n, a1[t][3] * inv_sqrt_n);
+#pragma unroll
+        for (int w = 0; w < 4; ++w)
+          top[t] = __builtin_elementwise_max(top[t], __builtin_bit_cast(u16x2_t, o[t][p].v[w] & 0x7FFF7FFFu));
+      }
     }
-    uint32_t mag = top.x > top.y ? top.x : top.y;
+#pragma unroll
+    for (int t = 0; t < G; ++t) {
+      const int j = here[t].j;
+      int32_t* packed = static_cast<int32_t*>(jobs.out[j]);
+      uint16_t* scale = static_cast<uint16_t*>(jobs.scale[j]);
+      uint16_t* rotated = static_cast<uint16_t*>(jobs.rotated[j]);
+      const int64_t row = here[t].row;
+      const bool keep = here[t].keep;
+      uint32_t mag = top[t].x > top[t].y ? top[t].x : top[t].y;
+#pragma unroll
+      for (int d = 16; d < 64; d <<= 1) {
+        const uint32_t other = (uint32_t)__shfl_xor((int)mag, d, kWave);
+        mag = other > mag ? other : mag;
+      }
+      // calculate_qparams, symmetric, in bf16 (helpers.py:101-122); 7.5 is a bf16 value: the
+      // product with its reciprocal rounds to the same bf16 as the quotient
+      const float sv = symmetric_scale<BF16>(bf16_to_f32((uint16_t)mag), mag > 0x7F80u, cfg.sym_div);
+      // Packed word 4 p + lq of the sub-row comes out of lane (l16, lq) for pair p.
+      // The 4 lanes of a sub-row swap words through a wave-private patch of LDS so
+      // that each stores NP neighbouring words (16 bytes at B = 128) instead of NP
+      // single ones 16 bytes apart.
+      int32_t* swap = &swap_lds[wave][l16][0];
+#pragma unroll
+      for (int p = 0; p < NP; ++p) {
+#ifdef CTMI_HQP_DIAG_NOQUANT
+        Vec<int32_t, 1> w;
+        w.v[0] = (int32_t)(o[t][p].v[0] ^ o[t][p].v[1] ^ o[t][p].v[2] ^ o[t][p].v[3]) + (int32_t)__float_as_uint(sv);
+#else
+        const Vec<int32_t, 1> w = quant_pack8<BF16, BF16, 4, false>(
+            __builtin_bit_cast(Vec<uint16_t, 8>, o[t][p]), sv, 0.0f, cfg.bit_min, cfg.bit_max);
+#endif
+        swap[4 * p + lq] = w.v[0];
+        if (rotated && keep)
+          stg<uint16_t, 8>(rotated + row * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o[t][p]));
+      }
+      asm volatile("" ::: "memory");  // the reads below are of other lanes' words
+      if (keep) {
+        if (lq == 0) scale[row] = f32_to_bf16(sv);
+        if (lq < NP) {
+          Vec<int32_t, 4> out4;
+#pragma unroll
+          for (int j4 = 0; j4 < 4; ++j4) out4.v[j4] = swap[4 * lq + j4];
+          CTMI_HQP_STORE<int32_t, 4>(packed + row * (B / 8) + 4 * lq, out4);
+        }
+      }
+      asm volatile("" ::: "memory");  // the next group's words must not overtake these reads
+    }
+  }
+}
+
+// ---------------------------------------------------------------- the same for Sylvester's matrix of 128
+// hadamard_quant_pack_kernel for the matrix the reference uses at this size (Sylvester's H_128,
+// with or without sign vectors; transform/utils/hadamard.py:65-100), with no matrix in memory:
+// H[k][c] = (-1)^popcount(k & c) splits, for the operand layout above (k = 32 ks + 8 q + e,
+// c = 32 p + 8 (m / 4) + 4 b + m % 4 for row m of tile 2 p + b), into
+//     (-1)^popcount(ks & p)  *  (-1)^(popcount(q & (m / 4)) + popcount(e & (4 b + m % 4))):
+// two fragments (b = 0, 1) a lane keeps in 8 registers serve all 32 products, and the sign
+// in front goes to the other operand (the sub-rows, negated once per group).  Sign vectors are
+// applied as sign-bit masks to the inputs and to the rounded outputs.  Without a matrix to set
+// up, a workgroup takes one chunk of sub-rows and exits (no loop over the tensor, nothing in
+// LDS, no barrier), like the streaming kernels of the other formats.
+#ifndef CTMI_SQP_GROUPS
+#define CTMI_SQP_GROUPS 2  // groups of 16 sub-rows a wavefront takes
+#endif
+#ifndef CTMI_SQP_FP32_MAX
+#define CTMI_SQP_FP32_MAX 1  // max |x| on the fp32 values (one instruction per two) or on the packed bf16 ones
+#endif
+#ifndef CTMI_SQP_NEG_FRAG
+#define CTMI_SQP_NEG_FRAG 0  // the sign in front of a product on the fragment (1) or on the sub-rows (0)
+#endif
+#ifndef CTMI_SQP_LOAD
+#define CTMI_SQP_LOAD ldg_nt
+#endif
+#ifndef CTMI_SQP_STORE
+#define CTMI_SQP_STORE stg_nt
+#endif
+constexpr int kSqpThreads = 256;
+constexpr int kSqpWaves = kSqpThreads / kWave;
+
+#ifndef CTMI_SQP_MIN_WAVES
+#define CTMI_SQP_MIN_WAVES 4
+#endif
+template <bool MANY, bool SIGN_IN, bool SIGN_OUT>
+__global__ void __launch_bounds__(kSqpThreads, CTMI_SQP_MIN_WAVES)
+sylvester128_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const float* __restrict__ s_in,
+                               const float* __restrict__ s_out, float inv_sqrt_n, QpCfg cfg) {
+  constexpr int B = 128, KS = 4, NP = 4, G = CTMI_SQP_GROUPS;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int l16 = lane & 15, lq = lane >> 4;
+  const int64_t g0 = ((int64_t)blockIdx.x * kSqpWaves + wave) * G;
+  if (g0 >= n_groups) return;
+
+  // where the groups' sub-rows are, and their loads (all issued before anything else)
+  int job[G];
+  int64_t row[G];
+  bool keep[G];
+  bf16x8_t xf[G][KS];
+#pragma unroll
+  for (int t = 0; t < G; ++t) {
+    int64_t g = g0 + t, local;
+    const bool live = g < n_groups;
+    if (!live) g = n_groups - 1;  // past the end: the last group again, nothing stored
+    job[t] = had_job<MANY>(jobs, g, &local);
+    row[t] = local * 16 + l16;
+    keep[t] = live && row[t] < jobs.n_sub[job[t]];
+    if (row[t] >= jobs.n_sub[job[t]]) row[t] = jobs.n_sub[job[t]] - 1;  // ragged last group
+    const uint16_t* src = static_cast<const uint16_t*>(jobs.x[job[t]]) + row[t] * B + 8 * lq;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      xf[t][ks] = __builtin_bit_cast(bf16x8_t, CTMI_SQP_LOAD<uint16_t, 8>(src + 32 * ks));
+  }
+  // sign-bit masks of this lane's inputs (k = 32 ks + 8 lq + e) and outputs (c = 32 p + 8 lq + e)
+  uint32_t flip_in[SIGN_IN ? KS : 1][4], flip_out[SIGN_OUT ? NP : 1][4];
+  auto masks = [&](const float* __restrict__ signs, uint32_t (*flip)[4]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const Vec<uint32_t, 4> lo = ldg<uint32_t, 4>(reinterpret_cast<const uint32_t*>(signs) + 32 * q + 8 * lq);
+      const Vec<uint32_t, 4> hi = ldg<uint32_t, 4>(reinterpret_cast<const uint32_t*>(signs) + 32 * q + 8 * lq + 4);
+      flip[q][0] = ((lo.v[0] >> 16) & 0x8000u) | (lo.v[1] & 0x80000000u);
+      flip[q][1] = ((lo.v[2] >> 16) & 0x8000u) | (lo.v[3] & 0x80000000u);
+      flip[q][2] = ((hi.v[0] >> 16) & 0x8000u) | (hi.v[1] & 0x80000000u);
+      flip[q][3] = ((hi.v[2] >> 16) & 0x8000u) | (hi.v[3] & 0x80000000u);
+    }
+  };
+  if constexpr (SIGN_IN) masks(s_in, flip_in);
+  if constexpr (SIGN_OUT) masks(s_out, flip_out);
+  // the two fragments: entry e of row m = l16 in the k block of lane quarter lq
+  u32x4_t frag[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const uint32_t rowbits = (uint32_t)(4 * b + (l16 & 3));
+      const uint32_t common = (uint32_t)__builtin_popcount(lq & (l16 >> 2));
+      const uint32_t lo = ((common + __builtin_popcount((2 * d) & rowbits)) & 1u) ? 0xBF80u : 0x3F80u;
+      const uint32_t hi = ((common + __builtin_popcount((2 * d + 1) & rowbits)) & 1u) ? 0xBF80u : 0x3F80u;
+      frag[b][d] = lo | (hi << 16);
+    }
+  const bf16x8_t f0 = __builtin_bit_cast(bf16x8_t, frag[0]), f1 = __builtin_bit_cast(bf16x8_t, frag[1]);
+#if CTMI_SQP_NEG_FRAG
+  const bf16x8_t f0n = __builtin_bit_cast(bf16x8_t, frag[0] ^ 0x80008000u);
+  const bf16x8_t f1n = __builtin_bit_cast(bf16x8_t, frag[1] ^ 0x80008000u);
+#endif
+
+#pragma unroll
+  for (int t = 0; t < G; ++t) {
+    if constexpr (SIGN_IN) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        u32x4_t xs = __builtin_bit_cast(u32x4_t, xf[t][ks]);
+#pragma unroll
+        for (int d = 0; d < 4; ++d) xs[d] ^= flip_in[ks][d];
+        xf[t][ks] = __builtin_bit_cast(bf16x8_t, xs);
+      }
+    }
+#if !CTMI_SQP_NEG_FRAG
+    bf16x8_t xneg[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      xneg[ks] = __builtin_bit_cast(bf16x8_t, __builtin_bit_cast(u32x4_t, xf[t][ks]) ^ 0x80008000u);
+#endif
+    Vec<uint32_t, 4> o[NP];  // the rotated sub-row in bf16: columns 32 p + 8 lq .. + 8
+    // max |x| of what this lane holds, on the fp32 values before they are rounded (rounding
+    // is monotonic: the largest magnitude stays the largest).  The maximum drops NaNs, and the
+    // min-max observer must not: a NaN among the inputs makes every output of the sub-row a
+    // NaN (one look at one value finds it), infinities among them make every output an
+    // infinity or a NaN (the maximum is then infinite); both go the exact way below.
+#if CTMI_SQP_FP32_MAX
+    float top = 0.0f;
+    bool odd = false;
+#else
+    typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+    u16x2_t top2 = {0, 0};
+#endif
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+      f32x4_t a0 = {0.0f, 0.0f, 0.0f, 0.0f}, a1 = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const bool minus = (__builtin_popcount(ks & p) & 1) != 0;
+#if CTMI_SQP_NEG_FRAG
+        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(minus ? f0n : f0, xf[t][ks], a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(minus ? f1n : f1, xf[t][ks], a1, 0, 0, 0);
+#else
+        const bf16x8_t xk = minus ? xneg[ks] : xf[t][ks];
+        a0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f0, xk, a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f1, xk, a1, 0, 0, 0);
+#endif
+      }
+      float v[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        v[e] = a0[e] * inv_sqrt_n;
+        v[4 + e] = a1[e] * inv_sqrt_n;
+      }
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {
+        o[p].v[w] = pack_bf16x2(v[2 * w], v[2 * w + 1]);
+        if constexpr (SIGN_OUT) o[p].v[w] ^= flip_out[p][w];
+#if CTMI_SQP_FP32_MAX
+        top = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[2 * w]), __builtin_fabsf(v[2 * w + 1])), top);
+#else
+        top2 = __builtin_elementwise_max(top2, __builtin_bit_cast(u16x2_t, o[p].v[w] & 0x7FFF7FFFu));
+#endif
+      }
+#if CTMI_SQP_FP32_MAX
+      if (p == 0) odd = v[0] != v[0];
+#endif
+    }
+    // max |x| of the sub-row: the 4 lanes l16 + 16 q agree through two lane exchanges
+    // (magnitudes of non-negative floats order like their bit patterns, a NaN above everything)
+#if !CTMI_SQP_FP32_MAX
+    // (bf16 magnitudes order like their bit patterns, a NaN above everything: the maximum is
+    // taken on the packed 16-bit halves, two elements per instruction)
+    uint32_t mag = (uint32_t)(top2.x > top2.y ? top2.x : top2.y) << 16;
+#else
+    uint32_t mag = __float_as_uint(top);
+    if (odd || !(top < __builtin_inff())) {
+      // the rare group with a NaN or an infinity: the maximum over the rounded values, bit by bit
+      mag = 0;
+#pragma unroll
+      for (int p = 0; p < NP; ++p)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const uint32_t lo = (o[p].v[w] & 0x7FFFu) << 16, hi = o[p].v[w] & 0x7FFF0000u;
+          mag = max(mag, max(lo, hi));
+        }
+    } else {
+      mag = (uint32_t)f32_to_bf16(__uint_as_float(mag)) << 16;  // rounded as the outputs are
+    }
+#endif
 #pragma unroll
     for (int d = 16; d < 64; d <<= 1) {
       const uint32_t other = (uint32_t)__shfl_xor((int)mag, d, kWave);
       mag = other > mag ? other : mag;
     }
-    // calculate_qparams, symmetric, in bf16 (helpers.py:101-122): the scheme is fixed
-    // here, so the general routine's dtype switches are spelled out instead
-    float sv = bf16_to_f32(f32_to_bf16(bf16_to_f32((uint16_t)mag) / cfg.sym_div));
-    sv = (sv != sv) ? sv : fmaxf(sv, 1.1920928955078125e-07f);
-    // Packed word 4 p + lq of the sub-row comes out of lane (l16, lq) for pair p.
-    // The 4 lanes of a sub-row swap words through a wave-private patch of LDS so
-    // that each stores NP neighbouring words (16 bytes at B = 128) instead of NP
-    // single ones 16 bytes apart.
-    int32_t* swap = &swap_lds[wave][l16][0];
+    mag >>= 16;
+    const float sv = symmetric_scale<BF16>(bf16_to_f32((uint16_t)mag), mag > 0x7F80u, cfg.sym_div);
+    const int j = job[t];
+    int32_t* packed = static_cast<int32_t*>(jobs.out[j]);
+    uint16_t* scale = static_cast<uint16_t*>(jobs.scale[j]);
+    uint16_t* rotated = static_cast<uint16_t*>(jobs.rotated[j]);
+    uint32_t w[NP];
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-      const Vec<int32_t, 1> w = quant_pack8<BF16, BF16, 4, false>(
-          __builtin_bit_cast(Vec<uint16_t, 8>, o[p]), sv, 0.0f, cfg.bit_min, cfg.bit_max);
-      swap[4 * p + lq] = w.v[0];
-      if (rotated && keep)
-        stg<uint16_t, 8>(rotated + row * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o[p]));
+      w[p] = (uint32_t)quant_pack8<BF16, BF16, 4, false>(__builtin_bit_cast(Vec<uint16_t, 8>, o[p]), sv, 0.0f,
+                                                         cfg.bit_min, cfg.bit_max).v[0];
+      if (rotated && keep[t])
+        CTMI_SQP_STORE<uint16_t, 8>(rotated + row[t] * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o[p]));
     }
-    asm volatile("" ::: "memory");  // the reads below are of other lanes' words
-    if (keep) {
-      if (lq == 0) scale[row] = f32_to_bf16(sv);
-      if (lq < NP) {
-        Vec<int32_t, 4> out4;
+    // Lane (l16, lq) holds packed words 4 p + lq of its sub-row; the 4 lanes of a sub-row
+    // transpose their 4 x 4 words in two exchanges (lanes 32 apart, then neighbouring rows
+    // of 16 lanes), after which lane lq stores words 4 lq .. 4 lq + 3: 16 bytes.
+    {
+      auto s02 = __builtin_amdgcn_permlane32_swap(w[0], w[2], false, false);
+      auto s13 = __builtin_amdgcn_permlane32_swap(w[1], w[3], false, false);
+      auto s01 = __builtin_amdgcn_permlane16_swap(s02[0], s13[0], false, false);
+      auto s23 = __builtin_amdgcn_permlane16_swap(s02[1], s13[1], false, false);
+      w[0] = s01[0];
+      w[1] = s01[1];
+      w[2] = s23[0];
+      w[3] = s23[1];
+    }
+    if (keep[t]) {
+      if (lq == 0) scale[row[t]] = f32_to_bf16(sv);
+      Vec<int32_t, 4> out4;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) out4.v[j] = swap[4 * lq + j];
-        stg<int32_t, 4>(packed + row * (B / 8) + 4 * lq, out4);
-      }
+      for (int q = 0; q < 4; ++q) out4.v[q] = (int32_t)w[q];
+      CTMI_SQP_STORE<int32_t, 4>(packed + row[t] * (B / 8) + 4 * lq, out4);
     }
-    asm volatile("" ::: "memory");  // the next group's words must not overtake these reads
   }
 }
 
@@ -1253,7 +1540,7 @@ static int hqp_check_job(const ctmi_hadamard_pack_job& j, int32_t b_dim) {
   if (j.numel == 0) return CTMI_OK;
   CTMI_REQUIRE(j.x && j.packed && j.scale, CTMI_ERR_VALUE, "NULL tensor pointer");
   CTMI_REQUIRE((uintptr_t)j.x % 16 == 0 && (uintptr_t)j.rotated % 16 == 0 &&
-                   (uintptr_t)j.packed % 4 == 0 && (uintptr_t)j.scale % 2 == 0,
+                   (uintptr_t)j.packed % 16 == 0 && (uintptr_t)j.scale % 2 == 0,
                CTMI_ERR_VALUE, "tensors must be 16-byte aligned");
   return CTMI_OK;
 }
@@ -1271,10 +1558,29 @@ static void hqp_launch(const HadJobs& t, int filled, int32_t b_dim, const void* 
   c.mt = c.zp_sub_dtype = c.scale_dtype = CTMI_BF16;
   c.zp_dtype = CTMI_I8;
   const int64_t n_groups = t.end[filled - 1];
-  const int64_t wgs = cdiv(n_groups, kHqpWaves);
+  const float inv = 1.0f / sqrtf((float)b_dim);
+  if (!mb_t) {  // Sylvester's matrix of 128 (checked by the caller)
+    const unsigned grid = (unsigned)cdiv(n_groups, kSqpWaves * CTMI_SQP_GROUPS);
+#define CTMI_SQP(MANY)                                                                                \
+  if (sign_in && sign_out)                                                                            \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, true, true>), grid, kSqpThreads, 0, st,  \
+                       t, n_groups, sign_in, sign_out, inv, c);                                       \
+  else if (sign_in)                                                                                   \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, true, false>), grid, kSqpThreads, 0, st, \
+                       t, n_groups, sign_in, sign_out, inv, c);                                       \
+  else if (sign_out)                                                                                  \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, false, true>), grid, kSqpThreads, 0, st, \
+                       t, n_groups, sign_in, sign_out, inv, c);                                       \
+  else                                                                                                \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, false, false>), grid, kSqpThreads, 0,    \
+                       st, t, n_groups, sign_in, sign_out, inv, c)
+    if (filled == 1) { CTMI_SQP(false); } else { CTMI_SQP(true); }
+#undef CTMI_SQP
+    return;
+  }
+  const int64_t wgs = cdiv(n_groups, kHqpWaves * CTMI_HQP_GROUPS);
   const int64_t cap = 256 * CTMI_HQP_WG_PER_CU;
   const unsigned grid = (unsigned)(wgs < cap ? wgs : cap);
-  const float inv = 1.0f / sqrtf((float)b_dim);
 #define CTMI_HQP(BB)                                                                             \
   if (filled == 1)                                                                               \
     hipLaunchKernelGGL((hadamard_quant_pack_kernel<BB, false>), grid, kHqpThreads, 0, st, t,     \
@@ -1300,8 +1606,10 @@ extern "C" int ctmi_hadamard_quant_pack_many(const ctmi_hadamard_pack_job* jobs,
     rc = hqp_check_job(jobs[i], b_dim);
     if (rc) return rc;
   }
-  CTMI_REQUIRE(n_jobs == 0 || (mb_t && (uintptr_t)mb_t % 16 == 0), CTMI_ERR_VALUE,
-               "the matrix must be given, 16-byte aligned");
+  CTMI_REQUIRE((mb_t || b_dim == 128) && (uintptr_t)mb_t % 16 == 0, CTMI_ERR_VALUE,
+               "the matrix must be given, 16-byte aligned (NULL stands for Sylvester's matrix of 128)");
+  CTMI_REQUIRE(mb_t || ((uintptr_t)sign_in % 16 == 0 && (uintptr_t)sign_out % 16 == 0), CTMI_ERR_VALUE,
+               "sign vectors must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   HadJobs t;
   clear_jobs(&t);

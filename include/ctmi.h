@@ -563,7 +563,13 @@ int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n_jobs, int3
  * by the min-max observer, calculate_qparams and the quantize + pack_to_int32 of
  * ctmi_pack_quantized_compress.  Same bits as those calls in sequence.
  * packed: int32 [numel / 8]; scale: bf16 [numel / b_dim] (the group scales, row
- * major); rotated: optional bf16 [numel] copy of the rotated tensor, or NULL. */
+ * major); rotated: optional bf16 [numel] copy of the rotated tensor, or NULL.
+ * mb_t == NULL with b_dim == 128 stands for Sylvester's matrix of that order (what
+ * deterministic_hadamard_matrix and random_hadamard_matrix build at this size,
+ * transform/utils/hadamard.py:38-100): no matrix is read, and workgroups stream through
+ * the tensor without a set-up phase; the sign vectors must then be 16-byte aligned.  A
+ * rotated output that is exactly zero carries the sign of its sign_out entry there (-0
+ * where the kernel with a matrix gives +0); codes and scales do not depend on it. */
 int ctmi_hadamard_quant_pack(const void* x, int32_t io_dtype, int64_t numel, int32_t b_dim,
                              const void* mb_t, const float* sign_in, const float* sign_out,
                              int32_t num_bits, int32_t symmetric, int32_t* packed, void* scale,
