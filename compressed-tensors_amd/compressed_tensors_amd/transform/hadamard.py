@@ -232,6 +232,12 @@ def _aligned(*tensors) -> bool:
     return all(t is None or t.data_ptr() % 16 == 0 for t in tensors)
 
 
+def _matrix_free(n: int, dtype, *tensors) -> bool:
+    """does the fused rotation + quantization by Sylvester's matrix of order n run without a
+    matrix argument?"""
+    return n == 128 and dtype == torch.bfloat16 and _aligned(*tensors)
+
+
 def hadamard_apply(
     value: Tensor,
     n: int,
@@ -272,7 +278,7 @@ def hadamard_apply(
     out = torch.empty_like(x)
     _lib.check(
         lib.ctmi_hadamard_apply(
-            x.data_ptr(), out.data_ptr(), code, x.numel(), a, b, _lib.ptr(ma_t), mb_t.data_ptr(),
+            x.data_ptr(), out.data_ptr(), code, x.numel(), a, b, _lib.ptr(ma_t), _lib.ptr(mb_t),
             _lib.ptr(s_in), _lib.ptr(s_out), _lib.stream_of(dev),
         )
     )
@@ -400,7 +406,7 @@ def _quantize_pack(values, n, args, sign_in, sign_out, matrix_t, return_rotated,
         mb_t = None
         if matrix_t is not None:
             mb_t = matrix_t.to(device=dev, dtype=torch.bfloat16).contiguous()
-        elif n != 128 or not _aligned(s_in, s_out):
+        elif not _matrix_free(n, torch.bfloat16, s_in, s_out):
             mb_t = _sylvester_bf16(n, dev)
         _lib.check(lib.ctmi_hadamard_quant_pack_many(
             jobs, len(xs), code, n, _lib.ptr(mb_t), _lib.ptr(s_in), _lib.ptr(s_out), 4, 1, stream))
@@ -467,7 +473,7 @@ def hadamard_apply_many(
     for job, x, out in zip(jobs, xs, outs):
         job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()
     _lib.check(
-        lib.ctmi_hadamard_apply_many(jobs, len(xs), code, a, b, _lib.ptr(ma_t), mb_t.data_ptr(),
+        lib.ctmi_hadamard_apply_many(jobs, len(xs), code, a, b, _lib.ptr(ma_t), _lib.ptr(mb_t),
                                      _lib.ptr(s_in), _lib.ptr(s_out), _lib.stream_of(dev))
     )
     return outs
