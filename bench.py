@@ -162,7 +162,7 @@ class Op:
     fused operation replaces, one call per weight against one call for all)"""
 
     def __init__(self, name, calls, nbytes, kernel, primary=True, mfma_flops=None, launches=None,
-                 useful_flops=None):
+                 useful_flops=None, passes_bytes=None):
         self.name, self.calls, self.nbytes, self.kernel = name, calls, nbytes, kernel
         self.primary = primary
         self.mfma_flops = mfma_flops  # flops the kernel issues on the matrix cores, per pass
@@ -171,6 +171,11 @@ class Op:
         self.useful_flops = mfma_flops if useful_flops is None else useful_flops
         # launches of `kernel` per pass: one per call unless a call chains several
         self.launches = len(calls) if launches is None else launches
+        # bytes the operation has to move when its result needs more than one pass over the
+        # input (sparse-bitmask compression: the values' positions depend on a prefix sum over
+        # the whole tensor, so the tensor is read once for the mask and counts and once more
+        # to be compacted): the floor of the method, next to the format's algorithmic bytes
+        self.passes_bytes = passes_bytes
         self.ms = 0.0
 
 
@@ -420,7 +425,11 @@ def other_workload(torch, name, seed):
         bm_bytes = copies * (2 * nb + nb // 8 + 8 * 8192) + 2 * nnz_total
         s24_bytes = copies24 * (n24 + n24 // 2 + n24 // 8)
         fused24_bytes = copies24 * (2 * n24 + n24 // 2 + n24 // 8)  # what the one-pass form has to move
-        ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes, "bitmask_compact_rows_kernel"),
+        # two passes over the dense tensor: (dense in, bitmask + counts out), a scan of the counts,
+        # (dense + bitmask + offsets in, values out)
+        bm_passes = copies * (2 * 2 * nb + 2 * (nb // 8) + 3 * 8 * 8192) + 2 * nnz_total
+        ops = [Op("sparse-bitmask compress, 8192x8192 bf16, 50 % zeros (mask+offsets, then compaction)", c_calls, bm_bytes,
+                  "bitmask_compact_rows_kernel", passes_bytes=bm_passes),
                Op("sparse-bitmask decompress (positions from the bitmask alone)", d_calls, bm_bytes, "bitmask_scatter_tiles_kernel"),
                Op("sparse-24-bitmask compress, 14336x4096 fp8", s_calls, s24_bytes, "sparse24_compress_kernel"),
                Op("sparse-24-bitmask decompress", t_calls, s24_bytes, "sparse24_scatter_kernel"),
@@ -912,6 +921,9 @@ def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True, only
                "ms": op.ms, "algorithmic_bytes": op.nbytes,
                "for_comparison_only": not op.primary}
         row["launches"] = op.launches
+        if op.passes_bytes is not None:
+            row["bytes_of_its_passes"] = op.passes_bytes
+            row["frac_of_hbm_peak_on_bytes_of_its_passes"] = op.passes_bytes / (op.ms * 1e-3) / 1e9 / HBM_PEAK_GBS
         if op.mfma_flops is not None:
             row["mfma_TFLOPs"] = op.mfma_flops / (op.ms * 1e-3) / 1e12
             row["mfma_utilisation"] = op.mfma_flops / (op.ms * 1e-3) / MFMA_BF16_PEAK
