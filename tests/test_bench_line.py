@@ -66,6 +66,8 @@ def test_stdout_line_is_short_and_complete(tmp_path):
     for key in ("value", "unit", "cores", "kind", "sample"):
         assert key in line["cpu_baseline"], key
     assert set(line["configs_frac"]) == set(bench.OTHER_WORKLOADS)
+    whole, slowest = line["configs_frac"]["sparse"]
+    assert abs(whole - 1e9 / 0.123456 / 1e6 / 8000.0) < 5e-3 and abs(slowest - 0.1543) < 1e-3  # three digits
     assert abs(line["api_level"]["frac_of_hbm_peak"] - 0.4879) < 1e-4
     assert abs(line["roofline"]["frac"] - out["roofline"]["frac"]) < 1e-3
 
