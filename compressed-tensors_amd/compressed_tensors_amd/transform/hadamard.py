@@ -140,17 +140,32 @@ def load_hadamard_table(path: Optional[str] = None) -> Dict[int, Tensor]:
     return _table_cache[path]
 
 
+_sylvester_entries: Dict[str, Dict[int, bool]] = {}
+
+
+def _is_sylvester_entry(path: str, k: int, block: Tensor) -> bool:
+    """does entry k of the table at `path` equal Sylvester's matrix?  Compared once per
+    (path, k)."""
+    seen = _sylvester_entries.setdefault(os.path.abspath(path), {})
+    if k not in seen:
+        seen[k] = is_pow2(k) and torch.equal(block, deterministic_hadamard_matrix(k, torch.int8))
+    return seen[k]
+
+
 def known_hadamard_block(n: int, table_path: Optional[str] = None) -> Tuple[int, Optional[Tensor]]:
     """(K, H_K) as the reference's _fetch_hadamard_divisor picks it (hadamard.py:102-129):
-    the largest K of the table with n / K a power of two.  For a power of two n other than
-    32 that block is Sylvester's matrix of order min(n, 256) - true of the reference's
-    table - and no table is needed: returns (K, None)."""
-    if is_pow2(n) and n != 32:
+    the largest K of the table with n / K a power of two.  H_K is None where the block is
+    Sylvester's matrix, so that the whole transform is Sylvester(n): an entry of the table
+    is compared with Sylvester's matrix before that is said of it.  With no table at hand a
+    power of two other than 32 gives (min(n, 256), None), which is what the reference's
+    table holds."""
+    path = table_path or _default_table_path()
+    if path is None and is_pow2(n) and n != 32:
         return min(n, 256), None
-    table = load_hadamard_table(table_path)
+    table = load_hadamard_table(path)
     for k in sorted(table, reverse=True):
         if n % k == 0 and is_pow2(n // k):
-            return k, table[k]
+            return k, (None if _is_sylvester_entry(path, k, table[k]) else table[k])
     raise ValueError(f"Cannot construct random hadamard matrix of size {n}")
 
 

@@ -196,6 +196,31 @@ def test_table_loader_rejects_what_is_not_hadamard(tmp_path, hadamard_table_path
     assert known_hadamard_block(4096) == (256, None) and known_hadamard_block(16) == (16, None)
 
 
+def test_power_of_two_entry_of_a_table_is_compared_with_sylvester(tmp_path):
+    """a table whose entry for 4 is a Hadamard matrix other than Sylvester's is used as it
+    is; one that holds Sylvester's matrix takes the matrix-free route (block None)"""
+    from safetensors.torch import save_file
+
+    from compressed_tensors_amd.transform import (
+        deterministic_hadamard_matrix, known_hadamard_block, random_hadamard_matrix)
+
+    syl = deterministic_hadamard_matrix(4, torch.int8)
+    other = syl[[1, 0, 2, 3]].contiguous()
+    other[2] = -other[2]
+    plain, odd = tmp_path / "plain.safetensors", tmp_path / "odd.safetensors"
+    save_file({"4": syl}, str(plain))
+    save_file({"4": other}, str(odd))
+    assert known_hadamard_block(16, str(plain)) == (4, None)
+    k, block = known_hadamard_block(16, str(odd))
+    assert k == 4 and torch.equal(block, other)
+    g1, g2 = torch.Generator().manual_seed(5), torch.Generator().manual_seed(5)
+    want = oh.random_hadamard_matrix(16, dtype=torch.float32, gen=g1, table={4: other})
+    got = random_hadamard_matrix(16, torch.float32, gen=g2, table_path=str(odd))
+    assert torch.equal(got, want)
+    assert not torch.equal(got, random_hadamard_matrix(
+        16, torch.float32, gen=torch.Generator().manual_seed(5), table_path=str(plain)))
+
+
 def test_matrix_core_split_follows_the_largest_block_rule(ctmi, hadamard_table_path):
     """host logic only (the library's `supported` queries touch no GPU): for the sizes the
     reference builds from its table - the largest block that leaves a power of two,
