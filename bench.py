@@ -64,16 +64,29 @@ PROFILES = ROOT / "profiles"
 MFMA_BF16_PEAK = 2.5e15  # dense bf16 MFMA, published peak
 
 
-def measured_traffic(workload, kernel):
+def measured_traffic(workload, kernel, operation=None):
     """HBM bytes per launch from the committed counter summaries: lines of the form
-    `traffic_bytes_per_launch <workload> <kernel> <bytes>` in profiles/*pmc_traffic*.txt
-    (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, KiB per dispatch, each scaled by what
-    the same counter reads for a plain 1 GiB copy).  -> (bytes or None, file name or None)"""
+    `traffic_bytes_per_launch <workload> <kernel> <bytes> [op=<operation>]` in
+    profiles/*pmc_traffic*.txt (rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE, KiB per
+    dispatch, each scaled by what the same counter reads for a plain 1 GiB copy).  A line
+    that names the operation (counters of a run with --only-op) wins over one for the kernel
+    alone; where a kernel has lines with operations and none of them is this one, nothing is
+    returned (another operation's launches move other bytes).
+    -> (bytes or None, file name or None)"""
+    by_kernel, tagged = None, False
     for path in sorted(PROFILES.glob("*pmc_traffic*.txt")):
         for line in path.read_text().splitlines():
-            f = line.split()
-            if len(f) == 4 and f[0] == "traffic_bytes_per_launch" and f[1] == workload and f[2] == kernel:
-                return float(f[3]), f"profiles/{path.name}"
+            f = line.split(None, 4)
+            if len(f) < 4 or f[0] != "traffic_bytes_per_launch" or f[1] != workload or f[2] != kernel:
+                continue
+            if len(f) == 5:
+                tagged = True
+                if operation is not None and f[4].strip() == "op=" + operation:
+                    return float(f[3]), f"profiles/{path.name}"
+            elif by_kernel is None:
+                by_kernel = (float(f[3]), f"profiles/{path.name}")
+    if by_kernel is not None and not tagged:
+        return by_kernel
     return None, None
 
 
@@ -307,8 +320,8 @@ def other_workload(torch, name, seed):
             a_dyn.append(dynamic(x, out, 4096, targs))
             acts.append(x)
         na = 8 * 8192 * 4096
-        ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_kernel", launches=chained(len(entries))),
-               Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_kernel", launches=chained(len(entries))),
+        ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_many_kernel", launches=chained(len(entries))),
+               Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_many_kernel", launches=chained(len(entries))),
                Op("weights one-shot: per-channel observer (224 calls)", w_obs, 2 * n, "observe_wide_kernel", primary=False),
                Op("weights one-shot: quantize with those scales (224 calls)", w_q, 3 * n, "qdq_vec_kernel", primary=False),
                Op("weights one-shot: scales + fp8 codes in one pass (224 calls)", w_one, 3 * n, "dynamic_rows_kernel", primary=False),
@@ -900,10 +913,11 @@ def cpu_baseline_other(torch, workload, seed):
 def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True, only_op=None):
     """one of the other configurations -> its result object (same fields as the headline
     line, plus the per-operation table).  only_op: time just the operations whose name contains
-    this text (a counter run then sees the launches of that operation and no others)"""
+    this text, or equals it after a leading "=" (a counter run then sees the launches of that operation and no others)"""
     metric, ops, keep = other_workload(torch, workload, seed)
     if only_op:
-        ops = [op for op in ops if only_op in op.name]
+        exact = only_op.startswith("=")
+        ops = [op for op in ops if (op.name == only_op[1:] if exact else only_op in op.name)]
         if not ops:
             raise SystemExit(f"no operation of {workload} is named like {only_op!r}")
         for op in ops:
@@ -915,7 +929,7 @@ def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True, only
     # operations aside); every operation's own rate is in `operations`
     slow = max((op for op in ops if op.primary), key=lambda op: op.ms)
     n_launch = slow.launches
-    traffic, traffic_source = measured_traffic(workload, slow.kernel)
+    traffic, traffic_source = measured_traffic(workload, slow.kernel, slow.name)
 
     def op_row(op):
         row = {"name": op.name, "kernel": op.kernel, "GBs": op.nbytes / (op.ms * 1e-3) / 1e9,

@@ -647,9 +647,10 @@ int ctmi_kron_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, 
 int ctmi_block_matmul(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t h,
                       const float* w, void* stream);
 
-/* Plain device-to-device copy of `bytes` bytes (a multiple of 16): the known
- * quantity against which hardware byte counters are calibrated when profiling.
- * No counterpart in the reference. */
+/* Diagnostics, not part of the path: a plain device-to-device copy of `bytes` bytes (a
+ * multiple of 16), the known quantity against which hardware byte counters are calibrated
+ * when profiling (bench.py --calib-copies).  Nothing in the library or its host mirror
+ * calls it.  No counterpart in the reference. */
 int ctmi_calib_copy(const void* src, void* dst, int64_t bytes, void* stream);
 
 /* The 4096-entry keep table used by the 2:4 kernels (host copy, for tests). */
