@@ -990,18 +990,28 @@ def run_other(torch, workload, seed, steps, warmup, with_cpu_baseline=True, only
     return out
 
 
-def api_level(torch, seed, steps):
+API_FORMATS = (
+    # format, weight scheme, algorithmic bytes per element and direction
+    ("pack-quantized", dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP),
+     2 + 2 / GROUP + 0.5),
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel"), 3.0),
+    ("nvfp4-pack-quantized", dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group",
+                                  group_size=16), 2 + 1 / 16 + 0.5),
+)
+
+
+def api_level_format(torch, seed, steps, fmt, spec, bytes_per_element):
     """ModelCompressor.compress_model + decompress_model on a module tree of 224 bf16 Linear
-    layers with the Llama-3-8B shapes (scales attached beforehand by the observer): the cost
-    of the host mirror above the C ABI, next to the kernel-level headline"""
+    layers with the Llama-3-8B shapes (scales attached beforehand by the observer), one format"""
     from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
     from compressed_tensors_amd.quantization import (
         QuantizationArgs, QuantizationConfig, QuantizationScheme, observe_weight_qparams,
     )
+    from compressed_tensors_amd.quantization.helpers import generate_gparam
 
     dev = torch.device("cuda:0")
     gen = torch.Generator(device=dev).manual_seed(seed)
-    args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
+    args = QuantizationArgs(**spec)
 
     class Layer(torch.nn.Module):
         def __init__(self):
@@ -1016,18 +1026,23 @@ def api_level(torch, seed, steps):
     model = torch.nn.Module()
     model.layers = torch.nn.ModuleList([Layer() for _ in range(32)])
     config = QuantizationConfig(
-        config_groups={"group_0": QuantizationScheme(targets=["Linear"], weights=args)},
-        format="pack-quantized")
+        config_groups={"group_0": QuantizationScheme(targets=["Linear"], weights=args)}, format=fmt)
     apply_quantization_scheme(model, config)
     n = 0
     for m in model.modules():
         if isinstance(m, torch.nn.Linear):
-            scale, zp = observe_weight_qparams(m.weight.data, args)
+            if spec["strategy"] == "tensor_group":
+                lo, hi = torch.aminmax(m.weight.data)
+                gs = generate_gparam(lo.reshape(1), hi.reshape(1))
+                m.register_parameter("weight_global_scale", torch.nn.Parameter(gs, requires_grad=False))
+                scale, zp = observe_weight_qparams(m.weight.data, args, global_scale=gs)
+            else:
+                scale, zp = observe_weight_qparams(m.weight.data, args)
             m.register_parameter("weight_scale", torch.nn.Parameter(scale, requires_grad=False))
             m.register_parameter("weight_zero_point", torch.nn.Parameter(zp, requires_grad=False))
             n += m.weight.numel()
     mc = ModelCompressor(quantization_config=config)
-    per_dir = 2 * n + 2 * (n // GROUP) + n // 2
+    per_dir = bytes_per_element * n
     comp, deco = [], []
     for it in range(steps + 1):  # first pass is the warm-up
         torch.cuda.synchronize()
@@ -1042,16 +1057,28 @@ def api_level(torch, seed, steps):
             comp.append(t1 - t0)
             deco.append(t2 - t1)
     c_s, d_s = statistics.median(comp), statistics.median(deco)
+    del model, mc
+    torch.cuda.empty_cache()
     return {
-        "what": "ModelCompressor.compress_model + decompress_model, 224 torch.nn.Linear (bf16, on the "
-                "GPU) of the Llama-3-8B shapes, pack-quantized W4A16 g128, wall time incl. the Python "
-                "harness, parameter swaps and allocation of the outputs",
         "compress_model_ms": c_s * 1e3, "decompress_model_ms": d_s * 1e3,
         "compress_GBs": per_dir / c_s / 1e9, "decompress_GBs": per_dir / d_s / 1e9,
         "roundtrip_GBs": 2 * per_dir / (c_s + d_s) / 1e9,
         "frac_of_hbm_peak": 2 * per_dir / (c_s + d_s) / 1e9 / HBM_PEAK_GBS,
         "passes": steps, "statistic": "median",
     }
+
+
+def api_level(torch, seed, steps):
+    """the cost of the host mirror above the C ABI, next to the kernel-level figures: the
+    headline's format at the top level of the result, the int8 / fp8 and nvfp4 formats under
+    `other_formats`"""
+    out = {"what": "ModelCompressor.compress_model + decompress_model, 224 torch.nn.Linear (bf16, on the "
+                   "GPU) of the Llama-3-8B shapes, pack-quantized W4A16 g128, wall time incl. the Python "
+                   "harness, parameter swaps and allocation of the outputs"}
+    out.update(api_level_format(torch, seed, steps, *API_FORMATS[0]))
+    out["other_formats"] = {fmt: api_level_format(torch, seed, steps, fmt, spec, bpe)
+                            for fmt, spec, bpe in API_FORMATS[1:]}
+    return out
 
 
 OTHER_WORKLOADS = ("fp8-w8a8", "sparse", "nvfp4", "hadamard", "one-shot")
@@ -1100,6 +1127,8 @@ def short_line(out, details_path=None):
         line["mfma_frac"] = _sig(out["mfma_utilisation"]["frac"], 3)
     if "api_level" in out:
         line["api_level"] = pick(out["api_level"], ("frac_of_hbm_peak", "compress_model_ms", "decompress_model_ms"))
+        for fmt, res in out["api_level"].get("other_formats", {}).items():
+            line["api_level"][fmt] = _sig(res["frac_of_hbm_peak"], 3)
     if details_path:
         line["details"] = os.path.relpath(details_path, ROOT)
     text = json.dumps(line, separators=(",", ":"))

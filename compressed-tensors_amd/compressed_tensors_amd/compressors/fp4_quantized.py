@@ -12,6 +12,9 @@ from torch import Tensor
 
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
+from compressed_tensors_amd.compressors.job_tables import (
+    FLOAT_DTYPES, args_key, module_chunks, module_table, slab_outputs,
+)
 from compressed_tensors_amd.compressors.quantized_base import (
     BaseQuantizationCompressor, LazyDenseOutputs,
 )
@@ -325,6 +328,130 @@ def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progre
 
 
 NVFP4PackedCompressor.compress = _compress_state_dict_batched
+
+
+# ---------------------------------------------------------------------------------------------
+# Module pathways (ModelCompressor.compress_model / decompress_model): a 2-D float weight on the
+# GPU with fp8 group scales and an fp32 global scale goes into a job table written by columns;
+# everything else takes the state-dict path.
+_OWN = ("weight", "weight_packed", "weight_scale", "weight_zero_point", "weight_global_scale", "bias")
+_SCALE_DTYPES = FLOAT_DTYPES + (torch.float8_e4m3fn,)
+
+
+def _own_only(params) -> bool:
+    for name, p in params.items():
+        if p is not None and name not in _OWN:
+            return False
+    return True
+
+
+def _table_ready(t, device) -> bool:
+    return t is not None and t.device == device and t.is_contiguous()
+
+
+def _compress_modules_fast(self, members, names_to_scheme) -> None:
+    """NVFP4PackedCompressor.compress_modules: compress_module (compressors/base.py:125-151,
+    fp4_quantized.py:84-106) for every (prefix, module) pair, one ctmi_nvfp4_compress_many
+    call per 64"""
+    entry = _lib.load().ctmi_nvfp4_compress_many
+    table = module_table(self)
+    new_param = torch.nn.Parameter
+    slow, arg_keys = [], {}
+    for lo, hi in module_chunks(len(members)):
+        picked, shapes, device = [], [], None
+        for prefix, module in members[lo:hi]:
+            params = module._parameters
+            w, scale, zp, gs = (params.get(n) for n in ("weight", "weight_scale", "weight_zero_point",
+                                                        "weight_global_scale"))
+            args = names_to_scheme[prefix].weights
+            key = arg_keys.get(id(args))
+            if key is None:
+                key = arg_keys[id(args)] = args_key(args)
+            if (w is None or w.ndim != 2 or w.numel() == 0 or w.shape[1] % 2 or w.dtype not in FLOAT_DTYPES
+                    or w.device.type != "cuda" or not w.is_contiguous()
+                    or not _table_ready(scale, w.device) or scale.dtype not in _SCALE_DTYPES or scale.ndim != 2
+                    or not _table_ready(gs, w.device) or gs.dtype is not torch.float32 or gs.numel() != 1
+                    or (zp is not None and not _table_ready(zp, w.device))
+                    or not _own_only(params) or (device is not None and device != w.device)):
+                slow.append((prefix, module))
+                continue
+            device = w.device
+            picked.append((params, w, scale, zp, gs, args, key))
+            shapes.append((w.shape[0], w.shape[1] // 2))
+        if not picked:
+            continue
+        packed = slab_outputs(shapes, torch.uint8, device)
+        for (params, w, scale, zp, gs, args, key), out in zip(picked, packed):
+            rows, cols = w.shape
+            tkey = ("c", rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
+            which = table.template(tkey)
+            if which < 0:
+                which = table.add_template(tkey, build_qparams(w, scale, zp, args, None, gs))
+            table.add(w.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(w.dtype), which,
+                      scale.data_ptr(), 0 if zp is None else zp.data_ptr(), gs.data_ptr())
+        table.launch(entry, _lib.stream_of(device))
+        # the kernels are enqueued: the modules get their new parameters while the GPU works
+        for (params, w, scale, zp, gs, args, key), out in zip(picked, packed):
+            rest = [(n, p) for n, p in params.items()
+                    if n not in ("weight", "weight_packed") and not (n == "weight_zero_point" and args.symmetric)]
+            params.clear()
+            params["weight_packed"] = new_param(out, requires_grad=False)
+            params.update(rest)
+    if slow:
+        BaseQuantizationCompressor.compress_modules(self, slow, names_to_scheme)
+
+
+def _decompress_modules_fast(self, members, names_to_scheme) -> None:
+    """NVFP4PackedCompressor.decompress_modules: decompress_module (compressors/base.py:165-190,
+    fp4_quantized.py:108-123) for every (prefix, module) pair"""
+    entry = _lib.load().ctmi_nvfp4_decompress_many
+    table = module_table(self)
+    new_param = torch.nn.Parameter
+    slow = []
+    for lo, hi in module_chunks(len(members)):
+        picked, shapes, device = [], [], None
+        for prefix, module in members[lo:hi]:
+            params = module._parameters
+            packed, scale, gs = (params.get(n) for n in ("weight_packed", "weight_scale", "weight_global_scale"))
+            if (packed is None or packed.dtype is not torch.uint8 or packed.ndim != 2 or packed.numel() == 0
+                    or packed.device.type != "cuda" or not packed.is_contiguous()
+                    or not _table_ready(scale, packed.device) or scale.dtype not in _SCALE_DTYPES
+                    or scale.ndim != 2 or scale.shape[0] != packed.shape[0] or scale.shape[1] <= 1
+                    or (2 * packed.shape[1]) % scale.shape[1]
+                    or not _table_ready(gs, packed.device) or gs.dtype is not torch.float32 or gs.numel() != 1
+                    or params.get("weight_zero_point") is not None
+                    or not _own_only(params) or (device is not None and device != packed.device)):
+                slow.append((prefix, module))
+                continue
+            device = packed.device
+            picked.append((params, packed, scale, gs))
+            shapes.append((packed.shape[0], 2 * packed.shape[1]))
+        if not picked:
+            continue
+        # (several groups per row: the reference's group path, which honours the bf16 it asks for)
+        dense = slab_outputs(shapes, torch.bfloat16, device)
+        out_code = _lib.dtype_code(torch.bfloat16)
+        for (params, packed, scale, gs), out, shape in zip(picked, dense, shapes):
+            tkey = ("d", shape, scale.shape, scale.dtype)
+            which = table.template(tkey)
+            if which < 0:
+                carrier = _ShapeOnly(torch.Size(shape), torch.bfloat16)
+                plan = build_qparams(carrier, scale, None, infer_dequant_args(carrier, scale), None, gs)
+                if not plan.grouped:
+                    raise RuntimeError(f"group scales expected, got shape {tuple(scale.shape)}")
+                plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_FLOAT, 4
+                which = table.add_template(tkey, plan)
+            table.add(packed.data_ptr(), out.data_ptr(), shape[0], shape[1], out_code, which,
+                      scale.data_ptr(), 0, gs.data_ptr())
+        table.launch(entry, _lib.stream_of(device))
+        for (params, packed, scale, gs), out in zip(picked, dense):
+            params["weight"] = new_param(out, requires_grad=False)
+    if slow:
+        BaseQuantizationCompressor.decompress_modules(self, slow, names_to_scheme)
+
+
+NVFP4PackedCompressor.compress_modules = _compress_modules_fast
+NVFP4PackedCompressor.decompress_modules = _decompress_modules_fast
 
 
 @BaseCompressor.register(name=CompressionFormat.mxfp4_pack_quantized.value)

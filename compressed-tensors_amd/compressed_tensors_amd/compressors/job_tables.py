@@ -16,24 +16,35 @@ import torch
 
 from compressed_tensors_amd import _lib
 
-__all__ = ["WeightJobTable", "slab_outputs"]
+__all__ = ["WeightJobTable", "slab_outputs", "module_table", "module_chunks", "args_key", "FLOAT_DTYPES"]
 
-_JOB = np.dtype(_lib.WeightJob)
 _QP = np.dtype(_lib.QParams)
-assert _JOB.itemsize == ctypes.sizeof(_lib.WeightJob) and _QP.itemsize == ctypes.sizeof(_lib.QParams)
-_JOB_PTR = ctypes.POINTER(_lib.WeightJob)
+assert _QP.itemsize == ctypes.sizeof(_lib.QParams)
+
+FLOAT_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+_CHUNK_MODULES = 64   # modules per call of the C ABI on the module pathways
 
 _SLAB_BYTES = 1 << 30   # outputs of one shape share an allocation up to this size
 _ALIGN = 256            # ... if each of them keeps this alignment inside it
 
 
 class WeightJobTable:
-    """Rows are added with `add`; `launch` writes them into a `ctmi_weight_job` array and
-    hands it to a many-weight entry point.  `add_template` registers the part of a job's
-    qparams that holds no scale or zero-point address (as `build_qparams` made it for one
-    weight of the combination; its other addresses must be NULL)."""
+    """Rows are added with `add`; `launch` writes them into an array of `job_struct` and hands
+    it to a many-weight entry point.  `add_template` registers the part of a job's qparams
+    that holds no scale, zero-point or global-scale address (as `build_qparams` made it for
+    one weight of the combination).
 
-    def __init__(self):
+    job_struct: `ctmi_weight_job` (source, destination, rows, cols, dtype of the dense side,
+    reserved, qparams) or `ctmi_qdq_job`, which has the same layout with the dtypes of input
+    and output in the two 32-bit members."""
+
+    def __init__(self, job_struct=_lib.WeightJob):
+        self._job = np.dtype(job_struct)
+        assert self._job.itemsize == ctypes.sizeof(job_struct)
+        names = self._job.names
+        assert len(names) == 7 and names[2:4] == ("rows", "cols") and names[6] == "qp"
+        self._f_src, self._f_dst, self._f_dtype, self._f_dtype2 = names[0], names[1], names[4], names[5]
+        self._job_ptr = ctypes.POINTER(job_struct)
         self._templates: List[np.ndarray] = []
         self._template_of: Dict[Tuple, int] = {}
         self.clear()
@@ -42,6 +53,7 @@ class WeightJobTable:
         """drop the rows added since the last launch"""
         self.src, self.dst, self.rows, self.cols, self.dense_dtype = [], [], [], [], []
         self.scale, self.zero_point, self.which = [], [], []
+        self.global_scale, self.second_dtype = [], []
 
     @property
     def n_templates(self) -> int:
@@ -53,47 +65,76 @@ class WeightJobTable:
 
     def add_template(self, key, plan) -> int:
         qp = np.frombuffer(bytes(plan.qp), dtype=_QP).copy()
-        if int(qp["col_group"][0]) or int(qp["global_scale"][0]):
-            raise ValueError("a template cannot hold the address of a column-group table or a global scale")
+        if int(qp["col_group"][0]):
+            raise ValueError("a template cannot hold the address of a column-group table")
         qp["scale"] = 0
         qp["zero_point"] = 0
+        qp["global_scale"] = 0
         self._templates.append(qp)
         self._stacked = np.concatenate(self._templates)
         self._template_of[key] = len(self._templates) - 1
         return len(self._templates) - 1
 
     def add(self, src: int, dst: int, rows: int, cols: int, dense_dtype: int, which: int,
-            scale: int, zero_point: int = 0) -> None:
+            scale: int, zero_point: int = 0, global_scale: int = 0, second_dtype: int = 0) -> None:
+        """dense_dtype / second_dtype: the two 32-bit members of the job (ctmi_weight_job: dtype
+        of the dense side, reserved; ctmi_qdq_job: dtype of the input, of the output)"""
         self.src.append(src)
         self.dst.append(dst)
         self.rows.append(rows)
         self.cols.append(cols)
         self.dense_dtype.append(dense_dtype)
+        self.second_dtype.append(second_dtype)
         self.which.append(which)
         self.scale.append(scale)
         self.zero_point.append(zero_point)
+        self.global_scale.append(global_scale)
 
     def __len__(self):
         return len(self.src)
 
-    def launch(self, entry, stream: int) -> None:
-        """one call of `entry(jobs, n, stream)` for the rows added since the last launch"""
+    def launch(self, entry, *args) -> None:
+        """one call of `entry(jobs, n, *args)` for the rows added since the last launch"""
         n = len(self.src)
         if n == 0:
             return
-        tab = np.zeros(n, _JOB)
-        tab["src"] = self.src
-        tab["dst"] = self.dst
+        tab = np.zeros(n, self._job)
+        tab[self._f_src] = self.src
+        tab[self._f_dst] = self.dst
         tab["rows"] = self.rows
         tab["cols"] = self.cols
-        tab["dense_dtype"] = self.dense_dtype
+        tab[self._f_dtype] = self.dense_dtype
+        tab[self._f_dtype2] = self.second_dtype
         qp = self._stacked[self.which]
         qp["scale"] = self.scale
         qp["zero_point"] = self.zero_point
+        qp["global_scale"] = self.global_scale
         tab["qp"] = qp
         self.clear()
         # the entry points read the table before they return: it need not outlive the call
-        _lib.check(entry(ctypes.cast(tab.ctypes.data, _JOB_PTR), n, stream))
+        _lib.check(entry(ctypes.cast(tab.ctypes.data, self._job_ptr), n, *args))
+
+
+def module_chunks(n):
+    """(lo, hi) ranges of at most 64 modules"""
+    for at in range(0, n, _CHUNK_MODULES):
+        yield at, min(at + _CHUNK_MODULES, n)
+
+
+def module_table(compressor, job_struct=_lib.WeightJob) -> WeightJobTable:
+    """the compressor's job table for the module pathways: its templates (the pointer-free
+    part of a weight's qparams per shape / dtype / scheme) stay valid from call to call"""
+    table = compressor.__dict__.get("_table")
+    if table is None or table.n_templates > 512:
+        table = compressor.__dict__["_table"] = WeightJobTable(job_struct)
+    table.clear()  # rows a failed call may have left behind
+    return table
+
+
+def args_key(args):
+    """what of a QuantizationArgs decides a weight's qparams plan"""
+    return (args.num_bits, args.type, args.symmetric, args.strategy, args.group_size,
+            None if args.block_structure is None else tuple(args.block_structure))
 
 
 def slab_outputs(shapes: List[Tuple[int, ...]], dtype: torch.dtype, device) -> List[torch.Tensor]:

@@ -10,6 +10,9 @@ from torch import Tensor
 
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
+from compressed_tensors_amd.compressors.job_tables import (
+    FLOAT_DTYPES, args_key, module_chunks, module_table, slab_outputs,
+)
 from compressed_tensors_amd.compressors.quantized_base import (
     BaseQuantizationCompressor, LazyDenseOutputs,
 )
@@ -333,6 +336,124 @@ def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progre
 
 
 NaiveQuantizationCompressor.compress = _compress_state_dict_batched
+
+
+# ---------------------------------------------------------------------------------------------
+# Module pathways (ModelCompressor.compress_model / decompress_model): the common case - a 2-D
+# float weight on the GPU whose module holds nothing but weight, scale, zero point and bias -
+# goes into a job table written by columns; everything else takes the state-dict path.
+_PLAIN = ("weight", "weight_scale", "weight_zero_point", "bias")
+
+
+def _plain(params) -> bool:
+    """no activation ordering, no global scale, no activation qparams: nothing the table
+    would have to carry besides scale and zero point"""
+    for name, p in params.items():
+        if p is not None and name not in _PLAIN:
+            return False
+    return True
+
+
+def _compress_modules_fast(self, members, names_to_scheme) -> None:
+    """NaiveQuantizationCompressor.compress_modules: compress_module (compressors/base.py:125-151,
+    naive_quantized.py:79-114) for every (prefix, module) pair, one ctmi_qdq_many call per 64"""
+    entry = _lib.load().ctmi_qdq_many
+    table = module_table(self, _lib.QdqJob)
+    new_param = torch.nn.Parameter
+    slow, arg_keys = [], {}
+    for lo, hi in module_chunks(len(members)):
+        picked, shapes, device, code_dtype = [], [], None, None
+        for prefix, module in members[lo:hi]:
+            params = module._parameters
+            w, scale, zp = params.get("weight"), params.get("weight_scale"), params.get("weight_zero_point")
+            args = names_to_scheme[prefix].weights
+            key = arg_keys.get(id(args))
+            if key is None:
+                key = arg_keys[id(args)] = (args_key(args), args.pytorch_dtype() if args.num_bits <= 8 else None)
+            if (w is None or scale is None or w.ndim != 2 or w.numel() == 0 or w.dtype not in FLOAT_DTYPES
+                    or w.device.type != "cuda" or not w.is_contiguous() or scale.ndim == 0
+                    or scale.dtype not in FLOAT_DTYPES or scale.device != w.device
+                    or not scale.is_contiguous()
+                    or (zp is not None and (zp.device != w.device or not zp.is_contiguous()))
+                    or key[1] is None or not _plain(params)
+                    or (device is not None and (device, code_dtype) != (w.device, key[1]))):
+                slow.append((prefix, module))
+                continue
+            device, code_dtype = w.device, key[1]
+            picked.append((params, w, scale, zp, args, key))
+            shapes.append(tuple(w.shape))
+        if not picked:
+            continue
+        codes = slab_outputs(shapes, code_dtype, device)
+        out_code = _lib.dtype_code(code_dtype)
+        for (params, w, scale, zp, args, key), out in zip(picked, codes):
+            rows, cols = w.shape
+            tkey = ("c", rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
+            which = table.template(tkey)
+            if which < 0:
+                which = table.add_template(tkey, build_qparams(w, scale, zp, args, None, None))
+            table.add(w.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(w.dtype), which,
+                      scale.data_ptr(), 0 if zp is None else zp.data_ptr(), 0, out_code)
+        table.launch(entry, 1, 0, _lib.stream_of(device))
+        # the kernels are enqueued: the modules get their new parameters while the GPU works
+        for (params, w, scale, zp, args, key), out in zip(picked, codes):
+            params["weight"] = new_param(out, requires_grad=False)
+            if args.symmetric and zp is not None:  # a symmetric scheme stores no zero points
+                del params["weight_zero_point"]
+    if slow:
+        BaseQuantizationCompressor.compress_modules(self, slow, names_to_scheme)
+
+
+def _decompress_modules_fast(self, members, names_to_scheme) -> None:
+    """NaiveQuantizationCompressor.decompress_modules: decompress_module
+    (compressors/base.py:165-190, naive_quantized.py:116-136) for every (prefix, module) pair"""
+    entry = _lib.load().ctmi_qdq_many
+    table = module_table(self, _lib.QdqJob)
+    new_param = torch.nn.Parameter
+    slow = []
+    for lo, hi in module_chunks(len(members)):
+        picked, shapes, dtype, device = [], [], None, None
+        for prefix, module in members[lo:hi]:
+            params = module._parameters
+            codes, scale, zp = params.get("weight"), params.get("weight_scale"), params.get("weight_zero_point")
+            if (codes is None or scale is None or codes.ndim != 2 or codes.numel() == 0
+                    or codes.dtype not in (torch.int8, torch.float8_e4m3fn)
+                    or codes.device.type != "cuda" or not codes.is_contiguous()
+                    or scale.dtype not in FLOAT_DTYPES or scale.device != codes.device
+                    or not scale.is_contiguous()
+                    or (zp is not None and (zp.device != codes.device or not zp.is_contiguous()))
+                    or not _plain(params)
+                    or (dtype is not None and (dtype, device) != (scale.dtype, codes.device))):
+                slow.append((prefix, module))
+                continue
+            dtype, device = scale.dtype, codes.device
+            picked.append((params, codes, scale, zp))
+            shapes.append(tuple(codes.shape))
+        if not picked:
+            continue
+        dense = slab_outputs(shapes, dtype, device)
+        out_code = _lib.dtype_code(dtype)
+        for (params, codes, scale, zp), out in zip(picked, dense):
+            rows, cols = codes.shape
+            tkey = ("d", rows, cols, codes.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype)
+            which = table.template(tkey)
+            if which < 0:
+                # dequantize(x_q, scale, zero_point, g_idx=None): the strategy follows from the
+                # two shapes, the output dtype is the scale's (naive_quantized.py:116-136)
+                carrier = _ShapeOnly(codes.shape, codes.dtype)
+                which = table.add_template(
+                    tkey, build_qparams(carrier, scale, zp, infer_dequant_args(carrier, scale), None, None))
+            table.add(codes.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(codes.dtype), which,
+                      scale.data_ptr(), 0 if zp is None else zp.data_ptr(), 0, out_code)
+        table.launch(entry, 0, 1, _lib.stream_of(device))
+        for (params, codes, scale, zp), out in zip(picked, dense):
+            params["weight"] = new_param(out, requires_grad=False)
+    if slow:
+        BaseQuantizationCompressor.decompress_modules(self, slow, names_to_scheme)
+
+
+NaiveQuantizationCompressor.compress_modules = _compress_modules_fast
+NaiveQuantizationCompressor.decompress_modules = _decompress_modules_fast
 
 
 @BaseCompressor.register(name=CompressionFormat.int_quantized.value)

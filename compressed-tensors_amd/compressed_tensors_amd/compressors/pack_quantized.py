@@ -15,7 +15,9 @@ from torch import Tensor
 
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
-from compressed_tensors_amd.compressors.job_tables import WeightJobTable, slab_outputs
+from compressed_tensors_amd.compressors.job_tables import (
+    FLOAT_DTYPES, args_key, module_chunks, module_table, slab_outputs,
+)
 from compressed_tensors_amd.compressors.quantized_base import (
     BaseQuantizationCompressor, LazyDenseOutputs,
 )
@@ -606,29 +608,10 @@ PackedQuantizationCompressor.compress = _compress_state_dict_batched
 # Module pathways (ModelCompressor.compress_model / decompress_model): the common case - a 2-D
 # float weight on the GPU with group or channel scales, symmetric, no activation ordering - goes
 # into a job table written by columns; everything else takes the state-dict path above.
-_CHUNK_MODULES = 64   # modules per call of the C ABI
-_FLOAT_DTYPES = (torch.bfloat16, torch.float16, torch.float32)
+_FLOAT_DTYPES = FLOAT_DTYPES
 # what compression takes away from a module or writes anew (a symmetric scheme stores no zero points)
 _REPLACED = ("weight", "weight_zero_point", "weight_packed", "weight_shape")
-
-
-def _chunks(n):
-    for at in range(0, n, _CHUNK_MODULES):
-        yield at, min(at + _CHUNK_MODULES, n)
-
-
-def _module_table(self) -> WeightJobTable:
-    """the compressor's job table for the module pathways: its templates (the pointer-free
-    part of a weight's qparams per shape / dtype / scheme) stay valid from call to call"""
-    table = self.__dict__.get("_table")
-    if table is None or table.n_templates > 512:
-        table = self.__dict__["_table"] = WeightJobTable()
-    table.clear()  # rows a failed call may have left behind
-    return table
-
-
-def _args_key(args: QuantizationArgs):
-    return (args.num_bits, args.type, args.symmetric, args.strategy, args.group_size)
+_chunks, _module_table, _args_key = module_chunks, module_table, args_key
 
 
 def _compress_modules_fast(self, members, names_to_scheme) -> None:

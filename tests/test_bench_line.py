@@ -43,7 +43,12 @@ def _canned(bench):
         "hbm_roofline_frac": 0.8142, "roofline": roofline, "parity": "p" * 300, "cpu_baseline": cpu,
         "configs": configs,
         "api_level": {"what": "w" * 300, "compress_model_ms": 4.894932000013341,
-                      "decompress_model_ms": 4.101406000003749, "frac_of_hbm_peak": 0.48790287070046295},
+                      "decompress_model_ms": 4.101406000003749, "frac_of_hbm_peak": 0.48790287070046295,
+                      "other_formats": {
+                          "float-quantized": {"compress_model_ms": 3.35, "decompress_model_ms": 3.49,
+                                              "frac_of_hbm_peak": 0.76612345, "what": "w" * 200},
+                          "nvfp4-pack-quantized": {"compress_model_ms": 3.07, "decompress_model_ms": 2.98,
+                                                   "frac_of_hbm_peak": 0.73912345}}},
     }
 
 
@@ -69,6 +74,7 @@ def test_stdout_line_is_short_and_complete(tmp_path):
     whole, slowest = line["configs_frac"]["sparse"]
     assert abs(whole - 1e9 / 0.123456 / 1e6 / 8000.0) < 5e-3 and abs(slowest - 0.1543) < 1e-3  # three digits
     assert abs(line["api_level"]["frac_of_hbm_peak"] - 0.4879) < 1e-4
+    assert line["api_level"]["float-quantized"] == 0.766 and line["api_level"]["nvfp4-pack-quantized"] == 0.739
     assert abs(line["roofline"]["frac"] - out["roofline"]["frac"]) < 1e-3
 
 

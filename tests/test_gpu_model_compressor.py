@@ -397,3 +397,89 @@ def test_module_pathway_equals_state_dict_pathway(gpu):
         assert_bit_equal(m.weight.data, single.cpu(), f"{name} decompressed")
         assert m.weight.dtype == m.weight_scale.dtype
         assert dense_before[f"{name}.weight"].shape == m.weight.shape
+
+
+@pytest.mark.parametrize("fmt,spec", [
+    ("float-quantized", dict(num_bits=8, type="float", symmetric=True, strategy="channel")),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=64)),
+    ("int-quantized", dict(num_bits=8, type="int", symmetric=True, strategy="tensor")),
+    ("nvfp4-pack-quantized", dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)),
+], ids=["fp8-channel", "int8-asym-group", "int8-tensor", "nvfp4"])
+def test_module_pathway_of_the_other_formats(fmt, spec, gpu):
+    """compress_model / decompress_model for the int8 / fp8 and nvfp4 formats (job tables written
+    by columns): the same parameters as compress(state_dict) leaves, codes equal to the oracle's,
+    dense weights equal to the per-weight decompression; modules the table does not take
+    (activation ordering, a bias-carrying one, an fp32 one) among them; forward runs afterwards"""
+    from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme, observe_weight_qparams,
+    )
+    from compressed_tensors_amd.quantization.helpers import generate_gparam
+
+    announce("module pathway", fmt, spec)
+    torch.manual_seed(7)
+
+    class Mixed(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            self.a = torch.nn.ModuleList([torch.nn.Linear(256, 64 + 16 * i, bias=False) for i in range(9)])
+            self.b = torch.nn.ModuleList([torch.nn.Linear(128, 48, bias=True) for _ in range(3)])
+            self.c = torch.nn.Linear(256, 32, bias=False)   # activation ordering (where the format has it)
+            self.e = torch.nn.Linear(128, 16, bias=False)   # fp32 weight
+
+    model = Mixed().to(torch.bfloat16).to(gpu)
+    model.e.float()
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    config = QuantizationConfig(
+        config_groups={"g0": QuantizationScheme(targets=["Linear"], weights=args)}, format=fmt)
+    apply_quantization_scheme(model, config)
+    nvfp4 = spec["strategy"] == "tensor_group"
+    grouped = spec["strategy"] == "group"
+    oracle_in = {}
+    for name, m in model.named_modules():
+        if getattr(m, "quantization_scheme", None) is None:
+            continue
+        w = m.weight.data
+        gs = None
+        if nvfp4:
+            mn, mx = torch.aminmax(w)
+            gs = generate_gparam(mn.reshape(1), mx.reshape(1))
+            m.register_parameter("weight_global_scale", torch.nn.Parameter(gs, requires_grad=False))
+        scale, zp = observe_weight_qparams(w, args, global_scale=gs) if nvfp4 else observe_weight_qparams(w, args)
+        m.register_parameter("weight_scale", torch.nn.Parameter(scale, requires_grad=False))
+        m.register_parameter("weight_zero_point", torch.nn.Parameter(zp, requires_grad=False))
+        if name == "c" and grouped:
+            g_idx = (torch.randperm(256, device=gpu) // 64).to(torch.int32)
+            m.register_parameter("weight_g_idx", torch.nn.Parameter(g_idx, requires_grad=False))
+        elif name != "c":
+            oracle_in[name] = (w.cpu(), scale.cpu(), zp.cpu(), None if gs is None else gs.cpu())
+    mc = ModelCompressor(quantization_config=config)
+    want = mc.compress(model)
+    mc.compress_model(model)
+    got = {n: p.data for n, p in model.named_parameters()}
+    assert set(got) == set(want)
+    for name in want:
+        assert_bit_equal(got[name], want[name].to(got[name].device), name)
+    assert model.b[0].bias is not None and model.a[0].bias is None and "bias" in model.a[0]._parameters
+    for name, (w, s, z, gs) in oracle_in.items():
+        if nvfp4:
+            assert_bit_equal(got[f"{name}.weight_packed"], op.nvfp4_compress(w, s, gs, oargs), f"{name} codes")
+        else:
+            assert_bit_equal(got[f"{name}.weight"], op.naive_compress(w, s, oargs, zero_point=z), f"{name} codes")
+    compressed = {n: p.data for n, p in model.named_parameters()}
+    mc.decompress_model(model)
+    comp = mc.quantization_compressor[fmt]
+    for name, m in model.named_modules():
+        scheme = getattr(m, "quantization_scheme", None)
+        if scheme is None:
+            continue
+        data = {k[len(name) + 1:]: v for k, v in compressed.items() if k.startswith(name + ".")}
+        single = comp.decompress_weight(compressed_data=data, quantization_args=scheme.weights)
+        assert_bit_equal(m.weight.data, single.cpu(), f"{name} decompressed")
+        assert m.weight.dtype == single.dtype and m.weight.shape == single.shape
+        x = torch.randn(2, m.in_features, device=gpu).to(m.weight.dtype)
+        assert_bit_equal(m(x), torch.nn.functional.linear(x, single, m.bias).cpu(), f"{name} forward")
+    # a second round starts from modules that hold both the codes' leftovers and the dense weight
+    mc.compress_model(model)
+    again = {n: p.data for n, p in model.named_parameters()}
+    assert set(again) == set(want)
