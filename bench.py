@@ -1057,6 +1057,22 @@ def api_level_format(torch, seed, steps, fmt, spec, bytes_per_element):
             comp.append(t1 - t0)
             deco.append(t2 - t1)
     c_s, d_s = statistics.median(comp), statistics.median(deco)
+    # the state-dict pathway: compress(model) -> compressed state dict, decompress(state dict, model)
+    comp, deco = [], []
+    for it in range(steps + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        state = mc.compress(model)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        mc.decompress(state, model)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        del state
+        if it:
+            comp.append(t1 - t0)
+            deco.append(t2 - t1)
+    cs_s, ds_s = statistics.median(comp), statistics.median(deco)
     del model, mc
     torch.cuda.empty_cache()
     return {
@@ -1064,6 +1080,10 @@ def api_level_format(torch, seed, steps, fmt, spec, bytes_per_element):
         "compress_GBs": per_dir / c_s / 1e9, "decompress_GBs": per_dir / d_s / 1e9,
         "roundtrip_GBs": 2 * per_dir / (c_s + d_s) / 1e9,
         "frac_of_hbm_peak": 2 * per_dir / (c_s + d_s) / 1e9 / HBM_PEAK_GBS,
+        "state_dict_pathway": {
+            "what": "compress(model) -> compressed state dict, decompress(state dict, model)",
+            "compress_ms": cs_s * 1e3, "decompress_ms": ds_s * 1e3,
+            "frac_of_hbm_peak": 2 * per_dir / (cs_s + ds_s) / 1e9 / HBM_PEAK_GBS},
         "passes": steps, "statistic": "median",
     }
 
@@ -1127,6 +1147,8 @@ def short_line(out, details_path=None):
         line["mfma_frac"] = _sig(out["mfma_utilisation"]["frac"], 3)
     if "api_level" in out:
         line["api_level"] = pick(out["api_level"], ("frac_of_hbm_peak", "compress_model_ms", "decompress_model_ms"))
+        if "state_dict_pathway" in out["api_level"]:
+            line["api_level"]["state_dict_pathway"] = _sig(out["api_level"]["state_dict_pathway"]["frac_of_hbm_peak"], 3)
         for fmt, res in out["api_level"].get("other_formats", {}).items():
             line["api_level"][fmt] = _sig(res["frac_of_hbm_peak"], 3)
     if details_path:

@@ -13,7 +13,7 @@ from torch import Tensor
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
 from compressed_tensors_amd.compressors.job_tables import (
-    FLOAT_DTYPES, args_key, module_chunks, module_table, slab_outputs,
+    FLOAT_DTYPES, args_key, on_gpu, run_table,
 )
 from compressed_tensors_amd.compressors.quantized_base import (
     BaseQuantizationCompressor, LazyDenseOutputs,
@@ -279,26 +279,39 @@ class Fp4WeightBatch(LazyDenseOutputs):
 
 
 def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,
-                                 compression_device=None, **kwargs):
+                                 compression_device=None, precomputed=None, **kwargs):
     """BaseQuantizationCompressor.compress (quantized_compressors/base.py:69-161) with
     every nvfp4 weight handed to the C ABI in one call: same keys, dtypes and values as
     the per-weight loop."""
     jobs, names = [], []
-    for name in list(model_state.keys()):
-        if not name.endswith("weight"):
-            continue
-        prefix = name[: -len("weight")]
-        scale = model_state.get(prefix + "weight_scale", None)
-        gs = model_state.get(prefix + "weight_global_scale", None)
-        weight = model_state[name]
-        if scale is None or gs is None or weight.ndim != 2 or weight.numel() == 0:
-            continue  # the per-weight path below deals with it (or raises as the reference does)
-        module_path = prefix[:-1] if prefix.endswith(".") else prefix
-        jobs.append(dict(weight=weight, scale=scale, global_scale=gs,
-                         zero_point=model_state.get(prefix + "weight_zero_point", None),
-                         quantization_args=names_to_scheme[module_path].weights))
-        names.append(name)
-    packed_by_name = dict(zip(names, Fp4WeightBatch(jobs).compress())) if jobs else {}
+
+    def candidates():
+        # (a generator: the first many-weight call goes out while later names are still looked at)
+        for name in list(model_state.keys()):
+            if not name.endswith("weight") or (precomputed is not None and name in precomputed):
+                continue
+            prefix = name[: -len("weight")]
+            scale = model_state.get(prefix + "weight_scale", None)
+            gs = model_state.get(prefix + "weight_global_scale", None)
+            weight = model_state[name]
+            if scale is None or gs is None or weight.ndim != 2 or weight.numel() == 0:
+                continue  # the per-weight path below deals with it (or raises as the reference does)
+            module_path = prefix[:-1] if prefix.endswith(".") else prefix
+            job = dict(weight=weight, scale=scale, global_scale=gs,
+                       zero_point=model_state.get(prefix + "weight_zero_point", None),
+                       quantization_args=names_to_scheme[module_path].weights)
+            jobs.append(job)
+            names.append(name)
+            yield (weight, scale, job["zero_point"], gs, None, job["quantization_args"])
+
+    # the common case through the job table written by columns, the rest as one batch of its own
+    outs = _table_compress(self, candidates())
+    packed_by_name = dict(precomputed or {})  # (what the caller enqueued from the modules already)
+    packed_by_name.update((names[k], out) for k, out in enumerate(outs) if out is not None)
+    left = [k for k, out in enumerate(outs) if out is None]
+    if left:
+        for k, packed in zip(left, Fp4WeightBatch([jobs[k] for k in left]).compress()):
+            packed_by_name[names[k]] = packed
 
     def move(t):
         return t if compression_device is None else t.to(compression_device)
@@ -345,58 +358,115 @@ def _own_only(params) -> bool:
     return True
 
 
-def _table_ready(t, device) -> bool:
-    return t is not None and t.device == device and t.is_contiguous()
+class _CompressSpec:
+    """what run_table needs for ctmi_nvfp4_compress_many.  Records are (weight, scale,
+    zero_point, global_scale, g_idx, args); the reference does not forward g_idx to quantize().
+    Taken: a 2-D float weight on the GPU with 2-D scales and an fp32 global scale of one value."""
+    job_struct = _lib.WeightJob
+
+    def __init__(self):
+        self._args = {}
+
+    def key(self, rec):
+        w, scale, zp, gs, g_idx, args = rec
+        if (not on_gpu(w) or w.ndim != 2 or w.numel() == 0 or w.shape[1] % 2 or w.dtype not in FLOAT_DTYPES
+                or not on_gpu(scale, w.device) or scale.dtype not in _SCALE_DTYPES or scale.ndim != 2
+                or not on_gpu(gs, w.device) or gs.dtype is not torch.float32 or gs.numel() != 1
+                or (zp is not None and not on_gpu(zp, w.device))):
+            return None
+        k = self._args.get(id(args))
+        if k is None:
+            k = self._args[id(args)] = args_key(args)
+        return ("c", w.shape, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, k)
+
+    def out_spec(self, rec):
+        w = rec[0]
+        return (w.shape[0], w.shape[1] // 2), torch.uint8, w.device
+
+    def plan(self, rec):
+        w, scale, zp, gs, g_idx, args = rec
+        return build_qparams(w, scale, zp, args, None, gs)
+
+    def row(self, rec, out):
+        w, scale, zp, gs = rec[0], rec[1], rec[2], rec[3]
+        return (w.data_ptr(), out.data_ptr(), w.shape[0], w.shape[1], _lib.dtype_code(w.dtype),
+                scale.data_ptr(), 0 if zp is None else zp.data_ptr(), gs.data_ptr(), 0)
+
+
+class _DecompressSpec:
+    """... for ctmi_nvfp4_decompress_many.  Records are (compressed entries of one weight under
+    their local names, args).  Taken: packed bytes, several group scales per row and an fp32
+    global scale on the GPU (the reference's group path, which honours the bf16 it asks for)."""
+    job_struct = _lib.WeightJob
+
+    def key(self, rec):
+        data = rec[0]
+        packed, scale, gs = data.get("weight_packed"), data.get("weight_scale"), data.get("weight_global_scale")
+        if (not on_gpu(packed) or packed.dtype is not torch.uint8 or packed.ndim != 2 or packed.numel() == 0
+                or not on_gpu(scale, packed.device) or scale.dtype not in _SCALE_DTYPES
+                or scale.ndim != 2 or scale.shape[0] != packed.shape[0] or scale.shape[1] <= 1
+                or (2 * packed.shape[1]) % scale.shape[1]
+                or not on_gpu(gs, packed.device) or gs.dtype is not torch.float32 or gs.numel() != 1):
+            return None
+        return ("d", packed.shape, scale.shape, scale.dtype)
+
+    def out_spec(self, rec):
+        packed = rec[0]["weight_packed"]
+        return (packed.shape[0], 2 * packed.shape[1]), torch.bfloat16, packed.device
+
+    def plan(self, rec):
+        data = rec[0]
+        packed, scale = data["weight_packed"], data["weight_scale"]
+        carrier = _ShapeOnly(torch.Size((packed.shape[0], 2 * packed.shape[1])), torch.bfloat16)
+        plan = build_qparams(carrier, scale, None, infer_dequant_args(carrier, scale), None,
+                             data["weight_global_scale"])
+        if not plan.grouped:
+            raise RuntimeError(f"group scales expected, got shape {tuple(scale.shape)}")
+        plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_FLOAT, 4
+        return plan
+
+    def row(self, rec, out):
+        data = rec[0]
+        packed = data["weight_packed"]
+        return (packed.data_ptr(), out.data_ptr(), packed.shape[0], 2 * packed.shape[1],
+                _lib.dtype_code(torch.bfloat16), data["weight_scale"].data_ptr(), 0,
+                data["weight_global_scale"].data_ptr(), 0)
+
+
+def _table_compress(self, recs) -> list:
+    """packed bytes per (weight, scale, zero_point, global_scale, g_idx, args) record from
+    many-weight calls; None where the record is not one the job table takes"""
+    return run_table(self, recs, _CompressSpec(), _lib.load().ctmi_nvfp4_compress_many)
+
+
+def _table_decompress(self, recs) -> list:
+    """dense weights per (compressed entries, args) record; None where the table does not take it"""
+    return run_table(self, recs, _DecompressSpec(), _lib.load().ctmi_nvfp4_decompress_many)
 
 
 def _compress_modules_fast(self, members, names_to_scheme) -> None:
     """NVFP4PackedCompressor.compress_modules: compress_module (compressors/base.py:125-151,
-    fp4_quantized.py:84-106) for every (prefix, module) pair, one ctmi_nvfp4_compress_many
-    call per 64"""
-    entry = _lib.load().ctmi_nvfp4_compress_many
-    table = module_table(self)
+    fp4_quantized.py:84-106) for every (prefix, module) pair"""
     new_param = torch.nn.Parameter
-    slow, arg_keys = [], {}
-    for lo, hi in module_chunks(len(members)):
-        picked, shapes, device = [], [], None
-        for prefix, module in members[lo:hi]:
+    recs = []
+    for prefix, module in members:
+        params = module._parameters
+        ok = _own_only(params)
+        recs.append((params.get("weight") if ok else None, params.get("weight_scale"),
+                     params.get("weight_zero_point"), params.get("weight_global_scale"), None,
+                     names_to_scheme[prefix].weights))
+    outs = _table_compress(self, recs)
+    # the kernels are enqueued: the modules get their new parameters while the GPU works
+    for (prefix, module), rec, out in zip(members, recs, outs):
+        if out is not None:
             params = module._parameters
-            w, scale, zp, gs = (params.get(n) for n in ("weight", "weight_scale", "weight_zero_point",
-                                                        "weight_global_scale"))
-            args = names_to_scheme[prefix].weights
-            key = arg_keys.get(id(args))
-            if key is None:
-                key = arg_keys[id(args)] = args_key(args)
-            if (w is None or w.ndim != 2 or w.numel() == 0 or w.shape[1] % 2 or w.dtype not in FLOAT_DTYPES
-                    or w.device.type != "cuda" or not w.is_contiguous()
-                    or not _table_ready(scale, w.device) or scale.dtype not in _SCALE_DTYPES or scale.ndim != 2
-                    or not _table_ready(gs, w.device) or gs.dtype is not torch.float32 or gs.numel() != 1
-                    or (zp is not None and not _table_ready(zp, w.device))
-                    or not _own_only(params) or (device is not None and device != w.device)):
-                slow.append((prefix, module))
-                continue
-            device = w.device
-            picked.append((params, w, scale, zp, gs, args, key))
-            shapes.append((w.shape[0], w.shape[1] // 2))
-        if not picked:
-            continue
-        packed = slab_outputs(shapes, torch.uint8, device)
-        for (params, w, scale, zp, gs, args, key), out in zip(picked, packed):
-            rows, cols = w.shape
-            tkey = ("c", rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
-            which = table.template(tkey)
-            if which < 0:
-                which = table.add_template(tkey, build_qparams(w, scale, zp, args, None, gs))
-            table.add(w.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(w.dtype), which,
-                      scale.data_ptr(), 0 if zp is None else zp.data_ptr(), gs.data_ptr())
-        table.launch(entry, _lib.stream_of(device))
-        # the kernels are enqueued: the modules get their new parameters while the GPU works
-        for (params, w, scale, zp, gs, args, key), out in zip(picked, packed):
+            symmetric = rec[5].symmetric
             rest = [(n, p) for n, p in params.items()
-                    if n not in ("weight", "weight_packed") and not (n == "weight_zero_point" and args.symmetric)]
+                    if n not in ("weight", "weight_packed") and not (n == "weight_zero_point" and symmetric)]
             params.clear()
             params["weight_packed"] = new_param(out, requires_grad=False)
             params.update(rest)
+    slow = [members[i] for i, out in enumerate(outs) if out is None]
     if slow:
         BaseQuantizationCompressor.compress_modules(self, slow, names_to_scheme)
 
@@ -404,52 +474,33 @@ def _compress_modules_fast(self, members, names_to_scheme) -> None:
 def _decompress_modules_fast(self, members, names_to_scheme) -> None:
     """NVFP4PackedCompressor.decompress_modules: decompress_module (compressors/base.py:165-190,
     fp4_quantized.py:108-123) for every (prefix, module) pair"""
-    entry = _lib.load().ctmi_nvfp4_decompress_many
-    table = module_table(self)
     new_param = torch.nn.Parameter
-    slow = []
-    for lo, hi in module_chunks(len(members)):
-        picked, shapes, device = [], [], None
-        for prefix, module in members[lo:hi]:
-            params = module._parameters
-            packed, scale, gs = (params.get(n) for n in ("weight_packed", "weight_scale", "weight_global_scale"))
-            if (packed is None or packed.dtype is not torch.uint8 or packed.ndim != 2 or packed.numel() == 0
-                    or packed.device.type != "cuda" or not packed.is_contiguous()
-                    or not _table_ready(scale, packed.device) or scale.dtype not in _SCALE_DTYPES
-                    or scale.ndim != 2 or scale.shape[0] != packed.shape[0] or scale.shape[1] <= 1
-                    or (2 * packed.shape[1]) % scale.shape[1]
-                    or not _table_ready(gs, packed.device) or gs.dtype is not torch.float32 or gs.numel() != 1
-                    or params.get("weight_zero_point") is not None
-                    or not _own_only(params) or (device is not None and device != packed.device)):
-                slow.append((prefix, module))
-                continue
-            device = packed.device
-            picked.append((params, packed, scale, gs))
-            shapes.append((packed.shape[0], 2 * packed.shape[1]))
-        if not picked:
-            continue
-        # (several groups per row: the reference's group path, which honours the bf16 it asks for)
-        dense = slab_outputs(shapes, torch.bfloat16, device)
-        out_code = _lib.dtype_code(torch.bfloat16)
-        for (params, packed, scale, gs), out, shape in zip(picked, dense, shapes):
-            tkey = ("d", shape, scale.shape, scale.dtype)
-            which = table.template(tkey)
-            if which < 0:
-                carrier = _ShapeOnly(torch.Size(shape), torch.bfloat16)
-                plan = build_qparams(carrier, scale, None, infer_dequant_args(carrier, scale), None, gs)
-                if not plan.grouped:
-                    raise RuntimeError(f"group scales expected, got shape {tuple(scale.shape)}")
-                plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_FLOAT, 4
-                which = table.add_template(tkey, plan)
-            table.add(packed.data_ptr(), out.data_ptr(), shape[0], shape[1], out_code, which,
-                      scale.data_ptr(), 0, gs.data_ptr())
-        table.launch(entry, _lib.stream_of(device))
-        for (params, packed, scale, gs), out in zip(picked, dense):
-            params["weight"] = new_param(out, requires_grad=False)
+    recs = []
+    for _, module in members:
+        params = module._parameters
+        ok = _own_only(params) and params.get("weight_zero_point") is None
+        recs.append((params if ok else {}, None))
+    outs = _table_decompress(self, recs)
+    for (prefix, module), out in zip(members, outs):
+        if out is not None:
+            module._parameters["weight"] = new_param(out, requires_grad=False)
+    slow = [members[i] for i, out in enumerate(outs) if out is None]
     if slow:
         BaseQuantizationCompressor.decompress_modules(self, slow, names_to_scheme)
 
 
+def _decompress_weights_batched(self, items) -> list:
+    """NVFP4PackedCompressor.decompress_weight for a list of (compressed_data,
+    quantization_args) pairs: many-weight calls where the job table takes them"""
+    outs = _table_decompress(self, items)
+    for k, out in enumerate(outs):
+        if out is None:
+            outs[k] = self.decompress_weight(compressed_data=items[k][0], quantization_args=items[k][1])
+    return outs
+
+
+NVFP4PackedCompressor.decompress_weights = _decompress_weights_batched
+NVFP4PackedCompressor.table_compress = _table_compress
 NVFP4PackedCompressor.compress_modules = _compress_modules_fast
 NVFP4PackedCompressor.decompress_modules = _decompress_modules_fast
 

@@ -16,7 +16,8 @@ import torch
 
 from compressed_tensors_amd import _lib
 
-__all__ = ["WeightJobTable", "slab_outputs", "module_table", "module_chunks", "args_key", "FLOAT_DTYPES"]
+__all__ = ["WeightJobTable", "slab_outputs", "module_table", "module_chunks", "args_key", "FLOAT_DTYPES",
+           "run_table", "on_gpu"]
 
 _QP = np.dtype(_lib.QParams)
 assert _QP.itemsize == ctypes.sizeof(_lib.QParams)
@@ -115,10 +116,17 @@ class WeightJobTable:
         _lib.check(entry(ctypes.cast(tab.ctypes.data, self._job_ptr), n, *args))
 
 
+_RAMP = (16, 32)  # the first calls are short: the GPU starts while the later rows are written
+
+
 def module_chunks(n):
-    """(lo, hi) ranges of at most 64 modules"""
-    for at in range(0, n, _CHUNK_MODULES):
-        yield at, min(at + _CHUNK_MODULES, n)
+    """(lo, hi) ranges over n weights: 16, 32, then 64 at a time"""
+    at, k = 0, 0
+    while at < n:
+        size = _RAMP[k] if k < len(_RAMP) else _CHUNK_MODULES
+        yield at, min(at + size, n)
+        at += size
+        k += 1
 
 
 def module_table(compressor, job_struct=_lib.WeightJob) -> WeightJobTable:
@@ -135,6 +143,64 @@ def args_key(args):
     """what of a QuantizationArgs decides a weight's qparams plan"""
     return (args.num_bits, args.type, args.symmetric, args.strategy, args.group_size,
             None if args.block_structure is None else tuple(args.block_structure))
+
+
+def on_gpu(t, device=None) -> bool:
+    """is `t` a contiguous tensor on a GPU (on `device`, if given)?"""
+    return (t is not None and t.device.type == "cuda" and t.is_contiguous()
+            and (device is None or t.device == device))
+
+
+def run_table(compressor, recs, spec, entry, *entry_args) -> list:
+    """The many-weight call `entry(jobs, n, *entry_args, stream)` for the records of `recs`
+    that `spec` takes; returns one output tensor per record, None for those it does not take
+    (the caller treats them one by one).  `spec` describes a format and direction:
+      spec.job_struct       ctmi_weight_job or ctmi_qdq_job
+      spec.key(rec)         template key (what decides the qparams besides addresses), or None
+      spec.out_spec(rec)    (shape, dtype, device) of the output
+      spec.plan(rec)        the QPlan of build_qparams for this record (made once per key)
+      spec.row(rec, out)    (src, dst, rows, cols, dtype code, scale, zero_point, global_scale,
+                             second dtype code): addresses and sizes of the job
+    Outputs of one shape share allocations; calls are short at first, so that the GPU starts
+    while later rows are still being written."""
+    outs: list = []
+    pending: Dict[Tuple, List] = {}   # (dtype, device) of the outputs -> rows waiting for their call
+    calls: Dict[Tuple, int] = {}      # ... -> calls made so far (the first ones are short)
+    table = None
+
+    def flush(group):
+        nonlocal table
+        part = pending.pop(group)
+        if table is None:
+            table = module_table(compressor, spec.job_struct)
+        dtype, device = group
+        slabs = slab_outputs([shape for _, _, _, shape in part], dtype, device)
+        for (i, rec, key, _), out in zip(part, slabs):
+            which = table.template(key)
+            if which < 0:
+                which = table.add_template(key, spec.plan(rec))
+            src, dst, rows, cols, code, scale, zp, gs, code2 = spec.row(rec, out)
+            table.add(src, dst, rows, cols, code, which, scale, zp, gs, code2)
+            outs[i] = out
+        table.launch(entry, *entry_args, _lib.stream_of(device))
+        calls[group] = calls.get(group, 0) + 1
+
+    # `recs` may be a generator: a call goes out as soon as its rows are there
+    for i, rec in enumerate(recs):
+        outs.append(None)
+        key = spec.key(rec)
+        if key is None:
+            continue
+        shape, dtype, device = spec.out_spec(rec)
+        group = (dtype, device)
+        rows = pending.setdefault(group, [])
+        rows.append((i, rec, key, tuple(shape)))
+        k = calls.get(group, 0)
+        if len(rows) >= (_RAMP[k] if k < len(_RAMP) else _CHUNK_MODULES):
+            flush(group)
+    for group in list(pending):
+        flush(group)
+    return outs
 
 
 def slab_outputs(shapes: List[Tuple[int, ...]], dtype: torch.dtype, device) -> List[torch.Tensor]:

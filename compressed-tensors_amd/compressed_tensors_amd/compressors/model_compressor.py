@@ -34,8 +34,13 @@ __all__ = ["ModelCompressor", "map_module_to_scheme", "match_named_modules",
 # Modules per batch of the in-memory pathways.  The host needs somewhat less time per module
 # than the GPU: batches (multiples of the 8 weights of a launch) grow by about half from one to
 # the next, and the GPU hardly waits after the first.
+_GRAD_DTYPES = (torch.float16, torch.float32, torch.bfloat16)
 _BATCHES = (8, 16, 24, 32, 48)
 _BATCH = 64
+
+
+def _data(p):
+    return None if p is None else p.data
 
 
 def _set_plain(module: Module, name: str, value) -> None:
@@ -139,7 +144,11 @@ class ModelCompressor:
     # ----- state dict pathways ----- #
     def compress(self, model: Module, state_dict: Optional[Dict[str, Tensor]] = None,
                  show_progress: bool = False) -> Dict[str, Tensor]:
+        precomputed = None
         if state_dict is None:
+            # the weights are where the modules hold them: their kernels are enqueued before
+            # the state dict is even put together
+            precomputed = self._enqueue_from_modules(model)
             state_dict = model.state_dict()
         stacked = self._compress_quantized_24(model, state_dict)
         if stacked:
@@ -150,7 +159,8 @@ class ModelCompressor:
             module_to_scheme = map_module_to_scheme(model)
             quant_compressor = next(iter(self.quantization_compressor.values()))
             state_dict = quant_compressor.compress(
-                state_dict, names_to_scheme=module_to_scheme, show_progress=show_progress
+                state_dict, names_to_scheme=module_to_scheme, show_progress=show_progress,
+                precomputed=precomputed,
             )
             if self.quantization_config.format != CompressionFormat.dense.value:
                 self.quantization_config.quantization_status = QuantizationStatus.COMPRESSED.value
@@ -162,6 +172,36 @@ class ModelCompressor:
         for entries in stacked.values():
             state_dict.update(entries)
         return state_dict
+
+    def _enqueue_from_modules(self, model: Module) -> Optional[Dict[str, Tensor]]:
+        """{name of a dense weight in the state dict: its compressed tensor} for the weights
+        the quantization compressor's job table takes, their kernels enqueued; None where
+        that does not apply (sparsity in play, several formats, no table for the format)"""
+        if (self.quantization_compressor is None or len(self.quantization_compressor) != 1
+                or self.sparsity_compressor is not None):
+            return None
+        compressor = next(iter(self.quantization_compressor.values()))
+        table_compress = getattr(compressor, "table_compress", None)
+        if table_compress is None:
+            return None
+        names = []
+
+        def weights():
+            for prefix, module in model.named_modules():
+                scheme = _scheme_of(module)
+                if scheme is None or scheme.weights is None or "_fsdp_wrapped_module." in prefix:
+                    continue
+                params = module._parameters
+                w, scale = params.get("weight"), params.get("weight_scale")
+                if w is None or scale is None:
+                    continue
+                names.append(f"{prefix}.weight" if prefix else "weight")
+                yield (w.data, scale.data, _data(params.get("weight_zero_point")),
+                       _data(params.get("weight_global_scale")), _data(params.get("weight_g_idx")),
+                       scheme.weights)
+
+        outs = table_compress(weights())
+        return {name: out for name, out in zip(names, outs) if out is not None}
 
     def _compress_quantized_24(self, model: Module, state_dict: Dict[str, Tensor],
                                targets: Optional[Set[str]] = None,
@@ -288,14 +328,20 @@ class ModelCompressor:
             for name, data in dense.items():
                 self._assign(model, name, data)
         if quant_compressor is not None:
-            names_to_scheme = map_module_to_scheme(model)
+            names_to_scheme, modules = {}, {}
+            for name, module in model.named_modules():  # one walk: schemes and where the results go
+                modules[name] = module
+                scheme = _scheme_of(module)
+                if scheme is not None and scheme.weights is not None:
+                    names_to_scheme[name.replace("_fsdp_wrapped_module.", "")] = scheme
             for mod_path, data in quant_compressor.decompress(state, names_to_scheme=names_to_scheme):
-                for param_name, param_data in data.items():
-                    if param_name == "weight" or hasattr(self._module(model, mod_path), param_name):
-                        self._assign(model, f"{mod_path}.{param_name}", param_data)
-            for module in model.modules():
-                if getattr(module, "quantization_scheme", None) is not None:
-                    module.quantization_status = QuantizationStatus.FROZEN
+                module = modules.get(mod_path)
+                if module is None:
+                    module = self._module(model, mod_path)
+                self._assign_own(model, module, mod_path, data)
+            for module in modules.values():
+                if _scheme_of(module) is not None:
+                    _set_plain(module, "quantization_status", QuantizationStatus.FROZEN)
 
     def update_config(self, save_directory: str) -> None:
         """write the compression configs into `config.json` under `save_directory`, next
@@ -440,6 +486,28 @@ class ModelCompressor:
 
     _own_parameters = staticmethod(own_parameters)
     _swap_parameters = staticmethod(swap_parameters)
+
+    def _assign_own(self, model: Module, module: Module, mod_path: str, data: Dict[str, Tensor]) -> None:
+        """_assign for the entries of one module: the dense weight, and what else of `data` the
+        module has an attribute for.  Parameters the module already holds are replaced in
+        their slots; anything else goes through _assign."""
+        params = module._parameters
+        device = None
+        for p in params.values():
+            if p is not None:
+                device = p.device
+                break
+        for param_name, value in data.items():
+            if param_name in params and device is not None:
+                held = params[param_name]
+                # (a parameter the module keeps on another device - the shape of a packed weight
+                # lives on the host - stays there)
+                target = device if held is None else held.device
+                if value.device != target:
+                    value = value.to(target)
+                params[param_name] = torch.nn.Parameter(value, requires_grad=value.dtype in _GRAD_DTYPES)
+            elif param_name == "weight" or hasattr(module, param_name):
+                self._assign(model, f"{mod_path}.{param_name}", value)
 
     def _assign(self, model: Module, full_name: str, data: Tensor) -> None:
         prefix, _, param_name = full_name.rpartition(".")

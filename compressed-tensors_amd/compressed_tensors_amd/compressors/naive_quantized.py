@@ -11,7 +11,7 @@ from torch import Tensor
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
 from compressed_tensors_amd.compressors.job_tables import (
-    FLOAT_DTYPES, args_key, module_chunks, module_table, slab_outputs,
+    FLOAT_DTYPES, args_key, on_gpu, run_table,
 )
 from compressed_tensors_amd.compressors.quantized_base import (
     BaseQuantizationCompressor, LazyDenseOutputs,
@@ -284,30 +284,43 @@ class NaiveQuantizationCompressor(BaseQuantizationCompressor):
 
 
 def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,
-                                 compression_device=None, **kwargs):
+                                 compression_device=None, precomputed=None, **kwargs):
     """BaseQuantizationCompressor.compress (quantized_compressors/base.py:69-161) with
     every quantizable weight handed to the C ABI in one call: same keys, dtypes and
     values as the per-weight loop."""
     jobs, names = [], []
-    for name in list(model_state.keys()):
-        if not name.endswith("weight"):
-            continue
-        prefix = name[: -len("weight")]
-        scale = model_state.get(prefix + "weight_scale", None)
-        if scale is None:
-            continue
-        if model_state.get(prefix + "weight_global_scale", None) is not None:
-            raise ValueError("global_scale is not supported for the NaiveQuantizationCompressor")
-        module_path = prefix[:-1] if prefix.endswith(".") else prefix
-        args = names_to_scheme[module_path].weights
-        weight = model_state[name]
-        if not can_quantize(weight, args) or weight.ndim < 1 or weight.numel() == 0:
-            continue  # the per-weight path below passes it through
-        jobs.append(dict(weight=weight, scale=scale, quantization_args=args,
-                         zero_point=model_state.get(prefix + "weight_zero_point", None),
-                         g_idx=model_state.get(prefix + "weight_g_idx", None)))
-        names.append(name)
-    codes_by_name = dict(zip(names, QuantizedWeightBatch(jobs).compress())) if jobs else {}
+
+    def candidates():
+        # (a generator: the first many-weight call goes out while later names are still looked at)
+        for name in list(model_state.keys()):
+            if not name.endswith("weight") or (precomputed is not None and name in precomputed):
+                continue
+            prefix = name[: -len("weight")]
+            scale = model_state.get(prefix + "weight_scale", None)
+            if scale is None:
+                continue
+            if model_state.get(prefix + "weight_global_scale", None) is not None:
+                raise ValueError("global_scale is not supported for the NaiveQuantizationCompressor")
+            module_path = prefix[:-1] if prefix.endswith(".") else prefix
+            args = names_to_scheme[module_path].weights
+            weight = model_state[name]
+            if not can_quantize(weight, args) or weight.ndim < 1 or weight.numel() == 0:
+                continue  # the per-weight path below passes it through
+            job = dict(weight=weight, scale=scale, quantization_args=args,
+                       zero_point=model_state.get(prefix + "weight_zero_point", None),
+                       g_idx=model_state.get(prefix + "weight_g_idx", None))
+            jobs.append(job)
+            names.append(name)
+            yield (weight, scale, job["zero_point"], None, job["g_idx"], args)
+
+    # the common case through the job table written by columns, the rest as one batch of its own
+    outs = _table_compress(self, candidates())
+    codes_by_name = dict(precomputed or {})  # (what the caller enqueued from the modules already)
+    codes_by_name.update((names[k], out) for k, out in enumerate(outs) if out is not None)
+    left = [k for k, out in enumerate(outs) if out is None]
+    if left:
+        for k, codes in zip(left, QuantizedWeightBatch([jobs[k] for k in left]).compress()):
+            codes_by_name[names[k]] = codes
 
     def move(t):
         return t if compression_device is None else t.to(compression_device)
@@ -354,52 +367,108 @@ def _plain(params) -> bool:
     return True
 
 
+class _CompressSpec:
+    """what run_table needs for ctmi_qdq_many, quantizing.  Records are (weight, scale,
+    zero_point, global_scale, g_idx, args).  Taken: a 2-D float weight on the GPU with float
+    scales of one dimension or more, no activation ordering."""
+    job_struct = _lib.QdqJob
+
+    def __init__(self):
+        self._args = {}
+
+    def key(self, rec):
+        w, scale, zp, gs, g_idx, args = rec
+        k = self._args.get(id(args))
+        if k is None:
+            k = self._args[id(args)] = (args_key(args), args.pytorch_dtype() if args.num_bits <= 8 else None)
+        if (gs is not None or g_idx is not None or not on_gpu(w) or w.ndim != 2 or w.numel() == 0
+                or w.dtype not in FLOAT_DTYPES or not on_gpu(scale, w.device) or scale.ndim == 0
+                or scale.dtype not in FLOAT_DTYPES or (zp is not None and not on_gpu(zp, w.device))
+                or k[1] is None):
+            return None
+        return ("c", w.shape, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, k)
+
+    def out_spec(self, rec):
+        return rec[0].shape, self._args[id(rec[5])][1], rec[0].device
+
+    def plan(self, rec):
+        w, scale, zp, gs, g_idx, args = rec
+        return build_qparams(w, scale, zp, args, None, None)
+
+    def row(self, rec, out):
+        w, scale, zp = rec[0], rec[1], rec[2]
+        return (w.data_ptr(), out.data_ptr(), w.shape[0], w.shape[1], _lib.dtype_code(w.dtype),
+                scale.data_ptr(), 0 if zp is None else zp.data_ptr(), 0, _lib.dtype_code(out.dtype))
+
+
+class _DecompressSpec:
+    """... dequantizing.  Records are (compressed entries of one weight under their local
+    names, args).  Taken: int8 / fp8 codes and float scales on the GPU, no activation
+    ordering."""
+    job_struct = _lib.QdqJob
+
+    def key(self, rec):
+        data = rec[0]
+        codes, scale, zp = data.get("weight"), data.get("weight_scale"), data.get("weight_zero_point")
+        if (data.get("weight_g_idx") is not None or not on_gpu(codes) or codes.ndim != 2 or codes.numel() == 0
+                or codes.dtype not in (torch.int8, torch.float8_e4m3fn)
+                or not on_gpu(scale, codes.device) or scale.dtype not in FLOAT_DTYPES
+                or (zp is not None and not on_gpu(zp, codes.device))):
+            return None
+        return ("d", codes.shape, codes.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype)
+
+    def out_spec(self, rec):
+        data = rec[0]
+        return data["weight"].shape, data["weight_scale"].dtype, data["weight"].device
+
+    def plan(self, rec):
+        # dequantize(x_q, scale, zero_point, g_idx=None): the strategy follows from the two
+        # shapes, the output dtype is the scale's (naive_quantized.py:116-136)
+        data = rec[0]
+        codes, scale = data["weight"], data["weight_scale"]
+        carrier = _ShapeOnly(codes.shape, codes.dtype)
+        return build_qparams(carrier, scale, data.get("weight_zero_point"),
+                             infer_dequant_args(carrier, scale), None, None)
+
+    def row(self, rec, out):
+        data = rec[0]
+        codes, scale, zp = data["weight"], data["weight_scale"], data.get("weight_zero_point")
+        return (codes.data_ptr(), out.data_ptr(), codes.shape[0], codes.shape[1], _lib.dtype_code(codes.dtype),
+                scale.data_ptr(), 0 if zp is None else zp.data_ptr(), 0, _lib.dtype_code(out.dtype))
+
+
+def _table_compress(self, recs) -> list:
+    """codes per (weight, scale, zero_point, global_scale, g_idx, args) record from many-weight
+    calls; None where the record is not one the job table takes"""
+    return run_table(self, recs, _CompressSpec(), _lib.load().ctmi_qdq_many, 1, 0)
+
+
+def _table_decompress(self, recs) -> list:
+    """dense weights per (compressed entries, args) record; None where the table does not take it"""
+    return run_table(self, recs, _DecompressSpec(), _lib.load().ctmi_qdq_many, 0, 1)
+
+
 def _compress_modules_fast(self, members, names_to_scheme) -> None:
     """NaiveQuantizationCompressor.compress_modules: compress_module (compressors/base.py:125-151,
-    naive_quantized.py:79-114) for every (prefix, module) pair, one ctmi_qdq_many call per 64"""
-    entry = _lib.load().ctmi_qdq_many
-    table = module_table(self, _lib.QdqJob)
+    naive_quantized.py:79-114) for every (prefix, module) pair"""
     new_param = torch.nn.Parameter
-    slow, arg_keys = [], {}
-    for lo, hi in module_chunks(len(members)):
-        picked, shapes, device, code_dtype = [], [], None, None
-        for prefix, module in members[lo:hi]:
+    recs, plain = [], []
+    for prefix, module in members:
+        params = module._parameters
+        ok = _plain(params)
+        plain.append(ok)
+        # (a module that holds more than weight, scale, zero point and bias: the state-dict path)
+        recs.append((params.get("weight") if ok else None, params.get("weight_scale"),
+                     params.get("weight_zero_point"), None, None, names_to_scheme[prefix].weights))
+    outs = _table_compress(self, recs)
+    # the kernels are enqueued: the modules get their new parameters while the GPU works
+    for (prefix, module), rec, out in zip(members, recs, outs):
+        if out is not None:
             params = module._parameters
-            w, scale, zp = params.get("weight"), params.get("weight_scale"), params.get("weight_zero_point")
-            args = names_to_scheme[prefix].weights
-            key = arg_keys.get(id(args))
-            if key is None:
-                key = arg_keys[id(args)] = (args_key(args), args.pytorch_dtype() if args.num_bits <= 8 else None)
-            if (w is None or scale is None or w.ndim != 2 or w.numel() == 0 or w.dtype not in FLOAT_DTYPES
-                    or w.device.type != "cuda" or not w.is_contiguous() or scale.ndim == 0
-                    or scale.dtype not in FLOAT_DTYPES or scale.device != w.device
-                    or not scale.is_contiguous()
-                    or (zp is not None and (zp.device != w.device or not zp.is_contiguous()))
-                    or key[1] is None or not _plain(params)
-                    or (device is not None and (device, code_dtype) != (w.device, key[1]))):
-                slow.append((prefix, module))
-                continue
-            device, code_dtype = w.device, key[1]
-            picked.append((params, w, scale, zp, args, key))
-            shapes.append(tuple(w.shape))
-        if not picked:
-            continue
-        codes = slab_outputs(shapes, code_dtype, device)
-        out_code = _lib.dtype_code(code_dtype)
-        for (params, w, scale, zp, args, key), out in zip(picked, codes):
-            rows, cols = w.shape
-            tkey = ("c", rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
-            which = table.template(tkey)
-            if which < 0:
-                which = table.add_template(tkey, build_qparams(w, scale, zp, args, None, None))
-            table.add(w.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(w.dtype), which,
-                      scale.data_ptr(), 0 if zp is None else zp.data_ptr(), 0, out_code)
-        table.launch(entry, 1, 0, _lib.stream_of(device))
-        # the kernels are enqueued: the modules get their new parameters while the GPU works
-        for (params, w, scale, zp, args, key), out in zip(picked, codes):
             params["weight"] = new_param(out, requires_grad=False)
-            if args.symmetric and zp is not None:  # a symmetric scheme stores no zero points
+            if rec[5].symmetric and rec[2] is not None:  # a symmetric scheme stores no zero points
                 del params["weight_zero_point"]
+    slow = [members[i] for i, out in enumerate(outs) if out is None]
     if slow:
         BaseQuantizationCompressor.compress_modules(self, slow, names_to_scheme)
 
@@ -407,51 +476,29 @@ def _compress_modules_fast(self, members, names_to_scheme) -> None:
 def _decompress_modules_fast(self, members, names_to_scheme) -> None:
     """NaiveQuantizationCompressor.decompress_modules: decompress_module
     (compressors/base.py:165-190, naive_quantized.py:116-136) for every (prefix, module) pair"""
-    entry = _lib.load().ctmi_qdq_many
-    table = module_table(self, _lib.QdqJob)
     new_param = torch.nn.Parameter
-    slow = []
-    for lo, hi in module_chunks(len(members)):
-        picked, shapes, dtype, device = [], [], None, None
-        for prefix, module in members[lo:hi]:
-            params = module._parameters
-            codes, scale, zp = params.get("weight"), params.get("weight_scale"), params.get("weight_zero_point")
-            if (codes is None or scale is None or codes.ndim != 2 or codes.numel() == 0
-                    or codes.dtype not in (torch.int8, torch.float8_e4m3fn)
-                    or codes.device.type != "cuda" or not codes.is_contiguous()
-                    or scale.dtype not in FLOAT_DTYPES or scale.device != codes.device
-                    or not scale.is_contiguous()
-                    or (zp is not None and (zp.device != codes.device or not zp.is_contiguous()))
-                    or not _plain(params)
-                    or (dtype is not None and (dtype, device) != (scale.dtype, codes.device))):
-                slow.append((prefix, module))
-                continue
-            dtype, device = scale.dtype, codes.device
-            picked.append((params, codes, scale, zp))
-            shapes.append(tuple(codes.shape))
-        if not picked:
-            continue
-        dense = slab_outputs(shapes, dtype, device)
-        out_code = _lib.dtype_code(dtype)
-        for (params, codes, scale, zp), out in zip(picked, dense):
-            rows, cols = codes.shape
-            tkey = ("d", rows, cols, codes.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype)
-            which = table.template(tkey)
-            if which < 0:
-                # dequantize(x_q, scale, zero_point, g_idx=None): the strategy follows from the
-                # two shapes, the output dtype is the scale's (naive_quantized.py:116-136)
-                carrier = _ShapeOnly(codes.shape, codes.dtype)
-                which = table.add_template(
-                    tkey, build_qparams(carrier, scale, zp, infer_dequant_args(carrier, scale), None, None))
-            table.add(codes.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(codes.dtype), which,
-                      scale.data_ptr(), 0 if zp is None else zp.data_ptr(), 0, out_code)
-        table.launch(entry, 0, 1, _lib.stream_of(device))
-        for (params, codes, scale, zp), out in zip(picked, dense):
-            params["weight"] = new_param(out, requires_grad=False)
+    recs = [(module._parameters if _plain(module._parameters) else {}, None) for _, module in members]
+    outs = _table_decompress(self, recs)
+    for (prefix, module), out in zip(members, outs):
+        if out is not None:
+            module._parameters["weight"] = new_param(out, requires_grad=False)
+    slow = [members[i] for i, out in enumerate(outs) if out is None]
     if slow:
         BaseQuantizationCompressor.decompress_modules(self, slow, names_to_scheme)
 
 
+def _decompress_weights_batched(self, items) -> list:
+    """NaiveQuantizationCompressor.decompress_weight for a list of (compressed_data,
+    quantization_args) pairs: many-weight calls where the job table takes them"""
+    outs = _table_decompress(self, items)
+    for k, out in enumerate(outs):
+        if out is None:
+            outs[k] = self.decompress_weight(compressed_data=items[k][0], quantization_args=items[k][1])
+    return outs
+
+
+NaiveQuantizationCompressor.decompress_weights = _decompress_weights_batched
+NaiveQuantizationCompressor.table_compress = _table_compress
 NaiveQuantizationCompressor.compress_modules = _compress_modules_fast
 NaiveQuantizationCompressor.decompress_modules = _decompress_modules_fast
 

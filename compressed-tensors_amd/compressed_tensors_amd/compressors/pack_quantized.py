@@ -16,7 +16,7 @@ from torch import Tensor
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import BaseCompressor, to_gpu
 from compressed_tensors_amd.compressors.job_tables import (
-    FLOAT_DTYPES, args_key, module_chunks, module_table, slab_outputs,
+    FLOAT_DTYPES, args_key, on_gpu, run_table,
 )
 from compressed_tensors_amd.compressors.quantized_base import (
     BaseQuantizationCompressor, LazyDenseOutputs,
@@ -323,18 +323,32 @@ class PackedQuantizationCompressor(BaseQuantizationCompressor):
         return out
 
 
+class _Leftover(list):
+    """(compressed entries, args) pairs the job table did not take"""
+    _no_table = True
+
+
 def _decompress_weights_batched(self, items) -> list:
     """PackedQuantizationCompressor.decompress_weight (pack_quantized.py:147-183) for a list
     of (compressed_data, quantization_args) pairs from one ctmi_pack_quantized_decompress_many
     call; same tensors as the per-weight calls"""
+    if not items:
+        return []
+    if not getattr(items, "_no_table", False):
+        # the common case through the job table written by columns, the rest below
+        outs = _table_decompress(self, items)
+        left = [k for k, out in enumerate(outs) if out is None]
+        if left:
+            rest = _Leftover(items[k] for k in left)
+            for k, out in zip(left, _decompress_weights_batched(self, rest)):
+                outs[k] = out
+        return outs
     if len(items) > _CHUNK:  # the GPU starts on the first chunk while the rest is prepared
         outs = []
         for at in range(0, len(items), _CHUNK):
-            outs += _decompress_weights_batched(self, items[at:at + _CHUNK])
+            outs += _decompress_weights_batched(self, _Leftover(items[at:at + _CHUNK]))
         return outs
     n = len(items)
-    if n == 0:
-        return []
     jobs = (_lib.WeightJob * n)()
     outs, keep, device = [], [], None
     for i, (data, args) in enumerate(items):
@@ -535,37 +549,52 @@ class ObservedWeightBatch:
 
 
 def _compress_state_dict_batched(self, model_state, names_to_scheme, show_progress=False,
-                                 compression_device=None, **kwargs):
+                                 compression_device=None, precomputed=None, **kwargs):
     """BaseQuantizationCompressor.compress for pack-quantized with every weight
     handed to the C ABI in one call (same keys, dtypes and shapes as the
     per-weight loop)."""
     jobs, order = [], []
-    for name in list(model_state.keys()):
-        if not name.endswith("weight"):
-            continue
-        prefix = name[: -len("weight")]
-        scale = model_state.get(prefix + "weight_scale", None)
-        if scale is None:
-            continue
-        module_path = prefix[:-1] if prefix.endswith(".") else prefix
-        args = names_to_scheme[module_path].weights
-        weight = model_state[name]
-        if model_state.get(prefix + "weight_global_scale", None) is not None:
-            raise ValueError("global_scale is not supported for the PackQuantizationCompressor")
-        if not can_quantize(weight, args) or weight.ndim != 2:
-            continue  # handled by the per-weight path below
-        jobs.append(dict(name=name, weight=weight, scale=scale,
-                         zero_point=model_state.get(prefix + "weight_zero_point", None),
-                         g_idx=model_state.get(prefix + "weight_g_idx", None),
-                         quantization_args=args))
-        order.append((name, prefix, args))
-    packed_by_name = {}
-    # a few launches' worth of weights per call: the GPU works on one chunk while the
-    # host prepares the job table of the next
-    for at in range(0, len(jobs), _CHUNK):
-        batch = PackedWeightBatch(jobs[at:at + _CHUNK])
-        for (name, prefix, args), packed in zip(order[at:at + _CHUNK], batch.compress()):
-            packed_by_name[name] = packed
+
+    def candidates():
+        # (a generator: the first many-weight call goes out while later names are still looked at)
+        for name in list(model_state.keys()):
+            if not name.endswith("weight") or (precomputed is not None and name in precomputed):
+                continue
+            prefix = name[: -len("weight")]
+            scale = model_state.get(prefix + "weight_scale", None)
+            if scale is None:
+                continue
+            module_path = prefix[:-1] if prefix.endswith(".") else prefix
+            args = names_to_scheme[module_path].weights
+            weight = model_state[name]
+            if model_state.get(prefix + "weight_global_scale", None) is not None:
+                raise ValueError("global_scale is not supported for the PackQuantizationCompressor")
+            if not can_quantize(weight, args) or weight.ndim != 2:
+                continue  # handled by the per-weight path below
+            job = dict(name=name, weight=weight, scale=scale,
+                       zero_point=model_state.get(prefix + "weight_zero_point", None),
+                       g_idx=model_state.get(prefix + "weight_g_idx", None),
+                       quantization_args=args)
+            jobs.append(job)
+            order.append((name, prefix, args))
+            yield (weight, scale, job["zero_point"], None, job["g_idx"], args)
+
+    packed_by_name = dict(precomputed or {})  # (what the caller enqueued from the modules already)
+    # the common case through the job table written by columns ...
+    outs = _table_compress(self, candidates())
+    left = []
+    for k, out in enumerate(outs):
+        if out is None:
+            left.append(k)
+        else:
+            packed_by_name[order[k][0]] = out
+    # ... the rest (asymmetric, activation-ordered, not yet on the GPU) a few launches' worth
+    # of weights per call: the GPU works on one chunk while the host prepares the next
+    for at in range(0, len(left), _CHUNK):
+        part = left[at:at + _CHUNK]
+        batch = PackedWeightBatch([jobs[k] for k in part])
+        for k, packed in zip(part, batch.compress()):
+            packed_by_name[order[k][0]] = packed
 
     def move(t):
         return t if compression_device is None else t.to(compression_device)
@@ -611,62 +640,126 @@ PackedQuantizationCompressor.compress = _compress_state_dict_batched
 _FLOAT_DTYPES = FLOAT_DTYPES
 # what compression takes away from a module or writes anew (a symmetric scheme stores no zero points)
 _REPLACED = ("weight", "weight_zero_point", "weight_packed", "weight_shape")
-_chunks, _module_table, _args_key = module_chunks, module_table, args_key
+_args_key = args_key
+
+
+class _CompressSpec:
+    """what run_table needs for ctmi_pack_quantized_compress_many.  Records are
+    (weight, scale, zero_point, global_scale, g_idx, args).  Taken: a 2-D float weight on the
+    GPU, group or channel scales, symmetric, no activation ordering."""
+    job_struct = _lib.WeightJob
+
+    def __init__(self):
+        self._args = {}
+
+    def key(self, rec):
+        w, scale, zp, gs, g_idx, args = rec
+        k = self._args.get(id(args))
+        if k is None:
+            k = self._args[id(args)] = _args_key(args)
+        if (gs is not None or g_idx is not None or not on_gpu(w) or w.ndim != 2 or w.numel() == 0
+                or w.dtype not in _FLOAT_DTYPES or not on_gpu(scale, w.device)
+                or scale.dtype not in _FLOAT_DTYPES or (zp is not None and not on_gpu(zp, w.device))
+                or not k[2] or k[3] not in _PACKABLE or k[1] != "int" or not 1 <= k[0] <= 8):
+            return None
+        return ("c", w.shape, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, k)
+
+    def out_spec(self, rec):
+        w, args = rec[0], rec[5]
+        return (w.shape[0], -(-w.shape[1] // (32 // args.num_bits))), torch.int32, w.device
+
+    def plan(self, rec):
+        w, scale, zp, gs, g_idx, args = rec
+        # the zero points of a symmetric scheme (all zero) take part in the arithmetic as they
+        # are, as in the reference's compress_weight
+        return build_qparams(w, scale, zp, args, None, None)
+
+    def row(self, rec, out):
+        w, scale, zp = rec[0], rec[1], rec[2]
+        return (w.data_ptr(), out.data_ptr(), w.shape[0], w.shape[1], _lib.dtype_code(w.dtype),
+                scale.data_ptr(), 0 if zp is None else zp.data_ptr(), 0, 0)
+
+
+class _DecompressSpec:
+    """... for ctmi_pack_quantized_decompress_many.  Records are (compressed entries of one
+    weight under their local names, args).  Taken: packed words and 2-D float scales on the
+    GPU, symmetric (no zero points), no activation ordering."""
+    job_struct = _lib.WeightJob
+
+    def __init__(self):
+        self._shapes = {}
+
+    def key(self, rec):
+        data, args = rec
+        packed, scale, ws = data.get("weight_packed"), data.get("weight_scale"), data.get("weight_shape")
+        if (ws is None or not on_gpu(packed) or packed.dtype is not torch.int32 or packed.ndim != 2
+                or not on_gpu(scale, packed.device) or scale.ndim != 2 or scale.dtype not in _FLOAT_DTYPES
+                or not args.symmetric or args.strategy not in _PACKABLE or not 1 <= args.num_bits <= 8
+                or data.get("weight_zero_point") is not None or data.get("weight_g_idx") is not None
+                or (isinstance(ws, Tensor) and ws.device.type != "cpu")):
+            return None
+        shape = tuple(ws.flatten().tolist() if isinstance(ws, Tensor) else [int(d) for d in ws])
+        if len(shape) != 2 or packed.shape != (shape[0], -(-shape[1] // (32 // args.num_bits))):
+            return None
+        self._shapes[id(data)] = shape
+        return ("d", shape, scale.shape, scale.dtype, args.num_bits)
+
+    def out_spec(self, rec):
+        data = rec[0]
+        return self._shapes[id(data)], data["weight_scale"].dtype, data["weight_packed"].device
+
+    def plan(self, rec):
+        data, args = rec
+        # dequantize(x_q, scale, zero_point=None, args=None): the strategy follows from the two
+        # shapes, the output dtype is the scale's (pack_quantized.py:176-181)
+        scale = data["weight_scale"]
+        carrier = _ShapeOnly(self._shapes[id(data)], torch.int8)
+        plan = build_qparams(carrier, scale, None, infer_dequant_args(carrier, scale), None, None)
+        plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_INT, args.num_bits
+        return plan
+
+    def row(self, rec, out):
+        data = rec[0]
+        scale = data["weight_scale"]
+        shape = self._shapes[id(data)]
+        return (data["weight_packed"].data_ptr(), out.data_ptr(), shape[0], shape[1],
+                _lib.dtype_code(scale.dtype), scale.data_ptr(), 0, 0, 0)
+
+
+def _table_compress(self, recs) -> list:
+    """packed words per (weight, scale, zero_point, global_scale, g_idx, args) record from
+    many-weight calls; None where the record is not one the job table takes"""
+    return run_table(self, recs, _CompressSpec(), _lib.load().ctmi_pack_quantized_compress_many)
+
+
+def _table_decompress(self, recs) -> list:
+    """dense weights per (compressed entries, args) record; None where the table does not take it"""
+    return run_table(self, recs, _DecompressSpec(), _lib.load().ctmi_pack_quantized_decompress_many)
 
 
 def _compress_modules_fast(self, members, names_to_scheme) -> None:
     """PackedQuantizationCompressor.compress_modules: compress_module
     (compressors/base.py:125-151, pack_quantized.py:88-146) for every (prefix, module) pair"""
-    entry = _lib.load().ctmi_pack_quantized_compress_many
-    table = _module_table(self)
     new_param = torch.nn.Parameter
-    slow, arg_keys = [], {}
-    for lo, hi in _chunks(len(members)):
-        picked, shapes, device = [], [], None
-        for prefix, module in members[lo:hi]:
-            params = module._parameters
-            w, scale, zp = params.get("weight"), params.get("weight_scale"), params.get("weight_zero_point")
-            args = names_to_scheme[prefix].weights
-            key = arg_keys.get(id(args))
-            if key is None:
-                key = arg_keys[id(args)] = _args_key(args)
-            if (w is None or scale is None or w.ndim != 2 or w.dtype not in _FLOAT_DTYPES
-                    or w.device.type != "cuda" or not w.is_contiguous()
-                    or scale.dtype not in _FLOAT_DTYPES or scale.device != w.device
-                    or not scale.is_contiguous()
-                    or (zp is not None and (zp.device != w.device or not zp.is_contiguous()))
-                    or not key[2] or key[3] not in _PACKABLE or key[1] != "int" or not 1 <= key[0] <= 8
-                    or (device is not None and device != w.device)
-                    or params.get("weight_g_idx") is not None
-                    or params.get("weight_global_scale") is not None):
-                slow.append((prefix, module))
-                continue
-            device = w.device
-            rows, cols = w.shape
-            picked.append((params, w, scale, zp, args, key, rows, cols))
-            shapes.append((rows, -(-cols // (32 // key[0]))))
-        if not picked:
-            continue
-        packed = slab_outputs(shapes, torch.int32, device)
-        dims = torch.tensor([(p[6], p[7]) for p in picked]).unbind(0)  # every weight_shape, one host tensor
-        for (params, w, scale, zp, args, key, rows, cols), out in zip(picked, packed):
-            tkey = ("c", rows, cols, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, key)
-            which = table.template(tkey)
-            if which < 0:
-                # the zero points of a symmetric scheme (all zero) take part in the arithmetic
-                # as they are, as in the reference's compress_weight
-                plan = build_qparams(w, scale, zp, args, None, None)
-                which = table.add_template(tkey, plan)
-            table.add(w.data_ptr(), out.data_ptr(), rows, cols, _lib.dtype_code(w.dtype), which,
-                      scale.data_ptr(), 0 if zp is None else zp.data_ptr())
-        table.launch(entry, _lib.stream_of(device))
-        # the kernels are enqueued: the modules get their new parameters while the GPU works
-        for (params, w, scale, zp, args, key, rows, cols), out, dim in zip(picked, packed, dims):
+    recs = []
+    for prefix, module in members:
+        params = module._parameters
+        recs.append((params.get("weight"), params.get("weight_scale"), params.get("weight_zero_point"),
+                     params.get("weight_global_scale"), params.get("weight_g_idx"),
+                     names_to_scheme[prefix].weights))
+    outs = _table_compress(self, recs)
+    # the kernels are enqueued: the modules get their new parameters while the GPU works
+    taken = [i for i, out in enumerate(outs) if out is not None]
+    if taken:
+        dims = torch.tensor([tuple(recs[i][0].shape) for i in taken]).unbind(0)  # every weight_shape, one host tensor
+        for i, dim in zip(taken, dims):
+            params = members[i][1]._parameters
             rest = [(n, p) for n, p in params.items() if n not in _REPLACED]
             params.clear()
-            params["weight_packed"] = new_param(out, requires_grad=False)
+            params["weight_packed"] = new_param(outs[i], requires_grad=False)
             params["weight_shape"] = new_param(dim, requires_grad=False)
             params.update(rest)
+    slow = [members[i] for i, out in enumerate(outs) if out is None]
     if slow:
         BaseQuantizationCompressor.compress_modules(self, slow, names_to_scheme)
 
@@ -674,54 +767,17 @@ def _compress_modules_fast(self, members, names_to_scheme) -> None:
 def _decompress_modules_fast(self, members, names_to_scheme) -> None:
     """PackedQuantizationCompressor.decompress_modules: decompress_module
     (compressors/base.py:165-190, pack_quantized.py:147-183) for every (prefix, module) pair"""
-    entry = _lib.load().ctmi_pack_quantized_decompress_many
-    table = _module_table(self)
     new_param = torch.nn.Parameter
-    slow = []
-    for lo, hi in _chunks(len(members)):
-        picked, shapes, dtype, device = [], [], None, None
-        for prefix, module in members[lo:hi]:
-            params = module._parameters
-            packed, scale, ws = params.get("weight_packed"), params.get("weight_scale"), params.get("weight_shape")
-            args = names_to_scheme[prefix].weights
-            if (packed is None or scale is None or ws is None or ws.device.type != "cpu"
-                    or packed.dtype is not torch.int32 or packed.ndim != 2 or packed.device.type != "cuda"
-                    or not packed.is_contiguous() or scale.ndim != 2 or scale.dtype not in _FLOAT_DTYPES
-                    or scale.device != packed.device or not scale.is_contiguous()
-                    or not args.symmetric or args.strategy not in _PACKABLE or not 1 <= args.num_bits <= 8
-                    or params.get("weight_zero_point") is not None
-                    or params.get("weight_g_idx") is not None
-                    or (dtype is not None and (dtype, device) != (scale.dtype, packed.device))):
-                slow.append((prefix, module))
-                continue
-            shape = tuple(ws.tolist())
-            if len(shape) != 2 or packed.shape != (shape[0], -(-shape[1] // (32 // args.num_bits))):
-                slow.append((prefix, module))
-                continue
-            dtype, device = scale.dtype, packed.device
-            picked.append((params, packed, scale, args.num_bits, shape))
-            shapes.append(shape)
-        if not picked:
-            continue
-        dense = slab_outputs(shapes, dtype, device)
-        for (params, packed, scale, num_bits, shape), out in zip(picked, dense):
-            tkey = ("d", shape, scale.shape, scale.dtype, num_bits)
-            which = table.template(tkey)
-            if which < 0:
-                # dequantize(x_q, scale, zero_point=None, args=None): the strategy follows from
-                # the two shapes, the output dtype is the scale's (pack_quantized.py:176-181)
-                carrier = _ShapeOnly(shape, torch.int8)
-                plan = build_qparams(carrier, scale, None, infer_dequant_args(carrier, scale), None, None)
-                plan.qp.qtype, plan.qp.num_bits = _lib.QTYPE_INT, num_bits
-                which = table.add_template(tkey, plan)
-            table.add(packed.data_ptr(), out.data_ptr(), shape[0], shape[1], _lib.dtype_code(scale.dtype),
-                      which, scale.data_ptr())
-        table.launch(entry, _lib.stream_of(device))
-        for (params, packed, scale, num_bits, shape), out in zip(picked, dense):
-            params["weight"] = new_param(out, requires_grad=False)
+    recs = [(module._parameters, names_to_scheme[prefix].weights) for prefix, module in members]
+    outs = _table_decompress(self, recs)
+    for (prefix, module), out in zip(members, outs):
+        if out is not None:
+            module._parameters["weight"] = new_param(out, requires_grad=False)
+    slow = [members[i] for i, out in enumerate(outs) if out is None]
     if slow:
         BaseQuantizationCompressor.decompress_modules(self, slow, names_to_scheme)
 
 
+PackedQuantizationCompressor.table_compress = _table_compress
 PackedQuantizationCompressor.compress_modules = _compress_modules_fast
 PackedQuantizationCompressor.decompress_modules = _decompress_modules_fast

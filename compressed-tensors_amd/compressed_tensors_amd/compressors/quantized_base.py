@@ -159,14 +159,15 @@ class BaseQuantizationCompressor(BaseCompressor):
         self, state_dict: Dict[str, Tensor], names_to_scheme: Dict[str, Any]
     ) -> Generator[Tuple[str, Dict[str, Tensor]], None, None]:
         nested = nest_state_dict(state_dict, self.compression_param_names)
-        for module_path, weight_data in nested.items():
-            weight_data = dict(weight_data)
-            if "weight_scale" in weight_data:
-                quant_args = names_to_scheme[module_path].weights
-                weight_data["weight"] = self.decompress_weight(
-                    compressed_data=weight_data, quantization_args=quant_args
-                )
-                yield module_path, weight_data
+        todo = [(module_path, dict(weight_data)) for module_path, weight_data in nested.items()
+                if "weight_scale" in weight_data]
+        # every weight of the state dict in many-weight calls where the format has them: the
+        # kernels are enqueued before the first module is handed back
+        dense = self.decompress_weights(
+            [(weight_data, names_to_scheme[module_path].weights) for module_path, weight_data in todo])
+        for (module_path, weight_data), weight in zip(todo, dense):
+            weight_data["weight"] = weight
+            yield module_path, weight_data
 
     def decompress_weights(self, items) -> list:
         """decompress_weight for a list of (compressed_data, quantization_args) pairs;

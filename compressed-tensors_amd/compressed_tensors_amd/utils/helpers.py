@@ -114,6 +114,16 @@ def nest_state_dict(state_dict, params_to_nest, return_unmatched_params: bool = 
     {module_path: {param_name: tensor}} (+ the entries that matched nothing).
     Reference: utils/safetensors_load.py:251-291."""
     nested, unmatched = {}, {}
+    names = set(params_to_nest)
+    if not any("." in n for n in names):
+        # every name is a last component: one split per key
+        for key, value in state_dict.items():
+            module_path, _, last = key.rpartition(".")
+            if module_path and last in names:
+                nested.setdefault(module_path, {})[last] = value
+            else:
+                unmatched[key] = value
+        return (nested, unmatched) if return_unmatched_params else nested
     for key, value in state_dict.items():
         hit = False
         for param_name in params_to_nest:

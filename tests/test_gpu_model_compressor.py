@@ -455,6 +455,12 @@ def test_module_pathway_of_the_other_formats(fmt, spec, gpu):
             oracle_in[name] = (w.cpu(), scale.cpu(), zp.cpu(), None if gs is None else gs.cpu())
     mc = ModelCompressor(quantization_config=config)
     want = mc.compress(model)
+    # (compress(model) enqueues from the modules before it builds the state dict; given the
+    # state dict it cannot: same entries, same order)
+    given = mc.compress(model, state_dict=model.state_dict())
+    assert list(given) == list(want)
+    for name in want:
+        assert_bit_equal(given[name], want[name].to(given[name].device), f"{name} from a given state dict")
     mc.compress_model(model)
     got = {n: p.data for n, p in model.named_parameters()}
     assert set(got) == set(want)
