@@ -26,7 +26,9 @@ __all__ = [
     "sparse24_bitmask_compress_many",
     "sparse24_bitmask_decompress_many",
     "quantize_sparse24_compress",
+    "quantize_sparse24_compress_many",
     "sparse24_decompress_dequantize",
+    "sparse24_decompress_dequantize_many",
     "get_24_bytemasks",
 ]
 
@@ -240,6 +242,109 @@ def sparse24_decompress_dequantize(values: Tensor, bitmask: Tensor, original_sha
         )
     )
     return out
+
+
+# What decides the qparams of a stacked weight besides addresses -> (the qparams as bytes, does
+# the fused kernel take the layout?): a model has a handful of such combinations.
+_stacked_compress_plans: Dict[Tuple, Tuple[bytes, bool]] = {}
+_stacked_decompress_plans: Dict[Tuple, Tuple[bytes, bool]] = {}
+_FLOATS = (torch.bfloat16, torch.float16, torch.float32)
+
+
+def quantize_sparse24_compress_many(recs) -> List[Optional[Tuple[Tensor, Tensor]]]:
+    """quantize_sparse24_compress for (weight, scale, zero_point, args) records whose tensors are
+    on the GPU already: one kernel per weight as there, but the qparams of a (shape, dtype,
+    scheme) combination are derived once, outputs of one shape share allocations and nothing
+    else happens between the launches.  None for records this does not take."""
+    import ctypes
+
+    from compressed_tensors_amd.compressors.job_tables import args_key, on_gpu, slab_outputs
+    from compressed_tensors_amd.quantization.forward import build_qparams
+
+    lib = _lib.load()
+    outs: List[Optional[Tuple[Tensor, Tensor]]] = [None] * len(recs)
+    groups: Dict[Tuple, List] = {}
+    for i, (w, scale, zp, args) in enumerate(recs):
+        if (not on_gpu(w) or w.ndim != 2 or w.numel() == 0 or w.dtype not in _FLOATS
+                or w.data_ptr() % (8 * w.element_size()) or not on_gpu(scale, w.device)
+                or scale.dtype not in _FLOATS or scale.ndim == 0 or args.num_bits > 8
+                or (zp is not None and not on_gpu(zp, w.device))):
+            continue
+        key = (w.shape, w.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype, args_key(args))
+        plan = _stacked_compress_plans.get(key)
+        if plan is None:
+            if len(_stacked_compress_plans) > 1024:
+                _stacked_compress_plans.clear()
+            qplan = build_qparams(w, scale, zp, args, None, None)
+            ok = bool(lib.ctmi_quantize_sparse24_compress_supported(
+                _lib.dtype_code(w.dtype), w.shape[0], w.shape[1], ctypes.byref(qplan.qp)))
+            plan = _stacked_compress_plans[key] = (bytes(qplan.qp), ok)
+        if plan[1]:
+            groups.setdefault((args.pytorch_dtype(), w.device), []).append((i, plan[0]))
+    for (code_dtype, device), items in groups.items():
+        stream = _lib.stream_of(device)
+        values = slab_outputs([(recs[i][0].shape[0], recs[i][0].shape[1] // 2) for i, _ in items], code_dtype, device)
+        bitmasks = slab_outputs([(recs[i][0].shape[0], recs[i][0].shape[1] // 8) for i, _ in items], torch.uint8, device)
+        for (i, raw), v, b in zip(items, values, bitmasks):
+            w, scale, zp, _ = recs[i]
+            qp = _lib.QParams.from_buffer_copy(raw)
+            qp.scale = scale.data_ptr()
+            qp.zero_point = None if zp is None else zp.data_ptr()
+            _lib.check(lib.ctmi_quantize_sparse24_compress(
+                w.data_ptr(), _lib.dtype_code(w.dtype), v.data_ptr(), b.data_ptr(), w.shape[0], w.shape[1],
+                ctypes.byref(qp), stream))
+            outs[i] = (v, b)
+    return outs
+
+
+def sparse24_decompress_dequantize_many(recs) -> List[Optional[Tensor]]:
+    """sparse24_decompress_dequantize for (values, bitmask, shape, scale, zero_point) records
+    whose tensors are on the GPU already (shape: a pair of ints); None for records this does
+    not take"""
+    import ctypes
+
+    from compressed_tensors_amd.compressors.job_tables import on_gpu, slab_outputs
+    from compressed_tensors_amd.quantization.forward import _ShapeOnly, build_qparams, infer_dequant_args
+
+    lib = _lib.load()
+    outs: List[Optional[Tensor]] = [None] * len(recs)
+    groups: Dict[Tuple, List] = {}
+    for i, (values, bitmask, shape, scale, zp) in enumerate(recs):
+        if (len(shape) != 2 or not on_gpu(values) or values.dtype not in (torch.int8, torch.float8_e4m3fn)
+                or not on_gpu(bitmask, values.device) or not on_gpu(scale, values.device)
+                or scale.dtype not in _FLOATS or (zp is not None and not on_gpu(zp, values.device))):
+            continue
+        rows, cols = shape
+        if (rows == 0 or cols == 0 or cols % 8 or values.numel() * 2 != rows * cols
+                or bitmask.numel() * 8 != rows * cols or values.data_ptr() % 4):
+            continue
+        key = (rows, cols, values.dtype, scale.shape, scale.dtype, None if zp is None else zp.dtype)
+        plan = _stacked_decompress_plans.get(key)
+        if plan is None:
+            if len(_stacked_decompress_plans) > 1024:
+                _stacked_decompress_plans.clear()
+            codes = _ShapeOnly((rows, cols), values.dtype)
+            qplan = build_qparams(codes, scale, zp, infer_dequant_args(codes, scale), None, None)
+            ok = bool(lib.ctmi_sparse24_decompress_dequantize_supported(
+                _lib.dtype_code(values.dtype), _lib.dtype_code(scale.dtype), rows, cols, ctypes.byref(qplan.qp)))
+            ok = ok and lib.ctmi_sparse24_dequantize_tmp_bytes(rows, cols) == 0
+            plan = _stacked_decompress_plans[key] = (bytes(qplan.qp), ok)
+        if plan[1]:
+            groups.setdefault((scale.dtype, values.device), []).append((i, plan[0]))
+    for (dtype, device), items in groups.items():
+        stream = _lib.stream_of(device)
+        dense = slab_outputs([tuple(recs[i][2]) for i, _ in items], dtype, device)
+        ocode = _lib.dtype_code(dtype)
+        for (i, raw), out in zip(items, dense):
+            values, bitmask, shape, scale, zp = recs[i]
+            qp = _lib.QParams.from_buffer_copy(raw)
+            qp.scale = scale.data_ptr()
+            qp.zero_point = None if zp is None else zp.data_ptr()
+            _lib.check(lib.ctmi_sparse24_decompress_dequantize(
+                values.data_ptr(), values.numel(), _lib.dtype_code(values.dtype), bitmask.data_ptr(),
+                out.data_ptr(), ocode, None, shape[0], shape[1], ctypes.byref(qp), stream))
+            outs[i] = out
+    return outs
 
 
 def sparse24_bitmask_decompress(

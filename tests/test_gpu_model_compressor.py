@@ -142,9 +142,18 @@ def test_fp8_plus_sparse24_stack(gpu):
     other = copy.deepcopy(model)
     for name in cpu:
         other.get_submodule(name).weight.data.zero_()
-    with mock.patch.object(mc, "_decompress_quantized_24", wraps=mc._decompress_quantized_24) as fused:
+    from compressed_tensors_amd.compressors import sparse_24_bitmask as s24
+
+    taken = []
+
+    def spy(recs, inner=s24.sparse24_decompress_dequantize_many):
+        out = inner(recs)
+        taken.extend(o is not None for o in out)
+        return out
+
+    with mock.patch.object(s24, "sparse24_decompress_dequantize_many", spy):
         mc.decompress(dict(state), other)
-    assert fused.call_count == len(cpu)
+    assert len(taken) == len(cpu) and all(taken)  # every module through the one-pass kernel
     for name in cpu:
         assert_bit_equal(other.get_submodule(name).weight.data, want[name], f"{name} from the state dict")
         assert_bit_equal(other.get_submodule(name).weight_scale.data, cpu[name][1], f"{name}.weight_scale")
@@ -155,9 +164,10 @@ def test_fp8_plus_sparse24_stack(gpu):
         assert_bit_equal(module.compressed.data, state[f"{name}.compressed"], f"{name}.compressed in memory")
         assert_bit_equal(module.bitmask.data, state[f"{name}.bitmask"], f"{name}.bitmask in memory")
         assert not hasattr(module, "weight")
-    with mock.patch.object(mc, "_decompress_quantized_24", wraps=mc._decompress_quantized_24) as fused:
+    taken.clear()
+    with mock.patch.object(s24, "sparse24_decompress_dequantize_many", spy):
         mc.decompress_model(model)
-    assert fused.call_count == len(cpu)
+    assert len(taken) == len(cpu) and all(taken)  # every module through the one-pass kernel
     for name in cpu:
         assert_bit_equal(model.get_submodule(name).weight.data, want[name], f"{name} decompressed")
 
@@ -489,3 +499,45 @@ def test_module_pathway_of_the_other_formats(fmt, spec, gpu):
     mc.compress_model(model)
     again = {n: p.data for n, p in model.named_parameters()}
     assert set(again) == set(want)
+
+
+@pytest.mark.parametrize("fmt", ["sparse-24-bitmask", "sparse-bitmask"])
+def test_sparsity_only_model_in_memory(fmt, gpu):
+    """compress_model / decompress_model with a sparsity compressor alone (the targets of a
+    batch share one call of the compressor): the modules hold what compress(model) returns,
+    the way back is lossless, forward runs"""
+    from compressed_tensors_amd.compressors import ModelCompressor
+    from compressed_tensors_amd.config import SparsityCompressionConfig
+
+    announce("sparsity-only model", fmt)
+    torch.manual_seed(9)
+    model = Tiny(layers=2).to(torch.bfloat16).to(gpu)
+    dense = {}
+    for name, m in model.named_modules():
+        if isinstance(m, torch.nn.Linear):
+            keep = osp.get_24_bytemasks(m.weight.data.cpu()).to(gpu)
+            m.weight.data = torch.where(keep, m.weight.data, torch.zeros_like(m.weight.data))
+            dense[name] = m.weight.data.clone()
+    scfg = SparsityCompressionConfig(format=fmt, targets=["Linear"], ignore=["lm_head"],
+                                     sparsity_structure="2:4" if fmt == "sparse-24-bitmask" else "unstructured")
+    mc = ModelCompressor(sparsity_config=scfg)
+    want = mc.compress(model)
+    mc.compress_model(model)
+    got = {n: p.data for n, p in model.named_parameters()}
+    assert set(got) == set(want)
+    for name in want:
+        assert_bit_equal(got[name], want[name].to(got[name].device), name)
+    for name in dense:
+        if name == "lm_head":
+            continue
+        values, bitmask = (osp.sparse24_bitmask_compress(dense[name].cpu()) if fmt == "sparse-24-bitmask"
+                           else osp.bitmask_compress(dense[name].cpu())[:2])
+        assert_bit_equal(got[f"{name}.compressed"], values, f"{name}.compressed")
+        assert_bit_equal(got[f"{name}.bitmask"], bitmask, f"{name}.bitmask")
+        assert not hasattr(model.get_submodule(name), "weight")
+    mc.decompress_model(model)
+    for name, w in dense.items():
+        m = model.get_submodule(name)
+        assert_bit_equal(m.weight.data, w.cpu(), f"{name} restored")
+        x = torch.randn(2, m.in_features, device=gpu).bfloat16()
+        assert_bit_equal(m(x), torch.nn.functional.linear(x, w).cpu(), f"{name} forward")
