@@ -337,6 +337,7 @@ def other_workload(torch, name, seed):
         copies = 6
         c_calls, d_calls, s_calls, t_calls, two_step, one_step = [], [], [], [], [], []
         back_two, back_one, s16_calls, t16_calls, pk_calls, up_calls = [], [], [], [], [], []
+        stacked_jobs = []
         nb = 8192 * 8192
         nnz_total = 0
         for _ in range(copies):
@@ -420,6 +421,16 @@ def other_workload(torch, name, seed):
                   tmp_dq.data_ptr(), rows, cols, ctypes.byref(plan.qp), st)
             back_two.append(lambda d=d, dq=dq: (_lib.check(lib.ctmi_sparse24_decompress(*d)), _lib.check(lib.ctmi_qdq(*dq))))
             back_one.append(lambda fd=fd: _lib.check(lib.ctmi_sparse24_decompress_dequantize(*fd)))
+            stacked_jobs.append((w, values, bitmask, back, rows, cols, plan))
+        # the stacked case for all weights from one call (8 per launch)
+        qc, qd = (_lib.Stacked24Job * copies24)(), (_lib.Stacked24Job * copies24)()
+        for k, (w, values, bitmask, back, rows, cols, plan) in enumerate(stacked_jobs):
+            for job, dense_side in ((qc[k], w), (qd[k], back)):
+                job.dense, job.values, job.bitmask = dense_side.data_ptr(), values.data_ptr(), bitmask.data_ptr()
+                job.rows, job.cols = rows, cols
+                job.dense_dtype, job.values_dtype, job.qp = code(dense_side.dtype), code(FP8), plan.qp
+        qcm, qdm = (qc, copies24, st), (qd, copies24, st)
+        keep.extend([qc, qd])
         cj, dj = (_lib.Sparse24Job * copies24)(), (_lib.Sparse24Job * copies24)()
         for k, (q, values, bitmask, dense, rows, cols) in enumerate(s24_jobs):
             for job, full in ((cj[k], q), (dj[k], dense)):
@@ -463,7 +474,13 @@ def other_workload(torch, name, seed):
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
                Op("bf16 -> fp8 codes -> 2:4 compress, one pass", one_step, fused24_bytes, "quant_sparse24_compress_kernel"),
                Op("2:4 decompress -> fp8 codes -> bf16, two steps", back_two, fused24_bytes, "qdq_vec_kernel", primary=False),
-               Op("2:4 decompress -> fp8 codes -> bf16, one pass", back_one, fused24_bytes, "sparse24_scatter_dequant_kernel")]
+               Op("2:4 decompress -> fp8 codes -> bf16, one pass", back_one, fused24_bytes, "sparse24_scatter_dequant_kernel"),
+               Op("bf16 -> fp8 codes -> 2:4 compress, one pass, all 16 in one call (8 per launch)",
+                  [lambda: _lib.check(lib.ctmi_quantize_sparse24_compress_many(*qcm))], fused24_bytes,
+                  "quant_sparse24_compress_chain_kernel", launches=chained(copies24)),
+               Op("2:4 decompress -> fp8 codes -> bf16, one pass, all 16 in one call (8 per launch)",
+                  [lambda: _lib.check(lib.ctmi_sparse24_decompress_dequantize_many(*qdm))], fused24_bytes,
+                  "sparse24_scatter_dequant_chain_kernel", launches=chained(copies24))]
         return "sparse-bitmask / sparse-24-bitmask compress+decompress GB/s", ops, keep
 
     if name == "nvfp4":

@@ -129,6 +129,21 @@ class ObservePackJob(ctypes.Structure):
     ]
 
 
+class Stacked24Job(ctypes.Structure):
+    """ctmi_stacked24_job"""
+
+    _fields_ = [
+        ("dense", c_void_p),
+        ("values", c_void_p),
+        ("bitmask", c_void_p),
+        ("rows", c_int64),
+        ("cols", c_int64),
+        ("dense_dtype", c_int32),
+        ("values_dtype", c_int32),
+        ("qp", QParams),
+    ]
+
+
 class QdqJob(ctypes.Structure):
     """ctmi_qdq_job"""
 
@@ -201,6 +216,8 @@ SIGNATURES = {
         [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_int64,
          POINTER(QParams), c_void_p],
     ),
+    "ctmi_quantize_sparse24_compress_many": (c_int32, [POINTER(Stacked24Job), c_int64, c_void_p]),
+    "ctmi_sparse24_decompress_dequantize_many": (c_int32, [POINTER(Stacked24Job), c_int64, c_void_p]),
     "ctmi_bitmask_tmp_bytes": (c_int64, [c_int64, c_int64]),
     "ctmi_bitmask_count": (
         c_int32,

@@ -251,11 +251,34 @@ _stacked_decompress_plans: Dict[Tuple, Tuple[bytes, bool]] = {}
 _FLOATS = (torch.bfloat16, torch.float16, torch.float32)
 
 
+def _stacked_call(entry, rows, device) -> None:
+    """one many-weight call for `rows` = (dense, values, bitmask, n_rows, n_cols, dense code,
+    values code, qparams bytes, scale, zero_point) tuples: the job table written by columns"""
+    import ctypes
+
+    import numpy as np
+
+    job_t, qp_t = np.dtype(_lib.Stacked24Job), np.dtype(_lib.QParams)
+    tab = np.zeros(len(rows), job_t)
+    cols = list(zip(*rows))
+    for name, col in zip(("dense", "values", "bitmask", "rows", "cols", "dense_dtype", "values_dtype"), cols):
+        tab[name] = col
+    qp = np.frombuffer(b"".join(cols[7]), dtype=qp_t).copy()
+    qp["scale"] = cols[8]
+    qp["zero_point"] = cols[9]
+    tab["qp"] = qp
+    _lib.check(entry(ctypes.cast(tab.ctypes.data, ctypes.POINTER(_lib.Stacked24Job)), len(rows),
+                     _lib.stream_of(device)))
+
+
+_STACKED_CALL = 32  # weights per call (4 launches of 8): the GPU starts while later rows are written
+
+
 def quantize_sparse24_compress_many(recs) -> List[Optional[Tuple[Tensor, Tensor]]]:
     """quantize_sparse24_compress for (weight, scale, zero_point, args) records whose tensors are
-    on the GPU already: one kernel per weight as there, but the qparams of a (shape, dtype,
-    scheme) combination are derived once, outputs of one shape share allocations and nothing
-    else happens between the launches.  None for records this does not take."""
+    on the GPU already, through ctmi_quantize_sparse24_compress_many (8 weights per launch):
+    the qparams of a (shape, dtype, scheme) combination are derived once, outputs of one shape
+    share allocations.  None for records this does not take."""
     import ctypes
 
     from compressed_tensors_amd.compressors.job_tables import args_key, on_gpu, slab_outputs
@@ -282,25 +305,26 @@ def quantize_sparse24_compress_many(recs) -> List[Optional[Tuple[Tensor, Tensor]
         if plan[1]:
             groups.setdefault((args.pytorch_dtype(), w.device), []).append((i, plan[0]))
     for (code_dtype, device), items in groups.items():
-        stream = _lib.stream_of(device)
-        values = slab_outputs([(recs[i][0].shape[0], recs[i][0].shape[1] // 2) for i, _ in items], code_dtype, device)
-        bitmasks = slab_outputs([(recs[i][0].shape[0], recs[i][0].shape[1] // 8) for i, _ in items], torch.uint8, device)
-        for (i, raw), v, b in zip(items, values, bitmasks):
-            w, scale, zp, _ = recs[i]
-            qp = _lib.QParams.from_buffer_copy(raw)
-            qp.scale = scale.data_ptr()
-            qp.zero_point = None if zp is None else zp.data_ptr()
-            _lib.check(lib.ctmi_quantize_sparse24_compress(
-                w.data_ptr(), _lib.dtype_code(w.dtype), v.data_ptr(), b.data_ptr(), w.shape[0], w.shape[1],
-                ctypes.byref(qp), stream))
-            outs[i] = (v, b)
+        vcode = _lib.dtype_code(code_dtype)
+        for at in range(0, len(items), _STACKED_CALL):
+            part = items[at:at + _STACKED_CALL]
+            values = slab_outputs([(recs[i][0].shape[0], recs[i][0].shape[1] // 2) for i, _ in part], code_dtype, device)
+            bitmasks = slab_outputs([(recs[i][0].shape[0], recs[i][0].shape[1] // 8) for i, _ in part], torch.uint8, device)
+            rows = []
+            for (i, raw), v, b in zip(part, values, bitmasks):
+                w, scale, zp, _ = recs[i]
+                rows.append((w.data_ptr(), v.data_ptr(), b.data_ptr(), w.shape[0], w.shape[1],
+                             _lib.dtype_code(w.dtype), vcode, raw, scale.data_ptr(),
+                             0 if zp is None else zp.data_ptr()))
+                outs[i] = (v, b)
+            _stacked_call(lib.ctmi_quantize_sparse24_compress_many, rows, device)
     return outs
 
 
 def sparse24_decompress_dequantize_many(recs) -> List[Optional[Tensor]]:
     """sparse24_decompress_dequantize for (values, bitmask, shape, scale, zero_point) records
-    whose tensors are on the GPU already (shape: a pair of ints); None for records this does
-    not take"""
+    whose tensors are on the GPU already (shape: a pair of ints), through
+    ctmi_sparse24_decompress_dequantize_many; None for records this does not take"""
     import ctypes
 
     from compressed_tensors_amd.compressors.job_tables import on_gpu, slab_outputs
@@ -327,23 +351,22 @@ def sparse24_decompress_dequantize_many(recs) -> List[Optional[Tensor]]:
             qplan = build_qparams(codes, scale, zp, infer_dequant_args(codes, scale), None, None)
             ok = bool(lib.ctmi_sparse24_decompress_dequantize_supported(
                 _lib.dtype_code(values.dtype), _lib.dtype_code(scale.dtype), rows, cols, ctypes.byref(qplan.qp)))
-            ok = ok and lib.ctmi_sparse24_dequantize_tmp_bytes(rows, cols) == 0
             plan = _stacked_decompress_plans[key] = (bytes(qplan.qp), ok)
         if plan[1]:
             groups.setdefault((scale.dtype, values.device), []).append((i, plan[0]))
     for (dtype, device), items in groups.items():
-        stream = _lib.stream_of(device)
-        dense = slab_outputs([tuple(recs[i][2]) for i, _ in items], dtype, device)
         ocode = _lib.dtype_code(dtype)
-        for (i, raw), out in zip(items, dense):
-            values, bitmask, shape, scale, zp = recs[i]
-            qp = _lib.QParams.from_buffer_copy(raw)
-            qp.scale = scale.data_ptr()
-            qp.zero_point = None if zp is None else zp.data_ptr()
-            _lib.check(lib.ctmi_sparse24_decompress_dequantize(
-                values.data_ptr(), values.numel(), _lib.dtype_code(values.dtype), bitmask.data_ptr(),
-                out.data_ptr(), ocode, None, shape[0], shape[1], ctypes.byref(qp), stream))
-            outs[i] = out
+        for at in range(0, len(items), _STACKED_CALL):
+            part = items[at:at + _STACKED_CALL]
+            dense = slab_outputs([tuple(recs[i][2]) for i, _ in part], dtype, device)
+            rows = []
+            for (i, raw), out in zip(part, dense):
+                values, bitmask, shape, scale, zp = recs[i]
+                rows.append((out.data_ptr(), values.data_ptr(), bitmask.data_ptr(), shape[0], shape[1],
+                             ocode, _lib.dtype_code(values.dtype), raw, scale.data_ptr(),
+                             0 if zp is None else zp.data_ptr()))
+                outs[i] = out
+            _stacked_call(lib.ctmi_sparse24_decompress_dequantize_many, rows, device)
     return outs
 
 

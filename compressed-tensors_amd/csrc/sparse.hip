@@ -12,9 +12,11 @@
 // are stored in row-major order of the set bits.
 #include <atomic>
 #include <cstddef>
+#include <cstring>
 #include <mutex>
 #include <type_traits>
 #include <unordered_map>
+#include <vector>
 
 #include "ctmi_device.h"
 #include "ctmi_host.h"
@@ -1023,6 +1025,20 @@ struct S24Table {
 };
 static_assert(offsetof(S24Table, chunk_end) == 0 && offsetof(S24Table, n_items) == 32, "find_job_index");
 
+// The stacked kernels (codes AND 2:4 in one pass) for up to 8 weights per launch.  compress: src
+// the dense weight, dst the values; decompress: src the values, dst the dense weight; an item is
+// 8 neighbouring elements of the dense side.
+struct QS24Table {  // the kernel's only argument: find_job_index reads its head
+  uint32_t chunk_end[kMaxJobs];  // running total of workgroups, job 0 .. j (unused: 0xFFFFFFFF)
+  uint32_t n_items[kMaxJobs];
+  ChainJob job[kMaxJobs];
+  uint8_t* bitmask[kMaxJobs];
+  int64_t rows[kMaxJobs];        // (decompress: what the repair needs)
+  float qmin, qmax;
+  uint32_t slot;
+};
+static_assert(offsetof(QS24Table, chunk_end) == 0 && offsetof(QS24Table, n_items) == 32, "find_job_index");
+
 // The general scatter of a whole tensor, rows dealt round-robin to the workgroups of the
 // launch; where a row's values start is the number of set bits before it, which each
 // workgroup counts by itself as it moves from one of its rows to the next (rows are whole
@@ -1245,6 +1261,95 @@ sparse24_repair_dequant_kernel(const uint8_t* __restrict__ values, int64_t nvalu
     counted = r + 1;
   }
   s24_repair_done(slot);
+}
+
+// sparse24_scatter_dequant_kernel / sparse24_repair_dequant_kernel for the weights of a
+// QS24Table: a workgroup finds its weight in the table's head, a malformed bitmask sets the
+// weight's bit in the launch's verdict word, the kernel behind redoes the weights named there.
+template <typename FT, int QK, bool HAS_ZP, bool FLAT>
+__global__ void __launch_bounds__(kBlock) sparse24_scatter_dequant_chain_kernel(const QS24Table t) {
+  using FR = typename FT::raw;
+  constexpr int U = kS24DqU;
+  __shared__ uint32_t lut[32];
+  if (threadIdx.x < 32) lut[threadIdx.x] = s24_selector<1>((int)threadIdx.x);
+  __syncthreads();
+  uint32_t local, n_items;
+  const uint32_t ji = find_job_index(blockIdx.x, &local, &n_items);
+  const ChainJob job = t.job[ji];
+  const uint8_t* __restrict__ bitmask = t.bitmask[ji];
+  const uint8_t* __restrict__ values = static_cast<const uint8_t*>(job.src);
+  const FR* __restrict__ scale = static_cast<const FR*>(job.scale);
+  const uint8_t* __restrict__ zp = reinterpret_cast<const uint8_t*>(job.zp);
+  FR* __restrict__ out = static_cast<FR*>(job.dst);
+  const uint32_t i0 = local * (kBlock * U) + threadIdx.x;
+  uint8_t m[U], zraw[U];
+  uint32_t v[U];
+  FR sraw[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    uint32_t i = i0 + k * kBlock;
+    if (i >= n_items) i = n_items - 1;  // past the end: re-read the last item (not stored)
+    const uint32_t si = chain_scale_index<FLAT>(i, job);
+    m[k] = bitmask[i];
+    v[k] = reinterpret_cast<const uint32_t*>(values)[i];
+    sraw[k] = scale[si];
+    zraw[k] = 0;
+    if constexpr (HAS_ZP) zraw[k] = zp[si];
+  }
+  bool bad = false;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t i = i0 + k * kBlock;
+    const uint32_t bits = m[k];
+    uint32_t n = bits - ((bits >> 1) & 0x55u);
+    n = (n & 0x33u) + ((n >> 2) & 0x33u);  // set bits per group of 4
+    bad |= i < n_items && n != 0x22u;
+    Vec<uint32_t, 2> cw;  // 8 codes out of 4: one v_perm_b32 per group
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      cw.v[q] = __builtin_amdgcn_perm(0u, v[k], lut[((bits >> (4 * q)) & 15u) + 16 * q]);
+    const Vec<uint8_t, 8> codes = __builtin_bit_cast(Vec<uint8_t, 8>, cw);
+    const Vec<FR, 8> o = dequant_codes8<FT, QK, HAS_ZP>(codes, sraw[k], zraw[k]);
+    if (i < n_items) stg_nt<FR, 8>(out + (int64_t)i * 8, o);
+  }
+  s24_report(t.slot, ji, bad);
+}
+
+template <typename FT, int QK, bool HAS_ZP, bool FLAT>
+__global__ void __launch_bounds__(kBlock) sparse24_repair_dequant_chain_kernel(const QS24Table t) {
+  using FR = typename FT::raw;
+  const uint32_t todo = s24_bad_jobs(t.slot);
+  if (todo == 0) return;
+  __shared__ int scan_s[kWaves];
+  __shared__ int64_t red[kWaves];
+  __shared__ uint8_t stage[kBlock * 8];
+  for (int q = 0; q < kMaxJobs; ++q) {
+    if (!((todo >> q) & 1u)) continue;
+    const ChainJob job = t.job[q];
+    const uint8_t* bitmask = t.bitmask[q];
+    const uint8_t* values = static_cast<const uint8_t*>(job.src);
+    const FR* scale = static_cast<const FR*>(job.scale);
+    const uint8_t* zp = reinterpret_cast<const uint8_t*>(job.zp);
+    FR* out = static_cast<FR*>(job.dst);
+    const int64_t rows = t.rows[q], pc = (int64_t)t.n_items[q] / rows, nvalues = (int64_t)t.n_items[q] * 4;
+    int64_t src = 0, counted = 0;  // set bits in rows [0, counted)
+    for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+      int64_t c = 0;
+      for (int64_t b = counted * pc + threadIdx.x; b < r * pc; b += kBlock) c += __popc((uint32_t)bitmask[b]);
+      src += block_sum(c, red);
+      scatter_row_to<uint8_t>(values, nvalues, bitmask + r * pc, src, pc, 0xffu, scan_s, stage,
+                              [&](int64_t b, const Vec<uint8_t, 8>& codes) {
+                                const int64_t i = r * pc + b;
+                                const uint32_t si = chain_scale_index<FLAT>((uint32_t)i, job);
+                                uint8_t zraw = 0;
+                                if constexpr (HAS_ZP) zraw = zp[si];
+                                stg<FR, 8>(out + i * 8,
+                                           dequant_codes8<FT, QK, HAS_ZP>(codes, scale[si], zraw));
+                              });
+      counted = r + 1;
+    }
+  }
+  s24_repair_done(t.slot);
 }
 
 // ------------------------------------------------------------------ 2:4 selection
@@ -1542,6 +1647,46 @@ quant_sparse24_compress_kernel(const typename FT::raw* __restrict__ x,
     qdq_vec8<FT, kKindFloat, kOut, QK, HAS_ZP>(a[k], unused_c, FT::to_f32(sraw[k]), z, qmin, qmax,
                                                &unused_f, &codes);
     store_survivors24<uint8_t, CTMI_I8, 8>(codes, values, bitmask, i, i < nitems);
+  }
+}
+
+// ... for the weights of a QS24Table
+template <typename FT, int QK, bool HAS_ZP, bool FLAT>
+__global__ void __launch_bounds__(kBlock) quant_sparse24_compress_chain_kernel(const QS24Table t) {
+  using FR = typename FT::raw;
+  constexpr int U = 4;
+  constexpr int kOut = QK == 0 ? kKindI8 : kKindF8;
+  uint32_t local, nitems;
+  const uint32_t ji = find_job_index(blockIdx.x, &local, &nitems);
+  const ChainJob job = t.job[ji];
+  uint8_t* __restrict__ bitmask = t.bitmask[ji];
+  const FR* __restrict__ x = static_cast<const FR*>(job.src);
+  const FR* __restrict__ scale = static_cast<const FR*>(job.scale);
+  const uint8_t* __restrict__ zp = reinterpret_cast<const uint8_t*>(job.zp);
+  uint8_t* __restrict__ values = static_cast<uint8_t*>(job.dst);
+  const uint32_t i0 = local * (kBlock * U) + threadIdx.x;
+  Vec<FR, 8> a[U];
+  FR sraw[U];
+  uint8_t zraw[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t i = i0 + k * kBlock;
+    const uint32_t at = i < nitems ? i : nitems - 1;  // past the end: re-read, not stored
+    const uint32_t si = chain_scale_index<FLAT>(at, job);
+    a[k] = ldg_nt<FR, 8>(x + (int64_t)at * 8);
+    sraw[k] = scale[si];
+    if constexpr (HAS_ZP) zraw[k] = zp[si];
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t i = i0 + k * kBlock;
+    Vec<FR, 8> unused_f;
+    Vec<uint8_t, 8> codes, unused_c;
+    float z = 0.0f;  // the zero point as the reference adds it (zero_point.to(x.dtype))
+    if constexpr (HAS_ZP) z = QK == 0 ? (float)(int8_t)zraw[k] : f8e4m3_to_f32(zraw[k]);
+    qdq_vec8<FT, kKindFloat, kOut, QK, HAS_ZP>(a[k], unused_c, FT::to_f32(sraw[k]), z, t.qmin, t.qmax,
+                                               &unused_f, &codes);
+    store_survivors24<uint8_t, CTMI_I8, 8>(codes, values, bitmask, (int64_t)i, i < nitems);
   }
 }
 
@@ -2232,4 +2377,174 @@ extern "C" int ctmi_sparse24_decompress_dequantize(const void* values, int64_t n
 #undef CTMI_S24DQ_K
 #undef CTMI_S24DQ
   return check_launch("ctmi_sparse24_decompress_dequantize");
+}
+
+// ---- the stacked entry points for a list of weights
+namespace ctmi {
+namespace {
+
+struct StackedKey {
+  int sd, qk;
+  bool has_zp, flat;
+  float qmin, qmax;
+  bool operator==(const StackedKey& o) const {
+    return sd == o.sd && qk == o.qk && has_zp == o.has_zp && flat == o.flat && qmin == o.qmin &&
+           qmax == o.qmax;
+  }
+};
+
+struct StackedPlan {
+  StackedKey key;
+  VecJob job;
+  uint8_t* bitmask;
+  int64_t rows;
+};
+
+template <bool COMPRESS, typename FT, int QK>
+void launch_stacked_chain2(const StackedKey& k, const QS24Table& t, unsigned grid, hipStream_t st) {
+#define CTMI_ST(ZP, FLAT)                                                                              \
+  if constexpr (COMPRESS) {                                                                            \
+    hipLaunchKernelGGL((quant_sparse24_compress_chain_kernel<FT, QK, ZP, FLAT>), grid, kBlock, 0, st, t); \
+  } else {                                                                                             \
+    hipLaunchKernelGGL((sparse24_scatter_dequant_chain_kernel<FT, QK, ZP, FLAT>), grid, kBlock, 0, st, t); \
+    hipLaunchKernelGGL((sparse24_repair_dequant_chain_kernel<FT, QK, ZP, FLAT>), kS24RepairGrid, kBlock, 0, \
+                       st, t);                                                                         \
+  }
+  if (k.has_zp) { if (k.flat) { CTMI_ST(true, true) } else { CTMI_ST(true, false) } }
+  else { if (k.flat) { CTMI_ST(false, true) } else { CTMI_ST(false, false) } }
+#undef CTMI_ST
+}
+
+template <bool COMPRESS>
+void launch_stacked_chain(const StackedKey& k, const QS24Table& t, unsigned grid, hipStream_t st) {
+#define CTMI_ST1(FT)                                                        \
+  if (k.qk == 0) launch_stacked_chain2<COMPRESS, FT, 0>(k, t, grid, st);    \
+  else launch_stacked_chain2<COMPRESS, FT, 1>(k, t, grid, st)
+  if (k.sd == CTMI_BF16) { CTMI_ST1(BF16); }
+  else if (k.sd == CTMI_F16) { CTMI_ST1(F16); }
+  else { CTMI_ST1(F32); }
+#undef CTMI_ST1
+}
+
+// weights that share a kernel instance (dtype, code kind, zero points, scale numbering,
+// quantization range) into common launches, 8 per launch
+template <bool COMPRESS>
+void run_stacked(std::vector<StackedPlan>& plans, hipStream_t st) {
+  constexpr int per_chunk = kBlock * (COMPRESS ? 4 : kS24DqU);
+  std::vector<char> done(plans.size(), 0);
+  for (size_t i = 0; i < plans.size(); ++i) {
+    if (done[i]) continue;
+    const StackedKey key = plans[i].key;
+    QS24Table t;
+    std::memset(&t, 0, sizeof(t));
+    int n = 0;
+    uint64_t chunks = 0;
+    auto reset = [&]() {
+      n = 0;
+      chunks = 0;
+      for (int k = 0; k < kMaxJobs; ++k) t.chunk_end[k] = 0xFFFFFFFFu;
+    };
+    reset();
+    t.qmin = key.qmin;
+    t.qmax = key.qmax;
+    auto flush = [&]() {
+      if (n == 0) return;
+      if (!COMPRESS) t.slot = s24_slot_of(st);
+      launch_stacked_chain<COMPRESS>(key, t, (unsigned)chunks, st);
+      reset();
+    };
+    for (size_t j = i; j < plans.size(); ++j) {
+      if (done[j] || !(plans[j].key == key)) continue;
+      const uint64_t c = (uint64_t)cdiv(plans[j].job.g.nvec, per_chunk);
+      if (n == kMaxJobs || chunks + c >= (1ull << 31)) flush();
+      t.job[n] = make_chain_job(plans[j].job);
+      t.n_items[n] = plans[j].job.g.nvec;
+      t.bitmask[n] = plans[j].bitmask;
+      t.rows[n] = plans[j].rows;
+      chunks += c;
+      t.chunk_end[n] = (uint32_t)chunks;
+      ++n;
+      done[j] = 1;
+    }
+    flush();
+  }
+}
+
+}  // namespace
+}  // namespace ctmi
+
+extern "C" int ctmi_quantize_sparse24_compress_many(const ctmi_stacked24_job* jobs, int64_t n,
+                                                    void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  std::vector<StackedPlan> plans;
+  plans.reserve((size_t)n);
+  for (int64_t i = 0; i < n; ++i) {  // every job is looked at before anything is enqueued
+    const ctmi_stacked24_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 0 && j.cols >= 0, CTMI_ERR_VALUE, "negative shape");
+    int rc = check_qparams(&j.qp, j.rows, j.cols);
+    if (rc) return rc;
+    if (j.rows == 0 || j.cols == 0) continue;
+    CTMI_REQUIRE(ctmi_quantize_sparse24_compress_supported(j.dense_dtype, j.rows, j.cols, &j.qp),
+                 CTMI_ERR_UNSUPPORTED,
+                 "job %lld: no fused kernel for this layout: quantize, then compress the codes",
+                 (long long)i);
+    CTMI_REQUIRE(j.dense && j.values && j.bitmask, CTMI_ERR_VALUE, "NULL tensor pointer");
+    CTMI_REQUIRE((uintptr_t)j.dense % (8 * dtype_size(j.dense_dtype)) == 0 && (uintptr_t)j.values % 4 == 0,
+                 CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+    CTMI_REQUIRE(j.rows * j.cols / 8 < (1ll << 31), CTMI_ERR_UNSUPPORTED, "job %lld: tensor too large",
+                 (long long)i);
+    StackedPlan p;
+    vec_geometry(&j.qp, j.rows, j.cols, &p.job.g);
+    float qmin, qmax;
+    rc = quant_range(j.qp.qtype, j.qp.num_bits, &qmin, &qmax);
+    if (rc) return rc;
+    p.key = StackedKey{j.dense_dtype, j.qp.qtype == CTMI_QTYPE_INT ? 0 : 1, j.qp.zero_point != nullptr,
+                       flat_geometry(p.job.g), qmin, qmax};
+    p.job.src = j.dense;
+    p.job.dst = j.values;
+    p.job.scale = j.qp.scale;
+    p.job.zp = (const int8_t*)j.qp.zero_point;
+    p.bitmask = j.bitmask;
+    p.rows = j.rows;
+    plans.push_back(p);
+  }
+  run_stacked<true>(plans, (hipStream_t)stream);
+  return check_launch("ctmi_quantize_sparse24_compress_many");
+}
+
+extern "C" int ctmi_sparse24_decompress_dequantize_many(const ctmi_stacked24_job* jobs, int64_t n,
+                                                        void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  std::vector<StackedPlan> plans;
+  plans.reserve((size_t)n);
+  for (int64_t i = 0; i < n; ++i) {
+    const ctmi_stacked24_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 0 && j.cols >= 0, CTMI_ERR_VALUE, "negative shape");
+    int rc = check_qparams(&j.qp, j.rows, j.cols);
+    if (rc) return rc;
+    if (j.rows == 0 || j.cols == 0) continue;
+    CTMI_REQUIRE(ctmi_sparse24_decompress_dequantize_supported(j.values_dtype, j.dense_dtype, j.rows,
+                                                               j.cols, &j.qp),
+                 CTMI_ERR_UNSUPPORTED,
+                 "job %lld: no fused kernel for this layout: decompress the codes, then dequantize",
+                 (long long)i);
+    CTMI_REQUIRE(j.dense && j.values && j.bitmask, CTMI_ERR_VALUE, "NULL tensor pointer");
+    CTMI_REQUIRE((uintptr_t)j.dense % (8 * dtype_size(j.dense_dtype)) == 0 && (uintptr_t)j.values % 4 == 0,
+                 CTMI_ERR_VALUE, "tensors must be aligned to 8 elements");
+    CTMI_REQUIRE(j.rows * j.cols / 8 < (1ll << 31), CTMI_ERR_UNSUPPORTED, "job %lld: tensor too large",
+                 (long long)i);
+    StackedPlan p;
+    vec_geometry(&j.qp, j.rows, j.cols, &p.job.g);
+    p.key = StackedKey{j.dense_dtype, j.values_dtype == CTMI_I8 ? 0 : 1, j.qp.zero_point != nullptr,
+                       flat_geometry(p.job.g), 0.0f, 0.0f};
+    p.job.src = j.values;
+    p.job.dst = const_cast<void*>(j.dense);
+    p.job.scale = j.qp.scale;
+    p.job.zp = (const int8_t*)j.qp.zero_point;
+    p.bitmask = j.bitmask;
+    p.rows = j.rows;
+    plans.push_back(p);
+  }
+  run_stacked<false>(plans, (hipStream_t)stream);
+  return check_launch("ctmi_sparse24_decompress_dequantize_many");
 }

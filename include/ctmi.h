@@ -328,6 +328,29 @@ int ctmi_sparse24_decompress_dequantize(const void* values, int64_t nvalues, int
                                         void* tmp, int64_t rows, int64_t cols,
                                         const ctmi_qparams* qp, void* stream);
 
+/* One weight for the many-weight forms of the two entry points above.  dense: the dense
+ * weight (read by compress, written by decompress), dense_dtype its dtype; values: the codes
+ * that survive, [rows, cols/2] of values_dtype (CTMI_I8 or CTMI_F8E4M3; compress derives it
+ * from qp and ignores the member); bitmask: uint8 [rows, cols/8]. */
+typedef struct ctmi_stacked24_job {
+  void* dense;
+  void* values;
+  uint8_t* bitmask;
+  int64_t rows, cols;
+  int32_t dense_dtype;
+  int32_t values_dtype;
+  ctmi_qparams qp;
+} ctmi_stacked24_job;
+
+/* ModelCompressor.compress / decompress over the weights of a model that are both quantized
+ * to int8 / fp8 codes and 2:4 compressed (model_compressor.py:638-667, :572-604): n weights
+ * from one call, same results as n calls of ctmi_quantize_sparse24_compress /
+ * ctmi_sparse24_decompress_dequantize.  Every job is validated before anything is enqueued
+ * (a layout without a fused kernel: CTMI_ERR_UNSUPPORTED, nothing enqueued); weights that
+ * share a kernel instance are chained into common launches, 8 per launch. */
+int ctmi_quantize_sparse24_compress_many(const ctmi_stacked24_job* jobs, int64_t n, void* stream);
+int ctmi_sparse24_decompress_dequantize_many(const ctmi_stacked24_job* jobs, int64_t n, void* stream);
+
 /* A1.  calculate_qparams (quantization/utils/helpers.py:67-146), elementwise
  * over n (min, max) pairs of dtype mm_dtype.  mm_is_0d != 0 when the reference
  * would see 0-d min/max tensors (their zero-point subtraction then promotes to

@@ -763,3 +763,55 @@ def test_sparse24_decompress_many_launches_back_to_back(gpu):
         torch.cuda.synchronize()
         for i, (got, want) in enumerate(outs):
             assert_bit_equal(got, want, f"launch {i} of {len(which)} on {len(set(which))} stream(s)")
+
+
+def test_stacked_kernels_for_many_weights_in_one_call(gpu):
+    """ctmi_quantize_sparse24_compress_many / ctmi_sparse24_decompress_dequantize_many (8 weights
+    per launch) against the single-weight entry points: 19 weights of mixed shapes, dtypes,
+    strategies (channel, group, tensor), code kinds (fp8, int8) and zero points; one of them with
+    a bitmask that is not 2:4 on the way back (the repair pass names it alone)"""
+    from compressed_tensors_amd.compressors.sparse_24_bitmask import (
+        quantize_sparse24_compress, quantize_sparse24_compress_many,
+        sparse24_decompress_dequantize, sparse24_decompress_dequantize_many,
+    )
+    from compressed_tensors_amd.quantization import QuantizationArgs, observe_weight_qparams
+
+    announce("stacked kernels, many weights")
+    g = torch.Generator().manual_seed(31)
+    specs = [
+        dict(num_bits=8, type="float", symmetric=True, strategy="channel"),
+        dict(num_bits=8, type="int", symmetric=True, strategy="group", group_size=64),
+        dict(num_bits=8, type="int", symmetric=False, strategy="channel"),
+        dict(num_bits=8, type="float", symmetric=True, strategy="tensor"),
+    ]
+    shapes = [(64, 256), (96, 512), (8, 64), (200, 1024), (33, 128)]
+    recs, single = [], []
+    for k in range(19):
+        args = QuantizationArgs(**specs[k % len(specs)])
+        dtype = (torch.bfloat16, torch.float16, torch.float32)[k % 3]
+        w = (torch.randn(shapes[k % len(shapes)], generator=g) * 0.05).to(dtype).to(gpu)
+        scale, zp = observe_weight_qparams(w, args)
+        recs.append((w, scale, zp, args))
+        single.append(quantize_sparse24_compress(w, scale, args, zero_point=zp))
+    many = quantize_sparse24_compress_many(recs)
+    assert all(m is not None for m in many)
+    for k, ((values, bitmask), (want_values, want_bitmask)) in enumerate(zip(many, single)):
+        assert values.dtype == want_values.dtype
+        assert_bit_equal(values, want_values.cpu(), f"weight {k} values")
+        assert_bit_equal(bitmask, want_bitmask.cpu(), f"weight {k} bitmask")
+    # the way back; weight 11 gets a bitmask with a group of three and one of one
+    back = []
+    for k, ((w, scale, zp, args), (values, bitmask)) in enumerate(zip(recs, many)):
+        zp_back = None if args.symmetric else zp
+        if k == 11:
+            bitmask = bitmask.clone()
+            bitmask[0, 0] = 0b00010111
+        back.append((values, bitmask, tuple(w.shape), scale, zp_back))
+    want = [sparse24_decompress_dequantize(v, b, shape, s, zero_point=z) for v, b, shape, s, z in back]
+    got = sparse24_decompress_dequantize_many(back)
+    for k, (a, b) in enumerate(zip(got, want)):
+        assert a is not None and a.dtype == b.dtype and a.shape == b.shape
+        assert_bit_equal(a, b.cpu(), f"weight {k} restored")
+    # what the many-weight helpers do not take comes back as None (the caller goes one by one)
+    assert quantize_sparse24_compress_many([(recs[0][0].cpu(), recs[0][1], None, recs[0][3])]) == [None]
+    assert sparse24_decompress_dequantize_many([(many[0][0].cpu(), many[0][1], (64, 256), recs[0][1], None)]) == [None]
