@@ -541,3 +541,90 @@ def test_sparsity_only_model_in_memory(fmt, gpu):
         assert_bit_equal(m.weight.data, w.cpu(), f"{name} restored")
         x = torch.randn(2, m.in_features, device=gpu).bfloat16()
         assert_bit_equal(m(x), torch.nn.functional.linear(x, w).cpu(), f"{name} forward")
+
+
+@pytest.mark.parametrize("fmt", ["pack-quantized", "int-quantized", "float-quantized", "nvfp4-pack-quantized"])
+def test_module_pathway_on_a_seeded_mixture(fmt, gpu):
+    """40 Linear modules of mixed shapes (some whose outputs cannot share an allocation), dtypes
+    and schemes in one model: compress_model leaves in every module what compress_weight gives
+    for it alone, decompress_model what decompress_weight gives"""
+    import random
+
+    from compressed_tensors_amd.compressors import ModelCompressor, apply_quantization_scheme
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme, observe_weight_qparams,
+    )
+    from compressed_tensors_amd.quantization.helpers import generate_gparam
+
+    announce("seeded mixture", fmt)
+    rng = random.Random(fmt)
+    torch.manual_seed(len(fmt))
+    if fmt == "pack-quantized":
+        specs = [dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128),
+                 dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=32),
+                 dict(num_bits=8, type="int", symmetric=True, strategy="channel"),
+                 dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=64)]
+    elif fmt == "int-quantized":
+        specs = [dict(num_bits=8, type="int", symmetric=True, strategy="channel"),
+                 dict(num_bits=8, type="int", symmetric=False, strategy="group", group_size=32),
+                 dict(num_bits=8, type="int", symmetric=True, strategy="tensor")]
+    elif fmt == "float-quantized":
+        specs = [dict(num_bits=8, type="float", symmetric=True, strategy="channel"),
+                 dict(num_bits=8, type="float", symmetric=True, strategy="group", group_size=128),
+                 dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[16, 64])]
+    else:
+        specs = [dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)]
+    ins, outs = [128, 256, 384, 1024], [16, 24, 40, 64, 72, 200]
+    model = torch.nn.Module()
+    model.m = torch.nn.ModuleList()
+    groups = {}
+    for i in range(40):
+        spec = specs[rng.randrange(len(specs))]
+        dtype = rng.choice([torch.bfloat16, torch.bfloat16, torch.float16, torch.float32])
+        if fmt == "nvfp4-pack-quantized":
+            dtype = rng.choice([torch.bfloat16, torch.float16])
+        lin = torch.nn.Linear(rng.choice(ins), rng.choice(outs), bias=rng.random() < 0.3).to(dtype).to(gpu)
+        if spec.get("strategy") == "block":
+            lin = torch.nn.Linear(rng.choice([128, 256]), rng.choice([16, 64]), bias=False).to(dtype).to(gpu)
+        model.m.append(lin)
+        groups.setdefault(tuple(sorted((k, str(v)) for k, v in spec.items())), (spec, []))[1].append(f"m.{i}")
+    config = QuantizationConfig(config_groups={
+        f"g{k}": QuantizationScheme(targets=names, weights=QuantizationArgs(**spec))
+        for k, (spec, names) in enumerate(groups.values())}, format=fmt)
+    apply_quantization_scheme(model, config)
+    mc = ModelCompressor(quantization_config=config)
+    comp = mc.quantization_compressor[fmt]
+    want = {}
+    for name, m in model.named_modules():
+        scheme = getattr(m, "quantization_scheme", None)
+        if scheme is None:
+            continue
+        args, w = scheme.weights, m.weight.data
+        gs = None
+        if args.strategy == "tensor_group":
+            lo, hi = torch.aminmax(w)
+            gs = generate_gparam(lo.reshape(1), hi.reshape(1))
+            m.register_parameter("weight_global_scale", torch.nn.Parameter(gs, requires_grad=False))
+            scale, zp = observe_weight_qparams(w, args, global_scale=gs)
+        else:
+            scale, zp = observe_weight_qparams(w, args)
+        m.register_parameter("weight_scale", torch.nn.Parameter(scale, requires_grad=False))
+        m.register_parameter("weight_zero_point", torch.nn.Parameter(zp, requires_grad=False))
+        kw = dict(weight=w.clone(), scale=scale, zero_point=zp, quantization_args=args)
+        if gs is not None:
+            kw["global_scale"] = gs
+        want[name] = comp.compress_weight(**kw)
+    assert len(want) == 40
+    mc.compress_model(model)
+    for name, single in want.items():
+        m = model.get_submodule(name)
+        for key, value in single.items():
+            assert_bit_equal(getattr(m, key).data, value.cpu(), f"{name}.{key}")
+    held = {name: {k: p.data for k, p in model.get_submodule(name)._parameters.items() if p is not None}
+            for name in want}
+    mc.decompress_model(model)
+    for name, data in held.items():
+        m = model.get_submodule(name)
+        single = comp.decompress_weight(compressed_data=data, quantization_args=m.quantization_scheme.weights)
+        assert_bit_equal(m.weight.data, single.cpu(), f"{name} decompressed")
+        assert m.weight.dtype == single.dtype
