@@ -2508,6 +2508,7 @@ extern "C" int ctmi_quantize_sparse24_compress_many(const ctmi_stacked24_job* jo
     p.rows = j.rows;
     plans.push_back(p);
   }
+  if (plans.empty()) return CTMI_OK;  // nothing to enqueue
   run_stacked<true>(plans, (hipStream_t)stream);
   return check_launch("ctmi_quantize_sparse24_compress_many");
 }
@@ -2545,6 +2546,7 @@ extern "C" int ctmi_sparse24_decompress_dequantize_many(const ctmi_stacked24_job
     p.rows = j.rows;
     plans.push_back(p);
   }
+  if (plans.empty()) return CTMI_OK;
   run_stacked<false>(plans, (hipStream_t)stream);
   return check_launch("ctmi_sparse24_decompress_dequantize_many");
 }

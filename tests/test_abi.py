@@ -322,3 +322,43 @@ def test_sylvester_entry_point_errors(ctmi):
     # the same kernel behind ctmi_kron_matmul (h = 1, Sylvester inner factor)
     rc = ctmi.ctmi_kron_matmul(0x1008, 0x2000, _lib.BF16, 4096, 1, 4096, 0x3000, None, None, 1, 1.0, None)
     assert rc == _lib.CTMI_ERR_VALUE and "aligned" in _err(ctmi)
+
+
+def test_stacked_and_activation_ordered_entry_points_check_their_arguments(ctmi):
+    """the many-weight forms of the fp8 / int8 + 2:4 kernels and the one-pass kernel for
+    activation-ordered weights: every job is looked at on the host before anything is enqueued"""
+    jobs = (_lib.Stacked24Job * 2)()
+    for j, cols in zip(jobs, (64, 68)):
+        j.dense, j.values, j.bitmask, j.rows, j.cols = 0x1000, 0x2000, 0x3000, 4, cols
+        j.dense_dtype, j.values_dtype = _lib.BF16, _lib.F8E4M3
+        j.qp = _qp(scale=0x4000, scale_dtype=_lib.BF16, qtype=_lib.QTYPE_FLOAT, num_bits=8,
+                   s_rows=4, s_cols=1, blk_rows=1, blk_cols=cols)
+    # rows of 68 elements are not whole bitmask bytes: the second job stops the whole call
+    assert ctmi.ctmi_quantize_sparse24_compress_many(jobs, 2, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert "job 1" in _err(ctmi)
+    assert ctmi.ctmi_sparse24_decompress_dequantize_many(jobs, 2, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert ctmi.ctmi_quantize_sparse24_compress_many(None, 0, None) == _lib.CTMI_OK
+    assert ctmi.ctmi_sparse24_decompress_dequantize_many(None, 0, None) == _lib.CTMI_OK
+    assert ctmi.ctmi_quantize_sparse24_compress_many(None, 2, None) == _lib.CTMI_ERR_VALUE
+    jobs[1].cols = 64
+    jobs[1].qp.blk_cols = 64
+    jobs[1].values = 0
+    assert ctmi.ctmi_quantize_sparse24_compress_many(jobs, 2, None) == _lib.CTMI_ERR_VALUE
+    # what the single-weight query says holds for the list
+    assert ctmi.ctmi_quantize_sparse24_compress_supported(_lib.BF16, 4, 64, ctypes.byref(jobs[0].qp)) == 1
+    assert ctmi.ctmi_quantize_sparse24_compress_supported(_lib.BF16, 4, 68, ctypes.byref(jobs[0].qp)) == 0
+    # activation-ordered one pass: rows that fit a workgroup's registers, at most 256 groups a row
+    assert ctmi.ctmi_observe_pack_quantized_gidx_supported(_lib.BF16, 64, 4096, 128, 4) == 1
+    assert ctmi.ctmi_observe_pack_quantized_gidx_supported(_lib.BF16, 64, 4100, 4, 4) == 0   # cols % 8
+    assert ctmi.ctmi_observe_pack_quantized_gidx_supported(_lib.BF16, 64, 16392, 8, 4) == 0  # too wide
+    assert ctmi.ctmi_observe_pack_quantized_gidx_supported(_lib.BF16, 64, 4096, 8, 4) == 0   # 512 groups
+    assert ctmi.ctmi_observe_pack_quantized_gidx_supported(_lib.BF16, 64, 4096, 128, 3) == 0
+    rc = ctmi.ctmi_observe_pack_quantized_gidx(0x1000, _lib.BF16, 64, 4096, 8, 4, 1, None, 0x2000, 0x3000,
+                                               None, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED and "separately" in _err(ctmi)
+    rc = ctmi.ctmi_observe_pack_quantized_gidx(None, _lib.BF16, 64, 4096, 128, 4, 1, None, 0x2000, 0x3000,
+                                               None, None)
+    assert rc == _lib.CTMI_ERR_VALUE
+    rc = ctmi.ctmi_observe_pack_quantized_gidx(0x1000, _lib.I8, 64, 4096, 128, 4, 1, None, 0x2000, 0x3000,
+                                               None, None)
+    assert rc == _lib.CTMI_ERR_UNSUPPORTED
