@@ -344,3 +344,45 @@ def test_fused_rotation_quantization_packing_at_full_size(n, gpu):
         want = op.pack_quantized_compress(yc, o_scale, oargs, zero_point=o_zp)["weight_packed"]
         assert_bit_equal(fused["weight_scale"][sl], o_scale, f"scales {sl}")
         assert_bit_equal(fused["weight_packed"][sl], want, f"packed {sl}")
+
+
+def test_whole_tensors_against_the_oracle(gpu):
+    """one whole 4096 x 4096 weight per format against the oracle, every byte (the row slices
+    above leave most rows to GPU-vs-GPU comparisons): fp8 per channel with outliers (codes and
+    dequantized weight) and nvfp4 g16 (scales, packed codes, dequantized weight)"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.quantization import QuantizationArgs, observe_weight_qparams
+
+    g = torch.Generator(device=gpu).manual_seed(21)
+    w = torch.randn(4096, 4096, generator=g, device=gpu) * 0.02
+    w = torch.where(torch.rand(4096, 4096, generator=g, device=gpu) < 1e-3, w * 20, w).bfloat16()
+    wc = w.cpu()
+
+    announce("whole tensor fp8", tuple(w.shape))
+    spec = dict(num_bits=8, type="float", symmetric=True, strategy="channel")
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    scale, zp = observe_weight_qparams(w, args)
+    o_scale, o_zp = oq.observe_weight(wc, oargs)
+    assert_bit_equal(scale, o_scale, "fp8 scales")
+    comp = BaseCompressor.load_from_registry("float-quantized")
+    codes = comp.compress_weight(weight=w, scale=scale, zero_point=zp, quantization_args=args)["weight"]
+    want = op.naive_compress(wc, o_scale, oargs, zero_point=o_zp)
+    assert_bit_equal(codes, want, "fp8 codes")
+    dense = comp.decompress_weight({"weight": codes, "weight_scale": scale}, quantization_args=args)
+    assert_bit_equal(dense, op.naive_decompress(dict(weight=want, weight_scale=o_scale)), "fp8 dense")
+
+    announce("whole tensor nvfp4", tuple(w.shape))
+    spec = dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16)
+    args, oargs = QuantizationArgs(**spec), oq._Args(**spec)
+    gs, scale, zp = _nvfp4_scales(w, args, gpu)
+    mn, mx = torch.aminmax(wc)
+    o_gs = oq.generate_gparam(mn.reshape(1), mx.reshape(1))
+    o_scale, o_zp = oq.observe_weight(wc, oargs, global_scale=o_gs)
+    assert_bit_equal(gs, o_gs, "nvfp4 global scale")
+    assert_bit_equal(scale, o_scale, "nvfp4 scales")
+    comp = BaseCompressor.load_from_registry("nvfp4-pack-quantized")
+    packed = comp.compress_weight(weight=w, scale=scale, global_scale=gs, quantization_args=args)["weight_packed"]
+    want = op.nvfp4_compress(wc, o_scale, o_gs, oargs, zero_point=o_zp)
+    assert_bit_equal(packed, want, "nvfp4 packed")
+    dense = comp.decompress_weight({"weight_packed": packed, "weight_scale": scale, "weight_global_scale": gs})
+    assert_bit_equal(dense, op.nvfp4_decompress(want, o_scale, o_gs), "nvfp4 dense")
