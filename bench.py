@@ -253,6 +253,17 @@ def other_workload(torch, name, seed):
              zp.data_ptr(), code(zp.dtype), None, None, st)
         return lambda: _lib.check(lib.ctmi_observe_qparams(*a))
 
+    def observe_many(items, args):
+        """items: (x, blk_cols, scale, zp): one ctmi_observe_qparams_many call for the list"""
+        jobs = (_lib.ObserveJob * len(items))()
+        for j, (x, blk_cols, scale, zp) in zip(jobs, items):
+            j.x, j.scale, j.zero_point, j.global_scale = x.data_ptr(), scale.data_ptr(), zp.data_ptr(), None
+            j.rows, j.cols, j.blk_cols, j.x_dtype = x.numel() // x.shape[-1], x.shape[-1], blk_cols, code(x.dtype)
+        keep.extend([jobs, items])
+        qtype = _lib.QTYPE_FLOAT if args.type == "float" else _lib.QTYPE_INT
+        a = (jobs, len(items), qtype, args.num_bits, int(args.symmetric), -1, code(items[0][3].dtype), st)
+        return lambda: _lib.check(lib.ctmi_observe_qparams_many(*a))
+
     def dynamic(x, out, blk_cols, args, gscale=None):
         keep.extend([x, out, gscale])
         rows = x.numel() // x.shape[-1]
@@ -280,6 +291,8 @@ def other_workload(torch, name, seed):
         # one-shot: scales + fp8 codes from one pass over weights that have no scales yet,
         # against the observer and the quantizer one after the other (one call per weight each)
         w_obs, w_q, w_one = [], [], []
+        w_obs_many = [observe_many([(e["weight"], e["weight"].shape[1], e["scale"], e["observed_zp"])
+                                    for e in entries], args)]
         for e, codes in zip(entries, batch.codes):
             w, sc = e["weight"], e["scale"]
             r, c = w.shape
@@ -323,6 +336,8 @@ def other_workload(torch, name, seed):
         ops = [Op("weights: quantize to fp8, per channel (224 tensors)", q_calls, 3 * n, "qdq_vec_many_kernel", launches=chained(len(entries))),
                Op("weights: dequantize from fp8 (224 tensors)", d_calls, 3 * n, "qdq_vec_many_kernel", launches=chained(len(entries))),
                Op("weights one-shot: per-channel observer (224 calls)", w_obs, 2 * n, "observe_wide_kernel", primary=False),
+               Op("weights one-shot: per-channel observer, one call (8 per launch)", w_obs_many, 2 * n,
+                  "observe_wide_chain_kernel", launches=chained(len(entries))),
                Op("weights one-shot: quantize with those scales (224 calls)", w_q, 3 * n, "qdq_vec_kernel", primary=False),
                Op("weights one-shot: scales + fp8 codes in one pass (224 calls)", w_one, 3 * n, "dynamic_rows_kernel", primary=False),
                Op("weights one-shot: scales + fp8 codes in one pass, one call (8 per launch)", w_many, 3 * n, "dynamic_rows_many_kernel", launches=chained(len(entries))),
@@ -582,7 +597,7 @@ def other_workload(torch, name, seed):
     if name == "one-shot":
         # the Llama-3-8B-shaped set, no scales yet: observer + qparams + quantize + pack
         args = QuantizationArgs(num_bits=4, type="int", symmetric=True, strategy="group", group_size=GROUP)
-        sep_obs, sep_cmp, fused, job_fields, n, keep2 = [], [], [], [], 0, []
+        sep_obs, sep_cmp, fused, job_fields, n, keep2, obs_zps = [], [], [], [], 0, [], []
         for _, r, c in shapes_for("llama3-8b-w4a16"):
             w = randn(r, c, 0.02)
             scale, zp = observe_weight_qparams(w, args)
@@ -590,6 +605,7 @@ def other_workload(torch, name, seed):
             plan = build_qparams(w, scale, None, args, None, None)
             keep.extend([w, scale, zp, packed, plan])
             keep2.append((w, scale, packed))
+            obs_zps.append(zp)
             sep_obs.append(observe(w, GROUP, args, scale, zp))
             ca = (w.data_ptr(), code(w.dtype), packed.data_ptr(), r, c, ctypes.byref(plan.qp), st)
             sep_cmp.append(lambda ca=ca: _lib.check(lib.ctmi_pack_quantized_compress(*ca)))
@@ -604,6 +620,7 @@ def other_workload(torch, name, seed):
              j.num_bits, j.symmetric) = f
         keep.append(jobs)
         many = [lambda: _lib.check(lib.ctmi_observe_pack_quantized_many(jobs, len(job_fields), st))]
+        sep_obs_many = [observe_many([(w, GROUP, scale, zp) for (w, scale, _), zp in zip(keep2, obs_zps)], args)]
         # the same set with activation ordering (one random g_idx per row length): the group of
         # a column is looked up, min / max meet in LDS
         from compressed_tensors_amd.quantization.forward import _column_groups
@@ -625,6 +642,8 @@ def other_workload(torch, name, seed):
         keep.append(col_groups)
         g = n // GROUP
         ops = [Op("observer + qparams, group 128 (224 tensors, one call each)", sep_obs, 2 * n + 3 * g, "observe_flat_kernel", primary=False),
+               Op("observer + qparams, group 128, all 224 tensors in one call (8 per launch)", sep_obs_many, 2 * n + 3 * g,
+                  "observe_flat_chain_kernel", launches=chained(len(job_fields))),
                Op("quantize + pack with those scales (one call each)", sep_cmp, 2 * n + 2 * g + n // 2, "pq_compress_vec_kernel", primary=False),
                Op("observer + qparams + quantize + pack in one pass (one call each)", fused, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel", primary=False),
                Op("the same, all 224 tensors in one call (8 per launch)", many, 2 * n + 2 * g + n // 2, "observe_pack_groups_kernel", launches=chained(len(job_fields))),

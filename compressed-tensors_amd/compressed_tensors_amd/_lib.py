@@ -129,6 +129,22 @@ class ObservePackJob(ctypes.Structure):
     ]
 
 
+class ObserveJob(ctypes.Structure):
+    """ctmi_observe_job"""
+
+    _fields_ = [
+        ("x", c_void_p),
+        ("scale", c_void_p),
+        ("zero_point", c_void_p),
+        ("global_scale", c_void_p),
+        ("rows", c_int64),
+        ("cols", c_int64),
+        ("blk_cols", c_int64),
+        ("x_dtype", c_int32),
+        ("reserved", c_int32),
+    ]
+
+
 class Stacked24Job(ctypes.Structure):
     """ctmi_stacked24_job"""
 
@@ -216,6 +232,8 @@ SIGNATURES = {
         [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int32, c_void_p, c_int64, c_int64,
          POINTER(QParams), c_void_p],
     ),
+    "ctmi_observe_qparams_many": (
+        c_int32, [POINTER(ObserveJob), c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p]),
     "ctmi_quantize_sparse24_compress_many": (c_int32, [POINTER(Stacked24Job), c_int64, c_void_p]),
     "ctmi_sparse24_decompress_dequantize_many": (c_int32, [POINTER(Stacked24Job), c_int64, c_void_p]),
     "ctmi_bitmask_tmp_bytes": (c_int64, [c_int64, c_int64]),

@@ -7,8 +7,12 @@
 //
 // calculate_qparams is evaluated in the dtype of the min/max tensors (each op
 // rounded to it), except where the reference's operands promote to fp32.
+#include <cstring>
+#include <vector>
+
 #include "ctmi_device.h"
 #include "ctmi_host.h"
+#include "job_table.h"
 #include "qparams.h"
 #include "minmax.h"
 
@@ -272,6 +276,91 @@ static bool observe_streaming(const void* x, const float* gscale, const ObserveO
   return false;
 }
 
+// ---- the streaming forms for several tensors per launch (scales and zero points only)
+struct ObsChainJob {
+  const void* x;
+  void* scale;
+  void* zp;
+  const float* gscale;
+};
+struct ObsChainTable {  // the kernel's only argument: find_job_index reads its head
+  uint32_t chunk_end[kMaxJobs];  // running total of workgroups, job 0 .. j (unused: 0xFFFFFFFF)
+  uint32_t n_items[kMaxJobs];    // flat: vectors of the tensor; wide: its segments
+  ObsChainJob job[kMaxJobs];
+  uint32_t per[kMaxJobs];        // wide: vectors per segment
+  int L;                         // flat: vectors per segment (one value per launch)
+  QpCfg c;
+};
+static_assert(offsetof(ObsChainTable, chunk_end) == 0 && offsetof(ObsChainTable, n_items) == 32,
+              "find_job_index");
+
+template <typename XT>
+__global__ void __launch_bounds__(256) observe_flat_chain_kernel(const ObsChainTable t) {
+  constexpr int U = kObsUnroll;
+  uint32_t local, nvec;
+  const ObsChainJob job = t.job[find_job_index(blockIdx.x, &local, &nvec)];
+  const typename XT::raw* __restrict__ x = static_cast<const typename XT::raw*>(job.x);
+  const int L = t.L;
+  const float gs = job.gscale ? job.gscale[0] : 1.0f;
+  const uint32_t v0 = local * (256 * U) + threadIdx.x;
+  Vec<typename XT::raw, 8> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const uint32_t v = v0 + k * 256;  // past the end: re-read the last vector (nothing is emitted for it)
+    a[k] = ldg<typename XT::raw, 8>(x + (int64_t)(v < nvec ? v : nvec - 1) * 8);
+  }
+  __shared__ float seg_lo[256 * U], seg_hi[256 * U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    float lo = __builtin_inff(), hi = -__builtin_inff();
+    bool unordered = false;
+    vec_minmax<XT>(a[k], &lo, &hi, &unordered);
+    group_minmax(L, &lo, &hi);
+    if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
+    if ((threadIdx.x & (L - 1)) == 0) {
+      const int slot = (k * 256 + threadIdx.x) / L;
+      seg_lo[slot] = lo;
+      seg_hi[slot] = hi;
+    }
+  }
+  __syncthreads();
+  const ObserveOut o{job.scale, job.zp, nullptr, nullptr};
+  const int per_wg = 256 * U / L;
+  const int64_t first = (int64_t)local * per_wg, n_seg = nvec / L;
+  for (int i = threadIdx.x; i < per_wg && first + i < n_seg; i += 256)
+    emit_segment<XT>(o, first + i, seg_lo[i], seg_hi[i], gs, t.c);
+}
+
+template <typename XT>
+__global__ void __launch_bounds__(256) observe_wide_chain_kernel(const ObsChainTable t) {
+  constexpr int U = 8;
+  uint32_t local, n_segments;
+  const uint32_t ji = find_job_index(blockIdx.x, &local, &n_segments);
+  const ObsChainJob job = t.job[ji];
+  const int64_t items = t.per[ji];
+  const float gs = job.gscale ? job.gscale[0] : 1.0f;
+  const int lane = threadIdx.x & 63;
+  const int64_t s = (int64_t)local * 4 + (threadIdx.x >> 6);
+  if (s >= n_segments) return;
+  const typename XT::raw* p = static_cast<const typename XT::raw*>(job.x) + s * items * 8;
+  float lo = __builtin_inff(), hi = -__builtin_inff();
+  bool unordered = false;
+  for (int64_t i0 = 0; i0 < items; i0 += 64 * U) {
+    Vec<typename XT::raw, 8> a[U];
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int64_t i = i0 + k * 64 + lane;
+      a[k] = ldg_nt<typename XT::raw, 8>(p + (i < items ? i : items - 1) * 8);
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) vec_minmax<XT>(a[k], &lo, &hi, &unordered);
+  }
+  group_minmax(64, &lo, &hi);
+  if (group_any(64, unordered)) lo = hi = __builtin_nanf("");
+  const ObserveOut o{job.scale, job.zp, nullptr, nullptr};
+  if (lane == 0) emit_segment<XT>(o, s, lo, hi, gs, t.c);
+}
+
 // stage 2: fold `blk_rows` consecutive rows of a [rows, n_seg] min/max table;
 // one workgroup per output cell
 template <typename XT>
@@ -471,4 +560,101 @@ extern "C" int ctmi_observe_qparams(const void* x, int32_t x_dtype, int64_t rows
                          (XT::raw*)max_out, g, c);
   });
   return check_launch("ctmi_observe_qparams");
+}
+
+// A2 + A1 for a list of tensors: tensors whose cells stream (see observe_streaming) and share
+// a dtype and a kind of kernel go into common launches, 8 per launch; any other tensor gets
+// the launch ctmi_observe_qparams would give it.
+extern "C" int ctmi_observe_qparams_many(const ctmi_observe_job* jobs, int64_t n, int32_t qtype,
+                                         int32_t num_bits, int32_t symmetric, int32_t scale_dtype,
+                                         int32_t zp_dtype, void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  struct Plan {
+    QpCfg c;
+    SegGeom g;
+    int kind;  // 0: a launch of its own, 1: flat, 2: wide
+    int64_t items;
+  };
+  std::vector<Plan> plans((size_t)n);
+  for (int64_t i = 0; i < n; ++i) {  // every job is looked at before anything is enqueued
+    const ctmi_observe_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 1 && j.cols >= 1, CTMI_ERR_VALUE, "job %lld: cannot observe an empty tensor",
+                 (long long)i);
+    CTMI_REQUIRE(j.blk_cols >= 1, CTMI_ERR_VALUE, "job %lld: empty cell", (long long)i);
+    Plan& p = plans[i];
+    const bool fp4_global = qtype == CTMI_QTYPE_FLOAT && num_bits == 4 && symmetric && j.global_scale;
+    int rc = fill_qpcfg(&p.c, qtype, num_bits, symmetric, j.x_dtype, 0, j.global_scale != nullptr,
+                        scale_dtype < 0 ? (fp4_global ? CTMI_F8E4M3 : j.x_dtype) : scale_dtype,
+                        zp_dtype);
+    if (rc) return rc;
+    CTMI_REQUIRE(j.x && j.scale, CTMI_ERR_VALUE, "job %lld: NULL tensor pointer", (long long)i);
+    seg_geometry(&p.g, j.x, dtype_size(j.x_dtype), j.rows, j.cols, j.blk_cols);
+    p.items = p.g.seg_cols / 8;
+    p.kind = 0;
+    const bool nvfp4_case = p.c.fp4_global && j.blk_cols == 16 && dtype_size(j.x_dtype) == 2;
+    if (p.g.vec && p.g.cols % p.g.seg_cols == 0 && !nvfp4_case &&
+        j.rows * j.cols / 8 < (1ll << 31)) {
+      if (p.items <= 64 && (p.items & (p.items - 1)) == 0) p.kind = 1;
+      else if (p.items > 64) p.kind = 2;
+    }
+  }
+  hipStream_t st = (hipStream_t)stream;
+  std::vector<char> done((size_t)n, 0);
+  for (int64_t i = 0; i < n; ++i) {
+    if (plans[i].kind != 0) continue;
+    const ctmi_observe_job& j = jobs[i];
+    int rc = ctmi_observe_qparams(j.x, j.x_dtype, j.rows, j.cols, j.blk_cols, qtype, num_bits, symmetric,
+                                  j.global_scale, j.scale, plans[i].c.scale_dtype, j.zero_point,
+                                  zp_dtype, nullptr, nullptr, stream);
+    if (rc) return rc;
+    done[i] = 1;
+  }
+  for (int64_t i = 0; i < n; ++i) {
+    if (done[i]) continue;
+    const Plan& lead = plans[i];
+    const int xd = jobs[i].x_dtype;
+    ObsChainTable t;
+    std::memset(&t, 0, sizeof(t));
+    t.c = lead.c;
+    t.L = (int)lead.items;
+    int cnt = 0;
+    uint64_t chunks = 0;
+    auto reset = [&]() {
+      cnt = 0;
+      chunks = 0;
+      for (int k = 0; k < kMaxJobs; ++k) t.chunk_end[k] = 0xFFFFFFFFu;
+    };
+    reset();
+    auto flush = [&]() {
+      if (cnt == 0) return;
+      CTMI_DISPATCH_XT(xd, {
+        if (lead.kind == 1)
+          hipLaunchKernelGGL(observe_flat_chain_kernel<XT>, (unsigned)chunks, 256, 0, st, t);
+        else
+          hipLaunchKernelGGL(observe_wide_chain_kernel<XT>, (unsigned)chunks, 256, 0, st, t);
+      });
+      reset();
+    };
+    for (int64_t k = i; k < n; ++k) {
+      const Plan& p = plans[k];
+      // (the scale dtype follows from the tensor's dtype and the global scale: part of what
+      // tensors of one launch share)
+      if (done[k] || p.kind != lead.kind || jobs[k].x_dtype != xd || p.c.scale_dtype != lead.c.scale_dtype ||
+          p.c.fp4_global != lead.c.fp4_global || (lead.kind == 1 && p.items != lead.items))
+        continue;
+      const int64_t nvec = jobs[k].rows * jobs[k].cols / 8;
+      const int64_t n_segments = jobs[k].rows * p.g.n_seg;
+      const uint64_t c = (uint64_t)(lead.kind == 1 ? cdiv(nvec, 256 * kObsUnroll) : cdiv(n_segments, 4));
+      if (cnt == kMaxJobs || chunks + c >= (1ull << 31)) flush();
+      t.job[cnt] = ObsChainJob{jobs[k].x, jobs[k].scale, jobs[k].zero_point, jobs[k].global_scale};
+      t.n_items[cnt] = (uint32_t)(lead.kind == 1 ? nvec : n_segments);
+      t.per[cnt] = (uint32_t)p.items;
+      chunks += c;
+      t.chunk_end[cnt] = (uint32_t)chunks;
+      ++cnt;
+      done[k] = 1;
+    }
+    flush();
+  }
+  return n ? check_launch("ctmi_observe_qparams_many") : CTMI_OK;
 }

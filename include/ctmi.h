@@ -457,6 +457,29 @@ typedef struct ctmi_observe_nvfp4_job {
 } ctmi_observe_nvfp4_job;
 int ctmi_observe_nvfp4_compress_many(const ctmi_observe_nvfp4_job* jobs, int64_t n, void* stream);
 
+/* One tensor for ctmi_observe_qparams_many: x [rows, cols] of x_dtype, cells of 1 x blk_cols
+ * elements; scale / zero_point [rows, ceil(cols / blk_cols)] (zero_point optional);
+ * global_scale: the fp32 scalar of a tensor_group (nvfp4) scheme, else NULL. */
+typedef struct ctmi_observe_job {
+  const void* x;
+  void* scale;
+  void* zero_point;
+  const float* global_scale;
+  int64_t rows, cols, blk_cols;
+  int32_t x_dtype;
+  int32_t reserved;
+} ctmi_observe_job;
+
+/* A2 + A1 for the weights of a model in one call: what a calibration pass with the min-max
+ * observer does module by module (tests/mock_observer.py:38-113 followed by calculate_qparams,
+ * quantization/utils/helpers.py:67-146).  Same results as n calls of ctmi_observe_qparams
+ * without min_out / max_out; tensors that share a dtype and a kernel are chained into common
+ * launches, 8 per launch.  scale_dtype < 0: the dtype the reference produces for each tensor
+ * (its own, or float8_e4m3fn for fp4 with a global scale).  Every job is validated before
+ * anything is enqueued. */
+int ctmi_observe_qparams_many(const ctmi_observe_job* jobs, int64_t n, int32_t qtype, int32_t num_bits,
+                              int32_t symmetric, int32_t scale_dtype, int32_t zp_dtype, void* stream);
+
 /* A26.  Dynamic activation quantization in one pass (forward_quantize with
  * args.dynamic, quantization/lifecycle/forward.py:414-451): the scales of
  * compute_dynamic_scales_and_zp (quantization/utils/helpers.py:149-205, via

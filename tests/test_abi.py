@@ -362,3 +362,26 @@ def test_stacked_and_activation_ordered_entry_points_check_their_arguments(ctmi)
     rc = ctmi.ctmi_observe_pack_quantized_gidx(0x1000, _lib.I8, 64, 4096, 128, 4, 1, None, 0x2000, 0x3000,
                                                None, None)
     assert rc == _lib.CTMI_ERR_UNSUPPORTED
+
+
+def test_many_weight_observer_checks_every_job_first(ctmi):
+    """ctmi_observe_qparams_many: the whole list is validated on the host before any launch"""
+    jobs = (_lib.ObserveJob * 2)()
+    for j in jobs:
+        j.x, j.scale, j.zero_point, j.rows, j.cols, j.blk_cols, j.x_dtype = 0x1000, 0x2000, 0x3000, 4, 256, 128, _lib.BF16
+    call = ctmi.ctmi_observe_qparams_many
+    assert call(None, 0, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) == _lib.CTMI_OK
+    assert call(None, 2, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) == _lib.CTMI_ERR_VALUE
+    assert call(jobs, -1, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) == _lib.CTMI_ERR_VALUE
+    jobs[1].rows = 0
+    assert call(jobs, 2, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) == _lib.CTMI_ERR_VALUE
+    assert "job 1" in _err(ctmi)
+    jobs[1].rows, jobs[1].blk_cols = 4, 0
+    assert call(jobs, 2, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) == _lib.CTMI_ERR_VALUE
+    jobs[1].blk_cols, jobs[1].scale = 128, 0
+    assert call(jobs, 2, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) == _lib.CTMI_ERR_VALUE
+    assert "job 1" in _err(ctmi)
+    jobs[1].scale, jobs[1].x_dtype = 0x2000, _lib.I8  # an integer tensor has no observer
+    assert call(jobs, 2, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) != _lib.CTMI_OK
+    jobs[1].x_dtype = _lib.BF16
+    assert call(jobs, 2, _lib.QTYPE_FLOAT, 4, 0, -1, _lib.F8E4M3, None) != _lib.CTMI_OK  # asymmetric fp4

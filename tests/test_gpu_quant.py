@@ -449,6 +449,59 @@ def test_quantized_weight_batch_matches_single_calls(gpu):
         assert d.dtype == back.dtype and torch.equal(d.view(torch.int16), back.view(torch.int16))
 
 
+MANY_OBS = [
+    dict(num_bits=4, type="int", symmetric=True, strategy="group", group_size=128),
+    dict(num_bits=4, type="int", symmetric=False, strategy="group", group_size=32),
+    dict(num_bits=8, type="float", symmetric=True, strategy="channel"),
+    dict(num_bits=8, type="int", symmetric=False, strategy="channel"),
+    dict(num_bits=4, type="float", symmetric=True, strategy="tensor_group", group_size=16),
+    dict(num_bits=8, type="int", symmetric=True, strategy="tensor"),
+]
+
+
+@pytest.mark.parametrize("spec", MANY_OBS, ids=[f"{s['type']}{s['num_bits']}-{s['strategy']}" for s in MANY_OBS])
+def test_observer_for_many_weights_in_one_call(spec, gpu):
+    """ctmi_observe_qparams_many (8 weights per launch) against the oracle's observer and
+    against one call per weight: mixed shapes and dtypes in one list, more than 8 weights of
+    a kind, rows longer than one wave covers, shapes no vectorised kernel takes, NaN and
+    infinite elements, and (fp4) global scales."""
+    from compressed_tensors_amd.quantization import observe_weight_qparams, observe_weights_qparams
+
+    announce("observe_many", spec)
+    args, oargs = _pair(spec)
+    shapes = [(64, 512), (8, 4096), (33, 128), (16, 14336), (128, 1024), (5, 96), (16, 16), (256, 256),
+              (3, 4128), (40, 640), (7, 48), (48, 96), (24, 8192), (12, 384), (9, 32), (4, 1024),
+              (2, 4096), (64, 64), (1, 16), (32, 2048)]
+    if spec.get("group_size", 16) > 16:
+        shapes = [(r, -(-c // spec["group_size"]) * spec["group_size"]) for r, c in shapes]
+    dtypes = [torch.bfloat16, torch.bfloat16, torch.float16, torch.bfloat16, torch.float32]
+    ws, gss = [], []
+    for i, shape in enumerate(shapes):
+        w = _weights(shape, dtypes[i % len(dtypes)], seed=100 + i)
+        if i == 5:  # (no global scale for this one)
+            w[2, 40] = float("inf")
+        if i == 7:  # (what a NaN becomes is compared with the single call only)
+            w[3, 17] = float("nan")
+        ws.append(w)
+        gss.append(None)
+        if spec["strategy"] == "tensor_group" and i % 3 != 2:
+            gss[-1] = oq.generate_gparam(*torch.aminmax(ws[i if i != 7 else 0]))
+    wg = [w.to(gpu) for w in ws]
+    gg = [None if g is None else g.to(gpu) for g in gss]
+    got = observe_weights_qparams(wg, args, global_scales=gg if any(g is not None for g in gg) else None)
+    assert len(got) == len(ws)
+    for i, (w, gs, (scale, zp)) in enumerate(zip(ws, gss, got)):
+        if i != 7:
+            o_scale, o_zp = oq.observe_weight(w, oargs, global_scale=gs)
+            assert_bit_equal(scale, o_scale, f"scale {i} {tuple(w.shape)} {w.dtype}")
+            assert_bit_equal(zp, o_zp, f"zero_point {i} {tuple(w.shape)} {w.dtype}")
+        one_s, one_z = observe_weight_qparams(wg[i], args, global_scale=gg[i])
+        assert one_s.dtype == scale.dtype and one_s.shape == scale.shape and one_z.dtype == zp.dtype
+        assert torch.equal(one_s.view(torch.uint8), scale.view(torch.uint8))
+        assert torch.equal(one_z.view(torch.uint8), zp.view(torch.uint8))
+    assert observe_weights_qparams([], args) == []
+
+
 def test_mxfp4_scale_helpers_on_every_input(gpu):
     """round_to_power_2 and generate_mxfp4_scales on all 65 536 bfloat16 patterns,
     convert_mxfp4_exp_scale on all 256 exponents, against the oracle"""
