@@ -310,15 +310,25 @@ def other_workload(torch, name, seed):
         om = (oq_jobs, len(entries), 1, 8, 1, -1, code(FP8), st)
         w_many = [lambda om=om: _lib.check(lib.ctmi_observe_quantize_many(*om))]
         # block strategy (128 x 128 cells): the same one pass, a block per workgroup
-        w_blk = []
+        w_blk, blk_scales = [], []
         for e, codes in zip(entries, batch.codes):
             w = e["weight"]
             r, c = w.shape
             sb = torch.empty(r // 128, c // 128, dtype=w.dtype, device=dev)
-            keep.append(sb)
+            blk_scales.append(sb)
             ob = (w.data_ptr(), code(w.dtype), codes.data_ptr(), r, c, 128, 128, 1, 8, 1, sb.data_ptr(),
                   code(sb.dtype), None, code(FP8), st)
             w_blk.append(lambda ob=ob: _lib.check(lib.ctmi_observe_quantize_blocks(*ob)))
+        bjobs = (_lib.ObserveQuantizeBlocksJob * len(entries))()
+        for job, e, codes, sb in zip(bjobs, entries, batch.codes, blk_scales):
+            w = e["weight"]
+            job.x, job.codes, job.scale, job.zero_point = w.data_ptr(), codes.data_ptr(), sb.data_ptr(), None
+            job.rows, job.cols, job.blk_rows, job.blk_cols = w.shape[0], w.shape[1], 128, 128
+            job.x_dtype = code(w.dtype)
+        keep.append(bjobs)
+        bm = (bjobs, len(entries), 1, 8, 1, -1, code(FP8), st)
+        w_blk_many = [lambda bm=bm: _lib.check(lib.ctmi_observe_quantize_blocks_many(*bm))]
+        keep.append(blk_scales)
         acts, a_obs, a_fq, a_dyn = [], [], [], []
         targs = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="token",
                                  dynamic=True)
@@ -343,6 +353,8 @@ def other_workload(torch, name, seed):
                Op("weights one-shot: scales + fp8 codes in one pass, one call (8 per launch)", w_many, 3 * n, "dynamic_rows_many_kernel", launches=chained(len(entries))),
                Op("weights one-shot, 128x128 blocks: scales + fp8 codes in one pass (224 calls)", w_blk, 3 * n,
                   "observe_quantize_blocks_kernel", primary=False),
+               Op("weights one-shot, 128x128 blocks: scales + fp8 codes in one pass, one call (8 per launch)", w_blk_many,
+                  3 * n, "observe_quantize_blocks_many_kernel", launches=chained(len(entries))),
                Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
                Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel"),
                Op("activations: scales + fake-quantize in one pass (8 x 8192x4096)", a_dyn, 4 * na, "dynamic_rows_kernel")]

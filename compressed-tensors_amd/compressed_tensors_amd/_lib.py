@@ -120,6 +120,14 @@ class ObserveQuantizeJob(ctypes.Structure):
                 ("reserved", c_int32)]
 
 
+class ObserveQuantizeBlocksJob(ctypes.Structure):
+    """mirror of `struct ctmi_observe_quantize_blocks_job`"""
+
+    _fields_ = [("x", c_void_p), ("codes", c_void_p), ("scale", c_void_p), ("zero_point", c_void_p),
+                ("rows", c_int64), ("cols", c_int64), ("blk_rows", c_int64), ("blk_cols", c_int64),
+                ("x_dtype", c_int32), ("reserved", c_int32)]
+
+
 class ObservePackJob(ctypes.Structure):
     """ctmi_observe_pack_job"""
     _fields_ = [
@@ -363,6 +371,10 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_int32, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int32, c_int32, c_int32,
          c_void_p, c_int32, c_void_p, c_int32, c_void_p],
+    ),
+    "ctmi_observe_quantize_blocks_many": (
+        c_int32,
+        [POINTER(ObserveQuantizeBlocksJob), c_int64, c_int32, c_int32, c_int32, c_int32, c_int32, c_void_p],
     ),
     "ctmi_observe_quantize_many": (
         c_int32,

@@ -96,6 +96,8 @@ def observe_and_compress_weights(weights, quantization_args: QuantizationArgs):
     lib = _lib.load()
     qtype = _lib.QTYPE_INT if args.type == "int" else _lib.QTYPE_FLOAT
     results = [None] * len(weights)
+    if args.strategy == QuantizationStrategy.BLOCK.value:
+        return _observe_and_compress_blocks_many(weights, args, qtype)
     batch = []
     for i, weight in enumerate(weights):
         w = to_gpu(weight)
@@ -133,6 +135,46 @@ def observe_and_compress_weights(weights, quantization_args: QuantizationArgs):
             job.x_dtype = _lib.dtype_code(w.dtype)
         dev = batch[0][0].device
         _lib.check(lib.ctmi_observe_quantize_many(
+            jobs, len(batch), qtype, args.num_bits, int(args.symmetric), -1,
+            _lib.dtype_code(_zp_dtype(args)), _lib.stream_of(dev)))
+    return results
+
+
+def _observe_and_compress_blocks_many(weights, args: QuantizationArgs, qtype: int):
+    """the block strategy of observe_and_compress_weights: ctmi_observe_quantize_blocks_many for
+    the weights whose blocks fit a workgroup's registers, the single-weight path for the rest"""
+    from compressed_tensors_amd.quantization.helpers import _zp_dtype
+
+    lib = _lib.load()
+    bh, bw = args.block_structure
+    results = [None] * len(weights)
+    batches = {}
+    for i, weight in enumerate(weights):
+        w = to_gpu(weight)
+        w = w.contiguous() if w.ndim == 2 else w
+        if not (w.ndim == 2 and w.numel() > 0 and can_quantize(w, args)
+                and w.data_ptr() % (8 * w.element_size()) == 0
+                and lib.ctmi_observe_quantize_blocks_supported(
+                    _lib.dtype_code(w.dtype), w.shape[0], w.shape[1], bh, bw, qtype, args.num_bits)):
+            comp = BaseCompressor.load_from_registry(CompressionFormat.naive_quantized.value)
+            results[i] = comp.observe_and_compress_weight(weight, args)
+            continue
+        rows, cols = w.shape
+        out = {"weight": torch.empty((rows, cols), dtype=args.pytorch_dtype(), device=w.device),
+               "weight_scale": torch.empty((rows // bh, cols // bw), dtype=w.dtype, device=w.device)}
+        if not args.symmetric:
+            out["weight_zero_point"] = torch.empty((rows // bh, cols // bw), dtype=_zp_dtype(args),
+                                                   device=w.device)
+        results[i] = out
+        batches.setdefault(w.device, []).append((w, out))
+    for dev, batch in batches.items():
+        jobs = (_lib.ObserveQuantizeBlocksJob * len(batch))()
+        for job, (w, out) in zip(jobs, batch):
+            job.x, job.codes, job.scale = w.data_ptr(), out["weight"].data_ptr(), out["weight_scale"].data_ptr()
+            job.zero_point = _lib.ptr(out.get("weight_zero_point"))
+            job.rows, job.cols, job.blk_rows, job.blk_cols = w.shape[0], w.shape[1], bh, bw
+            job.x_dtype = _lib.dtype_code(w.dtype)
+        _lib.check(lib.ctmi_observe_quantize_blocks_many(
             jobs, len(batch), qtype, args.num_bits, int(args.symmetric), -1,
             _lib.dtype_code(_zp_dtype(args)), _lib.stream_of(dev)))
     return results

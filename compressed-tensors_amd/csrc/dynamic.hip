@@ -202,6 +202,31 @@ __global__ void __launch_bounds__(256) dynamic_rows_many_kernel(DynJobs t, QpCfg
                                       t.items[j], s - first, c);
 }
 
+// Blocks of up to kDynMaxJobs tensors per launch (one workgroup per block, as above)
+struct DynBlockJobs {
+  const void* x[kDynMaxJobs];
+  void* out[kDynMaxJobs];
+  DynOut o[kDynMaxJobs];
+  int64_t end[kDynMaxJobs];  // running total of blocks, job 0 .. j (unused: INT64_MAX)
+  int items[kDynMaxJobs];
+  CellLayout g[kDynMaxJobs];
+};
+
+template <typename FT, int QK, bool SYM, int U>
+__global__ void __launch_bounds__(256) observe_quantize_blocks_many_kernel(DynBlockJobs t, QpCfg c) {
+  const int64_t s = blockIdx.x;
+  int j = 0;
+  int64_t first = 0;
+#pragma unroll
+  for (int i = 0; i < kDynMaxJobs - 1; ++i) {
+    const bool past = s >= t.end[i];
+    j = past ? i + 1 : j;
+    first = past ? t.end[i] : first;
+  }
+  rows_segment<FT, QK, SYM, U, true, true>(static_cast<const typename FT::raw*>(t.x[j]), t.out[j], t.o[j],
+                                           t.items[j], s - first, c, t.g[j]);
+}
+
 // Segments of L vectors, L a power of two <= 64 (group strategies): L neighbouring
 // lanes own a segment; memory is one run of vectors numbered like the segments.
 template <typename FT, int QK, bool SYM, bool CODES>
@@ -532,4 +557,101 @@ extern "C" int ctmi_observe_quantize_many(const ctmi_observe_quantize_job* jobs,
     if (rc) return rc;
   }
   return CTMI_OK;
+}
+
+// vectors-per-thread class of a block (items = vectors of 8 elements in a block)
+static int block_class(int64_t items) { return items <= 256 ? 1 : items <= 512 ? 2 : items <= 1024 ? 4 : 8; }
+
+template <typename FT, int QK, bool SYM>
+static void launch_blocks_many(const DynBlockJobs& t, int filled, int u, const QpCfg& c, hipStream_t st) {
+  const unsigned grid = (unsigned)t.end[filled - 1];
+#define CTMI_BM(UU) \
+  hipLaunchKernelGGL((observe_quantize_blocks_many_kernel<FT, QK, SYM, UU>), grid, 256, 0, st, t, c)
+  if (u == 1) CTMI_BM(1);
+  else if (u == 2) CTMI_BM(2);
+  else if (u == 4) CTMI_BM(4);
+  else CTMI_BM(8);
+#undef CTMI_BM
+}
+
+extern "C" int ctmi_observe_quantize_blocks_many(const ctmi_observe_quantize_blocks_job* jobs, int64_t n,
+                                                 int32_t qtype, int32_t num_bits, int32_t symmetric,
+                                                 int32_t scale_dtype, int32_t zp_dtype, void* stream) {
+  CTMI_REQUIRE(n >= 0 && (jobs || n == 0), CTMI_ERR_VALUE, "bad job list");
+  if (n == 0) return CTMI_OK;
+  for (int64_t i = 0; i < n; ++i) {  // everything is looked at before anything is enqueued
+    const ctmi_observe_quantize_blocks_job& j = jobs[i];
+    CTMI_REQUIRE(j.rows >= 1 && j.cols >= 1, CTMI_ERR_VALUE, "job %lld: cannot observe an empty tensor",
+                 (long long)i);
+    CTMI_REQUIRE(j.blk_rows >= 1 && j.blk_cols >= 1, CTMI_ERR_VALUE, "job %lld: empty cell", (long long)i);
+    QpCfg c;
+    int rc = fill_qpcfg(&c, qtype, num_bits, symmetric, j.x_dtype, 0, false,
+                        scale_dtype < 0 ? j.x_dtype : scale_dtype, zp_dtype);
+    if (rc) return rc;
+    CTMI_REQUIRE(j.x && j.codes && j.scale, CTMI_ERR_VALUE, "job %lld: NULL tensor pointer", (long long)i);
+    CTMI_REQUIRE(ctmi_observe_quantize_blocks_supported(j.x_dtype, j.rows, j.cols, j.blk_rows, j.blk_cols,
+                                                        qtype, num_bits),
+                 CTMI_ERR_UNSUPPORTED,
+                 "job %lld: no fused kernel for this layout (blocks must tile the tensor, be a multiple "
+                 "of 8 wide and hold at most 16384 elements)", (long long)i);
+    CTMI_REQUIRE((uintptr_t)j.x % (8 * dtype_size(j.x_dtype)) == 0 && (uintptr_t)j.codes % 8 == 0,
+                 CTMI_ERR_VALUE, "job %lld: tensors must be aligned to 8 elements", (long long)i);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const int qk = qtype == CTMI_QTYPE_INT ? 0 : 1;
+  // blocks of one size class and dtype share launches, kDynMaxJobs tensors at a time
+  const int dts[3] = {CTMI_BF16, CTMI_F16, CTMI_F32};
+  const int classes[4] = {1, 2, 4, 8};
+  for (int d = 0; d < 3; ++d) {
+    QpCfg c;
+    fill_qpcfg(&c, qtype, num_bits, symmetric, dts[d], 0, false, scale_dtype < 0 ? dts[d] : scale_dtype,
+               zp_dtype);
+    for (int k = 0; k < 4; ++k) {
+      DynBlockJobs t;
+      int filled = 0;
+      auto reset = [&]() {
+        filled = 0;
+        for (int q = 0; q < kDynMaxJobs; ++q) {
+          t.x[q] = nullptr;
+          t.out[q] = nullptr;
+          t.o[q] = DynOut{nullptr, nullptr};
+          t.end[q] = INT64_MAX;
+          t.items[q] = 1;
+          t.g[q] = CellLayout{1, 1, 1, 1};
+        }
+      };
+      auto flush = [&]() {
+        if (!filled) return;
+#define CTMI_BM_SYM(FT, QK)                                                    \
+  (symmetric ? launch_blocks_many<FT, QK, true>(t, filled, classes[k], c, st)  \
+             : launch_blocks_many<FT, QK, false>(t, filled, classes[k], c, st))
+#define CTMI_BM_FT(FT) (qk == 0 ? CTMI_BM_SYM(FT, 0) : CTMI_BM_SYM(FT, 1))
+        if (dts[d] == CTMI_BF16) CTMI_BM_FT(BF16);
+        else if (dts[d] == CTMI_F16) CTMI_BM_FT(F16);
+        else CTMI_BM_FT(F32);
+#undef CTMI_BM_SYM
+#undef CTMI_BM_FT
+        reset();
+      };
+      reset();
+      for (int64_t i = 0; i < n; ++i) {
+        const ctmi_observe_quantize_blocks_job& j = jobs[i];
+        const int64_t items = j.blk_rows * j.blk_cols / 8;
+        if (j.x_dtype != dts[d] || block_class(items) != classes[k]) continue;
+        const int64_t blocks = (j.rows / j.blk_rows) * (j.cols / j.blk_cols);  // < 2^31 (checked above)
+        const int64_t before = filled ? t.end[filled - 1] : 0;
+        if (filled == kDynMaxJobs || before + blocks >= (1ll << 31)) flush();
+        t.x[filled] = j.x;
+        t.out[filled] = j.codes;
+        t.o[filled] = DynOut{j.scale, j.zero_point};
+        t.items[filled] = (int)items;
+        t.g[filled] = CellLayout{(int)(j.blk_cols / 8), (int)(j.cols / 8), (int)(j.cols / j.blk_cols),
+                                 (int)j.blk_rows};
+        t.end[filled] = (filled ? t.end[filled - 1] : 0) + blocks;
+        ++filled;
+      }
+      flush();
+    }
+  }
+  return check_launch("ctmi_observe_quantize_blocks_many");
 }

@@ -705,6 +705,12 @@ tile_popcount_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
 // is handed from one workgroup to another inside a launch: the end of the count
 // kernel is what makes its stores visible, and the library keeps no state of its own.
 constexpr int kGroupTiles = 64;
+#ifndef CTMI_SCATTER_TILES
+#define CTMI_SCATTER_TILES 1
+#endif
+// tiles a scatter workgroup takes (8192x8192 bf16, half the bits set: 1 and 2 run alike,
+// 4 is a fifth slower: the kernel is not waiting for memory latency)
+constexpr int kScatterTiles = CTMI_SCATTER_TILES;
 constexpr int kGroupThreads = 1024;
 constexpr int kMaxGroups = 1024;
 struct TileInfo {
@@ -772,7 +778,10 @@ tile_popcount_groups_kernel(const uint8_t* __restrict__ bitmask, int64_t nbytes,
 // store instruction of the wavefront writes 1 KB without gaps (whole memory lines; with
 // a lane's 16 elements side by side a store would leave every other 16 bytes to the
 // next one, and the device moves such halves noticeably slower).
-template <typename R, bool GROUPED>
+//
+// A workgroup takes T neighbouring tiles (of one group) and goes through them side by
+// side: bitmask bytes and values of all T are asked for before anything is waited for.
+template <typename R, bool GROUPED, int T>
 __global__ void __launch_bounds__(kBlock)
 bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
                              const uint8_t* __restrict__ bitmask,
@@ -780,137 +789,182 @@ bitmask_scatter_tiles_kernel(const R* __restrict__ values, int64_t nvalues,
                              const int64_t* __restrict__ tile_offsets,
                              const TileInfo* __restrict__ info,
                              const int32_t* __restrict__ group_total, R* __restrict__ out,
-                             int64_t numel) {
+                             int64_t numel, int64_t ntiles) {
   constexpr int VE = 16 / (int)sizeof(R);  // elements of a piece
   constexpr int NP = 16 / VE;              // pieces of a lane
   constexpr int P = (NP + 1) / 2;
+  constexpr int kStage = kTileElems + 2 * VE + 16;
+  constexpr int kRoundsIn = (kTileElems + 2 * VE) / (kBlock * VE) + 1;  // vectors a lane stages
   static_assert(kTileElems == kWaves * kWave * 16, "1024 elements per wavefront");
-  __shared__ int wtot[kWaves];
-  // the tile's values, up to VE - 1 before them and room for the reads of unset
+  static_assert(kGroupTiles % T == 0, "the tiles of a workgroup share a group");
+  __shared__ int wtot[T][kWaves];
+  // a tile's values, up to VE - 1 before them and room for the reads of unset
   // elements behind the last one
-  __shared__ __align__(16) R stage[kTileElems + 2 * VE + 16];
+  __shared__ __align__(16) R stage[T][kStage];
   const int tid = threadIdx.x, lane = lane_id(), wave = tid / kWave;
-  const int64_t tile = blockIdx.x;
-  int64_t excl;
-  int total;
-  if constexpr (GROUPED) {
-    // set bits before the tile's group: every wavefront adds the totals of the earlier
-    // groups up by itself (no more than kMaxGroups / kWave loads a lane, all in flight
-    // together, and no barrier)
-    const int group = (int)(tile / kGroupTiles);
-    int part[kMaxGroups / kWave];
-#pragma unroll
-    for (int k = 0; k < kMaxGroups / kWave; ++k) {
-      const int g = k * kWave + lane;
-      part[k] = (k * kWave < group && g < group) ? group_total[g] : 0;
-    }
-    // (a tensor on this path has at most kMaxGroups * kGroupTiles * kTileElems = 2^28 elements)
-    int sum = 0;
-#pragma unroll
-    for (int k = 0; k < kMaxGroups / kWave; ++k) sum += part[k];
-#pragma unroll
-    for (int d = kWave / 2; d > 0; d >>= 1) sum += __shfl_xor(sum, d, kWave);
-    const TileInfo ti = info[tile];
-    excl = (int64_t)sum + ti.before;
-    total = ti.count;
-  } else {
-    excl = tile_offsets[tile];
-    total = (int)tile_counts[tile];
-  }
-
+  const int64_t tile0 = (int64_t)blockIdx.x * T;
   // the lane's pieces and their bits (numel is a multiple of 16: a piece is inside
   // the tensor as a whole or not at all)
-  const int64_t elem0 = tile * kTileElems + wave * (kWave * 16) + lane * VE;
-  uint32_t bits[NP];
+  uint32_t bits[T][NP];
 #pragma unroll
-  for (int q = 0; q < NP; ++q) {
-    const int64_t elem = elem0 + q * (kWave * VE);
-    bits[q] = 0;
-    if (elem < numel) {
-      if constexpr (VE == 16) bits[q] = reinterpret_cast<const uint16_t*>(bitmask)[elem >> 4];
-      else bits[q] = ((uint32_t)bitmask[elem >> 3] >> (elem & 7)) & ((1u << VE) - 1u);
-    }
-  }
-  // values [excl, excl + total) -> LDS, from the 16-byte boundary below excl; lanes
-  // count in elements from there, `have` of which exist
-  const int64_t base = excl & ~(int64_t)(VE - 1);
-  const int off = (int)(excl - base);
-  const int nvecs = (off + total + VE - 1) / VE;
-  const int64_t left = nvalues - base;
-  const int have = (int)(left < 0 ? 0 : left > kTileElems + 2 * VE ? kTileElems + 2 * VE : left);
-  const R* from = values + base;
-  for (int i = tid; i < nvecs; i += kBlock) {
-    const int e0 = i * VE;
-    Vec<R, VE> v;
+  for (int t = 0; t < T; ++t) {
+    const int64_t elem0 = (tile0 + t) * kTileElems + wave * (kWave * 16) + lane * VE;
 #pragma unroll
-    for (int e = 0; e < VE; ++e) v.v[e] = (R)0;
-    if (e0 < have) {
-      // an aligned vector that starts inside the buffer never leaves its page
-      v = ldg<R, VE>(from + e0);
-      if (e0 + VE > have) {  // set bits beyond the values read as zero
-#pragma unroll
-        for (int e = 0; e < VE; ++e)
-          if (e0 + e >= have) v.v[e] = (R)0;
+    for (int q = 0; q < NP; ++q) {
+      const int64_t elem = elem0 + q * (kWave * VE);
+      bits[t][q] = 0;
+      if (elem < numel) {
+        if constexpr (VE == 16) bits[t][q] = reinterpret_cast<const uint16_t*>(bitmask)[elem >> 4];
+        else bits[t][q] = ((uint32_t)bitmask[elem >> 3] >> (elem & 7)) & ((1u << VE) - 1u);
       }
     }
-    *reinterpret_cast<Vec<R, VE>*>(stage + e0) = v;
   }
-  // Ranks.  In the tile's order a wavefront's piece q of all lanes comes before its
-  // piece q + 1.  Two pieces' counts ride through one scan as 16-bit fields.
-  int first[NP];
-  int wave_total = 0;
+  int64_t excl[T];
+  int total[T];
+  if constexpr (GROUPED) {
+    // set bits before the tiles' group: every wavefront adds the totals of the earlier
+    // groups up by itself, four neighbouring totals a lane and round (group_total is
+    // aligned to 16 bytes and readable up to the next multiple of 4 totals), 256 groups a
+    // round, and no barrier.  The number of rounds is the same for the whole workgroup.
+    // (a tensor on this path has at most kMaxGroups * kGroupTiles * kTileElems = 2^28 elements)
+    const int group = (int)(tile0 / kGroupTiles);
+    constexpr int kRounds = kMaxGroups / (4 * kWave);
+    const auto counted = [&](const u32x4_t v, int first) {  // of four totals from group `first` on
+      const int left = group - first;
+      return (int)v.x + (left > 1 ? (int)v.y : 0) + (left > 2 ? (int)v.z : 0) + (left > 3 ? (int)v.w : 0);
+    };
+    int sum = 0;
+    if (lane * 4 < group)
+      sum = counted(*reinterpret_cast<const u32x4_t*>(group_total + lane * 4), lane * 4);
+    if (group > 4 * kWave) {  // tensors beyond 2^26 elements: the other rounds, loads first
+      u32x4_t part[kRounds];
 #pragma unroll
-  for (int p = 0; p < P; ++p) {
-    uint32_t cnt2 = (uint32_t)__popc(bits[2 * p]);
-    if (2 * p + 1 < NP) cnt2 |= (uint32_t)__popc(bits[2 * p + 1]) << 16;
-    const uint32_t inc2 = (uint32_t)wave_inclusive_scan((int)cnt2);
-    const uint32_t all2 = (uint32_t)__builtin_amdgcn_readlane((int)inc2, kWave - 1);
-    const uint32_t below2 = inc2 - cnt2;
-    first[2 * p] = wave_total + (int)(below2 & 0xffffu);
-    wave_total += (int)(all2 & 0xffffu);
-    if (2 * p + 1 < NP) {
-      first[2 * p + 1] = wave_total + (int)(below2 >> 16);
-      wave_total += (int)(all2 >> 16);
+      for (int k = 1; k < kRounds; ++k) {
+        part[k] = u32x4_t{0, 0, 0, 0};
+        if (k * 4 * kWave + lane * 4 < group)
+          part[k] = *reinterpret_cast<const u32x4_t*>(group_total + k * 4 * kWave + lane * 4);
+      }
+#pragma unroll
+      for (int k = 1; k < kRounds; ++k) sum += counted(part[k], k * 4 * kWave + lane * 4);
+    }
+    sum = __builtin_amdgcn_readlane(wave_inclusive_scan(sum), kWave - 1);
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const TileInfo ti = tile0 + t < ntiles ? info[tile0 + t] : TileInfo{0, 0};
+      excl[t] = (int64_t)sum + ti.before;
+      total[t] = ti.count;
+    }
+  } else {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const bool in = tile0 + t < ntiles;
+      excl[t] = in ? tile_offsets[tile0 + t] : 0;
+      total[t] = in ? (int)tile_counts[tile0 + t] : 0;
     }
   }
-  if (lane == 0) wtot[wave] = wave_total;
-  __syncthreads();
-  int before = off;
+
+  // values [excl, excl + total) -> LDS, from the 16-byte boundary below excl; lanes
+  // count in elements from there, `have` of which exist.  All loads of all tiles first.
+  int off[T];
+  Vec<R, VE> in[T][kRoundsIn] = {};
 #pragma unroll
-  for (int w = 0; w < kWaves; ++w) {
-    const int t = wtot[w];
-    before += w < wave ? t : 0;
+  for (int t = 0; t < T; ++t) {
+    const int64_t base = excl[t] & ~(int64_t)(VE - 1);
+    off[t] = (int)(excl[t] - base);
+    const int nvecs = (off[t] + total[t] + VE - 1) / VE;
+    const int64_t left = nvalues - base;
+    const int have = (int)(left < 0 ? 0 : left > kTileElems + 2 * VE ? kTileElems + 2 * VE : left);
+    const R* from = values + base;
+#pragma unroll
+    for (int r = 0; r < kRoundsIn; ++r) {
+      const int e0 = (r * kBlock + tid) * VE;
+      // an aligned vector that starts inside the buffer never leaves its page
+      if (r * kBlock + tid < nvecs && e0 < have) in[t][r] = ldg<R, VE>(from + e0);
+    }
   }
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    const int64_t base = excl[t] & ~(int64_t)(VE - 1);
+    const int nvecs = (off[t] + total[t] + VE - 1) / VE;
+    const int64_t left = nvalues - base;
+    const int have = (int)(left < 0 ? 0 : left > kTileElems + 2 * VE ? kTileElems + 2 * VE : left);
+#pragma unroll
+    for (int r = 0; r < kRoundsIn; ++r) {
+      const int e0 = (r * kBlock + tid) * VE;
+      if (r * kBlock + tid < nvecs) {
+        Vec<R, VE> v = in[t][r];
+        if (e0 + VE > have) {  // set bits beyond the values read as zero
+#pragma unroll
+          for (int e = 0; e < VE; ++e)
+            if (e0 + e >= have) v.v[e] = (R)0;
+        }
+        *reinterpret_cast<Vec<R, VE>*>(&stage[t][e0]) = v;
+      }
+    }
+  }
+  // Ranks.  In a tile's order a wavefront's piece q of all lanes comes before its
+  // piece q + 1.  Two pieces' counts ride through one scan as 16-bit fields.
+  int first[T][NP];
+#pragma unroll
+  for (int t = 0; t < T; ++t) {
+    int wave_total = 0;
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      uint32_t cnt2 = (uint32_t)__popc(bits[t][2 * p]);
+      if (2 * p + 1 < NP) cnt2 |= (uint32_t)__popc(bits[t][2 * p + 1]) << 16;
+      const uint32_t inc2 = (uint32_t)wave_inclusive_scan((int)cnt2);
+      const uint32_t all2 = (uint32_t)__builtin_amdgcn_readlane((int)inc2, kWave - 1);
+      const uint32_t below2 = inc2 - cnt2;
+      first[t][2 * p] = wave_total + (int)(below2 & 0xffffu);
+      wave_total += (int)(all2 & 0xffffu);
+      if (2 * p + 1 < NP) {
+        first[t][2 * p + 1] = wave_total + (int)(below2 >> 16);
+        wave_total += (int)(all2 >> 16);
+      }
+    }
+    if (lane == 0) wtot[t][wave] = wave_total;
+  }
+  __syncthreads();
   // Element j of a piece is value number popcount(bits below j) of the piece's if bit j
   // is set.  Every element is read, set or not (the place is inside the staged image
   // either way), and cleared by a mask afterwards: no branch per element.
 #pragma unroll
-  for (int q = 0; q < NP; ++q) {
-    const int64_t elem = elem0 + q * (kWave * VE);
-    if (elem < numel) {
-      const uint32_t mine = bits[q];
-      const int at = before + first[q];
-      Vec<R, VE> o;
-      if constexpr (sizeof(R) == 2) {
-        uint32_t w2[VE / 2];
+  for (int t = 0; t < T; ++t) {
+    int before = off[t];
 #pragma unroll
-        for (int h = 0; h < VE / 2; ++h) {
-          const uint32_t lo = stage[at + __popc(mine & ((1u << (2 * h)) - 1u))];
-          const uint32_t hi = stage[at + __popc(mine & ((1u << (2 * h + 1)) - 1u))];
-          const uint32_t keep_lo = (uint32_t)((int32_t)(mine << (31 - 2 * h)) >> 31);
-          const uint32_t keep_hi = (uint32_t)((int32_t)(mine << (30 - 2 * h)) >> 31);
-          w2[h] = (lo | (hi << 16)) & ((keep_lo & 0xffffu) | (keep_hi & 0xffff0000u));
-        }
-        o = __builtin_bit_cast(Vec<R, VE>, w2);
-      } else {
+    for (int w = 0; w < kWaves; ++w) {
+      const int wt = wtot[t][w];
+      before += w < wave ? wt : 0;
+    }
+    const int64_t elem0 = (tile0 + t) * kTileElems + wave * (kWave * 16) + lane * VE;
 #pragma unroll
-        for (int j = 0; j < VE; ++j) {
-          const R v = stage[at + __popc(mine & ((1u << j) - 1u))];
-          const R keep = (R)(0 - (R)((mine >> j) & 1u));
-          o.v[j] = v & keep;
+    for (int q = 0; q < NP; ++q) {
+      const int64_t elem = elem0 + q * (kWave * VE);
+      if (elem < numel) {
+        const uint32_t mine = bits[t][q];
+        const R* st = &stage[t][before + first[t][q]];
+        Vec<R, VE> o;
+        if constexpr (sizeof(R) == 2) {
+          uint32_t w2[VE / 2];
+#pragma unroll
+          for (int h = 0; h < VE / 2; ++h) {
+            const uint32_t lo = st[__popc(mine & ((1u << (2 * h)) - 1u))];
+            const uint32_t hi = st[__popc(mine & ((1u << (2 * h + 1)) - 1u))];
+            const uint32_t keep_lo = (uint32_t)((int32_t)(mine << (31 - 2 * h)) >> 31);
+            const uint32_t keep_hi = (uint32_t)((int32_t)(mine << (30 - 2 * h)) >> 31);
+            w2[h] = (lo | (hi << 16)) & ((keep_lo & 0xffffu) | (keep_hi & 0xffff0000u));
+          }
+          o = __builtin_bit_cast(Vec<R, VE>, w2);
+        } else {
+#pragma unroll
+          for (int j = 0; j < VE; ++j) {
+            const R v = st[__popc(mine & ((1u << j) - 1u))];
+            const R keep = (R)(0 - (R)((mine >> j) & 1u));
+            o.v[j] = v & keep;
+          }
         }
+        stg_nt<R, VE>(out + elem, o);
       }
-      stg_nt<R, VE>(out + elem, o);
     }
   }
 }
@@ -1943,7 +1997,10 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
     const bool grouped = ngroups <= kMaxGroups;
     if (grouped) {
       info = (TileInfo*)tmp;
-      totals = (int32_t*)(info + ntiles);  // set bits of each group
+      // set bits of each group, from the next 16-byte boundary (the scatter kernel reads
+      // four totals per load); ctmi_bitmask_tmp_bytes leaves room for that and for the
+      // round-up of the last four
+      totals = (int32_t*)(((uintptr_t)(info + ntiles) + 15) & ~(uintptr_t)15);
       hipLaunchKernelGGL(tile_popcount_groups_kernel, (unsigned)ngroups, kGroupThreads, 0, st,
                          bitmask, rows * pc, info, totals, ntiles);
     } else {
@@ -1956,13 +2013,13 @@ static int scatter_entry(const void* values, int64_t nvalues, int32_t elem_size,
     }
 #define CTMI_TILES(R)                                                                              \
   if (grouped)                                                                                     \
-    hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, true>), (unsigned)ntiles, kBlock, 0, st,   \
-                       (const R*)values, nvalues, bitmask, counts, offs, info, totals, (R*)out,    \
-                       numel);                                                                     \
+    hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, true, kScatterTiles>),                     \
+                       (unsigned)cdiv(ntiles, kScatterTiles), kBlock, 0, st, (const R*)values,     \
+                       nvalues, bitmask, counts, offs, info, totals, (R*)out, numel, ntiles);      \
   else                                                                                             \
-    hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, false>), (unsigned)ntiles, kBlock, 0, st,  \
-                       (const R*)values, nvalues, bitmask, counts, offs, info, totals, (R*)out,    \
-                       numel)
+    hipLaunchKernelGGL((bitmask_scatter_tiles_kernel<R, false, kScatterTiles>),                    \
+                       (unsigned)cdiv(ntiles, kScatterTiles), kBlock, 0, st, (const R*)values,     \
+                       nvalues, bitmask, counts, offs, info, totals, (R*)out, numel, ntiles)
     if (elem_size == 1) { CTMI_TILES(uint8_t); }
     else if (elem_size == 2) { CTMI_TILES(uint16_t); }
     else { CTMI_TILES(uint32_t); }

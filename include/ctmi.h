@@ -544,6 +544,22 @@ int ctmi_observe_quantize_many(const ctmi_observe_quantize_job* jobs, int64_t n,
                                int32_t num_bits, int32_t symmetric, int32_t scale_dtype,
                                int32_t zp_dtype, void* stream);
 
+/* ctmi_observe_quantize_blocks for every weight of a state dict in one call (blocks of one
+ * size class share launches, eight weights at a time).  Every job must be one that
+ * ctmi_observe_quantize_blocks_supported accepts; the whole list is checked before anything
+ * is enqueued.  scale_dtype < 0: every weight's scales in its own dtype. */
+typedef struct ctmi_observe_quantize_blocks_job {
+  const void* x;
+  void* codes;
+  void* scale;      /* [rows / blk_rows, cols / blk_cols] */
+  void* zero_point; /* optional */
+  int64_t rows, cols, blk_rows, blk_cols;
+  int32_t x_dtype, reserved;
+} ctmi_observe_quantize_blocks_job;
+int ctmi_observe_quantize_blocks_many(const ctmi_observe_quantize_blocks_job* jobs, int64_t n,
+                                      int32_t qtype, int32_t num_bits, int32_t symmetric,
+                                      int32_t scale_dtype, int32_t zp_dtype, void* stream);
+
 /* MXFP4 group scales (quantization/utils/mxfp4_utils.py): powers of two held as
  * uint8 exponents.  x / out of the first two are bfloat16 group maxima, n values.
  *   ctmi_mxfp4_round_to_power_2   :41-73  (x + 32) & 0xFF80 on the bf16 bits

@@ -385,3 +385,27 @@ def test_many_weight_observer_checks_every_job_first(ctmi):
     assert call(jobs, 2, _lib.QTYPE_INT, 4, 1, -1, _lib.I8, None) != _lib.CTMI_OK
     jobs[1].x_dtype = _lib.BF16
     assert call(jobs, 2, _lib.QTYPE_FLOAT, 4, 0, -1, _lib.F8E4M3, None) != _lib.CTMI_OK  # asymmetric fp4
+
+
+def test_many_weight_block_one_shot_checks_every_job_first(ctmi):
+    """ctmi_observe_quantize_blocks_many: what the single-weight query refuses stops the whole call"""
+    jobs = (_lib.ObserveQuantizeBlocksJob * 2)()
+    for j in jobs:
+        j.x, j.codes, j.scale, j.rows, j.cols, j.blk_rows, j.blk_cols, j.x_dtype = (
+            0x1000, 0x2000, 0x3000, 256, 512, 128, 128, _lib.BF16)
+    call = ctmi.ctmi_observe_quantize_blocks_many
+    fp8 = (_lib.QTYPE_FLOAT, 8, 1, -1, _lib.F8E4M3, None)
+    assert call(None, 0, *fp8) == _lib.CTMI_OK
+    assert call(None, 2, *fp8) == _lib.CTMI_ERR_VALUE
+    jobs[1].blk_rows = 256  # 32768 elements: more than a workgroup's registers hold
+    assert call(jobs, 2, *fp8) == _lib.CTMI_ERR_UNSUPPORTED
+    assert "job 1" in _err(ctmi)
+    assert ctmi.ctmi_observe_quantize_blocks_supported(_lib.BF16, 256, 512, 256, 128, _lib.QTYPE_FLOAT, 8) == 0
+    jobs[1].blk_rows, jobs[1].cols = 128, 520  # blocks do not tile the rows
+    assert call(jobs, 2, *fp8) == _lib.CTMI_ERR_UNSUPPORTED
+    jobs[1].cols, jobs[1].codes = 512, 0
+    assert call(jobs, 2, *fp8) == _lib.CTMI_ERR_VALUE
+    jobs[1].codes, jobs[1].x = 0x2000, 0x1002  # not aligned to 8 elements
+    assert call(jobs, 2, *fp8) == _lib.CTMI_ERR_VALUE
+    jobs[1].x, jobs[1].rows = 0x1000, 0
+    assert call(jobs, 2, *fp8) == _lib.CTMI_ERR_VALUE

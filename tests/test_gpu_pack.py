@@ -945,6 +945,52 @@ def test_naive_observe_and_compress_in_one_pass(fmt, spec, shape, dtype, gpu):
     assert got["weight"].dtype == args.pytorch_dtype()
 
 
+BLOCKS_MANY = [
+    dict(num_bits=8, type="float", symmetric=True, strategy="block", block_structure=[128, 128]),
+    dict(num_bits=8, type="int", symmetric=False, strategy="block", block_structure=[16, 64]),
+    dict(num_bits=8, type="float", symmetric=False, strategy="block", block_structure=[32, 128]),
+]
+
+
+@pytest.mark.parametrize("spec", BLOCKS_MANY, ids=[f"{s['type']}-{s['block_structure'][0]}x{s['block_structure'][1]}" for s in BLOCKS_MANY])
+def test_block_observe_and_compress_many_weights(spec, gpu):
+    """block strategy, a list of weights from one call (ctmi_observe_quantize_blocks_many): the
+    oracle's observer, calculate_qparams and naive compression bit for bit, and the single
+    call; more weights than a launch takes, three dtypes, a weight of a single all-zero block"""
+    from compressed_tensors_amd.compressors import BaseCompressor, observe_and_compress_weights
+
+    announce("one-shot blocks, many weights", spec)
+    args, oargs = _pair(spec)
+    bh, bw = spec["block_structure"]
+    mult = [(2, 4), (1, 32), (8, 1), (1, 1), (3, 5), (16, 2), (4, 4), (2, 9), (1, 2), (5, 3), (6, 6)]
+    dtypes = [torch.bfloat16, torch.float16, torch.bfloat16, torch.float32]
+    g = torch.Generator().manual_seed(17)
+    ws = []
+    for i, (a, b) in enumerate(mult):
+        w = torch.randn(a * bh, b * bw, generator=g) * 0.02
+        w[torch.rand(w.shape, generator=g) < 0.002] *= 20
+        w = w.to(dtypes[i % len(dtypes)])
+        w.view(-1)[1] = -0.0
+        if i == 3:
+            w[:] = 0  # an all-zero block: the scale is clamped from below
+        ws.append(w)
+    got = observe_and_compress_weights([w.to(gpu) for w in ws], args)
+    comp = BaseCompressor.load_from_registry("naive-quantized")
+    assert len(got) == len(ws)
+    for i, (w, out) in enumerate(zip(ws, got)):
+        scale, zp = oq.observe_weight(w, oargs)
+        want = op.naive_compress(w, scale, oargs, zero_point=zp)
+        assert set(out) == ({"weight", "weight_scale"} | (set() if spec["symmetric"] else {"weight_zero_point"}))
+        assert_bit_equal(out["weight_scale"], scale, f"scale {i}")
+        if not spec["symmetric"]:
+            assert_bit_equal(out["weight_zero_point"], zp, f"zero point {i}")
+        assert_bit_equal(out["weight"], want, f"codes {i}")
+        single = comp.observe_and_compress_weight(w.to(gpu), args)
+        for key in single:
+            assert_bit_equal(out[key], single[key].cpu(), f"single call, weight {i} {key}")
+    assert observe_and_compress_weights([], args) == []
+
+
 def test_naive_observe_and_compress_many_weights(gpu):
     """observe_and_compress_weights == observe_and_compress_weight weight by weight: more
     weights than a launch takes, rows of every length class, two dtypes, a weight whose
