@@ -118,6 +118,52 @@ def test_bitmask_empty_and_state_dict(gpu):
     assert "a.bias" in restored and "b.weight" in restored
 
 
+def test_bitmask_compress_of_a_state_dict_waits_for_the_gpu_once(gpu, monkeypatch):
+    """BitmaskCompressor.compress over several targets (bitmask_compress_many): the oracle's
+    values, bitmasks and row offsets for every weight, the key order of the loop over
+    compress_weight, other entries passed through, and one read-back of the counts for all"""
+    from compressed_tensors_amd.compressors import BaseCompressor
+    from compressed_tensors_amd.compressors import sparse_bitmask as sb
+
+    announce("sparse-bitmask state dict")
+    state, dense = {}, {}
+    for i, (shape, dtype, sparsity) in enumerate(BM[:9] + [((4, 16), torch.bfloat16, 1.0)]):
+        x = (_sparse_tensor(shape, dtype, sparsity, seed=50 + i) if dtype != torch.int8
+             else (torch.arange(shape[0] * shape[1]).reshape(shape) % 3).to(torch.int8))
+        dense[f"m{i}"] = x
+        state[f"m{i}.weight"] = x.to(gpu)
+        state[f"m{i}.bias"] = torch.full((shape[0],), float(i), device=gpu)
+    state["emb.weight"] = torch.ones(3, 5, device=gpu)  # not a target
+    state["norm.weight"] = torch.ones(7, device=gpu)    # 1-D and not a target either
+    targets = set(dense)
+    calls = []
+    real = sb.bitmask_compress_many
+    monkeypatch.setattr(sb, "bitmask_compress_many", lambda ts: calls.append(len(ts)) or real(ts))
+    comp = BaseCompressor.load_from_registry("sparse-bitmask")
+    out = comp.compress(state, compression_targets=targets)
+    assert calls == [len(dense)]
+    want_keys = []
+    for name in state:
+        prefix = name[: -len(".weight")]
+        if name.endswith(".weight") and prefix in targets:
+            want_keys += [f"{prefix}.{p}" for p in ("shape", "compressed", "bitmask", "row_offsets")]
+        else:
+            want_keys.append(name)
+    assert list(out) == want_keys
+    for name, x in dense.items():
+        o_values, o_bitmask, o_offsets = osp.bitmask_compress(x)
+        assert_bit_equal(out[f"{name}.compressed"], o_values, f"{name} values")
+        assert_bit_equal(out[f"{name}.bitmask"], o_bitmask, f"{name} bitmask")
+        assert_bit_equal(out[f"{name}.row_offsets"], o_offsets, f"{name} row_offsets")
+        assert out[f"{name}.shape"].tolist() == list(x.shape)
+    assert out["emb.weight"] is state["emb.weight"]
+    back = dict(comp.decompress(out))
+    for name, x in dense.items():
+        o_values, o_bitmask, _ = osp.bitmask_compress(x)  # (-0.0 is dropped: comes back as 0.0)
+        assert_bit_equal(back[f"{name}.weight"], osp.bitmask_decompress(o_values, o_bitmask, list(x.shape)),
+                         f"{name} round trip")
+
+
 def _prune24(x):
     keep = osp.get_24_bytemasks(x)
     return torch.where(keep, x, torch.zeros_like(x))
