@@ -675,14 +675,20 @@ def other_workload(torch, name, seed):
             mb = deterministic_hadamard_matrix(b_dim, torch.bfloat16, dev).contiguous()
             ma = deterministic_hadamard_matrix(a_dim, torch.bfloat16, dev).contiguous() if a_dim > 1 else None
             keep.extend([q, mb, ma])
+            # size 128: no matrix argument stands for Sylvester's matrix (the kernel that keeps none
+            # in memory); the kernel that is handed the matrix is timed beside it on one line
+            mbp = None if a_dim == 1 else mb.data_ptr()
+            rows_kernel = "sylvester128_quant_pack_kernel" if a_dim == 1 else "hadamard_kron_kernel"
             for label, xs in tensors.items():
-                calls = []
+                calls, with_matrix = [], []
                 for x in xs:
                     out = torch.empty_like(x)
                     keep.extend([x, out])
                     a = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), a_dim, b_dim,
-                         _lib.ptr(ma), mb.data_ptr(), q.data_ptr(), None, st)
+                         _lib.ptr(ma), mbp, q.data_ptr(), None, st)
                     calls.append(lambda a=a: _lib.check(lib.ctmi_hadamard_apply(*a)))
+                    am = a[:7] + (mb.data_ptr(),) + a[8:]
+                    with_matrix.append(lambda am=am: _lib.check(lib.ctmi_hadamard_apply(*am)))
                 nb = sum(4 * x.numel() for x in xs)
                 # matrix-core flops per element: 2 b for the one product of a block-b rotation;
                 # 2 b + 3 * 2 a for a Kronecker pair (the fp32 result of the first product goes
@@ -693,21 +699,25 @@ def other_workload(torch, name, seed):
                 # size 4096 on the matrix cores: kept to compare with the butterfly kernel below,
                 # which is what hadamard_apply picks for this size
                 ops.append(Op(f"random-sign Hadamard, size {n}{' (matrix cores)' if a_dim > 1 else ''}: {label}",
-                              calls, nb, "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
+                              calls, nb, rows_kernel,
                               primary=a_dim == 1 and not label.startswith("weights 4096x4096"), mfma_flops=flops,
                               useful_flops=useful))
+                if a_dim == 1 and label.startswith("weights 14336x4096"):
+                    ops.append(Op(f"random-sign Hadamard, size {n}, any matrix of 128 (passed as an argument): {label}",
+                                  with_matrix, nb, "hadamard_rows_kernel", primary=False, mfma_flops=flops,
+                                  useful_flops=useful))
                 if label.startswith("weights 4096x4096"):
                     jobs = (_lib.HadamardJob * len(xs))()
                     outs = [torch.empty_like(x) for x in xs]
                     for job, x, out in zip(jobs, xs, outs):
                         job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()
                     keep.extend([jobs, outs])
-                    m = (jobs, len(xs), code(xs[0].dtype), a_dim, b_dim, _lib.ptr(ma), mb.data_ptr(),
+                    m = (jobs, len(xs), code(xs[0].dtype), a_dim, b_dim, _lib.ptr(ma), mbp,
                          q.data_ptr(), None, st)
                     ops.append(Op(f"random-sign Hadamard, size {n}{' (matrix cores)' if a_dim > 1 else ''}: {label}, "
                                   "one call (8 per launch)",
                                   [lambda m=m: _lib.check(lib.ctmi_hadamard_apply_many(*m))], nb,
-                                  "hadamard_rows_kernel" if a_dim == 1 else "hadamard_kron_kernel",
+                                  rows_kernel,
                                   primary=a_dim == 1, mfma_flops=flops, useful_flops=useful,
                                   launches=chained(len(xs))))
         # sizes 4096 and 8192 as butterflies in registers (ctmi_sylvester_apply_many): what

@@ -248,8 +248,8 @@ def _aligned(*tensors) -> bool:
 
 
 def _matrix_free(n: int, dtype, *tensors) -> bool:
-    """does the fused rotation + quantization by Sylvester's matrix of order n run without a
-    matrix argument?"""
+    """does the rotation (alone or fused with the quantization) by Sylvester's matrix of order
+    n run without a matrix argument?"""
     return n == 128 and dtype == torch.bfloat16 and _aligned(*tensors)
 
 
@@ -291,6 +291,8 @@ def hadamard_apply(
     s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
     s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
     out = torch.empty_like(x)
+    if matrix_t is None and _matrix_free(n, x.dtype, x, out, s_in, s_out):
+        mb_t = None  # Sylvester's matrix of 128: the kernel that keeps no matrix in memory
     _lib.check(
         lib.ctmi_hadamard_apply(
             x.data_ptr(), out.data_ptr(), code, x.numel(), a, b, _lib.ptr(ma_t), _lib.ptr(mb_t),
@@ -484,6 +486,8 @@ def hadamard_apply_many(
     s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
     s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
     outs = [torch.empty_like(x) for x in xs]
+    if matrix_t is None and _matrix_free(n, dtype, s_in, s_out, *xs, *outs):
+        mb_t = None  # Sylvester's matrix of 128: the kernel that keeps no matrix in memory
     jobs = (_lib.HadamardJob * len(xs))()
     for job, x, out in zip(jobs, xs, outs):
         job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()

@@ -490,6 +490,9 @@ fwht_mfma_kernel(FwhtTable tab, const float* __restrict__ sign_in, const float* 
   }
 }
 
+#ifndef CTMI_FWHT_STREAM_FROM
+#define CTMI_FWHT_STREAM_FROM 8192
+#endif
 // A workgroup takes every grid-th run, so all workgroups have to be resident together and
 // carry equally many runs: one that starts when another has finished runs alone for as long
 // again.  How many fit a compute unit (registers, LDS) is the runtime's to say; *resident_wgs
@@ -497,7 +500,7 @@ fwht_mfma_kernel(FwhtTable tab, const float* __restrict__ sign_in, const float* 
 template <typename Kernel>
 int launch_persistent(Kernel kern, int threads, int* resident_wgs, const FwhtTable& tab,
                       const float* sign_in, const float* sign_out, const float* w0, float scale,
-                      const QpCfg& cfg, hipStream_t st) {
+                      const QpCfg& cfg, hipStream_t st, int64_t stream_from = INT64_MAX) {
   if (*resident_wgs == 0) {
     int per_cu = 0, dev = 0, cus = 0;
     hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kern, threads, 0);
@@ -507,7 +510,9 @@ int launch_persistent(Kernel kern, int threads, int* resident_wgs, const FwhtTab
     *resident_wgs = (per_cu > 0 ? per_cu : 1) * (cus > 0 ? cus : 256);
   }
   const int64_t resident = *resident_wgs;
-  const int64_t runs_each = (tab.total + resident - 1) / resident;
+  // (stream_from: from that many runs on a workgroup takes one run and leaves, and the
+  // hardware hands out the runs)
+  const int64_t runs_each = tab.total >= stream_from ? 1 : (tab.total + resident - 1) / resident;
   const unsigned grid = (unsigned)((tab.total + runs_each - 1) / runs_each);
   hipLaunchKernelGGL(kern, grid, threads, 0, st, tab, sign_in, sign_out, w0, scale, cfg);
   return CTMI_OK;
@@ -525,8 +530,11 @@ template <bool SIGN_IN, bool SIGN_OUT, bool MANY, bool QUANT>
 int launch_fwht_mfma_variant(const FwhtTable& tab, const float* sign_in, const float* sign_out,
                              const float* w0, float scale, const QpCfg& cfg, hipStream_t st) {
   static int resident_wgs = 0;
+  // The rotation alone on 8192 runs or more: one run per workgroup (14336x4096: 0.70 of the HBM
+  // peak against 0.65 with every workgroup resident and looping; at 4096 runs the loop wins,
+  // 0.62 against 0.50, and with the quantization behind it the loop wins at every size).
   return launch_persistent(fwht_mfma_kernel<SIGN_IN, SIGN_OUT, MANY, QUANT>, kWave, &resident_wgs, tab,
-                           sign_in, sign_out, w0, scale, cfg, st);
+                           sign_in, sign_out, w0, scale, cfg, st, QUANT ? INT64_MAX : CTMI_FWHT_STREAM_FROM);
 }
 
 template <bool QUANT>

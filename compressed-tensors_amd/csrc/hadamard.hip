@@ -755,11 +755,22 @@ constexpr int kSqpWaves = kSqpThreads / kWave;
 #ifndef CTMI_SQP_MIN_WAVES
 #define CTMI_SQP_MIN_WAVES 4
 #endif
-template <bool MANY, bool SIGN_IN, bool SIGN_OUT>
+// QUANT = false: the rotation alone (jobs.out takes the rotated sub-rows, whole groups on
+// their way out through the image as well, so that loads and stores are both whole lines).
+#ifndef CTMI_SR_GROUPS
+#define CTMI_SR_GROUPS 1  // the rotation alone: groups of 16 sub-rows a wavefront takes (14336x4096: 1: 0.76 of the HBM peak, 2: 0.73, 4: 0.69)
+#endif
+#ifndef CTMI_SR_STORE
+#define CTMI_SR_STORE stg_nt
+#endif
+#ifndef CTMI_SR_IMAGE_MANY
+#define CTMI_SR_IMAGE_MANY 1  // the rotation alone: launches over several tensors use the image too
+#endif
+template <bool MANY, bool SIGN_IN, bool SIGN_OUT, bool QUANT = true>
 __global__ void __launch_bounds__(kSqpThreads, CTMI_SQP_MIN_WAVES)
 sylvester128_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const float* __restrict__ s_in,
                     const float* __restrict__ s_out, float inv_sqrt_n, QpCfg cfg) {
-  constexpr int B = 128, KS = 4, NP = 4, G = CTMI_SQP_GROUPS;
+  constexpr int B = 128, KS = 4, NP = 4, G = QUANT ? CTMI_SQP_GROUPS : CTMI_SR_GROUPS;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int l16 = lane & 15, lq = lane >> 4;
@@ -774,7 +785,7 @@ sylvester128_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const float* __re
   // pieces hit different banks.  A ragged last group is loaded in the operand layout directly.
   // (launches over several tensors load in the operand layout throughout: with the image they
   // measured 10 % slower, launches of one tensor 6 % faster)
-  constexpr bool kImage = CTMI_SQP_IMAGE && !MANY;
+  constexpr bool kImage = QUANT ? (CTMI_SQP_IMAGE && !MANY) : (!MANY || CTMI_SR_IMAGE_MANY);
   constexpr int kPitch = (2 * B + 16) / 4;  // dwords between sub-rows of the image
   __shared__ __attribute__((aligned(16))) uint32_t image_lds[kSqpWaves][kImage ? G * 16 * kPitch : 1];
   int job[G];
@@ -899,15 +910,55 @@ sylvester128_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const float* __re
       for (int w = 0; w < 4; ++w) {
         o[p].v[w] = pack_bf16x2(v[2 * w], v[2 * w + 1]);
         if constexpr (SIGN_OUT) o[p].v[w] ^= flip_out[p][w];
+        if constexpr (QUANT) {
 #if CTMI_SQP_FP32_MAX
-        top = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[2 * w]), __builtin_fabsf(v[2 * w + 1])), top);
+          top = __builtin_fmaxf(__builtin_fmaxf(__builtin_fabsf(v[2 * w]), __builtin_fabsf(v[2 * w + 1])), top);
 #else
-        top2 = __builtin_elementwise_max(top2, __builtin_bit_cast(u16x2_t, o[p].v[w] & 0x7FFF7FFFu));
+          top2 = __builtin_elementwise_max(top2, __builtin_bit_cast(u16x2_t, o[p].v[w] & 0x7FFF7FFFu));
 #endif
+        }
       }
 #if CTMI_SQP_FP32_MAX
-      if (p == 0) odd = v[0] != v[0];
+      if (QUANT && p == 0) odd = v[0] != v[0];
 #endif
+    }
+    // A sum that cancels exactly is +0 whatever the column's sign (the sign belongs to the
+    // matrix, the accumulator starts at +0): zeros among the outputs that leave as rotated
+    // values give back the sign bit the mask put on them.
+    auto unsigned_zeros = [](uint32_t w) -> uint32_t {
+      typedef uint16_t u16x2_t __attribute__((ext_vector_type(2)));
+      const u16x2_t one = {1, 1};
+      const u16x2_t nz = __builtin_elementwise_min(__builtin_bit_cast(u16x2_t, w & 0x7FFF7FFFu), one);
+      return w & ((__builtin_bit_cast(uint32_t, nz) << 15) | 0x7FFF7FFFu);
+    };
+    if constexpr (!QUANT) {
+      if constexpr (SIGN_OUT) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+          for (int w = 0; w < 4; ++w) o[p].v[w] = unsigned_zeros(o[p].v[w]);
+      }
+      uint16_t* dst = static_cast<uint16_t*>(jobs.out[job[t]]);
+      if (whole[t] && keep[t]) {
+        // back through the image: the lane's pieces of sub-row l16, then the stretch as it
+        // lies in memory (keep is true for every lane of a whole group)
+        uint32_t* img = &image_lds[wave][t * 16 * kPitch];
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+          *reinterpret_cast<u32x4_t*>(&img[l16 * kPitch + 16 * p + 4 * lq]) = __builtin_bit_cast(u32x4_t, o[p]);
+        const int64_t at = (row[t] - l16) * B + lane * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const int j = ks * kWave + lane;
+          const u32x4_t piece = *reinterpret_cast<const u32x4_t*>(&img[(j >> 4) * kPitch + (j & 15) * 4]);
+          CTMI_SR_STORE<uint16_t, 8>(dst + at + 512 * ks, __builtin_bit_cast(Vec<uint16_t, 8>, piece));
+        }
+      } else if (!whole[t] && keep[t]) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+          CTMI_SR_STORE<uint16_t, 8>(dst + row[t] * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o[p]));
+      }
+      continue;
     }
     // max |x| of the sub-row: the 4 lanes l16 + 16 q agree through two lane exchanges
     // (magnitudes of non-negative floats order like their bit patterns, a NaN above everything)
@@ -947,8 +998,14 @@ sylvester128_quant_pack_kernel(HadJobs jobs, int64_t n_groups, const float* __re
     for (int p = 0; p < NP; ++p) {
       w[p] = (uint32_t)quant_pack8<BF16, BF16, 4, false>(__builtin_bit_cast(Vec<uint16_t, 8>, o[p]), sv, 0.0f,
                                                          cfg.bit_min, cfg.bit_max).v[0];
-      if (rotated && keep[t])
-        CTMI_SQP_STORE<uint16_t, 8>(rotated + row[t] * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, o[p]));
+      if (rotated && keep[t]) {
+        Vec<uint32_t, 4> r = o[p];
+        if constexpr (SIGN_OUT) {
+#pragma unroll
+          for (int d = 0; d < 4; ++d) r.v[d] = unsigned_zeros(r.v[d]);
+        }
+        CTMI_SQP_STORE<uint16_t, 8>(rotated + row[t] * B + 32 * p + 8 * lq, __builtin_bit_cast(Vec<uint16_t, 8>, r));
+      }
     }
     // Lane (l16, lq) holds packed words 4 p + lq of its sub-row; the 4 lanes of a sub-row
     // transpose their 4 x 4 words in two exchanges (lanes 32 apart, then neighbouring rows
@@ -994,6 +1051,30 @@ static void sylvester128_launch(const HadJobs& t, int filled, const float* sign_
                        n_groups, sign_in, sign_out, inv, c)
   if (filled == 1) { CTMI_SQP(false); } else { CTMI_SQP(true); }
 #undef CTMI_SQP
+}
+
+// the rotation alone; jobs: t.end counts groups of 16 sub-rows (a tensor's last one may be ragged)
+static void sylvester128_rows_launch(const HadJobs& t, int filled, const float* sign_in,
+                                     const float* sign_out, hipStream_t st) {
+  const int64_t n_groups = t.end[filled - 1];
+  const float inv = 1.0f / sqrtf(128.0f);
+  const unsigned grid = (unsigned)cdiv(n_groups, kSqpWaves * CTMI_SR_GROUPS);
+  const QpCfg c{};
+#define CTMI_SR(MANY)                                                                                   \
+  if (sign_in && sign_out)                                                                              \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, true, true, false>), grid, kSqpThreads, 0, \
+                       st, t, n_groups, sign_in, sign_out, inv, c);                                     \
+  else if (sign_in)                                                                                     \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, true, false, false>), grid, kSqpThreads,   \
+                       0, st, t, n_groups, sign_in, sign_out, inv, c);                                  \
+  else if (sign_out)                                                                                    \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, false, true, false>), grid, kSqpThreads,   \
+                       0, st, t, n_groups, sign_in, sign_out, inv, c);                                  \
+  else                                                                                                  \
+    hipLaunchKernelGGL((sylvester128_quant_pack_kernel<MANY, false, false, false>), grid, kSqpThreads,  \
+                       0, st, t, n_groups, sign_in, sign_out, inv, c)
+  if (filled == 1) { CTMI_SR(false); } else { CTMI_SR(true); }
+#undef CTMI_SR
 }
 
 // ---------------------------------------------------------------- Kronecker sizes, bf16, no LDS staging
@@ -1410,6 +1491,11 @@ extern "C" int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_
   return 0;
 }
 
+// does the rotation by Sylvester's matrix of 128 run without a matrix argument?
+static bool sylvester128_rows_ok(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
+  return a_dim == 1 && b_dim == 128 && io_dtype == CTMI_BF16;
+}
+
 extern "C" int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype) {
   return a_dim > 1 && block_sylvester64_supported(a_dim, b_dim, io_dtype, false);
 }
@@ -1426,8 +1512,9 @@ extern "C" int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, i
   CTMI_REQUIRE(numel % n == 0, CTMI_ERR_VALUE,
                "tensor size %lld is not a multiple of the transform size %lld", (long long)numel,
                (long long)n);
-  if (!mb_t && a_dim > 1) {
+  if (!mb_t && (a_dim > 1 || sylvester128_rows_ok(a_dim, b_dim, io_dtype))) {
     // Mb = Sylvester's matrix: the product with Ma on the matrix cores, butterflies for Mb
+    // (or, for a block of 128, the kernel that keeps no matrix in memory)
     ctmi_hadamard_job job;
     job.x = x;
     job.out = out;
@@ -1476,6 +1563,40 @@ extern "C" int ctmi_hadamard_apply_many(const ctmi_hadamard_job* jobs, int64_t n
   CTMI_REQUIRE(a_dim >= 1 && b_dim >= 1, CTMI_ERR_VALUE, "bad factor sizes");
   CTMI_REQUIRE(io_dtype == CTMI_BF16 || io_dtype == CTMI_F16 || io_dtype == CTMI_F32,
                CTMI_ERR_UNSUPPORTED, "transforms take float16/bfloat16/float32 tensors");
+  if (!mb_t && sylvester128_rows_ok(a_dim, b_dim, io_dtype)) {
+    // Sylvester's matrix of 128 on bfloat16 tensors: no matrix in memory, any number of sub-rows
+    for (int64_t i = 0; i < n_jobs; ++i) {
+      const ctmi_hadamard_job& j = jobs[i];
+      CTMI_REQUIRE(j.numel >= 0 && j.numel % b_dim == 0, CTMI_ERR_VALUE,
+                   "job %lld: tensor size %lld is not a multiple of the transform size %d", (long long)i,
+                   (long long)j.numel, b_dim);
+      CTMI_REQUIRE(j.numel == 0 || (j.x && j.out), CTMI_ERR_VALUE, "job %lld: NULL tensor pointer", (long long)i);
+      CTMI_REQUIRE((uintptr_t)j.x % 16 == 0 && (uintptr_t)j.out % 16 == 0, CTMI_ERR_VALUE,
+                   "tensors must be 16-byte aligned");
+    }
+    CTMI_REQUIRE((uintptr_t)sign_in % 16 == 0 && (uintptr_t)sign_out % 16 == 0, CTMI_ERR_VALUE,
+                 "sign vectors must be 16-byte aligned");
+    HadJobs t;
+    clear_jobs(&t);
+    int filled = 0;
+    bool any = false;
+    for (int64_t i = 0; i <= n_jobs; ++i) {
+      if (i < n_jobs && jobs[i].numel > 0) {
+        t.x[filled] = jobs[i].x;
+        t.out[filled] = jobs[i].out;
+        t.n_sub[filled] = jobs[i].numel / b_dim;
+        t.end[filled] = (filled ? t.end[filled - 1] : 0) + cdiv(jobs[i].numel / b_dim, (int64_t)16);
+        ++filled;
+      }
+      if (filled == kHadMaxJobs || (i == n_jobs && filled)) {
+        sylvester128_rows_launch(t, filled, sign_in, sign_out, (hipStream_t)stream);
+        clear_jobs(&t);
+        filled = 0;
+        any = true;
+      }
+    }
+    return any ? check_launch("ctmi_hadamard_apply_many") : CTMI_OK;
+  }
   const bool sylvester_inner = !mb_t && a_dim > 1;
   if (sylvester_inner)
     CTMI_REQUIRE(ctmi_hadamard_sylvester_inner_supported(a_dim, b_dim, io_dtype) && !(sign_in && sign_out),

@@ -600,7 +600,10 @@ int ctmi_hadamard_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype);
  * block of its table, so the sizes met are 192 x 16 = 3072, 224 x 16 = 3584, 160 x 32 = 5120,
  * 224 x 32 = 7168, 224 x 64 = 14336, 224 x 128 = 28672 ...), bfloat16 or float16 tensors,
  * signs on one side
- * (ctmi_hadamard_sylvester_inner_supported). */
+ * (ctmi_hadamard_sylvester_inner_supported).
+ * mb_t == NULL with a_dim == 1, b_dim == 128 and bfloat16 tensors: Sylvester's matrix of 128
+ * (what the reference uses at this size) from a kernel that keeps no matrix in memory; same
+ * bits as with the matrix passed.  Tensors and sign vectors 16-byte aligned. */
 int ctmi_hadamard_sylvester_inner_supported(int32_t a_dim, int32_t b_dim, int32_t io_dtype);
 int ctmi_hadamard_apply(const void* x, void* out, int32_t io_dtype, int64_t numel, int32_t a_dim,
                         int32_t b_dim, const void* ma_t, const void* mb_t, const float* sign_in,

@@ -280,6 +280,60 @@ def test_many_tensors_in_one_call(n, dtype, gpu):
                 assert_bit_equal(y, hadamard_apply(x, n, **signs), f"tensor {i} ({rows[i]} rows)")
 
 
+@pytest.mark.parametrize("signs", ["none", "in", "out", "both"])
+def test_sylvester128_without_a_matrix(signs, gpu):
+    """Sylvester's matrix of 128 on bfloat16 tensors runs from a kernel that keeps no matrix in
+    memory (no matrix_t): the same bits as the kernel that is handed the matrix, one tensor
+    per call and several per call, whole and ragged groups of 16 sub-rows, in place; and the
+    fp64 product by the explicit matrix within one ulp"""
+    from compressed_tensors_amd import _lib
+    from compressed_tensors_amd.transform import hadamard_apply, hadamard_apply_many
+    from compressed_tensors_amd.transform.hadamard import _sylvester_bf16
+
+    announce("sylvester 128, no matrix", signs)
+    n = 128
+    g = torch.Generator().manual_seed(5)
+    q_in = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float() if signs in ("in", "both") else None
+    q_out = (torch.randint(0, 2, (n,), generator=g) * 2 - 1).float() if signs in ("out", "both") else None
+    kw = dict(sign_in=q_in, sign_out=q_out)
+    shapes = [(16, 128), (64, 512), (5, 256), (33, 384), (1, 128), (2048, 256), (7, 1152), (48, 128), (16, 256), (3, 128)]
+    xs = [(torch.randn(s, generator=g) * 0.05).bfloat16().to(gpu) for s in shapes]
+    xs[2][0, 3] = float("inf")
+    xs[3][1, 200] = float("nan")
+    matrix_t = _sylvester_bf16(n, gpu)
+    lib = _lib.load()
+    many = hadamard_apply_many(xs, n, **kw)
+    with_matrix = hadamard_apply_many(xs, n, matrix_t=matrix_t, **kw)
+    h = oh.deterministic_hadamard_matrix(n, dtype=torch.float64)
+    def same(got, want, what):  # bit for bit; a NaN is a NaN whatever its sign bit
+        got, want = got.cpu(), want.cpu()
+        nan = torch.isnan(want.float())
+        assert torch.equal(torch.isnan(got.float()), nan), f"{what}: NaNs"
+        assert_bit_equal(torch.where(nan, torch.zeros_like(got), got), torch.where(nan, torch.zeros_like(want), want), what)
+
+    for i, (x, y, w) in enumerate(zip(xs, many, with_matrix)):
+        same(y, w, f"tensor {i} {tuple(x.shape)}: no matrix vs matrix")
+        same(hadamard_apply(x, n, **kw), w, f"tensor {i}: single call")
+        if i not in (2, 3):
+            v = x.cpu().double().reshape(-1, n)
+            if q_in is not None:
+                v = v * q_in.double()
+            exact = v @ h
+            if q_out is not None:
+                exact = exact * q_out.double()
+            exact = (exact / n ** 0.5).reshape(x.shape).to(torch.bfloat16)
+            _assert_within_ulp(y, exact, f"tensor {i} vs fp64")
+    # in place
+    z = xs[1].clone()
+    lib_jobs = (_lib.HadamardJob * 1)()
+    lib_jobs[0].x, lib_jobs[0].out, lib_jobs[0].numel = z.data_ptr(), z.data_ptr(), z.numel()
+    s_in = None if q_in is None else q_in.to(gpu)
+    s_out = None if q_out is None else q_out.to(gpu)
+    _lib.check(lib.ctmi_hadamard_apply_many(lib_jobs, 1, _lib.dtype_code(z.dtype), 1, n, None, None,
+                                            _lib.ptr(s_in), _lib.ptr(s_out), _lib.stream_of(z.device)))
+    assert_bit_equal(z, with_matrix[1].cpu(), "in place")
+
+
 @pytest.mark.parametrize("n", [128, 4096, 2048, 1024])
 def test_fused_many_tensors_in_one_call(n, gpu):
     """hadamard_quantize_pack_many == hadamard_quantize_pack tensor by tensor"""
