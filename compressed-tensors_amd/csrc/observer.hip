@@ -294,7 +294,9 @@ struct ObsChainTable {  // the kernel's only argument: find_job_index reads its 
 static_assert(offsetof(ObsChainTable, chunk_end) == 0 && offsetof(ObsChainTable, n_items) == 32,
               "find_job_index");
 
-template <typename XT>
+// SYM (16-bit tensors, symmetric scheme): only max |x| matters, taken on the packed magnitude
+// bits (two elements per instruction; the min / max form keeps the vector ALUs 95 % busy).
+template <typename XT, bool SYM>
 __global__ void __launch_bounds__(256) observe_flat_chain_kernel(const ObsChainTable t) {
   constexpr int U = kObsUnroll;
   uint32_t local, nvec;
@@ -313,10 +315,17 @@ __global__ void __launch_bounds__(256) observe_flat_chain_kernel(const ObsChainT
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     float lo = __builtin_inff(), hi = -__builtin_inff();
-    bool unordered = false;
-    vec_minmax<XT>(a[k], &lo, &hi, &unordered);
-    group_minmax(L, &lo, &hi);
-    if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
+    if constexpr (SYM) {
+      const uint32_t m = group_umax(L, absmax8_bits<XT>(a[k]));
+      constexpr uint32_t kInf = XT::id == CTMI_BF16 ? 0x7f80u : 0x7c00u;
+      hi = m > kInf ? __builtin_nanf("") : XT::to_f32((typename XT::raw)m);
+      lo = -hi;
+    } else {
+      bool unordered = false;
+      vec_minmax<XT>(a[k], &lo, &hi, &unordered);
+      group_minmax(L, &lo, &hi);
+      if (group_any(L, unordered)) lo = hi = __builtin_nanf("");
+    }
     if ((threadIdx.x & (L - 1)) == 0) {
       const int slot = (k * 256 + threadIdx.x) / L;
       seg_lo[slot] = lo;
@@ -628,9 +637,14 @@ extern "C" int ctmi_observe_qparams_many(const ctmi_observe_job* jobs, int64_t n
     auto flush = [&]() {
       if (cnt == 0) return;
       CTMI_DISPATCH_XT(xd, {
-        if (lead.kind == 1)
-          hipLaunchKernelGGL(observe_flat_chain_kernel<XT>, (unsigned)chunks, 256, 0, st, t);
-        else
+        if (lead.kind == 1) {
+          if constexpr (sizeof(typename XT::raw) == 2) {
+            if (symmetric) hipLaunchKernelGGL((observe_flat_chain_kernel<XT, true>), (unsigned)chunks, 256, 0, st, t);
+            else hipLaunchKernelGGL((observe_flat_chain_kernel<XT, false>), (unsigned)chunks, 256, 0, st, t);
+          } else {
+            hipLaunchKernelGGL((observe_flat_chain_kernel<XT, false>), (unsigned)chunks, 256, 0, st, t);
+          }
+        } else
           hipLaunchKernelGGL(observe_wide_chain_kernel<XT>, (unsigned)chunks, 256, 0, st, t);
       });
       reset();
