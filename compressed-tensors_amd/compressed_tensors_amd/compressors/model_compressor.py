@@ -1,13 +1,17 @@
 """ModelCompressor: model-level compress / decompress on the GPU.
 
 Same entry points as the reference (compressors/model_compressors/model_compressor.py):
-  __init__ :309-345, compress_model :453-539, decompress_model :541-617,
-  compress :621-676, decompress :678-767, map_module_to_scheme :896-907.
+  from_pretrained :116-130, from_compression_config :133-169, from_pretrained_model :171-231,
+  parse_sparsity_config :233-251, parse_quantization_config :254-289, __init__ :309-345,
+  get_missing_module_keys :347-394, get_unexpected_file_keys :396-449,
+  compress_model :453-539, decompress_model :541-617, compress :621-676,
+  decompress :678-767, update_config :769-817, map_module_to_scheme :896-907.
 The reference moves every module to the CPU first (its comment "in the future,
 support compression on same device", :483 / :566); here tensors are compressed
 on the GPU they live on.  Modules carry their scheme in `quantization_scheme`
 (set by `apply_quantization_scheme` below or by the caller).
 """
+import logging
 import re
 from typing import Dict, List, Optional, Set
 
@@ -25,7 +29,7 @@ from compressed_tensors_amd.config import (
 )
 from compressed_tensors_amd.compressors.quantized_base import own_parameters, swap_parameters
 from compressed_tensors_amd.quantization.quant_scheme import QuantizationConfig, QuantizationScheme
-from compressed_tensors_amd.utils.helpers import load_safetensors_state_dict, nest_state_dict
+from compressed_tensors_amd.utils.helpers import load_safetensors_state_dict, merge_names, nest_state_dict
 
 __all__ = ["ModelCompressor", "map_module_to_scheme", "match_named_modules",
            "apply_quantization_scheme"]
@@ -440,24 +444,142 @@ class ModelCompressor:
             json.dump(config_data, config_file, indent=2, sort_keys=True)
 
     @classmethod
-    def from_compression_config(cls, compression_config: Optional[Dict]):
-        """a compressor from the `quantization_config` entry of a config.json (the
-        dict form; model_compressor.py:164-206)"""
-        if not compression_config:
+    def from_pretrained(cls, pretrained_model_name_or_path: str, **kwargs) -> Optional["ModelCompressor"]:
+        """a compressor from the `quantization_config` (or `compression_config`) entry of a
+        model's config (model_compressor.py:116-130); None for a model that is not
+        compressed.  A directory (or a config.json) on disk is read as JSON; anything else
+        goes through transformers' AutoConfig."""
+        import json
+        import os
+
+        path = str(pretrained_model_name_or_path)
+        config_file = os.path.join(path, "config.json") if os.path.isdir(path) else path
+        if os.path.isfile(config_file):
+            with open(config_file, "r") as file:
+                data = json.load(file)
+            compression_config = data.get(QUANTIZATION_CONFIG_NAME) or data.get("compression_config")
+        else:
+            from transformers import AutoConfig
+
+            config = AutoConfig.from_pretrained(pretrained_model_name_or_path, **kwargs)
+            compression_config = getattr(config, QUANTIZATION_CONFIG_NAME, None)
+        return cls.from_compression_config(compression_config)
+
+    @staticmethod
+    def parse_sparsity_config(compression_config) -> Optional[Dict]:
+        """the sparsity config nested inside a quantization / compression config, a dict or an
+        object with `sparsity_config` / `quantization_config` attributes (transformers'
+        CompressedTensorsConfig); an empty one is None (model_compressor.py:233-251)"""
+        if compression_config is None:
             return None
-        data = dict(compression_config)
-        sparsity = data.pop(SPARSITY_CONFIG_NAME, None) or None
+        if not isinstance(compression_config, dict):
+            s_config = getattr(compression_config, SPARSITY_CONFIG_NAME, None)
+            return s_config.model_dump() if s_config is not None else None
+        return compression_config.get(SPARSITY_CONFIG_NAME, None) or None
+
+    @staticmethod
+    def parse_quantization_config(compression_config) -> Optional[Dict]:
+        """every field that is not the sparsity config, the transform config or metadata; None
+        if nothing but metadata is left (model_compressor.py:254-289)"""
+        from copy import deepcopy
+
+        if compression_config is None:
+            return None
+        if not isinstance(compression_config, dict):
+            q_config = getattr(compression_config, QUANTIZATION_CONFIG_NAME, None)
+            return q_config.model_dump() if q_config is not None else None
+        data = deepcopy(compression_config)
+        data.pop(SPARSITY_CONFIG_NAME, None)
         data.pop("transform_config", None)
+        quant_method = data.pop("quant_method", None)
         data.pop("version", None)
-        sparsity_config = SparsityCompressionConfig(**sparsity) if sparsity else None
-        quantization_config = None
-        if data.get("config_groups"):
+        if not data:
+            return None
+        if quant_method is not None:
+            data["quant_method"] = quant_method
+        return data
+
+    @classmethod
+    def from_compression_config(cls, compression_config):
+        """a compressor from the `quantization_config` entry of a config.json or from
+        transformers' CompressedTensorsConfig (model_compressor.py:133-169); None if it names
+        neither a sparsity nor a quantization config"""
+        if compression_config is None:
+            return None
+        sparsity = cls.parse_sparsity_config(compression_config)
+        quantization = cls.parse_quantization_config(compression_config)
+        if sparsity is None and quantization is None:
+            return None
+        sparsity_config = quantization_config = None
+        if sparsity is not None:
+            sparsity_config = SparsityCompressionConfig.load_from_registry(sparsity.get("format"), **sparsity)
+        if quantization is not None and quantization.get("config_groups"):
             allowed = ("config_groups", "format", "quantization_status", "global_compression_ratio",
                        "ignore", "kv_cache_scheme", "quant_method")
-            quantization_config = QuantizationConfig(**{k: v for k, v in data.items() if k in allowed})
+            quantization_config = QuantizationConfig(**{k: v for k, v in quantization.items() if k in allowed})
         if sparsity_config is None and quantization_config is None:
             return None
         return cls(sparsity_config=sparsity_config, quantization_config=quantization_config)
+
+    @classmethod
+    def from_pretrained_model(cls, model: Module, sparsity_config_or_format=None,
+                              quantization_format: Optional[str] = None,
+                              sparsity_config=None) -> Optional["ModelCompressor"]:
+        """a compressor for a model in memory from the schemes its modules carry
+        (model_compressor.py:171-231): the quantization format of every module is inferred
+        (or set to `quantization_format`), the quantization config is read off the model;
+        sparsity_config_or_format: a SparsityCompressionConfig, a format name or None.  None
+        if there is nothing to compress."""
+        from compressed_tensors_amd.config import infer_and_set_per_module_quantization_format
+
+        if sparsity_config:
+            logging.getLogger(__name__).warning("sparsity_config is deprecated, use sparsity_config_or_format")
+            sparsity_config_or_format = sparsity_config
+        if sparsity_config_or_format and isinstance(sparsity_config_or_format, str):
+            sparsity_config = SparsityCompressionConfig.load_from_registry(sparsity_config_or_format)
+        else:
+            sparsity_config = sparsity_config_or_format
+        formats = infer_and_set_per_module_quantization_format(
+            model, sparsity_structure=sparsity_config.sparsity_structure if sparsity_config is not None else None,
+            quantization_format=quantization_format)
+        quantization_config = QuantizationConfig.from_pretrained(model, format=formats)
+        transform_config = getattr(model, "transform_config", None)
+        if not any((quantization_config, sparsity_config, transform_config)):
+            return None
+        return cls(sparsity_config=sparsity_config, quantization_config=quantization_config,
+                   transform_config=transform_config, compression_formats=formats)
+
+    def get_missing_module_keys(self, model: Module) -> List[str]:
+        """the `weight` keys a compressed checkpoint of `model` does not hold: targets of the
+        sparsity compressor and, for pack-quantized, of the quantization schemes
+        (model_compressor.py:347-394)"""
+        missing = set()
+        if self.sparsity_compressor and self.sparsity_config.format != CompressionFormat.dense.value:
+            missing.update(merge_names(name, "weight") for name, _ in match_named_modules(
+                model, self.sparsity_config.targets, self.sparsity_config.ignore))
+        if (self.quantization_compressor
+                and self.quantization_config.format == CompressionFormat.pack_quantized.value):
+            for scheme in self.quantization_config.config_groups.values():
+                missing.update(merge_names(name, "weight") for name, _ in match_named_modules(
+                    model, scheme.targets, self.quantization_config.ignore))
+        return list(missing)
+
+    def get_unexpected_file_keys(self, model: Module) -> List[str]:
+        """the keys a compressed checkpoint holds that `model` has no parameter for: the
+        compression parameters of every target (model_compressor.py:396-449)"""
+        unexpected = set()
+        if self.sparsity_compressor and self.sparsity_config.format != CompressionFormat.dense.value:
+            unexpected.update(
+                merge_names(name, param)
+                for name, _ in match_named_modules(model, self.sparsity_config.targets, self.sparsity_config.ignore)
+                for param in self.sparsity_compressor.compression_param_names)
+        if self.quantization_compressor:
+            for scheme in self.quantization_config.config_groups.values():
+                targets = list(match_named_modules(model, scheme.targets, self.quantization_config.ignore))
+                for compressor in self.quantization_compressor.values():
+                    unexpected.update(merge_names(name, param) for name, _ in targets
+                                      for param in compressor.compression_param_names if param != "weight")
+        return list(unexpected)
 
     # ----- in-memory pathways ----- #
     def _stream(self, model: Module, module_to_scheme: Dict[str, QuantizationScheme],

@@ -14,6 +14,7 @@ __all__ = [
     "QuantizationStatus",
     "SPARSITY_CONFIG_NAME",
     "QUANTIZATION_CONFIG_NAME",
+    "infer_and_set_per_module_quantization_format",
 ]
 
 SPARSITY_CONFIG_NAME = "sparsity_config"
@@ -83,3 +84,66 @@ class SparsityCompressionConfig:
 
     def model_dump(self) -> Dict[str, Any]:
         return dict(self.__dict__)
+
+    @classmethod
+    def load_from_registry(cls, name, **kwargs) -> "SparsityCompressionConfig":
+        """the config of a sparsity format by its registry name (config/base.py:97-114; the
+        reference registers one subclass per format, with the same fields)"""
+        fields = ("targets", "ignore", "global_sparsity", "sparsity_structure")
+        return cls(format=name, **{k: v for k, v in kwargs.items() if k in fields})
+
+    def __eq__(self, other) -> bool:
+        return isinstance(other, SparsityCompressionConfig) and self.model_dump() == other.model_dump()
+
+    __hash__ = None
+
+
+def _quant_compression_format(input_args, weight_args, sparsity_structure=None) -> CompressionFormat:
+    """the format a module's weight and input arguments ask for (config/format.py:32-84)"""
+    two_four = SparsityStructure(sparsity_structure) == SparsityStructure.TWO_FOUR
+    if weight_args.num_bits == 4 and weight_args.type == "float":
+        return CompressionFormat.nvfp4_pack_quantized
+    if input_args is None:  # weight only: W4A16, W8A16
+        if not (weight_args.num_bits in (4, 8) and weight_args.type == "int"):
+            return CompressionFormat.naive_quantized
+        if two_four and weight_args.strategy in ("channel", "group"):
+            return CompressionFormat.marlin_24
+        return CompressionFormat.pack_quantized
+    if weight_args.type == "float" and weight_args.num_bits == 8:
+        return CompressionFormat.float_quantized
+    if weight_args.type == "int":
+        return CompressionFormat.int_quantized
+    return CompressionFormat.naive_quantized
+
+
+def infer_and_set_per_module_quantization_format(model, sparsity_structure: Optional[str] = None,
+                                                 quantization_format: Optional[str] = None) -> Optional[List[str]]:
+    """sets `quantization_scheme.format` of every quantized module (the global format if one
+    is given, else the module's own, else the inferred one) and returns the distinct formats
+    of the model, None if no module is quantized (config/format.py:87-159)"""
+    import logging
+
+    formats: List[str] = []
+    for module in model.modules():
+        scheme = getattr(module, "quantization_scheme", None)
+        if scheme is None or not any(
+                a is not None for a in (scheme.weights, scheme.input_activations, scheme.output_activations)):
+            continue
+        if scheme.weights is not None:
+            inferred = _quant_compression_format(scheme.input_activations, scheme.weights, sparsity_structure).value
+            if quantization_format is not None:
+                if quantization_format != inferred:
+                    logging.getLogger(__name__).warning(
+                        "The provided format for the module does not match the inferred format. "
+                        "Compression may fail ")
+                scheme.format = quantization_format
+            elif scheme.format is not None:
+                if scheme.format != inferred:
+                    logging.getLogger(__name__).warning(
+                        "The provided format for the module does not match the inferred format. "
+                        "Compression may fail ")
+            else:
+                scheme.format = inferred
+        if scheme.format and scheme.format not in formats:
+            formats.append(scheme.format)
+    return formats or None

@@ -49,6 +49,11 @@ class QuantizationScheme:
             if args is not None and args.actorder is not None:
                 raise ValueError("Cannot apply actorder to activations")
 
+    def __eq__(self, other) -> bool:
+        return isinstance(other, QuantizationScheme) and self.model_dump() == other.model_dump()
+
+    __hash__ = None
+
     def model_dump(self) -> Dict[str, Any]:
         return {
             "targets": self.targets,
@@ -89,6 +94,69 @@ class QuantizationConfig:
         self.ignore = ignore or []
         self.kv_cache_scheme = kv_cache_scheme
         self.quant_method = quant_method
+
+    def __eq__(self, other) -> bool:
+        return isinstance(other, QuantizationConfig) and self.model_dump() == other.model_dump()
+
+    __hash__ = None
+
+    @classmethod
+    def model_validate(cls, data) -> "QuantizationConfig":
+        """a config from its plain-dict form (fields this class does not have are dropped)"""
+        if isinstance(data, QuantizationConfig):
+            return data
+        fields = ("config_groups", "format", "quantization_status", "global_compression_ratio", "ignore",
+                  "kv_cache_scheme", "quant_method")
+        return cls(**{k: v for k, v in dict(data).items() if k in fields})
+
+    @staticmethod
+    def from_pretrained(model, format=None) -> Optional["QuantizationConfig"]:
+        """the config of a model whose modules carry `quantization_scheme`
+        (quantization/quant_config.py:166-260): one group per distinct scheme, modules of a
+        quantized class without a scheme on the ignore list, the status of the last quantized
+        module; None if nothing is quantized.  format: a format, a list of formats
+        ("mixed-precision" if more than one) or None (int-quantized for a compressed model,
+        dense otherwise)."""
+        from compressed_tensors_amd.config import CompressionFormat, QuantizationStatus
+        from compressed_tensors_amd.modeling import IMPL_ATTR
+        from compressed_tensors_amd.quantization.initialize import is_attention_module
+
+        def quantized(module) -> bool:
+            scheme = getattr(module, "quantization_scheme", None)
+            return scheme is not None and any(
+                a is not None for a in (scheme.weights, scheme.input_activations, scheme.output_activations))
+
+        schemes: List[QuantizationScheme] = []
+        status = None
+        quantized_types = set()
+        unquantized: Dict[str, List[str]] = {}
+        kv_cache_scheme = None
+        for name, module in model.named_modules():
+            layer_type = type(module).__name__
+            attention = is_attention_module(module)
+            has_group = quantized(module) and (not attention or hasattr(module, IMPL_ATTR))
+            if has_group:
+                status = getattr(module, "quantization_status", status)
+                quantized_types.add(layer_type)
+                if module.quantization_scheme not in schemes:
+                    schemes.append(module.quantization_scheme)
+            if quantized(module) and attention:
+                status = getattr(module, "quantization_status", status)
+                kv_cache_scheme = module.quantization_scheme.input_activations
+            if not has_group:
+                unquantized.setdefault(layer_type, []).append(name)
+        if not schemes and kv_cache_scheme is None:
+            return None
+        ignore = [n for layer_type, names in unquantized.items() if layer_type in quantized_types for n in names]
+        if format is None:
+            compressed = getattr(status, "value", status) == QuantizationStatus.COMPRESSED.value
+            format = (CompressionFormat.int_quantized if compressed else CompressionFormat.dense).value
+        elif isinstance(format, (list, tuple)):
+            format = CompressionFormat.mixed_precision.value if len(format) > 1 else format[0]
+        return QuantizationConfig(
+            config_groups={f"group_{i}": scheme for i, scheme in enumerate(schemes)},
+            quantization_status=status, kv_cache_scheme=kv_cache_scheme,
+            global_compression_ratio=None, format=format, ignore=ignore)
 
     def model_dump(self, exclude=None) -> Dict[str, Any]:
         """plain-dict form, as written into a model's config.json"""
