@@ -11,6 +11,9 @@ __all__ = [
     "CompressionFormat",
     "SparsityStructure",
     "SparsityCompressionConfig",
+    "DenseSparsityConfig",
+    "BitmaskConfig",
+    "Sparse24BitMaskConfig",
     "QuantizationStatus",
     "SPARSITY_CONFIG_NAME",
     "QUANTIZATION_CONFIG_NAME",
@@ -96,6 +99,28 @@ class SparsityCompressionConfig:
         return isinstance(other, SparsityCompressionConfig) and self.model_dump() == other.model_dump()
 
     __hash__ = None
+
+
+class DenseSparsityConfig(SparsityCompressionConfig):
+    """config/dense.py:26-43: sparse tensors stored as they are"""
+
+    def __init__(self, format: str = CompressionFormat.dense.value, **kwargs):
+        super().__init__(format=format, **kwargs)
+
+
+class BitmaskConfig(SparsityCompressionConfig):
+    """config/sparse_bitmask.py:26-40"""
+
+    def __init__(self, format: str = CompressionFormat.sparse_bitmask.value, **kwargs):
+        super().__init__(format=format, **kwargs)
+
+
+class Sparse24BitMaskConfig(SparsityCompressionConfig):
+    """config/sparse_24_bitmask.py:27-40: 2:4 by default"""
+
+    def __init__(self, format: str = CompressionFormat.sparse_24_bitmask.value,
+                 sparsity_structure: Optional[str] = SparsityStructure.TWO_FOUR.value, **kwargs):
+        super().__init__(format=format, sparsity_structure=sparsity_structure, **kwargs)
 
 
 def _quant_compression_format(input_args, weight_args, sparsity_structure=None) -> CompressionFormat:

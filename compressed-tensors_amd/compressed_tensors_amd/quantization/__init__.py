@@ -4,3 +4,4 @@ from .helpers import *  # noqa: F401,F403
 from .forward import *  # noqa: F401,F403
 from .initialize import *  # noqa: F401,F403
 from .mxfp4_utils import *  # noqa: F401,F403
+from .lifecycle import *  # noqa: F401,F403

@@ -27,6 +27,7 @@ __all__ = [
     "dequantize",
     "fake_quantize",
     "forward_quantize",
+    "wrap_module_forward_quantized",
     "build_qparams",
 ]
 
@@ -405,3 +406,48 @@ def forward_quantize(
         x=value, scale=scale, zero_point=zero_point, args=args, g_idx=g_idx,
         global_scale=global_scale,
     )
+
+
+def wrap_module_forward_quantized(module: torch.nn.Module, scheme) -> None:
+    """replace `module.forward` by one that fake-quantizes what the scheme names around the
+    original call (forward.py:355-412): the input, the weight (put back afterwards; not for
+    a compressed module, whose weight already lies on the grid) and the output (left alone
+    while a static output scheme is being calibrated).  `module.quantization_enabled = False`
+    switches all of it off."""
+    from functools import wraps
+
+    original = module.forward.__func__ if hasattr(module.forward, "__func__") else module.forward.func
+    # a module that is initialized again is wrapped once, around the forward it came with
+    original = getattr(original, "_wraps_forward", original)
+
+    @wraps(original)
+    def wrapped_forward(self, *args, **kwargs):
+        call = original.__get__(module, module.__class__)
+        if not getattr(module, "quantization_enabled", True):
+            return call(*args, **kwargs)
+        status = getattr(module, "quantization_status", None)
+        status = str(getattr(status, "value", status))
+        compressed = status == "compressed"
+        input_ = args[0]
+        if scheme.input_activations is not None:
+            input_ = forward_quantize(module, input_, "input", scheme.input_activations)
+        # (a CompressedLinear's weight was decompressed from codes: it lies on the grid already,
+        # and its zero points may still be in their packed form)
+        swap_weight = scheme.weights is not None and not compressed and not hasattr(module, "compressor")
+        if swap_weight:
+            kept = self.weight.data
+            self.weight.data = forward_quantize(module, self.weight.data, "weight", scheme.weights)
+        try:
+            output = call(input_, *args[1:], **kwargs)
+        finally:
+            if swap_weight:
+                self.weight.data = kept
+        if scheme.output_activations is not None:
+            if status == "calibration" and not scheme.output_activations.dynamic:
+                return output
+            output = forward_quantize(module, output, "output", scheme.output_activations)
+        return output
+
+    wrapped_forward._wraps_forward = original
+    setattr(module, "forward", wrapped_forward.__get__(module, module.__class__))
+

@@ -150,6 +150,10 @@ def initialize_module_for_quantization(
     if scheme.output_activations is not None:
         initialize_qparams(module, "output", scheme.output_activations, weight.shape[:-1],
                            weight.dtype, force_zero_point)
+    # forward calls act on the scheme from here on (forward.py:355-412)
+    from compressed_tensors_amd.quantization.forward import wrap_module_forward_quantized
+
+    wrap_module_forward_quantized(module, scheme)
     module.quantization_scheme = scheme
     module.quantization_status = QuantizationStatus.INITIALIZED
 

@@ -628,3 +628,57 @@ def test_module_pathway_on_a_seeded_mixture(fmt, gpu):
         single = comp.decompress_weight(compressed_data=data, quantization_args=m.quantization_scheme.weights)
         assert_bit_equal(m.weight.data, single.cpu(), f"{name} decompressed")
         assert m.weight.dtype == single.dtype
+
+
+def test_wrapped_forward_and_in_place_weight_compression(gpu):
+    """a module under apply_quantization_config: forward fake-quantizes the input (dynamic per
+    token), the weight (put back afterwards) and the output as the scheme says (forward.py:355-412),
+    bit for bit what fake_quantize gives on the same tensors; compress_quantized_weights leaves
+    the oracle's int8 codes in the weight (compressed.py:33-73)"""
+    from compressed_tensors_amd.quantization import (
+        QuantizationArgs, QuantizationConfig, QuantizationScheme, apply_quantization_config,
+        compress_quantized_weights, fake_quantize, observe_weight_qparams)
+    from compressed_tensors_amd.quantization.helpers import compute_dynamic_scales_and_zp
+    from oracle import quant as oq
+
+    announce("wrapped forward")
+    torch.manual_seed(3)
+    w_spec = dict(num_bits=4, type="int", strategy="group", group_size=16, symmetric=False)
+    i_spec = dict(num_bits=8, type="int", strategy="token", dynamic=True, symmetric=True)
+    o_spec = dict(num_bits=8, type="float", strategy="tensor", dynamic=False, symmetric=True)
+    scheme = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(**w_spec),
+                                input_activations=QuantizationArgs(**i_spec),
+                                output_activations=QuantizationArgs(**o_spec))
+    model = torch.nn.Sequential(torch.nn.Linear(64, 32, bias=True)).to(torch.bfloat16).to(gpu)
+    apply_quantization_config(model, QuantizationConfig(config_groups={"g": scheme}, quantization_status="frozen"))
+    lin = model[0]
+    w = lin.weight.data.clone()
+    scale, zp = observe_weight_qparams(w, scheme.weights)
+    lin.weight_scale.data.copy_(scale)
+    lin.weight_zero_point.data.copy_(zp)
+    lin.output_scale.data.fill_(0.01)
+    x = torch.randn(2, 5, 64, device=gpu).bfloat16()
+    got = model(x)
+    s, z = compute_dynamic_scales_and_zp(x, scheme.input_activations)
+    xq = fake_quantize(x, s, z, scheme.input_activations)
+    wq = fake_quantize(w, scale, zp, scheme.weights)
+    out = torch.nn.functional.linear(xq, wq, lin.bias)
+    want = fake_quantize(out, lin.output_scale.data, lin.output_zero_point.data, scheme.output_activations)
+    assert_bit_equal(got, want.cpu(), "forward")
+    assert_bit_equal(lin.weight.data, w.cpu(), "the weight is put back")
+    # the pieces against the oracle
+    assert_bit_equal(wq, oq.fake_quantize(w.cpu(), scale.cpu(), zp.cpu(), oq._Args(**w_spec)), "weight on the grid")
+    # calibration of a static output scheme leaves the output alone
+    lin.quantization_status = "calibration"
+    assert_bit_equal(model(x), out.cpu(), "calibration")
+    lin.quantization_status = "frozen"
+    lin.quantization_enabled = False
+    assert_bit_equal(model(x), torch.nn.functional.linear(x, w, lin.bias).cpu(), "disabled")
+    lin.quantization_enabled = True
+    model.apply(compress_quantized_weights)
+    assert lin.weight.dtype == torch.int8 and not lin.weight.requires_grad
+    assert str(getattr(lin.quantization_status, "value", lin.quantization_status)) == "compressed"
+    assert_bit_equal(lin.weight.data, oq.quantize(w.cpu(), scale.cpu(), zp.cpu(), oq._Args(**w_spec), dtype=torch.int8),
+                     "int8 codes")
+    model.apply(compress_quantized_weights)  # a second time changes nothing
+    assert lin.weight.dtype == torch.int8
