@@ -27,6 +27,10 @@ __all__ = [
     "get_weight_mappings",
     "get_nested_weight_mappings",
     "get_quantization_parameter_to_path_mapping",
+    "get_safetensors_folder",
+    "match_param_name",
+    "is_quantization_param",
+    "get_nested_mappings_from_state_dict",
     "iter_tensors",
     "CheckpointReader",
     "save_file",
@@ -100,6 +104,40 @@ def get_nested_weight_mappings(model_path: str, params_to_nest: Iterable[str],
         if return_unmatched_params and not matched:
             unmatched[key] = location
     return (nested, unmatched) if return_unmatched_params else nested
+
+
+def get_safetensors_folder(pretrained_model_name_or_path: str, cache_dir: Optional[str] = None) -> str:
+    """the folder that holds a model's safetensors files: a local path as it is, anything else
+    through transformers' cache (utils/safetensors_load.py:42-81)"""
+    path = str(pretrained_model_name_or_path)
+    if os.path.exists(path):
+        return os.path.abspath(path)
+    from transformers.utils import cached_file
+
+    for name in (SAFE_WEIGHTS_NAME, SAFE_WEIGHTS_INDEX_NAME):
+        found = cached_file(path, name, cache_dir=cache_dir, _raise_exceptions_for_missing_entries=False)
+        if found is not None:
+            return os.path.split(found)[0]
+    raise ValueError(f"Could not locate safetensors weight or index file from {path}.")
+
+
+def match_param_name(full_name: str, param_name: str) -> Optional[str]:
+    """the module path of `full_name` if it ends in `.param_name` (utils/safetensors_load.py:99-112)"""
+    return _module_of(full_name, param_name)
+
+
+def is_quantization_param(name: str) -> bool:
+    """utils/safetensors_load.py:308-322"""
+    return name.endswith(("_scale", "zero_point", "g_idx"))
+
+
+def get_nested_mappings_from_state_dict(state_dict, params_to_nest: Iterable[str],
+                                        return_unmatched_params: bool = False):
+    """module path -> {compression parameter -> tensor} for a state dict in memory
+    (utils/safetensors_load.py:251-305)"""
+    from compressed_tensors_amd.utils.helpers import nest_state_dict
+
+    return nest_state_dict(state_dict, tuple(params_to_nest), return_unmatched_params=return_unmatched_params)
 
 
 def get_quantization_parameter_to_path_mapping(model_path: str) -> Dict[str, str]:

@@ -145,3 +145,21 @@ def test_update_config_and_back(tmp_path):
     os.remove(tmp_path / "config.json")
     ModelCompressor().update_config(str(tmp_path))
     assert not (tmp_path / "config.json").exists()
+
+
+def test_helper_names_of_the_reference(tmp_path):
+    """utils/safetensors_load.py: match_param_name :99-112, is_quantization_param :308-322,
+    get_nested_mappings_from_state_dict :251-305, get_safetensors_folder :42-81 (local paths)"""
+    from compressed_tensors_amd.utils.safetensors_io import (
+        get_nested_mappings_from_state_dict, get_safetensors_folder, is_quantization_param, match_param_name)
+
+    assert match_param_name("model.layers.0.q_proj.weight_scale", "weight_scale") == "model.layers.0.q_proj"
+    assert match_param_name("model.layers.0.q_proj.weight_scale", "weight") is None
+    assert match_param_name("weight_scale", "weight_scale") is None
+    assert [is_quantization_param(n) for n in ("a.weight_scale", "a.input_zero_point", "a.weight_g_idx", "a.weight",
+                                                "a.bitmask")] == [True, True, True, False, False]
+    state = {"a.weight": torch.ones(1), "a.weight_scale": torch.ones(1), "b.bias": torch.ones(1)}
+    nested, rest = get_nested_mappings_from_state_dict(state, ["weight", "weight_scale"], return_unmatched_params=True)
+    assert set(nested) == {"a"} and set(nested["a"]) == {"weight", "weight_scale"} and set(rest) == {"b.bias"}
+    assert get_nested_mappings_from_state_dict(state, ["bias"]) == {"b": {"bias": state["b.bias"]}}
+    assert get_safetensors_folder(str(tmp_path)) == str(tmp_path.resolve())
