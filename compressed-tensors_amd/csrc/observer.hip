@@ -194,7 +194,7 @@ observe_flat_kernel(const typename XT::raw* __restrict__ x, const float* gscale,
   for (int k = 0; k < U; ++k) {
     // past the end: re-read the last vector (nothing is emitted for it)
     const int64_t v = v0 + k * 256;
-    a[k] = ldg<typename XT::raw, 8>(x + (v < nvec ? v : nvec - 1) * 8);
+    a[k] = ldg_nt<typename XT::raw, 8>(x + (v < nvec ? v : nvec - 1) * 8);  // read once
   }
   // The segments' results go through LDS so that the scale arithmetic and the
   // stores run on full wavefronts, one segment per lane, instead of on one lane
@@ -309,7 +309,7 @@ __global__ void __launch_bounds__(256) observe_flat_chain_kernel(const ObsChainT
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     const uint32_t v = v0 + k * 256;  // past the end: re-read the last vector (nothing is emitted for it)
-    a[k] = ldg<typename XT::raw, 8>(x + (int64_t)(v < nvec ? v : nvec - 1) * 8);
+    a[k] = ldg_nt<typename XT::raw, 8>(x + (int64_t)(v < nvec ? v : nvec - 1) * 8);
   }
   __shared__ float seg_lo[256 * U], seg_hi[256 * U];
 #pragma unroll
