@@ -12,7 +12,6 @@ on the GPU they live on.  Modules carry their scheme in `quantization_scheme`
 (set by `apply_quantization_scheme` below or by the caller).
 """
 import logging
-import re
 from typing import Dict, List, Optional, Set
 
 import torch
@@ -30,6 +29,7 @@ from compressed_tensors_amd.config import (
 from compressed_tensors_amd.compressors.quantized_base import own_parameters, swap_parameters
 from compressed_tensors_amd.quantization.quant_scheme import QuantizationConfig, QuantizationScheme
 from compressed_tensors_amd.utils.helpers import load_safetensors_state_dict, merge_names, nest_state_dict
+from compressed_tensors_amd.utils.match import match_named_modules
 
 __all__ = ["ModelCompressor", "map_module_to_scheme", "match_named_modules",
            "apply_quantization_scheme"]
@@ -71,23 +71,6 @@ def _set_plain(module: Module, name: str, value) -> None:
     """module.<name> = value for a value that is no parameter, buffer or module (without the
     checks Module.__setattr__ makes for those)"""
     object.__setattr__(module, name, value)
-
-
-def _matches(name: str, module: Module, target: str) -> bool:
-    if target.startswith("re:"):
-        return re.match(target[3:], name) is not None
-    return target == name or target == module.__class__.__name__
-
-
-def match_named_modules(model: Module, targets: Optional[List[str]],
-                        ignore: Optional[List[str]] = None):
-    """(name, module) pairs whose name or class matches a target and no ignore entry
-    (reference: utils/match.py:40-100; `re:` prefixes are regular expressions)."""
-    for name, module in model.named_modules():
-        if any(_matches(name, module, t) for t in (targets or [])) and not any(
-            _matches(name, module, t) for t in (ignore or [])
-        ):
-            yield name, module
 
 
 def apply_quantization_scheme(model: Module, config: QuantizationConfig) -> None:

@@ -86,9 +86,9 @@ def disable_quantization(module: Module) -> None:
 
 
 def _matching_targets(name: str, module: Module, targets):
-    from compressed_tensors_amd.compressors.model_compressor import _matches
+    from compressed_tensors_amd.utils.match import match_targets
 
-    return [t for t in targets if _matches(name, module, t)]
+    return match_targets(name, module, targets)
 
 
 def apply_quantization_config(model: Module, config: Optional[QuantizationConfig],

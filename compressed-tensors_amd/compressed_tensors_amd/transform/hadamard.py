@@ -37,6 +37,7 @@ from torch import Tensor
 from compressed_tensors_amd import _lib
 from compressed_tensors_amd.compressors.base import to_gpu
 from compressed_tensors_amd.registry import RegistryMixin
+from compressed_tensors_amd.utils.internal import InternalModule
 
 __all__ = [
     "is_pow2",
@@ -59,6 +60,7 @@ __all__ = [
     "HadamardFactory",
     "RandomHadamardFactory",
     "HadamardTransform",
+    "TransformBase",
 ]
 
 _FLOATS = (torch.float32, torch.float16, torch.bfloat16)
@@ -527,28 +529,85 @@ class TransformLocation(str, Enum):
         return self not in (TransformLocation.WEIGHT_INPUT, TransformLocation.WEIGHT_OUTPUT)
 
 
+def _torch_dtype(value) -> torch.dtype:
+    """a torch.dtype, or its name with or without the "torch." in front (utils/type.py:30-40)"""
+    if isinstance(value, torch.dtype):
+        return value
+    found = getattr(torch, str(value).removeprefix("torch."), None) if isinstance(value, str) else None
+    if not isinstance(found, torch.dtype):
+        raise ValueError(f"No such torch dtype `{value}`")
+    return found
+
+
+def _only_fields(cls, data: Dict, fields) -> None:
+    extra = set(data) - set(fields)
+    if extra:  # the reference's models forbid extra fields
+        raise ValueError(f"{cls.__name__}: unexpected field(s) {sorted(extra)}")
+
+
 class TransformArgs:
+    """how and where a transform is applied (transform/transform_args.py:56-85)"""
+    _FIELDS = ("targets", "location", "inverse", "ignore")
+
     def __init__(self, targets: List[str], location, inverse: bool = False,
                  ignore: Optional[List[str]] = None):
         self.targets = [targets] if isinstance(targets, str) else list(targets)
         self.location = TransformLocation(location)
         self.inverse = bool(inverse)
-        self.ignore = list(ignore or [])
+        self.ignore = [ignore] if isinstance(ignore, str) else list(ignore or [])
 
     def is_online(self) -> bool:
         return self.location.is_online()
 
+    def model_dump(self) -> Dict:
+        return {"targets": list(self.targets), "location": self.location.value,
+                "inverse": self.inverse, "ignore": list(self.ignore)}
+
+    @classmethod
+    def model_validate(cls, data) -> "TransformArgs":
+        if isinstance(data, cls):
+            return data
+        _only_fields(cls, data, cls._FIELDS)
+        return cls(**data)
+
+    def __eq__(self, other) -> bool:
+        return isinstance(other, TransformArgs) and self.model_dump() == other.model_dump()
+
+    def __repr__(self) -> str:
+        return f"TransformArgs({self.model_dump()})"
+
 
 class TransformScheme:
+    """a transform type and the places of a model it goes to (transform/transform_scheme.py:25-55)"""
+    _FIELDS = ("type", "apply", "randomize", "requires_grad", "head_dim", "precision")
+
     def __init__(self, type: str, apply: Optional[List[TransformArgs]] = None,
                  randomize: bool = False, requires_grad: bool = False,
-                 head_dim: Optional[int] = None, precision: torch.dtype = torch.float32):
+                 head_dim: Optional[int] = None, precision=torch.float32):
         self.type = type
-        self.apply = list(apply or [])
-        self.randomize = randomize
-        self.requires_grad = requires_grad
+        self.apply = [TransformArgs.model_validate(a) for a in (apply or [])]
+        self.randomize = bool(randomize)
+        self.requires_grad = bool(requires_grad)
         self.head_dim = head_dim
-        self.precision = precision
+        self.precision = _torch_dtype(precision)
+
+    def model_dump(self) -> Dict:
+        return {"type": self.type, "apply": [a.model_dump() for a in self.apply],
+                "randomize": self.randomize, "requires_grad": self.requires_grad,
+                "head_dim": self.head_dim, "precision": str(self.precision)}
+
+    @classmethod
+    def model_validate(cls, data) -> "TransformScheme":
+        if isinstance(data, cls):
+            return data
+        _only_fields(cls, data, cls._FIELDS)
+        return cls(**data)
+
+    def __eq__(self, other) -> bool:
+        return isinstance(other, TransformScheme) and self.model_dump() == other.model_dump()
+
+    def __repr__(self) -> str:
+        return f"TransformScheme({self.model_dump()})"
 
 
 def _kernel_takes(value: Tensor, matrix: Tensor) -> bool:
@@ -656,7 +715,36 @@ def _matrix_core_split(lib, k: int, b: int, code: int) -> Optional[Tuple[int, in
     return None
 
 
-class HadamardTransform(torch.nn.Module):
+class TransformBase(InternalModule):
+    """A transform as applied at one location of one kind of module
+    (transform/factory/base.py:196-213)."""
+
+    args: TransformArgs
+
+    def forward(self, value: Tensor) -> Tensor:
+        raise NotImplementedError()
+
+    def forward_many(self, values: List[Tensor]) -> List[Tensor]:
+        """forward on every tensor of a list (the weights of the modules one TransformArgs
+        entry names); kernels that take several tensors per launch override it"""
+        return [self.forward(v) for v in values]
+
+    def same_as(self):
+        """a key that two transforms share if forward does the same in both"""
+        return id(self)
+
+    def right_inverse(self, value: Tensor) -> Tensor:
+        self.args.inverse = not self.args.inverse
+        try:
+            return self.forward(value)
+        finally:
+            self.args.inverse = not self.args.inverse
+
+    def __repr__(self) -> str:
+        return f"{type(self).__name__}(inverse={self.args.inverse})"
+
+
+class HadamardTransform(TransformBase):
     """W = diag(signs) * H, optionally row/column permuted by `perm` (W[perm][:, perm]),
     where H = Sylvester(size) or, with `block` = a known K x K Hadamard matrix,
     H = block^T (x) Sylvester(size / K) as the reference builds it for sizes that are not
@@ -698,6 +786,66 @@ class HadamardTransform(torch.nn.Module):
             h = self.signs.to(self.precision).cpu().unsqueeze(1) * h
         return h
 
+    def _orientation(self) -> Tuple[bool, bool]:
+        left, transposed = _orientation(self.args.location, self.module_type)
+        if self.args.inverse:
+            transposed = not transposed
+        if left:
+            # M @ V = (V^T @ M^T)^T: the transposed value is multiplied by the other orientation
+            transposed = not transposed
+        return left, transposed
+
+    def same_as(self):
+        return (self.size, id(self.signs), id(self.perm), id(self.block), self.args.location,
+                self.args.inverse, self.module_type, self.precision)
+
+    def forward_many(self, values: List[Tensor]) -> List[Tensor]:
+        """Sylvester sizes the butterfly or matrix-core kernels take: all tensors in
+        launches of 8 (ctmi_hadamard_apply_many); anything else one by one"""
+        n = self.size
+        if (len(values) < 2 or self.block is not None or self.perm is not None
+                or len({v.dtype for v in values}) != 1 or values[0].dtype not in _FLOATS
+                or not hadamard_kernel_exists(n, values[0].dtype)):
+            return [self.forward(v) for v in values]
+        left, transposed = self._orientation()
+        xs = [to_gpu(v) for v in values]
+        if left:
+            xs = [x.transpose(0, -1) for x in xs]
+        s_in, s_out = (None, self.signs) if transposed else (self.signs, None)
+        ys = hadamard_apply_many(xs, n, sign_in=s_in, sign_out=s_out)
+        return [y.transpose(0, -1).contiguous() for y in ys] if left else ys
+
+    def _save_to_state_dict(self, destination, prefix, keep_vars):
+        """the entries the reference's transform holds as parameters: the dense matrix and
+        the permutation (transform/factory/hadamard.py:84-101)"""
+        super()._save_to_state_dict(destination, prefix, keep_vars)
+        destination[prefix + "weight"] = self.weight
+        if self.perm is not None:
+            destination[prefix + "perm"] = self.perm
+
+    def _load_from_state_dict(self, state_dict, prefix, local_metadata, strict, missing_keys,
+                              unexpected_keys, error_msgs):
+        """a saved dense matrix must be the one this transform stands for; its signs (the
+        first column of diag(signs) H) and the permutation are taken over"""
+        weight = state_dict.pop(prefix + "weight", None)
+        perm = state_dict.pop(prefix + "perm", None)
+        if perm is not None:
+            self.perm = perm.to(torch.int64).cpu()
+        if weight is not None:
+            if tuple(weight.shape) != (self.size, self.size):
+                error_msgs.append(f"{prefix}weight: {tuple(weight.shape)} is not {self.size} x {self.size}")
+            else:
+                # row i of diag(signs) H is signs[i] times row i of H, whose first entry is +-1
+                had_signs, self.signs = self.signs, None
+                unsigned_first = self.weight[:, 0].to(torch.float64)
+                saved = weight.detach().to("cpu", torch.float64)
+                self.signs = (saved[:, 0] * unsigned_first).to(torch.float32)
+                if not torch.equal(self.weight.to(torch.float64), saved):
+                    self.signs = had_signs
+                    error_msgs.append(f"{prefix}weight is not a sign-scaled Hadamard matrix of this construction")
+        super()._load_from_state_dict(state_dict, prefix, local_metadata, strict, missing_keys,
+                                      unexpected_keys, error_msgs)
+
     def _explicit_factor(self, h: int, transposed: bool, device) -> Tensor:
         """fp32 [h, h] factor w of W = diag(q) (w (x) S) for x W, of W^T for x W^T"""
         key = (str(device), transposed)
@@ -711,12 +859,7 @@ class HadamardTransform(torch.nn.Module):
         return self._factor[key]
 
     def forward(self, value: Tensor) -> Tensor:
-        left, transposed = _orientation(self.args.location, self.module_type)
-        if self.args.inverse:
-            transposed = not transposed
-        if left:
-            # M @ V = (V^T @ M^T)^T: the transposed value is multiplied by the other orientation
-            transposed = not transposed
+        left, transposed = self._orientation()
         value = to_gpu(value)
         n = self.size
         lib = _lib.load()
@@ -790,8 +933,8 @@ class HadamardTransform(torch.nn.Module):
 
 
 class TransformFactory(RegistryMixin):
-    """name -> factory registry with the reference's `from_scheme` entry
-    (transform/factory/base.py:53-92); module hooking is left to the caller."""
+    """name -> factory registry with the reference's `from_scheme` entry, and the
+    application of a scheme to a model (transform/factory/base.py:53-193)."""
 
     def __init__(self, name: str, scheme: TransformScheme, seed: Optional[int] = None):
         self.name = name
@@ -803,6 +946,89 @@ class TransformFactory(RegistryMixin):
     @classmethod
     def from_scheme(cls, scheme: TransformScheme, **kwargs):
         return cls.get_value_from_registry(scheme.type)(scheme=scheme, **kwargs)
+
+    def create_transform(self, module: torch.nn.Module, args: TransformArgs) -> "TransformBase":
+        raise NotImplementedError()
+
+    def apply_to_model(self, model: torch.nn.Module, use_tqdm: bool = True) -> None:
+        """create the scheme's transforms and put them into the model
+        (transform/factory/base.py:94-110).  The entries of `scheme.apply` are taken in order;
+        the weights one entry names are rotated together, several tensors per launch."""
+        from compressed_tensors_amd.utils.match import match_named_modules
+
+        entries = [(arg, [m for _, m in match_named_modules(model, arg.targets, arg.ignore)])
+                   for arg in self.scheme.apply]
+        bar = None
+        if use_tqdm:
+            import tqdm
+
+            bar = tqdm.tqdm(total=sum(len(ms) for _, ms in entries), desc=f"Applying {self.name} transforms")
+        for arg, modules in entries:
+            if arg.location in (TransformLocation.WEIGHT_INPUT, TransformLocation.WEIGHT_OUTPUT):
+                self._fuse_into_weights(modules, arg)
+            else:
+                for module in modules:
+                    self._apply_to_module(model, module, arg)
+            if bar is not None:
+                bar.update(len(modules))
+        if bar is not None:
+            bar.close()
+
+    def _fuse_into_weights(self, modules: List[torch.nn.Module], args: TransformArgs) -> None:
+        """weight <- transform(weight) for every module (transform/factory/base.py:143-160);
+        modules whose transforms are the same (size, signs, permutation) and whose weights
+        share a dtype go through forward_many"""
+        if self.scheme.requires_grad:
+            raise NotImplementedError(
+                "transforms that are trained (requires_grad) are not supported: the kernels "
+                "have no backward")
+        groups: Dict[tuple, List] = {}
+        for module in modules:
+            assert hasattr(module, "weight")
+            transform = self.create_transform(module, args)
+            key = (transform.same_as(), module.weight.dtype, str(module.weight.device))
+            groups.setdefault(key, []).append((module, transform))
+        with torch.no_grad():
+            for members in groups.values():
+                outs = members[0][1].forward_many([m.weight.data for m, _ in members])
+                for (module, _), out in zip(members, outs):
+                    module.weight.data = out.to(device=module.weight.device, dtype=module.weight.dtype)
+
+    def _apply_to_module(self, model: torch.nn.Module, module: torch.nn.Module,
+                         args: TransformArgs) -> None:
+        """one transform at one module: weights are rotated on the spot, the other locations
+        get the transform as a submodule `<name>_<location>` and a hook that calls it
+        (transform/factory/base.py:112-193)"""
+        location = TransformLocation(args.location)
+        if location in (TransformLocation.WEIGHT_INPUT, TransformLocation.WEIGHT_OUTPUT):
+            self._fuse_into_weights([module], args)
+            return
+        transform = self.create_transform(module, args)
+        module.register_module(f"{self.name}_{location.value}", transform)
+        if location == TransformLocation.INPUT:
+            module.register_forward_pre_hook(
+                lambda _, inputs: transform(inputs[0]).to(inputs[0].device), prepend=True)
+        elif location == TransformLocation.OUTPUT:
+            module.register_forward_hook(lambda _, _inputs, output: transform(output).to(output.device))
+        elif location in (TransformLocation.Q_ATTN, TransformLocation.K_CACHE):
+            from transformers import PreTrainedModel
+
+            from compressed_tensors_amd.modeling import (initialize_hooked_attention,
+                                                         initialize_hooked_kv_cache,
+                                                         register_key_hook, register_query_hook)
+
+            if not isinstance(model, PreTrainedModel):
+                raise ValueError(f"Cannot hook attention of model: {model}")
+            if location == TransformLocation.Q_ATTN:
+                initialize_hooked_attention(model, module)
+                register_query_hook(
+                    module, lambda _, query_states: transform(query_states).to(query_states.device))
+            else:
+                initialize_hooked_kv_cache(model, module)
+                register_key_hook(
+                    module, lambda _, key_states: transform(key_states).to(key_states.device))
+        else:
+            raise NotImplementedError()
 
 
 def _transform_size(module: torch.nn.Module, location: TransformLocation,

@@ -1,0 +1,244 @@
+"""GPU: a transform configuration applied to a model (reference:
+tests/test_transform/factory/test_correctness.py, test_serialization.py).  Weights rotated
+several per launch are compared, bit for bit, with the one-tensor call and, within one ulp,
+with the oracle's fp64 product by the explicit matrix; a transform and its inverse at two
+places of a model leave the model's output where it was."""
+import pytest
+import torch
+
+from gpu_util import announce, assert_bit_equal
+from oracle import hadamard as oh
+
+pytestmark = pytest.mark.gpu
+
+
+class Stack(torch.nn.Module):
+    def __init__(self, *sizes, dtype=torch.float32):
+        super().__init__()
+        self.fcs = torch.nn.ModuleList(
+            [torch.nn.Linear(a, b, bias=False, dtype=dtype) for a, b in zip(sizes, sizes[1:])])
+
+    def forward(self, x):
+        for fc in self.fcs:
+            x = fc(x)
+        return x
+
+
+def _ulp(t):
+    bits = {torch.bfloat16: 8, torch.float16: 11, torch.float32: 24}[t.dtype]
+    mag = t.double().abs().clamp_min(2.0 ** -126)
+    return torch.exp2(torch.floor(torch.log2(mag)) - (bits - 1))
+
+
+@pytest.mark.parametrize("kind", ["hadamard", "random-hadamard", "random-matrix"])
+@pytest.mark.parametrize("randomize", [False, True])
+def test_a_transform_and_its_inverse_cancel_in_a_model(kind, randomize, gpu):
+    """test_correctness.py:94-121 (test_correctness_model), fp32 on the GPU: the output of
+    fcs[0] is transformed, the input weights of fcs[1] take the inverse; the input of fcs[2]
+    is transformed online, its input weights take the inverse"""
+    from compressed_tensors_amd.transform import (TransformArgs, TransformConfig, TransformScheme,
+                                                  apply_transform_config)
+
+    announce("transform model", kind, randomize)
+    torch.manual_seed(7)
+    model = Stack(64, 128, 256, 32).to(gpu)
+    x = torch.rand(5, 3, 64, device=gpu)
+    with torch.no_grad():
+        want = model(x)
+    config = TransformConfig(config_groups={"": TransformScheme(type=kind, randomize=randomize, apply=[
+        TransformArgs(targets="fcs.0", location="weight_output"),
+        TransformArgs(targets="fcs.1", location="weight_input", inverse=True),
+        TransformArgs(targets="fcs.2", location="input"),
+        TransformArgs(targets="fcs.2", location="weight_input", inverse=True),
+    ])})
+    apply_transform_config(model, config)
+    assert model.transform_config is config
+    # online transforms stay as submodules named after the scheme and the location; the ones
+    # multiplied into weights are gone
+    assert [n for n, _ in model.fcs[2].named_children()] == ["_input"]
+    assert [n for n, _ in model.fcs[0].named_children()] == []
+    with torch.no_grad():
+        got = model(x)
+    # a random matrix is not orthogonal: its condition number is what the tolerance pays for
+    tol = 1e-5 if kind != "random-matrix" else 5e-3
+    assert torch.allclose(want, got, atol=tol * float(want.abs().max().clamp_min(1.0)), rtol=0.0), \
+        float((want - got).abs().max())
+
+
+@pytest.mark.parametrize("location", ["weight_input", "weight_output"])
+def test_weights_of_one_entry_are_rotated_together(location, gpu, monkeypatch):
+    """The modules one TransformArgs entry names go through the many-tensor entry point; what
+    it leaves in a weight is what the one-tensor call leaves there, and within one ulp of the
+    fp64 product with the explicit matrix (factory/base.py:143-160, factory/hadamard.py:103-121)"""
+    import compressed_tensors_amd.transform.hadamard as th
+    from compressed_tensors_amd.transform import TransformArgs, TransformFactory, TransformScheme
+
+    announce("transform weights together", location)
+    torch.manual_seed(3)
+    model = Stack(*([256] * 12), dtype=torch.bfloat16).to(gpu)
+    model.fcs.append(torch.nn.Linear(256, 512, bias=False, dtype=torch.bfloat16, device=gpu)
+                     if location == "weight_input" else
+                     torch.nn.Linear(512, 256, bias=False, dtype=torch.bfloat16, device=gpu))
+    before = [fc.weight.detach().clone() for fc in model.fcs]
+    calls = []
+    real = th.hadamard_apply_many
+    monkeypatch.setattr(th, "hadamard_apply_many",
+                        lambda values, *a, **k: calls.append(len(values)) or real(values, *a, **k))
+    scheme = TransformScheme(type="random-hadamard", head_dim=128,
+                             apply=[TransformArgs(targets="Linear", location=location)])
+    factory = TransformFactory.from_scheme(scheme, name="R", seed=5)
+    factory.apply_to_model(model, use_tqdm=False)
+    assert calls == [len(model.fcs)], calls  # one call for all 12 weights
+    tfm = factory.create_transform(model.fcs[0], scheme.apply[0])
+    w64 = tfm.weight.double()
+    for fc, old in zip(model.fcs, before):
+        assert fc.weight.dtype == torch.bfloat16 and fc.weight.shape == old.shape
+        assert_bit_equal(fc.weight.data, tfm(old), "many-tensor launch against the one-tensor call")
+        want = oh.hadamard_forward(w64, old.cpu(), location, torch.nn.Linear, False, None)
+        err = (fc.weight.detach().cpu().double() - want.double()).abs()
+        tol = _ulp(want) + 2.0 ** -21 * want.double().abs().amax(-1, keepdim=True)
+        assert bool((err <= tol).all()), float((err / tol).max())
+
+
+def test_online_transform_is_saved_with_the_matrix_the_reference_holds(gpu):
+    """the state dict of a model with an online transform names `<scheme>_<location>.weight`
+    (and `.perm`), the dense matrix (factory/hadamard.py:84-101); loading it into a transform
+    built from another seed makes that one the same"""
+    from compressed_tensors_amd.transform import TransformArgs, TransformFactory, TransformScheme
+
+    announce("transform state dict")
+    model = Stack(128, 64).to(gpu)
+    scheme = TransformScheme(type="random-hadamard", randomize=True,
+                             apply=[TransformArgs(targets="Linear", location="input")])
+    TransformFactory.from_scheme(scheme, name="u", seed=1).apply_to_model(model, use_tqdm=False)
+    state = model.state_dict()
+    assert set(state) == {"fcs.0.weight", "fcs.0.u_input.weight", "fcs.0.u_input.perm"}
+    w = state["fcs.0.u_input.weight"]
+    assert w.shape == (128, 128) and w.dtype == torch.float32
+    assert torch.equal(w.abs(), torch.ones_like(w))
+    assert torch.equal(w @ w.T, 128 * torch.eye(128))
+    x = torch.randn(4, 128, device=gpu)
+    with torch.no_grad():
+        want = model(x)
+
+    other = Stack(128, 64).to(gpu)
+    TransformFactory.from_scheme(scheme, name="u", seed=2).apply_to_model(other, use_tqdm=False)
+    assert not torch.equal(other.fcs[0].u_input.weight, w)
+    other.load_state_dict(state)
+    assert torch.equal(other.fcs[0].u_input.weight, w)
+    assert torch.equal(other.fcs[0].u_input.perm, state["fcs.0.u_input.perm"])
+    with torch.no_grad():
+        assert_bit_equal(other(x), want, "the loaded transform")
+
+    bad = dict(state)
+    bad["fcs.0.u_input.weight"] = torch.rand(128, 128)
+    with pytest.raises(RuntimeError, match="not a sign-scaled Hadamard"):
+        other.load_state_dict(bad)
+
+
+def test_trained_transforms_are_refused(gpu):
+    from compressed_tensors_amd.transform import TransformArgs, TransformFactory, TransformScheme
+
+    model = Stack(128, 64).to(gpu)
+    scheme = TransformScheme(type="hadamard", requires_grad=True,
+                             apply=[TransformArgs(targets="Linear", location="weight_input")])
+    with pytest.raises(NotImplementedError, match="requires_grad"):
+        TransformFactory.from_scheme(scheme, name="t").apply_to_model(model, use_tqdm=False)
+
+
+def test_attention_locations_need_a_transformers_model(gpu):
+    from compressed_tensors_amd.transform import TransformArgs, TransformFactory, TransformScheme
+
+    model = Stack(128, 64).to(gpu)
+    scheme = TransformScheme(type="hadamard", head_dim=64,
+                             apply=[TransformArgs(targets="Linear", location="q_attn")])
+    with pytest.raises(ValueError, match="Cannot hook attention"):
+        TransformFactory.from_scheme(scheme, name="t").apply_to_model(model, use_tqdm=False)
+
+
+@pytest.mark.parametrize("kind", ["hadamard", "random-hadamard", "random-matrix"])
+@pytest.mark.parametrize("embed_loc", ["weight_output", "output"])
+@pytest.mark.parametrize("linear_loc", ["input", "weight_input"])
+def test_embedding_and_the_linear_behind_it(kind, embed_loc, linear_loc, gpu):
+    """test_correctness.py:62-91 (test_correctness_embedding)"""
+    from compressed_tensors_amd.transform import (TransformArgs, TransformConfig, TransformScheme,
+                                                  apply_transform_config)
+
+    announce("transform embedding", kind, embed_loc, linear_loc)
+    torch.manual_seed(11)
+    model = torch.nn.Sequential(torch.nn.Embedding(32, 64), torch.nn.Linear(64, 128, bias=False)).to(gpu)
+    ids = torch.randint(0, 32, (17, 5), device=gpu)
+    with torch.no_grad():
+        want = model(ids)
+    apply_transform_config(model, TransformConfig(config_groups={"": TransformScheme(type=kind, apply=[
+        TransformArgs(targets="Embedding", location=embed_loc),
+        TransformArgs(targets="Linear", location=linear_loc, inverse=True)])}))
+    with torch.no_grad():
+        got = model(ids)
+    tol = 1e-5 if kind != "random-matrix" else 5e-3
+    assert torch.allclose(want, got, atol=tol * float(want.abs().max().clamp_min(1.0)), rtol=0.0), \
+        float((want - got).abs().max())
+
+
+def _tiny_llama(gpu):
+    transformers = pytest.importorskip("transformers")
+    config = transformers.LlamaConfig(
+        hidden_size=64, intermediate_size=128, num_hidden_layers=2, num_attention_heads=4,
+        num_key_value_heads=2, vocab_size=96, max_position_embeddings=64)
+    torch.manual_seed(0)
+    return transformers.LlamaForCausalLM(config).eval().to(gpu)
+
+
+@pytest.mark.parametrize("kind", ["hadamard", "random-hadamard", "random-matrix"])
+def test_value_and_output_projections_per_head(kind, gpu):
+    """test_correctness.py:130-164 (test_correctness_attention_heads) on a two-layer Llama:
+    the values are rotated per head in v_proj's weight, o_proj's weight takes the inverse"""
+    from compressed_tensors_amd.transform import (TransformArgs, TransformConfig, TransformScheme,
+                                                  apply_transform_config)
+
+    announce("transform heads", kind)
+    model = _tiny_llama(gpu)
+    ids = (torch.arange(20, device=gpu).reshape(2, 10) * 7) % 96
+    with torch.no_grad():
+        want = model(ids).logits
+    v_before = model.model.layers[0].self_attn.v_proj.weight.detach().clone()
+    apply_transform_config(model, TransformConfig(config_groups={"R2": TransformScheme(
+        type=kind, head_dim=16, apply=[
+            TransformArgs(targets="re:.*v_proj$", location="weight_output"),
+            TransformArgs(targets="re:.*o_proj$", location="weight_input", inverse=True)])}))
+    assert not torch.equal(model.model.layers[0].self_attn.v_proj.weight, v_before)
+    with torch.no_grad():
+        got = model(ids).logits
+    tol = 1e-5 if kind != "random-matrix" else 5e-3
+    assert torch.allclose(want, got, atol=tol * float(want.abs().max().clamp_min(1.0)), rtol=0.0), \
+        float((want - got).abs().max())
+
+
+@pytest.mark.parametrize("kind", ["hadamard", "random-hadamard"])
+def test_queries_and_keys_rotated_alike(kind, gpu):
+    """test_correctness.py:167-200 (test_correctness_query_key_locations): the same orthogonal
+    matrix on the queries (after rope) and on the keys going into the cache leaves q k^T alone"""
+    from compressed_tensors_amd.modeling import IMPL_ATTR, KV_CACHE_ATTR
+    from compressed_tensors_amd.transform import (TransformArgs, TransformConfig, TransformScheme,
+                                                  apply_transform_config)
+
+    announce("transform q/k", kind)
+    model = _tiny_llama(gpu)
+    ids = (torch.arange(20, device=gpu).reshape(2, 10) * 7) % 96
+    with torch.no_grad():
+        want = model(ids).logits
+    apply_transform_config(model, TransformConfig(config_groups={"R3": TransformScheme(
+        type=kind, head_dim=16, apply=[
+            TransformArgs(targets="re:.*self_attn$", location="q_attn"),
+            TransformArgs(targets="re:.*self_attn$", location="k_cache")])}))
+    attn = model.model.layers[1].self_attn
+    assert hasattr(attn, IMPL_ATTR) and hasattr(attn, KV_CACHE_ATTR)
+    assert hasattr(attn, "R3_q_attn") and hasattr(attn, "R3_k_cache")
+    seen = []
+    real = attn.R3_q_attn.forward
+    attn.R3_q_attn.forward = lambda v: seen.append(tuple(v.shape)) or real(v)
+    with torch.no_grad():
+        got = model(ids).logits
+    assert seen == [(2, 4, 10, 16)]
+    assert torch.allclose(want, got, atol=1e-5 * float(want.abs().max().clamp_min(1.0)), rtol=0.0), \
+        float((want - got).abs().max())
