@@ -754,7 +754,8 @@ class HadamardTransform(TransformBase):
 
     def __init__(self, size: int, signs: Optional[Tensor], perm: Optional[Tensor],
                  scheme: TransformScheme, args: TransformArgs, module_type: type,
-                 precision: torch.dtype = torch.float32, block: Optional[Tensor] = None):
+                 precision: torch.dtype = torch.float32, block: Optional[Tensor] = None,
+                 dense: Optional[Dict] = None):
         super().__init__()
         if block is None and not is_pow2(size):
             raise ValueError("Cannot construct deterministic hadamard of size != 2^n")
@@ -772,10 +773,22 @@ class HadamardTransform(TransformBase):
         self.precision = precision
         self._scale = torch.tensor(size, dtype=torch.float64).sqrt()
         self._factor: Dict[tuple, Tensor] = {}
+        # dense matrices built on demand (state dicts, the library-GEMM path), shared by the
+        # transforms a factory makes for one size
+        self._dense: Dict[tuple, Tensor] = {} if dense is None else dense
+
+    _dynamic_tied_weights_keys: List[str] = ["weight", "perm"]
 
     @property
     def weight(self) -> Tensor:
-        """the dense matrix the reference would hold (before `perm`)"""
+        """the dense matrix the reference would hold (before `perm`); one tensor for all
+        transforms that share signs and precision"""
+        key = (id(self.signs), self.precision)
+        if key not in self._dense:
+            self._dense[key] = self._build_weight()
+        return self._dense[key]
+
+    def _build_weight(self) -> Tensor:
         if self.block is None:
             h = deterministic_hadamard_matrix(self.size, self.precision, torch.device("cpu"))
         else:
@@ -837,6 +850,7 @@ class HadamardTransform(TransformBase):
             else:
                 # row i of diag(signs) H is signs[i] times row i of H, whose first entry is +-1
                 had_signs, self.signs = self.signs, None
+                self._dense = {}  # its own matrices from here on
                 unsigned_first = self.weight[:, 0].to(torch.float64)
                 saved = weight.detach().to("cpu", torch.float64)
                 self.signs = (saved[:, 0] * unsigned_first).to(torch.float32)
@@ -1060,6 +1074,7 @@ class HadamardFactory(TransformFactory):
         self._signs: Dict[int, Optional[Tensor]] = {}
         self._blocks: Dict[int, Optional[Tensor]] = {}
         self._perms: Dict[int, Tensor] = {}
+        self._dense: Dict[int, Dict] = {}
 
     def _create_signs(self, size: int) -> Optional[Tensor]:
         return None
@@ -1079,7 +1094,8 @@ class HadamardFactory(TransformFactory):
             perm = self._perms[size]
         precision = self.scheme.precision if args.is_online() else torch.float64
         return HadamardTransform(size, self._signs[size], perm, self.scheme, args, type(module),
-                                 precision=precision, block=self._blocks[size])
+                                 precision=precision, block=self._blocks[size],
+                                 dense=self._dense.setdefault(size, {}))
 
 
 @TransformFactory.register("random-hadamard")

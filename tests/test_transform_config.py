@@ -162,3 +162,32 @@ def test_narrow_match():
     assert is_narrow_match(m, "re:layers.0.*", "layers.0") is True
     assert is_narrow_match(m, "re:layers.0.*", "layers.0.q_proj") is False  # the parent matches too
     assert is_narrow_match(m, ["Linear"], "layers.0.q_proj") is True
+
+
+@pytest.mark.parametrize("kind", ["hadamard", "random-hadamard"])
+@pytest.mark.parametrize("randomize", [True, False])
+def test_transforms_of_one_size_share_their_matrix(kind, randomize):
+    """tests/test_transform/factory/test_memory.py:33-66: online transforms of the same size
+    hold one matrix between them (here: none until a state dict asks, then one)"""
+    from collections import Counter
+
+    from compressed_tensors_amd.transform import TransformBase, apply_transform_config
+
+    sizes = (2, 2, 4, 4, 8, 8)
+    model = torch.nn.Sequential(*[torch.nn.Linear(a, b, bias=False) for a, b in zip(sizes, sizes[1:])])
+    apply_transform_config(model, TransformConfig(config_groups={"": TransformScheme(
+        type=kind, randomize=randomize, apply=[TransformArgs(targets="Linear", location="input"),
+                                               TransformArgs(targets="Linear", location="output")])}))
+    assert model.transform_config.config_groups[""].type == kind
+    transforms = [m for m in model.modules() if isinstance(m, TransformBase)]
+    assert len(transforms) == 10
+    count = Counter(id(t.weight) for t in transforms)
+    by_size = {t.weight.shape[0]: id(t.weight) for t in transforms}
+    assert len(count) == len(by_size) == 3
+    assert (count[by_size[2]], count[by_size[4]], count[by_size[8]]) == (3, 4, 3)
+    state = model.state_dict()
+    assert state["0._input.weight"].data_ptr() == state["1._input.weight"].data_ptr()
+    assert ("0._input.perm" in state) == randomize
+    for t in transforms:  # Hadamard: W W^T = n I
+        w = t.weight.double()
+        assert torch.equal(w @ w.T, w.shape[0] * torch.eye(w.shape[0], dtype=torch.float64))
