@@ -1146,6 +1146,48 @@ def api_level_format(torch, seed, steps, fmt, spec, bytes_per_element):
     }
 
 
+def api_level_transform(torch, seed, steps):
+    """TransformFactory.apply_to_model on the same module tree: a random-sign Hadamard rotation
+    of block size 128 multiplied into the input side of all 224 weights (bf16 in, bf16 out:
+    4 bytes per element), wall time incl. module matching and the parameter updates"""
+    from compressed_tensors_amd.transform import TransformArgs, TransformFactory, TransformScheme
+
+    dev = torch.device("cuda:0")
+    gen = torch.Generator(device=dev).manual_seed(seed)
+
+    class Layer(torch.nn.Module):
+        def __init__(self):
+            super().__init__()
+            for name, r, c in LLAMA3_8B_LAYER:
+                lin = torch.nn.Linear(1, 1, bias=False)
+                lin.in_features, lin.out_features = c, r
+                lin.weight.data = (torch.randn(r, c, generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+                lin.weight.requires_grad_(False)
+                setattr(self, name, lin)
+
+    model = torch.nn.Module()
+    model.layers = torch.nn.ModuleList([Layer() for _ in range(32)])
+    n = sum(m.weight.numel() for m in model.modules() if isinstance(m, torch.nn.Linear))
+    scheme = TransformScheme(type="random-hadamard", head_dim=128,
+                             apply=[TransformArgs(targets="Linear", location="weight_input")])
+    times = []
+    for it in range(steps + 1):  # first pass is the warm-up
+        factory = TransformFactory.from_scheme(scheme, name="R", seed=seed)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        factory.apply_to_model(model, use_tqdm=False)
+        torch.cuda.synchronize()
+        if it:
+            times.append(time.perf_counter() - t0)
+    t = statistics.median(times)
+    del model
+    torch.cuda.empty_cache()
+    return {"what": "TransformFactory.apply_to_model: random-hadamard, head_dim 128, weight_input of 224 "
+                    "torch.nn.Linear (bf16, Llama-3-8B shapes)",
+            "apply_to_model_ms": t * 1e3, "GBs": 4 * n / t / 1e9,
+            "frac_of_hbm_peak": 4 * n / t / 1e9 / HBM_PEAK_GBS, "passes": steps, "statistic": "median"}
+
+
 def api_level(torch, seed, steps):
     """the cost of the host mirror above the C ABI, next to the kernel-level figures: the
     headline's format at the top level of the result, the int8 / fp8 and nvfp4 formats under
@@ -1156,6 +1198,7 @@ def api_level(torch, seed, steps):
     out.update(api_level_format(torch, seed, steps, *API_FORMATS[0]))
     out["other_formats"] = {fmt: api_level_format(torch, seed, steps, fmt, spec, bpe)
                             for fmt, spec, bpe in API_FORMATS[1:]}
+    out["transform"] = api_level_transform(torch, seed, steps)
     return out
 
 
@@ -1209,6 +1252,8 @@ def short_line(out, details_path=None):
             line["api_level"]["state_dict_pathway"] = _sig(out["api_level"]["state_dict_pathway"]["frac_of_hbm_peak"], 3)
         for fmt, res in out["api_level"].get("other_formats", {}).items():
             line["api_level"][fmt] = _sig(res["frac_of_hbm_peak"], 3)
+        if "transform" in out["api_level"]:
+            line["api_level"]["hadamard128"] = _sig(out["api_level"]["transform"]["frac_of_hbm_peak"], 3)
     if details_path:
         line["details"] = os.path.relpath(details_path, ROOT)
     text = json.dumps(line, separators=(",", ":"))

@@ -447,12 +447,17 @@ def hadamard_apply_many(
     sign_out: Optional[Tensor] = None,
     matrix_t: Optional[Tensor] = None,
     kernel: Optional[str] = None,
+    in_place: bool = False,
 ) -> List[Tensor]:
     """hadamard_apply on several tensors of one dtype that share the matrix and the
     signs (the weights of a model under one transform scheme), from one call: the
-    kernels take 8 tensors per launch."""
+    kernels take 8 tensors per launch.  in_place: the tensors (contiguous, on the GPU)
+    are overwritten with their transforms and returned (a workgroup has read all of a
+    run of n elements before it writes any of it)."""
     if not values:
         return []
+    if in_place and not all(v.is_cuda and v.is_contiguous() for v in values):
+        raise ValueError("tensors transformed in place are contiguous tensors on the GPU")
     xs = [to_gpu(v).contiguous() for v in values]
     dtype, dev = xs[0].dtype, xs[0].device
     if dtype not in _FLOATS:
@@ -467,7 +472,7 @@ def hadamard_apply_many(
     if _butterfly(n, dtype, kernel, matrix_t):
         s_in, s_out = _sign(sign_in, dev), _sign(sign_out, dev)
         if _aligned(s_in, s_out, *xs) or kernel == "butterfly":
-            outs = [torch.empty_like(x) for x in xs]
+            outs = xs if in_place else [torch.empty_like(x) for x in xs]
             jobs = (_lib.HadamardJob * len(xs))()
             for job, x, out in zip(jobs, xs, outs):
                 job.x, job.out, job.numel = x.data_ptr(), out.data_ptr(), x.numel()
@@ -487,7 +492,7 @@ def hadamard_apply_many(
         ma_t = _sylvester_bf16(a, dev) if a > 1 else None
     s_in = None if sign_in is None else sign_in.to(device=dev, dtype=torch.float32).contiguous()
     s_out = None if sign_out is None else sign_out.to(device=dev, dtype=torch.float32).contiguous()
-    outs = [torch.empty_like(x) for x in xs]
+    outs = xs if in_place else [torch.empty_like(x) for x in xs]
     if matrix_t is None and _matrix_free(n, dtype, s_in, s_out, *xs, *outs):
         mb_t = None  # Sylvester's matrix of 128: the kernel that keeps no matrix in memory
     jobs = (_lib.HadamardJob * len(xs))()
@@ -724,9 +729,10 @@ class TransformBase(InternalModule):
     def forward(self, value: Tensor) -> Tensor:
         raise NotImplementedError()
 
-    def forward_many(self, values: List[Tensor]) -> List[Tensor]:
+    def forward_many(self, values: List[Tensor], in_place: bool = False) -> List[Tensor]:
         """forward on every tensor of a list (the weights of the modules one TransformArgs
-        entry names); kernels that take several tensors per launch override it"""
+        entry names); kernels that take several tensors per launch override it.  in_place:
+        the tensors may be overwritten with their transforms (and returned)"""
         return [self.forward(v) for v in values]
 
     def same_as(self):
@@ -812,11 +818,11 @@ class HadamardTransform(TransformBase):
         return (self.size, id(self.signs), id(self.perm), id(self.block), self.args.location,
                 self.args.inverse, self.module_type, self.precision)
 
-    def forward_many(self, values: List[Tensor]) -> List[Tensor]:
+    def forward_many(self, values: List[Tensor], in_place: bool = False) -> List[Tensor]:
         """Sylvester sizes the butterfly or matrix-core kernels take: all tensors in
         launches of 8 (ctmi_hadamard_apply_many); anything else one by one"""
         n = self.size
-        if (len(values) < 2 or self.block is not None or self.perm is not None
+        if (not values or self.block is not None or self.perm is not None
                 or len({v.dtype for v in values}) != 1 or values[0].dtype not in _FLOATS
                 or not hadamard_kernel_exists(n, values[0].dtype)):
             return [self.forward(v) for v in values]
@@ -825,7 +831,8 @@ class HadamardTransform(TransformBase):
         if left:
             xs = [x.transpose(0, -1) for x in xs]
         s_in, s_out = (None, self.signs) if transposed else (self.signs, None)
-        ys = hadamard_apply_many(xs, n, sign_in=s_in, sign_out=s_out)
+        in_place = in_place and not left and all(x.is_cuda and x.is_contiguous() for x in xs)
+        ys = hadamard_apply_many(xs, n, sign_in=s_in, sign_out=s_out, in_place=in_place)
         return [y.transpose(0, -1).contiguous() for y in ys] if left else ys
 
     def _save_to_state_dict(self, destination, prefix, keep_vars):
@@ -967,46 +974,82 @@ class TransformFactory(RegistryMixin):
     def apply_to_model(self, model: torch.nn.Module, use_tqdm: bool = True) -> None:
         """create the scheme's transforms and put them into the model
         (transform/factory/base.py:94-110).  The entries of `scheme.apply` are taken in order;
-        the weights one entry names are rotated together, several tensors per launch."""
+        the weights one entry names are rotated together, several tensors per launch, while
+        the walk over the model goes on."""
         from compressed_tensors_amd.utils.match import match_named_modules
 
-        entries = [(arg, [m for _, m in match_named_modules(model, arg.targets, arg.ignore)])
-                   for arg in self.scheme.apply]
         bar = None
         if use_tqdm:
             import tqdm
 
-            bar = tqdm.tqdm(total=sum(len(ms) for _, ms in entries), desc=f"Applying {self.name} transforms")
-        for arg, modules in entries:
+            bar = tqdm.tqdm(desc=f"Applying {self.name} transforms")
+        tick = (lambda k: None) if bar is None else bar.update
+        for arg in self.scheme.apply:
+            modules = (m for _, m in match_named_modules(model, arg.targets, arg.ignore))
             if arg.location in (TransformLocation.WEIGHT_INPUT, TransformLocation.WEIGHT_OUTPUT):
-                self._fuse_into_weights(modules, arg)
+                self._fuse_into_weights(modules, arg, tick)
             else:
                 for module in modules:
                     self._apply_to_module(model, module, arg)
-            if bar is not None:
-                bar.update(len(modules))
+                    tick(1)
         if bar is not None:
             bar.close()
 
-    def _fuse_into_weights(self, modules: List[torch.nn.Module], args: TransformArgs) -> None:
-        """weight <- transform(weight) for every module (transform/factory/base.py:143-160);
-        modules whose transforms are the same (size, signs, permutation) and whose weights
-        share a dtype go through forward_many"""
+    # modules per call of forward_many when weights are rotated: short calls first, so that
+    # the GPU starts while the host still walks the rest of the model
+    _FUSE_BATCHES = (8, 24, 64)
+
+    def _transform_key(self, module: torch.nn.Module, args: TransformArgs):
+        """modules with equal keys get equal transforms at `args` (one is created for all
+        of them); None: one transform per module"""
+        return None
+
+    def _fuse_into_weights(self, modules, args: TransformArgs, tick=lambda k: None) -> None:
+        """weight <- transform(weight) for every module (transform/factory/base.py:143-160).
+        Modules whose transforms are the same (size, signs, permutation) and whose weights
+        share dtype and device collect into calls of forward_many, in place where the kernel
+        allows it; a call goes out as soon as it is full."""
         if self.scheme.requires_grad:
             raise NotImplementedError(
                 "transforms that are trained (requires_grad) are not supported: the kernels "
                 "have no backward")
-        groups: Dict[tuple, List] = {}
+        made: Dict = {}     # _transform_key -> (transform, its same_as())
+        pending: Dict = {}  # (same_as, dtype, device) -> [transform, modules, weight addresses, calls made]
+
+        def flush(entry):
+            transform, batch = entry[0], entry[1]
+            with torch.no_grad():
+                outs = transform.forward_many([m.weight.data for m in batch], in_place=True)
+                for module, out in zip(batch, outs):
+                    w = module.weight
+                    if out.data_ptr() != w.data_ptr():
+                        w.data = out.to(device=w.device, dtype=w.dtype)
+            tick(len(batch))
+            entry[1], entry[2], entry[3] = [], set(), entry[3] + 1
+
         for module in modules:
             assert hasattr(module, "weight")
-            transform = self.create_transform(module, args)
-            key = (transform.same_as(), module.weight.dtype, str(module.weight.device))
-            groups.setdefault(key, []).append((module, transform))
-        with torch.no_grad():
-            for members in groups.values():
-                outs = members[0][1].forward_many([m.weight.data for m, _ in members])
-                for (module, _), out in zip(members, outs):
-                    module.weight.data = out.to(device=module.weight.device, dtype=module.weight.dtype)
+            key = self._transform_key(module, args)
+            if key is None or key not in made:
+                transform = self.create_transform(module, args)
+                found = (transform, transform.same_as())
+                if key is not None:
+                    made[key] = found
+            else:
+                found = made[key]
+            w = module.weight
+            entry = pending.setdefault((found[1], w.dtype, w.device), [found[0], [], set(), 0])
+            # a weight two modules share is transformed once per module, as in the reference's
+            # loop over modules: never twice in one call
+            if w.data_ptr() in entry[2]:
+                flush(entry)
+            entry[1].append(module)
+            entry[2].add(w.data_ptr())
+            if len(entry[1]) >= self._FUSE_BATCHES[min(entry[3], len(self._FUSE_BATCHES) - 1)]:
+                flush(entry)
+        for entry in pending.values():
+            if entry[1]:
+                flush(entry)
 
     def _apply_to_module(self, model: torch.nn.Module, module: torch.nn.Module,
                          args: TransformArgs) -> None:
@@ -1081,6 +1124,9 @@ class HadamardFactory(TransformFactory):
 
     def _create_block(self, size: int) -> Optional[Tensor]:
         return None
+
+    def _transform_key(self, module: torch.nn.Module, args: TransformArgs):
+        return (_transform_size(module, args.location, self.scheme.head_dim), type(module))
 
     def create_transform(self, module: torch.nn.Module, args: TransformArgs) -> HadamardTransform:
         size = _transform_size(module, args.location, self.scheme.head_dim)

@@ -63,6 +63,9 @@ class RandomMatrixFactory(TransformFactory):
     def _create_inverse(self, weight: Parameter) -> Parameter:
         return Parameter(high_precision_invert(weight.data).contiguous(), requires_grad=False)
 
+    def _transform_key(self, module: Module, args: TransformArgs):
+        return (_transform_size(module, args.location, self.scheme.head_dim), type(module))
+
     def create_transform(self, module: Module, args: TransformArgs) -> RandomMatrixTransform:
         size = _transform_size(module, args.location, self.scheme.head_dim)
         own = next(module.parameters(recurse=False), None)

@@ -37,14 +37,19 @@ def _name_matches(name: str, target: str, fused: Optional[Fused] = None) -> bool
     return name == target
 
 
+_CLASS_NAMES: Dict[type, frozenset] = {}
+
+
 def _class_matches(module: torch.nn.Module, target: str) -> bool:
     """match.py:315-336: any torch module class among the module's bases carries the name
     (vLLM's LinearBase counts as Linear)"""
-    for cls in type(module).__mro__:
-        if issubclass(cls, torch.nn.Module) and (
-                cls.__name__ == target or (target == "Linear" and cls.__name__ == "LinearBase")):
-            return True
-    return False
+    names = _CLASS_NAMES.get(type(module))
+    if names is None:
+        found = {c.__name__ for c in type(module).__mro__ if issubclass(c, torch.nn.Module)}
+        if "LinearBase" in found:
+            found.add("Linear")
+        names = _CLASS_NAMES[type(module)] = frozenset(found)
+    return target in names
 
 
 def _one(name: str, module: torch.nn.Module, target: str, fused: Optional[Fused]) -> bool:

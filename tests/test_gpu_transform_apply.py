@@ -75,7 +75,7 @@ def test_weights_of_one_entry_are_rotated_together(location, gpu, monkeypatch):
 
     announce("transform weights together", location)
     torch.manual_seed(3)
-    model = Stack(*([256] * 12), dtype=torch.bfloat16).to(gpu)
+    model = Stack(*([256] * 13), dtype=torch.bfloat16).to(gpu)
     model.fcs.append(torch.nn.Linear(256, 512, bias=False, dtype=torch.bfloat16, device=gpu)
                      if location == "weight_input" else
                      torch.nn.Linear(512, 256, bias=False, dtype=torch.bfloat16, device=gpu))
@@ -88,7 +88,7 @@ def test_weights_of_one_entry_are_rotated_together(location, gpu, monkeypatch):
                              apply=[TransformArgs(targets="Linear", location=location)])
     factory = TransformFactory.from_scheme(scheme, name="R", seed=5)
     factory.apply_to_model(model, use_tqdm=False)
-    assert calls == [len(model.fcs)], calls  # one call for all 12 weights
+    assert calls == [8, len(model.fcs) - 8], calls  # a short first call, the rest in the next
     tfm = factory.create_transform(model.fcs[0], scheme.apply[0])
     w64 = tfm.weight.double()
     for fc, old in zip(model.fcs, before):
@@ -242,3 +242,41 @@ def test_queries_and_keys_rotated_alike(kind, gpu):
     assert seen == [(2, 4, 10, 16)]
     assert torch.allclose(want, got, atol=1e-5 * float(want.abs().max().clamp_min(1.0)), rtol=0.0), \
         float((want - got).abs().max())
+
+
+def test_a_weight_two_modules_share_is_transformed_once_per_module(gpu):
+    """tied weights: the reference's loop over modules transforms the shared tensor at every
+    module that holds it (factory/base.py:143-160); two jobs of one launch never share it"""
+    from compressed_tensors_amd.transform import TransformArgs, TransformFactory, TransformScheme
+
+    announce("transform tied weights")
+    torch.manual_seed(2)
+    model = Stack(128, 128, 128, dtype=torch.bfloat16).to(gpu)
+    model.fcs[1].weight = model.fcs[0].weight
+    before = model.fcs[0].weight.detach().clone()
+    scheme = TransformScheme(type="hadamard", apply=[TransformArgs(targets="Linear", location="weight_input")])
+    factory = TransformFactory.from_scheme(scheme, name="t")
+    factory.apply_to_model(model, use_tqdm=False)
+    assert model.fcs[1].weight is model.fcs[0].weight
+    tfm = factory.create_transform(model.fcs[0], scheme.apply[0])
+    assert_bit_equal(model.fcs[0].weight.data, tfm(tfm(before)), "transformed at both modules")
+
+
+@pytest.mark.parametrize("n,dtype", [(128, torch.bfloat16), (4096, torch.bfloat16), (64, torch.float32),
+                                     (2048, torch.float16)])
+def test_many_tensors_in_place(n, dtype, gpu):
+    """the many-tensor call may overwrite its inputs: same bits as into fresh outputs"""
+    from compressed_tensors_amd.transform import hadamard_apply_many, random_hadamard_signs
+
+    announce("transform in place", n, dtype)
+    g = torch.Generator().manual_seed(n)
+    xs = [torch.randn(r, 2 * n, generator=g).to(dtype).to(gpu) for r in (48, 3, 130, 64, 16, 7, 33, 256, 5)]
+    q = random_hadamard_signs(n, g)
+    want = hadamard_apply_many(xs, n, sign_in=q)
+    ptrs = [x.data_ptr() for x in xs]
+    got = hadamard_apply_many(xs, n, sign_in=q, in_place=True)
+    assert [y.data_ptr() for y in got] == ptrs
+    for y, w in zip(got, want):
+        assert_bit_equal(y, w, f"in place, size {n}")
+    with pytest.raises(ValueError, match="in place"):
+        hadamard_apply_many([xs[0].t()], n, in_place=True)
