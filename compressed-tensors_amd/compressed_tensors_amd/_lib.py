@@ -190,6 +190,8 @@ SIGNATURES = {
         c_int32,
         [c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int64, _QP, c_int32, c_int32, c_void_p],
     ),
+    "ctmi_round_to_quantized_type": (
+        c_int32, [c_void_p, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p]),
     "ctmi_qdq_many": (c_int32, [POINTER(QdqJob), c_int64, c_int32, c_int32, c_void_p]),
     "ctmi_pack_to_int32": (
         c_int32,

@@ -15,6 +15,9 @@ __all__ = [
     "BitmaskConfig",
     "Sparse24BitMaskConfig",
     "QuantizationStatus",
+    "LIFECYCLE_ORDER",
+    "DEFAULT_QUANTIZATION_METHOD",
+    "DEFAULT_QUANTIZATION_FORMAT",
     "SPARSITY_CONFIG_NAME",
     "QUANTIZATION_CONFIG_NAME",
     "infer_and_set_per_module_quantization_format",
@@ -61,10 +64,52 @@ class SparsityStructure(Enum):
 
 
 class QuantizationStatus(str, Enum):
+    """where a quantized layer is in its life; statuses compare by that order, and any
+    status is at or beyond None (quantization/quant_config.py:39-99)"""
     INITIALIZED = "initialized"
     CALIBRATION = "calibration"
     FROZEN = "frozen"
     COMPRESSED = "compressed"
+
+    @classmethod
+    def lifecycle_order(cls) -> List["QuantizationStatus"]:
+        return list(cls)
+
+    def _rank_against(self, other):
+        if not isinstance(other, QuantizationStatus):
+            raise NotImplementedError
+        order = LIFECYCLE_ORDER
+        return order.index(self), order.index(other)
+
+    def __ge__(self, other):
+        if other is None:
+            return True
+        a, b = self._rank_against(other)
+        return a >= b
+
+    def __gt__(self, other):
+        if other is None:
+            return True
+        a, b = self._rank_against(other)
+        return a > b
+
+    def __lt__(self, other):
+        if other is None:
+            return False
+        a, b = self._rank_against(other)
+        return a < b
+
+    def __le__(self, other):
+        if other is None:
+            return False
+        a, b = self._rank_against(other)
+        return a <= b
+
+
+LIFECYCLE_ORDER = [QuantizationStatus.INITIALIZED, QuantizationStatus.CALIBRATION,
+                   QuantizationStatus.FROZEN, QuantizationStatus.COMPRESSED]
+DEFAULT_QUANTIZATION_METHOD = "compressed-tensors"
+DEFAULT_QUANTIZATION_FORMAT = "fakequant"
 
 
 class SparsityCompressionConfig:

@@ -36,10 +36,20 @@ __all__ = [
     "can_quantize",
     "get_torch_bit_depth",
     "strategy_cdiv",
+    "KV_CACHE_TARGETS",
+    "is_kv_cache_quant_scheme",
 ]
 
 _LOGGER = logging.getLogger(__name__)
 _FLOATS = (torch.float32, torch.float16, torch.bfloat16)
+
+KV_CACHE_TARGETS = ["re:.*self_attn$"]
+
+
+def is_kv_cache_quant_scheme(scheme) -> bool:
+    """does a scheme name the attention modules whose keys and values go into the cache
+    (helpers.py:394-411)"""
+    return any(target in KV_CACHE_TARGETS for target in scheme.targets)
 
 
 def is_fp4(quantization_args: QuantizationArgs) -> bool:

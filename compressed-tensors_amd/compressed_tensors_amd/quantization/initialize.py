@@ -91,7 +91,7 @@ def initialize_qparams(
             raise ValueError("Group quant requires at least 1 observed dimension")
         num_groups = strategy_cdiv(observed_shape[-1], args.group_size, strategy)
         expected_shape = (*observed_shape[:-1], num_groups)
-        if args.actorder == ActivationOrdering.GROUP.value:
+        if ActivationOrdering.GROUP == args.actorder:  # or its other name, dynamic
             _register(module, f"{base_name}_g_idx",
                       torch.full((observed_shape[-1],), -1, device=device, dtype=torch.int))
     elif strategy == QuantizationStrategy.BLOCK.value:

@@ -5,7 +5,10 @@ bitorder="little" (reference: utils/helpers.py:302-339) on the GPU; shard /
 combine helpers mirror utils/helpers.py:237-299; merge_names mirrors
 utils/safetensors_load.py:115-125.
 """
-from typing import List
+import contextlib
+import warnings
+from functools import wraps
+from typing import Any, Callable, Dict, List, Optional
 
 import torch
 
@@ -25,6 +28,14 @@ __all__ = [
     "get_num_attn_heads",
     "get_num_kv_heads",
     "get_head_dim",
+    "Aliasable",
+    "ParameterizedDefaultDict",
+    "patch_attr",
+    "deprecated",
+    "replace_module",
+    "fix_fsdp_module_name",
+    "is_compressed_tensors_config",
+    "infer_compressor_from_model_config",
 ]
 
 
@@ -197,3 +208,127 @@ def get_head_dim(config) -> int:
         return config.hidden_size // config.num_attention_heads
     raise ValueError("Cannot determine head_dim from config. Config must define either `head_dim` "
                      f"or both `hidden_size` and `num_attention_heads`. {config}")
+
+
+# ------------------------------------------------------------------ small host utilities
+FSDP_WRAPPER_NAME = "_fsdp_wrapped_module"
+
+
+def fix_fsdp_module_name(name: str) -> str:
+    """a module name without FSDP's wrapper component, wherever it sits (utils/helpers.py:80-90)"""
+    return name.replace(FSDP_WRAPPER_NAME + ".", "").replace("." + FSDP_WRAPPER_NAME, "")
+
+
+def replace_module(model: torch.nn.Module, name: str, new_module: torch.nn.Module) -> None:
+    """put `new_module` where the dotted `name` points (utils/helpers.py:118-127)"""
+    parent_name, _, child = name.rpartition(".")
+    parent = model.get_submodule(parent_name) if parent_name else model
+    setattr(parent, child, new_module)
+
+
+def is_compressed_tensors_config(compression_config: Any) -> bool:
+    """is this transformers' CompressedTensorsConfig (False where transformers has none;
+    utils/helpers.py:130-142)"""
+    try:
+        from transformers.utils.quantization_config import CompressedTensorsConfig
+    except ImportError:
+        return False
+    return isinstance(compression_config, CompressedTensorsConfig)
+
+
+def infer_compressor_from_model_config(pretrained_model_name_or_path: str):
+    """the sparsity compressor a model's config.json names, or None (utils/helpers.py:56-77)"""
+    from transformers import AutoConfig
+
+    from compressed_tensors_amd.compressors import BaseCompressor, ModelCompressor
+    from compressed_tensors_amd.config import SparsityCompressionConfig
+
+    config = AutoConfig.from_pretrained(pretrained_model_name_or_path)
+    sparsity = ModelCompressor.parse_sparsity_config(getattr(config, "quantization_config", None)
+                                                     or getattr(config, "compression_config", None))
+    if sparsity is None:
+        return None
+    fmt = sparsity.get("format")
+    return BaseCompressor.load_from_registry(
+        fmt, config=SparsityCompressionConfig.load_from_registry(fmt, **sparsity))
+
+
+def deprecated(future_name: Optional[str] = None, message: Optional[str] = None) -> Callable:
+    """decorator: calling the function warns (DeprecationWarning) that it will go, and what
+    to call instead (utils/helpers.py:176-203)"""
+    def decorator(func):
+        text = message
+        if text is None:
+            text = f"{func.__name__} is deprecated and will be removed in a future release"
+            if future_name is not None:
+                text += f". Please use {future_name} instead."
+
+        @wraps(func)
+        def wrapped(*args, **kwargs):
+            warnings.warn(text, DeprecationWarning, stacklevel=2)
+            return func(*args, **kwargs)
+
+        return wrapped
+
+    return decorator
+
+
+class Aliasable:
+    """mixin for enums some of whose members are other names for a member: equality and
+    hashing go by the member an alias stands for (utils/helpers.py:206-234)"""
+
+    @staticmethod
+    def get_aliases() -> Dict[str, str]:
+        raise NotImplementedError()
+
+    def _canonical(self, value):
+        return self.get_aliases().get(value, value)
+
+    def __eq__(self, other):
+        other_value = other.value if isinstance(other, type(self)) else other
+        try:
+            return self._canonical(self.value) == self._canonical(other_value)
+        except TypeError:  # an unhashable `other` is no member
+            return False
+
+    def __ne__(self, other):
+        return not self.__eq__(other)
+
+    def __hash__(self):
+        return hash(self._canonical(self.value))
+
+
+@contextlib.contextmanager
+def patch_attr(base: object, attr: str, value: Any):
+    """`base.attr = value` inside the with block; afterwards the old value is back, or the
+    attribute gone if there was none (utils/helpers.py:343-368)"""
+    missing = object()
+    before = getattr(base, attr, missing)
+    setattr(base, attr, value)
+    try:
+        yield
+    finally:
+        if before is missing:
+            delattr(base, attr)
+        else:
+            setattr(base, attr, before)
+
+
+class ParameterizedDefaultDict(dict):
+    """a defaultdict whose factory is given the missing key (a tuple key as its arguments)
+    and, through get(), keyword arguments that are not part of the key
+    (utils/helpers.py:371-401)"""
+
+    def __init__(self, default_factory: Callable[..., Any]):
+        super().__init__()
+        self.default_factory = default_factory
+        self._factory_kwargs: Dict[str, Any] = {}
+
+    def __missing__(self, key: Any) -> Any:
+        args = key if isinstance(key, tuple) else (key,)
+        value = self[key] = self.default_factory(*args, **self._factory_kwargs)
+        return value
+
+    def get(self, *args, factory_kwargs: Optional[Dict[str, Any]] = None) -> Any:
+        with patch_attr(self, "_factory_kwargs", dict(factory_kwargs or {})):
+            return self[args]

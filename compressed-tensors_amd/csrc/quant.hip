@@ -81,6 +81,47 @@ bool nvfp4_qdq_try_vectorised(const void* x, int x_dtype, void* out, int out_dty
 bool qdq_gidx_try(const void* x, int x_dtype, void* out, int out_dtype, int64_t rows, int64_t cols,
                   const ctmi_qparams* qp, int do_q, int do_dq, hipStream_t st);
 
+// ------------------------------------------------------------------ round_to_quantized_type
+// quant_args.py:384-408 on its own: every element to the nearest value of the quantized
+// type, in the tensor's dtype, no scale and no clamp.  MODE 0: torch.round (ties to
+// even); 1: to float8_e4m3fn and back; 2: FP4_E2M1_DATA.cast_to_fp4.
+template <typename XT, int MODE>
+__global__ void __launch_bounds__(256)
+round_to_type_kernel(const typename XT::raw* __restrict__ x, typename XT::raw* __restrict__ out,
+                     int64_t n) {
+  constexpr int VE = 16 / (int)sizeof(typename XT::raw);
+  const auto one = [](float v) {
+    if constexpr (MODE == 0) return rintf(v);
+    else if constexpr (MODE == 1) return f8e4m3_to_f32(f32_to_f8e4m3(v));
+    else return cast_to_fp4(v);
+  };
+  const int64_t nvec = n / VE;
+  for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
+    Vec<typename XT::raw, VE> a = ldg_nt<typename XT::raw, VE>(x + v * VE);
+#pragma unroll
+    for (int j = 0; j < VE; ++j) a.v[j] = XT::from_f32(one(XT::to_f32(a.v[j])));
+    stg_nt<typename XT::raw, VE>(out + v * VE, a);
+  }
+  if (blockIdx.x == 0 && threadIdx.x < n - nvec * VE) {
+    const int64_t i = nvec * VE + threadIdx.x;
+    out[i] = XT::from_f32(one(XT::to_f32(x[i])));
+  }
+}
+
+template <typename XT>
+static void round_to_type_launch(const void* x, void* out, int64_t n, int mode, hipStream_t st) {
+  using R = typename XT::raw;
+  constexpr int VE = 16 / (int)sizeof(R);
+  int64_t want = cdiv(n / VE, 256 * 4);
+  const unsigned grid = (unsigned)(want < 1 ? 1 : want > (1 << 20) ? (1 << 20) : want);
+  if (mode == 0)
+    hipLaunchKernelGGL((round_to_type_kernel<XT, 0>), grid, 256, 0, st, (const R*)x, (R*)out, n);
+  else if (mode == 1)
+    hipLaunchKernelGGL((round_to_type_kernel<XT, 1>), grid, 256, 0, st, (const R*)x, (R*)out, n);
+  else
+    hipLaunchKernelGGL((round_to_type_kernel<XT, 2>), grid, 256, 0, st, (const R*)x, (R*)out, n);
+}
+
 // ------------------------------------------------------------------ host side
 static int fill_cfg(const ctmi_qparams* qp, int x_dtype, QuantCfg* q) {
   int rc = quant_range(qp->qtype, qp->num_bits, &q->qmin, &q->qmax);
@@ -145,6 +186,27 @@ static void qdq_enqueue_generic(const void* x, int32_t x_dtype, void* out, int32
   dim3 block(256);
   dim3 grid((unsigned)cdiv(cols, 256), (unsigned)(rows < 32768 ? rows : 32768));
   hipLaunchKernelGGL(qdq_generic_kernel, grid, block, 0, st, a);
+}
+
+extern "C" int ctmi_round_to_quantized_type(const void* x, void* out, int32_t dtype, int64_t n,
+                                           int32_t qtype, int32_t num_bits, void* stream) {
+  CTMI_REQUIRE(n >= 0, CTMI_ERR_VALUE, "negative size");
+  CTMI_REQUIRE(dtype == CTMI_F32 || dtype == CTMI_F16 || dtype == CTMI_BF16, CTMI_ERR_UNSUPPORTED,
+               "round_to_quantized_type needs a float16/bfloat16/float32 tensor");
+  CTMI_REQUIRE(qtype == CTMI_QTYPE_INT || qtype == CTMI_QTYPE_FLOAT, CTMI_ERR_VALUE,
+               "Invalid quantization type %d", qtype);
+  CTMI_REQUIRE(qtype == CTMI_QTYPE_INT || num_bits == 4 || num_bits == 8, CTMI_ERR_UNSUPPORTED,
+               "Only num_bits in (4, 8) are supported");
+  if (n == 0) return CTMI_OK;
+  CTMI_REQUIRE(x != nullptr && out != nullptr, CTMI_ERR_VALUE, "NULL tensor pointer");
+  CTMI_REQUIRE((uintptr_t)x % 16 == 0 && (uintptr_t)out % 16 == 0, CTMI_ERR_VALUE,
+               "tensors must be 16-byte aligned");
+  const int mode = qtype == CTMI_QTYPE_INT ? 0 : num_bits == 8 ? 1 : 2;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == CTMI_BF16) round_to_type_launch<BF16>(x, out, n, mode, st);
+  else if (dtype == CTMI_F16) round_to_type_launch<F16>(x, out, n, mode, st);
+  else round_to_type_launch<F32>(x, out, n, mode, st);
+  return check_launch("ctmi_round_to_quantized_type");
 }
 
 extern "C" int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_dtype, int64_t rows,

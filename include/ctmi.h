@@ -89,6 +89,15 @@ int ctmi_qdq(const void* x, int32_t x_dtype, void* out, int32_t out_dtype, int64
              int64_t cols, const ctmi_qparams* qp, int32_t do_quantize, int32_t do_dequantize,
              void* stream);
 
+/* A8 on its own.  round_to_quantized_type (quantization/quant_args.py:384-408): every
+ * element of a float16 / bfloat16 / float32 tensor of n elements rounded to the nearest
+ * value of the quantized type and kept in the tensor's dtype: INT torch.round (ties to
+ * even), FLOAT with 8 bits through float8_e4m3fn and back, FLOAT with 4 bits
+ * FP4_E2M1_DATA.cast_to_fp4 (:55-68).  No scale, no clamp; out may be x.
+ * Other bit widths of FLOAT: CTMI_ERR_UNSUPPORTED, as the reference's NotImplementedError. */
+int ctmi_round_to_quantized_type(const void* x, void* out, int32_t dtype, int64_t n,
+                                 int32_t qtype, int32_t num_bits, void* stream);
+
 /* One tensor of a state dict for ctmi_qdq_many. */
 typedef struct ctmi_qdq_job {
   const void* x;

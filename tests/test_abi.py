@@ -409,3 +409,16 @@ def test_many_weight_block_one_shot_checks_every_job_first(ctmi):
     assert call(jobs, 2, *fp8) == _lib.CTMI_ERR_VALUE
     jobs[1].x, jobs[1].rows = 0x1000, 0
     assert call(jobs, 2, *fp8) == _lib.CTMI_ERR_VALUE
+
+
+def test_round_to_quantized_type_argument_checks(ctmi):
+    """quant_args.py:384-408: FLOAT with other than 4 or 8 bits is not implemented, an unknown
+    type is a value error; both are told before any GPU call"""
+    f = ctmi.ctmi_round_to_quantized_type
+    assert f(None, None, _lib.BF16, 0, 0, 8, None) == 0
+    assert f(None, None, _lib.BF16, 16, 1, 6, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert b"Only num_bits in (4, 8)" in ctmi.ctmi_last_error()
+    assert f(None, None, _lib.BF16, 16, 2, 8, None) == _lib.CTMI_ERR_VALUE
+    assert f(None, None, _lib.I8, 16, 0, 8, None) == _lib.CTMI_ERR_UNSUPPORTED
+    assert f(None, None, _lib.F32, 16, 0, 8, None) == _lib.CTMI_ERR_VALUE  # NULL tensors
+    assert f(None, None, _lib.F32, -1, 0, 8, None) == _lib.CTMI_ERR_VALUE

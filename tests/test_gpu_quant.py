@@ -760,3 +760,51 @@ def test_quantize_dequantize_with_activation_ordering(spec, shape, dtype, gpu):
                      oq.dequantize(want_q, scale, zp_arg, args=oargs, g_idx=g_idx), "dequantize")
     assert_bit_equal(fake_quantize(w.to(gpu), dev(scale), dev(zp_arg), args, g_idx=dev(g_idx)),
                      oq.fake_quantize(w, scale, zp_arg, oargs, g_idx=g_idx), "fake_quantize")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32], ids=["bf16", "f16", "f32"])
+@pytest.mark.parametrize("kind,num_bits", [("int", 8), ("float", 8), ("float", 4)])
+def test_round_to_quantized_type_on_every_pattern(kind, num_bits, dtype, gpu):
+    """A8 on its own (quant_args.py:384-408): all 65 536 patterns of a 16-bit float (for
+    float32: those of bfloat16 widened, ties and near-ties of every grid added) through
+    round_to_quantized_type, against the oracle, bit for bit; NaNs where the oracle has NaNs"""
+    from compressed_tensors_amd.quantization import FP4_E2M1_DATA, round_to_quantized_type
+
+    announce("round_to_quantized_type", kind, num_bits, dtype)
+    args, oargs = _pair(dict(num_bits=num_bits, type=kind, symmetric=True, strategy="tensor"))
+    if dtype == torch.float32:
+        x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.bfloat16).float()
+        ties = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 0.5, 1.5, 2.5, 3.5, 447.0, 448.0, 464.0,
+                             465.0, 2.0 ** -9, 2.0 ** -10, 1.5 * 2.0 ** -9, 17.0, 18.0, 19.0, 0.0])
+        near = torch.cat([ties, torch.nextafter(ties, torch.tensor(1e9)), torch.nextafter(ties, torch.tensor(-1e9))])
+        x = torch.cat([x, near, -near, torch.randn(4099, generator=torch.Generator().manual_seed(1)) * 100])
+    else:
+        x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype).clone()
+    x = torch.cat([x, x[:5]])  # a length that is no multiple of the kernel's vector
+    want = oq.round_to_quantized_type(x.clone(), oargs)
+    got = round_to_quantized_type(x.to(gpu), args)
+    assert got.dtype == dtype and got.shape == x.shape and got.is_cuda
+    got = got.cpu()
+    nan = torch.isnan(want.float())
+    assert torch.equal(torch.isnan(got.float()), nan), "NaNs"
+    assert torch.equal(bits_of(got)[~nan], bits_of(want)[~nan])
+    if kind == "float" and num_bits == 4:
+        again = FP4_E2M1_DATA.cast_to_fp4(x.to(gpu)).cpu()
+        assert torch.equal(bits_of(again)[~nan], bits_of(want)[~nan])
+    # a 2-d view that is not contiguous
+    m = x[:65536].reshape(256, 256).t()
+    assert_bit_equal(round_to_quantized_type(m.to(gpu), args).cpu().nan_to_num(0.0),
+                     oq.round_to_quantized_type(m.clone(), oargs).nan_to_num(0.0), "transposed")
+
+
+def test_round_to_quantized_type_refuses_what_the_reference_refuses(gpu):
+    from compressed_tensors_amd.quantization import QuantizationArgs, round_to_quantized_type
+
+    x = torch.zeros(8, device=gpu)
+    args = QuantizationArgs(num_bits=8, type="float", symmetric=True, strategy="tensor")
+    args.num_bits = 6
+    with pytest.raises(NotImplementedError, match="Only num_bits in"):
+        round_to_quantized_type(x, args)
+    args.type = "complex"
+    with pytest.raises(ValueError, match="Invalid quantization type"):
+        round_to_quantized_type(x, args)
