@@ -7,6 +7,8 @@ they are what model configs on disk name.
 from enum import Enum, unique
 from typing import Any, Dict, List, Optional
 
+from compressed_tensors_amd.registry import RegistryMixin
+
 __all__ = [
     "CompressionFormat",
     "SparsityStructure",
@@ -20,11 +22,17 @@ __all__ = [
     "DEFAULT_QUANTIZATION_FORMAT",
     "SPARSITY_CONFIG_NAME",
     "QUANTIZATION_CONFIG_NAME",
+    "TRANSFORM_CONFIG_NAME",
+    "COMPRESSION_VERSION_NAME",
+    "QUANTIZATION_METHOD_NAME",
     "infer_and_set_per_module_quantization_format",
 ]
 
 SPARSITY_CONFIG_NAME = "sparsity_config"
 QUANTIZATION_CONFIG_NAME = "quantization_config"
+TRANSFORM_CONFIG_NAME = "transform_config"
+COMPRESSION_VERSION_NAME = "version"
+QUANTIZATION_METHOD_NAME = "quant_method"
 
 
 @unique
@@ -112,9 +120,10 @@ DEFAULT_QUANTIZATION_METHOD = "compressed-tensors"
 DEFAULT_QUANTIZATION_FORMAT = "fakequant"
 
 
-class SparsityCompressionConfig:
+class SparsityCompressionConfig(RegistryMixin):
     """format / targets / ignore / global_sparsity / sparsity_structure
-    (reference: config/base.py:97-114)."""
+    (reference: config/base.py:97-114); the configs of the formats register under the
+    format's name."""
 
     def __init__(
         self,
@@ -135,10 +144,11 @@ class SparsityCompressionConfig:
 
     @classmethod
     def load_from_registry(cls, name, **kwargs) -> "SparsityCompressionConfig":
-        """the config of a sparsity format by its registry name (config/base.py:97-114; the
-        reference registers one subclass per format, with the same fields)"""
-        fields = ("targets", "ignore", "global_sparsity", "sparsity_structure")
-        return cls(format=name, **{k: v for k, v in kwargs.items() if k in fields})
+        """the config class registered for a sparsity format, built from the fields of a
+        config.json entry (config/base.py:97-114; other keys of the entry are ignored, as
+        the reference's models ignore them)"""
+        fields = ("format", "targets", "ignore", "global_sparsity", "sparsity_structure")
+        return cls.get_value_from_registry(name)(**{k: v for k, v in kwargs.items() if k in fields})
 
     def __eq__(self, other) -> bool:
         return isinstance(other, SparsityCompressionConfig) and self.model_dump() == other.model_dump()
@@ -146,6 +156,7 @@ class SparsityCompressionConfig:
     __hash__ = None
 
 
+@SparsityCompressionConfig.register(name=CompressionFormat.dense.value)
 class DenseSparsityConfig(SparsityCompressionConfig):
     """config/dense.py:26-43: sparse tensors stored as they are"""
 
@@ -153,6 +164,7 @@ class DenseSparsityConfig(SparsityCompressionConfig):
         super().__init__(format=format, **kwargs)
 
 
+@SparsityCompressionConfig.register(name=CompressionFormat.sparse_bitmask.value)
 class BitmaskConfig(SparsityCompressionConfig):
     """config/sparse_bitmask.py:26-40"""
 
@@ -160,6 +172,7 @@ class BitmaskConfig(SparsityCompressionConfig):
         super().__init__(format=format, **kwargs)
 
 
+@SparsityCompressionConfig.register(name=CompressionFormat.sparse_24_bitmask.value)
 class Sparse24BitMaskConfig(SparsityCompressionConfig):
     """config/sparse_24_bitmask.py:27-40: 2:4 by default"""
 

@@ -4,11 +4,11 @@ from typing import Dict
 
 import torch
 
+from compressed_tensors_amd.config import TRANSFORM_CONFIG_NAME
+
 from .hadamard import TransformFactory, TransformScheme
 
-__all__ = ["TransformConfig", "apply_transform_config", "TRANSFORM_CONFIG_NAME"]
-
-TRANSFORM_CONFIG_NAME = "transform_config"
+__all__ = ["TransformConfig", "apply_transform_config"]
 
 
 class TransformConfig:
