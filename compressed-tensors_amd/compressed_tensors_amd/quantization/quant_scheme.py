@@ -86,14 +86,36 @@ class QuantizationConfig:
         for name, scheme in config_groups.items():
             if isinstance(scheme, dict):
                 scheme = QuantizationScheme(**scheme)
+            elif not isinstance(scheme, QuantizationScheme):
+                # a list of targets under the name of a preset scheme (quant_config.py:148-160)
+                scheme = preset_name_to_scheme(name=name, targets=list(scheme))
             groups[name] = scheme
         self.config_groups = groups
         self.format = format
         self.quantization_status = quantization_status
         self.global_compression_ratio = global_compression_ratio
         self.ignore = ignore or []
+        if isinstance(kv_cache_scheme, dict):
+            kv_cache_scheme = QuantizationArgs(**kv_cache_scheme)
         self.kv_cache_scheme = kv_cache_scheme
         self.quant_method = quant_method
+
+    def to_dict(self) -> Dict[str, Any]:
+        """model_dump under the name transformers' quantizer calls (quant_config.py:162-164)"""
+        return self.model_dump()
+
+    def requires_calibration_data(self) -> bool:
+        """are there scales only data can give: a kv cache scheme, static or locally dynamic
+        input activations, static output activations (quant_config.py:262-278)"""
+        if self.kv_cache_scheme is not None:
+            return True
+        for scheme in self.config_groups.values():
+            inputs, outputs = scheme.input_activations, scheme.output_activations
+            if inputs is not None and inputs.dynamic in (False, DynamicType.LOCAL, DynamicType.LOCAL.value):
+                return True
+            if outputs is not None and not outputs.dynamic:
+                return True
+        return False
 
     def __eq__(self, other) -> bool:
         return isinstance(other, QuantizationConfig) and self.model_dump() == other.model_dump()

@@ -102,3 +102,30 @@ def test_module_helpers():
     except ImportError:
         return
     assert is_compressed_tensors_config(config) is True
+
+
+def test_quantization_config_presets_and_calibration_needs():
+    """quant_config.py:148-164, 262-278; tests/test_quantization/test_quant_config.py"""
+    from compressed_tensors_amd.quantization import QuantizationConfig, QuantizationScheme
+
+    config = QuantizationConfig(config_groups={"W4A16": ["Linear"], "w8a8": ["Conv2d"]})
+    w4, w8 = config.config_groups["W4A16"], config.config_groups["w8a8"]
+    assert isinstance(w4, QuantizationScheme) and w4.targets == ["Linear"] and w4.weights.num_bits == 4
+    assert w4.input_activations is None and w8.targets == ["Conv2d"] and w8.input_activations.dynamic is True
+    assert not config.requires_calibration_data()  # weights only, and inputs quantized per token on the fly
+    assert config.to_dict() == config.model_dump()
+    with pytest.raises(KeyError, match="Unknown preset scheme name"):
+        QuantizationConfig(config_groups={"W5A5": ["Linear"]})
+
+    static_in = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(),
+                                   input_activations=QuantizationArgs(num_bits=8))
+    assert QuantizationConfig(config_groups={"g": static_in}).requires_calibration_data()
+    local = QuantizationScheme(targets=["Linear"], weights=QuantizationArgs(),
+                               input_activations=QuantizationArgs(num_bits=4, type="float", strategy="tensor_group",
+                                                                  group_size=16, dynamic="local"))
+    assert QuantizationConfig(config_groups={"g": local}).requires_calibration_data()
+    static_out = QuantizationScheme(targets=["Linear"], output_activations=QuantizationArgs(num_bits=8))
+    assert QuantizationConfig(config_groups={"g": static_out}).requires_calibration_data()
+    kv = QuantizationConfig(config_groups={"W4A16": ["Linear"]}, kv_cache_scheme={"num_bits": 8, "type": "float"})
+    assert kv.requires_calibration_data() and kv.kv_cache_scheme.type == "float"
+    assert QuantizationConfig.model_validate(kv.model_dump()) == kv
