@@ -85,12 +85,6 @@ def disable_quantization(module: Module) -> None:
     module.quantization_enabled = False
 
 
-def _matching_targets(name: str, module: Module, targets):
-    from compressed_tensors_amd.utils.match import match_targets
-
-    return match_targets(name, module, targets)
-
-
 def apply_quantization_config(model: Module, config: Optional[QuantizationConfig],
                               run_compressed: bool = False):
     """attach the schemes of `config` to the modules they target and give these their
@@ -117,18 +111,18 @@ def apply_quantization_config(model: Module, config: Optional[QuantizationConfig
     for scheme in config.config_groups.values():
         for target in scheme.targets:
             target_to_scheme[target] = scheme
-    for name, module in list(model.named_modules()):
-        matched = _matching_targets(name, module, target_to_scheme)
-        if not matched or _matching_targets(name, module, config.ignore or []):
-            continue
-        scheme = target_to_scheme[matched[0]]
+    from compressed_tensors_amd.utils.match import is_narrow_match, match_named_modules, match_targets
+
+    # a target that names no module is worth a warning; of several targets that name a module
+    # the most specific decides: its name, then a pattern, then a class (apply.py:140-160)
+    for name, module in list(match_named_modules(model, target_to_scheme, config.ignore, warn_on_fail=True)):
+        scheme = target_to_scheme[match_targets(name, module, target_to_scheme)[0]]
         module.quantization_scheme = scheme
         if (run_compressed and isinstance(module, torch.nn.Linear)
                 and config.format != CompressionFormat.dense.value):
             CompressedLinear.from_linear(module, quantization_scheme=scheme, quantization_format=config.format)
         else:
-            if is_attention_module(module) and any(
-                    not t.startswith("re:") and t == name for t in scheme.targets):
+            if is_attention_module(module) and is_narrow_match(model, scheme.targets, name):
                 initialize_hooked_attention(model, module)
             initialize_module_for_quantization(module, force_zero_point=force_zero_point)
         module.quantization_status = status

@@ -87,10 +87,10 @@ def match_named_modules(model: torch.nn.Module, targets: Optional[Iterable[str]]
     for name, module in model.named_modules():
         if isinstance(module, InternalModule):
             continue
-        hit = next((t for t in targets if _one(name, module, t, fused)), None)
-        if hit is None:
+        if warn_on_fail and unmatched:  # every target that names the module has found one
+            unmatched.difference_update([t for t in unmatched if _one(name, module, t, fused)])
+        if not any(_one(name, module, t, fused) for t in targets):
             continue
-        unmatched.discard(hit)
         if not any(_one(name, module, t, fused) for t in ignore):
             yield name, module
     if warn_on_fail:

@@ -159,3 +159,47 @@ def test_statuses_compare_by_lifecycle_order_and_metadata_names():
 
     assert is_kv_cache_quant_scheme(QuantizationScheme(targets=["re:.*self_attn$"]))
     assert not is_kv_cache_quant_scheme(QuantizationScheme(targets=["Linear"]))
+
+
+def test_the_most_specific_target_decides_and_unmatched_targets_warn(caplog):
+    """tests/test_quantization/lifecycle/test_apply.py:73-119, 312-344: a module's name beats a
+    pattern, a pattern beats a class, whatever the order of the groups"""
+    def group(bits, target):
+        return {"weights": {"num_bits": bits}, "targets": [target]}
+
+    config = QuantizationConfig(config_groups={
+        "group_1": group(8, "Linear"), "group_2": group(4, "re:.*up_proj"),
+        "group_3": group(2, "layers.0.up_proj"), "group_4": group(6, "re:.*foobarbaz")},
+        ignore=["lm_head", "re:.*gate"])
+    config.quantization_status = QuantizationStatus.CALIBRATION
+    model = Tiny()
+    with caplog.at_level("WARNING"):
+        apply_quantization_config(model, config)
+    # one target and one ignore entry name no module
+    assert "Could not match `re:.*foobarbaz`" in caplog.text and caplog.text.count("Could not match") == 1
+    bits = {name: m.quantization_scheme.weights.num_bits for name, m in model.named_modules()
+            if hasattr(m, "quantization_scheme")}
+    assert bits == {"layers.0.q_proj": 8, "layers.0.up_proj": 2, "layers.1.q_proj": 8, "layers.1.up_proj": 4}
+    assert model.layers[0].q_proj.quantization_status == QuantizationStatus.CALIBRATION
+    assert not hasattr(model.lm_head, "quantization_scheme")
+
+
+def test_a_second_config_replaces_what_the_first_left():
+    """tests/test_quantization/lifecycle/test_apply.py:347-442"""
+    fp8 = QuantizationArgs(num_bits=8, type="float", strategy="tensor", symmetric=True, dynamic=False)
+    first = QuantizationConfig(config_groups={"group_0": QuantizationScheme(
+        targets=[r"re:.*(q|up)_proj$"], weights=fp8, input_activations=fp8)}, ignore=["lm_head"])
+    second = QuantizationConfig(config_groups={"group_0": QuantizationScheme(
+        targets=[r"re:.*up_proj$"],
+        weights=QuantizationArgs(num_bits=4, type="int", strategy="group", group_size=16, symmetric=False))},
+        ignore=["lm_head"])
+    model = Tiny()
+    apply_quantization_config(model, first)
+    apply_quantization_config(model, second)
+    for block in model.layers:
+        up, q = block.up_proj, block.q_proj
+        assert not hasattr(up, "input_scale") and not hasattr(up, "input_zero_point")
+        assert up.weight_scale.shape == (64, 2) and up.weight_zero_point.shape == (64, 2)
+        assert up.quantization_scheme.weights.num_bits == 4
+        assert q.input_scale.shape == q.input_zero_point.shape == q.weight_scale.shape == (1,)
+        assert q.quantization_scheme.weights.type == "float"
