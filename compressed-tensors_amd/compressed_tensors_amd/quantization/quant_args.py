@@ -67,6 +67,8 @@ def _round_on_gpu(tensor: torch.Tensor, qtype: int, num_bits: int) -> torch.Tens
 
     _lib.require_gpu(tensor)
     x = tensor.contiguous()
+    if x.data_ptr() % 16:  # a view that starts inside a buffer: the kernel reads 16 bytes a lane
+        x = x.clone()
     out = torch.empty_like(x)
     _lib.check(_lib.load().ctmi_round_to_quantized_type(
         x.data_ptr(), out.data_ptr(), _lib.dtype_code(x.dtype), x.numel(), qtype, num_bits,

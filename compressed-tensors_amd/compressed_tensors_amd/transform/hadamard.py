@@ -249,6 +249,12 @@ def _aligned(*tensors) -> bool:
     return all(t is None or t.data_ptr() % 16 == 0 for t in tensors)
 
 
+def _on_16_bytes(x: Tensor) -> Tensor:
+    """x, or a copy of it if it starts inside a buffer off a 16-byte boundary (the kernels
+    read and write 16 bytes a lane)"""
+    return x.clone() if x.data_ptr() % 16 else x
+
+
 def _matrix_free(n: int, dtype, *tensors) -> bool:
     """does the rotation (alone or fused with the quantization) by Sylvester's matrix of order
     n run without a matrix argument?"""
@@ -268,7 +274,7 @@ def hadamard_apply(
     the explicit matrix whose transpose is `matrix_t` (bf16, entries exact in bf16).
     kernel: "mfma" / "butterfly" to pick between the two implementations of the Sylvester
     sizes 1024 ... 8192 (default: the faster one)."""
-    x = to_gpu(value).contiguous()
+    x = _on_16_bytes(to_gpu(value).contiguous())
     if x.dtype not in _FLOATS:
         raise NotImplementedError(f"transforms of dtype {x.dtype} are not supported")
     if x.shape[-1] % n != 0:
@@ -456,9 +462,10 @@ def hadamard_apply_many(
     run of n elements before it writes any of it)."""
     if not values:
         return []
-    if in_place and not all(v.is_cuda and v.is_contiguous() for v in values):
-        raise ValueError("tensors transformed in place are contiguous tensors on the GPU")
-    xs = [to_gpu(v).contiguous() for v in values]
+    if in_place and not all(v.is_cuda and v.is_contiguous() and v.data_ptr() % 16 == 0 for v in values):
+        raise ValueError("tensors transformed in place are contiguous tensors on the GPU that start on "
+                         "16-byte boundaries")
+    xs = [_on_16_bytes(to_gpu(v).contiguous()) for v in values]
     dtype, dev = xs[0].dtype, xs[0].device
     if dtype not in _FLOATS:
         raise NotImplementedError(f"transforms of dtype {dtype} are not supported")
@@ -831,7 +838,8 @@ class HadamardTransform(TransformBase):
         if left:
             xs = [x.transpose(0, -1) for x in xs]
         s_in, s_out = (None, self.signs) if transposed else (self.signs, None)
-        in_place = in_place and not left and all(x.is_cuda and x.is_contiguous() for x in xs)
+        in_place = in_place and not left and all(
+            x.is_cuda and x.is_contiguous() and x.data_ptr() % 16 == 0 for x in xs)
         ys = hadamard_apply_many(xs, n, sign_in=s_in, sign_out=s_out, in_place=in_place)
         return [y.transpose(0, -1).contiguous() for y in ys] if left else ys
 

@@ -791,6 +791,9 @@ def test_round_to_quantized_type_on_every_pattern(kind, num_bits, dtype, gpu):
     if kind == "float" and num_bits == 4:
         again = FP4_E2M1_DATA.cast_to_fp4(x.to(gpu)).cpu()
         assert torch.equal(bits_of(again)[~nan], bits_of(want)[~nan])
+    # a view that starts in the middle of a buffer
+    assert_bit_equal(round_to_quantized_type(x.to(gpu)[3:1000], args).cpu().nan_to_num(0.0),
+                     want[3:1000].nan_to_num(0.0), "offset view")
     # a 2-d view that is not contiguous
     m = x[:65536].reshape(256, 256).t()
     assert_bit_equal(round_to_quantized_type(m.to(gpu), args).cpu().nan_to_num(0.0),

@@ -280,3 +280,12 @@ def test_many_tensors_in_place(n, dtype, gpu):
         assert_bit_equal(y, w, f"in place, size {n}")
     with pytest.raises(ValueError, match="in place"):
         hadamard_apply_many([xs[0].t()], n, in_place=True)
+    # a tensor that starts off a 16-byte boundary: not in place, and through a copy otherwise
+    flat = torch.cat([x.flatten() for x in xs[:2]])
+    inner = flat[1:1 + xs[0].numel()].view_as(xs[0])
+    inner.copy_(want[0])  # any values
+    assert inner.data_ptr() % 16 != 0
+    with pytest.raises(ValueError, match="in place"):
+        hadamard_apply_many([inner], n, in_place=True)
+    assert_bit_equal(hadamard_apply_many([inner], n, sign_in=q)[0],
+                     hadamard_apply_many([inner.clone()], n, sign_in=q)[0], "off a 16-byte boundary")
