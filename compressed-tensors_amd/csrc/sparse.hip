@@ -1563,8 +1563,8 @@ __device__ __forceinline__ void store_survivors24_any(const Vec<R, N>& a, R* __r
 #pragma unroll
   for (int bq = 0; bq < N / 8; ++bq) m.v[bq] = (uint8_t)((keep_all >> (8 * bq)) & 0xffu);
   if (keep_item) {
-    stg<R, N / 2>(values + i * (N / 2), o);
-    stg<uint8_t, N / 8>(bitmask + i * (N / 8), m);
+    stg_nt<R, N / 2>(values + i * (N / 2), o);
+    stg_nt<uint8_t, N / 8>(bitmask + i * (N / 8), m);
   }
 }
 
@@ -1594,8 +1594,8 @@ __device__ __forceinline__ void store_survivors24_bytes(const Vec<uint8_t, N>& a
 #pragma unroll
   for (int bq = 0; bq < N / 8; ++bq) m.v[bq] = (uint8_t)((keep_all >> (8 * bq)) & 0xffu);
   if (keep_item) {
-    stg<uint32_t, G / 2>(reinterpret_cast<uint32_t*>(values + i * (N / 2)), o);
-    stg<uint8_t, N / 8>(bitmask + i * (N / 8), m);
+    stg_nt<uint32_t, G / 2>(reinterpret_cast<uint32_t*>(values + i * (N / 2)), o);
+    stg_nt<uint8_t, N / 8>(bitmask + i * (N / 8), m);
   }
 }
 
