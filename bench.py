@@ -604,6 +604,24 @@ def other_workload(torch, name, seed):
         ops += [Op("nvfp4 activations: group-16 scales (16 x 4096x4096)", o_calls, 2 * na + na // 16, "observe_flat_kernel"),
                 Op("nvfp4 activations: fake-quantize (16 x 4096x4096)", f_calls, 4 * na + na // 16, "nvfp4_qdq_vec_kernel"),
                 Op("nvfp4 activations: scales + fake-quantize in one pass (16 x 4096x4096)", y_calls, 4 * na, "nvfp4_dynamic_kernel")]
+        # A13 / A14 on their own: values already on the e2m1 grid <-> two codes a byte
+        grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], device=dev)
+        p4_calls, u4_calls, n4 = [], [], 0
+        for _ in range(16):
+            r, c = 14336, 4096
+            x = (grid[torch.randint(0, 8, (r, c), generator=gen, device=dev)]
+                 * (torch.randint(0, 2, (r, c), generator=gen, device=dev) * 2 - 1)).to(torch.bfloat16)
+            codes = torch.empty(r, c // 2, dtype=torch.uint8, device=dev)
+            back = torch.empty_like(x)
+            keep.extend([x, codes, back])
+            pa = (x.data_ptr(), code(x.dtype), codes.data_ptr(), r, c, st)
+            ua = (codes.data_ptr(), back.data_ptr(), code(back.dtype), r, c, st)
+            _lib.check(lib.ctmi_pack_fp4_to_uint8(*pa))
+            p4_calls.append(lambda pa=pa: _lib.check(lib.ctmi_pack_fp4_to_uint8(*pa)))
+            u4_calls.append(lambda ua=ua: _lib.check(lib.ctmi_unpack_fp4_from_uint8(*ua)))
+            n4 += r * c
+        ops += [Op("pack_fp4_to_uint8 alone, bf16 14336x4096 (x16)", p4_calls, 2 * n4 + n4 // 2, "fp4_pack_vec_kernel"),
+                Op("unpack_fp4_from_uint8 alone, to bf16 (x16)", u4_calls, 2 * n4 + n4 // 2, "fp4_unpack_vec_kernel")]
         return "nvfp4-pack-quantized compress/decompress + activation fake-quantize GB/s", ops, keep
 
     if name == "one-shot":
@@ -663,6 +681,24 @@ def other_workload(torch, name, seed):
                   gidx_cmp, 2 * n + 2 * g + n // 2, "pq_gidx_compress_kernel", primary=False),
                Op("activation ordering (g_idx): observer + qparams + quantize + pack in one pass (one call each)",
                   gidx_one, 2 * n + 2 * g + n // 2, "observe_pack_table_kernel", primary=False)]
+        # A9 / A10 on their own: int8 codes <-> packed words (callers that hold codes already)
+        pk_calls, up_calls, n_codes = [], [], 0
+        for _ in range(16):
+            r, c = 14336, 4096
+            codes = torch.randint(-8, 8, (r, c), generator=gen, device=dev, dtype=torch.int8)
+            words = torch.empty(r, c // 8, dtype=torch.int32, device=dev)
+            back = torch.empty_like(codes)
+            keep.extend([codes, words, back])
+            pa = (codes.data_ptr(), words.data_ptr(), r, c, 4, 1, st)
+            ua = (words.data_ptr(), back.data_ptr(), r, c, 4, 1, st)
+            _lib.check(lib.ctmi_pack_to_int32(*pa))
+            pk_calls.append(lambda pa=pa: _lib.check(lib.ctmi_pack_to_int32(*pa)))
+            up_calls.append(lambda ua=ua: _lib.check(lib.ctmi_unpack_from_int32(*ua)))
+            n_codes += r * c
+        ops += [Op("pack_to_int32 alone: int8 codes -> 4-bit words, 14336x4096 (x16)", pk_calls, n_codes + n_codes // 2,
+                   "pack_dim1_vec_kernel"),
+                Op("unpack_from_int32 alone, 14336x4096 (x16)", up_calls, n_codes + n_codes // 2,
+                   "unpack_dim1_vec_kernel")]
         return "one-shot W4A16 g128 compression GB/s (no scales given), Llama-3-8B-shaped weights", ops, keep
 
     if name == "hadamard":

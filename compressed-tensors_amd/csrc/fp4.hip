@@ -50,20 +50,77 @@ __device__ __forceinline__ int fp4_nearest_code_rt(float x, int xdt) {
   return fp4_nearest_code<CTMI_F32>(x);
 }
 
+// 8 fp32 values -> 8 e2m1 codes (element i in bits [4i, 4i+4)) with the hardware
+// converter: round to nearest even on the e2m1 grid = the reference's bucket
+// boundaries (quant_args.py:55-68), saturating at +-6, sign kept.
+__device__ __forceinline__ uint32_t fp4_pack8_hw(const float* t) {
+  uint32_t w = 0;
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[0], t[1], 1.0f, 0);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[2], t[3], 1.0f, 1);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[4], t[5], 1.0f, 2);
+  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[6], t[7], 1.0f, 3);
+  return w;
+}
+
+// 8 codes of a dword -> 8 fp32 values (exact; code 8 is -0.0)
+__device__ __forceinline__ void fp4_unpack8_hw(uint32_t w, float* t) {
+  typedef float f32x2 __attribute__((ext_vector_type(2)));
+  f32x2 r;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0); t[0] = r.x; t[1] = r.y;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1); t[2] = r.x; t[3] = r.y;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2); t[4] = r.x; t[5] = r.y;
+  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3); t[6] = r.x; t[7] = r.y;
+}
+
 // ------------------------------------------------------------------ standalone pack / unpack
-// one thread per 8 elements (cols % 8 == 0) -> one 32-bit store
+// 8 elements -> one 32-bit word; a lane takes kFp4Vecs of them, all loads first; the tensor is
+// read and written once: streaming loads and stores
+constexpr int kFp4Vecs = 4;
+
 template <typename XT>
 __global__ void __launch_bounds__(256)
 fp4_pack_vec_kernel(const typename XT::raw* __restrict__ x, uint32_t* __restrict__ out,
                     int64_t nvec) {
-  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
-       v += (int64_t)gridDim.x * blockDim.x) {
-    Vec<typename XT::raw, 8> a = ldg<typename XT::raw, 8>(x + v * 8);
-    uint32_t acc = 0;
+  constexpr int U = kFp4Vecs;
+  constexpr int H = 16 / (int)sizeof(typename XT::raw);  // elements of a 16-byte load
+  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  Vec<typename XT::raw, H> a[U][8 / H];
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
-      acc |= (uint32_t)fp4_nearest_code<XT::id>(XT::to_f32(a.v[i])) << (4 * i);
-    out[v] = acc;
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    const typename XT::raw* at = x + (v < nvec ? v : nvec - 1) * 8;  // past the end: re-read, not stored
+#pragma unroll
+    for (int h = 0; h < 8 / H; ++h) a[k][h] = ldg_nt<typename XT::raw, H>(at + h * H);
+  }
+  // A quantized tensor holds values of the grid only: the hardware converter gives their
+  // codes, and converting back tells whether a value was one (bit for bit, so that -0.0 and
+  // NaNs are told apart).  If any lane of the wavefront met another value, the wavefront goes
+  // through the reference's nearest-value search instead (one branch for all its elements).
+  uint32_t acc[U];
+  bool off_grid = false;
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    float t[8], back[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) t[i] = XT::to_f32(a[k][i / H].v[i % H]);
+    acc[k] = fp4_pack8_hw(t);
+    fp4_unpack8_hw(acc[k], back);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) off_grid |= f2u(back[i]) != f2u(t[i]);
+  }
+  if (__builtin_amdgcn_ballot_w64(off_grid) != 0) {
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      acc[k] = 0;
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+        acc[k] |= (uint32_t)fp4_nearest_code<XT::id>(XT::to_f32(a[k][i / H].v[i % H])) << (4 * i);
+    }
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    if (v < nvec) __builtin_nontemporal_store(acc[k], out + v);
   }
 }
 
@@ -82,13 +139,30 @@ template <typename OT>
 __global__ void __launch_bounds__(256)
 fp4_unpack_vec_kernel(const uint32_t* __restrict__ in, typename OT::raw* __restrict__ out,
                       int64_t nvec) {
-  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
-       v += (int64_t)gridDim.x * blockDim.x) {
-    const uint32_t w = in[v];
-    float f[8];
+  constexpr int U = kFp4Vecs;
+  constexpr int H = 16 / (int)sizeof(typename OT::raw);  // elements of a 16-byte store
+  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  uint32_t w[U];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) f[i] = fp4_decode((int)((w >> (4 * i)) & 15u));
-    stg<typename OT::raw, 8>(out + v * 8, pack8_from_f32<OT>(f));  // sixteen values, none a NaN
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    w[k] = __builtin_nontemporal_load(in + (v < nvec ? v : nvec - 1));
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    float f[8];
+    fp4_unpack8_hw(w[k], f);
+    const Vec<typename OT::raw, 8> o = pack8_from_f32<OT>(f);  // values of the grid, none a NaN
+    if (v < nvec) {
+#pragma unroll
+      for (int h = 0; h < 8 / H; ++h) {
+        Vec<typename OT::raw, H> part;
+#pragma unroll
+        for (int e = 0; e < H; ++e) part.v[e] = o.v[h * H + e];
+        stg_nt<typename OT::raw, H>(out + v * 8 + h * H, part);
+      }
+    }
   }
 }
 
@@ -179,28 +253,6 @@ __global__ void __launch_bounds__(256) nvfp4_decompress_generic_kernel(Fp4Args a
 #endif
 constexpr int kFp4Tuning[2] = {CTMI_FP4_TUNING};
 constexpr int kFp4Block = kFp4Tuning[0], kFp4Unroll = kFp4Tuning[1];
-
-// 8 fp32 values -> 8 e2m1 codes (element i in bits [4i, 4i+4)) with the hardware
-// converter: round to nearest even on the e2m1 grid = the reference's bucket
-// boundaries (quant_args.py:55-68), saturating at +-6, sign kept.
-__device__ __forceinline__ uint32_t fp4_pack8_hw(const float* t) {
-  uint32_t w = 0;
-  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[0], t[1], 1.0f, 0);
-  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[2], t[3], 1.0f, 1);
-  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[4], t[5], 1.0f, 2);
-  w = __builtin_amdgcn_cvt_scalef32_pk_fp4_f32(w, t[6], t[7], 1.0f, 3);
-  return w;
-}
-
-// 8 codes of a dword -> 8 fp32 values (exact; code 8 is -0.0)
-__device__ __forceinline__ void fp4_unpack8_hw(uint32_t w, float* t) {
-  typedef float f32x2 __attribute__((ext_vector_type(2)));
-  f32x2 r;
-  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 0); t[0] = r.x; t[1] = r.y;
-  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 1); t[2] = r.x; t[3] = r.y;
-  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 2); t[4] = r.x; t[5] = r.y;
-  r = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(w, 1.0f, 3); t[6] = r.x; t[7] = r.y;
-}
 
 // The reference's chain for 8 elements: x / s, + zp, clamp to +-6, cast_to_fp4
 // (forward.py:471-482, quant_args.py:55-68), one exact division per element.
@@ -990,7 +1042,7 @@ extern "C" int ctmi_pack_fp4_to_uint8(const void* x, int32_t x_dtype, uint8_t* o
   const int64_t n = rows * cols;
   if (n % 8 == 0 && (uintptr_t)x % (8 * dtype_size(x_dtype)) == 0 && (uintptr_t)out % 4 == 0) {
     const int64_t nvec = n / 8;
-    const int grid = grid_for(nvec, 256);
+    const unsigned grid = (unsigned)cdiv(nvec, 256 * kFp4Vecs);
     if (x_dtype == CTMI_BF16) hipLaunchKernelGGL(fp4_pack_vec_kernel<BF16>, grid, 256, 0, st, (const uint16_t*)x, (uint32_t*)out, nvec);
     else if (x_dtype == CTMI_F16) hipLaunchKernelGGL(fp4_pack_vec_kernel<F16>, grid, 256, 0, st, (const uint16_t*)x, (uint32_t*)out, nvec);
     else hipLaunchKernelGGL(fp4_pack_vec_kernel<F32>, grid, 256, 0, st, (const float*)x, (uint32_t*)out, nvec);
@@ -1012,7 +1064,7 @@ extern "C" int ctmi_unpack_fp4_from_uint8(const uint8_t* in, void* out, int32_t 
   const int64_t n = rows * cols;
   if (n % 8 == 0 && (uintptr_t)out % (8 * dtype_size(out_dtype)) == 0 && (uintptr_t)in % 4 == 0) {
     const int64_t nvec = n / 8;
-    const int grid = grid_for(nvec, 256);
+    const unsigned grid = (unsigned)cdiv(nvec, 256 * kFp4Vecs);
     if (out_dtype == CTMI_BF16) hipLaunchKernelGGL(fp4_unpack_vec_kernel<BF16>, grid, 256, 0, st, (const uint32_t*)in, (uint16_t*)out, nvec);
     else if (out_dtype == CTMI_F16) hipLaunchKernelGGL(fp4_unpack_vec_kernel<F16>, grid, 256, 0, st, (const uint32_t*)in, (uint16_t*)out, nvec);
     else hipLaunchKernelGGL(fp4_unpack_vec_kernel<F32>, grid, 256, 0, st, (const uint32_t*)in, (float*)out, nvec);

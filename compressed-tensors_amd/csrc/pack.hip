@@ -46,25 +46,38 @@ pack_dim1_kernel(const int8_t* __restrict__ in, int32_t* __restrict__ out, int64
   }
 }
 
-// 4- or 8-bit, cols % 16 == 0: 16 input bytes per thread.
+// vectors a lane of the streaming pack / unpack kernels takes, all of them asked for before
+// any is used
+constexpr int kPackVecs = 4;
+
+// 4- or 8-bit, cols % 16 == 0: 16 input bytes per vector.  The tensor is read and written
+// once: streaming loads and stores.
 template <int BITS>
 __global__ void __launch_bounds__(256)
 pack_dim1_vec_kernel(const int8_t* __restrict__ in, int32_t* __restrict__ out, int64_t nvec) {
   constexpr int W = BITS * 16 / 32;  // words produced per 16 inputs
   constexpr int PF = 32 / BITS;
   constexpr int OFF = 1 << (BITS - 1);
-  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
-       v += (int64_t)gridDim.x * blockDim.x) {
-    Vec<int8_t, 16> a = ldg<int8_t, 16>(in + v * 16);
+  constexpr int U = kPackVecs;
+  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  Vec<int8_t, 16> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    a[k] = ldg_nt<int8_t, 16>(in + (v < nvec ? v : nvec - 1) * 16);  // past the end: re-read, not stored
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
     Vec<int32_t, W> o;
 #pragma unroll
     for (int w = 0; w < W; ++w) {
       uint32_t acc = 0;
 #pragma unroll
-      for (int i = 0; i < PF; ++i) acc += (uint32_t)(uint8_t)(a.v[w * PF + i] + OFF) << (BITS * i);
+      for (int i = 0; i < PF; ++i) acc += (uint32_t)(uint8_t)(a[k].v[w * PF + i] + OFF) << (BITS * i);
       o.v[w] = (int32_t)acc;
     }
-    stg<int32_t, W>(out + v * W, o);
+    if (v < nvec) stg_nt<int32_t, W>(out + v * W, o);
   }
 }
 
@@ -112,7 +125,7 @@ unpack_kernel(const int32_t* __restrict__ in, int8_t* __restrict__ out, int64_t 
   }
 }
 
-// 4- or 8-bit, packed_dim 1, cols % 16 == 0: 16 output bytes per thread.
+// 4- or 8-bit, packed_dim 1, cols % 16 == 0: 16 output bytes per vector
 template <int BITS>
 __global__ void __launch_bounds__(256)
 unpack_dim1_vec_kernel(const int32_t* __restrict__ in, int8_t* __restrict__ out, int64_t nvec) {
@@ -120,16 +133,24 @@ unpack_dim1_vec_kernel(const int32_t* __restrict__ in, int8_t* __restrict__ out,
   constexpr int PF = 32 / BITS;
   constexpr int OFF = 1 << (BITS - 1);
   constexpr uint32_t MASK = (1u << BITS) - 1u;
-  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < nvec;
-       v += (int64_t)gridDim.x * blockDim.x) {
-    Vec<int32_t, W> a = ldg<int32_t, W>(in + v * W);
+  constexpr int U = kPackVecs;
+  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  Vec<int32_t, W> a[U];
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
+    a[k] = ldg_nt<int32_t, W>(in + (v < nvec ? v : nvec - 1) * W);  // past the end: re-read, not stored
+  }
+#pragma unroll
+  for (int k = 0; k < U; ++k) {
+    const int64_t v = v0 + k * 256;
     Vec<int8_t, 16> o;
 #pragma unroll
     for (int w = 0; w < W; ++w)
 #pragma unroll
       for (int i = 0; i < PF; ++i)
-        o.v[w * PF + i] = (int8_t)((int)(((uint32_t)a.v[w] >> (BITS * i)) & MASK) - OFF);
-    stg<int8_t, 16>(out + v * 16, o);
+        o.v[w * PF + i] = (int8_t)((int)(((uint32_t)a[k].v[w] >> (BITS * i)) & MASK) - OFF);
+    if (v < nvec) stg_nt<int8_t, 16>(out + v * 16, o);
   }
 }
 
@@ -416,7 +437,7 @@ extern "C" int ctmi_pack_to_int32(const int8_t* in, int32_t* out, int64_t rows, 
                      ((uintptr_t)in % 16 == 0) && ((uintptr_t)out % 8 == 0);
     if (vec) {
       const int64_t nvec = rows * cols / 16;
-      const int grid = grid_for(nvec, 256);
+      const unsigned grid = (unsigned)cdiv(nvec, 256 * kPackVecs);
       if (num_bits == 4) hipLaunchKernelGGL(pack_dim1_vec_kernel<4>, grid, 256, 0, st, in, out, nvec);
       else hipLaunchKernelGGL(pack_dim1_vec_kernel<8>, grid, 256, 0, st, in, out, nvec);
     } else {
@@ -445,7 +466,7 @@ extern "C" int ctmi_unpack_from_int32(const int32_t* in, int8_t* out, int64_t ro
                    ((uintptr_t)out % 16 == 0) && ((uintptr_t)in % 8 == 0);
   if (vec) {
     const int64_t nvec = rows * cols / 16;
-    const int grid = grid_for(nvec, 256);
+    const unsigned grid = (unsigned)cdiv(nvec, 256 * kPackVecs);
     if (num_bits == 4) hipLaunchKernelGGL(unpack_dim1_vec_kernel<4>, grid, 256, 0, st, in, out, nvec);
     else hipLaunchKernelGGL(unpack_dim1_vec_kernel<8>, grid, 256, 0, st, in, out, nvec);
   } else {

@@ -522,6 +522,31 @@ def test_fp4_pack_off_grid_inputs(dtype, shape, gpu):
                          op.unpack_fp4_from_uint8(want, *shape, dtype=out_dtype), "fp4 unpack")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_fp4_pack_every_16_bit_pattern_and_mixed_tensors(dtype, gpu):
+    """pack_fp4_to_uint8 (fp4_quantized.py:135-178) on all 65 536 patterns of a 16-bit float
+    (values of the grid, others, both zeros, infinities, NaNs), and on a large tensor of grid
+    values with a few others strewn in: wavefronts with and without a value off the grid"""
+    from compressed_tensors_amd.compressors import pack_fp4_to_uint8, unpack_fp4_from_uint8
+
+    announce("fp4 every pattern", dtype)
+    x = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(dtype).reshape(256, 256).clone()
+    assert_bit_equal(pack_fp4_to_uint8(x.to(gpu)), op.pack_fp4_to_uint8(x), "every pattern")
+    g = torch.Generator().manual_seed(5)
+    grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0])
+    y = (grid[torch.randint(0, 8, (520, 2048), generator=g)]
+         * (torch.randint(0, 2, (520, 2048), generator=g) * 2 - 1)).to(dtype)
+    flat = y.view(-1)
+    where = torch.randint(0, flat.numel(), (40,), generator=g)
+    flat[where] = (torch.randn(40, generator=g) * 3).to(dtype)
+    flat[where[:4]] = torch.tensor([float("nan"), float("inf"), -float("inf"), 0.75]).to(dtype)
+    packed = pack_fp4_to_uint8(y.to(gpu))
+    assert_bit_equal(packed, op.pack_fp4_to_uint8(y), "grid values with a few others")
+    for out_dtype in (torch.bfloat16, torch.float16, torch.float32):
+        assert_bit_equal(unpack_fp4_from_uint8(packed, 520, 2048, dtype=out_dtype),
+                         op.unpack_fp4_from_uint8(packed.cpu(), 520, 2048, dtype=out_dtype), "unpack")
+
+
 @pytest.mark.parametrize("shape,dtype", [((64, 256), torch.bfloat16), ((24, 48), torch.bfloat16),
                                          ((32, 128), torch.float16), ((8, 64), torch.float32)])
 def test_nvfp4_compressor(shape, dtype, gpu):
