@@ -358,12 +358,22 @@ def other_workload(torch, name, seed):
                Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
                Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel"),
                Op("activations: scales + fake-quantize in one pass (8 x 8192x4096)", a_dyn, 4 * na, "dynamic_rows_kernel")]
+        # A8 on its own: every element to the nearest fp8 value, dtype kept
+        r_calls, nr = [], 0
+        for _ in range(8):
+            x = randn(14336, 4096)
+            out = torch.empty_like(x)
+            keep.extend([x, out])
+            ra = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), 1, 8, st)
+            r_calls.append(lambda ra=ra: _lib.check(lib.ctmi_round_to_quantized_type(*ra)))
+            nr += x.numel()
+        ops.append(Op("round_to_quantized_type alone (fp8), bf16 14336x4096 (x8)", r_calls, 4 * nr, "round_to_type_kernel"))
         return "fp8 W8A8 quantize/dequantize GB/s, Llama-3-8B-shaped weights + per-token activations", ops, keep
 
     if name == "sparse":
         copies = 6
         c_calls, d_calls, s_calls, t_calls, two_step, one_step = [], [], [], [], [], []
-        back_two, back_one, s16_calls, t16_calls, pk_calls, up_calls = [], [], [], [], [], []
+        back_two, back_one, s16_calls, t16_calls, pk_calls, up_calls, bm_calls = [], [], [], [], [], [], []
         stacked_jobs = []
         nb = 8192 * 8192
         nnz_total = 0
@@ -422,6 +432,8 @@ def other_workload(torch, name, seed):
             bools_back = torch.empty_like(bools)
             packed = torch.empty(rows, cols // 8, dtype=torch.uint8, device=dev)
             keep.extend([bools, bools_back, packed])
+            bm = (w.data_ptr(), code(w.dtype), bools_back.data_ptr(), w.numel(), st)
+            bm_calls.append(lambda bm=bm: _lib.check(lib.ctmi_get_24_bytemasks(*bm)))
             pk = (bools.data_ptr(), packed.data_ptr(), rows, cols, st)
             up = (packed.data_ptr(), bools_back.data_ptr(), rows, cols, st)
             _lib.check(lib.ctmi_pack_bitmasks(*pk))
@@ -496,6 +508,7 @@ def other_workload(torch, name, seed):
                Op("sparse-24-bitmask decompress, bf16, all 16 in one call (8 per launch)",
                   [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm16))],
                   2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel", launches=chained(copies24)),
+               Op("get_24_bytemasks, 14336x4096 bf16 -> bool", bm_calls, copies24 * (2 * n24 + n24), "bytemask24_vec_kernel"),
                Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies24 * (n24 + n24 // 8), "pack_bitmasks"),
                Op("unpack_bitmasks", up_calls, copies24 * (n24 + n24 // 8), "unpack_bitmasks"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),

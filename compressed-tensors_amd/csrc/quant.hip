@@ -92,15 +92,32 @@ round_to_type_kernel(const typename XT::raw* __restrict__ x, typename XT::raw* _
   constexpr int VE = 16 / (int)sizeof(typename XT::raw);
   const auto one = [](float v) {
     if constexpr (MODE == 0) return rintf(v);
-    else if constexpr (MODE == 1) return f8e4m3_to_f32(f32_to_f8e4m3(v));
+    else if constexpr (MODE == 1) {
+      // the hardware converter: nearest even, NaN beyond the largest value's rounding range,
+      // as torch's cast (checked on every 16-bit pattern)
+      return __builtin_amdgcn_cvt_f32_fp8(__builtin_amdgcn_cvt_pk_fp8_f32(v, v, 0, false), 0);
+    }
     else return cast_to_fp4(v);
   };
+  // 4 vectors a lane, all of them asked for before any is used; the tensor is read and
+  // written once: streaming loads and stores
+  constexpr int U = 4;
   const int64_t nvec = n / VE;
-  for (int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x; v < nvec; v += (int64_t)gridDim.x * 256) {
-    Vec<typename XT::raw, VE> a = ldg_nt<typename XT::raw, VE>(x + v * VE);
+  const int64_t v0 = (int64_t)blockIdx.x * (256 * U) + threadIdx.x;
+  Vec<typename XT::raw, VE> a[U];
+  if (nvec > 0) {
 #pragma unroll
-    for (int j = 0; j < VE; ++j) a.v[j] = XT::from_f32(one(XT::to_f32(a.v[j])));
-    stg_nt<typename XT::raw, VE>(out + v * VE, a);
+    for (int k = 0; k < U; ++k) {
+      const int64_t v = v0 + k * 256;
+      a[k] = ldg_nt<typename XT::raw, VE>(x + (v < nvec ? v : nvec - 1) * VE);  // past the end: re-read, not stored
+    }
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+      const int64_t v = v0 + k * 256;
+#pragma unroll
+      for (int j = 0; j < VE; ++j) a[k].v[j] = XT::from_f32(one(XT::to_f32(a[k].v[j])));
+      if (v < nvec) stg_nt<typename XT::raw, VE>(out + v * VE, a[k]);
+    }
   }
   if (blockIdx.x == 0 && threadIdx.x < n - nvec * VE) {
     const int64_t i = nvec * VE + threadIdx.x;
@@ -112,8 +129,8 @@ template <typename XT>
 static void round_to_type_launch(const void* x, void* out, int64_t n, int mode, hipStream_t st) {
   using R = typename XT::raw;
   constexpr int VE = 16 / (int)sizeof(R);
-  int64_t want = cdiv(n / VE, 256 * 4);
-  const unsigned grid = (unsigned)(want < 1 ? 1 : want > (1 << 20) ? (1 << 20) : want);
+  const int64_t want = cdiv(n / VE, 256 * 4);
+  const unsigned grid = (unsigned)(want < 1 ? 1 : want);
   if (mode == 0)
     hipLaunchKernelGGL((round_to_type_kernel<XT, 0>), grid, 256, 0, st, (const R*)x, (R*)out, n);
   else if (mode == 1)

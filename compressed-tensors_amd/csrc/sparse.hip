@@ -1499,12 +1499,12 @@ bytemask24_vec_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64
     int64_t i = i0 + k * kBlock;
     if (i >= nitems) i = nitems - 1;  // re-read, not stored
     if constexpr (sizeof(R) * N == 16) {
-      a[k] = ldg<R, N>(x + i * N);
+      a[k] = ldg_nt<R, N>(x + i * N);
     } else {
 #pragma unroll
       for (int h = 0; h < (int)(sizeof(R) * N / 16); ++h) {
         constexpr int PER = 16 / sizeof(R);
-        const Vec<R, PER> part = ldg<R, PER>(x + i * N + h * PER);
+        const Vec<R, PER> part = ldg_nt<R, PER>(x + i * N + h * PER);
 #pragma unroll
         for (int j = 0; j < PER; ++j) a[k].v[h * PER + j] = part.v[j];
       }
@@ -1520,7 +1520,7 @@ bytemask24_vec_kernel(const R* __restrict__ x, uint8_t* __restrict__ mask, int64
       const uint32_t kq = (keep >> (4 * q)) & 15u;
       o.v[q] = (kq | (kq << 7) | (kq << 14) | (kq << 21)) & 0x01010101u;
     }
-    if (i < nitems) stg<uint32_t, N / 4>(reinterpret_cast<uint32_t*>(mask + i * N), o);
+    if (i < nitems) stg_nt<uint32_t, N / 4>(reinterpret_cast<uint32_t*>(mask + i * N), o);
   }
 }
 
