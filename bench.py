@@ -32,6 +32,9 @@ that no pass finds its input in the last-level cache:
                     quantize and pack, as separate passes and as one
   hadamard          block-128 and full 4096 rotations of 8192 x 4096 activations and of
                     4096 x 4096 / 14336 x 4096 weights
+  standalone        single reference functions called on their own, one call per 14336 x 4096
+                    tensor: round_to_quantized_type, pack_to_int32 / unpack_from_int32,
+                    pack_fp4_to_uint8 / unpack_fp4_from_uint8, get_24_bytemasks
   api               ModelCompressor.compress_model / decompress_model on a module tree of the
                     default set's 224 weights (wall time of the host mirror above the C ABI)
 """
@@ -358,22 +361,12 @@ def other_workload(torch, name, seed):
                Op("activations: per-token min-max + scales (8 x 8192x4096)", a_obs, 2 * na, "observe_wide_kernel"),
                Op("activations: per-token fp8 fake-quantize (8 x 8192x4096)", a_fq, 4 * na, "qdq_vec_kernel"),
                Op("activations: scales + fake-quantize in one pass (8 x 8192x4096)", a_dyn, 4 * na, "dynamic_rows_kernel")]
-        # A8 on its own: every element to the nearest fp8 value, dtype kept
-        r_calls, nr = [], 0
-        for _ in range(8):
-            x = randn(14336, 4096)
-            out = torch.empty_like(x)
-            keep.extend([x, out])
-            ra = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), 1, 8, st)
-            r_calls.append(lambda ra=ra: _lib.check(lib.ctmi_round_to_quantized_type(*ra)))
-            nr += x.numel()
-        ops.append(Op("round_to_quantized_type alone (fp8), bf16 14336x4096 (x8)", r_calls, 4 * nr, "round_to_type_kernel"))
         return "fp8 W8A8 quantize/dequantize GB/s, Llama-3-8B-shaped weights + per-token activations", ops, keep
 
     if name == "sparse":
         copies = 6
         c_calls, d_calls, s_calls, t_calls, two_step, one_step = [], [], [], [], [], []
-        back_two, back_one, s16_calls, t16_calls, pk_calls, up_calls, bm_calls = [], [], [], [], [], [], []
+        back_two, back_one, s16_calls, t16_calls, pk_calls, up_calls = [], [], [], [], [], []
         stacked_jobs = []
         nb = 8192 * 8192
         nnz_total = 0
@@ -432,8 +425,6 @@ def other_workload(torch, name, seed):
             bools_back = torch.empty_like(bools)
             packed = torch.empty(rows, cols // 8, dtype=torch.uint8, device=dev)
             keep.extend([bools, bools_back, packed])
-            bm = (w.data_ptr(), code(w.dtype), bools_back.data_ptr(), w.numel(), st)
-            bm_calls.append(lambda bm=bm: _lib.check(lib.ctmi_get_24_bytemasks(*bm)))
             pk = (bools.data_ptr(), packed.data_ptr(), rows, cols, st)
             up = (packed.data_ptr(), bools_back.data_ptr(), rows, cols, st)
             _lib.check(lib.ctmi_pack_bitmasks(*pk))
@@ -508,7 +499,6 @@ def other_workload(torch, name, seed):
                Op("sparse-24-bitmask decompress, bf16, all 16 in one call (8 per launch)",
                   [lambda: _lib.check(lib.ctmi_sparse24_decompress_many(*dm16))],
                   2 * s24_bytes - copies24 * (n24 // 8), "sparse24_scatter_kernel", launches=chained(copies24)),
-               Op("get_24_bytemasks, 14336x4096 bf16 -> bool", bm_calls, copies24 * (2 * n24 + n24), "bytemask24_vec_kernel"),
                Op("pack_bitmasks, 14336x4096 bool", pk_calls, copies24 * (n24 + n24 // 8), "pack_bitmasks"),
                Op("unpack_bitmasks", up_calls, copies24 * (n24 + n24 // 8), "unpack_bitmasks"),
                Op("bf16 -> fp8 codes -> 2:4 compress, two steps (14336x4096)", two_step, fused24_bytes, "qdq_vec_kernel", primary=False),
@@ -617,24 +607,6 @@ def other_workload(torch, name, seed):
         ops += [Op("nvfp4 activations: group-16 scales (16 x 4096x4096)", o_calls, 2 * na + na // 16, "observe_flat_kernel"),
                 Op("nvfp4 activations: fake-quantize (16 x 4096x4096)", f_calls, 4 * na + na // 16, "nvfp4_qdq_vec_kernel"),
                 Op("nvfp4 activations: scales + fake-quantize in one pass (16 x 4096x4096)", y_calls, 4 * na, "nvfp4_dynamic_kernel")]
-        # A13 / A14 on their own: values already on the e2m1 grid <-> two codes a byte
-        grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], device=dev)
-        p4_calls, u4_calls, n4 = [], [], 0
-        for _ in range(16):
-            r, c = 14336, 4096
-            x = (grid[torch.randint(0, 8, (r, c), generator=gen, device=dev)]
-                 * (torch.randint(0, 2, (r, c), generator=gen, device=dev) * 2 - 1)).to(torch.bfloat16)
-            codes = torch.empty(r, c // 2, dtype=torch.uint8, device=dev)
-            back = torch.empty_like(x)
-            keep.extend([x, codes, back])
-            pa = (x.data_ptr(), code(x.dtype), codes.data_ptr(), r, c, st)
-            ua = (codes.data_ptr(), back.data_ptr(), code(back.dtype), r, c, st)
-            _lib.check(lib.ctmi_pack_fp4_to_uint8(*pa))
-            p4_calls.append(lambda pa=pa: _lib.check(lib.ctmi_pack_fp4_to_uint8(*pa)))
-            u4_calls.append(lambda ua=ua: _lib.check(lib.ctmi_unpack_fp4_from_uint8(*ua)))
-            n4 += r * c
-        ops += [Op("pack_fp4_to_uint8 alone, bf16 14336x4096 (x16)", p4_calls, 2 * n4 + n4 // 2, "fp4_pack_vec_kernel"),
-                Op("unpack_fp4_from_uint8 alone, to bf16 (x16)", u4_calls, 2 * n4 + n4 // 2, "fp4_unpack_vec_kernel")]
         return "nvfp4-pack-quantized compress/decompress + activation fake-quantize GB/s", ops, keep
 
     if name == "one-shot":
@@ -694,6 +666,22 @@ def other_workload(torch, name, seed):
                   gidx_cmp, 2 * n + 2 * g + n // 2, "pq_gidx_compress_kernel", primary=False),
                Op("activation ordering (g_idx): observer + qparams + quantize + pack in one pass (one call each)",
                   gidx_one, 2 * n + 2 * g + n // 2, "observe_pack_table_kernel", primary=False)]
+        return "one-shot W4A16 g128 compression GB/s (no scales given), Llama-3-8B-shaped weights", ops, keep
+
+    if name == "standalone":
+        # the entry points of single reference functions called on their own (a caller that
+        # holds codes, a mask or a tensor to round already): one call per 14336x4096 tensor
+        ops = []
+        # A8 on its own: every element to the nearest fp8 value, dtype kept
+        r_calls, nr = [], 0
+        for _ in range(8):
+            x = randn(14336, 4096)
+            out = torch.empty_like(x)
+            keep.extend([x, out])
+            ra = (x.data_ptr(), out.data_ptr(), code(x.dtype), x.numel(), 1, 8, st)
+            r_calls.append(lambda ra=ra: _lib.check(lib.ctmi_round_to_quantized_type(*ra)))
+            nr += x.numel()
+        ops.append(Op("round_to_quantized_type alone (fp8), bf16 14336x4096 (x8)", r_calls, 4 * nr, "round_to_type_kernel"))
         # A9 / A10 on their own: int8 codes <-> packed words (callers that hold codes already)
         pk_calls, up_calls, n_codes = [], [], 0
         for _ in range(16):
@@ -712,7 +700,35 @@ def other_workload(torch, name, seed):
                    "pack_dim1_vec_kernel"),
                 Op("unpack_from_int32 alone, 14336x4096 (x16)", up_calls, n_codes + n_codes // 2,
                    "unpack_dim1_vec_kernel")]
-        return "one-shot W4A16 g128 compression GB/s (no scales given), Llama-3-8B-shaped weights", ops, keep
+        # A13 / A14 on their own: values already on the e2m1 grid <-> two codes a byte
+        grid = torch.tensor([0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0], device=dev)
+        p4_calls, u4_calls, n4 = [], [], 0
+        for _ in range(16):
+            r, c = 14336, 4096
+            x = (grid[torch.randint(0, 8, (r, c), generator=gen, device=dev)]
+                 * (torch.randint(0, 2, (r, c), generator=gen, device=dev) * 2 - 1)).to(torch.bfloat16)
+            codes = torch.empty(r, c // 2, dtype=torch.uint8, device=dev)
+            back = torch.empty_like(x)
+            keep.extend([x, codes, back])
+            pa = (x.data_ptr(), code(x.dtype), codes.data_ptr(), r, c, st)
+            ua = (codes.data_ptr(), back.data_ptr(), code(back.dtype), r, c, st)
+            _lib.check(lib.ctmi_pack_fp4_to_uint8(*pa))
+            p4_calls.append(lambda pa=pa: _lib.check(lib.ctmi_pack_fp4_to_uint8(*pa)))
+            u4_calls.append(lambda ua=ua: _lib.check(lib.ctmi_unpack_fp4_from_uint8(*ua)))
+            n4 += r * c
+        ops += [Op("pack_fp4_to_uint8 alone, bf16 14336x4096 (x16)", p4_calls, 2 * n4 + n4 // 2, "fp4_pack_vec_kernel"),
+                Op("unpack_fp4_from_uint8 alone, to bf16 (x16)", u4_calls, 2 * n4 + n4 // 2, "fp4_unpack_vec_kernel")]
+        # A20 on its own: the top-2-of-4 mask of a dense tensor, one bool per element
+        bm_calls, nbm = [], 0
+        for _ in range(8):
+            w = randn(14336, 4096, 0.02)
+            mask = torch.empty(w.shape, dtype=torch.bool, device=dev)
+            keep.extend([w, mask])
+            bm = (w.data_ptr(), code(w.dtype), mask.data_ptr(), w.numel(), st)
+            bm_calls.append(lambda bm=bm: _lib.check(lib.ctmi_get_24_bytemasks(*bm)))
+            nbm += w.numel()
+        ops.append(Op("get_24_bytemasks alone, bf16 14336x4096 -> bool (x8)", bm_calls, 3 * nbm, "bytemask24_vec_kernel"))
+        return "single reference functions called on their own, GB/s", ops, keep
 
     if name == "hadamard":
         ops = []
@@ -1008,6 +1024,13 @@ def cpu_baseline_other(torch, workload, seed):
         def run():
             s, z = oquant.observe_weight(w, oargs)
             opack.pack_quantized_compress(w, s, oargs, zero_point=z)
+    elif workload == "standalone":
+        codes = torch.randint(-8, 8, (14336, 4096), generator=g, dtype=torch.int8)
+        n = codes.numel()
+        nbytes, what = 2 * (n + n // 2), "pack_to_int32 + unpack_from_int32 of 14336x4096 int8 codes (4 bits)"
+
+        def run():
+            opack.unpack_from_int32(opack.pack_to_int32(codes, 4), 4, codes.shape)
     else:
         return None
     med = median_time(run)
@@ -1251,7 +1274,7 @@ def api_level(torch, seed, steps):
     return out
 
 
-OTHER_WORKLOADS = ("fp8-w8a8", "sparse", "nvfp4", "hadamard", "one-shot")
+OTHER_WORKLOADS = ("fp8-w8a8", "sparse", "nvfp4", "hadamard", "one-shot", "standalone")
 
 MAX_LINE = 1500  # characters of the line on stdout: what reads it keeps a short tail only
 
