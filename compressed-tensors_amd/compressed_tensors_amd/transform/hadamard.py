@@ -821,6 +821,16 @@ class HadamardTransform(TransformBase):
             transposed = not transposed
         return left, transposed
 
+    def _signs_on(self, device) -> Optional[Tensor]:
+        """the sign vector as fp32 on `device`, copied there once (a call per forward pass
+        must not pay a host-to-device copy)"""
+        if self.signs is None:
+            return None
+        key = ("signs", id(self.signs), str(device))
+        if key not in self._factor:
+            self._factor[key] = self.signs.to(device=device, dtype=torch.float32).contiguous()
+        return self._factor[key]
+
     def same_as(self):
         return (self.size, id(self.signs), id(self.perm), id(self.block), self.args.location,
                 self.args.inverse, self.module_type, self.precision)
@@ -837,7 +847,8 @@ class HadamardTransform(TransformBase):
         xs = [to_gpu(v) for v in values]
         if left:
             xs = [x.transpose(0, -1) for x in xs]
-        s_in, s_out = (None, self.signs) if transposed else (self.signs, None)
+        signs = self._signs_on(xs[0].device)
+        s_in, s_out = (None, signs) if transposed else (signs, None)
         in_place = in_place and not left and all(
             x.is_cuda and x.is_contiguous() and x.data_ptr() % 16 == 0 for x in xs)
         ys = hadamard_apply_many(xs, n, sign_in=s_in, sign_out=s_out, in_place=in_place)
@@ -920,14 +931,18 @@ class HadamardTransform(TransformBase):
         s_in = s_out = None
         if self.signs is not None:
             if transposed:
-                s_out = self.signs
+                s_out = self._signs_on(x.device)
             else:
-                s_in = self.signs
+                s_in = self._signs_on(x.device)
         if self.perm is not None:
             # W' = W[p][:, p]:  x W' = ((x scattered to p) W) gathered at p
-            p = self.perm.to(x.device)
+            key = ("perm", id(self.perm), str(x.device))
+            if key not in self._factor:  # the permutation and its inverse, on the device once
+                on_device = self.perm.to(x.device)
+                self._factor[key] = (on_device, torch.argsort(on_device))
+            p, p_inverse = self._factor[key]
             blocks = x.unflatten(-1, (x.shape[-1] // n, n))
-            x = blocks.index_select(-1, torch.argsort(p)).flatten(-2, -1)
+            x = blocks.index_select(-1, p_inverse).flatten(-2, -1)
         if mfma:
             y = hadamard_apply(x, n, sign_in=s_in, sign_out=s_out)
         elif big is not None:

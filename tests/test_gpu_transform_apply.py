@@ -289,3 +289,30 @@ def test_many_tensors_in_place(n, dtype, gpu):
         hadamard_apply_many([inner], n, in_place=True)
     assert_bit_equal(hadamard_apply_many([inner], n, sign_in=q)[0],
                      hadamard_apply_many([inner.clone()], n, sign_in=q)[0], "off a 16-byte boundary")
+
+
+def test_online_transform_keeps_its_signs_and_permutation_on_the_device(gpu):
+    """a forward pass through an online transform copies nothing from the host: sign vector
+    and permutation go to the device at the first call and stay"""
+    from compressed_tensors_amd.transform import TransformArgs, TransformFactory, TransformScheme
+
+    announce("transform device copies")
+    model = Stack(256, 64, dtype=torch.bfloat16).to(gpu)
+    scheme = TransformScheme(type="random-hadamard", randomize=True, head_dim=128,
+                             apply=[TransformArgs(targets="Linear", location="input")])
+    TransformFactory.from_scheme(scheme, name="R", seed=4).apply_to_model(model, use_tqdm=False)
+    tfm = model.fcs[0].R_input
+    assert tfm.signs.device.type == "cpu" and tfm.perm.device.type == "cpu"
+    x = torch.randn(3, 256, device=gpu, dtype=torch.bfloat16)
+    with torch.no_grad():
+        first = model(x)
+    kept = {k[0]: v for k, v in tfm._factor.items() if k[0] in ("signs", "perm")}
+    assert kept["signs"].is_cuda and kept["signs"].dtype == torch.float32
+    assert all(t.is_cuda for t in kept["perm"])
+    before = {k: (v.data_ptr() if torch.is_tensor(v) else tuple(t.data_ptr() for t in v))
+              for k, v in tfm._factor.items() if k[0] in ("signs", "perm")}
+    with torch.no_grad():
+        assert_bit_equal(model(x), first, "second call")
+    after = {k: (v.data_ptr() if torch.is_tensor(v) else tuple(t.data_ptr() for t in v))
+             for k, v in tfm._factor.items() if k[0] in ("signs", "perm")}
+    assert after == before
